@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu] [--no-extra]
+
+Prints ONE JSON line.  The headline is the fp16 paged-attention decode step (configuration 3
+of BASELINE.json): a "step" is one hipattn_paged_attention call on the whole synthetic batch
+(KV-cache write of the new tokens + split-context decode + merge), inputs resident in HBM.
+`value` is algorithmic KV bytes / wall time of a step; `roofline` is the same byte count over
+the average duration of the dominant kernel (the split-context decode kernel), measured with
+HIP events recorded by the library around that launch.  Unless --no-extra is given, the other
+configurations are measured the same way and reported under "workloads" in the same line
+(c2: bf16 causal prefill SDPA in TFLOP/s against the dense bf16 MFMA peak; c4: u8-KV decode;
+c5: mixed chunked prefill + decode).  `cpu_baseline` times the CPU oracle (a restatement, not
+OpenVINO's CPU plugin: OpenVINO is not installed) on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_steps(hip, fn, steps, warmup):
+    """fn(i) enqueues one step on the default stream.  Returns (ms per step, dominant-kernel ms)."""
+    for i in range(warmup):
+        fn(i)
+    hip.check(hip.lib().hipattn_stream_synchronize(None))
+    befores = [hip.Event() for _ in range(steps)]
+    afters = [hip.Event() for _ in range(steps)]
+    start, stop = hip.Event(), hip.Event()
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        hip.profile_dominant_kernel(befores[i], afters[i])
+        fn(i)
+    hip.profile_dominant_kernel(None, None)
+    stop.record()
+    stop.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = start.elapsed_ms(stop) / steps
+    kern = [befores[i].elapsed_ms(afters[i]) for i in range(steps)]
+    for e in befores + afters + [start, stop]:
+        e.close()
+    return ev_ms, wall_ms, sum(kern) / len(kern)
+
+
+def bench_paged(hip, case, steps, warmup, name):
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import helpers as H
+    from openvino_contrib_amd import workloads as W
+
+    dev = H.PagedDeviceCase(hip, case)
+    desc = H.pa_desc(hip, case)
+    ws_bytes = hip.paged_attention_workspace_size(desc)
+    ws = hip.DeviceBuffer(ws_bytes) if ws_bytes else None
+
+    def step(_):
+        hip.paged_attention(desc, dev.q, dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                            dev.subsequence_begins, dev.block_indices, dev.block_indices_begins, dev.out, ws)
+
+    ms, wall_ms, kern_ms = time_steps(hip, step, steps, warmup)
+    path = hip.last_kernel_path()
+    kv_bytes = W.paged_kv_bytes(case)
+    flops = W.paged_flops(case)
+    res = {
+        "workload": name, "kernel_path": path, "ms_per_step": ms, "host_ms_per_step": wall_ms,
+        "dominant_kernel_ms": kern_ms, "kv_bytes": kv_bytes, "flops": flops, "workspace_bytes": ws_bytes,
+        "kv_gbs": kv_bytes / (ms * 1e-3) / 1e9, "tflops": flops / (ms * 1e-3) / 1e12,
+    }
+    dev.free()
+    if ws:
+        ws.free()
+    return res
+
+
+def bench_sdpa(hip, case, steps, warmup, name):
+    from openvino_contrib_amd import workloads as W
+
+    desc = hip.SdpaDesc(case["dtype"], case["B"], case["Hq"], case["Hkv"], case["Lq"], case["Lk"], case["D"], 1, 0.0)
+    q = hip.DeviceBuffer.from_numpy(case["q_store"])
+    k = hip.DeviceBuffer.from_numpy(case["k_store"])
+    v = hip.DeviceBuffer.from_numpy(case["v_store"])
+    out = hip.DeviceBuffer(case["q_store"].nbytes)
+
+    def step(_):
+        hip.sdpa(desc, q, k, v, out)
+
+    ms, wall_ms, kern_ms = time_steps(hip, step, steps, warmup)
+    flops = W.sdpa_flops(case["B"], case["Hq"], case["Lq"], case["Lk"], case["D"], True)
+    res = {"workload": name, "kernel_path": hip.last_kernel_path(), "ms_per_step": ms, "host_ms_per_step": wall_ms,
+           "dominant_kernel_ms": kern_ms, "flops": flops, "tflops": flops / (ms * 1e-3) / 1e12}
+    for b in (q, k, v, out):
+        b.free()
+    return res
+
+
+def roofline_hbm(res, traffic=None):
+    a = res["kv_bytes"] / (res["dominant_kernel_ms"] * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
+            "traffic": traffic, "kernel": "paged_decode_kernel"}
+
+
+def roofline_mfma(res):
+    a = res["flops"] / (res["dominant_kernel_ms"] * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "sdpa_flash_kernel"}
+
+
+def cpu_baseline_paged(case, n_seqs, budget_s=20.0):
+    """Oracle (port) on the first n_seqs sequences of the case, attention only."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import oracle as O
+    from openvino_contrib_amd import workloads as W
+
+    n = min(n_seqs, case["S"])
+    sub = dict(case)
+    sub["S"] = n
+    sub["past_lens"] = case["past_lens"][:n]
+    sub["subsequence_begins"] = case["subsequence_begins"][:n + 1]
+    sub["block_indices_begins"] = case["block_indices_begins"][:n + 1]
+    T = int(sub["subsequence_begins"][-1])
+    kc, vc = case["key_cache"], case["value_cache"]
+    best = None
+    t_end = time.perf_counter() + budget_s
+    reps = 0
+    while reps < 3 and (reps == 0 or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        O.paged_attention(case["q"][:T], case["k_new"][:T], case["v_new"][:T], kc, vc, case["cache_dtype"],
+                          sub["past_lens"], sub["subsequence_begins"], case["block_indices"],
+                          sub["block_indices_begins"], case["Hq"], case["Hkv"], case["D"], case["block_size"],
+                          sliding_window=case["sliding_window"], do_write=False)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        reps += 1
+    b = W.paged_kv_bytes(sub)
+    return {"value": b / best / 1e9, "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+            "sample": "oracle paged attention (no cache write) on the first %d of %d sequences, best of %d, %.2f s"
+                      % (n, case["S"], reps, best)}
+
+
+def cpu_baseline_sdpa(case, budget_s=20.0):
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O
+    from openvino_contrib_amd import workloads as W
+
+    G = case["Hq"] // case["Hkv"]
+    t0 = time.perf_counter()
+    O.sdpa(case["q"][:1, :G], case["k"][:1, :1], case["v"][:1, :1], causal=True)
+    dt = time.perf_counter() - t0
+    fl = W.sdpa_flops(1, G, case["Lq"], case["Lk"], case["D"], True)
+    return {"value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
+            "sample": "oracle fp32 SDPA on batch 0, kv head 0 (%d of %d query heads), %.2f s"
+                      % (G, case["B"] * case["Hq"], dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-extra", action="store_true", help="measure the headline workload only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
+
+    from openvino_contrib_amd import capi as hip
+    from openvino_contrib_amd import workloads as W
+
+    hip.lib()
+    if hip.device_count() < 1:
+        sys.exit("bench.py: no HIP device")
+    hip.check(hip.lib().hipattn_set_device(0))
+    info = hip.device_info(0)
+    log("device:", info.name.decode(), info.arch.decode(), info.compute_units, "CUs")
+
+    names = {"c2": "config2: bf16 causal prefill SDPA B4 Hq32 Hkv8 L2048 D128",
+             "c3": "config3: fp16 paged decode, 64 seq x 1 token, ctx U[512,8192], blk 32, Hq32 Hkv8 D128",
+             "c4": "config4: u8-KV paged decode, 128 seq, ctx U[1024,16384], Hq64 Hkv8 D128",
+             "c5": "config5: 8x512 prefill chunks + 120 decode, window 4096, bf16 q, fp16 cache, Hq64 Hkv8 D128"}
+    makers = {"c2": W.config2, "c3": W.config3, "c4": W.config4, "c5": W.config5}
+    order = [args.workload] + ([w for w in ("c3", "c2", "c4", "c5") if w != args.workload] if not args.no_extra else [])
+    results, cpu = {}, {}
+    for w in order:
+        t0 = time.perf_counter()
+        case = makers[w]()
+        log("%s: inputs generated in %.1f s" % (w, time.perf_counter() - t0))
+        if w == "c2":
+            r = bench_sdpa(hip, case, args.steps, args.warmup, names[w])
+            r["roofline"] = roofline_mfma(r)
+        else:
+            r = bench_paged(hip, case, args.steps, args.warmup, names[w])
+            r["roofline"] = roofline_hbm(r)
+            if w == "c5":
+                t_ideal = max(r["kv_bytes"] / (HBM_PEAK_GBS * 1e9), r["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12))
+                r["ideal_ms"] = t_ideal * 1e3
+                r["frac_of_ideal"] = t_ideal * 1e3 / r["ms_per_step"]
+        log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f"
+            % (w, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"]))
+        if not args.no_cpu and w == args.workload:
+            cpu = cpu_baseline_sdpa(case) if w == "c2" else cpu_baseline_paged(case, 8)
+            log("cpu baseline:", cpu)
+        results[w] = r
+        del case
+
+    head = results[args.workload]
+    is_sdpa = args.workload == "c2"
+    line = {
+        "metric": "prefill SDPA TFLOPS" if is_sdpa else "paged-attn decode KV GB/s",
+        "value": head["tflops"] if is_sdpa else head["kv_gbs"],
+        "unit": "TFLOP/s" if is_sdpa else "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if is_sdpa else ("u8" if args.workload == "c4" else "f16"),
+        "data": "synthetic",
+        "config": {"workload": head["workload"], "kernel_path": head["kernel_path"],
+                   "device": info.name.decode(), "arch": info.arch.decode()},
+        "roofline": head["roofline"],
+        "cpu_baseline": cpu if cpu else None,
+        "workloads": {k: v for k, v in results.items()},
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,203 @@
+/*
+ * hipattn - thin C ABI over the MI355X (gfx950) attention kernels.
+ *
+ * This is the boundary the C++ plugin operators (SdpaOp, PagedAttentionOp), the tests
+ * and the benchmark call.  Plain C: pointers, sizes and POD descriptors; no C++ or
+ * framework types.  Every pointer named "device" must be device memory of the current
+ * HIP device; all calls are asynchronous on the given stream unless stated; nothing
+ * here allocates behind the caller's back: scratch memory comes in through the
+ * workspace arguments (the counterpart of the reference's WorkbufferRequest,
+ * modules/nvidia_plugin/src/cuda_operation_base.hpp:114-117).  Functions return a
+ * status code and never throw; hipattn_last_error_string() describes the last failure
+ * on the calling thread.
+ *
+ * Reference citations are relative to modules/nvidia_plugin/ of openvino_contrib.
+ */
+#ifndef HIPATTN_H_
+#define HIPATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPATTN_VERSION_MAJOR 0
+#define HIPATTN_VERSION_MINOR 1
+
+typedef enum hipattn_status {
+    HIPATTN_OK = 0,
+    HIPATTN_INVALID_ARGUMENT = 1,   /* null pointer, negative size, inconsistent descriptor */
+    HIPATTN_UNSUPPORTED = 2,        /* valid request this build has no kernel for */
+    HIPATTN_WORKSPACE_TOO_SMALL = 3,
+    HIPATTN_HIP_ERROR = 4,          /* a HIP runtime call failed; see hipattn_last_error_string */
+    HIPATTN_NO_DEVICE = 5
+} hipattn_status;
+
+typedef enum hipattn_dtype {
+    HIPATTN_F32 = 0,
+    HIPATTN_F16 = 1,
+    HIPATTN_BF16 = 2,
+    HIPATTN_U8 = 3 /* KV cache only: rows of [scale f32][zero-point f32][head_dim bytes] */
+} hipattn_dtype;
+
+typedef struct hipattn_stream_t* hipattn_stream; /* a hipStream_t; NULL is the default stream */
+typedef struct hipattn_event_t* hipattn_event;   /* a hipEvent_t */
+
+typedef struct hipattn_device_info {
+    char name[128];
+    char arch[32];            /* "gfx950" on MI355X */
+    int compute_units;
+    int wavefront_size;
+    int lds_bytes_per_workgroup;
+    int clock_mhz;
+    size_t global_mem_bytes;
+} hipattn_device_info;
+
+/* ---- device layer: replaces CUDA::Device / Stream / Allocation / Event wrappers
+ *      (src/cuda/runtime.hpp:62-324, src/cuda/event.hpp:11-29) -------------------------- */
+
+const char* hipattn_last_error_string(void);
+const char* hipattn_status_string(hipattn_status status);
+int hipattn_version(void); /* major * 1000 + minor */
+
+hipattn_status hipattn_device_count(int* count);
+hipattn_status hipattn_set_device(int device);
+hipattn_status hipattn_get_device_info(int device, hipattn_device_info* info);
+
+hipattn_status hipattn_stream_create(hipattn_stream* stream); /* default priority, non-blocking */
+hipattn_status hipattn_stream_destroy(hipattn_stream stream);
+hipattn_status hipattn_stream_synchronize(hipattn_stream stream);
+
+/* runtime.hpp:188-229, 235, 273-281 (DefaultAllocation, Allocation, Stream::malloc) */
+hipattn_status hipattn_malloc(void** device_ptr, size_t bytes);
+hipattn_status hipattn_free(void* device_ptr);
+hipattn_status hipattn_malloc_async(void** device_ptr, size_t bytes, hipattn_stream stream);
+hipattn_status hipattn_free_async(void* device_ptr, hipattn_stream stream);
+/* pinned host memory for staging (allocated, never registered) */
+hipattn_status hipattn_host_malloc(void** host_ptr, size_t bytes);
+hipattn_status hipattn_host_free(void* host_ptr);
+
+/* runtime.hpp:236-252, 267-285 (Stream::upload / download / transfer / memset) */
+hipattn_status hipattn_memcpy_h2d_async(void* device_dst, const void* host_src, size_t bytes, hipattn_stream stream);
+hipattn_status hipattn_memcpy_d2h_async(void* host_dst, const void* device_src, size_t bytes, hipattn_stream stream);
+hipattn_status hipattn_memcpy_d2d_async(void* device_dst, const void* device_src, size_t bytes, hipattn_stream stream);
+/* byte fill done by a kernel (safe to record into a captured graph) */
+hipattn_status hipattn_fill_async(void* device_dst, int byte_value, size_t bytes, hipattn_stream stream);
+
+hipattn_status hipattn_event_create(hipattn_event* event);
+hipattn_status hipattn_event_destroy(hipattn_event event);
+hipattn_status hipattn_event_record(hipattn_event event, hipattn_stream stream);
+hipattn_status hipattn_event_synchronize(hipattn_event event);
+hipattn_status hipattn_event_elapsed_ms(hipattn_event start, hipattn_event stop, float* ms);
+
+/* ---- v13::ScaledDotProductAttention -------------------------------------------------
+ * Replaces the decomposed chain the reference executes after
+ * ScaledDotProductAttentionDecomposition (src/transformer/cuda_graph_transformer.cpp:151-156):
+ * MatMulOp (src/ops/matmul.cpp:185-227), scale Multiply (src/ops/multiply.cpp:43), the
+ * causal mask Range/GreaterEqual/Select/Add (src/ops/select.cpp:50-91, src/ops/add.cpp:17-43),
+ * SoftmaxOp (src/ops/softmax.cpp:178-193) and the second MatMulOp, with one fused kernel.
+ *
+ * q [batch, num_heads_q, len_q, head_dim], k and v [batch, num_heads_kv, len_kv, head_dim],
+ * out like q; all contiguous and of `dtype`.  Query head h reads kv head
+ * h / (num_heads_q / num_heads_kv).  causal != 0: query row i sees keys j <= i
+ * (lower-triangular, top-left aligned).  scale <= 0 selects 1/sqrt(head_dim).
+ * Softmax and accumulation are fp32 whatever `dtype` is. */
+typedef struct hipattn_sdpa_desc {
+    hipattn_dtype dtype;
+    int batch;
+    int num_heads_q;
+    int num_heads_kv;
+    int len_q;
+    int len_kv;
+    int head_dim;
+    int causal;
+    float scale;
+} hipattn_sdpa_desc;
+
+hipattn_status hipattn_sdpa_workspace_size(const hipattn_sdpa_desc* desc, size_t* bytes);
+hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const void* k, const void* v, void* out,
+                            void* workspace, size_t workspace_bytes, hipattn_stream stream);
+
+/* ---- PagedAttentionExtension --------------------------------------------------------
+ * No counterpart in the reference (its only KV-cache mechanism is the contiguous
+ * variable state, src/cuda_variable_state.hpp:135-160, src/ops/read_value.cpp:31-72,
+ * src/ops/assign.cpp:29-56, and its nearest scatter is src/kernels/scatter_nd_update.cu:19-34).
+ * Argument order follows the OpenVINO operator's inputs.
+ *
+ *   q                     [num_tokens, num_heads_q * head_dim]              q_dtype
+ *   k_new, v_new          [num_tokens, num_heads_kv * head_dim]             kv_dtype
+ *   key_cache,value_cache [num_blocks, num_heads_kv, block_size, row]       cache_dtype
+ *                         row = head_dim elements, or for HIPATTN_U8
+ *                         [scale f32][zero-point f32][head_dim bytes] per token and head
+ *   past_lens             [num_seqs] i32      tokens already cached per sequence
+ *   subsequence_begins    [num_seqs + 1] i32  token offsets of each sequence in this batch
+ *   block_indices         [...] i32           physical block ids, sequence after sequence
+ *   block_indices_begins  [num_seqs + 1] i32  offsets into block_indices
+ *   out                   [num_tokens, num_heads_q * head_dim]              out_dtype
+ *
+ * Step 1 (unless HIPATTN_PA_SKIP_CACHE_WRITE): token i of sequence s is written at
+ * logical position p = past_lens[s] + i, physical block
+ * block_indices[block_indices_begins[s] + p / block_size], row p % block_size; u8 caches
+ * are quantised on the fly.  Blocks outside the table or outside [0, num_blocks) are skipped.
+ * Step 2: that token attends cache positions j, max(0, p - sliding_window + 1) <= j <= p
+ * (all of 0..p when sliding_window <= 0).
+ * All index arrays live in device memory; the host only passes upper bounds:
+ * max_context_len >= max_s(past_lens[s] + q_len[s]) sizes the split of the context. */
+enum {
+    HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */
+    HIPATTN_PA_FORCE_GENERIC = 2     /* use the shape-generic kernels (testing aid) */
+};
+
+typedef struct hipattn_pa_desc {
+    hipattn_dtype q_dtype;     /* F16, BF16 or F32 */
+    hipattn_dtype kv_dtype;    /* type of k_new / v_new: F16, BF16 or F32 */
+    hipattn_dtype cache_dtype; /* F16, BF16, F32 or U8 */
+    hipattn_dtype out_dtype;   /* F16, BF16 or F32 */
+    int num_heads_q;
+    int num_heads_kv;
+    int head_dim;
+    int block_size;
+    int num_blocks;
+    int num_tokens;
+    int num_seqs;
+    int max_context_len;
+    int sliding_window;
+    float scale;       /* <= 0 selects 1/sqrt(head_dim) */
+    int flags;         /* HIPATTN_PA_* */
+    int decode_chunk;  /* tokens per split of a decode context; 0 = choose */
+} hipattn_pa_desc;
+
+hipattn_status hipattn_paged_attention_workspace_size(const hipattn_pa_desc* desc, size_t* bytes);
+hipattn_status hipattn_paged_attention(const hipattn_pa_desc* desc, const void* q, const void* k_new,
+                                       const void* v_new, void* key_cache, void* value_cache,
+                                       const int32_t* past_lens, const int32_t* subsequence_begins,
+                                       const int32_t* block_indices, const int32_t* block_indices_begins, void* out,
+                                       void* workspace, size_t workspace_bytes, hipattn_stream stream);
+
+/* Step 1 alone: the device-side KV-cache block writer. */
+hipattn_status hipattn_kv_cache_write(const hipattn_pa_desc* desc, const void* k_new, const void* v_new,
+                                      void* key_cache, void* value_cache, const int32_t* past_lens,
+                                      const int32_t* subsequence_begins, const int32_t* block_indices,
+                                      const int32_t* block_indices_begins, hipattn_stream stream);
+
+/* Bytes of one cache row (per token and kv head) for a cache type. */
+size_t hipattn_cache_row_bytes(hipattn_dtype cache_dtype, int head_dim);
+
+/* Measurement aid (no reference counterpart; the reference's per-op profiler wraps whole
+ * Execute calls with events, src/cuda_profiler.hpp:141-146).  While a pair of events is set
+ * on the calling thread, hipattn_sdpa / hipattn_paged_attention record `before` immediately
+ * ahead of and `after` immediately behind the launch of their dominant kernel (the flash
+ * kernel, or the split-context decode kernel when the batch has decode sequences), on the
+ * call's stream.  Pass NULLs to switch it off. */
+hipattn_status hipattn_profile_dominant_kernel(hipattn_event before, hipattn_event after);
+
+/* Name of the kernel path the last attention call on this thread dispatched to
+ * ("flash_mfma", "generic", "decode_mfma+merge", ...).  Diagnostic only. */
+const char* hipattn_last_kernel_path(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPATTN_H_ */

@@ -1,0 +1,76 @@
+"""Build recipe for libhipattn.so (HIP kernels + C ABI), gfx950 only.
+
+hipcc cross-compiles without a GPU.  The library is built in-tree, next to the sources
+(openvino_contrib_amd/csrc/libhipattn.so), so that it travels with the source tree.
+"""
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+INCLUDE = os.path.join(os.path.dirname(_HERE), "include")
+LIB_PATH = os.path.join(CSRC, "libhipattn.so")
+
+SOURCES = [
+    "hipattn_api.hip",
+    "kv_cache_write.hip",
+    "attention_generic.hip",
+    "paged_decode.hip",
+    "flash_prefill.hip",
+]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fvisibility=hidden",
+    "-Wall",
+    "-Wno-unused-function",
+    # keep hipcc from forming packed fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I" + INCLUDE,
+    "-I" + CSRC,
+]
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; libhipattn cannot be built")
+    return exe
+
+
+def _compile(src, extra):
+    obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
+    cmd = [hipcc()] + HIPCC_FLAGS + list(extra) + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s" % (src, r.stderr[-4000:]))
+    return obj, r.stderr
+
+
+def build_library(verbose=False, extra_flags=(), jobs=4):
+    """Compile every HIP source and link libhipattn.so.  Always recompiles."""
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(lambda s: _compile(s, extra_flags), SOURCES))
+    objs = [o for o, _ in results]
+    if verbose:
+        for _, err in results:
+            lines = [l for l in err.splitlines() if "packed-fp32-ops" not in l]
+            if lines:
+                print("\n".join(lines), file=sys.stderr)
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s" % r.stderr[-4000:])
+    for o in objs:
+        os.remove(o)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

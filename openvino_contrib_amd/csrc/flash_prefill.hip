@@ -1,0 +1,440 @@
+// Flash-style attention for prefill on gfx950: dense v13::ScaledDotProductAttention and the
+// multi-token (chunked prefill) sequences of PagedAttentionExtension share one kernel body.
+//
+// A workgroup of four wavefronts owns 128 query rows of one query head (32 rows per
+// wavefront) and walks the keys in tiles of 64.  K tiles are staged in LDS row-major, V tiles
+// transposed (the 4x8 patch each thread loads is transposed in registers on the way in), the
+// next tile's global loads are in flight while the current one is consumed.  Both products
+// run on v_mfma_f32_32x32x16 (f16 or bf16) with fp32 accumulation:
+//   S^T = K Q^T   (M = 32 keys, N = 32 query rows, contraction over head_dim)
+//   O^T = V^T P^T (M = 32 head-dim rows, N = 32 query rows, contraction over keys)
+// Computing the scores transposed leaves each lane with 8 consecutive-in-operand keys of one
+// query row, i.e. the accumulator of the first product already is the B operand of the
+// second; the softmax statistics of a row live in the two lanes l and l+32 and need a single
+// cross-lane exchange.  Scale, causal mask, sliding window and the online softmax (exp2
+// domain) are fused; fully masked key tiles are never visited.
+//
+// Replaces the reference's decomposed chain, which writes and re-reads the [B,H,Lq,Lk] score
+// tensor four times: MatMulOp::Execute (src/ops/matmul.cpp:185-227), Multiply
+// (src/ops/multiply.cpp:43), Select/Add mask (src/ops/select.cpp:50-91, src/ops/add.cpp:17-43),
+// SoftmaxOp::Execute (src/ops/softmax.cpp:178-193), TransposeOp (src/ops/transpose.cpp:87-135)
+// and ConvertOp (src/ops/convert.cpp:60).
+#include "device_common.hpp"
+#include "kernels.hpp"
+
+namespace hipattn {
+
+namespace flash {
+
+constexpr int kD = 128;
+constexpr int kTileQ = 128;   // query rows per workgroup
+constexpr int kTileK = 64;    // keys per LDS tile
+constexpr int kThreads = 256;
+constexpr int kKRow = 272;    // bytes per K row in LDS (256 + 16 pad)
+constexpr int kVRow = 136;    // bytes per V^T row in LDS (64 keys * 2 + 8 pad)
+
+template <bool kBf16>
+struct Mfma;
+template <>
+struct Mfma<false> {
+    using vec8 = half8_t;
+    static __device__ __forceinline__ float16_t mma(vec8 a, vec8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint16_t cvt(float x) { return float_to_f16_bits(x); }
+};
+template <>
+struct Mfma<true> {
+    using vec8 = bf16x8_t;
+    static __device__ __forceinline__ float16_t mma(vec8 a, vec8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint16_t cvt(float x) {
+        __bf16 b = (__bf16)x;
+        return __builtin_bit_cast(uint16_t, b);
+    }
+};
+
+// What one workgroup works on.
+struct Tile {
+    const uint16_t* q;   // first query row of the tile, this head
+    int64_t q_stride;    // elements between consecutive query rows
+    void* out;           // output base (element (0,0) of the tile's first row, this head)
+    int64_t out_stride;
+    int rows;            // valid query rows (<= 128)
+    int pos0;            // sequence position of query row 0
+    int kv_len;          // keys available
+    int causal;
+    int window;
+    int q_dtype;         // HIPATTN_F16 / HIPATTN_BF16 (converted to the MFMA type when they differ)
+    int out_dtype;
+    // keys / values
+    const uint8_t* k;
+    const uint8_t* v;
+    const int32_t* table;   // paged: this sequence's block ids; dense: nullptr
+    int table_len;
+    int num_blocks;
+    int64_t block_stride;   // paged: bytes between physical blocks
+    int block_size;
+};
+
+__device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key, bool& ok) {
+    ok = key < t.kv_len;
+    if (!ok) return 0;
+    if (t.table == nullptr) return (int64_t)key * (kD * 2);
+    const int lb = key / t.block_size;
+    const int pb = t.table[lb];
+    if (pb < 0 || pb >= t.num_blocks) {
+        ok = false;
+        return 0;
+    }
+    return (int64_t)pb * t.block_stride + (int64_t)(key % t.block_size) * (kD * 2);
+}
+
+template <bool kBf16>
+__device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t, int row, int d0) {
+    using vec8 = typename Mfma<kBf16>::vec8;
+    uint4_t raw = {0u, 0u, 0u, 0u};
+    if (row < t.rows) raw = *(const uint4_t*)(t.q + (int64_t)row * t.q_stride + d0);
+    const bool q_is_bf16 = (t.q_dtype == HIPATTN_BF16);
+    if (q_is_bf16 == kBf16) return __builtin_bit_cast(vec8, raw);
+    // widen through fp32 and round to the MFMA element type
+    uint4_t cv;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        float lo, hi;
+        if (q_is_bf16) {
+            lo = __uint_as_float(raw[w] << 16);
+            hi = __uint_as_float(raw[w] & 0xffff0000u);
+        } else {
+            lo = f16_bits_to_float((uint16_t)(raw[w] & 0xffffu));
+            hi = f16_bits_to_float((uint16_t)(raw[w] >> 16));
+        }
+        cv[w] = (uint32_t)Mfma<kBf16>::cvt(lo) | ((uint32_t)Mfma<kBf16>::cvt(hi) << 16);
+    }
+    return __builtin_bit_cast(vec8, cv);
+}
+
+template <bool kBf16>
+__device__ __forceinline__ void run_tile(const Tile& t, uint8_t* k_lds, uint8_t* v_lds, float scale) {
+    using M = Mfma<kBf16>;
+    using vec8 = typename M::vec8;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int n32 = lane & 31, hi = lane >> 5;
+    const int row = wave * 32 + n32;  // query row inside the tile
+    const float c = scale * kLog2e;
+
+    // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
+    vec8 qf[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) qf[i] = load_q_frag<kBf16>(t, row, i * 16 + hi * 8);
+
+    // key range this tile has to visit
+    int kv_hi = t.kv_len;
+    if (t.causal) kv_hi = min(kv_hi, t.pos0 + t.rows);
+    int kv_lo = 0;
+    if (t.window > 0) kv_lo = max(0, t.pos0 - t.window + 1);
+    kv_lo = (kv_lo / kTileK) * kTileK;
+
+    float16_t o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+    const int my_pos = t.pos0 + row;  // position of this lane's query row
+
+    // global -> register staging: thread (c16, r16) loads K rows r16 + 16k and V rows r16*4 + j
+    const int c16 = tid & 15, r16 = tid >> 4;
+    uint4_t kreg[4], vreg[4];
+    auto load_regs = [&](int tile_start) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            bool ok;
+            int64_t off = kv_row_offset(t, tile_start + r16 + 16 * k, ok);
+            kreg[k] = ok ? *(const uint4_t*)(t.k + off + c16 * 16) : (uint4_t){0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            bool ok;
+            int64_t off = kv_row_offset(t, tile_start + r16 * 4 + j, ok);
+            vreg[j] = ok ? *(const uint4_t*)(t.v + off + c16 * 16) : (uint4_t){0u, 0u, 0u, 0u};
+        }
+    };
+    auto store_lds = [&]() {
+#pragma unroll
+        for (int k = 0; k < 4; k++) *(uint4_t*)(k_lds + (r16 + 16 * k) * kKRow + c16 * 16) = kreg[k];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            uint2_t w;
+            if (e & 1) {
+                w[0] = (vreg[0][e >> 1] >> 16) | (vreg[1][e >> 1] & 0xffff0000u);
+                w[1] = (vreg[2][e >> 1] >> 16) | (vreg[3][e >> 1] & 0xffff0000u);
+            } else {
+                w[0] = (vreg[0][e >> 1] & 0xffffu) | (vreg[1][e >> 1] << 16);
+                w[1] = (vreg[2][e >> 1] & 0xffffu) | (vreg[3][e >> 1] << 16);
+            }
+            *(uint2_t*)(v_lds + (c16 * 8 + e) * kVRow + r16 * 8) = w;
+        }
+    };
+
+    if (kv_lo < kv_hi) load_regs(kv_lo);
+    for (int ts = kv_lo; ts < kv_hi; ts += kTileK) {
+        __syncthreads();  // everyone is done reading the previous tile
+        store_lds();
+        __syncthreads();
+        if (ts + kTileK < kv_hi) load_regs(ts + kTileK);
+
+        // ---- S^T = K Q^T
+        float16_t s[2];
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const vec8 a = *(const vec8*)(k_lds + (mt * 32 + n32) * kKRow + (i * 16 + hi * 8) * 2);
+                s[mt] = M::mma(a, qf[i], s[mt]);
+            }
+        }
+        // ---- scale + mask.  Register r of tile mt is key ts + mt*32 + 8*(r/4) + 4*hi + r%4.
+        const bool all_valid = (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
+                               (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float x = s[mt][r] * c;
+                if (!all_valid) {
+                    const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+                    bool ok = key < t.kv_len;
+                    if (t.causal) ok = ok && key <= my_pos;
+                    if (t.window > 0) ok = ok && key > my_pos - t.window;
+                    x = ok ? x : -INFINITY;
+                }
+                s[mt][r] = x;
+                mloc = fmaxf(mloc, x);
+            }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // row with nothing to attend yet
+        const float alpha = fast_exp2(m_run - m_safe);
+        m_run = m_new;
+        float lsum = 0.0f;
+        vec8 pf[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            uint4_t pw;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w] - m_safe);
+                const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1] - m_safe);
+                lsum += p0 + p1;
+                pw[w] = (uint32_t)M::cvt(p0) | ((uint32_t)M::cvt(p1) << 16);
+            }
+            pf[ks] = __builtin_bit_cast(vec8, pw);
+        }
+        l_run = l_run * alpha + lsum;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) o[dt] *= alpha;
+        }
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint8_t* vrow = v_lds + (dt * 32 + n32) * kVRow + (ks * 16 + 4 * hi) * 2;
+                uint4_t aw;
+                const uint2_t a0 = *(const uint2_t*)(vrow);
+                const uint2_t a1 = *(const uint2_t*)(vrow + 16);
+                aw[0] = a0[0];
+                aw[1] = a0[1];
+                aw[2] = a1[0];
+                aw[3] = a1[1];
+                o[dt] = M::mma(__builtin_bit_cast(vec8, aw), pf[ks], o[dt]);
+            }
+        }
+    }
+
+    // ---- normalise and store.  o[dt][r] is head-dim dt*32 + 8*(r/4) + 4*hi + r%4 of `row`.
+    l_run += __shfl_xor(l_run, 32, 64);
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    if (row < t.rows) {
+        const int64_t obase = (int64_t)row * t.out_stride;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                const int d = dt * 32 + 8 * rq + 4 * hi;
+                if (t.out_dtype == HIPATTN_F32) {
+                    float4 v4 = make_float4(o[dt][rq * 4] * inv, o[dt][rq * 4 + 1] * inv, o[dt][rq * 4 + 2] * inv,
+                                            o[dt][rq * 4 + 3] * inv);
+                    *(float4*)((float*)t.out + obase + d) = v4;
+                } else {
+                    uint2_t w;
+                    if (t.out_dtype == HIPATTN_F16) {
+                        w[0] = (uint32_t)float_to_f16_bits(o[dt][rq * 4] * inv) |
+                               ((uint32_t)float_to_f16_bits(o[dt][rq * 4 + 1] * inv) << 16);
+                        w[1] = (uint32_t)float_to_f16_bits(o[dt][rq * 4 + 2] * inv) |
+                               ((uint32_t)float_to_f16_bits(o[dt][rq * 4 + 3] * inv) << 16);
+                    } else {
+                        w[0] = (uint32_t)float_to_bf16_bits(o[dt][rq * 4] * inv) |
+                               ((uint32_t)float_to_bf16_bits(o[dt][rq * 4 + 1] * inv) << 16);
+                        w[1] = (uint32_t)float_to_bf16_bits(o[dt][rq * 4 + 2] * inv) |
+                               ((uint32_t)float_to_bf16_bits(o[dt][rq * 4 + 3] * inv) << 16);
+                    }
+                    *(uint2_t*)((uint16_t*)t.out + obase + d) = w;
+                }
+            }
+    }
+}
+
+template <bool kBf16>
+__global__ __launch_bounds__(kThreads) void sdpa_flash_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t k_lds[kTileK * kKRow];
+    __shared__ __attribute__((aligned(16))) uint8_t v_lds[kD * kVRow];
+    const int n_tiles = (p.len_q + kTileQ - 1) / kTileQ;
+    const int qt = n_tiles - 1 - (int)blockIdx.x;  // heaviest (latest) causal tiles first
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int G = p.num_heads_q / p.num_heads_kv;
+    Tile t;
+    const int64_t qoff = (((int64_t)b * p.num_heads_q + h) * p.len_q + (int64_t)qt * kTileQ) * kD;
+    t.q = (const uint16_t*)p.q + qoff;
+    t.q_stride = kD;
+    t.out = (uint16_t*)p.out + qoff;
+    t.out_stride = kD;
+    t.rows = min(kTileQ, p.len_q - qt * kTileQ);
+    t.pos0 = qt * kTileQ;
+    t.kv_len = p.len_kv;
+    t.causal = p.causal;
+    t.window = 0;
+    t.q_dtype = p.dtype;
+    t.out_dtype = p.dtype;
+    const int64_t kvoff = ((int64_t)b * p.num_heads_kv + h / G) * p.len_kv * (kD * 2);
+    t.k = (const uint8_t*)p.k + kvoff;
+    t.v = (const uint8_t*)p.v + kvoff;
+    t.table = nullptr;
+    t.table_len = 0;
+    t.num_blocks = 0;
+    t.block_stride = 0;
+    t.block_size = 1;
+    run_tile<kBf16>(t, k_lds, v_lds, p.scale);
+}
+
+// Exclusive prefix of query tiles per sequence (sequences with a single token have none:
+// they belong to the decode kernel).  One workgroup; sequences are split evenly over threads.
+__global__ __launch_bounds__(256) void paged_prefill_plan_kernel(PagedParams p) {
+    __shared__ int partial[256];
+    const int tid = threadIdx.x;
+    const int per = (p.num_seqs + 255) / 256;
+    const int s0 = min(tid * per, p.num_seqs), s1 = min(s0 + per, p.num_seqs);
+    int sum = 0;
+    for (int s = s0; s < s1; s++) {
+        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
+        sum += qlen > 1 ? (qlen + kTileQ - 1) / kTileQ : 0;
+    }
+    partial[tid] = sum;
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int i = 0; i < 256; i++) {
+            int v = partial[i];
+            partial[i] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+    int run = partial[tid];
+    for (int s = s0; s < s1; s++) {
+        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
+        p.tile_prefix[s] = run;
+        run += qlen > 1 ? (qlen + kTileQ - 1) / kTileQ : 0;
+    }
+    if (s1 == p.num_seqs && s0 < p.num_seqs) p.tile_prefix[p.num_seqs] = run;
+}
+
+template <bool kBf16>
+__global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t k_lds[kTileK * kKRow];
+    __shared__ __attribute__((aligned(16))) uint8_t v_lds[kD * kVRow];
+    const int total = p.tile_prefix[p.num_seqs];
+    const int tile_id = total - 1 - (int)blockIdx.x;
+    if (tile_id < 0) return;
+    // sequence owning this tile: largest s with tile_prefix[s] <= tile_id
+    int lo = 0, hi_s = p.num_seqs;
+    while (hi_s - lo > 1) {
+        const int mid = (lo + hi_s) >> 1;
+        if (p.tile_prefix[mid] <= tile_id)
+            lo = mid;
+        else
+            hi_s = mid;
+    }
+    const int s = lo;
+    const int qt = tile_id - p.tile_prefix[s];
+    const int h = blockIdx.y;
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const int t0 = p.subsequence_begins[s];
+    const int qlen = p.subsequence_begins[s + 1] - t0;
+    const int past = p.past_lens[s];
+    const int tb0 = p.block_indices_begins[s];
+    const int table_len = p.block_indices_begins[s + 1] - tb0;
+    Tile t;
+    const int64_t row0 = (int64_t)(t0 + qt * kTileQ) * p.num_heads_q + h;
+    t.q = (const uint16_t*)p.q + row0 * kD;
+    t.q_stride = (int64_t)p.num_heads_q * kD;
+    t.out = (p.out_dtype == HIPATTN_F32) ? (void*)((float*)p.out + row0 * kD) : (void*)((uint16_t*)p.out + row0 * kD);
+    t.out_stride = (int64_t)p.num_heads_q * kD;
+    t.rows = min(kTileQ, qlen - qt * kTileQ);
+    t.pos0 = past + qt * kTileQ;
+    t.kv_len = min(past + qlen, table_len * p.block_size);
+    t.causal = 1;
+    t.window = p.sliding_window;
+    t.q_dtype = p.q_dtype;
+    t.out_dtype = p.out_dtype;
+    const int64_t head_off = (int64_t)(h / G) * p.block_size * (kD * 2);
+    t.k = p.key_cache + head_off;
+    t.v = p.value_cache + head_off;
+    t.table = p.block_indices + tb0;
+    t.table_len = table_len;
+    t.num_blocks = p.num_blocks;
+    t.block_stride = (int64_t)p.num_heads_kv * p.block_size * (kD * 2);
+    t.block_size = p.block_size;
+    run_tile<kBf16>(t, k_lds, v_lds, p.scale);
+}
+
+}  // namespace flash
+
+bool sdpa_flash_supported(const SdpaParams& p) {
+    return p.head_dim == flash::kD && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16);
+}
+
+hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe) {
+    if (p.batch == 0 || p.len_q == 0) return hipSuccess;
+    const int n_tiles = (p.len_q + flash::kTileQ - 1) / flash::kTileQ;
+    dim3 grid(n_tiles, p.num_heads_q, p.batch);
+    if (probe.before) (void)hipEventRecord(probe.before, stream);
+    if (p.dtype == HIPATTN_BF16)
+        hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
+    else
+        hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
+    hipError_t e = hipGetLastError();
+    if (probe.after) (void)hipEventRecord(probe.after, stream);
+    return e;
+}
+
+hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
+    hipLaunchKernelGGL(flash::paged_prefill_plan_kernel, dim3(1), dim3(256), 0, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    dim3 grid(p.max_q_tiles, p.num_heads_q);
+    if (p.cache_dtype == HIPATTN_BF16)
+        hipLaunchKernelGGL(flash::paged_prefill_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
+    else
+        hipLaunchKernelGGL(flash::paged_prefill_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace hipattn

@@ -1,0 +1,418 @@
+// C ABI of libhipattn (include/hipattn.h): argument validation, kernel dispatch and a thin
+// layer over the HIP runtime.  Nothing here throws; failures come back as status codes with
+// a per-thread message.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "hipattn.h"
+#include "kernels.hpp"
+
+#define HIPATTN_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+thread_local char g_error[512] = "";
+thread_local const char* g_kernel_path = "none";
+thread_local hipattn::KernelProbe g_probe;
+
+hipattn_status fail(hipattn_status st, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return st;
+}
+
+hipattn_status hip_fail(hipError_t e, const char* what) {
+    return fail(HIPATTN_HIP_ERROR, "%s: %s (%s)", what, hipGetErrorString(e), hipGetErrorName(e));
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e_ = (expr);                         \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+inline hipStream_t as_stream(hipattn_stream s) { return reinterpret_cast<hipStream_t>(s); }
+inline hipEvent_t as_event(hipattn_event e) { return reinterpret_cast<hipEvent_t>(e); }
+
+bool is_float_dtype(int d) { return d == HIPATTN_F32 || d == HIPATTN_F16 || d == HIPATTN_BF16; }
+
+float resolve_scale(float scale, int head_dim) { return scale > 0.0f ? scale : 1.0f / std::sqrt((float)head_dim); }
+
+hipattn_status validate_sdpa(const hipattn_sdpa_desc* d) {
+    if (!d) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: null descriptor");
+    if (!is_float_dtype(d->dtype)) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: dtype %d is not f32/f16/bf16", d->dtype);
+    if (d->batch < 0 || d->len_q < 0 || d->len_kv < 0)
+        return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: negative extent (batch %d, len_q %d, len_kv %d)", d->batch,
+                    d->len_q, d->len_kv);
+    if (d->num_heads_q <= 0 || d->num_heads_kv <= 0 || d->num_heads_q % d->num_heads_kv)
+        return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: num_heads_q %d must be a positive multiple of num_heads_kv %d",
+                    d->num_heads_q, d->num_heads_kv);
+    if (d->head_dim <= 0) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: head_dim %d", d->head_dim);
+    if (d->head_dim > 512) return fail(HIPATTN_UNSUPPORTED, "sdpa: head_dim %d > 512", d->head_dim);
+    return HIPATTN_OK;
+}
+
+hipattn_status validate_pa(const hipattn_pa_desc* d, bool need_q) {
+    if (!d) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: null descriptor");
+    if (need_q && (!is_float_dtype(d->q_dtype) || !is_float_dtype(d->out_dtype)))
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: q/out dtype must be f32/f16/bf16");
+    if (!is_float_dtype(d->cache_dtype) && d->cache_dtype != HIPATTN_U8)
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: cache dtype %d", d->cache_dtype);
+    if (!(d->flags & HIPATTN_PA_SKIP_CACHE_WRITE) && !is_float_dtype(d->kv_dtype))
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: kv dtype %d", d->kv_dtype);
+    if (d->num_heads_q <= 0 || d->num_heads_kv <= 0 || d->num_heads_q % d->num_heads_kv)
+        return fail(HIPATTN_INVALID_ARGUMENT,
+                    "paged_attention: num_heads_q %d must be a positive multiple of num_heads_kv %d", d->num_heads_q,
+                    d->num_heads_kv);
+    if (d->head_dim <= 0 || d->block_size <= 0)
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: head_dim %d, block_size %d", d->head_dim,
+                    d->block_size);
+    if (d->head_dim > 512) return fail(HIPATTN_UNSUPPORTED, "paged_attention: head_dim %d > 512", d->head_dim);
+    if (d->num_blocks < 0 || d->num_tokens < 0 || d->num_seqs < 0 || d->max_context_len < 0)
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: negative extent");
+    if (d->cache_dtype == HIPATTN_U8 && d->head_dim % 8)
+        return fail(HIPATTN_UNSUPPORTED, "paged_attention: u8 cache needs head_dim %% 8 == 0 (row alignment)");
+    return HIPATTN_OK;
+}
+
+hipattn::KvWriteParams make_write_params(const hipattn_pa_desc* d, const void* k_new, const void* v_new,
+                                         void* key_cache, void* value_cache, const int32_t* past_lens,
+                                         const int32_t* subsequence_begins, const int32_t* block_indices,
+                                         const int32_t* block_indices_begins) {
+    hipattn::KvWriteParams w{};
+    w.k_new = k_new;
+    w.v_new = v_new;
+    w.key_cache = (uint8_t*)key_cache;
+    w.value_cache = (uint8_t*)value_cache;
+    w.past_lens = past_lens;
+    w.subsequence_begins = subsequence_begins;
+    w.block_indices = block_indices;
+    w.block_indices_begins = block_indices_begins;
+    w.kv_dtype = d->kv_dtype;
+    w.cache_dtype = d->cache_dtype;
+    w.num_tokens = d->num_tokens;
+    w.num_seqs = d->num_seqs;
+    w.num_heads_kv = d->num_heads_kv;
+    w.head_dim = d->head_dim;
+    w.block_size = d->block_size;
+    w.num_blocks = d->num_blocks;
+    return w;
+}
+
+hipattn::PagedParams make_paged_params(const hipattn_pa_desc* d) {
+    hipattn::PagedParams p{};
+    p.q_dtype = d->q_dtype;
+    p.cache_dtype = d->cache_dtype;
+    p.out_dtype = d->out_dtype;
+    p.num_heads_q = d->num_heads_q;
+    p.num_heads_kv = d->num_heads_kv;
+    p.head_dim = d->head_dim;
+    p.block_size = d->block_size;
+    p.num_blocks = d->num_blocks;
+    p.num_tokens = d->num_tokens;
+    p.num_seqs = d->num_seqs;
+    p.max_context_len = d->max_context_len;
+    p.sliding_window = d->sliding_window;
+    p.scale = resolve_scale(d->scale, d->head_dim);
+    p.chunk_tokens = d->decode_chunk;
+    return p;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------- misc
+HIPATTN_EXPORT const char* hipattn_last_error_string(void) { return g_error; }
+
+HIPATTN_EXPORT const char* hipattn_status_string(hipattn_status status) {
+    switch (status) {
+        case HIPATTN_OK: return "ok";
+        case HIPATTN_INVALID_ARGUMENT: return "invalid argument";
+        case HIPATTN_UNSUPPORTED: return "unsupported";
+        case HIPATTN_WORKSPACE_TOO_SMALL: return "workspace too small";
+        case HIPATTN_HIP_ERROR: return "HIP runtime error";
+        case HIPATTN_NO_DEVICE: return "no HIP device";
+    }
+    return "unknown status";
+}
+
+HIPATTN_EXPORT int hipattn_version(void) { return HIPATTN_VERSION_MAJOR * 1000 + HIPATTN_VERSION_MINOR; }
+
+HIPATTN_EXPORT const char* hipattn_last_kernel_path(void) { return g_kernel_path; }
+
+HIPATTN_EXPORT hipattn_status hipattn_profile_dominant_kernel(hipattn_event before, hipattn_event after) {
+    if ((before == nullptr) != (after == nullptr))
+        return fail(HIPATTN_INVALID_ARGUMENT, "profile_dominant_kernel: pass two events or two NULLs");
+    g_probe.before = reinterpret_cast<hipEvent_t>(before);
+    g_probe.after = reinterpret_cast<hipEvent_t>(after);
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT size_t hipattn_cache_row_bytes(hipattn_dtype cache_dtype, int head_dim) {
+    switch (cache_dtype) {
+        case HIPATTN_F32: return 4 * (size_t)head_dim;
+        case HIPATTN_F16:
+        case HIPATTN_BF16: return 2 * (size_t)head_dim;
+        case HIPATTN_U8: return (size_t)head_dim + 8;
+    }
+    return 0;
+}
+
+// ----------------------------------------------------------------------- device layer
+HIPATTN_EXPORT hipattn_status hipattn_device_count(int* count) {
+    if (!count) return fail(HIPATTN_INVALID_ARGUMENT, "device_count: null output");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *count = 0;
+        (void)hipGetLastError();
+        return fail(HIPATTN_NO_DEVICE, "hipGetDeviceCount: %s", hipGetErrorString(e));
+    }
+    *count = n;
+    return n > 0 ? HIPATTN_OK : fail(HIPATTN_NO_DEVICE, "no HIP device visible");
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_set_device(int device) {
+    HIP_TRY(hipSetDevice(device));
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_get_device_info(int device, hipattn_device_info* info) {
+    if (!info) return fail(HIPATTN_INVALID_ARGUMENT, "get_device_info: null output");
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    memset(info, 0, sizeof(*info));
+    snprintf(info->name, sizeof(info->name), "%s", prop.name);
+    // gcnArchName is "gfx950:sramecc+:xnack-"; keep the processor name only
+    snprintf(info->arch, sizeof(info->arch), "%s", prop.gcnArchName);
+    if (char* colon = strchr(info->arch, ':')) *colon = 0;
+    info->compute_units = prop.multiProcessorCount;
+    info->wavefront_size = prop.warpSize;
+    info->lds_bytes_per_workgroup = (int)prop.sharedMemPerBlock;
+    info->clock_mhz = prop.clockRate / 1000;
+    info->global_mem_bytes = prop.totalGlobalMem;
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_stream_create(hipattn_stream* stream) {
+    if (!stream) return fail(HIPATTN_INVALID_ARGUMENT, "stream_create: null output");
+    hipStream_t s;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = reinterpret_cast<hipattn_stream>(s);
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_stream_destroy(hipattn_stream stream) {
+    HIP_TRY(hipStreamDestroy(as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_stream_synchronize(hipattn_stream stream) {
+    HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_malloc(void** device_ptr, size_t bytes) {
+    if (!device_ptr) return fail(HIPATTN_INVALID_ARGUMENT, "malloc: null output");
+    *device_ptr = nullptr;
+    if (bytes == 0) return HIPATTN_OK;
+    HIP_TRY(hipMalloc(device_ptr, bytes));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_free(void* device_ptr) {
+    if (!device_ptr) return HIPATTN_OK;
+    HIP_TRY(hipFree(device_ptr));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_malloc_async(void** device_ptr, size_t bytes, hipattn_stream stream) {
+    if (!device_ptr) return fail(HIPATTN_INVALID_ARGUMENT, "malloc_async: null output");
+    *device_ptr = nullptr;
+    if (bytes == 0) return HIPATTN_OK;
+    HIP_TRY(hipMallocAsync(device_ptr, bytes, as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_free_async(void* device_ptr, hipattn_stream stream) {
+    if (!device_ptr) return HIPATTN_OK;
+    HIP_TRY(hipFreeAsync(device_ptr, as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_host_malloc(void** host_ptr, size_t bytes) {
+    if (!host_ptr) return fail(HIPATTN_INVALID_ARGUMENT, "host_malloc: null output");
+    *host_ptr = nullptr;
+    if (bytes == 0) return HIPATTN_OK;
+    HIP_TRY(hipHostMalloc(host_ptr, bytes, hipHostMallocDefault));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_host_free(void* host_ptr) {
+    if (!host_ptr) return HIPATTN_OK;
+    HIP_TRY(hipHostFree(host_ptr));
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_memcpy_h2d_async(void* device_dst, const void* host_src, size_t bytes,
+                                                       hipattn_stream stream) {
+    if (bytes == 0) return HIPATTN_OK;
+    if (!device_dst || !host_src) return fail(HIPATTN_INVALID_ARGUMENT, "memcpy_h2d: null pointer");
+    HIP_TRY(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_memcpy_d2h_async(void* host_dst, const void* device_src, size_t bytes,
+                                                       hipattn_stream stream) {
+    if (bytes == 0) return HIPATTN_OK;
+    if (!host_dst || !device_src) return fail(HIPATTN_INVALID_ARGUMENT, "memcpy_d2h: null pointer");
+    HIP_TRY(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_memcpy_d2d_async(void* device_dst, const void* device_src, size_t bytes,
+                                                       hipattn_stream stream) {
+    if (bytes == 0) return HIPATTN_OK;
+    if (!device_dst || !device_src) return fail(HIPATTN_INVALID_ARGUMENT, "memcpy_d2d: null pointer");
+    HIP_TRY(hipMemcpyAsync(device_dst, device_src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_fill_async(void* device_dst, int byte_value, size_t bytes,
+                                                 hipattn_stream stream) {
+    if (bytes == 0) return HIPATTN_OK;
+    if (!device_dst) return fail(HIPATTN_INVALID_ARGUMENT, "fill: null pointer");
+    HIP_TRY(hipattn::launch_fill_bytes(device_dst, byte_value, bytes, as_stream(stream)));
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_event_create(hipattn_event* event) {
+    if (!event) return fail(HIPATTN_INVALID_ARGUMENT, "event_create: null output");
+    hipEvent_t e;
+    HIP_TRY(hipEventCreate(&e));
+    *event = reinterpret_cast<hipattn_event>(e);
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_event_destroy(hipattn_event event) {
+    HIP_TRY(hipEventDestroy(as_event(event)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_event_record(hipattn_event event, hipattn_stream stream) {
+    HIP_TRY(hipEventRecord(as_event(event), as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_event_synchronize(hipattn_event event) {
+    HIP_TRY(hipEventSynchronize(as_event(event)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_event_elapsed_ms(hipattn_event start, hipattn_event stop, float* ms) {
+    if (!ms) return fail(HIPATTN_INVALID_ARGUMENT, "event_elapsed_ms: null output");
+    HIP_TRY(hipEventElapsedTime(ms, as_event(start), as_event(stop)));
+    return HIPATTN_OK;
+}
+
+// ------------------------------------------------------------------------------- SDPA
+HIPATTN_EXPORT hipattn_status hipattn_sdpa_workspace_size(const hipattn_sdpa_desc* desc, size_t* bytes) {
+    if (!bytes) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa_workspace_size: null output");
+    *bytes = 0;
+    return validate_sdpa(desc);
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const void* k, const void* v,
+                                           void* out, void* workspace, size_t workspace_bytes,
+                                           hipattn_stream stream) {
+    (void)workspace;
+    (void)workspace_bytes;
+    if (hipattn_status st = validate_sdpa(desc)) return st;
+    const int64_t out_elems = (int64_t)desc->batch * desc->num_heads_q * desc->len_q * desc->head_dim;
+    if (out_elems == 0) return HIPATTN_OK;
+    if (!q || !out) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: null q/out");
+    if (desc->len_kv > 0 && (!k || !v)) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: null k/v");
+    hipattn::SdpaParams p{};
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.out = out;
+    p.dtype = desc->dtype;
+    p.batch = desc->batch;
+    p.num_heads_q = desc->num_heads_q;
+    p.num_heads_kv = desc->num_heads_kv;
+    p.len_q = desc->len_q;
+    p.len_kv = desc->len_kv;
+    p.head_dim = desc->head_dim;
+    p.causal = desc->causal != 0;
+    p.scale = resolve_scale(desc->scale, desc->head_dim);
+    if (hipattn::sdpa_flash_supported(p)) {
+        g_kernel_path = "sdpa_flash_mfma";
+        HIP_TRY(hipattn::launch_sdpa_flash(p, as_stream(stream), g_probe));
+    } else {
+        g_kernel_path = "sdpa_generic";
+        HIP_TRY(hipattn::launch_sdpa_generic(p, as_stream(stream)));
+    }
+    return HIPATTN_OK;
+}
+
+// ------------------------------------------------------------------- paged attention
+HIPATTN_EXPORT hipattn_status hipattn_kv_cache_write(const hipattn_pa_desc* desc, const void* k_new, const void* v_new,
+                                                     void* key_cache, void* value_cache, const int32_t* past_lens,
+                                                     const int32_t* subsequence_begins, const int32_t* block_indices,
+                                                     const int32_t* block_indices_begins, hipattn_stream stream) {
+    if (hipattn_status st = validate_pa(desc, false)) return st;
+    if (!is_float_dtype(desc->kv_dtype)) return fail(HIPATTN_INVALID_ARGUMENT, "kv_cache_write: kv dtype %d", desc->kv_dtype);
+    if (desc->num_tokens == 0 || desc->num_seqs == 0) return HIPATTN_OK;
+    if (!k_new || !v_new || !key_cache || !value_cache || !past_lens || !subsequence_begins || !block_indices ||
+        !block_indices_begins)
+        return fail(HIPATTN_INVALID_ARGUMENT, "kv_cache_write: null pointer");
+    hipattn::KvWriteParams w = make_write_params(desc, k_new, v_new, key_cache, value_cache, past_lens,
+                                                 subsequence_begins, block_indices, block_indices_begins);
+    HIP_TRY(hipattn::launch_kv_cache_write(w, as_stream(stream)));
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_paged_attention_workspace_size(const hipattn_pa_desc* desc, size_t* bytes) {
+    if (!bytes) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_workspace_size: null output");
+    *bytes = 0;
+    if (hipattn_status st = validate_pa(desc, true)) return st;
+    hipattn::PagedParams p = make_paged_params(desc);
+    if (!(desc->flags & HIPATTN_PA_FORCE_GENERIC) && hipattn::paged_fast_supported(p))
+        *bytes = hipattn::paged_fast_workspace_bytes(p);
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* desc, const void* q, const void* k_new,
+                                                      const void* v_new, void* key_cache, void* value_cache,
+                                                      const int32_t* past_lens, const int32_t* subsequence_begins,
+                                                      const int32_t* block_indices,
+                                                      const int32_t* block_indices_begins, void* out, void* workspace,
+                                                      size_t workspace_bytes, hipattn_stream stream) {
+    if (hipattn_status st = validate_pa(desc, true)) return st;
+    if (desc->num_tokens == 0 || desc->num_seqs == 0) return HIPATTN_OK;
+    if (!q || !out || !key_cache || !value_cache || !past_lens || !subsequence_begins || !block_indices ||
+        !block_indices_begins)
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: null pointer");
+    if (!(desc->flags & HIPATTN_PA_SKIP_CACHE_WRITE)) {
+        if (!k_new || !v_new) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: null k_new/v_new");
+        hipattn::KvWriteParams w = make_write_params(desc, k_new, v_new, key_cache, value_cache, past_lens,
+                                                     subsequence_begins, block_indices, block_indices_begins);
+        HIP_TRY(hipattn::launch_kv_cache_write(w, as_stream(stream)));
+    }
+    hipattn::PagedParams p = make_paged_params(desc);
+    p.q = q;
+    p.key_cache = (const uint8_t*)key_cache;
+    p.value_cache = (const uint8_t*)value_cache;
+    p.past_lens = past_lens;
+    p.subsequence_begins = subsequence_begins;
+    p.block_indices = block_indices;
+    p.block_indices_begins = block_indices_begins;
+    p.out = out;
+    if (!(desc->flags & HIPATTN_PA_FORCE_GENERIC) && hipattn::paged_fast_supported(p)) {
+        const size_t need = hipattn::paged_fast_workspace_bytes(p);
+        if (need > 0 && (!workspace || workspace_bytes < need))
+            return fail(HIPATTN_WORKSPACE_TOO_SMALL, "paged_attention: workspace %zu bytes, need %zu", workspace_bytes,
+                        need);
+        if ((uintptr_t)workspace % 16)
+            return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: workspace must be 16-byte aligned");
+        hipattn::paged_fast_plan(p, workspace);
+        g_kernel_path = "paged_mfma";
+        HIP_TRY(hipattn::launch_paged_fast(p, as_stream(stream), g_probe));
+    } else {
+        g_kernel_path = "paged_generic";
+        HIP_TRY(hipattn::launch_paged_generic(p, as_stream(stream)));
+    }
+    return HIPATTN_OK;
+}

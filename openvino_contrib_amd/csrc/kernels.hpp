@@ -1,0 +1,107 @@
+// Parameter blocks and host-side launchers of the attention kernels (internal to the
+// library; the public boundary is include/hipattn.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hipattn.h"
+
+namespace hipattn {
+
+struct KvWriteParams {
+    const void* k_new;
+    const void* v_new;
+    uint8_t* key_cache;
+    uint8_t* value_cache;
+    const int32_t* past_lens;
+    const int32_t* subsequence_begins;
+    const int32_t* block_indices;
+    const int32_t* block_indices_begins;
+    int kv_dtype;
+    int cache_dtype;
+    int num_tokens;
+    int num_seqs;
+    int num_heads_kv;
+    int head_dim;
+    int block_size;
+    int num_blocks;
+};
+
+struct SdpaParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* out;
+    int dtype;
+    int batch;
+    int num_heads_q;
+    int num_heads_kv;
+    int len_q;
+    int len_kv;
+    int head_dim;
+    int causal;
+    float scale;  // already resolved (> 0)
+};
+
+struct PagedParams {
+    const void* q;
+    const uint8_t* key_cache;
+    const uint8_t* value_cache;
+    const int32_t* past_lens;
+    const int32_t* subsequence_begins;
+    const int32_t* block_indices;
+    const int32_t* block_indices_begins;
+    void* out;
+    int q_dtype;
+    int cache_dtype;
+    int out_dtype;
+    int num_heads_q;
+    int num_heads_kv;
+    int head_dim;
+    int block_size;
+    int num_blocks;
+    int num_tokens;
+    int num_seqs;
+    int max_context_len;
+    int sliding_window;
+    float scale;  // already resolved (> 0)
+    // split-context decode: partial results live in the caller's workspace
+    int chunk_tokens;     // tokens per split (multiple of block_size)
+    int max_chunks;       // ceil(max attended tokens / chunk_tokens)
+    float* part_out;      // [num_seqs, num_heads_q, max_chunks, head_dim]
+    float* part_ml;       // [num_seqs, num_heads_q, max_chunks, 2] running max (log2 domain) and sum
+    // chunked prefill: query-tile schedule built on the device
+    int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
+    int max_q_tiles;      // grid upper bound
+    // shape-generic kernel only: skip sequences with exactly one token (the decode kernel has them)
+    int generic_skip_single;
+};
+
+// Optional event pair recorded around the dominant kernel of a call (measurement aid).
+struct KernelProbe {
+    hipEvent_t before = nullptr;
+    hipEvent_t after = nullptr;
+};
+
+hipError_t launch_kv_cache_write(const KvWriteParams& p, hipStream_t stream);
+
+// shape-generic fp32 VALU kernels: any head_dim <= 512, any block size, every dtype
+hipError_t launch_sdpa_generic(const SdpaParams& p, hipStream_t stream);
+hipError_t launch_paged_generic(const PagedParams& p, hipStream_t stream);
+
+// MFMA flash kernels (head_dim 64 or 128, f16 / bf16)
+bool sdpa_flash_supported(const SdpaParams& p);
+hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
+
+// paged attention fast paths: split-context decode (+ merge) and chunked prefill
+bool paged_fast_supported(const PagedParams& p);
+size_t paged_fast_workspace_bytes(const PagedParams& p);
+void paged_fast_plan(PagedParams& p, void* workspace);  // fills chunking fields and workspace pointers
+hipError_t launch_paged_fast(const PagedParams& p, hipStream_t stream, const KernelProbe& probe);
+hipError_t launch_paged_decode(const PagedParams& p, hipStream_t stream, const KernelProbe& probe);  // + merge
+hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream);  // plan + flash over the block table
+
+hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t stream);
+
+}  // namespace hipattn

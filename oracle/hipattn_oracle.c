@@ -1,0 +1,415 @@
+/*
+ * CPU oracle for the attention hot path.  TEST INFRASTRUCTURE ONLY: this file is the
+ * checker that tests, the smoke check and the benchmark's cpu_baseline leg compare the
+ * HIP kernels against.  Nothing in the shipped library links or calls it.
+ *
+ * The reference plugin holds no attention kernel of its own: it rewrites
+ * v13::ScaledDotProductAttention into Multiply / MatMul / Select / Add / Softmax / MatMul
+ * (modules/nvidia_plugin/src/transformer/cuda_graph_transformer.cpp:151-156) and runs
+ * those on cuBLAS and cuDNN (src/ops/matmul.cpp:204-226, src/ops/softmax.cpp:184-192).
+ * The arithmetic itself lives in OpenVINO 2025.3.0 (wheel/requirements.txt:4), which is
+ * not part of the reference tree, so this file restates the published operator
+ * definitions:
+ *
+ *   oracle_sdpa_f32            softmax(scale * Q K^T + causal mask) V, fp32, GQA by head
+ *                              group, top-left aligned lower-triangular mask
+ *                              (model built as in tests/functional/shared_tests_instances/
+ *                              single_layer_tests/scaled_dot_product_attention.cpp:48-69;
+ *                              batch broadcast rules as src/ops/matmul.cpp:128-175;
+ *                              max-subtracted softmax as src/ops/softmax.cpp:75-147).
+ *                              Pinned by: fp64 brute force, torch's CPU
+ *                              scaled_dot_product_attention fixtures, invariants.
+ *   oracle_kv_cache_write      slot(s, p) = block_indices[begins[s] + p / bs] * bs + p % bs,
+ *                              row scatter in the spirit of
+ *                              src/kernels/scatter_nd_update.cu:19-34; out-of-range block
+ *                              ids are skipped, never written
+ *                              (tests/unit/kernels/scatter_update.cpp:59-86).
+ *                              Pinned by: brute force in numpy, write-then-gather identity,
+ *                              canary fill.
+ *   oracle_paged_attention     PagedAttentionExtension: cache write, then every query token
+ *                              attends cache positions (p - W, p] of its own sequence.
+ *                              PARITY UNPINNED against OpenVINO: the op does not occur in
+ *                              the reference tree and OpenVINO is not installed.  Pinned
+ *                              by reduction to oracle_sdpa_f32 after a gather through the
+ *                              block table, and by block-permutation invariance.
+ *   oracle_quant_u8_row /      asymmetric per-token, per-head u8 rows
+ *   oracle_dequant_u8_row      [scale f32][zero-point f32][D bytes].  PARITY UNPINNED
+ *                              against OpenVINO (rounding mode and row layout are restated
+ *                              from the published CPU plugin behaviour, not checked).
+ *                              Pinned by |x - x^| <= scale/2 and min/max round trip.
+ *
+ * All arithmetic is fp32 with fp64 softmax sums.  Compiled with OpenMP; the number of
+ * threads is whatever omp_get_max_threads() says (reported by oracle_num_threads()).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <float.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_BF16 = 2, ORACLE_U8 = 3 };
+
+ORACLE_API int oracle_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+ORACLE_API void oracle_set_num_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
+
+/* ---------------------------------------------------------------- scalar conversions */
+
+static inline uint32_t f32_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static inline float bits_f32(uint32_t u) {
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* IEEE binary16 -> binary32, exact. */
+ORACLE_API float oracle_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    if (exp == 0) {
+        if (man == 0) return bits_f32(sign);
+        /* subnormal: value = man * 2^-24 */
+        float v = (float)man * 5.9604644775390625e-8f;
+        return sign ? -v : v;
+    }
+    if (exp == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
+    return bits_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+/* binary32 -> binary16, round to nearest even, subnormals kept, overflow to inf. */
+ORACLE_API uint16_t oracle_f32_to_f16(float f) {
+    uint32_t x = f32_bits(f);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t ax = x & 0x7fffffffu;
+    if (ax >= 0x7f800000u) { /* inf / nan */
+        if (ax > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((ax >> 13) & 0x3ffu));
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (ax >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* >= 65520 rounds to inf */
+    if (ax < 0x33000001u) return sign;                        /* <= 2^-25 rounds to zero */
+    int32_t e = (int32_t)(ax >> 23) - 127;
+    uint32_t m = (ax & 0x7fffffu) | 0x800000u;
+    if (e < -14) {
+        /* subnormal half: shift so that the unit is 2^-24 */
+        int shift = -14 - e + 13; /* 14..24 */
+        uint32_t q = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (q & 1u))) q++;
+        return (uint16_t)(sign | q);
+    }
+    uint32_t q = ((uint32_t)(e + 15) << 10) | ((m >> 13) & 0x3ffu);
+    uint32_t rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+}
+
+ORACLE_API float oracle_bf16_to_f32(uint16_t b) { return bits_f32((uint32_t)b << 16); }
+
+/* binary32 -> bfloat16, round to nearest even. */
+ORACLE_API uint16_t oracle_f32_to_bf16(float f) {
+    uint32_t x = f32_bits(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+    uint32_t lsb = (x >> 16) & 1u;
+    x += 0x7fffu + lsb;
+    return (uint16_t)(x >> 16);
+}
+
+ORACLE_API void oracle_f32_to_f16_array(const float* src, uint16_t* dst, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) dst[i] = oracle_f32_to_f16(src[i]);
+}
+ORACLE_API void oracle_f16_to_f32_array(const uint16_t* src, float* dst, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) dst[i] = oracle_f16_to_f32(src[i]);
+}
+ORACLE_API void oracle_f32_to_bf16_array(const float* src, uint16_t* dst, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) dst[i] = oracle_f32_to_bf16(src[i]);
+}
+ORACLE_API void oracle_bf16_to_f32_array(const uint16_t* src, float* dst, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) dst[i] = oracle_bf16_to_f32(src[i]);
+}
+
+/* ------------------------------------------------------------------- u8 quantisation */
+
+/*
+ * One cache row of a u8 cache: [scale f32][zp f32][D x u8].
+ *   scale = (max - min) / 255   (0 -> 1e-4 so that a constant row survives)
+ *   zp    = -min / scale + 0   (the sum turns -0 into +0)
+ *   q     = clamp(rint(fma(x, 1/scale, zp)), 0, 255)     (round half to even)
+ *   x^    = (q - zp) * scale
+ */
+ORACLE_API void oracle_quant_u8_row(const float* x, int D, uint8_t* row) {
+    float mn = FLT_MAX, mx = -FLT_MAX;
+    for (int d = 0; d < D; d++) {
+        mn = x[d] < mn ? x[d] : mn;
+        mx = x[d] > mx ? x[d] : mx;
+    }
+    float scale = (mx - mn) / 255.0f;
+    if (scale == 0.0f) scale = 0.0001f;
+    float zp = -mn / scale + 0.0f;
+    float inv = 1.0f / scale;
+    memcpy(row, &scale, 4);
+    memcpy(row + 4, &zp, 4);
+    for (int d = 0; d < D; d++) {
+        float t = rintf(fmaf(x[d], inv, zp));
+        t = t < 0.0f ? 0.0f : (t > 255.0f ? 255.0f : t);
+        row[8 + d] = (uint8_t)t;
+    }
+}
+
+ORACLE_API void oracle_dequant_u8_row(const uint8_t* row, int D, float* x) {
+    float scale, zp;
+    memcpy(&scale, row, 4);
+    memcpy(&zp, row + 4, 4);
+    for (int d = 0; d < D; d++) x[d] = ((float)row[8 + d] - zp) * scale;
+}
+
+ORACLE_API void oracle_quant_u8_rows(const float* x, int64_t n, int D, uint8_t* rows) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) oracle_quant_u8_row(x + i * D, D, rows + i * (D + 8));
+}
+
+ORACLE_API void oracle_dequant_u8_rows(const uint8_t* rows, int64_t n, int D, float* x) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) oracle_dequant_u8_row(rows + i * (D + 8), D, x + i * D);
+}
+
+static inline int64_t cache_row_bytes(int dtype, int D) {
+    switch (dtype) {
+        case ORACLE_F32: return 4 * (int64_t)D;
+        case ORACLE_F16:
+        case ORACLE_BF16: return 2 * (int64_t)D;
+        default: return (int64_t)D + 8;
+    }
+}
+
+static void cache_row_store(int dtype, const float* x, int D, uint8_t* row) {
+    switch (dtype) {
+        case ORACLE_F32: memcpy(row, x, 4 * (size_t)D); break;
+        case ORACLE_F16:
+            for (int d = 0; d < D; d++) ((uint16_t*)row)[d] = oracle_f32_to_f16(x[d]);
+            break;
+        case ORACLE_BF16:
+            for (int d = 0; d < D; d++) ((uint16_t*)row)[d] = oracle_f32_to_bf16(x[d]);
+            break;
+        default: oracle_quant_u8_row(x, D, row);
+    }
+}
+
+static void cache_row_load(int dtype, const uint8_t* row, int D, float* x) {
+    switch (dtype) {
+        case ORACLE_F32: memcpy(x, row, 4 * (size_t)D); break;
+        case ORACLE_F16:
+            for (int d = 0; d < D; d++) x[d] = oracle_f16_to_f32(((const uint16_t*)row)[d]);
+            break;
+        case ORACLE_BF16:
+            for (int d = 0; d < D; d++) x[d] = oracle_bf16_to_f32(((const uint16_t*)row)[d]);
+            break;
+        default: oracle_dequant_u8_row(row, D, x);
+    }
+}
+
+/* ------------------------------------------------------------------------ dense SDPA */
+
+static inline float dotf(const float* a, const float* b, int n) {
+    float s = 0.0f;
+#pragma omp simd reduction(+ : s)
+    for (int i = 0; i < n; i++) s += a[i] * b[i];
+    return s;
+}
+
+/*
+ * One query row against keys [j0, j1) given as row pointers computed by the caller's
+ * stride; scores buffer must hold j1 - j0 floats.
+ */
+static void attend_row(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0, int j1,
+                       int D, float scale, float* scores, float* out) {
+    int n = j1 - j0;
+    if (n <= 0) {
+        for (int d = 0; d < D; d++) out[d] = 0.0f;
+        return;
+    }
+    float m = -INFINITY;
+    for (int j = 0; j < n; j++) {
+        float s = scale * dotf(q, kbase + (int64_t)(j0 + j) * kv_stride, D);
+        scores[j] = s;
+        m = s > m ? s : m;
+    }
+    double l = 0.0;
+    for (int j = 0; j < n; j++) {
+        float p = expf(scores[j] - m);
+        scores[j] = p;
+        l += (double)p;
+    }
+    for (int d = 0; d < D; d++) out[d] = 0.0f;
+    for (int j = 0; j < n; j++) {
+        const float* v = vbase + (int64_t)(j0 + j) * kv_stride;
+        float p = scores[j];
+        for (int d = 0; d < D; d++) out[d] += p * v[d];
+    }
+    float inv = (float)(1.0 / l);
+    for (int d = 0; d < D; d++) out[d] *= inv;
+}
+
+/*
+ * q [B,Hq,Lq,D], k,v [B,Hkv,Lk,D], out [B,Hq,Lq,D]; query head h reads kv head
+ * h / (Hq/Hkv).  causal: row i sees keys j <= i (top-left aligned, as the operator
+ * specification's tril(ones(Lq,Lk))).  scale <= 0 selects 1/sqrt(D).
+ */
+ORACLE_API int oracle_sdpa_f32(const float* q, const float* k, const float* v, float* out, int B, int Hq, int Hkv,
+                               int Lq, int Lk, int D, int causal, float scale) {
+    if (B < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Lq < 0 || Lk < 0 || D <= 0) return 1;
+    if (scale <= 0.0f) scale = 1.0f / sqrtf((float)D);
+    int G = Hq / Hkv;
+    int64_t rows = (int64_t)B * Hq * Lq;
+#pragma omp parallel
+    {
+        float* scores = (float*)malloc(sizeof(float) * (size_t)(Lk > 0 ? Lk : 1));
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t r = 0; r < rows; r++) {
+            int i = (int)(r % Lq);
+            int h = (int)((r / Lq) % Hq);
+            int b = (int)(r / ((int64_t)Lq * Hq));
+            const float* kb = k + ((int64_t)b * Hkv + h / G) * Lk * D;
+            const float* vb = v + ((int64_t)b * Hkv + h / G) * Lk * D;
+            int j1 = causal ? (i + 1 < Lk ? i + 1 : Lk) : Lk;
+            attend_row(q + r * D, kb, vb, D, 0, j1, D, scale, scores, out + r * D);
+        }
+        free(scores);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------ paged KV cache */
+
+/*
+ * Scatter the new key/value rows of a batch into the paged caches.
+ *   k_new, v_new        [T, Hkv*D] fp32 (already rounded to the activation type by the caller)
+ *   key_cache/value_cache  [num_blocks, Hkv, block_size, row_bytes(dtype, D)]
+ *   past_lens [S], subsequence_begins [S+1], block_indices [..], block_indices_begins [S+1]
+ * Token i of sequence s goes to logical position p = past_lens[s] + i, i.e. physical
+ * block block_indices[block_indices_begins[s] + p / block_size], row p % block_size.
+ * A logical block beyond the sequence's table, or a physical id outside [0, num_blocks),
+ * is skipped.  Returns the number of skipped token rows.
+ */
+ORACLE_API int64_t oracle_kv_cache_write(const float* k_new, const float* v_new, uint8_t* key_cache,
+                                         uint8_t* value_cache, int cache_dtype, const int32_t* past_lens,
+                                         const int32_t* subsequence_begins, const int32_t* block_indices,
+                                         const int32_t* block_indices_begins, int S, int Hkv, int D, int block_size,
+                                         int num_blocks) {
+    int64_t rb = cache_row_bytes(cache_dtype, D);
+    int64_t skipped = 0;
+    for (int s = 0; s < S; s++) {
+        int t0 = subsequence_begins[s], t1 = subsequence_begins[s + 1];
+        int nb = block_indices_begins[s + 1] - block_indices_begins[s];
+        for (int t = t0; t < t1; t++) {
+            int p = past_lens[s] + (t - t0);
+            int lb = p / block_size;
+            if (p < 0 || lb >= nb) {
+                skipped++;
+                continue;
+            }
+            int pb = block_indices[block_indices_begins[s] + lb];
+            if (pb < 0 || pb >= num_blocks) {
+                skipped++;
+                continue;
+            }
+            for (int h = 0; h < Hkv; h++) {
+                int64_t off = (((int64_t)pb * Hkv + h) * block_size + p % block_size) * rb;
+                cache_row_store(cache_dtype, k_new + ((int64_t)t * Hkv + h) * D, D, key_cache + off);
+                cache_row_store(cache_dtype, v_new + ((int64_t)t * Hkv + h) * D, D, value_cache + off);
+            }
+        }
+    }
+    return skipped;
+}
+
+/*
+ * Gather one sequence's first n cache rows of kv head h through its block table into a
+ * contiguous fp32 [n, D] array (used by the oracle itself and by tests that reduce the
+ * paged case to the dense one).
+ */
+ORACLE_API void oracle_gather_cache_rows(const uint8_t* cache, int cache_dtype, const int32_t* seq_blocks, int n,
+                                         int h, int Hkv, int D, int block_size, float* dst) {
+    int64_t rb = cache_row_bytes(cache_dtype, D);
+    for (int p = 0; p < n; p++) {
+        int pb = seq_blocks[p / block_size];
+        int64_t off = (((int64_t)pb * Hkv + h) * block_size + p % block_size) * rb;
+        cache_row_load(cache_dtype, cache + off, D, dst + (int64_t)p * D);
+    }
+}
+
+/*
+ * PagedAttentionExtension, restated.
+ *   q [T, Hq*D] fp32, out [T, Hq*D] fp32.
+ *   do_write != 0: first scatter k_new / v_new (oracle_kv_cache_write).
+ * Query token i of sequence s sits at position p = past_lens[s] + i and attends cache
+ * positions j with max(0, p - W + 1) <= j <= p when W = sliding_window > 0, else 0..p.
+ * scale <= 0 selects 1/sqrt(D).
+ */
+ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const float* v_new, uint8_t* key_cache,
+                                      uint8_t* value_cache, int cache_dtype, const int32_t* past_lens,
+                                      const int32_t* subsequence_begins, const int32_t* block_indices,
+                                      const int32_t* block_indices_begins, int S, int Hq, int Hkv, int D,
+                                      int block_size, int num_blocks, float scale, int sliding_window, int do_write,
+                                      float* out) {
+    if (S < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || block_size <= 0) return 1;
+    if (scale <= 0.0f) scale = 1.0f / sqrtf((float)D);
+    if (do_write)
+        oracle_kv_cache_write(k_new, v_new, key_cache, value_cache, cache_dtype, past_lens, subsequence_begins,
+                              block_indices, block_indices_begins, S, Hkv, D, block_size, num_blocks);
+    int G = Hq / Hkv;
+    /* work items: (sequence, kv head); gathered K/V are shared by the G query heads */
+    int64_t items = (int64_t)S * Hkv;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int64_t it = 0; it < items; it++) {
+        int s = (int)(it / Hkv), h = (int)(it % Hkv);
+        int t0 = subsequence_begins[s], qlen = subsequence_begins[s + 1] - t0;
+        if (qlen <= 0) continue;
+        int ctx = past_lens[s] + qlen;
+        float* kbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
+        float* vbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
+        float* scores = (float*)malloc(sizeof(float) * (size_t)ctx);
+        const int32_t* blocks = block_indices + block_indices_begins[s];
+        oracle_gather_cache_rows(key_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, kbuf);
+        oracle_gather_cache_rows(value_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, vbuf);
+        for (int i = 0; i < qlen; i++) {
+            int p = past_lens[s] + i;
+            int j0 = 0;
+            if (sliding_window > 0 && p - sliding_window + 1 > 0) j0 = p - sliding_window + 1;
+            for (int g = 0; g < G; g++) {
+                int64_t row = ((int64_t)(t0 + i) * Hq + (h * G + g)) * D;
+                attend_row(q + row, kbuf, vbuf, D, j0, p + 1, D, scale, scores, out + row);
+            }
+        }
+        free(kbuf);
+        free(vbuf);
+        free(scores);
+    }
+    return 0;
+}

@@ -1,0 +1,196 @@
+"""ctypes loader for the CPU oracle (oracle/hipattn_oracle.c).
+
+Test infrastructure only: imported by tests/, the smoke check and the benchmark's
+cpu_baseline leg.  The product package never imports this module.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libhipattn_oracle.so")
+
+F32, F16, BF16, U8 = 0, 1, 2, 3
+
+_lib = None
+
+
+def build(force=False):
+    """Compile the oracle with the Makefile beside it."""
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        vp, i32, i64, f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+        L.oracle_num_threads.restype = i32
+        L.oracle_set_num_threads.argtypes = [i32]
+        L.oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.oracle_f16_to_f32.restype = f32
+        L.oracle_f32_to_f16.argtypes = [f32]
+        L.oracle_f32_to_f16.restype = ctypes.c_uint16
+        L.oracle_f32_to_bf16.argtypes = [f32]
+        L.oracle_f32_to_bf16.restype = ctypes.c_uint16
+        for n in ("oracle_f32_to_f16_array", "oracle_f16_to_f32_array", "oracle_f32_to_bf16_array",
+                  "oracle_bf16_to_f32_array"):
+            getattr(L, n).argtypes = [vp, vp, i64]
+            getattr(L, n).restype = None
+        L.oracle_quant_u8_row.argtypes = [vp, i32, vp]
+        L.oracle_quant_u8_row.restype = None
+        L.oracle_dequant_u8_row.argtypes = [vp, i32, vp]
+        L.oracle_dequant_u8_row.restype = None
+        L.oracle_quant_u8_rows.argtypes = [vp, i64, i32, vp]
+        L.oracle_quant_u8_rows.restype = None
+        L.oracle_dequant_u8_rows.argtypes = [vp, i64, i32, vp]
+        L.oracle_dequant_u8_rows.restype = None
+        L.oracle_sdpa_f32.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, f32]
+        L.oracle_sdpa_f32.restype = i32
+        L.oracle_kv_cache_write.argtypes = [vp, vp, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32]
+        L.oracle_kv_cache_write.restype = i64
+        L.oracle_gather_cache_rows.argtypes = [vp, i32, vp, i32, i32, i32, i32, i32, vp]
+        L.oracle_gather_cache_rows.restype = None
+        L.oracle_paged_attention.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
+                                             f32, i32, i32, vp]
+        L.oracle_paged_attention.restype = i32
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dt):
+    a = np.ascontiguousarray(a, dtype=dt)
+    return a
+
+
+def num_threads():
+    return lib().oracle_num_threads()
+
+
+def set_num_threads(n):
+    lib().oracle_set_num_threads(int(n))
+
+
+# ----------------------------------------------------------------------------- conversions
+def f32_to_f16_bits(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().oracle_f32_to_f16_array(_p(x), _p(out), x.size)
+    return out
+
+
+def f16_bits_to_f32(h):
+    h = _c(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().oracle_f16_to_f32_array(_p(h), _p(out), h.size)
+    return out
+
+
+def f32_to_bf16_bits(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().oracle_f32_to_bf16_array(_p(x), _p(out), x.size)
+    return out
+
+
+def bf16_bits_to_f32(b):
+    b = _c(b, np.uint16)
+    out = np.empty(b.shape, np.float32)
+    lib().oracle_bf16_to_f32_array(_p(b), _p(out), b.size)
+    return out
+
+
+def round_to(x, dtype):
+    """fp32 array rounded to the storage type and expanded back to fp32."""
+    if dtype == F32:
+        return _c(x, np.float32).copy()
+    if dtype == F16:
+        return f16_bits_to_f32(f32_to_f16_bits(x))
+    if dtype == BF16:
+        return bf16_bits_to_f32(f32_to_bf16_bits(x))
+    raise ValueError(dtype)
+
+
+def cache_row_bytes(dtype, D):
+    return {F32: 4 * D, F16: 2 * D, BF16: 2 * D, U8: D + 8}[dtype]
+
+
+def quant_u8_rows(x):
+    """x [..., D] fp32 -> uint8 [..., D + 8] rows of [scale][zp][D bytes]."""
+    x = _c(x, np.float32)
+    D = x.shape[-1]
+    flat = x.reshape(-1, D)
+    out = np.empty((flat.shape[0], D + 8), np.uint8)
+    lib().oracle_quant_u8_rows(_p(flat), flat.shape[0], D, _p(out))
+    return out.reshape(x.shape[:-1] + (D + 8,))
+
+
+def dequant_u8_rows(rows):
+    rows = _c(rows, np.uint8)
+    D = rows.shape[-1] - 8
+    flat = rows.reshape(-1, D + 8)
+    out = np.empty((flat.shape[0], D), np.float32)
+    lib().oracle_dequant_u8_rows(_p(flat), flat.shape[0], D, _p(out))
+    return out.reshape(rows.shape[:-1] + (D,))
+
+
+# ------------------------------------------------------------------------------ operators
+def sdpa(q, k, v, causal=False, scale=0.0):
+    """q [B,Hq,Lq,D], k/v [B,Hkv,Lk,D] fp32 -> out [B,Hq,Lq,D] fp32."""
+    q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
+    B, Hq, Lq, D = q.shape
+    _, Hkv, Lk, _ = k.shape
+    out = np.empty_like(q)
+    rc = lib().oracle_sdpa_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, Lq, Lk, D, int(bool(causal)), float(scale))
+    if rc:
+        raise ValueError("oracle_sdpa_f32: bad arguments")
+    return out
+
+
+def kv_cache_write(k_new, v_new, key_cache, value_cache, cache_dtype, past_lens, subsequence_begins, block_indices,
+                   block_indices_begins, Hkv, D, block_size):
+    """In-place scatter into uint8-viewed caches [num_blocks, Hkv, block_size, row_bytes]."""
+    k_new, v_new = _c(k_new, np.float32), _c(v_new, np.float32)
+    pl, sb = _c(past_lens, np.int32), _c(subsequence_begins, np.int32)
+    bi, bb = _c(block_indices, np.int32), _c(block_indices_begins, np.int32)
+    assert key_cache.dtype == np.uint8 and value_cache.dtype == np.uint8
+    assert key_cache.flags.c_contiguous and value_cache.flags.c_contiguous
+    num_blocks = key_cache.shape[0]
+    return lib().oracle_kv_cache_write(_p(k_new), _p(v_new), _p(key_cache), _p(value_cache), cache_dtype, _p(pl),
+                                       _p(sb), _p(bi), _p(bb), len(pl), Hkv, D, block_size, num_blocks)
+
+
+def gather_cache_rows(cache, cache_dtype, seq_blocks, n, h, Hkv, D, block_size):
+    seq_blocks = _c(seq_blocks, np.int32)
+    out = np.empty((n, D), np.float32)
+    lib().oracle_gather_cache_rows(_p(cache), cache_dtype, _p(seq_blocks), n, h, Hkv, D, block_size, _p(out))
+    return out
+
+
+def paged_attention(q, k_new, v_new, key_cache, value_cache, cache_dtype, past_lens, subsequence_begins,
+                    block_indices, block_indices_begins, Hq, Hkv, D, block_size, scale=0.0, sliding_window=0,
+                    do_write=True):
+    """q [T, Hq*D] fp32; caches are uint8 views, updated in place when do_write. Returns out [T, Hq*D]."""
+    q = _c(q, np.float32)
+    k_new, v_new = _c(k_new, np.float32), _c(v_new, np.float32)
+    pl, sb = _c(past_lens, np.int32), _c(subsequence_begins, np.int32)
+    bi, bb = _c(block_indices, np.int32), _c(block_indices_begins, np.int32)
+    assert key_cache.dtype == np.uint8 and value_cache.dtype == np.uint8
+    out = np.zeros_like(q)
+    rc = lib().oracle_paged_attention(_p(q), _p(k_new), _p(v_new), _p(key_cache), _p(value_cache), cache_dtype,
+                                      _p(pl), _p(sb), _p(bi), _p(bb), len(pl), Hq, Hkv, D, block_size,
+                                      key_cache.shape[0], float(scale), int(sliding_window), int(bool(do_write)),
+                                      _p(out))
+    if rc:
+        raise ValueError("oracle_paged_attention: bad arguments")
+    return out

@@ -1,0 +1,283 @@
+"""GPU parity tests: every call goes through the C ABI (libhipattn.so) and is compared with the
+CPU oracle on the same seeded inputs.
+
+Bars: cache bytes after the writer / the op's step 1 are bit-exact; attention outputs are
+within max-abs 2e-3 (fp16), 1e-2 (bf16 or u8 cache), 1e-4 for the fp32 kernel, against the
+oracle's fp32 result computed from the same stored (rounded / quantised) inputs.
+"""
+import numpy as np
+import pytest
+
+import helpers as H
+from openvino_contrib_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+TOL = {W.F32: 1e-4, W.F16: 2e-3, W.BF16: 1e-2}
+
+
+def announce(*args):
+    print("[case]", *args, flush=True)
+
+
+# ------------------------------------------------------------------------------ KV writer
+@pytest.mark.parametrize("kv_dtype,cache_dtype", [(W.F16, W.F16), (W.BF16, W.F16), (W.F32, W.F16), (W.F16, W.U8),
+                                                  (W.BF16, W.U8), (W.F32, W.U8), (W.BF16, W.BF16), (W.F32, W.F32),
+                                                  (W.F16, W.F32)])
+def test_kv_cache_write_bit_exact(hip, oracle, kv_dtype, cache_dtype):
+    announce("kv_write", kv_dtype, cache_dtype)
+    seqs = [(0, 70), (31, 1), (32, 1), (100, 33), (5, 0), (63, 2), (1000, 1)]
+    case = W.make_paged_case(51, seqs, 8, 4, 128, 32, W.F16, kv_dtype, cache_dtype)
+    # exercise tiny, huge and fp16-subnormal magnitudes in the new rows
+    scale = np.ones(case["T"], np.float32)
+    scale[::5] = 1e-6
+    scale[1::7] = 1e4
+    for name in ("k_new", "v_new"):
+        st, val = W.to_storage(case[name] * scale[:, None], kv_dtype)
+        case[name], case[name + "_store"] = val, st
+    case["k_new"][3, :128] = 0.75  # constant row: zero range in the quantiser
+    case["k_new_store"], case["k_new"] = W.to_storage(case["k_new"], kv_dtype)
+    dev = H.PagedDeviceCase(hip, case)
+    desc = H.pa_desc(hip, case)
+    hip.kv_cache_write(desc, dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                       dev.subsequence_begins, dev.block_indices, dev.block_indices_begins)
+    kc, vc = dev.caches()
+    okc, ovc = case["key_cache"].copy(), case["value_cache"].copy()
+    with np.errstate(over="ignore"):
+        oracle.kv_cache_write(case["k_new"], case["v_new"], okc, ovc, cache_dtype, case["past_lens"],
+                              case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], 4, 128,
+                              32)
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    # untouched rows keep their bytes: exactly T * Hkv rows differ from the initial pool
+    assert (kc != case["key_cache"]).any(axis=-1).sum() == case["T"] * 4
+    dev.free()
+
+
+def test_kv_cache_write_skips_invalid_targets(hip, oracle):
+    announce("kv_write invalid targets")
+    case = W.make_paged_case(52, [(3, 40), (0, 33)], 4, 2, 64, 16, W.F16, W.F16, W.F16)
+    case["block_indices"][0] = case["num_blocks"] + 5
+    case["block_indices"][1] = -1
+    # sequence 1's table is one block short of what its tokens need
+    case["block_indices_begins"][2] -= 1
+    dev = H.PagedDeviceCase(hip, case)
+    hip.kv_cache_write(H.pa_desc(hip, case), dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                       dev.subsequence_begins, dev.block_indices, dev.block_indices_begins)
+    kc, vc = dev.caches()
+    okc, ovc = case["key_cache"].copy(), case["value_cache"].copy()
+    skipped = oracle.kv_cache_write(case["k_new"], case["v_new"], okc, ovc, W.F16, case["past_lens"],
+                                    case["subsequence_begins"], case["block_indices"], case["block_indices_begins"],
+                                    2, 64, 16)
+    assert skipped == 13 + 16 + 1
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    dev.free()
+
+
+# ------------------------------------------------------------------------------------ SDPA
+@pytest.mark.parametrize("shape", [(1, 1, 1, 4, 4, 8), (1, 4, 4, 16, 16, 32), (1, 8, 8, 32, 32, 64),
+                                   (1, 4, 4, 2, 2, 8), (2, 8, 2, 33, 47, 64), (1, 2, 1, 5, 300, 80),
+                                   (1, 2, 2, 70, 70, 256)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [W.F32, W.F16])
+def test_sdpa_small_shapes(hip, oracle, shape, causal, dtype):
+    """Shapes of the reference's SDPA test (scaled_dot_product_attention.cpp:76-104) and odd ones;
+    its f16 threshold is 0.025, the bar here is 2e-3."""
+    announce("sdpa small", shape, causal, dtype)
+    B, Hq, Hkv, Lq, Lk, D = shape
+    case = W.make_sdpa_case(61, B, Hq, Hkv, Lq, Lk, D, dtype)
+    out, path = H.run_sdpa(hip, case, causal)
+    ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+    assert path == "sdpa_generic"
+    assert H.max_abs(out, ref) <= TOL[dtype]
+
+
+def test_sdpa_golden_fixture_on_gpu(hip):
+    announce("sdpa golden")
+    import os
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sdpa_golden.npz"))
+    for name in ("ref_small", "ref_medium", "ref_llm", "ref_3d", "gqa", "rect", "long_row"):
+        q, k, v = z[name + "/q"], z[name + "/k"], z[name + "/v"]
+        case = {"B": q.shape[0], "Hq": q.shape[1], "Hkv": k.shape[1], "Lq": q.shape[2], "Lk": k.shape[2],
+                "D": q.shape[3], "dtype": W.F32, "q_store": q, "k_store": k, "v_store": v}
+        for causal in (False, True):
+            out, _ = H.run_sdpa(hip, case, causal)
+            assert H.max_abs(out, z["%s/out_causal%d" % (name, int(causal))]) <= 1e-4, (name, causal)
+
+
+@pytest.mark.parametrize("dtype", [W.F16, W.BF16])
+@pytest.mark.parametrize("shape,causal", [
+    ((1, 1, 1, 1, 1, 128), True), ((1, 2, 1, 63, 63, 128), True), ((1, 2, 2, 64, 64, 128), False),
+    ((1, 4, 2, 65, 65, 128), True), ((2, 4, 1, 128, 128, 128), True), ((1, 2, 1, 129, 129, 128), True),
+    ((1, 8, 2, 300, 300, 128), True), ((1, 2, 1, 200, 1000, 128), False), ((1, 2, 1, 1000, 200, 128), True),
+    ((1, 4, 4, 1000, 1000, 128), True), ((1, 2, 2, 77, 500, 128), True)])
+def test_sdpa_flash(hip, oracle, dtype, shape, causal):
+    announce("sdpa flash", dtype, shape, causal)
+    B, Hq, Hkv, Lq, Lk, D = shape
+    case = W.make_sdpa_case(62, B, Hq, Hkv, Lq, Lk, D, dtype)
+    out, path = H.run_sdpa(hip, case, causal)
+    assert path == "sdpa_flash_mfma"
+    ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+    assert np.isfinite(out).all()
+    assert H.max_abs(out, ref) <= TOL[dtype]
+
+
+def test_sdpa_scale_and_empty(hip, oracle):
+    announce("sdpa scale/empty")
+    case = W.make_sdpa_case(63, 1, 2, 1, 90, 90, 128, W.F16)
+    out, _ = H.run_sdpa(hip, case, True, scale=0.05)
+    assert H.max_abs(out, oracle.sdpa(case["q"], case["k"], case["v"], causal=True, scale=0.05)) <= 2e-3
+    # len_q == 0 is a no-op; len_kv == 0 yields zeros (nothing to attend)
+    desc = hip.SdpaDesc(W.F16, 1, 2, 1, 0, 16, 128, 0, 0.0)
+    hip.check(hip.lib().hipattn_sdpa(desc, None, None, None, None, None, 0, None))
+    case0 = W.make_sdpa_case(64, 1, 2, 1, 5, 0, 128, W.F16)
+    case0["k_store"] = np.zeros((1,), np.uint16)
+    case0["v_store"] = np.zeros((1,), np.uint16)
+    out0, _ = H.run_sdpa(hip, case0, False)
+    assert np.all(out0 == 0)
+    # invalid descriptors are rejected with a status, not a crash
+    bad = hip.SdpaDesc(W.F16, 1, 3, 2, 4, 4, 128, 0, 0.0)
+    assert hip.lib().hipattn_sdpa(bad, None, None, None, None, None, 0, None) == hip.INVALID_ARGUMENT
+
+
+# ------------------------------------------------------------------------------ paged decode
+DECODE_CTX = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 500, 511, 512, 513, 1023, 1024, 1025, 2000, 3001]
+
+
+@pytest.mark.parametrize("cache_dtype,q_dtype,Hq", [(W.F16, W.F16, 32), (W.F16, W.BF16, 8), (W.U8, W.F16, 64),
+                                                    (W.U8, W.BF16, 16), (W.F16, W.F16, 128)])
+@pytest.mark.parametrize("chunk", [0, 128, 256])
+def test_paged_decode(hip, oracle, cache_dtype, q_dtype, Hq, chunk):
+    announce("paged decode", cache_dtype, q_dtype, Hq, chunk)
+    seqs = [(c - 1, 1) for c in DECODE_CTX]
+    case = W.make_paged_case(71, seqs, Hq, 8, 128, 32, q_dtype, q_dtype, cache_dtype)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run(decode_chunk=chunk)
+    assert path == "paged_mfma"
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    tol = 1e-2 if (cache_dtype == W.U8 or q_dtype == W.BF16) else 2e-3
+    assert np.isfinite(out).all()
+    assert H.max_abs(out, ref) <= tol
+    # the shape-generic kernels agree as well (second, independent device implementation)
+    out_g, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic"
+    assert H.max_abs(out_g, ref) <= tol
+    dev.free()
+
+
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
+@pytest.mark.parametrize("window", [1, 31, 32, 100, 640, 5000])
+def test_paged_decode_sliding_window(hip, oracle, cache_dtype, window):
+    announce("paged decode window", cache_dtype, window)
+    seqs = [(c - 1, 1) for c in DECODE_CTX]
+    case = W.make_paged_case(72, seqs, 32, 8, 128, 32, W.F16, W.F16, cache_dtype, sliding_window=window)
+    dev = H.PagedDeviceCase(hip, case)
+    out, _ = dev.run(decode_chunk=128)
+    ref, _, _ = H.oracle_paged(oracle, case)
+    assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3)
+    dev.free()
+
+
+def test_paged_decode_ignores_garbage_beyond_context(hip, oracle):
+    """Cache rows no sequence has written yet may hold NaN / Inf patterns."""
+    announce("paged decode garbage")
+    seqs = [(c - 1, 1) for c in (5, 33, 70, 257)]
+    for cache_dtype in (W.F16, W.U8):
+        case = W.make_paged_case(73, seqs, 32, 8, 128, 32, W.F16, W.F16, cache_dtype)
+        for s, (past, _) in enumerate(seqs):
+            ctx = past + 1
+            last = case["block_indices"][case["block_indices_begins"][s + 1] - 1]
+            r = ctx % 32
+            if r:
+                case["key_cache"][last, :, r:] = 0xFF
+                case["value_cache"][last, :, r:] = 0xFF
+        dev = H.PagedDeviceCase(hip, case)
+        out, _ = dev.run()
+        ref, _, _ = H.oracle_paged(oracle, case)
+        assert np.isfinite(out).all()
+        assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3)
+        dev.free()
+
+
+def test_paged_block_permutation_is_bit_identical(hip):
+    announce("paged permutation")
+    seqs = [(c - 1, 1) for c in (700, 64, 1500, 33)] + [(100, 200)]
+    case = W.make_paged_case(74, seqs, 32, 8, 128, 32, W.F16, W.F16, W.F16)
+    dev = H.PagedDeviceCase(hip, case)
+    out, _ = dev.run(decode_chunk=256)
+    rng = np.random.default_rng(2)
+    perm = rng.permutation(case["num_blocks"])
+    case2 = dict(case)
+    case2["block_indices"] = perm[case["block_indices"]].astype(np.int32)
+    case2["key_cache"] = np.empty_like(case["key_cache"])
+    case2["value_cache"] = np.empty_like(case["value_cache"])
+    case2["key_cache"][perm] = case["key_cache"]
+    case2["value_cache"][perm] = case["value_cache"]
+    dev2 = H.PagedDeviceCase(hip, case2)
+    out2, _ = dev2.run(decode_chunk=256)
+    np.testing.assert_array_equal(out, out2)
+    dev.free()
+    dev2.free()
+
+
+# ----------------------------------------------------------------- mixed prefill + decode
+@pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.F16, W.F16, 0), (W.BF16, W.F16, 0), (W.BF16, W.F16, 300),
+                                                        (W.F16, W.F16, 64), (W.F16, W.U8, 0), (W.F16, W.U8, 100)])
+def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window):
+    announce("paged mixed", q_dtype, cache_dtype, window)
+    seqs = [(0, 130), (37, 1), (500, 1), (100, 257), (0, 2), (999, 1), (31, 97), (64, 1), (700, 128), (5, 0)]
+    case = W.make_paged_case(81, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run(decode_chunk=128)
+    assert path == "paged_mfma"
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    tol = 1e-2 if (cache_dtype == W.U8 or q_dtype == W.BF16) else 2e-3
+    assert np.isfinite(out).all()
+    assert H.max_abs(out, ref) <= tol
+    dev.free()
+
+
+@pytest.mark.parametrize("shape", [(6, 2, 64, 16, W.F16, W.F16), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
+                                   (4, 1, 128, 16, W.F16, W.U8), (34, 2, 128, 32, W.F16, W.F16)])
+def test_paged_generic_shapes(hip, oracle, shape):
+    """Head sizes, block sizes and GQA ratios outside the MFMA fast path."""
+    announce("paged generic", shape)
+    Hq, Hkv, D, bs, qd, cd = shape
+    seqs = [(0, 9), (37, 1), (31, 2), (5, 40), (64, 1), (200, 1)]
+    case = W.make_paged_case(82, seqs, Hq, Hkv, D, bs, qd, qd, cd, sliding_window=0)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run()
+    assert path == "paged_generic"
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    tol = 1e-2 if (cd in (W.U8, W.BF16) or qd == W.BF16) else (1e-4 if qd == W.F32 else 2e-3)
+    assert H.max_abs(out, ref) <= tol
+    dev.free()
+
+
+def test_paged_errors(hip):
+    announce("paged errors")
+    case = W.make_paged_case(83, [(100, 1), (700, 1)], 32, 8, 128, 32, W.F16, W.F16, W.F16)
+    dev = H.PagedDeviceCase(hip, case)
+    desc = H.pa_desc(hip, case, decode_chunk=128)
+    need = hip.paged_attention_workspace_size(desc)
+    assert need > 0
+    small = hip.DeviceBuffer(need - 1)
+    small.nbytes = need - 1
+    with pytest.raises(hip.HipAttnError) as e:
+        hip.paged_attention(desc, dev.q, dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                            dev.subsequence_begins, dev.block_indices, dev.block_indices_begins, dev.out, small)
+    assert e.value.status == hip.WORKSPACE_TOO_SMALL
+    with pytest.raises(hip.HipAttnError) as e:
+        hip.paged_attention(desc, dev.q, None, None, dev.key_cache, dev.value_cache, dev.past_lens,
+                            dev.subsequence_begins, dev.block_indices, dev.block_indices_begins, dev.out, small)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    dev.free()

@@ -1,0 +1,289 @@
+"""Pins the CPU oracle (oracle/hipattn_oracle.c) without any GPU.
+
+Checks are chosen so that a plausible mistake fails one of them: a wrong mask offset fails the
+torch fixtures and the first-row identity, a transposed GQA mapping fails the repeated-KV
+identity, a wrong block/row index in the scatter fails the brute-force map, a wrong window
+bound fails the explicit-mask comparison, a wrong rounding fails the bit comparisons.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from openvino_contrib_amd import workloads as W
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sdpa_golden.npz")
+
+
+def brute_sdpa_f64(q, k, v, causal, scale=None, mask=None):
+    """Closed form softmax(scale q k^T + mask) v in fp64 with explicit Python loops over heads."""
+    q, k, v = q.astype(np.float64), k.astype(np.float64), v.astype(np.float64)
+    B, Hq, Lq, D = q.shape
+    Hkv, Lk = k.shape[1], k.shape[2]
+    G = Hq // Hkv
+    scale = 1.0 / np.sqrt(D) if scale is None else scale
+    out = np.zeros_like(q)
+    for b in range(B):
+        for h in range(Hq):
+            s = scale * q[b, h] @ k[b, h // G].T
+            if causal:
+                i = np.arange(Lq)[:, None]
+                j = np.arange(Lk)[None, :]
+                s = np.where(j <= i, s, -np.inf)
+            if mask is not None:
+                s = np.where(mask, s, -np.inf)
+            s = s - s.max(axis=1, keepdims=True)
+            p = np.exp(s)
+            p /= p.sum(axis=1, keepdims=True)
+            out[b, h] = p @ v[b, h // G]
+    return out
+
+
+# ------------------------------------------------------------------------------------ SDPA
+@pytest.mark.parametrize("name", ["ref_small", "ref_medium", "ref_llm", "ref_3d", "gqa", "rect", "long_row"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_sdpa_matches_torch_fixture(oracle, name, causal):
+    z = np.load(GOLDEN)
+    out = oracle.sdpa(z[name + "/q"], z[name + "/k"], z[name + "/v"], causal=causal)
+    np.testing.assert_allclose(out, z["%s/out_causal%d" % (name, int(causal))], atol=2e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 2, 5, 9, 8), (2, 6, 3, 12, 12, 16), (1, 4, 1, 9, 4, 32)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_sdpa_matches_fp64_brute_force(oracle, shape, causal):
+    B, Hq, Hkv, Lq, Lk, D = shape
+    c = W.make_sdpa_case(7, B, Hq, Hkv, Lq, Lk, D, W.F32)
+    out = oracle.sdpa(c["q"], c["k"], c["v"], causal=causal, scale=0.37)
+    ref = brute_sdpa_f64(c["q"], c["k"], c["v"], causal, scale=0.37)
+    np.testing.assert_allclose(out, ref, atol=2e-6, rtol=1e-5)
+
+
+def test_sdpa_invariants(oracle):
+    c = W.make_sdpa_case(11, 2, 4, 2, 10, 10, 16, W.F32)
+    q, k, v = c["q"], c["k"], c["v"]
+    out = oracle.sdpa(q, k, v, causal=True)
+    # causal row 0 sees only key 0
+    G = 2
+    for h in range(4):
+        np.testing.assert_allclose(out[:, h, 0], v[:, h // G, 0], atol=1e-6)
+    # GQA == MHA with K/V repeated along heads
+    out_mha = oracle.sdpa(q, np.repeat(k, G, axis=1), np.repeat(v, G, axis=1), causal=True)
+    np.testing.assert_array_equal(out, out_mha)
+    # uniform V gives V back; adding a constant to every score of a row changes nothing
+    vu = np.broadcast_to(v[:, :, :1], v.shape).copy()
+    np.testing.assert_allclose(oracle.sdpa(q, k, vu, causal=False), np.repeat(vu[:, :, :1], G, axis=1).repeat(10, 2),
+                               atol=1e-6)
+    # batch permutation equivariance
+    np.testing.assert_array_equal(oracle.sdpa(q[::-1], k[::-1], v[::-1], causal=True), out[::-1])
+    # default scale is 1/sqrt(D)
+    np.testing.assert_array_equal(oracle.sdpa(q, k, v, causal=True, scale=0.0),
+                                  oracle.sdpa(q, k, v, causal=True, scale=np.float32(1 / np.sqrt(np.float32(16)))))
+
+
+def test_sdpa_empty_and_bad_args(oracle):
+    q = np.zeros((1, 2, 0, 8), np.float32)
+    k = np.zeros((1, 2, 5, 8), np.float32)
+    assert oracle.sdpa(q, k, k).shape == (1, 2, 0, 8)
+    q = np.ones((1, 2, 3, 8), np.float32)
+    k = np.zeros((1, 2, 0, 8), np.float32)
+    assert np.all(oracle.sdpa(q, k, k) == 0)  # nothing to attend: zeros, not NaN
+    with pytest.raises(ValueError):
+        oracle.sdpa(np.ones((1, 3, 2, 8), np.float32), np.ones((1, 2, 2, 8), np.float32),
+                    np.ones((1, 2, 2, 8), np.float32))
+
+
+# ------------------------------------------------------------------------------ conversions
+def test_f16_bf16_conversions_bit_exact(oracle):
+    rng = np.random.default_rng(3)
+    x = np.concatenate([
+        rng.standard_normal(4096).astype(np.float32),
+        (rng.standard_normal(4096) * 1e-6).astype(np.float32),   # fp16 subnormal range
+        (rng.standard_normal(1024) * 3e4).astype(np.float32),    # near fp16 overflow
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, -1e9, 2.0 ** -24, 2.0 ** -25, 3 * 2.0 ** -26,
+                  np.inf, -np.inf], np.float32),
+    ])
+    with np.errstate(over="ignore"):
+        np.testing.assert_array_equal(oracle.f32_to_f16_bits(x), x.astype(np.float16).view(np.uint16))
+    h = np.arange(0, 65536, dtype=np.uint32).astype(np.uint16)
+    finite = (h & 0x7C00) != 0x7C00
+    np.testing.assert_array_equal(oracle.f16_bits_to_f32(h)[finite], h.view(np.float16).astype(np.float32)[finite])
+    # every finite half survives the round trip
+    np.testing.assert_array_equal(oracle.f32_to_f16_bits(oracle.f16_bits_to_f32(h[finite])), h[finite])
+    import torch
+    tb = torch.from_numpy(x[:-2]).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    np.testing.assert_array_equal(oracle.f32_to_bf16_bits(x[:-2]), tb)
+    np.testing.assert_array_equal(W.f32_to_bf16_bits(x[:-2]), tb)
+    np.testing.assert_array_equal(W.f32_to_f16_bits(x[:9000]), oracle.f32_to_f16_bits(x[:9000]))
+
+
+# ---------------------------------------------------------------------------- u8 rows
+def test_u8_quant_invariants(oracle):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((500, 128)).astype(np.float32)
+    x[7] = 1.25       # constant row
+    x[8, :] = 0.0
+    rows = oracle.quant_u8_rows(x)
+    scale = rows[:, 0:4].copy().view(np.float32)[:, 0]
+    zp = rows[:, 4:8].copy().view(np.float32)[:, 0]
+    q = rows[:, 8:]
+    xh = oracle.dequant_u8_rows(rows)
+    # layout and formula, restated independently in fp64
+    np.testing.assert_allclose(scale[:7], (x[:7].max(1).astype(np.float64) - x[:7].min(1)) / 255.0, rtol=1e-6)
+    assert scale[7] == np.float32(0.0001) and scale[8] == np.float32(0.0001)
+    np.testing.assert_allclose(zp, -x.min(1).astype(np.float64) / scale, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(xh, (q.astype(np.float64) - zp[:, None]) * scale[:, None], rtol=1e-6, atol=1e-7)
+    # error bound and extreme values
+    assert np.all(np.abs(xh - x) <= scale[:, None] * 0.5 * (1 + 1e-4) + 1e-6)
+    rowsel = np.arange(500) != 7
+    assert np.all(q[rowsel & (np.arange(500) != 8)].min(1) == 0)
+    assert np.all(q[rowsel & (np.arange(500) != 8)].max(1) == 255)
+    # the workload generator's numpy quantiser agrees (bytes within one step, scale/zp exactly)
+    rows_np = W.quantize_u8_rows(x)
+    np.testing.assert_array_equal(rows_np[:, :8], rows[:, :8])
+    assert np.abs(rows_np[:, 8:].astype(np.int32) - q.astype(np.int32)).max() <= 1
+    assert (rows_np[:, 8:] != q).mean() < 1e-3
+
+
+# -------------------------------------------------------------------------- KV scatter
+def _brute_scatter(case, cache_dtype):
+    """Independent restatement of the slot map in plain Python."""
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    D, Hkv, bs = case["D"], case["Hkv"], case["block_size"]
+    for s in range(case["S"]):
+        t0, t1 = case["subsequence_begins"][s], case["subsequence_begins"][s + 1]
+        for t in range(t0, t1):
+            p = case["past_lens"][s] + (t - t0)
+            blk = case["block_indices"][case["block_indices_begins"][s] + p // bs]
+            for h in range(Hkv):
+                kc[blk, h, p % bs] = W.cache_rows_from_f32(case["k_new"][t, h * D:(h + 1) * D][None], cache_dtype)[0]
+                vc[blk, h, p % bs] = W.cache_rows_from_f32(case["v_new"][t, h * D:(h + 1) * D][None], cache_dtype)[0]
+    return kc, vc
+
+
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.BF16, W.F32])
+def test_kv_write_matches_brute_force(oracle, cache_dtype):
+    case = W.make_paged_case(21, [(0, 5), (31, 1), (32, 1), (40, 30), (7, 0), (63, 2)], 4, 2, 16, 32, W.F16, W.F16,
+                             cache_dtype)
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    skipped = oracle.kv_cache_write(case["k_new"], case["v_new"], kc, vc, cache_dtype, case["past_lens"],
+                                    case["subsequence_begins"], case["block_indices"], case["block_indices_begins"],
+                                    2, 16, 32)
+    assert skipped == 0
+    bk, bv = _brute_scatter(case, cache_dtype)
+    np.testing.assert_array_equal(kc, bk)
+    np.testing.assert_array_equal(vc, bv)
+    # exactly T * Hkv rows changed in each cache (values are random, so a rewritten row differs)
+    changed = (kc != case["key_cache"]).any(axis=-1).sum()
+    assert changed == case["T"] * 2
+
+
+def test_kv_write_then_gather_is_identity_and_skips_bad_blocks(oracle):
+    case = W.make_paged_case(22, [(3, 40), (0, 33)], 2, 2, 8, 16, W.F32, W.F32, W.F32)
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    oracle.kv_cache_write(case["k_new"], case["v_new"], kc, vc, W.F32, case["past_lens"], case["subsequence_begins"],
+                          case["block_indices"], case["block_indices_begins"], 2, 8, 16)
+    for s, (past, n) in enumerate([(3, 40), (0, 33)]):
+        blocks = case["block_indices"][case["block_indices_begins"][s]:case["block_indices_begins"][s + 1]]
+        for h in range(2):
+            rows = oracle.gather_cache_rows(kc, W.F32, blocks, past + n, h, 2, 8, 16)
+            t0 = case["subsequence_begins"][s]
+            np.testing.assert_array_equal(rows[past:], case["k_new"][t0:t0 + n, h * 8:(h + 1) * 8])
+    # out-of-range physical ids and positions past the table are skipped, nothing is written
+    # (expectation of modules/nvidia_plugin/tests/unit/kernels/scatter_update.cpp:59-86)
+    bad = case["block_indices"].copy()
+    bad[0] = case["num_blocks"] + 5
+    bad[1] = -1
+    kc2, vc2 = case["key_cache"].copy(), case["value_cache"].copy()
+    skipped = oracle.kv_cache_write(case["k_new"], case["v_new"], kc2, vc2, W.F32, case["past_lens"],
+                                    case["subsequence_begins"], bad, case["block_indices_begins"], 2, 8, 16)
+    assert skipped == (16 - 3) + 16  # positions 3..15 -> block 0, 16..31 -> block 1
+    short = case["block_indices_begins"].copy()
+    short[1] -= 1  # hide sequence 0's last block
+    short_idx = np.concatenate([case["block_indices"][:2], case["block_indices"][3:]])
+    short[2] -= 1
+    kc3, vc3 = case["key_cache"].copy(), case["value_cache"].copy()
+    skipped = oracle.kv_cache_write(case["k_new"], case["v_new"], kc3, vc3, W.F32, case["past_lens"],
+                                    case["subsequence_begins"], short_idx, short, 2, 8, 16)
+    assert skipped == (3 + 40) - 32
+
+
+# ---------------------------------------------------------------------- paged attention
+def _dense_reference(oracle, case, s, scale=None):
+    """Paged attention of sequence s via gather + dense SDPA with an explicit brute-force mask."""
+    D, Hq, Hkv, bs, Wn = case["D"], case["Hq"], case["Hkv"], case["block_size"], case["sliding_window"]
+    past = int(case["past_lens"][s])
+    t0, t1 = int(case["subsequence_begins"][s]), int(case["subsequence_begins"][s + 1])
+    n = t1 - t0
+    ctx = past + n
+    blocks = case["block_indices"][case["block_indices_begins"][s]:case["block_indices_begins"][s + 1]]
+    k = np.stack([oracle.gather_cache_rows(case["kc_after"], case["cache_dtype"], blocks, ctx, h, Hkv, D, bs)
+                  for h in range(Hkv)])[None]
+    v = np.stack([oracle.gather_cache_rows(case["vc_after"], case["cache_dtype"], blocks, ctx, h, Hkv, D, bs)
+                  for h in range(Hkv)])[None]
+    q = case["q"][t0:t1].reshape(n, Hq, D).transpose(1, 0, 2)[None]
+    i = past + np.arange(n)[:, None]
+    j = np.arange(ctx)[None, :]
+    mask = j <= i
+    if Wn > 0:
+        mask &= j > i - Wn
+    out = brute_sdpa_f64(q, k, v, causal=False, scale=scale, mask=mask)
+    return out[0].transpose(1, 0, 2).reshape(n, Hq * D)
+
+
+@pytest.mark.parametrize("cache_dtype,window", [(W.F16, 0), (W.F32, 0), (W.U8, 0), (W.F16, 24), (W.BF16, 7)])
+def test_paged_attention_reduces_to_dense(oracle, cache_dtype, window):
+    seqs = [(0, 9), (37, 1), (31, 2), (5, 40), (64, 1)]
+    case = W.make_paged_case(31, seqs, 4, 2, 16, 16, W.F32, W.F32, cache_dtype, sliding_window=window)
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    out = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc, vc, cache_dtype, case["past_lens"],
+                                 case["subsequence_begins"], case["block_indices"], case["block_indices_begins"],
+                                 4, 2, 16, 16, sliding_window=window)
+    case["kc_after"], case["vc_after"] = kc, vc
+    for s in range(len(seqs)):
+        t0, t1 = case["subsequence_begins"][s], case["subsequence_begins"][s + 1]
+        np.testing.assert_allclose(out[t0:t1], _dense_reference(oracle, case, s), atol=3e-6, rtol=1e-5)
+    # the op's own write equals the stand-alone writer
+    kc2, vc2 = case["key_cache"].copy(), case["value_cache"].copy()
+    oracle.kv_cache_write(case["k_new"], case["v_new"], kc2, vc2, cache_dtype, case["past_lens"],
+                          case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], 2, 16, 16)
+    np.testing.assert_array_equal(kc, kc2)
+    np.testing.assert_array_equal(vc, vc2)
+
+
+def test_paged_attention_block_permutation_invariance_and_window(oracle):
+    seqs = [(20, 12), (50, 1), (0, 3)]
+    case = W.make_paged_case(32, seqs, 4, 2, 16, 8, W.F32, W.F32, W.F16)
+    args = lambda c, kc, vc, w: (c["q"], c["k_new"], c["v_new"], kc, vc, W.F16, c["past_lens"],
+                                 c["subsequence_begins"], c["block_indices"], c["block_indices_begins"], 4, 2, 16, 8)
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    out = oracle.paged_attention(*args(case, kc, vc, 0))
+    # move every physical block to a new place and permute the table accordingly: bit-identical
+    rng = np.random.default_rng(1)
+    perm = rng.permutation(case["num_blocks"])
+    case2 = dict(case)
+    case2["block_indices"] = perm[case["block_indices"]].astype(np.int32)
+    kc2 = np.empty_like(case["key_cache"])
+    vc2 = np.empty_like(case["value_cache"])
+    kc2[perm] = case["key_cache"]
+    vc2[perm] = case["value_cache"]
+    out2 = oracle.paged_attention(*args(case2, kc2, vc2, 0))
+    np.testing.assert_array_equal(out, out2)
+    # a window at least as long as every context changes nothing; a short one does
+    kc3, vc3 = case["key_cache"].copy(), case["value_cache"].copy()
+    out3 = oracle.paged_attention(*args(case, kc3, vc3, 0), sliding_window=51)
+    np.testing.assert_array_equal(out, out3)
+    kc4, vc4 = case["key_cache"].copy(), case["value_cache"].copy()
+    out4 = oracle.paged_attention(*args(case, kc4, vc4, 0), sliding_window=4)
+    assert np.abs(out4 - out).max() > 1e-3
+    # chunked prefill: sequence 0 fed as 5 + 7 tokens gives the same rows as 12 at once
+    caseA = W.make_paged_case(33, [(20, 12)], 4, 2, 16, 8, W.F32, W.F32, W.F32)
+    kcA, vcA = caseA["key_cache"].copy(), caseA["value_cache"].copy()
+    full = oracle.paged_attention(*args(caseA, kcA, vcA, 0)[:5], W.F32, *args(caseA, kcA, vcA, 0)[6:])
+    kcB, vcB = caseA["key_cache"].copy(), caseA["value_cache"].copy()
+    parts = []
+    for past, lo, hi in ((20, 0, 5), (25, 5, 12)):
+        parts.append(oracle.paged_attention(caseA["q"][lo:hi], caseA["k_new"][lo:hi], caseA["v_new"][lo:hi], kcB, vcB,
+                                            W.F32, np.array([past], np.int32), np.array([0, hi - lo], np.int32),
+                                            caseA["block_indices"], caseA["block_indices_begins"], 4, 2, 16, 8))
+    np.testing.assert_allclose(np.concatenate(parts), full, atol=1e-6)
+    np.testing.assert_array_equal(kcA, kcB)
