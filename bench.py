@@ -73,7 +73,9 @@ def bench_paged(hip, case, steps, warmup, name):
     path = hip.last_kernel_path()
     kv_bytes = W.paged_kv_bytes(case)
     flops = W.paged_flops(case)
+    decode_only = W.paged_kv_bytes(case, decode_only=True)  # what the split-context decode kernel reads
     res = {
+        "decode_kv_bytes": decode_only,
         "workload": name, "kernel_path": path, "ms_per_step": ms, "host_ms_per_step": wall_ms,
         "dominant_kernel_ms": kern_ms, "kv_bytes": kv_bytes, "flops": flops, "workspace_bytes": ws_bytes,
         "kv_gbs": kv_bytes / (ms * 1e-3) / 1e9, "tflops": flops / (ms * 1e-3) / 1e12,
@@ -106,7 +108,7 @@ def bench_sdpa(hip, case, steps, warmup, name):
 
 
 def roofline_hbm(res, traffic=None):
-    a = res["kv_bytes"] / (res["dominant_kernel_ms"] * 1e-3) / 1e9
+    a = res["decode_kv_bytes"] / (res["dominant_kernel_ms"] * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
             "traffic": traffic, "kernel": "paged_decode_kernel"}
 
@@ -117,37 +119,27 @@ def roofline_mfma(res):
             "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "sdpa_flash_kernel"}
 
 
-def cpu_baseline_paged(case, n_seqs, budget_s=20.0):
-    """Oracle (port) on the first n_seqs sequences of the case, attention only."""
+def cpu_baseline_paged(case, budget_s=12.0):
+    """Oracle (port, OpenMP over sequences x kv heads) on the whole batch, attention only,
+    repeated until about budget_s seconds of CPU work have been spent."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
-    import numpy as np
     import oracle as O
     from openvino_contrib_amd import workloads as W
 
-    n = min(n_seqs, case["S"])
-    sub = dict(case)
-    sub["S"] = n
-    sub["past_lens"] = case["past_lens"][:n]
-    sub["subsequence_begins"] = case["subsequence_begins"][:n + 1]
-    sub["block_indices_begins"] = case["block_indices_begins"][:n + 1]
-    T = int(sub["subsequence_begins"][-1])
     kc, vc = case["key_cache"], case["value_cache"]
-    best = None
-    t_end = time.perf_counter() + budget_s
-    reps = 0
-    while reps < 3 and (reps == 0 or time.perf_counter() < t_end):
+    times = []
+    t_begin = time.perf_counter()
+    while not times or (time.perf_counter() - t_begin < budget_s and len(times) < 200):
         t0 = time.perf_counter()
-        O.paged_attention(case["q"][:T], case["k_new"][:T], case["v_new"][:T], kc, vc, case["cache_dtype"],
-                          sub["past_lens"], sub["subsequence_begins"], case["block_indices"],
-                          sub["block_indices_begins"], case["Hq"], case["Hkv"], case["D"], case["block_size"],
+        O.paged_attention(case["q"], case["k_new"], case["v_new"], kc, vc, case["cache_dtype"], case["past_lens"],
+                          case["subsequence_begins"], case["block_indices"], case["block_indices_begins"],
+                          case["Hq"], case["Hkv"], case["D"], case["block_size"],
                           sliding_window=case["sliding_window"], do_write=False)
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
-        reps += 1
-    b = W.paged_kv_bytes(sub)
-    return {"value": b / best / 1e9, "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
-            "sample": "oracle paged attention (no cache write) on the first %d of %d sequences, best of %d, %.2f s"
-                      % (n, case["S"], reps, best)}
+        times.append(time.perf_counter() - t0)
+    mean = sum(times) / len(times)
+    return {"value": W.paged_kv_bytes(case) / mean / 1e9, "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+            "sample": "oracle paged attention (no cache write) on all %d sequences of the workload, mean of %d passes, "
+                      "%.1f s of CPU work" % (case["S"], len(times), sum(times))}
 
 
 def cpu_baseline_sdpa(case, budget_s=20.0):
@@ -156,13 +148,20 @@ def cpu_baseline_sdpa(case, budget_s=20.0):
     from openvino_contrib_amd import workloads as W
 
     G = case["Hq"] // case["Hkv"]
-    t0 = time.perf_counter()
-    O.sdpa(case["q"][:1, :G], case["k"][:1, :1], case["v"][:1, :1], causal=True)
-    dt = time.perf_counter() - t0
-    fl = W.sdpa_flops(1, G, case["Lq"], case["Lk"], case["D"], True)
-    return {"value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
-            "sample": "oracle fp32 SDPA on batch 0, kv head 0 (%d of %d query heads), %.2f s"
-                      % (G, case["B"] * case["Hq"], dt)}
+    times = []
+    t_begin = time.perf_counter()
+    n = 0
+    while not times or (time.perf_counter() - t_begin < budget_s and n < case["B"] * case["Hkv"]):
+        b, hkv = divmod(n, case["Hkv"])
+        t0 = time.perf_counter()
+        O.sdpa(case["q"][b:b + 1, hkv * G:(hkv + 1) * G], case["k"][b:b + 1, hkv:hkv + 1],
+               case["v"][b:b + 1, hkv:hkv + 1], causal=True)
+        times.append(time.perf_counter() - t0)
+        n += 1
+    fl = W.sdpa_flops(1, G, case["Lq"], case["Lk"], case["D"], True) * len(times)
+    return {"value": fl / sum(times) / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
+            "sample": "oracle fp32 SDPA on %d of %d (batch, kv head) groups of the workload, %.1f s of CPU work"
+                      % (len(times), case["B"] * case["Hkv"], sum(times))}
 
 
 def main():
@@ -170,7 +169,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy"],
+                    help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="measure the headline workload only")
     args = ap.parse_args()
@@ -185,7 +185,29 @@ def main():
         sys.exit("bench.py: no HIP device")
     hip.check(hip.lib().hipattn_set_device(0))
     info = hip.device_info(0)
-    log("device:", info.name.decode(), info.arch.decode(), info.compute_units, "CUs")
+    dev_name = info.name.decode() or ("AMD " + info.arch.decode())
+    log("device:", dev_name, info.arch.decode(), info.compute_units, "CUs")
+
+    if args.workload == "copy":
+        # Known-size traffic for scaling FETCH_SIZE / WRITE_SIZE: a device-to-device copy of 1 GiB
+        # (1 GiB read + 1 GiB written per launch) and a 1 GiB fill kernel (1 GiB written).
+        n = 1 << 30
+        src, dst = hip.DeviceBuffer(n), hip.DeviceBuffer(n)
+        src.fill(1)
+        dst.fill(2)
+        hip.check(hip.lib().hipattn_stream_synchronize(None))
+        e0, e1, e2 = hip.Event(), hip.Event(), hip.Event()
+        e0.record()
+        for _ in range(args.steps):
+            hip.check(hip.lib().hipattn_memcpy_d2d_async(dst.ptr, src.ptr, n, None))
+        e1.record()
+        for _ in range(args.steps):
+            dst.fill(3)
+        e2.record()
+        e2.synchronize()
+        print(json.dumps({"workload": "copy", "bytes_per_launch": n, "launches_each": args.steps,
+                          "d2d_copy_ms": e0.elapsed_ms(e1) / args.steps, "fill_ms": e1.elapsed_ms(e2) / args.steps}))
+        return
 
     names = {"c2": "config2: bf16 causal prefill SDPA B4 Hq32 Hkv8 L2048 D128",
              "c3": "config3: fp16 paged decode, 64 seq x 1 token, ctx U[512,8192], blk 32, Hq32 Hkv8 D128",
@@ -211,7 +233,7 @@ def main():
         log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f"
             % (w, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"]))
         if not args.no_cpu and w == args.workload:
-            cpu = cpu_baseline_sdpa(case) if w == "c2" else cpu_baseline_paged(case, 8)
+            cpu = cpu_baseline_sdpa(case) if w == "c2" else cpu_baseline_paged(case)
             log("cpu baseline:", cpu)
         results[w] = r
         del case
@@ -227,7 +249,7 @@ def main():
         "dtype": "bf16" if is_sdpa else ("u8" if args.workload == "c4" else "f16"),
         "data": "synthetic",
         "config": {"workload": head["workload"], "kernel_path": head["kernel_path"],
-                   "device": info.name.decode(), "arch": info.arch.decode()},
+                   "device": dev_name, "arch": info.arch.decode(), "compute_units": info.compute_units},
         "roofline": head["roofline"],
         "cpu_baseline": cpu if cpu else None,
         "workloads": {k: v for k, v in results.items()},

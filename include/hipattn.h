@@ -143,8 +143,10 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * are quantised on the fly.  Blocks outside the table or outside [0, num_blocks) are skipped.
  * Step 2: that token attends cache positions j, max(0, p - sliding_window + 1) <= j <= p
  * (all of 0..p when sliding_window <= 0).
- * All index arrays live in device memory; the host only passes upper bounds:
- * max_context_len >= max_s(past_lens[s] + q_len[s]) sizes the split of the context. */
+ * All index arrays live in device memory and are only read there; the split of the work is
+ * planned on the device.  max_context_len (>= max_s(past_lens[s] + q_len[s])) is advisory.
+ * A sequence may contribute no token to a batch, with one exception: a batch with
+ * num_tokens == num_seqs is taken to hold exactly one token per sequence (pure decode). */
 enum {
     HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */
     HIPATTN_PA_FORCE_GENERIC = 2     /* use the shape-generic kernels (testing aid) */
@@ -166,7 +168,7 @@ typedef struct hipattn_pa_desc {
     int sliding_window;
     float scale;       /* <= 0 selects 1/sqrt(head_dim) */
     int flags;         /* HIPATTN_PA_* */
-    int decode_chunk;  /* tokens per split of a decode context; 0 = choose */
+    int decode_waves;  /* wavefronts the decode contexts are spread over; 0 = as many as the device keeps resident */
 } hipattn_pa_desc;
 
 hipattn_status hipattn_paged_attention_workspace_size(const hipattn_pa_desc* desc, size_t* bytes);

@@ -69,7 +69,7 @@ class PaDesc(ctypes.Structure):
         ("sliding_window", ctypes.c_int),
         ("scale", ctypes.c_float),
         ("flags", ctypes.c_int),
-        ("decode_chunk", ctypes.c_int),
+        ("decode_waves", ctypes.c_int),
     ]
 
 

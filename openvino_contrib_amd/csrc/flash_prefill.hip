@@ -324,38 +324,6 @@ __global__ __launch_bounds__(kThreads) void sdpa_flash_kernel(SdpaParams p) {
     run_tile<kBf16>(t, k_lds, v_lds, p.scale);
 }
 
-// Exclusive prefix of query tiles per sequence (sequences with a single token have none:
-// they belong to the decode kernel).  One workgroup; sequences are split evenly over threads.
-__global__ __launch_bounds__(256) void paged_prefill_plan_kernel(PagedParams p) {
-    __shared__ int partial[256];
-    const int tid = threadIdx.x;
-    const int per = (p.num_seqs + 255) / 256;
-    const int s0 = min(tid * per, p.num_seqs), s1 = min(s0 + per, p.num_seqs);
-    int sum = 0;
-    for (int s = s0; s < s1; s++) {
-        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
-        sum += qlen > 1 ? (qlen + kTileQ - 1) / kTileQ : 0;
-    }
-    partial[tid] = sum;
-    __syncthreads();
-    if (tid == 0) {
-        int run = 0;
-        for (int i = 0; i < 256; i++) {
-            int v = partial[i];
-            partial[i] = run;
-            run += v;
-        }
-    }
-    __syncthreads();
-    int run = partial[tid];
-    for (int s = s0; s < s1; s++) {
-        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
-        p.tile_prefix[s] = run;
-        run += qlen > 1 ? (qlen + kTileQ - 1) / kTileQ : 0;
-    }
-    if (s1 == p.num_seqs && s0 < p.num_seqs) p.tile_prefix[p.num_seqs] = run;
-}
-
 template <bool kBf16>
 __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t k_lds[kTileK * kKRow];
@@ -426,9 +394,6 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
 }
 
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL(flash::paged_prefill_plan_kernel, dim3(1), dim3(256), 0, stream, p);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
     dim3 grid(p.max_q_tiles, p.num_heads_q);
     if (p.cache_dtype == HIPATTN_BF16)
         hipLaunchKernelGGL(flash::paged_prefill_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);

@@ -76,6 +76,8 @@ hipattn_status validate_pa(const hipattn_pa_desc* d, bool need_q) {
     if (d->head_dim > 512) return fail(HIPATTN_UNSUPPORTED, "paged_attention: head_dim %d > 512", d->head_dim);
     if (d->num_blocks < 0 || d->num_tokens < 0 || d->num_seqs < 0 || d->max_context_len < 0)
         return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: negative extent");
+    if (d->decode_waves < 0 || d->decode_waves > 65536)
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: decode_waves %d outside [0, 65536]", d->decode_waves);
     if (d->cache_dtype == HIPATTN_U8 && d->head_dim % 8)
         return fail(HIPATTN_UNSUPPORTED, "paged_attention: u8 cache needs head_dim %% 8 == 0 (row alignment)");
     return HIPATTN_OK;
@@ -120,7 +122,7 @@ hipattn::PagedParams make_paged_params(const hipattn_pa_desc* d) {
     p.max_context_len = d->max_context_len;
     p.sliding_window = d->sliding_window;
     p.scale = resolve_scale(d->scale, d->head_dim);
-    p.chunk_tokens = d->decode_chunk;
+    p.num_waves = d->decode_waves > 0 ? d->decode_waves : 0;
     return p;
 }
 
@@ -385,12 +387,10 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* des
     if (!q || !out || !key_cache || !value_cache || !past_lens || !subsequence_begins || !block_indices ||
         !block_indices_begins)
         return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: null pointer");
-    if (!(desc->flags & HIPATTN_PA_SKIP_CACHE_WRITE)) {
-        if (!k_new || !v_new) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: null k_new/v_new");
-        hipattn::KvWriteParams w = make_write_params(desc, k_new, v_new, key_cache, value_cache, past_lens,
-                                                     subsequence_begins, block_indices, block_indices_begins);
-        HIP_TRY(hipattn::launch_kv_cache_write(w, as_stream(stream)));
-    }
+    const bool do_write = !(desc->flags & HIPATTN_PA_SKIP_CACHE_WRITE);
+    if (do_write && (!k_new || !v_new)) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: null k_new/v_new");
+    hipattn::KvWriteParams w = make_write_params(desc, k_new, v_new, key_cache, value_cache, past_lens,
+                                                 subsequence_begins, block_indices, block_indices_begins);
     hipattn::PagedParams p = make_paged_params(desc);
     p.q = q;
     p.key_cache = (const uint8_t*)key_cache;
@@ -409,9 +409,10 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* des
             return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: workspace must be 16-byte aligned");
         hipattn::paged_fast_plan(p, workspace);
         g_kernel_path = "paged_mfma";
-        HIP_TRY(hipattn::launch_paged_fast(p, as_stream(stream), g_probe));
+        HIP_TRY(hipattn::launch_paged_fast(p, do_write ? &w : nullptr, as_stream(stream), g_probe));
     } else {
         g_kernel_path = "paged_generic";
+        if (do_write) HIP_TRY(hipattn::launch_kv_cache_write(w, as_stream(stream)));
         HIP_TRY(hipattn::launch_paged_generic(p, as_stream(stream)));
     }
     return HIPATTN_OK;

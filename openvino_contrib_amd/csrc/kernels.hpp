@@ -66,11 +66,12 @@ struct PagedParams {
     int max_context_len;
     int sliding_window;
     float scale;  // already resolved (> 0)
-    // split-context decode: partial results live in the caller's workspace
-    int chunk_tokens;     // tokens per split (multiple of block_size)
-    int max_chunks;       // ceil(max attended tokens / chunk_tokens)
-    float* part_out;      // [num_seqs, num_heads_q, max_chunks, head_dim]
-    float* part_ml;       // [num_seqs, num_heads_q, max_chunks, 2] running max (log2 domain) and sum
+    // decode: the batch's block-heads are cut into num_waves equal pieces (one per wavefront);
+    // pieces that do not cover a whole (sequence, kv head) segment leave partials in the workspace
+    int num_waves;        // wavefronts (= single-wavefront workgroups) of the decode kernel
+    int32_t* blk_prefix;  // [num_seqs + 1] exclusive prefix of attended blocks of decode sequences
+    float* part_out;      // [num_waves + num_seqs*num_heads_kv, G, head_dim] unnormalised outputs
+    float* part_ml;       // [num_waves + num_seqs*num_heads_kv, G, 2] running max (log2 domain) and sum
     // chunked prefill: query-tile schedule built on the device
     int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
     int max_q_tiles;      // grid upper bound
@@ -94,13 +95,14 @@ hipError_t launch_paged_generic(const PagedParams& p, hipStream_t stream);
 bool sdpa_flash_supported(const SdpaParams& p);
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
 
-// paged attention fast paths: split-context decode (+ merge) and chunked prefill
+// paged attention fast paths: plan + stream-K decode + merge, and chunked prefill
 bool paged_fast_supported(const PagedParams& p);
 size_t paged_fast_workspace_bytes(const PagedParams& p);
 void paged_fast_plan(PagedParams& p, void* workspace);  // fills chunking fields and workspace pointers
-hipError_t launch_paged_fast(const PagedParams& p, hipStream_t stream, const KernelProbe& probe);
-hipError_t launch_paged_decode(const PagedParams& p, hipStream_t stream, const KernelProbe& probe);  // + merge
-hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream);  // plan + flash over the block table
+// write == nullptr skips the KV-cache write of the new tokens
+hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
+                             const KernelProbe& probe);
+hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream);  // flash over the block table (needs the plan)
 
 hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t stream);
 

@@ -1,106 +1,31 @@
 // Device-side KV-cache block writer: scatters the new key/value rows of a batch into the
 // paged caches, converting or quantising on the way.  HBM-bound byte moving: one wavefront
-// per (token, kv head), 128-bit friendly contiguous rows, no staging.
+// per (token, kv head), contiguous rows, no staging.
 //
 // Nearest reference analogue: the row scatter of src/kernels/scatter_nd_update.cu:19-34,
 // 36-79 (which first copies the whole input, scatter_nd_update.cu:170-171; this writer
 // touches only the new rows) and the whole-state copies of
 // src/cuda_variable_state.hpp:135-160.  Out-of-range targets are skipped as in
 // tests/unit/kernels/scatter_update.cpp:59-86.
-#include "device_common.hpp"
-#include "kernels.hpp"
+#include "kv_cache_write.hpp"
 
 namespace hipattn {
 
-// sequence that owns token t: largest s with subsequence_begins[s] <= t
-__device__ __forceinline__ int find_sequence(const int32_t* __restrict__ begins, int num_seqs, int t) {
-    int lo = 0, hi = num_seqs;  // invariant: begins[lo] <= t < begins[hi]
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (begins[mid] <= t)
-            lo = mid;
-        else
-            hi = mid;
-    }
-    return lo;
-}
-
 template <int kMaxPerLane>
-__global__ __launch_bounds__(64) void kv_cache_write_kernel(KvWriteParams p) {
-    const int t = blockIdx.x;
-    const int h = blockIdx.y;
-    const int lane = threadIdx.x;
-    if (t >= p.num_tokens) return;
-    // tokens outside every sequence (padding after the last subsequence) are ignored
-    if (t < p.subsequence_begins[0] || t >= p.subsequence_begins[p.num_seqs]) return;
-    const int s = find_sequence(p.subsequence_begins, p.num_seqs, t);
-    const int pos = p.past_lens[s] + (t - p.subsequence_begins[s]);
-    if (pos < 0) return;
-    const int lb = pos / p.block_size;
-    const int tb0 = p.block_indices_begins[s];
-    if (lb >= p.block_indices_begins[s + 1] - tb0) return;
-    const int pb = p.block_indices[tb0 + lb];
-    if (pb < 0 || pb >= p.num_blocks) return;
-
-    const int D = p.head_dim;
-    const int64_t rb = cache_row_bytes(p.cache_dtype, D);
-    const int64_t row_off = (((int64_t)pb * p.num_heads_kv + h) * p.block_size + pos % p.block_size) * rb;
-    const int64_t src_off = ((int64_t)t * p.num_heads_kv + h) * D;
-
-#pragma unroll
-    for (int which = 0; which < 2; which++) {
-        const void* src = which ? p.v_new : p.k_new;
-        uint8_t* row = (which ? p.value_cache : p.key_cache) + row_off;
-        float x[kMaxPerLane];
-        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
-#pragma unroll
-        for (int i = 0; i < kMaxPerLane; i++) {
-            int d = lane + i * 64;
-            if (d < D) {
-                x[i] = load_scalar(src, src_off + d, p.kv_dtype);
-                mn = fminf(mn, x[i]);
-                mx = fmaxf(mx, x[i]);
-            } else {
-                x[i] = 0.0f;
-            }
-        }
-        if (p.cache_dtype == HIPATTN_U8) {
-            mn = wave_min(mn);
-            mx = wave_max(mx);
-            float scale = (mx - mn) / 255.0f;
-            if (scale == 0.0f) scale = 0.0001f;
-            const float zp = -mn / scale + 0.0f;  // -0 becomes +0
-            const float inv = 1.0f / scale;
-            if (lane == 0) {
-                ((float*)row)[0] = scale;
-                ((float*)row)[1] = zp;
-            }
-#pragma unroll
-            for (int i = 0; i < kMaxPerLane; i++) {
-                int d = lane + i * 64;
-                if (d < D) {
-                    float q = rintf(fmaf(x[i], inv, zp));
-                    q = fminf(fmaxf(q, 0.0f), 255.0f);
-                    row[8 + d] = (uint8_t)q;
-                }
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < kMaxPerLane; i++) {
-                int d = lane + i * 64;
-                if (d < D) store_scalar(row, d, p.cache_dtype, x[i]);
-            }
-        }
-    }
+__global__ __launch_bounds__(256) void kv_cache_write_kernel(KvWriteParams p) {
+    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);  // (token, kv head) pair of this wavefront
+    if (pair >= p.num_tokens * p.num_heads_kv) return;
+    kv_cache_write_pair<kMaxPerLane>(p, pair / p.num_heads_kv, pair % p.num_heads_kv, threadIdx.x & 63);
 }
 
 hipError_t launch_kv_cache_write(const KvWriteParams& p, hipStream_t stream) {
     if (p.num_tokens == 0 || p.num_seqs == 0) return hipSuccess;
-    dim3 grid(p.num_tokens, p.num_heads_kv);
+    const int64_t pairs = (int64_t)p.num_tokens * p.num_heads_kv;
+    dim3 grid((unsigned)((pairs + 3) / 4));
     if (p.head_dim <= 128)
-        hipLaunchKernelGGL(kv_cache_write_kernel<2>, grid, dim3(64), 0, stream, p);
+        hipLaunchKernelGGL(kv_cache_write_kernel<2>, grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL(kv_cache_write_kernel<8>, grid, dim3(64), 0, stream, p);
+        hipLaunchKernelGGL(kv_cache_write_kernel<8>, grid, dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -1,14 +1,25 @@
-// Split-context paged-attention decode for gfx950 (one new token per sequence).
+// Paged-attention decode for gfx950 (sequences with exactly one new token), scheduled
+// stream-K style over the whole batch.
 //
-// Work decomposition: grid (chunk, kv head, sequence).  A workgroup of four wavefronts owns
-// `chunk_tokens` consecutive cache positions of one kv head of one sequence and serves the
-// whole GQA group (all query heads sharing that kv head, up to 16) so that every KV byte is
-// read from HBM exactly once.  Wavefront w walks the chunk's 32-token blocks w, w+4, ...;
-// per block it reads the block-table entry, streams the 8 KiB (fp16) or 4352 B (u8) of K and
-// of V for this head straight from global memory into MFMA operand registers, and keeps an
-// online softmax.  Partial (max, sum, output) triples are merged across the four wavefronts
-// in LDS and, when the context spans several chunks, across chunks by paged_merge_kernel
-// (a log-sum-exp reduction).
+// Work decomposition.  The unit of work is one 32-token cache block of one kv head of one
+// sequence ("block-head": 8 KiB of K plus 8 KiB of V in fp16, 2 x 4352 B in u8).  All
+// block-heads of the batch are laid out on one line, ordered (sequence, kv head, block), and
+// the line is cut into `num_waves` equal pieces; wavefront w owns piece w.  The kernel is
+// launched with exactly as many single-wavefront workgroups as fit on the device at once, so
+// every wavefront streams the same number of bytes and they all finish together: no tail, no
+// per-chunk launch cost, no dependence on how the contexts happen to be distributed.  A piece
+// that covers a whole (sequence, kv head) segment writes the final output rows; otherwise the
+// wavefront leaves a partial (running max, sum, unnormalised output) per query head in the
+// workspace and paged_merge_kernel combines the pieces of a segment with a log-sum-exp
+// reduction.  The
+// per-sequence block counts and their prefix sum come from the plan workgroup of the prologue
+// kernel, which reads past_lens / subsequence_begins on the device: the host never sees the
+// lengths.  The same launch performs the operator's KV-cache write.
+//
+// One wavefront serves the whole GQA group (all query heads sharing the kv head, up to 16),
+// so every KV byte is read from HBM exactly once.  Per block it streams K and V straight from
+// global memory into MFMA operand registers (two register stages: the next block's loads are
+// in flight while the current block is consumed) and keeps an online softmax.
 //
 // MFMA use (v_mfma_f32_16x16x32_f16).  Scores are computed transposed, S^T = K Q^T, with the
 // 16 tokens of a tile on the M side and the (padded) 16 query heads on the N side; the
@@ -32,13 +43,12 @@
 
 #include "device_common.hpp"
 #include "kernels.hpp"
+#include "kv_cache_write.hpp"
 
 namespace hipattn {
 
-constexpr int kD = 128;           // head size of the fast path
-constexpr int kBS = 32;           // cache block size of the fast path
-constexpr int kDecodeWaves = 4;
-constexpr int kDecodeThreads = 64 * kDecodeWaves;
+constexpr int kD = 128;   // head size of the fast path
+constexpr int kBS = 32;   // cache block size of the fast path
 
 struct DecodeRange {
     int valid;        // sequence is a decode sequence with something to attend
@@ -46,10 +56,10 @@ struct DecodeRange {
     int ctx;          // attended positions end (exclusive)
     int j0;           // attended positions begin
     int first_block;  // logical block holding j0
-    int end_block;    // one past the logical block holding ctx - 1
+    int nb;           // number of logical blocks attended (0 when not valid)
 };
 
-// Range of cache positions a decode sequence attends; shared by the decode and merge kernels.
+// Range of cache positions a decode sequence attends; shared by the plan, decode and merge kernels.
 __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int s) {
     DecodeRange r;
     const int t0 = p.subsequence_begins[s];
@@ -61,7 +71,7 @@ __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int s)
     if (p.sliding_window > 0 && r.ctx - p.sliding_window > 0) r.j0 = r.ctx - p.sliding_window;
     if (r.ctx <= 0) r.valid = 0;
     r.first_block = r.j0 / p.block_size;
-    r.end_block = (r.ctx + p.block_size - 1) / p.block_size;
+    r.nb = r.valid ? (r.ctx + p.block_size - 1) / p.block_size - r.first_block : 0;
     return r;
 }
 
@@ -251,194 +261,294 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
     }
 }
 
-template <bool kU8>
-__global__ __launch_bounds__(kDecodeThreads) void paged_decode_kernel(PagedParams p) {
-    __shared__ float o_lds[kDecodeWaves][16][kD + 4];
-    __shared__ float ml_lds[kDecodeWaves][2][16];
 
-    const int chunk = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
-    const DecodeRange rg = decode_range(p, s);
-    if (!rg.valid) return;
-    const int blocks_per_chunk = p.chunk_tokens / kBS;
-    const int b_begin = rg.first_block + chunk * blocks_per_chunk;
-    if (b_begin >= rg.end_block) return;
-    const int b_end = min(b_begin + blocks_per_chunk, rg.end_block);
-    const int n_chunks = (rg.end_block - rg.first_block + blocks_per_chunk - 1) / blocks_per_chunk;
-
+// ---- plan ----------------------------------------------------------------------------------
+// Exclusive prefix sums over the sequences of (a) attended blocks of decode sequences and
+// (b) 128-row query tiles of multi-token sequences.  One workgroup; sequences are split evenly
+// over the threads.
+__device__ __forceinline__ void plan_block(const PagedParams& p) {
+    __shared__ int part_blk[256];
+    __shared__ int part_tile[256];
     const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int lane = tid & 63, n16 = lane & 15, kg = lane >> 4;
-    const int G = p.num_heads_q / p.num_heads_kv;
-    const float c = p.scale * kLog2e;
+    const int per = (p.num_seqs + 255) / 256;
+    const int s0 = min(tid * per, p.num_seqs), s1 = min(s0 + per, p.num_seqs);
+    int blk = 0, tile = 0;
+    for (int s = s0; s < s1; s++) {
+        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
+        blk += decode_range(p, s).nb;
+        tile += qlen > 1 ? (qlen + 127) / 128 : 0;
+    }
+    part_blk[tid] = blk;
+    part_tile[tid] = tile;
+    __syncthreads();
+    if (tid == 0) {
+        int rb = 0, rt = 0;
+        for (int i = 0; i < 256; i++) {
+            const int vb = part_blk[i], vt = part_tile[i];
+            part_blk[i] = rb;
+            part_tile[i] = rt;
+            rb += vb;
+            rt += vt;
+        }
+    }
+    __syncthreads();
+    blk = part_blk[tid];
+    tile = part_tile[tid];
+    for (int s = s0; s < s1; s++) {
+        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
+        p.blk_prefix[s] = blk;
+        p.tile_prefix[s] = tile;
+        blk += decode_range(p, s).nb;
+        tile += qlen > 1 ? (qlen + 127) / 128 : 0;
+    }
+    if (s1 == p.num_seqs && s0 < p.num_seqs) {
+        p.blk_prefix[p.num_seqs] = blk;
+        p.tile_prefix[p.num_seqs] = tile;
+    }
+}
 
-    // Q^T operand: lane (head n16, kg) holds Q[head][kg*32 + i*8 .. +8]; padding heads are zero
-    half8_t qf[4];
-    float sumq = 0.0f;
-    {
-        const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kD;
+// One launch for step 1 of the operator and the schedule: workgroups [0, write_blocks) scatter
+// the new K/V rows into the caches (four (token, kv head) pairs each), workgroup write_blocks
+// plans.  The plan reads lengths only, never the cache, so the two parts do not interact.
+__global__ __launch_bounds__(256) void paged_prologue_kernel(KvWriteParams wp, PagedParams p, int write_blocks) {
+    if ((int)blockIdx.x < write_blocks) {
+        const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+        if (pair < wp.num_tokens * wp.num_heads_kv)
+            kv_cache_write_pair<2>(wp, pair / wp.num_heads_kv, pair % wp.num_heads_kv, threadIdx.x & 63);
+    } else {
+        plan_block(p);
+    }
+}
+
+// Largest s in [0, n) with prefix[s] <= x; requires prefix[0] <= x.  64-ary search: every round
+// is one vector load and one ballot, so a batch of 4096 sequences needs two rounds.
+__device__ __forceinline__ int locate_sequence(const int32_t* __restrict__ prefix, int n, int x, int lane) {
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        const int step = (hi - lo + 63) / 64;
+        const int idx = lo + lane * step;
+        const bool ok = idx < hi && prefix[idx] <= x;
+        const int k = __builtin_popcountll(__builtin_amdgcn_ballot_w64(ok)) - 1;  // prefix is monotone
+        lo = lo + k * step;
+        hi = min(hi, lo + step);
+    }
+    return lo;
+}
+
+// First block-head of wavefront w's piece.
+__device__ __forceinline__ int64_t piece_begin(int w, int64_t total, int num_waves) {
+    return (int64_t)w * total / num_waves;
+}
+
+// eight consecutive output elements, one 16-byte store for the 16-bit types
+__device__ __forceinline__ void store_out8(void* out, int64_t elem, int dtype, const float (&o)[8]) {
+    if (dtype == HIPATTN_F32) {
+        float* po = (float*)out + elem;
+        *(float4*)(po) = make_float4(o[0], o[1], o[2], o[3]);
+        *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
+        return;
+    }
+    uint4_t w;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            if (n16 < G) {
-                qf[i] = load_q8(p.q, qrow + kg * 32 + i * 8, p.q_dtype);
-            } else {
+    for (int i = 0; i < 4; i++) {
+        const uint32_t lo = dtype == HIPATTN_F16 ? float_to_f16_bits(o[2 * i]) : float_to_bf16_bits(o[2 * i]);
+        const uint32_t hi = dtype == HIPATTN_F16 ? float_to_f16_bits(o[2 * i + 1]) : float_to_bf16_bits(o[2 * i + 1]);
+        w[i] = lo | (hi << 16);
+    }
+    *(uint4_t*)((uint16_t*)out + elem) = w;
+}
+
+// Log-sum-exp reduction of the partials that pieces w_first..w_last left for query head g of
+// segment (s, h), done by one wavefront.  Pieces are taken 64 at a time: lane i fetches the
+// (max, sum) pair of piece i, the weights come out of two wavefront reductions, and the output
+// rows are then accumulated with independent loads (lane l owns head-dim 2l and 2l + 1).
+__device__ __forceinline__ void merge_segment_head(const PagedParams& p, int s, int h, int g, int token, int w_first,
+                                                   int w_last, int64_t total, int lane) {
+    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv, W = p.num_waves;
+    const bool sparse = total < W;  // only then can a piece be empty
+    float m_run = -INFINITY, l_run = 0.0f, ox = 0.0f, oy = 0.0f;
+    for (int w0 = w_first; w0 <= w_last; w0 += 64) {
+        const int w = w0 + lane;
+        bool have = w <= w_last;
+        if (have && sparse) have = piece_begin(w, total, W) < piece_begin(w + 1, total, W);
+        const int64_t slot = (int64_t)w + (int64_t)s * Hkv + h;
+        float mw = -INFINITY, lw = 0.0f;
+        if (have) {
+            const float2 ml = *(const float2*)(p.part_ml + (slot * G + g) * 2);
+            mw = ml.x;
+            lw = ml.y;
+        }
+        const float m_new = fmaxf(m_run, wave_max(mw));
+        const float rescale = (m_run == -INFINITY) ? 0.0f : fast_exp2(m_run - m_new);
+        const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - m_new);
+        l_run = l_run * rescale + wave_sum(f * lw);
+        ox *= rescale;
+        oy *= rescale;
+        m_run = m_new;
+        const uint64_t live = __builtin_amdgcn_ballot_w64(have);
+        const int n = min(64, w_last - w0 + 1);
+        for (int i = 0; i < n; i++) {
+            if (!((live >> i) & 1)) continue;
+            const float fi = __shfl(f, i, 64);
+            const int64_t sl = (int64_t)(w0 + i) + (int64_t)s * Hkv + h;
+            const float2 v = *(const float2*)(p.part_out + (sl * G + g) * kD + 2 * lane);
+            ox = fmaf(fi, v.x, ox);
+            oy = fmaf(fi, v.y, oy);
+        }
+    }
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    const int64_t o = ((int64_t)token * p.num_heads_q + (int64_t)h * G + g) * kD + 2 * lane;
+    if (p.out_dtype == HIPATTN_F32) {
+        *(float2*)((float*)p.out + o) = make_float2(ox * inv, oy * inv);
+    } else {
+        const uint32_t lo = p.out_dtype == HIPATTN_F16 ? float_to_f16_bits(ox * inv) : float_to_bf16_bits(ox * inv);
+        const uint32_t hi = p.out_dtype == HIPATTN_F16 ? float_to_f16_bits(oy * inv) : float_to_bf16_bits(oy * inv);
+        *(uint32_t*)((uint16_t*)p.out + o) = lo | (hi << 16);
+    }
+}
+
+template <bool kU8>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p) {
+    const int w = blockIdx.x;
+    const int lane = threadIdx.x, n16 = lane & 15, kg = lane >> 4;
+    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
+    const float c = p.scale * kLog2e;
+    const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
+    int64_t L = piece_begin(w, total, p.num_waves);
+    const int64_t L_end = piece_begin(w + 1, total, p.num_waves);
+    if (L >= L_end) return;
+
+    constexpr int64_t kRowBytes = kU8 ? (kD + 8) : (2 * kD);
+    const int64_t block_stride = (int64_t)Hkv * kBS * kRowBytes;
+    int s = locate_sequence(p.blk_prefix, p.num_seqs, (int)(L / Hkv), lane);
+
+    while (L < L_end) {
+        while (s + 1 < p.num_seqs && (int64_t)p.blk_prefix[s + 1] * Hkv <= L) s++;  // next sequence with blocks
+        const DecodeRange rg = decode_range(p, s);
+        const int nb = rg.nb;
+        if (nb <= 0) break;  // cannot happen for a consistent plan; never loop forever
+        const int64_t seq_L0 = (int64_t)p.blk_prefix[s] * Hkv;
+        const int h = (int)((L - seq_L0) / nb);
+        const int b_rel = (int)((L - seq_L0) % nb);
+        const int64_t seg_L1 = seq_L0 + (int64_t)(h + 1) * nb;
+        const int n = (int)(min(L_end, seg_L1) - L);  // blocks of this segment in this piece
+        const bool whole = (b_rel == 0) && (L + n == seg_L1);
+        const int lb0 = rg.first_block + b_rel;        // first logical block
+        const int32_t* table = p.block_indices + p.block_indices_begins[s] + lb0;
+        const int64_t head_off = (int64_t)h * kBS * kRowBytes;
+
+        // Q^T operand: lane (head n16, kg) holds Q[head][kg*32 + i*8 .. +8]; padding heads are zero
+        half8_t qf[4];
+        float sumq = 0.0f;
+        {
+            const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kD;
 #pragma unroll
-                for (int e = 0; e < 8; e++) qf[i][e] = (half_t)0.0f;
+            for (int i = 0; i < 4; i++) {
+                if (n16 < G) {
+                    qf[i] = load_q8(p.q, qrow + kg * 32 + i * 8, p.q_dtype);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) qf[i][e] = (half_t)0.0f;
+                }
+                if constexpr (kU8) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) sumq += (float)qf[i][e];
+                }
             }
             if constexpr (kU8) {
-#pragma unroll
-                for (int e = 0; e < 8; e++) sumq += (float)qf[i][e];
+                sumq += __shfl_xor(sumq, 16, 64);
+                sumq += __shfl_xor(sumq, 32, 64);
             }
         }
+
+        WaveState st;
+        st.m = -INFINITY;
+        st.l = 0.0f;
+        st.corr = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) st.acc[e] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+        // blocks in groups of 64: one vector load fetches the group's block-table entries
+        for (int g0 = 0; g0 < n; g0 += 64) {
+            const int gn = min(64, n - g0);
+            const int my_pb = lane < gn ? table[g0 + lane] : -1;
+            auto issue = [&](BlockRegs<kU8>& regs, int i) -> bool {
+                const int pb = __builtin_amdgcn_readlane(my_pb, i);
+                if (pb < 0 || pb >= p.num_blocks) return false;  // never read outside the cache
+                const int64_t off = (int64_t)pb * block_stride + head_off;
+                load_block<kU8>(regs, p.key_cache + off, p.value_cache + off, n16, kg);
+                return true;
+            };
+            // two register stages: block i+1 is in flight while block i is consumed
+            BlockRegs<kU8> ra, rb;
+            bool ok_a = issue(ra, 0), ok_b = false;
+            int i = 0;
+            while (i < gn) {
+                ok_b = (i + 1 < gn) ? issue(rb, i + 1) : false;
+                if (ok_a) process_block<kU8>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
+                if (i + 1 >= gn) break;
+                ok_a = (i + 2 < gn) ? issue(ra, i + 2) : false;
+                if (ok_b) process_block<kU8>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
+                i += 2;
+            }
+        }
+
+        // ---- this wavefront's result for the segment
+        float l = st.l, corr = st.corr;
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
         if constexpr (kU8) {
-            sumq += __shfl_xor(sumq, 16, 64);
-            sumq += __shfl_xor(sumq, 32, 64);
+            corr += __shfl_xor(corr, 16, 64);
+            corr += __shfl_xor(corr, 32, 64);
         }
-    }
-
-    WaveState st;
-    st.m = -INFINITY;
-    st.l = 0.0f;
-    st.corr = 0.0f;
+        const int64_t slot = (int64_t)w + (int64_t)s * Hkv + h;  // unique per (piece, segment)
+        if (n16 < G) {
+            const float inv = whole ? (l > 0.0f ? 1.0f / l : 0.0f) : 1.0f;
+            // acc[e][r] is head-dim (kg*4 + r)*8 + e: eight consecutive outputs per r
 #pragma unroll
-    for (int e = 0; e < 8; e++) st.acc[e] = (float4_t){0.f, 0.f, 0.f, 0.f};
-
-    const int32_t* table = p.block_indices + p.block_indices_begins[s];
-    constexpr int64_t kRowBytes = kU8 ? (kD + 8) : (2 * kD);
-    const int64_t block_stride = (int64_t)p.num_heads_kv * kBS * kRowBytes;
-    const int64_t head_off = (int64_t)h * kBS * kRowBytes;
-
-    auto block_ptrs = [&](int lb, const uint8_t*& kb, const uint8_t*& vb) -> bool {
-        const int pb = table[lb];
-        if (pb < 0 || pb >= p.num_blocks) return false;  // never read outside the cache
-        const int64_t off = (int64_t)pb * block_stride + head_off;
-        kb = p.key_cache + off;
-        vb = p.value_cache + off;
-        return true;
-    };
-
-    // two register stages: the loads of block i+4 are in flight while block i is consumed
-    BlockRegs<kU8> ra, rb;
-    const uint8_t *kb = nullptr, *vb = nullptr;
-    int lb = b_begin + wave;
-    bool va = false, vb_ok = false;
-    if (lb < b_end) {
-        va = block_ptrs(lb, kb, vb);
-        if (va) load_block<kU8>(ra, kb, vb, n16, kg);
-    }
-    while (lb < b_end) {
-        const int lb_next = lb + kDecodeWaves;
-        vb_ok = false;
-        if (lb_next < b_end) {
-            vb_ok = block_ptrs(lb_next, kb, vb);
-            if (vb_ok) load_block<kU8>(rb, kb, vb, n16, kg);
-        }
-        if (va) process_block<kU8>(st, ra, qf, sumq, c, lb * kBS, rg.j0, rg.ctx, kg);
-        if (lb_next >= b_end) break;
-        const int lb_next2 = lb_next + kDecodeWaves;
-        va = false;
-        if (lb_next2 < b_end) {
-            va = block_ptrs(lb_next2, kb, vb);
-            if (va) load_block<kU8>(ra, kb, vb, n16, kg);
-        }
-        if (vb_ok) process_block<kU8>(st, rb, qf, sumq, c, lb_next * kBS, rg.j0, rg.ctx, kg);
-        lb = lb_next2;
-    }
-
-    // ---- merge the four wavefronts through LDS
-    float l = st.l, corr = st.corr;
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    if constexpr (kU8) {
-        corr += __shfl_xor(corr, 16, 64);
-        corr += __shfl_xor(corr, 32, 64);
-    }
-    if (kg == 0) {
-        ml_lds[wave][0][n16] = st.m;
-        ml_lds[wave][1][n16] = l;
-    }
+            for (int r = 0; r < 4; r++) {
+                float o[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            float v = st.acc[e][r];
-            if constexpr (kU8) v -= corr;
-            o_lds[wave][n16][(kg * 4 + r) * 8 + e] = v;
-        }
-    __syncthreads();
-
-    // thread -> (head g, 8 consecutive head-dim slots)
-    for (int item = tid; item < G * (kD / 8); item += kDecodeThreads) {
-        const int g = item / (kD / 8), d0 = (item % (kD / 8)) * 8;
-        float mt = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < kDecodeWaves; w++) mt = fmaxf(mt, ml_lds[w][0][g]);
-        float lt = 0.0f;
-        float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w = 0; w < kDecodeWaves; w++) {
-            const float mw = ml_lds[w][0][g];
-            const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - mt);
-            lt += f * ml_lds[w][1][g];
-#pragma unroll
-            for (int e = 0; e < 8; e++) o[e] += f * o_lds[w][g][d0 + e];
-        }
-        const int hq = h * G + g;
-        if (n_chunks == 1) {
-            const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
-            const int64_t orow = ((int64_t)rg.token * p.num_heads_q + hq) * kD + d0;
-#pragma unroll
-            for (int e = 0; e < 8; e++) store_scalar(p.out, orow + e, p.out_dtype, o[e] * inv);
-        } else {
-            const int64_t slot = ((int64_t)s * p.num_heads_q + hq) * p.max_chunks + chunk;
-            float* po = p.part_out + slot * kD + d0;
-            *(float4*)(po) = make_float4(o[0], o[1], o[2], o[3]);
-            *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
-            if (d0 == 0) {
-                p.part_ml[slot * 2] = mt;
-                p.part_ml[slot * 2 + 1] = lt;
+                for (int e = 0; e < 8; e++) {
+                    float v = st.acc[e][r];
+                    if constexpr (kU8) v -= corr;
+                    o[e] = v * inv;
+                }
+                const int d0 = (kg * 4 + r) * 8;
+                if (whole) {
+                    store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * kD + d0, p.out_dtype, o);
+                } else {
+                    float* po = p.part_out + (slot * G + n16) * kD + d0;
+                    *(float4*)(po) = make_float4(o[0], o[1], o[2], o[3]);
+                    *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
+                }
+            }
+            if (!whole && kg == 0) {
+                p.part_ml[(slot * G + n16) * 2] = st.m;
+                p.part_ml[(slot * G + n16) * 2 + 1] = l;
             }
         }
+        L += n;
     }
 }
 
-// Log-sum-exp reduction of the per-chunk partials of one (sequence, query head).
-__global__ __launch_bounds__(kD) void paged_merge_kernel(PagedParams p) {
-    const int hq = blockIdx.x, s = blockIdx.y;
+// Combines the partials of every (sequence, kv head) segment that more than one piece worked
+// on.  A separate launch: the kernel boundary is what makes the partials visible, which is far
+// cheaper here than device-scope fences inside the streaming kernel (those write back and
+// invalidate whole L2 caches and cost the decode kernel almost half of its bandwidth).
+__global__ __launch_bounds__(256) void paged_merge_kernel(PagedParams p) {
+    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
+    const int s = blockIdx.x / Hkv, h = blockIdx.x % Hkv;  // one workgroup per segment
     const DecodeRange rg = decode_range(p, s);
-    if (!rg.valid) return;
-    const int blocks_per_chunk = p.chunk_tokens / kBS;
-    int n_chunks = (rg.end_block - rg.first_block + blocks_per_chunk - 1) / blocks_per_chunk;
-    if (n_chunks <= 1) return;  // the decode kernel already wrote the final row
-    if (n_chunks > p.max_chunks) n_chunks = p.max_chunks;  // caller understated max_context_len: stay in bounds
-    const int d = threadIdx.x;
-    const int64_t slot0 = ((int64_t)s * p.num_heads_q + hq) * p.max_chunks;
-    float mt = -INFINITY;
-    for (int ch = 0; ch < n_chunks; ch++) mt = fmaxf(mt, p.part_ml[(slot0 + ch) * 2]);
-    float lt = 0.0f, o = 0.0f;
-    for (int ch = 0; ch < n_chunks; ch++) {
-        const float f = fast_exp2(p.part_ml[(slot0 + ch) * 2] - mt);
-        lt += f * p.part_ml[(slot0 + ch) * 2 + 1];
-        o += f * p.part_out[(slot0 + ch) * kD + d];
-    }
-    const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
-    store_scalar(p.out, ((int64_t)rg.token * p.num_heads_q + hq) * kD + d, p.out_dtype, o * inv);
-}
-
-hipError_t launch_paged_decode(const PagedParams& p, hipStream_t stream, const KernelProbe& probe) {
-    dim3 grid(p.max_chunks, p.num_heads_kv, p.num_seqs);
-    if (probe.before) (void)hipEventRecord(probe.before, stream);
-    if (p.cache_dtype == HIPATTN_U8)
-        hipLaunchKernelGGL(paged_decode_kernel<true>, grid, dim3(kDecodeThreads), 0, stream, p);
-    else
-        hipLaunchKernelGGL(paged_decode_kernel<false>, grid, dim3(kDecodeThreads), 0, stream, p);
-    hipError_t e = hipGetLastError();
-    if (probe.after) (void)hipEventRecord(probe.after, stream);
-    if (e != hipSuccess) return e;
-    if (p.max_chunks > 1) {
-        hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_heads_q, p.num_seqs), dim3(kD), 0, stream, p);
-        e = hipGetLastError();
-    }
-    return e;
+    if (rg.nb <= 0) return;
+    const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
+    if (total <= 0) return;
+    const int64_t L0 = (int64_t)p.blk_prefix[s] * Hkv + (int64_t)h * rg.nb, L1 = L0 + rg.nb;
+    const int w_first = (int)(((L0 + 1) * p.num_waves - 1) / total);  // piece holding block-head L0
+    const int w_last = (int)((L1 * p.num_waves - 1) / total);        // piece holding block-head L1 - 1
+    if (w_first >= w_last) return;  // a single piece covered the segment and wrote the final rows
+    for (int g = threadIdx.x >> 6; g < G; g += 4)  // one wavefront per query head of the group
+        merge_segment_head(p, s, h, g, rg.token, w_first, w_last, total, threadIdx.x & 63);
 }
 
 // ---- host side of the fast path ---------------------------------------------------------
@@ -450,59 +560,77 @@ bool paged_fast_supported(const PagedParams& p) {
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_U8);
 }
 
-// Largest number of 32-token blocks a decode sequence can attend.
-static int max_decode_blocks(const PagedParams& p) {
-    int blocks = (p.max_context_len + kBS - 1) / kBS;
-    if (p.sliding_window > 0) blocks = std::min(blocks, (p.sliding_window + kBS - 1) / kBS + 1);
-    return std::max(blocks, 1);
+// Wavefronts the decode kernel keeps resident: it needs up to 256 registers per lane, i.e. two
+// wavefronts per SIMD, eight per compute unit.
+static int resident_decode_waves() {
+    static thread_local int cached_device = -1, cached_waves = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 2048;
+    if (dev != cached_device) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        cached_device = dev;
+        cached_waves = cus * 8;
+    }
+    return cached_waves;
 }
 
-// Tokens per split: enough workgroups to fill 256 CUs several times over while keeping the
-// partial-result traffic (520 B per query head and split) small against the KV bytes read.
-static int choose_chunk_tokens(const PagedParams& p) {
-    if (p.chunk_tokens > 0) return std::max(kBS, (p.chunk_tokens / kBS) * kBS);
-    const int64_t total_blocks = (int64_t)p.num_seqs * p.num_heads_kv * max_decode_blocks(p);
-    const int min_chunk = (p.cache_dtype == HIPATTN_U8) ? 1024 : 512;
-    int chunk = 4096;
-    while (chunk > min_chunk && total_blocks * kBS / chunk < 4096) chunk >>= 1;
-    while (chunk > 128 && total_blocks * kBS / chunk < 512) chunk >>= 1;
-    return chunk;
+static int choose_num_waves(const PagedParams& p) {
+    if (p.num_waves > 0) return p.num_waves;
+    return resident_decode_waves();
 }
 
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 size_t paged_fast_workspace_bytes(const PagedParams& p) {
-    const int chunk = choose_chunk_tokens(p);
-    const int max_chunks = (max_decode_blocks(p) * kBS + chunk - 1) / chunk;
-    size_t bytes = align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
-    if (max_chunks > 1) {
-        const size_t slots = (size_t)p.num_seqs * p.num_heads_q * max_chunks;
-        bytes += align_up(slots * kD * sizeof(float), 256) + align_up(slots * 2 * sizeof(float), 256);
-    }
-    return bytes;
+    const int W = choose_num_waves(p);
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const size_t slots = (size_t)W + (size_t)p.num_seqs * p.num_heads_kv;
+    return 2 * align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256) +
+           align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
 }
 
 void paged_fast_plan(PagedParams& p, void* workspace) {
-    p.chunk_tokens = choose_chunk_tokens(p);
-    p.max_chunks = (max_decode_blocks(p) * kBS + p.chunk_tokens - 1) / p.chunk_tokens;
+    p.num_waves = choose_num_waves(p);
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const size_t slots = (size_t)p.num_waves + (size_t)p.num_seqs * p.num_heads_kv;
     uint8_t* w = (uint8_t*)workspace;
     p.tile_prefix = (int32_t*)w;
     w += align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
-    p.part_out = nullptr;
-    p.part_ml = nullptr;
-    if (p.max_chunks > 1) {
-        const size_t slots = (size_t)p.num_seqs * p.num_heads_q * p.max_chunks;
-        p.part_out = (float*)w;
-        w += align_up(slots * kD * sizeof(float), 256);
-        p.part_ml = (float*)w;
-    }
+    p.blk_prefix = (int32_t*)w;
+    w += align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
+    p.part_out = (float*)w;
+    w += align_up(slots * G * kD * sizeof(float), 256);
+    p.part_ml = (float*)w;
     // query tiles of multi-token sequences: each has >= 2 tokens and wastes at most one tile
     const int multi = std::min(p.num_seqs, p.num_tokens / 2);
-    p.max_q_tiles = p.num_tokens / 128 + multi;
+    // one token per sequence: a pure decode batch, no query tiles at all
+    p.max_q_tiles = (p.num_tokens == p.num_seqs) ? 0 : p.num_tokens / 128 + multi;
 }
 
-hipError_t launch_paged_fast(const PagedParams& p, hipStream_t stream, const KernelProbe& probe) {
-    hipError_t e = launch_paged_decode(p, stream, probe);
+hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
+                             const KernelProbe& probe) {
+    // prologue: KV-cache write of the new tokens (optional) + plan, one launch
+    KvWriteParams wp{};
+    int write_blocks = 0;
+    if (write) {
+        wp = *write;
+        if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head_dim 128 only
+        write_blocks = (int)(((int64_t)wp.num_tokens * wp.num_heads_kv + 3) / 4);
+    }
+    hipLaunchKernelGGL(paged_prologue_kernel, dim3(write_blocks + 1), dim3(256), 0, stream, wp, p, write_blocks);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (probe.before) (void)hipEventRecord(probe.before, stream);
+    if (p.cache_dtype == HIPATTN_U8)
+        hipLaunchKernelGGL(paged_decode_kernel<true>, dim3(p.num_waves), dim3(64), 0, stream, p);
+    else
+        hipLaunchKernelGGL(paged_decode_kernel<false>, dim3(p.num_waves), dim3(64), 0, stream, p);
+    e = hipGetLastError();
+    if (probe.after) (void)hipEventRecord(probe.after, stream);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_seqs * p.num_heads_kv), dim3(256), 0, stream, p);
+    e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.max_q_tiles > 0) {
         if (p.cache_dtype == HIPATTN_U8) {

@@ -160,15 +160,16 @@ def make_paged_case(seed, seqs, Hq, Hkv, D, block_size, q_dtype, kv_dtype, cache
     }
 
 
-def paged_kv_bytes(case):
-    """Algorithmic KV bytes of the call: every attended (position, kv head) row of K and of V once."""
+def paged_kv_bytes(case, decode_only=False):
+    """Algorithmic KV bytes of the call: every attended (position, kv head) row of K and of V once.
+    decode_only restricts the sum to sequences with exactly one new token."""
     W = case["sliding_window"]
     rb = cache_row_bytes(case["cache_dtype"], case["D"])
     total = 0
     for s in range(case["S"]):
         past = int(case["past_lens"][s])
         qlen = int(case["subsequence_begins"][s + 1] - case["subsequence_begins"][s])
-        if qlen <= 0:
+        if qlen <= 0 or (decode_only and qlen != 1):
             continue
         ctx = past + qlen
         lo = max(0, past - W + 1) if W > 0 else 0  # first position any token of the sequence attends

@@ -147,13 +147,13 @@ DECODE_CTX = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 500, 511, 512, 513, 1
 
 @pytest.mark.parametrize("cache_dtype,q_dtype,Hq", [(W.F16, W.F16, 32), (W.F16, W.BF16, 8), (W.U8, W.F16, 64),
                                                     (W.U8, W.BF16, 16), (W.F16, W.F16, 128)])
-@pytest.mark.parametrize("chunk", [0, 128, 256])
-def test_paged_decode(hip, oracle, cache_dtype, q_dtype, Hq, chunk):
-    announce("paged decode", cache_dtype, q_dtype, Hq, chunk)
+@pytest.mark.parametrize("waves", [0, 5, 100, 3000])
+def test_paged_decode(hip, oracle, cache_dtype, q_dtype, Hq, waves):
+    announce("paged decode", cache_dtype, q_dtype, Hq, waves)
     seqs = [(c - 1, 1) for c in DECODE_CTX]
     case = W.make_paged_case(71, seqs, Hq, 8, 128, 32, q_dtype, q_dtype, cache_dtype)
     dev = H.PagedDeviceCase(hip, case)
-    out, path = dev.run(decode_chunk=chunk)
+    out, path = dev.run(decode_waves=waves)
     assert path == "paged_mfma"
     ref, okc, ovc = H.oracle_paged(oracle, case)
     kc, vc = dev.caches()
@@ -176,7 +176,7 @@ def test_paged_decode_sliding_window(hip, oracle, cache_dtype, window):
     seqs = [(c - 1, 1) for c in DECODE_CTX]
     case = W.make_paged_case(72, seqs, 32, 8, 128, 32, W.F16, W.F16, cache_dtype, sliding_window=window)
     dev = H.PagedDeviceCase(hip, case)
-    out, _ = dev.run(decode_chunk=128)
+    out, _ = dev.run(decode_waves=128)
     ref, _, _ = H.oracle_paged(oracle, case)
     assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3)
     dev.free()
@@ -208,7 +208,7 @@ def test_paged_block_permutation_is_bit_identical(hip):
     seqs = [(c - 1, 1) for c in (700, 64, 1500, 33)] + [(100, 200)]
     case = W.make_paged_case(74, seqs, 32, 8, 128, 32, W.F16, W.F16, W.F16)
     dev = H.PagedDeviceCase(hip, case)
-    out, _ = dev.run(decode_chunk=256)
+    out, _ = dev.run(decode_waves=256)
     rng = np.random.default_rng(2)
     perm = rng.permutation(case["num_blocks"])
     case2 = dict(case)
@@ -218,7 +218,7 @@ def test_paged_block_permutation_is_bit_identical(hip):
     case2["key_cache"][perm] = case["key_cache"]
     case2["value_cache"][perm] = case["value_cache"]
     dev2 = H.PagedDeviceCase(hip, case2)
-    out2, _ = dev2.run(decode_chunk=256)
+    out2, _ = dev2.run(decode_waves=256)
     np.testing.assert_array_equal(out, out2)
     dev.free()
     dev2.free()
@@ -232,7 +232,7 @@ def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window):
     seqs = [(0, 130), (37, 1), (500, 1), (100, 257), (0, 2), (999, 1), (31, 97), (64, 1), (700, 128), (5, 0)]
     case = W.make_paged_case(81, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
     dev = H.PagedDeviceCase(hip, case)
-    out, path = dev.run(decode_chunk=128)
+    out, path = dev.run(decode_waves=128)
     assert path == "paged_mfma"
     ref, okc, ovc = H.oracle_paged(oracle, case)
     kc, vc = dev.caches()
@@ -267,7 +267,7 @@ def test_paged_errors(hip):
     announce("paged errors")
     case = W.make_paged_case(83, [(100, 1), (700, 1)], 32, 8, 128, 32, W.F16, W.F16, W.F16)
     dev = H.PagedDeviceCase(hip, case)
-    desc = H.pa_desc(hip, case, decode_chunk=128)
+    desc = H.pa_desc(hip, case, decode_waves=128)
     need = hip.paged_attention_workspace_size(desc)
     assert need > 0
     small = hip.DeviceBuffer(need - 1)
