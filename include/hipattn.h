@@ -149,7 +149,11 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * num_tokens == num_seqs is taken to hold exactly one token per sequence (pure decode). */
 enum {
     HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */
-    HIPATTN_PA_FORCE_GENERIC = 2     /* use the shape-generic kernels (testing aid) */
+    HIPATTN_PA_FORCE_GENERIC = 2,    /* use the shape-generic kernels (testing aid) */
+    HIPATTN_PA_TRACE_WAVES = 4       /* diagnostic: the decode kernel leaves, in the last
+                                        decode_waves * 32 bytes of the workspace, four int64 per
+                                        wavefront: entry, first block consumed, exit (100 MHz
+                                        ticks) and units of work */
 };
 
 typedef struct hipattn_pa_desc {

@@ -69,14 +69,21 @@ struct PagedParams {
     // decode: the batch's block-heads are cut into num_waves equal pieces (one per wavefront);
     // pieces that do not cover a whole (sequence, kv head) segment leave partials in the workspace
     int num_waves;        // wavefronts (= single-wavefront workgroups) of the decode kernel
-    int32_t* blk_prefix;  // [num_seqs + 1] exclusive prefix of attended blocks of decode sequences
-    float* part_out;      // [num_waves + num_seqs*num_heads_kv, G, head_dim] unnormalised outputs
-    float* part_ml;       // [num_waves + num_seqs*num_heads_kv, G, 2] running max (log2 domain) and sum
+    int switch_cost;      // block-times a wavefront is charged for starting on a new segment
+    int dyn_pieces;       // pieces of the last quarter of the work line, handed out on demand
+    int dyn_groups;       // wavefront groups, each with its own ticket counter and every dyn_groups-th piece
+    int32_t* dyn_counter; // [64] ticket counters (zeroed by the plan)
+    int32_t* blk_prefix;  // [num_seqs + 1] exclusive prefix of work-line units of decode sequences
+    void* seq_info;       // [num_seqs] 32-byte records: what each decode sequence attends (written by the plan)
+    float* part_out;      // [num_waves + dyn_pieces + num_seqs*num_heads_kv, G, head_dim] unnormalised outputs
+    float* part_ml;       // [same, G, 2] running max (log2 domain) and sum
     // chunked prefill: query-tile schedule built on the device
     int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
     int max_q_tiles;      // grid upper bound
     // shape-generic kernel only: skip sequences with exactly one token (the decode kernel has them)
     int generic_skip_single;
+    // diagnostic (HIPATTN_PA_TRACE_WAVES): per decode wavefront {entry, first block consumed, exit, line units}
+    int64_t* wave_trace;
 };
 
 // Optional event pair recorded around the dominant kernel of a call (measurement aid).

@@ -40,6 +40,7 @@
 // src/ops/assign.cpp:52-54) and materialises the scores in HBM (src/ops/matmul.cpp:204-226,
 // src/ops/softmax.cpp:184-192).
 #include <algorithm>
+#include <cstdlib>
 
 #include "device_common.hpp"
 #include "kernels.hpp"
@@ -50,16 +51,20 @@ namespace hipattn {
 constexpr int kD = 128;   // head size of the fast path
 constexpr int kBS = 32;   // cache block size of the fast path
 
-struct DecodeRange {
+struct alignas(32) DecodeRange {
     int valid;        // sequence is a decode sequence with something to attend
     int token;        // row of q / out
     int ctx;          // attended positions end (exclusive)
     int j0;           // attended positions begin
     int first_block;  // logical block holding j0
     int nb;           // number of logical blocks attended (0 when not valid)
+    int table_begin;  // offset of the sequence's block table in block_indices
+    int pad;
 };
+static_assert(sizeof(DecodeRange) == 32, "one 32-byte record per sequence");
 
-// Range of cache positions a decode sequence attends; shared by the plan, decode and merge kernels.
+// Range of cache positions a decode sequence attends.  Computed once per call by the plan and
+// stored per sequence (seq_info), so that the decode and merge kernels fetch it with one load.
 __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int s) {
     DecodeRange r;
     const int t0 = p.subsequence_begins[s];
@@ -72,6 +77,8 @@ __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int s)
     if (r.ctx <= 0) r.valid = 0;
     r.first_block = r.j0 / p.block_size;
     r.nb = r.valid ? (r.ctx + p.block_size - 1) / p.block_size - r.first_block : 0;
+    r.table_begin = p.block_indices_begins[s];
+    r.pad = 0;
     return r;
 }
 
@@ -262,6 +269,12 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
 }
 
 
+// Length of one (sequence, kv head) segment on the work line: its blocks plus `switch_cost`
+// units that stand for the time a wavefront loses when it starts on a new segment (dependent
+// loads of the sequence's lengths, its block table and the queries).  Cutting the line into
+// equal pieces then equalises time, not just bytes.
+__device__ __forceinline__ int line_units(int nb, int switch_cost) { return nb > 0 ? nb + switch_cost : 0; }
+
 // ---- plan ----------------------------------------------------------------------------------
 // Exclusive prefix sums over the sequences of (a) attended blocks of decode sequences and
 // (b) 128-row query tiles of multi-token sequences.  One workgroup; sequences are split evenly
@@ -270,12 +283,13 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
     __shared__ int part_blk[256];
     __shared__ int part_tile[256];
     const int tid = threadIdx.x;
+    if (tid < 64) p.dyn_counter[tid] = 0;  // tickets for the dynamic pieces of this call, one counter per group
     const int per = (p.num_seqs + 255) / 256;
     const int s0 = min(tid * per, p.num_seqs), s1 = min(s0 + per, p.num_seqs);
     int blk = 0, tile = 0;
     for (int s = s0; s < s1; s++) {
         const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
-        blk += decode_range(p, s).nb;
+        blk += line_units(decode_range(p, s).nb, p.switch_cost);
         tile += qlen > 1 ? (qlen + 127) / 128 : 0;
     }
     part_blk[tid] = blk;
@@ -298,7 +312,9 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
         const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
         p.blk_prefix[s] = blk;
         p.tile_prefix[s] = tile;
-        blk += decode_range(p, s).nb;
+        const DecodeRange rg = decode_range(p, s);
+        ((DecodeRange*)p.seq_info)[s] = rg;
+        blk += line_units(rg.nb, p.switch_cost);
         tile += qlen > 1 ? (qlen + 127) / 128 : 0;
     }
     if (s1 == p.num_seqs && s0 < p.num_seqs) {
@@ -335,10 +351,29 @@ __device__ __forceinline__ int locate_sequence(const int32_t* __restrict__ prefi
     return lo;
 }
 
-// First block-head of wavefront w's piece.
-__device__ __forceinline__ int64_t piece_begin(int w, int64_t total, int num_waves) {
-    return (int64_t)w * total / num_waves;
-}
+// How the work line [0, total) is cut into pieces.  Pieces 0 .. W-1 are the static ones, one per
+// wavefront, and share the first three quarters of the line equally; pieces W .. W+P-1 share the
+// last quarter and are handed out on demand (an atomic counter), so wavefronts that run faster
+// -- older ones win the arbitration for the memory pipeline, some XCDs see more bandwidth --
+// take more of them and all wavefronts finish together.
+struct Line {
+    int64_t total, t_static, t_dyn;
+    int W, P;
+    __device__ __forceinline__ Line(int64_t total_, int W_, int P_) : total(total_), W(W_), P(P_) {
+        t_dyn = P_ > 0 ? total_ / 4 : 0;
+        t_static = total_ - t_dyn;
+    }
+    // first line unit of piece id (id may be W + P: the end of the line)
+    __device__ __forceinline__ int64_t begin(int id) const {
+        if (id <= W) return (int64_t)id * t_static / W;
+        return t_static + (int64_t)(id - W) * t_dyn / P;
+    }
+    // the (non-empty) piece that holds line unit pos, 0 <= pos < total
+    __device__ __forceinline__ int piece_at(int64_t pos) const {
+        if (pos < t_static) return (int)(((pos + 1) * W - 1) / t_static);
+        return W + (int)(((pos - t_static + 1) * P - 1) / t_dyn);
+    }
+};
 
 // eight consecutive output elements, one 16-byte store for the 16-bit types
 __device__ __forceinline__ void store_out8(void* out, int64_t elem, int dtype, const float (&o)[8]) {
@@ -358,20 +393,18 @@ __device__ __forceinline__ void store_out8(void* out, int64_t elem, int dtype, c
     *(uint4_t*)((uint16_t*)out + elem) = w;
 }
 
-// Log-sum-exp reduction of the partials that pieces w_first..w_last left for query head g of
+// Log-sum-exp reduction of the partials that pieces id_first..id_last left for query head g of
 // segment (s, h), done by one wavefront.  Pieces are taken 64 at a time: lane i fetches the
 // (max, sum) pair of piece i, the weights come out of two wavefront reductions, and the output
 // rows are then accumulated with independent loads (lane l owns head-dim 2l and 2l + 1).
-__device__ __forceinline__ void merge_segment_head(const PagedParams& p, int s, int h, int g, int token, int w_first,
-                                                   int w_last, int64_t total, int lane) {
-    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv, W = p.num_waves;
-    const bool sparse = total < W;  // only then can a piece be empty
+__device__ __forceinline__ void merge_segment_head(const PagedParams& p, const Line& line, int s, int h, int g,
+                                                   int token, int id_first, int id_last, int lane) {
+    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
     float m_run = -INFINITY, l_run = 0.0f, ox = 0.0f, oy = 0.0f;
-    for (int w0 = w_first; w0 <= w_last; w0 += 64) {
-        const int w = w0 + lane;
-        bool have = w <= w_last;
-        if (have && sparse) have = piece_begin(w, total, W) < piece_begin(w + 1, total, W);
-        const int64_t slot = (int64_t)w + (int64_t)s * Hkv + h;
+    for (int id0 = id_first; id0 <= id_last; id0 += 64) {
+        const int id = id0 + lane;
+        const bool have = id <= id_last && line.begin(id) < line.begin(id + 1);  // skip empty pieces
+        const int64_t slot = (int64_t)id + (int64_t)s * Hkv + h;
         float mw = -INFINITY, lw = 0.0f;
         if (have) {
             const float2 ml = *(const float2*)(p.part_ml + (slot * G + g) * 2);
@@ -386,11 +419,11 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, int s, 
         oy *= rescale;
         m_run = m_new;
         const uint64_t live = __builtin_amdgcn_ballot_w64(have);
-        const int n = min(64, w_last - w0 + 1);
+        const int n = min(64, id_last - id0 + 1);
         for (int i = 0; i < n; i++) {
             if (!((live >> i) & 1)) continue;
             const float fi = __shfl(f, i, 64);
-            const int64_t sl = (int64_t)(w0 + i) + (int64_t)s * Hkv + h;
+            const int64_t sl = (int64_t)(id0 + i) + (int64_t)s * Hkv + h;
             const float2 v = *(const float2*)(p.part_out + (sl * G + g) * kD + 2 * lane);
             ox = fmaf(fi, v.x, ox);
             oy = fmaf(fi, v.y, oy);
@@ -414,27 +447,52 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
     const float c = p.scale * kLog2e;
     const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
-    int64_t L = piece_begin(w, total, p.num_waves);
-    const int64_t L_end = piece_begin(w + 1, total, p.num_waves);
-    if (L >= L_end) return;
+    if (total <= 0) return;
+    const Line line(total, p.num_waves, p.dyn_pieces);
+    // diagnostic: entry time, time the first block was consumed, exit time, units done (100 MHz clock)
+    int64_t t_entry = 0, t_first = 0, units_done = 0;
+    int blocks_done = 0;
+    if (p.wave_trace) t_entry = wall_clock64();
 
     constexpr int64_t kRowBytes = kU8 ? (kD + 8) : (2 * kD);
     const int64_t block_stride = (int64_t)Hkv * kBS * kRowBytes;
-    int s = locate_sequence(p.blk_prefix, p.num_seqs, (int)(L / Hkv), lane);
+
+    // The static piece first, then dynamic pieces for as long as there are any.  The ticket for
+    // the next dynamic piece is drawn before the current piece is worked on, so its latency is hidden.
+    // Tickets come from one counter per group of wavefronts (a single counter would serialise
+    // thousands of same-address atomics); group g owns the dynamic pieces g, g + groups, ...
+    // A group mixes wavefronts of every XCD and of both dispatch halves (w / 8 mod groups).
+    const int group = (w >> 3) % p.dyn_groups;
+    int piece = w;
+    for (;;) {
+    int ticket_lane0 = 0;
+    if (p.dyn_pieces > 0 && lane == 0) ticket_lane0 = atomicAdd(p.dyn_counter + group, 1);
+    int64_t L = line.begin(piece);
+    const int64_t L_end = line.begin(piece + 1);
+    units_done += L_end - L;
+    int s = L < L_end ? locate_sequence(p.blk_prefix, p.num_seqs, (int)(L / Hkv), lane) : 0;
 
     while (L < L_end) {
         while (s + 1 < p.num_seqs && (int64_t)p.blk_prefix[s + 1] * Hkv <= L) s++;  // next sequence with blocks
-        const DecodeRange rg = decode_range(p, s);
+        const DecodeRange rg = ((const DecodeRange*)p.seq_info)[s];
         const int nb = rg.nb;
         if (nb <= 0) break;  // cannot happen for a consistent plan; never loop forever
+        const int seglen = nb + p.switch_cost;
         const int64_t seq_L0 = (int64_t)p.blk_prefix[s] * Hkv;
-        const int h = (int)((L - seq_L0) / nb);
-        const int b_rel = (int)((L - seq_L0) % nb);
-        const int64_t seg_L1 = seq_L0 + (int64_t)(h + 1) * nb;
-        const int n = (int)(min(L_end, seg_L1) - L);  // blocks of this segment in this piece
-        const bool whole = (b_rel == 0) && (L + n == seg_L1);
+        const int h = (int)((L - seq_L0) / seglen);
+        const int64_t seg_B0 = seq_L0 + (int64_t)h * seglen + p.switch_cost;  // line position of the segment's block 0
+        const int64_t seg_L1 = seg_B0 + nb;                        // end of the segment
+        const int64_t from = max(L, seg_B0), to = min(L_end, seg_L1);
+        if (from >= to) {  // the piece ends inside the switch-cost units: no block of this segment is ours
+            L = to;
+            continue;
+        }
+        const int b_rel = (int)(from - seg_B0);
+        const int n = (int)(to - from);  // blocks of this segment in this piece
+        const bool whole = (n == nb);
+        L = from;
         const int lb0 = rg.first_block + b_rel;        // first logical block
-        const int32_t* table = p.block_indices + p.block_indices_begins[s] + lb0;
+        const int32_t* table = p.block_indices + rg.table_begin + lb0;
         const int64_t head_off = (int64_t)h * kBS * kRowBytes;
 
         // Q^T operand: lane (head n16, kg) holds Q[head][kg*32 + i*8 .. +8]; padding heads are zero
@@ -486,6 +544,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             while (i < gn) {
                 ok_b = (i + 1 < gn) ? issue(rb, i + 1) : false;
                 if (ok_a) process_block<kU8>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
+                if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
+                blocks_done = 1;
                 if (i + 1 >= gn) break;
                 ok_a = (i + 2 < gn) ? issue(ra, i + 2) : false;
                 if (ok_b) process_block<kU8>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
@@ -501,7 +561,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             corr += __shfl_xor(corr, 16, 64);
             corr += __shfl_xor(corr, 32, 64);
         }
-        const int64_t slot = (int64_t)w + (int64_t)s * Hkv + h;  // unique per (piece, segment)
+        const int64_t slot = (int64_t)piece + (int64_t)s * Hkv + h;  // unique per (piece, segment)
         if (n16 < G) {
             const float inv = whole ? (l > 0.0f ? 1.0f / l : 0.0f) : 1.0f;
             // acc[e][r] is head-dim (kg*4 + r)*8 + e: eight consecutive outputs per r
@@ -530,6 +590,17 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         }
         L += n;
     }
+    if (p.dyn_pieces <= 0) break;
+    const int next = group + __shfl(ticket_lane0, 0, 64) * p.dyn_groups;
+    if (next >= p.dyn_pieces) break;  // this group's share of the line is used up (every wavefront gets here)
+    piece = p.num_waves + next;
+    }
+    if (p.wave_trace && lane == 0) {
+        p.wave_trace[w * 4 + 0] = t_entry;
+        p.wave_trace[w * 4 + 1] = t_first;
+        p.wave_trace[w * 4 + 2] = wall_clock64();
+        p.wave_trace[w * 4 + 3] = units_done;
+    }
 }
 
 // Combines the partials of every (sequence, kv head) segment that more than one piece worked
@@ -539,16 +610,17 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 __global__ __launch_bounds__(256) void paged_merge_kernel(PagedParams p) {
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
     const int s = blockIdx.x / Hkv, h = blockIdx.x % Hkv;  // one workgroup per segment
-    const DecodeRange rg = decode_range(p, s);
+    const DecodeRange rg = ((const DecodeRange*)p.seq_info)[s];
     if (rg.nb <= 0) return;
     const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
     if (total <= 0) return;
-    const int64_t L0 = (int64_t)p.blk_prefix[s] * Hkv + (int64_t)h * rg.nb, L1 = L0 + rg.nb;
-    const int w_first = (int)(((L0 + 1) * p.num_waves - 1) / total);  // piece holding block-head L0
-    const int w_last = (int)((L1 * p.num_waves - 1) / total);        // piece holding block-head L1 - 1
-    if (w_first >= w_last) return;  // a single piece covered the segment and wrote the final rows
+    const Line line(total, p.num_waves, p.dyn_pieces);
+    const int seglen = rg.nb + p.switch_cost;
+    const int64_t L0 = (int64_t)p.blk_prefix[s] * Hkv + (int64_t)h * seglen + p.switch_cost, L1 = L0 + rg.nb;
+    const int id_first = line.piece_at(L0), id_last = line.piece_at(L1 - 1);
+    if (id_first >= id_last) return;  // a single piece covered the segment and wrote the final rows
     for (int g = threadIdx.x >> 6; g < G; g += 4)  // one wavefront per query head of the group
-        merge_segment_head(p, s, h, g, rg.token, w_first, w_last, total, threadIdx.x & 63);
+        merge_segment_head(p, line, s, h, g, rg.token, id_first, id_last, threadIdx.x & 63);
 }
 
 // ---- host side of the fast path ---------------------------------------------------------
@@ -575,33 +647,63 @@ static int resident_decode_waves() {
     return cached_waves;
 }
 
+// fp16 caches stream best with one wavefront per SIMD; the u8 path has more arithmetic per
+// byte and wants both resident wavefronts to cover it.
 static int choose_num_waves(const PagedParams& p) {
     if (p.num_waves > 0) return p.num_waves;
-    return resident_decode_waves();
+    const int resident = resident_decode_waves();
+    return p.cache_dtype == HIPATTN_U8 ? resident : resident / 2;
 }
 
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// On-demand pieces per wavefront for the last quarter of the line.  Off by default: a wavefront
+// that starts on a new piece pays a chain of dependent loads (ticket, sequence, block table,
+// first block) before it streams again, and on MI355X that costs more than the better balance
+// at the end of the kernel wins back.  HIPATTN_DECODE_DYN_PIECES_PER_WAVE switches it on (tuning aid).
+static int choose_dyn_pieces(int num_waves) {
+    const char* e = getenv("HIPATTN_DECODE_DYN_PIECES_PER_WAVE");
+    const int v = e ? atoi(e) : 0;
+    return num_waves * std::min(std::max(v, 0), 64);
+}
+
 size_t paged_fast_workspace_bytes(const PagedParams& p) {
     const int W = choose_num_waves(p);
     const int G = p.num_heads_q / p.num_heads_kv;
-    const size_t slots = (size_t)W + (size_t)p.num_seqs * p.num_heads_kv;
-    return 2 * align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256) +
-           align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
+    const size_t slots = (size_t)W + choose_dyn_pieces(W) + (size_t)p.num_seqs * p.num_heads_kv;
+    return 256 + 2 * align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256) + align_up((size_t)p.num_seqs * 32, 256) +
+           align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256) +
+           (p.wave_trace ? align_up((size_t)W * 4 * sizeof(int64_t), 256) : 0);
+}
+
+// Block-times charged per segment start; HIPATTN_DECODE_SWITCH_COST overrides (tuning aid).
+static int choose_switch_cost() {
+    const char* e = getenv("HIPATTN_DECODE_SWITCH_COST");
+    const int v = e ? atoi(e) : 3;
+    return std::min(std::max(v, 0), 64);
 }
 
 void paged_fast_plan(PagedParams& p, void* workspace) {
     p.num_waves = choose_num_waves(p);
+    p.switch_cost = choose_switch_cost();
+    p.dyn_pieces = choose_dyn_pieces(p.num_waves);
+    p.dyn_groups = std::min(64, std::max(1, p.num_waves / 32));  // every group has at least one wavefront
     const int G = p.num_heads_q / p.num_heads_kv;
-    const size_t slots = (size_t)p.num_waves + (size_t)p.num_seqs * p.num_heads_kv;
+    const size_t slots = (size_t)p.num_waves + p.dyn_pieces + (size_t)p.num_seqs * p.num_heads_kv;
     uint8_t* w = (uint8_t*)workspace;
+    p.dyn_counter = (int32_t*)w;
+    w += 256;
     p.tile_prefix = (int32_t*)w;
     w += align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
     p.blk_prefix = (int32_t*)w;
     w += align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
+    p.seq_info = w;
+    w += align_up((size_t)p.num_seqs * 32, 256);
     p.part_out = (float*)w;
     w += align_up(slots * G * kD * sizeof(float), 256);
     p.part_ml = (float*)w;
+    w += align_up(slots * G * 2 * sizeof(float), 256);
+    if (p.wave_trace) p.wave_trace = (int64_t*)w;  // requested: the last 32 bytes per wavefront of the workspace
     // query tiles of multi-token sequences: each has >= 2 tokens and wastes at most one tile
     const int multi = std::min(p.num_seqs, p.num_tokens / 2);
     // one token per sequence: a pure decode batch, no query tiles at all

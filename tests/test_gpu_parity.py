@@ -182,6 +182,24 @@ def test_paged_decode_sliding_window(hip, oracle, cache_dtype, window):
     dev.free()
 
 
+@pytest.mark.parametrize("env", [{"HIPATTN_DECODE_DYN_PIECES_PER_WAVE": "4"}, {"HIPATTN_DECODE_SWITCH_COST": "0"},
+                                 {"HIPATTN_DECODE_DYN_PIECES_PER_WAVE": "2", "HIPATTN_DECODE_SWITCH_COST": "9"}])
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
+def test_paged_decode_schedule_knobs(hip, oracle, env, cache_dtype, monkeypatch):
+    """The schedule of the decode kernel (on-demand pieces, segment-start cost) never changes results."""
+    announce("paged decode knobs", env, cache_dtype)
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    seqs = [(c - 1, 1) for c in DECODE_CTX]
+    case = W.make_paged_case(75, seqs, 32, 8, 128, 32, W.F16, W.F16, cache_dtype, sliding_window=700)
+    ref, _, _ = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case)
+    for waves in (0, 40, 300, 4000):
+        out, _ = dev.run(decode_waves=waves)
+        assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3), waves
+    dev.free()
+
+
 def test_paged_decode_ignores_garbage_beyond_context(hip, oracle):
     """Cache rows no sequence has written yet may hold NaN / Inf patterns."""
     announce("paged decode garbage")
