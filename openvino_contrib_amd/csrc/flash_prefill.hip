@@ -3,8 +3,11 @@
 //
 // A workgroup of four wavefronts owns 128 query rows of one query head (32 rows per
 // wavefront) and walks the keys in tiles of 64.  K tiles are staged in LDS row-major, V tiles
-// transposed (the 4x8 patch each thread loads is transposed in registers on the way in), the
-// next tile's global loads are in flight while the current one is consumed.  Both products
+// transposed (the 4x8 patch each thread loads is transposed in registers on the way in).  LDS
+// holds two stages: while tile i is consumed, tile i+1 is written to the other stage and the
+// global loads of tile i+2 are in flight, with one workgroup barrier per tile.  The kernel is
+// held to 256 registers so that two workgroups share a compute unit and one workgroup's MFMA
+// phase overlaps the other's softmax arithmetic.  Both products
 // run on v_mfma_f32_32x32x16 (f16 or bf16) with fp32 accumulation:
 //   S^T = K Q^T   (M = 32 keys, N = 32 query rows, contraction over head_dim)
 //   O^T = V^T P^T (M = 32 head-dim rows, N = 32 query rows, contraction over keys)
@@ -32,6 +35,8 @@ constexpr int kTileK = 64;    // keys per LDS tile
 constexpr int kThreads = 256;
 constexpr int kKRow = 272;    // bytes per K row in LDS (256 + 16 pad)
 constexpr int kVRow = 136;    // bytes per V^T row in LDS (64 keys * 2 + 8 pad)
+constexpr int kKBytes = kTileK * kKRow;          // K part of a stage
+constexpr int kStageBytes = kKBytes + kD * kVRow;  // K tile + V^T tile
 
 template <bool kBf16>
 struct Mfma;
@@ -42,6 +47,11 @@ struct Mfma<false> {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ uint16_t cvt(float x) { return float_to_f16_bits(x); }
+    static __device__ __forceinline__ uint32_t cvt2(float lo, float hi) {
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        const half2_t h = __builtin_convertvector((float2_t){lo, hi}, half2_t);
+        return __builtin_bit_cast(uint32_t, h);
+    }
 };
 template <>
 struct Mfma<true> {
@@ -52,6 +62,12 @@ struct Mfma<true> {
     static __device__ __forceinline__ uint16_t cvt(float x) {
         __bf16 b = (__bf16)x;
         return __builtin_bit_cast(uint16_t, b);
+    }
+    static __device__ __forceinline__ uint32_t cvt2(float lo, float hi) {
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        const bf16x2_t h = __builtin_convertvector((float2_t){lo, hi}, bf16x2_t);
+        return __builtin_bit_cast(uint32_t, h);
     }
 };
 
@@ -76,19 +92,20 @@ struct Tile {
     int num_blocks;
     int64_t block_stride;   // paged: bytes between physical blocks
     int block_size;
+    int block_shift;        // log2(block_size)
 };
 
 __device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key, bool& ok) {
     ok = key < t.kv_len;
     if (!ok) return 0;
     if (t.table == nullptr) return (int64_t)key * (kD * 2);
-    const int lb = key / t.block_size;
+    const int lb = key >> t.block_shift;  // block_size is a power of two on this path
     const int pb = t.table[lb];
     if (pb < 0 || pb >= t.num_blocks) {
         ok = false;
         return 0;
     }
-    return (int64_t)pb * t.block_stride + (int64_t)(key % t.block_size) * (kD * 2);
+    return (int64_t)pb * t.block_stride + (int64_t)(key & (t.block_size - 1)) * (kD * 2);
 }
 
 template <bool kBf16>
@@ -115,8 +132,116 @@ __device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t,
     return __builtin_bit_cast(vec8, cv);
 }
 
+// One 64-key tile against this wavefront's 32 query rows.  kMasked is false for tiles that every
+// query row of the workgroup sees completely (the common case), so that the inner loops carry no
+// per-element predicate at all.
+//
+// Online softmax with a lazily updated reference: p = exp2((s - m_ref) c) is a valid numerator
+// for any reference m_ref as long as it cannot overflow, so the accumulators are rescaled only
+// when some row's maximum has grown by more than 2^8 (exp2 domain) over its reference, which
+// after the first few tiles is rare.
+template <bool kBf16, bool kMasked>
+__device__ __forceinline__ void consume_tile(const Tile& t, const uint8_t* k_lds, const uint8_t* v_lds,
+                                             const typename Mfma<kBf16>::vec8 (&qf)[8], float16_t (&o)[4],
+                                             float& m_ref, float& l_run, float c, int ts, int my_pos, int n32,
+                                             int hi) {
+    using M = Mfma<kBf16>;
+    using vec8 = typename M::vec8;
+    // ---- S^T = K Q^T
+    float16_t s[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const vec8 a = *(const vec8*)(k_lds + (mt * 32 + n32) * kKRow + (i * 16 + hi * 8) * 2);
+            s[mt] = M::mma(a, qf[i], s[mt]);
+        }
+    }
+    // ---- mask (register r of tile mt is key ts + mt*32 + 8*(r/4) + 4*hi + r%4) and row maximum
+    float m_tile = -INFINITY;
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            if constexpr (kMasked) {
+                const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+                bool ok = key < t.kv_len;
+                if (t.causal) ok = ok && key <= my_pos;
+                if (t.window > 0) ok = ok && key > my_pos - t.window;
+                s[mt][r] = ok ? s[mt][r] : -INFINITY;
+            }
+            m_tile = fmaxf(m_tile, s[mt][r]);
+        }
+    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));  // the row lives in lanes l and l + 32
+    const bool grow = m_tile * c > m_ref * c + 8.0f || (m_ref == -INFINITY && m_tile != -INFINITY);
+    if (__builtin_amdgcn_ballot_w64(grow)) {
+        const float m_new = fmaxf(m_ref, m_tile);
+        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // row with nothing to attend yet
+        const float alpha = fast_exp2((m_ref - m_safe) * c);        // exp2(-inf) = 0 the first time
+        l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) o[dt] *= alpha;
+        m_ref = m_new;
+    }
+    const float neg_mc = (m_ref == -INFINITY) ? 0.0f : -m_ref * c;
+    float lsum = 0.0f;
+    vec8 pf[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+        uint4_t pw;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float p0 = fast_exp2(fmaf(s[ks >> 1][(ks & 1) * 8 + 2 * w], c, neg_mc));
+            const float p1 = fast_exp2(fmaf(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1], c, neg_mc));
+            lsum += p0 + p1;
+            pw[w] = M::cvt2(p0, p1);
+        }
+        pf[ks] = __builtin_bit_cast(vec8, pw);
+    }
+    l_run += lsum;
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            const uint8_t* vrow = v_lds + (dt * 32 + n32) * kVRow + (ks * 16 + 4 * hi) * 2;
+            const uint2_t a0 = *(const uint2_t*)(vrow);
+            const uint2_t a1 = *(const uint2_t*)(vrow + 16);
+            const uint4_t aw = {a0[0], a0[1], a1[0], a1[1]};
+            o[dt] = M::mma(__builtin_bit_cast(vec8, aw), pf[ks], o[dt]);
+        }
+    }
+}
+
+template <int kOutDtype>
+__device__ __forceinline__ void store_rows(const Tile& t, const float16_t (&o)[4], float inv, int row, int hi) {
+    // o[dt][r] is head-dim dt*32 + 8*(r/4) + 4*hi + r%4 of `row`: four consecutive outputs per (dt, r/4)
+    const int64_t obase = (int64_t)row * t.out_stride;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            const int d = dt * 32 + 8 * rq + 4 * hi;
+            const float x0 = o[dt][rq * 4] * inv, x1 = o[dt][rq * 4 + 1] * inv, x2 = o[dt][rq * 4 + 2] * inv,
+                        x3 = o[dt][rq * 4 + 3] * inv;
+            if constexpr (kOutDtype == HIPATTN_F32) {
+                *(float4*)((float*)t.out + obase + d) = make_float4(x0, x1, x2, x3);
+            } else if constexpr (kOutDtype == HIPATTN_F16) {
+                const uint2_t w = {Mfma<false>::cvt2(x0, x1), Mfma<false>::cvt2(x2, x3)};
+                *(uint2_t*)((uint16_t*)t.out + obase + d) = w;
+            } else {
+                const uint2_t w = {Mfma<true>::cvt2(x0, x1), Mfma<true>::cvt2(x2, x3)};
+                *(uint2_t*)((uint16_t*)t.out + obase + d) = w;
+            }
+        }
+}
+
+// lds: two stages of (K tile, V^T tile); the stage for tile i+1 is filled while tile i is consumed,
+// so the loop needs one workgroup barrier per tile.
 template <bool kBf16>
-__device__ __forceinline__ void run_tile(const Tile& t, uint8_t* k_lds, uint8_t* v_lds, float scale) {
+__device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scale) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     const int tid = threadIdx.x;
@@ -142,7 +267,7 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* k_lds, uint8_t*
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
+    float m_ref = -INFINITY, l_run = 0.0f;
     const int my_pos = t.pos0 + row;  // position of this lane's query row
 
     // global -> register staging: thread (c16, r16) loads K rows r16 + 16k and V rows r16*4 + j
@@ -162,7 +287,7 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* k_lds, uint8_t*
             vreg[j] = ok ? *(const uint4_t*)(t.v + off + c16 * 16) : (uint4_t){0u, 0u, 0u, 0u};
         }
     };
-    auto store_lds = [&]() {
+    auto store_lds = [&](uint8_t* k_lds, uint8_t* v_lds) {
 #pragma unroll
         for (int k = 0; k < 4; k++) *(uint4_t*)(k_lds + (r16 + 16 * k) * kKRow + c16 * 16) = kreg[k];
 #pragma unroll
@@ -179,123 +304,49 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* k_lds, uint8_t*
         }
     };
 
-    if (kv_lo < kv_hi) load_regs(kv_lo);
+    if (kv_lo < kv_hi) {
+        load_regs(kv_lo);
+        store_lds(lds, lds + kKBytes);
+        if (kv_lo + kTileK < kv_hi) load_regs(kv_lo + kTileK);
+    }
+    __syncthreads();
+    int stage = 0;
     for (int ts = kv_lo; ts < kv_hi; ts += kTileK) {
-        __syncthreads();  // everyone is done reading the previous tile
-        store_lds();
-        __syncthreads();
-        if (ts + kTileK < kv_hi) load_regs(ts + kTileK);
-
-        // ---- S^T = K Q^T
-        float16_t s[2];
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const vec8 a = *(const vec8*)(k_lds + (mt * 32 + n32) * kKRow + (i * 16 + hi * 8) * 2);
-                s[mt] = M::mma(a, qf[i], s[mt]);
-            }
-        }
-        // ---- scale + mask.  Register r of tile mt is key ts + mt*32 + 8*(r/4) + 4*hi + r%4.
+        const uint8_t* k_lds = lds + stage * kStageBytes;
+        const uint8_t* v_lds = k_lds + kKBytes;
         const bool all_valid = (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
                                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
-        float mloc = -INFINITY;
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                float x = s[mt][r] * c;
-                if (!all_valid) {
-                    const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
-                    bool ok = key < t.kv_len;
-                    if (t.causal) ok = ok && key <= my_pos;
-                    if (t.window > 0) ok = ok && key > my_pos - t.window;
-                    x = ok ? x : -INFINITY;
-                }
-                s[mt][r] = x;
-                mloc = fmaxf(mloc, x);
-            }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-        const float m_new = fmaxf(m_run, mloc);
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // row with nothing to attend yet
-        const float alpha = fast_exp2(m_run - m_safe);
-        m_run = m_new;
-        float lsum = 0.0f;
-        vec8 pf[4];
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            uint4_t pw;
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w] - m_safe);
-                const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1] - m_safe);
-                lsum += p0 + p1;
-                pw[w] = (uint32_t)M::cvt(p0) | ((uint32_t)M::cvt(p1) << 16);
-            }
-            pf[ks] = __builtin_bit_cast(vec8, pw);
+        if (all_valid)
+            consume_tile<kBf16, false>(t, k_lds, v_lds, qf, o, m_ref, l_run, c, ts, my_pos, n32, hi);
+        else
+            consume_tile<kBf16, true>(t, k_lds, v_lds, qf, o, m_ref, l_run, c, ts, my_pos, n32, hi);
+        if (ts + kTileK < kv_hi) {
+            // the other stage was last read one iteration ago; every wavefront has passed the
+            // barrier that ended that iteration
+            uint8_t* nk = lds + (stage ^ 1) * kStageBytes;
+            store_lds(nk, nk + kKBytes);
+            if (ts + 2 * kTileK < kv_hi) load_regs(ts + 2 * kTileK);
         }
-        l_run = l_run * alpha + lsum;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) o[dt] *= alpha;
-        }
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const uint8_t* vrow = v_lds + (dt * 32 + n32) * kVRow + (ks * 16 + 4 * hi) * 2;
-                uint4_t aw;
-                const uint2_t a0 = *(const uint2_t*)(vrow);
-                const uint2_t a1 = *(const uint2_t*)(vrow + 16);
-                aw[0] = a0[0];
-                aw[1] = a0[1];
-                aw[2] = a1[0];
-                aw[3] = a1[1];
-                o[dt] = M::mma(__builtin_bit_cast(vec8, aw), pf[ks], o[dt]);
-            }
-        }
+        __syncthreads();
+        stage ^= 1;
     }
 
-    // ---- normalise and store.  o[dt][r] is head-dim dt*32 + 8*(r/4) + 4*hi + r%4 of `row`.
+    // ---- normalise and store
     l_run += __shfl_xor(l_run, 32, 64);
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
     if (row < t.rows) {
-        const int64_t obase = (int64_t)row * t.out_stride;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                const int d = dt * 32 + 8 * rq + 4 * hi;
-                if (t.out_dtype == HIPATTN_F32) {
-                    float4 v4 = make_float4(o[dt][rq * 4] * inv, o[dt][rq * 4 + 1] * inv, o[dt][rq * 4 + 2] * inv,
-                                            o[dt][rq * 4 + 3] * inv);
-                    *(float4*)((float*)t.out + obase + d) = v4;
-                } else {
-                    uint2_t w;
-                    if (t.out_dtype == HIPATTN_F16) {
-                        w[0] = (uint32_t)float_to_f16_bits(o[dt][rq * 4] * inv) |
-                               ((uint32_t)float_to_f16_bits(o[dt][rq * 4 + 1] * inv) << 16);
-                        w[1] = (uint32_t)float_to_f16_bits(o[dt][rq * 4 + 2] * inv) |
-                               ((uint32_t)float_to_f16_bits(o[dt][rq * 4 + 3] * inv) << 16);
-                    } else {
-                        w[0] = (uint32_t)float_to_bf16_bits(o[dt][rq * 4] * inv) |
-                               ((uint32_t)float_to_bf16_bits(o[dt][rq * 4 + 1] * inv) << 16);
-                        w[1] = (uint32_t)float_to_bf16_bits(o[dt][rq * 4 + 2] * inv) |
-                               ((uint32_t)float_to_bf16_bits(o[dt][rq * 4 + 3] * inv) << 16);
-                    }
-                    *(uint2_t*)((uint16_t*)t.out + obase + d) = w;
-                }
-            }
+        if (t.out_dtype == HIPATTN_F32)
+            store_rows<HIPATTN_F32>(t, o, inv, row, hi);
+        else if (t.out_dtype == HIPATTN_F16)
+            store_rows<HIPATTN_F16>(t, o, inv, row, hi);
+        else
+            store_rows<HIPATTN_BF16>(t, o, inv, row, hi);
     }
 }
 
 template <bool kBf16>
-__global__ __launch_bounds__(kThreads) void sdpa_flash_kernel(SdpaParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t k_lds[kTileK * kKRow];
-    __shared__ __attribute__((aligned(16))) uint8_t v_lds[kD * kVRow];
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
     const int n_tiles = (p.len_q + kTileQ - 1) / kTileQ;
     const int qt = n_tiles - 1 - (int)blockIdx.x;  // heaviest (latest) causal tiles first
     const int h = blockIdx.y, b = blockIdx.z;
@@ -321,13 +372,14 @@ __global__ __launch_bounds__(kThreads) void sdpa_flash_kernel(SdpaParams p) {
     t.num_blocks = 0;
     t.block_stride = 0;
     t.block_size = 1;
-    run_tile<kBf16>(t, k_lds, v_lds, p.scale);
+    t.block_shift = 0;
+    run_tile<kBf16>(t, lds, p.scale);
 }
 
+// (not held to 256 registers: with the block-table addressing on top that would spill)
 template <bool kBf16>
 __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t k_lds[kTileK * kKRow];
-    __shared__ __attribute__((aligned(16))) uint8_t v_lds[kD * kVRow];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
     const int total = p.tile_prefix[p.num_seqs];
     const int tile_id = total - 1 - (int)blockIdx.x;
     if (tile_id < 0) return;
@@ -370,7 +422,8 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) 
     t.num_blocks = p.num_blocks;
     t.block_stride = (int64_t)p.num_heads_kv * p.block_size * (kD * 2);
     t.block_size = p.block_size;
-    run_tile<kBf16>(t, k_lds, v_lds, p.scale);
+    t.block_shift = __builtin_ctz(p.block_size);
+    run_tile<kBf16>(t, lds, p.scale);
 }
 
 }  // namespace flash
