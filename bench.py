@@ -113,6 +113,17 @@ def bench_sdpa(hip, case, steps, warmup, name):
     return res
 
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script (summaries and the scaling against a plain 1 GiB copy: profiles/*.txt).  Hardware
+# counters cannot be read from inside this process, so these are the recorded figures for the
+# default seeds; None where no counter run exists.
+MEASURED_TRAFFIC_BYTES = {
+    "c3": (563496.0 * 2.0 + 3031.4) * 1024,
+    "c4": (1220723.0 * 2.0 + 12255.3) * 1024,
+    "c2": (136289.7 * 2.0 + 67566.2) * 1024,
+}
+
+
 def roofline_hbm(res, traffic=None):
     a = res["decode_kv_bytes"] / (res["dominant_kernel_ms"] * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
@@ -122,7 +133,8 @@ def roofline_hbm(res, traffic=None):
 def roofline_mfma(res):
     a = res["flops"] / (res["dominant_kernel_ms"] * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "sdpa_flash_kernel"}
+            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get("c2"),
+            "kernel": "sdpa_flash_kernel"}
 
 
 def cpu_baseline_paged(case, budget_s=12.0):
@@ -231,7 +243,7 @@ def main():
             r["roofline"] = roofline_mfma(r)
         else:
             r = bench_paged(hip, case, args.steps, args.warmup, names[w])
-            r["roofline"] = roofline_hbm(r)
+            r["roofline"] = roofline_hbm(r, MEASURED_TRAFFIC_BYTES.get(w))
             if w == "c5":
                 t_ideal = max(r["kv_bytes"] / (HBM_PEAK_GBS * 1e9), r["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                 r["ideal_ms"] = t_ideal * 1e3
