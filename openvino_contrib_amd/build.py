@@ -72,5 +72,25 @@ def build_library(verbose=False, extra_flags=(), jobs=4):
     return LIB_PATH
 
 
+PLUGIN_LIB_PATH = os.path.join(CSRC, "libhip_plugin.so")
+PLUGIN_SOURCES = ["plugin/ops.cpp", "plugin/plugin.cpp", "plugin/c_api.cpp"]
+
+
+def build_plugin():
+    """Compile the host-side plugin layer (plain C++17, reaches the GPU only through libhipattn's C ABI)."""
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("build libhipattn.so first")
+    cxx = shutil.which("g++") or "g++"
+    cmd = [cxx, "-std=c++17", "-O2", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wextra", "-pthread",
+           "-I" + INCLUDE, "-I" + os.path.join(CSRC, "plugin")]
+    cmd += [os.path.join(CSRC, s) for s in PLUGIN_SOURCES]
+    cmd += ["-L" + CSRC, "-lhipattn", "-Wl,-rpath,$ORIGIN", "-o", PLUGIN_LIB_PATH]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("plugin build failed:\n%s" % r.stderr[-6000:])
+    return PLUGIN_LIB_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_plugin())

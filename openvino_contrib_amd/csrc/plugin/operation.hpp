@@ -1,0 +1,148 @@
+// Per-operator contract and registry of the "HIP" plugin.
+//
+// Mirrors the reference's contract -- IOperationExec / OperationBase
+// (modules/nvidia_plugin/src/cuda_operation_base.hpp:33-149), OperationRegistry and
+// OPERATION_REGISTER (src/cuda_operation_registry.hpp:48-109, 133-143) -- with one deliberate
+// difference: operators are shape-polymorphic.  The reference resolves dynamic shapes by cloning
+// a statically shaped operator per distinct input shape (src/cuda_dynamic_operation.cpp:128-230,
+// LRU of 300); attention inputs change shape on every step (tokens in the batch, block tables),
+// so here Execute() receives the runtime shapes with the pointers and the operator object stays
+// immutable and shared by all concurrent requests.
+#pragma once
+
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "graph.hpp"
+#include "hip_device.hpp"
+
+namespace hip_plugin {
+
+using TensorID = size_t;
+
+struct Configuration;  // plugin.hpp
+
+struct CreationContext {
+    int device_id = 0;
+    bool op_benchmark = false;
+};
+
+// One operand at run time: device pointer, element type, concrete shape.  `host` is a host copy of
+// the same bytes when the request has one (small index / scalar inputs set from host memory).
+struct TensorView {
+    void* device = nullptr;
+    const void* host = nullptr;
+    ElementType type = ElementType::dynamic;
+    Shape shape;
+    size_t byte_size() const { return (size_t)shape_size(shape) * element_size(type); }
+};
+
+struct WorkbufferRequest {
+    std::vector<size_t> immutable_sizes;  // filled once at compile time (unused by the attention ops)
+    std::vector<size_t> mutable_sizes;    // per-request scratch
+};
+
+struct Workbuffers {
+    std::vector<void*> mutable_buffers;
+    std::vector<size_t> mutable_sizes;
+};
+
+struct InferenceRequestContext {
+    const Stream& stream;
+    bool profiling = false;
+};
+
+class OperationBase {
+public:
+    using Ptr = std::shared_ptr<OperationBase>;
+    using IndexCollection = std::vector<TensorID>;
+    using Inputs = const std::vector<TensorView>&;
+    using Outputs = const std::vector<TensorView>&;
+
+    OperationBase(const CreationContext&, const Node& node, IndexCollection&& input_ids, IndexCollection&& output_ids)
+        : node_name_(node.friendly_name),
+          type_name_(node.type_name),
+          input_ids_(std::move(input_ids)),
+          output_ids_(std::move(output_ids)) {}
+    virtual ~OperationBase() = default;
+
+    // Concrete output shapes for concrete input shapes (what validate_and_infer_types gives a clone
+    // in the reference, src/cuda_dynamic_operation.cpp:419-468).
+    virtual std::vector<Shape> InferOutputShapes(const std::vector<Shape>& input_shapes) const = 0;
+    // Scratch the operator needs for these shapes; the request provides it in Execute().
+    virtual WorkbufferRequest GetWorkBufferRequest(const std::vector<TensorView>& /*inputs*/) const { return {}; }
+    // Enqueue the operator on context.stream.  const: one instance serves every request.
+    virtual void Execute(const InferenceRequestContext& context, Inputs inputs, Outputs outputs,
+                         const Workbuffers& workbuffers) const = 0;
+    // Outputs that alias an input buffer and are updated in place (input index per output, -1 = none).
+    virtual int InplaceInputOf(size_t /*output*/) const { return -1; }
+
+    const std::string& GetName() const { return node_name_; }
+    const std::string& GetTypeName() const { return type_name_; }
+    const IndexCollection& GetInputIds() const { return input_ids_; }
+    const IndexCollection& GetOutputIds() const { return output_ids_; }
+
+protected:
+    std::string node_name_;
+    std::string type_name_;
+    const IndexCollection input_ids_;
+    const IndexCollection output_ids_;
+};
+
+class OperationRegistry final {
+public:
+    using IndexCollection = OperationBase::IndexCollection;
+    using OperationBuilder = std::function<OperationBase::Ptr(const CreationContext&, const std::shared_ptr<Node>&,
+                                                              IndexCollection&&, IndexCollection&&)>;
+    template <typename TOperation>
+    class Register {
+    public:
+        explicit Register(const std::string& type_name) {
+            getInstance().registerOp(type_name, [](const CreationContext& context, const std::shared_ptr<Node>& node,
+                                                   IndexCollection&& in, IndexCollection&& out) -> OperationBase::Ptr {
+                return std::make_shared<TOperation>(context, *node, std::move(in), std::move(out));
+            });
+        }
+    };
+
+    static OperationRegistry& getInstance() {
+        static OperationRegistry registry;
+        return registry;
+    }
+    bool hasOperation(const std::shared_ptr<Node>& node) const { return builders_.count(node->type_name) != 0; }
+    // Throws when the type is unknown or the operator's constructor rejects the node: that is how
+    // query_model learns what is supported (src/cuda_plugin.cpp:171-188).
+    OperationBase::Ptr createOperation(const CreationContext& context, const std::shared_ptr<Node>& node,
+                                       IndexCollection&& in, IndexCollection&& out) const {
+        auto it = builders_.find(node->type_name);
+        if (it == builders_.end())
+            HIP_PLUGIN_THROW("operation '" + node->type_name + "' (node '" + node->friendly_name +
+                             "') is not supported by the HIP plugin");
+        return it->second(context, node, std::move(in), std::move(out));
+    }
+    std::vector<std::string> registeredTypes() const {
+        std::vector<std::string> names;
+        for (auto& kv : builders_) names.push_back(kv.first);
+        return names;
+    }
+
+private:
+    void registerOp(const std::string& type_name, OperationBuilder&& builder) {
+        if (!builders_.emplace(type_name, std::move(builder)).second)
+            throw std::runtime_error("Operation " + type_name + " is already registered !!");
+    }
+    std::map<std::string, OperationBuilder> builders_;
+};
+
+}  // namespace hip_plugin
+
+// Registers `type` (derived from OperationBase, constructible from
+// (const CreationContext&, const Node&, IndexCollection&&, IndexCollection&&)) for nodes whose
+// type name is `name`.
+#define HIP_OPERATION_REGISTER(type, name)                                                              \
+    extern "C" {                                                                                        \
+    [[maybe_unused]] const ::hip_plugin::OperationRegistry::Register<type> hip_plugin_op_register_##name{#name}; \
+    }

@@ -1,0 +1,210 @@
+"""ctypes binding of libhip_plugin.so (include/hip_plugin.h): the C++ Plugin / CompiledModel /
+InferRequest classes of the "HIP" device, driven from Python by the tests."""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libhip_plugin.so")
+
+F32, F16, BF16, U8, I32 = 0, 1, 2, 3, 100
+_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, U8: np.uint8, I32: np.int32}
+
+_vp, _i, _sz, _cp = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_char_p
+_P = ctypes.POINTER
+_i64p = _P(ctypes.c_int64)
+SYMBOLS = {
+    "hip_plugin_last_error": (_cp, []),
+    "hip_plugin_create": (_i, [_P(_vp)]),
+    "hip_plugin_destroy": (None, [_vp]),
+    "hip_plugin_set_property": (_i, [_vp, _cp, _cp]),
+    "hip_plugin_get_property": (_i, [_vp, _cp, ctypes.c_char_p, _sz]),
+    "hip_plugin_compile_model": (_i, [_vp, _vp, _cp, _P(_vp)]),
+    "hip_plugin_query_model": (_i, [_vp, _vp, ctypes.c_char_p, _sz]),
+    "hip_plugin_registered_operations": (_i, [ctypes.c_char_p, _sz]),
+    "hip_model_create_sdpa": (_i, [_i, _i, _i64p, _i64p, _i, _i, _P(_vp)]),
+    "hip_model_create_paged_attention": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, _P(_vp)]),
+    "hip_model_create_unsupported": (_i, [_P(_vp)]),
+    "hip_model_destroy": (None, [_vp]),
+    "hip_compiled_model_destroy": (None, [_vp]),
+    "hip_compiled_model_num_inputs": (_i, [_vp]),
+    "hip_compiled_model_input_name": (_i, [_vp, _i, ctypes.c_char_p, _sz]),
+    "hip_compiled_model_get_property": (_i, [_vp, _cp, ctypes.c_char_p, _sz]),
+    "hip_compiled_model_create_infer_request": (_i, [_vp, _P(_vp)]),
+    "hip_infer_request_destroy": (None, [_vp]),
+    "hip_infer_request_set_input": (_i, [_vp, _i, _vp, _i, _i, _i, _i64p]),
+    "hip_infer_request_infer": (_i, [_vp]),
+    "hip_infer_request_start_async": (_i, [_vp]),
+    "hip_infer_request_wait": (_i, [_vp]),
+    "hip_infer_request_output_info": (_i, [_vp, _i, _P(_i), _P(_i), _i64p, _P(_sz)]),
+    "hip_infer_request_copy_output": (_i, [_vp, _i, _vp, _sz]),
+    "hip_infer_request_profiling": (_i, [_vp, ctypes.c_char_p, _sz]),
+}
+
+_lib = None
+
+
+class PluginError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(message)
+        self.code = code
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise PluginError(-1, "%s is missing: run __graft_entry__.build()" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def _check(code):
+    if code != 0:
+        raise PluginError(code, lib().hip_plugin_last_error().decode())
+
+
+def _shape(s):
+    return (ctypes.c_int64 * len(s))(*[int(x) for x in s])
+
+
+def _text(fn, *args, size=1 << 16):
+    buf = ctypes.create_string_buffer(size)
+    _check(fn(*args, buf, size))
+    return buf.value.decode()
+
+
+def registered_operations():
+    return _text(lib().hip_plugin_registered_operations).split(",")
+
+
+class Model:
+    def __init__(self, handle):
+        self.handle = handle
+
+    @classmethod
+    def sdpa(cls, dtype, q_shape, kv_shape, causal, with_scale_input=False):
+        h = _vp()
+        _check(lib().hip_model_create_sdpa(dtype, len(q_shape), _shape(q_shape), _shape(kv_shape), int(causal),
+                                           int(with_scale_input), ctypes.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def paged_attention(cls, q_dtype, kv_dtype, cache_dtype, Hq, Hkv, D, block_size, alibi_len=0):
+        h = _vp()
+        _check(lib().hip_model_create_paged_attention(q_dtype, kv_dtype, cache_dtype, Hq, Hkv, D, block_size,
+                                                      alibi_len, ctypes.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def unsupported(cls):
+        h = _vp()
+        _check(lib().hip_model_create_unsupported(ctypes.byref(h)))
+        return cls(h)
+
+    def __del__(self):
+        if self.handle:
+            lib().hip_model_destroy(self.handle)
+            self.handle = None
+
+
+class InferRequest:
+    def __init__(self, handle):
+        self.handle = handle
+        self._keep = {}
+
+    def set_input(self, index, array, dtype):
+        """Host tensor: wrapped, not copied (kept alive here until replaced)."""
+        array = np.ascontiguousarray(array, _NP[dtype])
+        self._keep[index] = array
+        _check(lib().hip_infer_request_set_input(self.handle, index, array.ctypes.data_as(_vp), 0, dtype, array.ndim,
+                                                 _shape(array.shape)))
+
+    def set_device_input(self, index, device_ptr, dtype, shape):
+        _check(lib().hip_infer_request_set_input(self.handle, index, device_ptr, 1, dtype, len(shape), _shape(shape)))
+
+    def infer(self):
+        _check(lib().hip_infer_request_infer(self.handle))
+
+    def start_async(self):
+        _check(lib().hip_infer_request_start_async(self.handle))
+
+    def wait(self):
+        _check(lib().hip_infer_request_wait(self.handle))
+
+    def output(self, index=0):
+        dt, rank, nbytes = _i(0), _i(0), _sz(0)
+        shape = (ctypes.c_int64 * 8)()
+        _check(lib().hip_infer_request_output_info(self.handle, index, ctypes.byref(dt), ctypes.byref(rank), shape,
+                                                   ctypes.byref(nbytes)))
+        out = np.empty([shape[i] for i in range(rank.value)], _NP[dt.value])
+        _check(lib().hip_infer_request_copy_output(self.handle, index, out.ctypes.data_as(_vp), out.nbytes))
+        return out, dt.value
+
+    def profiling(self):
+        rows = []
+        for line in _text(lib().hip_infer_request_profiling, self.handle).splitlines():
+            name, typ, us = line.split("|")
+            rows.append((name, typ, float(us)))
+        return rows
+
+    def __del__(self):
+        if self.handle:
+            lib().hip_infer_request_destroy(self.handle)
+            self.handle = None
+
+
+class CompiledModel:
+    def __init__(self, handle):
+        self.handle = handle
+
+    def input_names(self):
+        n = lib().hip_compiled_model_num_inputs(self.handle)
+        return [_text(lib().hip_compiled_model_input_name, self.handle, i, size=256) for i in range(n)]
+
+    def get_property(self, key):
+        return _text(lib().hip_compiled_model_get_property, self.handle, key.encode(), size=4096)
+
+    def create_infer_request(self):
+        h = _vp()
+        _check(lib().hip_compiled_model_create_infer_request(self.handle, ctypes.byref(h)))
+        return InferRequest(h)
+
+    def __del__(self):
+        if self.handle:
+            lib().hip_compiled_model_destroy(self.handle)
+            self.handle = None
+
+
+class Plugin:
+    def __init__(self):
+        h = _vp()
+        _check(lib().hip_plugin_create(ctypes.byref(h)))
+        self.handle = h
+
+    def set_property(self, key, value):
+        _check(lib().hip_plugin_set_property(self.handle, key.encode(), str(value).encode()))
+
+    def get_property(self, key):
+        return _text(lib().hip_plugin_get_property, self.handle, key.encode(), size=4096)
+
+    def query_model(self, model):
+        names = _text(lib().hip_plugin_query_model, self.handle, model.handle)
+        return names.split(",") if names else []
+
+    def compile_model(self, model, properties=None):
+        text = ";".join("%s=%s" % kv for kv in (properties or {}).items()).encode() if properties else None
+        h = _vp()
+        _check(lib().hip_plugin_compile_model(self.handle, model.handle, text, ctypes.byref(h)))
+        return CompiledModel(h)
+
+    def __del__(self):
+        if self.handle:
+            lib().hip_plugin_destroy(self.handle)
+            self.handle = None
