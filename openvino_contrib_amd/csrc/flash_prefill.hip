@@ -29,6 +29,29 @@ namespace hipattn {
 
 namespace flash {
 
+// Diagnostic build only (a probe that includes this file with HIPATTN_FLASH_TRACE defined):
+// lane 0 of selected wavefronts stores the shader clock at the phase boundaries of every tile.
+#ifdef HIPATTN_FLASH_TRACE
+__device__ long long* g_flash_trace = nullptr;
+struct PhaseClock {
+    long long acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    long long last = 0;
+};
+// phase k = time since the previous stamp; totals are stored once, after the last tile
+#define FLASH_STAMP(t, tile, k)                                                   \
+    do {                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                        \
+        const long long stamp_ = (long long)__builtin_readcyclecounter();         \
+        __builtin_amdgcn_sched_barrier(0);                                        \
+        (t).clk.acc[k] += stamp_ - (t).clk.last;                                  \
+        (t).clk.last = stamp_;                                                    \
+    } while (0)
+#else
+#define FLASH_STAMP(t, tile, k) \
+    do {                        \
+    } while (0)
+#endif
+
 constexpr int kD = 128;
 constexpr int kTileQ = 128;   // query rows per workgroup
 constexpr int kTileK = 64;    // keys per LDS tile
@@ -93,6 +116,10 @@ struct Tile {
     int64_t block_stride;   // paged: bytes between physical blocks
     int block_size;
     int block_shift;        // log2(block_size)
+#ifdef HIPATTN_FLASH_TRACE
+    long long* trace;
+    mutable PhaseClock clk;
+#endif
 };
 
 __device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key, bool& ok) {
@@ -159,6 +186,7 @@ __device__ __forceinline__ void consume_tile(const Tile& t, const uint8_t* k_lds
             s[mt] = M::mma(a, qf[i], s[mt]);
         }
     }
+    FLASH_STAMP(t, ts / kTileK, 1);
     // ---- mask (register r of tile mt is key ts + mt*32 + 8*(r/4) + 4*hi + r%4) and row maximum
     float m_tile = -INFINITY;
 #pragma unroll
@@ -201,6 +229,7 @@ __device__ __forceinline__ void consume_tile(const Tile& t, const uint8_t* k_lds
         pf[ks] = __builtin_bit_cast(vec8, pw);
     }
     l_run += lsum;
+    FLASH_STAMP(t, ts / kTileK, 2);
     // ---- O^T += V^T P^T
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
@@ -270,7 +299,9 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scal
     float m_ref = -INFINITY, l_run = 0.0f;
     const int my_pos = t.pos0 + row;  // position of this lane's query row
 
-    // global -> register staging: thread (c16, r16) loads K rows r16 + 16k and V rows r16*4 + j
+    // global -> register staging: thread (c16, r16) loads 16-byte chunk c16 of K rows r16 + 16k
+    // and chunk r16 of V rows c16*4 + j: the 16 lanes that share an LDS write instruction then
+    // hold 16 consecutive key quads of one V^T row (a contiguous 128-byte write, no bank conflicts)
     const int c16 = tid & 15, r16 = tid >> 4;
     uint4_t kreg[4], vreg[4];
     auto load_regs = [&](int tile_start) {
@@ -283,8 +314,8 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scal
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             bool ok;
-            int64_t off = kv_row_offset(t, tile_start + r16 * 4 + j, ok);
-            vreg[j] = ok ? *(const uint4_t*)(t.v + off + c16 * 16) : (uint4_t){0u, 0u, 0u, 0u};
+            int64_t off = kv_row_offset(t, tile_start + c16 * 4 + j, ok);
+            vreg[j] = ok ? *(const uint4_t*)(t.v + off + r16 * 16) : (uint4_t){0u, 0u, 0u, 0u};
         }
     };
     auto store_lds = [&](uint8_t* k_lds, uint8_t* v_lds) {
@@ -300,7 +331,7 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scal
                 w[0] = (vreg[0][e >> 1] & 0xffffu) | (vreg[1][e >> 1] << 16);
                 w[1] = (vreg[2][e >> 1] & 0xffffu) | (vreg[3][e >> 1] << 16);
             }
-            *(uint2_t*)(v_lds + (c16 * 8 + e) * kVRow + r16 * 8) = w;
+            *(uint2_t*)(v_lds + (r16 * 8 + e) * kVRow + c16 * 8) = w;
         }
     };
 
@@ -311,26 +342,38 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scal
     }
     __syncthreads();
     int stage = 0;
+#ifdef HIPATTN_FLASH_TRACE
+    t.clk.last = (long long)__builtin_readcyclecounter();
+#endif
     for (int ts = kv_lo; ts < kv_hi; ts += kTileK) {
         const uint8_t* k_lds = lds + stage * kStageBytes;
         const uint8_t* v_lds = k_lds + kKBytes;
+        FLASH_STAMP(t, ts / kTileK, 0);
         const bool all_valid = (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
                                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
         if (all_valid)
             consume_tile<kBf16, false>(t, k_lds, v_lds, qf, o, m_ref, l_run, c, ts, my_pos, n32, hi);
         else
             consume_tile<kBf16, true>(t, k_lds, v_lds, qf, o, m_ref, l_run, c, ts, my_pos, n32, hi);
+        FLASH_STAMP(t, ts / kTileK, 3);
         if (ts + kTileK < kv_hi) {
             // the other stage was last read one iteration ago; every wavefront has passed the
             // barrier that ended that iteration
             uint8_t* nk = lds + (stage ^ 1) * kStageBytes;
             store_lds(nk, nk + kKBytes);
+            FLASH_STAMP(t, ts / kTileK, 4);
             if (ts + 2 * kTileK < kv_hi) load_regs(ts + 2 * kTileK);
         }
+        FLASH_STAMP(t, ts / kTileK, 5);
         __syncthreads();
+        FLASH_STAMP(t, ts / kTileK, 6);
         stage ^= 1;
     }
 
+#ifdef HIPATTN_FLASH_TRACE
+    if (t.trace)
+        for (int k = 0; k < 8; k++) t.trace[k] = t.clk.acc[k];
+#endif
     // ---- normalise and store
     l_run += __shfl_xor(l_run, 32, 64);
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
@@ -344,27 +387,42 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scal
     }
 }
 
-template <bool kBf16>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
-    const int n_tiles = (p.len_q + kTileQ - 1) / kTileQ;
-    const int qt = n_tiles - 1 - (int)blockIdx.x;  // heaviest (latest) causal tiles first
-    const int h = blockIdx.y, b = blockIdx.z;
+// Launch index -> work item: workgroups go to the eight XCDs round-robin by launch index and
+// each XCD has its own L2, so index i becomes item (i % 8) * (n / 8) + i / 8.  An XCD then walks
+// a contiguous range of items ordered (batch, kv head, query tile descending, query head in
+// group): the workgroups resident on it at one time share one K/V head, which stays in that L2,
+// and the heaviest (latest) causal tiles of a head come first.
+struct SdpaItem {
+    int b, h, qt;
+};
+__device__ __forceinline__ SdpaItem sdpa_item(const SdpaParams& p, int n_tiles) {
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const int n_items = (int)gridDim.x;
+    int item = (int)blockIdx.x;
+    if ((n_items & 7) == 0) item = (item & 7) * (n_items >> 3) + (item >> 3);
+    SdpaItem it;
+    it.qt = n_tiles - 1 - (item / G) % n_tiles;
+    it.h = ((item / (G * n_tiles)) % p.num_heads_kv) * G + item % G;
+    it.b = item / (G * n_tiles * p.num_heads_kv);
+    return it;
+}
+
+__device__ __forceinline__ Tile sdpa_tile(const SdpaParams& p, const SdpaItem& it, int tile_rows) {
     const int G = p.num_heads_q / p.num_heads_kv;
     Tile t;
-    const int64_t qoff = (((int64_t)b * p.num_heads_q + h) * p.len_q + (int64_t)qt * kTileQ) * kD;
+    const int64_t qoff = (((int64_t)it.b * p.num_heads_q + it.h) * p.len_q + (int64_t)it.qt * tile_rows) * kD;
     t.q = (const uint16_t*)p.q + qoff;
     t.q_stride = kD;
     t.out = (uint16_t*)p.out + qoff;
     t.out_stride = kD;
-    t.rows = min(kTileQ, p.len_q - qt * kTileQ);
-    t.pos0 = qt * kTileQ;
+    t.rows = min(tile_rows, p.len_q - it.qt * tile_rows);
+    t.pos0 = it.qt * tile_rows;
     t.kv_len = p.len_kv;
     t.causal = p.causal;
     t.window = 0;
     t.q_dtype = p.dtype;
     t.out_dtype = p.dtype;
-    const int64_t kvoff = ((int64_t)b * p.num_heads_kv + h / G) * p.len_kv * (kD * 2);
+    const int64_t kvoff = ((int64_t)it.b * p.num_heads_kv + it.h / G) * p.len_kv * (kD * 2);
     t.k = (const uint8_t*)p.k + kvoff;
     t.v = (const uint8_t*)p.v + kvoff;
     t.table = nullptr;
@@ -373,6 +431,27 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     t.block_stride = 0;
     t.block_size = 1;
     t.block_shift = 0;
+    return t;
+}
+
+template <bool kBf16>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
+#ifdef HIPATTN_FLASH_LDS_PAD  // diagnostic: forces one workgroup per compute unit
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes + HIPATTN_FLASH_LDS_PAD];
+#else
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
+#endif
+    const int n_tiles = (p.len_q + kTileQ - 1) / kTileQ;
+    const SdpaItem it = sdpa_item(p, n_tiles);
+    Tile t = sdpa_tile(p, it, kTileQ);
+#ifdef HIPATTN_FLASH_TRACE
+    {
+        const int wg = it.h + p.num_heads_q * it.b;
+        t.trace = (g_flash_trace && it.qt == n_tiles - 1 && (threadIdx.x & 63) == 0)
+                      ? g_flash_trace + (int64_t)(wg * 4 + (threadIdx.x >> 6)) * 8
+                      : nullptr;
+    }
+#endif
     run_tile<kBf16>(t, lds, p.scale);
 }
 
@@ -423,6 +502,9 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) 
     t.block_stride = (int64_t)p.num_heads_kv * p.block_size * (kD * 2);
     t.block_size = p.block_size;
     t.block_shift = __builtin_ctz(p.block_size);
+#ifdef HIPATTN_FLASH_TRACE
+    t.trace = nullptr;
+#endif
     run_tile<kBf16>(t, lds, p.scale);
 }
 
@@ -435,7 +517,7 @@ bool sdpa_flash_supported(const SdpaParams& p) {
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe) {
     if (p.batch == 0 || p.len_q == 0) return hipSuccess;
     const int n_tiles = (p.len_q + flash::kTileQ - 1) / flash::kTileQ;
-    dim3 grid(n_tiles, p.num_heads_q, p.batch);
+    dim3 grid(n_tiles * p.num_heads_q * p.batch);
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     if (p.dtype == HIPATTN_BF16)
         hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
