@@ -2,13 +2,14 @@
 // multi-token (chunked prefill) sequences of PagedAttentionExtension share one kernel body.
 //
 // A workgroup of four wavefronts owns 128 query rows of one query head (32 rows per
-// wavefront) and walks the keys in tiles of 64.  K tiles are staged in LDS row-major, V tiles
-// transposed (the 4x8 patch each thread loads is transposed in registers on the way in).  LDS
-// holds two stages: while tile i is consumed, tile i+1 is written to the other stage and the
-// global loads of tile i+2 are in flight, with one workgroup barrier per tile.  The kernel is
-// held to 256 registers so that two workgroups share a compute unit and one workgroup's MFMA
-// phase overlaps the other's softmax arithmetic.  Both products
-// run on v_mfma_f32_32x32x16 (f16 or bf16) with fp32 accumulation:
+// wavefront) and walks the keys in tiles of 64.  K and V tiles go from global memory straight
+// into LDS (global_load_lds_dwordx4: no staging registers, no LDS write instructions), both
+// row-major with the 16-byte chunks of a row XOR-swizzled so that fragment reads are free of
+// bank conflicts; the V^T operand is read with the transposing LDS load ds_read_b64_tr_b16.
+// LDS holds two stages: the loads of tile i+1 are issued at the top of iteration i into the
+// stage that tile i-1 occupied, with one workgroup barrier per tile.  The kernel is held to 256
+// registers so that two workgroups share a compute unit.  Both products run on
+// v_mfma_f32_32x32x16 (f16 or bf16) with fp32 accumulation:
 //   S^T = K Q^T   (M = 32 keys, N = 32 query rows, contraction over head_dim)
 //   O^T = V^T P^T (M = 32 head-dim rows, N = 32 query rows, contraction over keys)
 // Computing the scores transposed leaves each lane with 8 consecutive-in-operand keys of one
@@ -33,6 +34,7 @@ namespace flash {
 // lane 0 of selected wavefronts stores the shader clock at the phase boundaries of every tile.
 #ifdef HIPATTN_FLASH_TRACE
 __device__ long long* g_flash_trace = nullptr;
+__device__ long long* g_flash_wg_trace = nullptr;  // per workgroup: wall start/end (100 MHz), cycles start/end, hw id
 struct PhaseClock {
     long long acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     long long last = 0;
@@ -56,10 +58,12 @@ constexpr int kD = 128;
 constexpr int kTileQ = 128;   // query rows per workgroup
 constexpr int kTileK = 64;    // keys per LDS tile
 constexpr int kThreads = 256;
-constexpr int kKRow = 272;    // bytes per K row in LDS (256 + 16 pad)
-constexpr int kVRow = 136;    // bytes per V^T row in LDS (64 keys * 2 + 8 pad)
-constexpr int kKBytes = kTileK * kKRow;          // K part of a stage
-constexpr int kStageBytes = kKBytes + kD * kVRow;  // K tile + V^T tile
+constexpr int kRowBytes = kD * 2;                // a K or V row in LDS: 16 chunks of 16 bytes
+constexpr int kKBytes = kTileK * kRowBytes;      // K part of a stage
+constexpr int kStageBytes = 2 * kKBytes;         // K tile + V tile
+
+#define HIPATTN_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define HIPATTN_GLOBAL_PTR(p) ((__attribute__((address_space(1))) void*)(p))
 
 template <bool kBf16>
 struct Mfma;
@@ -122,17 +126,15 @@ struct Tile {
 #endif
 };
 
-__device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key, bool& ok) {
-    ok = key < t.kv_len;
-    if (!ok) return 0;
-    if (t.table == nullptr) return (int64_t)key * (kD * 2);
+// Byte offset of a key's row from t.k / t.v.  Keys past the end are redirected to the last valid
+// key and block ids outside the cache are clamped: such rows only ever meet a probability of
+// zero (or are unspecified input), but they must be readable and finite.
+__device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key) {
+    key = min(key, t.kv_len - 1);
+    if (t.table == nullptr) return (int64_t)key * kRowBytes;
     const int lb = key >> t.block_shift;  // block_size is a power of two on this path
-    const int pb = t.table[lb];
-    if (pb < 0 || pb >= t.num_blocks) {
-        ok = false;
-        return 0;
-    }
-    return (int64_t)pb * t.block_stride + (int64_t)(key & (t.block_size - 1)) * (kD * 2);
+    const int pb = min(max(t.table[lb], 0), t.num_blocks - 1);
+    return (int64_t)pb * t.block_stride + (int64_t)(key & (t.block_size - 1)) * kRowBytes;
 }
 
 template <bool kBf16>
@@ -159,49 +161,111 @@ __device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t,
     return __builtin_bit_cast(vec8, cv);
 }
 
-// One 64-key tile against this wavefront's 32 query rows.  kMasked is false for tiles that every
-// query row of the workgroup sees completely (the common case), so that the inner loops carry no
-// per-element predicate at all.
+typedef __attribute__((address_space(3))) uint8_t lds_byte;
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// LDS layout of a K or V tile: row r (a key) at byte r * 256, its 16-byte chunk c stored at chunk
+// position c ^ swz(r), with swz(r) = r % 16 for K and 4 * (r % 4) for V.
+//
+// K fragment (A operand of S^T = K Q^T, k-step i): lane (n32, hi) reads chunk 2i + hi of row
+// mt*32 + n32 with one ds_read_b128; sixteen consecutive lanes hit sixteen different positions.
+//
+// V^T fragment (A operand of O^T = V^T P^T, k-step ks, head-dim tile dt): the lane holding
+// head-dim d = dt*32 + n32 needs V[key][d] for the keys 16ks + 4hi + {0..3} and 16ks + 8 + 4hi +
+// {0..3}.  ds_read_b64_tr_b16 gives lane i of a 16-lane group element j = what lane 4j + i/4 of
+// the group addressed, taken at 16-bit index i % 4: so lane i addresses row key0 + i/4, head-dim
+// d0 + 4 (i % 4) .. +3 (d0 = dt*32 + 16 * (group & 1), key0 = 16ks + 4 * (group >> 1)), and
+// receives V[key0 + j][d0 + i].  Two such reads, eight rows apart, make one fragment.
+struct FragOffsets {
+    int k[8];  // + mt * 32 rows
+    int v[4];  // per dt; + ks * 16 rows (+ 8 rows for the second half)
+};
+
+__device__ __forceinline__ FragOffsets frag_offsets(int lane) {
+    FragOffsets f;
+    const int n32 = lane & 31, hi = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < 8; i++) f.k[i] = n32 * kRowBytes + (((2 * i + hi) ^ (n32 & 15)) << 4);
+    const int g = lane >> 4, i16 = lane & 15;
+    const int vrow = 4 * (g >> 1) + (i16 >> 2);  // row % 4 == i16 / 4
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+        f.v[dt] = vrow * kRowBytes + (((4 * dt + 2 * (g & 1) + ((i16 & 3) >> 1)) ^ (4 * (i16 >> 2))) << 4) + 8 * (i16 & 1);
+    return f;
+}
+
+template <bool kBf16>
+__device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte* v_lds, const FragOffsets& f, int ks,
+                                                                  int dt) {
+    typedef __attribute__((address_space(3))) short4_t lds_short4;
+    const lds_byte* p = v_lds + f.v[dt] + ks * 16 * kRowBytes;
+    const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)p);
+    const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p + 8 * kRowBytes));
+    typedef short short8_t __attribute__((ext_vector_type(8)));
+    const short8_t a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+    return __builtin_bit_cast(typename Mfma<kBf16>::vec8, a);
+}
+
+// One 64-key tile against this wavefront's 32 query rows.  `masked` is false for tiles that every
+// query row of the workgroup sees completely (the common case).
+//
+// LDS latency is taken out of the MFMA chains by issuing fragment reads in batches ahead of
+// their use: all sixteen K fragments before the first score MFMA, and the first half of the V^T
+// fragments right behind the score MFMAs, so that they arrive during the softmax arithmetic.
 //
 // Online softmax with a lazily updated reference: p = exp2((s - m_ref) c) is a valid numerator
 // for any reference m_ref as long as it cannot overflow, so the accumulators are rescaled only
 // when some row's maximum has grown by more than 2^8 (exp2 domain) over its reference, which
 // after the first few tiles is rare.
-template <bool kBf16, bool kMasked>
-__device__ __forceinline__ void consume_tile(const Tile& t, const uint8_t* k_lds, const uint8_t* v_lds,
-                                             const typename Mfma<kBf16>::vec8 (&qf)[8], float16_t (&o)[4],
-                                             float& m_ref, float& l_run, float c, int ts, int my_pos, int n32,
-                                             int hi) {
+template <bool kBf16, typename AfterScores>
+__device__ __forceinline__ void consume_tile(const Tile& t, const lds_byte* k_lds, const lds_byte* v_lds,
+                                             const FragOffsets& f, const typename Mfma<kBf16>::vec8 (&qf)[8],
+                                             float16_t (&o)[4], float& m_ref, float& l_run, float c, int ts, int my_pos,
+                                             int hi, bool masked, AfterScores&& after_scores) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
+    typedef __attribute__((address_space(3))) vec8 lds_vec8;
     // ---- S^T = K Q^T
+    vec8 kf[2][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) kf[mt][i] = *(const lds_vec8*)(k_lds + f.k[i] + mt * 32 * kRowBytes);
+    __builtin_amdgcn_sched_barrier(0);
     float16_t s[2];
-#pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const vec8 a = *(const vec8*)(k_lds + (mt * 32 + n32) * kKRow + (i * 16 + hi * 8) * 2);
-            s[mt] = M::mma(a, qf[i], s[mt]);
-        }
-    }
-    FLASH_STAMP(t, ts / kTileK, 1);
-    // ---- mask (register r of tile mt is key ts + mt*32 + 8*(r/4) + 4*hi + r%4) and row maximum
-    float m_tile = -INFINITY;
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            if constexpr (kMasked) {
+        for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) s[mt] = M::mma(kf[mt][i], qf[i], s[mt]);
+    vec8 vf[2][4];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) vf[ks][dt] = read_v_frag<kBf16>(v_lds, f, ks, dt);
+    after_scores();
+    FLASH_STAMP(t, ts / kTileK, 1);
+    // ---- mask (register r of tile mt is key ts + mt*32 + 8*(r/4) + 4*hi + r%4) and row maximum
+    if (masked) {
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
                 const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
                 bool ok = key < t.kv_len;
                 if (t.causal) ok = ok && key <= my_pos;
                 if (t.window > 0) ok = ok && key > my_pos - t.window;
                 s[mt][r] = ok ? s[mt][r] : -INFINITY;
             }
-            m_tile = fmaxf(m_tile, s[mt][r]);
-        }
+    }
+    float m_tile = -INFINITY;
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, s[mt][r]);
     m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));  // the row lives in lanes l and l + 32
     const bool grow = m_tile * c > m_ref * c + 8.0f || (m_ref == -INFINITY && m_tile != -INFINITY);
     if (__builtin_amdgcn_ballot_w64(grow)) {
@@ -231,17 +295,19 @@ __device__ __forceinline__ void consume_tile(const Tile& t, const uint8_t* k_lds
     l_run += lsum;
     FLASH_STAMP(t, ts / kTileK, 2);
     // ---- O^T += V^T P^T
+    vec8 vg[2][4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
+    for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            const uint8_t* vrow = v_lds + (dt * 32 + n32) * kVRow + (ks * 16 + 4 * hi) * 2;
-            const uint2_t a0 = *(const uint2_t*)(vrow);
-            const uint2_t a1 = *(const uint2_t*)(vrow + 16);
-            const uint4_t aw = {a0[0], a0[1], a1[0], a1[1]};
-            o[dt] = M::mma(__builtin_bit_cast(vec8, aw), pf[ks], o[dt]);
-        }
-    }
+        for (int dt = 0; dt < 4; dt++) vg[ks][dt] = read_v_frag<kBf16>(v_lds, f, 2 + ks, dt);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) o[dt] = M::mma(vf[ks][dt], pf[ks], o[dt]);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) o[dt] = M::mma(vg[ks][dt], pf[2 + ks], o[dt]);
 }
 
 template <int kOutDtype>
@@ -267,14 +333,15 @@ __device__ __forceinline__ void store_rows(const Tile& t, const float16_t (&o)[4
         }
 }
 
-// lds: two stages of (K tile, V^T tile); the stage for tile i+1 is filled while tile i is consumed,
-// so the loop needs one workgroup barrier per tile.
+// lds: two stages of (K tile, V tile); stage (i+1)%2 is filled while tile i is consumed, so the
+// loop needs one workgroup barrier per tile.
 template <bool kBf16>
-__device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scale) {
+__device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, float scale) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
+    lds_byte* const lds = (lds_byte*)lds_generic;
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int n32 = lane & 31, hi = lane >> 5;
     const int row = wave * 32 + n32;  // query row inside the tile
     const float c = scale * kLog2e;
@@ -298,73 +365,62 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds, float scal
         for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
     float m_ref = -INFINITY, l_run = 0.0f;
     const int my_pos = t.pos0 + row;  // position of this lane's query row
+    const FragOffsets f = frag_offsets(lane);
 
-    // global -> register staging: thread (c16, r16) loads 16-byte chunk c16 of K rows r16 + 16k
-    // and chunk r16 of V rows c16*4 + j: the 16 lanes that share an LDS write instruction then
-    // hold 16 consecutive key quads of one V^T row (a contiguous 128-byte write, no bank conflicts)
-    const int c16 = tid & 15, r16 = tid >> 4;
-    uint4_t kreg[4], vreg[4];
-    auto load_regs = [&](int tile_start) {
+    // global -> LDS: one instruction moves four rows (64 lanes x 16 bytes, LDS address = wave-uniform
+    // base + lane * 16); wavefront w issues the four instructions of rows 16w .. 16w + 15 of the K
+    // tile and of the V tile.  Lane l fills chunk position l % 16 of row 16w + 4k + l / 16, i.e. it
+    // fetches chunk (l % 16) ^ swz(row).
+    const int lrow = lane >> 4, lpos = lane & 15;
+    auto load_k_tile = [&](int tile_start, lds_byte* k_lds) {
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            bool ok;
-            int64_t off = kv_row_offset(t, tile_start + r16 + 16 * k, ok);
-            kreg[k] = ok ? *(const uint4_t*)(t.k + off + c16 * 16) : (uint4_t){0u, 0u, 0u, 0u};
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            bool ok;
-            int64_t off = kv_row_offset(t, tile_start + c16 * 4 + j, ok);
-            vreg[j] = ok ? *(const uint4_t*)(t.v + off + r16 * 16) : (uint4_t){0u, 0u, 0u, 0u};
+            const int r = 16 * wave + 4 * k + lrow;
+            const int64_t off = kv_row_offset(t, tile_start + r) + ((lpos ^ (r & 15)) << 4);
+            __builtin_amdgcn_global_load_lds(HIPATTN_GLOBAL_PTR(t.k + off), HIPATTN_LDS_PTR(k_lds + (16 * wave + 4 * k) * kRowBytes),
+                                             16, 0, 0);
         }
     };
-    auto store_lds = [&](uint8_t* k_lds, uint8_t* v_lds) {
+    auto load_v_tile = [&](int tile_start, lds_byte* v_lds) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) *(uint4_t*)(k_lds + (r16 + 16 * k) * kKRow + c16 * 16) = kreg[k];
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            uint2_t w;
-            if (e & 1) {
-                w[0] = (vreg[0][e >> 1] >> 16) | (vreg[1][e >> 1] & 0xffff0000u);
-                w[1] = (vreg[2][e >> 1] >> 16) | (vreg[3][e >> 1] & 0xffff0000u);
-            } else {
-                w[0] = (vreg[0][e >> 1] & 0xffffu) | (vreg[1][e >> 1] << 16);
-                w[1] = (vreg[2][e >> 1] & 0xffffu) | (vreg[3][e >> 1] << 16);
-            }
-            *(uint2_t*)(v_lds + (r16 * 8 + e) * kVRow + c16 * 8) = w;
+        for (int k = 0; k < 4; k++) {
+            const int r = 16 * wave + 4 * k + lrow;
+            const int64_t off = kv_row_offset(t, tile_start + r) + ((lpos ^ (4 * (r & 3))) << 4);
+            __builtin_amdgcn_global_load_lds(HIPATTN_GLOBAL_PTR(t.v + off), HIPATTN_LDS_PTR(v_lds + (16 * wave + 4 * k) * kRowBytes),
+                                             16, 0, 0);
         }
     };
 
     if (kv_lo < kv_hi) {
-        load_regs(kv_lo);
-        store_lds(lds, lds + kKBytes);
-        if (kv_lo + kTileK < kv_hi) load_regs(kv_lo + kTileK);
+        load_k_tile(kv_lo, lds);
+        load_v_tile(kv_lo, lds + kKBytes);
     }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's rows are in LDS
     __syncthreads();
     int stage = 0;
 #ifdef HIPATTN_FLASH_TRACE
     t.clk.last = (long long)__builtin_readcyclecounter();
 #endif
-    for (int ts = kv_lo; ts < kv_hi; ts += kTileK) {
-        const uint8_t* k_lds = lds + stage * kStageBytes;
-        const uint8_t* v_lds = k_lds + kKBytes;
+    // `cur` and `next` are the two stages: the restrict qualifiers tell the compiler that the LDS
+    // writes of the asynchronous loads cannot alias the fragment reads of the same iteration, so
+    // that it does not wait for the loads before every LDS read.
+    auto iteration = [&](int ts, const lds_byte* __restrict__ cur, lds_byte* __restrict__ next) {
+        const bool has_next = ts + kTileK < kv_hi;
         FLASH_STAMP(t, ts / kTileK, 0);
+        if (has_next) load_k_tile(ts + kTileK, next);
+        FLASH_STAMP(t, ts / kTileK, 5);
         const bool all_valid = (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
                                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
-        if (all_valid)
-            consume_tile<kBf16, false>(t, k_lds, v_lds, qf, o, m_ref, l_run, c, ts, my_pos, n32, hi);
-        else
-            consume_tile<kBf16, true>(t, k_lds, v_lds, qf, o, m_ref, l_run, c, ts, my_pos, n32, hi);
+        consume_tile<kBf16>(t, cur, cur + kKBytes, f, qf, o, m_ref, l_run, c, ts, my_pos, hi, !all_valid, [&] {
+            if (has_next) load_v_tile(ts + kTileK, next + kKBytes);
+        });
         FLASH_STAMP(t, ts / kTileK, 3);
-        if (ts + kTileK < kv_hi) {
-            // the other stage was last read one iteration ago; every wavefront has passed the
-            // barrier that ended that iteration
-            uint8_t* nk = lds + (stage ^ 1) * kStageBytes;
-            store_lds(nk, nk + kKBytes);
-            FLASH_STAMP(t, ts / kTileK, 4);
-            if (ts + 2 * kTileK < kv_hi) load_regs(ts + 2 * kTileK);
-        }
-        FLASH_STAMP(t, ts / kTileK, 5);
+    };
+    for (int ts = kv_lo; ts < kv_hi; ts += kTileK) {
+        // the other stage was last read one iteration ago; every wavefront has passed the barrier
+        // that ended that iteration
+        iteration(ts, lds + stage * kStageBytes, lds + (stage ^ 1) * kStageBytes);
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
         __syncthreads();
         FLASH_STAMP(t, ts / kTileK, 6);
         stage ^= 1;
@@ -452,7 +508,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                       : nullptr;
     }
 #endif
+#ifdef HIPATTN_FLASH_TRACE
+    long long w0 = 0, c0 = 0;
+    if (g_flash_wg_trace) {
+        w0 = wall_clock64();
+        c0 = (long long)__builtin_readcyclecounter();
+    }
+#endif
     run_tile<kBf16>(t, lds, p.scale);
+#ifdef HIPATTN_FLASH_TRACE
+    if (g_flash_wg_trace && threadIdx.x == 0) {
+        long long* r = g_flash_wg_trace + (int64_t)blockIdx.x * 8;
+        r[0] = w0;
+        r[1] = wall_clock64();
+        r[2] = c0;
+        r[3] = (long long)__builtin_readcyclecounter();
+        r[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID
+        r[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
+        r[6] = it.qt;
+    }
+#endif
 }
 
 // (not held to 256 registers: with the block-table addressing on top that would spill)
