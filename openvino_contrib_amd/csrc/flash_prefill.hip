@@ -79,6 +79,11 @@ struct Mfma<false> {
         const half2_t h = __builtin_convertvector((float2_t){lo, hi}, half2_t);
         return __builtin_bit_cast(uint32_t, h);
     }
+    // acc + lo + hi of a packed pair (v_dot2_f32_f16 against ones)
+    static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
+        const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, packed), ones, acc, false);
+    }
 };
 template <>
 struct Mfma<true> {
@@ -95,6 +100,12 @@ struct Mfma<true> {
         typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
         const bf16x2_t h = __builtin_convertvector((float2_t){lo, hi}, bf16x2_t);
         return __builtin_bit_cast(uint32_t, h);
+    }
+    // acc + lo + hi of a packed pair (v_dot2_f32_bf16 against ones)
+    static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, packed), ones, acc, false);
     }
 };
 
@@ -137,14 +148,14 @@ __device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key) {
     return (int64_t)pb * t.block_stride + (int64_t)(key & (t.block_size - 1)) * kRowBytes;
 }
 
+// Q fragment, multiplied by c = scale * log2(e) and rounded to the MFMA element type: the first
+// product then yields the exponents of the softmax directly.
 template <bool kBf16>
-__device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t, int row, int d0) {
+__device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t, int row, int d0, float c) {
     using vec8 = typename Mfma<kBf16>::vec8;
     uint4_t raw = {0u, 0u, 0u, 0u};
     if (row < t.rows) raw = *(const uint4_t*)(t.q + (int64_t)row * t.q_stride + d0);
     const bool q_is_bf16 = (t.q_dtype == HIPATTN_BF16);
-    if (q_is_bf16 == kBf16) return __builtin_bit_cast(vec8, raw);
-    // widen through fp32 and round to the MFMA element type
     uint4_t cv;
 #pragma unroll
     for (int w = 0; w < 4; w++) {
@@ -156,13 +167,21 @@ __device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t,
             lo = f16_bits_to_float((uint16_t)(raw[w] & 0xffffu));
             hi = f16_bits_to_float((uint16_t)(raw[w] >> 16));
         }
-        cv[w] = (uint32_t)Mfma<kBf16>::cvt(lo) | ((uint32_t)Mfma<kBf16>::cvt(hi) << 16);
+        cv[w] = Mfma<kBf16>::cvt2(lo * c, hi * c);
     }
     return __builtin_bit_cast(vec8, cv);
 }
 
 typedef __attribute__((address_space(3))) uint8_t lds_byte;
 typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// Lanes l and l + 32 exchange a value in the vector ALU (v_permlane32_swap: the upper half of the
+// first operand is swapped with the lower half of the second); both get (value of l, value of l + 32).
+__device__ __forceinline__ void pair_values(float x, float& lo, float& hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
 
 // LDS layout of a K or V tile: row r (a key) at byte r * 256, its 16-byte chunk c stored at chunk
 // position c ^ swz(r), with swz(r) = r % 16 for K and 4 * (r % 4) for V.
@@ -213,15 +232,24 @@ __device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte
 // their use: all sixteen K fragments before the first score MFMA, and the first half of the V^T
 // fragments right behind the score MFMAs, so that they arrive during the softmax arithmetic.
 //
-// Online softmax with a lazily updated reference: p = exp2((s - m_ref) c) is a valid numerator
-// for any reference m_ref as long as it cannot overflow, so the accumulators are rescaled only
-// when some row's maximum has grown by more than 2^8 (exp2 domain) over its reference, which
-// after the first few tiles is rare.
+// Online softmax with a lazily updated reference.  The scores come out of the first product as
+// exponents x = s c - ref, because Q carries the factor c and the accumulator of the product is
+// initialised with -ref (a 16-register tuple per lane: all sixteen belong to one query row), so
+// a probability costs one v_exp_f32 and half a conversion.  p = exp2(x) is a valid numerator for
+// any reference as long as it cannot overflow: ref is raised, and the accumulators rescaled,
+// only when some row's largest exponent exceeds 8, which after the first few tiles is rare.
+// Row sums are taken from the rounded probabilities, two per v_dot2 instruction.
+struct SoftmaxState {
+    float16_t neg_ref;  // -ref in every element
+    float l_run;        // this lane's half of the row sum
+    bool started;       // the row has met a key it may attend to
+};
+
 template <bool kBf16, typename AfterScores>
 __device__ __forceinline__ void consume_tile(const Tile& t, const lds_byte* k_lds, const lds_byte* v_lds,
                                              const FragOffsets& f, const typename Mfma<kBf16>::vec8 (&qf)[8],
-                                             float16_t (&o)[4], float& m_ref, float& l_run, float c, int ts, int my_pos,
-                                             int hi, bool masked, AfterScores&& after_scores) {
+                                             float16_t (&o)[4], SoftmaxState& st, int ts, int my_pos, int hi, bool masked,
+                                             AfterScores&& after_scores) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     typedef __attribute__((address_space(3))) vec8 lds_vec8;
@@ -234,11 +262,9 @@ __device__ __forceinline__ void consume_tile(const Tile& t, const lds_byte* k_ld
     __builtin_amdgcn_sched_barrier(0);
     float16_t s[2];
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++)
+    for (int mt = 0; mt < 2; mt++) s[mt] = M::mma(kf[mt][0], qf[0], st.neg_ref);
 #pragma unroll
-        for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; i++)
+    for (int i = 1; i < 8; i++)
 #pragma unroll
         for (int mt = 0; mt < 2; mt++) s[mt] = M::mma(kf[mt][i], qf[i], s[mt]);
     vec8 vf[2][4];
@@ -266,33 +292,40 @@ __device__ __forceinline__ void consume_tile(const Tile& t, const lds_byte* k_ld
     for (int mt = 0; mt < 2; mt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, s[mt][r]);
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));  // the row lives in lanes l and l + 32
-    const bool grow = m_tile * c > m_ref * c + 8.0f || (m_ref == -INFINITY && m_tile != -INFINITY);
-    if (__builtin_amdgcn_ballot_w64(grow)) {
-        const float m_new = fmaxf(m_ref, m_tile);
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // row with nothing to attend yet
-        const float alpha = fast_exp2((m_ref - m_safe) * c);        // exp2(-inf) = 0 the first time
-        l_run *= alpha;
+    {  // the row lives in lanes l and l + 32
+        float lo, hi2;
+        pair_values(m_tile, lo, hi2);
+        m_tile = fmaxf(lo, hi2);
+    }
+    const bool seen = m_tile != -INFINITY;
+    if (__builtin_amdgcn_ballot_w64(m_tile > 8.0f || (seen && !st.started))) {
+        // move the reference to this tile's maximum: up for a started row, anywhere for a new one
+        // (whose accumulators are still zero)
+        const float delta = st.started ? fmaxf(m_tile, 0.0f) : (seen ? m_tile : 0.0f);
+        const float alpha = fast_exp2(-fmaxf(delta, 0.0f));
+        st.l_run *= alpha;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) o[dt] *= alpha;
-        m_ref = m_new;
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) s[mt] -= delta;
+        st.neg_ref -= delta;
+        st.started = st.started || seen;
     }
-    const float neg_mc = (m_ref == -INFINITY) ? 0.0f : -m_ref * c;
-    float lsum = 0.0f;
+    float lsum = st.l_run;
     vec8 pf[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
         uint4_t pw;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            const float p0 = fast_exp2(fmaf(s[ks >> 1][(ks & 1) * 8 + 2 * w], c, neg_mc));
-            const float p1 = fast_exp2(fmaf(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1], c, neg_mc));
-            lsum += p0 + p1;
+            const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w]);
+            const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1]);
             pw[w] = M::cvt2(p0, p1);
+            lsum = M::add_pair(pw[w], lsum);
         }
         pf[ks] = __builtin_bit_cast(vec8, pw);
     }
-    l_run += lsum;
+    st.l_run = lsum;
     FLASH_STAMP(t, ts / kTileK, 2);
     // ---- O^T += V^T P^T
     vec8 vg[2][4];
@@ -349,7 +382,7 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, fl
     // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
     vec8 qf[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) qf[i] = load_q_frag<kBf16>(t, row, i * 16 + hi * 8);
+    for (int i = 0; i < 8; i++) qf[i] = load_q_frag<kBf16>(t, row, i * 16 + hi * 8, c);
 
     // key range this tile has to visit
     int kv_hi = t.kv_len;
@@ -363,7 +396,11 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, fl
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
-    float m_ref = -INFINITY, l_run = 0.0f;
+    SoftmaxState st;
+#pragma unroll
+    for (int r = 0; r < 16; r++) st.neg_ref[r] = 0.0f;
+    st.l_run = 0.0f;
+    st.started = false;
     const int my_pos = t.pos0 + row;  // position of this lane's query row
     const FragOffsets f = frag_offsets(lane);
 
@@ -407,13 +444,14 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, fl
     auto iteration = [&](int ts, const lds_byte* __restrict__ cur, lds_byte* __restrict__ next) {
         const bool has_next = ts + kTileK < kv_hi;
         FLASH_STAMP(t, ts / kTileK, 0);
-        if (has_next) load_k_tile(ts + kTileK, next);
+        if (has_next) {
+            load_k_tile(ts + kTileK, next);
+            load_v_tile(ts + kTileK, next + kKBytes);
+        }
         FLASH_STAMP(t, ts / kTileK, 5);
         const bool all_valid = (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
                                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
-        consume_tile<kBf16>(t, cur, cur + kKBytes, f, qf, o, m_ref, l_run, c, ts, my_pos, hi, !all_valid, [&] {
-            if (has_next) load_v_tile(ts + kTileK, next + kKBytes);
-        });
+        consume_tile<kBf16>(t, cur, cur + kKBytes, f, qf, o, st, ts, my_pos, hi, !all_valid, [&] {});
         FLASH_STAMP(t, ts / kTileK, 3);
     };
     for (int ts = kv_lo; ts < kv_hi; ts += kTileK) {
@@ -431,8 +469,10 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, fl
         for (int k = 0; k < 8; k++) t.trace[k] = t.clk.acc[k];
 #endif
     // ---- normalise and store
-    l_run += __shfl_xor(l_run, 32, 64);
-    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    float l_lo, l_hi;
+    pair_values(st.l_run, l_lo, l_hi);
+    const float l_row = l_lo + l_hi;
+    const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
     if (row < t.rows) {
         if (t.out_dtype == HIPATTN_F32)
             store_rows<HIPATTN_F32>(t, o, inv, row, hi);
