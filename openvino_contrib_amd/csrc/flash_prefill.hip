@@ -1,15 +1,24 @@
 // Flash-style attention for prefill on gfx950: dense v13::ScaledDotProductAttention and the
 // multi-token (chunked prefill) sequences of PagedAttentionExtension share one kernel body.
 //
-// A workgroup of four wavefronts owns 128 query rows of one query head (32 rows per
-// wavefront) and walks the keys in tiles of 64.  K and V tiles go from global memory straight
-// into LDS (global_load_lds_dwordx4: no staging registers, no LDS write instructions), both
-// row-major with the 16-byte chunks of a row XOR-swizzled so that fragment reads are free of
-// bank conflicts; the V^T operand is read with the transposing LDS load ds_read_b64_tr_b16.
-// LDS holds two stages: the loads of tile i+1 are issued at the top of iteration i into the
-// stage that tile i-1 occupied, with one workgroup barrier per tile.  The kernel is held to 256
-// registers so that two workgroups share a compute unit.  Both products run on
-// v_mfma_f32_32x32x16 (f16 or bf16) with fp32 accumulation:
+// A workgroup has eight wavefronts in two groups of four.  Each group owns 128 query rows (32
+// per wavefront) of one query head; the two groups work on two heads of the same K/V head (or on
+// two consecutive query tiles of one head), so they share every K and V tile.  Keys are walked
+// in tiles of 64.  K and V tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4: no staging registers, no LDS write instructions), row-major with
+// the 16-byte chunks of a row XOR-swizzled so that fragment reads are free of bank conflicts;
+// the V^T operand is read with the transposing LDS load ds_read_b64_tr_b16.  LDS holds a ring of
+// three K and three V stages, filled two tiles ahead.
+//
+// One wavefront of each group sits on every SIMD, and the two alternate between a matrix phase
+// (O += P V of one tile, then the scores of the next) and a vector phase (mask, running
+// reference, exp2, conversion and row sums of the scores just computed, plus the issue of the
+// global->LDS loads), separated by workgroup barriers: while one group feeds the matrix core the
+// other keeps the vector ALU busy, by construction rather than by chance.  A SIMD runs an MFMA
+// stream at full rate next to another wavefront's VALU stream, but a single wavefront cannot
+// overlap the two beyond a handful of instructions.
+//
+// Both products run on v_mfma_f32_32x32x16 (f16 or bf16) with fp32 accumulation:
 //   S^T = K Q^T   (M = 32 keys, N = 32 query rows, contraction over head_dim)
 //   O^T = V^T P^T (M = 32 head-dim rows, N = 32 query rows, contraction over keys)
 // Computing the scores transposed leaves each lane with 8 consecutive-in-operand keys of one
@@ -31,39 +40,61 @@ namespace hipattn {
 namespace flash {
 
 // Diagnostic build only (a probe that includes this file with HIPATTN_FLASH_TRACE defined):
-// lane 0 of selected wavefronts stores the shader clock at the phase boundaries of every tile.
+// thread 0 of every workgroup stores wall clock (100 MHz) and shader clock at entry and exit.
 #ifdef HIPATTN_FLASH_TRACE
-__device__ long long* g_flash_trace = nullptr;
-__device__ long long* g_flash_wg_trace = nullptr;  // per workgroup: wall start/end (100 MHz), cycles start/end, hw id
+__device__ long long* g_flash_wg_trace = nullptr;
+__device__ long long* g_flash_phase_trace = nullptr;  // per wavefront: 8 accumulated phase times (shader clocks)
+__device__ long long* g_flash_raw_trace = nullptr;    // workgroup 0: raw stamps of tiles 10 and 11, per wavefront
 struct PhaseClock {
     long long acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     long long last = 0;
+    long long raw[8];
+    int tile = 0;
 };
-// phase k = time since the previous stamp; totals are stored once, after the last tile
-#define FLASH_STAMP(t, tile, k)                                                   \
-    do {                                                                          \
-        __builtin_amdgcn_sched_barrier(0);                                        \
-        const long long stamp_ = (long long)__builtin_readcyclecounter();         \
-        __builtin_amdgcn_sched_barrier(0);                                        \
-        (t).clk.acc[k] += stamp_ - (t).clk.last;                                  \
-        (t).clk.last = stamp_;                                                    \
+// phase k = time since the previous stamp
+#define FLASH_STAMP(clk, k)                                               \
+    do {                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                \
+        const long long stamp_ = (long long)__builtin_readcyclecounter(); \
+        __builtin_amdgcn_sched_barrier(0);                                \
+        (clk).acc[k] += stamp_ - (clk).last;                              \
+        (clk).last = stamp_;                                              \
+        if ((clk).tile == 10) (clk).raw[k] = stamp_;                      \
     } while (0)
 #else
-#define FLASH_STAMP(t, tile, k) \
-    do {                        \
+#define FLASH_STAMP(clk, k) \
+    do {                    \
     } while (0)
 #endif
 
 constexpr int kD = 128;
-constexpr int kTileQ = 128;   // query rows per workgroup
+constexpr int kTileQ = 128;   // query rows per group of four wavefronts
 constexpr int kTileK = 64;    // keys per LDS tile
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
+constexpr int kStages = 3;    // ring of K stages and ring of V stages
 constexpr int kRowBytes = kD * 2;                // a K or V row in LDS: 16 chunks of 16 bytes
-constexpr int kKBytes = kTileK * kRowBytes;      // K part of a stage
-constexpr int kStageBytes = 2 * kKBytes;         // K tile + V tile
+constexpr int kKBytes = kTileK * kRowBytes;      // one K or V stage
+constexpr int kLdsBytes = 2 * kStages * kKBytes;
 
-#define HIPATTN_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-#define HIPATTN_GLOBAL_PTR(p) ((__attribute__((address_space(1))) void*)(p))
+// global -> LDS load of 16 bytes per lane: lane l's data lands at LDS byte lds_base + 16 l
+// (lds_base wave-uniform, carried in M0).  Issued as inline assembly on purpose: the compiler
+// treats the intrinsic form as a flat access that may touch LDS and from then on waits for all
+// outstanding LDS reads and loads at every use (s_waitcnt 0), which serialises the fragment
+// prefetch.  The waiting these loads need is done by hand (barrier_keeping_loads).
+typedef __attribute__((address_space(3))) uint8_t lds_byte;
+__device__ __forceinline__ void load_to_lds_16(const uint8_t* global_base, uint32_t lane_offset, lds_byte* lds_base) {
+    // global_base wave-uniform, lane_offset per lane
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(global_base), "s"((uint32_t)(uintptr_t)lds_base)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void load_to_lds_16(const uint8_t* lane_address, lds_byte* lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(lane_address), "s"((uint32_t)(uintptr_t)lds_base)
+                 : "memory", "m0");
+}
 
 template <bool kBf16>
 struct Mfma;
@@ -78,11 +109,6 @@ struct Mfma<false> {
         typedef float float2_t __attribute__((ext_vector_type(2)));
         const half2_t h = __builtin_convertvector((float2_t){lo, hi}, half2_t);
         return __builtin_bit_cast(uint32_t, h);
-    }
-    // acc + lo + hi of a packed pair (v_dot2_f32_f16 against ones)
-    static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
-        const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, packed), ones, acc, false);
     }
 };
 template <>
@@ -101,28 +127,22 @@ struct Mfma<true> {
         const bf16x2_t h = __builtin_convertvector((float2_t){lo, hi}, bf16x2_t);
         return __builtin_bit_cast(uint32_t, h);
     }
-    // acc + lo + hi of a packed pair (v_dot2_f32_bf16 against ones)
-    static __device__ __forceinline__ float add_pair(uint32_t packed, float acc) {
-        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-        const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, packed), ones, acc, false);
-    }
 };
 
-// What one workgroup works on.
+// What one group of four wavefronts works on.
 struct Tile {
     const uint16_t* q;   // first query row of the tile, this head
     int64_t q_stride;    // elements between consecutive query rows
     void* out;           // output base (element (0,0) of the tile's first row, this head)
     int64_t out_stride;
-    int rows;            // valid query rows (<= 128)
+    int rows;            // valid query rows (<= 128); 0: this group has nothing to do
     int pos0;            // sequence position of query row 0
     int kv_len;          // keys available
     int causal;
     int window;
     int q_dtype;         // HIPATTN_F16 / HIPATTN_BF16 (converted to the MFMA type when they differ)
     int out_dtype;
-    // keys / values
+    // keys / values: the same for both groups of a workgroup
     const uint8_t* k;
     const uint8_t* v;
     const int32_t* table;   // paged: this sequence's block ids; dense: nullptr
@@ -131,11 +151,21 @@ struct Tile {
     int64_t block_stride;   // paged: bytes between physical blocks
     int block_size;
     int block_shift;        // log2(block_size)
-#ifdef HIPATTN_FLASH_TRACE
-    long long* trace;
-    mutable PhaseClock clk;
-#endif
 };
+
+// Keys [lo, hi) a tile has to visit, lo rounded down to a tile boundary.
+__device__ __forceinline__ void key_range(const Tile& t, int& lo, int& hi) {
+    if (t.rows <= 0) {
+        lo = hi = 0;
+        return;
+    }
+    hi = t.kv_len;
+    if (t.causal) hi = min(hi, t.pos0 + t.rows);
+    lo = 0;
+    if (t.window > 0) lo = max(0, t.pos0 - t.window + 1);
+    lo = (lo / kTileK) * kTileK;
+    if (hi < lo) hi = lo;
+}
 
 // Byte offset of a key's row from t.k / t.v.  Keys past the end are redirected to the last valid
 // key and block ids outside the cache are clamped: such rows only ever meet a probability of
@@ -172,7 +202,6 @@ __device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t,
     return __builtin_bit_cast(vec8, cv);
 }
 
-typedef __attribute__((address_space(3))) uint8_t lds_byte;
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
 // Lanes l and l + 32 exchange a value in the vector ALU (v_permlane32_swap: the upper half of the
@@ -195,29 +224,30 @@ __device__ __forceinline__ void pair_values(float x, float& lo, float& hi) {
 // the group addressed, taken at 16-bit index i % 4: so lane i addresses row key0 + i/4, head-dim
 // d0 + 4 (i % 4) .. +3 (d0 = dt*32 + 16 * (group & 1), key0 = 16ks + 4 * (group >> 1)), and
 // receives V[key0 + j][d0 + i].  Two such reads, eight rows apart, make one fragment.
+//
+// Both fragment addresses are (one per-lane base) ^ (a compile-time constant): the swizzle term
+// of the lane sits in address bits that the base leaves zero.
 struct FragOffsets {
-    int k[8];  // + mt * 32 rows
-    int v[4];  // per dt; + ks * 16 rows (+ 8 rows for the second half)
+    int k;  // K fragment (mt, i):  (k ^ (i << 5)) + mt * 32 rows
+    int v;  // V^T fragment (ks, dt): (v ^ (dt << 6)) + ks * 16 rows (+ 8 rows for the second half)
 };
 
 __device__ __forceinline__ FragOffsets frag_offsets(int lane) {
     FragOffsets f;
-    const int n32 = lane & 31, hi = lane >> 5;
-#pragma unroll
-    for (int i = 0; i < 8; i++) f.k[i] = n32 * kRowBytes + (((2 * i + hi) ^ (n32 & 15)) << 4);
+    const int n32 = lane & 31, hi = lane >> 5, x = n32 & 15;
+    // chunk (2i + hi) ^ x = 2 (i ^ (x >> 1)) + (hi ^ (x & 1))
+    f.k = n32 * kRowBytes + ((x >> 1) << 5) + ((hi ^ (x & 1)) << 4);
     const int g = lane >> 4, i16 = lane & 15;
     const int vrow = 4 * (g >> 1) + (i16 >> 2);  // row % 4 == i16 / 4
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++)
-        f.v[dt] = vrow * kRowBytes + (((4 * dt + 2 * (g & 1) + ((i16 & 3) >> 1)) ^ (4 * (i16 >> 2))) << 4) + 8 * (i16 & 1);
+    // chunk (4dt + 2(g&1) + (i16 % 4) / 2) ^ 4 (i16 / 4) = 4 (dt ^ (i16 / 4)) + 2 (g & 1) + (i16 % 4) / 2
+    f.v = vrow * kRowBytes + ((i16 >> 2) << 6) + ((2 * (g & 1) + ((i16 & 3) >> 1)) << 4) + 8 * (i16 & 1);
     return f;
 }
 
 template <bool kBf16>
-__device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte* v_lds, const FragOffsets& f, int ks,
-                                                                  int dt) {
+__device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte* v_lds, int v_off, int ks, int dt) {
     typedef __attribute__((address_space(3))) short4_t lds_short4;
-    const lds_byte* p = v_lds + f.v[dt] + ks * 16 * kRowBytes;
+    const lds_byte* p = v_lds + (v_off ^ (dt << 6)) + ks * 16 * kRowBytes;
     const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)p);
     const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p + 8 * kRowBytes));
     typedef short short8_t __attribute__((ext_vector_type(8)));
@@ -225,56 +255,26 @@ __device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte
     return __builtin_bit_cast(typename Mfma<kBf16>::vec8, a);
 }
 
-// One 64-key tile against this wavefront's 32 query rows.  `masked` is false for tiles that every
-// query row of the workgroup sees completely (the common case).
-//
-// LDS latency is taken out of the MFMA chains by issuing fragment reads in batches ahead of
-// their use: all sixteen K fragments before the first score MFMA, and the first half of the V^T
-// fragments right behind the score MFMAs, so that they arrive during the softmax arithmetic.
-//
 // Online softmax with a lazily updated reference.  The scores come out of the first product as
 // exponents x = s c - ref, because Q carries the factor c and the accumulator of the product is
 // initialised with -ref (a 16-register tuple per lane: all sixteen belong to one query row), so
 // a probability costs one v_exp_f32 and half a conversion.  p = exp2(x) is a valid numerator for
 // any reference as long as it cannot overflow: ref is raised, and the accumulators rescaled,
 // only when some row's largest exponent exceeds 8, which after the first few tiles is rare.
-// Row sums are taken from the rounded probabilities, two per v_dot2 instruction.
 struct SoftmaxState {
     float16_t neg_ref;  // -ref in every element
     float l_run;        // this lane's half of the row sum
     bool started;       // the row has met a key it may attend to
 };
 
-template <bool kBf16, typename AfterScores>
-__device__ __forceinline__ void consume_tile(const Tile& t, const lds_byte* k_lds, const lds_byte* v_lds,
-                                             const FragOffsets& f, const typename Mfma<kBf16>::vec8 (&qf)[8],
-                                             float16_t (&o)[4], SoftmaxState& st, int ts, int my_pos, int hi, bool masked,
-                                             AfterScores&& after_scores) {
+// Mask, reference update and probabilities of the tile that starts at key ts (register r of s[mt]
+// is key ts + mt*32 + 8*(r/4) + 4*hi + r%4).  `masked` is false for tiles that every query row of
+// the group sees completely (the common case).
+template <bool kBf16>
+__device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], float16_t (&o)[4], SoftmaxState& st,
+                                             typename Mfma<kBf16>::vec8 (&pf)[4], int ts, int my_pos, int hi, bool masked) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
-    typedef __attribute__((address_space(3))) vec8 lds_vec8;
-    // ---- S^T = K Q^T
-    vec8 kf[2][8];
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++) kf[mt][i] = *(const lds_vec8*)(k_lds + f.k[i] + mt * 32 * kRowBytes);
-    __builtin_amdgcn_sched_barrier(0);
-    float16_t s[2];
-#pragma unroll
-    for (int mt = 0; mt < 2; mt++) s[mt] = M::mma(kf[mt][0], qf[0], st.neg_ref);
-#pragma unroll
-    for (int i = 1; i < 8; i++)
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++) s[mt] = M::mma(kf[mt][i], qf[i], s[mt]);
-    vec8 vf[2][4];
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) vf[ks][dt] = read_v_frag<kBf16>(v_lds, f, ks, dt);
-    after_scores();
-    FLASH_STAMP(t, ts / kTileK, 1);
-    // ---- mask (register r of tile mt is key ts + mt*32 + 8*(r/4) + 4*hi + r%4) and row maximum
     if (masked) {
 #pragma unroll
         for (int mt = 0; mt < 2; mt++)
@@ -312,7 +312,6 @@ __device__ __forceinline__ void consume_tile(const Tile& t, const lds_byte* k_ld
         st.started = st.started || seen;
     }
     float lsum = st.l_run;
-    vec8 pf[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
         uint4_t pw;
@@ -321,26 +320,102 @@ __device__ __forceinline__ void consume_tile(const Tile& t, const lds_byte* k_ld
             const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w]);
             const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1]);
             pw[w] = M::cvt2(p0, p1);
-            lsum = M::add_pair(pw[w], lsum);
+            lsum += p0 + p1;  // (not v_dot2: dot instructions wait for the matrix core, which the other group keeps busy)
         }
         pf[ks] = __builtin_bit_cast(vec8, pw);
     }
     st.l_run = lsum;
-    FLASH_STAMP(t, ts / kTileK, 2);
-    // ---- O^T += V^T P^T
-    vec8 vg[2][4];
+}
+
+// The fragments of a product are read from LDS in batches of four, each batch one batch of MFMAs
+// ahead of its use; sched_barrier keeps the compiler from sinking the reads back to their uses.
+template <bool kBf16>
+__device__ __forceinline__ void read_v_batch(const lds_byte* v_lds, const FragOffsets& f, int ks,
+                                             typename Mfma<kBf16>::vec8 (&vf)[4]) {
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int dt = 0; dt < 4; dt++) vf[dt] = read_v_frag<kBf16>(v_lds, f.v, ks, dt);
+}
+template <bool kBf16>
+__device__ __forceinline__ void read_k_batch(const lds_byte* k_lds, const FragOffsets& f, int b,
+                                             typename Mfma<kBf16>::vec8 (&kf)[4]) {  // k-steps 2b, 2b+1 of both key halves
+    typedef __attribute__((address_space(3))) typename Mfma<kBf16>::vec8 lds_vec8;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) vg[ks][dt] = read_v_frag<kBf16>(v_lds, f, 2 + ks, dt);
+    for (int u = 0; u < 4; u++)
+        kf[u] = *(const lds_vec8*)(k_lds + (f.k ^ ((2 * b + (u >> 1)) << 5)) + (u & 1) * 32 * kRowBytes);
+}
+
+// O^T += V^T P^T for one tile
+template <bool kBf16>
+__device__ __forceinline__ void tile_accumulate(const lds_byte* v_lds, const FragOffsets& f,
+                                                const typename Mfma<kBf16>::vec8 (&pf)[4], float16_t (&o)[4]) {
+    using M = Mfma<kBf16>;
+    using vec8 = typename M::vec8;
+    vec8 vf[2][4];
+    read_v_batch<kBf16>(v_lds, f, 0, vf[0]);
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int ks = 0; ks < 4; ks++) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks < 3) read_v_batch<kBf16>(v_lds, f, ks + 1, vf[(ks + 1) & 1]);
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) o[dt] = M::mma(vf[ks][dt], pf[ks], o[dt]);
+        for (int dt = 0; dt < 4; dt++) o[dt] = M::mma(vf[ks & 1][dt], pf[ks], o[dt]);
+    }
+}
+
+// S^T = K Q^T - ref for one 64-key tile
+template <bool kBf16>
+__device__ __forceinline__ void tile_scores(const lds_byte* k_lds, const FragOffsets& f,
+                                            const typename Mfma<kBf16>::vec8 (&qf)[8], const float16_t& neg_ref,
+                                            float16_t (&s)[2]) {
+    using M = Mfma<kBf16>;
+    using vec8 = typename M::vec8;
+    vec8 kf[2][4];
+    read_k_batch<kBf16>(k_lds, f, 0, kf[0]);
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int b = 0; b < 4; b++) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (b < 3) read_k_batch<kBf16>(k_lds, f, b + 1, kf[(b + 1) & 1]);
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) o[dt] = M::mma(vg[ks][dt], pf[2 + ks], o[dt]);
+        for (int u = 0; u < 4; u++) {
+            const int i = 2 * b + (u >> 1), mt = u & 1;
+            s[mt] = M::mma(kf[b & 1][u], qf[i], i == 0 ? neg_ref : s[mt]);
+        }
+    }
+}
+
+// The matrix phase of the steady state: O^T += V^T P^T for one tile, then the scores of the next;
+// the first K fragments are read while the last P V MFMAs run.
+template <bool kBf16>
+__device__ __forceinline__ void tile_accumulate_and_scores(const lds_byte* v_lds, const lds_byte* k_lds,
+                                                           const FragOffsets& f,
+                                                           const typename Mfma<kBf16>::vec8 (&pf)[4], float16_t (&o)[4],
+                                                           const typename Mfma<kBf16>::vec8 (&qf)[8],
+                                                           const float16_t& neg_ref, float16_t (&s)[2]) {
+    using M = Mfma<kBf16>;
+    using vec8 = typename M::vec8;
+    vec8 fr[3][4];  // batches b, b+1, b+2: reads run two batches (8 MFMAs) ahead of their use
+    auto read_batch = [&](int b) {
+        if (b < 4)
+            read_v_batch<kBf16>(v_lds, f, b, fr[b % 3]);
+        else
+            read_k_batch<kBf16>(k_lds, f, b - 4, fr[b % 3]);
+    };
+    read_batch(0);
+    read_batch(1);
+#pragma unroll
+    for (int b = 0; b < 8; b++) {  // batches 0..3: P V (ks = b); 4..7: scores (k-steps 2(b-4), 2(b-4)+1)
+        __builtin_amdgcn_sched_barrier(0);
+        if (b + 2 < 8) read_batch(b + 2);
+        if (b < 4) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) o[dt] = M::mma(fr[b % 3][dt], pf[b], o[dt]);
+        } else {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = 2 * (b - 4) + (u >> 1), mt = u & 1;
+                s[mt] = M::mma(fr[b % 3][u], qf[i], i == 0 ? neg_ref : s[mt]);
+            }
+        }
+    }
 }
 
 template <int kOutDtype>
@@ -366,30 +441,80 @@ __device__ __forceinline__ void store_rows(const Tile& t, const float16_t (&o)[4
         }
 }
 
-// lds: two stages of (K tile, V tile); stage (i+1)%2 is filled while tile i is consumed, so the
-// loop needs one workgroup barrier per tile.
+// Wave-uniform address of the 8 consecutive rows that start at key0 (a multiple of 8 below
+// kv_len): they lie in one block of a paged cache.
+__device__ __forceinline__ const uint8_t* row_group_base(const Tile& t, const uint8_t* base, int key0) {
+    if (t.table == nullptr) return base + (int64_t)key0 * kRowBytes;
+    const int pb = min(max(t.table[key0 >> t.block_shift], 0), t.num_blocks - 1);
+    return base + (int64_t)pb * t.block_stride + (int64_t)(key0 & (t.block_size - 1)) * kRowBytes;
+}
+
+// Workgroup barrier that lets the `keep` most recent global->LDS loads of this wavefront stay in
+// flight (__syncthreads would wait for all of them): s_waitcnt vmcnt(keep) lgkmcnt(0), then
+// s_barrier.  Loads complete in order, so everything issued earlier has landed in LDS.
+template <int kKeep>
+__device__ __forceinline__ void barrier_keeping() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | (kKeep & 15) | ((kKeep >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0, 2 or 4 (wave-uniform)
+    if (keep >= 4)
+        barrier_keeping<4>();
+    else if (keep >= 2)
+        barrier_keeping<2>();
+    else
+        barrier_keeping<0>();
+}
+
+// The loop of one wavefront.  t is the tile of this wavefront's group; [kv_lo, kv_hi) is the key
+// range of the workgroup (the union of both groups' ranges, kv_lo a multiple of 64).
+//
+// Phases, numbered from 0 and separated by workgroup barriers: group 0 computes the scores of
+// tile j in phase 2j, their softmax in phase 2j+1 and P V in phase 2j+2 (together with the
+// scores of tile j+1); group 1 does the same one phase later.  K(j) is therefore read in phases
+// 2j and 2j+1, V(j) in phases 2j+2 and 2j+3.  Load batch B(x) = {K(x+2), V(x+1)} goes into the
+// ring stages of K(x-1) and V(x-2); every wavefront issues its rows of B(x) in a vector phase
+// (group 0 in phase 2x+1, group 1 in phase 2x), and at each barrier waits for all of its loads
+// except the latest batch, which puts B(x) in LDS two phases before its first use.
 template <bool kBf16>
-__device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, float scale) {
+__device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     lds_byte* const lds = (lds_byte*)lds_generic;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int group = wave >> 2;
     const int n32 = lane & 31, hi = lane >> 5;
-    const int row = wave * 32 + n32;  // query row inside the tile
+    const int row = (wave & 3) * 32 + n32;  // query row inside the group's tile
     const float c = scale * kLog2e;
+    const int n = (kv_hi - kv_lo + kTileK - 1) / kTileK;  // tiles of the workgroup
+    if (n <= 0) {
+        // nothing to attend to: rows of zeros (the reference's softmax over an empty set is undefined)
+        if (row < t.rows) {
+            float16_t z[4];
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) z[dt][r] = 0.0f;
+            if (t.out_dtype == HIPATTN_F32)
+                store_rows<HIPATTN_F32>(t, z, 0.0f, row, hi);
+            else
+                store_rows<HIPATTN_F16>(t, z, 0.0f, row, hi);  // zero bits are the same in f16 and bf16
+        }
+        return;
+    }
+    auto unmasked = [&](int j) {
+        const int ts = kv_lo + j * kTileK;
+        return (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
+               (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
+    };
 
     // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
     vec8 qf[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) qf[i] = load_q_frag<kBf16>(t, row, i * 16 + hi * 8, c);
-
-    // key range this tile has to visit
-    int kv_hi = t.kv_len;
-    if (t.causal) kv_hi = min(kv_hi, t.pos0 + t.rows);
-    int kv_lo = 0;
-    if (t.window > 0) kv_lo = max(0, t.pos0 - t.window + 1);
-    kv_lo = (kv_lo / kTileK) * kTileK;
 
     float16_t o[4];
 #pragma unroll
@@ -405,69 +530,108 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, fl
     const FragOffsets f = frag_offsets(lane);
 
     // global -> LDS: one instruction moves four rows (64 lanes x 16 bytes, LDS address = wave-uniform
-    // base + lane * 16); wavefront w issues the four instructions of rows 16w .. 16w + 15 of the K
-    // tile and of the V tile.  Lane l fills chunk position l % 16 of row 16w + 4k + l / 16, i.e. it
-    // fetches chunk (l % 16) ^ swz(row).
+    // base + lane * 16); wavefront w issues the two instructions of rows 8w .. 8w + 7 of a K or V
+    // tile.  Lane l fills chunk position l % 16 of row r = 8w + 4k + l / 16, i.e. it fetches chunk
+    // (l % 16) ^ swz(r): for K that is ((l%16) ^ (l/16) ^ 8(w%2)) ^ 4k, for V (l%16) ^ 4(l/16).
     const int lrow = lane >> 4, lpos = lane & 15;
-    auto load_k_tile = [&](int tile_start, lds_byte* k_lds) {
+    const uint32_t k_lane = (uint32_t)(((lpos ^ lrow ^ (8 * (wave & 1))) << 4) + lrow * kRowBytes);
+    const uint32_t v_lane = (uint32_t)(((lpos ^ (4 * lrow)) << 4) + lrow * kRowBytes);
+    lds_byte* const k_ring = lds;
+    lds_byte* const v_ring = lds + kStages * kKBytes;
+    // this wavefront's rows of tile j into `stage`; returns the number of instructions issued
+    auto load_rows = [&](bool is_k, int j, lds_byte* stage) -> int {
+        if (j >= n) return 0;
+        const uint8_t* base = is_k ? t.k : t.v;
+        lds_byte* const dst = stage + 8 * wave * kRowBytes;
+        const int key0 = kv_lo + j * kTileK + 8 * wave;
+        if (key0 + 8 <= t.kv_len) {
+            const uint8_t* gb = row_group_base(t, base, key0);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int r = 16 * wave + 4 * k + lrow;
-            const int64_t off = kv_row_offset(t, tile_start + r) + ((lpos ^ (r & 15)) << 4);
-            __builtin_amdgcn_global_load_lds(HIPATTN_GLOBAL_PTR(t.k + off), HIPATTN_LDS_PTR(k_lds + (16 * wave + 4 * k) * kRowBytes),
-                                             16, 0, 0);
-        }
-    };
-    auto load_v_tile = [&](int tile_start, lds_byte* v_lds) {
+            for (int k = 0; k < 2; k++) {
+                const uint32_t off = (is_k ? (k_lane ^ (uint32_t)(k << 6)) : v_lane) + (uint32_t)(4 * k * kRowBytes);
+                load_to_lds_16(gb, off, dst + 4 * k * kRowBytes);
+            }
+        } else {  // the rows at the end of the sequence: per-lane clamped
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int r = 16 * wave + 4 * k + lrow;
-            const int64_t off = kv_row_offset(t, tile_start + r) + ((lpos ^ (4 * (r & 3))) << 4);
-            __builtin_amdgcn_global_load_lds(HIPATTN_GLOBAL_PTR(t.v + off), HIPATTN_LDS_PTR(v_lds + (16 * wave + 4 * k) * kRowBytes),
-                                             16, 0, 0);
+            for (int k = 0; k < 2; k++) {
+                const int r = 8 * (wave & 1) + 4 * k + lrow;
+                const int chunk = is_k ? (lpos ^ r) : (lpos ^ (4 * lrow));
+                const int64_t off = kv_row_offset(t, key0 + 4 * k + lrow) + (chunk << 4);
+                load_to_lds_16(base + off, dst + 4 * k * kRowBytes);
+            }
         }
+        return 2;
     };
+    auto k_stage = [&](int j) { return k_ring + (j % kStages) * kKBytes; };
+    auto v_stage = [&](int j) { return v_ring + (j % kStages) * kKBytes; };
 
-    if (kv_lo < kv_hi) {
-        load_k_tile(kv_lo, lds);
-        load_v_tile(kv_lo, lds + kKBytes);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's rows are in LDS
-    __syncthreads();
-    int stage = 0;
+    // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
+    load_rows(true, 0, k_stage(0));
+    load_rows(false, 0, v_stage(0));
+    load_rows(true, 1, k_stage(1));
+    int recent = 0;
+    if (group == 1) recent = load_rows(true, 2, k_stage(2)) + load_rows(false, 1, v_stage(1));
+    barrier_keeping_loads(recent);
+    if (group == 1) barrier_keeping_loads(recent);  // group 1 sits out phase 0
+
+    float16_t s[2];
+    vec8 pf[4];
+    tile_scores<kBf16>(k_stage(0), f, qf, st.neg_ref, s);
+    barrier_keeping_loads(recent);
 #ifdef HIPATTN_FLASH_TRACE
-    t.clk.last = (long long)__builtin_readcyclecounter();
+    PhaseClock clk;
+    clk.last = (long long)__builtin_readcyclecounter();
 #endif
-    // `cur` and `next` are the two stages: the restrict qualifiers tell the compiler that the LDS
-    // writes of the asynchronous loads cannot alias the fragment reads of the same iteration, so
-    // that it does not wait for the loads before every LDS read.
-    auto iteration = [&](int ts, const lds_byte* __restrict__ cur, lds_byte* __restrict__ next) {
-        const bool has_next = ts + kTileK < kv_hi;
-        FLASH_STAMP(t, ts / kTileK, 0);
-        if (has_next) {
-            load_k_tile(ts + kTileK, next);
-            load_v_tile(ts + kTileK, next + kKBytes);
-        }
-        FLASH_STAMP(t, ts / kTileK, 5);
-        const bool all_valid = (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
-                               (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
-        consume_tile<kBf16>(t, cur, cur + kKBytes, f, qf, o, st, ts, my_pos, hi, !all_valid, [&] {});
-        FLASH_STAMP(t, ts / kTileK, 3);
+    // The two phases of tile j.  Both groups run every tile of the workgroup's key range: a tile
+    // outside a group's own range is fully masked and contributes probabilities of zero.  The
+    // restrict qualifiers tell the compiler that the LDS writes of the asynchronous loads cannot
+    // alias the fragment reads, so that it does not wait for all loads before every LDS read; the
+    // barriers do the waiting that is needed.
+    auto two_phases = [&](int j, bool last, const lds_byte* __restrict__ k_next, const lds_byte* __restrict__ v_cur,
+                          lds_byte* __restrict__ k_fill, lds_byte* __restrict__ v_fill) {
+        // ---- vector phase
+#ifdef HIPATTN_FLASH_TRACE
+        clk.tile = j;
+#endif
+        FLASH_STAMP(clk, 0);
+        recent = load_rows(true, j + group + 2, k_fill) + load_rows(false, j + group + 1, v_fill);
+        FLASH_STAMP(clk, 1);
+        tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
+        // (the probabilities are complete before the barrier: the compiler may not move their
+        // arithmetic into the matrix phase)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) asm volatile("" : "+v"(pf[ks]));
+        FLASH_STAMP(clk, 2);
+        // the matrix phase runs at raised priority (set before the barrier, so that it holds from
+        // the first instruction after it): otherwise the other group's instruction stream, which
+        // never stalls for long, keeps this wavefront's MFMAs from issuing
+        __builtin_amdgcn_s_setprio(3);
+        barrier_keeping_loads(recent);
+        FLASH_STAMP(clk, 3);
+        // ---- matrix phase
+        if (!last)
+            tile_accumulate_and_scores<kBf16>(v_cur, k_next, f, pf, o, qf, st.neg_ref, s);
+        else
+            tile_accumulate<kBf16>(v_cur, f, pf, o);
+        __builtin_amdgcn_s_setprio(0);
+        FLASH_STAMP(clk, 5);
+        barrier_keeping_loads(recent);
+        FLASH_STAMP(clk, 6);
     };
-    for (int ts = kv_lo; ts < kv_hi; ts += kTileK) {
-        // the other stage was last read one iteration ago; every wavefront has passed the barrier
-        // that ended that iteration
-        iteration(ts, lds + stage * kStageBytes, lds + (stage ^ 1) * kStageBytes);
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-        __syncthreads();
-        FLASH_STAMP(t, ts / kTileK, 6);
-        stage ^= 1;
-    }
-
+    for (int j = 0; j < n - 1; j++)
+        two_phases(j, false, k_stage(j + 1), v_stage(j), k_stage(j + group + 2), v_stage(j + group + 1));
+    two_phases(n - 1, true, k_stage(n), v_stage(n - 1), k_stage(n + group + 1), v_stage(n + group));
+    if (group == 0) barrier_keeping_loads(0);  // as many barriers as group 1
 #ifdef HIPATTN_FLASH_TRACE
-    if (t.trace)
-        for (int k = 0; k < 8; k++) t.trace[k] = t.clk.acc[k];
+    if (g_flash_phase_trace && lane == 0) {
+        long long* r = g_flash_phase_trace + ((int64_t)blockIdx.x * 8 + wave) * 8;
+        for (int k = 0; k < 7; k++) r[k] = clk.acc[k];
+        r[7] = n;
+    }
+    if (g_flash_raw_trace && lane == 0 && blockIdx.x == 0 && n >= 12)
+        for (int k = 0; k < 8; k++) g_flash_raw_trace[wave * 16 + k] = clk.raw[k];
 #endif
+
     // ---- normalise and store
     float l_lo, l_hi;
     pair_values(st.l_run, l_lo, l_hi);
@@ -485,40 +649,40 @@ __device__ __forceinline__ void run_tile(const Tile& t, uint8_t* lds_generic, fl
 
 // Launch index -> work item: workgroups go to the eight XCDs round-robin by launch index and
 // each XCD has its own L2, so index i becomes item (i % 8) * (n / 8) + i / 8.  An XCD then walks
-// a contiguous range of items ordered (batch, kv head, query tile descending, query head in
-// group): the workgroups resident on it at one time share one K/V head, which stays in that L2,
-// and the heaviest (latest) causal tiles of a head come first.
-struct SdpaItem {
-    int b, h, qt;
-};
-__device__ __forceinline__ SdpaItem sdpa_item(const SdpaParams& p, int n_tiles) {
+// a contiguous range of items ordered (batch, kv head, query tile descending, pair): the
+// workgroups resident on it at one time share one K/V head, which stays in that L2, and the
+// heaviest (latest) causal tiles of a head come first.  With an even number of query heads per
+// kv head the two groups of a workgroup take two heads at the same query tile; otherwise they
+// take two consecutive query tiles of one head.
+__device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) {
     const int G = p.num_heads_q / p.num_heads_kv;
+    const int n_qt = (p.len_q + kTileQ - 1) / kTileQ;
+    const bool pair_heads = (G & 1) == 0;
+    const int slots = pair_heads ? n_qt : (n_qt + 1) / 2;  // query positions of a head's workgroups
+    const int lanes = pair_heads ? G / 2 : G;              // workgroups per query position
     const int n_items = (int)gridDim.x;
     int item = (int)blockIdx.x;
     if ((n_items & 7) == 0) item = (item & 7) * (n_items >> 3) + (item >> 3);
-    SdpaItem it;
-    it.qt = n_tiles - 1 - (item / G) % n_tiles;
-    it.h = ((item / (G * n_tiles)) % p.num_heads_kv) * G + item % G;
-    it.b = item / (G * n_tiles * p.num_heads_kv);
-    return it;
-}
-
-__device__ __forceinline__ Tile sdpa_tile(const SdpaParams& p, const SdpaItem& it, int tile_rows) {
-    const int G = p.num_heads_q / p.num_heads_kv;
+    const int li = item % lanes;
+    const int slot = slots - 1 - (item / lanes) % slots;
+    const int hkv = (item / (lanes * slots)) % p.num_heads_kv;
+    const int b = item / (lanes * slots * p.num_heads_kv);
+    const int h = hkv * G + (pair_heads ? 2 * li + group : li);
+    const int qt = pair_heads ? slot : 2 * slot + group;
     Tile t;
-    const int64_t qoff = (((int64_t)it.b * p.num_heads_q + it.h) * p.len_q + (int64_t)it.qt * tile_rows) * kD;
+    const int64_t qoff = (((int64_t)b * p.num_heads_q + h) * p.len_q + (int64_t)min(qt, n_qt - 1) * kTileQ) * kD;
     t.q = (const uint16_t*)p.q + qoff;
     t.q_stride = kD;
     t.out = (uint16_t*)p.out + qoff;
     t.out_stride = kD;
-    t.rows = min(tile_rows, p.len_q - it.qt * tile_rows);
-    t.pos0 = it.qt * tile_rows;
+    t.rows = qt < n_qt ? min(kTileQ, p.len_q - qt * kTileQ) : 0;
+    t.pos0 = qt * kTileQ;
     t.kv_len = p.len_kv;
     t.causal = p.causal;
     t.window = 0;
     t.q_dtype = p.dtype;
     t.out_dtype = p.dtype;
-    const int64_t kvoff = ((int64_t)it.b * p.num_heads_kv + it.h / G) * p.len_kv * (kD * 2);
+    const int64_t kvoff = ((int64_t)b * p.num_heads_kv + hkv) * p.len_kv * (kD * 2);
     t.k = (const uint8_t*)p.k + kvoff;
     t.v = (const uint8_t*)p.v + kvoff;
     t.table = nullptr;
@@ -531,23 +695,28 @@ __device__ __forceinline__ Tile sdpa_tile(const SdpaParams& p, const SdpaItem& i
 }
 
 template <bool kBf16>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
-#ifdef HIPATTN_FLASH_LDS_PAD  // diagnostic: forces one workgroup per compute unit
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes + HIPATTN_FLASH_LDS_PAD];
-#else
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
-#endif
-    const int n_tiles = (p.len_q + kTileQ - 1) / kTileQ;
-    const SdpaItem it = sdpa_item(p, n_tiles);
-    Tile t = sdpa_tile(p, it, kTileQ);
-#ifdef HIPATTN_FLASH_TRACE
-    {
-        const int wg = it.h + p.num_heads_q * it.b;
-        t.trace = (g_flash_trace && it.qt == n_tiles - 1 && (threadIdx.x & 63) == 0)
-                      ? g_flash_trace + (int64_t)(wg * 4 + (threadIdx.x >> 6)) * 8
-                      : nullptr;
+__device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t* lds, float scale) {
+    int lo0, hi0, lo1, hi1;
+    key_range(t0, lo0, hi0);
+    key_range(t1, lo1, hi1);
+    int kv_lo, kv_hi;
+    if (hi0 <= lo0) {
+        kv_lo = lo1;
+        kv_hi = hi1;
+    } else if (hi1 <= lo1) {
+        kv_lo = lo0;
+        kv_hi = hi0;
+    } else {
+        kv_lo = min(lo0, lo1);
+        kv_hi = max(hi0, hi1);
     }
-#endif
+    const int group = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
+    run_pair<kBf16>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
+}
+
+template <bool kBf16>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
 #ifdef HIPATTN_FLASH_TRACE
     long long w0 = 0, c0 = 0;
     if (g_flash_wg_trace) {
@@ -555,7 +724,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         c0 = (long long)__builtin_readcyclecounter();
     }
 #endif
-    run_tile<kBf16>(t, lds, p.scale);
+    const Tile t0 = sdpa_group_tile(p, 0), t1 = sdpa_group_tile(p, 1);
+    run_both<kBf16>(t0, t1, lds, p.scale);
 #ifdef HIPATTN_FLASH_TRACE
     if (g_flash_wg_trace && threadIdx.x == 0) {
         long long* r = g_flash_wg_trace + (int64_t)blockIdx.x * 8;
@@ -565,30 +735,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         r[3] = (long long)__builtin_readcyclecounter();
         r[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID
         r[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
-        r[6] = it.qt;
+        r[6] = t0.pos0 / kTileQ;
     }
 #endif
 }
 
-// (not held to 256 registers: with the block-table addressing on top that would spill)
-template <bool kBf16>
-__global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
-    const int total = p.tile_prefix[p.num_seqs];
-    const int tile_id = total - 1 - (int)blockIdx.x;
-    if (tile_id < 0) return;
-    // sequence owning this tile: largest s with tile_prefix[s] <= tile_id
-    int lo = 0, hi_s = p.num_seqs;
-    while (hi_s - lo > 1) {
-        const int mid = (lo + hi_s) >> 1;
-        if (p.tile_prefix[mid] <= tile_id)
-            lo = mid;
-        else
-            hi_s = mid;
-    }
-    const int s = lo;
-    const int qt = tile_id - p.tile_prefix[s];
-    const int h = blockIdx.y;
+// One workgroup per (128-row query tile of a multi-token sequence, pair of query heads).  With an
+// odd number of query heads per kv head the second group has no work and only helps loading.
+__device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, int qt, int h, bool has_work) {
     const int G = p.num_heads_q / p.num_heads_kv;
     const int t0 = p.subsequence_begins[s];
     const int qlen = p.subsequence_begins[s + 1] - t0;
@@ -601,7 +755,7 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) 
     t.q_stride = (int64_t)p.num_heads_q * kD;
     t.out = (p.out_dtype == HIPATTN_F32) ? (void*)((float*)p.out + row0 * kD) : (void*)((uint16_t*)p.out + row0 * kD);
     t.out_stride = (int64_t)p.num_heads_q * kD;
-    t.rows = min(kTileQ, qlen - qt * kTileQ);
+    t.rows = has_work ? min(kTileQ, qlen - qt * kTileQ) : 0;
     t.pos0 = past + qt * kTileQ;
     t.kv_len = min(past + qlen, table_len * p.block_size);
     t.causal = 1;
@@ -617,10 +771,32 @@ __global__ __launch_bounds__(kThreads) void paged_prefill_kernel(PagedParams p) 
     t.block_stride = (int64_t)p.num_heads_kv * p.block_size * (kD * 2);
     t.block_size = p.block_size;
     t.block_shift = __builtin_ctz(p.block_size);
-#ifdef HIPATTN_FLASH_TRACE
-    t.trace = nullptr;
-#endif
-    run_tile<kBf16>(t, lds, p.scale);
+    return t;
+}
+
+template <bool kBf16>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+    const int total = p.tile_prefix[p.num_seqs];
+    const int tile_id = total - 1 - (int)blockIdx.x;
+    if (tile_id < 0) return;
+    // sequence owning this tile: largest s with tile_prefix[s] <= tile_id
+    int lo = 0, hi_s = p.num_seqs;
+    while (hi_s - lo > 1) {
+        const int mid = (lo + hi_s) >> 1;
+        if (p.tile_prefix[mid] <= tile_id)
+            lo = mid;
+        else
+            hi_s = mid;
+    }
+    const int s = lo;
+    const int qt = tile_id - p.tile_prefix[s];
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const bool pair_heads = (G & 1) == 0;
+    const int h0 = pair_heads ? 2 * (int)blockIdx.y : (int)blockIdx.y;
+    const Tile t0 = paged_group_tile(p, s, qt, h0, true);
+    const Tile t1 = paged_group_tile(p, s, qt, pair_heads ? h0 + 1 : h0, pair_heads);
+    run_both<kBf16>(t0, t1, lds, p.scale);
 }
 
 }  // namespace flash
@@ -631,8 +807,11 @@ bool sdpa_flash_supported(const SdpaParams& p) {
 
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe) {
     if (p.batch == 0 || p.len_q == 0) return hipSuccess;
-    const int n_tiles = (p.len_q + flash::kTileQ - 1) / flash::kTileQ;
-    dim3 grid(n_tiles * p.num_heads_q * p.batch);
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const int n_qt = (p.len_q + flash::kTileQ - 1) / flash::kTileQ;
+    const bool pair_heads = (G & 1) == 0;
+    const int per_kv_head = pair_heads ? (G / 2) * n_qt : G * ((n_qt + 1) / 2);
+    dim3 grid(per_kv_head * p.num_heads_kv * p.batch);
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     if (p.dtype == HIPATTN_BF16)
         hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
@@ -644,7 +823,8 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
 }
 
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
-    dim3 grid(p.max_q_tiles, p.num_heads_q);
+    const int G = p.num_heads_q / p.num_heads_kv;
+    dim3 grid(p.max_q_tiles, (G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q);
     if (p.cache_dtype == HIPATTN_BF16)
         hipLaunchKernelGGL(flash::paged_prefill_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
     else
