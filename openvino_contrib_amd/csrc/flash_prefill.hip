@@ -609,10 +609,17 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         barrier_keeping_loads(recent);
         FLASH_STAMP(clk, 3);
         // ---- matrix phase
+        // fragment addresses of this tile: per-lane offset + stage address, so that every read is
+        // one XOR with a constant plus an immediate offset (the stage addresses are multiples of
+        // 16 KB and leave the XORed bits alone)
+        FragOffsets fs;
+        fs.k = f.k + (int)(uintptr_t)k_next;
+        fs.v = f.v + (int)(uintptr_t)v_cur;
+        const lds_byte* const zero = (const lds_byte*)0;
         if (!last)
-            tile_accumulate_and_scores<kBf16>(v_cur, k_next, f, pf, o, qf, st.neg_ref, s);
+            tile_accumulate_and_scores<kBf16>(zero, zero, fs, pf, o, qf, st.neg_ref, s);
         else
-            tile_accumulate<kBf16>(v_cur, f, pf, o);
+            tile_accumulate<kBf16>(zero, fs, pf, o);
         __builtin_amdgcn_s_setprio(0);
         FLASH_STAMP(clk, 5);
         barrier_keeping_loads(recent);
@@ -716,7 +723,7 @@ __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t
 
 template <bool kBf16>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
 #ifdef HIPATTN_FLASH_TRACE
     long long w0 = 0, c0 = 0;
     if (g_flash_wg_trace) {
@@ -776,7 +783,7 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
 
 template <bool kBf16>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
     const int total = p.tile_prefix[p.num_seqs];
     const int tile_id = total - 1 - (int)blockIdx.x;
     if (tile_id < 0) return;
