@@ -442,10 +442,10 @@ __device__ __forceinline__ void store_rows(const Tile& t, const float16_t (&o)[4
 }
 
 // Wave-uniform address of the 8 consecutive rows that start at key0 (a multiple of 8 below
-// kv_len): they lie in one block of a paged cache.
-__device__ __forceinline__ const uint8_t* row_group_base(const Tile& t, const uint8_t* base, int key0) {
+// kv_len): they lie in one block of a paged cache, whose table entry is `entry`.
+__device__ __forceinline__ const uint8_t* row_group_base(const Tile& t, const uint8_t* base, int key0, int entry) {
     if (t.table == nullptr) return base + (int64_t)key0 * kRowBytes;
-    const int pb = min(max(t.table[key0 >> t.block_shift], 0), t.num_blocks - 1);
+    const int pb = min(max(entry, 0), t.num_blocks - 1);
     return base + (int64_t)pb * t.block_stride + (int64_t)(key0 & (t.block_size - 1)) * kRowBytes;
 }
 
@@ -539,13 +539,14 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     lds_byte* const k_ring = lds;
     lds_byte* const v_ring = lds + kStages * kKBytes;
     // this wavefront's rows of tile j into `stage`; returns the number of instructions issued
-    auto load_rows = [&](bool is_k, int j, lds_byte* stage) -> int {
+    // (entry: the block table entry of these rows, see table_entry below; ignored for dense K/V)
+    auto load_rows = [&](bool is_k, int j, lds_byte* stage, int entry) -> int {
         if (j >= n) return 0;
         const uint8_t* base = is_k ? t.k : t.v;
         lds_byte* const dst = stage + 8 * wave * kRowBytes;
         const int key0 = kv_lo + j * kTileK + 8 * wave;
         if (key0 + 8 <= t.kv_len) {
-            const uint8_t* gb = row_group_base(t, base, key0);
+            const uint8_t* gb = row_group_base(t, base, key0, entry);
 #pragma unroll
             for (int k = 0; k < 2; k++) {
                 const uint32_t off = (is_k ? (k_lane ^ (uint32_t)(k << 6)) : v_lane) + (uint32_t)(4 * k * kRowBytes);
@@ -562,15 +563,32 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         }
         return 2;
     };
+    // Block table entry of this wavefront's rows of tile j (0 when there is none), read through
+    // the scalar cache in the vector phase, so that no scalar load is outstanding during a
+    // matrix phase (which would turn every partial wait for LDS fragments into a full one).
+    // (As inline assembly, because behind the compiler fences of the barriers an ordinary load of
+    // the table becomes a vector load that is waited for at once, together with every load to LDS
+    // in flight.  The wait for the scalar load is part of the statement: the compiler takes the
+    // output register as written when the statement ends and may reuse it at any time after.)
+    auto table_entry = [&](int j) -> int {
+        const int key0 = kv_lo + j * kTileK + 8 * wave;
+        if (t.table == nullptr || j >= n || key0 + 8 > t.kv_len) return 0;
+        int entry;
+        asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(entry) : "s"(t.table + (key0 >> t.block_shift)));
+        return entry;
+    };
     auto k_stage = [&](int j) { return k_ring + (j % kStages) * kKBytes; };
     auto v_stage = [&](int j) { return v_ring + (j % kStages) * kKBytes; };
 
     // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
-    load_rows(true, 0, k_stage(0));
-    load_rows(false, 0, v_stage(0));
-    load_rows(true, 1, k_stage(1));
+    const int e0 = table_entry(0), e1 = table_entry(1), e2 = table_entry(2), e3 = table_entry(3);
+    load_rows(true, 0, k_stage(0), e0);
+    load_rows(false, 0, v_stage(0), e0);
+    load_rows(true, 1, k_stage(1), e1);
     int recent = 0;
-    if (group == 1) recent = load_rows(true, 2, k_stage(2)) + load_rows(false, 1, v_stage(1));
+    if (group == 1) recent = load_rows(true, 2, k_stage(2), e2) + load_rows(false, 1, v_stage(1), e1);
+    // entries of the tiles the first iteration loads: K(group + 2) and V(group + 1)
+    int entry_v = group ? e2 : e1, entry_k = group ? e3 : e2;
     barrier_keeping_loads(recent);
     if (group == 1) barrier_keeping_loads(recent);  // group 1 sits out phase 0
 
@@ -594,7 +612,9 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         clk.tile = j;
 #endif
         FLASH_STAMP(clk, 0);
-        recent = load_rows(true, j + group + 2, k_fill) + load_rows(false, j + group + 1, v_fill);
+        recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
+        entry_v = entry_k;  // the next iteration loads V of the tile whose K was loaded now
+        entry_k = table_entry(j + group + 3);
         FLASH_STAMP(clk, 1);
         tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
         // (the probabilities are complete before the barrier: the compiler may not move their
