@@ -111,7 +111,10 @@ def test_sdpa_golden_fixture_on_gpu(hip):
     ((1, 1, 1, 1, 1, 128), True), ((1, 2, 1, 63, 63, 128), True), ((1, 2, 2, 64, 64, 128), False),
     ((1, 4, 2, 65, 65, 128), True), ((2, 4, 1, 128, 128, 128), True), ((1, 2, 1, 129, 129, 128), True),
     ((1, 8, 2, 300, 300, 128), True), ((1, 2, 1, 200, 1000, 128), False), ((1, 2, 1, 1000, 200, 128), True),
-    ((1, 4, 4, 1000, 1000, 128), True), ((1, 2, 2, 77, 500, 128), True)])
+    ((1, 4, 4, 1000, 1000, 128), True), ((1, 2, 2, 77, 500, 128), True),
+    # odd GQA ratios pair two query tiles of one head in a workgroup; 5 tiles leave one group idle
+    ((1, 6, 2, 400, 400, 128), True), ((2, 3, 1, 260, 700, 128), False), ((1, 3, 3, 600, 600, 128), True),
+    ((1, 2, 1, 1600, 1600, 128), True)])
 def test_sdpa_flash(hip, oracle, dtype, shape, causal):
     announce("sdpa flash", dtype, shape, causal)
     B, Hq, Hkv, Lq, Lk, D = shape
@@ -245,10 +248,11 @@ def test_paged_block_permutation_is_bit_identical(hip):
 # ----------------------------------------------------------------- mixed prefill + decode
 @pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.F16, W.F16, 0), (W.BF16, W.F16, 0), (W.BF16, W.F16, 300),
                                                         (W.F16, W.F16, 64), (W.F16, W.U8, 0), (W.F16, W.U8, 100)])
-def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window):
-    announce("paged mixed", q_dtype, cache_dtype, window)
+@pytest.mark.parametrize("heads", [(16, 4), (12, 4), (4, 4)])  # even GQA ratio (head pairs), odd ratios (one group idle)
+def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window, heads):
+    announce("paged mixed", q_dtype, cache_dtype, window, heads)
     seqs = [(0, 130), (37, 1), (500, 1), (100, 257), (0, 2), (999, 1), (31, 97), (64, 1), (700, 128), (5, 0)]
-    case = W.make_paged_case(81, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    case = W.make_paged_case(81, seqs, heads[0], heads[1], 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
     dev = H.PagedDeviceCase(hip, case)
     out, path = dev.run(decode_waves=128)
     assert path == "paged_mfma"
