@@ -102,12 +102,18 @@ __device__ __forceinline__ half8_t load_q8(const void* q, int64_t elem, int q_dt
     return r;
 }
 
-// four bytes of `w` selected pairwise -> two exact fp16 integers (0..255)
-__device__ __forceinline__ uint32_t bytes_to_half2(uint32_t lo_src, uint32_t hi_src, uint32_t sel) {
-    // v_perm_b32: selector bytes 0..3 pick from lo_src, 4..7 from hi_src, 0x0c yields 0x00
-    uint32_t x = __builtin_amdgcn_perm(hi_src, lo_src, sel) | 0x64006400u;  // 1024 + byte, twice
-    half2_t h = __builtin_bit_cast(half2_t, x) - (half2_t){(half_t)1024.0f, (half_t)1024.0f};
-    return __builtin_bit_cast(uint32_t, h);
+// u8 -> fp16 operands.  0x6400 | byte is the fp16 number 1024 + byte, exactly.  The operands keep
+// that bias: it adds 1024 * sum(q) to a score and 1024 * sum(p') to an output, which are folded
+// into the zero-point terms the kernel subtracts anyway (the products are exact in fp32 and the
+// sums stay far inside its 24 bits), so the bias costs no instruction.
+constexpr float kByteBias = 1024.0f;
+// two bytes of one word (selector bytes 0..3 = its bytes, 4 = the bias byte 0x64)
+__device__ __forceinline__ uint32_t bytes_to_biased_half2(uint32_t src, uint32_t sel) {
+    return __builtin_amdgcn_perm(0x64646464u, src, sel);
+}
+// one byte of each of two words (selector bytes 0..3 pick from lo_src, 4..7 from hi_src, 0x0c yields 0x00)
+__device__ __forceinline__ uint32_t bytes_to_biased_half2(uint32_t lo_src, uint32_t hi_src, uint32_t sel) {
+    return __builtin_amdgcn_perm(hi_src, lo_src, sel) | 0x64006400u;
 }
 
 template <bool kU8>
@@ -182,10 +188,10 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
                 a = as_half8(b.k[t][i]);
             } else {
                 uint4_t w;
-                w[0] = bytes_to_half2(b.k[t][i][0], 0u, 0x0c010c00u);
-                w[1] = bytes_to_half2(b.k[t][i][0], 0u, 0x0c030c02u);
-                w[2] = bytes_to_half2(b.k[t][i][1], 0u, 0x0c010c00u);
-                w[3] = bytes_to_half2(b.k[t][i][1], 0u, 0x0c030c02u);
+                w[0] = bytes_to_biased_half2(b.k[t][i][0], 0x04010400u);
+                w[1] = bytes_to_biased_half2(b.k[t][i][0], 0x04030402u);
+                w[2] = bytes_to_biased_half2(b.k[t][i][1], 0x04010400u);
+                w[3] = bytes_to_biased_half2(b.k[t][i][1], 0x04030402u);
                 a = as_half8(w);
             }
             s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[i], s[t], 0, 0, 0);
@@ -201,7 +207,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
             const int j = t * 4 + r;
             const int tok = tok_base + t * 16 + kg * 4 + r;
             float x = s[t][r];
-            if constexpr (kU8) x = b.ksz[j].x * (x - b.ksz[j].y * sumq);
+            if constexpr (kU8) x = b.ksz[j].x * (x - (b.ksz[j].y + kByteBias) * sumq);
             x = (tok >= j0 && tok < ctx) ? x * c : -INFINITY;
             sv[j] = x;
             mloc = fmaxf(mloc, x);
@@ -236,7 +242,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
         if constexpr (kU8) {
             pj *= b.vsz[j].x;
             const half_t ph = (half_t)pj;
-            csum = fmaf((float)ph, b.vsz[j].y, csum);
+            csum = fmaf((float)ph, b.vsz[j].y + kByteBias, csum);
             pf[j] = ph;
         } else {
             pf[j] = (half_t)pj;
@@ -262,7 +268,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
             const uint32_t sel = 0x0c000c00u | ((4u + (e & 3)) << 16) | (uint32_t)(e & 3);
 #pragma unroll
             for (int jp = 0; jp < 4; jp++)
-                w[jp] = bytes_to_half2(b.v[2 * jp][e >> 2], b.v[2 * jp + 1][e >> 2], sel);
+                w[jp] = bytes_to_biased_half2(b.v[2 * jp][e >> 2], b.v[2 * jp + 1][e >> 2], sel);
         }
         st.acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(w), pf, st.acc[e], 0, 0, 0);
     }
