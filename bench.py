@@ -27,12 +27,31 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16
 
 
+CLOCK_RAMP_MS = 100.0  # untimed load ahead of the warmup steps, see time_steps
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
 def time_steps(hip, fn, steps, warmup):
-    """fn(i) enqueues one step on the default stream.  Returns (ms per step, dominant-kernel ms)."""
+    """fn(i) enqueues one step on the default stream.  Returns (ms per step, dominant-kernel ms).
+
+    Before the `warmup` untimed steps the same step runs untimed for CLOCK_RAMP_MS of GPU time: the
+    shader clock of an idle MI355X takes some tens of milliseconds of load to reach its sustained
+    level (a sub-millisecond step measured from idle runs 15-20 % slower than the same step in a
+    serving loop), and a handful of warmup steps is over long before that."""
+    ramp0, ramp1 = hip.Event(), hip.Event()
+    ramped = 0.0
+    while ramped < CLOCK_RAMP_MS:
+        ramp0.record()
+        for i in range(32):
+            fn(i)
+        ramp1.record()
+        ramp1.synchronize()
+        ramped += ramp0.elapsed_ms(ramp1)
+    ramp0.close()
+    ramp1.close()
     for i in range(warmup):
         fn(i)
     hip.check(hip.lib().hipattn_stream_synchronize(None))
@@ -186,8 +205,8 @@ def cpu_baseline_sdpa(case, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -268,7 +287,8 @@ def main():
         "dtype": "bf16" if is_sdpa else ("u8" if args.workload == "c4" else "f16"),
         "data": "synthetic",
         "config": {"workload": head["workload"], "kernel_path": head["kernel_path"],
-                   "device": dev_name, "arch": info.arch.decode(), "compute_units": info.compute_units},
+                   "device": dev_name, "arch": info.arch.decode(), "compute_units": info.compute_units,
+                   "clock_ramp_ms": CLOCK_RAMP_MS},
         "roofline": head["roofline"],
         "cpu_baseline": cpu if cpu else None,
         "workloads": {k: v for k, v in results.items()},
