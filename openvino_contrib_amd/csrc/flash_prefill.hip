@@ -179,12 +179,15 @@ __device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key) {
 }
 
 // Q fragment, multiplied by c = scale * log2(e) and rounded to the MFMA element type: the first
-// product then yields the exponents of the softmax directly.
+// product then yields the exponents of the softmax directly.  Loading and converting are separate
+// steps, so that all loads of a wavefront (and the first K/V tiles) are in flight together; rows
+// past the end of the tile repeat its last row (their results are never stored).
+__device__ __forceinline__ uint4_t load_q_raw(const Tile& t, int row, int d0) {
+    return *(const uint4_t*)(t.q + (int64_t)min(row, t.rows - 1) * t.q_stride + d0);
+}
 template <bool kBf16>
-__device__ __forceinline__ typename Mfma<kBf16>::vec8 load_q_frag(const Tile& t, int row, int d0, float c) {
+__device__ __forceinline__ typename Mfma<kBf16>::vec8 convert_q_frag(const Tile& t, uint4_t raw, float c) {
     using vec8 = typename Mfma<kBf16>::vec8;
-    uint4_t raw = {0u, 0u, 0u, 0u};
-    if (row < t.rows) raw = *(const uint4_t*)(t.q + (int64_t)row * t.q_stride + d0);
     const bool q_is_bf16 = (t.q_dtype == HIPATTN_BF16);
     uint4_t cv;
 #pragma unroll
@@ -441,6 +444,36 @@ __device__ __forceinline__ void store_rows(const Tile& t, const float16_t (&o)[4
         }
 }
 
+// 16-bit outputs of a wavefront's 32 rows, transposed through 8 KB of LDS (free once the key loop
+// is over) so that the global stores are whole rows: the accumulator layout gives a lane 8 bytes
+// in each of 16 places of one row, a wavefront-wide store of which touches 32 rows 16 bytes at a
+// time.  LDS rows are 256 bytes with the 16-byte chunks XOR-swizzled by the row number; one store
+// instruction then writes four complete rows (16 lanes x 16 bytes each).
+template <bool kOutBf16>
+__device__ __forceinline__ void store_rows_via_lds(const Tile& t, const float16_t (&o)[4], float inv, lds_byte* stage,
+                                                   int row0, int lane) {
+    const int n32 = lane & 31, hi = lane >> 5;
+    typedef __attribute__((address_space(3))) uint2_t lds_uint2;
+    typedef __attribute__((address_space(3))) uint4_t lds_uint4;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            const float x0 = o[dt][rq * 4] * inv, x1 = o[dt][rq * 4 + 1] * inv, x2 = o[dt][rq * 4 + 2] * inv,
+                        x3 = o[dt][rq * 4 + 3] * inv;
+            const uint2_t w = {Mfma<kOutBf16>::cvt2(x0, x1), Mfma<kOutBf16>::cvt2(x2, x3)};
+            const int chunk = dt * 4 + rq;  // head-dim dt*32 + 8*rq .. +8; this lane has its half `hi`
+            *(lds_uint2*)(stage + n32 * kRowBytes + ((chunk ^ (n32 & 15)) << 4) + hi * 8) = w;
+        }
+    const int lrow = lane >> 4, chunk = lane & 15;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const int r = 4 * k + lrow;
+        const uint4_t w = *(const lds_uint4*)(stage + r * kRowBytes + ((chunk ^ (r & 15)) << 4));
+        if (row0 + r < t.rows) *(uint4_t*)((uint16_t*)t.out + (int64_t)(row0 + r) * t.out_stride + chunk * 8) = w;
+    }
+}
+
 // Wave-uniform address of the 8 consecutive rows that start at key0 (a multiple of 8 below
 // kv_len): they lie in one block of a paged cache, whose table entry is `entry`.
 __device__ __forceinline__ const uint8_t* row_group_base(const Tile& t, const uint8_t* base, int key0, int entry) {
@@ -511,10 +544,14 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
     };
 
-    // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
-    vec8 qf[8];
+    // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8 (loads issued here, converted below)
+    uint4_t q_raw[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) qf[i] = load_q_frag<kBf16>(t, row, i * 16 + hi * 8, c);
+    for (int i = 0; i < 8; i++) q_raw[i] = uint4_t{0u, 0u, 0u, 0u};
+    if (t.rows > 0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) q_raw[i] = load_q_raw(t, row, i * 16 + hi * 8);
+    }
 
     float16_t o[4];
 #pragma unroll
@@ -589,6 +626,9 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     if (group == 1) recent = load_rows(true, 2, k_stage(2), e2) + load_rows(false, 1, v_stage(1), e1);
     // entries of the tiles the first iteration loads: K(group + 2) and V(group + 1)
     int entry_v = group ? e2 : e1, entry_k = group ? e3 : e2;
+    vec8 qf[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) qf[i] = convert_q_frag<kBf16>(t, q_raw[i], c);
     barrier_keeping_loads(recent);
     if (group == 1) barrier_keeping_loads(recent);  // group 1 sits out phase 0
 
@@ -664,13 +704,15 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     pair_values(st.l_run, l_lo, l_hi);
     const float l_row = l_lo + l_hi;
     const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
-    if (row < t.rows) {
-        if (t.out_dtype == HIPATTN_F32)
-            store_rows<HIPATTN_F32>(t, o, inv, row, hi);
-        else if (t.out_dtype == HIPATTN_F16)
-            store_rows<HIPATTN_F16>(t, o, inv, row, hi);
-        else
-            store_rows<HIPATTN_BF16>(t, o, inv, row, hi);
+    // (every wavefront is past its last read of the K/V ring here: the final barrier of the loop)
+    lds_byte* const out_stage = lds + wave * (32 * kRowBytes);
+    const int row0 = (wave & 3) * 32;
+    if (t.out_dtype == HIPATTN_F32) {
+        if (row < t.rows) store_rows<HIPATTN_F32>(t, o, inv, row, hi);
+    } else if (t.out_dtype == HIPATTN_F16) {
+        store_rows_via_lds<false>(t, o, inv, out_stage, row0, lane);
+    } else {
+        store_rows_via_lds<true>(t, o, inv, out_stage, row0, lane);
     }
 }
 
