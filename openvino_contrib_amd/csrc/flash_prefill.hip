@@ -74,7 +74,9 @@ constexpr int kThreads = 512;
 constexpr int kStages = 3;    // ring of K stages and ring of V stages
 constexpr int kRowBytes = kD * 2;                // a K or V row in LDS: 16 chunks of 16 bytes
 constexpr int kKBytes = kTileK * kRowBytes;      // one K or V stage
-constexpr int kLdsBytes = 2 * kStages * kKBytes;
+constexpr int kRingBytes = 2 * kStages * kKBytes;
+constexpr int kWaveStageBytes = 32 * kRowBytes;  // a wavefront's 32 query rows (in) or output rows (out), 16-bit
+constexpr int kLdsBytes = kRingBytes + 8 * kWaveStageBytes;
 
 // global -> LDS load of 16 bytes per lane: lane l's data lands at LDS byte lds_base + 16 l
 // (lds_base wave-uniform, carried in M0).  Issued as inline assembly on purpose: the compiler
@@ -179,12 +181,7 @@ __device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key) {
 }
 
 // Q fragment, multiplied by c = scale * log2(e) and rounded to the MFMA element type: the first
-// product then yields the exponents of the softmax directly.  Loading and converting are separate
-// steps, so that all loads of a wavefront (and the first K/V tiles) are in flight together; rows
-// past the end of the tile repeat its last row (their results are never stored).
-__device__ __forceinline__ uint4_t load_q_raw(const Tile& t, int row, int d0) {
-    return *(const uint4_t*)(t.q + (int64_t)min(row, t.rows - 1) * t.q_stride + d0);
-}
+// product then yields the exponents of the softmax directly.
 template <bool kBf16>
 __device__ __forceinline__ typename Mfma<kBf16>::vec8 convert_q_frag(const Tile& t, uint4_t raw, float c) {
     using vec8 = typename Mfma<kBf16>::vec8;
@@ -544,13 +541,21 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
     };
 
-    // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8 (loads issued here, converted below)
-    uint4_t q_raw[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) q_raw[i] = uint4_t{0u, 0u, 0u, 0u};
+    // The wavefront's 32 query rows go to its own 8 KB of LDS with eight global->LDS loads of four
+    // whole rows each, laid out like a K tile (chunk c of row r at position c ^ (r % 16)): the
+    // fragment of k-step i, head-dim i*16 + hi*8 .. +8 of row n32, is then one conflict-free
+    // ds_read_b128.  Rows past the end of the tile repeat its last row (never stored).  A lane
+    // loading its fragments straight from global memory would touch 32 rows per instruction.
+    lds_byte* const wave_stage = lds + kRingBytes + wave * kWaveStageBytes;
     if (t.rows > 0) {
+        const int lr = lane >> 4, lp = lane & 15;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q_raw[i] = load_q_raw(t, row, i * 16 + hi * 8);
+        for (int k = 0; k < 8; k++) {
+            const int r = 4 * k + lr;
+            const int qrow = min((wave & 3) * 32 + r, t.rows - 1);
+            const uint8_t* src = (const uint8_t*)(t.q + (int64_t)qrow * t.q_stride) + ((lp ^ (r & 15)) << 4);
+            load_to_lds_16(src, wave_stage + 4 * k * kRowBytes);
+        }
     }
 
     float16_t o[4];
@@ -626,10 +631,16 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     if (group == 1) recent = load_rows(true, 2, k_stage(2), e2) + load_rows(false, 1, v_stage(1), e1);
     // entries of the tiles the first iteration loads: K(group + 2) and V(group + 1)
     int entry_v = group ? e2 : e1, entry_k = group ? e3 : e2;
+    barrier_keeping_loads(recent);  // (also: this wavefront's query rows have landed)
+    // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
     vec8 qf[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) qf[i] = convert_q_frag<kBf16>(t, q_raw[i], c);
-    barrier_keeping_loads(recent);
+    for (int i = 0; i < 8; i++) {
+        typedef __attribute__((address_space(3))) uint4_t lds_uint4;
+        uint4_t raw = {0u, 0u, 0u, 0u};
+        if (t.rows > 0) raw = *(const lds_uint4*)(wave_stage + (f.k ^ (i << 5)));
+        qf[i] = convert_q_frag<kBf16>(t, raw, c);
+    }
     if (group == 1) barrier_keeping_loads(recent);  // group 1 sits out phase 0
 
     float16_t s[2];
@@ -704,8 +715,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     pair_values(st.l_run, l_lo, l_hi);
     const float l_row = l_lo + l_hi;
     const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
-    // (every wavefront is past its last read of the K/V ring here: the final barrier of the loop)
-    lds_byte* const out_stage = lds + wave * (32 * kRowBytes);
+    lds_byte* const out_stage = wave_stage;
     const int row0 = (wave & 3) * 32;
     if (t.out_dtype == HIPATTN_F32) {
         if (row < t.rows) store_rows<HIPATTN_F32>(t, o, inv, row, hi);
