@@ -440,37 +440,33 @@ __device__ __forceinline__ void store_rows(const Tile& t, const float16_t (&o)[4
         }
 }
 
-// 16-bit outputs of a wavefront's 32 rows, transposed through 2 KB of LDS so that the global
-// stores are contiguous pieces of rows: the accumulator layout gives a lane 8 bytes in each of 16
-// places of one row, a wavefront-wide store of which touches 32 rows 16 bytes at a time.  The
-// rows go out in four rounds of 32 head-dim elements (64 bytes of every row): a round is staged
-// as 32 rows of 64 bytes, the 16-byte chunks XOR-swizzled by the row number, and leaves as two
-// store instructions of 16 rows x 64 bytes.
+// 16-bit outputs of a wavefront's 32 rows, transposed through 8 KB of LDS (free once the key loop
+// is over) so that the global stores are whole rows: the accumulator layout gives a lane 8 bytes
+// in each of 16 places of one row, a wavefront-wide store of which touches 32 rows 16 bytes at a
+// time.  LDS rows are 256 bytes with the 16-byte chunks XOR-swizzled by the row number; one store
+// instruction then writes four complete rows (16 lanes x 16 bytes each).
 template <bool kOutBf16>
 __device__ __forceinline__ void store_rows_via_lds(const Tile& t, const float16_t (&o)[4], float inv, lds_byte* stage,
                                                    int row0, int lane) {
-    asm volatile("" : "+v"(lane));  // (the addresses below are computed here, once per item, not kept in registers)
     const int n32 = lane & 31, hi = lane >> 5;
     typedef __attribute__((address_space(3))) uint2_t lds_uint2;
     typedef __attribute__((address_space(3))) uint4_t lds_uint4;
-    const int lrow = lane >> 2, chunk = lane & 3;
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++) {
+    for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int rq = 0; rq < 4; rq++) {
             const float x0 = o[dt][rq * 4] * inv, x1 = o[dt][rq * 4 + 1] * inv, x2 = o[dt][rq * 4 + 2] * inv,
                         x3 = o[dt][rq * 4 + 3] * inv;
             const uint2_t w = {Mfma<kOutBf16>::cvt2(x0, x1), Mfma<kOutBf16>::cvt2(x2, x3)};
-            // head-dim dt*32 + 8*rq .. +8 is chunk rq of the round; this lane has its half `hi`
-            *(lds_uint2*)(stage + n32 * 64 + ((rq ^ ((n32 >> 1) & 3)) << 4) + hi * 8) = w;
+            const int chunk = dt * 4 + rq;  // head-dim dt*32 + 8*rq .. +8; this lane has its half `hi`
+            *(lds_uint2*)(stage + n32 * kRowBytes + ((chunk ^ (n32 & 15)) << 4) + hi * 8) = w;
         }
+    const int lrow = lane >> 4, chunk = lane & 15;
 #pragma unroll
-        for (int k = 0; k < 2; k++) {
-            const int r = 16 * k + lrow;
-            const uint4_t w = *(const lds_uint4*)(stage + r * 64 + ((chunk ^ ((r >> 1) & 3)) << 4));
-            if (row0 + r < t.rows)
-                *(uint4_t*)((uint16_t*)t.out + (int64_t)(row0 + r) * t.out_stride + dt * 32 + chunk * 8) = w;
-        }
+    for (int k = 0; k < 8; k++) {
+        const int r = 4 * k + lrow;
+        const uint4_t w = *(const lds_uint4*)(stage + r * kRowBytes + ((chunk ^ (r & 15)) << 4));
+        if (row0 + r < t.rows) *(uint4_t*)((uint16_t*)t.out + (int64_t)(row0 + r) * t.out_stride + chunk * 8) = w;
     }
 }
 
@@ -492,14 +488,8 @@ __device__ __forceinline__ void barrier_keeping() {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 }
-__device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep: 0, 2 or 4, plus 8 (wave-uniform)
-    if (keep >= 12)
-        barrier_keeping<12>();
-    else if (keep >= 10)
-        barrier_keeping<10>();
-    else if (keep >= 8)
-        barrier_keeping<8>();
-    else if (keep >= 4)
+__device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0, 2 or 4 (wave-uniform)
+    if (keep >= 4)
         barrier_keeping<4>();
     else if (keep >= 2)
         barrier_keeping<2>();
@@ -507,65 +497,18 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep: 0, 2
         barrier_keeping<0>();
 }
 
-// One unit of work of a workgroup, as one of its two groups sees it.
-struct Item {
-    Tile t;     // this group's tile
-    int kv_lo;  // first key of the workgroup's key range (the union of both groups' ranges), a multiple of 64
-    int n;      // 64-key tiles in that range
-};
-
-// (the tiles are passed as "mine" and "the other group's", not selected by group number here: a
-// run-time choice between two structures would put both in scratch memory)
-__device__ __forceinline__ void make_item(const Tile& mine, const Tile& other, Item& it) {
-    int lo0, hi0, lo1, hi1;
-    key_range(mine, lo0, hi0);
-    key_range(other, lo1, hi1);
-    int kv_lo, kv_hi;
-    if (hi0 <= lo0) {
-        kv_lo = lo1;
-        kv_hi = hi1;
-    } else if (hi1 <= lo1) {
-        kv_lo = lo0;
-        kv_hi = hi0;
-    } else {
-        kv_lo = min(lo0, lo1);
-        kv_hi = max(hi0, hi1);
-    }
-    it.t = mine;
-    it.kv_lo = kv_lo;
-    it.n = (kv_hi - kv_lo + kTileK - 1) / kTileK;
-}
-
-// What the loads issued ahead for the following item need to know of it (dense K/V only).
-struct NextItem {
-    const uint8_t* k;
-    const uint8_t* v;
-    const uint16_t* q;
-    int64_t q_stride;
-    int rows, kv_len, kv_lo, n;
-    bool valid;
-};
-
-// The loop of one wavefront over the items feed(round, group, item) hands this workgroup
-// (round = 0, 1, ... until it returns false; the same answer in every wavefront).
+// The loop of one wavefront.  t is the tile of this wavefront's group; [kv_lo, kv_hi) is the key
+// range of the workgroup (the union of both groups' ranges, kv_lo a multiple of 64).
 //
-// Phases of an item, numbered from 0 and separated by workgroup barriers: group 0 computes the
-// scores of tile j in phase 2j, their softmax in phase 2j+1 and P V in phase 2j+2 (together with
-// the scores of tile j+1); group 1 does the same one phase later.  K(j) is therefore read in
-// phases 2j and 2j+1, V(j) in phases 2j+2 and 2j+3.  Load batch B(x) = {K(x+2), V(x+1)} goes into
-// the ring stages of K(x-1) and V(x-2); every wavefront issues its rows of B(x) in a vector phase
+// Phases, numbered from 0 and separated by workgroup barriers: group 0 computes the scores of
+// tile j in phase 2j, their softmax in phase 2j+1 and P V in phase 2j+2 (together with the
+// scores of tile j+1); group 1 does the same one phase later.  K(j) is therefore read in phases
+// 2j and 2j+1, V(j) in phases 2j+2 and 2j+3.  Load batch B(x) = {K(x+2), V(x+1)} goes into the
+// ring stages of K(x-1) and V(x-2); every wavefront issues its rows of B(x) in a vector phase
 // (group 0 in phase 2x+1, group 1 in phase 2x), and at each barrier waits for all of its loads
 // except the latest batch, which puts B(x) in LDS two phases before its first use.
-//
-// The tiles of consecutive items form one sequence through the ring: tile n + i of an item with
-// n tiles is tile i of the item after it, so the last iterations of an item load the first K and
-// V tiles of the next one (and the first iteration its query rows), and a workgroup starts its
-// second and later items with their data already in LDS.  k_issued / v_issued count the tiles of
-// that sequence, from tile 0 of the current item, whose rows this wavefront has issued; tiles are
-// issued strictly in order, and a tile past the end of the following item is not available until
-// the workgroup has moved on.
-template <bool kBf16, bool kPaged, typename Feed>
-__device__ __forceinline__ void run_items(Feed&& feed, uint8_t* lds_generic, float scale) {
+template <bool kBf16>
+__device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     lds_byte* const lds = (lds_byte*)lds_generic;
@@ -575,6 +518,56 @@ __device__ __forceinline__ void run_items(Feed&& feed, uint8_t* lds_generic, flo
     const int n32 = lane & 31, hi = lane >> 5;
     const int row = (wave & 3) * 32 + n32;  // query row inside the group's tile
     const float c = scale * kLog2e;
+    const int n = (kv_hi - kv_lo + kTileK - 1) / kTileK;  // tiles of the workgroup
+    if (n <= 0) {
+        // nothing to attend to: rows of zeros (the reference's softmax over an empty set is undefined)
+        if (row < t.rows) {
+            float16_t z[4];
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) z[dt][r] = 0.0f;
+            if (t.out_dtype == HIPATTN_F32)
+                store_rows<HIPATTN_F32>(t, z, 0.0f, row, hi);
+            else
+                store_rows<HIPATTN_F16>(t, z, 0.0f, row, hi);  // zero bits are the same in f16 and bf16
+        }
+        return;
+    }
+    auto unmasked = [&](int j) {
+        const int ts = kv_lo + j * kTileK;
+        return (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
+               (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
+    };
+
+    // The wavefront's 32 query rows go to its own 8 KB of LDS with eight global->LDS loads of four
+    // whole rows each, laid out like a K tile (chunk c of row r at position c ^ (r % 16)): the
+    // fragment of k-step i, head-dim i*16 + hi*8 .. +8 of row n32, is then one conflict-free
+    // ds_read_b128.  Rows past the end of the tile repeat its last row (never stored).  A lane
+    // loading its fragments straight from global memory would touch 32 rows per instruction.
+    lds_byte* const wave_stage = lds + kRingBytes + wave * kWaveStageBytes;
+    if (t.rows > 0) {
+        const int lr = lane >> 4, lp = lane & 15;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int r = 4 * k + lr;
+            const int qrow = min((wave & 3) * 32 + r, t.rows - 1);
+            const uint8_t* src = (const uint8_t*)(t.q + (int64_t)qrow * t.q_stride) + ((lp ^ (r & 15)) << 4);
+            load_to_lds_16(src, wave_stage + 4 * k * kRowBytes);
+        }
+    }
+
+    float16_t o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+    SoftmaxState st;
+#pragma unroll
+    for (int r = 0; r < 16; r++) st.neg_ref[r] = 0.0f;
+    st.l_run = 0.0f;
+    st.started = false;
+    const int my_pos = t.pos0 + row;  // position of this lane's query row
     const FragOffsets f = frag_offsets(lane);
 
     // global -> LDS: one instruction moves four rows (64 lanes x 16 bytes, LDS address = wave-uniform
@@ -586,297 +579,170 @@ __device__ __forceinline__ void run_items(Feed&& feed, uint8_t* lds_generic, flo
     const uint32_t v_lane = (uint32_t)(((lpos ^ (4 * lrow)) << 4) + lrow * kRowBytes);
     lds_byte* const k_ring = lds;
     lds_byte* const v_ring = lds + kStages * kKBytes;
-    // The wavefront's 32 query rows go to its own 8 KB of LDS with eight global->LDS loads of four
-    // whole rows each, laid out like a K tile (chunk c of row r at position c ^ (r % 16)): the
-    // fragment of k-step i, head-dim i*16 + hi*8 .. +8 of row n32, is then one conflict-free
-    // ds_read_b128.  Rows past the end of the tile repeat its last row (never stored).  A lane
-    // loading its fragments straight from global memory would touch 32 rows per instruction.
-    lds_byte* const wave_stage = lds + kRingBytes + wave * kWaveStageBytes;
-    auto issue_q = [&](const uint16_t* q, int64_t q_stride, int rows) __attribute__((always_inline)) -> int {
-        if (rows <= 0) return 0;
-        int lr = lrow, lp = lpos;
-        asm volatile("" : "+v"(lr), "+v"(lp));  // (once per item: computed here, not kept live through the key loop)
+    // this wavefront's rows of tile j into `stage`; returns the number of instructions issued
+    // (entry: the block table entry of these rows, see table_entry below; ignored for dense K/V)
+    auto load_rows = [&](bool is_k, int j, lds_byte* stage, int entry) -> int {
+        if (j >= n) return 0;
+        const uint8_t* base = is_k ? t.k : t.v;
+        lds_byte* const dst = stage + 8 * wave * kRowBytes;
+        const int key0 = kv_lo + j * kTileK + 8 * wave;
+        if (key0 + 8 <= t.kv_len) {
+            const uint8_t* gb = row_group_base(t, base, key0, entry);
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const int r = 4 * k + lr;
-            const int qrow = min((wave & 3) * 32 + r, rows - 1);
-            const uint8_t* src = (const uint8_t*)(q + (int64_t)qrow * q_stride) + ((lp ^ (r & 15)) << 4);
-            load_to_lds_16(src, wave_stage + 4 * k * kRowBytes);
+            for (int k = 0; k < 2; k++) {
+                const uint32_t off = (is_k ? (k_lane ^ (uint32_t)(k << 6)) : v_lane) + (uint32_t)(4 * k * kRowBytes);
+                load_to_lds_16(gb, off, dst + 4 * k * kRowBytes);
+            }
+        } else {  // the rows at the end of the sequence: per-lane clamped
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int r = 8 * (wave & 1) + 4 * k + lrow;
+                const int chunk = is_k ? (lpos ^ r) : (lpos ^ (4 * lrow));
+                const int64_t off = kv_row_offset(t, key0 + 4 * k + lrow) + (chunk << 4);
+                load_to_lds_16(base + off, dst + 4 * k * kRowBytes);
+            }
         }
-        return 8;
+        return 2;
     };
+    // Block table entry of this wavefront's rows of tile j (0 when there is none), read through
+    // the scalar cache in the vector phase, so that no scalar load is outstanding during a
+    // matrix phase (which would turn every partial wait for LDS fragments into a full one).
+    // (As inline assembly, because behind the compiler fences of the barriers an ordinary load of
+    // the table becomes a vector load that is waited for at once, together with every load to LDS
+    // in flight.  The wait for the scalar load is part of the statement: the compiler takes the
+    // output register as written when the statement ends and may reuse it at any time after.)
+    auto table_entry = [&](int j) -> int {
+        const int key0 = kv_lo + j * kTileK + 8 * wave;
+        if (t.table == nullptr || j >= n || key0 + 8 > t.kv_len) return 0;
+        int entry;
+        asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(entry) : "s"(t.table + (key0 >> t.block_shift)));
+        return entry;
+    };
+    auto k_stage = [&](int j) { return k_ring + (j % kStages) * kKBytes; };
+    auto v_stage = [&](int j) { return v_ring + (j % kStages) * kKBytes; };
 
-    Item it;
-    int round = 0;
-    if (!feed(round, group, it)) return;
-    NextItem nx;
-    int vbase = 0;                    // ring stage of tile 0 of the current item
-    int k_issued = 0, v_issued = 0;   // see above
-    // where this wavefront's rows of the next K / V tile to be issued go (the stages in ring order)
-    lds_byte* const k_dst_last = k_ring + (kStages - 1) * kKBytes + 8 * wave * kRowBytes;
-    lds_byte* const v_dst_last = v_ring + (kStages - 1) * kKBytes + 8 * wave * kRowBytes;
-    lds_byte* k_dst = k_ring + 8 * wave * kRowBytes;
-    lds_byte* v_dst = v_ring + 8 * wave * kRowBytes;
-    bool q_issued = false;            // the current item's query rows are in, or on their way to, the stage
-
-    while (true) {
-        const Tile& t = it.t;
-        const int kv_lo = it.kv_lo, n = it.n;
-        nx.valid = false;
-        if constexpr (!kPaged) {  // (a paged cache is never loaded ahead: one item per workgroup)
-            Item probe_item;
-            if (feed(round + 1, group, probe_item)) {
-                const Tile& u = probe_item.t;
-                nx.valid = true;
-                nx.k = u.k;
-                nx.v = u.v;
-                nx.q = u.q;
-                nx.q_stride = u.q_stride;
-                nx.rows = u.rows;
-                nx.kv_len = u.kv_len;
-                nx.kv_lo = probe_item.kv_lo;
-                nx.n = probe_item.n;
-            }
+    // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
+    const int e0 = table_entry(0), e1 = table_entry(1), e2 = table_entry(2), e3 = table_entry(3);
+    load_rows(true, 0, k_stage(0), e0);
+    load_rows(false, 0, v_stage(0), e0);
+    load_rows(true, 1, k_stage(1), e1);
+    int recent = 0;
+    if (group == 1) recent = load_rows(true, 2, k_stage(2), e2) + load_rows(false, 1, v_stage(1), e1);
+    // entries of the tiles the first iteration loads: K(group + 2) and V(group + 1)
+    int entry_v = group ? e2 : e1, entry_k = group ? e3 : e2;
+    barrier_keeping_loads(recent);  // (also: this wavefront's query rows have landed)
+    // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
+    vec8 qf[8];
+    {
+        typedef __attribute__((address_space(3))) uint4_t lds_uint4;
+        uint4_t raw[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            raw[i] = uint4_t{0u, 0u, 0u, 0u};
+            if (t.rows > 0) raw[i] = *(const lds_uint4*)(wave_stage + (f.k ^ (i << 5)));
         }
-        if (n <= 0) {
-            // nothing to attend to: rows of zeros (the reference's softmax over an empty set is undefined)
-            if (row < t.rows) {
-                float16_t z[4];
+        if (t.q_dtype == HIPATTN_BF16) {  // (one wave-uniform branch, not a choice per element)
 #pragma unroll
-                for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) z[dt][r] = 0.0f;
-                if (t.out_dtype == HIPATTN_F32)
-                    store_rows<HIPATTN_F32>(t, z, 0.0f, row, hi);
-                else
-                    store_rows<HIPATTN_F16>(t, z, 0.0f, row, hi);  // zero bits are the same in f16 and bf16
-            }
+            for (int i = 0; i < 8; i++) qf[i] = convert_q_frag<kBf16, true>(raw[i], c);
         } else {
-            auto unmasked = [&](int j) __attribute__((always_inline)) {
-                const int ts = kv_lo + j * kTileK;
-                return (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
-                       (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
-            };
-            // Block table entry of this wavefront's rows of tile j of the current item (0 when there
-            // is none), read through the scalar cache in the vector phase, so that no scalar load is
-            // outstanding during a matrix phase (which would turn every partial wait for LDS
-            // fragments into a full one).  (As inline assembly, because behind the compiler fences of
-            // the barriers an ordinary load of the table becomes a vector load that is waited for at
-            // once, together with every load to LDS in flight.  The wait for the scalar load is part
-            // of the statement: the compiler takes the output register as written when the
-            // statement ends and may reuse it at any time after.)
-            auto table_entry = [&](int j) __attribute__((always_inline)) -> int {
-                if constexpr (!kPaged) return 0;
-                const int key0 = kv_lo + j * kTileK + 8 * wave;
-                if (t.table == nullptr || j >= n || key0 + 8 > t.kv_len) return 0;
-                int entry;
-                asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)"
-                             : "=s"(entry)
-                             : "s"(t.table + (key0 >> t.block_shift)));
-                return entry;
-            };
-            // entries of tiles v_issued, v_issued + 1, v_issued + 2 (K runs one or two tiles ahead of V)
-            int ev0 = table_entry(v_issued), ev1 = table_entry(v_issued + 1), ev2 = table_entry(v_issued + 2);
-            // tiles of the sequence that can be loaded now: this item's and (dense only) the next one's
-            const int n_avail = n + ((!kPaged && nx.valid) ? nx.n : 0);
-            const int nx_lo_adj = nx.valid ? nx.kv_lo - n * kTileK : 0;  // first key of tile jv >= n: nx_lo_adj + 64 jv
-            // This wavefront's rows (8w .. 8w+7) of tile jv < n_avail of the sequence into dst.
-            auto load_tile = [&](bool is_k, int jv, int entry, lds_byte* dst) __attribute__((always_inline)) {
-                const bool cur = kPaged || jv < n;
-                const uint8_t* const base = cur ? (is_k ? t.k : t.v) : (is_k ? nx.k : nx.v);
-                const int key0 = (cur ? kv_lo : nx_lo_adj) + jv * kTileK + 8 * wave;
-                const int len = cur ? t.kv_len : nx.kv_len;
-                if (key0 + 8 <= len) {
-                    const uint8_t* gb = kPaged ? row_group_base(t, base, key0, entry) : base + (int64_t)key0 * kRowBytes;
 #pragma unroll
-                    for (int k = 0; k < 2; k++) {
-                        const uint32_t off =
-                            (is_k ? (k_lane ^ (uint32_t)(k << 6)) : v_lane) + (uint32_t)(4 * k * kRowBytes);
-                        load_to_lds_16(gb, off, dst + 4 * k * kRowBytes);
-                    }
-                } else {  // the rows at the end of the sequence: clamped per lane
-                    int lr = lrow;
-                    asm volatile("" : "+v"(lr));  // (keeps these rarely used addresses out of the loop's live registers)
-#pragma unroll
-                    for (int k = 0; k < 2; k++) {
-                        const uint32_t chunk_bytes = (is_k ? (k_lane ^ (uint32_t)(k << 6)) : v_lane) & 0xf0u;
-                        const int key = min(key0 + 4 * k + lr, len - 1);
-                        const int64_t off = kPaged ? kv_row_offset(t, key) : (int64_t)key * kRowBytes;
-                        load_to_lds_16(base + off + chunk_bytes, dst + 4 * k * kRowBytes);
-                    }
-                }
-            };
-            // tries the next K tile (if wanted up to k_upto) and the next V tile (up to v_upto), in
-            // that order; returns the number of load instructions issued
-            auto issue_next = [&](int k_upto, int v_upto) __attribute__((always_inline)) -> int {
-                int count = 0;
-                if (k_issued <= k_upto && k_issued < n_avail) {
-                    const int d = k_issued - v_issued;
-                    const int e0 = ev0, e1 = ev1, e2 = ev2;  // (values first: no choice between references)
-                    load_tile(true, k_issued, d <= 0 ? e0 : (d == 1 ? e1 : e2), k_dst);
-                    count += 2;
-                    k_issued++;
-                    k_dst = (k_dst == k_dst_last) ? k_dst - (kStages - 1) * kKBytes : k_dst + kKBytes;
-                }
-                if (v_issued <= v_upto && v_issued < k_issued && v_issued < n_avail) {
-                    load_tile(false, v_issued, ev0, v_dst);
-                    count += 2;
-                    v_issued++;
-                    v_dst = (v_dst == v_dst_last) ? v_dst - (kStages - 1) * kKBytes : v_dst + kKBytes;
-                    ev0 = ev1;
-                    ev1 = ev2;
-                    ev2 = table_entry(v_issued + 2);
-                }
-                return count;
-            };
-
-            // ---- prologue: this item's query rows, K(0), V(0), K(1) and, from group 1, its rows
-            // of B(0) -- whatever of them the previous item has not issued already
-            if (!q_issued) issue_q(t.q, t.q_stride, t.rows);
-            q_issued = false;
-#pragma nounroll
-            for (int u = 0; u < 3; u++) issue_next(1 + group, group);
-            barrier_keeping<0>();
-            // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
-            vec8 qf[8];
-            {
-                typedef __attribute__((address_space(3))) uint4_t lds_uint4;
-                uint4_t raw[8];
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    raw[i] = uint4_t{0u, 0u, 0u, 0u};
-                    if (t.rows > 0) raw[i] = *(const lds_uint4*)(wave_stage + (f.k ^ (i << 5)));
-                }
-                if (t.q_dtype == HIPATTN_BF16) {
-#pragma unroll
-                    for (int i = 0; i < 8; i++) qf[i] = convert_q_frag<kBf16, true>(raw[i], c);
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 8; i++) qf[i] = convert_q_frag<kBf16, false>(raw[i], c);
-                }
-            }
-            float16_t o[4];
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
-            SoftmaxState st;
-#pragma unroll
-            for (int r = 0; r < 16; r++) st.neg_ref[r] = 0.0f;
-            st.l_run = 0.0f;
-            st.started = false;
-            const int my_pos = t.pos0 + row;  // position of this lane's query row
-            int recent = 0;
-            if (group == 1) barrier_keeping<0>();  // group 1 sits out phase 0
-
-            auto k_stage = [&](int j) __attribute__((always_inline)) { return k_ring + ((vbase + j) % kStages) * kKBytes; };
-            auto v_stage = [&](int j) __attribute__((always_inline)) { return v_ring + ((vbase + j) % kStages) * kKBytes; };
-            float16_t s[2];
-            vec8 pf[4];
-            tile_scores<kBf16>(k_stage(0), f, qf, st.neg_ref, s);
-            barrier_keeping<0>();
-#ifdef HIPATTN_FLASH_TRACE
-            PhaseClock clk;
-            clk.last = (long long)__builtin_readcyclecounter();
-#endif
-            // The two phases of tile j.  Both groups run every tile of the workgroup's key range: a
-            // tile outside a group's own range is fully masked and contributes probabilities of zero.
-            auto two_phases = [&](int j, bool last, const lds_byte* k_next, const lds_byte* v_cur) __attribute__((always_inline)) {
-                // ---- vector phase
-#ifdef HIPATTN_FLASH_TRACE
-                clk.tile = j;
-#endif
-                FLASH_STAMP(clk, 0);
-                recent = issue_next(j + group + 2, j + group + 1);
-                if (j == 0 && nx.valid) {
-                    // the query rows of the following item (this item's are in registers by now)
-                    recent += issue_q(nx.q, nx.q_stride, nx.rows);
-                    q_issued = true;
-                }
-                FLASH_STAMP(clk, 1);
-                tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
-                // (the probabilities are complete before the barrier: the compiler may not move their
-                // arithmetic into the matrix phase)
-#pragma unroll
-                for (int ks = 0; ks < 4; ks++) asm volatile("" : "+v"(pf[ks]));
-                FLASH_STAMP(clk, 2);
-                // the matrix phase runs at raised priority (set before the barrier, so that it holds
-                // from the first instruction after it): otherwise the other group's instruction
-                // stream, which never stalls for long, keeps this wavefront's MFMAs from issuing
-                __builtin_amdgcn_s_setprio(3);
-                barrier_keeping_loads(recent);
-                FLASH_STAMP(clk, 3);
-                // ---- matrix phase
-                // fragment addresses of this tile: per-lane offset + stage address, so that every read
-                // is one XOR with a constant plus an immediate offset (the stage addresses are
-                // multiples of 16 KB and leave the XORed bits alone)
-                FragOffsets fs;
-                fs.k = f.k + (int)(uintptr_t)k_next;
-                fs.v = f.v + (int)(uintptr_t)v_cur;
-                const lds_byte* const zero = (const lds_byte*)0;
-                if (!last)
-                    tile_accumulate_and_scores<kBf16>(zero, zero, fs, pf, o, qf, st.neg_ref, s);
-                else
-                    tile_accumulate<kBf16>(zero, fs, pf, o);
-                __builtin_amdgcn_s_setprio(0);
-                FLASH_STAMP(clk, 5);
-                barrier_keeping_loads(recent);
-                FLASH_STAMP(clk, 6);
-            };
-            for (int j = 0; j < n - 1; j++) two_phases(j, false, k_stage(j + 1), v_stage(j));
-            two_phases(n - 1, true, k_stage(n), v_stage(n - 1));
-            if (group == 0) barrier_keeping_loads(recent);  // as many barriers as group 1
-#ifdef HIPATTN_FLASH_TRACE
-            if (g_flash_phase_trace && lane == 0 && round == 0) {
-                long long* r = g_flash_phase_trace + ((int64_t)blockIdx.x * 8 + wave) * 8;
-                for (int k = 0; k < 7; k++) r[k] = clk.acc[k];
-                r[7] = n;
-            }
-            if (g_flash_raw_trace && lane == 0 && blockIdx.x == 0 && round == 0 && n >= 12)
-                for (int k = 0; k < 8; k++) g_flash_raw_trace[wave * 16 + k] = clk.raw[k];
-#endif
-
-            // ---- normalise and store.  Every wavefront is past its last read of V(n-1) here (the
-            // final barrier above), and nothing is loaded into that stage before the first
-            // iteration of the next item, which lies behind that item's first barrier: it is the
-            // staging area of the output rows, 2 KB per wavefront.
-            float l_lo, l_hi;
-            pair_values(st.l_run, l_lo, l_hi);
-            const float l_row = l_lo + l_hi;
-            const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
-            lds_byte* const out_stage = v_ring + ((vbase + n - 1) % kStages) * kKBytes + wave * 2048;
-            const int row0 = (wave & 3) * 32;
-            if (t.out_dtype == HIPATTN_F32) {
-                if (row < t.rows) store_rows<HIPATTN_F32>(t, o, inv, row, hi);
-            } else if (t.out_dtype == HIPATTN_F16) {
-                store_rows_via_lds<false>(t, o, inv, out_stage, row0, lane);
-            } else {
-                store_rows_via_lds<true>(t, o, inv, out_stage, row0, lane);
-            }
+            for (int i = 0; i < 8; i++) qf[i] = convert_q_frag<kBf16, false>(raw[i], c);
         }
-        // ---- next item
-        if constexpr (kPaged) break;
-        round++;
-        if (!feed(round, group, it)) break;
-        vbase = (vbase + max(n, 0)) % kStages;
-        k_issued = max(k_issued - max(n, 0), 0);
-        v_issued = max(v_issued - max(n, 0), 0);
+    }
+    if (group == 1) barrier_keeping_loads(recent);  // group 1 sits out phase 0
+
+    float16_t s[2];
+    vec8 pf[4];
+    tile_scores<kBf16>(k_stage(0), f, qf, st.neg_ref, s);
+    barrier_keeping_loads(recent);
+#ifdef HIPATTN_FLASH_TRACE
+    PhaseClock clk;
+    clk.last = (long long)__builtin_readcyclecounter();
+#endif
+    // The two phases of tile j.  Both groups run every tile of the workgroup's key range: a tile
+    // outside a group's own range is fully masked and contributes probabilities of zero.  The
+    // restrict qualifiers tell the compiler that the LDS writes of the asynchronous loads cannot
+    // alias the fragment reads, so that it does not wait for all loads before every LDS read; the
+    // barriers do the waiting that is needed.
+    auto two_phases = [&](int j, bool last, const lds_byte* __restrict__ k_next, const lds_byte* __restrict__ v_cur,
+                          lds_byte* __restrict__ k_fill, lds_byte* __restrict__ v_fill) {
+        // ---- vector phase
+#ifdef HIPATTN_FLASH_TRACE
+        clk.tile = j;
+#endif
+        FLASH_STAMP(clk, 0);
+        recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
+        entry_v = entry_k;  // the next iteration loads V of the tile whose K was loaded now
+        entry_k = table_entry(j + group + 3);
+        FLASH_STAMP(clk, 1);
+        tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
+        // (the probabilities are complete before the barrier: the compiler may not move their
+        // arithmetic into the matrix phase)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) asm volatile("" : "+v"(pf[ks]));
+        FLASH_STAMP(clk, 2);
+        // the matrix phase runs at raised priority (set before the barrier, so that it holds from
+        // the first instruction after it): otherwise the other group's instruction stream, which
+        // never stalls for long, keeps this wavefront's MFMAs from issuing
+        __builtin_amdgcn_s_setprio(3);
+        barrier_keeping_loads(recent);
+        FLASH_STAMP(clk, 3);
+        // ---- matrix phase
+        // fragment addresses of this tile: per-lane offset + stage address, so that every read is
+        // one XOR with a constant plus an immediate offset (the stage addresses are multiples of
+        // 16 KB and leave the XORed bits alone)
+        FragOffsets fs;
+        fs.k = f.k + (int)(uintptr_t)k_next;
+        fs.v = f.v + (int)(uintptr_t)v_cur;
+        const lds_byte* const zero = (const lds_byte*)0;
+        if (!last)
+            tile_accumulate_and_scores<kBf16>(zero, zero, fs, pf, o, qf, st.neg_ref, s);
+        else
+            tile_accumulate<kBf16>(zero, fs, pf, o);
+        __builtin_amdgcn_s_setprio(0);
+        FLASH_STAMP(clk, 5);
+        barrier_keeping_loads(recent);
+        FLASH_STAMP(clk, 6);
+    };
+    for (int j = 0; j < n - 1; j++)
+        two_phases(j, false, k_stage(j + 1), v_stage(j), k_stage(j + group + 2), v_stage(j + group + 1));
+    two_phases(n - 1, true, k_stage(n), v_stage(n - 1), k_stage(n + group + 1), v_stage(n + group));
+    if (group == 0) barrier_keeping_loads(0);  // as many barriers as group 1
+#ifdef HIPATTN_FLASH_TRACE
+    if (g_flash_phase_trace && lane == 0) {
+        long long* r = g_flash_phase_trace + ((int64_t)blockIdx.x * 8 + wave) * 8;
+        for (int k = 0; k < 7; k++) r[k] = clk.acc[k];
+        r[7] = n;
+    }
+    if (g_flash_raw_trace && lane == 0 && blockIdx.x == 0 && n >= 12)
+        for (int k = 0; k < 8; k++) g_flash_raw_trace[wave * 16 + k] = clk.raw[k];
+#endif
+
+    // ---- normalise and store
+    float l_lo, l_hi;
+    pair_values(st.l_run, l_lo, l_hi);
+    const float l_row = l_lo + l_hi;
+    const float inv = l_row > 0.0f ? 1.0f / l_row : 0.0f;
+    lds_byte* const out_stage = wave_stage;
+    const int row0 = (wave & 3) * 32;
+    if (t.out_dtype == HIPATTN_F32) {
+        if (row < t.rows) store_rows<HIPATTN_F32>(t, o, inv, row, hi);
+    } else if (t.out_dtype == HIPATTN_F16) {
+        store_rows_via_lds<false>(t, o, inv, out_stage, row0, lane);
+    } else {
+        store_rows_via_lds<true>(t, o, inv, out_stage, row0, lane);
     }
 }
 
-// Number of work items of a dense call, and item -> tiles.  Items are ordered (batch, kv head,
-// query tile descending, pair): consecutive items share one K/V head, and the heaviest (latest)
-// causal tiles of a head come first.  With an even number of query heads per kv head the two
-// groups of a workgroup take two heads at the same query tile; otherwise they take two
-// consecutive query tiles of one head.
-__device__ __host__ __forceinline__ int sdpa_item_count(const SdpaParams& p) {
-    const int G = p.num_heads_q / p.num_heads_kv;
-    const int n_qt = (p.len_q + kTileQ - 1) / kTileQ;
-    const int per_kv_head = (G & 1) == 0 ? (G / 2) * n_qt : G * ((n_qt + 1) / 2);
-    return per_kv_head * p.num_heads_kv * p.batch;
-}
+// Launch index -> work item: workgroups go to the eight XCDs round-robin by launch index and
+// each XCD has its own L2, so index i becomes item (i % 8) * (n / 8) + i / 8.  An XCD then walks
+// a contiguous range of items ordered (batch, kv head, query tile descending, pair): the
+// workgroups resident on it at one time share one K/V head, which stays in that L2, and the
+// heaviest (latest) causal tiles of a head come first.  With an even number of query heads per
+// kv head the two groups of a workgroup take two heads at the same query tile; otherwise they
+// take two consecutive query tiles of one head.
 // a / b for wave-uniform 0 <= a < 2^22 and 1 <= b < 2^22: a float reciprocal and one correction
-// step instead of the long 32-bit division sequence (an item is decoded several times per item).
+// step instead of the long 32-bit division sequence.
 __device__ __forceinline__ int small_div(int a, int b) {
     int q = (int)((float)a * __builtin_amdgcn_rcpf((float)b));  // off by at most one
     const int r = a - q * b;
@@ -884,12 +750,15 @@ __device__ __forceinline__ int small_div(int a, int b) {
     q -= (r < 0) ? 1 : 0;
     return q;
 }
-__device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int item, int group) {
+__device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) {
     const int G = small_div(p.num_heads_q, p.num_heads_kv);
     const int n_qt = (p.len_q + kTileQ - 1) / kTileQ;
     const bool pair_heads = (G & 1) == 0;
     const int slots = pair_heads ? n_qt : (n_qt + 1) / 2;  // query positions of a head's workgroups
     const int lanes = pair_heads ? G / 2 : G;              // workgroups per query position
+    const int n_items = (int)gridDim.x;
+    int item = (int)blockIdx.x;
+    if ((n_items & 7) == 0) item = (item & 7) * (n_items >> 3) + (item >> 3);
     const int by_lane = small_div(item, lanes), li = item - by_lane * lanes;
     const int by_slot = small_div(by_lane, slots), slot = slots - 1 - (by_lane - by_slot * slots);
     const int b = small_div(by_slot, p.num_heads_kv), hkv = by_slot - b * p.num_heads_kv;
@@ -920,38 +789,28 @@ __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int item, i
     return t;
 }
 
-// The dense kernel is persistent: the launch has one workgroup per compute unit (a workgroup
-// takes a whole one: 160 KB of LDS, eight wavefronts of 256 registers), and workgroup w works
-// through its share of the items in rounds.  Workgroups go to the eight XCDs round-robin by
-// launch index and each XCD has its own L2, so the items are cut into eight contiguous ranges,
-// one per XCD: the workgroups resident on an XCD at one time then share one K/V head, which
-// stays in that L2.  Within its range a workgroup takes item w' of the even rounds and item
-// W' - 1 - w' of the odd ones (w' its index among the W' workgroups of the XCD): the causal
-// weights of a round fall with the item index, and the reversal pairs a heavy item with a light
-// one, so that all workgroups finish together without a work queue.
-struct SdpaFeed {
-    const SdpaParams& p;
-    int n_items;
-    __device__ __forceinline__ bool operator()(int round, int group, Item& it) const {
-        const int W = (int)gridDim.x, w = (int)blockIdx.x;
-        int item;
-        if ((n_items & 7) == 0 && (W & 7) == 0) {
-            const int wx = W >> 3, per = n_items >> 3, lw = w >> 3;
-            const int local = round * wx + ((round & 1) ? wx - 1 - lw : lw);
-            if (local >= per) return false;
-            item = (w & 7) * per + local;
-        } else {
-            item = round * W + ((round & 1) ? W - 1 - w : w);
-            if (item >= n_items) return false;
-        }
-        make_item(sdpa_group_tile(p, item, group), sdpa_group_tile(p, item, group ^ 1), it);
-        return true;
+template <bool kBf16>
+__device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t* lds, float scale) {
+    int lo0, hi0, lo1, hi1;
+    key_range(t0, lo0, hi0);
+    key_range(t1, lo1, hi1);
+    int kv_lo, kv_hi;
+    if (hi0 <= lo0) {
+        kv_lo = lo1;
+        kv_hi = hi1;
+    } else if (hi1 <= lo1) {
+        kv_lo = lo0;
+        kv_hi = hi0;
+    } else {
+        kv_lo = min(lo0, lo1);
+        kv_hi = max(hi0, hi1);
     }
-};
+    const int group = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
+    run_pair<kBf16>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
+}
 
 template <bool kBf16>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p,
-                                                                                                        int n_items) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
 #ifdef HIPATTN_FLASH_TRACE
     long long w0 = 0, c0 = 0;
@@ -960,7 +819,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         c0 = (long long)__builtin_readcyclecounter();
     }
 #endif
-    run_items<kBf16, false>(SdpaFeed{p, n_items}, lds, p.scale);
+    const Tile t0 = sdpa_group_tile(p, 0), t1 = sdpa_group_tile(p, 1);
+    run_both<kBf16>(t0, t1, lds, p.scale);
 #ifdef HIPATTN_FLASH_TRACE
     if (g_flash_wg_trace && threadIdx.x == 0) {
         long long* r = g_flash_wg_trace + (int64_t)blockIdx.x * 8;
@@ -970,7 +830,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         r[3] = (long long)__builtin_readcyclecounter();
         r[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID
         r[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
-        r[6] = 0;
+        r[6] = t0.pos0 / kTileQ;
     }
 #endif
 }
@@ -1009,20 +869,6 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
     return t;
 }
 
-// the single item of a paged workgroup
-struct PagedFeed {
-    const PagedParams& p;
-    int s, qt, h0;
-    bool pair_heads;
-    __device__ __forceinline__ bool operator()(int round, int group, Item& it) const {
-        if (round > 0) return false;
-        // group 0 always has work; group 1 takes the second head of the pair, if there is one
-        make_item(paged_group_tile(p, s, qt, pair_heads ? h0 + group : h0, pair_heads || group == 0),
-                  paged_group_tile(p, s, qt, pair_heads ? h0 + (group ^ 1) : h0, pair_heads || group == 1), it);
-        return true;
-    }
-};
-
 template <bool kBf16>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
@@ -1043,38 +889,32 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int G = p.num_heads_q / p.num_heads_kv;
     const bool pair_heads = (G & 1) == 0;
     const int h0 = pair_heads ? 2 * (int)blockIdx.y : (int)blockIdx.y;
-    run_items<kBf16, true>(PagedFeed{p, s, qt, h0, pair_heads}, lds, p.scale);
+    const Tile t0 = paged_group_tile(p, s, qt, h0, true);
+    const Tile t1 = paged_group_tile(p, s, qt, pair_heads ? h0 + 1 : h0, pair_heads);
+    run_both<kBf16>(t0, t1, lds, p.scale);
 }
 
 }  // namespace flash
 
 bool sdpa_flash_supported(const SdpaParams& p) {
-    return p.head_dim == flash::kD && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16);
-}
-
-// compute units of the current device (a persistent launch has one workgroup per unit)
-static int current_device_compute_units() {
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int cus = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        cached[dev] = cus;
-    }
-    return cached[dev];
+    if (p.head_dim != flash::kD || !(p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16)) return false;
+    // the kernel decodes its launch index with small_div: the number of workgroups must stay below 2^22
+    const int64_t q_tiles = ((int64_t)p.len_q + flash::kTileQ - 1) / flash::kTileQ;
+    return (int64_t)p.batch * p.num_heads_q * q_tiles < (int64_t(1) << 22);
 }
 
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe) {
     if (p.batch == 0 || p.len_q == 0) return hipSuccess;
-    const int n_items = flash::sdpa_item_count(p);
-    const int cus = current_device_compute_units();
-    dim3 grid(n_items < cus ? n_items : cus);
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const int n_qt = (p.len_q + flash::kTileQ - 1) / flash::kTileQ;
+    const bool pair_heads = (G & 1) == 0;
+    const int per_kv_head = pair_heads ? (G / 2) * n_qt : G * ((n_qt + 1) / 2);
+    dim3 grid(per_kv_head * p.num_heads_kv * p.batch);
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     if (p.dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p, n_items);
+        hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
     else
-        hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p, n_items);
+        hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     return e;
