@@ -488,6 +488,28 @@ __device__ __forceinline__ void barrier_keeping() {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 }
+// Waits until at most `keep` (even, <= 10, wave-uniform) of this wavefront's global->LDS loads are
+// in flight, without a barrier: enough for data that only this wavefront reads.
+template <int kKeep>
+__device__ __forceinline__ void wait_keeping() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (kKeep & 15) | ((kKeep >> 4) << 14));  // vmcnt only
+    asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ void wait_keeping_loads(int keep) {
+    if (keep >= 10)
+        wait_keeping<10>();
+    else if (keep >= 8)
+        wait_keeping<8>();
+    else if (keep >= 6)
+        wait_keeping<6>();
+    else if (keep >= 4)
+        wait_keeping<4>();
+    else if (keep >= 2)
+        wait_keeping<2>();
+    else
+        wait_keeping<0>();
+}
 __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0, 2 or 4 (wave-uniform)
     if (keep >= 4)
         barrier_keeping<4>();
@@ -623,14 +645,15 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
 
     // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
     const int e0 = table_entry(0), e1 = table_entry(1), e2 = table_entry(2), e3 = table_entry(3);
-    load_rows(true, 0, k_stage(0), e0);
-    load_rows(false, 0, v_stage(0), e0);
-    load_rows(true, 1, k_stage(1), e1);
+    const int first = load_rows(true, 0, k_stage(0), e0) + load_rows(false, 0, v_stage(0), e0) +
+                      load_rows(true, 1, k_stage(1), e1);
     int recent = 0;
     if (group == 1) recent = load_rows(true, 2, k_stage(2), e2) + load_rows(false, 1, v_stage(1), e1);
     // entries of the tiles the first iteration loads: K(group + 2) and V(group + 1)
     int entry_v = group ? e2 : e1, entry_k = group ? e3 : e2;
-    barrier_keeping_loads(recent);  // (also: this wavefront's query rows have landed)
+    // The query rows were issued first and nobody else reads them: they are converted while the
+    // K and V tiles are still on their way.
+    wait_keeping_loads(first + recent);
     // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
     vec8 qf[8];
     {
@@ -649,6 +672,9 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             for (int i = 0; i < 8; i++) qf[i] = convert_q_frag<kBf16, false>(raw[i], c);
         }
     }
+#pragma unroll
+    for (int i = 0; i < 8; i++) asm volatile("" : "+v"(qf[i]));  // (converted before the wait below, not after)
+    barrier_keeping_loads(recent);
     if (group == 1) barrier_keeping_loads(recent);  // group 1 sits out phase 0
 
     float16_t s[2];
@@ -707,7 +733,6 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     for (int j = 0; j < n - 1; j++)
         two_phases(j, false, k_stage(j + 1), v_stage(j), k_stage(j + group + 2), v_stage(j + group + 1));
     two_phases(n - 1, true, k_stage(n), v_stage(n - 1), k_stage(n + group + 1), v_stage(n + group));
-    if (group == 0) barrier_keeping_loads(0);  // as many barriers as group 1
 #ifdef HIPATTN_FLASH_TRACE
     if (g_flash_phase_trace && lane == 0) {
         long long* r = g_flash_phase_trace + ((int64_t)blockIdx.x * 8 + wave) * 8;
@@ -732,6 +757,8 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     } else {
         store_rows_via_lds<true>(t, o, inv, out_stage, row0, lane);
     }
+    // as many barriers as group 1, whose last phase runs while group 0 stores its rows
+    if (group == 0) barrier_keeping_loads(0);
 }
 
 // Launch index -> work item: workgroups go to the eight XCDs round-robin by launch index and
