@@ -41,6 +41,7 @@
 // src/ops/softmax.cpp:184-192).
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "device_common.hpp"
 #include "kernels.hpp"
@@ -116,6 +117,10 @@ __device__ __forceinline__ uint32_t bytes_to_biased_half2(uint32_t lo_src, uint3
     return __builtin_amdgcn_perm(hi_src, lo_src, sel) | 0x64006400u;
 }
 
+#ifndef HIPATTN_U8_STAGES
+#define HIPATTN_U8_STAGES 3
+#endif
+
 template <bool kU8>
 struct BlockRegs;
 
@@ -129,9 +134,18 @@ template <>
 struct BlockRegs<true> {
     uint2_t k[2][4];  // 8 bytes each
     uint2_t v[8];
-    float2 ksz[8];    // (scale, zp) of K for token j = tile*4 + r of this lane
-    float2 vsz[8];
+    // (scale, zp) of one token: lane (i = lane & 15, kg) holds those of the K row (i < 8) or V row
+    // (i >= 8) of token j = i & 7 of its 16-lane row, i.e. of token (j >> 2) * 16 + kg * 4 + (j & 3);
+    // the lanes of the row read them with a DPP row broadcast.  (Loading all eight pairs of K and
+    // of V into every lane costs sixteen load instructions and 32 registers per block.)
+    float2 sz;
 };
+
+// value of lane kLane of the caller's 16-lane row (v_mov_b32 row_newbcast, folded into the consumer where possible)
+template <int kLane>
+__device__ __forceinline__ float row_broadcast(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x150 + kLane, 0xf, 0xf, false));
+}
 
 template <bool kU8>
 __device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* kbase, const uint8_t* vbase, int n16,
@@ -160,9 +174,11 @@ __device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* kba
             for (int r = 0; r < 4; r++) {
                 const int tok = t * 16 + kg * 4 + r;
                 b.v[t * 4 + r] = *(const uint2_t*)(vbase + tok * kRow + 8 + n16 * 8);
-                b.ksz[t * 4 + r] = *(const float2*)(kbase + tok * kRow);
-                b.vsz[t * 4 + r] = *(const float2*)(vbase + tok * kRow);
             }
+        {
+            const int j = n16 & 7, tok = (j >> 2) * 16 + kg * 4 + (j & 3);
+            b.sz = *(const float2*)((n16 < 8 ? kbase : vbase) + tok * kRow);
+        }
     }
 }
 
@@ -200,6 +216,25 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
     // ---- mask, scale, online softmax.  Lane holds tokens tok_base + t*16 + kg*4 + r.
     float sv[8];
     float mloc = -INFINITY;
+    // u8: this lane's token's scale, zero-point plus byte bias, and their product (see BlockRegs)
+    float sz_scale = 0.0f, sz_zero = 0.0f, sz_prod = 0.0f;
+    const bool partial = (tok_base < j0) || (tok_base + kBS > ctx);  // wavefront-uniform
+    if constexpr (kU8) {
+        sz_scale = b.sz.x;
+        sz_zero = b.sz.y + kByteBias;
+        if (partial) {
+            // Rows outside the attended range may hold anything (never-written cache memory): their
+            // probability is exactly zero, and their scale and zero-point are cleared so that
+            // 0 * NaN cannot occur.
+            const int j = ((int)threadIdx.x & 7), tok = tok_base + (j >> 2) * 16 + kg * 4 + (j & 3);
+            if (!(tok >= j0 && tok < ctx)) sz_scale = sz_zero = 0.0f;
+        }
+        sz_prod = sz_scale * sz_zero;
+    }
+    auto dequant_score = [&](auto jc, float x) {
+        constexpr int j = decltype(jc)::value;
+        return fmaf(row_broadcast<j>(sz_scale), x, -(row_broadcast<j>(sz_prod) * sumq));
+    };
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -207,7 +242,18 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
             const int j = t * 4 + r;
             const int tok = tok_base + t * 16 + kg * 4 + r;
             float x = s[t][r];
-            if constexpr (kU8) x = b.ksz[j].x * (x - (b.ksz[j].y + kByteBias) * sumq);
+            if constexpr (kU8) {
+                switch (j) {
+                    case 0: x = dequant_score(std::integral_constant<int, 0>{}, x); break;
+                    case 1: x = dequant_score(std::integral_constant<int, 1>{}, x); break;
+                    case 2: x = dequant_score(std::integral_constant<int, 2>{}, x); break;
+                    case 3: x = dequant_score(std::integral_constant<int, 3>{}, x); break;
+                    case 4: x = dequant_score(std::integral_constant<int, 4>{}, x); break;
+                    case 5: x = dequant_score(std::integral_constant<int, 5>{}, x); break;
+                    case 6: x = dequant_score(std::integral_constant<int, 6>{}, x); break;
+                    default: x = dequant_score(std::integral_constant<int, 7>{}, x); break;
+                }
+            }
             x = (tok >= j0 && tok < ctx) ? x * c : -INFINITY;
             sv[j] = x;
             mloc = fmaxf(mloc, x);
@@ -219,17 +265,12 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
     st.m = m_new;
     // Rows outside the attended range may hold anything (never-written cache memory): their
     // probability is exactly zero, and fp16 V rows are cleared so that 0 * NaN cannot occur.
-    const bool partial = (tok_base < j0) || (tok_base + kBS > ctx);  // wavefront-uniform
-    if (partial) {
+    if constexpr (!kU8) {
+        if (partial) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int tok = tok_base + (j >> 2) * 16 + kg * 4 + (j & 3);
-            if (!(tok >= j0 && tok < ctx)) {
-                if constexpr (kU8) {
-                    b.vsz[j] = make_float2(0.0f, 0.0f);
-                } else {
-                    b.v[j] = (uint4_t){0u, 0u, 0u, 0u};
-                }
+            for (int j = 0; j < 8; j++) {
+                const int tok = tok_base + (j >> 2) * 16 + kg * 4 + (j & 3);
+                if (!(tok >= j0 && tok < ctx)) b.v[j] = (uint4_t){0u, 0u, 0u, 0u};
             }
         }
     }
@@ -240,9 +281,20 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
         float pj = fast_exp2(sv[j] - m_new);
         lsum += pj;
         if constexpr (kU8) {
-            pj *= b.vsz[j].x;
+            float vs, vz;  // scale and zero-point (plus bias) of V's token j: lanes 8 + j of the row
+            switch (j) {
+                case 0: vs = row_broadcast<8>(sz_scale); vz = row_broadcast<8>(sz_zero); break;
+                case 1: vs = row_broadcast<9>(sz_scale); vz = row_broadcast<9>(sz_zero); break;
+                case 2: vs = row_broadcast<10>(sz_scale); vz = row_broadcast<10>(sz_zero); break;
+                case 3: vs = row_broadcast<11>(sz_scale); vz = row_broadcast<11>(sz_zero); break;
+                case 4: vs = row_broadcast<12>(sz_scale); vz = row_broadcast<12>(sz_zero); break;
+                case 5: vs = row_broadcast<13>(sz_scale); vz = row_broadcast<13>(sz_zero); break;
+                case 6: vs = row_broadcast<14>(sz_scale); vz = row_broadcast<14>(sz_zero); break;
+                default: vs = row_broadcast<15>(sz_scale); vz = row_broadcast<15>(sz_zero); break;
+            }
+            pj *= vs;
             const half_t ph = (half_t)pj;
-            csum = fmaf((float)ph, b.vsz[j].y + kByteBias, csum);
+            csum = fmaf((float)ph, vz, csum);
             pf[j] = ph;
         } else {
             pf[j] = (half_t)pj;
@@ -543,19 +595,44 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 load_block<kU8>(regs, p.key_cache + off, p.value_cache + off, n16, kg);
                 return true;
             };
-            // two register stages: block i+1 is in flight while block i is consumed
-            BlockRegs<kU8> ra, rb;
-            bool ok_a = issue(ra, 0), ok_b = false;
-            int i = 0;
-            while (i < gn) {
-                ok_b = (i + 1 < gn) ? issue(rb, i + 1) : false;
-                if (ok_a) process_block<kU8>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
-                if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
-                blocks_done = 1;
-                if (i + 1 >= gn) break;
-                ok_a = (i + 2 < gn) ? issue(ra, i + 2) : false;
-                if (ok_b) process_block<kU8>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
-                i += 2;
+            if constexpr (!kU8) {
+                // two register stages: block i+1 is in flight while block i is consumed
+                BlockRegs<kU8> ra, rb;
+                bool ok_a = issue(ra, 0), ok_b = false;
+                int i = 0;
+                while (i < gn) {
+                    ok_b = (i + 1 < gn) ? issue(rb, i + 1) : false;
+                    if (ok_a) process_block<kU8>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
+                    if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
+                    blocks_done = 1;
+                    if (i + 1 >= gn) break;
+                    ok_a = (i + 2 < gn) ? issue(ra, i + 2) : false;
+                    if (ok_b) process_block<kU8>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
+                    i += 2;
+                }
+            } else {
+                // kStages register stages: blocks i+1 .. i+kStages-1 are in flight while block i is
+                // consumed.  A wavefront's loads in flight are what keeps HBM busy (eight wavefronts
+                // per compute unit): a u8 block-head is 8.5 KB against 16 KB in fp16 and its stage
+                // takes half as many registers, so the u8 kernel keeps one block more in flight.
+                constexpr int kStages = HIPATTN_U8_STAGES;
+                BlockRegs<kU8> regs[kStages];
+                bool ok[kStages];
+#pragma unroll
+                for (int u = 0; u < kStages - 1; u++) ok[u] = (u < gn) ? issue(regs[u], u) : false;
+                for (int i = 0; i < gn; i += kStages) {
+#pragma unroll
+                    for (int u = 0; u < kStages; u++) {
+                        const int idx = i + u;
+                        if (idx >= gn) break;
+                        constexpr int kLast = kStages - 1;
+                        ok[(u + kLast) % kStages] =
+                            (idx + kLast < gn) ? issue(regs[(u + kLast) % kStages], idx + kLast) : false;
+                        if (ok[u]) process_block<kU8>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kBS, rg.j0, rg.ctx, kg);
+                        if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
+                        blocks_done = 1;
+                    }
+                }
             }
         }
 
