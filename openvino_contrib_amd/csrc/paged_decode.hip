@@ -118,7 +118,7 @@ __device__ __forceinline__ uint32_t bytes_to_biased_half2(uint32_t lo_src, uint3
 }
 
 #ifndef HIPATTN_U8_STAGES
-#define HIPATTN_U8_STAGES 3
+#define HIPATTN_U8_STAGES 2
 #endif
 
 template <bool kU8>
@@ -612,9 +612,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 }
             } else {
                 // kStages register stages: blocks i+1 .. i+kStages-1 are in flight while block i is
-                // consumed.  A wavefront's loads in flight are what keeps HBM busy (eight wavefronts
-                // per compute unit): a u8 block-head is 8.5 KB against 16 KB in fp16 and its stage
-                // takes half as many registers, so the u8 kernel keeps one block more in flight.
+                // consumed.  (Measured on the 128-sequence u8 workload: two stages 452 us, three 455 us,
+                // four spill registers and fall to 629 us.)
                 constexpr int kStages = HIPATTN_U8_STAGES;
                 BlockRegs<kU8> regs[kStages];
                 bool ok[kStages];
