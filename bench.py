@@ -203,15 +203,20 @@ def cpu_baseline_sdpa(case, budget_s=20.0):
 
 
 def main():
+    global CLOCK_RAMP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters")
+    ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
+                    help="untimed GPU time of the step run ahead of the warmup steps (0 for hardware-counter runs, "
+                         "which only count bytes)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="measure the headline workload only")
     args = ap.parse_args()
+    CLOCK_RAMP_MS = args.ramp_ms
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
 
