@@ -137,10 +137,10 @@ def bench_sdpa(hip, case, steps, warmup, name):
 # counters cannot be read from inside this process, so these are the recorded figures for the
 # default seeds; None where no counter run exists.
 MEASURED_TRAFFIC_BYTES = {
-    "c3": (563487.2 * 2.0 + 3031.0) * 1024,
-    "c4": (1220709.5 * 2.0 + 12253.3) * 1024,
-    "c2": (49280.2 * 2.0 + 65536.0) * 1024,
-    "c5": (786661.7 * 2.0 + 7602.2) * 1024,  # the decode kernel of the mixed step
+    "c3": (563502.7 * 2.0 + 3031.8) * 1024,
+    "c4": (1220744.2 * 2.0 + 12203.6) * 1024,
+    "c2": (49294.0 * 2.0 + 65536.0) * 1024,
+    "c5": (786659.0 * 2.0 + 7600.9) * 1024,  # the decode kernel of the mixed step
 }
 
 
