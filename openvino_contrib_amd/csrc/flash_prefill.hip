@@ -264,6 +264,7 @@ struct SoftmaxState {
     float16_t neg_ref;  // -ref in every element
     float l_run;        // this lane's half of the row sum
     bool started;       // the row has met a key it may attend to
+    bool all_started;   // wave-uniform: every row of the wavefront has
 };
 
 // Mask, reference update and probabilities of the tile that starts at key ts (register r of s[mt]
@@ -285,6 +286,36 @@ __device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], f
                 if (t.window > 0) ok = ok && key > my_pos - t.window;
                 s[mt][r] = ok ? s[mt][r] : -INFINITY;
             }
+    }
+    // probabilities of the tile against the current reference, and this lane's share of their sum
+    auto probabilities = [&]() __attribute__((always_inline)) -> float {
+        float sum = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            uint4_t pw;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w]);
+                const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1]);
+                pw[w] = M::cvt2(p0, p1);
+                sum += p0 + p1;  // (not v_dot2: dot instructions wait for the matrix core, which the other group keeps busy)
+            }
+            pf[ks] = __builtin_bit_cast(vec8, pw);
+        }
+        return sum;
+    };
+    // Common case (an unmasked tile, every row already has a reference): no row maximum at all.
+    // The exponentials are taken against the standing reference and the tile's row sums tell
+    // whether that was safe: a sum below 2^24 bounds every probability, and anything else (large,
+    // infinite, NaN) sends the wavefront through the careful path below, which redoes the tile
+    // from the untouched scores.  Sixteen v_max3, the cross-lane exchange and the compare of the
+    // maximum are then spent only on the first tile of a row, on masked tiles and on outliers.
+    if (!masked && st.all_started) {
+        const float sum = probabilities();
+        if (!__builtin_amdgcn_ballot_w64(!(sum < 16777216.0f))) {
+            st.l_run += sum;
+            return;
+        }
     }
     float m_tile = -INFINITY;
 #pragma unroll
@@ -309,21 +340,9 @@ __device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], f
         for (int mt = 0; mt < 2; mt++) s[mt] -= delta;
         st.neg_ref -= delta;
         st.started = st.started || seen;
+        st.all_started = __builtin_amdgcn_ballot_w64(!st.started) == 0;
     }
-    float lsum = st.l_run;
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-        uint4_t pw;
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-            const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w]);
-            const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1]);
-            pw[w] = M::cvt2(p0, p1);
-            lsum += p0 + p1;  // (not v_dot2: dot instructions wait for the matrix core, which the other group keeps busy)
-        }
-        pf[ks] = __builtin_bit_cast(vec8, pw);
-    }
-    st.l_run = lsum;
+    st.l_run += probabilities();
 }
 
 // The fragments of a product are read from LDS in batches of four, each batch one batch of MFMAs
@@ -589,6 +608,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     for (int r = 0; r < 16; r++) st.neg_ref[r] = 0.0f;
     st.l_run = 0.0f;
     st.started = false;
+    st.all_started = false;
     const int my_pos = t.pos0 + row;  // position of this lane's query row
     const FragOffsets f = frag_offsets(lane);
 
