@@ -208,8 +208,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy"],
-                    help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters")
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy", "mfma"],
+                    help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
+                         "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
                     help="untimed GPU time of the step run ahead of the warmup steps (0 for hardware-counter runs, "
                          "which only count bytes)")
@@ -230,6 +231,18 @@ def main():
     info = hip.device_info(0)
     dev_name = info.name.decode() or ("AMD " + info.arch.decode())
     log("device:", dev_name, info.arch.decode(), info.compute_units, "CUs")
+
+    if args.workload == "mfma":
+        # What the device sustains on v_mfma_f32_32x32x16_bf16 alone, and at which shader clock, with
+        # random and with all-zero operands (the power an MFMA draws follows the bits that toggle).
+        import ctypes
+        out = {"workload": "mfma", "peak_tflops": MFMA_BF16_PEAK_TFLOPS}
+        for name, zero in (("random_operands", 0), ("zero_operands", 1)):
+            tf, ghz = ctypes.c_double(), ctypes.c_double()
+            hip.check(hip.lib().hipattn_mfma_yardstick(zero, max(args.steps, 50), ctypes.byref(tf), ctypes.byref(ghz), None))
+            out[name] = {"tflops": tf.value, "shader_ghz": ghz.value, "frac_of_peak": tf.value / MFMA_BF16_PEAK_TFLOPS}
+        print(json.dumps(out))
+        return
 
     if args.workload == "copy":
         # Known-size traffic for scaling FETCH_SIZE / WRITE_SIZE: a device-to-device copy of 1 GiB

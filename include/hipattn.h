@@ -85,6 +85,12 @@ hipattn_status hipattn_memcpy_d2h_async(void* host_dst, const void* device_src, 
 hipattn_status hipattn_memcpy_d2d_async(void* device_dst, const void* device_src, size_t bytes, hipattn_stream stream);
 /* byte fill done by a kernel (safe to record into a captured graph) */
 hipattn_status hipattn_fill_async(void* device_dst, int byte_value, size_t bytes, hipattn_stream stream);
+/* Diagnostic without a counterpart in the reference: the rate (TFLOP/s) and shader clock (GHz) the
+ * current device sustains on register-fed v_mfma_f32_32x32x16_bf16 alone, with all-zero or with
+ * random operands; the yardstick for the MFMA-bound kernels, as a plain copy is for the
+ * HBM-bound ones.  Runs 2 x launches kernels (half of them untimed), allocates and frees its own
+ * few KB, and synchronises the stream. */
+hipattn_status hipattn_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz, hipattn_stream stream);
 
 hipattn_status hipattn_event_create(hipattn_event* event);
 hipattn_status hipattn_event_destroy(hipattn_event event);

@@ -20,6 +20,7 @@ SOURCES = [
     "attention_generic.hip",
     "paged_decode.hip",
     "flash_prefill.hip",
+    "yardstick.hip",
 ]
 
 HIPCC_FLAGS = [

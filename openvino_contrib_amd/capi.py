@@ -96,6 +96,7 @@ SYMBOLS = {
     "hipattn_memcpy_d2h_async": (_i, [_vp, _vp, _sz, _vp]),
     "hipattn_memcpy_d2d_async": (_i, [_vp, _vp, _sz, _vp]),
     "hipattn_fill_async": (_i, [_vp, _i, _sz, _vp]),
+    "hipattn_mfma_yardstick": (_i, [_i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), _vp]),
     "hipattn_event_create": (_i, [_P(_vp)]),
     "hipattn_event_destroy": (_i, [_vp]),
     "hipattn_event_record": (_i, [_vp, _vp]),

@@ -284,6 +284,14 @@ HIPATTN_EXPORT hipattn_status hipattn_fill_async(void* device_dst, int byte_valu
     return HIPATTN_OK;
 }
 
+HIPATTN_EXPORT hipattn_status hipattn_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz,
+                                                     hipattn_stream stream) {
+    if (!tflops || !shader_ghz) return fail(HIPATTN_INVALID_ARGUMENT, "mfma_yardstick: null output");
+    if (launches < 1 || launches > 100000) return fail(HIPATTN_INVALID_ARGUMENT, "mfma_yardstick: launches out of range");
+    HIP_TRY(hipattn::run_mfma_yardstick(zero_data, launches, tflops, shader_ghz, as_stream(stream)));
+    return HIPATTN_OK;
+}
+
 HIPATTN_EXPORT hipattn_status hipattn_event_create(hipattn_event* event) {
     if (!event) return fail(HIPATTN_INVALID_ARGUMENT, "event_create: null output");
     hipEvent_t e;

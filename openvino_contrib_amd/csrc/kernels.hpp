@@ -112,5 +112,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream);  // flash over the block table (needs the plan)
 
 hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t stream);
+// diagnostic: sustained register-fed bf16 MFMA rate and shader clock of the current device (yardstick.hip)
+hipError_t run_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz, hipStream_t stream);
 
 }  // namespace hipattn

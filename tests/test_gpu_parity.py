@@ -303,3 +303,15 @@ def test_paged_errors(hip):
                             dev.subsequence_begins, dev.block_indices, dev.block_indices_begins, dev.out, small)
     assert e.value.status == hip.INVALID_ARGUMENT
     dev.free()
+
+
+@pytest.mark.gpu
+def test_mfma_yardstick_reports_a_plausible_rate(hip):
+    """The diagnostic that bench.py --workload mfma prints: register-fed bf16 MFMAs only."""
+    import ctypes
+    tf, ghz = ctypes.c_double(), ctypes.c_double()
+    hip.check(hip.lib().hipattn_mfma_yardstick(1, 20, ctypes.byref(tf), ctypes.byref(ghz), None))
+    assert 500.0 < tf.value < 2600.0   # never above the 2.5 PFLOP/s dense bf16 peak (plus timer slack)
+    assert 1.0 < ghz.value < 2.6
+    assert hip.lib().hipattn_mfma_yardstick(0, 0, ctypes.byref(tf), ctypes.byref(ghz), None) == hip.INVALID_ARGUMENT
+
