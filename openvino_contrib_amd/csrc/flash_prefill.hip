@@ -8,15 +8,18 @@
 // (global_load_lds_dwordx4: no staging registers, no LDS write instructions), row-major with
 // the 16-byte chunks of a row XOR-swizzled so that fragment reads are free of bank conflicts;
 // the V^T operand is read with the transposing LDS load ds_read_b64_tr_b16.  LDS holds a ring of
-// three K and three V stages, filled two tiles ahead.
+// three K and three V stages, filled two tiles ahead, and 8 KB per wavefront through which its
+// query rows come in and its output rows go out as whole rows (160 KB in all: one workgroup per
+// compute unit).
 //
 // One wavefront of each group sits on every SIMD, and the two alternate between a matrix phase
 // (O += P V of one tile, then the scores of the next) and a vector phase (mask, running
 // reference, exp2, conversion and row sums of the scores just computed, plus the issue of the
 // global->LDS loads), separated by workgroup barriers: while one group feeds the matrix core the
-// other keeps the vector ALU busy, by construction rather than by chance.  A SIMD runs an MFMA
-// stream at full rate next to another wavefront's VALU stream, but a single wavefront cannot
-// overlap the two beyond a handful of instructions.
+// other keeps the vector ALU busy, by construction rather than by chance.  (A variant in which
+// every wavefront interleaves the exponentials of one tile with its own score MFMAs of the next
+// needs about 5 % fewer cycles and takes the same time: with real data the kernel runs at the
+// machine's power limit, and the clock settles lower for the denser instruction stream.)
 //
 // Both products run on v_mfma_f32_32x32x16 (f16 or bf16) with fp32 accumulation:
 //   S^T = K Q^T   (M = 32 keys, N = 32 query rows, contraction over head_dim)
