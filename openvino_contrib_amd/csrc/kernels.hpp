@@ -26,7 +26,17 @@ struct KvWriteParams {
     int head_dim;
     int block_size;
     int num_blocks;
+    // kv heads one wavefront writes (set by kv_write_wavefronts): 1 for small batches, all of a
+    // token's heads for large ones, where looking up the token's slot per head would dominate
+    int heads_per_wave;
 };
+
+// Wavefronts the writer needs for p (and p.heads_per_wave, which it sets).
+inline int64_t kv_write_wavefronts(KvWriteParams& p) {
+    const int64_t pairs = (int64_t)p.num_tokens * p.num_heads_kv;
+    p.heads_per_wave = pairs > 16384 ? p.num_heads_kv : 1;
+    return (int64_t)p.num_tokens * ((p.num_heads_kv + p.heads_per_wave - 1) / p.heads_per_wave);
+}
 
 struct SdpaParams {
     const void* q;

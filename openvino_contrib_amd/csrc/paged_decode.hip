@@ -382,13 +382,11 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
 }
 
 // One launch for step 1 of the operator and the schedule: workgroups [0, write_blocks) scatter
-// the new K/V rows into the caches (four (token, kv head) pairs each), workgroup write_blocks
+// the new K/V rows into the caches (four wavefronts of the writer each), workgroup write_blocks
 // plans.  The plan reads lengths only, never the cache, so the two parts do not interact.
 __global__ __launch_bounds__(256) void paged_prologue_kernel(KvWriteParams wp, PagedParams p, int write_blocks) {
     if ((int)blockIdx.x < write_blocks) {
-        const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
-        if (pair < wp.num_tokens * wp.num_heads_kv)
-            kv_cache_write_pair<2>(wp, pair / wp.num_heads_kv, pair % wp.num_heads_kv, threadIdx.x & 63);
+        kv_cache_write_wave<2>(wp, (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), threadIdx.x & 63);
     } else {
         plan_block(p);
     }
@@ -800,7 +798,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     if (write) {
         wp = *write;
         if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head_dim 128 only
-        write_blocks = (int)(((int64_t)wp.num_tokens * wp.num_heads_kv + 3) / 4);
+        write_blocks = (int)((kv_write_wavefronts(wp) + 3) / 4);
     }
     hipLaunchKernelGGL(paged_prologue_kernel, dim3(write_blocks + 1), dim3(256), 0, stream, wp, p, write_blocks);
     hipError_t e = hipGetLastError();
