@@ -922,23 +922,40 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
 template <bool kBf16>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
-    const int total = p.tile_prefix[p.num_seqs];
-    const int tile_id = total - 1 - (int)blockIdx.x;
-    if (tile_id < 0) return;
-    // sequence owning this tile: largest s with tile_prefix[s] <= tile_id
+    // Launch index -> work item.  The workgroups that run on one XCD at a time should share K/V in
+    // its L2, and the XCDs should get equal work although sequences differ in length.  With a
+    // multiple of eight kv heads, XCD x (launch index modulo 8) takes kv heads x, x + 8, ... of
+    // every sequence; its items are ordered (sequence, kv head, query tile descending, head slot),
+    // so the workgroups of one (sequence, kv head), which read the same K/V, run together.  Other
+    // head counts keep that order without the split.  The number of items is only known here (the
+    // grid is an upper bound): indices past the end leave at once.
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const bool pair_heads = (G & 1) == 0;
+    const int slots = pair_heads ? G / 2 : G;  // workgroups per (query tile, kv head)
+    const bool split = (p.num_heads_kv & 7) == 0;
+    const int heads_here = split ? p.num_heads_kv >> 3 : p.num_heads_kv;  // kv heads per sequence in this list
+    const int per_tile = heads_here * slots;                              // items of the list per query tile
+    const int items = p.tile_prefix[p.num_seqs] * per_tile;
+    const int item = split ? (int)blockIdx.x >> 3 : (int)blockIdx.x;
+    if (item >= items) return;
+    // sequence owning the item: largest s with tile_prefix[s] * per_tile <= item
     int lo = 0, hi_s = p.num_seqs;
     while (hi_s - lo > 1) {
         const int mid = (lo + hi_s) >> 1;
-        if (p.tile_prefix[mid] <= tile_id)
+        if (p.tile_prefix[mid] * per_tile <= item)
             lo = mid;
         else
             hi_s = mid;
     }
     const int s = lo;
-    const int qt = tile_id - p.tile_prefix[s];
-    const int G = p.num_heads_q / p.num_heads_kv;
-    const bool pair_heads = (G & 1) == 0;
-    const int h0 = pair_heads ? 2 * (int)blockIdx.y : (int)blockIdx.y;
+    const int tiles_s = p.tile_prefix[s + 1] - p.tile_prefix[s];
+    int r = item - p.tile_prefix[s] * per_tile;
+    const int head_here = r / (tiles_s * slots);
+    r -= head_here * tiles_s * slots;
+    const int qt = tiles_s - 1 - r / slots;  // the later (heavier) tiles of a sequence first
+    const int li = r % slots;
+    const int hkv = split ? ((int)blockIdx.x & 7) + 8 * head_here : head_here;
+    const int h0 = hkv * G + (pair_heads ? 2 * li : li);
     const Tile t0 = paged_group_tile(p, s, qt, h0, true);
     const Tile t1 = paged_group_tile(p, s, qt, pair_heads ? h0 + 1 : h0, pair_heads);
     run_both<kBf16>(t0, t1, lds, p.scale);
@@ -972,7 +989,7 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
 
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
     const int G = p.num_heads_q / p.num_heads_kv;
-    dim3 grid(p.max_q_tiles, (G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q);
+    dim3 grid((unsigned)((int64_t)p.max_q_tiles * ((G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q)));
     if (p.cache_dtype == HIPATTN_BF16)
         hipLaunchKernelGGL(flash::paged_prefill_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
     else
