@@ -140,7 +140,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c3": (563502.7 * 2.0 + 3031.8) * 1024,
     "c4": (1220744.2 * 2.0 + 12203.6) * 1024,
     "c2": (49294.0 * 2.0 + 65536.0) * 1024,
-    "c5": (786659.0 * 2.0 + 7600.9) * 1024,  # the decode kernel of the mixed step
+    "c5": (786678.2 * 2.0 + 7603.4) * 1024,  # the decode kernel of the mixed step
 }
 
 
