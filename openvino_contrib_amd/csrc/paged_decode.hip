@@ -21,13 +21,13 @@
 // global memory into MFMA operand registers (two register stages: the next block's loads are
 // in flight while the current block is consumed) and keeps an online softmax.
 //
-// MFMA use (v_mfma_f32_16x16x32_f16).  Scores are computed transposed, S^T = K Q^T, with the
+// MFMA use (v_mfma_f32_16x16x32_f16; _bf16 for bf16 caches).  Scores are computed transposed, S^T = K Q^T, with the
 // 16 tokens of a tile on the M side and the (padded) 16 query heads on the N side; the
 // accumulator layout then gives each lane four consecutive tokens of one head, which is
 // exactly the B-operand layout the second product O^T = V^T P^T needs, so P never moves
 // between lanes.  The contraction index of an MFMA can be permuted freely as long as both
 // operands use the same permutation; that freedom is used to make every global load a
-// contiguous 16-byte (fp16) or 8-byte (u8) piece of a cache row:
+// contiguous 16-byte (fp16, bf16) or 8-byte (u8) piece of a cache row:
 //   K operand: lane (tok = lane & 15, kg = lane >> 4) holds K[tok][kg*32 + i*8 .. +8], i = 0..3
 //   V operand: lane (c = lane & 15, kg) loads V[tok(kg,j)][c*8 .. +8] for its 8 tokens j and
 //              transposes the 8x8 patch in registers; MFMA e then yields O[:, c*8 + e].
@@ -88,17 +88,50 @@ __device__ __forceinline__ uint32_t pack_hi(uint32_t a, uint32_t b) { return (a 
 
 __device__ __forceinline__ half8_t as_half8(uint4_t v) { return __builtin_bit_cast(half8_t, v); }
 
-// 8 consecutive query elements as fp16 (bf16 queries are widened exactly)
-__device__ __forceinline__ half8_t load_q8(const void* q, int64_t elem, int q_dtype) {
-    if (q_dtype == HIPATTN_F16) {
-        return as_half8(*(const uint4_t*)((const uint16_t*)q + elem));
+// Element type of the MFMA operands: fp16 for fp16 and u8 caches, bf16 for bf16 caches.
+template <bool kBf16>
+struct Op16;
+template <>
+struct Op16<false> {
+    using vec8 = half8_t;
+    static __device__ __forceinline__ vec8 from_bits(uint4_t v) { return __builtin_bit_cast(vec8, v); }
+    static __device__ __forceinline__ float4_t mma(vec8 a, vec8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ void set(vec8& v, int i, float x) { v[i] = (half_t)x; }
+    static __device__ __forceinline__ float get(const vec8& v, int i) { return (float)v[i]; }
+};
+template <>
+struct Op16<true> {
+    using vec8 = bf16x8_t;
+    static __device__ __forceinline__ vec8 from_bits(uint4_t v) { return __builtin_bit_cast(vec8, v); }
+    static __device__ __forceinline__ float4_t mma(vec8 a, vec8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void set(vec8& v, int i, float x) { v[i] = (__bf16)x; }
+    static __device__ __forceinline__ float get(const vec8& v, int i) { return (float)v[i]; }
+};
+
+// 8 consecutive query elements in the operand type (same type: the bits; otherwise converted:
+// bf16 -> fp16 is exact inside the fp16 range, fp16 -> bf16 rounds to 8 bits)
+template <bool kBf16>
+__device__ __forceinline__ typename Op16<kBf16>::vec8 load_q8(const void* q, int64_t elem, int q_dtype) {
+    using O = Op16<kBf16>;
     const uint4_t raw = *(const uint4_t*)((const uint16_t*)q + elem);
-    half8_t r;
+    if (q_dtype == (kBf16 ? HIPATTN_BF16 : HIPATTN_F16)) return O::from_bits(raw);
+    typename O::vec8 r;
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-        r[2 * w] = (half_t)__uint_as_float(raw[w] << 16);
-        r[2 * w + 1] = (half_t)__uint_as_float(raw[w] & 0xffff0000u);
+        float lo, hi;
+        if constexpr (kBf16) {  // fp16 queries
+            lo = f16_bits_to_float((uint16_t)(raw[w] & 0xffffu));
+            hi = f16_bits_to_float((uint16_t)(raw[w] >> 16));
+        } else {  // bf16 queries
+            lo = __uint_as_float(raw[w] << 16);
+            hi = __uint_as_float(raw[w] & 0xffff0000u);
+        }
+        O::set(r, 2 * w, lo);
+        O::set(r, 2 * w + 1, hi);
     }
     return r;
 }
@@ -189,8 +222,8 @@ struct WaveState {
     float4_t acc[8];  // acc[e][r] = O[head][(kg*4 + r)*8 + e]
 };
 
-template <bool kU8>
-__device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, const half8_t (&qf)[4], float sumq,
+template <bool kU8, bool kBf16>
+__device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, const typename Op16<kBf16>::vec8 (&qf)[4], float sumq,
                                               float c, int tok_base, int j0, int ctx, int kg) {
     // ---- S^T = K Q^T : two tiles of 16 tokens x 16 heads
     float4_t s[2];
@@ -199,18 +232,18 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
         s[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            half8_t a;
+            typename Op16<kBf16>::vec8 a;
             if constexpr (!kU8) {
-                a = as_half8(b.k[t][i]);
+                a = Op16<kBf16>::from_bits(b.k[t][i]);
             } else {
                 uint4_t w;
                 w[0] = bytes_to_biased_half2(b.k[t][i][0], 0x04010400u);
                 w[1] = bytes_to_biased_half2(b.k[t][i][0], 0x04030402u);
                 w[2] = bytes_to_biased_half2(b.k[t][i][1], 0x04010400u);
                 w[3] = bytes_to_biased_half2(b.k[t][i][1], 0x04030402u);
-                a = as_half8(w);
+                a = Op16<kBf16>::from_bits(w);
             }
-            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[i], s[t], 0, 0, 0);
+            s[t] = Op16<kBf16>::mma(a, qf[i], s[t]);
         }
     }
     // ---- mask, scale, online softmax.  Lane holds tokens tok_base + t*16 + kg*4 + r.
@@ -274,7 +307,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
             }
         }
     }
-    half8_t pf;
+    typename Op16<kBf16>::vec8 pf;
     float lsum = 0.0f, csum = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
@@ -293,11 +326,10 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
                 default: vs = row_broadcast<15>(sz_scale); vz = row_broadcast<15>(sz_zero); break;
             }
             pj *= vs;
-            const half_t ph = (half_t)pj;
-            csum = fmaf((float)ph, vz, csum);
-            pf[j] = ph;
+            Op16<kBf16>::set(pf, j, pj);
+            csum = fmaf(Op16<kBf16>::get(pf, j), vz, csum);
         } else {
-            pf[j] = (half_t)pj;
+            Op16<kBf16>::set(pf, j, pj);
         }
     }
     st.l = st.l * alpha + lsum;
@@ -322,7 +354,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
             for (int jp = 0; jp < 4; jp++)
                 w[jp] = bytes_to_biased_half2(b.v[2 * jp][e >> 2], b.v[2 * jp + 1][e >> 2], sel);
         }
-        st.acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(w), pf, st.acc[e], 0, 0, 0);
+        st.acc[e] = Op16<kBf16>::mma(Op16<kBf16>::from_bits(w), pf, st.acc[e]);
     }
 }
 
@@ -496,8 +528,9 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
     }
 }
 
-template <bool kU8>
+template <bool kU8, bool kBf16>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p) {
+    static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
     const int w = blockIdx.x;
     const int lane = threadIdx.x, n16 = lane & 15, kg = lane >> 4;
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
@@ -552,21 +585,21 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         const int64_t head_off = (int64_t)h * kBS * kRowBytes;
 
         // Q^T operand: lane (head n16, kg) holds Q[head][kg*32 + i*8 .. +8]; padding heads are zero
-        half8_t qf[4];
+        typename Op16<kBf16>::vec8 qf[4];
         float sumq = 0.0f;
         {
             const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kD;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 if (n16 < G) {
-                    qf[i] = load_q8(p.q, qrow + kg * 32 + i * 8, p.q_dtype);
+                    qf[i] = load_q8<kBf16>(p.q, qrow + kg * 32 + i * 8, p.q_dtype);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) qf[i][e] = (half_t)0.0f;
+                    for (int e = 0; e < 8; e++) Op16<kBf16>::set(qf[i], e, 0.0f);
                 }
                 if constexpr (kU8) {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) sumq += (float)qf[i][e];
+                    for (int e = 0; e < 8; e++) sumq += Op16<kBf16>::get(qf[i], e);
                 }
             }
             if constexpr (kU8) {
@@ -600,12 +633,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 int i = 0;
                 while (i < gn) {
                     ok_b = (i + 1 < gn) ? issue(rb, i + 1) : false;
-                    if (ok_a) process_block<kU8>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
+                    if (ok_a) process_block<kU8, kBf16>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
                     if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
                     blocks_done = 1;
                     if (i + 1 >= gn) break;
                     ok_a = (i + 2 < gn) ? issue(ra, i + 2) : false;
-                    if (ok_b) process_block<kU8>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
+                    if (ok_b) process_block<kU8, kBf16>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
                     i += 2;
                 }
             } else {
@@ -625,7 +658,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                         constexpr int kLast = kStages - 1;
                         ok[(u + kLast) % kStages] =
                             (idx + kLast < gn) ? issue(regs[(u + kLast) % kStages], idx + kLast) : false;
-                        if (ok[u]) process_block<kU8>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kBS, rg.j0, rg.ctx, kg);
+                        if (ok[u]) process_block<kU8, kBf16>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kBS, rg.j0, rg.ctx, kg);
                         if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
                         blocks_done = 1;
                     }
@@ -709,7 +742,7 @@ bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     return p.head_dim == kD && p.block_size == kBS && G <= 16 &&
            (p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16) &&
-           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_U8);
+           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
 }
 
 // Wavefronts the decode kernel keeps resident: it needs up to 256 registers per lane, i.e. two
@@ -805,9 +838,11 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     if (e != hipSuccess) return e;
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     if (p.cache_dtype == HIPATTN_U8)
-        hipLaunchKernelGGL(paged_decode_kernel<true>, dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<true, false>), dim3(p.num_waves), dim3(64), 0, stream, p);
+    else if (p.cache_dtype == HIPATTN_BF16)
+        hipLaunchKernelGGL((paged_decode_kernel<false, true>), dim3(p.num_waves), dim3(64), 0, stream, p);
     else
-        hipLaunchKernelGGL(paged_decode_kernel<false>, dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<false, false>), dim3(p.num_waves), dim3(64), 0, stream, p);
     e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     if (e != hipSuccess) return e;

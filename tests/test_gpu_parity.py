@@ -149,7 +149,8 @@ DECODE_CTX = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 500, 511, 512, 513, 1
 
 
 @pytest.mark.parametrize("cache_dtype,q_dtype,Hq", [(W.F16, W.F16, 32), (W.F16, W.BF16, 8), (W.U8, W.F16, 64),
-                                                    (W.U8, W.BF16, 16), (W.F16, W.F16, 128)])
+                                                    (W.U8, W.BF16, 16), (W.F16, W.F16, 128), (W.BF16, W.BF16, 32),
+                                                    (W.BF16, W.F16, 16)])
 @pytest.mark.parametrize("waves", [0, 5, 100, 3000])
 def test_paged_decode(hip, oracle, cache_dtype, q_dtype, Hq, waves):
     announce("paged decode", cache_dtype, q_dtype, Hq, waves)
@@ -162,7 +163,7 @@ def test_paged_decode(hip, oracle, cache_dtype, q_dtype, Hq, waves):
     kc, vc = dev.caches()
     np.testing.assert_array_equal(kc, okc)
     np.testing.assert_array_equal(vc, ovc)
-    tol = 1e-2 if (cache_dtype == W.U8 or q_dtype == W.BF16) else 2e-3
+    tol = 1e-2 if (cache_dtype in (W.U8, W.BF16) or q_dtype == W.BF16) else 2e-3
     assert np.isfinite(out).all()
     assert H.max_abs(out, ref) <= tol
     # the shape-generic kernels agree as well (second, independent device implementation)
@@ -247,7 +248,8 @@ def test_paged_block_permutation_is_bit_identical(hip):
 
 # ----------------------------------------------------------------- mixed prefill + decode
 @pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.F16, W.F16, 0), (W.BF16, W.F16, 0), (W.BF16, W.F16, 300),
-                                                        (W.F16, W.F16, 64), (W.F16, W.U8, 0), (W.F16, W.U8, 100)])
+                                                        (W.F16, W.F16, 64), (W.F16, W.U8, 0), (W.F16, W.U8, 100),
+                                                        (W.BF16, W.BF16, 0), (W.BF16, W.BF16, 200)])
 @pytest.mark.parametrize("heads", [(16, 4), (12, 4), (4, 4)])  # even GQA ratio (head pairs), odd ratios (one group idle)
 def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window, heads):
     announce("paged mixed", q_dtype, cache_dtype, window, heads)
@@ -260,7 +262,7 @@ def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window, heads):
     kc, vc = dev.caches()
     np.testing.assert_array_equal(kc, okc)
     np.testing.assert_array_equal(vc, ovc)
-    tol = 1e-2 if (cache_dtype == W.U8 or q_dtype == W.BF16) else 2e-3
+    tol = 1e-2 if (cache_dtype in (W.U8, W.BF16) or q_dtype == W.BF16) else 2e-3
     assert np.isfinite(out).all()
     assert H.max_abs(out, ref) <= tol
     dev.free()
