@@ -885,8 +885,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #endif
 }
 
-// One workgroup per (128-row query tile of a multi-token sequence, pair of query heads).  With an
-// odd number of query heads per kv head the second group has no work and only helps loading.
+// One workgroup per (128-row query tile of a multi-token sequence, pair of query heads) or, with an
+// odd number of query heads per kv head, per (pair of query tiles, query head).
 __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, int qt, int h, bool has_work) {
     const int G = p.num_heads_q / p.num_heads_kv;
     const int t0 = p.subsequence_begins[s];
@@ -956,8 +956,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int li = r % slots;
     const int hkv = split ? ((int)blockIdx.x & 7) + 8 * head_here : head_here;
     const int h0 = hkv * G + (pair_heads ? 2 * li : li);
+    // The two groups take two query heads of the kv head at one query tile or, with an odd number
+    // of query heads per kv head, two consecutive query tiles of one head: the item of the even
+    // tile does both, the item of the odd tile has nothing left to do.
+    if (!pair_heads && (qt & 1)) return;
     const Tile t0 = paged_group_tile(p, s, qt, h0, true);
-    const Tile t1 = paged_group_tile(p, s, qt, pair_heads ? h0 + 1 : h0, pair_heads);
+    const Tile t1 = pair_heads ? paged_group_tile(p, s, qt, h0 + 1, true) : paged_group_tile(p, s, qt + 1, h0, qt + 1 < tiles_s);
     run_both<kBf16>(t0, t1, lds, p.scale);
 }
 
