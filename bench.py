@@ -208,7 +208,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy", "mfma"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "copy", "mfma"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
                          "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
@@ -269,7 +269,9 @@ def main():
              "c3": "config3: fp16 paged decode, 64 seq x 1 token, ctx U[512,8192], blk 32, Hq32 Hkv8 D128",
              "c4": "config4: u8-KV paged decode, 128 seq, ctx U[1024,16384], Hq64 Hkv8 D128",
              "c5": "config5: 8x512 prefill chunks + 120 decode, window 4096, bf16 q, fp16 cache, Hq64 Hkv8 D128"}
-    makers = {"c2": W.config2, "c3": W.config3, "c4": W.config4, "c5": W.config5}
+    names["c5u8"] = "config5's batch on a u8 cache (not one of the reference configurations: the u8 load path of the prefill kernel)"
+    makers = {"c2": W.config2, "c3": W.config3, "c4": W.config4, "c5": W.config5,
+              "c5u8": lambda: W.config5(cache_dtype=W.U8)}
     order = [args.workload] + ([w for w in ("c3", "c2", "c4", "c5") if w != args.workload] if not args.no_extra else [])
     results, cpu = {}, {}
     for w in order:
@@ -282,7 +284,7 @@ def main():
         else:
             r = bench_paged(hip, case, args.steps, args.warmup, names[w])
             r["roofline"] = roofline_hbm(r, MEASURED_TRAFFIC_BYTES.get(w))
-            if w == "c5":
+            if w in ("c5", "c5u8"):
                 t_ideal = max(r["kv_bytes"] / (HBM_PEAK_GBS * 1e9), r["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                 r["ideal_ms"] = t_ideal * 1e3
                 r["frac_of_ideal"] = t_ideal * 1e3 / r["ms_per_step"]
@@ -302,7 +304,7 @@ def main():
         "unit": "TFLOP/s" if is_sdpa else "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if is_sdpa else ("u8" if args.workload == "c4" else "f16"),
+        "dtype": "bf16" if is_sdpa else ("u8" if args.workload in ("c4", "c5u8") else "f16"),
         "data": "synthetic",
         "config": {"workload": head["workload"], "kernel_path": head["kernel_path"],
                    "device": dev_name, "arch": info.arch.decode(), "compute_units": info.compute_units,

@@ -158,6 +158,32 @@ struct Tile {
     int block_shift;        // log2(block_size)
 };
 
+// u8 caches: rows of 8 bytes (float scale, float zero-point) + 128 payload bytes.  The u8 variant
+// of the kernel loads them into registers, dequantises to fp16 and writes the result into the
+// same LDS stages (same layout) the 16-bit caches are loaded into directly; everything behind
+// that is the fp16 kernel.
+constexpr int kU8RowBytes = kD + 8;
+struct U8Rows {
+    uint2_t k_lo, k_hi, v_lo, v_hi;  // this lane's 16 payload bytes of a K row and of a V row
+    float2 k_sz, v_sz;               // the rows' (scale, zero-point)
+    int jk, jv;                      // tiles they belong to (-1: none)
+};
+// two bytes of a word (selected by `sel`) as fp16 numbers 1024 + byte
+__device__ __forceinline__ half2_t biased_half2(uint32_t w, uint32_t sel) {
+    return __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, w, sel));
+}
+// 8 payload bytes -> 8 dequantised fp16 values: (byte - zp) * scale, as (byte) * scale + off in
+// packed fp16 (1024 + byte is exact in fp16, and so is the subtraction of 1024)
+__device__ __forceinline__ uint4_t dequant8(uint2_t w, half2_t scale, half2_t off) {
+    const half2_t bias = {(half_t)1024.0f, (half_t)1024.0f};
+    uint4_t r;
+    r[0] = __builtin_bit_cast(uint32_t, (biased_half2(w[0], 0x04010400u) - bias) * scale + off);
+    r[1] = __builtin_bit_cast(uint32_t, (biased_half2(w[0], 0x04030402u) - bias) * scale + off);
+    r[2] = __builtin_bit_cast(uint32_t, (biased_half2(w[1], 0x04010400u) - bias) * scale + off);
+    r[3] = __builtin_bit_cast(uint32_t, (biased_half2(w[1], 0x04030402u) - bias) * scale + off);
+    return r;
+}
+
 // Keys [lo, hi) a tile has to visit, lo rounded down to a tile boundary.
 __device__ __forceinline__ void key_range(const Tile& t, int& lo, int& hi) {
     if (t.rows <= 0) {
@@ -551,8 +577,9 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0,
 // ring stages of K(x-1) and V(x-2); every wavefront issues its rows of B(x) in a vector phase
 // (group 0 in phase 2x+1, group 1 in phase 2x), and at each barrier waits for all of its loads
 // except the latest batch, which puts B(x) in LDS two phases before its first use.
-template <bool kBf16>
+template <bool kBf16, bool kU8 = false>
 __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
+    static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16");
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     lds_byte* const lds = (lds_byte*)lds_generic;
@@ -665,18 +692,94 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     };
     auto k_stage = [&](int j) { return k_ring + (j % kStages) * kKBytes; };
     auto v_stage = [&](int j) { return v_ring + (j % kStages) * kKBytes; };
+    // ---- u8 caches: lane l of wavefront w handles 16 payload bytes (piece l % 8) of row 8w + l / 8
+    const int u8_row = 8 * wave + (lane >> 3), u8_piece = lane & 7;
+    // address of this lane's row of tile j (entry: the block table entry of the wavefront's rows)
+    auto u8_row_address = [&](const uint8_t* base, int j, int entry) __attribute__((always_inline)) -> const uint8_t* {
+        const int key0 = kv_lo + j * kTileK + 8 * wave;
+        int key = kv_lo + j * kTileK + u8_row;
+        int pb;
+        if (key0 + 8 <= t.kv_len) {
+            pb = entry;
+        } else {  // rows at the end of the sequence repeat its last row
+            key = min(key, t.kv_len - 1);
+            pb = t.table[key >> t.block_shift];
+        }
+        pb = min(max(pb, 0), t.num_blocks - 1);
+        return base + (int64_t)pb * t.block_stride + (int64_t)(key & (t.block_size - 1)) * kU8RowBytes;
+    };
+    auto u8_fetch = [&](int jk, int ek, int jv, int ev) __attribute__((always_inline)) -> U8Rows {
+        U8Rows x;
+        x.k_lo = x.k_hi = x.v_lo = x.v_hi = uint2_t{0u, 0u};
+        x.k_sz = x.v_sz = make_float2(0.0f, 0.0f);
+        x.jk = jk < n ? jk : -1;
+        x.jv = jv < n ? jv : -1;
+        if (x.jk >= 0) {
+            const uint8_t* row = u8_row_address(t.k, jk, ek);
+            x.k_sz = *(const float2*)row;
+            x.k_lo = *(const uint2_t*)(row + 8 + 16 * u8_piece);
+            x.k_hi = *(const uint2_t*)(row + 16 + 16 * u8_piece);
+        }
+        if (x.jv >= 0) {
+            const uint8_t* row = u8_row_address(t.v, jv, ev);
+            x.v_sz = *(const float2*)row;
+            x.v_lo = *(const uint2_t*)(row + 8 + 16 * u8_piece);
+            x.v_hi = *(const uint2_t*)(row + 16 + 16 * u8_piece);
+        }
+        return x;
+    };
+    // dequantises the rows and writes them where the 16-bit path loads them (chunk c of row r at
+    // position c ^ (r % 16) for K, c ^ 4 (r % 4) for V); this lane has chunks 2 piece and 2 piece + 1
+    auto u8_store = [&](const U8Rows& x) __attribute__((always_inline)) {
+        typedef __attribute__((address_space(3))) uint4_t lds_uint4;
+        if (x.jk >= 0) {
+            const half2_t sc = {(half_t)x.k_sz.x, (half_t)x.k_sz.x};
+            const float o32 = -x.k_sz.y * x.k_sz.x;
+            const half2_t of = {(half_t)o32, (half_t)o32};
+            lds_byte* const rowp = k_stage(x.jk) + u8_row * kRowBytes;
+            *(lds_uint4*)(rowp + (((2 * u8_piece) ^ (u8_row & 15)) << 4)) = dequant8(x.k_lo, sc, of);
+            *(lds_uint4*)(rowp + (((2 * u8_piece + 1) ^ (u8_row & 15)) << 4)) = dequant8(x.k_hi, sc, of);
+        }
+        if (x.jv >= 0) {
+            const half2_t sc = {(half_t)x.v_sz.x, (half_t)x.v_sz.x};
+            const float o32 = -x.v_sz.y * x.v_sz.x;
+            const half2_t of = {(half_t)o32, (half_t)o32};
+            lds_byte* const rowp = v_stage(x.jv) + u8_row * kRowBytes;
+            *(lds_uint4*)(rowp + (((2 * u8_piece) ^ (4 * (u8_row & 3))) << 4)) = dequant8(x.v_lo, sc, of);
+            *(lds_uint4*)(rowp + (((2 * u8_piece + 1) ^ (4 * (u8_row & 3))) << 4)) = dequant8(x.v_hi, sc, of);
+        }
+    };
+    // the workgroup barrier of the u8 variant: LDS writes done, register loads may stay in flight
+    auto phase_barrier = [&](int keep) __attribute__((always_inline)) {
+        if constexpr (kU8)
+            barrier_keeping<63>();
+        else
+            barrier_keeping_loads(keep);
+    };
 
     // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
     const int e0 = table_entry(0), e1 = table_entry(1), e2 = table_entry(2), e3 = table_entry(3);
-    const int first = load_rows(true, 0, k_stage(0), e0) + load_rows(false, 0, v_stage(0), e0) +
-                      load_rows(true, 1, k_stage(1), e1);
-    int recent = 0;
-    if (group == 1) recent = load_rows(true, 2, k_stage(2), e2) + load_rows(false, 1, v_stage(1), e1);
+    int first = 0, recent = 0;
+    U8Rows pending;  // u8: rows fetched in one iteration, dequantised and written in the next
+    pending.jk = pending.jv = -1;
+    if constexpr (kU8) {
+        const U8Rows a = u8_fetch(0, e0, 0, e0), b = u8_fetch(1, e1, n, 0);
+        if (group == 1) pending = u8_fetch(2, e2, 1, e1);  // its rows of B(0), written in the first iteration
+        u8_store(a);
+        u8_store(b);
+    } else {
+        first = load_rows(true, 0, k_stage(0), e0) + load_rows(false, 0, v_stage(0), e0) +
+                load_rows(true, 1, k_stage(1), e1);
+        if (group == 1) recent = load_rows(true, 2, k_stage(2), e2) + load_rows(false, 1, v_stage(1), e1);
+    }
     // entries of the tiles the first iteration loads: K(group + 2) and V(group + 1)
     int entry_v = group ? e2 : e1, entry_k = group ? e3 : e2;
     // The query rows were issued first and nobody else reads them: they are converted while the
     // K and V tiles are still on their way.
-    wait_keeping_loads(first + recent);
+    if constexpr (kU8)
+        wait_keeping<0>();
+    else
+        wait_keeping_loads(first + recent);
     // Q^T operand: k-step i covers head-dim i*16 + hi*8 .. +8
     vec8 qf[8];
     {
@@ -697,13 +800,13 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) asm volatile("" : "+v"(qf[i]));  // (converted before the wait below, not after)
-    barrier_keeping_loads(recent);
-    if (group == 1) barrier_keeping_loads(recent);  // group 1 sits out phase 0
+    phase_barrier(recent);
+    if (group == 1) phase_barrier(recent);  // group 1 sits out phase 0
 
     float16_t s[2];
     vec8 pf[4];
     tile_scores<kBf16>(k_stage(0), f, qf, st.neg_ref, s);
-    barrier_keeping_loads(recent);
+    phase_barrier(recent);
 #ifdef HIPATTN_FLASH_TRACE
     PhaseClock clk;
     clk.last = (long long)__builtin_readcyclecounter();
@@ -720,7 +823,14 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         clk.tile = j;
 #endif
         FLASH_STAMP(clk, 0);
-        recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
+        if constexpr (kU8) {
+            // rows fetched one iteration ago go into their stages, two phases before their first
+            // use; the rows of this iteration's batch are fetched into registers
+            u8_store(pending);
+            pending = u8_fetch(j + group + 2, entry_k, j + group + 1, entry_v);
+        } else {
+            recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
+        }
         entry_v = entry_k;  // the next iteration loads V of the tile whose K was loaded now
         entry_k = table_entry(j + group + 3);
         FLASH_STAMP(clk, 1);
@@ -734,7 +844,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         // the first instruction after it): otherwise the other group's instruction stream, which
         // never stalls for long, keeps this wavefront's MFMAs from issuing
         __builtin_amdgcn_s_setprio(3);
-        barrier_keeping_loads(recent);
+        phase_barrier(recent);
         FLASH_STAMP(clk, 3);
         // ---- matrix phase
         // fragment addresses of this tile: per-lane offset + stage address, so that every read is
@@ -750,7 +860,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             tile_accumulate<kBf16>(zero, fs, pf, o);
         __builtin_amdgcn_s_setprio(0);
         FLASH_STAMP(clk, 5);
-        barrier_keeping_loads(recent);
+        phase_barrier(recent);
         FLASH_STAMP(clk, 6);
     };
     for (int j = 0; j < n - 1; j++)
@@ -781,7 +891,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         store_rows_via_lds<true>(t, o, inv, out_stage, row0, lane);
     }
     // as many barriers as group 1, whose last phase runs while group 0 stores its rows
-    if (group == 0) barrier_keeping_loads(0);
+    if (group == 0) phase_barrier(0);
 }
 
 // Launch index -> work item: workgroups go to the eight XCDs round-robin by launch index and
@@ -839,7 +949,7 @@ __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) 
     return t;
 }
 
-template <bool kBf16>
+template <bool kBf16, bool kU8 = false>
 __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t* lds, float scale) {
     int lo0, hi0, lo1, hi1;
     key_range(t0, lo0, hi0);
@@ -856,7 +966,7 @@ __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t
         kv_hi = max(hi0, hi1);
     }
     const int group = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
-    run_pair<kBf16>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
+    run_pair<kBf16, kU8>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
 }
 
 template <bool kBf16>
@@ -907,19 +1017,20 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
     t.window = p.sliding_window;
     t.q_dtype = p.q_dtype;
     t.out_dtype = p.out_dtype;
-    const int64_t head_off = (int64_t)(h / G) * p.block_size * (kD * 2);
+    const int row_bytes = p.cache_dtype == HIPATTN_U8 ? kU8RowBytes : kD * 2;
+    const int64_t head_off = (int64_t)(h / G) * p.block_size * row_bytes;
     t.k = p.key_cache + head_off;
     t.v = p.value_cache + head_off;
     t.table = p.block_indices + tb0;
     t.table_len = table_len;
     t.num_blocks = p.num_blocks;
-    t.block_stride = (int64_t)p.num_heads_kv * p.block_size * (kD * 2);
+    t.block_stride = (int64_t)p.num_heads_kv * p.block_size * row_bytes;
     t.block_size = p.block_size;
     t.block_shift = __builtin_ctz(p.block_size);
     return t;
 }
 
-template <bool kBf16>
+template <bool kBf16, bool kU8>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
     // Launch index -> work item.  The workgroups that run on one XCD at a time should share K/V in
@@ -962,7 +1073,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (!pair_heads && (qt & 1)) return;
     const Tile t0 = paged_group_tile(p, s, qt, h0, true);
     const Tile t1 = pair_heads ? paged_group_tile(p, s, qt, h0 + 1, true) : paged_group_tile(p, s, qt + 1, h0, qt + 1 < tiles_s);
-    run_both<kBf16>(t0, t1, lds, p.scale);
+    run_both<kBf16, kU8>(t0, t1, lds, p.scale);
 }
 
 }  // namespace flash
@@ -995,9 +1106,11 @@ hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
     const int G = p.num_heads_q / p.num_heads_kv;
     dim3 grid((unsigned)((int64_t)p.max_q_tiles * ((G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q)));
     if (p.cache_dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL(flash::paged_prefill_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
+        hipLaunchKernelGGL((flash::paged_prefill_kernel<true, false>), grid, dim3(flash::kThreads), 0, stream, p);
+    else if (p.cache_dtype == HIPATTN_U8)
+        hipLaunchKernelGGL((flash::paged_prefill_kernel<false, true>), grid, dim3(flash::kThreads), 0, stream, p);
     else
-        hipLaunchKernelGGL(flash::paged_prefill_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
+        hipLaunchKernelGGL((flash::paged_prefill_kernel<false, false>), grid, dim3(flash::kThreads), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -850,13 +850,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.max_q_tiles > 0) {
-        if (p.cache_dtype == HIPATTN_U8) {
-            PagedParams g = p;
-            g.generic_skip_single = 1;
-            e = launch_paged_generic(g, stream);
-        } else {
-            e = launch_paged_prefill(p, stream);
-        }
+        e = launch_paged_prefill(p, stream);
     }
     return e;
 }

@@ -79,3 +79,9 @@ def test_config4_u8_paged_decode(hip, oracle):
 def test_config5_mixed_batch(hip, oracle):
     announce("C5 8x512 prefill + 120 decode, window 4096, bf16 q, fp16 cache")
     _run_paged_config(hip, oracle, W.config5(), 1e-2, "C5")
+
+
+def test_config5_mixed_batch_u8_cache(hip, oracle):
+    """Configuration 5's batch on a u8 cache: the chunks go through the flash kernel's u8 loads."""
+    announce("C5 with a u8 cache")
+    _run_paged_config(hip, oracle, W.config5(cache_dtype=W.U8), 1e-2, "C5-u8")
