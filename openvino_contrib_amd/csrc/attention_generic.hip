@@ -134,7 +134,6 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void paged_generic_kernel(Page
     const int h = (int)(r % p.num_heads_q);
     if (t < p.subsequence_begins[0] || t >= p.subsequence_begins[p.num_seqs]) return;
     const int s = find_sequence_of_token(p.subsequence_begins, p.num_seqs, t);
-    if (p.generic_skip_single && p.subsequence_begins[s + 1] - p.subsequence_begins[s] == 1) return;
     const int pos = p.past_lens[s] + (t - p.subsequence_begins[s]);
     const int D = p.head_dim;
     const int G = p.num_heads_q / p.num_heads_kv;

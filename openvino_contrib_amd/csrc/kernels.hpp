@@ -90,8 +90,6 @@ struct PagedParams {
     // chunked prefill: query-tile schedule built on the device
     int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
     int max_q_tiles;      // grid upper bound
-    // shape-generic kernel only: skip sequences with exactly one token (the decode kernel has them)
-    int generic_skip_single;
     // diagnostic (HIPATTN_PA_TRACE_WAVES): per decode wavefront {entry, first block consumed, exit, line units}
     int64_t* wave_trace;
 };
