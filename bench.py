@@ -288,6 +288,9 @@ def main():
                 t_ideal = max(r["kv_bytes"] / (HBM_PEAK_GBS * 1e9), r["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                 r["ideal_ms"] = t_ideal * 1e3
                 r["frac_of_ideal"] = t_ideal * 1e3 / r["ms_per_step"]
+                r["roofline"]["note"] = ("mixed batch: the decode kernel runs beside the chunks' flash kernel on a share "
+                                         "of the compute units, so its duration is not a whole-chip figure; "
+                                         "frac_of_ideal is the one for this step")
         log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f"
             % (w, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"]))
         if not args.no_cpu and w == args.workload:

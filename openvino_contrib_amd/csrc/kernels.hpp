@@ -83,6 +83,13 @@ struct PagedParams {
     int dyn_pieces;       // pieces of the last quarter of the work line, handed out on demand
     int dyn_groups;       // wavefront groups, each with its own ticket counter and every dyn_groups-th piece
     int32_t* dyn_counter; // [64] ticket counters (zeroed by the plan)
+    // mixed batches: the decode kernel keeps only some compute units (eight wavefronts each) and the
+    // chunks' flash kernel runs beside it on the others; the plan decides how many from the work
+    // of the two parts and leaves the wavefront count in plan_waves[0] (num_waves is then the most
+    // it may choose).  overlap_share scales the decode part's share (1 = as modelled).
+    int overlap;          // 0: decode, merge and prefill kernels run one after the other
+    float overlap_share;
+    int32_t* plan_waves;  // [1]
     int32_t* blk_prefix;  // [num_seqs + 1] exclusive prefix of work-line units of decode sequences
     void* seq_info;       // [num_seqs] 32-byte records: what each decode sequence attends (written by the plan)
     float* part_out;      // [num_waves + dyn_pieces + num_seqs*num_heads_kv, G, head_dim] unnormalised outputs

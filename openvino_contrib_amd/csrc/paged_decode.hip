@@ -35,11 +35,24 @@
 // scale is folded into the score / probability and the zero-point into a rank-one
 // correction (q.(k - zp) s = s (q.k) - s zp sum(q)).
 //
+// Mixed batches (decode sequences and multi-token chunks in one call).  The chunks go to the flash
+// kernel over the block table, which is bound by the matrix cores; the decode sequences are bound
+// by HBM.  Each of the two kernels needs whole compute units (registers, LDS), so they cannot
+// share one, but they can share the chip: the decode kernel is then launched with eight
+// wavefronts to a workgroup -- a workgroup owns a compute unit -- directly behind the prologue,
+// and the flash kernel on a side stream that waits for the prologue too and takes the other
+// compute units (and every one the decode workgroups give back).  How many compute units the
+// decode part keeps is decided by the plan on the device, in proportion to the work of the two
+// parts (cache bytes to stream against key tiles to multiply), so that both end together;
+// workgroups beyond that number leave at once.  The caller's stream waits for the side stream
+// before the call returns, so to the caller the call is still one piece of work in stream order.
+//
 // No counterpart in the reference: its decode path copies the whole contiguous KV state
 // three times per token (src/cuda_variable_state.hpp:135-160, src/ops/read_value.cpp:65-71,
 // src/ops/assign.cpp:52-54) and materialises the scores in HBM (src/ops/matmul.cpp:204-226,
 // src/ops/softmax.cpp:184-192).
 #include <algorithm>
+#include <mutex>
 #include <cstdlib>
 #include <type_traits>
 
@@ -372,27 +385,54 @@ __device__ __forceinline__ int line_units(int nb, int switch_cost) { return nb >
 __device__ __forceinline__ void plan_block(const PagedParams& p) {
     __shared__ int part_blk[256];
     __shared__ int part_tile[256];
+    __shared__ float part_keys[256];
     const int tid = threadIdx.x;
     if (tid < 64) p.dyn_counter[tid] = 0;  // tickets for the dynamic pieces of this call, one counter per group
     const int per = (p.num_seqs + 255) / 256;
     const int s0 = min(tid * per, p.num_seqs), s1 = min(s0 + per, p.num_seqs);
     int blk = 0, tile = 0;
+    float key_tiles = 0.0f;  // 64-key tiles the flash kernel works through, summed over 128-row query tiles
     for (int s = s0; s < s1; s++) {
         const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
         blk += line_units(decode_range(p, s).nb, p.switch_cost);
         tile += qlen > 1 ? (qlen + 127) / 128 : 0;
+        if (p.overlap && qlen > 1) {
+            const int past = p.past_lens[s];
+            for (int r0 = 0; r0 < qlen; r0 += 128) {
+                int keys = past + min(qlen, r0 + 128);
+                if (p.sliding_window > 0) keys = min(keys, p.sliding_window + 128);
+                key_tiles += (float)((keys + 63) >> 6);
+            }
+        }
     }
     part_blk[tid] = blk;
     part_tile[tid] = tile;
+    part_keys[tid] = key_tiles;
     __syncthreads();
     if (tid == 0) {
         int rb = 0, rt = 0;
+        float rk = 0.0f;
         for (int i = 0; i < 256; i++) {
             const int vb = part_blk[i], vt = part_tile[i];
             part_blk[i] = rb;
             part_tile[i] = rt;
             rb += vb;
             rt += vt;
+            rk += part_keys[i];
+        }
+        if (p.overlap) {
+            // Compute-unit time of the two parts, in microseconds, as measured with both running:
+            // a compute unit of the decode kernel streams about 33 GB/s of fp16 cache (u8: 24 GB/s),
+            // one of the flash kernel does a 128-row x 64-key tile of one head in about 1.2 us
+            // (u8 caches, dequantised on the way: 1.7 us).  Each part gets compute units in
+            // proportion to its work, so that both end together.
+            const bool u8 = p.cache_dtype == HIPATTN_U8;
+            const float decode_us = (float)rb * p.num_heads_kv * (u8 ? 8704.0f / 24000.0f : 16384.0f / 33000.0f) * p.overlap_share;
+            const float prefill_us = rk * p.num_heads_q * (u8 ? 1.7f : 1.2f);
+            const int cus = p.num_waves >> 3;
+            int mine = (int)ceilf(cus * decode_us / fmaxf(decode_us + prefill_us, 1.0f));
+            mine = max(1, min(mine, cus));
+            p.plan_waves[0] = mine * 8;
         }
     }
     __syncthreads();
@@ -528,16 +568,22 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
     }
 }
 
-template <bool kU8, bool kBf16>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p) {
+// kWaves wavefronts to a workgroup.  1 is the ordinary launch.  With 8 a workgroup owns a compute
+// unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
+// leave the others free for a kernel that runs beside this one.
+template <bool kU8, bool kBf16, int kWaves>
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
-    const int w = blockIdx.x;
-    const int lane = threadIdx.x, n16 = lane & 15, kg = lane >> 4;
+    const int w = kWaves == 1 ? blockIdx.x : blockIdx.x * kWaves + (threadIdx.x >> 6);
+    const int lane = kWaves == 1 ? threadIdx.x : (threadIdx.x & 63), n16 = lane & 15, kg = lane >> 4;
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
     const float c = p.scale * kLog2e;
     const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
     if (total <= 0) return;
-    const Line line(total, p.num_waves, p.dyn_pieces);
+    // eight to a workgroup: the plan has chosen how many of the launched wavefronts work
+    const int num_waves = kWaves == 1 ? p.num_waves : p.plan_waves[0];
+    if (w >= num_waves) return;
+    const Line line(total, num_waves, p.dyn_pieces);
     // diagnostic: entry time, time the first block was consumed, exit time, units done (100 MHz clock)
     int64_t t_entry = 0, t_first = 0, units_done = 0;
     int blocks_done = 0;
@@ -706,7 +752,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     if (p.dyn_pieces <= 0) break;
     const int next = group + __shfl(ticket_lane0, 0, 64) * p.dyn_groups;
     if (next >= p.dyn_pieces) break;  // this group's share of the line is used up (every wavefront gets here)
-    piece = p.num_waves + next;
+    piece = num_waves + next;
     }
     if (p.wave_trace && lane == 0) {
         p.wave_trace[w * 4 + 0] = t_entry;
@@ -727,7 +773,7 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(PagedParams p) {
     if (rg.nb <= 0) return;
     const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
     if (total <= 0) return;
-    const Line line(total, p.num_waves, p.dyn_pieces);
+    const Line line(total, p.overlap ? p.plan_waves[0] : p.num_waves, p.dyn_pieces);
     const int seglen = rg.nb + p.switch_cost;
     const int64_t L0 = (int64_t)p.blk_prefix[s] * Hkv + (int64_t)h * seglen + p.switch_cost, L1 = L0 + rg.nb;
     const int id_first = line.piece_at(L0), id_last = line.piece_at(L1 - 1);
@@ -762,9 +808,25 @@ static int resident_decode_waves() {
 
 // fp16 caches stream best with one wavefront per SIMD; the u8 path has more arithmetic per
 // byte and wants both resident wavefronts to cover it.
-static int choose_num_waves(const PagedParams& p) {
+// Upper bound of the 128-row query tiles of the batch's multi-token sequences (the lengths stay
+// on the device): each such sequence has at least 2 tokens and wastes at most one tile.
+static int query_tile_bound(const PagedParams& p) {
+    if (p.num_tokens == p.num_seqs) return 0;  // one token per sequence: a pure decode batch
+    return p.num_tokens / 128 + std::min(p.num_seqs, p.num_tokens / 2);
+}
+
+// Mixed batches run the decode kernel beside the chunks' flash kernel unless the caller fixed the
+// number of decode wavefronts or HIPATTN_MIXED_OVERLAP=0 asks for one kernel after the other.
+static bool overlap_wanted(const PagedParams& p) {
+    if (query_tile_bound(p) == 0 || p.num_waves > 0) return false;
+    const char* e = getenv("HIPATTN_MIXED_OVERLAP");
+    return !(e && atoi(e) == 0);
+}
+
+static int choose_num_waves(const PagedParams& p, bool overlap) {
     if (p.num_waves > 0) return p.num_waves;
     const int resident = resident_decode_waves();
+    if (overlap) return resident;  // the most the plan may choose
     return p.cache_dtype == HIPATTN_U8 ? resident : resident / 2;
 }
 
@@ -774,17 +836,19 @@ static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // that starts on a new piece pays a chain of dependent loads (ticket, sequence, block table,
 // first block) before it streams again, and on MI355X that costs more than the better balance
 // at the end of the kernel wins back.  HIPATTN_DECODE_DYN_PIECES_PER_WAVE switches it on (tuning aid).
-static int choose_dyn_pieces(int num_waves) {
+static int choose_dyn_pieces(int num_waves, bool overlap) {
+    if (overlap) return 0;
     const char* e = getenv("HIPATTN_DECODE_DYN_PIECES_PER_WAVE");
     const int v = e ? atoi(e) : 0;
     return num_waves * std::min(std::max(v, 0), 64);
 }
 
 size_t paged_fast_workspace_bytes(const PagedParams& p) {
-    const int W = choose_num_waves(p);
+    const bool overlap = overlap_wanted(p);
+    const int W = choose_num_waves(p, overlap);
     const int G = p.num_heads_q / p.num_heads_kv;
-    const size_t slots = (size_t)W + choose_dyn_pieces(W) + (size_t)p.num_seqs * p.num_heads_kv;
-    return 256 + 2 * align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256) + align_up((size_t)p.num_seqs * 32, 256) +
+    const size_t slots = (size_t)W + choose_dyn_pieces(W, overlap) + (size_t)p.num_seqs * p.num_heads_kv;
+    return 512 + 2 * align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256) + align_up((size_t)p.num_seqs * 32, 256) +
            align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256) +
            (p.wave_trace ? align_up((size_t)W * 4 * sizeof(int64_t), 256) : 0);
 }
@@ -797,14 +861,22 @@ static int choose_switch_cost() {
 }
 
 void paged_fast_plan(PagedParams& p, void* workspace) {
-    p.num_waves = choose_num_waves(p);
+    const bool overlap = overlap_wanted(p);  // asks whether the caller fixed num_waves: before it is filled in
+    p.overlap = overlap ? 1 : 0;
+    p.num_waves = choose_num_waves(p, overlap);
     p.switch_cost = choose_switch_cost();
-    p.dyn_pieces = choose_dyn_pieces(p.num_waves);
+    p.dyn_pieces = choose_dyn_pieces(p.num_waves, overlap);
+    {
+        const char* e = getenv("HIPATTN_MIXED_DECODE_SHARE_PERCENT");  // tuning aid
+        p.overlap_share = e ? std::min(std::max(atoi(e), 10), 1000) / 100.0f : 1.0f;
+    }
     p.dyn_groups = std::min(64, std::max(1, p.num_waves / 32));  // every group has at least one wavefront
     const int G = p.num_heads_q / p.num_heads_kv;
     const size_t slots = (size_t)p.num_waves + p.dyn_pieces + (size_t)p.num_seqs * p.num_heads_kv;
     uint8_t* w = (uint8_t*)workspace;
     p.dyn_counter = (int32_t*)w;
+    w += 256;
+    p.plan_waves = (int32_t*)w;
     w += 256;
     p.tile_prefix = (int32_t*)w;
     w += align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
@@ -817,10 +889,34 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     p.part_ml = (float*)w;
     w += align_up(slots * G * 2 * sizeof(float), 256);
     if (p.wave_trace) p.wave_trace = (int64_t*)w;  // requested: the last 32 bytes per wavefront of the workspace
-    // query tiles of multi-token sequences: each has >= 2 tokens and wastes at most one tile
-    const int multi = std::min(p.num_seqs, p.num_tokens / 2);
-    // one token per sequence: a pure decode batch, no query tiles at all
-    p.max_q_tiles = (p.num_tokens == p.num_seqs) ? 0 : p.num_tokens / 128 + multi;
+    p.max_q_tiles = query_tile_bound(p);
+}
+
+// One side stream and a fork/join pair of events per device, made on first use and kept until the
+// process ends.  The mutex keeps the record/wait pairs of concurrent callers apart.
+struct SideStream {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    std::mutex mutex;
+};
+
+static SideStream* side_stream() {
+    static std::mutex table_mutex;
+    static SideStream* table[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> guard(table_mutex);
+    if (!table[dev]) {
+        SideStream* s = new SideStream;
+        if (hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking) != hipSuccess ||
+            hipEventCreateWithFlags(&s->fork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&s->join, hipEventDisableTiming) != hipSuccess) {
+            delete s;
+            return nullptr;
+        }
+        table[dev] = s;
+    }
+    return table[dev];
 }
 
 hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
@@ -836,13 +932,43 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     hipLaunchKernelGGL(paged_prologue_kernel, dim3(write_blocks + 1), dim3(256), 0, stream, wp, p, write_blocks);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    if (p.max_q_tiles > 0 && p.overlap) {
+        // Mixed batch: the decode sequences stream from HBM on a few compute units while the
+        // chunks' flash kernel, on a side stream, has the others; both only need the prologue's
+        // results.  The decode kernel stays on the caller's stream, directly behind the prologue,
+        // so that it is dispatched first and gets its compute units at once.
+        SideStream* side = side_stream();
+        if (!side) return hipErrorOutOfMemory;
+        std::lock_guard<std::mutex> guard(side->mutex);
+        if ((e = hipEventRecord(side->fork, stream)) != hipSuccess) return e;
+        if ((e = hipStreamWaitEvent(side->stream, side->fork, 0)) != hipSuccess) return e;
+        if (probe.before) (void)hipEventRecord(probe.before, stream);
+        const dim3 grid(p.num_waves / 8), block(512);
+        if (p.cache_dtype == HIPATTN_U8)
+            hipLaunchKernelGGL((paged_decode_kernel<true, false, 8>), grid, block, 0, stream, p);
+        else if (p.cache_dtype == HIPATTN_BF16)
+            hipLaunchKernelGGL((paged_decode_kernel<false, true, 8>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((paged_decode_kernel<false, false, 8>), grid, block, 0, stream, p);
+        e = hipGetLastError();
+        if (probe.after) (void)hipEventRecord(probe.after, stream);
+        const hipError_t e_prefill = launch_paged_prefill(p, side->stream);
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_seqs * p.num_heads_kv), dim3(256), 0, stream, p);
+            e = hipGetLastError();
+        }
+        // always join, also after an error, so the caller's stream never runs ahead of the side stream
+        hipError_t e_join = hipEventRecord(side->join, side->stream);
+        if (e_join == hipSuccess) e_join = hipStreamWaitEvent(stream, side->join, 0);
+        return e != hipSuccess ? e : (e_prefill != hipSuccess ? e_prefill : e_join);
+    }
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     if (p.cache_dtype == HIPATTN_U8)
-        hipLaunchKernelGGL((paged_decode_kernel<true, false>), dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<true, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p);
     else if (p.cache_dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL((paged_decode_kernel<false, true>), dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<false, true, 1>), dim3(p.num_waves), dim3(64), 0, stream, p);
     else
-        hipLaunchKernelGGL((paged_decode_kernel<false, false>), dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<false, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p);
     e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     if (e != hipSuccess) return e;

@@ -268,6 +268,41 @@ def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window, heads):
     dev.free()
 
 
+@pytest.mark.parametrize("env", [{}, {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "10"},
+                                 {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "1000"}, {"HIPATTN_MIXED_OVERLAP": "0"}])
+@pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.BF16, W.F16, 0), (W.F16, W.U8, 300), (W.BF16, W.BF16, 0)])
+def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, window, monkeypatch):
+    """With no fixed wavefront count the decode kernel of a mixed batch runs beside the chunks' flash
+    kernel on a share of the compute units that the plan picks on the device; whatever the share
+    (forced small and large here, and the one-after-the-other order), the results are the same, also
+    when calls follow each other without a synchronisation in between."""
+    announce("paged mixed side by side", env, q_dtype, cache_dtype, window)
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    batches = [
+        [(0, 130), (37, 1), (500, 1), (100, 257), (0, 2), (999, 1), (31, 97), (64, 1), (700, 128), (5, 0)],
+        [(0, 300), (210, 45)],                                       # no decode sequence at all
+        [(c - 1, 1) for c in DECODE_CTX] + [(3, 2)],                 # nearly all decode
+    ]
+    tol = 1e-2
+    for i, seqs in enumerate(batches):
+        case = W.make_paged_case(90 + i, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+        ref, okc, ovc = H.oracle_paged(oracle, case)
+        dev = H.PagedDeviceCase(hip, case)
+        out, path = dev.run()
+        assert path == "paged_mfma"
+        kc, vc = dev.caches()
+        np.testing.assert_array_equal(kc, okc)
+        np.testing.assert_array_equal(vc, ovc)
+        assert np.isfinite(out).all()
+        # N(0, 1) values and short contexts give outputs beyond 2, where the 16-bit output type alone
+        # rounds by up to 0.008: the bound is relative there
+        assert (np.abs(out - ref) <= tol * np.maximum(1.0, np.abs(ref))).all(), i
+        out2, _ = dev.run()  # the same tokens written again: same caches, same result
+        np.testing.assert_array_equal(out, out2)
+        dev.free()
+
+
 @pytest.mark.parametrize("shape", [(6, 2, 64, 16, W.F16, W.F16), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
                                    (4, 1, 128, 16, W.F16, W.U8), (34, 2, 128, 32, W.F16, W.F16)])
 def test_paged_generic_shapes(hip, oracle, shape):
