@@ -29,10 +29,22 @@ struct KvWriteParams {
     // kv heads one wavefront writes (set by kv_write_wavefronts): 1 for small batches, all of a
     // token's heads for large ones, where looking up the token's slot per head would dominate
     int heads_per_wave;
+    // head size 128, 16-bit new rows, 16-byte aligned pointers (set by kv_write_wavefronts): a
+    // wavefront writes four kv heads of a token with 16-byte loads
+    int vector_rows;
 };
 
 // Wavefronts the writer needs for p (and p.heads_per_wave, which it sets).
 inline int64_t kv_write_wavefronts(KvWriteParams& p) {
+    const auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const bool bits16 = p.kv_dtype == HIPATTN_F16 || p.kv_dtype == HIPATTN_BF16;
+    const bool cache_ok = p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8;
+    p.vector_rows = (p.head_dim == 128 && bits16 && cache_ok && aligned16(p.k_new) && aligned16(p.v_new) &&
+                     aligned16(p.key_cache) && aligned16(p.value_cache)) ? 1 : 0;
+    if (p.vector_rows) {
+        p.heads_per_wave = 4;
+        return (int64_t)p.num_tokens * ((p.num_heads_kv + 3) / 4);
+    }
     const int64_t pairs = (int64_t)p.num_tokens * p.num_heads_kv;
     p.heads_per_wave = pairs > 16384 ? p.num_heads_kv : 1;
     return (int64_t)p.num_tokens * ((p.num_heads_kv + p.heads_per_wave - 1) / p.heads_per_wave);

@@ -7,39 +7,125 @@
 
 namespace hipattn {
 
-// sequence that owns token t: largest s with subsequence_begins[s] <= t
-__device__ __forceinline__ int find_sequence(const int32_t* __restrict__ begins, int num_seqs, int t) {
-    int lo = 0, hi = num_seqs;  // invariant: begins[lo] <= t < begins[hi]
+// Largest s in [0, n) with prefix[s] <= x; requires prefix[0] <= x.  64-ary search: every round
+// is one vector load and one ballot, so a batch of 4096 sequences needs two rounds.
+__device__ __forceinline__ int locate_sequence(const int32_t* __restrict__ prefix, int n, int x, int lane) {
+    int lo = 0, hi = n;
     while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (begins[mid] <= t)
-            lo = mid;
-        else
-            hi = mid;
+        const int step = (hi - lo + 63) / 64;
+        const int idx = lo + lane * step;
+        const bool ok = idx < hi && prefix[idx] <= x;
+        const int k = __builtin_popcountll(__builtin_amdgcn_ballot_w64(ok)) - 1;  // prefix is monotone
+        lo = lo + k * step;
+        hi = min(hi, lo + step);
     }
     return lo;
 }
 
+// Where token t goes: physical block and position inside it; false when it has no valid target
+// (padding tokens outside every sequence, positions beyond the sequence's block table, block
+// numbers outside the pool).  A chain of dependent loads, done once per wavefront.
+__device__ __forceinline__ bool kv_write_slot(const KvWriteParams& p, int t, int lane, int& pb, int& pos) {
+    if (t >= p.num_tokens) return false;
+    if (t < p.subsequence_begins[0] || t >= p.subsequence_begins[p.num_seqs]) return false;
+    const int s = locate_sequence(p.subsequence_begins, p.num_seqs, t, lane);
+    pos = p.past_lens[s] + (t - p.subsequence_begins[s]);
+    if (pos < 0) return false;
+    const int lb = pos / p.block_size;
+    const int tb0 = p.block_indices_begins[s];
+    if (lb >= p.block_indices_begins[s + 1] - tb0) return false;
+    pb = p.block_indices[tb0 + lb];
+    return pb >= 0 && pb < p.num_blocks;
+}
+
+__device__ __forceinline__ float bits16_to_float(uint32_t bits, int dtype) {
+    return dtype == HIPATTN_F16 ? f16_bits_to_float((uint16_t)bits) : bf16_bits_to_float((uint16_t)bits);
+}
+__device__ __forceinline__ uint32_t float_to_bits16(float x, int dtype) {
+    return dtype == HIPATTN_F16 ? float_to_f16_bits(x) : float_to_bf16_bits(x);
+}
+
+// Head size 128 with 16-bit new rows (p.vector_rows): the wavefront takes four kv heads of one
+// token, which lie side by side in k_new / v_new, with one 16-byte load per lane for K and one for
+// V -- 16 lanes and 8 elements each to a head -- and writes the cache rows with 16-byte (16-bit
+// caches) or 8-byte (u8) stores.  The arithmetic is that of the element-wise path below, value
+// for value (the quantiser's minimum and maximum do not depend on the order of the reduction).
+__device__ __forceinline__ void kv_cache_write_rows128(const KvWriteParams& p, int64_t wv, int lane) {
+    const int chunks = (p.num_heads_kv + 3) >> 2;
+    const int t = (int)(wv / chunks);
+    const int h = (int)(wv % chunks) * 4 + (lane >> 4);
+    const int d0 = (lane & 15) * 8;
+    int pb = 0, pos = 0;
+    if (!kv_write_slot(p, t, lane, pb, pos)) return;  // wavefront-uniform
+    const bool active = h < p.num_heads_kv;
+    const int hh = active ? h : 0;  // idle lanes follow head 0 and store nothing
+    const int64_t src_off = ((int64_t)t * p.num_heads_kv + hh) * 128 + d0;
+    const uint4_t kraw = *(const uint4_t*)((const uint16_t*)p.k_new + src_off);
+    const uint4_t vraw = *(const uint4_t*)((const uint16_t*)p.v_new + src_off);
+    const int64_t rb = cache_row_bytes(p.cache_dtype, 128);
+    const int64_t row_off = (((int64_t)pb * p.num_heads_kv + hh) * p.block_size + pos % p.block_size) * rb;
+#pragma unroll
+    for (int which = 0; which < 2; which++) {
+        const uint4_t raw = which ? vraw : kraw;
+        uint8_t* row = (which ? p.value_cache : p.key_cache) + row_off;
+        if (p.cache_dtype == p.kv_dtype) {
+            if (active) *(uint4_t*)(row + d0 * 2) = raw;
+            continue;
+        }
+        float x[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) x[i] = bits16_to_float((raw[i >> 1] >> ((i & 1) * 16)) & 0xffffu, p.kv_dtype);
+        if (p.cache_dtype == HIPATTN_U8) {
+            float mn = x[0], mx = x[0];
+#pragma unroll
+            for (int i = 1; i < 8; i++) {
+                mn = fminf(mn, x[i]);
+                mx = fmaxf(mx, x[i]);
+            }
+#pragma unroll
+            for (int m = 1; m < 16; m <<= 1) {  // over the 16 lanes of the head
+                mn = fminf(mn, __shfl_xor(mn, m, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+            }
+            float scale = (mx - mn) / 255.0f;
+            if (scale == 0.0f) scale = 0.0001f;
+            const float zp = -mn / scale + 0.0f;  // -0 becomes +0
+            const float inv = 1.0f / scale;
+            uint32_t q[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = (uint32_t)fminf(fmaxf(rintf(fmaf(x[i], inv, zp)), 0.0f), 255.0f);
+            uint2_t packed;
+            packed[0] = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+            packed[1] = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
+            if (active) {
+                *(uint2_t*)(row + 8 + d0) = packed;
+                if ((lane & 15) == 0) *(float2*)row = make_float2(scale, zp);
+            }
+        } else {  // the other 16-bit type
+            uint4_t out;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                out[i] = float_to_bits16(x[2 * i], p.cache_dtype) | (float_to_bits16(x[2 * i + 1], p.cache_dtype) << 16);
+            if (active) *(uint4_t*)(row + d0 * 2) = out;
+        }
+    }
+}
+
 // Wavefront `wv` of the writer: the K rows and the V rows of one token for p.heads_per_wave kv
-// heads.  The token's slot (sequence by binary search, position, block table entry: a chain of
-// dependent loads) is looked up once per wavefront.
+// heads, element by element: any head size, any pair of types.  The token's slot is looked up once
+// per wavefront.
 template <int kMaxPerLane>
 __device__ __forceinline__ void kv_cache_write_wave(const KvWriteParams& p, int64_t wv, int lane) {
+    if (p.vector_rows) {
+        kv_cache_write_rows128(p, wv, lane);
+        return;
+    }
     const int hpw = p.heads_per_wave;
     const int groups = (p.num_heads_kv + hpw - 1) / hpw;
     const int t = (int)(wv / groups);
     const int h_begin = (int)(wv % groups) * hpw, h_end = min(h_begin + hpw, p.num_heads_kv);
-    if (t >= p.num_tokens) return;
-    // tokens outside every sequence (padding after the last subsequence) are ignored
-    if (t < p.subsequence_begins[0] || t >= p.subsequence_begins[p.num_seqs]) return;
-    const int s = find_sequence(p.subsequence_begins, p.num_seqs, t);
-    const int pos = p.past_lens[s] + (t - p.subsequence_begins[s]);
-    if (pos < 0) return;
-    const int lb = pos / p.block_size;
-    const int tb0 = p.block_indices_begins[s];
-    if (lb >= p.block_indices_begins[s + 1] - tb0) return;
-    const int pb = p.block_indices[tb0 + lb];
-    if (pb < 0 || pb >= p.num_blocks) return;
+    int pb = 0, pos = 0;
+    if (!kv_write_slot(p, t, lane, pb, pos)) return;
 
     const int D = p.head_dim;
     const int64_t rb = cache_row_bytes(p.cache_dtype, D);

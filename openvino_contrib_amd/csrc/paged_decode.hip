@@ -464,21 +464,6 @@ __global__ __launch_bounds__(256) void paged_prologue_kernel(KvWriteParams wp, P
     }
 }
 
-// Largest s in [0, n) with prefix[s] <= x; requires prefix[0] <= x.  64-ary search: every round
-// is one vector load and one ballot, so a batch of 4096 sequences needs two rounds.
-__device__ __forceinline__ int locate_sequence(const int32_t* __restrict__ prefix, int n, int x, int lane) {
-    int lo = 0, hi = n;
-    while (hi - lo > 1) {
-        const int step = (hi - lo + 63) / 64;
-        const int idx = lo + lane * step;
-        const bool ok = idx < hi && prefix[idx] <= x;
-        const int k = __builtin_popcountll(__builtin_amdgcn_ballot_w64(ok)) - 1;  // prefix is monotone
-        lo = lo + k * step;
-        hi = min(hi, lo + step);
-    }
-    return lo;
-}
-
 // How the work line [0, total) is cut into pieces.  Pieces 0 .. W-1 are the static ones, one per
 // wavefront, and share the first three quarters of the line equally; pieces W .. W+P-1 share the
 // last quarter and are handed out on demand (an atomic counter), so wavefronts that run faster

@@ -54,6 +54,28 @@ def test_kv_cache_write_bit_exact(hip, oracle, kv_dtype, cache_dtype):
     dev.free()
 
 
+@pytest.mark.parametrize("Hkv", [1, 3, 6, 8])
+@pytest.mark.parametrize("kv_dtype,cache_dtype", [(W.F16, W.F16), (W.BF16, W.F16), (W.F16, W.U8), (W.F16, W.BF16)])
+def test_kv_cache_write_head_counts(hip, oracle, Hkv, kv_dtype, cache_dtype):
+    """Head size 128 with 16-bit rows takes four heads to a wavefront: head counts that are not a
+    multiple of four leave lanes idle in the last one."""
+    announce("kv_write heads", Hkv, kv_dtype, cache_dtype)
+    seqs = [(0, 70), (31, 1), (100, 33), (5, 0), (63, 2)]
+    case = W.make_paged_case(53, seqs, Hkv, Hkv, 128, 32, W.F16, kv_dtype, cache_dtype)
+    dev = H.PagedDeviceCase(hip, case)
+    desc = H.pa_desc(hip, case)
+    hip.kv_cache_write(desc, dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                       dev.subsequence_begins, dev.block_indices, dev.block_indices_begins)
+    kc, vc = dev.caches()
+    okc, ovc = case["key_cache"].copy(), case["value_cache"].copy()
+    oracle.kv_cache_write(case["k_new"], case["v_new"], okc, ovc, cache_dtype, case["past_lens"],
+                          case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], Hkv, 128, 32)
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    assert (kc != case["key_cache"]).any(axis=-1).sum() == case["T"] * Hkv
+    dev.free()
+
+
 def test_kv_cache_write_skips_invalid_targets(hip, oracle):
     announce("kv_write invalid targets")
     case = W.make_paged_case(52, [(3, 40), (0, 33)], 4, 2, 64, 16, W.F16, W.F16, W.F16)
