@@ -325,6 +325,42 @@ def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, 
         dev.free()
 
 
+def test_paged_mixed_batches_from_two_host_threads(hip, oracle):
+    """Mixed-batch calls share one side stream per device; two host threads with a stream, a
+    workspace and tensors of their own each must not disturb each other."""
+    import threading
+
+    announce("paged mixed, two host threads")
+    batches = [[(0, 130), (37, 1), (500, 1), (100, 257), (999, 1)], [(10, 200), (640, 1), (64, 1), (3, 1), (0, 64)]]
+    cases = [W.make_paged_case(97 + i, b, 16, 4, 128, 32, W.F16, W.F16, W.F16) for i, b in enumerate(batches)]
+    refs = [H.oracle_paged(oracle, c)[0] for c in cases]
+    devs = [H.PagedDeviceCase(hip, c) for c in cases]
+    streams = [hip.Stream(), hip.Stream()]
+    results, errors = [None, None], []
+
+    def worker(i):
+        try:
+            hip.check(hip.lib().hipattn_set_device(0))
+            outs = [devs[i].run(stream=streams[i])[0] for _ in range(6)]
+            for o in outs[1:]:
+                np.testing.assert_array_equal(o, outs[0])
+            results[i] = outs[0]
+        except Exception as e:  # reported by the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not any(t.is_alive() for t in threads), "a worker is stuck"
+    assert not errors, errors
+    for i in range(2):
+        assert H.max_abs(results[i], refs[i]) <= 2e-3
+        devs[i].free()
+        streams[i].close()
+
+
 @pytest.mark.parametrize("shape", [(6, 2, 64, 16, W.F16, W.F16), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
                                    (4, 1, 128, 16, W.F16, W.U8), (34, 2, 128, 32, W.F16, W.F16)])
 def test_paged_generic_shapes(hip, oracle, shape):
