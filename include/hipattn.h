@@ -4,10 +4,10 @@
  * This is the boundary the C++ plugin operators (SdpaOp, PagedAttentionOp), the tests
  * and the benchmark call.  Plain C: pointers, sizes and POD descriptors; no C++ or
  * framework types.  Every pointer named "device" must be device memory of the current
- * HIP device; all calls are asynchronous on the given stream unless stated; nothing
- * here allocates behind the caller's back: scratch memory comes in through the
- * workspace arguments (the counterpart of the reference's WorkbufferRequest,
- * modules/nvidia_plugin/src/cuda_operation_base.hpp:114-117).  Functions return a
+ * HIP device; all calls are asynchronous on the given stream unless stated; no
+ * attention call allocates device memory behind the caller's back: scratch memory comes
+ * in through the workspace arguments (the counterpart of the reference's
+ * WorkbufferRequest, modules/nvidia_plugin/src/cuda_operation_base.hpp:114-117).  Functions return a
  * status code and never throw; hipattn_last_error_string() describes the last failure
  * on the calling thread.
  *
@@ -152,7 +152,12 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * All index arrays live in device memory and are only read there; the split of the work is
  * planned on the device.  max_context_len (>= max_s(past_lens[s] + q_len[s])) is advisory.
  * A sequence may contribute no token to a batch, with one exception: a batch with
- * num_tokens == num_seqs is taken to hold exactly one token per sequence (pure decode). */
+ * num_tokens == num_seqs is taken to hold exactly one token per sequence (pure decode).
+ * A mixed batch (single-token and multi-token sequences) with decode_waves == 0 runs its two
+ * parts side by side: the call forks from `stream` onto a side stream that the library keeps per
+ * device (created by the first such call, default priority, never destroyed) and joins before it
+ * returns, so `stream` order is all the caller has to know, also under stream capture.  The
+ * environment variable HIPATTN_MIXED_OVERLAP=0 switches that off. */
 enum {
     HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */
     HIPATTN_PA_FORCE_GENERIC = 2,    /* use the shape-generic kernels (testing aid) */
