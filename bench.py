@@ -157,6 +157,23 @@ def roofline_mfma(res):
             "kernel": "sdpa_flash_kernel"}
 
 
+def oracle_kind():
+    """Which CPU implementation stands beside the GPU figure.  The reference's natural one is
+    OpenVINO's CPU plugin running the same single-operator model; it is used only where OpenVINO is
+    installed, which is probed here and said in the record either way."""
+    import importlib.util
+
+    if importlib.util.find_spec("openvino") is None:
+        return "restatement (openvino is not importable on this machine)"
+    try:
+        import openvino
+
+        version = getattr(openvino, "__version__", "unknown version")
+    except Exception as e:  # an installation that does not load is as good as none
+        return "restatement (openvino found but failed to import: %s)" % type(e).__name__
+    return "restatement (OpenVINO %s is importable; running the single-operator model on its CPU plugin is not wired up)" % version
+
+
 def cpu_baseline_paged(case, budget_s=12.0):
     """Oracle (port, OpenMP over sequences x kv heads) on the whole batch, attention only,
     repeated until about budget_s seconds of CPU work have been spent."""
@@ -176,6 +193,7 @@ def cpu_baseline_paged(case, budget_s=12.0):
         times.append(time.perf_counter() - t0)
     mean = sum(times) / len(times)
     return {"value": W.paged_kv_bytes(case) / mean / 1e9, "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+            "oracle": oracle_kind(),
             "sample": "oracle paged attention (no cache write) on all %d sequences of the workload, mean of %d passes, "
                       "%.1f s of CPU work" % (case["S"], len(times), sum(times))}
 
@@ -198,6 +216,7 @@ def cpu_baseline_sdpa(case, budget_s=20.0):
         n += 1
     fl = W.sdpa_flops(1, G, case["Lq"], case["Lk"], case["D"], True) * len(times)
     return {"value": fl / sum(times) / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
+            "oracle": oracle_kind(),
             "sample": "oracle fp32 SDPA on %d of %d (batch, kv head) groups of the workload, %.1f s of CPU work"
                       % (len(times), case["B"] * case["Hkv"], sum(times))}
 
