@@ -5,7 +5,7 @@
  * (modules/nvidia_plugin/tests/unit/dynamic_shape.cpp:165-172 constructs Plugin directly,
  * compiles a model, creates an infer request, sets tensors, infers and compares).  Under a real
  * ov::Core these entry points are replaced by OpenVINO's plugin ABI
- * (src/cuda_create_plugin.cpp:11-12); see INTEGRATION.md.
+ * (src/cuda_create_plugin.cpp:11-12): create_plugin_engine() returning the Plugin object.
  *
  * All functions return 0 on success and a non-zero code on failure;
  * hip_plugin_last_error() then holds the exception text ("file:line(function): message").
