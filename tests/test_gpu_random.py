@@ -1,0 +1,67 @@
+"""Randomly drawn paged-attention batches against the oracle (gpu).
+
+The hand-picked cases of test_gpu_parity.py sit on the boundaries that were thought of; these do
+not: head counts (GQA ratios 1..16, kv head counts that are not multiples of four), cache and query
+types, sliding windows, and batches that are all decode, all prefill or mixed, with sequence
+lengths on and off the block and tile boundaries.  Seeds are fixed, so a failure names its case.
+
+Bounds: cache bytes bit-exact; outputs within 2e-3 (fp16 operands) or 1e-2 (bf16 queries, u8
+caches) of the oracle's fp32 result, relative to max(1, |value|) because N(0, 1) values give
+outputs beyond 1 where the 16-bit output type alone rounds by more.  bf16 caches are held to 2e-2:
+their probabilities enter the second product as bf16 (8 significant bits), and with N(0, 1) values
+single elements of a few million reach 1.2e-2 (the 99.99th percentile is 3e-3).
+"""
+import numpy as np
+import pytest
+
+import helpers as H
+from openvino_contrib_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_batch(rng):
+    G = int(rng.choice([1, 2, 3, 4, 5, 8, 16]))
+    Hkv = int(rng.choice([1, 2, 3, 4, 8]))
+    cache = int(rng.choice([W.F16, W.BF16, W.U8]))
+    q_dtype = int(rng.choice([W.F16, W.BF16]))
+    window = int(rng.choice([0, 0, 1, 17, 64, 300, 1000]))
+    kind = str(rng.choice(["decode", "mixed", "prefill"]))
+    seqs = []
+    for _ in range(int(rng.integers(1, 40))):
+        past = int(rng.choice([0, 1, 31, 32, 33, 100, 500, 1500, int(rng.integers(0, 3000))]))
+        if kind == "decode":
+            q_len = 1
+        elif kind == "prefill":
+            q_len = int(rng.choice([2, 5, 64, 127, 128, 129, 300]))
+        else:
+            q_len = int(rng.choice([1, 1, 1, 0, 2, 64, 130, 257]))
+        seqs.append((past, q_len))
+    return kind, G * Hkv, Hkv, cache, q_dtype, window, seqs
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13, 14])
+def test_random_paged_batches(hip, oracle, seed):
+    rng = np.random.default_rng(seed)
+    worst = 0.0
+    for it in range(16):
+        kind, Hq, Hkv, cache, q_dtype, window, seqs = draw_batch(rng)
+        if sum(n for _, n in seqs) == 0:
+            continue
+        print("[case] random paged", seed, it, kind, "Hq", Hq, "Hkv", Hkv, "cache", cache, "q", q_dtype, "window", window,
+              "seqs", seqs, flush=True)
+        case = W.make_paged_case(seed * 100 + it, seqs, Hq, Hkv, 128, 32, q_dtype, q_dtype, cache, sliding_window=window)
+        ref, okc, ovc = H.oracle_paged(oracle, case)
+        dev = H.PagedDeviceCase(hip, case)
+        out, path = dev.run()
+        kc, vc = dev.caches()
+        dev.free()
+        assert path == "paged_mfma"
+        np.testing.assert_array_equal(kc, okc)
+        np.testing.assert_array_equal(vc, ovc)
+        assert np.isfinite(out).all()
+        tol = 2e-2 if cache == W.BF16 else (1e-2 if (cache == W.U8 or q_dtype == W.BF16) else 2e-3)
+        err = float((np.abs(out - ref) / np.maximum(1.0, np.abs(ref))).max())
+        worst = max(worst, err / tol)
+        assert err <= tol, (seed, it)
+    print("worst error / bound: %.2f" % worst)
