@@ -65,3 +65,32 @@ def test_random_paged_batches(hip, oracle, seed):
         worst = max(worst, err / tol)
         assert err <= tol, (seed, it)
     print("worst error / bound: %.2f" % worst)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_sdpa_shapes(hip, oracle, seed):
+    """Dense SDPA: batch, GQA ratio, head size (128 takes the MFMA kernel for 16-bit types, the
+    others and fp32 the shape-generic one), square and rectangular score matrices, causal or not."""
+    rng = np.random.default_rng(seed)
+    worst = {}
+    for it in range(24):
+        G = int(rng.choice([1, 2, 3, 4, 5, 8]))
+        Hkv = int(rng.choice([1, 2, 3]))
+        B = int(rng.choice([1, 2, 3]))
+        D = int(rng.choice([128, 128, 128, 64, 32]))
+        dtype = int(rng.choice([W.F16, W.BF16, W.F32]))
+        Lq = int(rng.choice([1, 2, 31, 64, 127, 128, 129, 255, 256, 257, 300, 511, 700, int(rng.integers(1, 900))]))
+        Lk = Lq if rng.random() < 0.5 else int(rng.choice([1, 63, 64, 65, 200, 513, 1000, int(rng.integers(1, 1200))]))
+        causal = bool(rng.random() < 0.6)
+        print("[case] random sdpa", seed, it, "B", B, "Hq", G * Hkv, "Hkv", Hkv, "Lq", Lq, "Lk", Lk, "D", D, "dtype", dtype,
+              "causal", causal, flush=True)
+        case = W.make_sdpa_case(seed * 100 + it, B, G * Hkv, Hkv, Lq, Lk, D, dtype, std=0.5 if dtype == W.BF16 else 1.0)
+        out, path = H.run_sdpa(hip, case, causal)
+        ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+        rows = np.isfinite(ref)  # a row that attends to no key at all is unspecified in the oracle as well
+        tol = {W.F32: 1e-4, W.F16: 2e-3, W.BF16: 1e-2}[dtype]
+        err = np.abs(out - ref)[rows] / np.maximum(1.0, np.abs(ref[rows]))
+        e = float(err.max()) if err.size else 0.0
+        worst[path] = max(worst.get(path, 0.0), e / tol)
+        assert e <= tol, (seed, it, path)
+    print("worst error / bound by kernel path:", worst)
