@@ -156,7 +156,8 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * A mixed batch (single-token and multi-token sequences) with decode_waves == 0 runs its two
  * parts side by side: the call forks from `stream` onto a side stream that the library keeps per
  * device (created by the first such call, default priority, never destroyed) and joins before it
- * returns, so `stream` order is all the caller has to know, also under stream capture.  The
+ * returns, so `stream` order is all the caller has to know, also under stream capture (make the
+ * first such call on a device outside a capture: creating a stream is not a capturable operation).  The
  * environment variable HIPATTN_MIXED_OVERLAP=0 switches that off. */
 enum {
     HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */
