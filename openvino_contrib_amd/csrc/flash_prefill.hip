@@ -577,8 +577,9 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0,
 // ring stages of K(x-1) and V(x-2); every wavefront issues its rows of B(x) in a vector phase
 // (group 0 in phase 2x+1, group 1 in phase 2x), and at each barrier waits for all of its loads
 // except the latest batch, which puts B(x) in LDS two phases before its first use.
-template <bool kBf16, bool kU8 = false>
+template <bool kBf16, bool kU8 = false, bool kPaged = true>
 __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
+    static_assert(kPaged || !kU8, "dense K/V are 16-bit");
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16");
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
@@ -677,13 +678,15 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         return 2;
     };
     // Block table entry of this wavefront's rows of tile j (0 when there is none), read through
-    // the scalar cache in the vector phase, so that no scalar load is outstanding during a
-    // matrix phase (which would turn every partial wait for LDS fragments into a full one).
+    // the scalar cache at the end of a matrix phase, behind its last fragment wait: a scalar load
+    // outstanding while fragments are still being waited for would turn every partial wait for LDS
+    // fragments into a full one.
     // (As inline assembly, because behind the compiler fences of the barriers an ordinary load of
     // the table becomes a vector load that is waited for at once, together with every load to LDS
     // in flight.  The wait for the scalar load is part of the statement: the compiler takes the
     // output register as written when the statement ends and may reuse it at any time after.)
     auto table_entry = [&](int j) -> int {
+        if constexpr (!kPaged) return 0;
         const int key0 = kv_lo + j * kTileK + 8 * wave;
         if (t.table == nullptr || j >= n || key0 + 8 > t.kv_len) return 0;
         int entry;
@@ -757,6 +760,21 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             barrier_keeping_loads(keep);
     };
 
+    // Dense K/V: tile j's eight rows of this wavefront are keys kv_lo + 64 j + 8 wave + [0, 8); for the
+    // first fast_tiles tiles all of them exist, and their loads are two instructions on a source
+    // address that advances by one tile per iteration (fill_k / fill_v: the rows of the tiles that
+    // iteration j fills, K(j + group + 2) and V(j + group + 1)).
+    int fast_tiles = 0;
+    const uint8_t* fill_k = nullptr;
+    const uint8_t* fill_v = nullptr;
+    const uint32_t k_lane1 = (k_lane ^ 64u) + 4 * kRowBytes, v_lane1 = v_lane + 4 * kRowBytes;
+    if constexpr (!kPaged) {
+        const int room = t.kv_len - kv_lo - 8 * wave - 8;
+        fast_tiles = room >= 0 ? min(n, room / kTileK + 1) : 0;
+        fill_k = t.k + (int64_t)(kv_lo + (group + 2) * kTileK + 8 * wave) * kRowBytes;
+        fill_v = t.v + (int64_t)(kv_lo + (group + 1) * kTileK + 8 * wave) * kRowBytes;
+    }
+
     // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
     const int e0 = table_entry(0), e1 = table_entry(1), e2 = table_entry(2), e3 = table_entry(3);
     int first = 0, recent = 0;
@@ -816,8 +834,16 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     // restrict qualifiers tell the compiler that the LDS writes of the asynchronous loads cannot
     // alias the fragment reads, so that it does not wait for all loads before every LDS read; the
     // barriers do the waiting that is needed.
-    auto two_phases = [&](int j, bool last, const lds_byte* __restrict__ k_next, const lds_byte* __restrict__ v_cur,
-                          lds_byte* __restrict__ k_fill, lds_byte* __restrict__ v_fill) {
+    // The four stages an iteration touches walk round their rings in step: their indices are carried
+    // (add, compare, select) instead of taking j modulo the ring length four times per iteration;
+    // index * 16 KB keeps the stage addresses visibly aligned for the fragment address arithmetic.
+    int i_kn = 1 % kStages, i_vc = 0, i_kf = (group + 2) % kStages, i_vf = (group + 1) % kStages;
+    auto bump = [](int& i) __attribute__((always_inline)) { i = (i + 1 == kStages) ? 0 : i + 1; };
+    auto two_phases = [&](int j, bool last) {
+        const lds_byte* __restrict__ const k_next = k_ring + i_kn * kKBytes;
+        const lds_byte* __restrict__ const v_cur = v_ring + i_vc * kKBytes;
+        lds_byte* __restrict__ const k_fill = k_ring + i_kf * kKBytes;
+        lds_byte* __restrict__ const v_fill = v_ring + i_vf * kKBytes;
         // ---- vector phase
 #ifdef HIPATTN_FLASH_TRACE
         clk.tile = j;
@@ -828,11 +854,21 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             // use; the rows of this iteration's batch are fetched into registers
             u8_store(pending);
             pending = u8_fetch(j + group + 2, entry_k, j + group + 1, entry_v);
+        } else if constexpr (!kPaged) {
+            if (j + group + 2 < fast_tiles) {  // then the rows of V(j + group + 1) exist as well
+                lds_byte* const kd = k_fill + 8 * wave * kRowBytes;
+                lds_byte* const vd = v_fill + 8 * wave * kRowBytes;
+                load_to_lds_16(fill_k, k_lane, kd);
+                load_to_lds_16(fill_k, k_lane1, kd + 4 * kRowBytes);
+                load_to_lds_16(fill_v, v_lane, vd);
+                load_to_lds_16(fill_v, v_lane1, vd + 4 * kRowBytes);
+                recent = 4;
+            } else {
+                recent = load_rows(true, j + group + 2, k_fill, 0) + load_rows(false, j + group + 1, v_fill, 0);
+            }
         } else {
             recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
         }
-        entry_v = entry_k;  // the next iteration loads V of the tile whose K was loaded now
-        entry_k = table_entry(j + group + 3);
         FLASH_STAMP(clk, 1);
         tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
         // (the probabilities are complete before the barrier: the compiler may not move their
@@ -860,12 +896,30 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             tile_accumulate<kBf16>(zero, fs, pf, o);
         __builtin_amdgcn_s_setprio(0);
         FLASH_STAMP(clk, 5);
+        // The next iteration's stages and source rows are worked out here, where the wavefront would
+        // otherwise only wait at the barrier for the other group's vector phase; behind the barrier
+        // this scalar arithmetic would sit at the head of its own vector phase.
+        bump(i_kn);
+        bump(i_vc);
+        bump(i_kf);
+        bump(i_vf);
+        if constexpr (kPaged) {
+            // (every fragment read of the matrix phase has been waited for by now, so the scalar
+            // load's own wait costs the phase nothing)
+            entry_v = entry_k;  // the next iteration loads V of the tile whose K was loaded now
+            entry_k = table_entry(j + group + 3);
+        }
+        if constexpr (!kPaged) {
+            fill_k += kTileK * kRowBytes;
+            fill_v += kTileK * kRowBytes;
+            asm volatile("" : "+s"(fill_k), "+s"(fill_v));
+        }
+        asm volatile("" : "+s"(i_kn), "+s"(i_vc), "+s"(i_kf), "+s"(i_vf));
         phase_barrier(recent);
         FLASH_STAMP(clk, 6);
     };
-    for (int j = 0; j < n - 1; j++)
-        two_phases(j, false, k_stage(j + 1), v_stage(j), k_stage(j + group + 2), v_stage(j + group + 1));
-    two_phases(n - 1, true, k_stage(n), v_stage(n - 1), k_stage(n + group + 1), v_stage(n + group));
+    for (int j = 0; j < n - 1; j++) two_phases(j, false);
+    two_phases(n - 1, true);
 #ifdef HIPATTN_FLASH_TRACE
     if (g_flash_phase_trace && lane == 0) {
         long long* r = g_flash_phase_trace + ((int64_t)blockIdx.x * 8 + wave) * 8;
@@ -949,7 +1003,7 @@ __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) 
     return t;
 }
 
-template <bool kBf16, bool kU8 = false>
+template <bool kBf16, bool kU8 = false, bool kPaged = true>
 __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t* lds, float scale) {
     int lo0, hi0, lo1, hi1;
     key_range(t0, lo0, hi0);
@@ -966,7 +1020,7 @@ __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t
         kv_hi = max(hi0, hi1);
     }
     const int group = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
-    run_pair<kBf16, kU8>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
+    run_pair<kBf16, kU8, kPaged>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
 }
 
 template <bool kBf16>
@@ -980,7 +1034,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
 #endif
     const Tile t0 = sdpa_group_tile(p, 0), t1 = sdpa_group_tile(p, 1);
-    run_both<kBf16>(t0, t1, lds, p.scale);
+    run_both<kBf16, false, false>(t0, t1, lds, p.scale);
 #ifdef HIPATTN_FLASH_TRACE
     if (g_flash_wg_trace && threadIdx.x == 0) {
         long long* r = g_flash_wg_trace + (int64_t)blockIdx.x * 8;
