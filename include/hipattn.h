@@ -152,7 +152,9 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * All index arrays live in device memory and are only read there; the split of the work is
  * planned on the device.  max_context_len (>= max_s(past_lens[s] + q_len[s])) is advisory.
  * A sequence may contribute no token to a batch, with one exception: a batch with
- * num_tokens == num_seqs is taken to hold exactly one token per sequence (pure decode).
+ * num_tokens == num_seqs is taken to hold exactly one token per sequence (pure decode: the host
+ * cannot see the lengths, and a decode step should not pay for a launch that finds nothing to
+ * do), unless HIPATTN_PA_ANY_LENGTHS says otherwise.
  * A mixed batch (single-token and multi-token sequences) with decode_waves == 0 runs its two
  * parts side by side: the call forks from `stream` onto a side stream that the library keeps per
  * device (created by the first such call, default priority, never destroyed) and joins before it
@@ -162,6 +164,8 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
 enum {
     HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */
     HIPATTN_PA_FORCE_GENERIC = 2,    /* use the shape-generic kernels (testing aid) */
+    HIPATTN_PA_ANY_LENGTHS = 8,      /* num_tokens == num_seqs does not mean one token per sequence
+                                        here (a batch with empty sequences beside longer ones) */
     HIPATTN_PA_TRACE_WAVES = 4       /* diagnostic: the decode kernel leaves, in the last
                                         decode_waves * 32 bytes of the workspace, four int64 per
                                         wavefront: entry, first block consumed, exit (100 MHz

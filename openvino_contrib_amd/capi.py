@@ -16,6 +16,8 @@ OK, INVALID_ARGUMENT, UNSUPPORTED, WORKSPACE_TOO_SMALL, HIP_ERROR, NO_DEVICE = r
 F32, F16, BF16, U8 = 0, 1, 2, 3
 PA_SKIP_CACHE_WRITE = 1
 PA_FORCE_GENERIC = 2
+PA_TRACE_WAVES = 4
+PA_ANY_LENGTHS = 8
 
 DTYPE_BYTES = {F32: 4, F16: 2, BF16: 2, U8: 1}
 

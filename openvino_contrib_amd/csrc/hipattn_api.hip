@@ -123,6 +123,7 @@ hipattn::PagedParams make_paged_params(const hipattn_pa_desc* d) {
     p.sliding_window = d->sliding_window;
     p.scale = resolve_scale(d->scale, d->head_dim);
     p.num_waves = d->decode_waves > 0 ? d->decode_waves : 0;
+    p.any_lengths = (d->flags & HIPATTN_PA_ANY_LENGTHS) ? 1 : 0;
     p.wave_trace = (d->flags & HIPATTN_PA_TRACE_WAVES) ? reinterpret_cast<int64_t*>(1) : nullptr;  // placed by the plan
     return p;
 }

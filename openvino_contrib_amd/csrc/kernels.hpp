@@ -109,6 +109,7 @@ struct PagedParams {
     // chunked prefill: query-tile schedule built on the device
     int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
     int max_q_tiles;      // grid upper bound
+    int any_lengths;      // num_tokens == num_seqs may still hide multi-token sequences (HIPATTN_PA_ANY_LENGTHS)
     // diagnostic (HIPATTN_PA_TRACE_WAVES): per decode wavefront {entry, first block consumed, exit, line units}
     int64_t* wave_trace;
 };

@@ -796,7 +796,7 @@ static int resident_decode_waves() {
 // Upper bound of the 128-row query tiles of the batch's multi-token sequences (the lengths stay
 // on the device): each such sequence has at least 2 tokens and wastes at most one tile.
 static int query_tile_bound(const PagedParams& p) {
-    if (p.num_tokens == p.num_seqs) return 0;  // one token per sequence: a pure decode batch
+    if (p.num_tokens == p.num_seqs && !p.any_lengths) return 0;  // one token per sequence: a pure decode batch
     return p.num_tokens / 128 + std::min(p.num_seqs, p.num_tokens / 2);
 }
 

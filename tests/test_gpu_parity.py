@@ -325,6 +325,27 @@ def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, 
         dev.free()
 
 
+def test_paged_as_many_tokens_as_sequences_but_not_one_each(hip, oracle):
+    """num_tokens == num_seqs normally means a pure decode batch (the host cannot see the lengths);
+    a batch that only looks like one -- an empty sequence beside a two-token one -- needs the
+    HIPATTN_PA_ANY_LENGTHS flag, and with it goes through the mixed-batch path."""
+    announce("paged T == S with mixed lengths")
+    for cache_dtype in (W.F16, W.U8):
+        case = W.make_paged_case(99, [(1500, 1), (100, 2), (31, 0)], 24, 3, 128, 32, W.F16, W.F16, cache_dtype,
+                                 sliding_window=64)
+        assert case["T"] == case["S"]
+        ref, okc, ovc = H.oracle_paged(oracle, case)
+        dev = H.PagedDeviceCase(hip, case)
+        out, path = dev.run(flags=hip.PA_ANY_LENGTHS)
+        assert path == "paged_mfma"
+        kc, vc = dev.caches()
+        np.testing.assert_array_equal(kc, okc)
+        np.testing.assert_array_equal(vc, ovc)
+        assert np.isfinite(out).all()
+        assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3)
+        dev.free()
+
+
 def test_paged_mixed_batches_from_two_host_threads(hip, oracle):
     """Mixed-batch calls share one side stream per device; two host threads with a stream, a
     workspace and tensors of their own each must not disturb each other."""
