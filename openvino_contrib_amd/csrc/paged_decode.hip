@@ -383,9 +383,9 @@ __device__ __forceinline__ int line_units(int nb, int switch_cost) { return nb >
 // (b) 128-row query tiles of multi-token sequences.  One workgroup; sequences are split evenly
 // over the threads.
 __device__ __forceinline__ void plan_block(const PagedParams& p) {
-    __shared__ int part_blk[256];
-    __shared__ int part_tile[256];
-    __shared__ float part_keys[256];
+    __shared__ int wave_blk[4];
+    __shared__ int wave_tile[4];
+    __shared__ float wave_keys[4];
     const int tid = threadIdx.x;
     if (tid < 64) p.dyn_counter[tid] = 0;  // tickets for the dynamic pieces of this call, one counter per group
     const int per = (p.num_seqs + 255) / 256;
@@ -405,39 +405,53 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
             }
         }
     }
-    part_blk[tid] = blk;
-    part_tile[tid] = tile;
-    part_keys[tid] = key_tiles;
-    __syncthreads();
-    if (tid == 0) {
-        int rb = 0, rt = 0;
-        float rk = 0.0f;
-        for (int i = 0; i < 256; i++) {
-            const int vb = part_blk[i], vt = part_tile[i];
-            part_blk[i] = rb;
-            part_tile[i] = rt;
-            rb += vb;
-            rt += vt;
-            rk += part_keys[i];
-        }
-        if (p.overlap) {
-            // Compute-unit time of the two parts, in microseconds, as measured with both running:
-            // a compute unit of the decode kernel streams about 33 GB/s of fp16 cache (u8: 24 GB/s),
-            // one of the flash kernel does a 128-row x 64-key tile of one head in about 1.2 us
-            // (u8 caches, dequantised on the way: 1.7 us).  Each part gets compute units in
-            // proportion to its work, so that both end together.
-            const bool u8 = p.cache_dtype == HIPATTN_U8;
-            const float decode_us = (float)rb * p.num_heads_kv * (u8 ? 8704.0f / 24000.0f : 16384.0f / 33000.0f) * p.overlap_share;
-            const float prefill_us = rk * p.num_heads_q * (u8 ? 1.7f : 1.2f);
-            const int cus = p.num_waves >> 3;
-            int mine = (int)ceilf(cus * decode_us / fmaxf(decode_us + prefill_us, 1.0f));
-            mine = max(1, min(mine, cus));
-            p.plan_waves[0] = mine * 8;
+    // Exclusive prefix sums over the 256 threads: a scan inside each wavefront (six shuffle steps),
+    // then the totals of the wavefronts ahead.  (One thread adding up 256 values in LDS took about as
+    // long as the rest of the launch.)
+    const int lane = tid & 63, wv = tid >> 6;
+    int scan_blk = blk, scan_tile = tile;
+    float scan_keys = key_tiles;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int ub = __shfl_up(scan_blk, d, 64), ut = __shfl_up(scan_tile, d, 64);
+        const float uk = __shfl_up(scan_keys, d, 64);
+        if (lane >= d) {
+            scan_blk += ub;
+            scan_tile += ut;
+            scan_keys += uk;
         }
     }
+    if (lane == 63) {
+        wave_blk[wv] = scan_blk;
+        wave_tile[wv] = scan_tile;
+        wave_keys[wv] = scan_keys;
+    }
     __syncthreads();
-    blk = part_blk[tid];
-    tile = part_tile[tid];
+    int ahead_blk = 0, ahead_tile = 0, total_blk = 0;
+    float total_keys = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        ahead_blk += w < wv ? wave_blk[w] : 0;
+        ahead_tile += w < wv ? wave_tile[w] : 0;
+        total_blk += wave_blk[w];
+        total_keys += wave_keys[w];
+    }
+    if (tid == 0 && p.overlap) {
+        // Compute-unit time of the two parts, in microseconds, as measured with both running:
+        // a compute unit of the decode kernel streams about 33 GB/s of fp16 cache (u8: 24 GB/s),
+        // one of the flash kernel does a 128-row x 64-key tile of one head in about 1.2 us
+        // (u8 caches, dequantised on the way: 1.7 us).  Each part gets compute units in
+        // proportion to its work, so that both end together.
+        const bool u8 = p.cache_dtype == HIPATTN_U8;
+        const float decode_us = (float)total_blk * p.num_heads_kv * (u8 ? 8704.0f / 24000.0f : 16384.0f / 33000.0f) * p.overlap_share;
+        const float prefill_us = total_keys * p.num_heads_q * (u8 ? 1.7f : 1.2f);
+        const int cus = p.num_waves >> 3;
+        int mine = (int)ceilf(cus * decode_us / fmaxf(decode_us + prefill_us, 1.0f));
+        mine = max(1, min(mine, cus));
+        p.plan_waves[0] = mine * 8;
+    }
+    blk = ahead_blk + scan_blk - blk;
+    tile = ahead_tile + scan_tile - tile;
     for (int s = s0; s < s1; s++) {
         const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
         p.blk_prefix[s] = blk;
