@@ -24,10 +24,15 @@ CAPTURE_MODE_RELAXED = 2
 
 def hip_runtime():
     """The HIP runtime library this process already has loaded (the one libhipattn.so links to)."""
+    import os
+
     with open("/proc/self/maps") as f:
-        paths = {line.split()[-1] for line in f if "libamdhip64" in line}
+        paths = sorted({line.split()[-1] for line in f if "libamdhip64" in line})
     assert paths, "libhipattn.so is loaded, so the HIP runtime must be"
-    rt = ctypes.CDLL(sorted(paths)[0])
+    # another copy may be mapped as well (a Python package that bundles its own): take the ROCm
+    # installation's, which is the one libhipattn.so is linked against
+    rocm = [q for q in paths if os.path.realpath(q).startswith(os.path.realpath("/opt/rocm"))]
+    rt = ctypes.CDLL((rocm or paths)[0])
     vp = ctypes.c_void_p
     rt.hipStreamBeginCapture.argtypes = [vp, ctypes.c_int]
     rt.hipStreamEndCapture.argtypes = [vp, ctypes.POINTER(vp)]
