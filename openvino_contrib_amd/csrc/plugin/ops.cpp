@@ -189,6 +189,18 @@ private:
         d.sliding_window = host_scalar<int32_t>(in[kSlidingWindow], "sliding_window", 0, false);
         d.max_context_len = host_scalar<int32_t>(in[kMaxContextLen], "max_context_len", 0, false);
         d.flags = 0;
+        // As many tokens as sequences normally means one token each, and the kernels plan for that
+        // without looking; when the lengths came from a host tensor they are looked at here, so that
+        // a batch that only resembles a decode step (an empty sequence beside a longer one) is
+        // announced as what it is.
+        if (d.num_tokens == d.num_seqs && in[kSubsequenceBegins].host != nullptr) {
+            const int32_t* begins = static_cast<const int32_t*>(in[kSubsequenceBegins].host);
+            for (int s = 0; s < d.num_seqs; s++)
+                if (begins[s + 1] - begins[s] != 1) {
+                    d.flags |= HIPATTN_PA_ANY_LENGTHS;
+                    break;
+                }
+        }
         d.decode_waves = 0;
         return d;
     }

@@ -69,10 +69,15 @@ def test_sdpa_dynamic_shapes_one_compiled_model(hip, oracle):
         compiled.create_infer_request().infer()
 
 
-@pytest.mark.parametrize("cache_dtype,q_dtype,window", [(W.F16, W.F16, 0), (W.U8, W.F16, 0), (W.F16, W.BF16, 200)])
-def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_dtype, window):
-    print("[plugin] paged attention", cache_dtype, q_dtype, window, flush=True)
-    seqs = [(0, 130), (37, 1), (500, 1), (100, 257), (999, 1), (64, 1)]
+MIXED_BATCH = [(0, 130), (37, 1), (500, 1), (100, 257), (999, 1), (64, 1)]
+LOOKS_LIKE_DECODE = [(1500, 1), (100, 2), (31, 0)]  # as many tokens as sequences, but not one each
+
+
+@pytest.mark.parametrize("cache_dtype,q_dtype,window,seqs", [(W.F16, W.F16, 0, MIXED_BATCH), (W.U8, W.F16, 0, MIXED_BATCH),
+                                                              (W.F16, W.BF16, 200, MIXED_BATCH),
+                                                              (W.F16, W.F16, 64, LOOKS_LIKE_DECODE)])
+def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_dtype, window, seqs):
+    print("[plugin] paged attention", cache_dtype, q_dtype, window, seqs, flush=True)
     case = W.make_paged_case(94, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
     plugin = P.Plugin()
     plugin.set_property("PERF_COUNT", "YES")
