@@ -805,8 +805,10 @@ static int resident_decode_waves() {
     return cached_waves;
 }
 
-// fp16 caches stream best with one wavefront per SIMD; the u8 path has more arithmetic per
-// byte and wants both resident wavefronts to cover it.
+// fp16 caches stream best with one wavefront per SIMD (four per compute unit; three measure the
+// same); the u8 path has more arithmetic per byte and wants more: six per compute unit measured
+// 1.5 % faster than all eight on the 128-sequence u8 configuration, counts that do not divide
+// evenly over the compute units 5-10 % slower.
 // Upper bound of the 128-row query tiles of the batch's multi-token sequences (the lengths stay
 // on the device): each such sequence has at least 2 tokens and wastes at most one tile.
 static int query_tile_bound(const PagedParams& p) {
@@ -826,7 +828,7 @@ static int choose_num_waves(const PagedParams& p, bool overlap) {
     if (p.num_waves > 0) return p.num_waves;
     const int resident = resident_decode_waves();
     if (overlap) return resident;  // the most the plan may choose
-    return p.cache_dtype == HIPATTN_U8 ? resident : resident / 2;
+    return p.cache_dtype == HIPATTN_U8 ? resident / 4 * 3 : resident / 2;
 }
 
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
