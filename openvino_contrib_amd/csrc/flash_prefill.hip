@@ -335,13 +335,15 @@ __device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], f
     };
     // Common case (an unmasked tile, every row already has a reference): no row maximum at all.
     // The exponentials are taken against the standing reference and the tile's row sums tell
-    // whether that was safe: a sum below 2^24 bounds every probability, and anything else (large,
-    // infinite, NaN) sends the wavefront through the careful path below, which redoes the tile
-    // from the untouched scores.  Sixteen v_max3, the cross-lane exchange and the compare of the
+    // whether that was safe: a sum below the bound (2^24; 2^15 where the probabilities become fp16,
+    // which ends at 65504) bounds every probability, and anything else (large, infinite, NaN)
+    // sends the wavefront through the careful path below, which redoes the tile from the
+    // untouched scores.  Sixteen v_max3, the cross-lane exchange and the compare of the
     // maximum are then spent only on the first tile of a row, on masked tiles and on outliers.
     if (!masked && st.all_started) {
         const float sum = probabilities();
-        if (!__builtin_amdgcn_ballot_w64(!(sum < 16777216.0f))) {
+        constexpr float kSafeSum = kBf16 ? 16777216.0f : 32768.0f;
+        if (!__builtin_amdgcn_ballot_w64(!(sum < kSafeSum))) {
             st.l_run += sum;
             return;
         }

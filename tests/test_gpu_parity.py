@@ -148,6 +148,34 @@ def test_sdpa_flash(hip, oracle, dtype, shape, causal):
     assert H.max_abs(out, ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [W.F16, W.BF16])
+@pytest.mark.parametrize("profile", ["ramp", "step16", "step40", "spike"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_sdpa_flash_scores_that_grow_along_the_keys(hip, oracle, dtype, profile, causal):
+    """Later keys score far above the earlier ones, so that the running reference of the softmax
+    has to move after the first tile: by a slow ramp (3 bits per 64-key tile), by a step of
+    about 16 or 40 bits (2^16 is beyond fp16, 2^40 beyond the sum check of either type) and by a
+    single key 30 bits above everything else."""
+    announce("sdpa growing scores", dtype, profile, causal)
+    B, Hq, Hkv, L, D = 1, 4, 2, 1024, 128
+    rng = np.random.Generator(np.random.PCG64(71))
+    gain = {"ramp": np.linspace(0.0, 3.0, L), "step16": np.where(np.arange(L) >= 600, 1.0, 0.0),
+            "step40": np.where(np.arange(L) >= 600, 2.5, 0.0),
+            "spike": np.where(np.arange(L) == 777, 1.9, 0.0)}[profile].astype(np.float32)
+    # scores in nats are about 128 / sqrt(128) * gain = 11.3 gain, plus noise of about 0.3
+    q = 0.3 * rng.standard_normal((B, Hq, L, D), dtype=np.float32) + 1.0
+    k = 0.3 * rng.standard_normal((B, Hkv, L, D), dtype=np.float32) + gain[None, None, :, None]
+    v = rng.standard_normal((B, Hkv, L, D), dtype=np.float32)
+    case = {"B": B, "Hq": Hq, "Hkv": Hkv, "Lq": L, "Lk": L, "D": D, "dtype": dtype}
+    for name, x in (("q", q), ("k", k), ("v", v)):
+        case[name + "_store"], case[name] = W.to_storage(x, dtype)
+    out, path = H.run_sdpa(hip, case, causal)
+    assert path == "sdpa_flash_mfma"
+    ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+    assert np.isfinite(out).all()
+    assert float(np.max(np.abs(out - ref) / np.maximum(1.0, np.abs(ref)))) <= TOL[dtype]
+
+
 def test_sdpa_scale_and_empty(hip, oracle):
     announce("sdpa scale/empty")
     case = W.make_sdpa_case(63, 1, 2, 1, 90, 90, 128, W.F16)
