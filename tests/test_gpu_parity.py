@@ -318,6 +318,51 @@ def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window, heads):
     dev.free()
 
 
+@pytest.mark.parametrize("q_dtype,cache_dtype", [(W.F16, W.F16), (W.BF16, W.F16), (W.F16, W.U8), (W.BF16, W.BF16)])
+@pytest.mark.parametrize("profile", ["ramp", "step16", "step40"])
+def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dtype, profile):
+    """Chunks and decode tokens whose later keys score far above the earlier ones (see the dense
+    test of the same name): the keys of every sequence, in the cache and among the new tokens, are
+    rewritten so that their scores rise with the position."""
+    announce("paged growing scores", q_dtype, cache_dtype, profile)
+    seqs = [(0, 700), (900, 1), (1500, 1), (400, 300), (2000, 1), (63, 1)]
+    Hq, Hkv, D, bs = 8, 2, 128, 32
+    case = W.make_paged_case(83, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype)
+    rng = np.random.Generator(np.random.PCG64(84))
+
+    def gain(pos, total):
+        x = pos / max(total - 1, 1)
+        if profile == "ramp":
+            return 3.0 * x
+        return (1.0 if profile == "step16" else 2.5) * (x >= 0.6)
+
+    T = case["T"]
+    q = 0.3 * rng.standard_normal((T, Hq * D), dtype=np.float32) + 1.0
+    k_new = 0.3 * rng.standard_normal((T, Hkv * D), dtype=np.float32)
+    for s, (past, n) in enumerate(seqs):
+        total = past + n
+        g = np.array([gain(pos, total) for pos in range(total)], np.float32)
+        rows = 0.3 * rng.standard_normal((past, Hkv, D), dtype=np.float32) + g[:past, None, None]
+        for pos in range(past):
+            blk = case["block_indices"][case["block_indices_begins"][s] + pos // bs]
+            case["key_cache"][blk, :, pos % bs] = W.cache_rows_from_f32(rows[pos], cache_dtype)
+        t0 = case["subsequence_begins"][s]
+        k_new[t0:t0 + n] += g[past:, None]
+    case["q_store"], case["q"] = W.to_storage(q, q_dtype)
+    case["k_new_store"], case["k_new"] = W.to_storage(k_new, q_dtype)
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run()
+    assert path == "paged_mfma"
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    assert np.isfinite(out).all()
+    tol = 2e-2 if cache_dtype == W.BF16 else 1e-2
+    assert (np.abs(out - ref) <= tol * np.maximum(1.0, np.abs(ref))).all()
+    dev.free()
+
+
 @pytest.mark.parametrize("env", [{}, {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "10"},
                                  {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "1000"}, {"HIPATTN_MIXED_OVERLAP": "0"}])
 @pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.BF16, W.F16, 0), (W.F16, W.U8, 300), (W.BF16, W.BF16, 0)])
