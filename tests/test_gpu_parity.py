@@ -326,14 +326,15 @@ def test_paged_mixed_batch(hip, oracle, q_dtype, cache_dtype, window, heads):
 
 @pytest.mark.parametrize("q_dtype,cache_dtype", [(W.F16, W.F16), (W.BF16, W.F16), (W.F16, W.U8), (W.BF16, W.BF16)])
 @pytest.mark.parametrize("profile", ["ramp", "step16", "step40", "fall", "wide"])
-def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dtype, profile):
+@pytest.mark.parametrize("window", [0, 300])
+def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dtype, profile, window):
     """Chunks and decode tokens whose later keys score far above the earlier ones (see the dense
     test of the same name): the keys of every sequence, in the cache and among the new tokens, are
     rewritten so that their scores rise with the position."""
-    announce("paged growing scores", q_dtype, cache_dtype, profile)
+    announce("paged growing scores", q_dtype, cache_dtype, profile, window)
     seqs = [(0, 700), (900, 1), (1500, 1), (400, 300), (2000, 1), (63, 1)]
     Hq, Hkv, D, bs = 8, 2, 128, 32
-    case = W.make_paged_case(83, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype)
+    case = W.make_paged_case(83, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
     rng = np.random.Generator(np.random.PCG64(84))
 
     def gain(pos, total):
