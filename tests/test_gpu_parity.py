@@ -182,6 +182,28 @@ def test_sdpa_flash_scores_that_grow_along_the_keys(hip, oracle, dtype, profile,
     assert float(np.max(np.abs(out - ref) / np.maximum(1.0, np.abs(ref)))) <= tol
 
 
+@pytest.mark.parametrize("dtype", [W.F32, W.F16])
+@pytest.mark.parametrize("profile", ["ramp", "step40", "fall"])
+def test_sdpa_generic_scores_that_grow_along_the_keys(hip, oracle, dtype, profile):
+    announce("sdpa generic growing scores", dtype, profile)
+    B, Hq, Hkv, Lq, Lk, D = 1, 4, 2, 200, 700, 64
+    rng = np.random.Generator(np.random.PCG64(72))
+    gain = {"ramp": np.linspace(0.0, 4.0, Lk), "step40": np.where(np.arange(Lk) >= 400, 3.5, 0.0),
+            "fall": np.linspace(4.0, 0.0, Lk)}[profile].astype(np.float32)  # 8 nats per unit of gain
+    q = 0.3 * rng.standard_normal((B, Hq, Lq, D), dtype=np.float32) + 1.0
+    k = 0.3 * rng.standard_normal((B, Hkv, Lk, D), dtype=np.float32) + gain[None, None, :, None]
+    v = rng.standard_normal((B, Hkv, Lk, D), dtype=np.float32)
+    case = {"B": B, "Hq": Hq, "Hkv": Hkv, "Lq": Lq, "Lk": Lk, "D": D, "dtype": dtype}
+    for name, x in (("q", q), ("k", k), ("v", v)):
+        case[name + "_store"], case[name] = W.to_storage(x, dtype)
+    for causal in (False, True):
+        out, path = H.run_sdpa(hip, case, causal)
+        assert path == "sdpa_generic"
+        ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+        assert np.isfinite(out).all()
+        assert float(np.max(np.abs(out - ref) / np.maximum(1.0, np.abs(ref)))) <= TOL[dtype]
+
+
 def test_sdpa_scale_and_empty(hip, oracle):
     announce("sdpa scale/empty")
     case = W.make_sdpa_case(63, 1, 2, 1, 90, 90, 128, W.F16)
@@ -374,6 +396,12 @@ def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dt
         tol = {W.BF16: 3e-2, W.U8: 2e-2}.get(cache_dtype, 1e-2)
     err = np.abs(out - ref) / np.maximum(1.0, np.abs(ref))
     assert float(err.max()) <= tol
+    # the fp32 kernel that serves the shapes the MFMA kernels do not, on the same call
+    out_g, path_g = dev.run(flags=hip.PA_FORCE_GENERIC | hip.PA_SKIP_CACHE_WRITE)
+    assert path_g == "paged_generic"
+    assert np.isfinite(out_g).all()
+    # (its own error is below 1e-3; the rest is the 16-bit output type)
+    assert float((np.abs(out_g - ref) / np.maximum(1.0, np.abs(ref))).max()) <= (8e-3 if q_dtype == W.BF16 else 2e-3)
     dev.free()
 
 
