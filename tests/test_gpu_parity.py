@@ -405,6 +405,34 @@ def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dt
     dev.free()
 
 
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
+@pytest.mark.parametrize("mixed", [False, True])
+def test_paged_batch_of_thousands_of_sequences(hip, oracle, cache_dtype, mixed):
+    """More sequences than two rounds of the kernels' 64-ary search over the batch cover (4096),
+    some of them without a token, short contexts, so that most wavefronts cross many sequences."""
+    announce("paged thousands of sequences", cache_dtype, mixed)
+    rng = np.random.Generator(np.random.PCG64(85))
+    seqs = [(int(rng.integers(0, 70)), int(rng.choice([1, 1, 1, 1, 0]))) for _ in range(4500)]
+    if mixed:
+        seqs[7] = (100, 200)
+        seqs[2200] = (0, 77)
+        seqs[4499] = (300, 129)
+    else:
+        seqs = [(p, 1) for p, _ in seqs]
+    case = W.make_paged_case(86, seqs, 8, 2, 128, 32, W.F16, W.F16, cache_dtype)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run()
+    assert path == "paged_mfma"
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    assert np.isfinite(out).all()
+    tol = 1e-2 if cache_dtype == W.U8 else 2e-3
+    assert float((np.abs(out - ref) / np.maximum(1.0, np.abs(ref))).max()) <= tol
+    dev.free()
+
+
 @pytest.mark.parametrize("env", [{}, {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "10"},
                                  {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "1000"}, {"HIPATTN_MIXED_OVERLAP": "0"}])
 @pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.BF16, W.F16, 0), (W.F16, W.U8, 300), (W.BF16, W.BF16, 0)])
