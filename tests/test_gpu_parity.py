@@ -405,6 +405,26 @@ def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dt
     dev.free()
 
 
+def test_paged_pool_beyond_two_gib_and_long_contexts(hip, oracle):
+    """Caches of 2.7 GB each, so that most physical blocks lie beyond the reach of 32-bit byte
+    offsets, and contexts of up to 131072 tokens (4096 table entries, 2048 key tiles) for a decode
+    token and for a chunk."""
+    announce("paged large pool, long contexts")
+    seqs = [(131071, 1), (130000, 200), (100000, 1), (50, 1)]
+    case = W.make_paged_case(87, seqs, 8, 8, 128, 32, W.F16, W.F16, W.F16, spare_blocks=30000)
+    assert case["key_cache"].nbytes > (5 << 29) and int(case["block_indices"].max()) * 65536 > (1 << 31)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run()
+    assert path == "paged_mfma"
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    kc, vc = dev.caches()
+    assert np.array_equal(kc, okc) and np.array_equal(vc, ovc)
+    del kc, vc, okc, ovc
+    assert np.isfinite(out).all()
+    assert H.max_abs(out, ref) <= 2e-3
+    dev.free()
+
+
 @pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
 @pytest.mark.parametrize("mixed", [False, True])
 def test_paged_batch_of_thousands_of_sequences(hip, oracle, cache_dtype, mixed):
