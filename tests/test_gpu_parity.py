@@ -204,6 +204,30 @@ def test_sdpa_generic_scores_that_grow_along_the_keys(hip, oracle, dtype, profil
         assert float(np.max(np.abs(out - ref) / np.maximum(1.0, np.abs(ref)))) <= TOL[dtype]
 
 
+def test_sdpa_flash_tensors_beyond_two_gib(hip, oracle):
+    """Query and output tensors of 2^30 elements (2 GiB of bf16) and 65536 keys per head, causal:
+    rows spread over the tensor are compared with the oracle, each as one query row over the keys it
+    sees; every output element must have been written."""
+    announce("sdpa flash beyond 2 GiB")
+    B, Hq, Hkv, L, D = 1, 128, 8, 65536, 128
+    rng = np.random.Generator(np.random.PCG64(73))
+    period = 4096  # the query rows repeat with this period along the sequence (their positions do not)
+    q_st, q_val = W.to_storage(rng.standard_normal((B, Hq, period, D), dtype=np.float32), W.BF16)
+    k_st, k_val = W.to_storage(rng.standard_normal((B, Hkv, L, D), dtype=np.float32), W.BF16)
+    v_st, v_val = W.to_storage(rng.standard_normal((B, Hkv, L, D), dtype=np.float32), W.BF16)
+    case = {"B": B, "Hq": Hq, "Hkv": Hkv, "Lq": L, "Lk": L, "D": D, "dtype": W.BF16,
+            "q_store": np.tile(q_st, (1, 1, L // period, 1)), "k_store": k_st, "v_store": v_st}
+    assert case["q_store"].nbytes == 1 << 31
+    out, path = H.run_sdpa(hip, case, True)
+    assert path == "sdpa_flash_mfma"
+    assert np.isfinite(out).all()
+    for h, row in ((0, 0), (5, 4095), (64, 40000), (100, 12345), (127, 65408), (127, 65535)):
+        kvh = h // (Hq // Hkv)
+        ref = oracle.sdpa(q_val[:, h:h + 1, row % period:row % period + 1], k_val[:, kvh:kvh + 1, :row + 1],
+                          v_val[:, kvh:kvh + 1, :row + 1], causal=False)
+        assert H.max_abs(out[0, h, row], ref[0, 0, 0]) <= TOL[W.BF16], (h, row)
+
+
 def test_sdpa_scale_and_empty(hip, oracle):
     announce("sdpa scale/empty")
     case = W.make_sdpa_case(63, 1, 2, 1, 90, 90, 128, W.F16)
