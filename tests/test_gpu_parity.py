@@ -605,6 +605,14 @@ def test_paged_errors(hip):
         hip.paged_attention(desc, dev.q, None, None, dev.key_cache, dev.value_cache, dev.past_lens,
                             dev.subsequence_begins, dev.block_indices, dev.block_indices_begins, dev.out, small)
     assert e.value.status == hip.INVALID_ARGUMENT
+    # a call without tokens or without sequences does nothing, whatever the pointers are
+    for T, S in ((0, 2), (3, 0), (0, 0)):
+        empty = hip.PaDesc(W.F16, W.F16, W.F16, W.F16, 32, 8, 128, 32, case["num_blocks"], T, S, 0, 0, 0.0, 0, 0)
+        before = dev.out.download(np.uint16, (case["T"], 32 * 128))
+        assert hip.lib().hipattn_paged_attention(empty, None, None, None, None, None, None, None, None, None, None,
+                                                 None, 0, None) == hip.OK
+        assert hip.lib().hipattn_kv_cache_write(empty, None, None, None, None, None, None, None, None, None) == hip.OK
+        np.testing.assert_array_equal(before, dev.out.download(np.uint16, (case["T"], 32 * 128)))
     dev.free()
 
 
