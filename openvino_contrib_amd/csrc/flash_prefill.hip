@@ -572,13 +572,22 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0,
 // The loop of one wavefront.  t is the tile of this wavefront's group; [kv_lo, kv_hi) is the key
 // range of the workgroup (the union of both groups' ranges, kv_lo a multiple of 64).
 //
-// Phases, numbered from 0 and separated by workgroup barriers: group 0 computes the scores of
-// tile j in phase 2j, their softmax in phase 2j+1 and P V in phase 2j+2 (together with the
-// scores of tile j+1); group 1 does the same one phase later.  K(j) is therefore read in phases
-// 2j and 2j+1, V(j) in phases 2j+2 and 2j+3.  Load batch B(x) = {K(x+2), V(x+1)} goes into the
-// ring stages of K(x-1) and V(x-2); every wavefront issues its rows of B(x) in a vector phase
-// (group 0 in phase 2x+1, group 1 in phase 2x), and at each barrier waits for all of its loads
-// except the latest batch, which puts B(x) in LDS two phases before its first use.
+// Phases, numbered from 0: group 0 computes the scores of tile j in phase 2j, their softmax in
+// phase 2j+1 and P V in phase 2j+2 (together with the scores of tile j+1); group 1 does the same
+// one phase later.  K(j) is therefore read in phases 2j and 2j+1, V(j) in phases 2j+2 and 2j+3.
+// Load batch B(x) = {K(x+2), V(x+1)} goes into the ring stages of K(x-1) and V(x-2); every
+// wavefront issues its rows of B(x) in a vector phase (group 0 in phase 2x+1, group 1 in phase
+// 2x).
+//
+// One workgroup barrier per tile: before every even phase, i.e. for group 0 between its vector
+// and its matrix phase, for group 1 behind its matrix phase; at it a wavefront waits for all of
+// its loads except the latest batch.  That is all the data needs.  What is read from phase 2j+2
+// on -- K(j+1) and V(j) -- was issued by group 0 in phase 2j-1 and by group 1 in phase 2j-2, and
+// at the barrier before phase 2j+2 neither batch is the issuing wavefront's latest any more.  What
+// is overwritten by loads issued from phase 2j+2 on -- the stages of K(j) and V(j-1) -- was last
+// read in phase 2j+1.  Between the barriers each group runs one matrix and one vector phase, in
+// opposite order, so that the matrix core and the vector units are both in use; the odd phase
+// boundaries are not enforced, the two groups only drift by what their phases differ in length.
 template <bool kBf16, bool kU8 = false, bool kPaged = true>
 __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
     static_assert(kPaged || !kU8, "dense K/V are 16-bit");
@@ -882,7 +891,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         // the first instruction after it): otherwise the other group's instruction stream, which
         // never stalls for long, keeps this wavefront's MFMAs from issuing
         __builtin_amdgcn_s_setprio(3);
-        phase_barrier(recent);
+        if (group == 0) phase_barrier(recent);  // (group 1 passes from its vector phase straight into its matrix phase)
         FLASH_STAMP(clk, 3);
         // ---- matrix phase
         // fragment addresses of this tile: per-lane offset + stage address, so that every read is
@@ -917,7 +926,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             asm volatile("" : "+s"(fill_k), "+s"(fill_v));
         }
         asm volatile("" : "+s"(i_kn), "+s"(i_vc), "+s"(i_kf), "+s"(i_vf));
-        phase_barrier(recent);
+        if (group == 1) phase_barrier(recent);
         FLASH_STAMP(clk, 6);
     };
     for (int j = 0; j < n - 1; j++) two_phases(j, false);

@@ -439,12 +439,12 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
     if (tid == 0 && p.overlap) {
         // Compute-unit time of the two parts, in microseconds, as measured with both running:
         // a compute unit of the decode kernel streams about 33 GB/s of fp16 cache (u8: 24 GB/s),
-        // one of the flash kernel does a 128-row x 64-key tile of one head in about 1.2 us
-        // (u8 caches, dequantised on the way: 1.7 us).  Each part gets compute units in
+        // one of the flash kernel does a 128-row x 64-key tile of one head in about 1.1 us
+        // (u8 caches, dequantised on the way: 1.4 us).  Each part gets compute units in
         // proportion to its work, so that both end together.
         const bool u8 = p.cache_dtype == HIPATTN_U8;
         const float decode_us = (float)total_blk * p.num_heads_kv * (u8 ? 8704.0f / 24000.0f : 16384.0f / 33000.0f) * p.overlap_share;
-        const float prefill_us = total_keys * p.num_heads_q * (u8 ? 1.7f : 1.2f);
+        const float prefill_us = total_keys * p.num_heads_q * (u8 ? 1.4f : 1.1f);
         const int cus = p.num_waves >> 3;
         int mine = (int)ceilf(cus * decode_us / fmaxf(decode_us + prefill_us, 1.0f));
         mine = max(1, min(mine, cus));
