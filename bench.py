@@ -81,8 +81,7 @@ def time_steps(hip, fn, steps, warmup):
 
 
 def bench_paged(hip, case, steps, warmup, name):
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import helpers as H
+    from openvino_contrib_amd import device_case as H
     from openvino_contrib_amd import workloads as W
 
     dev = H.PagedDeviceCase(hip, case)
@@ -255,10 +254,16 @@ def main():
         # What the device sustains on v_mfma_f32_32x32x16_bf16 alone, and at which shader clock, with
         # random and with all-zero operands (the power an MFMA draws follows the bits that toggle).
         import ctypes
+        from openvino_contrib_amd import build as hip_build
+        if not os.path.exists(hip_build.YARDSTICK_LIB_PATH):
+            sys.exit("bench.py: %s is missing (python -m openvino_contrib_amd.build)" % hip_build.YARDSTICK_LIB_PATH)
+        yard = ctypes.CDLL(hip_build.YARDSTICK_LIB_PATH)
         out = {"workload": "mfma", "peak_tflops": MFMA_BF16_PEAK_TFLOPS}
         for name, zero in (("random_operands", 0), ("zero_operands", 1)):
             tf, ghz = ctypes.c_double(), ctypes.c_double()
-            hip.check(hip.lib().hipattn_mfma_yardstick(zero, max(args.steps, 50), ctypes.byref(tf), ctypes.byref(ghz), None))
+            rc = yard.mfma_yardstick(zero, max(args.steps, 50), ctypes.byref(tf), ctypes.byref(ghz))
+            if rc != 0:
+                sys.exit("bench.py: mfma_yardstick failed with HIP error %d" % rc)
             out[name] = {"tflops": tf.value, "shader_ghz": ghz.value, "frac_of_peak": tf.value / MFMA_BF16_PEAK_TFLOPS}
         print(json.dumps(out))
         return

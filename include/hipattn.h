@@ -24,7 +24,7 @@ extern "C" {
 #endif
 
 #define HIPATTN_VERSION_MAJOR 0
-#define HIPATTN_VERSION_MINOR 1
+#define HIPATTN_VERSION_MINOR 2
 
 typedef enum hipattn_status {
     HIPATTN_OK = 0,
@@ -85,12 +85,6 @@ hipattn_status hipattn_memcpy_d2h_async(void* host_dst, const void* device_src, 
 hipattn_status hipattn_memcpy_d2d_async(void* device_dst, const void* device_src, size_t bytes, hipattn_stream stream);
 /* byte fill done by a kernel (safe to record into a captured graph) */
 hipattn_status hipattn_fill_async(void* device_dst, int byte_value, size_t bytes, hipattn_stream stream);
-/* Diagnostic without a counterpart in the reference: the rate (TFLOP/s) and shader clock (GHz) the
- * current device sustains on register-fed v_mfma_f32_32x32x16_bf16 alone, with all-zero or with
- * random operands; the yardstick for the MFMA-bound kernels, as a plain copy is for the
- * HBM-bound ones.  Runs 2 x launches kernels (half of them untimed), allocates and frees its own
- * few KB, and synchronises the stream. */
-hipattn_status hipattn_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz, hipattn_stream stream);
 
 hipattn_status hipattn_event_create(hipattn_event* event);
 hipattn_status hipattn_event_destroy(hipattn_event event);
@@ -126,6 +120,22 @@ hipattn_status hipattn_sdpa_workspace_size(const hipattn_sdpa_desc* desc, size_t
 hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const void* k, const void* v, void* out,
                             void* workspace, size_t workspace_bytes, hipattn_stream stream);
 
+/* The same operator with its optional attention_mask input, which the reference executes as the
+ * Add / Select nodes of the decomposition (src/ops/add.cpp:17-43, src/ops/select.cpp:50-91).
+ * The mask is addressed as [batch, num_heads_q, len_q, len_kv] through strides in elements; a
+ * stride of 0 broadcasts that dimension.  dtype F32 / F16 / BF16: the value is added to the
+ * scaled score; dtype U8: boolean, nonzero = the key takes part, zero = probability zero.  As the
+ * operator specifies, the mask is ignored when desc->causal is set.  A query row whose keys are
+ * all masked out yields zeros.  mask_desc and mask are both NULL or both set. */
+typedef struct hipattn_mask_desc {
+    hipattn_dtype dtype;
+    int64_t stride[4];
+} hipattn_mask_desc;
+
+hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q, const void* k, const void* v,
+                                   const hipattn_mask_desc* mask_desc, const void* mask, void* out, void* workspace,
+                                   size_t workspace_bytes, hipattn_stream stream);
+
 /* ---- PagedAttentionExtension --------------------------------------------------------
  * No counterpart in the reference (its only KV-cache mechanism is the contiguous
  * variable state, src/cuda_variable_state.hpp:135-160, src/ops/read_value.cpp:31-72,
@@ -151,25 +161,29 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * (all of 0..p when sliding_window <= 0).
  * All index arrays live in device memory and are only read there; the split of the work is
  * planned on the device.  max_context_len (>= max_s(past_lens[s] + q_len[s])) is advisory.
- * A sequence may contribute no token to a batch, with one exception: a batch with
- * num_tokens == num_seqs is taken to hold exactly one token per sequence (pure decode: the host
- * cannot see the lengths, and a decode step should not pay for a launch that finds nothing to
- * do), unless HIPATTN_PA_ANY_LENGTHS says otherwise.
+ * A sequence may contribute any number of tokens to a batch, none included.  A batch with
+ * num_tokens == num_seqs is planned per token (the host cannot see the lengths, and a decode
+ * step should not pay for a prefill launch that finds nothing to do): every token is a decode
+ * row with its own context length, whichever sequence it belongs to, so the result is right
+ * for any split of the tokens over the sequences; HIPATTN_PA_ANY_LENGTHS only changes how fast
+ * such a batch runs when it does hold long multi-token sequences.
+ * A single-token row with nothing to attend (an empty block table) gets an output row of zeros.
+ * Block ids outside [0, num_blocks) in a table: the decode and the shape-generic kernels skip
+ * those blocks (probability zero); the MFMA chunked-prefill kernel redirects them to a valid
+ * block, so reads stay inside the cache and the affected rows are unspecified.
  * A mixed batch (single-token and multi-token sequences) with decode_waves == 0 runs its two
  * parts side by side: the call forks from `stream` onto a side stream that the library keeps per
  * device (created by the first such call, default priority, never destroyed) and joins before it
  * returns, so `stream` order is all the caller has to know, also under stream capture (make the
  * first such call on a device outside a capture: creating a stream is not a capturable operation).  The
- * environment variable HIPATTN_MIXED_OVERLAP=0 switches that off. */
+ * option "mixed_overlap" = 0 (hipattn_set_option) switches that off. */
 enum {
     HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */
     HIPATTN_PA_FORCE_GENERIC = 2,    /* use the shape-generic kernels (testing aid) */
-    HIPATTN_PA_ANY_LENGTHS = 8,      /* num_tokens == num_seqs does not mean one token per sequence
-                                        here (a batch with empty sequences beside longer ones) */
-    HIPATTN_PA_TRACE_WAVES = 4       /* diagnostic: the decode kernel leaves, in the last
-                                        decode_waves * 32 bytes of the workspace, four int64 per
-                                        wavefront: entry, first block consumed, exit (100 MHz
-                                        ticks) and units of work */
+    HIPATTN_PA_ANY_LENGTHS = 8       /* performance hint for a batch with num_tokens == num_seqs that
+                                        holds multi-token sequences beside empty ones: send those to
+                                        the chunked-prefill kernel instead of treating each of their
+                                        tokens as a decode row */
 };
 
 typedef struct hipattn_pa_desc {
@@ -214,6 +228,19 @@ size_t hipattn_cache_row_bytes(hipattn_dtype cache_dtype, int head_dim);
  * kernel, or the split-context decode kernel when the batch has decode sequences), on the
  * call's stream.  Pass NULLs to switch it off. */
 hipattn_status hipattn_profile_dominant_kernel(hipattn_event before, hipattn_event after);
+
+/* Process-wide schedule options (no reference counterpart; the reference's knobs are OpenVINO
+ * properties, src/cuda_config.cpp:20-79).  value < 0 restores the default.  Names:
+ *   "mixed_overlap"               1 (default): the decode part of a mixed batch runs beside the
+ *                                 chunks' kernel; 0: one kernel after the other
+ *   "mixed_decode_share_percent"  scales the compute units the plan gives the decode part (100)
+ *   "decode_switch_cost"          block-times charged per (sequence, kv head) start when the decode
+ *                                 work is cut into equal pieces (3)
+ *   "decode_dyn_pieces_per_wave"  on-demand pieces per wavefront for the last quarter of the
+ *                                 decode work (0 = none)
+ * HIPATTN_<NAME IN CAPITALS> in the environment gives an option its initial value; the
+ * environment is read once per process. */
+hipattn_status hipattn_set_option(const char* name, int value);
 
 /* Name of the kernel path the last attention call on this thread dispatched to
  * ("flash_mfma", "generic", "decode_mfma+merge", ...).  Diagnostic only. */

@@ -20,7 +20,6 @@ SOURCES = [
     "attention_generic.hip",
     "paged_decode.hip",
     "flash_prefill.hip",
-    "yardstick.hip",
 ]
 
 HIPCC_FLAGS = [
@@ -73,6 +72,18 @@ def build_library(verbose=False, extra_flags=(), jobs=4):
     return LIB_PATH
 
 
+YARDSTICK_LIB_PATH = os.path.join(CSRC, "bench", "libmfma_yardstick.so")
+
+
+def build_bench_tools():
+    """The MFMA yardstick of bench.py --workload mfma: a library of its own, not part of libhipattn."""
+    cmd = [hipcc()] + HIPCC_FLAGS + ["-shared", os.path.join(CSRC, "bench", "mfma_yardstick.hip"), "-o", YARDSTICK_LIB_PATH]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on mfma_yardstick.hip:\n%s" % r.stderr[-4000:])
+    return YARDSTICK_LIB_PATH
+
+
 PLUGIN_LIB_PATH = os.path.join(CSRC, "libhip_plugin.so")
 PLUGIN_SOURCES = ["plugin/ops.cpp", "plugin/plugin.cpp", "plugin/c_api.cpp"]
 
@@ -95,3 +106,4 @@ def build_plugin():
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_plugin())
+    print(build_bench_tools())

@@ -16,7 +16,6 @@ OK, INVALID_ARGUMENT, UNSUPPORTED, WORKSPACE_TOO_SMALL, HIP_ERROR, NO_DEVICE = r
 F32, F16, BF16, U8 = 0, 1, 2, 3
 PA_SKIP_CACHE_WRITE = 1
 PA_FORCE_GENERIC = 2
-PA_TRACE_WAVES = 4
 PA_ANY_LENGTHS = 8
 
 DTYPE_BYTES = {F32: 4, F16: 2, BF16: 2, U8: 1}
@@ -51,6 +50,13 @@ class SdpaDesc(ctypes.Structure):
         ("head_dim", ctypes.c_int),
         ("causal", ctypes.c_int),
         ("scale", ctypes.c_float),
+    ]
+
+
+class MaskDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int),
+        ("stride", ctypes.c_int64 * 4),
     ]
 
 
@@ -98,7 +104,6 @@ SYMBOLS = {
     "hipattn_memcpy_d2h_async": (_i, [_vp, _vp, _sz, _vp]),
     "hipattn_memcpy_d2d_async": (_i, [_vp, _vp, _sz, _vp]),
     "hipattn_fill_async": (_i, [_vp, _i, _sz, _vp]),
-    "hipattn_mfma_yardstick": (_i, [_i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), _vp]),
     "hipattn_event_create": (_i, [_P(_vp)]),
     "hipattn_event_destroy": (_i, [_vp]),
     "hipattn_event_record": (_i, [_vp, _vp]),
@@ -106,8 +111,10 @@ SYMBOLS = {
     "hipattn_event_elapsed_ms": (_i, [_vp, _vp, _P(_f)]),
     "hipattn_sdpa_workspace_size": (_i, [_P(SdpaDesc), _P(_sz)]),
     "hipattn_sdpa": (_i, [_P(SdpaDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "hipattn_sdpa_masked": (_i, [_P(SdpaDesc), _vp, _vp, _vp, _P(MaskDesc), _vp, _vp, _vp, _sz, _vp]),
     "hipattn_paged_attention_workspace_size": (_i, [_P(PaDesc), _P(_sz)]),
     "hipattn_paged_attention": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "hipattn_set_option": (_i, [ctypes.c_char_p, _i]),
     "hipattn_kv_cache_write": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "hipattn_cache_row_bytes": (_sz, [_i, _i]),
     "hipattn_last_kernel_path": (ctypes.c_char_p, []),
@@ -259,6 +266,14 @@ def sdpa(desc, q, k, v, out, workspace=None, stream=None):
                              _h(stream)))
 
 
+def sdpa_masked(desc, q, k, v, mask_dtype, mask_strides, mask, out, workspace=None, stream=None):
+    """SDPA with an attention mask (DeviceBuffer) addressed as [batch, head, query, key] by strides in elements."""
+    md = MaskDesc(mask_dtype, (ctypes.c_int64 * 4)(*mask_strides))
+    check(lib().hipattn_sdpa_masked(ctypes.byref(desc), q.ptr, k.ptr, v.ptr, ctypes.byref(md), mask.ptr, out.ptr,
+                                    workspace.ptr if workspace else None, workspace.nbytes if workspace else 0,
+                                    _h(stream)))
+
+
 def paged_attention_workspace_size(desc):
     n = _sz(0)
     check(lib().hipattn_paged_attention_workspace_size(ctypes.byref(desc), ctypes.byref(n)))
@@ -271,6 +286,11 @@ def paged_attention(desc, q, k_new, v_new, key_cache, value_cache, past_lens, su
         ctypes.byref(desc), q.ptr, k_new.ptr if k_new else None, v_new.ptr if v_new else None, key_cache.ptr,
         value_cache.ptr, past_lens.ptr, subsequence_begins.ptr, block_indices.ptr, block_indices_begins.ptr,
         out.ptr, workspace.ptr if workspace else None, workspace.nbytes if workspace else 0, _h(stream)))
+
+
+def set_option(name, value):
+    """Process-wide schedule option (see include/hipattn.h); value < 0 restores the default."""
+    check(lib().hipattn_set_option(name.encode(), int(value)))
 
 
 def kv_cache_write(desc, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins, block_indices,

@@ -14,12 +14,32 @@ constexpr int kGenericMaxD = 512;
 constexpr int kGenericSlots = kGenericMaxD / 64;
 constexpr int kWavesPerBlock = 4;
 
+// No additive term on the scores.
+struct NoBias {
+    __device__ __forceinline__ float operator()(int) const { return 0.0f; }
+};
+
+// One row of an attention mask: element j at row + j * stride (stride 0: broadcast over the keys).
+// Boolean masks (u8, nonzero = the key takes part) become 0 / -inf; float masks are added to the
+// scaled scores, as ScaledDotProductAttention specifies.
+struct MaskRow {
+    const uint8_t* row;
+    int64_t stride;  // elements
+    int dtype;       // HIPATTN_F32 / F16 / BF16, or HIPATTN_U8 for boolean
+    __device__ __forceinline__ float operator()(int j) const {
+        if (dtype == HIPATTN_U8) return row[j * stride] ? 0.0f : -INFINITY;
+        return load_scalar(row, j * stride, dtype);
+    }
+};
+
 // Attend one query row to keys [j0, j1).  q_lds holds the row in fp32; KV yields row
-// pointers.  Every lane of the wavefront must call this; the result for head-dim slot
-// d = lane + 64 * i is returned in o[i], already normalised.
-template <typename KV>
-__device__ __forceinline__ void attend_row_wave(const float* q_lds, const KV& kv, int j0, int j1, int D, float scale,
-                                                float (&o)[kGenericSlots]) {
+// pointers and says which keys exist (a key in a block outside the cache has probability zero);
+// bias(j) is added to the scaled score of key j.  Every lane of the wavefront must call this; the
+// result for head-dim slot d = lane + 64 * i is returned in o[i], already normalised.  A row that
+// can attend nothing (empty range, every key masked with -inf) yields zeros.
+template <typename KV, typename Bias>
+__device__ __forceinline__ void attend_row_wave(const float* q_lds, const KV& kv, const Bias& bias, int j0, int j1, int D,
+                                                float scale, float (&o)[kGenericSlots]) {
     const int lane = threadIdx.x & 63;
     float m = -INFINITY, l = 0.0f;
 #pragma unroll
@@ -28,15 +48,16 @@ __device__ __forceinline__ void attend_row_wave(const float* q_lds, const KV& kv
     for (int base = j0; base < j1; base += 64) {
         const int j = base + lane;
         float s = -INFINITY;
-        if (j < j1) {
+        if (j < j1 && kv.exists(j)) {
             const uint8_t* krow = kv.k_row(j);
             float acc = 0.0f;
             for (int d = 0; d < D; d++) acc = fmaf(q_lds[d], load_cache_elem(krow, d, kv.dtype), acc);
-            s = acc * c;
+            s = fmaf(acc, c, bias(j) * kLog2e);
         }
         const float m_new = fmaxf(m, wave_max(s));
+        if (m_new == -INFINITY) continue;  // nothing attended so far (wave-uniform)
         const float alpha = fast_exp2(m - m_new);  // exp2(-inf) = 0 on the first tile
-        const float pj = (j < j1) ? fast_exp2(s - m_new) : 0.0f;
+        const float pj = (s != -INFINITY) ? fast_exp2(s - m_new) : 0.0f;
         l = l * alpha + wave_sum(pj);
         m = m_new;
 #pragma unroll
@@ -44,6 +65,7 @@ __device__ __forceinline__ void attend_row_wave(const float* q_lds, const KV& kv
         const int n = min(64, j1 - base);
         for (int jj = 0; jj < n; jj++) {
             const float pb = __shfl(pj, jj, 64);
+            if (pb == 0.0f) continue;  // (wave-uniform) masked keys may be unreadable or hold anything
             const uint8_t* vrow = kv.v_row(base + jj);
 #pragma unroll
             for (int i = 0; i < kGenericSlots; i++) {
@@ -62,6 +84,7 @@ struct DenseKV {
     const uint8_t* v;
     int64_t row_bytes;
     int dtype;
+    __device__ __forceinline__ bool exists(int) const { return true; }
     __device__ __forceinline__ const uint8_t* k_row(int j) const { return k + j * row_bytes; }
     __device__ __forceinline__ const uint8_t* v_row(int j) const { return v + j * row_bytes; }
 };
@@ -76,10 +99,13 @@ struct PagedKV {
     int block_size;
     int dtype;
     int num_blocks;
+    // a block id outside the cache: its keys are skipped (probability zero), as the decode kernel does
+    __device__ __forceinline__ bool exists(int j) const {
+        const int pb = blocks[j / block_size];
+        return pb >= 0 && pb < num_blocks;
+    }
     __device__ __forceinline__ int64_t off(int j) const {
-        // a block id outside the cache is clamped: the result is unspecified but no read leaves the cache
-        const int pb = min(max(blocks[j / block_size], 0), num_blocks - 1);
-        return (int64_t)pb * block_stride + head_off + (int64_t)(j % block_size) * row_bytes;
+        return (int64_t)blocks[j / block_size] * block_stride + head_off + (int64_t)(j % block_size) * row_bytes;
     }
     __device__ __forceinline__ const uint8_t* k_row(int j) const { return k + off(j); }
     __device__ __forceinline__ const uint8_t* v_row(int j) const { return v + off(j); }
@@ -104,7 +130,14 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void sdpa_generic_kernel(SdpaP
     DenseKV kv{(const uint8_t*)p.k + kv_off, (const uint8_t*)p.v + kv_off, rb, p.dtype};
     const int j1 = p.causal ? min(i + 1, p.len_kv) : p.len_kv;
     float o[kGenericSlots];
-    attend_row_wave(q_lds[wave], kv, 0, j1, D, p.scale, o);
+    if (p.mask && !p.causal) {  // (the operator ignores attention_mask when causal is set)
+        const int64_t moff = (int64_t)b * p.mask_stride[0] + (int64_t)h * p.mask_stride[1] + (int64_t)i * p.mask_stride[2];
+        const MaskRow bias{(const uint8_t*)p.mask + moff * (p.mask_dtype == HIPATTN_U8 ? 1 : dtype_bytes(p.mask_dtype)),
+                           p.mask_stride[3], p.mask_dtype};
+        attend_row_wave(q_lds[wave], kv, bias, 0, j1, D, p.scale, o);
+    } else {
+        attend_row_wave(q_lds[wave], kv, NoBias{}, 0, j1, D, p.scale, o);
+    }
 #pragma unroll
     for (int s = 0; s < kGenericSlots; s++) {
         const int d = lane + 64 * s;
@@ -156,7 +189,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void paged_generic_kernel(Page
     int j0 = 0;
     if (p.sliding_window > 0 && pos - p.sliding_window + 1 > 0) j0 = pos - p.sliding_window + 1;
     float o[kGenericSlots];
-    attend_row_wave(q_lds[wave], kv, j0, j1, D, p.scale, o);
+    attend_row_wave(q_lds[wave], kv, NoBias{}, j0, j1, D, p.scale, o);
 #pragma unroll
     for (int sl = 0; sl < kGenericSlots; sl++) {
         const int d = lane + 64 * sl;

@@ -3,11 +3,13 @@
 // v_mfma_f32_32x32x16_bf16, and at which shader clock?  The published peak (2.5 PFLOP/s dense
 // bf16) assumes 2.4 GHz; under load the clock is set by the power management, and the power an
 // MFMA draws depends on how many operand bits toggle, so the answer differs between all-zero
-// operands and random ones.  Not part of the attention path; used by bench.py --workload mfma.
+// operands and random ones.  Not part of the attention path and not part of libhipattn: built into a
+// library of its own (libmfma_yardstick.so) that only bench.py --workload mfma loads.
 #include <vector>
 
+#include <hip/hip_runtime.h>
+
 #include "device_common.hpp"
-#include "kernels.hpp"
 
 namespace hipattn {
 
@@ -60,8 +62,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 }  // namespace
 
-// Runs the kernel `launches` times after as many untimed ones (clock ramp); synchronises the stream.
-hipError_t run_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz, hipStream_t stream) {
+// Runs the kernel `launches` times after as many untimed ones (clock ramp) on the default stream and
+// synchronises it.
+static hipError_t run_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz) {
+    hipStream_t stream = nullptr;
     int dev = 0, cus = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
@@ -108,3 +112,10 @@ hipError_t run_mfma_yardstick(int zero_data, int launches, double* tflops, doubl
 }
 
 }  // namespace hipattn
+
+// Returns 0 on success, a hipError_t value otherwise.
+extern "C" __attribute__((visibility("default"))) int mfma_yardstick(int zero_data, int launches, double* tflops,
+                                                                     double* shader_ghz) {
+    if (!tflops || !shader_ghz || launches < 1 || launches > 100000) return (int)hipErrorInvalidValue;
+    return (int)hipattn::run_mfma_yardstick(zero_data, launches, tflops, shader_ghz);
+}

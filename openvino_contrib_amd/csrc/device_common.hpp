@@ -103,6 +103,10 @@ __device__ __forceinline__ void store_scalar(void* base, int64_t idx, int dtype,
     }
 }
 
+__host__ __device__ __forceinline__ int dtype_bytes(int dtype) {
+    return dtype == HIPATTN_F32 ? 4 : (dtype == HIPATTN_U8 ? 1 : 2);
+}
+
 __host__ __device__ __forceinline__ int64_t cache_row_bytes(int cache_dtype, int head_dim) {
     switch (cache_dtype) {
         case HIPATTN_F32: return 4 * (int64_t)head_dim;

@@ -76,6 +76,8 @@ hipattn_status validate_pa(const hipattn_pa_desc* d, bool need_q) {
     if (d->head_dim > 512) return fail(HIPATTN_UNSUPPORTED, "paged_attention: head_dim %d > 512", d->head_dim);
     if (d->num_blocks < 0 || d->num_tokens < 0 || d->num_seqs < 0 || d->max_context_len < 0)
         return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: negative extent");
+    if (d->num_blocks == 0 && d->num_tokens > 0 && d->num_seqs > 0)
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: %d tokens but a cache of no blocks", d->num_tokens);
     if (d->decode_waves < 0 || d->decode_waves > 65536)
         return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: decode_waves %d outside [0, 65536]", d->decode_waves);
     if (d->cache_dtype == HIPATTN_U8 && d->head_dim % 8)
@@ -124,7 +126,6 @@ hipattn::PagedParams make_paged_params(const hipattn_pa_desc* d) {
     p.scale = resolve_scale(d->scale, d->head_dim);
     p.num_waves = d->decode_waves > 0 ? d->decode_waves : 0;
     p.any_lengths = (d->flags & HIPATTN_PA_ANY_LENGTHS) ? 1 : 0;
-    p.wave_trace = (d->flags & HIPATTN_PA_TRACE_WAVES) ? reinterpret_cast<int64_t*>(1) : nullptr;  // placed by the plan
     return p;
 }
 
@@ -154,6 +155,12 @@ HIPATTN_EXPORT hipattn_status hipattn_profile_dominant_kernel(hipattn_event befo
         return fail(HIPATTN_INVALID_ARGUMENT, "profile_dominant_kernel: pass two events or two NULLs");
     g_probe.before = reinterpret_cast<hipEvent_t>(before);
     g_probe.after = reinterpret_cast<hipEvent_t>(after);
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_set_option(const char* name, int value) {
+    if (!name) return fail(HIPATTN_INVALID_ARGUMENT, "set_option: null name");
+    if (!hipattn::set_option(name, value)) return fail(HIPATTN_INVALID_ARGUMENT, "set_option: no option named '%s'", name);
     return HIPATTN_OK;
 }
 
@@ -285,14 +292,6 @@ HIPATTN_EXPORT hipattn_status hipattn_fill_async(void* device_dst, int byte_valu
     return HIPATTN_OK;
 }
 
-HIPATTN_EXPORT hipattn_status hipattn_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz,
-                                                     hipattn_stream stream) {
-    if (!tflops || !shader_ghz) return fail(HIPATTN_INVALID_ARGUMENT, "mfma_yardstick: null output");
-    if (launches < 1 || launches > 100000) return fail(HIPATTN_INVALID_ARGUMENT, "mfma_yardstick: launches out of range");
-    HIP_TRY(hipattn::run_mfma_yardstick(zero_data, launches, tflops, shader_ghz, as_stream(stream)));
-    return HIPATTN_OK;
-}
-
 HIPATTN_EXPORT hipattn_status hipattn_event_create(hipattn_event* event) {
     if (!event) return fail(HIPATTN_INVALID_ARGUMENT, "event_create: null output");
     hipEvent_t e;
@@ -325,12 +324,21 @@ HIPATTN_EXPORT hipattn_status hipattn_sdpa_workspace_size(const hipattn_sdpa_des
     return validate_sdpa(desc);
 }
 
-HIPATTN_EXPORT hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const void* k, const void* v,
-                                           void* out, void* workspace, size_t workspace_bytes,
-                                           hipattn_stream stream) {
+HIPATTN_EXPORT hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q, const void* k,
+                                                  const void* v, const hipattn_mask_desc* mask_desc, const void* mask,
+                                                  void* out, void* workspace, size_t workspace_bytes,
+                                                  hipattn_stream stream) {
     (void)workspace;
     (void)workspace_bytes;
     if (hipattn_status st = validate_sdpa(desc)) return st;
+    if ((mask == nullptr) != (mask_desc == nullptr))
+        return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: a mask needs a mask descriptor and the other way round");
+    if (mask_desc) {
+        if (!is_float_dtype(mask_desc->dtype) && mask_desc->dtype != HIPATTN_U8)
+            return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: mask dtype %d (f32, f16, bf16, or u8 for boolean)", mask_desc->dtype);
+        for (int i = 0; i < 4; i++)
+            if (mask_desc->stride[i] < 0) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: negative mask stride");
+    }
     const int64_t out_elems = (int64_t)desc->batch * desc->num_heads_q * desc->len_q * desc->head_dim;
     if (out_elems == 0) return HIPATTN_OK;
     if (!q || !out) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa: null q/out");
@@ -349,7 +357,12 @@ HIPATTN_EXPORT hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const 
     p.head_dim = desc->head_dim;
     p.causal = desc->causal != 0;
     p.scale = resolve_scale(desc->scale, desc->head_dim);
-    if (hipattn::sdpa_flash_supported(p)) {
+    if (mask && !p.causal) {  // the operator ignores attention_mask when causal is set
+        p.mask = mask;
+        p.mask_dtype = mask_desc->dtype;
+        for (int i = 0; i < 4; i++) p.mask_stride[i] = mask_desc->stride[i];
+    }
+    if (!p.mask && hipattn::sdpa_flash_supported(p)) {
         g_kernel_path = "sdpa_flash_mfma";
         HIP_TRY(hipattn::launch_sdpa_flash(p, as_stream(stream), g_probe));
     } else {
@@ -357,6 +370,12 @@ HIPATTN_EXPORT hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const 
         HIP_TRY(hipattn::launch_sdpa_generic(p, as_stream(stream)));
     }
     return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const void* k, const void* v,
+                                           void* out, void* workspace, size_t workspace_bytes,
+                                           hipattn_stream stream) {
+    return hipattn_sdpa_masked(desc, q, k, v, nullptr, nullptr, out, workspace, workspace_bytes, stream);
 }
 
 // ------------------------------------------------------------------- paged attention
@@ -386,12 +405,14 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention_workspace_size(const hipat
     return HIPATTN_OK;
 }
 
-HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* desc, const void* q, const void* k_new,
-                                                      const void* v_new, void* key_cache, void* value_cache,
-                                                      const int32_t* past_lens, const int32_t* subsequence_begins,
-                                                      const int32_t* block_indices,
-                                                      const int32_t* block_indices_begins, void* out, void* workspace,
-                                                      size_t workspace_bytes, hipattn_stream stream) {
+namespace {
+// Body of both paged-attention entry points.  static_scratch: the workspace is the library's
+// static device array and nothing may be allocated or created on the way.
+hipattn_status paged_attention_impl(const hipattn_pa_desc* desc, const void* q, const void* k_new, const void* v_new,
+                                    void* key_cache, void* value_cache, const int32_t* past_lens,
+                                    const int32_t* subsequence_begins, const int32_t* block_indices,
+                                    const int32_t* block_indices_begins, void* out, void* workspace,
+                                    size_t workspace_bytes, hipattn_stream stream, bool static_scratch) {
     if (hipattn_status st = validate_pa(desc, true)) return st;
     if (desc->num_tokens == 0 || desc->num_seqs == 0) return HIPATTN_OK;
     if (!q || !out || !key_cache || !value_cache || !past_lens || !subsequence_begins || !block_indices ||
@@ -410,8 +431,10 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* des
     p.block_indices = block_indices;
     p.block_indices_begins = block_indices_begins;
     p.out = out;
+    p.no_side_stream = static_scratch ? 1 : 0;  // (creating the side stream of a mixed batch allocates)
     if (!(desc->flags & HIPATTN_PA_FORCE_GENERIC) && hipattn::paged_fast_supported(p)) {
         const size_t need = hipattn::paged_fast_workspace_bytes(p);
+        (void)static_scratch;
         if (need > 0 && (!workspace || workspace_bytes < need))
             return fail(HIPATTN_WORKSPACE_TOO_SMALL, "paged_attention: workspace %zu bytes, need %zu", workspace_bytes,
                         need);
@@ -426,4 +449,15 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* des
         HIP_TRY(hipattn::launch_paged_generic(p, as_stream(stream)));
     }
     return HIPATTN_OK;
+}
+}  // namespace
+
+HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* desc, const void* q, const void* k_new,
+                                                      const void* v_new, void* key_cache, void* value_cache,
+                                                      const int32_t* past_lens, const int32_t* subsequence_begins,
+                                                      const int32_t* block_indices,
+                                                      const int32_t* block_indices_begins, void* out, void* workspace,
+                                                      size_t workspace_bytes, hipattn_stream stream) {
+    return paged_attention_impl(desc, q, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins,
+                                block_indices, block_indices_begins, out, workspace, workspace_bytes, stream, false);
 }

@@ -64,6 +64,11 @@ struct SdpaParams {
     int head_dim;
     int causal;
     float scale;  // already resolved (> 0)
+    // optional attention mask (nullptr: none; ignored when causal), broadcast over [batch, head, query, key]
+    // by strides in elements; F32 / F16 / BF16 are added to the scaled scores, U8 is boolean (nonzero = attend)
+    const void* mask;
+    int mask_dtype;
+    int64_t mask_stride[4];
 };
 
 struct PagedParams {
@@ -109,9 +114,10 @@ struct PagedParams {
     // chunked prefill: query-tile schedule built on the device
     int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
     int max_q_tiles;      // grid upper bound
-    int any_lengths;      // num_tokens == num_seqs may still hide multi-token sequences (HIPATTN_PA_ANY_LENGTHS)
-    // diagnostic (HIPATTN_PA_TRACE_WAVES): per decode wavefront {entry, first block consumed, exit, line units}
-    int64_t* wave_trace;
+    int any_lengths;      // a batch with num_tokens == num_seqs sends its multi-token sequences to the
+                          // chunked-prefill kernel too (HIPATTN_PA_ANY_LENGTHS); without it such a batch is
+                          // planned per token and every token is a decode row
+    int no_side_stream;   // mixed batches run one kernel after the other on the caller's stream
 };
 
 // Optional event pair recorded around the dominant kernel of a call (measurement aid).
@@ -140,7 +146,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream);  // flash over the block table (needs the plan)
 
 hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t stream);
-// diagnostic: sustained register-fed bf16 MFMA rate and shader clock of the current device (yardstick.hip)
-hipError_t run_mfma_yardstick(int zero_data, int launches, double* tflops, double* shader_ghz, hipStream_t stream);
 
+// Schedule option by name (see paged_decode.hip); value < 0 restores the default.  false: no such option.
+bool set_option(const char* name, int value);
 }  // namespace hipattn

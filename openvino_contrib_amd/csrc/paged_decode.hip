@@ -52,8 +52,10 @@
 // src/ops/assign.cpp:52-54) and materialises the scores in HBM (src/ops/matmul.cpp:204-226,
 // src/ops/softmax.cpp:184-192).
 #include <algorithm>
-#include <mutex>
+#include <atomic>
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include "device_common.hpp"
@@ -66,33 +68,60 @@ constexpr int kD = 128;   // head size of the fast path
 constexpr int kBS = 32;   // cache block size of the fast path
 
 struct alignas(32) DecodeRange {
-    int valid;        // sequence is a decode sequence with something to attend
+    int valid;        // the record is a single-token row with something to attend
     int token;        // row of q / out
     int ctx;          // attended positions end (exclusive)
     int j0;           // attended positions begin
     int first_block;  // logical block holding j0
     int nb;           // number of logical blocks attended (0 when not valid)
     int table_begin;  // offset of the sequence's block table in block_indices
-    int pad;
+    int empty_row;    // a single-token row with nothing to attend: its output row is zeros
 };
 static_assert(sizeof(DecodeRange) == 32, "one 32-byte record per sequence");
 
-// Range of cache positions a decode sequence attends.  Computed once per call by the plan and
-// stored per sequence (seq_info), so that the decode and merge kernels fetch it with one load.
-__device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int s) {
+// Sequence that owns token t: the last s with subsequence_begins[s] <= t.
+__device__ __forceinline__ int sequence_of_token(const PagedParams& p, int t) {
+    int lo = 0, hi = p.num_seqs;  // begins[lo] <= t < begins[hi]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (p.subsequence_begins[mid] <= t)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+// Range of cache positions a single-token row attends.  Computed once per call by the plan and
+// stored per record (seq_info), so that the decode and merge kernels fetch it with one load.
+//
+// Records are per sequence when the batch may hold multi-token sequences (max_q_tiles > 0: those go
+// to the chunked-prefill kernel and only sequences of exactly one token are decode rows).  A batch
+// with as many tokens as sequences is planned per TOKEN instead (max_q_tiles == 0, no prefill
+// launch): record i is token i, whichever sequence it belongs to, so a batch that only looks like
+// a decode step -- an empty sequence beside a two-token one -- still gets every row right; its
+// extra tokens are simply decode rows with their own context length.
+__device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int i) {
     DecodeRange r;
-    const int t0 = p.subsequence_begins[s];
-    r.valid = (p.subsequence_begins[s + 1] - t0 == 1);
-    r.token = t0;
+    int s = i, pos_in_seq = 0;
+    bool single = true;
+    if (p.max_q_tiles == 0) {
+        if (!(p.subsequence_begins[i] == i && p.subsequence_begins[i + 1] == i + 1)) s = sequence_of_token(p, i);
+        pos_in_seq = i - p.subsequence_begins[s];
+        r.token = i;
+    } else {
+        r.token = p.subsequence_begins[s];
+        single = (p.subsequence_begins[s + 1] - r.token == 1);
+    }
     const int table_tokens = (p.block_indices_begins[s + 1] - p.block_indices_begins[s]) * p.block_size;
-    r.ctx = min(p.past_lens[s] + 1, table_tokens);
+    r.ctx = min(p.past_lens[s] + pos_in_seq + 1, table_tokens);
     r.j0 = 0;
     if (p.sliding_window > 0 && r.ctx - p.sliding_window > 0) r.j0 = r.ctx - p.sliding_window;
-    if (r.ctx <= 0) r.valid = 0;
+    r.valid = single && r.ctx > 0;
+    r.empty_row = single && r.ctx <= 0;
     r.first_block = r.j0 / p.block_size;
     r.nb = r.valid ? (r.ctx + p.block_size - 1) / p.block_size - r.first_block : 0;
     r.table_begin = p.block_indices_begins[s];
-    r.pad = 0;
     return r;
 }
 
@@ -395,7 +424,7 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
     for (int s = s0; s < s1; s++) {
         const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
         blk += line_units(decode_range(p, s).nb, p.switch_cost);
-        tile += qlen > 1 ? (qlen + 127) / 128 : 0;
+        tile += (qlen > 1 && p.max_q_tiles > 0) ? (qlen + 127) / 128 : 0;
         if (p.overlap && qlen > 1) {
             const int past = p.past_lens[s];
             for (int r0 = 0; r0 < qlen; r0 += 128) {
@@ -458,8 +487,17 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
         p.tile_prefix[s] = tile;
         const DecodeRange rg = decode_range(p, s);
         ((DecodeRange*)p.seq_info)[s] = rg;
+        if (rg.empty_row) {  // (rare: an empty block table) nothing will visit this row
+            const int64_t n = (int64_t)p.num_heads_q * p.head_dim, o0 = (int64_t)rg.token * n;
+            for (int64_t e = 0; e < n; e++) {
+                if (p.out_dtype == HIPATTN_F32)
+                    ((float*)p.out)[o0 + e] = 0.0f;
+                else
+                    ((uint16_t*)p.out)[o0 + e] = 0;
+            }
+        }
         blk += line_units(rg.nb, p.switch_cost);
-        tile += qlen > 1 ? (qlen + 127) / 128 : 0;
+        tile += (qlen > 1 && p.max_q_tiles > 0) ? (qlen + 127) / 128 : 0;
     }
     if (s1 == p.num_seqs && s0 < p.num_seqs) {
         p.blk_prefix[p.num_seqs] = blk;
@@ -583,10 +621,6 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     const int num_waves = kWaves == 1 ? p.num_waves : p.plan_waves[0];
     if (w >= num_waves) return;
     const Line line(total, num_waves, p.dyn_pieces);
-    // diagnostic: entry time, time the first block was consumed, exit time, units done (100 MHz clock)
-    int64_t t_entry = 0, t_first = 0, units_done = 0;
-    int blocks_done = 0;
-    if (p.wave_trace) t_entry = wall_clock64();
 
     constexpr int64_t kRowBytes = kU8 ? (kD + 8) : (2 * kD);
     const int64_t block_stride = (int64_t)Hkv * kBS * kRowBytes;
@@ -603,7 +637,6 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     if (p.dyn_pieces > 0 && lane == 0) ticket_lane0 = atomicAdd(p.dyn_counter + group, 1);
     int64_t L = line.begin(piece);
     const int64_t L_end = line.begin(piece + 1);
-    units_done += L_end - L;
     int s = L < L_end ? locate_sequence(p.blk_prefix, p.num_seqs, (int)(L / Hkv), lane) : 0;
 
     while (L < L_end) {
@@ -679,8 +712,6 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                 while (i < gn) {
                     ok_b = (i + 1 < gn) ? issue(rb, i + 1) : false;
                     if (ok_a) process_block<kU8, kBf16>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
-                    if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
-                    blocks_done = 1;
                     if (i + 1 >= gn) break;
                     ok_a = (i + 2 < gn) ? issue(ra, i + 2) : false;
                     if (ok_b) process_block<kU8, kBf16>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
@@ -704,8 +735,6 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                         ok[(u + kLast) % kStages] =
                             (idx + kLast < gn) ? issue(regs[(u + kLast) % kStages], idx + kLast) : false;
                         if (ok[u]) process_block<kU8, kBf16>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kBS, rg.j0, rg.ctx, kg);
-                        if (p.wave_trace && blocks_done == 0) t_first = wall_clock64();
-                        blocks_done = 1;
                     }
                 }
             }
@@ -753,12 +782,6 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     if (next >= p.dyn_pieces) break;  // this group's share of the line is used up (every wavefront gets here)
     piece = num_waves + next;
     }
-    if (p.wave_trace && lane == 0) {
-        p.wave_trace[w * 4 + 0] = t_entry;
-        p.wave_trace[w * 4 + 1] = t_first;
-        p.wave_trace[w * 4 + 2] = wall_clock64();
-        p.wave_trace[w * 4 + 3] = units_done;
-    }
 }
 
 // Combines the partials of every (sequence, kv head) segment that more than one piece worked
@@ -779,6 +802,52 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(PagedParams p) {
     if (id_first >= id_last) return;  // a single piece covered the segment and wrote the final rows
     for (int g = threadIdx.x >> 6; g < G; g += 4)  // one wavefront per query head of the group
         merge_segment_head(p, line, s, h, g, rg.token, id_first, id_last, threadIdx.x & 63);
+}
+
+
+// Schedule options: process-wide, changed with set_option (hipattn_set_option in the C ABI).  The
+// environment variable HIPATTN_<NAME IN CAPITALS> gives an option its initial value; the
+// environment is read once, when the first option is looked at, never on the call path.
+namespace {
+struct Option {
+    const char* name;
+    const char* env;
+    int dflt, lo, hi;
+    std::atomic<int> value;
+};
+Option g_options[] = {
+    // 0: one kernel after the other for mixed batches; 1: decode beside the chunks' flash kernel
+    {"mixed_overlap", "HIPATTN_MIXED_OVERLAP", 1, 0, 1, {1}},
+    // block-times a (sequence, kv head) segment start is charged on the decode work line
+    {"decode_switch_cost", "HIPATTN_DECODE_SWITCH_COST", 3, 0, 64, {3}},
+    // on-demand pieces per wavefront for the last quarter of the decode work line (0: none)
+    {"decode_dyn_pieces_per_wave", "HIPATTN_DECODE_DYN_PIECES_PER_WAVE", 0, 0, 64, {0}},
+    // scales the compute units the plan gives the decode part of a mixed batch (100 = as modelled)
+    {"mixed_decode_share_percent", "HIPATTN_MIXED_DECODE_SHARE_PERCENT", 100, 10, 1000, {100}},
+};
+enum { kOptMixedOverlap = 0, kOptSwitchCost, kOptDynPieces, kOptSharePercent };
+
+void init_options_from_environment() {
+    static std::once_flag once;
+    std::call_once(once, [] {
+        for (Option& o : g_options)
+            if (const char* e = getenv(o.env)) o.value.store(std::min(std::max(atoi(e), o.lo), o.hi));
+    });
+}
+int option(int which) {
+    init_options_from_environment();
+    return g_options[which].value.load(std::memory_order_relaxed);
+}
+}  // namespace
+
+bool set_option(const char* name, int value) {
+    init_options_from_environment();
+    for (Option& o : g_options)
+        if (strcmp(o.name, name) == 0) {
+            o.value.store(value < 0 ? o.dflt : std::min(std::max(value, o.lo), o.hi));
+            return true;
+        }
+    return false;
 }
 
 // ---- host side of the fast path ---------------------------------------------------------
@@ -817,11 +886,10 @@ static int query_tile_bound(const PagedParams& p) {
 }
 
 // Mixed batches run the decode kernel beside the chunks' flash kernel unless the caller fixed the
-// number of decode wavefronts or HIPATTN_MIXED_OVERLAP=0 asks for one kernel after the other.
+// number of decode wavefronts or the option mixed_overlap = 0 asks for one kernel after the other.
 static bool overlap_wanted(const PagedParams& p) {
-    if (query_tile_bound(p) == 0 || p.num_waves > 0) return false;
-    const char* e = getenv("HIPATTN_MIXED_OVERLAP");
-    return !(e && atoi(e) == 0);
+    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
+    return option(kOptMixedOverlap) != 0;
 }
 
 static int choose_num_waves(const PagedParams& p, bool overlap) {
@@ -836,12 +904,10 @@ static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // On-demand pieces per wavefront for the last quarter of the line.  Off by default: a wavefront
 // that starts on a new piece pays a chain of dependent loads (ticket, sequence, block table,
 // first block) before it streams again, and on MI355X that costs more than the better balance
-// at the end of the kernel wins back.  HIPATTN_DECODE_DYN_PIECES_PER_WAVE switches it on (tuning aid).
+// at the end of the kernel wins back.  The option decode_dyn_pieces_per_wave switches it on.
 static int choose_dyn_pieces(int num_waves, bool overlap) {
     if (overlap) return 0;
-    const char* e = getenv("HIPATTN_DECODE_DYN_PIECES_PER_WAVE");
-    const int v = e ? atoi(e) : 0;
-    return num_waves * std::min(std::max(v, 0), 64);
+    return num_waves * option(kOptDynPieces);
 }
 
 size_t paged_fast_workspace_bytes(const PagedParams& p) {
@@ -850,27 +916,17 @@ size_t paged_fast_workspace_bytes(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     const size_t slots = (size_t)W + choose_dyn_pieces(W, overlap) + (size_t)p.num_seqs * p.num_heads_kv;
     return 512 + 2 * align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256) + align_up((size_t)p.num_seqs * 32, 256) +
-           align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256) +
-           (p.wave_trace ? align_up((size_t)W * 4 * sizeof(int64_t), 256) : 0);
+           align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
 }
 
-// Block-times charged per segment start; HIPATTN_DECODE_SWITCH_COST overrides (tuning aid).
-static int choose_switch_cost() {
-    const char* e = getenv("HIPATTN_DECODE_SWITCH_COST");
-    const int v = e ? atoi(e) : 3;
-    return std::min(std::max(v, 0), 64);
-}
 
 void paged_fast_plan(PagedParams& p, void* workspace) {
     const bool overlap = overlap_wanted(p);  // asks whether the caller fixed num_waves: before it is filled in
     p.overlap = overlap ? 1 : 0;
     p.num_waves = choose_num_waves(p, overlap);
-    p.switch_cost = choose_switch_cost();
+    p.switch_cost = option(kOptSwitchCost);
     p.dyn_pieces = choose_dyn_pieces(p.num_waves, overlap);
-    {
-        const char* e = getenv("HIPATTN_MIXED_DECODE_SHARE_PERCENT");  // tuning aid
-        p.overlap_share = e ? std::min(std::max(atoi(e), 10), 1000) / 100.0f : 1.0f;
-    }
+    p.overlap_share = option(kOptSharePercent) / 100.0f;
     p.dyn_groups = std::min(64, std::max(1, p.num_waves / 32));  // every group has at least one wavefront
     const int G = p.num_heads_q / p.num_heads_kv;
     const size_t slots = (size_t)p.num_waves + p.dyn_pieces + (size_t)p.num_seqs * p.num_heads_kv;
@@ -889,7 +945,6 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     w += align_up(slots * G * kD * sizeof(float), 256);
     p.part_ml = (float*)w;
     w += align_up(slots * G * 2 * sizeof(float), 256);
-    if (p.wave_trace) p.wave_trace = (int64_t*)w;  // requested: the last 32 bytes per wavefront of the workspace
     p.max_q_tiles = query_tile_bound(p);
 }
 

@@ -19,6 +19,11 @@
  *                              max-subtracted softmax as src/ops/softmax.cpp:75-147).
  *                              Pinned by: fp64 brute force, torch's CPU
  *                              scaled_dot_product_attention fixtures, invariants.
+ *   oracle_sdpa_mask_f32       the same with the operator's attention_mask input (additive;
+ *                              boolean masks converted to 0 / -inf), the Add node of the
+ *                              decomposed graph (src/ops/add.cpp:17-43).  Pinned by torch's
+ *                              CPU routine with attn_mask (float, boolean, broadcast) and by
+ *                              explicit causal mask == causal flag.
  *   oracle_kv_cache_write      slot(s, p) = block_indices[begins[s] + p / bs] * bs + p % bs,
  *                              row scatter in the spirit of
  *                              src/kernels/scatter_nd_update.cu:19-34; out-of-range block
@@ -247,8 +252,9 @@ static inline float dotf(const float* a, const float* b, int n) {
  * One query row against keys [j0, j1) given as row pointers computed by the caller's
  * stride; scores buffer must hold j1 - j0 floats.
  */
-static void attend_row(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0, int j1,
-                       int D, float scale, float* scores, float* out) {
+static void attend_row_biased(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0,
+                              int j1, int D, float scale, const float* bias, int64_t bias_stride, float* scores,
+                              float* out) {
     int n = j1 - j0;
     if (n <= 0) {
         for (int d = 0; d < D; d++) out[d] = 0.0f;
@@ -257,6 +263,7 @@ static void attend_row(const float* q, const float* kbase, const float* vbase, i
     float m = -INFINITY;
     for (int j = 0; j < n; j++) {
         float s = scale * dotf(q, kbase + (int64_t)(j0 + j) * kv_stride, D);
+        if (bias) s += bias[(int64_t)(j0 + j) * bias_stride];
         scores[j] = s;
         m = s > m ? s : m;
     }
@@ -274,6 +281,11 @@ static void attend_row(const float* q, const float* kbase, const float* vbase, i
     }
     float inv = (float)(1.0 / l);
     for (int d = 0; d < D; d++) out[d] *= inv;
+}
+
+static void attend_row(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0, int j1,
+                       int D, float scale, float* scores, float* out) {
+    attend_row_biased(q, kbase, vbase, kv_stride, j0, j1, D, scale, NULL, 0, scores, out);
 }
 
 /*
@@ -299,6 +311,43 @@ ORACLE_API int oracle_sdpa_f32(const float* q, const float* k, const float* v, f
             const float* vb = v + ((int64_t)b * Hkv + h / G) * Lk * D;
             int j1 = causal ? (i + 1 < Lk ? i + 1 : Lk) : Lk;
             attend_row(q + r * D, kb, vb, D, 0, j1, D, scale, scores, out + r * D);
+        }
+        free(scores);
+    }
+    return 0;
+}
+
+/*
+ * The same operator with its attention_mask input: softmax(scale * Q K^T + mask) V.  mask is the
+ * additive form (a boolean mask is 0 where true and -inf where false, as the operator
+ * specification converts it), addressed as [B,Hq,Lq,Lk] through element strides, 0 = broadcast;
+ * it replaces the Add node of the decomposed graph (src/ops/add.cpp:17-43, numpy broadcast as
+ * src/ops/elementwise_binary.hpp:15-77).  With causal set the mask is ignored, as the operator
+ * specifies.  A row whose keys are all masked with -inf comes out as NaN (exp(-inf - -inf)),
+ * like the library routine that pins this function.
+ * Pinned by torch's CPU scaled_dot_product_attention(attn_mask=...) fixtures (float and boolean,
+ * broadcast and full) and by reduction: a causal mask passed explicitly equals causal = 1.
+ */
+ORACLE_API int oracle_sdpa_mask_f32(const float* q, const float* k, const float* v, float* out, int B, int Hq,
+                                    int Hkv, int Lq, int Lk, int D, int causal, float scale, const float* mask,
+                                    const int64_t* mask_stride) {
+    if (!mask || causal) return oracle_sdpa_f32(q, k, v, out, B, Hq, Hkv, Lq, Lk, D, causal, scale);
+    if (B < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Lq < 0 || Lk < 0 || D <= 0) return 1;
+    if (scale <= 0.0f) scale = 1.0f / sqrtf((float)D);
+    int G = Hq / Hkv;
+    int64_t rows = (int64_t)B * Hq * Lq;
+#pragma omp parallel
+    {
+        float* scores = (float*)malloc(sizeof(float) * (size_t)(Lk > 0 ? Lk : 1));
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t r = 0; r < rows; r++) {
+            int i = (int)(r % Lq);
+            int h = (int)((r / Lq) % Hq);
+            int b = (int)(r / ((int64_t)Lq * Hq));
+            const float* kb = k + ((int64_t)b * Hkv + h / G) * Lk * D;
+            const float* vb = v + ((int64_t)b * Hkv + h / G) * Lk * D;
+            const float* mrow = mask + b * mask_stride[0] + h * mask_stride[1] + i * mask_stride[2];
+            attend_row_biased(q + r * D, kb, vb, D, 0, Lk, D, scale, mrow, mask_stride[3], scores, out + r * D);
         }
         free(scores);
     }
@@ -392,6 +441,15 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
         int t0 = subsequence_begins[s], qlen = subsequence_begins[s + 1] - t0;
         if (qlen <= 0) continue;
         int ctx = past_lens[s] + qlen;
+        /* positions beyond the sequence's block table do not exist (their writes were skipped) */
+        int table_tokens = (block_indices_begins[s + 1] - block_indices_begins[s]) * block_size;
+        if (ctx > table_tokens) ctx = table_tokens;
+        if (ctx <= 0) {
+            for (int i = 0; i < qlen; i++)
+                for (int g = 0; g < G; g++)
+                    memset(out + ((int64_t)(t0 + i) * Hq + (h * G + g)) * D, 0, sizeof(float) * (size_t)D);
+            continue;
+        }
         float* kbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
         float* vbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
         float* scores = (float*)malloc(sizeof(float) * (size_t)ctx);
@@ -404,7 +462,8 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
             if (sliding_window > 0 && p - sliding_window + 1 > 0) j0 = p - sliding_window + 1;
             for (int g = 0; g < G; g++) {
                 int64_t row = ((int64_t)(t0 + i) * Hq + (h * G + g)) * D;
-                attend_row(q + row, kbuf, vbuf, D, j0, p + 1, D, scale, scores, out + row);
+                attend_row(q + row, kbuf, vbuf, D, j0 < ctx ? j0 : ctx, p + 1 < ctx ? p + 1 : ctx, D, scale, scores,
+                           out + row);
             }
         }
         free(kbuf);

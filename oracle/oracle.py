@@ -53,6 +53,8 @@ def lib():
         L.oracle_dequant_u8_rows.restype = None
         L.oracle_sdpa_f32.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, f32]
         L.oracle_sdpa_f32.restype = i32
+        L.oracle_sdpa_mask_f32.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, f32, vp, vp]
+        L.oracle_sdpa_mask_f32.restype = i32
         L.oracle_kv_cache_write.argtypes = [vp, vp, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32]
         L.oracle_kv_cache_write.restype = i64
         L.oracle_gather_cache_rows.argtypes = [vp, i32, vp, i32, i32, i32, i32, i32, vp]
@@ -154,6 +156,30 @@ def sdpa(q, k, v, causal=False, scale=0.0):
     rc = lib().oracle_sdpa_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, Lq, Lk, D, int(bool(causal)), float(scale))
     if rc:
         raise ValueError("oracle_sdpa_f32: bad arguments")
+    return out
+
+
+def sdpa_masked(q, k, v, mask, causal=False, scale=0.0):
+    """SDPA with an attention mask broadcastable to [B,Hq,Lq,Lk]: float = added to the scaled scores,
+    bool = True takes part (the operator's two mask forms)."""
+    q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
+    B, Hq, Lq, D = q.shape
+    _, Hkv, Lk, _ = k.shape
+    mask = np.asarray(mask)
+    if mask.dtype == np.bool_:
+        mask = np.where(mask, np.float32(0.0), np.float32(-np.inf))
+    mask = _c(mask, np.float32)
+    while mask.ndim < 4:
+        mask = mask[None]
+    strides = np.zeros(4, np.int64)
+    for ax, full in enumerate((B, Hq, Lq, Lk)):
+        assert mask.shape[ax] in (1, full), "mask shape %s does not broadcast to %s" % (mask.shape, (B, Hq, Lq, Lk))
+        strides[ax] = mask.strides[ax] // 4 if mask.shape[ax] == full and full > 1 else 0
+    out = np.empty_like(q)
+    rc = lib().oracle_sdpa_mask_f32(_p(q), _p(k), _p(v), _p(out), B, Hq, Hkv, Lq, Lk, D, int(bool(causal)),
+                                    float(scale), _p(mask), _p(strides))
+    if rc:
+        raise ValueError("oracle_sdpa_mask_f32: bad arguments")
     return out
 
 

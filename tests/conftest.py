@@ -30,3 +30,18 @@ def hip():
     assert capi.device_count() > 0, "no HIP device: GPU tests must run on the GPU box"
     capi.check(capi.lib().hipattn_set_device(0))
     return capi
+
+
+@pytest.fixture
+def schedule_options(hip):
+    """Sets process-wide schedule options of the library for one test and restores the defaults after it."""
+    touched = []
+
+    def apply(options):
+        for name, value in options.items():
+            hip.set_option(name, value)
+            touched.append(name)
+
+    yield apply
+    for name in touched:
+        hip.set_option(name, -1)

@@ -1,88 +1,7 @@
-"""Shared plumbing of the GPU parity tests: move a synthetic case through the C ABI and bring
-the results back as fp32 numpy arrays."""
-import numpy as np
-
-from openvino_contrib_amd import workloads as W
-
-
-def storage_to_f32(arr, dtype):
-    if dtype == W.F32:
-        return arr.astype(np.float32)
-    if dtype == W.F16:
-        return W.f16_bits_to_f32(arr)
-    return W.bf16_bits_to_f32(arr)
-
-
-def run_sdpa(hip, case, causal, scale=0.0):
-    desc = hip.SdpaDesc(case["dtype"], case["B"], case["Hq"], case["Hkv"], case["Lq"], case["Lk"], case["D"],
-                        int(causal), scale)
-    q = hip.DeviceBuffer.from_numpy(case["q_store"])
-    k = hip.DeviceBuffer.from_numpy(case["k_store"])
-    v = hip.DeviceBuffer.from_numpy(case["v_store"])
-    out = hip.DeviceBuffer(case["q_store"].nbytes)
-    out.fill(0xFF)  # NaN pattern: rows the kernel fails to write show up
-    ws_bytes = hip.sdpa_workspace_size(desc)
-    ws = hip.DeviceBuffer(ws_bytes) if ws_bytes else None
-    hip.sdpa(desc, q, k, v, out, ws)
-    res = out.download(W.np_storage_dtype(case["dtype"]), case["q_store"].shape)
-    path = hip.last_kernel_path()
-    for b in (q, k, v, out):
-        b.free()
-    return storage_to_f32(res, case["dtype"]), path
-
-
-def pa_desc(hip, case, out_dtype=None, flags=0, decode_waves=0, scale=0.0, max_context_len=None):
-    return hip.PaDesc(case["q_dtype"], case["kv_dtype"], case["cache_dtype"],
-                      case["q_dtype"] if out_dtype is None else out_dtype, case["Hq"], case["Hkv"], case["D"],
-                      case["block_size"], case["num_blocks"], case["T"], case["S"],
-                      case["max_context_len"] if max_context_len is None else max_context_len,
-                      case["sliding_window"], scale, flags, decode_waves)
-
-
-class PagedDeviceCase:
-    """Device copies of one paged-attention call."""
-
-    def __init__(self, hip, case, out_dtype=None):
-        self.hip, self.case = hip, case
-        self.out_dtype = case["q_dtype"] if out_dtype is None else out_dtype
-        up = hip.DeviceBuffer.from_numpy
-        self.q = up(case["q_store"])
-        self.k_new = up(case["k_new_store"])
-        self.v_new = up(case["v_new_store"])
-        self.key_cache = up(case["key_cache"])
-        self.value_cache = up(case["value_cache"])
-        self.past_lens = up(case["past_lens"])
-        self.subsequence_begins = up(case["subsequence_begins"])
-        self.block_indices = up(case["block_indices"])
-        self.block_indices_begins = up(case["block_indices_begins"])
-        self.out_elems = case["T"] * case["Hq"] * case["D"]
-        self.out = hip.DeviceBuffer(self.out_elems * hip.DTYPE_BYTES[self.out_dtype])
-
-    def run(self, flags=0, decode_waves=0, scale=0.0, max_context_len=None, stream=None):
-        hip = self.hip
-        desc = pa_desc(hip, self.case, self.out_dtype, flags, decode_waves, scale, max_context_len)
-        nbytes = hip.paged_attention_workspace_size(desc)
-        ws = hip.DeviceBuffer(nbytes) if nbytes else None
-        self.out.fill(0xFF)
-        hip.paged_attention(desc, self.q, self.k_new, self.v_new, self.key_cache, self.value_cache, self.past_lens,
-                            self.subsequence_begins, self.block_indices, self.block_indices_begins, self.out, ws,
-                            stream)
-        path = hip.last_kernel_path()
-        res = self.out.download(W.np_storage_dtype(self.out_dtype), (self.case["T"], self.case["Hq"] * self.case["D"]),
-                                stream)
-        if ws:
-            ws.free()
-        return storage_to_f32(res, self.out_dtype), path
-
-    def caches(self):
-        kc = self.key_cache.download(np.uint8, self.case["key_cache"].shape)
-        vc = self.value_cache.download(np.uint8, self.case["value_cache"].shape)
-        return kc, vc
-
-    def free(self):
-        for b in (self.q, self.k_new, self.v_new, self.key_cache, self.value_cache, self.past_lens,
-                  self.subsequence_begins, self.block_indices, self.block_indices_begins, self.out):
-            b.free()
+"""Shared plumbing of the GPU parity tests: the device-side case runners of the package plus the
+oracle call they are compared with."""
+from openvino_contrib_amd.device_case import (PagedDeviceCase, max_abs, pa_desc, run_sdpa, run_sdpa_masked,  # noqa: F401
+                                              storage_to_f32)
 
 
 def oracle_paged(oracle, case, scale=0.0):
@@ -94,5 +13,3 @@ def oracle_paged(oracle, case, scale=0.0):
     return out, kc, vc
 
 
-def max_abs(a, b):
-    return float(np.max(np.abs(a.astype(np.float64) - b.astype(np.float64)))) if a.size else 0.0

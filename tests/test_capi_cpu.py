@@ -31,11 +31,13 @@ def test_struct_layout_matches_header():
     # 9 and 16 four-byte fields, no padding
     assert ctypes.sizeof(capi.SdpaDesc) == 36
     assert ctypes.sizeof(capi.PaDesc) == 64
+    # int + four int64, the int64s aligned to 8
+    assert ctypes.sizeof(capi.MaskDesc) == 40 and capi.MaskDesc.stride.offset == 8
 
 
 def test_non_compute_calls_work_without_a_device():
     L = capi.lib()
-    assert L.hipattn_version() == 1
+    assert L.hipattn_version() == 2
     assert L.hipattn_status_string(capi.UNSUPPORTED) == b"unsupported"
     assert capi.cache_row_bytes(capi.U8, 128) == 136
     assert capi.cache_row_bytes(capi.F16, 128) == 256
@@ -55,3 +57,8 @@ def test_non_compute_calls_work_without_a_device():
     pa.head_dim = 128
     pa.cache_dtype = 9
     assert L.hipattn_paged_attention_workspace_size(ctypes.byref(pa), ctypes.byref(n)) == capi.INVALID_ARGUMENT
+    # options are process-wide host state: no device needed
+    assert L.hipattn_set_option(b"decode_switch_cost", 5) == capi.OK
+    assert L.hipattn_set_option(b"decode_switch_cost", -1) == capi.OK
+    assert L.hipattn_set_option(b"no_such_option", 1) == capi.INVALID_ARGUMENT
+    assert b"no_such_option" in L.hipattn_last_error_string()

@@ -228,6 +228,61 @@ def test_sdpa_flash_tensors_beyond_two_gib(hip, oracle):
         assert H.max_abs(out[0, h, row], ref[0, 0, 0]) <= TOL[W.BF16], (h, row)
 
 
+@pytest.mark.parametrize("dtype,tol", [(W.F32, 1e-4), (W.F16, 2e-3), (W.BF16, 1e-2)])
+@pytest.mark.parametrize("mask_kind", ["bool_full", "float_full", "float_2d", "bool_keys", "half_per_head"])
+def test_sdpa_with_attention_mask(hip, oracle, dtype, tol, mask_kind):
+    """The operator's attention_mask input through hipattn_sdpa_masked: boolean and additive masks,
+    full and broadcast shapes, against the oracle on the same stored values (max-abs)."""
+    announce("sdpa mask", dtype, mask_kind)
+    B, Hq, Hkv, Lq, Lk, D = 2, 4, 2, 70, 130, 128
+    case = W.make_sdpa_case(61, B, Hq, Hkv, Lq, Lk, D, dtype)
+    rng = np.random.default_rng(62)
+    if mask_kind == "bool_full":
+        mask = rng.random((B, Hq, Lq, Lk)) < 0.5
+        mask[..., 5] = True
+    elif mask_kind == "bool_keys":
+        mask = rng.random((B, 1, 1, Lk)) < 0.3
+        mask[..., 0] = True
+    elif mask_kind == "float_full":
+        mask = (2.0 * rng.standard_normal((B, Hq, Lq, Lk))).astype(np.float32)
+        mask[0, 1, 3, 10:] = -np.inf
+    elif mask_kind == "float_2d":
+        mask = (2.0 * rng.standard_normal((Lq, Lk))).astype(np.float32)
+    else:
+        mask = rng.standard_normal((1, Hq, 1, 1)).astype(np.float16)  # a constant per head: no effect on the result
+    out, path = H.run_sdpa_masked(hip, case, mask)
+    assert path == "sdpa_generic"
+    ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask.astype(np.float32) if mask.dtype == np.float16 else mask)
+    assert np.isfinite(out).all()
+    assert H.max_abs(out, ref) <= tol
+    if mask_kind == "half_per_head":
+        assert H.max_abs(out, oracle.sdpa(case["q"], case["k"], case["v"])) <= tol
+
+
+def test_sdpa_mask_is_ignored_when_causal_and_masked_rows_are_zeros(hip, oracle):
+    announce("sdpa mask causal / empty rows")
+    case = W.make_sdpa_case(63, 1, 8, 2, 200, 200, 128, W.BF16, std=0.5)
+    desc = hip.SdpaDesc(W.BF16, 1, 8, 2, 200, 200, 128, 1, 0.0)
+    bufs = [hip.DeviceBuffer.from_numpy(case[n]) for n in ("q_store", "k_store", "v_store")]
+    mask = hip.DeviceBuffer.from_numpy(np.zeros((200, 200), np.uint8))  # would mask everything
+    out = hip.DeviceBuffer(case["q_store"].nbytes)
+    hip.sdpa_masked(desc, bufs[0], bufs[1], bufs[2], W.U8, [0, 0, 200, 1], mask, out)
+    assert hip.last_kernel_path() == "sdpa_flash_mfma"  # causal set: the mask plays no part
+    res = H.storage_to_f32(out.download(np.uint16, case["q_store"].shape), W.BF16)
+    assert H.max_abs(res, oracle.sdpa(case["q"], case["k"], case["v"], causal=True)) <= 1e-2
+    for b in bufs + [mask, out]:
+        b.free()
+    # a row with every key masked out has nothing to attend: zeros (the operator's softmax is undefined there)
+    m = np.ones((200, 200), bool)
+    m[17] = False
+    res, _ = H.run_sdpa_masked(hip, case, m)
+    assert not res[:, :, 17].any()
+    m[17, 0] = True
+    ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], m)
+    keep = np.arange(200) != 17
+    assert H.max_abs(res[:, :, keep], ref[:, :, keep]) <= 1e-2
+
+
 def test_sdpa_scale_and_empty(hip, oracle):
     announce("sdpa scale/empty")
     case = W.make_sdpa_case(63, 1, 2, 1, 90, 90, 128, W.F16)
@@ -288,14 +343,13 @@ def test_paged_decode_sliding_window(hip, oracle, cache_dtype, window):
     dev.free()
 
 
-@pytest.mark.parametrize("env", [{"HIPATTN_DECODE_DYN_PIECES_PER_WAVE": "4"}, {"HIPATTN_DECODE_SWITCH_COST": "0"},
-                                 {"HIPATTN_DECODE_DYN_PIECES_PER_WAVE": "2", "HIPATTN_DECODE_SWITCH_COST": "9"}])
+@pytest.mark.parametrize("env", [{"decode_dyn_pieces_per_wave": 4}, {"decode_switch_cost": 0},
+                                 {"decode_dyn_pieces_per_wave": 2, "decode_switch_cost": 9}])
 @pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
-def test_paged_decode_schedule_knobs(hip, oracle, env, cache_dtype, monkeypatch):
+def test_paged_decode_schedule_knobs(hip, oracle, env, cache_dtype, schedule_options):
     """The schedule of the decode kernel (on-demand pieces, segment-start cost) never changes results."""
     announce("paged decode knobs", env, cache_dtype)
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    schedule_options(env)
     seqs = [(c - 1, 1) for c in DECODE_CTX]
     case = W.make_paged_case(75, seqs, 32, 8, 128, 32, W.F16, W.F16, cache_dtype, sliding_window=700)
     ref, _, _ = H.oracle_paged(oracle, case)
@@ -477,17 +531,16 @@ def test_paged_batch_of_thousands_of_sequences(hip, oracle, cache_dtype, mixed):
     dev.free()
 
 
-@pytest.mark.parametrize("env", [{}, {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "10"},
-                                 {"HIPATTN_MIXED_DECODE_SHARE_PERCENT": "1000"}, {"HIPATTN_MIXED_OVERLAP": "0"}])
+@pytest.mark.parametrize("env", [{}, {"mixed_decode_share_percent": 10},
+                                 {"mixed_decode_share_percent": 1000}, {"mixed_overlap": 0}])
 @pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.BF16, W.F16, 0), (W.F16, W.U8, 300), (W.BF16, W.BF16, 0)])
-def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, window, monkeypatch):
+def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, window, schedule_options):
     """With no fixed wavefront count the decode kernel of a mixed batch runs beside the chunks' flash
     kernel on a share of the compute units that the plan picks on the device; whatever the share
     (forced small and large here, and the one-after-the-other order), the results are the same, also
     when calls follow each other without a synchronisation in between."""
     announce("paged mixed side by side", env, q_dtype, cache_dtype, window)
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    schedule_options(env)
     batches = [
         [(0, 130), (37, 1), (500, 1), (100, 257), (0, 2), (999, 1), (31, 97), (64, 1), (700, 128), (5, 0)],
         [(0, 300), (210, 45)],                                       # no decode sequence at all
@@ -512,25 +565,68 @@ def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, 
         dev.free()
 
 
-def test_paged_as_many_tokens_as_sequences_but_not_one_each(hip, oracle):
-    """num_tokens == num_seqs normally means a pure decode batch (the host cannot see the lengths);
-    a batch that only looks like one -- an empty sequence beside a two-token one -- needs the
-    HIPATTN_PA_ANY_LENGTHS flag, and with it goes through the mixed-batch path."""
-    announce("paged T == S with mixed lengths")
+@pytest.mark.parametrize("flags", [0, 8])
+def test_paged_as_many_tokens_as_sequences_but_not_one_each(hip, oracle, flags):
+    """num_tokens == num_seqs normally is a pure decode batch (the host cannot see the lengths); a
+    batch that only looks like one -- an empty sequence beside a two-token one -- must come out right
+    all the same: planned per token without a flag (every token a decode row), through the
+    mixed-batch path with HIPATTN_PA_ANY_LENGTHS."""
+    announce("paged T == S with mixed lengths", flags)
+    assert flags in (0, hip.PA_ANY_LENGTHS)
+    batches = [[(1500, 1), (100, 2), (31, 0)], [(5, 0), (0, 3), (200, 0), (64, 1), (77, 0), (31, 2)], [(0, 0), (40, 2)]]
     for cache_dtype in (W.F16, W.U8):
-        case = W.make_paged_case(99, [(1500, 1), (100, 2), (31, 0)], 24, 3, 128, 32, W.F16, W.F16, cache_dtype,
-                                 sliding_window=64)
-        assert case["T"] == case["S"]
-        ref, okc, ovc = H.oracle_paged(oracle, case)
+        for i, seqs in enumerate(batches):
+            case = W.make_paged_case(99 + i, seqs, 24, 3, 128, 32, W.F16, W.F16, cache_dtype, sliding_window=64)
+            assert case["T"] == case["S"]
+            ref, okc, ovc = H.oracle_paged(oracle, case)
+            dev = H.PagedDeviceCase(hip, case)
+            out, path = dev.run(flags=flags)
+            assert path == "paged_mfma"
+            kc, vc = dev.caches()
+            np.testing.assert_array_equal(kc, okc)
+            np.testing.assert_array_equal(vc, ovc)
+            assert np.isfinite(out).all()
+            assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3), (i, cache_dtype)
+            dev.free()
+
+
+def test_paged_decode_row_with_an_empty_block_table_is_zeros(hip, oracle):
+    """A single-token sequence whose block table is empty has nothing to attend: zeros on every path."""
+    announce("paged decode empty table")
+    case = W.make_paged_case(98, [(40, 1), (7, 1), (300, 1)], 16, 4, 128, 32, W.F16, W.F16, W.F16)
+    ref, _, _ = H.oracle_paged(oracle, case)  # rows 0 and 2 do not depend on sequence 1
+    b = case["block_indices_begins"]
+    n1 = int(b[2] - b[1])
+    case["block_indices"] = np.concatenate([case["block_indices"][:b[1]], case["block_indices"][b[2]:]]).astype(np.int32)
+    b[2:] -= n1  # sequence 1 now owns no block
+    ref[1] = 0.0
+    ref_again, _, _ = H.oracle_paged(oracle, case)
+    np.testing.assert_array_equal(ref, ref_again)
+    for flags in (0, hip.PA_FORCE_GENERIC):
         dev = H.PagedDeviceCase(hip, case)
-        out, path = dev.run(flags=hip.PA_ANY_LENGTHS)
-        assert path == "paged_mfma"
-        kc, vc = dev.caches()
-        np.testing.assert_array_equal(kc, okc)
-        np.testing.assert_array_equal(vc, ovc)
-        assert np.isfinite(out).all()
-        assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3)
+        out, _ = dev.run(flags=flags)
+        assert H.max_abs(out, ref) <= 2e-3, flags
+        assert not out[1].any(), flags
         dev.free()
+
+
+def test_paged_generic_skips_blocks_outside_the_cache(hip, oracle):
+    """A block id outside [0, num_blocks) in a table: the decode and the shape-generic kernels give
+    its keys probability zero, i.e. the result of the same sequence attending only its valid blocks
+    (checked as: both paths agree with each other and are finite)."""
+    announce("paged invalid block ids")
+    case = W.make_paged_case(97, [(95, 1), (200, 1)], 8, 2, 128, 32, W.F16, W.F16, W.F16)
+    b = case["block_indices_begins"]
+    case["block_indices"][b[0] + 1] = -7                    # second block of sequence 0
+    case["block_indices"][b[1] + 2] = case["num_blocks"] + 3  # third block of sequence 1
+    outs = []
+    for flags in (hip.PA_SKIP_CACHE_WRITE, hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC):
+        dev = H.PagedDeviceCase(hip, case)
+        out, _ = dev.run(flags=flags)
+        assert np.isfinite(out).all()
+        outs.append(out)
+        dev.free()
+    assert H.max_abs(outs[0], outs[1]) <= 2e-3
 
 
 def test_paged_mixed_batches_from_two_host_threads(hip, oracle):
@@ -620,9 +716,11 @@ def test_paged_errors(hip):
 def test_mfma_yardstick_reports_a_plausible_rate(hip):
     """The diagnostic that bench.py --workload mfma prints: register-fed bf16 MFMAs only."""
     import ctypes
+    from openvino_contrib_amd import build as hip_build
+    yard = ctypes.CDLL(hip_build.YARDSTICK_LIB_PATH)  # a bench-only library, not part of libhipattn
     tf, ghz = ctypes.c_double(), ctypes.c_double()
-    hip.check(hip.lib().hipattn_mfma_yardstick(1, 20, ctypes.byref(tf), ctypes.byref(ghz), None))
+    assert yard.mfma_yardstick(1, 20, ctypes.byref(tf), ctypes.byref(ghz)) == 0
     assert 500.0 < tf.value < 2600.0   # never above the 2.5 PFLOP/s dense bf16 peak (plus timer slack)
     assert 1.0 < ghz.value < 2.6
-    assert hip.lib().hipattn_mfma_yardstick(0, 0, ctypes.byref(tf), ctypes.byref(ghz), None) == hip.INVALID_ARGUMENT
+    assert yard.mfma_yardstick(0, 0, ctypes.byref(tf), ctypes.byref(ghz)) != 0
 

@@ -58,6 +58,40 @@ def test_sdpa_matches_fp64_brute_force(oracle, shape, causal):
     np.testing.assert_allclose(out, ref, atol=2e-6, rtol=1e-5)
 
 
+@pytest.mark.parametrize("name", ["float_full", "float_2d", "float_per_batch", "bool_full", "bool_keys"])
+def test_sdpa_mask_matches_torch_fixture(oracle, name):
+    """attention_mask input: float masks are added to the scaled scores, boolean masks select keys;
+    fixtures from torch's CPU routine with attn_mask, broadcast shapes included."""
+    z = np.load(GOLDEN)
+    p = "mask_" + name
+    out = oracle.sdpa_masked(z[p + "/q"], z[p + "/k"], z[p + "/v"], z[p + "/mask"])
+    np.testing.assert_allclose(out, z[p + "/out"], atol=2e-6, rtol=1e-5)
+
+
+def test_sdpa_mask_reductions(oracle):
+    c = W.make_sdpa_case(12, 2, 4, 2, 11, 11, 16, W.F32)
+    q, k, v = c["q"], c["k"], c["v"]
+    tril = np.tril(np.ones((11, 11), bool))
+    # an explicit lower-triangular boolean mask is the causal flag
+    np.testing.assert_allclose(oracle.sdpa_masked(q, k, v, tril), oracle.sdpa(q, k, v, causal=True), atol=1e-6)
+    # ... and so is its additive form; a mask of zeros changes nothing; with causal set the mask is ignored
+    add = np.where(tril, 0.0, -np.inf).astype(np.float32)
+    np.testing.assert_array_equal(oracle.sdpa_masked(q, k, v, add), oracle.sdpa_masked(q, k, v, tril))
+    np.testing.assert_array_equal(oracle.sdpa_masked(q, k, v, np.zeros((1, 1, 1, 11), np.float32)), oracle.sdpa(q, k, v))
+    np.testing.assert_array_equal(oracle.sdpa_masked(q, k, v, np.full((11, 11), -3.0, np.float32), causal=True),
+                                  oracle.sdpa(q, k, v, causal=True))
+    # a per-row constant shifts every score of the row: no change (softmax shift invariance)
+    rowc = np.arange(11, dtype=np.float32)[:, None] * np.ones((1, 11), np.float32)
+    np.testing.assert_allclose(oracle.sdpa_masked(q, k, v, rowc), oracle.sdpa(q, k, v), atol=1e-5)
+    # fp64 brute force with a random boolean mask over batch and heads
+    rng = np.random.default_rng(5)
+    m = rng.random((2, 4, 11, 11)) < 0.5
+    m[..., 3] = True
+    ref = np.stack([np.stack([brute_sdpa_f64(q[b:b + 1, h:h + 1], k[b:b + 1, h // 2:h // 2 + 1], v[b:b + 1, h // 2:h // 2 + 1],
+                                             False, mask=m[b, h])[0, 0] for h in range(4)]) for b in range(2)])
+    np.testing.assert_allclose(oracle.sdpa_masked(q, k, v, m), ref, atol=2e-6, rtol=1e-5)
+
+
 def test_sdpa_invariants(oracle):
     c = W.make_sdpa_case(11, 2, 4, 2, 10, 10, 16, W.F32)
     q, k, v = c["q"], c["k"], c["v"]
