@@ -212,6 +212,23 @@ hipattn_status hipattn_paged_attention(const hipattn_pa_desc* desc, const void* 
                                        const int32_t* block_indices, const int32_t* block_indices_begins, void* out,
                                        void* workspace, size_t workspace_bytes, hipattn_stream stream);
 
+/* The same operator for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference (its operators get scratch from the memory manager's per-request blob,
+ * src/cuda_operation_base.hpp:114-117).  No workspace argument: scratch is a static device array
+ * of HIPATTN_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs on, and the call
+ * makes no hipMalloc / hipFree, creates no stream or event and calls no allocating routine.  A
+ * batch whose plan needs more (hipattn_paged_attention_workspace_size tells) is refused with
+ * HIPATTN_WORKSPACE_TOO_SMALL.  Mixed batches run their kernels one after the other on `stream`
+ * (no side stream).  All calls on one GPU share the array: calls that overlap in time on one GPU,
+ * on whatever streams, race; one after the other is fine. */
+#define HIPATTN_NOALLOC_SCRATCH_BYTES (16u << 20)
+hipattn_status hipattn_paged_attention_noalloc(const hipattn_pa_desc* desc, const void* q, const void* k_new,
+                                               const void* v_new, void* key_cache, void* value_cache,
+                                               const int32_t* past_lens, const int32_t* subsequence_begins,
+                                               const int32_t* block_indices, const int32_t* block_indices_begins,
+                                               void* out, hipattn_stream stream);
+
 /* Step 1 alone: the device-side KV-cache block writer. */
 hipattn_status hipattn_kv_cache_write(const hipattn_pa_desc* desc, const void* k_new, const void* v_new,
                                       void* key_cache, void* value_cache, const int32_t* past_lens,

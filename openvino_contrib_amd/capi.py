@@ -114,6 +114,7 @@ SYMBOLS = {
     "hipattn_sdpa_masked": (_i, [_P(SdpaDesc), _vp, _vp, _vp, _P(MaskDesc), _vp, _vp, _vp, _sz, _vp]),
     "hipattn_paged_attention_workspace_size": (_i, [_P(PaDesc), _P(_sz)]),
     "hipattn_paged_attention": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "hipattn_paged_attention_noalloc": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "hipattn_set_option": (_i, [ctypes.c_char_p, _i]),
     "hipattn_kv_cache_write": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "hipattn_cache_row_bytes": (_sz, [_i, _i]),
@@ -288,9 +289,21 @@ def paged_attention(desc, q, k_new, v_new, key_cache, value_cache, past_lens, su
         out.ptr, workspace.ptr if workspace else None, workspace.nbytes if workspace else 0, _h(stream)))
 
 
+def paged_attention_noalloc(desc, q, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins,
+                            block_indices, block_indices_begins, out, stream=None):
+    """The entry point that allocates nothing: scratch is the library's static device array."""
+    check(lib().hipattn_paged_attention_noalloc(
+        ctypes.byref(desc), q.ptr, k_new.ptr if k_new else None, v_new.ptr if v_new else None, key_cache.ptr,
+        value_cache.ptr, past_lens.ptr, subsequence_begins.ptr, block_indices.ptr, block_indices_begins.ptr,
+        out.ptr, _h(stream)))
+
+
 def set_option(name, value):
     """Process-wide schedule option (see include/hipattn.h); value < 0 restores the default."""
     check(lib().hipattn_set_option(name.encode(), int(value)))
+
+
+NOALLOC_SCRATCH_BYTES = 16 << 20
 
 
 def kv_cache_write(desc, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins, block_indices,

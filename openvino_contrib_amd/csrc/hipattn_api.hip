@@ -434,7 +434,13 @@ hipattn_status paged_attention_impl(const hipattn_pa_desc* desc, const void* q, 
     p.no_side_stream = static_scratch ? 1 : 0;  // (creating the side stream of a mixed batch allocates)
     if (!(desc->flags & HIPATTN_PA_FORCE_GENERIC) && hipattn::paged_fast_supported(p)) {
         const size_t need = hipattn::paged_fast_workspace_bytes(p);
-        (void)static_scratch;
+        if (static_scratch) {
+            if (need > (size_t)HIPATTN_NOALLOC_SCRATCH_BYTES)
+                return fail(HIPATTN_WORKSPACE_TOO_SMALL,
+                            "paged_attention_noalloc: this batch needs %zu bytes of scratch, the static scratch holds %zu; "
+                            "use hipattn_paged_attention with a workspace", need, (size_t)HIPATTN_NOALLOC_SCRATCH_BYTES);
+            HIP_TRY(hipattn::paged_static_scratch(&workspace, &workspace_bytes));
+        }
         if (need > 0 && (!workspace || workspace_bytes < need))
             return fail(HIPATTN_WORKSPACE_TOO_SMALL, "paged_attention: workspace %zu bytes, need %zu", workspace_bytes,
                         need);
@@ -460,4 +466,15 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention(const hipattn_pa_desc* des
                                                       size_t workspace_bytes, hipattn_stream stream) {
     return paged_attention_impl(desc, q, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins,
                                 block_indices, block_indices_begins, out, workspace, workspace_bytes, stream, false);
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_paged_attention_noalloc(const hipattn_pa_desc* desc, const void* q,
+                                                              const void* k_new, const void* v_new, void* key_cache,
+                                                              void* value_cache, const int32_t* past_lens,
+                                                              const int32_t* subsequence_begins,
+                                                              const int32_t* block_indices,
+                                                              const int32_t* block_indices_begins, void* out,
+                                                              hipattn_stream stream) {
+    return paged_attention_impl(desc, q, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins,
+                                block_indices, block_indices_begins, out, nullptr, 0, stream, true);
 }

@@ -149,4 +149,7 @@ hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t str
 
 // Schedule option by name (see paged_decode.hip); value < 0 restores the default.  false: no such option.
 bool set_option(const char* name, int value);
+// Address and size of the current device's copy of the static scratch array (resolved once per device).
+hipError_t paged_static_scratch(void** ptr, size_t* bytes);
+
 }  // namespace hipattn

@@ -948,6 +948,35 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     p.max_q_tiles = query_tile_bound(p);
 }
 
+// ---- scratch of the entry point that allocates nothing (hipattn_paged_attention_noalloc) ------
+// A file-scope device array stands in for the caller's workspace: every GPU the library runs on
+// holds its own copy until the process ends.  In host code the array's name is not a device
+// address; the address on the current device comes from hipGetSymbolAddress, once per device, and
+// that pointer is what kernels and host calls get.  Calls that overlap on one GPU share the array
+// and race; it keeps the previous call's contents (the plan clears the ticket counters, everything
+// else is written before it is read).
+constexpr size_t kStaticScratchBytes = HIPATTN_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+hipError_t paged_static_scratch(void** ptr, size_t* bytes) {
+    static std::mutex mutex;
+    static void* address[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(mutex);
+    if (!address[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        address[dev] = p;
+    }
+    *ptr = address[dev];
+    *bytes = kStaticScratchBytes;
+    return hipSuccess;
+}
+
 // One side stream and a fork/join pair of events per device, made on first use and kept until the
 // process ends.  The mutex keeps the record/wait pairs of concurrent callers apart.
 struct SideStream {

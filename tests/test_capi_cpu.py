@@ -62,3 +62,11 @@ def test_non_compute_calls_work_without_a_device():
     assert L.hipattn_set_option(b"decode_switch_cost", -1) == capi.OK
     assert L.hipattn_set_option(b"no_such_option", 1) == capi.INVALID_ARGUMENT
     assert b"no_such_option" in L.hipattn_last_error_string()
+    # the entry point that allocates nothing refuses what its static scratch cannot hold before it
+    # touches any device
+    huge = capi.PaDesc(capi.F16, capi.F16, capi.F16, capi.F16, 128, 8, 128, 32, 8, 4096, 4096, 64, 0, 0.0, 0, 0)
+    assert L.hipattn_paged_attention_workspace_size(ctypes.byref(huge), ctypes.byref(n)) == capi.OK
+    assert n.value > capi.NOALLOC_SCRATCH_BYTES
+    one = ctypes.c_void_p(16)
+    assert L.hipattn_paged_attention_noalloc(ctypes.byref(huge), one, one, one, one, one, one, one, one, one, one,
+                                             None) == capi.WORKSPACE_TOO_SMALL
