@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu] [--no-extra] [--no-plugin]
 
 Prints ONE JSON line.  The headline is the fp16 paged-attention decode step (configuration 3
 of BASELINE.json): a "step" is one hipattn_paged_attention call on the whole synthetic batch
@@ -11,8 +11,10 @@ the average duration of the dominant kernel (the split-context decode kernel), m
 HIP events recorded by the library around that launch.  Unless --no-extra is given, the other
 configurations are measured the same way and reported under "workloads" in the same line
 (c2: bf16 causal prefill SDPA in TFLOP/s against the dense bf16 MFMA peak; c4: u8-KV decode;
-c5: mixed chunked prefill + decode).  `cpu_baseline` times the CPU oracle (a restatement, not
-OpenVINO's CPU plugin: OpenVINO is not installed) on a bounded sample of the same workload.
+c5: mixed chunked prefill + decode), each with a `cpu_baseline` of its own.  `cpu_baseline` times
+the CPU oracle (a restatement, not OpenVINO's CPU plugin: OpenVINO is not installed) on a bounded
+sample of the same workload.  `plugin_ms_per_step` of the headline workload is the same step through
+the plugin layer's InferRequest::infer with device-resident tensors.
 """
 import argparse
 import json
@@ -110,6 +112,49 @@ def bench_paged(hip, case, steps, warmup, name):
     return res
 
 
+def bench_paged_through_plugin(hip, case, steps, warmup):
+    """The same step through the plugin layer: Plugin -> CompiledModel -> InferRequest::infer ->
+    PagedAttentionOp -> C ABI, every tensor device-resident (remote tensors over the buffers of the raw
+    measurement, the output included), the scalar inputs on the host.  Host wall time per infer():
+    each call enqueues the operator on the worker's stream and waits for it, as OpenVINO's synchronous
+    infer does, so this is launch + execution + synchronisation, not a pipelined rate."""
+    from openvino_contrib_amd import device_case as H
+    from openvino_contrib_amd import plugin_capi as P
+    import numpy as np
+
+    dev = H.PagedDeviceCase(hip, case)
+    plugin = P.Plugin()
+    compiled = plugin.compile_model(P.Model.paged_attention(case["q_dtype"], case["kv_dtype"], case["cache_dtype"],
+                                                            case["Hq"], case["Hkv"], case["D"], case["block_size"]))
+    req = compiled.create_infer_request()
+    T, S = case["T"], case["S"]
+    row = case["key_cache"].shape[3] // hip.DTYPE_BYTES[case["cache_dtype"]]
+    cache_shape = list(case["key_cache"].shape[:3]) + [row]
+    req.set_device_input(0, dev.q.ptr, case["q_dtype"], [T, case["Hq"] * case["D"]])
+    req.set_device_input(1, dev.k_new.ptr, case["kv_dtype"], [T, case["Hkv"] * case["D"]])
+    req.set_device_input(2, dev.v_new.ptr, case["kv_dtype"], [T, case["Hkv"] * case["D"]])
+    req.set_device_input(3, dev.key_cache.ptr, case["cache_dtype"], cache_shape)
+    req.set_device_input(4, dev.value_cache.ptr, case["cache_dtype"], cache_shape)
+    req.set_device_input(5, dev.past_lens.ptr, P.I32, [S])
+    req.set_device_input(6, dev.subsequence_begins.ptr, P.I32, [S + 1])
+    req.set_device_input(7, dev.block_indices.ptr, P.I32, [len(case["block_indices"])])
+    req.set_device_input(8, dev.block_indices_begins.ptr, P.I32, [S + 1])
+    req.set_input(9, np.zeros((0,), np.float32), P.F32)
+    req.set_input(10, np.array([case["sliding_window"]], np.int32), P.I32)
+    req.set_input(11, np.zeros((0,), np.float32), P.F32)
+    req.set_input(12, np.array([case["max_context_len"]], np.int32), P.I32)
+    req.set_device_output(0, dev.out.ptr, case["q_dtype"], [T, case["Hq"] * case["D"]])
+    for _ in range(max(warmup, 20)):
+        req.infer()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        req.infer()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    del req, compiled, plugin
+    dev.free()
+    return ms
+
+
 def bench_sdpa(hip, case, steps, warmup, name):
     from openvino_contrib_amd import workloads as W
 
@@ -131,28 +176,35 @@ def bench_sdpa(hip, case, steps, warmup, name):
     return res
 
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script (summaries and the scaling against a plain 1 GiB copy: profiles/*.txt).  Hardware
-# counters cannot be read from inside this process, so these are the recorded figures for the
-# default seeds; None where no counter run exists.
-MEASURED_TRAFFIC_BYTES = {
-    "c3": (563515.7 * 2.0 + 3032.7) * 1024,
-    "c4": (1220078.5 * 2.0 + 10000.2) * 1024,
-    "c2": (49294.2 * 2.0 + 65536.0) * 1024,
-    "c5": (786210.7 * 2.0 + 6033.6) * 1024,  # the decode kernel of the mixed step
+# HBM bytes per launch of the dominant kernel.  Hardware counters cannot be read from inside this
+# process, so these are RECORDED figures: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch from
+# rocprofv3 --pmc runs of this script on the default seeds (scale factors from a plain 1 GiB copy,
+# profiles/copy_calibration.txt); the file each pair of numbers was read from is named beside it.
+RECORDED_TRAFFIC = {
+    "c3": ((563515.7 * 2.0 + 3032.7) * 1024, "profiles/paged_decode_kernel_config3_fp16.txt"),
+    "c4": ((1220078.5 * 2.0 + 10000.2) * 1024, "profiles/paged_decode_kernel_config4_u8.txt"),
+    "c2": ((49293.6 * 2.0 + 65536.0) * 1024, "profiles/sdpa_flash_kernel_config2_bf16.txt"),
+    "c5": ((786210.7 * 2.0 + 6033.6) * 1024, "profiles/paged_attention_config5_mixed.txt"),  # the decode kernel of the mixed step
 }
 
 
-def roofline_hbm(res, traffic=None):
+def recorded_traffic(w):
+    t = RECORDED_TRAFFIC.get(w)
+    return (t[0], "recorded, not measured in this run: " + t[1]) if t else (None, None)
+
+
+def roofline_hbm(res, w):
     a = res["decode_kv_bytes"] / (res["dominant_kernel_ms"] * 1e-3) / 1e9
+    traffic, source = recorded_traffic(w)
     return {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
-            "traffic": traffic, "kernel": "paged_decode_kernel"}
+            "traffic": traffic, "traffic_source": source, "kernel": "paged_decode_kernel"}
 
 
 def roofline_mfma(res):
     a = res["flops"] / (res["dominant_kernel_ms"] * 1e-3) / 1e12
+    traffic, source = recorded_traffic("c2")
     return {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get("c2"),
+            "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic, "traffic_source": source,
             "kernel": "sdpa_flash_kernel"}
 
 
@@ -234,6 +286,7 @@ def main():
                          "which only count bytes)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="measure the headline workload only")
+    ap.add_argument("--no-plugin", action="store_true", help="skip the timing through the plugin layer")
     args = ap.parse_args()
     CLOCK_RAMP_MS = args.ramp_ms
     if args.gpus != 1:
@@ -307,7 +360,7 @@ def main():
             r["roofline"] = roofline_mfma(r)
         else:
             r = bench_paged(hip, case, args.steps, args.warmup, names[w])
-            r["roofline"] = roofline_hbm(r, MEASURED_TRAFFIC_BYTES.get(w))
+            r["roofline"] = roofline_hbm(r, w)
             if w in ("c5", "c5u8"):
                 t_ideal = max(r["kv_bytes"] / (HBM_PEAK_GBS * 1e9), r["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                 r["ideal_ms"] = t_ideal * 1e3
@@ -317,9 +370,19 @@ def main():
                                          "frac_of_ideal is the one for this step")
         log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f"
             % (w, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"]))
-        if not args.no_cpu and w == args.workload:
-            cpu = cpu_baseline_sdpa(case) if w == "c2" else cpu_baseline_paged(case)
-            log("cpu baseline:", cpu)
+        if w == args.workload and w != "c2" and not args.no_plugin:
+            r["plugin_ms_per_step"] = bench_paged_through_plugin(hip, case, args.steps, args.warmup)
+            r["plugin_overhead_ms"] = r["plugin_ms_per_step"] - r["ms_per_step"]
+            log("%s through InferRequest::infer: %.3f ms/step (raw C ABI, back to back: %.3f)"
+                % (w, r["plugin_ms_per_step"], r["ms_per_step"]))
+        if not args.no_cpu:
+            # the headline gets the larger budget; every other workload a bounded sample beside its figure
+            budget = 12.0 if w == args.workload else 6.0
+            c = cpu_baseline_sdpa(case, budget) if w == "c2" else cpu_baseline_paged(case, budget)
+            r["cpu_baseline"] = c
+            if w == args.workload:
+                cpu = c
+            log("%s cpu baseline:" % w, c)
         results[w] = r
         del case
 

@@ -86,6 +86,14 @@ hipattn_status hipattn_memcpy_d2d_async(void* device_dst, const void* device_src
 /* byte fill done by a kernel (safe to record into a captured graph) */
 hipattn_status hipattn_fill_async(void* device_dst, int byte_value, size_t bytes, hipattn_stream stream);
 
+/* out = a + b over `count` elements of equal shape: the element-wise sum the reference runs as
+ * AddCudaOp (src/ops/add.cpp:17-43, src/kernels/details/elementwise_binary.cuh:24-46), here for the
+ * stateful models around the attention operators.  dtype: HIPATTN_F32 / F16 / BF16 (added in fp32,
+ * rounded once) or HIPATTN_I32. */
+#define HIPATTN_I32 100
+hipattn_status hipattn_add_async(void* device_out, const void* device_a, const void* device_b, int64_t count,
+                                 int dtype, hipattn_stream stream);
+
 hipattn_status hipattn_event_create(hipattn_event* event);
 hipattn_status hipattn_event_destroy(hipattn_event event);
 hipattn_status hipattn_event_record(hipattn_event event, hipattn_stream stream);

@@ -85,16 +85,20 @@ def build_bench_tools():
 
 
 PLUGIN_LIB_PATH = os.path.join(CSRC, "libhip_plugin.so")
-PLUGIN_SOURCES = ["plugin/ops.cpp", "plugin/plugin.cpp", "plugin/c_api.cpp"]
+PLUGIN_SOURCES = ["plugin/src/hip_ops.cpp", "plugin/src/hip_plugin.cpp", "plugin/src/hip_create_plugin.cpp",
+                  "plugin/test_facade/c_api.cpp"]
 
 
 def build_plugin():
-    """Compile the host-side plugin layer (plain C++17, reaches the GPU only through libhipattn's C ABI)."""
+    """Compile the host-side plugin layer (plain C++17, reaches the GPU only through libhipattn's C ABI)
+    against the stand-in for OpenVINO's developer headers (plugin/standin/), plus the C facade the
+    tests drive it through.  Where the OpenVINO developer package is installed, plugin/CMakeLists.txt
+    builds the same sources against the real headers instead."""
     if not os.path.exists(LIB_PATH):
         raise RuntimeError("build libhipattn.so first")
     cxx = shutil.which("g++") or "g++"
     cmd = [cxx, "-std=c++17", "-O2", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wextra", "-pthread",
-           "-I" + INCLUDE, "-I" + os.path.join(CSRC, "plugin")]
+           "-I" + INCLUDE, "-I" + os.path.join(CSRC, "plugin", "src"), "-I" + os.path.join(CSRC, "plugin", "standin")]
     cmd += [os.path.join(CSRC, s) for s in PLUGIN_SOURCES]
     cmd += ["-L" + CSRC, "-lhipattn", "-Wl,-rpath,$ORIGIN", "-o", PLUGIN_LIB_PATH]
     r = subprocess.run(cmd, capture_output=True, text=True)

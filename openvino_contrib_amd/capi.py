@@ -104,6 +104,7 @@ SYMBOLS = {
     "hipattn_memcpy_d2h_async": (_i, [_vp, _vp, _sz, _vp]),
     "hipattn_memcpy_d2d_async": (_i, [_vp, _vp, _sz, _vp]),
     "hipattn_fill_async": (_i, [_vp, _i, _sz, _vp]),
+    "hipattn_add_async": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, _vp]),
     "hipattn_event_create": (_i, [_P(_vp)]),
     "hipattn_event_destroy": (_i, [_vp]),
     "hipattn_event_record": (_i, [_vp, _vp]),

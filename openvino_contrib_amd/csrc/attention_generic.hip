@@ -219,6 +219,26 @@ __global__ void fill_bytes_kernel(uint8_t* dst, uint8_t value, size_t bytes) {
     for (; i < bytes; i += stride) dst[i] = value;
 }
 
+// out[i] = a[i] + b[i]; the floating types add in fp32 and round once, i32 wraps
+__global__ void add_kernel(const void* a, const void* b, void* out, int64_t n, int dtype) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        if (dtype < 0)
+            ((int32_t*)out)[i] = (int32_t)((uint32_t)((const int32_t*)a)[i] + (uint32_t)((const int32_t*)b)[i]);
+        else
+            store_scalar(out, i, dtype, load_scalar(a, i, dtype) + load_scalar(b, i, dtype));
+    }
+}
+
+hipError_t launch_add(const void* a, const void* b, void* out, int64_t n, int dtype, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(add_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a, b, out, n, dtype);
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t stream) {
     if (bytes == 0) return hipSuccess;
     size_t blocks = (bytes + 255) / 256;

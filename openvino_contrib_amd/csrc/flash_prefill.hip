@@ -42,34 +42,6 @@ namespace hipattn {
 
 namespace flash {
 
-// Diagnostic build only (a probe that includes this file with HIPATTN_FLASH_TRACE defined):
-// thread 0 of every workgroup stores wall clock (100 MHz) and shader clock at entry and exit.
-#ifdef HIPATTN_FLASH_TRACE
-__device__ long long* g_flash_wg_trace = nullptr;
-__device__ long long* g_flash_phase_trace = nullptr;  // per wavefront: 8 accumulated phase times (shader clocks)
-__device__ long long* g_flash_raw_trace = nullptr;    // workgroup 0: raw stamps of tiles 10 and 11, per wavefront
-struct PhaseClock {
-    long long acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    long long last = 0;
-    long long raw[8];
-    int tile = 0;
-};
-// phase k = time since the previous stamp
-#define FLASH_STAMP(clk, k)                                               \
-    do {                                                                  \
-        __builtin_amdgcn_sched_barrier(0);                                \
-        const long long stamp_ = (long long)__builtin_readcyclecounter(); \
-        __builtin_amdgcn_sched_barrier(0);                                \
-        (clk).acc[k] += stamp_ - (clk).last;                              \
-        (clk).last = stamp_;                                              \
-        if ((clk).tile == 10) (clk).raw[k] = stamp_;                      \
-    } while (0)
-#else
-#define FLASH_STAMP(clk, k) \
-    do {                    \
-    } while (0)
-#endif
-
 constexpr int kD = 128;
 constexpr int kTileQ = 128;   // query rows per group of four wavefronts
 constexpr int kTileK = 64;    // keys per LDS tile
@@ -836,10 +808,6 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     vec8 pf[4];
     tile_scores<kBf16>(k_stage(0), f, qf, st.neg_ref, s);
     phase_barrier(recent);
-#ifdef HIPATTN_FLASH_TRACE
-    PhaseClock clk;
-    clk.last = (long long)__builtin_readcyclecounter();
-#endif
     // The two phases of tile j.  Both groups run every tile of the workgroup's key range: a tile
     // outside a group's own range is fully masked and contributes probabilities of zero.  The
     // restrict qualifiers tell the compiler that the LDS writes of the asynchronous loads cannot
@@ -856,10 +824,6 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         lds_byte* __restrict__ const k_fill = k_ring + i_kf * kKBytes;
         lds_byte* __restrict__ const v_fill = v_ring + i_vf * kKBytes;
         // ---- vector phase
-#ifdef HIPATTN_FLASH_TRACE
-        clk.tile = j;
-#endif
-        FLASH_STAMP(clk, 0);
         if constexpr (kU8) {
             // rows fetched one iteration ago go into their stages, two phases before their first
             // use; the rows of this iteration's batch are fetched into registers
@@ -880,19 +844,16 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         } else {
             recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
         }
-        FLASH_STAMP(clk, 1);
         tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
         // (the probabilities are complete before the barrier: the compiler may not move their
         // arithmetic into the matrix phase)
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) asm volatile("" : "+v"(pf[ks]));
-        FLASH_STAMP(clk, 2);
         // the matrix phase runs at raised priority (set before the barrier, so that it holds from
         // the first instruction after it): otherwise the other group's instruction stream, which
         // never stalls for long, keeps this wavefront's MFMAs from issuing
         __builtin_amdgcn_s_setprio(3);
         if (group == 0) phase_barrier(recent);  // (group 1 passes from its vector phase straight into its matrix phase)
-        FLASH_STAMP(clk, 3);
         // ---- matrix phase
         // fragment addresses of this tile: per-lane offset + stage address, so that every read is
         // one XOR with a constant plus an immediate offset (the stage addresses are multiples of
@@ -906,7 +867,6 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         else
             tile_accumulate<kBf16>(zero, fs, pf, o);
         __builtin_amdgcn_s_setprio(0);
-        FLASH_STAMP(clk, 5);
         // The next iteration's stages and source rows are worked out here, where the wavefront would
         // otherwise only wait at the barrier for the other group's vector phase; behind the barrier
         // this scalar arithmetic would sit at the head of its own vector phase.
@@ -927,19 +887,9 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         }
         asm volatile("" : "+s"(i_kn), "+s"(i_vc), "+s"(i_kf), "+s"(i_vf));
         if (group == 1) phase_barrier(recent);
-        FLASH_STAMP(clk, 6);
     };
     for (int j = 0; j < n - 1; j++) two_phases(j, false);
     two_phases(n - 1, true);
-#ifdef HIPATTN_FLASH_TRACE
-    if (g_flash_phase_trace && lane == 0) {
-        long long* r = g_flash_phase_trace + ((int64_t)blockIdx.x * 8 + wave) * 8;
-        for (int k = 0; k < 7; k++) r[k] = clk.acc[k];
-        r[7] = n;
-    }
-    if (g_flash_raw_trace && lane == 0 && blockIdx.x == 0 && n >= 12)
-        for (int k = 0; k < 8; k++) g_flash_raw_trace[wave * 16 + k] = clk.raw[k];
-#endif
 
     // ---- normalise and store
     float l_lo, l_hi;
@@ -1037,27 +987,8 @@ __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t
 template <bool kBf16>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_kernel(SdpaParams p) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
-#ifdef HIPATTN_FLASH_TRACE
-    long long w0 = 0, c0 = 0;
-    if (g_flash_wg_trace) {
-        w0 = wall_clock64();
-        c0 = (long long)__builtin_readcyclecounter();
-    }
-#endif
     const Tile t0 = sdpa_group_tile(p, 0), t1 = sdpa_group_tile(p, 1);
     run_both<kBf16, false, false>(t0, t1, lds, p.scale);
-#ifdef HIPATTN_FLASH_TRACE
-    if (g_flash_wg_trace && threadIdx.x == 0) {
-        long long* r = g_flash_wg_trace + (int64_t)blockIdx.x * 8;
-        r[0] = w0;
-        r[1] = wall_clock64();
-        r[2] = c0;
-        r[3] = (long long)__builtin_readcyclecounter();
-        r[4] = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID
-        r[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
-        r[6] = t0.pos0 / kTileQ;
-    }
-#endif
 }
 
 // One workgroup per (128-row query tile of a multi-token sequence, pair of query heads) or, with an

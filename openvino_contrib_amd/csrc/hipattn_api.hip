@@ -292,6 +292,16 @@ HIPATTN_EXPORT hipattn_status hipattn_fill_async(void* device_dst, int byte_valu
     return HIPATTN_OK;
 }
 
+HIPATTN_EXPORT hipattn_status hipattn_add_async(void* device_out, const void* device_a, const void* device_b,
+                                                int64_t count, int dtype, hipattn_stream stream) {
+    if (count < 0) return fail(HIPATTN_INVALID_ARGUMENT, "add: negative count");
+    if (count == 0) return HIPATTN_OK;
+    if (!device_out || !device_a || !device_b) return fail(HIPATTN_INVALID_ARGUMENT, "add: null pointer");
+    if (dtype != HIPATTN_I32 && !is_float_dtype(dtype)) return fail(HIPATTN_INVALID_ARGUMENT, "add: dtype %d", dtype);
+    HIP_TRY(hipattn::launch_add(device_a, device_b, device_out, count, dtype == HIPATTN_I32 ? -1 : dtype, as_stream(stream)));
+    return HIPATTN_OK;
+}
+
 HIPATTN_EXPORT hipattn_status hipattn_event_create(hipattn_event* event) {
     if (!event) return fail(HIPATTN_INVALID_ARGUMENT, "event_create: null output");
     hipEvent_t e;

@@ -146,6 +146,8 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream);  // flash over the block table (needs the plan)
 
 hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t stream);
+// out = a + b over n elements; dtype is a HIPATTN_F32 / F16 / BF16 value, or -1 for int32
+hipError_t launch_add(const void* a, const void* b, void* out, int64_t n, int dtype, hipStream_t stream);
 
 // Schedule option by name (see paged_decode.hip); value < 0 restores the default.  false: no such option.
 bool set_option(const char* name, int value);

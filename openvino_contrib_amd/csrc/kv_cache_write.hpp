@@ -45,11 +45,60 @@ __device__ __forceinline__ uint32_t float_to_bits16(float x, int dtype) {
     return dtype == HIPATTN_F16 ? float_to_f16_bits(x) : float_to_bf16_bits(x);
 }
 
+// Eight consecutive elements (d0 .. d0 + 7) of a new 128-element row, given as the 16 bytes `raw` of
+// the kv type, go into the cache row at `row`, converted or quantised.  Sixteen consecutive lanes
+// (a 16-lane group) hold one row between them; the u8 quantiser's minimum and maximum are reduced
+// over that group, so every lane of the group must call this together (`active` false: take part
+// in the reduction, store nothing).  The arithmetic is that of the element-wise path below, value
+// for value (the quantiser's minimum and maximum do not depend on the order of the reduction).
+__device__ __forceinline__ void kv_store_row8(const KvWriteParams& p, uint4_t raw, uint8_t* row, int d0, bool active,
+                                              int lane) {
+    if (p.cache_dtype == p.kv_dtype) {
+        if (active) *(uint4_t*)(row + d0 * 2) = raw;
+        return;
+    }
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[i] = bits16_to_float((raw[i >> 1] >> ((i & 1) * 16)) & 0xffffu, p.kv_dtype);
+    if (p.cache_dtype == HIPATTN_U8) {
+        float mn = x[0], mx = x[0];
+#pragma unroll
+        for (int i = 1; i < 8; i++) {
+            mn = fminf(mn, x[i]);
+            mx = fmaxf(mx, x[i]);
+        }
+#pragma unroll
+        for (int m = 1; m < 16; m <<= 1) {  // over the 16 lanes of the row
+            mn = fminf(mn, __shfl_xor(mn, m, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+        }
+        float scale = (mx - mn) / 255.0f;
+        if (scale == 0.0f) scale = 0.0001f;
+        const float zp = -mn / scale + 0.0f;  // -0 becomes +0
+        const float inv = 1.0f / scale;
+        uint32_t q[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = (uint32_t)fminf(fmaxf(rintf(fmaf(x[i], inv, zp)), 0.0f), 255.0f);
+        uint2_t packed;
+        packed[0] = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+        packed[1] = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
+        if (active) {
+            *(uint2_t*)(row + 8 + d0) = packed;
+            if ((lane & 15) == 0) *(float2*)row = make_float2(scale, zp);
+        }
+    } else {  // the other 16-bit type
+        uint4_t out;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            out[i] = float_to_bits16(x[2 * i], p.cache_dtype) | (float_to_bits16(x[2 * i + 1], p.cache_dtype) << 16);
+        if (active) *(uint4_t*)(row + d0 * 2) = out;
+    }
+}
+
 // Head size 128 with 16-bit new rows (p.vector_rows): the wavefront takes four kv heads of one
 // token, which lie side by side in k_new / v_new, with one 16-byte load per lane for K and one for
 // V -- 16 lanes and 8 elements each to a head -- and writes the cache rows with 16-byte (16-bit
-// caches) or 8-byte (u8) stores.  The arithmetic is that of the element-wise path below, value
-// for value (the quantiser's minimum and maximum do not depend on the order of the reduction).
+// caches) or 8-byte (u8) stores.
 __device__ __forceinline__ void kv_cache_write_rows128(const KvWriteParams& p, int64_t wv, int lane) {
     const int chunks = (p.num_heads_kv + 3) >> 2;
     const int t = (int)(wv / chunks);
@@ -64,51 +113,23 @@ __device__ __forceinline__ void kv_cache_write_rows128(const KvWriteParams& p, i
     const uint4_t vraw = *(const uint4_t*)((const uint16_t*)p.v_new + src_off);
     const int64_t rb = cache_row_bytes(p.cache_dtype, 128);
     const int64_t row_off = (((int64_t)pb * p.num_heads_kv + hh) * p.block_size + pos % p.block_size) * rb;
-#pragma unroll
-    for (int which = 0; which < 2; which++) {
-        const uint4_t raw = which ? vraw : kraw;
-        uint8_t* row = (which ? p.value_cache : p.key_cache) + row_off;
-        if (p.cache_dtype == p.kv_dtype) {
-            if (active) *(uint4_t*)(row + d0 * 2) = raw;
-            continue;
-        }
-        float x[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) x[i] = bits16_to_float((raw[i >> 1] >> ((i & 1) * 16)) & 0xffffu, p.kv_dtype);
-        if (p.cache_dtype == HIPATTN_U8) {
-            float mn = x[0], mx = x[0];
-#pragma unroll
-            for (int i = 1; i < 8; i++) {
-                mn = fminf(mn, x[i]);
-                mx = fmaxf(mx, x[i]);
-            }
-#pragma unroll
-            for (int m = 1; m < 16; m <<= 1) {  // over the 16 lanes of the head
-                mn = fminf(mn, __shfl_xor(mn, m, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, m, 64));
-            }
-            float scale = (mx - mn) / 255.0f;
-            if (scale == 0.0f) scale = 0.0001f;
-            const float zp = -mn / scale + 0.0f;  // -0 becomes +0
-            const float inv = 1.0f / scale;
-            uint32_t q[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) q[i] = (uint32_t)fminf(fmaxf(rintf(fmaf(x[i], inv, zp)), 0.0f), 255.0f);
-            uint2_t packed;
-            packed[0] = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
-            packed[1] = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
-            if (active) {
-                *(uint2_t*)(row + 8 + d0) = packed;
-                if ((lane & 15) == 0) *(float2*)row = make_float2(scale, zp);
-            }
-        } else {  // the other 16-bit type
-            uint4_t out;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                out[i] = float_to_bits16(x[2 * i], p.cache_dtype) | (float_to_bits16(x[2 * i + 1], p.cache_dtype) << 16);
-            if (active) *(uint4_t*)(row + d0 * 2) = out;
-        }
-    }
+    kv_store_row8(p, kraw, p.key_cache + row_off, d0, active, lane);
+    kv_store_row8(p, vraw, p.value_cache + row_off, d0, active, lane);
+}
+
+// The K row and the V row of ONE (token, kv head) pair, head size 128, 16-bit new rows, written by
+// one wavefront that already knows the slot: lanes 0-15 take the K row, lanes 16-31 the V row.
+// This is what a decode wavefront does for the sequence whose last cache block it is about to read.
+__device__ __forceinline__ void kv_cache_write_pair128(const KvWriteParams& p, int t, int h, int pb, int pos, int lane) {
+    const int which = lane >> 4;  // 0: K, 1: V, 2 and 3: idle
+    const bool active = which < 2;
+    const int d0 = (lane & 15) * 8;
+    const int64_t src_off = ((int64_t)t * p.num_heads_kv + h) * 128 + d0;
+    const uint16_t* src = (const uint16_t*)((which & 1) ? p.v_new : p.k_new);
+    const uint4_t raw = *(const uint4_t*)(src + src_off);
+    const int64_t rb = cache_row_bytes(p.cache_dtype, 128);
+    const int64_t row_off = (((int64_t)pb * p.num_heads_kv + h) * p.block_size + pos % p.block_size) * rb;
+    kv_store_row8(p, raw, ((which & 1) ? p.value_cache : p.key_cache) + row_off, d0, active, lane);
 }
 
 // Wavefront `wv` of the writer: the K rows and the V rows of one token for p.heads_per_wave kv

@@ -68,11 +68,11 @@ constexpr int kD = 128;   // head size of the fast path
 constexpr int kBS = 32;   // cache block size of the fast path
 
 struct alignas(32) DecodeRange {
-    int valid;        // the record is a single-token row with something to attend
+    int write_pos;    // cache position of the row's own new token when it has a slot in the table, else -1
     int token;        // row of q / out
     int ctx;          // attended positions end (exclusive)
     int j0;           // attended positions begin
-    int first_block;  // logical block holding j0
+    int new_begin;    // cache position of the first token its sequence contributes to this batch (past_lens)
     int nb;           // number of logical blocks attended (0 when not valid)
     int table_begin;  // offset of the sequence's block table in block_indices
     int empty_row;    // a single-token row with nothing to attend: its output row is zeros
@@ -105,23 +105,33 @@ __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int i)
     DecodeRange r;
     int s = i, pos_in_seq = 0;
     bool single = true;
+    // everything a row of an ordinary decode batch needs is fetched at once, on the guess that row i is
+    // sequence i (one level of memory latency instead of two); a guess that fails is redone below
+    const int b0 = p.subsequence_begins[i], b1 = p.subsequence_begins[i + 1];
+    int tb0 = p.block_indices_begins[i], tb1 = p.block_indices_begins[i + 1], past = p.past_lens[i];
     if (p.max_q_tiles == 0) {
-        if (!(p.subsequence_begins[i] == i && p.subsequence_begins[i + 1] == i + 1)) s = sequence_of_token(p, i);
+        if (!(b0 == i && b1 == i + 1)) {
+            s = sequence_of_token(p, i);
+            tb0 = p.block_indices_begins[s];
+            tb1 = p.block_indices_begins[s + 1];
+            past = p.past_lens[s];
+        }
         pos_in_seq = i - p.subsequence_begins[s];
         r.token = i;
     } else {
-        r.token = p.subsequence_begins[s];
-        single = (p.subsequence_begins[s + 1] - r.token == 1);
+        r.token = b0;
+        single = (b1 - b0 == 1);
     }
-    const int table_tokens = (p.block_indices_begins[s + 1] - p.block_indices_begins[s]) * p.block_size;
-    r.ctx = min(p.past_lens[s] + pos_in_seq + 1, table_tokens);
+    const int table_tokens = (tb1 - tb0) * p.block_size;
+    r.ctx = min(past + pos_in_seq + 1, table_tokens);
     r.j0 = 0;
     if (p.sliding_window > 0 && r.ctx - p.sliding_window > 0) r.j0 = r.ctx - p.sliding_window;
-    r.valid = single && r.ctx > 0;
+    const bool valid = single && r.ctx > 0;
+    r.write_pos = (single && past + pos_in_seq < table_tokens) ? past + pos_in_seq : -1;
     r.empty_row = single && r.ctx <= 0;
-    r.first_block = r.j0 / p.block_size;
-    r.nb = r.valid ? (r.ctx + p.block_size - 1) / p.block_size - r.first_block : 0;
-    r.table_begin = p.block_indices_begins[s];
+    r.new_begin = past;
+    r.nb = valid ? (r.ctx + p.block_size - 1) / p.block_size - r.j0 / p.block_size : 0;
+    r.table_begin = tb0;
     return r;
 }
 
@@ -407,6 +417,16 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
 // equal pieces then equalises time, not just bytes.
 __device__ __forceinline__ int line_units(int nb, int switch_cost) { return nb > 0 ? nb + switch_cost : 0; }
 
+__device__ __forceinline__ void zero_output_row(const PagedParams& p, int token) {
+    const int64_t n = (int64_t)p.num_heads_q * p.head_dim, o0 = (int64_t)token * n;
+    for (int64_t e = 0; e < n; e++) {
+        if (p.out_dtype == HIPATTN_F32)
+            ((float*)p.out)[o0 + e] = 0.0f;
+        else
+            ((uint16_t*)p.out)[o0 + e] = 0;
+    }
+}
+
 // ---- plan ----------------------------------------------------------------------------------
 // Exclusive prefix sums over the sequences of (a) attended blocks of decode sequences and
 // (b) 128-row query tiles of multi-token sequences.  One workgroup; sequences are split evenly
@@ -487,15 +507,7 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
         p.tile_prefix[s] = tile;
         const DecodeRange rg = decode_range(p, s);
         ((DecodeRange*)p.seq_info)[s] = rg;
-        if (rg.empty_row) {  // (rare: an empty block table) nothing will visit this row
-            const int64_t n = (int64_t)p.num_heads_q * p.head_dim, o0 = (int64_t)rg.token * n;
-            for (int64_t e = 0; e < n; e++) {
-                if (p.out_dtype == HIPATTN_F32)
-                    ((float*)p.out)[o0 + e] = 0.0f;
-                else
-                    ((uint16_t*)p.out)[o0 + e] = 0;
-            }
-        }
+        if (rg.empty_row) zero_output_row(p, rg.token);  // (rare: an empty block table) nothing will visit this row
         blk += line_units(rg.nb, p.switch_cost);
         tile += (qlen > 1 && p.max_q_tiles > 0) ? (qlen + 127) / 128 : 0;
     }
@@ -605,17 +617,69 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
     }
 }
 
+// Pure decode batches of up to kSelfPlanMaxRows rows need no prologue launch: every wavefront works
+// out the schedule for itself (one record per row into LDS, lane-parallel, and a wavefront scan for
+// the prefix sums), which is shorter than the chain of dependent global loads through a plan another
+// kernel left behind, and the wavefront that is about to read the last cache block of a (row, kv
+// head) first writes that row's new K and V rows into it -- the operator's cache write, done by
+// the only wavefront that needs its result during this call.  Wavefront 0 leaves the plan in the
+// workspace for the merge kernel.
+constexpr int kSelfPlanMaxRows = 256;
+
 // kWaves wavefronts to a workgroup.  1 is the ordinary launch.  With 8 a workgroup owns a compute
 // unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
 // leave the others free for a kernel that runs beside this one.
-template <bool kU8, bool kBf16, int kWaves>
-__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p) {
+template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false>
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
+    static_assert(!kSelfPlan || kWaves == 1, "a wavefront that plans for itself is a workgroup of its own");
     const int w = kWaves == 1 ? blockIdx.x : blockIdx.x * kWaves + (threadIdx.x >> 6);
     const int lane = kWaves == 1 ? threadIdx.x : (threadIdx.x & 63), n16 = lane & 15, kg = lane >> 4;
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
     const float c = p.scale * kLog2e;
-    const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
+    __shared__ DecodeRange plan_rec[kSelfPlan ? kSelfPlanMaxRows : 1];
+    __shared__ int plan_prefix[kSelfPlan ? kSelfPlanMaxRows + 1 : 1];
+    if constexpr (kSelfPlan) {
+        int carry = 0;
+        for (int base = 0; base < p.num_seqs; base += 64) {
+            const int i = base + lane;
+            DecodeRange rg;
+            int units = 0;
+            if (i < p.num_seqs) {
+                rg = decode_range(p, i);
+                units = line_units(rg.nb, p.switch_cost);
+                plan_rec[i] = rg;
+            }
+            int scan = units;  // inclusive scan over the wavefront
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int up = __shfl_up(scan, d, 64);
+                if (lane >= d) scan += up;
+            }
+            if (i < p.num_seqs) {
+                plan_prefix[i] = carry + scan - units;
+                if (w == 0) {  // for the merge kernel
+                    ((DecodeRange*)p.seq_info)[i] = rg;
+                    p.blk_prefix[i] = carry + scan - units;
+                    if (rg.empty_row) zero_output_row(p, rg.token);
+                }
+            }
+            carry += __shfl(scan, 63, 64);
+        }
+        if (lane == 0) {
+            plan_prefix[p.num_seqs] = carry;
+            if (w == 0) p.blk_prefix[p.num_seqs] = carry;
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the records are in LDS (the wavefront is the whole workgroup)
+        __builtin_amdgcn_wave_barrier();
+    }
+    auto prefix_at = [&](int i) -> int {
+        if constexpr (kSelfPlan)
+            return plan_prefix[i];
+        else
+            return p.blk_prefix[i];
+    };
+    const int64_t total = (int64_t)prefix_at(p.num_seqs) * Hkv;
     if (total <= 0) return;
     // eight to a workgroup: the plan has chosen how many of the launched wavefronts work
     const int num_waves = kWaves == 1 ? p.num_waves : p.plan_waves[0];
@@ -637,15 +701,32 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     if (p.dyn_pieces > 0 && lane == 0) ticket_lane0 = atomicAdd(p.dyn_counter + group, 1);
     int64_t L = line.begin(piece);
     const int64_t L_end = line.begin(piece + 1);
-    int s = L < L_end ? locate_sequence(p.blk_prefix, p.num_seqs, (int)(L / Hkv), lane) : 0;
+    int s = 0;
+    if (L < L_end) {
+        if constexpr (kSelfPlan) {  // the last row whose prefix is <= L / Hkv (the prefix is monotone)
+            const int x = (int)(L / Hkv);
+            int cnt = 0;
+            for (int base = 0; base < p.num_seqs; base += 64) {
+                const int i = base + lane;
+                cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(i < p.num_seqs && plan_prefix[i] <= x));
+            }
+            s = max(cnt - 1, 0);
+        } else {
+            s = locate_sequence(p.blk_prefix, p.num_seqs, (int)(L / Hkv), lane);
+        }
+    }
 
     while (L < L_end) {
-        while (s + 1 < p.num_seqs && (int64_t)p.blk_prefix[s + 1] * Hkv <= L) s++;  // next sequence with blocks
-        const DecodeRange rg = ((const DecodeRange*)p.seq_info)[s];
+        while (s + 1 < p.num_seqs && (int64_t)prefix_at(s + 1) * Hkv <= L) s++;  // next sequence with blocks
+        DecodeRange rg;
+        if constexpr (kSelfPlan)
+            rg = plan_rec[s];
+        else
+            rg = ((const DecodeRange*)p.seq_info)[s];
         const int nb = rg.nb;
         if (nb <= 0) break;  // cannot happen for a consistent plan; never loop forever
         const int seglen = nb + p.switch_cost;
-        const int64_t seq_L0 = (int64_t)p.blk_prefix[s] * Hkv;
+        const int64_t seq_L0 = (int64_t)prefix_at(s) * Hkv;
         const int h = (int)((L - seq_L0) / seglen);
         const int64_t seg_B0 = seq_L0 + (int64_t)h * seglen + p.switch_cost;  // line position of the segment's block 0
         const int64_t seg_L1 = seg_B0 + nb;                        // end of the segment
@@ -658,10 +739,26 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         const int n = (int)(to - from);  // blocks of this segment in this piece
         const bool whole = (n == nb);
         L = from;
-        const int lb0 = rg.first_block + b_rel;        // first logical block
+        const int lb0 = rg.j0 / kBS + b_rel;            // first logical block
         const int32_t* table = p.block_indices + rg.table_begin + lb0;
         const int64_t head_off = (int64_t)h * kBS * kRowBytes;
 
+        if constexpr (kSelfPlan) {
+            // The new tokens of this call whose cache rows this piece is about to read go into the cache
+            // first: the row's own token (in the segment's last block) and, when its sequence
+            // contributes several tokens to the batch, the tokens ahead of it.  The same wavefront
+            // stores and then loads, and the stores are waited for below; a token that several rows
+            // attend is written by each of their wavefronts with the same bytes.
+            if (do_write && rg.write_pos >= 0) {
+                const int q_lo = max(rg.new_begin, lb0 * kBS), q_hi = min(rg.write_pos, (lb0 + n) * kBS - 1);
+                for (int q = q_lo; q <= q_hi; q++) {  // (wave-uniform; one pass for a decode row)
+                    const int pb_new = p.block_indices[rg.table_begin + q / kBS];
+                    if (pb_new >= 0 && pb_new < p.num_blocks)
+                        kv_cache_write_pair128(wp, rg.token - (rg.write_pos - q), h, pb_new, q, lane);
+                }
+                if (q_lo <= q_hi) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the rows have reached the cache
+            }
+        }
         // Q^T operand: lane (head n16, kg) holds Q[head][kg*32 + i*8 .. +8]; padding heads are zero
         typename Op16<kBf16>::vec8 qf[4];
         float sumq = 0.0f;
@@ -1006,7 +1103,6 @@ static SideStream* side_stream() {
 
 hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
                              const KernelProbe& probe) {
-    // prologue: KV-cache write of the new tokens (optional) + plan, one launch
     KvWriteParams wp{};
     int write_blocks = 0;
     if (write) {
@@ -1014,8 +1110,29 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head_dim 128 only
         write_blocks = (int)((kv_write_wavefronts(wp) + 3) / 4);
     }
+    hipError_t e = hipSuccess;
+    // A pure decode batch of few rows is one launch less: the decode wavefronts plan for themselves
+    // and write the new rows (see kSelfPlanMaxRows).
+    const bool self_plan = p.max_q_tiles == 0 && p.num_seqs <= kSelfPlanMaxRows && p.dyn_pieces == 0 &&
+                           (!write || wp.vector_rows);
+    if (self_plan) {
+        if (probe.before) (void)hipEventRecord(probe.before, stream);
+        const int do_write = write ? 1 : 0;
+        if (p.cache_dtype == HIPATTN_U8)
+            hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, true>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, do_write);
+        else if (p.cache_dtype == HIPATTN_BF16)
+            hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, true>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, do_write);
+        else
+            hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, true>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, do_write);
+        e = hipGetLastError();
+        if (probe.after) (void)hipEventRecord(probe.after, stream);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_seqs * p.num_heads_kv), dim3(256), 0, stream, p);
+        return hipGetLastError();
+    }
+    // prologue: KV-cache write of the new tokens (optional) + plan, one launch
     hipLaunchKernelGGL(paged_prologue_kernel, dim3(write_blocks + 1), dim3(256), 0, stream, wp, p, write_blocks);
-    hipError_t e = hipGetLastError();
+    e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.max_q_tiles > 0 && p.overlap) {
         // Mixed batch: the decode sequences stream from HBM on a few compute units while the
@@ -1030,11 +1147,11 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         if (probe.before) (void)hipEventRecord(probe.before, stream);
         const dim3 grid(p.num_waves / 8), block(512);
         if (p.cache_dtype == HIPATTN_U8)
-            hipLaunchKernelGGL((paged_decode_kernel<true, false, 8>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((paged_decode_kernel<true, false, 8>), grid, block, 0, stream, p, wp, 0);
         else if (p.cache_dtype == HIPATTN_BF16)
-            hipLaunchKernelGGL((paged_decode_kernel<false, true, 8>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((paged_decode_kernel<false, true, 8>), grid, block, 0, stream, p, wp, 0);
         else
-            hipLaunchKernelGGL((paged_decode_kernel<false, false, 8>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((paged_decode_kernel<false, false, 8>), grid, block, 0, stream, p, wp, 0);
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
         const hipError_t e_prefill = launch_paged_prefill(p, side->stream);
@@ -1049,11 +1166,11 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     }
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     if (p.cache_dtype == HIPATTN_U8)
-        hipLaunchKernelGGL((paged_decode_kernel<true, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<true, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);
     else if (p.cache_dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL((paged_decode_kernel<false, true, 1>), dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<false, true, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);
     else
-        hipLaunchKernelGGL((paged_decode_kernel<false, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p);
+        hipLaunchKernelGGL((paged_decode_kernel<false, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);
     e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     if (e != hipSuccess) return e;

@@ -8,28 +8,19 @@
 
 #include <cstddef>
 #include <memory>
-#include <stdexcept>
 #include <string>
 
 #include "hipattn.h"
+#include "openvino/core/except.hpp"
 
-namespace hip_plugin {
+namespace ov {
+namespace hip_gpu {
 
-// What ov::Exception would be under a real ov::Core.
-class Exception : public std::runtime_error {
-public:
-    explicit Exception(const std::string& what) : std::runtime_error(what) {}
-};
-class NotImplemented : public Exception {
-public:
-    explicit NotImplemented(const std::string& what) : Exception(what) {}
-};
-
-[[noreturn]] inline void throw_exception(const std::string& msg, const char* file, int line, const char* func) {
-    throw Exception(std::string(file) + ":" + std::to_string(line) + "(" + func + "): " + msg);
+[[noreturn]] inline void throw_ov_exception(const std::string& msg, const char* file, int line, const char* func) {
+    OPENVINO_THROW(file, ":", line, "(", func, "): ", msg);
 }
 
-#define HIP_PLUGIN_THROW(msg) ::hip_plugin::throw_exception((msg), __FILE__, __LINE__, __func__)
+#define HIP_PLUGIN_THROW(msg) ::ov::hip_gpu::throw_ov_exception((msg), __FILE__, __LINE__, __func__)
 #define HIP_PLUGIN_ASSERT(cond, msg) \
     do {                             \
         if (!(cond)) HIP_PLUGIN_THROW(std::string("assertion `" #cond "` failed: ") + (msg)); \
@@ -37,9 +28,9 @@ public:
 
 inline void throw_if_error(hipattn_status st, const char* file, int line, const char* func) {
     if (st != HIPATTN_OK)
-        throw_exception(std::string(hipattn_status_string(st)) + ": " + hipattn_last_error_string(), file, line, func);
+        throw_ov_exception(std::string(hipattn_status_string(st)) + ": " + hipattn_last_error_string(), file, line, func);
 }
-#define HIP_PLUGIN_CHECK(expr) ::hip_plugin::throw_if_error((expr), __FILE__, __LINE__, __func__)
+#define HIP_PLUGIN_CHECK(expr) ::ov::hip_gpu::throw_if_error((expr), __FILE__, __LINE__, __func__)
 
 class Stream {
 public:
@@ -56,6 +47,12 @@ public:
     }
     void download(void* dst, const void* src, size_t bytes) const {
         HIP_PLUGIN_CHECK(hipattn_memcpy_d2h_async(dst, src, bytes, stream_));
+    }
+    void transfer(void* dst, const void* src, size_t bytes) const {
+        HIP_PLUGIN_CHECK(hipattn_memcpy_d2d_async(dst, src, bytes, stream_));
+    }
+    void fill(void* dst, int byte_value, size_t bytes) const {
+        HIP_PLUGIN_CHECK(hipattn_fill_async(dst, byte_value, bytes, stream_));
     }
 
 private:
@@ -110,4 +107,5 @@ private:
     hipattn_event event_ = nullptr;
 };
 
-}  // namespace hip_plugin
+}  // namespace hip_gpu
+}  // namespace ov

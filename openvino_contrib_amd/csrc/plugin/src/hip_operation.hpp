@@ -10,20 +10,23 @@
 // immutable and shared by all concurrent requests.
 #pragma once
 
+#include <atomic>
 #include <functional>
 #include <map>
 #include <memory>
 #include <string>
 #include <vector>
 
-#include "graph.hpp"
 #include "hip_device.hpp"
+#include "openvino/core/node.hpp"
+#include "openvino/core/shape.hpp"
+#include "openvino/core/type/element_type.hpp"
 
-namespace hip_plugin {
+namespace ov {
+namespace hip_gpu {
 
 using TensorID = size_t;
-
-struct Configuration;  // plugin.hpp
+class VariableState;
 
 struct CreationContext {
     int device_id = 0;
@@ -31,13 +34,14 @@ struct CreationContext {
 };
 
 // One operand at run time: device pointer, element type, concrete shape.  `host` is a host copy of
-// the same bytes when the request has one (small index / scalar inputs set from host memory).
+// the same bytes when the request has one (small index / scalar inputs set from host memory, and
+// Constant nodes).
 struct TensorView {
     void* device = nullptr;
     const void* host = nullptr;
-    ElementType type = ElementType::dynamic;
-    Shape shape;
-    size_t byte_size() const { return (size_t)shape_size(shape) * element_size(type); }
+    ov::element::Type type;
+    ov::Shape shape;
+    size_t byte_size() const { return ov::shape_size(shape) * type.size(); }
 };
 
 struct WorkbufferRequest {
@@ -50,9 +54,38 @@ struct Workbuffers {
     std::vector<size_t> mutable_sizes;
 };
 
+// Set by InferRequest::cancel(); the executor looks at it between operators
+// (src/cancellation_token.hpp in the reference).
+class CancellationToken {
+public:
+    void cancel() { cancelled_.store(true); }
+    void reset() { cancelled_.store(false); }
+    bool is_cancelled() const { return cancelled_.load(); }
+
+private:
+    std::atomic<bool> cancelled_{false};
+};
+
+// Variable states of one infer request, by variable id (src/cuda_variable_state.hpp:186-238).
+class VariableContext {
+public:
+    void add(const std::string& id, const std::shared_ptr<VariableState>& state) { states_[id] = state; }
+    std::shared_ptr<VariableState> get(const std::string& id) const {
+        auto it = states_.find(id);
+        if (it == states_.end()) HIP_PLUGIN_THROW("no variable state with id '" + id + "'");
+        return it->second;
+    }
+    const std::map<std::string, std::shared_ptr<VariableState>>& all() const { return states_; }
+
+private:
+    std::map<std::string, std::shared_ptr<VariableState>> states_;
+};
+
 struct InferenceRequestContext {
     const Stream& stream;
     bool profiling = false;
+    const VariableContext* variables = nullptr;
+    const CancellationToken* cancellation = nullptr;
 };
 
 class OperationBase {
@@ -62,16 +95,17 @@ public:
     using Inputs = const std::vector<TensorView>&;
     using Outputs = const std::vector<TensorView>&;
 
-    OperationBase(const CreationContext&, const Node& node, IndexCollection&& input_ids, IndexCollection&& output_ids)
-        : node_name_(node.friendly_name),
-          type_name_(node.type_name),
+    OperationBase(const CreationContext&, const ov::Node& node, IndexCollection&& input_ids, IndexCollection&& output_ids)
+        : node_name_(node.get_friendly_name()),
+          type_name_(node.get_type_info().name),
           input_ids_(std::move(input_ids)),
           output_ids_(std::move(output_ids)) {}
     virtual ~OperationBase() = default;
 
     // Concrete output shapes for concrete input shapes (what validate_and_infer_types gives a clone
     // in the reference, src/cuda_dynamic_operation.cpp:419-468).
-    virtual std::vector<Shape> InferOutputShapes(const std::vector<Shape>& input_shapes) const = 0;
+    virtual std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& inputs,
+                                                     const InferenceRequestContext& context) const = 0;
     // Scratch the operator needs for these shapes; the request provides it in Execute().
     virtual WorkbufferRequest GetWorkBufferRequest(const std::vector<TensorView>& /*inputs*/) const { return {}; }
     // Enqueue the operator on context.stream.  const: one instance serves every request.
@@ -79,6 +113,8 @@ public:
                          const Workbuffers& workbuffers) const = 0;
     // Outputs that alias an input buffer and are updated in place (input index per output, -1 = none).
     virtual int InplaceInputOf(size_t /*output*/) const { return -1; }
+    // Host bytes the operator itself provides for an output (Constant); nullptr otherwise.
+    virtual const void* HostData(size_t /*output*/) const { return nullptr; }
 
     const std::string& GetName() const { return node_name_; }
     const std::string& GetTypeName() const { return type_name_; }
@@ -95,13 +131,13 @@ protected:
 class OperationRegistry final {
 public:
     using IndexCollection = OperationBase::IndexCollection;
-    using OperationBuilder = std::function<OperationBase::Ptr(const CreationContext&, const std::shared_ptr<Node>&,
+    using OperationBuilder = std::function<OperationBase::Ptr(const CreationContext&, const std::shared_ptr<ov::Node>&,
                                                               IndexCollection&&, IndexCollection&&)>;
     template <typename TOperation>
     class Register {
     public:
         explicit Register(const std::string& type_name) {
-            getInstance().registerOp(type_name, [](const CreationContext& context, const std::shared_ptr<Node>& node,
+            getInstance().registerOp(type_name, [](const CreationContext& context, const std::shared_ptr<ov::Node>& node,
                                                    IndexCollection&& in, IndexCollection&& out) -> OperationBase::Ptr {
                 return std::make_shared<TOperation>(context, *node, std::move(in), std::move(out));
             });
@@ -112,15 +148,17 @@ public:
         static OperationRegistry registry;
         return registry;
     }
-    bool hasOperation(const std::shared_ptr<Node>& node) const { return builders_.count(node->type_name) != 0; }
+    bool hasOperation(const std::shared_ptr<ov::Node>& node) const {
+        return builders_.count(node->get_type_info().name) != 0;
+    }
     // Throws when the type is unknown or the operator's constructor rejects the node: that is how
     // query_model learns what is supported (src/cuda_plugin.cpp:171-188).
-    OperationBase::Ptr createOperation(const CreationContext& context, const std::shared_ptr<Node>& node,
+    OperationBase::Ptr createOperation(const CreationContext& context, const std::shared_ptr<ov::Node>& node,
                                        IndexCollection&& in, IndexCollection&& out) const {
-        auto it = builders_.find(node->type_name);
+        auto it = builders_.find(node->get_type_info().name);
         if (it == builders_.end())
-            HIP_PLUGIN_THROW("operation '" + node->type_name + "' (node '" + node->friendly_name +
-                             "') is not supported by the HIP plugin");
+            HIP_PLUGIN_THROW(std::string("operation '") + node->get_type_info().name + "' (node '" +
+                             node->get_friendly_name() + "') is not supported by the HIP plugin");
         return it->second(context, node, std::move(in), std::move(out));
     }
     std::vector<std::string> registeredTypes() const {
@@ -132,17 +170,18 @@ public:
 private:
     void registerOp(const std::string& type_name, OperationBuilder&& builder) {
         if (!builders_.emplace(type_name, std::move(builder)).second)
-            throw std::runtime_error("Operation " + type_name + " is already registered !!");
+            throw std::runtime_error("HIP plugin: two operator classes claim the node type '" + type_name + "'");
     }
     std::map<std::string, OperationBuilder> builders_;
 };
 
-}  // namespace hip_plugin
+}  // namespace hip_gpu
+}  // namespace ov
 
 // Registers `type` (derived from OperationBase, constructible from
-// (const CreationContext&, const Node&, IndexCollection&&, IndexCollection&&)) for nodes whose
+// (const CreationContext&, const ov::Node&, IndexCollection&&, IndexCollection&&)) for nodes whose
 // type name is `name`.
-#define HIP_OPERATION_REGISTER(type, name)                                                              \
-    extern "C" {                                                                                        \
-    [[maybe_unused]] const ::hip_plugin::OperationRegistry::Register<type> hip_plugin_op_register_##name{#name}; \
+#define HIP_OPERATION_REGISTER(type, name)                                                                       \
+    extern "C" {                                                                                                 \
+    [[maybe_unused]] const ::ov::hip_gpu::OperationRegistry::Register<type> hip_plugin_op_register_##name{#name}; \
     }

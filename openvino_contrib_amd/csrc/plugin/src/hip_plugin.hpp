@@ -1,0 +1,262 @@
+// Plugin / CompiledModel / InferRequest / AsyncInferRequest of the "HIP" device.
+//
+// Shaped after the reference's Plugin : ov::IPlugin (modules/nvidia_plugin/src/cuda_plugin.hpp:18-83),
+// CompiledModel : ov::ICompiledModel (src/cuda_compiled_model.hpp:30-83), CudaInferRequest :
+// ov::ISyncInferRequest (src/cuda_infer_request.hpp:34-55), CudaAsyncInferRequest :
+// ov::IAsyncInferRequest (src/cuda_async_infer_request.hpp:14-29), CudaThreadPool
+// (src/cuda_thread_pool.hpp) and CudaVariableState (src/cuda_variable_state.hpp:31-183), with the
+// same base classes and virtual signatures.  The sources name only OpenVINO's own headers: they
+// compile against the developer package where it is installed and against the stand-in tree
+// (plugin/standin/) elsewhere.  What differs from the reference by design: no graph transformation
+// stage that decomposes attention, shape-polymorphic operators instead of per-shape clones, and a
+// remote context, because a paged KV cache has to stay on the device between infer calls.
+#pragma once
+
+#include <condition_variable>
+#include <deque>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "hip_device.hpp"
+#include "hip_operation.hpp"
+#include "openvino/core/any.hpp"
+#include "openvino/core/model.hpp"
+#include "openvino/op/util/variable.hpp"
+#include "openvino/runtime/iasync_infer_request.hpp"
+#include "openvino/runtime/icompiled_model.hpp"
+#include "openvino/runtime/iplugin.hpp"
+#include "openvino/runtime/iremote_context.hpp"
+#include "openvino/runtime/iremote_tensor.hpp"
+#include "openvino/runtime/isync_infer_request.hpp"
+#include "openvino/runtime/ivariable_state.hpp"
+#include "openvino/runtime/make_tensor.hpp"
+#include "openvino/runtime/profiling_info.hpp"
+#include "openvino/runtime/properties.hpp"
+#include "openvino/runtime/threading/itask_executor.hpp"
+
+namespace ov {
+namespace hip_gpu {
+
+// Value object rebuilt from an AnyMap over a base, as src/cuda_config.cpp:147-189 does.
+struct Configuration {
+    int device_id = 0;
+    ov::element::Type inference_precision = ov::element::dynamic;  // dynamic: keep the model's precision
+    bool enable_profiling = false;
+    int num_streams = 1;
+    std::string performance_mode = "LATENCY";
+
+    static Configuration from(const ov::AnyMap& properties, const Configuration& base, bool throw_on_unsupported = true);
+    ov::Any get(const std::string& name) const;
+    static const std::vector<std::string>& rw_properties();
+};
+
+// A tensor that lives in device memory: the KV caches, and anything else the caller keeps on the
+// device between infer calls.  Either owns its allocation or wraps a device pointer the caller
+// owns (property "DEV_PTR").
+class RemoteTensor : public ov::IRemoteTensor {
+public:
+    RemoteTensor(const ov::element::Type& type, const ov::Shape& shape, void* wrapped, const std::string& device_name);
+    void set_shape(ov::Shape shape) override;
+    const ov::element::Type& get_element_type() const override { return type_; }
+    const ov::Shape& get_shape() const override { return shape_; }
+    const ov::AnyMap& get_properties() const override { return properties_; }
+    const std::string& get_device_name() const override { return device_name_; }
+    void* device_ptr() const { return wrapped_ ? wrapped_ : owned_.get(); }
+
+private:
+    ov::element::Type type_;
+    ov::Shape shape_;
+    void* wrapped_ = nullptr;
+    Allocation owned_;
+    ov::AnyMap properties_;
+    std::string device_name_;
+};
+
+class RemoteContext : public ov::IRemoteContext {
+public:
+    RemoteContext(const std::string& device_name, int device_id);
+    const std::string& get_device_name() const override { return device_name_; }
+    const ov::AnyMap& get_property() const override { return properties_; }
+    ov::SoPtr<ov::IRemoteTensor> create_tensor(const ov::element::Type& type, const ov::Shape& shape,
+                                               const ov::AnyMap& params = {}) override;
+
+private:
+    std::string device_name_;
+    int device_id_;
+    ov::AnyMap properties_;
+};
+
+// Device-resident variable (ReadValue / Assign): grow-only capacity, logical shape, reset flag.
+class VariableState : public ov::IVariableState {
+public:
+    explicit VariableState(const ov::op::util::VariableInfo& info);
+    void set_state(const ov::SoPtr<ov::ITensor>& state) override;
+    ov::SoPtr<ov::ITensor> get_state() const override;
+    void reset() override;
+
+    // fast path of the operators: device to device on the request's stream
+    bool is_reset_state() const;
+    ov::Shape shape() const;
+    size_t byte_size() const;
+    void update_device_state(const Stream& stream, const void* src, const ov::Shape& new_shape);
+    void read_device_state(const Stream& stream, void* dst, size_t dst_bytes) const;
+
+private:
+    size_t logical_bytes() const { return type_.size() * ov::shape_size(current_shape_); }
+    mutable std::mutex mutex_;
+    ov::PartialShape data_shape_;
+    ov::element::Type type_;
+    ov::Shape initial_shape_, current_shape_;
+    Allocation buffer_;
+    bool is_reset_ = true;
+};
+
+// Worker threads of one device; each owns a stream.  Tasks handed to run() execute on one of them
+// (src/cuda_thread_pool.cpp:11-72); the stream of the executing thread is get_thread_context().
+struct ThreadContext {
+    Stream stream;
+};
+class ThreadPool : public ov::threading::ITaskExecutor {
+public:
+    ThreadPool(int device_id, unsigned num_threads);
+    ~ThreadPool() override;
+    void run(ov::threading::Task task) override;
+    const ThreadContext& get_thread_context();
+
+private:
+    void worker();
+    int device_id_;
+    std::mutex mutex_;
+    std::condition_variable wake_;
+    std::deque<ov::threading::Task> queue_;
+    bool stopping_ = false;
+    std::vector<std::thread> threads_;
+};
+
+class Plugin;
+class InferRequest;
+
+class CompiledModel : public ov::ICompiledModel {
+public:
+    CompiledModel(const std::shared_ptr<const ov::Model>& model, const Configuration& config,
+                  const std::shared_ptr<ov::threading::ITaskExecutor>& wait_executor,
+                  const std::shared_ptr<const ov::IPlugin>& plugin, bool loaded_from_cache);
+
+    std::shared_ptr<const ov::Model> get_runtime_model() const override { return model_; }
+    void export_model(std::ostream& model) const override;
+    std::shared_ptr<ov::IAsyncInferRequest> create_infer_request() const override;
+    void set_property(const ov::AnyMap& properties) override;
+    ov::Any get_property(const std::string& name) const override;
+
+    struct ExecStep {
+        std::shared_ptr<ov::Node> node;
+        OperationBase::Ptr op;
+    };
+    const std::vector<ExecStep>& exec_sequence() const { return exec_sequence_; }
+    size_t num_tensors() const { return num_tensors_; }
+    const std::vector<TensorID>& output_ids(const ov::Node* node) const { return output_ids_.at(node); }
+    const Configuration& config() const { return config_; }
+    const ov::ParameterVector& parameters() const { return exec_model_->get_parameters(); }
+    const ov::ResultVector& results() const { return exec_model_->get_results(); }
+
+protected:
+    std::shared_ptr<ov::ISyncInferRequest> create_sync_infer_request() const override;
+
+private:
+    std::shared_ptr<ov::Model> model_;             // what get_runtime_model / export_model hand out
+    std::shared_ptr<const ov::Model> exec_model_;  // the nodes the execution sequence refers to
+    Configuration config_;
+    std::shared_ptr<ov::threading::ITaskExecutor> wait_executor_;
+    bool loaded_from_cache_;
+    std::vector<ExecStep> exec_sequence_;
+    std::map<const ov::Node*, std::vector<TensorID>> output_ids_;  // per node: one TensorID per output port
+    size_t num_tensors_ = 0;
+};
+
+class InferRequest : public ov::ISyncInferRequest {
+public:
+    InferRequest(const std::shared_ptr<const CompiledModel>& compiled,
+                 const std::shared_ptr<ov::threading::ITaskExecutor>& wait_executor);
+
+    void infer() override;
+    std::vector<ov::SoPtr<ov::IVariableState>> query_state() const override;
+    std::vector<ov::ProfilingInfo> get_profiling_info() const override;
+
+    // stages of the asynchronous pipeline (src/cuda_infer_request.cpp:107-254)
+    void infer_preprocess();
+    void start_pipeline(const ThreadContext& thread_context);
+    void wait_pipeline(const ThreadContext& thread_context);
+    void infer_postprocess();
+    void cancel();
+
+private:
+    std::shared_ptr<const CompiledModel> compiled_;
+    std::shared_ptr<ov::threading::ITaskExecutor> wait_executor_;
+    std::vector<TensorView> views_;               // per TensorID, rebuilt by every infer
+    std::vector<Allocation> tensor_buffers_;      // per TensorID, grow-only
+    std::vector<Allocation> workbuffers_;         // per exec step
+    std::vector<std::unique_ptr<Event>> ev_begin_, ev_end_;
+    std::vector<size_t> ev_step_;
+    std::vector<ov::ProfilingInfo> profiling_;
+    VariableContext variables_;
+    CancellationToken cancellation_;
+};
+
+class AsyncInferRequest : public ov::IAsyncInferRequest {
+public:
+    AsyncInferRequest(const std::shared_ptr<InferRequest>& request,
+                      const std::shared_ptr<ov::threading::ITaskExecutor>& task_executor,
+                      const std::shared_ptr<ov::threading::ITaskExecutor>& wait_executor,
+                      const std::shared_ptr<ov::threading::ITaskExecutor>& callback_executor);
+    ~AsyncInferRequest() override;
+    void cancel() override;
+    void infer_thread_unsafe() override;
+
+private:
+    std::shared_ptr<InferRequest> request_;
+};
+
+class Plugin : public ov::IPlugin {
+public:
+    Plugin();
+    ~Plugin() override;
+
+    void set_property(const ov::AnyMap& properties) override;
+    ov::Any get_property(const std::string& name, const ov::AnyMap& arguments) const override;
+    std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
+                                                      const ov::AnyMap& properties) const override;
+    std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
+                                                      const ov::AnyMap& properties,
+                                                      const ov::SoPtr<ov::IRemoteContext>& context) const override;
+    std::shared_ptr<ov::ICompiledModel> import_model(std::istream& model_stream,
+                                                     const ov::AnyMap& properties) const override;
+    std::shared_ptr<ov::ICompiledModel> import_model(std::istream& model_stream,
+                                                     const ov::SoPtr<ov::IRemoteContext>& context,
+                                                     const ov::AnyMap& properties) const override;
+    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor& model_stream,
+                                                     const ov::AnyMap& properties) const override;
+    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor& model_stream,
+                                                     const ov::SoPtr<ov::IRemoteContext>& context,
+                                                     const ov::AnyMap& properties) const override;
+    ov::SupportedOpsMap query_model(const std::shared_ptr<const ov::Model>& model,
+                                    const ov::AnyMap& properties) const override;
+    ov::SoPtr<ov::IRemoteContext> create_context(const ov::AnyMap& remote_properties) const override;
+    ov::SoPtr<ov::IRemoteContext> get_default_context(const ov::AnyMap& remote_properties) const override;
+
+    bool is_operation_supported(const std::shared_ptr<ov::Node>& node, const Configuration& config) const;
+
+private:
+    std::shared_ptr<ov::threading::ITaskExecutor> get_stream_executor(const Configuration& config) const;
+    Configuration get_full_config(const ov::AnyMap& properties, bool throw_on_unsupported = true) const;
+    int device_count_ = 0;
+    Configuration config_;
+    mutable std::mutex mutex_;
+    mutable std::map<int, std::shared_ptr<ThreadPool>> device_thread_pool_;
+};
+
+}  // namespace hip_gpu
+}  // namespace ov

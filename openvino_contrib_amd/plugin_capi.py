@@ -8,8 +8,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libhip_plugin.so")
 
-F32, F16, BF16, U8, I32 = 0, 1, 2, 3, 100
-_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, U8: np.uint8, I32: np.int32}
+F32, F16, BF16, U8, I32, BOOL = 0, 1, 2, 3, 100, 101
+_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, U8: np.uint8, I32: np.int32, BOOL: np.bool_}
+OK, ERROR, OTHER_ERROR, NOT_IMPLEMENTED, CANCELLED, BUSY = range(6)
 
 _vp, _i, _sz, _cp = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_char_p
 _P = ctypes.POINTER
@@ -18,28 +19,41 @@ SYMBOLS = {
     "hip_plugin_last_error": (_cp, []),
     "hip_plugin_create": (_i, [_P(_vp)]),
     "hip_plugin_destroy": (None, [_vp]),
+    "hip_plugin_device_name": (_i, [_vp, ctypes.c_char_p, _sz]),
     "hip_plugin_set_property": (_i, [_vp, _cp, _cp]),
     "hip_plugin_get_property": (_i, [_vp, _cp, ctypes.c_char_p, _sz]),
     "hip_plugin_compile_model": (_i, [_vp, _vp, _cp, _P(_vp)]),
+    "hip_plugin_import_model": (_i, [_vp, _vp, _sz, _cp, _P(_vp)]),
     "hip_plugin_query_model": (_i, [_vp, _vp, ctypes.c_char_p, _sz]),
     "hip_plugin_registered_operations": (_i, [ctypes.c_char_p, _sz]),
-    "hip_model_create_sdpa": (_i, [_i, _i, _i64p, _i64p, _i, _i, _P(_vp)]),
-    "hip_model_create_paged_attention": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, _P(_vp)]),
+    "hip_model_create_sdpa": (_i, [_i, _i, _i64p, _i64p, _i, _i, _i, _i64p, _i, ctypes.c_float, _P(_vp)]),
+    "hip_model_create_paged_attention": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _P(_vp)]),
+    "hip_model_create_accumulator": (_i, [_i, _i, _i64p, _P(_vp)]),
     "hip_model_create_unsupported": (_i, [_P(_vp)]),
     "hip_model_destroy": (None, [_vp]),
     "hip_compiled_model_destroy": (None, [_vp]),
     "hip_compiled_model_num_inputs": (_i, [_vp]),
+    "hip_compiled_model_num_outputs": (_i, [_vp]),
     "hip_compiled_model_input_name": (_i, [_vp, _i, ctypes.c_char_p, _sz]),
     "hip_compiled_model_get_property": (_i, [_vp, _cp, ctypes.c_char_p, _sz]),
+    "hip_compiled_model_export": (_i, [_vp, _vp, _sz, _P(_sz)]),
     "hip_compiled_model_create_infer_request": (_i, [_vp, _P(_vp)]),
     "hip_infer_request_destroy": (None, [_vp]),
     "hip_infer_request_set_input": (_i, [_vp, _i, _vp, _i, _i, _i, _i64p]),
+    "hip_infer_request_set_output": (_i, [_vp, _i, _vp, _i, _i, _i, _i64p]),
     "hip_infer_request_infer": (_i, [_vp]),
     "hip_infer_request_start_async": (_i, [_vp]),
     "hip_infer_request_wait": (_i, [_vp]),
+    "hip_infer_request_cancel": (_i, [_vp]),
     "hip_infer_request_output_info": (_i, [_vp, _i, _P(_i), _P(_i), _i64p, _P(_sz)]),
     "hip_infer_request_copy_output": (_i, [_vp, _i, _vp, _sz]),
     "hip_infer_request_profiling": (_i, [_vp, ctypes.c_char_p, _sz]),
+    "hip_infer_request_num_states": (_i, [_vp]),
+    "hip_infer_request_state_name": (_i, [_vp, _i, ctypes.c_char_p, _sz]),
+    "hip_infer_request_state_reset": (_i, [_vp, _i]),
+    "hip_infer_request_state_info": (_i, [_vp, _i, _P(_i), _P(_i), _i64p, _P(_sz)]),
+    "hip_infer_request_state_get": (_i, [_vp, _i, _vp, _sz]),
+    "hip_infer_request_state_set": (_i, [_vp, _i, _vp, _i, _i, _i64p]),
 }
 
 _lib = None
@@ -89,17 +103,29 @@ class Model:
         self.handle = handle
 
     @classmethod
-    def sdpa(cls, dtype, q_shape, kv_shape, causal, with_scale_input=False):
+    def sdpa(cls, dtype, q_shape, kv_shape, causal, mask_dtype=None, mask_shape=(), scale=None, scale_constant=None):
+        """mask_dtype / mask_shape: the attention_mask input (None: absent).  scale=True: a scalar f32
+        Parameter named "scale"; scale_constant=x: a Constant holding x."""
         h = _vp()
+        mode, value = (2, float(scale_constant)) if scale_constant is not None else ((1, 0.0) if scale else (0, 0.0))
         _check(lib().hip_model_create_sdpa(dtype, len(q_shape), _shape(q_shape), _shape(kv_shape), int(causal),
-                                           int(with_scale_input), ctypes.byref(h)))
+                                           -1 if mask_dtype is None else mask_dtype, len(mask_shape),
+                                           _shape(mask_shape), mode, value, ctypes.byref(h)))
         return cls(h)
 
     @classmethod
-    def paged_attention(cls, q_dtype, kv_dtype, cache_dtype, Hq, Hkv, D, block_size, alibi_len=0):
+    def paged_attention(cls, q_dtype, kv_dtype, cache_dtype, Hq, Hkv, D, block_size, alibi_len=0, extra_inputs=0,
+                        extra_len=0, scores_result=False):
         h = _vp()
         _check(lib().hip_model_create_paged_attention(q_dtype, kv_dtype, cache_dtype, Hq, Hkv, D, block_size,
-                                                      alibi_len, ctypes.byref(h)))
+                                                      alibi_len, extra_inputs, extra_len, int(scores_result),
+                                                      ctypes.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def accumulator(cls, dtype, shape):
+        h = _vp()
+        _check(lib().hip_model_create_accumulator(dtype, len(shape), _shape(shape), ctypes.byref(h)))
         return cls(h)
 
     @classmethod
@@ -121,7 +147,7 @@ class InferRequest:
 
     def set_input(self, index, array, dtype):
         """Host tensor: wrapped, not copied (kept alive here until replaced)."""
-        array = np.ascontiguousarray(array, _NP[dtype])
+        array = np.asarray(array, dtype=_NP[dtype], order="C")  # (keeps a scalar's rank 0)
         self._keep[index] = array
         _check(lib().hip_infer_request_set_input(self.handle, index, array.ctypes.data_as(_vp), 0, dtype, array.ndim,
                                                  _shape(array.shape)))
@@ -129,8 +155,36 @@ class InferRequest:
     def set_device_input(self, index, device_ptr, dtype, shape):
         _check(lib().hip_infer_request_set_input(self.handle, index, device_ptr, 1, dtype, len(shape), _shape(shape)))
 
+    def set_device_output(self, index, device_ptr, dtype, shape):
+        """The output is left in the caller's device memory instead of a host tensor."""
+        _check(lib().hip_infer_request_set_output(self.handle, index, device_ptr, 1, dtype, len(shape), _shape(shape)))
+
     def infer(self):
         _check(lib().hip_infer_request_infer(self.handle))
+
+    def cancel(self):
+        _check(lib().hip_infer_request_cancel(self.handle))
+
+    def states(self):
+        n = lib().hip_infer_request_num_states(self.handle)
+        return [_text(lib().hip_infer_request_state_name, self.handle, i, size=256) for i in range(n)]
+
+    def state_reset(self, index=0):
+        _check(lib().hip_infer_request_state_reset(self.handle, index))
+
+    def state_get(self, index=0):
+        dt, rank, nbytes = _i(0), _i(0), _sz(0)
+        shape = (ctypes.c_int64 * 8)()
+        _check(lib().hip_infer_request_state_info(self.handle, index, ctypes.byref(dt), ctypes.byref(rank), shape,
+                                                  ctypes.byref(nbytes)))
+        out = np.empty([shape[i] for i in range(rank.value)], _NP[dt.value])
+        _check(lib().hip_infer_request_state_get(self.handle, index, out.ctypes.data_as(_vp), out.nbytes))
+        return out
+
+    def state_set(self, array, dtype, index=0):
+        array = np.ascontiguousarray(array, _NP[dtype])
+        _check(lib().hip_infer_request_state_set(self.handle, index, array.ctypes.data_as(_vp), dtype, array.ndim,
+                                                 _shape(array.shape)))
 
     def start_async(self):
         _check(lib().hip_infer_request_start_async(self.handle))
@@ -171,6 +225,17 @@ class CompiledModel:
     def get_property(self, key):
         return _text(lib().hip_compiled_model_get_property, self.handle, key.encode(), size=4096)
 
+    def num_outputs(self):
+        return lib().hip_compiled_model_num_outputs(self.handle)
+
+    def export_model(self):
+        """The bytes CompiledModel::export_model writes."""
+        n = _sz(0)
+        _check(lib().hip_compiled_model_export(self.handle, None, 0, ctypes.byref(n)))
+        buf = ctypes.create_string_buffer(max(n.value, 1))
+        _check(lib().hip_compiled_model_export(self.handle, buf, n.value, ctypes.byref(n)))
+        return buf.raw[:n.value]
+
     def create_infer_request(self):
         h = _vp()
         _check(lib().hip_compiled_model_create_infer_request(self.handle, ctypes.byref(h)))
@@ -193,6 +258,15 @@ class Plugin:
 
     def get_property(self, key):
         return _text(lib().hip_plugin_get_property, self.handle, key.encode(), size=4096)
+
+    def device_name(self):
+        return _text(lib().hip_plugin_device_name, self.handle, size=64)
+
+    def import_model(self, blob, properties=None):
+        text = ";".join("%s=%s" % kv for kv in (properties or {}).items()).encode() if properties else None
+        h = _vp()
+        _check(lib().hip_plugin_import_model(self.handle, blob, len(blob), text, ctypes.byref(h)))
+        return CompiledModel(h)
 
     def query_model(self, model):
         names = _text(lib().hip_plugin_query_model, self.handle, model.handle)

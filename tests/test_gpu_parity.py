@@ -179,7 +179,7 @@ def test_sdpa_flash_scores_that_grow_along_the_keys(hip, oracle, dtype, profile,
     ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
     assert np.isfinite(out).all()
     tol = TOL[dtype] if profile != "wide" else {W.F16: 4e-3, W.BF16: 3e-2}[dtype]
-    assert float(np.max(np.abs(out - ref) / np.maximum(1.0, np.abs(ref)))) <= tol
+    assert H.scaled_bound_error(out, ref, "sdpa flash %s dtype %d causal %d" % (profile, dtype, causal)) <= tol
 
 
 @pytest.mark.parametrize("dtype", [W.F32, W.F16])
@@ -201,7 +201,7 @@ def test_sdpa_generic_scores_that_grow_along_the_keys(hip, oracle, dtype, profil
         assert path == "sdpa_generic"
         ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
         assert np.isfinite(out).all()
-        assert float(np.max(np.abs(out - ref) / np.maximum(1.0, np.abs(ref)))) <= TOL[dtype]
+        assert H.scaled_bound_error(out, ref, "sdpa generic %s dtype %d causal %d" % (profile, dtype, causal)) <= TOL[dtype]
 
 
 def test_sdpa_flash_tensors_beyond_two_gib(hip, oracle):
@@ -472,14 +472,13 @@ def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dt
     if profile == "wide":  # (see the dense test: the precision of 16-bit probabilities on peaked rows)
         # and, for u8, of keys six units wide dequantised into fp16 operands
         tol = {W.BF16: 3e-2, W.U8: 2e-2}.get(cache_dtype, 1e-2)
-    err = np.abs(out - ref) / np.maximum(1.0, np.abs(ref))
-    assert float(err.max()) <= tol
+    assert H.scaled_bound_error(out, ref, "paged %s q %d cache %d window %d" % (profile, q_dtype, cache_dtype, window)) <= tol
     # the fp32 kernel that serves the shapes the MFMA kernels do not, on the same call
     out_g, path_g = dev.run(flags=hip.PA_FORCE_GENERIC | hip.PA_SKIP_CACHE_WRITE)
     assert path_g == "paged_generic"
     assert np.isfinite(out_g).all()
     # (its own error is below 1e-3; the rest is the 16-bit output type)
-    assert float((np.abs(out_g - ref) / np.maximum(1.0, np.abs(ref))).max()) <= (8e-3 if q_dtype == W.BF16 else 2e-3)
+    assert H.scaled_bound_error(out_g, ref, "paged generic %s q %d cache %d" % (profile, q_dtype, cache_dtype)) <= (8e-3 if q_dtype == W.BF16 else 2e-3)
     dev.free()
 
 
@@ -527,7 +526,7 @@ def test_paged_batch_of_thousands_of_sequences(hip, oracle, cache_dtype, mixed):
     np.testing.assert_array_equal(vc, ovc)
     assert np.isfinite(out).all()
     tol = 1e-2 if cache_dtype == W.U8 else 2e-3
-    assert float((np.abs(out - ref) / np.maximum(1.0, np.abs(ref))).max()) <= tol
+    assert H.scaled_bound_error(out, ref, "paged thousands of sequences cache %d mixed %d" % (cache_dtype, mixed)) <= tol
     dev.free()
 
 
@@ -559,7 +558,7 @@ def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, 
         assert np.isfinite(out).all()
         # N(0, 1) values and short contexts give outputs beyond 2, where the 16-bit output type alone
         # rounds by up to 0.008: the bound is relative there
-        assert (np.abs(out - ref) <= tol * np.maximum(1.0, np.abs(ref))).all(), i
+        assert H.scaled_bound_error(out, ref, "paged mixed side by side %d q %d cache %d" % (i, q_dtype, cache_dtype)) <= tol, i
         out2, _ = dev.run()  # the same tokens written again: same caches, same result
         np.testing.assert_array_equal(out, out2)
         dev.free()

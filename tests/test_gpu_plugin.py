@@ -81,9 +81,12 @@ def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_
     case = W.make_paged_case(94, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
     plugin = P.Plugin()
     plugin.set_property("PERF_COUNT", "YES")
-    compiled = plugin.compile_model(P.Model.paged_attention(q_dtype, q_dtype, cache_dtype, 16, 4, 128, 32))
+    # the operator's full signature: four empty optional inputs behind max_context_len and the scores output
+    compiled = plugin.compile_model(P.Model.paged_attention(q_dtype, q_dtype, cache_dtype, 16, 4, 128, 32,
+                                                            extra_inputs=4, extra_len=0, scores_result=True))
     assert compiled.input_names()[3:5] == ["key_cache", "value_cache"]
     assert compiled.get_property("EXECUTION_DEVICES") == "HIP.0"
+    assert compiled.num_outputs() == 2
     # the caches live on the device and are handed over as device tensors
     kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
     vc = hip.DeviceBuffer.from_numpy(case["value_cache"])
@@ -102,9 +105,15 @@ def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_
     req.set_input(10, np.array([window], np.int32), P.I32)
     req.set_input(11, np.zeros((0,), np.float32), W.F32)              # no alibi slopes
     req.set_input(12, np.array([case["max_context_len"]], np.int32), P.I32)
+    req.set_input(13, np.zeros((0,), np.int32), P.I32)                # score_aggregation_window: off
+    req.set_input(14, np.zeros((0,), np.int32), P.I32)                # no cache rotation
+    req.set_input(15, np.zeros((0,), np.int32), P.I32)
+    req.set_input(16, np.zeros((0,), np.float32), W.F32)
     req.start_async()
     req.wait()
     out, _ = req.output(0)
+    scores, _ = req.output(1)
+    assert scores.shape == (0,)
     out = H.storage_to_f32(out, q_dtype)
     ref, okc, ovc = H.oracle_paged(oracle, case)
     tol = 1e-2 if (cache_dtype == W.U8 or q_dtype == W.BF16) else 2e-3
@@ -113,7 +122,7 @@ def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_
     np.testing.assert_array_equal(kc.download(np.uint8, case["key_cache"].shape), okc)
     np.testing.assert_array_equal(vc.download(np.uint8, case["value_cache"].shape), ovc)
     prof = req.profiling()
-    assert [t for _, t, _ in prof] == ["PagedAttentionExtension", "Result"]
+    assert [t for _, t, _ in prof] == ["PagedAttentionExtension", "Result", "Result"]
     assert prof[0][2] > 0
     kc.free()
     vc.free()
@@ -131,3 +140,205 @@ def test_profiling_must_be_enabled(hip):
         req.profiling()
     with pytest.raises(P.PluginError):
         plugin.compile_model(P.Model.sdpa(W.F32, [1, 1, 4, 8], [1, 1, 4, 8], False), {"DEVICE_ID": 99})
+
+
+@pytest.mark.parametrize("dtype,tol", [(W.F32, 1e-4), (W.F16, 2e-3)])
+@pytest.mark.parametrize("mask_kind", ["bool_2d", "float_per_head", "none"])
+@pytest.mark.parametrize("scale_kind", ["default", "constant", "parameter"])
+def test_sdpa_with_mask_and_scale_inputs(hip, oracle, dtype, tol, mask_kind, scale_kind):
+    """attention_mask and scale inputs of v13::ScaledDotProductAttention through the plugin; the
+    reference executes them as Add / Select / Multiply nodes of the decomposed graph."""
+    print("[plugin] sdpa mask/scale", dtype, mask_kind, scale_kind, flush=True)
+    B, Hh, Lq, Lk, D = 2, 4, 33, 70, 64
+    case = W.make_sdpa_case(96, B, Hh, Hh, Lq, Lk, D, dtype)
+    rng = np.random.default_rng(97)
+    mask, mask_dtype = None, None
+    if mask_kind == "bool_2d":
+        mask = rng.random((Lq, Lk)) < 0.6
+        mask[:, 0] = True
+        mask_dtype = P.BOOL
+    elif mask_kind == "float_per_head":
+        mask = (1.5 * rng.standard_normal((1, Hh, Lq, Lk))).astype(np.float32)
+        mask_dtype = W.F32
+    scale = {"default": 0.0, "constant": 0.21, "parameter": 0.07}[scale_kind]
+    model = P.Model.sdpa(dtype, [-1, Hh, -1, D], [-1, Hh, -1, D], False, mask_dtype=mask_dtype,
+                         mask_shape=[-1] * (mask.ndim if mask is not None else 0),
+                         scale=(scale_kind == "parameter"), scale_constant=(scale if scale_kind == "constant" else None))
+    compiled = P.Plugin().compile_model(model)
+    req = compiled.create_infer_request()
+    for i, name in enumerate(("q", "k", "v")):
+        req.set_input(i, case[name + "_store"], dtype)
+    nxt = 3
+    if mask is not None or scale_kind != "default":
+        if mask is not None:
+            req.set_input(nxt, mask, mask_dtype)
+        else:
+            req.set_input(nxt, np.zeros((0,), W.np_storage_dtype(dtype)), dtype)  # the placeholder in front of scale
+        nxt += 1
+    if scale_kind == "parameter":
+        req.set_input(nxt, np.array(scale, np.float32), W.F32)
+    req.infer()
+    out, _ = req.output(0)
+    out = H.storage_to_f32(out, dtype)
+    if mask is not None:
+        ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask, scale=scale)
+    else:
+        ref = oracle.sdpa(case["q"], case["k"], case["v"], scale=scale)
+    assert H.max_abs(out, ref) <= tol
+
+
+@pytest.mark.parametrize("dtype,shape,pshape", [(W.F32, (1, 4, 20, 20), None), (W.F16, (1, 4, 20, 20), None),
+                                                (P.I32, (7, 4, 20, 20), None), (W.F32, (3, 4), (-1, 4)),
+                                                (W.F32, (0, 4), (-1, 4))])
+def test_read_value_assign_accumulator(hip, dtype, shape, pshape):
+    """The stateful model of the reference's test (tests/functional/shared_tests_instances/
+    single_layer_tests/read_value_assign.cpp:52-138, same shapes, precisions and input values,
+    the empty initial state included): y = ReadValue(init = x) + x, Assign(y).  After a reset the
+    variable reads as x, so the outputs run 2x, 3x, 4x; the state is device-resident."""
+    print("[plugin] accumulator", dtype, shape, pshape, flush=True)
+    n = int(np.prod(shape))
+    x = (np.arange(n) % 10 + 1).astype(np.float32).reshape(shape)
+    store = {W.F32: x, W.F16: W.to_storage(x, W.F16)[0], P.I32: x.astype(np.int32)}[dtype]
+    value = (lambda a: W.f16_bits_to_f32(a)) if dtype == W.F16 else (lambda a: a.astype(np.float32))
+    compiled = P.Plugin().compile_model(P.Model.accumulator(dtype, list(pshape or shape)))
+    req = compiled.create_infer_request()
+    assert req.states() == ["v0"]
+    req.set_input(0, store, dtype)
+    for k in (2, 3, 4):
+        req.infer()
+        out, _ = req.output(0)
+        assert out.shape == tuple(shape)
+        np.testing.assert_array_equal(value(out), k * x)
+        np.testing.assert_array_equal(value(req.state_get()), k * x)  # the state is what was assigned
+    req.state_reset()
+    assert req.state_get().shape == tuple(0 if (pshape and pshape[i] < 0) else shape[i] for i in range(len(shape)))
+    req.infer()
+    np.testing.assert_array_equal(value(req.output(0)[0]), 2 * x)  # after reset the variable reads as the init value
+    if n:
+        req.state_set(store, dtype)  # set_state: the next ReadValue returns it
+        req.infer()
+        np.testing.assert_array_equal(value(req.output(0)[0]), 2 * x)
+        req.infer()
+        np.testing.assert_array_equal(value(req.output(0)[0]), 3 * x)
+    # a second request of the same compiled model has a state of its own
+    other = compiled.create_infer_request()
+    other.set_input(0, store, dtype)
+    other.infer()
+    np.testing.assert_array_equal(value(other.output(0)[0]), 2 * x)
+
+
+def test_state_grows_with_a_dynamic_shape(hip):
+    """A variable with a dynamic extent takes the shape of what is assigned: grow-only capacity,
+    logical shape per step (src/cuda_variable_state.hpp:135-183)."""
+    compiled = P.Plugin().compile_model(P.Model.accumulator(W.F32, [-1, 4]))
+    req = compiled.create_infer_request()
+    for rows in (2, 5, 3):  # each new shape starts over from "state as large as the input"
+        x = np.arange(rows * 4, dtype=np.float32).reshape(rows, 4)
+        req.state_reset()
+        req.set_input(0, x, W.F32)
+        req.infer()
+        req.infer()
+        np.testing.assert_array_equal(req.output(0)[0], 3 * x)
+        assert req.state_get().shape == (rows, 4)
+
+
+def test_export_and_import_model(hip, oracle):
+    """export_model writes [u64][model][u64][weights]; import_model compiles from it and says so
+    (src/cuda_compiled_model.cpp:373-395, src/cuda_plugin.cpp:99-138)."""
+    import struct
+    plugin = P.Plugin()
+    model = P.Model.sdpa(W.F16, [1, 8, -1, 64], [1, 8, -1, 64], False, mask_dtype=P.BOOL, mask_shape=[-1, -1],
+                         scale_constant=0.2)
+    compiled = plugin.compile_model(model)
+    blob = compiled.export_model()
+    n_model = struct.unpack_from("<Q", blob, 0)[0]
+    n_weights = struct.unpack_from("<Q", blob, 8 + n_model)[0]
+    assert len(blob) == 16 + n_model + n_weights and b"ScaledDotProductAttention" in blob[8:8 + n_model]
+    assert compiled.get_property("LOADED_FROM_CACHE") == "NO"
+    imported = plugin.import_model(blob, {"LOADED_FROM_CACHE": "YES"})
+    assert imported.get_property("LOADED_FROM_CACHE") == "YES"
+    assert imported.input_names() == compiled.input_names() == ["query", "key", "value", "attention_mask"]
+    assert imported.export_model() == blob
+    case = W.make_sdpa_case(98, 1, 8, 8, 19, 40, 64, W.F16)
+    mask = np.random.default_rng(3).random((19, 40)) < 0.7
+    mask[:, 1] = True
+    outs = []
+    for cm in (compiled, imported):
+        req = cm.create_infer_request()
+        for i, name in enumerate(("q", "k", "v")):
+            req.set_input(i, case[name + "_store"], W.F16)
+        req.set_input(3, mask, P.BOOL)
+        req.infer()
+        outs.append(req.output(0)[0])
+    np.testing.assert_array_equal(outs[0], outs[1])
+    ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask, scale=0.2)
+    assert H.max_abs(H.storage_to_f32(outs[1], W.F16), ref) <= 2e-3
+    # a stateful model survives the round trip with its variable
+    acc = plugin.import_model(plugin.compile_model(P.Model.accumulator(W.F32, [-1, 4])).export_model())
+    req = acc.create_infer_request()
+    x = np.ones((2, 4), np.float32)
+    req.set_input(0, x, W.F32)
+    req.infer()
+    req.infer()
+    np.testing.assert_array_equal(req.output(0)[0], 3 * x)
+
+
+def test_async_pipeline_cancel_and_destruction(hip, oracle):
+    """start_async / wait / cancel and the destructor's stop_and_wait
+    (src/cuda_async_infer_request.cpp:26-61): a cancelled request ends with ov::Cancelled or, when
+    it had already finished, normally; either way it can be used again; destroying a request that
+    is still running waits for it."""
+    case = W.make_sdpa_case(99, 2, 8, 2, 600, 600, 128, W.BF16, std=0.5)
+    ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=True)
+    compiled = P.Plugin().compile_model(P.Model.sdpa(W.BF16, [-1, 8, -1, 128], [-1, 2, -1, 128], True))
+    req = compiled.create_infer_request()
+    for i, name in enumerate(("q", "k", "v")):
+        req.set_input(i, case[name + "_store"], W.BF16)
+    cancelled = 0
+    for _ in range(20):
+        req.start_async()
+        req.cancel()
+        try:
+            req.wait()
+        except P.PluginError as e:
+            assert e.code == P.CANCELLED
+            cancelled += 1
+    print("[plugin] cancelled", cancelled, "of 20", flush=True)
+    req.infer()  # usable after cancellation
+    assert H.max_abs(H.storage_to_f32(req.output(0)[0], W.BF16), ref) <= 1e-2
+    req.cancel()  # idle: no effect
+    req.start_async()
+    req.wait()
+    for _ in range(5):  # dropped while running: the destructor waits, nothing is left behind
+        r2 = compiled.create_infer_request()
+        for i, name in enumerate(("q", "k", "v")):
+            r2.set_input(i, case[name + "_store"], W.BF16)
+        r2.start_async()
+        del r2
+    # two requests in flight on the device's worker at once
+    reqs = [compiled.create_infer_request() for _ in range(3)]
+    for r in reqs:
+        for i, name in enumerate(("q", "k", "v")):
+            r.set_input(i, case[name + "_store"], W.BF16)
+        r.start_async()
+    for r in reqs:
+        r.wait()
+        assert H.max_abs(H.storage_to_f32(r.output(0)[0], W.BF16), ref) <= 1e-2
+
+
+def test_output_left_on_the_device(hip, oracle):
+    """An output port bound to a device tensor receives the result in place: nothing is downloaded."""
+    case = W.make_sdpa_case(100, 1, 8, 2, 130, 130, 128, W.F16)
+    compiled = P.Plugin().compile_model(P.Model.sdpa(W.F16, [-1, 8, -1, 128], [-1, 2, -1, 128], True))
+    req = compiled.create_infer_request()
+    bufs = [hip.DeviceBuffer.from_numpy(case[n + "_store"]) for n in ("q", "k", "v")]
+    out = hip.DeviceBuffer(case["q_store"].nbytes)
+    out.fill(0xFF)
+    for i, (b, n) in enumerate(zip(bufs, ("q", "k", "v"))):
+        req.set_device_input(i, b.ptr, W.F16, case[n + "_store"].shape)
+    req.set_device_output(0, out.ptr, W.F16, case["q_store"].shape)
+    req.infer()
+    res = H.storage_to_f32(out.download(np.uint16, case["q_store"].shape), W.F16)
+    assert H.max_abs(res, oracle.sdpa(case["q"], case["k"], case["v"], causal=True)) <= 2e-3
+    for b in bufs + [out]:
+        b.free()

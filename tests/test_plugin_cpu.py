@@ -25,23 +25,68 @@ def test_header_binding_and_exports_agree():
 
 def test_registry_holds_the_attention_operators():
     ops = P.registered_operations()
-    for name in ("Parameter", "Result", "Constant", "ScaledDotProductAttention", "PagedAttentionExtension"):
+    for name in ("Parameter", "Result", "Constant", "ScaledDotProductAttention", "PagedAttentionExtension", "ReadValue",
+                 "Assign", "Add"):
         assert name in ops
+
+
+def test_plugin_object_comes_from_create_plugin_engine():
+    """The facade asks the library's exported create_plugin_engine() for the plugin, as ov::Core would
+    (src/cuda_create_plugin.cpp:11-12)."""
+    L = ctypes.CDLL(P.LIB_PATH)
+    assert hasattr(L, "create_plugin_engine")
+    assert P.Plugin().device_name() == "HIP"
 
 
 def test_query_model_reports_supported_nodes():
     plugin = P.Plugin()
     sdpa = P.Model.sdpa(P.F16, [1, 8, -1, 64], [1, 8, -1, 64], True)
     assert sorted(plugin.query_model(sdpa)) == ["key", "out", "query", "sdpa", "value"]
-    # attention_mask / scale inputs: the operator's constructor throws, the node is reported unsupported
-    masked = P.Model.sdpa(P.F16, [1, 8, -1, 64], [1, 8, -1, 64], True, with_scale_input=True)
-    assert "sdpa" not in plugin.query_model(masked)
-    pa = P.Model.paged_attention(P.F16, P.F16, P.U8, 32, 8, 128, 32)
-    assert "paged_attention" in plugin.query_model(pa)
-    alibi = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, alibi_len=32)
-    assert "paged_attention" not in plugin.query_model(alibi)
     unknown = P.Model.unsupported()
     assert sorted(plugin.query_model(unknown)) == ["out", "x"]
+    stateful = P.Model.accumulator(P.F32, [-1, 4])
+    assert sorted(plugin.query_model(stateful)) == ["add", "assign", "out", "read_value", "x"]
+
+
+def test_sdpa_takes_the_operators_optional_inputs():
+    """attention_mask (boolean or floating, any broadcastable rank) and scale (Parameter or Constant)
+    are part of v13::ScaledDotProductAttention; the reference runs them through the decomposition."""
+    plugin = P.Plugin()
+    for kw in (dict(mask_dtype=P.BOOL, mask_shape=[-1, -1]), dict(mask_dtype=P.F16, mask_shape=[1, 8, -1, -1]),
+               dict(scale=True), dict(scale_constant=0.125), dict(mask_dtype=P.F32, mask_shape=[-1, -1], scale=True)):
+        model = P.Model.sdpa(P.F16, [1, 8, -1, 64], [1, 8, -1, 64], False, **kw)
+        assert "sdpa" in plugin.query_model(model), kw
+    # what stays unsupported: an integer mask, a mask of higher rank than the query
+    assert "sdpa" not in plugin.query_model(P.Model.sdpa(P.F16, [1, 8, -1, 64], [1, 8, -1, 64], False, mask_dtype=P.I32,
+                                                         mask_shape=[-1, -1]))
+    assert "sdpa" not in plugin.query_model(P.Model.sdpa(P.F16, [8, -1, 64], [8, -1, 64], False, mask_dtype=P.F16,
+                                                         mask_shape=[1, 8, -1, -1]))
+
+
+def test_paged_attention_takes_the_operators_full_signature():
+    """Exported models carry the inputs behind max_context_len (score aggregation, cache rotation,
+    sparse attention, sinks) and the scores output even when the features are off: such a node is
+    supported as long as those inputs are empty, and refused when they hold data."""
+    plugin = P.Plugin()
+    assert "paged_attention" in plugin.query_model(P.Model.paged_attention(P.F16, P.F16, P.U8, 32, 8, 128, 32))
+    for extra in (1, 4, 8):
+        pa = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=extra, extra_len=0,
+                                     scores_result=True)
+        names = plugin.query_model(pa)
+        assert "paged_attention" in names and "scores" in names, extra
+    rotated = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=4, extra_len=16)
+    assert "paged_attention" not in plugin.query_model(rotated)
+    unknown_inputs = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=9, extra_len=0)
+    assert "paged_attention" not in plugin.query_model(unknown_inputs)
+    alibi = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, alibi_len=32)
+    assert "paged_attention" not in plugin.query_model(alibi)
+
+
+def test_import_model_rejects_a_foreign_stream():
+    plugin = P.Plugin()
+    for blob in (b"", b"\x05\x00", b"\xff" * 32):
+        with pytest.raises(P.PluginError):
+            plugin.import_model(blob)
 
 
 def test_properties():
@@ -55,7 +100,7 @@ def test_properties():
     assert plugin.get_property("RANGE_FOR_ASYNC_INFER_REQUESTS") == "1 1 1"
     with pytest.raises(P.PluginError) as e:
         plugin.set_property("INFERENCE_PRECISION_HINT", "f64")
-    assert "INFERENCE_PRECISION_HINT" in str(e.value) and "plugin.cpp" in str(e.value)  # file:line(function): text
+    assert "INFERENCE_PRECISION_HINT" in str(e.value) and "hip_plugin.cpp" in str(e.value)  # file:line(function): text
     with pytest.raises(P.PluginError):
         plugin.set_property("NO_SUCH_PROPERTY", "1")
     with pytest.raises(P.PluginError):
