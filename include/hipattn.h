@@ -260,7 +260,7 @@ hipattn_status hipattn_profile_dominant_kernel(hipattn_event before, hipattn_eve
  *                                 chunks' kernel; 0: one kernel after the other
  *   "mixed_decode_share_percent"  scales the compute units the plan gives the decode part (100)
  *   "decode_switch_cost"          block-times charged per (sequence, kv head) start when the decode
- *                                 work is cut into equal pieces (3)
+ *                                 work is cut into equal pieces (5)
  *   "decode_dyn_pieces_per_wave"  on-demand pieces per wavefront for the last quarter of the
  *                                 decode work (0 = none)
  * HIPATTN_<NAME IN CAPITALS> in the environment gives an option its initial value; the

@@ -916,7 +916,7 @@ Option g_options[] = {
     // 0: one kernel after the other for mixed batches; 1: decode beside the chunks' flash kernel
     {"mixed_overlap", "HIPATTN_MIXED_OVERLAP", 1, 0, 1, {1}},
     // block-times a (sequence, kv head) segment start is charged on the decode work line
-    {"decode_switch_cost", "HIPATTN_DECODE_SWITCH_COST", 3, 0, 64, {3}},
+    {"decode_switch_cost", "HIPATTN_DECODE_SWITCH_COST", 5, 0, 64, {5}},
     // on-demand pieces per wavefront for the last quarter of the decode work line (0: none)
     {"decode_dyn_pieces_per_wave", "HIPATTN_DECODE_DYN_PIECES_PER_WAVE", 0, 0, 64, {0}},
     // scales the compute units the plan gives the decode part of a mixed batch (100 = as modelled)

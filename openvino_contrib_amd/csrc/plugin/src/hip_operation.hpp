@@ -113,6 +113,10 @@ public:
                          const Workbuffers& workbuffers) const = 0;
     // Outputs that alias an input buffer and are updated in place (input index per output, -1 = none).
     virtual int InplaceInputOf(size_t /*output*/) const { return -1; }
+    // Inputs the operator updates in place on the device (the KV caches of PagedAttentionExtension).
+    // When such an input was bound as a host tensor the request copies it back after the operator,
+    // so the caller's memory holds the update; device-resident tensors need nothing.
+    virtual std::vector<size_t> UpdatedInputs() const { return {}; }
     // Host bytes the operator itself provides for an output (Constant); nullptr otherwise.
     virtual const void* HostData(size_t /*output*/) const { return nullptr; }
 

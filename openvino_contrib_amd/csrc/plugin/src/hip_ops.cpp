@@ -278,6 +278,8 @@ public:
         return shapes;
     }
 
+    std::vector<size_t> UpdatedInputs() const override { return {kKeyCache, kValueCache}; }
+
     WorkbufferRequest GetWorkBufferRequest(const std::vector<TensorView>& inputs) const override {
         const hipattn_pa_desc d = describe(inputs);
         size_t bytes = 0;

@@ -649,6 +649,11 @@ void InferRequest::start_pipeline(const ThreadContext& thread_context) {
         }
         step.op->Execute(context, in, out, wb);
         if (profiling) ev_end_.back()->record(stream);
+        // an input the operator updated in place that the caller bound as host memory: the update goes
+        // back there (slow -- a KV cache belongs in a device tensor -- but never silently lost)
+        for (size_t idx : step.op->UpdatedInputs())
+            if (idx < in.size() && in[idx].host && in[idx].byte_size())
+                stream.download(const_cast<void*>(in[idx].host), in[idx].device, in[idx].byte_size());
     }
 
     // results into the host tensors of the output ports (device-bound outputs were written in place,

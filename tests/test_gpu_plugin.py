@@ -342,3 +342,32 @@ def test_output_left_on_the_device(hip, oracle):
     assert H.max_abs(res, oracle.sdpa(case["q"], case["k"], case["v"], causal=True)) <= 2e-3
     for b in bufs + [out]:
         b.free()
+
+
+def test_paged_attention_with_host_bound_caches_writes_them_back(hip, oracle):
+    """KV caches bound as host tensors are uploaded, updated by the operator and copied back, so the
+    caller's arrays hold the new rows (a device tensor avoids both copies; this is the slow, safe way)."""
+    seqs = [(37, 1), (0, 70), (500, 1)]
+    case = W.make_paged_case(101, seqs, 8, 2, 128, 32, W.F16, W.F16, W.F16)
+    compiled = P.Plugin().compile_model(P.Model.paged_attention(W.F16, W.F16, W.F16, 8, 2, 128, 32))
+    req = compiled.create_infer_request()
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    elem_shape = list(kc.shape[:3]) + [kc.shape[3] // 2]
+    req.set_input(0, case["q_store"], W.F16)
+    req.set_input(1, case["k_new_store"], W.F16)
+    req.set_input(2, case["v_new_store"], W.F16)
+    req.set_input(3, kc.view(np.uint16).reshape(elem_shape), W.F16)
+    req.set_input(4, vc.view(np.uint16).reshape(elem_shape), W.F16)
+    req.set_input(5, case["past_lens"], P.I32)
+    req.set_input(6, case["subsequence_begins"], P.I32)
+    req.set_input(7, case["block_indices"], P.I32)
+    req.set_input(8, case["block_indices_begins"], P.I32)
+    req.set_input(9, np.zeros((0,), np.float32), W.F32)
+    req.set_input(10, np.array([0], np.int32), P.I32)
+    req.set_input(11, np.zeros((0,), np.float32), W.F32)
+    req.set_input(12, np.array([case["max_context_len"]], np.int32), P.I32)
+    req.infer()
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    assert H.max_abs(H.storage_to_f32(req.output(0)[0], W.F16), ref) <= 2e-3
+    np.testing.assert_array_equal(kc, okc)  # the caller's own arrays now hold the new rows
+    np.testing.assert_array_equal(vc, ovc)
