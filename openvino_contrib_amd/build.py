@@ -53,23 +53,37 @@ def _compile(src, extra):
     return obj, r.stderr
 
 
-def build_library(verbose=False, extra_flags=(), jobs=4):
-    """Compile every HIP source and link libhipattn.so.  Always recompiles."""
+def _build_shared(sources, lib_path, verbose, extra_flags, jobs, link_flags=()):
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        results = list(ex.map(lambda s: _compile(s, extra_flags), SOURCES))
+        results = list(ex.map(lambda s: _compile(s, extra_flags), sources))
     objs = [o for o, _ in results]
     if verbose:
         for _, err in results:
             lines = [l for l in err.splitlines() if "packed-fp32-ops" not in l]
             if lines:
                 print("\n".join(lines), file=sys.stderr)
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path] + objs + list(link_flags)
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s" % r.stderr[-4000:])
     for o in objs:
         os.remove(o)
-    return LIB_PATH
+    return lib_path
+
+
+def build_library(verbose=False, extra_flags=(), jobs=4):
+    """Compile every HIP source and link libhipattn.so.  Always recompiles."""
+    return _build_shared(SOURCES, LIB_PATH, verbose, extra_flags, jobs)
+
+
+OPS_LIB_PATH = os.path.join(CSRC, "libhipops.so")
+OPS_SOURCES = ["ops/hipops_api.hip", "ops/layer_ops.hip", "ops/matmul.hip"]
+
+
+def build_ops_library(verbose=False, extra_flags=(), jobs=4):
+    """libhipops.so: the operators around attention (RMS norm, RoPE, MatMul over hipBLASLt, Gather,
+    Concat).  A library of its own because it links hipBLASLt."""
+    return _build_shared(OPS_SOURCES, OPS_LIB_PATH, verbose, extra_flags, jobs, link_flags=["-lhipblaslt"])
 
 
 YARDSTICK_LIB_PATH = os.path.join(CSRC, "bench", "libmfma_yardstick.so")
@@ -94,13 +108,13 @@ def build_plugin():
     against the stand-in for OpenVINO's developer headers (plugin/standin/), plus the C facade the
     tests drive it through.  Where the OpenVINO developer package is installed, plugin/CMakeLists.txt
     builds the same sources against the real headers instead."""
-    if not os.path.exists(LIB_PATH):
-        raise RuntimeError("build libhipattn.so first")
+    if not os.path.exists(LIB_PATH) or not os.path.exists(OPS_LIB_PATH):
+        raise RuntimeError("build libhipattn.so and libhipops.so first")
     cxx = shutil.which("g++") or "g++"
     cmd = [cxx, "-std=c++17", "-O2", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wextra", "-pthread",
            "-I" + INCLUDE, "-I" + os.path.join(CSRC, "plugin", "src"), "-I" + os.path.join(CSRC, "plugin", "standin")]
     cmd += [os.path.join(CSRC, s) for s in PLUGIN_SOURCES]
-    cmd += ["-L" + CSRC, "-lhipattn", "-Wl,-rpath,$ORIGIN", "-o", PLUGIN_LIB_PATH]
+    cmd += ["-L" + CSRC, "-lhipattn", "-lhipops", "-Wl,-rpath,$ORIGIN", "-o", PLUGIN_LIB_PATH]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("plugin build failed:\n%s" % r.stderr[-6000:])
@@ -109,5 +123,6 @@ def build_plugin():
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_ops_library(verbose=True))
     print(build_plugin())
     print(build_bench_tools())

@@ -1,0 +1,26 @@
+// Internal declarations shared by the sources of libhipops.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hipops.h"
+
+namespace hipops {
+
+// records the message for hipops_last_error_string() on this thread and returns `status`
+hipattn_status fail(hipattn_status status, const char* format, ...) __attribute__((format(printf, 2, 3)));
+
+hipattn_status rms_norm(const void* x, const void* gamma, void* out, int64_t rows, int64_t hidden, float eps, int x_dtype,
+                        int gamma_dtype, int out_dtype, hipStream_t stream);
+hipattn_status rope(const hipops_rope_desc* desc, const void* x, const void* cos, const void* sin, const int32_t* positions,
+                    void* out, hipStream_t stream);
+hipattn_status gather(const void* data, const void* indices, void* out, int64_t batch, int64_t outer, int64_t axis_dim,
+                      int64_t inner_bytes, int64_t num_indices, int index_dtype, hipStream_t stream);
+hipattn_status concat(const void* const* inputs, const int64_t* axis_bytes, int num_inputs, int64_t outer, void* out,
+                      hipStream_t stream);
+hipattn_status matmul_workspace_size(const hipops_matmul_desc* desc, size_t* bytes);
+hipattn_status matmul(const hipops_matmul_desc* desc, const void* a, const void* b, void* c, void* workspace,
+                      size_t workspace_bytes, hipStream_t stream);
+
+}  // namespace hipops

@@ -1,4 +1,4 @@
-"""ctypes loader for the CPU oracle (oracle/hipattn_oracle.c).
+"""ctypes loader for the CPU oracle (oracle/hipattn_oracle.c, oracle/layer_ops_oracle.c).
 
 Test infrastructure only: imported by tests/, the smoke check and the benchmark's
 cpu_baseline leg.  The product package never imports this module.
@@ -62,6 +62,16 @@ def lib():
         L.oracle_paged_attention.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                              f32, i32, i32, vp]
         L.oracle_paged_attention.restype = i32
+        L.oracle_rms_norm_f32.argtypes = [vp, vp, vp, i64, i64, f32]
+        L.oracle_rms_norm_f32.restype = None
+        L.oracle_rope_f32.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i64]
+        L.oracle_rope_f32.restype = None
+        L.oracle_matmul_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, i64, i64]
+        L.oracle_matmul_f32.restype = None
+        L.oracle_gather_bytes.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64]
+        L.oracle_gather_bytes.restype = None
+        L.oracle_concat_bytes.argtypes = [vp, vp, i32, i64, vp]
+        L.oracle_concat_bytes.restype = None
         _lib = L
     return _lib
 
@@ -219,4 +229,73 @@ def paged_attention(q, k_new, v_new, key_cache, value_cache, cache_dtype, past_l
                                       _p(out))
     if rc:
         raise ValueError("oracle_paged_attention: bad arguments")
+    return out
+
+
+# ---- the operators either side of attention (oracle/layer_ops_oracle.c) ------------------------
+def rms_norm(x, gamma=None, eps=1e-6):
+    """x [..., hidden] fp32, gamma [hidden] or None -> like x."""
+    x = _c(x, np.float32)
+    hidden = x.shape[-1]
+    g = None if gamma is None else _c(gamma, np.float32)
+    out = np.empty_like(x)
+    lib().oracle_rms_norm_f32(_p(x), _p(g) if g is not None else None, _p(out), x.size // hidden, hidden, float(eps))
+    return out
+
+
+def rope(x, cos, sin, positions=None, rotary_ndims=0, interleaved=False):
+    """x [tokens, heads, head_size] fp32; cos/sin [rows, rotary_ndims] (rotate-half) or
+    [rows, rotary_ndims/2] (adjacent pairs); positions int32 [tokens] or None (row = token)."""
+    x, cos, sin = _c(x, np.float32), _c(cos, np.float32), _c(sin, np.float32)
+    T, H, S = x.shape
+    rotary = rotary_ndims or S
+    assert cos.shape == sin.shape and cos.shape[1] == (rotary // 2 if interleaved else rotary)
+    pos = None if positions is None else _c(positions, np.int32)
+    out = np.empty_like(x)
+    lib().oracle_rope_f32(_p(x), _p(cos), _p(sin), _p(pos) if pos is not None else None, _p(out), T, H, S, rotary,
+                          int(bool(interleaved)), cos.shape[1])
+    return out
+
+
+def matmul(a, b, transpose_a=False, transpose_b=False):
+    """a [batch?, ., .], b [batch?, ., .] fp32 (2-D operands broadcast over the other's batch) -> [batch?, m, n]."""
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    batch = max(a.shape[0] if a.ndim == 3 else 1, b.shape[0] if b.ndim == 3 else 1)
+    m, k = (a.shape[-1], a.shape[-2]) if transpose_a else (a.shape[-2], a.shape[-1])
+    n = b.shape[-2] if transpose_b else b.shape[-1]
+    assert (b.shape[-1] if transpose_b else b.shape[-2]) == k
+    sa = m * k if a.ndim == 3 and a.shape[0] > 1 else 0
+    sb = k * n if b.ndim == 3 and b.shape[0] > 1 else 0
+    c = np.empty((batch, m, n), np.float32)
+    lib().oracle_matmul_f32(_p(a), _p(b), _p(c), m, n, k, batch, int(transpose_a), int(transpose_b), sa, sb)
+    return c if (a.ndim == 3 or b.ndim == 3) else c[0]
+
+
+def gather(data, indices, axis=0, batch_dims=0):
+    """Gather (opset 8 rules: negative indices wrap, rows out of range are zero) on any dtype."""
+    data = np.ascontiguousarray(data)
+    idx = _c(indices, np.int64)
+    batch = int(np.prod(data.shape[:batch_dims], dtype=np.int64))
+    outer = int(np.prod(data.shape[batch_dims:axis], dtype=np.int64))
+    axis_dim = data.shape[axis]
+    inner = int(np.prod(data.shape[axis + 1:], dtype=np.int64)) * data.dtype.itemsize
+    n_idx = int(np.prod(idx.shape[batch_dims:], dtype=np.int64))
+    out_shape = data.shape[:axis] + idx.shape[batch_dims:] + data.shape[axis + 1:]
+    out = np.empty(out_shape, data.dtype)
+    lib().oracle_gather_bytes(_p(data), _p(idx), _p(out), batch, outer, axis_dim, inner, n_idx)
+    return out
+
+
+def concat(arrays, axis):
+    arrays = [np.ascontiguousarray(a) for a in arrays]
+    first = arrays[0]
+    axis = axis % first.ndim
+    outer = int(np.prod(first.shape[:axis], dtype=np.int64))
+    tail = int(np.prod(first.shape[axis + 1:], dtype=np.int64)) * first.dtype.itemsize
+    widths = np.array([a.shape[axis] * tail for a in arrays], np.int64)
+    shape = list(first.shape)
+    shape[axis] = sum(a.shape[axis] for a in arrays)
+    out = np.empty(shape, first.dtype)
+    ptrs = (ctypes.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+    lib().oracle_concat_bytes(ptrs, _p(widths), len(arrays), outer, _p(out))
     return out

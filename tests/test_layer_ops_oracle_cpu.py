@@ -1,0 +1,120 @@
+"""Pins the CPU oracle of the operators around attention (oracle/layer_ops_oracle.c) without a GPU.
+
+Each function is checked against a library routine or a formulation that does not share its code:
+torch's rms_norm and the transformers library's rotary helpers (committed fixtures), complex
+multiplication, numpy's matmul / take / concatenate, and invariants a wrong sign, index or
+transposed operand breaks.
+"""
+import os
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "layer_ops_golden.npz")
+
+
+@pytest.fixture(scope="module")
+def golden():
+    return np.load(GOLDEN)
+
+
+@pytest.mark.parametrize("name", ["rms_small", "rms_odd", "rms_wide"])
+def test_rms_norm_matches_torch_fixture(oracle, golden, name):
+    out = oracle.rms_norm(golden[name + "/x"], golden[name + "/gamma"], float(golden[name + "/eps"]))
+    np.testing.assert_allclose(out, golden[name + "/out"], rtol=2e-6, atol=1e-7)
+
+
+def test_rms_norm_invariants(oracle):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((7, 96)).astype(np.float32)
+    out = oracle.rms_norm(x, None, 0.0)
+    np.testing.assert_allclose((out.astype(np.float64) ** 2).mean(-1), 1.0, rtol=1e-6)  # unit mean square
+    np.testing.assert_allclose(oracle.rms_norm(4.0 * x, None, 0.0), out, rtol=1e-6)       # scale invariance at eps 0
+    g = rng.standard_normal(96).astype(np.float32)
+    np.testing.assert_allclose(oracle.rms_norm(x, g, 1e-6), oracle.rms_norm(x, None, 1e-6) * g, rtol=1e-6)
+    big_eps = oracle.rms_norm(x, None, 1e6)  # eps dominates: out ~ x / 1000
+    np.testing.assert_allclose(big_eps, x / np.sqrt((x.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e6), rtol=1e-6)
+
+
+@pytest.mark.parametrize("name,rot,interleaved", [("llama", 16, False), ("llama_partial", 8, False), ("gptj", 16, True),
+                                                  ("gptj_partial", 8, True)])
+def test_rope_matches_transformers_fixture(oracle, golden, name, rot, interleaved):
+    out = oracle.rope(golden[name + "/x"], golden[name + "/cos"], golden[name + "/sin"], None, rot, interleaved)
+    np.testing.assert_allclose(out, golden[name + "/out"], rtol=0, atol=2e-6)
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_rope_is_a_complex_rotation(oracle, interleaved):
+    rng = np.random.default_rng(2)
+    T, H, S, rot = 9, 3, 32, 24
+    half = rot // 2
+    x = rng.standard_normal((T, H, S)).astype(np.float32)
+    theta = rng.uniform(0, 6.28, (50, half))
+    positions = rng.integers(0, 50, T).astype(np.int32)
+    if interleaved:
+        cos, sin = np.cos(theta), np.sin(theta)
+        z = x[..., 0:rot:2].astype(np.float64) + 1j * x[..., 1:rot:2]
+    else:
+        cos, sin = np.cos(np.tile(theta, 2)), np.sin(np.tile(theta, 2))
+        z = x[..., :half].astype(np.float64) + 1j * x[..., half:rot]
+    w = z * np.exp(1j * theta[positions])[:, None, :]
+    out = oracle.rope(x, cos, sin, positions, rot, interleaved)
+    if interleaved:
+        np.testing.assert_allclose(out[..., 0:rot:2], w.real, atol=2e-6)
+        np.testing.assert_allclose(out[..., 1:rot:2], w.imag, atol=2e-6)
+    else:
+        np.testing.assert_allclose(out[..., :half], w.real, atol=2e-6)
+        np.testing.assert_allclose(out[..., half:rot], w.imag, atol=2e-6)
+    assert np.array_equal(out[..., rot:], x[..., rot:])                     # the tail passes through
+    np.testing.assert_allclose(np.linalg.norm(out, axis=-1), np.linalg.norm(x, axis=-1), rtol=1e-6)
+    back = oracle.rope(out, cos, -sin, positions, rot, interleaved)          # rotate by -theta
+    np.testing.assert_allclose(back, x, atol=3e-6)
+    ident = oracle.rope(x, np.ones_like(cos), np.zeros_like(sin), positions, rot, interleaved)
+    assert np.array_equal(ident, x)
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_matches_numpy(oracle, ta, tb):
+    rng = np.random.default_rng(3)
+    m, n, k = 13, 7, 29
+    a = rng.standard_normal((3, k, m) if ta else (3, m, k)).astype(np.float32)
+    b = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)  # broadcast over the batch
+    ref = (np.swapaxes(a, 1, 2) if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+    np.testing.assert_allclose(oracle.matmul(a, b, ta, tb), ref, rtol=1e-6, atol=1e-6)
+    b3 = rng.standard_normal((3, n, k) if tb else (3, k, n)).astype(np.float32)
+    ref = (np.swapaxes(a, 1, 2) if ta else a).astype(np.float64) @ (np.swapaxes(b3, 1, 2) if tb else b3).astype(np.float64)
+    np.testing.assert_allclose(oracle.matmul(a, b3, ta, tb), ref, rtol=1e-6, atol=1e-6)
+    a2 = a[0]
+    ref = (a2.T if ta else a2).astype(np.float64) @ (np.swapaxes(b3, 1, 2) if tb else b3).astype(np.float64)
+    np.testing.assert_allclose(oracle.matmul(a2, b3, ta, tb), ref, rtol=1e-6, atol=1e-6)
+
+
+def test_gather_matches_numpy_take_and_zero_rule(oracle):
+    rng = np.random.default_rng(4)
+    data = rng.integers(0, 2 ** 16, (3, 4, 6, 5)).astype(np.uint16)
+    for axis in range(4):
+        n = data.shape[axis]
+        idx = rng.integers(-n, n, (2, 3))
+        assert np.array_equal(oracle.gather(data, idx, axis), np.take(data, idx, axis=axis))
+    idx = np.array([0, 6, -7, 5, -6])  # 6 and -7 fall outside an axis of 6
+    got = oracle.gather(data, idx, 2)
+    assert np.array_equal(got[:, :, [0, 3, 4]], data[:, :, [0, 5, 0]])
+    assert not got[:, :, [1, 2]].any()
+    # batch_dims = 1: every batch entry has its own indices
+    bidx = rng.integers(0, 6, (3, 4))
+    got = oracle.gather(data, bidx, 2, batch_dims=1)
+    ref = np.stack([np.take(data[b], bidx[b], axis=1) for b in range(3)])
+    assert np.array_equal(got, ref)
+    assert oracle.gather(data, np.zeros((0,), np.int64), 1).shape == (3, 0, 6, 5)
+
+
+def test_concat_matches_numpy(oracle):
+    rng = np.random.default_rng(5)
+    for axis in (0, 1, 2, -1):
+        parts = []
+        for w in (3, 0, 5, 1):
+            shape = [2, 4, 6]
+            shape[axis] = w
+            parts.append(rng.standard_normal(shape).astype(np.float32))
+        assert np.array_equal(oracle.concat(parts, axis), np.concatenate(parts, axis))
