@@ -73,6 +73,9 @@ int hip_model_create_paged_attention(int q_dtype, int kv_dtype, int cache_dtype,
 /* x -> ReadValue(init_value = x, "v0") -> Add(read, x) -> Assign("v0"), Result(add): the stateful
  * model of tests/functional/shared_tests_instances/single_layer_tests/read_value_assign.cpp:52-64 */
 int hip_model_create_accumulator(int dtype, int rank, const int64_t* shape, hip_model_t** model);
+/* a model from the stand-in text form (the first part of what export_model writes): one node per
+ * line, "<index> <type> <name> inputs=<producer>:<port>,... {key=value;...}", in topological order */
+int hip_model_create_from_text(const char* text, hip_model_t** model);
 /* a model holding one node of a type no plugin operator handles */
 int hip_model_create_unsupported(hip_model_t** model);
 void hip_model_destroy(hip_model_t* model);

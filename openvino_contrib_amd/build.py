@@ -99,7 +99,7 @@ def build_bench_tools():
 
 
 PLUGIN_LIB_PATH = os.path.join(CSRC, "libhip_plugin.so")
-PLUGIN_SOURCES = ["plugin/src/hip_ops.cpp", "plugin/src/hip_plugin.cpp", "plugin/src/hip_create_plugin.cpp",
+PLUGIN_SOURCES = ["plugin/src/hip_ops.cpp", "plugin/src/hip_layer_ops.cpp", "plugin/src/hip_plugin.cpp", "plugin/src/hip_create_plugin.cpp",
                   "plugin/test_facade/c_api.cpp"]
 
 

@@ -512,7 +512,7 @@ InferRequest::InferRequest(const std::shared_ptr<const CompiledModel>& compiled,
       wait_executor_(wait_executor),
       views_(compiled->num_tensors()),
       tensor_buffers_(compiled->num_tensors()),
-      workbuffers_(compiled->exec_sequence().size()) {
+      workbuffer_() {
     HIP_PLUGIN_CHECK(hipattn_set_device(compiled_->config().device_id));
     // host tensors for ports of known shape; dynamic outputs are shaped by infer_postprocess
     auto host_tensor = [](const ov::Output<const ov::Node>& port) {
@@ -621,9 +621,9 @@ void InferRequest::start_pipeline(const ThreadContext& thread_context) {
                 v.device = bound->second;
             } else {
                 v.device = tensor_buffers_[out_ids[o]].reserve(std::max<size_t>(v.byte_size(), 16));
-                if (const void* host = step.op->HostData(o)) {  // a Constant: uploaded on every infer, like a Parameter
+                if (const void* host = step.op->HostData(o)) {  // a Constant: uploaded once per request
                     v.host = host;
-                    if (v.byte_size()) stream.upload(v.device, host, v.byte_size());
+                    if (v.byte_size() && constants_on_device_.insert(out_ids[o]).second) stream.upload(v.device, host, v.byte_size());
                 }
             }
             out.push_back(v);
@@ -634,7 +634,8 @@ void InferRequest::start_pipeline(const ThreadContext& thread_context) {
         size_t total = 0;
         for (size_t b : req.mutable_sizes) total += (b + 255) / 256 * 256;
         if (total) {
-            char* base = (char*)workbuffers_[si].reserve(total);
+            // one arena for all steps: they run one after the other on the request's stream
+            char* base = (char*)workbuffer_.reserve(total);
             for (size_t b : req.mutable_sizes) {
                 wb.mutable_buffers.push_back(base);
                 wb.mutable_sizes.push_back(b);

@@ -17,6 +17,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <set>
 #include <string>
 #include <thread>
 #include <vector>
@@ -198,7 +199,8 @@ private:
     std::shared_ptr<ov::threading::ITaskExecutor> wait_executor_;
     std::vector<TensorView> views_;               // per TensorID, rebuilt by every infer
     std::vector<Allocation> tensor_buffers_;      // per TensorID, grow-only
-    std::vector<Allocation> workbuffers_;         // per exec step
+    Allocation workbuffer_;                       // scratch arena shared by the steps of one infer
+    std::set<TensorID> constants_on_device_;      // Constant outputs already uploaded
     std::vector<std::unique_ptr<Event>> ev_begin_, ev_end_;
     std::vector<size_t> ev_step_;
     std::vector<ov::ProfilingInfo> profiling_;

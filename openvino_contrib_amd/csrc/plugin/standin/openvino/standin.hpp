@@ -625,6 +625,180 @@ public:
     }
 };
 }  // namespace v1
+
+namespace v0 {
+// A [.., m, k] x B [.., k, n] with optional transposition of the last two axes of either operand
+class MatMul : public Node {
+public:
+    OPENVINO_OP("MatMul", "opset1")
+    MatMul(const Output<Node>& a, const Output<Node>& b, bool transpose_a = false, bool transpose_b = false)
+        : Node(OutputVector{a, b}), transpose_a_(transpose_a), transpose_b_(transpose_b) {
+        const PartialShape &sa = a.get_partial_shape(), &sb = b.get_partial_shape();
+        OPENVINO_ASSERT(sa.size() >= 2 && sb.size() >= 2, "MatMul operands must have rank 2 or more");
+        const PartialShape& lead = sa.size() >= sb.size() ? sa : sb;
+        std::vector<Dimension> dims(lead.begin(), lead.end() - 2);
+        dims.push_back(sa[sa.size() - (transpose_a ? 1 : 2)]);
+        dims.push_back(sb[sb.size() - (transpose_b ? 2 : 1)]);
+        set_output_type(0, a.get_element_type(), PartialShape(dims));
+    }
+    bool get_transpose_a() const { return transpose_a_; }
+    bool get_transpose_b() const { return transpose_b_; }
+    std::map<std::string, std::string> standin_attributes() const override {
+        return {{"transpose_a", transpose_a_ ? "true" : "false"}, {"transpose_b", transpose_b_ ? "true" : "false"}};
+    }
+
+private:
+    bool transpose_a_, transpose_b_;
+};
+
+class Concat : public Node {
+public:
+    OPENVINO_OP("Concat", "opset1")
+    Concat(const OutputVector& args, int64_t axis) : Node(args), axis_(axis) {
+        OPENVINO_ASSERT(!args.empty(), "Concat without inputs");
+        PartialShape out = args[0].get_partial_shape();
+        const int64_t ax = axis < 0 ? axis + (int64_t)out.size() : axis;
+        OPENVINO_ASSERT(ax >= 0 && ax < (int64_t)out.size(), "Concat axis out of range");
+        std::vector<Dimension> dims(out.begin(), out.end());
+        bool dynamic = false;
+        int64_t total = 0;
+        for (const auto& a : args) {
+            const auto& d = a.get_partial_shape()[ax];
+            if (d.is_dynamic())
+                dynamic = true;
+            else
+                total += d.get_length();
+        }
+        dims[ax] = dynamic ? Dimension::dynamic() : Dimension(total);
+        set_output_type(0, args[0].get_element_type(), PartialShape(dims));
+    }
+    int64_t get_axis() const { return axis_; }
+    std::map<std::string, std::string> standin_attributes() const override { return {{"axis", std::to_string(axis_)}}; }
+
+private:
+    int64_t axis_;
+};
+}  // namespace v0
+
+namespace util {
+// data, indices, axis (a Constant); batch_dims as attribute
+class GatherBase : public Node {
+public:
+    int64_t get_axis() const {
+        auto c = std::dynamic_pointer_cast<v0::Constant>(get_input_node_shared_ptr(2));
+        OPENVINO_ASSERT(c && c->get_byte_size() >= 4, "Gather axis must be a constant");
+        int64_t axis = 0;
+        if (c->get_output_element_type(0).size() == 8)
+            std::memcpy(&axis, c->get_data_ptr(), 8);
+        else {
+            int32_t a32;
+            std::memcpy(&a32, c->get_data_ptr(), 4);
+            axis = a32;
+        }
+        return axis < 0 ? axis + (int64_t)get_input_partial_shape(0).size() : axis;
+    }
+    int64_t get_batch_dims() const { return batch_dims_; }
+
+protected:
+    GatherBase(const Output<Node>& data, const Output<Node>& indices, const Output<Node>& axis, int64_t batch_dims)
+        : Node(OutputVector{data, indices, axis}), batch_dims_(batch_dims) {
+        const PartialShape &d = data.get_partial_shape(), &i = indices.get_partial_shape();
+        const int64_t ax = get_axis();
+        OPENVINO_ASSERT(ax >= 0 && ax < (int64_t)d.size() && batch_dims >= 0 && batch_dims <= ax, "Gather axis / batch_dims out of range");
+        std::vector<Dimension> dims(d.begin(), d.begin() + ax);
+        dims.insert(dims.end(), i.begin() + batch_dims, i.end());
+        dims.insert(dims.end(), d.begin() + ax + 1, d.end());
+        set_output_type(0, data.get_element_type(), PartialShape(dims));
+    }
+    int64_t batch_dims_;
+};
+}  // namespace util
+
+namespace v8 {
+class Gather : public util::GatherBase {
+public:
+    OPENVINO_OP("Gather", "opset8")
+    Gather(const Output<Node>& data, const Output<Node>& indices, const Output<Node>& axis, int64_t batch_dims = 0)
+        : util::GatherBase(data, indices, axis, batch_dims) {}
+    std::map<std::string, std::string> standin_attributes() const override {
+        return {{"batch_dims", std::to_string(batch_dims_)}};
+    }
+};
+}  // namespace v8
+
+namespace internal {
+// data, gamma; out = data / sqrt(mean(data^2, last axis) + epsilon) * gamma
+class RMS : public Node {
+public:
+    OPENVINO_OP("RMS", "ie_internal_opset")
+    RMS(const Output<Node>& data, const Output<Node>& gamma, double epsilon, const element::Type output_type = element::dynamic)
+        : Node(OutputVector{data, gamma}), epsilon_(epsilon), output_type_(output_type) {
+        set_output_type(0, output_type == element::dynamic ? data.get_element_type() : output_type, data.get_partial_shape());
+    }
+    double get_epsilon() const { return epsilon_; }
+    const element::Type& get_output_type() const { return output_type_; }
+    std::map<std::string, std::string> standin_attributes() const override {
+        std::ostringstream e;
+        e.precision(17);
+        e << epsilon_;
+        return {{"epsilon", e.str()}, {"output_type", output_type_.get_type_name()}};
+    }
+
+private:
+    double epsilon_;
+    element::Type output_type_;
+};
+
+// x, cos, sin [, position ids]; rotary position embedding with the layout described by Config
+class RoPE : public Node {
+public:
+    OPENVINO_OP("RoPE", "ie_internal_opset")
+    struct Config {
+        size_t slice_start = 0;  // slice of the innermost axis of x that holds the heads to rotate
+        size_t slice_stop = 0;
+        bool input_trans0213 = false;   // x comes as [batch, length, heads, size] instead of [batch, heads, length, size]
+        bool output_trans0213 = false;  // the output is wanted as [batch, length, heads, size]
+        bool is_interleaved = false;    // adjacent pairs instead of rotate-half
+        size_t rotary_ndims = 0;
+        bool is_chatglm = false;
+        bool support_2d_rope = false;
+        bool is_qwen = false;
+        bool use_rope_cache = false;
+        size_t head_cnt = 0;
+        size_t head_size = 0;
+        int gather_position_arg_id = 0;  // index of the position input, 0 = none
+    };
+    RoPE(const OutputVector& args, const Config& cfg) : Node(args), config_(cfg) {
+        OPENVINO_ASSERT(args.size() >= 3, "RoPE takes x, cos, sin [, positions]");
+        const PartialShape& x = args[0].get_partial_shape();
+        std::vector<Dimension> dims(x.begin(), x.end());
+        if (dims.size() == 2 && cfg.head_cnt && cfg.head_size) {  // [tokens, packed] -> [tokens, heads * size]
+            dims[1] = Dimension((int64_t)(cfg.head_cnt * cfg.head_size));
+        } else if (dims.size() == 3 && cfg.head_cnt && cfg.head_size) {  // [batch, length, packed] -> heads split out
+            dims[2] = Dimension((int64_t)cfg.head_cnt);
+            dims.push_back(Dimension((int64_t)cfg.head_size));
+            if (!cfg.output_trans0213) std::swap(dims[1], dims[2]);
+        } else if (dims.size() == 4 && cfg.input_trans0213 != cfg.output_trans0213) {
+            std::swap(dims[1], dims[2]);
+        }
+        set_output_type(0, args[0].get_element_type(), PartialShape(dims));
+    }
+    const Config& get_config() const { return config_; }
+    std::map<std::string, std::string> standin_attributes() const override {
+        auto b = [](bool v) { return std::string(v ? "true" : "false"); };
+        return {{"slice_start", std::to_string(config_.slice_start)}, {"slice_stop", std::to_string(config_.slice_stop)},
+                {"input_trans0213", b(config_.input_trans0213)}, {"output_trans0213", b(config_.output_trans0213)},
+                {"is_interleaved", b(config_.is_interleaved)}, {"rotary_ndims", std::to_string(config_.rotary_ndims)},
+                {"is_chatglm", b(config_.is_chatglm)}, {"support_2d_rope", b(config_.support_2d_rope)},
+                {"is_qwen", b(config_.is_qwen)}, {"use_rope_cache", b(config_.use_rope_cache)},
+                {"head_cnt", std::to_string(config_.head_cnt)}, {"head_size", std::to_string(config_.head_size)},
+                {"gather_position_arg_id", std::to_string(config_.gather_position_arg_id)}};
+    }
+
+private:
+    Config config_;
+};
+}  // namespace internal
 }  // namespace op
 
 using ParameterVector = std::vector<std::shared_ptr<op::v0::Parameter>>;
@@ -1064,6 +1238,30 @@ public:
                 n = a;
             } else if (type == "Add") {
                 n = std::make_shared<op::v1::Add>(inputs.at(0), inputs.at(1));
+            } else if (type == "MatMul") {
+                n = std::make_shared<op::v0::MatMul>(inputs.at(0), inputs.at(1), attrs["transpose_a"] == "true",
+                                                     attrs["transpose_b"] == "true");
+            } else if (type == "Concat") {
+                n = std::make_shared<op::v0::Concat>(inputs, std::stoll(attrs.at("axis")));
+            } else if (type == "Gather") {
+                n = std::make_shared<op::v8::Gather>(inputs.at(0), inputs.at(1), inputs.at(2),
+                                                     attrs.count("batch_dims") ? std::stoll(attrs["batch_dims"]) : 0);
+            } else if (type == "RMS") {
+                n = std::make_shared<op::internal::RMS>(inputs.at(0), inputs.at(1), std::stod(attrs.at("epsilon")),
+                                                        attrs.count("output_type") ? element::type_from_name(attrs["output_type"])
+                                                                                   : element::dynamic);
+            } else if (type == "RoPE") {
+                op::internal::RoPE::Config c;
+                auto num = [&](const char* k, size_t dflt) { return attrs.count(k) ? (size_t)std::stoull(attrs[k]) : dflt; };
+                auto flag = [&](const char* k) { return attrs.count(k) && attrs[k] == "true"; };
+                c.slice_start = num("slice_start", 0), c.slice_stop = num("slice_stop", 0);
+                c.input_trans0213 = flag("input_trans0213"), c.output_trans0213 = flag("output_trans0213");
+                c.is_interleaved = flag("is_interleaved"), c.rotary_ndims = num("rotary_ndims", 0);
+                c.is_chatglm = flag("is_chatglm"), c.support_2d_rope = flag("support_2d_rope");
+                c.is_qwen = flag("is_qwen"), c.use_rope_cache = flag("use_rope_cache");
+                c.head_cnt = num("head_cnt", 0), c.head_size = num("head_size", 0);
+                c.gather_position_arg_id = (int)num("gather_position_arg_id", 0);
+                n = std::make_shared<op::internal::RoPE>(inputs, c);
             } else {
                 OPENVINO_THROW("stand-in model stream holds an operator of type '", type, "'");
             }

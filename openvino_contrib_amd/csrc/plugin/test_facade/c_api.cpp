@@ -289,6 +289,12 @@ API int hip_model_create_accumulator(int dtype, int rank, const int64_t* shape, 
     });
 }
 
+// A model in the stand-in text form (what export_model writes): lets a test describe any graph of
+// the operators the stand-in knows.
+API int hip_model_create_from_text(const char* text, hip_model_t** model) {
+    return guarded([&] { *model = new hip_model_s{ov::standin::Core().read_model(std::string(text), ov::Tensor())}; });
+}
+
 namespace {
 class SuperOperation : public ov::Node {
 public:

@@ -29,6 +29,7 @@ SYMBOLS = {
     "hip_model_create_sdpa": (_i, [_i, _i, _i64p, _i64p, _i, _i, _i, _i64p, _i, ctypes.c_float, _P(_vp)]),
     "hip_model_create_paged_attention": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _P(_vp)]),
     "hip_model_create_accumulator": (_i, [_i, _i, _i64p, _P(_vp)]),
+    "hip_model_create_from_text": (_i, [_cp, _P(_vp)]),
     "hip_model_create_unsupported": (_i, [_P(_vp)]),
     "hip_model_destroy": (None, [_vp]),
     "hip_compiled_model_destroy": (None, [_vp]),
@@ -98,6 +99,45 @@ def registered_operations():
     return _text(lib().hip_plugin_registered_operations).split(",")
 
 
+_TYPE_NAMES = {F32: "f32", F16: "f16", BF16: "bf16", U8: "u8", I32: "i32", BOOL: "boolean"}
+
+
+class GraphText:
+    """Writes a graph in the stand-in text form, node by node: `add` returns the node's index, an
+    input is an index (output 0) or an (index, port) pair.  Parameters and Results take part in the
+    compiled model's inputs / outputs in the order they are added."""
+
+    def __init__(self, name="model"):
+        self.lines = ["standin-ir 1 " + name]
+
+    def add(self, type_name, name, inputs=(), **attrs):
+        idx = len(self.lines) - 1
+        ins = ",".join("%d:%d" % (i if isinstance(i, tuple) else (i, 0)) for i in inputs)
+        body = "".join("%s=%s;" % (k, ("true" if v else "false") if isinstance(v, bool) else v) for k, v in attrs.items())
+        self.lines.append("%d %s %s inputs=%s {%s}" % (idx, type_name, name, ins, body))
+        return idx
+
+    @staticmethod
+    def _shape(shape):
+        return "[" + ",".join("?" if d < 0 else str(d) for d in shape) + "]"
+
+    def parameter(self, name, dtype, shape):
+        return self.add("Parameter", name, element_type=_TYPE_NAMES.get(dtype, dtype), shape=self._shape(shape))
+
+    def constant(self, name, array, type_name):
+        array = np.ascontiguousarray(array)
+        return self.add("Constant", name, element_type=type_name, shape=self._shape(array.shape), data=array.tobytes().hex())
+
+    def result(self, name, source):
+        return self.add("Result", name, [source])
+
+    def text(self):
+        return "\n".join(self.lines) + "\n"
+
+    def model(self):
+        return Model.from_text(self.text())
+
+
 class Model:
     def __init__(self, handle):
         self.handle = handle
@@ -126,6 +166,13 @@ class Model:
     def accumulator(cls, dtype, shape):
         h = _vp()
         _check(lib().hip_model_create_accumulator(dtype, len(shape), _shape(shape), ctypes.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def from_text(cls, text):
+        """A model in the stand-in text form; GraphText builds it."""
+        h = _vp()
+        _check(lib().hip_model_create_from_text(text.encode(), ctypes.byref(h)))
         return cls(h)
 
     @classmethod

@@ -1,0 +1,257 @@
+"""The operators around attention through the plugin (compile_model on device "HIP", infer), each
+against the CPU oracle, and then chained into the attention half of a decoder layer:
+RMS -> q/k/v MatMul -> RoPE -> PagedAttentionExtension -> output MatMul -> residual Add."""
+import numpy as np
+import pytest
+
+from openvino_contrib_amd import device_case as H
+from openvino_contrib_amd import plugin_capi as P
+from openvino_contrib_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+F32, F16, BF16 = W.F32, W.F16, W.BF16
+ROUND = {F32: 2e-6, F16: 1e-3, BF16: 8e-3}
+
+
+def scaled_error(got, ref):
+    return float(np.max(np.abs(got - ref) / np.maximum(1.0, np.abs(ref))))
+
+
+def run(compiled, inputs):
+    """inputs: list of (array in storage form, dtype code)."""
+    req = compiled.create_infer_request()
+    for i, (a, dt) in enumerate(inputs):
+        req.set_input(i, a, dt)
+    req.infer()
+    return req
+
+
+def storage(x, dtype):
+    st, exact = W.to_storage(np.asarray(x, np.float32), dtype)
+    return st, exact
+
+
+@pytest.mark.parametrize("dtype", [BF16, F16, F32])
+def test_rms_through_the_plugin(hip, oracle, dtype):
+    rng = np.random.default_rng(1)
+    g = P.GraphText("rms")
+    x = g.parameter("x", dtype, [-1, -1, 256])
+    gamma_st, gamma = storage(1.0 + 0.2 * rng.standard_normal(256), dtype)
+    gm = g.constant("gamma", gamma_st, P._TYPE_NAMES[dtype])
+    g.result("out", g.add("RMS", "norm", [x, gm], epsilon=1e-5, output_type="dynamic"))
+    compiled = P.Plugin().compile_model(g.model())
+    for shape in ((2, 5, 256), (1, 1, 256), (3, 0, 256)):
+        x_st, xv = storage(rng.standard_normal(shape) * 3, dtype)
+        out, _ = run(compiled, [(x_st, dtype)]).output(0)
+        assert out.shape == shape
+        if out.size:
+            assert scaled_error(H.storage_to_f32(out, dtype), oracle.rms_norm(xv, gamma, 1e-5)) <= ROUND[dtype]
+
+
+def rope_tables(rows, rot, base=10000.0):
+    inv = base ** (-np.arange(0, rot, 2) / rot)
+    ang = np.arange(rows)[:, None] * inv[None, :]
+    return np.cos(np.tile(ang, 2)).astype(np.float32), np.sin(np.tile(ang, 2)).astype(np.float32)
+
+
+@pytest.mark.parametrize("in_t,out_t", [(False, False), (True, False), (True, True), (False, True)])
+def test_rope_rank4_layouts(hip, oracle, in_t, out_t):
+    rng = np.random.default_rng(2)
+    B, Hh, L, S = 2, 3, 7, 64
+    g = P.GraphText("rope4")
+    x = g.parameter("x", F16, [-1, -1, -1, S])
+    c = g.parameter("cos", F32, [-1, S])
+    s = g.parameter("sin", F32, [-1, S])
+    g.result("out", g.add("RoPE", "rope", [x, c, s], input_trans0213=in_t, output_trans0213=out_t, rotary_ndims=S))
+    compiled = P.Plugin().compile_model(g.model())
+    cos, sin = rope_tables(L, S)
+    xv = rng.standard_normal((B, Hh, L, S)).astype(np.float32)           # logical [batch, heads, length, size]
+    x_st, xv = storage(xv, F16)
+    feed = np.ascontiguousarray(x_st.transpose(0, 2, 1, 3)) if in_t else x_st
+    out, _ = run(compiled, [(feed, F16), (cos, F32), (sin, F32)]).output(0)
+    got = H.storage_to_f32(out, F16)
+    if out_t:
+        assert got.shape == (B, L, Hh, S)
+        got = got.transpose(0, 2, 1, 3)
+    ref = np.stack([oracle.rope(np.ascontiguousarray(xv[b].transpose(1, 0, 2)), cos, sin).transpose(1, 0, 2) for b in range(B)])
+    assert got.shape == ref.shape and scaled_error(got, ref) <= 2 * ROUND[F16]
+
+
+def test_rope_on_packed_tokens_with_positions(hip, oracle):
+    """The layout in front of PagedAttentionExtension: [tokens, packed q|k|v], the k heads rotated in a slice."""
+    rng = np.random.default_rng(3)
+    T, Hq, Hkv, S, rot = 19, 4, 2, 128, 64
+    packed = (Hq + 2 * Hkv) * S
+    g = P.GraphText("rope2")
+    x = g.parameter("qkv", BF16, [-1, packed])
+    c = g.parameter("cos", BF16, [-1, rot])
+    s = g.parameter("sin", BF16, [-1, rot])
+    pos = g.parameter("positions", P.I32, [-1])
+    g.result("k_rot", g.add("RoPE", "rope_k", [x, c, s, pos], slice_start=Hq * S, slice_stop=(Hq + Hkv) * S, head_cnt=Hkv,
+                            head_size=S, rotary_ndims=rot, gather_position_arg_id=3))
+    compiled = P.Plugin().compile_model(g.model())
+    cos, sin = rope_tables(500, rot)
+    cos_st, cos = storage(cos, BF16)
+    sin_st, sin = storage(sin, BF16)
+    x_st, xv = storage(rng.standard_normal((T, packed)), BF16)
+    positions = rng.integers(0, 500, T).astype(np.int32)
+    out, _ = run(compiled, [(x_st, BF16), (cos_st, BF16), (sin_st, BF16), (positions, P.I32)]).output(0)
+    assert out.shape == (T, Hkv * S)
+    ref = oracle.rope(xv[:, Hq * S:(Hq + Hkv) * S].reshape(T, Hkv, S), cos, sin, positions, rot).reshape(T, Hkv * S)
+    assert scaled_error(H.storage_to_f32(out, BF16), ref) <= 2 * ROUND[BF16]
+
+
+def test_rope_variants_the_plugin_refuses(hip):
+    plugin = P.Plugin()
+    for attrs in (dict(is_chatglm=True), dict(is_qwen=True), dict(support_2d_rope=True), dict(use_rope_cache=True),
+                  dict(gather_position_arg_id=2)):
+        g = P.GraphText("r")
+        x = g.parameter("x", F16, [-1, -1, -1, 64])
+        c = g.parameter("cos", F32, [-1, 64])
+        s = g.parameter("sin", F32, [-1, 64])
+        g.result("out", g.add("RoPE", "rope", [x, c, s], **attrs))
+        assert "rope" not in plugin.query_model(g.model())
+        with pytest.raises(P.PluginError):
+            plugin.compile_model(g.model())
+
+
+@pytest.mark.parametrize("a_shape,b_shape,ta,tb", [((37, 96), (80, 96), False, True), ((2, 3, 20, 48), (48, 16), False, False),
+                                                    ((4, 48, 20), (4, 48, 16), True, False), ((1, 64), (6, 24, 64), False, True)])
+def test_matmul_through_the_plugin(hip, oracle, a_shape, b_shape, ta, tb):
+    rng = np.random.default_rng(4)
+    g = P.GraphText("mm")
+    a = g.parameter("a", BF16, [-1] * (len(a_shape) - 1) + [a_shape[-1]])
+    b = g.parameter("b", BF16, list(b_shape))
+    g.result("out", g.add("MatMul", "mm", [a, b], transpose_a=ta, transpose_b=tb))
+    compiled = P.Plugin().compile_model(g.model())
+    a_st, av = storage(rng.standard_normal(a_shape), BF16)
+    b_st, bv = storage(rng.standard_normal(b_shape), BF16)
+    out, _ = run(compiled, [(a_st, BF16), (b_st, BF16)]).output(0)
+    a3 = av.reshape((-1,) + a_shape[-2:])
+    b3 = bv.reshape((-1,) + b_shape[-2:])
+    ref = oracle.matmul(a3 if a3.shape[0] > 1 else a3[0], b3 if b3.shape[0] > 1 else b3[0], ta, tb)
+    lead = a_shape[:-2] if len(a_shape) >= len(b_shape) and int(np.prod(a_shape[:-2])) >= int(np.prod(b_shape[:-2])) else b_shape[:-2]
+    assert out.shape == tuple(lead) + ref.shape[-2:]
+    assert scaled_error(H.storage_to_f32(out, BF16).reshape(ref.shape), ref) <= ROUND[BF16] + 1e-5
+
+
+def test_gather_embedding_and_concat_through_the_plugin(hip, oracle):
+    rng = np.random.default_rng(5)
+    g = P.GraphText("embed")
+    table_st, _ = storage(rng.standard_normal((300, 64)), F16)
+    table = g.constant("table", table_st, "f16")
+    ids = g.parameter("ids", P.I32, [-1])
+    axis = g.constant("axis", np.array(0, np.int64), "i64")
+    emb = g.add("Gather", "embed", [table, ids, axis], batch_dims=0)
+    extra = g.parameter("extra", F16, [-1, 16])
+    g.result("out", g.add("Concat", "cat", [emb, extra], axis=-1))
+    plugin = P.Plugin()
+    assert {"embed", "cat"} <= set(plugin.query_model(g.model()))
+    compiled = plugin.compile_model(g.model())
+    tokens = rng.integers(-300, 300, 23).astype(np.int32)
+    extra_st, _ = storage(rng.standard_normal((23, 16)), F16)
+    req = run(compiled, [(tokens, P.I32), (extra_st, F16)])
+    out, _ = req.output(0)
+    ref = oracle.concat([oracle.gather(table_st, tokens, 0), extra_st], 1)
+    assert np.array_equal(out, ref)
+    # the table is a Constant: a second infer on the same request reuses the device copy
+    tokens2 = rng.integers(0, 300, 5).astype(np.int32)
+    req.set_input(0, tokens2, P.I32)
+    req.set_input(1, extra_st[:5], F16)
+    req.infer()
+    out, _ = req.output(0)
+    assert np.array_equal(out, oracle.concat([oracle.gather(table_st, tokens2, 0), extra_st[:5]], 1))
+
+
+def test_attention_half_of_a_decoder_layer(hip, oracle):
+    """hidden -> RMS -> q, k, v projections -> RoPE(q), RoPE(k) -> PagedAttentionExtension (device-resident
+    cache, mixed prefill + decode batch) -> output projection -> + hidden, all on device "HIP", against
+    the chain of oracle functions with the same bf16 roundings between the operators."""
+    rng = np.random.default_rng(6)
+    Hq, Hkv, D, hidden, bs = 4, 2, 128, 512, 32
+    seqs = [(0, 70), (300, 1), (41, 1), (96, 33)]
+    case = W.make_paged_case(96, seqs, Hq, Hkv, D, bs, BF16, BF16, F16)
+    T = case["q"].shape[0]
+    g = P.GraphText("decoder_attention")
+    hid = g.parameter("hidden", BF16, [-1, hidden])
+    w = {n: g.parameter(n, BF16, [width, hidden if n != "wo" else Hq * D])
+         for n, width in (("wq", Hq * D), ("wk", Hkv * D), ("wv", Hkv * D), ("wo", hidden))}
+    cos_p = g.parameter("cos", F32, [-1, D])
+    sin_p = g.parameter("sin", F32, [-1, D])
+    pos_p = g.parameter("positions", P.I32, [-1])
+    kc_p = g.parameter("key_cache", F16, [-1, Hkv, bs, D])
+    vc_p = g.parameter("value_cache", F16, [-1, Hkv, bs, D])
+    idx = [g.parameter(n, P.I32, [-1]) for n in ("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")]
+    scale_p = g.parameter("scale", F32, [-1])
+    win_p = g.parameter("sliding_window", P.I32, [-1])
+    alibi_p = g.parameter("alibi_slopes", F32, [0])
+    mcl_p = g.parameter("max_context_len", P.I32, [-1])
+    gamma_st, gamma = storage(1.0 + 0.1 * rng.standard_normal(hidden), BF16)
+    norm = g.add("RMS", "input_norm", [hid, g.constant("gamma", gamma_st, "bf16")], epsilon=1e-5, output_type="dynamic")
+    q = g.add("MatMul", "q_proj", [norm, w["wq"]], transpose_a=False, transpose_b=True)
+    k = g.add("MatMul", "k_proj", [norm, w["wk"]], transpose_a=False, transpose_b=True)
+    v = g.add("MatMul", "v_proj", [norm, w["wv"]], transpose_a=False, transpose_b=True)
+    qr = g.add("RoPE", "q_rope", [q, cos_p, sin_p, pos_p], head_cnt=Hq, head_size=D, rotary_ndims=D, gather_position_arg_id=3)
+    kr = g.add("RoPE", "k_rope", [k, cos_p, sin_p, pos_p], head_cnt=Hkv, head_size=D, rotary_ndims=D, gather_position_arg_id=3)
+    pa = g.add("PagedAttentionExtension", "attention", [qr, kr, v, kc_p, vc_p] + idx + [scale_p, win_p, alibi_p, mcl_p])
+    o = g.add("MatMul", "o_proj", [pa, w["wo"]], transpose_a=False, transpose_b=True)
+    g.result("out", g.add("Add", "residual", [o, hid]))
+    plugin = P.Plugin()
+    plugin.set_property("PERF_COUNT", "YES")
+    supported = plugin.query_model(g.model())
+    assert {"input_norm", "q_proj", "q_rope", "k_rope", "attention", "o_proj", "residual"} <= set(supported)
+    compiled = plugin.compile_model(g.model())
+
+    hid_st, hv = storage(rng.standard_normal((T, hidden)), BF16)
+    weights = {n: storage(rng.standard_normal(shape) / np.sqrt(shape[1]), BF16)
+               for n, shape in (("wq", (Hq * D, hidden)), ("wk", (Hkv * D, hidden)), ("wv", (Hkv * D, hidden)), ("wo", (hidden, Hq * D)))}
+    positions = np.concatenate([np.arange(p, p + n) for p, n in seqs]).astype(np.int32)
+    cos, sin = rope_tables(int(positions.max()) + 1, D)
+    kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
+    vc = hip.DeviceBuffer.from_numpy(case["value_cache"])
+    dev_w = {n: hip.DeviceBuffer.from_numpy(st) for n, (st, _) in weights.items()}   # weights stay on the device
+    req = compiled.create_infer_request()
+    names = compiled.input_names()
+    host = {"hidden": (hid_st, BF16), "cos": (cos, F32), "sin": (sin, F32), "positions": (positions, P.I32),
+            "past_lens": (case["past_lens"], P.I32), "subsequence_begins": (case["subsequence_begins"], P.I32),
+            "block_indices": (case["block_indices"], P.I32), "block_indices_begins": (case["block_indices_begins"], P.I32),
+            "scale": (np.zeros((0,), np.float32), F32), "sliding_window": (np.array([0], np.int32), P.I32),
+            "alibi_slopes": (np.zeros((0,), np.float32), F32),
+            "max_context_len": (np.array([case["max_context_len"]], np.int32), P.I32)}
+    cache_shape = list(case["key_cache"].shape[:3]) + [D]
+    for i, n in enumerate(names):
+        if n in host:
+            req.set_input(i, *host[n])
+        elif n in dev_w:
+            req.set_device_input(i, dev_w[n].ptr, BF16, list(weights[n][0].shape))
+        elif n == "key_cache":
+            req.set_device_input(i, kc.ptr, F16, cache_shape)
+        elif n == "value_cache":
+            req.set_device_input(i, vc.ptr, F16, cache_shape)
+        else:
+            raise AssertionError("unexpected input " + n)
+    req.infer()
+    out, _ = req.output(0)
+    got = H.storage_to_f32(out, BF16)
+
+    r = lambda x: oracle.round_to(x, BF16)
+    n_ref = r(oracle.rms_norm(hv, gamma, 1e-5))
+    q_ref, k_ref, v_ref = (r(oracle.matmul(n_ref, weights[n][1], False, True)) for n in ("wq", "wk", "wv"))
+    qr_ref = r(oracle.rope(q_ref.reshape(T, Hq, D), cos, sin, positions)).reshape(T, Hq * D)
+    kr_ref = r(oracle.rope(k_ref.reshape(T, Hkv, D), cos, sin, positions)).reshape(T, Hkv * D)
+    okc, ovc = case["key_cache"].copy(), case["value_cache"].copy()
+    att = r(oracle.paged_attention(qr_ref, kr_ref, v_ref, okc, ovc, F16, case["past_lens"], case["subsequence_begins"],
+                                   case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs))
+    ref = r(r(oracle.matmul(att, weights["wo"][1], False, True)) + hv)
+    err = scaled_error(got, ref)
+    print("decoder attention block: scaled max error %.4g, plain %.4g" % (err, float(np.max(np.abs(got - ref)))), flush=True)
+    # every operator rounds to bf16 once (2^-9 relative) and a one-ulp difference in an intermediate
+    # spreads through the products that follow
+    assert err <= 3e-2
+    # the new tokens' keys went into the device-resident cache; a bf16 rounding difference in the
+    # projection in front of it may flip the last bit of an fp16 cache entry
+    kc_got = kc.download(np.uint8, case["key_cache"].shape).view(np.float16).astype(np.float32)
+    assert float(np.max(np.abs(kc_got - okc.view(np.float16).astype(np.float32)))) <= 0.07
+    types = [t for _, t, _ in req.profiling()]
+    assert types.count("MatMul") == 4 and types.count("RoPE") == 2 and "PagedAttentionExtension" in types

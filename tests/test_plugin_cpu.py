@@ -26,8 +26,36 @@ def test_header_binding_and_exports_agree():
 def test_registry_holds_the_attention_operators():
     ops = P.registered_operations()
     for name in ("Parameter", "Result", "Constant", "ScaledDotProductAttention", "PagedAttentionExtension", "ReadValue",
-                 "Assign", "Add"):
+                 "Assign", "Add", "RMS", "RoPE", "MatMul", "Gather", "Concat"):
         assert name in ops
+
+
+def test_query_model_on_the_operators_around_attention():
+    """A text-form graph of RMS / MatMul / RoPE / Gather / Concat nodes: supported ones are listed,
+    nodes an operator's constructor refuses are not (src/cuda_plugin.cpp:171-188)."""
+    import numpy as np
+
+    g = P.GraphText("layer")
+    ids = g.parameter("ids", P.I32, [-1])
+    table = g.constant("table", np.zeros((10, 64), np.uint16), "f16")
+    axis = g.constant("axis", np.array(0, np.int64), "i64")
+    emb = g.add("Gather", "embed", [table, ids, axis], batch_dims=0)
+    gamma = g.constant("gamma", np.zeros(64, np.uint16), "f16")
+    norm = g.add("RMS", "norm", [emb, gamma], epsilon=1e-6, output_type="dynamic")
+    w = g.parameter("w", P.F16, [128, 64])
+    proj = g.add("MatMul", "proj", [norm, w], transpose_a=False, transpose_b=True)
+    cos = g.parameter("cos", P.F32, [-1, 64])
+    sin = g.parameter("sin", P.F32, [-1, 64])
+    rope = g.add("RoPE", "rope", [proj, cos, sin], head_cnt=2, head_size=64, rotary_ndims=64)
+    glm = g.add("RoPE", "rope_glm", [proj, cos, sin], head_cnt=2, head_size=64, is_chatglm=True)
+    w32 = g.parameter("w32", P.F32, [128, 64])
+    mixed = g.add("MatMul", "mixed", [norm, w32], transpose_a=False, transpose_b=True)
+    cat = g.add("Concat", "cat", [rope, glm], axis=1)
+    g.result("out", cat)
+    g.result("out2", mixed)
+    supported = set(P.Plugin().query_model(g.model()))
+    assert {"embed", "norm", "proj", "rope", "cat"} <= supported
+    assert "rope_glm" not in supported and "mixed" not in supported
 
 
 def test_plugin_object_comes_from_create_plugin_engine():
