@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-cpu] [--no-extra] [--no-plugin]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer] [--no-cpu] [--no-extra] [--no-plugin]
 
 Prints ONE JSON line.  The headline is the fp16 paged-attention decode step (configuration 3
 of BASELINE.json): a "step" is one hipattn_paged_attention call on the whole synthetic batch
@@ -14,7 +14,9 @@ configurations are measured the same way and reported under "workloads" in the s
 c5: mixed chunked prefill + decode), each with a `cpu_baseline` of its own.  `cpu_baseline` times
 the CPU oracle (a restatement, not OpenVINO's CPU plugin: OpenVINO is not installed) on a bounded
 sample of the same workload.  `plugin_ms_per_step` of the headline workload is the same step through
-the plugin layer's InferRequest::infer with device-resident tensors.
+the plugin layer's InferRequest::infer with device-resident tensors.  The operators around attention
+(RMS norm, RoPE, MatMul, Gather, Concat of libhipops.so) ride along under "workloads" too, or alone
+with --workload layer.
 """
 import argparse
 import json
@@ -272,13 +274,157 @@ def cpu_baseline_sdpa(case, budget_s=20.0):
                       % (len(times), case["B"] * case["Hkv"], sum(times))}
 
 
+def bench_layer_ops(hip, steps, warmup, with_cpu):
+    """The operators around attention (libhipops.so) at the shapes of a decoder layer that feeds
+    configuration 2 (8,192 tokens, hidden 4,096, 32 query and 8 kv heads of 128) and of a 64-token
+    decode step.  Each operator is one kernel; its duration is the mean of `steps` back-to-back
+    launches between two events.  Rooflines: algorithmic bytes (every input and output byte once)
+    against 8 TB/s, or 2*m*n*k against the dense bf16 MFMA peak."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    from openvino_contrib_amd import ops_capi as ops
+    from openvino_contrib_amd import workloads as W
+
+    ops.lib()
+    rng = np.random.default_rng(2024)
+    T, hidden, Hq, Hkv, D, vocab = 8192, 4096, 32, 8, 128, 32000
+    BF16 = W.BF16
+
+    def dev(shape, scale=1.0):
+        st, exact = W.to_storage((rng.standard_normal(shape) * scale).astype(np.float32), BF16)
+        return hip.DeviceBuffer.from_numpy(st), exact
+
+    def timed(fn):
+        e0, e1 = hip.Event(), hip.Event()
+        ramped = 0.0
+        while ramped < CLOCK_RAMP_MS / 2:  # idle clocks, as in time_steps
+            e0.record()
+            for _ in range(64):
+                fn()
+            e1.record()
+            e1.synchronize()
+            ramped += e0.elapsed_ms(e1)
+        for _ in range(max(warmup, 3)):
+            fn()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_ms(e1) / steps
+        e0.close()
+        e1.close()
+        return ms
+
+    def cpu_time(fn, budget_s=2.0):
+        times, t_begin = [], time.perf_counter()
+        while not times or (time.perf_counter() - t_begin < budget_s and len(times) < 50):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        return sum(times) / len(times), len(times)
+
+    def hbm(name, ms, nbytes, kernel):
+        a = nbytes / (ms * 1e-3) / 1e9
+        return {"workload": name, "ms_per_step": ms, "dominant_kernel_ms": ms, "bytes": nbytes,
+                "roofline": {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
+                             "traffic": None, "kernel": kernel}}
+
+    out = {}
+    import oracle as O
+    sample = 256  # rows of the CPU samples
+
+    # RMS norm
+    dx, x = dev((T, hidden))
+    dg, g = dev((hidden,))
+    do = hip.DeviceBuffer(T * hidden * 2)
+    ms = timed(lambda: ops.rms_norm(dx, dg, do, T, hidden, 1e-5, BF16, BF16, BF16))
+    out["rms"] = hbm("RMS norm, %d x %d bf16" % (T, hidden), ms, 2 * T * hidden * 2 + hidden * 2, "rms_norm_vec_kernel")
+    if with_cpu:
+        t, n = cpu_time(lambda: O.rms_norm(x[:sample], g, 1e-5))
+        out["rms"]["cpu_baseline"] = {"value": (2 * sample * hidden * 4) / t / 1e9, "unit": "GB/s", "cores": O.num_threads(),
+                                      "kind": "port", "sample": "oracle (fp32) on %d of %d rows, mean of %d passes" % (sample, T, n)}
+
+    # RoPE on the query heads
+    pos = hip.DeviceBuffer.from_numpy(np.arange(T, dtype=np.int32) % 2048)
+    inv = 10000.0 ** (-np.arange(0, D, 2) / D)
+    ang = np.arange(2048)[:, None] * inv[None, :]
+    cos, sin = np.cos(np.tile(ang, 2)).astype(np.float32), np.sin(np.tile(ang, 2)).astype(np.float32)
+    dc, ds = hip.DeviceBuffer.from_numpy(cos), hip.DeviceBuffer.from_numpy(sin)
+    dq, q = dev((T, Hq, D))
+    dqo = hip.DeviceBuffer(T * Hq * D * 2)
+    rd = ops.RopeDesc(BF16, W.F32, T, Hq, D, D, 0, Hq * D, D, Hq * D, D, 2048, D)
+    ms = timed(lambda: ops.rope(rd, dq, dc, ds, pos, dqo))
+    out["rope"] = hbm("RoPE (rotate-half), %d tokens x %d heads x %d bf16, f32 tables" % (T, Hq, D), ms,
+                      2 * T * Hq * D * 2 + 2 * 2048 * D * 4 + T * 4, "rope_vec_kernel")
+    if with_cpu:
+        p = (np.arange(sample) % 2048).astype(np.int32)
+        t, n = cpu_time(lambda: O.rope(q[:sample], cos, sin, p))
+        out["rope"]["cpu_baseline"] = {"value": (2 * sample * Hq * D * 4) / t / 1e9, "unit": "GB/s", "cores": O.num_threads(),
+                                       "kind": "port", "sample": "oracle (fp32) on %d of %d tokens, mean of %d passes" % (sample, T, n)}
+
+    # Gather: embedding lookup
+    dt, table = dev((vocab, hidden))
+    ids = rng.integers(0, vocab, T).astype(np.int32)
+    dids = hip.DeviceBuffer.from_numpy(ids)
+    ms = timed(lambda: ops.gather(dt, dids, do, 1, 1, vocab, hidden * 2, T, ops.I32))
+    out["gather"] = hbm("Gather (embedding lookup), %d rows of %d bf16 from %d" % (T, hidden, vocab), ms,
+                        2 * T * hidden * 2 + T * 4, "gather_kernel")
+    if with_cpu:
+        tb = np.ascontiguousarray(table[:, :]).astype(np.float32)
+        t, n = cpu_time(lambda: O.gather(tb, ids[:sample], 0))
+        out["gather"]["cpu_baseline"] = {"value": (2 * sample * hidden * 4) / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                         "sample": "oracle (fp32 rows, one thread) on %d of %d indices, mean of %d passes" % (sample, T, n)}
+        del tb
+    dt.free()
+
+    # Concat of two halves along the last axis
+    da, _ = dev((T, hidden // 2))
+    db, _ = dev((T, hidden // 2))
+    ms = timed(lambda: ops.concat([da, db], [hidden, hidden], T, do))
+    out["concat"] = hbm("Concat of two [%d, %d] bf16 along the last axis" % (T, hidden // 2), ms, 2 * T * hidden * 2, "concat_kernel")
+
+    # MatMul: fused q|k|v projection of a prefill batch (MFMA-bound) and of a decode step (HBM-bound)
+    N = (Hq + 2 * Hkv) * D
+    dw, w = dev((N, hidden), 1.0 / 64)
+    for name, m in (("matmul_prefill", T), ("matmul_decode", 64)):
+        dc_out = hip.DeviceBuffer(m * N * 2)
+        md = ops.MatmulDesc(BF16, BF16, m, N, hidden, 1, 0, 1, 0, 0)
+        ws = hip.DeviceBuffer(ops.matmul_workspace_size(md))
+        ms = timed(lambda: ops.matmul(md, dx, dw, dc_out, ws))
+        flops = 2.0 * m * N * hidden
+        nbytes = (m * hidden + N * hidden + m * N) * 2
+        r = {"workload": "MatMul x[%d,%d] w[%d,%d]^T bf16 (q|k|v projection), hipBLASLt" % (m, hidden, N, hidden),
+             "ms_per_step": ms, "dominant_kernel_ms": ms, "flops": flops, "bytes": nbytes, "tflops": flops / (ms * 1e-3) / 1e12}
+        t_mfma, t_hbm = flops / (MFMA_BF16_PEAK_TFLOPS * 1e12), nbytes / (HBM_PEAK_GBS * 1e9)
+        if t_mfma >= t_hbm:
+            a = flops / (ms * 1e-3) / 1e12
+            r["roofline"] = {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "hipBLASLt GEMM"}
+        else:
+            a = nbytes / (ms * 1e-3) / 1e9
+            r["roofline"] = {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
+                             "traffic": None, "kernel": "hipBLASLt GEMM"}
+        if with_cpu:
+            rows = min(m, 16)
+            t, n = cpu_time(lambda: O.matmul(x[:rows], w, False, True), 3.0)
+            r["cpu_baseline"] = {"value": 2.0 * rows * N * hidden / t / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(),
+                                 "kind": "port", "sample": "oracle (fp64 accumulation) on %d of %d rows, mean of %d passes" % (rows, m, n)}
+        out[name] = r
+        dc_out.free()
+        ws.free()
+    for k, r in out.items():
+        log("%s: %.4f ms, roofline frac %.3f (%s)" % (k, r["ms_per_step"], r["roofline"]["frac"], r["roofline"]["bound"]))
+    return out
+
+
 def main():
     global CLOCK_RAMP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "copy", "mfma"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "copy", "mfma"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
                          "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
@@ -319,6 +465,11 @@ def main():
                 sys.exit("bench.py: mfma_yardstick failed with HIP error %d" % rc)
             out[name] = {"tflops": tf.value, "shader_ghz": ghz.value, "frac_of_peak": tf.value / MFMA_BF16_PEAK_TFLOPS}
         print(json.dumps(out))
+        return
+
+    if args.workload == "layer":
+        print(json.dumps({"workload": "layer", "steps": args.steps, "warmup": args.warmup,
+                          "workloads": bench_layer_ops(hip, args.steps, args.warmup, not args.no_cpu)}))
         return
 
     if args.workload == "copy":
@@ -385,6 +536,10 @@ def main():
             log("%s cpu baseline:" % w, c)
         results[w] = r
         del case
+
+    if not args.no_extra:
+        # the operators around attention, each with a roofline and a CPU figure of its own
+        results.update(bench_layer_ops(hip, args.steps, args.warmup, not args.no_cpu))
 
     head = results[args.workload]
     is_sdpa = args.workload == "c2"

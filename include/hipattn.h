@@ -24,7 +24,7 @@ extern "C" {
 #endif
 
 #define HIPATTN_VERSION_MAJOR 0
-#define HIPATTN_VERSION_MINOR 2
+#define HIPATTN_VERSION_MINOR 3
 
 typedef enum hipattn_status {
     HIPATTN_OK = 0,
@@ -219,6 +219,26 @@ hipattn_status hipattn_paged_attention(const hipattn_pa_desc* desc, const void* 
                                        const int32_t* past_lens, const int32_t* subsequence_begins,
                                        const int32_t* block_indices, const int32_t* block_indices_begins, void* out,
                                        void* workspace, size_t workspace_bytes, hipattn_stream stream);
+
+/* The operator's second output, "scores": for every cache position of every sequence the
+ * attention probability it received in this step, summed over the query heads and over the last
+ * score_aggregation_window[s] query tokens of its sequence (all of the sequence's new tokens when
+ * the pointer is NULL) - the figure a cache-eviction policy ranks tokens by.  No counterpart in the
+ * reference.  scores is f32; sequence s owns the past_lens[s] + new_tokens(s) entries that follow
+ * those of the sequences before it, so the caller sizes it with sum(past_lens) + num_tokens and
+ * passes that as scores_capacity (nothing is written beyond it).  Call it after
+ * hipattn_paged_attention of the same step, on the same stream: the cache must already hold the
+ * new tokens' keys.  Positions outside a query's sliding window and keys in blocks outside the cache
+ * count as probability zero, as in the attention itself.  The workspace holds one float per
+ * (token, query head).  Which tokens and heads OpenVINO aggregates over is restated from its
+ * documentation, not checked against it. */
+hipattn_status hipattn_paged_attention_scores_workspace_size(const hipattn_pa_desc* desc, size_t* bytes);
+hipattn_status hipattn_paged_attention_scores(const hipattn_pa_desc* desc, const void* q, const void* key_cache,
+                                              const int32_t* past_lens, const int32_t* subsequence_begins,
+                                              const int32_t* block_indices, const int32_t* block_indices_begins,
+                                              const int32_t* score_aggregation_window, float* scores,
+                                              int64_t scores_capacity, void* workspace, size_t workspace_bytes,
+                                              hipattn_stream stream);
 
 /* The same operator for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the

@@ -19,6 +19,7 @@ SOURCES = [
     "kv_cache_write.hip",
     "attention_generic.hip",
     "paged_decode.hip",
+    "paged_scores.hip",
     "flash_prefill.hip",
 ]
 

@@ -116,6 +116,8 @@ SYMBOLS = {
     "hipattn_paged_attention_workspace_size": (_i, [_P(PaDesc), _P(_sz)]),
     "hipattn_paged_attention": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hipattn_paged_attention_noalloc": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "hipattn_paged_attention_scores_workspace_size": (_i, [_P(PaDesc), _P(_sz)]),
+    "hipattn_paged_attention_scores": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int64, _vp, _sz, _vp]),
     "hipattn_set_option": (_i, [ctypes.c_char_p, _i]),
     "hipattn_kv_cache_write": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "hipattn_cache_row_bytes": (_sz, [_i, _i]),
@@ -297,6 +299,20 @@ def paged_attention_noalloc(desc, q, k_new, v_new, key_cache, value_cache, past_
         ctypes.byref(desc), q.ptr, k_new.ptr if k_new else None, v_new.ptr if v_new else None, key_cache.ptr,
         value_cache.ptr, past_lens.ptr, subsequence_begins.ptr, block_indices.ptr, block_indices_begins.ptr,
         out.ptr, _h(stream)))
+
+
+def paged_attention_scores(desc, q, key_cache, past_lens, subsequence_begins, block_indices, block_indices_begins,
+                           score_window, scores, capacity, stream=None):
+    """scores: DeviceBuffer of `capacity` floats.  The scratch (one float per token and head) is allocated here."""
+    n = _sz(0)
+    check(lib().hipattn_paged_attention_scores_workspace_size(ctypes.byref(desc), ctypes.byref(n)))
+    ws = DeviceBuffer(n.value)
+    check(lib().hipattn_paged_attention_scores(ctypes.byref(desc), q.ptr, key_cache.ptr, past_lens.ptr,
+                                               subsequence_begins.ptr, block_indices.ptr, block_indices_begins.ptr,
+                                               score_window.ptr if score_window is not None else None, scores.ptr,
+                                               capacity, ws.ptr, ws.nbytes, _h(stream)))
+    check(lib().hipattn_stream_synchronize(_h(stream)))
+    ws.free()
 
 
 def set_option(name, value):

@@ -3,6 +3,7 @@
 // a per-thread message.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -488,3 +489,60 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention_noalloc(const hipattn_pa_d
     return paged_attention_impl(desc, q, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins,
                                 block_indices, block_indices_begins, out, nullptr, 0, stream, true);
 }
+
+HIPATTN_EXPORT hipattn_status hipattn_paged_attention_scores_workspace_size(const hipattn_pa_desc* desc, size_t* bytes) {
+    if (!bytes) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_scores_workspace_size: null output");
+    *bytes = 0;
+    if (hipattn_status st = validate_pa(desc, true)) return st;
+    *bytes = (size_t)desc->num_tokens * desc->num_heads_q * sizeof(float);
+    return HIPATTN_OK;
+}
+
+HIPATTN_EXPORT hipattn_status hipattn_paged_attention_scores(const hipattn_pa_desc* desc, const void* q, const void* key_cache,
+                                                             const int32_t* past_lens, const int32_t* subsequence_begins,
+                                                             const int32_t* block_indices,
+                                                             const int32_t* block_indices_begins,
+                                                             const int32_t* score_aggregation_window, float* scores,
+                                                             int64_t scores_capacity, void* workspace,
+                                                             size_t workspace_bytes, hipattn_stream stream) {
+    if (hipattn_status st = validate_pa(desc, true)) return st;
+    if (scores_capacity < 0) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_scores: negative capacity");
+    if (desc->num_tokens == 0 || desc->num_seqs == 0 || scores_capacity == 0) return HIPATTN_OK;
+    if (!q || !key_cache || !past_lens || !subsequence_begins || !block_indices || !block_indices_begins || !scores)
+        return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_scores: null pointer");
+    if (desc->num_seqs > 65535) return fail(HIPATTN_UNSUPPORTED, "paged_attention_scores: %d sequences (at most 65535)", desc->num_seqs);
+    const size_t need = (size_t)desc->num_tokens * desc->num_heads_q * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+        return fail(HIPATTN_WORKSPACE_TOO_SMALL, "paged_attention_scores: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    if ((uintptr_t)workspace % 4) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_scores: workspace must be 4-byte aligned");
+    hipattn::ScoresParams p{};
+    p.q = q;
+    p.key_cache = (const uint8_t*)key_cache;
+    p.past_lens = past_lens;
+    p.subsequence_begins = subsequence_begins;
+    p.block_indices = block_indices;
+    p.block_indices_begins = block_indices_begins;
+    p.score_window = score_aggregation_window;
+    p.scores = scores;
+    p.scores_capacity = scores_capacity;
+    p.lse = (float*)workspace;
+    p.q_dtype = desc->q_dtype;
+    p.cache_dtype = desc->cache_dtype;
+    p.num_heads_q = desc->num_heads_q;
+    p.num_heads_kv = desc->num_heads_kv;
+    p.head_dim = desc->head_dim;
+    p.block_size = desc->block_size;
+    p.num_blocks = desc->num_blocks;
+    p.num_tokens = desc->num_tokens;
+    p.num_seqs = desc->num_seqs;
+    // no sequence is longer than its share of the cache, nor than the output
+    int64_t bound = (int64_t)desc->num_blocks * desc->block_size;
+    if (desc->max_context_len > 0) bound = std::min<int64_t>(bound, desc->max_context_len);
+    bound = std::min<int64_t>(bound, scores_capacity);
+    p.max_context_len = (int)std::min<int64_t>(bound, 0x7fffffff);
+    p.sliding_window = desc->sliding_window;
+    p.scale = desc->scale > 0.f ? desc->scale : 1.0f / sqrtf((float)desc->head_dim);
+    HIP_TRY(hipattn::launch_paged_scores(p, as_stream(stream)));
+    return HIPATTN_OK;
+}
+

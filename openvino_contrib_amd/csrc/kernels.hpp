@@ -149,6 +149,33 @@ hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t str
 // out = a + b over n elements; dtype is a HIPATTN_F32 / F16 / BF16 value, or -1 for int32
 hipError_t launch_add(const void* a, const void* b, void* out, int64_t n, int dtype, hipStream_t stream);
 
+// second output of PagedAttentionExtension: aggregated attention probabilities per key position
+struct ScoresParams {
+    const void* q;
+    const uint8_t* key_cache;
+    const int32_t* past_lens;
+    const int32_t* subsequence_begins;
+    const int32_t* block_indices;
+    const int32_t* block_indices_begins;
+    const int32_t* score_window;  // [num_seqs] or null: every new token of a sequence is aggregated
+    float* scores;
+    int64_t scores_capacity;      // floats
+    float* lse;                   // [num_tokens, num_heads_q] log2-domain log-sum-exp (workspace)
+    int q_dtype;
+    int cache_dtype;
+    int num_heads_q;
+    int num_heads_kv;
+    int head_dim;
+    int block_size;
+    int num_blocks;
+    int num_tokens;
+    int num_seqs;
+    int max_context_len;          // bound on past + new tokens of any sequence (sizes the grid)
+    int sliding_window;
+    float scale;                  // already resolved (> 0)
+};
+hipError_t launch_paged_scores(const ScoresParams& p, hipStream_t stream);
+
 // Schedule option by name (see paged_decode.hip); value < 0 restores the default.  false: no such option.
 bool set_option(const char* name, int value);
 // Address and size of the current device's copy of the static scratch array (resolved once per device).

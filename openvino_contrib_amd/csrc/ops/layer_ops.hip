@@ -50,7 +50,10 @@ __device__ __forceinline__ Float8 load8(const void* base, int64_t idx, int dtype
     return r;
 }
 
+// rounds to nearest even with the hardware's packed conversions
 __device__ __forceinline__ void store8(void* base, int64_t idx, int dtype, const Float8& r) {
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     if (dtype == HIPATTN_F32) {
         float4_t a, b;
 #pragma unroll
@@ -64,15 +67,11 @@ __device__ __forceinline__ void store8(void* base, int64_t idx, int dtype, const
         uint4_t raw;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            uint32_t lo, hi;
-            if (dtype == HIPATTN_F16) {
-                lo = float_to_f16_bits(r.v[2 * i]);
-                hi = float_to_f16_bits(r.v[2 * i + 1]);
-            } else {
-                lo = float_to_bf16_bits(r.v[2 * i]);
-                hi = float_to_bf16_bits(r.v[2 * i + 1]);
-            }
-            raw[i] = lo | (hi << 16);
+            const float2_t pair = {r.v[2 * i], r.v[2 * i + 1]};
+            if (dtype == HIPATTN_F16)
+                raw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, half2_t));
+            else
+                raw[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
         }
         *(uint4_t*)((uint16_t*)base + idx) = raw;
     }
@@ -183,54 +182,55 @@ struct RopeParams {
     int rot_items;       // of which rotate (the rest copy)
 };
 
-// One lane takes both halves of a rotation (eight elements i.. and eight elements i + half..,
-// or eight adjacent elements = four pairs), so that out may alias x.
+constexpr int kRopeMaxTable = 512;  // floats per table row the vector kernel stages (rotary_ndims up to 512)
+
+// One workgroup per token: its cos / sin rows go to LDS once, as floats, and every (head, piece)
+// of the token reads them from there.  One lane takes both halves of a rotation (eight elements
+// i.. and eight elements i + half.., or eight adjacent elements = four pairs), so out may alias x.
 __global__ __launch_bounds__(256) void rope_vec_kernel(RopeParams p) {
-    const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t heads_total = p.d.num_tokens * p.d.num_heads;
-    const int64_t th = item / p.items_per_head;
-    const int it = (int)(item - th * p.items_per_head);
-    if (th >= heads_total) return;
-    const int64_t t = th / p.d.num_heads;
-    const int h = (int)(th - t * p.d.num_heads);
-    const int64_t xb = t * p.d.x_token_stride + (int64_t)h * p.d.x_head_stride;
-    const int64_t ob = t * p.d.out_token_stride + (int64_t)h * p.d.out_head_stride;
-    if (it >= p.rot_items) {  // pass-through tail of the head
-        const int i = p.rotary + (it - p.rot_items) * 8;
-        store8(p.out, ob + i, p.d.dtype, load8(p.x, xb + i, p.d.dtype));
-        return;
-    }
+    __shared__ float cs[2][kRopeMaxTable];
+    const int64_t t = blockIdx.x;
     const int64_t pos = p.positions ? (int64_t)p.positions[t] : t;
     const int64_t tb = pos * p.d.table_row_stride;
-    if (p.d.interleaved) {
-        const int i = it * 8;  // elements i..i+7 = pairs i/2..i/2+3
-        const Float8 v = load8(p.x, xb + i, p.d.dtype);
-        float c[4], s[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            c[k] = load_scalar(p.cos, tb + i / 2 + k, p.d.table_dtype);
-            s[k] = load_scalar(p.sin, tb + i / 2 + k, p.d.table_dtype);
+    const int width = p.d.interleaved ? p.half : p.rotary;
+    for (int i = threadIdx.x; i < 2 * width; i += blockDim.x) {
+        const int which = i >= width, k = i - which * width;
+        cs[which][k] = load_scalar(which ? p.sin : p.cos, tb + k, p.d.table_dtype);
+    }
+    __syncthreads();
+    const int per_token = p.d.num_heads * p.items_per_head;
+    for (int item = threadIdx.x; item < per_token; item += blockDim.x) {
+        const int h = item / p.items_per_head;
+        const int it = item - h * p.items_per_head;
+        const int64_t xb = t * p.d.x_token_stride + (int64_t)h * p.d.x_head_stride;
+        const int64_t ob = t * p.d.out_token_stride + (int64_t)h * p.d.out_head_stride;
+        if (it >= p.rot_items) {  // pass-through tail of the head
+            const int i = p.rotary + (it - p.rot_items) * 8;
+            store8(p.out, ob + i, p.d.dtype, load8(p.x, xb + i, p.d.dtype));
+            continue;
         }
-        Float8 o;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            o.v[2 * k] = v.v[2 * k] * c[k] - v.v[2 * k + 1] * s[k];
-            o.v[2 * k + 1] = v.v[2 * k + 1] * c[k] + v.v[2 * k] * s[k];
-        }
-        store8(p.out, ob + i, p.d.dtype, o);
-    } else {
         const int i = it * 8;
-        const Float8 lo = load8(p.x, xb + i, p.d.dtype), hi = load8(p.x, xb + i + p.half, p.d.dtype);
-        const Float8 cl = load8(p.cos, tb + i, p.d.table_dtype), ch = load8(p.cos, tb + i + p.half, p.d.table_dtype);
-        const Float8 sl = load8(p.sin, tb + i, p.d.table_dtype), sh = load8(p.sin, tb + i + p.half, p.d.table_dtype);
-        Float8 ol, oh;
+        if (p.d.interleaved) {  // elements i..i+7 = pairs i/2..i/2+3
+            const Float8 v = load8(p.x, xb + i, p.d.dtype);
+            Float8 o;
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
-            ol.v[k] = lo.v[k] * cl.v[k] - hi.v[k] * sl.v[k];
-            oh.v[k] = hi.v[k] * ch.v[k] + lo.v[k] * sh.v[k];
+            for (int k = 0; k < 4; k++) {
+                const float c = cs[0][i / 2 + k], s = cs[1][i / 2 + k];
+                o.v[2 * k] = v.v[2 * k] * c - v.v[2 * k + 1] * s;
+                o.v[2 * k + 1] = v.v[2 * k + 1] * c + v.v[2 * k] * s;
+            }
+            store8(p.out, ob + i, p.d.dtype, o);
+        } else {
+            const Float8 lo = load8(p.x, xb + i, p.d.dtype), hi = load8(p.x, xb + i + p.half, p.d.dtype);
+            Float8 ol, oh;
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                ol.v[k] = lo.v[k] * cs[0][i + k] - hi.v[k] * cs[1][i + k];
+                oh.v[k] = hi.v[k] * cs[0][i + p.half + k] + lo.v[k] * cs[1][i + p.half + k];
+            }
+            store8(p.out, ob + i, p.d.dtype, ol);
+            store8(p.out, ob + i + p.half, p.d.dtype, oh);
         }
-        store8(p.out, ob + i, p.d.dtype, ol);
-        store8(p.out, ob + i + p.half, p.d.dtype, oh);
     }
 }
 
@@ -324,7 +324,6 @@ __global__ __launch_bounds__(256) void concat_kernel(ConcatParams p) {
 // ------------------------------------------------------------------------------ host side
 static bool aligned(const void* ptr, size_t a) { return ((uintptr_t)ptr % a) == 0; }
 static bool float_dtype(int d) { return d == HIPATTN_F32 || d == HIPATTN_F16 || d == HIPATTN_BF16; }
-static size_t vec_bytes(int dtype) { return dtype == HIPATTN_F32 ? 32 : 16; }  // eight elements; loads are 16-byte
 
 static hipattn_status launched(const char* what) {
     const hipError_t e = hipGetLastError();
@@ -342,12 +341,12 @@ hipattn_status rms_norm(const void* x, const void* gamma, void* out, int64_t row
     if (!(eps >= 0.f)) return fail(HIPATTN_INVALID_ARGUMENT, "rms_norm: eps must be >= 0");
     if (rows == 0) return HIPATTN_OK;
     if (!x || !out) return fail(HIPATTN_INVALID_ARGUMENT, "rms_norm: null pointer");
-    if ((rows + 3) / 4 > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "rms_norm: too many rows");
+    if (rows > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "rms_norm: too many rows");
     RmsParams p{x, gamma, out, rows, hidden, eps, x_dtype, gamma_dtype, out_dtype};
     const bool vec = hidden % 8 == 0 && aligned(x, 16) && aligned(out, 16) && (!gamma || aligned(gamma, 16));
     if (!vec) {
         hipLaunchKernelGGL(rms_norm_scalar_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
-    } else if (rows >= 2048 && hidden <= 4096) {
+    } else if (rows >= 2048 && hidden <= 1024) {
         // enough rows to fill the device with one wavefront each
         hipLaunchKernelGGL(rms_norm_vec_kernel<1>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
     } else {
@@ -380,25 +379,21 @@ hipattn_status rope(const hipops_rope_desc* d, const void* x, const void* cos, c
     p.d = *d;
     p.x = x, p.cos = cos, p.sin = sin, p.positions = positions, p.out = out;
     p.rotary = rotary, p.half = rotary / 2;
-    const size_t va = 16;
-    const bool x_vec = d->head_size % 8 == 0 && rotary % 8 == 0 && d->x_token_stride % 8 == 0 && d->x_head_stride % 8 == 0 &&
-                       d->out_token_stride % 8 == 0 && d->out_head_stride % 8 == 0 && aligned(x, va) && aligned(out, va);
-    const bool vec = x_vec && (d->interleaved ? true
-                                              : (p.half % 8 == 0 && d->table_row_stride % 8 == 0 && aligned(cos, va) && aligned(sin, va)));
-    const int64_t heads_total = d->num_tokens * d->num_heads;
-    int64_t items;
+    const bool vec = d->head_size % 8 == 0 && rotary % 8 == 0 && (d->interleaved || p.half % 8 == 0) && rotary <= kRopeMaxTable &&
+                     d->x_token_stride % 8 == 0 && d->x_head_stride % 8 == 0 && d->out_token_stride % 8 == 0 &&
+                     d->out_head_stride % 8 == 0 && aligned(x, 16) && aligned(out, 16);
     if (vec) {
+        if (d->num_tokens > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "rope: too many tokens for one launch");
         p.rot_items = d->interleaved ? rotary / 8 : p.half / 8;
         p.items_per_head = p.rot_items + (d->head_size - rotary) / 8;
-        items = heads_total * p.items_per_head;
+        const int per_token = d->num_heads * p.items_per_head;
+        const int threads = std::min(256, (per_token + kWave - 1) / kWave * kWave);
+        hipLaunchKernelGGL(rope_vec_kernel, dim3((unsigned)d->num_tokens), dim3(threads), 0, stream, p);
     } else {
-        items = heads_total * (p.half + (d->head_size - rotary));
-    }
-    if (blocks_for(items) > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "rope: too many elements for one launch");
-    if (vec)
-        hipLaunchKernelGGL(rope_vec_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
-    else
+        const int64_t items = d->num_tokens * d->num_heads * (int64_t)(p.half + (d->head_size - rotary));
+        if (blocks_for(items) > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "rope: too many elements for one launch");
         hipLaunchKernelGGL(rope_scalar_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
+    }
     return launched("rope");
 }
 

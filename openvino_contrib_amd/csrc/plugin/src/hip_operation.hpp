@@ -117,6 +117,9 @@ public:
     // When such an input was bound as a host tensor the request copies it back after the operator,
     // so the caller's memory holds the update; device-resident tensors need nothing.
     virtual std::vector<size_t> UpdatedInputs() const { return {}; }
+    // Told once, while the model is compiled, that nothing consumes this output: an operator may then
+    // skip producing it (the scores of PagedAttentionExtension).
+    virtual void MarkOutputUnused(size_t /*output*/) {}
     // Host bytes the operator itself provides for an output (Constant); nullptr otherwise.
     virtual const void* HostData(size_t /*output*/) const { return nullptr; }
 

@@ -9,6 +9,7 @@
 // src/ops/multiply.cpp:43); PagedAttentionOp has no counterpart there; ReadValueOp / AssignOp follow
 // src/ops/read_value.cpp:31-72 and src/ops/assign.cpp:29-56.  As in the reference, a constructor
 // that throws is how an unsupported node is reported (src/cuda_plugin.cpp:171-188).
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 
@@ -227,10 +228,10 @@ private:
     bool causal_ = false;
 };
 
-// Input order of the OpenVINO operator.  Everything from score_aggregation_window on belongs to
-// features this plugin does not implement (score output for cache eviction, cache rotation,
-// sparse attention, sinks); such inputs are accepted when they are empty, as exported models carry
-// them, and refused when they hold data.
+// Input order of the OpenVINO operator.  score_aggregation_window belongs to the scores output
+// (built: the aggregated probabilities a cache-eviction policy reads); everything behind it belongs
+// to features this plugin does not implement (cache rotation, sparse attention, sinks): such inputs
+// are accepted when they are empty, as exported models carry them, and refused when they hold data.
 enum PaInput {
     kQuery = 0, kKey, kValue, kKeyCache, kValueCache, kPastLens, kSubsequenceBegins, kBlockIndices,
     kBlockIndicesBegins, kScale, kSlidingWindow, kAlibiSlopes, kMaxContextLen, kPaRequiredInputs,
@@ -253,8 +254,10 @@ public:
             HIP_PLUGIN_THROW(who + std::to_string(num_inputs_) + " inputs: more than this plugin knows of");
         if (num_outputs_ < 1 || num_outputs_ > 2) HIP_PLUGIN_THROW(who + std::to_string(num_outputs_) + " outputs");
         for (size_t i = kPaRequiredInputs; i < num_inputs_; i++)
-            if (statically_non_empty(node.get_input_partial_shape(i)))
+            if (i != kScoreAggregationWindow && statically_non_empty(node.get_input_partial_shape(i)))
                 HIP_PLUGIN_THROW(who + kPaOptionalNames[i - kPaRequiredInputs] + " holds data: the feature is not supported");
+        if (num_inputs_ > kScoreAggregationWindow && node.get_input_element_type(kScoreAggregationWindow) != ov::element::i32)
+            HIP_PLUGIN_THROW(who + "score_aggregation_window must be i32");
         q_type_ = node.get_input_element_type(kQuery);
         kv_type_ = node.get_input_element_type(kKey);
         cache_type_ = node.get_input_element_type(kKeyCache);
@@ -272,9 +275,26 @@ public:
         out1_type_ = num_outputs_ > 1 ? node.get_output_element_type(1) : ov::element::dynamic;
     }
 
+    void MarkOutputUnused(size_t output) override {
+        if (output == 1) scores_wanted_ = false;
+    }
+
+    // scores: one value per cache position of every sequence, past and new; the output's extent is
+    // data (the sum of past_lens), so those must have come from host memory
     std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
         std::vector<ov::Shape> shapes{in.at(kQuery).shape};
-        if (num_outputs_ > 1) shapes.push_back(ov::Shape{0});  // scores: nothing is aggregated
+        if (num_outputs_ > 1) {
+            size_t total = 0;
+            if (scores_wanted_ && in[kQuery].shape.at(0) > 0) {
+                const TensorView& pl = in[kPastLens];
+                HIP_PLUGIN_ASSERT(pl.host != nullptr, "past_lens must be set from host memory when the scores output is used (it sizes that output)");
+                HIP_PLUGIN_ASSERT(out1_type_ == ov::element::f32, "the scores output must be f32, not " + out1_type_.get_type_name());
+                const int32_t* lens = (const int32_t*)pl.host;
+                for (size_t s = 0; s < ov::shape_size(pl.shape); s++) total += (size_t)std::max(lens[s], 0);
+                total += in[kQuery].shape[0];
+            }
+            shapes.push_back(ov::Shape{total});
+        }
         return shapes;
     }
 
@@ -285,7 +305,11 @@ public:
         size_t bytes = 0;
         HIP_PLUGIN_CHECK(hipattn_paged_attention_workspace_size(&d, &bytes));
         WorkbufferRequest r;
-        if (bytes) r.mutable_sizes.push_back(bytes);
+        r.mutable_sizes.push_back(bytes);
+        if (scores_wanted_ && num_outputs_ > 1) {
+            HIP_PLUGIN_CHECK(hipattn_paged_attention_scores_workspace_size(&d, &bytes));
+            r.mutable_sizes.push_back(bytes);
+        }
         return r;
     }
 
@@ -298,6 +322,20 @@ public:
             (const int32_t*)in[kPastLens].device, (const int32_t*)in[kSubsequenceBegins].device,
             (const int32_t*)in[kBlockIndices].device, (const int32_t*)in[kBlockIndicesBegins].device, out[0].device, ws,
             ws_bytes, context.stream.get()));
+        if (scores_wanted_ && out.size() > 1 && ov::shape_size(out[1].shape) > 0) {
+            const int32_t* window = nullptr;
+            if (num_inputs_ > kScoreAggregationWindow && ov::shape_size(in[kScoreAggregationWindow].shape) > 0) {
+                HIP_PLUGIN_ASSERT(ov::shape_size(in[kScoreAggregationWindow].shape) == (size_t)d.num_seqs,
+                                  "score_aggregation_window must hold one value per sequence");
+                window = (const int32_t*)in[kScoreAggregationWindow].device;
+            }
+            HIP_PLUGIN_ASSERT(wb.mutable_buffers.size() > 1, "no scratch for the scores");
+            HIP_PLUGIN_CHECK(hipattn_paged_attention_scores(
+                &d, in[kQuery].device, in[kKeyCache].device, (const int32_t*)in[kPastLens].device,
+                (const int32_t*)in[kSubsequenceBegins].device, (const int32_t*)in[kBlockIndices].device,
+                (const int32_t*)in[kBlockIndicesBegins].device, window, (float*)out[1].device,
+                (int64_t)ov::shape_size(out[1].shape), wb.mutable_buffers[1], wb.mutable_sizes[1], context.stream.get()));
+        }
     }
 
 private:
@@ -319,7 +357,7 @@ private:
         HIP_PLUGIN_ASSERT(q.size() == 2, "query must be [tokens, heads * head_size], got " + shape_str(q));
         HIP_PLUGIN_ASSERT(kc.size() == 4 && in[kValueCache].shape == kc, "key/value cache shapes " + shape_str(kc));
         for (size_t i = kPaRequiredInputs; i < num_inputs_; i++)
-            HIP_PLUGIN_ASSERT(ov::shape_size(in[i].shape) == 0,
+            HIP_PLUGIN_ASSERT(i == kScoreAggregationWindow || ov::shape_size(in[i].shape) == 0,
                               std::string(kPaOptionalNames[i - kPaRequiredInputs]) + " holds data: the feature is not supported");
         hipattn_pa_desc d{};
         to_hipattn_dtype(q_type_, d.q_dtype);
@@ -352,6 +390,7 @@ private:
     }
     ov::element::Type q_type_, kv_type_, cache_type_, out1_type_;
     size_t num_inputs_ = 0, num_outputs_ = 1;
+    bool scores_wanted_ = true;  // until the compiled model says nothing consumes output 1
 };
 
 // ReadValue: the variable's device buffer into the output; after a reset, the init_value input (or

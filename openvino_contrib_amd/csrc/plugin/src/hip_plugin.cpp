@@ -461,6 +461,16 @@ CompiledModel::CompiledModel(const std::shared_ptr<const ov::Model>& model, cons
         auto op = OperationRegistry::getInstance().createOperation(ctx, node, std::move(in), std::move(out));
         exec_sequence_.push_back({node, op});
     }
+    // outputs nothing consumes (neither an operator nor a Result) need not be produced
+    std::set<std::pair<const ov::Node*, size_t>> consumed;
+    for (const auto& node : ordered)
+        for (size_t i = 0; i < node->get_input_size(); i++) {
+            const auto src = node->input_value(i);
+            consumed.insert({src.get_node(), src.get_index()});
+        }
+    for (const auto& step : exec_sequence_)
+        for (size_t o = 0; o < step.node->get_output_size(); o++)
+            if (!consumed.count({step.node.get(), o})) step.op->MarkOutputUnused(o);
 }
 
 std::shared_ptr<ov::ISyncInferRequest> CompiledModel::create_sync_infer_request() const {

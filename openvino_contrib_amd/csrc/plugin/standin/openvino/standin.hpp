@@ -586,6 +586,11 @@ public:
         set_output_type(0, get_input_element_type(0), get_input_partial_shape(0));
         set_output_type(1, get_input_element_type(0), PartialShape{Dimension::dynamic()});
     }
+    // the operator lets a transformation pin the type of an output
+    void set_out_type(int index, const element::Type& type) { set_output_type((size_t)index, type, get_output_partial_shape(index)); }
+    std::map<std::string, std::string> standin_attributes() const override {
+        return {{"out0_type", get_output_element_type(0).get_type_name()}, {"out1_type", get_output_element_type(1).get_type_name()}};
+    }
 };
 
 namespace v6 {
@@ -1228,7 +1233,11 @@ public:
             } else if (type == "ScaledDotProductAttention") {
                 n = std::make_shared<op::v13::ScaledDotProductAttention>(inputs, attrs.at("causal") == "true");
             } else if (type == "PagedAttentionExtension") {
-                n = std::make_shared<op::PagedAttentionExtension>(inputs);
+                auto pa = std::make_shared<op::PagedAttentionExtension>(inputs);
+                for (int o = 0; o < 2; o++)
+                    if (attrs.count("out" + std::to_string(o) + "_type"))
+                        pa->set_out_type(o, element::type_from_name(attrs["out" + std::to_string(o) + "_type"]));
+                n = pa;
             } else if (type == "ReadValue") {
                 n = inputs.empty() ? std::make_shared<op::v6::ReadValue>(variable())
                                    : std::make_shared<op::v6::ReadValue>(inputs.at(0), variable());

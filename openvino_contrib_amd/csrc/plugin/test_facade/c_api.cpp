@@ -264,7 +264,10 @@ API int hip_model_create_paged_attention(int q_dtype, int kv_dtype, int cache_dt
         auto pa = std::make_shared<ov::op::PagedAttentionExtension>(in);
         pa->set_friendly_name("paged_attention");
         ov::ResultVector results{result("out", pa->output(0))};
-        if (with_scores_result) results.push_back(result("scores", pa->output(1)));
+        if (with_scores_result) {
+            pa->set_out_type(1, ov::element::f32);
+            results.push_back(result("scores", pa->output(1)));
+        }
         *model = new hip_model_s{std::make_shared<ov::Model>(results, params, "PagedAttention")};
     });
 }

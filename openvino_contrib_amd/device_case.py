@@ -102,6 +102,25 @@ class PagedDeviceCase:
             ws.free()
         return storage_to_f32(res, self.out_dtype), path
 
+    def scores(self, score_window=None, scale=0.0, max_context_len=None, stream=None):
+        """The operator's second output for the cache as it stands (call run() first): f32
+        [sum(past_lens) + tokens]."""
+        hip, case = self.hip, self.case
+        desc = pa_desc(hip, case, self.out_dtype, 0, 0, scale, max_context_len)
+        total = int(np.sum(case["past_lens"])) + case["T"]
+        out = hip.DeviceBuffer((total + 16) * 4)
+        out.fill(0xEE)
+        sw = None if score_window is None else hip.DeviceBuffer.from_numpy(np.asarray(score_window, np.int32))
+        hip.paged_attention_scores(desc, self.q, self.key_cache, self.past_lens, self.subsequence_begins,
+                                   self.block_indices, self.block_indices_begins, sw, out, total, stream)
+        res = out.download(np.float32, (total + 16,), stream)
+        out.free()
+        if sw is not None:
+            sw.free()
+        canary = np.frombuffer(b"\xee" * 4, np.float32)[0]
+        assert np.all(res[total:].view(np.uint32) == canary.view(np.uint32)), "scores written beyond the capacity"
+        return res[:total]
+
     def caches(self):
         kc = self.key_cache.download(np.uint8, self.case["key_cache"].shape)
         vc = self.value_cache.download(np.uint8, self.case["value_cache"].shape)

@@ -37,6 +37,12 @@
  *                              the reference tree and OpenVINO is not installed.  Pinned
  *                              by reduction to oracle_sdpa_f32 after a gather through the
  *                              block table, and by block-permutation invariance.
+ *   oracle_paged_attention_scores   the operator's second output: attention probability per
+ *                              cache position, summed over heads and the aggregated query
+ *                              tokens.  PARITY UNPINNED against OpenVINO.  Pinned by a numpy
+ *                              restatement over a dense gather, by sum = heads x aggregated
+ *                              tokens, and by scores-weighted values = attention output for a
+ *                              one-head, one-token sequence.
  *   oracle_quant_u8_row /      asymmetric per-token, per-head u8 rows
  *   oracle_dequant_u8_row      [scale f32][zero-point f32][D bytes].  PARITY UNPINNED
  *                              against OpenVINO (rounding mode and row layout are restated
@@ -470,5 +476,71 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
         free(vbuf);
         free(scores);
     }
+    return 0;
+}
+
+/* Second output of PagedAttentionExtension ("scores"): for every cache position of every
+ * sequence, the probability it received, summed over the query heads and over the last
+ * score_window[s] query tokens of the sequence (all of them when score_window is NULL).
+ * Reads the cache as it stands (call after the write).  scores must hold
+ * sum(past_lens[s] + new_tokens(s)) floats; sequence s starts where s-1 ends.  fp64 throughout.
+ * PARITY UNPINNED against OpenVINO (which tokens and heads are aggregated is restated from its
+ * operator documentation).  Pinned by: a numpy restatement over a dense gather of the keys, the sum
+ * of a sequence's scores (= heads x aggregated tokens), and agreement of the probabilities with
+ * the attention output (scores-weighted values of one head, one token). */
+ORACLE_API int oracle_paged_attention_scores(const float* q, const uint8_t* key_cache, int cache_dtype,
+                                             const int32_t* past_lens, const int32_t* subsequence_begins,
+                                             const int32_t* block_indices, const int32_t* block_indices_begins,
+                                             const int32_t* score_window, int S, int Hq, int Hkv, int D, int block_size,
+                                             float scale, int sliding_window, float* scores) {
+    if (S < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || block_size <= 0) return 1;
+    if (scale <= 0.0f) scale = 1.0f / sqrtf((float)D);
+    const int G = Hq / Hkv;
+    int64_t* starts = (int64_t*)malloc(sizeof(int64_t) * (size_t)(S + 1));
+    starts[0] = 0;
+    for (int s = 0; s < S; s++) starts[s + 1] = starts[s] + past_lens[s] + (subsequence_begins[s + 1] - subsequence_begins[s]);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int s = 0; s < S; s++) {
+        const int t0 = subsequence_begins[s], qlen = subsequence_begins[s + 1] - t0;
+        const int ctx_full = past_lens[s] + qlen;
+        float* out = scores + starts[s];
+        for (int j = 0; j < ctx_full; j++) out[j] = 0.0f;
+        int ctx = ctx_full;
+        const int table_tokens = (block_indices_begins[s + 1] - block_indices_begins[s]) * block_size;
+        if (ctx > table_tokens) ctx = table_tokens;
+        int w = qlen;
+        if (score_window) w = score_window[s] < 0 ? 0 : (score_window[s] < qlen ? score_window[s] : qlen);
+        if (ctx <= 0 || w <= 0) continue;
+        double* acc = (double*)calloc((size_t)ctx, sizeof(double));
+        double* sc = (double*)malloc(sizeof(double) * (size_t)ctx);
+        float* kbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
+        const int32_t* blocks = block_indices + block_indices_begins[s];
+        for (int h = 0; h < Hkv; h++) {
+            oracle_gather_cache_rows(key_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, kbuf);
+            for (int i = qlen - w; i < qlen; i++) {
+                const int p = past_lens[s] + i;
+                int j0 = 0, j1 = p + 1 < ctx ? p + 1 : ctx;
+                if (sliding_window > 0 && p - sliding_window + 1 > 0) j0 = p - sliding_window + 1;
+                if (j0 >= j1) continue;
+                for (int g = 0; g < G; g++) {
+                    const float* qr = q + ((int64_t)(t0 + i) * Hq + (h * G + g)) * D;
+                    double m = -INFINITY, l = 0.0;
+                    for (int j = j0; j < j1; j++) {
+                        double d = 0.0;
+                        for (int e = 0; e < D; e++) d += (double)qr[e] * (double)kbuf[(int64_t)j * D + e];
+                        sc[j] = d * (double)scale;
+                        if (sc[j] > m) m = sc[j];
+                    }
+                    for (int j = j0; j < j1; j++) l += exp(sc[j] - m);
+                    for (int j = j0; j < j1; j++) acc[j] += exp(sc[j] - m) / l;
+                }
+            }
+        }
+        for (int j = 0; j < ctx; j++) out[j] = (float)acc[j];
+        free(acc);
+        free(sc);
+        free(kbuf);
+    }
+    free(starts);
     return 0;
 }

@@ -62,6 +62,8 @@ def lib():
         L.oracle_paged_attention.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                              f32, i32, i32, vp]
         L.oracle_paged_attention.restype = i32
+        L.oracle_paged_attention_scores.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp]
+        L.oracle_paged_attention_scores.restype = i32
         L.oracle_rms_norm_f32.argtypes = [vp, vp, vp, i64, i64, f32]
         L.oracle_rms_norm_f32.restype = None
         L.oracle_rope_f32.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i64]
@@ -229,6 +231,24 @@ def paged_attention(q, k_new, v_new, key_cache, value_cache, cache_dtype, past_l
                                       _p(out))
     if rc:
         raise ValueError("oracle_paged_attention: bad arguments")
+    return out
+
+
+def paged_attention_scores(q, key_cache, cache_dtype, past_lens, subsequence_begins, block_indices, block_indices_begins,
+                           Hq, Hkv, D, block_size, score_window=None, scale=0.0, sliding_window=0):
+    """The operator's second output from the cache as it stands (after the step's write): f32
+    [sum(past_lens) + tokens], sequence after sequence."""
+    q = _c(q, np.float32)
+    pl, sb = _c(past_lens, np.int32), _c(subsequence_begins, np.int32)
+    bi, bb = _c(block_indices, np.int32), _c(block_indices_begins, np.int32)
+    sw = None if score_window is None else _c(score_window, np.int32)
+    total = int(pl.sum()) + int(sb[-1] - sb[0])
+    out = np.zeros(total, np.float32)
+    rc = lib().oracle_paged_attention_scores(_p(q), _p(key_cache), cache_dtype, _p(pl), _p(sb), _p(bi), _p(bb),
+                                             _p(sw) if sw is not None else None, len(pl), Hq, Hkv, D, block_size,
+                                             float(scale), int(sliding_window), _p(out))
+    if rc:
+        raise ValueError("oracle_paged_attention_scores: bad arguments")
     return out
 
 

@@ -723,3 +723,51 @@ def test_mfma_yardstick_reports_a_plausible_rate(hip):
     assert 1.0 < ghz.value < 2.6
     assert yard.mfma_yardstick(0, 0, ctypes.byref(tf), ctypes.byref(ghz)) != 0
 
+
+
+# ---- the operator's second output ("scores") ----------------------------------------------------
+SCORE_BATCHES = [
+    ([(30, 5), (0, 9), (65, 1), (12, 4)], None),
+    ([(30, 5), (0, 9), (65, 1), (12, 4)], [1, 3, 0, 2]),
+    ([(700, 1), (1500, 1), (31, 1)], None),
+    ([(100, 130), (0, 1)], [64, 5]),
+]
+
+
+@pytest.mark.parametrize("cache_dtype,q_dtype,Hq,Hkv,D,bs", [(W.F16, W.F16, 8, 2, 128, 32), (W.U8, W.BF16, 4, 4, 128, 32),
+                                                             (W.F32, W.F32, 4, 2, 64, 16), (W.BF16, W.BF16, 6, 3, 96, 8)])
+@pytest.mark.parametrize("batch", range(len(SCORE_BATCHES)))
+@pytest.mark.parametrize("window", [0, 40])
+def test_paged_attention_scores(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, bs, batch, window):
+    seqs, score_window = SCORE_BATCHES[batch]
+    print("[scores]", cache_dtype, q_dtype, Hq, Hkv, D, bs, seqs, score_window, window, flush=True)
+    case = W.make_paged_case(300 + batch, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    dev = H.PagedDeviceCase(hip, case)
+    dev.run()  # writes the new tokens' keys
+    got = dev.scores(score_window)
+    kc, _ = dev.caches()
+    ref = oracle.paged_attention_scores(case["q"], kc, cache_dtype, case["past_lens"], case["subsequence_begins"],
+                                        case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
+                                        score_window=score_window, sliding_window=window)
+    # a sum of up to heads x tokens probabilities, each from an fp32 dot product and exp2
+    bound = 2e-5 * max(1.0, float(ref.max()))
+    assert H.max_abs(got, ref) <= bound, (H.max_abs(got, ref), bound)
+    dev.free()
+
+
+def test_paged_attention_scores_arguments(hip):
+    case = W.make_paged_case(310, [(10, 2)], 4, 2, 64, 16, W.F16, W.F16, W.F16)
+    dev = H.PagedDeviceCase(hip, case)
+    desc = H.pa_desc(hip, case)
+    out = hip.DeviceBuffer(64)
+    L = hip.lib()
+    import ctypes
+    args = (dev.q.ptr, dev.key_cache.ptr, dev.past_lens.ptr, dev.subsequence_begins.ptr, dev.block_indices.ptr,
+            dev.block_indices_begins.ptr, None, out.ptr, 12)
+    assert L.hipattn_paged_attention_scores(ctypes.byref(desc), *args, None, 0, None) == hip.WORKSPACE_TOO_SMALL
+    ws = hip.DeviceBuffer(2 * 4 * 4)
+    assert L.hipattn_paged_attention_scores(ctypes.byref(desc), *args, ws.ptr, 8, None) == hip.WORKSPACE_TOO_SMALL
+    assert L.hipattn_paged_attention_scores(ctypes.byref(desc), *args, ws.ptr, 32, None) == hip.OK
+    assert L.hipattn_paged_attention_scores(ctypes.byref(desc), *(args[:-1] + (-1,)), ws.ptr, 32, None) == hip.INVALID_ARGUMENT
+    hip.check(L.hipattn_stream_synchronize(None))
+    dev.free()

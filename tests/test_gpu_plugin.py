@@ -113,9 +113,14 @@ def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_
     req.wait()
     out, _ = req.output(0)
     scores, _ = req.output(1)
-    assert scores.shape == (0,)
     out = H.storage_to_f32(out, q_dtype)
     ref, okc, ovc = H.oracle_paged(oracle, case)
+    # the scores Result is connected, so the second output is produced: every new token aggregated
+    ref_scores = oracle.paged_attention_scores(case["q"], okc, cache_dtype, case["past_lens"], case["subsequence_begins"],
+                                               case["block_indices"], case["block_indices_begins"], 16, 4, 128, 32,
+                                               sliding_window=window)
+    assert scores.dtype == np.float32 and scores.shape == ref_scores.shape
+    assert H.max_abs(scores, ref_scores) <= 2e-5 * max(1.0, float(ref_scores.max()))
     tol = 1e-2 if (cache_dtype == W.U8 or q_dtype == W.BF16) else 2e-3
     assert H.max_abs(out, ref) <= tol
     # the operator updated the device-resident caches in place, bit for bit as the oracle does
@@ -126,6 +131,51 @@ def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_
     assert prof[0][2] > 0
     kc.free()
     vc.free()
+
+
+def test_paged_attention_scores_over_an_aggregation_window(hip, oracle):
+    """score_aggregation_window holds one value per sequence: only that many of a sequence's last
+    query tokens are aggregated.  Without a consumer of output 1 nothing is computed for it."""
+    print("[plugin] paged attention scores with a window", flush=True)
+    seqs = MIXED_BATCH
+    window = [4, 1, 0, 300, 1, 1]
+    case = W.make_paged_case(97, seqs, 16, 4, 128, 32, W.F16, W.F16, W.F16)
+    plugin = P.Plugin()
+    for with_scores in (True, False):
+        compiled = plugin.compile_model(P.Model.paged_attention(W.F16, W.F16, W.F16, 16, 4, 128, 32, extra_inputs=1,
+                                                                extra_len=len(seqs), scores_result=with_scores))
+        kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
+        vc = hip.DeviceBuffer.from_numpy(case["value_cache"])
+        req = compiled.create_infer_request()
+        elem_shape = list(case["key_cache"].shape[:3]) + [128]
+        for i, (a, dt) in enumerate([(case["q_store"], W.F16), (case["k_new_store"], W.F16), (case["v_new_store"], W.F16)]):
+            req.set_input(i, a, dt)
+        req.set_device_input(3, kc.ptr, W.F16, elem_shape)
+        req.set_device_input(4, vc.ptr, W.F16, elem_shape)
+        for i, n in enumerate(("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")):
+            req.set_input(5 + i, case[n], P.I32)
+        req.set_input(9, np.zeros((0,), np.float32), W.F32)
+        req.set_input(10, np.array([0], np.int32), P.I32)
+        req.set_input(11, np.zeros((0,), np.float32), W.F32)
+        req.set_input(12, np.array([case["max_context_len"]], np.int32), P.I32)
+        req.set_input(13, np.array(window, np.int32), P.I32)
+        req.infer()
+        out, _ = req.output(0)
+        ref, okc, _ = H.oracle_paged(oracle, case)
+        assert H.max_abs(H.storage_to_f32(out, W.F16), ref) <= 2e-3
+        if with_scores:
+            scores, _ = req.output(1)
+            ref_scores = oracle.paged_attention_scores(case["q"], okc, W.F16, case["past_lens"], case["subsequence_begins"],
+                                                       case["block_indices"], case["block_indices_begins"], 16, 4, 128, 32,
+                                                       score_window=window)
+            assert scores.shape == ref_scores.shape
+            assert H.max_abs(scores, ref_scores) <= 2e-5 * max(1.0, float(ref_scores.max()))
+            begin = sum(p + n for p, n in seqs[:2])
+            assert not scores[begin:begin + sum(seqs[2])].any()  # a window of 0: nothing aggregated for that sequence
+        else:
+            assert compiled.num_outputs() == 1
+        kc.free()
+        vc.free()
 
 
 def test_profiling_must_be_enabled(hip):

@@ -321,3 +321,59 @@ def test_paged_attention_block_permutation_invariance_and_window(oracle):
                                             caseA["block_indices"], caseA["block_indices_begins"], 4, 2, 16, 8))
     np.testing.assert_allclose(np.concatenate(parts), full, atol=1e-6)
     np.testing.assert_array_equal(kcA, kcB)
+
+
+# ---- the operator's second output ("scores") ----------------------------------------------------
+def _dense_keys(oracle, case, s, h):
+    pl, bb = case["past_lens"], case["block_indices_begins"]
+    qlen = case["subsequence_begins"][s + 1] - case["subsequence_begins"][s]
+    return oracle.gather_cache_rows(case["key_cache"], case["cache_dtype"], case["block_indices"][bb[s]:bb[s + 1]],
+                                    int(pl[s] + qlen), h, case["Hkv"], case["D"], case["block_size"])
+
+
+@pytest.mark.parametrize("cache_dtype,window,score_window", [(W.F16, 0, None), (W.U8, 0, [1, 3, 0, 2]), (W.F32, 20, None),
+                                                              (W.BF16, 7, [2, 1, 1, 40])])
+def test_paged_scores_match_a_numpy_restatement(oracle, cache_dtype, window, score_window):
+    seqs = [(30, 5), (0, 9), (65, 1), (12, 4)]
+    Hq, Hkv, D, bs = 4, 2, 16, 8
+    case = W.make_paged_case(71, seqs, Hq, Hkv, D, bs, W.F32, W.F32, cache_dtype, sliding_window=window)
+    oracle.kv_cache_write(case["k_new"], case["v_new"], case["key_cache"], case["value_cache"], cache_dtype, case["past_lens"],
+                          case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], Hkv, D, bs)
+    got = oracle.paged_attention_scores(case["q"], case["key_cache"], cache_dtype, case["past_lens"], case["subsequence_begins"],
+                                        case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
+                                        score_window=score_window, sliding_window=window)
+    q = case["q"].reshape(-1, Hq, D).astype(np.float64)
+    ref, start = np.zeros_like(got, dtype=np.float64), 0
+    for s, (past, qlen) in enumerate(seqs):
+        ctx = past + qlen
+        t0 = case["subsequence_begins"][s]
+        w = qlen if score_window is None else min(qlen, score_window[s])
+        for h in range(Hq):
+            K = _dense_keys(oracle, case, s, h // (Hq // Hkv)).astype(np.float64)
+            for i in range(qlen - w, qlen):
+                p = past + i
+                j0 = max(0, p - window + 1) if window > 0 else 0
+                sc = (K[j0:p + 1] @ q[t0 + i, h]) / np.sqrt(D)
+                e = np.exp(sc - sc.max())
+                ref[start + j0:start + p + 1] += e / e.sum()
+        assert abs(got[start:start + ctx].sum() - Hq * w) < 1e-4  # every softmax sums to one
+        start += ctx
+    assert start == got.size
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+
+
+def test_paged_scores_are_the_probabilities_of_the_attention(oracle):
+    """One head, one new token: out = sum_j scores[j] * v[j], with out from the attention oracle."""
+    seqs = [(37, 1), (5, 1)]
+    case = W.make_paged_case(72, seqs, 1, 1, 32, 16, W.F32, W.F32, W.F32)
+    ref, kc, vc = None, case["key_cache"].copy(), case["value_cache"].copy()
+    out = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc, vc, W.F32, case["past_lens"],
+                                 case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], 1, 1, 32, 16)
+    sc = oracle.paged_attention_scores(case["q"], kc, W.F32, case["past_lens"], case["subsequence_begins"],
+                                       case["block_indices"], case["block_indices_begins"], 1, 1, 32, 16)
+    start = 0
+    for s, (past, qlen) in enumerate(seqs):
+        bb = case["block_indices_begins"]
+        V = oracle.gather_cache_rows(vc, W.F32, case["block_indices"][bb[s]:bb[s + 1]], past + 1, 0, 1, 32, 16)
+        np.testing.assert_allclose(sc[start:start + past + 1] @ V, out[s], rtol=1e-5, atol=1e-6)
+        start += past + 1

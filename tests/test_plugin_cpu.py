@@ -102,6 +102,8 @@ def test_paged_attention_takes_the_operators_full_signature():
                                      scores_result=True)
         names = plugin.query_model(pa)
         assert "paged_attention" in names and "scores" in names, extra
+    windowed = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=1, extra_len=16, scores_result=True)
+    assert "paged_attention" in plugin.query_model(windowed)  # score_aggregation_window may hold data
     rotated = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=4, extra_len=16)
     assert "paged_attention" not in plugin.query_model(rotated)
     unknown_inputs = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=9, extra_len=0)
