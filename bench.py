@@ -114,6 +114,50 @@ def bench_paged(hip, case, steps, warmup, name):
     return res
 
 
+def bench_paged_scores(hip, case, steps, name):
+    """The operator's second output for the same batch (every new token aggregated): two generic
+    kernels, each of which reads the whole K half of the attended cache, timed between two events."""
+    from openvino_contrib_amd import device_case as H
+    from openvino_contrib_amd import workloads as W
+    import ctypes
+    import numpy as np
+
+    dev = H.PagedDeviceCase(hip, case)
+    dev.run()
+    desc = H.pa_desc(hip, case)
+    total = int(np.sum(case["past_lens"])) + case["T"]
+    out = hip.DeviceBuffer(total * 4)
+    n = ctypes.c_size_t(0)
+    hip.check(hip.lib().hipattn_paged_attention_scores_workspace_size(ctypes.byref(desc), ctypes.byref(n)))
+    ws = hip.DeviceBuffer(n.value)
+
+    def call():
+        hip.check(hip.lib().hipattn_paged_attention_scores(
+            ctypes.byref(desc), dev.q.ptr, dev.key_cache.ptr, dev.past_lens.ptr, dev.subsequence_begins.ptr,
+            dev.block_indices.ptr, dev.block_indices_begins.ptr, None, out.ptr, total, ws.ptr, ws.nbytes, None))
+
+    steps = max(3, min(steps, 20))
+    for _ in range(2):
+        call()
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record()
+    for _ in range(steps):
+        call()
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / steps
+    k_bytes = W.paged_kv_bytes(case) // 2
+    a = (2 * k_bytes + total * 4) / (ms * 1e-3) / 1e9
+    dev.free()
+    out.free()
+    ws.free()
+    return {"workload": name, "ms_per_step": ms, "dominant_kernel_ms": ms, "steps": steps, "bytes": 2 * k_bytes + total * 4,
+            "roofline": {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
+                         "traffic": None, "kernel": "paged_lse_kernel + paged_scores_kernel",
+                         "note": "shape-generic fp32 kernels (one dot product per lane), compute-bound, not tuned; "
+                                 "the figure prices the two passes over the K rows against HBM"}}
+
+
 def bench_paged_through_plugin(hip, case, steps, warmup):
     """The same step through the plugin layer: Plugin -> CompiledModel -> InferRequest::infer ->
     PagedAttentionOp -> C ABI, every tensor device-resident (remote tensors over the buffers of the raw
@@ -526,6 +570,9 @@ def main():
             r["plugin_overhead_ms"] = r["plugin_ms_per_step"] - r["ms_per_step"]
             log("%s through InferRequest::infer: %.3f ms/step (raw C ABI, back to back: %.3f)"
                 % (w, r["plugin_ms_per_step"], r["ms_per_step"]))
+        if w == "c3" and not args.no_extra:
+            results["c3_scores"] = bench_paged_scores(hip, case, args.steps, "config3's batch: the scores output (all heads, the new token of every sequence)")
+            log("c3 scores output: %.3f ms" % results["c3_scores"]["ms_per_step"])
         if not args.no_cpu:
             # the headline gets the larger budget; every other workload a bounded sample beside its figure
             budget = 12.0 if w == args.workload else 6.0

@@ -735,7 +735,8 @@ SCORE_BATCHES = [
 
 
 @pytest.mark.parametrize("cache_dtype,q_dtype,Hq,Hkv,D,bs", [(W.F16, W.F16, 8, 2, 128, 32), (W.U8, W.BF16, 4, 4, 128, 32),
-                                                             (W.F32, W.F32, 4, 2, 64, 16), (W.BF16, W.BF16, 6, 3, 96, 8)])
+                                                             (W.F32, W.F32, 4, 2, 64, 16), (W.BF16, W.BF16, 6, 3, 96, 8),
+                                                             (W.F16, W.F16, 16, 1, 64, 32), (W.F16, W.F32, 2, 2, 256, 16)])
 @pytest.mark.parametrize("batch", range(len(SCORE_BATCHES)))
 @pytest.mark.parametrize("window", [0, 40])
 def test_paged_attention_scores(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, bs, batch, window):
