@@ -368,11 +368,18 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
             times.append(time.perf_counter() - t0)
         return sum(times) / len(times), len(times)
 
+    # HBM bytes per launch from rocprofv3 FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB (recorded, not measured in this run)
+    source = "recorded, not measured in this run: profiles/layer_ops_8192x4096_bf16.txt"
+    recorded = {"rms_norm_vec_kernel": (32883.2 * 2 + 65536.0) * 1024, "rope_vec_kernel": (36228.1 * 2 + 65536.0) * 1024,
+                "gather_kernel": (32501.6 * 2 + 65536.0) * 1024, "concat_kernel": (32787.9 * 2 + 65536.0) * 1024,
+                "matmul_prefill": (320729.2 * 2 + 98356.2) * 1024, "matmul_decode": (27236.2 * 2 + 768.0) * 1024}
+
     def hbm(name, ms, nbytes, kernel):
         a = nbytes / (ms * 1e-3) / 1e9
         return {"workload": name, "ms_per_step": ms, "dominant_kernel_ms": ms, "bytes": nbytes,
                 "roofline": {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
-                             "traffic": None, "kernel": kernel}}
+                             "traffic": recorded.get(kernel), "traffic_source": source if kernel in recorded else None,
+                             "kernel": kernel}}
 
     out = {}
     import oracle as O
@@ -444,11 +451,12 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
         if t_mfma >= t_hbm:
             a = flops / (ms * 1e-3) / 1e12
             r["roofline"] = {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                             "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "hipBLASLt GEMM"}
+                             "frac": a / MFMA_BF16_PEAK_TFLOPS, "traffic": recorded[name], "traffic_source": source,
+                             "kernel": "hipBLASLt GEMM"}
         else:
             a = nbytes / (ms * 1e-3) / 1e9
             r["roofline"] = {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
-                             "traffic": None, "kernel": "hipBLASLt GEMM"}
+                             "traffic": recorded[name], "traffic_source": source, "kernel": "hipBLASLt GEMM"}
         if with_cpu:
             rows = min(m, 16)
             t, n = cpu_time(lambda: O.matmul(x[:rows], w, False, True), 3.0)
