@@ -84,7 +84,10 @@ hipattn_status hipops_rope(const hipops_rope_desc* desc, const void* device_x, c
  * (same, or F32); accumulation is always fp32 (the reference lets cuBLAS accumulate f16 x f16 ->
  * f16 in half precision, matmul.cpp:84-87; fp32 is the tighter of the two).
  * The workspace may be NULL / 0; hipops_matmul_workspace_size gives the size that lets the
- * library choose among all of its algorithms. */
+ * library choose among all of its algorithms.  The first call with a new shape on a device times
+ * the library's candidate algorithms on the given operands (a few extra launches that write the
+ * same C, and one event synchronisation) and keeps the fastest; under stream capture it takes the
+ * library's first choice instead. */
 typedef struct hipops_matmul_desc {
     int ab_dtype;
     int c_dtype;

@@ -1,8 +1,8 @@
 // MatMul through hipBLASLt: a plain library GEMM with fp32 accumulation.  The operator's tensors
 // are row-major; hipBLASLt is column-major, so the product is taken transposed
 // (C^T = op(B)^T * op(A)^T) with the operands swapped and no data movement.  Descriptors and the
-// algorithm the heuristic picks are kept per (device, shape), so a repeated shape costs one
-// hipblasLtMatmul call.
+// algorithm are kept per (device, shape), so a repeated shape costs one hipblasLtMatmul call; the
+// algorithm is the fastest of the heuristic's candidates, timed once when the shape is first seen.
 #include <hipblaslt/hipblaslt.h>
 
 #include <map>
@@ -127,19 +127,50 @@ hipattn_status matmul(const hipops_matmul_desc* d, const void* a, const void* b,
         BLAS_CHECK(hipblasLtMatmulPreferenceCreate(&pref));
         const uint64_t max_ws = workspace_bytes;
         BLAS_CHECK(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws)));
-        constexpr int kAsk = 8;
+        constexpr int kAsk = 16;
         hipblasLtMatmulHeuristicResult_t found[kAsk];
         int n_found = 0;
         const hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(dev.handle, plan.desc, plan.first, plan.second, plan.result,
                                                                    plan.result, pref, kAsk, found, &n_found);
         hipblasLtMatmulPreferenceDestroy(pref);
         if (hs != HIPBLAS_STATUS_SUCCESS) return fail(HIPATTN_HIP_ERROR, "matmul: heuristic query failed with status %d", (int)hs);
-        int pick = -1;
-        for (int i = 0; i < n_found && pick < 0; i++)
-            if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes) pick = i;
+        int pick = -1, usable = 0;
+        for (int i = 0; i < n_found; i++)
+            if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes) {
+                if (pick < 0) pick = i;
+                usable++;
+            }
         if (pick < 0)
             return fail(HIPATTN_UNSUPPORTED, "matmul: hipBLASLt has no algorithm for m %lld n %lld k %lld batch %lld with %zu bytes of workspace",
                         (long long)d->m, (long long)d->n, (long long)d->k, (long long)d->batch, workspace_bytes);
+        // The heuristic's order is a guess: the first time a shape is seen, and unless the stream is
+        // being captured, every candidate runs a few times on the caller's own operands (each writes the
+        // same C) and the fastest is kept.  A candidate that fails to run is skipped.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (usable > 1 && hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
+            hipEvent_t e0 = nullptr, e1 = nullptr;
+            if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+                const float one = 1.0f, zero = 0.0f;
+                float best = 0.f;
+                for (int i = 0; i < n_found; i++) {
+                    if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > workspace_bytes) continue;
+                    constexpr int kRuns = 4;
+                    bool ok = true;
+                    for (int r = 0; r < kRuns + 1 && ok; r++) {  // the first run is not timed
+                        if (r == 1) ok = hipEventRecord(e0, stream) == hipSuccess;
+                        ok = ok && hipblasLtMatmul(dev.handle, plan.desc, &one, b, plan.first, a, plan.second, &zero, c, plan.result, c,
+                                                   plan.result, &found[i].algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+                    }
+                    float ms = 0.f;
+                    ok = ok && hipEventRecord(e1, stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+                         hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+                    if (ok && (best == 0.f || ms < best)) best = ms, pick = i;
+                }
+            }
+            if (e0) (void)hipEventDestroy(e0);
+            if (e1) (void)hipEventDestroy(e1);
+            (void)hipGetLastError();  // a candidate that could not launch must not poison the caller's next check
+        }
         plan.algo = found[pick].algo;
         plan.workspace = found[pick].workspaceSize;
         it = dev.plans.emplace(key, plan).first;
