@@ -21,6 +21,7 @@ SOURCES = [
     "paged_decode.hip",
     "paged_scores.hip",
     "flash_prefill.hip",
+    "flash_small.hip",
 ]
 
 HIPCC_FLAGS = [

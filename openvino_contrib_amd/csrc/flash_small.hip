@@ -1,0 +1,277 @@
+// Flash attention on the matrix cores for dense v13::ScaledDotProductAttention at head size 64
+// (f16 / bf16, causal or not, GQA): the shape of the reference's own f16 test and of the small
+// model families.  The same products and the same register layout as the head-size-128 kernel of
+// flash_prefill.hip -- S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16, the accumulator of the
+// first being the B operand of the second -- in a plain structure: four wavefronts per workgroup,
+// 32 query rows each, key tiles of 64 staged through registers into a double-buffered, swizzled LDS
+// tile, one workgroup barrier per tile, a straightforward online softmax.  Not tuned beyond
+// conflict-free LDS access; it replaces the fp32 VALU kernel for these shapes.
+//
+// Replaces the same decomposed chain as flash_prefill.hip (src/ops/matmul.cpp:185-227,
+// src/ops/softmax.cpp:178-193, src/ops/select.cpp:50-91 of the reference).
+#include "device_common.hpp"
+#include "kernels.hpp"
+
+namespace hipattn {
+
+namespace flash_small {
+
+constexpr int kD = 64;
+constexpr int kRowBytes = kD * 2;           // a K or V row in LDS: 8 chunks of 16 bytes
+constexpr int kTileK = 64;                  // keys per tile
+constexpr int kTileBytes = kTileK * kRowBytes;
+constexpr int kWaves = 4;
+constexpr int kTileQ = 32 * kWaves;         // query rows per workgroup
+
+template <bool kBf16>
+struct Mfma;
+template <>
+struct Mfma<false> {
+    using vec8 = half8_t;
+    static __device__ __forceinline__ float16_t mma(vec8 a, vec8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t cvt2(float lo, float hi) {
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector((float2_t){lo, hi}, half2_t));
+    }
+    static __device__ __forceinline__ float to_float(uint16_t bits) { return f16_bits_to_float(bits); }
+};
+template <>
+struct Mfma<true> {
+    using vec8 = bf16x8_t;
+    static __device__ __forceinline__ float16_t mma(vec8 a, vec8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t cvt2(float lo, float hi) {
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector((float2_t){lo, hi}, bf16x2_t));
+    }
+    static __device__ __forceinline__ float to_float(uint16_t bits) { return bf16_bits_to_float(bits); }
+};
+
+// both lanes of a pair (l, l + 32) get (value of l, value of l + 32)
+__device__ __forceinline__ void pair_values(float x, float& lo, float& hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
+
+// LDS position of the 16-byte chunk c (0..7) of row r of a tile.  K: chunk c ^ ((r >> 1) & 7), so
+// that sixteen lanes reading one chunk index of sixteen consecutive rows (a K fragment) hit sixteen
+// different 16-byte bank groups; V: chunk c ^ (4 * ((r >> 1) & 1)), so that the four rows a
+// transposing read touches at once lie in four different quarters of the banks.
+__device__ __forceinline__ int k_chunk_offset(int r, int c) { return r * kRowBytes + ((c ^ ((r >> 1) & 7)) << 4); }
+__device__ __forceinline__ int v_chunk_offset(int r, int c) { return r * kRowBytes + ((c ^ (((r >> 1) & 1) << 2)) << 4); }
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef short short8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) uint8_t lds_byte;
+typedef __attribute__((address_space(3))) short4_t lds_short4;
+
+// V^T fragment (A operand of O^T = V^T P^T) of k-step ks (16 keys) and head-dim tile dt (32 rows):
+// the lane holding head-dim d = dt*32 + n32 gets V[key][d] for keys 16ks + 4hi + {0..3} and
+// 16ks + 8 + 4hi + {0..3}: the keys its P^T registers of that k-step belong to.  ds_read_b64_tr_b16
+// hands lane i of a 16-lane group element j = what lane 4j + i/4 of the group addressed, at
+// 16-bit index i % 4; so lane i addresses row key0 + i/4, head-dim d0 + 4(i % 4).. and receives
+// V[key0 + j][d0 + i] (d0 = dt*32 + 16(group & 1), key0 = 16ks + 4(group >> 1)).
+template <bool kBf16>
+__device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte* v_lds, int lane, int ks, int dt) {
+    const int g = lane >> 4, i = lane & 15;
+    const int row = 16 * ks + 4 * (g >> 1) + (i >> 2);
+    const int d0 = dt * 32 + 16 * (g & 1) + 4 * (i & 3);  // first of this lane's four head-dim elements
+    const int c = d0 >> 3, within = (d0 & 7) * 2;
+    const lds_byte* p0 = v_lds + v_chunk_offset(row, c) + within;
+    const lds_byte* p1 = v_lds + v_chunk_offset(row + 8, c) + within;
+    const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)p0);
+    const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)p1);
+    const short8_t a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+    return __builtin_bit_cast(typename Mfma<kBf16>::vec8, a);
+}
+
+template <bool kBf16>
+__global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams p) {
+    using M = Mfma<kBf16>;
+    using vec8 = typename M::vec8;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][kTileBytes];  // [buffer][K, V]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int n32 = lane & 31, hi = lane >> 5;
+    const int q_tiles = (p.len_q + kTileQ - 1) / kTileQ;
+    const int qt = blockIdx.x % q_tiles;
+    const int h = (blockIdx.x / q_tiles) % p.num_heads_q;
+    const int b = blockIdx.x / (q_tiles * p.num_heads_q);
+    const int hkv = h / (p.num_heads_q / p.num_heads_kv);
+    const int q0 = qt * kTileQ;                      // first query row of the workgroup
+    const int my_row = q0 + wave * 32 + n32;         // this lane's query row (may lie beyond len_q)
+    const uint16_t* q = (const uint16_t*)p.q + ((int64_t)(b * p.num_heads_q + h) * p.len_q) * kD;
+    const uint8_t* k = (const uint8_t*)p.k + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
+    const uint8_t* v = (const uint8_t*)p.v + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
+
+    // keys this workgroup visits: all, or up to its last query row under the causal mask
+    const int kv_end = p.causal ? min(p.len_kv, min(q0 + kTileQ, p.len_q)) : p.len_kv;
+    const int tiles = (kv_end + kTileK - 1) / kTileK;
+
+    // Q^T fragments (B operand of S^T = K Q^T): lane (n32, hi) holds query row n32, head-dim
+    // elements 8 (2i + hi) .. + 7 for k-step i, times scale * log2(e)
+    vec8 qf[4];
+    {
+        const float c = p.scale * kLog2e;
+        const int row = min(my_row, p.len_q - 1);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint4_t raw = *(const uint4_t*)(q + (int64_t)row * kD + 8 * (2 * i + hi));
+            uint4_t cv;
+#pragma unroll
+            for (int w = 0; w < 4; w++)
+                cv[w] = M::cvt2(M::to_float((uint16_t)(raw[w] & 0xffffu)) * c, M::to_float((uint16_t)(raw[w] >> 16)) * c);
+            qf[i] = __builtin_bit_cast(vec8, cv);
+        }
+    }
+
+    // tile staging: 512 16-byte pieces per K tile and per V tile, two of each per thread
+    uint4_t stage[4];
+    auto fetch = [&](int tile) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const int piece = tid + 256 * s, r = piece >> 3, c = piece & 7;
+            const int key = min(tile * kTileK + r, p.len_kv - 1);  // rows past the end repeat the last key (masked later)
+            stage[s] = *(const uint4_t*)(k + (int64_t)key * kRowBytes + 16 * c);
+            stage[2 + s] = *(const uint4_t*)(v + (int64_t)key * kRowBytes + 16 * c);
+        }
+    };
+    auto deposit = [&](int buf) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const int piece = tid + 256 * s, r = piece >> 3, c = piece & 7;
+            *(uint4_t*)(lds[buf][0] + k_chunk_offset(r, c)) = stage[s];
+            *(uint4_t*)(lds[buf][1] + v_chunk_offset(r, c)) = stage[2 + s];
+        }
+    };
+
+    float16_t o[2];
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;  // the row's running maximum (both lanes of a pair agree) and this lane's share of the sum
+
+    if (tiles > 0) {
+        fetch(0);
+        deposit(0);
+    }
+    __syncthreads();
+    for (int j = 0; j < tiles; j++) {
+        const int buf = j & 1;
+        if (j + 1 < tiles) fetch(j + 1);  // in flight while this tile is computed
+        const lds_byte* k_lds = (const lds_byte*)lds[buf][0];
+        const lds_byte* v_lds = (const lds_byte*)lds[buf][1];
+        const int ts = j * kTileK;
+
+        // scores, transposed: register r of s[mt] is key ts + 32 mt + 8 (r / 4) + 4 hi + r % 4 of query row n32
+        float16_t s[2];
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = mt * 32 + n32;
+                const vec8 kf = __builtin_bit_cast(vec8, *(const __attribute__((address_space(3))) uint4_t*)(k_lds + k_chunk_offset(row, 2 * i + hi)));
+                s[mt] = M::mma(kf, qf[i], s[mt]);
+            }
+        }
+        // mask: keys past the end, and keys after the query under the causal flag
+        const bool edge = ts + kTileK > p.len_kv || (p.causal && ts + kTileK - 1 > q0 + wave * 32);
+        if (edge) {
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+                    const bool ok = key < p.len_kv && (!p.causal || key <= my_row);
+                    s[mt][r] = ok ? s[mt][r] : -INFINITY;
+                }
+        }
+        // online softmax in the exp2 domain; the row lives in lanes l and l + 32
+        float m_tile = -INFINITY;
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, s[mt][r]);
+        float m_lo, m_hi;
+        pair_values(m_tile, m_lo, m_hi);
+        const float m_new = fmaxf(m_run, fmaxf(m_lo, m_hi));
+        // a row that has met no key yet keeps everything at zero (exp2(-inf - -inf) would be NaN)
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = fast_exp2(m_run - m_use);
+        vec8 pf[4];
+        float sum = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            uint4_t pw;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w] - m_use);
+                const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1] - m_use);
+                pw[w] = M::cvt2(p0, p1);
+                sum += p0 + p1;
+            }
+            pf[ks] = __builtin_bit_cast(vec8, pw);
+        }
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+        // O^T += V^T P^T
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++) o[dt] = M::mma(read_v_frag<kBf16>(v_lds, lane, ks, dt), pf[ks], o[dt]);
+
+        if (j + 1 < tiles) deposit(buf ^ 1);  // the other buffer was last read before the previous barrier
+        __syncthreads();
+    }
+
+    // normalise and store: register r of o[dt] is head-dim 32 dt + 8 (r / 4) + 4 hi + r % 4 of query row n32
+    float l_lo, l_hi;
+    pair_values(l_run, l_lo, l_hi);
+    const float l = l_lo + l_hi;
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    if (my_row < p.len_q) {
+        uint16_t* out = (uint16_t*)p.out + ((int64_t)(b * p.num_heads_q + h) * p.len_q + my_row) * kD;
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint2_t w;
+                w[0] = M::cvt2(o[dt][4 * g] * inv, o[dt][4 * g + 1] * inv);
+                w[1] = M::cvt2(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
+                *(uint2_t*)(out + dt * 32 + 8 * g + 4 * hi) = w;
+            }
+    }
+}
+
+}  // namespace flash_small
+
+bool sdpa_flash_small_supported(const SdpaParams& p) {
+    return p.head_dim == flash_small::kD && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16) && p.mask == nullptr &&
+           p.len_kv > 0 && p.len_q > 0 && ((uintptr_t)p.q % 16) == 0 && ((uintptr_t)p.k % 16) == 0 &&
+           ((uintptr_t)p.v % 16) == 0 && ((uintptr_t)p.out % 8) == 0;
+}
+
+hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream) {
+    const int64_t q_tiles = (p.len_q + flash_small::kTileQ - 1) / flash_small::kTileQ;
+    const int64_t groups = q_tiles * p.num_heads_q * p.batch;
+    if (groups == 0) return hipSuccess;
+    if (groups > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (p.dtype == HIPATTN_BF16)
+        hipLaunchKernelGGL(flash_small::sdpa_flash_d64_kernel<true>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+    else
+        hipLaunchKernelGGL(flash_small::sdpa_flash_d64_kernel<false>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace hipattn

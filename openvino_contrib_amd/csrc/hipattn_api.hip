@@ -376,6 +376,9 @@ HIPATTN_EXPORT hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc,
     if (!p.mask && hipattn::sdpa_flash_supported(p)) {
         g_kernel_path = "sdpa_flash_mfma";
         HIP_TRY(hipattn::launch_sdpa_flash(p, as_stream(stream), g_probe));
+    } else if (hipattn::sdpa_flash_small_supported(p)) {
+        g_kernel_path = "sdpa_flash_mfma_d64";
+        HIP_TRY(hipattn::launch_sdpa_flash_small(p, as_stream(stream)));
     } else {
         g_kernel_path = "sdpa_generic";
         HIP_TRY(hipattn::launch_sdpa_generic(p, as_stream(stream)));

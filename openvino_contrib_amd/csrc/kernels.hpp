@@ -135,6 +135,9 @@ hipError_t launch_paged_generic(const PagedParams& p, hipStream_t stream);
 // MFMA flash kernels (head_dim 64 or 128, f16 / bf16)
 bool sdpa_flash_supported(const SdpaParams& p);
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
+// head size 64 on the matrix cores (flash_small.hip)
+bool sdpa_flash_small_supported(const SdpaParams& p);
+hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream);
 
 // paged attention fast paths: plan + stream-K decode + merge, and chunked prefill
 bool paged_fast_supported(const PagedParams& p);

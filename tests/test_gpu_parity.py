@@ -111,8 +111,31 @@ def test_sdpa_small_shapes(hip, oracle, shape, causal, dtype):
     case = W.make_sdpa_case(61, B, Hq, Hkv, Lq, Lk, D, dtype)
     out, path = H.run_sdpa(hip, case, causal)
     ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
-    assert path == "sdpa_generic"
+    assert path == ("sdpa_flash_mfma_d64" if (D == 64 and dtype == W.F16) else "sdpa_generic")
     assert H.max_abs(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [W.F16, W.BF16])
+@pytest.mark.parametrize("shape,causal", [
+    ((1, 8, 8, 32, 32, 64), False), ((1, 8, 8, 32, 32, 64), True),   # the reference test's f16 shape
+    ((1, 1, 1, 1, 1, 64), True), ((1, 2, 1, 63, 63, 64), True), ((1, 2, 2, 64, 64, 64), False),
+    ((1, 4, 2, 65, 65, 64), True), ((2, 4, 1, 128, 128, 64), True), ((1, 2, 1, 129, 129, 64), True),
+    ((1, 8, 2, 300, 300, 64), True), ((1, 2, 1, 200, 1000, 64), False), ((1, 2, 1, 1000, 200, 64), True),
+    ((2, 6, 3, 515, 515, 64), True), ((1, 2, 2, 77, 500, 64), True), ((1, 3, 1, 260, 700, 64), False),
+    ((1, 2, 1, 1600, 1600, 64), True), ((3, 5, 5, 1, 700, 64), False)])
+def test_sdpa_flash_head_size_64(hip, oracle, dtype, shape, causal):
+    """Head size 64 runs on the matrix cores too (its own kernel): edge lengths either side of the
+    64-key tile and the 128-row workgroup, GQA, rectangular shapes with the top-left aligned mask."""
+    announce("sdpa flash d64", dtype, shape, causal)
+    B, Hq, Hkv, Lq, Lk, D = shape
+    case = W.make_sdpa_case(63, B, Hq, Hkv, Lq, Lk, D, dtype)
+    out, path = H.run_sdpa(hip, case, causal)
+    assert path == "sdpa_flash_mfma_d64"
+    ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+    assert np.isfinite(out).all()
+    assert H.max_abs(out, ref) <= TOL[dtype]
+    out2, _ = H.run_sdpa(hip, case, causal, scale=0.05)
+    assert H.max_abs(out2, oracle.sdpa(case["q"], case["k"], case["v"], causal=causal, scale=0.05)) <= TOL[dtype]
 
 
 def test_sdpa_golden_fixture_on_gpu(hip):
@@ -182,9 +205,9 @@ def test_sdpa_flash_scores_that_grow_along_the_keys(hip, oracle, dtype, profile,
     assert H.scaled_bound_error(out, ref, "sdpa flash %s dtype %d causal %d" % (profile, dtype, causal)) <= tol
 
 
-@pytest.mark.parametrize("dtype", [W.F32, W.F16])
+@pytest.mark.parametrize("dtype", [W.F32, W.F16, W.BF16])
 @pytest.mark.parametrize("profile", ["ramp", "step40", "fall"])
-def test_sdpa_generic_scores_that_grow_along_the_keys(hip, oracle, dtype, profile):
+def test_sdpa_head_size_64_scores_that_grow_along_the_keys(hip, oracle, dtype, profile):
     announce("sdpa generic growing scores", dtype, profile)
     B, Hq, Hkv, Lq, Lk, D = 1, 4, 2, 200, 700, 64
     rng = np.random.Generator(np.random.PCG64(72))
@@ -198,10 +221,10 @@ def test_sdpa_generic_scores_that_grow_along_the_keys(hip, oracle, dtype, profil
         case[name + "_store"], case[name] = W.to_storage(x, dtype)
     for causal in (False, True):
         out, path = H.run_sdpa(hip, case, causal)
-        assert path == "sdpa_generic"
+        assert path == ("sdpa_generic" if dtype == W.F32 else "sdpa_flash_mfma_d64")  # fp16 at head size 64: the matrix-core kernel
         ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
         assert np.isfinite(out).all()
-        assert H.scaled_bound_error(out, ref, "sdpa generic %s dtype %d causal %d" % (profile, dtype, causal)) <= TOL[dtype]
+        assert H.scaled_bound_error(out, ref, "sdpa d64 %s dtype %d causal %d" % (profile, dtype, causal)) <= TOL[dtype]
 
 
 def test_sdpa_flash_tensors_beyond_two_gib(hip, oracle):
