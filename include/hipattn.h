@@ -100,6 +100,17 @@ hipattn_status hipattn_event_record(hipattn_event event, hipattn_stream stream);
 hipattn_status hipattn_event_synchronize(hipattn_event event);
 hipattn_status hipattn_event_elapsed_ms(hipattn_event start, hipattn_event stop, float* ms);
 
+/* Stream capture into an executable graph: replaces CUDA::GraphCapture / CUDA::GraphExec
+ * (src/cuda/graph.hpp), which the reference's CudaGraphTopologyRunner is built on
+ * (src/cuda_graph_topology_runner.cpp).  Every hipattn_* and hipops_* operator call is capturable
+ * (kernel launches and event fork / join only); allocation and host copies are not.
+ * hipattn_stream_end_capture instantiates the recorded graph and hands back the executable. */
+typedef struct hipattn_graph_t* hipattn_graph; /* a hipGraphExec_t */
+hipattn_status hipattn_stream_begin_capture(hipattn_stream stream);
+hipattn_status hipattn_stream_end_capture(hipattn_stream stream, hipattn_graph* graph);
+hipattn_status hipattn_graph_launch(hipattn_graph graph, hipattn_stream stream);
+hipattn_status hipattn_graph_destroy(hipattn_graph graph);
+
 /* ---- v13::ScaledDotProductAttention -------------------------------------------------
  * Replaces the decomposed chain the reference executes after
  * ScaledDotProductAttentionDecomposition (src/transformer/cuda_graph_transformer.cpp:151-156):

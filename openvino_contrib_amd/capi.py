@@ -110,6 +110,10 @@ SYMBOLS = {
     "hipattn_event_record": (_i, [_vp, _vp]),
     "hipattn_event_synchronize": (_i, [_vp]),
     "hipattn_event_elapsed_ms": (_i, [_vp, _vp, _P(_f)]),
+    "hipattn_stream_begin_capture": (_i, [_vp]),
+    "hipattn_stream_end_capture": (_i, [_vp, _P(_vp)]),
+    "hipattn_graph_launch": (_i, [_vp, _vp]),
+    "hipattn_graph_destroy": (_i, [_vp]),
     "hipattn_sdpa_workspace_size": (_i, [_P(SdpaDesc), _P(_sz)]),
     "hipattn_sdpa": (_i, [_P(SdpaDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "hipattn_sdpa_masked": (_i, [_P(SdpaDesc), _vp, _vp, _vp, _P(MaskDesc), _vp, _vp, _vp, _sz, _vp]),

@@ -328,6 +328,36 @@ HIPATTN_EXPORT hipattn_status hipattn_event_elapsed_ms(hipattn_event start, hipa
     return HIPATTN_OK;
 }
 
+// ------------------------------------------------------------------------------- graphs
+HIPATTN_EXPORT hipattn_status hipattn_stream_begin_capture(hipattn_stream stream) {
+    if (!stream) return fail(HIPATTN_INVALID_ARGUMENT, "stream_begin_capture: the default stream cannot be captured");
+    // relaxed: other threads of the process may go on using the device (allocating, copying) meanwhile
+    HIP_TRY(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_stream_end_capture(hipattn_stream stream, hipattn_graph* graph) {
+    if (!graph) return fail(HIPATTN_INVALID_ARGUMENT, "stream_end_capture: null output");
+    *graph = nullptr;
+    hipGraph_t recorded = nullptr;
+    HIP_TRY(hipStreamEndCapture(as_stream(stream), &recorded));
+    if (!recorded) return fail(HIPATTN_HIP_ERROR, "stream_end_capture: the capture was invalidated");
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, recorded, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(recorded);
+    if (e != hipSuccess) return fail(HIPATTN_HIP_ERROR, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    *graph = (hipattn_graph)exec;
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_graph_launch(hipattn_graph graph, hipattn_stream stream) {
+    if (!graph) return fail(HIPATTN_INVALID_ARGUMENT, "graph_launch: null graph");
+    HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph, as_stream(stream)));
+    return HIPATTN_OK;
+}
+HIPATTN_EXPORT hipattn_status hipattn_graph_destroy(hipattn_graph graph) {
+    if (graph) HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph));
+    return HIPATTN_OK;
+}
+
 // ------------------------------------------------------------------------------- SDPA
 HIPATTN_EXPORT hipattn_status hipattn_sdpa_workspace_size(const hipattn_sdpa_desc* desc, size_t* bytes) {
     if (!bytes) return fail(HIPATTN_INVALID_ARGUMENT, "sdpa_workspace_size: null output");

@@ -87,6 +87,31 @@ private:
     size_t capacity_ = 0;
 };
 
+// An executable graph recorded from a stream (CUDA::GraphExec in the reference, src/cuda/graph.hpp).
+class Graph {
+public:
+    Graph() = default;
+    ~Graph() { reset(); }
+    Graph(const Graph&) = delete;
+    Graph& operator=(const Graph&) = delete;
+    static void begin_capture(const Stream& s) { HIP_PLUGIN_CHECK(hipattn_stream_begin_capture(s.get())); }
+    // ends the capture on `s` and keeps what was recorded; returns false (and keeps nothing) when the
+    // recording could not be turned into an executable graph
+    bool end_capture(const Stream& s) {
+        reset();
+        return hipattn_stream_end_capture(s.get(), &graph_) == HIPATTN_OK && graph_ != nullptr;
+    }
+    void launch(const Stream& s) const { HIP_PLUGIN_CHECK(hipattn_graph_launch(graph_, s.get())); }
+    explicit operator bool() const { return graph_ != nullptr; }
+    void reset() {
+        if (graph_) hipattn_graph_destroy(graph_);
+        graph_ = nullptr;
+    }
+
+private:
+    hipattn_graph graph_ = nullptr;
+};
+
 class Event {
 public:
     Event() { HIP_PLUGIN_CHECK(hipattn_event_create(&event_)); }

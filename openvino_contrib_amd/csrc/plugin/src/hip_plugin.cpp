@@ -25,10 +25,15 @@ namespace ov {
 namespace hip_gpu {
 
 // ------------------------------------------------------------------------- Configuration
+// the counterpart of NVIDIA_USE_CUDA_GRAPH (include/nvidia/properties.hpp:30)
+static const char* const kUseGraphProperty = "HIP_USE_GRAPH";
+static const char* const kGraphMinOperatorsProperty = "HIP_GRAPH_MIN_OPERATORS";
+
 const std::vector<std::string>& Configuration::rw_properties() {
     static const std::vector<std::string> names = {ov::device::id.name(), ov::hint::inference_precision.name(),
                                                    ov::enable_profiling.name(), ov::num_streams.name(),
-                                                   ov::hint::performance_mode.name()};
+                                                   ov::hint::performance_mode.name(), kUseGraphProperty,
+                                                   kGraphMinOperatorsProperty};
     return names;
 }
 
@@ -61,6 +66,11 @@ Configuration Configuration::from(const ov::AnyMap& properties, const Configurat
             c.inference_precision = t;
         } else if (key == ov::enable_profiling.name()) {
             c.enable_profiling = value.as<bool>();
+        } else if (key == kUseGraphProperty) {
+            c.use_graph = value.as<bool>();
+        } else if (key == kGraphMinOperatorsProperty) {
+            c.graph_min_operators = value.as<int>();
+            if (c.graph_min_operators < 1) HIP_PLUGIN_THROW(std::string("property ") + kGraphMinOperatorsProperty + ": at least 1 expected");
         } else if (key == ov::num_streams.name()) {
             c.num_streams = value.as<int>();
             if (c.num_streams < 1) HIP_PLUGIN_THROW("property NUM_STREAMS must be positive");
@@ -79,6 +89,8 @@ ov::Any Configuration::get(const std::string& name) const {
     if (name == ov::device::id.name()) return std::to_string(device_id);
     if (name == ov::hint::inference_precision.name()) return inference_precision.get_type_name();
     if (name == ov::enable_profiling.name()) return enable_profiling;
+    if (name == kUseGraphProperty) return use_graph;
+    if (name == kGraphMinOperatorsProperty) return (int64_t)graph_min_operators;
     if (name == ov::num_streams.name()) return (int64_t)num_streams;
     if (name == ov::hint::performance_mode.name()) return performance_mode;
     HIP_PLUGIN_THROW("property '" + name + "' is not supported by the HIP plugin");
@@ -490,11 +502,16 @@ ov::Any CompiledModel::get_property(const std::string& name) const {
         return std::vector<std::string>{get_plugin()->get_device_name() + "." + std::to_string(config_.device_id)};
     if (name == ov::optimal_number_of_infer_requests.name()) return (int64_t)config_.num_streams;
     if (name == ov::loaded_from_cache.name()) return loaded_from_cache_;
+    // graphs recorded / launched by this model's requests so far (the reference reports the count it
+    // builds at compile time as NVIDIA_NUMBER_OF_CUDA_GRAPHS, include/nvidia/properties.hpp:35)
+    if (name == "HIP_NUMBER_OF_GRAPHS") return (int64_t)graphs_captured_.load();
+    if (name == "HIP_GRAPH_LAUNCHES") return (int64_t)graph_launches_.load();
     if (name == ov::supported_properties.name()) {
         std::vector<ov::PropertyName> all;
         for (auto& n : Configuration::rw_properties()) all.emplace_back(n, ov::PropertyMutability::RO);
         for (const char* n : {ov::supported_properties.name(), ov::model_name.name(), ov::execution_devices.name(),
-                              ov::optimal_number_of_infer_requests.name(), ov::loaded_from_cache.name()})
+                              ov::optimal_number_of_infer_requests.name(), ov::loaded_from_cache.name(), "HIP_NUMBER_OF_GRAPHS",
+                              "HIP_GRAPH_LAUNCHES"})
             all.emplace_back(n, ov::PropertyMutability::RO);
         return all;
     }
@@ -538,6 +555,16 @@ InferRequest::InferRequest(const std::shared_ptr<const CompiledModel>& compiled,
     for (const auto& port : get_outputs()) allocate_tensor(port, host_tensor(port));
     for (const auto& variable : compiled_->get_runtime_model()->get_variables())
         variables_.add(variable->get_info().variable_id, std::make_shared<VariableState>(variable->get_info()));
+    // ReadValue / Assign change host-side state while they enqueue: such a model runs operator by
+    // operator (the reference keeps stateful and dynamic models off its graph runner too,
+    // src/cuda_compiled_model.cpp:53-62)
+    int operators = 0;
+    for (const auto& step : compiled_->exec_sequence()) {
+        const std::string& type = step.op->GetTypeName();
+        operators += (type != "Parameter" && type != "Result" && type != "Constant");
+    }
+    graph_allowed_ = compiled_->config().use_graph && !compiled_->config().enable_profiling && variables_.all().empty() &&
+                     operators >= compiled_->config().graph_min_operators;
 }
 
 std::vector<ov::SoPtr<ov::IVariableState>> InferRequest::query_state() const {
@@ -575,97 +602,55 @@ void InferRequest::start_pipeline(const ThreadContext& thread_context) {
     ev_end_.clear();
     ev_step_.clear();
     profiling_.clear();
-    // The request's tensors are kept per port of the compiled model; port i belongs to parameter i /
-    // result i of the model the execution sequence was built from.
-    const auto& parameters = compiled_->parameters();
     const auto& results = compiled_->results();
-    std::map<const ov::Node*, ov::SoPtr<ov::ITensor>> input_tensors;
-    for (size_t i = 0; i < parameters.size(); i++) input_tensors[parameters[i].get()] = get_tensor(get_inputs().at(i));
-    // output ports bound to device tensors receive the operator's result in place
-    std::map<TensorID, void*> remote_outputs;
-    for (size_t i = 0; i < results.size(); i++) {
-        auto t = get_tensor(get_outputs().at(i));
-        if (auto remote = std::dynamic_pointer_cast<RemoteTensor>(t._ptr)) {
-            const auto src = results[i]->input_value(0);
-            remote_outputs[compiled_->output_ids(src.get_node()).at(src.get_index())] = remote->device_ptr();
-        }
-    }
 
-    const auto& sequence = compiled_->exec_sequence();
-    for (size_t si = 0; si < sequence.size(); si++) {
+    // Shapes, memory and scratch of every operator first (nothing is enqueued but uploads), then the
+    // operators themselves: one after the other, or as one graph when this infer is a repeat of the
+    // last one in everything the operators were handed.
+    prepare_steps(thread_context, context);
+    const bool graph_mode = graph_allowed_ && !profiling;
+    if (graph_mode) signature_ = make_signature();
+    if (graph_mode && graph_ && signature_ == last_signature_) {
         if (cancellation_.is_cancelled()) throw ov::Cancelled("Infer Request was canceled");
-        const auto& step = sequence[si];
-        const ov::Node& node = *step.node;
-        const auto& out_ids = step.op->GetOutputIds();
-        if (ov::as_type<const ov::op::v0::Parameter>(&node)) {
-            // bind or upload (the reference uploads every input on every infer,
-            // src/ops/parameter.cpp:24-33; device-resident tensors are passed through untouched)
-            auto t = input_tensors.at(&node);
-            TensorView v;
-            v.type = t->get_element_type();
-            v.shape = t->get_shape();
-            if (auto remote = std::dynamic_pointer_cast<RemoteTensor>(t._ptr)) {
-                v.device = remote->device_ptr();
-            } else {
-                v.host = t->data();
-                v.device = tensor_buffers_[out_ids[0]].reserve(std::max<size_t>(v.byte_size(), 16));
-                if (v.byte_size()) stream.upload(v.device, v.host, v.byte_size());
-            }
-            views_[out_ids[0]] = v;
-            continue;
+        graph_.launch(stream);
+        graph_launches_++;
+        compiled_->count_graph_launch();
+    } else if (graph_mode && signature_ == last_signature_) {
+        // the second infer in a row with this signature: everything it needs is allocated, record it
+        Graph::begin_capture(stream);
+        bool recorded = false;
+        try {
+            execute_steps(context, false);
+            recorded = graph_.end_capture(stream);
+        } catch (...) {
+            graph_.end_capture(stream);  // leave capture mode before the error travels on
+            graph_.reset();
+            throw;
         }
-        std::vector<TensorView> in;
-        for (TensorID id : step.op->GetInputIds()) in.push_back(views_[id]);
-        const std::vector<ov::Shape> out_shapes = step.op->InferOutputShapes(in, context);
-        std::vector<TensorView> out;
-        for (size_t o = 0; o < out_ids.size(); o++) {
-            TensorView v;
-            v.type = node.get_output_element_type(o);
-            v.shape = out_shapes.at(o);
-            const int alias = step.op->InplaceInputOf(o);
-            auto bound = remote_outputs.find(out_ids[o]);
-            if (alias >= 0) {
-                v.device = in.at(alias).device;
-                v.host = in.at(alias).host;
-            } else if (bound != remote_outputs.end()) {
-                v.device = bound->second;
-            } else {
-                v.device = tensor_buffers_[out_ids[o]].reserve(std::max<size_t>(v.byte_size(), 16));
-                if (const void* host = step.op->HostData(o)) {  // a Constant: uploaded once per request
-                    v.host = host;
-                    if (v.byte_size() && constants_on_device_.insert(out_ids[o]).second) stream.upload(v.device, host, v.byte_size());
-                }
-            }
-            out.push_back(v);
-            views_[out_ids[o]] = v;
+        if (recorded) {
+            graphs_captured_++;
+            compiled_->count_graph_captured();
+            graph_.launch(stream);
+            graph_launches_++;
+            compiled_->count_graph_launch();
+        } else {
+            graph_allowed_ = false;  // this model does not record: run it operator by operator from now on
+            execute_steps(context, false);
         }
-        const WorkbufferRequest req = step.op->GetWorkBufferRequest(in);
-        Workbuffers wb;
-        size_t total = 0;
-        for (size_t b : req.mutable_sizes) total += (b + 255) / 256 * 256;
-        if (total) {
-            // one arena for all steps: they run one after the other on the request's stream
-            char* base = (char*)workbuffer_.reserve(total);
-            for (size_t b : req.mutable_sizes) {
-                wb.mutable_buffers.push_back(base);
-                wb.mutable_sizes.push_back(b);
-                base += (b + 255) / 256 * 256;
-            }
-        }
-        if (profiling) {
-            ev_begin_.emplace_back(new Event());
-            ev_end_.emplace_back(new Event());
-            ev_step_.push_back(si);
-            ev_begin_.back()->record(stream);
-        }
-        step.op->Execute(context, in, out, wb);
-        if (profiling) ev_end_.back()->record(stream);
-        // an input the operator updated in place that the caller bound as host memory: the update goes
-        // back there (slow -- a KV cache belongs in a device tensor -- but never silently lost)
-        for (size_t idx : step.op->UpdatedInputs())
+    } else {
+        graph_.reset();
+        execute_steps(context, profiling);
+    }
+    if (graph_mode) last_signature_ = signature_;
+    // an input an operator updated in place that the caller bound as host memory: the update goes
+    // back there (slow -- a KV cache belongs in a device tensor -- but never silently lost)
+    const auto& sequence = compiled_->exec_sequence();
+    for (size_t si = 0; si < sequence.size(); si++)
+        for (size_t idx : sequence[si].op->UpdatedInputs()) {
+            const auto& in = prepared_[si].in;
             if (idx < in.size() && in[idx].host && in[idx].byte_size())
                 stream.download(const_cast<void*>(in[idx].host), in[idx].device, in[idx].byte_size());
-    }
+        }
 
     // results into the host tensors of the output ports (device-bound outputs were written in place,
     // or are copied device to device when they alias something else)
@@ -681,6 +666,140 @@ void InferRequest::start_pipeline(const ThreadContext& thread_context) {
         if (t->get_shape() != v.shape) t->set_shape(v.shape);
         if (v.byte_size()) stream.download(t->data(), v.device, v.byte_size());
     }
+}
+
+void InferRequest::prepare_steps(const ThreadContext& thread_context, const InferenceRequestContext& context) {
+    const Stream& stream = thread_context.stream;
+    // The request's tensors are kept per port of the compiled model; port i belongs to parameter i /
+    // result i of the model the execution sequence was built from.
+    const auto& parameters = compiled_->parameters();
+    const auto& results = compiled_->results();
+    std::map<const ov::Node*, ov::SoPtr<ov::ITensor>> input_tensors;
+    for (size_t i = 0; i < parameters.size(); i++) input_tensors[parameters[i].get()] = get_tensor(get_inputs().at(i));
+    // output ports bound to device tensors receive the operator's result in place
+    std::map<TensorID, void*> remote_outputs;
+    for (size_t i = 0; i < results.size(); i++) {
+        auto t = get_tensor(get_outputs().at(i));
+        if (auto remote = std::dynamic_pointer_cast<RemoteTensor>(t._ptr)) {
+            const auto src = results[i]->input_value(0);
+            remote_outputs[compiled_->output_ids(src.get_node()).at(src.get_index())] = remote->device_ptr();
+        }
+    }
+    const auto& sequence = compiled_->exec_sequence();
+    prepared_.assign(sequence.size(), PreparedStep{});
+    // scratch: one arena for all steps (they run one after the other on the request's stream), sized
+    // for the largest request before any pointer into it is handed out
+    std::vector<WorkbufferRequest> requests(sequence.size());
+    for (size_t si = 0; si < sequence.size(); si++) {
+        const auto& step = sequence[si];
+        const ov::Node& node = *step.node;
+        const auto& out_ids = step.op->GetOutputIds();
+        PreparedStep& ps = prepared_[si];
+        if (ov::as_type<const ov::op::v0::Parameter>(&node)) {
+            // bind or upload (the reference uploads every input on every infer,
+            // src/ops/parameter.cpp:24-33; device-resident tensors are passed through untouched)
+            auto t = input_tensors.at(&node);
+            TensorView v;
+            v.type = t->get_element_type();
+            v.shape = t->get_shape();
+            if (auto remote = std::dynamic_pointer_cast<RemoteTensor>(t._ptr)) {
+                v.device = remote->device_ptr();
+            } else {
+                v.host = t->data();
+                v.device = tensor_buffers_[out_ids[0]].reserve(std::max<size_t>(v.byte_size(), 16));
+                if (v.byte_size()) stream.upload(v.device, v.host, v.byte_size());
+            }
+            views_[out_ids[0]] = v;
+            ps.out.push_back(v);
+            continue;
+        }
+        for (TensorID id : step.op->GetInputIds()) ps.in.push_back(views_[id]);
+        const std::vector<ov::Shape> out_shapes = step.op->InferOutputShapes(ps.in, context);
+        for (size_t o = 0; o < out_ids.size(); o++) {
+            TensorView v;
+            v.type = node.get_output_element_type(o);
+            v.shape = out_shapes.at(o);
+            const int alias = step.op->InplaceInputOf(o);
+            auto bound = remote_outputs.find(out_ids[o]);
+            if (alias >= 0) {
+                v.device = ps.in.at(alias).device;
+                v.host = ps.in.at(alias).host;
+            } else if (bound != remote_outputs.end()) {
+                v.device = bound->second;
+            } else {
+                v.device = tensor_buffers_[out_ids[o]].reserve(std::max<size_t>(v.byte_size(), 16));
+                if (const void* host = step.op->HostData(o)) {  // a Constant: uploaded once per request
+                    v.host = host;
+                    if (v.byte_size() && constants_on_device_.insert(out_ids[o]).second) stream.upload(v.device, host, v.byte_size());
+                }
+            }
+            ps.out.push_back(v);
+            views_[out_ids[o]] = v;
+        }
+        requests[si] = step.op->GetWorkBufferRequest(ps.in);
+    }
+    size_t arena = 0;
+    for (const auto& req : requests) {
+        size_t total = 0;
+        for (size_t b : req.mutable_sizes) total += (b + 255) / 256 * 256;
+        arena = std::max(arena, total);
+    }
+    char* const arena_base = arena ? (char*)workbuffer_.reserve(arena) : nullptr;
+    for (size_t si = 0; si < sequence.size(); si++) {
+        char* base = arena_base;
+        for (size_t b : requests[si].mutable_sizes) {
+            prepared_[si].workbuffers.mutable_buffers.push_back(base);
+            prepared_[si].workbuffers.mutable_sizes.push_back(b);
+            base += (b + 255) / 256 * 256;
+        }
+    }
+}
+
+void InferRequest::execute_steps(const InferenceRequestContext& context, bool profiling) {
+    const auto& sequence = compiled_->exec_sequence();
+    for (size_t si = 0; si < sequence.size(); si++) {
+        const auto& step = sequence[si];
+        if (ov::as_type<const ov::op::v0::Parameter>(step.node.get())) continue;
+        if (cancellation_.is_cancelled()) throw ov::Cancelled("Infer Request was canceled");
+        if (profiling) {
+            ev_begin_.emplace_back(new Event());
+            ev_end_.emplace_back(new Event());
+            ev_step_.push_back(si);
+            ev_begin_.back()->record(context.stream);
+        }
+        step.op->Execute(context, prepared_[si].in, prepared_[si].out, prepared_[si].workbuffers);
+        if (profiling) ev_end_.back()->record(context.stream);
+    }
+}
+
+// Everything the operators of this infer were handed, as numbers: two infers with equal signatures
+// enqueue the same launches on the same memory.  Host-side values an operator may read while it
+// launches (scalars such as a scale, a window or a context bound) are part of it when they are
+// small; the shapes cover what larger host tensors decide (the extent of the scores output).
+std::vector<uint64_t> InferRequest::make_signature() const {
+    std::vector<uint64_t> sig;
+    auto add_view = [&](const TensorView& v) {
+        sig.push_back((uint64_t)(uintptr_t)v.device);
+        sig.push_back(v.shape.size());
+        for (size_t d : v.shape) sig.push_back(d);
+        const size_t bytes = v.byte_size();
+        if (v.host != nullptr && bytes > 0 && bytes <= 64) {
+            uint64_t words[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            std::memcpy(words, v.host, bytes);
+            sig.insert(sig.end(), words, words + (bytes + 7) / 8);
+        } else {
+            sig.push_back(v.host != nullptr);
+        }
+    };
+    for (const auto& ps : prepared_) {
+        for (const auto& v : ps.in) add_view(v);
+        for (const auto& v : ps.out) add_view(v);
+        for (size_t i = 0; i < ps.workbuffers.mutable_buffers.size(); i++) {
+            sig.push_back((uint64_t)(uintptr_t)ps.workbuffers.mutable_buffers[i]);
+            sig.push_back(ps.workbuffers.mutable_sizes[i]);
+        }
+    }
+    return sig;
 }
 
 void InferRequest::wait_pipeline(const ThreadContext& thread_context) { thread_context.stream.synchronize(); }

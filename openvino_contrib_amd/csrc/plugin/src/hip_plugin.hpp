@@ -17,6 +17,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <atomic>
 #include <set>
 #include <string>
 #include <thread>
@@ -49,6 +50,14 @@ struct Configuration {
     bool enable_profiling = false;
     int num_streams = 1;
     std::string performance_mode = "LATENCY";
+    // Replay the operator sequence of an infer request from a captured graph when nothing about it
+    // has changed (the reference's NVIDIA_USE_CUDA_GRAPH, nvidia/properties.hpp:30).
+    bool use_graph = true;
+    // ... for models of at least this many operators (Parameter, Result and Constant not counted).
+    // Measured on MI355X / ROCm 7.2 with 64-token RMS + MatMul layers: launching a graph costs more
+    // than two kernel launches and less than eight (2 kernels 35 us against 26 us one by one, 8 kernels
+    // 65 against 73, 32 kernels 173 against 225), so a lone attention operator stays off the graph.
+    int graph_min_operators = 6;
 
     static Configuration from(const ov::AnyMap& properties, const Configuration& base, bool throw_on_unsupported = true);
     ov::Any get(const std::string& name) const;
@@ -163,6 +172,8 @@ public:
     const Configuration& config() const { return config_; }
     const ov::ParameterVector& parameters() const { return exec_model_->get_parameters(); }
     const ov::ResultVector& results() const { return exec_model_->get_results(); }
+    void count_graph_captured() const { graphs_captured_++; }
+    void count_graph_launch() const { graph_launches_++; }
 
 protected:
     std::shared_ptr<ov::ISyncInferRequest> create_sync_infer_request() const override;
@@ -176,6 +187,7 @@ private:
     std::vector<ExecStep> exec_sequence_;
     std::map<const ov::Node*, std::vector<TensorID>> output_ids_;  // per node: one TensorID per output port
     size_t num_tensors_ = 0;
+    mutable std::atomic<size_t> graphs_captured_{0}, graph_launches_{0};
 };
 
 class InferRequest : public ov::ISyncInferRequest {
@@ -206,6 +218,29 @@ private:
     std::vector<ov::ProfilingInfo> profiling_;
     VariableContext variables_;
     CancellationToken cancellation_;
+
+    // What the operator sequence of one infer consists of once shapes are known and memory is bound.
+    struct PreparedStep {
+        std::vector<TensorView> in, out;
+        Workbuffers workbuffers;
+    };
+    std::vector<PreparedStep> prepared_;
+    // Graph replay (the reference's CudaGraphTopologyRunner, src/cuda_graph_topology_runner.cpp, for a
+    // model whose shapes may change from infer to infer): the signature of an infer is every pointer,
+    // shape, scratch address and small host-side value its operators were handed.  The second infer
+    // in a row with one signature is recorded into a graph, later ones replay it; a new signature
+    // starts over.
+    std::vector<uint64_t> signature_, last_signature_;
+    Graph graph_;
+    size_t graph_launches_ = 0, graphs_captured_ = 0;
+    bool graph_allowed_ = false;
+    std::vector<uint64_t> make_signature() const;
+    void prepare_steps(const ThreadContext& thread_context, const InferenceRequestContext& context);
+    void execute_steps(const InferenceRequestContext& context, bool profiling);
+
+public:
+    size_t graph_launches() const { return graph_launches_; }
+    size_t graphs_captured() const { return graphs_captured_; }
 };
 
 class AsyncInferRequest : public ov::IAsyncInferRequest {

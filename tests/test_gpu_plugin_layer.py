@@ -255,3 +255,155 @@ def test_attention_half_of_a_decoder_layer(hip, oracle):
     assert float(np.max(np.abs(kc_got - okc.view(np.float16).astype(np.float32)))) <= 0.07
     types = [t for _, t, _ in req.profiling()]
     assert types.count("MatMul") == 4 and types.count("RoPE") == 2 and "PagedAttentionExtension" in types
+
+
+def _small_chain(dtype=BF16):
+    """RMS -> MatMul -> RoPE with a position input: enough operators for a graph to matter."""
+    g = P.GraphText("chain")
+    x = g.parameter("x", dtype, [-1, 256])
+    w = g.parameter("w", dtype, [256, 256])
+    c = g.parameter("cos", F32, [-1, 64])
+    s = g.parameter("sin", F32, [-1, 64])
+    pos = g.parameter("positions", P.I32, [-1])
+    gamma_st, gamma = storage(np.linspace(0.5, 1.5, 256), dtype)
+    n = g.add("RMS", "norm", [x, g.constant("gamma", gamma_st, P._TYPE_NAMES[dtype])], epsilon=1e-5, output_type="dynamic")
+    m = g.add("MatMul", "proj", [n, w], transpose_a=False, transpose_b=True)
+    g.result("out", g.add("RoPE", "rope", [m, c, s, pos], head_cnt=4, head_size=64, rotary_ndims=64, gather_position_arg_id=3))
+    return g, gamma
+
+
+def _chain_reference(oracle, xv, wv, gamma, cos, sin, positions, dtype=BF16):
+    r = lambda a: oracle.round_to(a, dtype)
+    n = r(oracle.rms_norm(xv, gamma, 1e-5))
+    m = r(oracle.matmul(n, wv, False, True))
+    return r(oracle.rope(m.reshape(-1, 4, 64), cos, sin, positions)).reshape(-1, 256)
+
+
+def test_infer_request_replays_a_graph(hip, oracle):
+    """The second infer in a row that hands the operators the same pointers, shapes and small host
+    values is recorded into a graph and later ones replay it; host inputs are uploaded outside the
+    graph, so new values in the same tensors flow through a replay; anything else that changes (a
+    shape, a device pointer) sends the request back to operator-by-operator execution."""
+    rng = np.random.default_rng(8)
+    g, gamma = _small_chain()
+    # (three operators: below the size from which a graph pays and is used unasked)
+    compiled = P.Plugin().compile_model(g.model(), {"HIP_GRAPH_MIN_OPERATORS": "1"})
+    assert compiled.get_property("HIP_USE_GRAPH") == "YES"
+    T = 24
+    w_st, wv = storage(rng.standard_normal((256, 256)) / 16, BF16)
+    dw = hip.DeviceBuffer.from_numpy(w_st)
+    cos, sin = rope_tables(100, 64)
+    req = compiled.create_infer_request()
+    req.set_device_input(1, dw.ptr, BF16, [256, 256])
+    req.set_input(2, cos, F32)
+    req.set_input(3, sin, F32)
+
+    def step(x_st, positions):
+        req.set_input(0, x_st, BF16)
+        req.set_input(4, positions, P.I32)
+        req.infer()
+        out, _ = req.output(0)
+        return H.storage_to_f32(out, BF16)
+
+    counts = lambda: (int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")), int(compiled.get_property("HIP_GRAPH_LAUNCHES")))
+    x_st, xv = storage(rng.standard_normal((T, 256)), BF16)
+    positions = rng.integers(0, 100, T).astype(np.int32)
+    ref = _chain_reference(oracle, xv, wv, gamma, cos, sin, positions)
+    first = step(x_st, positions)
+    assert scaled_error(first, ref) <= 3e-2 and counts() == (0, 0)          # operator by operator
+    assert np.array_equal(step(x_st, positions), first) and counts() == (1, 1)  # recorded, then launched
+    assert np.array_equal(step(x_st, positions), first) and counts() == (1, 2)  # replayed
+    # new values in the same host tensors: uploaded ahead of the replay
+    x2_st, x2v = storage(rng.standard_normal((T, 256)), BF16)
+    positions2 = rng.integers(0, 100, T).astype(np.int32)
+    got = step(x2_st, positions2)
+    assert counts() == (1, 3)
+    assert scaled_error(got, _chain_reference(oracle, x2v, wv, gamma, cos, sin, positions2)) <= 3e-2
+    assert not np.array_equal(got, first)
+    # another number of tokens: no replay; twice more and the new shape has a graph of its own
+    x3_st, x3v = storage(rng.standard_normal((T + 5, 256)), BF16)
+    positions3 = rng.integers(0, 100, T + 5).astype(np.int32)
+    ref3 = _chain_reference(oracle, x3v, wv, gamma, cos, sin, positions3)
+    got3 = step(x3_st, positions3)
+    assert counts() == (1, 3) and scaled_error(got3, ref3) <= 3e-2
+    assert np.array_equal(step(x3_st, positions3), got3) and counts() == (2, 4)
+    assert np.array_equal(step(x3_st, positions3), got3) and counts() == (2, 5)
+    # a different weight tensor on the device: a new signature again
+    dw2 = hip.DeviceBuffer.from_numpy(w_st)
+    req.set_device_input(1, dw2.ptr, BF16, [256, 256])
+    assert np.array_equal(step(x3_st, positions3), got3) and counts() == (2, 5)
+
+
+def test_graph_replay_can_be_switched_off(hip, oracle):
+    rng = np.random.default_rng(9)
+    g, gamma = _small_chain()
+    plugin = P.Plugin()
+    compiled = plugin.compile_model(g.model(), {"HIP_USE_GRAPH": "NO", "HIP_GRAPH_MIN_OPERATORS": "1"})
+    w_st, _ = storage(rng.standard_normal((256, 256)) / 16, BF16)
+    cos, sin = rope_tables(50, 64)
+    x_st, _ = storage(rng.standard_normal((8, 256)), BF16)
+    positions = np.arange(8, dtype=np.int32)
+    req = compiled.create_infer_request()
+    outs = []
+    for _ in range(3):
+        for i, (a, dt) in enumerate([(x_st, BF16), (w_st, BF16), (cos, F32), (sin, F32), (positions, P.I32)]):
+            req.set_input(i, a, dt)
+        req.infer()
+        outs.append(req.output(0)[0])
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[2])
+    assert int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")) == 0
+    # profiling needs the operators one by one: it keeps the graph off as well
+    profiled = plugin.compile_model(g.model(), {"PERF_COUNT": "YES", "HIP_GRAPH_MIN_OPERATORS": "1"})
+    # and so does a model of fewer operators than a graph pays for (three here, six by default)
+    small = plugin.compile_model(g.model())
+    req = small.create_infer_request()
+    for _ in range(3):
+        for i, (a, dt) in enumerate([(x_st, BF16), (w_st, BF16), (cos, F32), (sin, F32), (positions, P.I32)]):
+            req.set_input(i, a, dt)
+        req.infer()
+    assert int(small.get_property("HIP_NUMBER_OF_GRAPHS")) == 0 and small.get_property("HIP_GRAPH_MIN_OPERATORS") == "6"
+    req = profiled.create_infer_request()
+    for _ in range(3):
+        for i, (a, dt) in enumerate([(x_st, BF16), (w_st, BF16), (cos, F32), (sin, F32), (positions, P.I32)]):
+            req.set_input(i, a, dt)
+        req.infer()
+    assert int(profiled.get_property("HIP_NUMBER_OF_GRAPHS")) == 0 and len(req.profiling()) > 0
+
+
+def test_paged_attention_decode_steps_replay_a_graph(hip, oracle):
+    """A decode-only PagedAttentionExtension step with device-resident tensors, replayed: the cache
+    write and the attention of every replay must be those of the eager step (same lengths: the
+    step is repeated, not advanced)."""
+    seqs = [(c - 1, 1) for c in (700, 64, 1500, 33, 2049, 5)]
+    case = W.make_paged_case(98, seqs, 16, 4, 128, 32, W.F16, W.F16, W.F16)
+    compiled = P.Plugin().compile_model(P.Model.paged_attention(W.F16, W.F16, W.F16, 16, 4, 128, 32), {"HIP_GRAPH_MIN_OPERATORS": "1"})
+    kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
+    vc = hip.DeviceBuffer.from_numpy(case["value_cache"])
+    dev = {n: hip.DeviceBuffer.from_numpy(case[n]) for n in ("q_store", "k_new_store", "v_new_store", "past_lens",
+                                                             "subsequence_begins", "block_indices", "block_indices_begins")}
+    req = compiled.create_infer_request()
+    T = case["q_store"].shape[0]
+    req.set_device_input(0, dev["q_store"].ptr, W.F16, [T, 16 * 128])
+    req.set_device_input(1, dev["k_new_store"].ptr, W.F16, [T, 4 * 128])
+    req.set_device_input(2, dev["v_new_store"].ptr, W.F16, [T, 4 * 128])
+    shape = list(case["key_cache"].shape[:3]) + [128]
+    req.set_device_input(3, kc.ptr, W.F16, shape)
+    req.set_device_input(4, vc.ptr, W.F16, shape)
+    for i, n in enumerate(("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")):
+        req.set_device_input(5 + i, dev[n].ptr, P.I32, list(case[n].shape))
+    req.set_input(9, np.zeros((0,), np.float32), W.F32)
+    req.set_input(10, np.array([0], np.int32), P.I32)
+    req.set_input(11, np.zeros((0,), np.float32), W.F32)
+    req.set_input(12, np.array([case["max_context_len"]], np.int32), P.I32)
+    from helpers import oracle_paged
+
+    ref, okc, ovc = oracle_paged(oracle, case)
+    outs = []
+    for _ in range(4):
+        req.infer()
+        outs.append(H.storage_to_f32(req.output(0)[0], W.F16))
+    assert H.max_abs(outs[0], ref) <= 2e-3
+    for o in outs[1:]:
+        assert np.array_equal(o, outs[0])
+    assert int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")) == 1 and int(compiled.get_property("HIP_GRAPH_LAUNCHES")) == 3
+    np.testing.assert_array_equal(kc.download(np.uint8, case["key_cache"].shape), okc)

@@ -128,6 +128,10 @@ def test_properties():
     plugin.set_property("INFERENCE_PRECISION_HINT", "bf16")
     assert plugin.get_property("INFERENCE_PRECISION_HINT") == "bf16"
     assert plugin.get_property("RANGE_FOR_ASYNC_INFER_REQUESTS") == "1 1 1"
+    # graph replay of repeated infers is on unless switched off (the reference's NVIDIA_USE_CUDA_GRAPH)
+    assert "HIP_USE_GRAPH" in plugin.get_property("SUPPORTED_PROPERTIES") and plugin.get_property("HIP_USE_GRAPH") == "YES"
+    plugin.set_property("HIP_USE_GRAPH", "NO")
+    assert plugin.get_property("HIP_USE_GRAPH") == "NO"
     with pytest.raises(P.PluginError) as e:
         plugin.set_property("INFERENCE_PRECISION_HINT", "f64")
     assert "INFERENCE_PRECISION_HINT" in str(e.value) and "hip_plugin.cpp" in str(e.value)  # file:line(function): text
