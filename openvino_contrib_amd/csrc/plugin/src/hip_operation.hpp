@@ -108,7 +108,11 @@ public:
                                                      const InferenceRequestContext& context) const = 0;
     // Scratch the operator needs for these shapes; the request provides it in Execute().
     virtual WorkbufferRequest GetWorkBufferRequest(const std::vector<TensorView>& /*inputs*/) const { return {}; }
-    // Enqueue the operator on context.stream.  const: one instance serves every request.
+    // Enqueue the operator on context.stream.  const: one instance serves every request.  Must only
+    // enqueue (kernel launches, device-to-device copies): a request may record the call into a graph
+    // and replay it.  Host bytes of an input (TensorView::host) may steer the launch only when the
+    // input holds at most 64 bytes -- those are part of the signature a replay is keyed by; whatever a
+    // larger host input decides has to show in InferOutputShapes.
     virtual void Execute(const InferenceRequestContext& context, Inputs inputs, Outputs outputs,
                          const Workbuffers& workbuffers) const = 0;
     // Outputs that alias an input buffer and are updated in place (input index per output, -1 = none).
