@@ -435,6 +435,23 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
     ms = timed(lambda: ops.concat([da, db], [hidden, hidden], T, do))
     out["concat"] = hbm("Concat of two [%d, %d] bf16 along the last axis" % (T, hidden // 2), ms, 2 * T * hidden * 2, "concat_kernel")
 
+    # gated MLP: GLU over the fused gate|up projection (width 14,336) and the unfused Swish and Multiply
+    ffn, Tm = 14336, 2048
+    dgu, gu = dev((Tm, 2 * ffn))
+    dmo = hip.DeviceBuffer(Tm * ffn * 2)
+    ms = timed(lambda: ops.glu(dgu, dmo, Tm, ffn, BF16))
+    out["glu"] = hbm("GLU (Swish), [%d, 2 x %d] bf16" % (Tm, ffn), ms, 3 * Tm * ffn * 2, "eltwise_vec_kernel(glu)")
+    if with_cpu:
+        t, n = cpu_time(lambda: O.glu(gu[:sample], 0, True))
+        out["glu"]["cpu_baseline"] = {"value": (3 * sample * ffn * 4) / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                      "sample": "oracle (fp32, one thread) on %d of %d rows, mean of %d passes" % (sample, Tm, n)}
+    ms = timed(lambda: ops.swish(dgu, dmo, Tm * ffn, BF16))
+    out["swish"] = hbm("Swish, %d x %d bf16" % (Tm, ffn), ms, 2 * Tm * ffn * 2, "eltwise_vec_kernel(swish)")
+    ms = timed(lambda: ops.multiply(dgu, dx, dmo, Tm * ffn, BF16))
+    out["multiply"] = hbm("Multiply, %d x %d bf16" % (Tm, ffn), ms, 3 * Tm * ffn * 2, "eltwise_vec_kernel(multiply)")
+    dgu.free()
+    dmo.free()
+
     # MatMul: fused q|k|v projection of a prefill batch (MFMA-bound) and of a decode step (HBM-bound)
     N = (Hq + 2 * Hkv) * D
     dw, w = dev((N, hidden), 1.0 / 64)

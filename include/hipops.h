@@ -1,6 +1,7 @@
 /*
  * hipops - thin C ABI over the operators that stand either side of attention in a decoder layer
- * on MI355X (gfx950): RMS normalisation, rotary position embedding, MatMul, Gather, Concat.
+ * on MI355X (gfx950): RMS normalisation, rotary position embedding, MatMul, Gather, Concat and the
+ * gated MLP's Swish, Multiply and GLU.
  *
  * Same conventions as hipattn.h, whose status codes, dtype codes and stream type it uses: plain C,
  * device pointers of the current HIP device, asynchronous on the given stream, nothing allocated
@@ -20,7 +21,7 @@ extern "C" {
 #endif
 
 #define HIPOPS_VERSION_MAJOR 0
-#define HIPOPS_VERSION_MINOR 1
+#define HIPOPS_VERSION_MINOR 2
 
 const char* hipops_last_error_string(void);
 int hipops_version(void); /* major * 1000 + minor */
@@ -99,6 +100,26 @@ typedef struct hipops_matmul_desc {
 hipattn_status hipops_matmul_workspace_size(const hipops_matmul_desc* desc, size_t* bytes);
 hipattn_status hipops_matmul(const hipops_matmul_desc* desc, const void* device_a, const void* device_b,
                              void* device_c, void* device_workspace, size_t workspace_bytes, hipattn_stream stream);
+
+/* ---- gated MLP pieces: Swish, Multiply, GLU --------------------------------------------------
+ * hipops_swish:    out = x / (1 + exp(-beta x))   SwishOp (src/ops/swish.cpp:41-59,
+ *                  src/kernels/swish.cu:17-19), beta from the operator's second input (default 1).
+ * hipops_multiply: out = a * b, equal shapes       MultiplyOp (src/ops/multiply.cpp:43 over
+ *                  src/kernels/details/elementwise_binary.cuh:24-46, without broadcasting).
+ * hipops_glu:      OpenVINO's fused gated linear unit (internal operator GLU, the fusion of
+ *                  VariadicSplit + Swish/Gelu + Multiply; the reference would run the three):
+ *                  x is [rows, 2 * width]; out[r, i] = act(x[r, g + i]) * x[r, u + i] with
+ *                  g = gate_first ? 0 : width and u = width - g, act one of HIPOPS_GLU_*.
+ * All three: fp32 arithmetic, one rounding to `dtype` (HIPATTN_F32 / F16 / BF16). */
+#define HIPOPS_GLU_SWISH 0
+#define HIPOPS_GLU_GELU 1      /* x * 0.5 (1 + erf(x / sqrt 2)) */
+#define HIPOPS_GLU_GELU_TANH 2 /* x * 0.5 (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))) */
+hipattn_status hipops_swish(const void* device_x, void* device_out, int64_t count, float beta, int dtype,
+                            hipattn_stream stream);
+hipattn_status hipops_multiply(const void* device_a, const void* device_b, void* device_out, int64_t count, int dtype,
+                               hipattn_stream stream);
+hipattn_status hipops_glu(const void* device_x, void* device_out, int64_t rows, int64_t width, int activation,
+                          int gate_first, int dtype, hipattn_stream stream);
 
 /* ---- Gather -----------------------------------------------------------------------------
  * Gather (opset 1/7/8) with batch_dims, as GatherOp sets it up (src/ops/gather.cpp:60-127) and

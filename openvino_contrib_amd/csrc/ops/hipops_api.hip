@@ -71,3 +71,17 @@ HIPOPS_API hipattn_status hipops_concat(const void* const* inputs, const int64_t
                                         void* out, hipattn_stream stream) {
     return guarded("hipops_concat", [&] { return concat(inputs, axis_bytes, num_inputs, outer, out, (hipStream_t)stream); });
 }
+
+HIPOPS_API hipattn_status hipops_swish(const void* x, void* out, int64_t count, float beta, int dtype, hipattn_stream stream) {
+    return guarded("hipops_swish", [&] { return swish(x, out, count, beta, dtype, (hipStream_t)stream); });
+}
+
+HIPOPS_API hipattn_status hipops_multiply(const void* a, const void* b, void* out, int64_t count, int dtype,
+                                          hipattn_stream stream) {
+    return guarded("hipops_multiply", [&] { return multiply(a, b, out, count, dtype, (hipStream_t)stream); });
+}
+
+HIPOPS_API hipattn_status hipops_glu(const void* x, void* out, int64_t rows, int64_t width, int activation, int gate_first,
+                                     int dtype, hipattn_stream stream) {
+    return guarded("hipops_glu", [&] { return glu(x, out, rows, width, activation, gate_first, dtype, (hipStream_t)stream); });
+}

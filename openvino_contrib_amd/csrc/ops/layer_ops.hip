@@ -267,6 +267,66 @@ __global__ __launch_bounds__(256) void rope_scalar_kernel(RopeParams p) {
     }
 }
 
+// ------------------------------------------------------------------------------ Swish, Multiply, GLU
+__device__ __forceinline__ float activate(float x, int activation, float beta) {
+    switch (activation) {
+        case HIPOPS_GLU_GELU: return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+        case HIPOPS_GLU_GELU_TANH: return 0.5f * x * (1.0f + tanhf(0.79788456080286536f * (x + 0.044715f * x * x * x)));
+        default: return x / (1.0f + __expf(-beta * x));
+    }
+}
+
+struct EltwiseParams {
+    const void* a;  // x (swish), a (multiply), the gate half's row 0 (glu)
+    const void* b;  // multiply: b; glu: the other half's row 0
+    void* out;
+    int64_t count;      // elements of out
+    int64_t width;      // glu: elements per output row (input rows are twice as long)
+    int op;             // 0 swish, 1 multiply, 2 glu
+    int activation;
+    float beta;
+    int dtype;
+};
+
+// eight output elements per lane
+__global__ __launch_bounds__(256) void eltwise_vec_kernel(EltwiseParams p) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i >= p.count) return;
+    int64_t ia = i;
+    if (p.op == 2) {  // row r of the output lies in row r of a 2 * width wide input
+        const int64_t r = i / p.width;
+        ia = r * 2 * p.width + (i - r * p.width);
+    }
+    const Float8 x = load8(p.a, ia, p.dtype);
+    Float8 o;
+    if (p.op == 0) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) o.v[k] = activate(x.v[k], HIPOPS_GLU_SWISH, p.beta);
+    } else {
+        const Float8 y = load8(p.b, ia, p.dtype);
+#pragma unroll
+        for (int k = 0; k < 8; k++) o.v[k] = (p.op == 1 ? x.v[k] : activate(x.v[k], p.activation, 1.0f)) * y.v[k];
+    }
+    store8(p.out, i, p.dtype, o);
+}
+
+__global__ __launch_bounds__(256) void eltwise_scalar_kernel(EltwiseParams p) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= p.count) return;
+    int64_t ia = i;
+    if (p.op == 2) {
+        const int64_t r = i / p.width;
+        ia = r * 2 * p.width + (i - r * p.width);
+    }
+    const float x = load_scalar(p.a, ia, p.dtype);
+    float o;
+    if (p.op == 0)
+        o = activate(x, HIPOPS_GLU_SWISH, p.beta);
+    else
+        o = (p.op == 1 ? x : activate(x, p.activation, 1.0f)) * load_scalar(p.b, ia, p.dtype);
+    store_scalar(p.out, i, p.dtype, o);
+}
+
 // ------------------------------------------------------------------------------ Gather / Concat
 template <typename V>
 __device__ __forceinline__ V zero_of() {
@@ -395,6 +455,59 @@ hipattn_status rope(const hipops_rope_desc* d, const void* x, const void* cos, c
         hipLaunchKernelGGL(rope_scalar_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
     }
     return launched("rope");
+}
+
+hipattn_status swish(const void* x, void* out, int64_t count, float beta, int dtype, hipStream_t stream) {
+    if (count < 0) return fail(HIPATTN_INVALID_ARGUMENT, "swish: negative count");
+    if (!float_dtype(dtype)) return fail(HIPATTN_UNSUPPORTED, "swish: dtype must be f32, f16 or bf16");
+    if (count == 0) return HIPATTN_OK;
+    if (!x || !out) return fail(HIPATTN_INVALID_ARGUMENT, "swish: null pointer");
+    EltwiseParams p{x, nullptr, out, count, 0, 0, HIPOPS_GLU_SWISH, beta, dtype};
+    const bool vec = count % 8 == 0 && aligned(x, 16) && aligned(out, 16);
+    const int64_t items = vec ? count / 8 : count;
+    if (blocks_for(items) > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "swish: too many elements for one launch");
+    if (vec)
+        hipLaunchKernelGGL(eltwise_vec_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(eltwise_scalar_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
+    return launched("swish");
+}
+
+hipattn_status multiply(const void* a, const void* b, void* out, int64_t count, int dtype, hipStream_t stream) {
+    if (count < 0) return fail(HIPATTN_INVALID_ARGUMENT, "multiply: negative count");
+    if (!float_dtype(dtype)) return fail(HIPATTN_UNSUPPORTED, "multiply: dtype must be f32, f16 or bf16");
+    if (count == 0) return HIPATTN_OK;
+    if (!a || !b || !out) return fail(HIPATTN_INVALID_ARGUMENT, "multiply: null pointer");
+    EltwiseParams p{a, b, out, count, 0, 1, 0, 1.0f, dtype};
+    const bool vec = count % 8 == 0 && aligned(a, 16) && aligned(b, 16) && aligned(out, 16);
+    const int64_t items = vec ? count / 8 : count;
+    if (blocks_for(items) > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "multiply: too many elements for one launch");
+    if (vec)
+        hipLaunchKernelGGL(eltwise_vec_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(eltwise_scalar_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
+    return launched("multiply");
+}
+
+hipattn_status glu(const void* x, void* out, int64_t rows, int64_t width, int activation, int gate_first, int dtype,
+                   hipStream_t stream) {
+    if (rows < 0 || width <= 0) return fail(HIPATTN_INVALID_ARGUMENT, "glu: rows %lld width %lld", (long long)rows, (long long)width);
+    if (!float_dtype(dtype)) return fail(HIPATTN_UNSUPPORTED, "glu: dtype must be f32, f16 or bf16");
+    if (activation < HIPOPS_GLU_SWISH || activation > HIPOPS_GLU_GELU_TANH) return fail(HIPATTN_INVALID_ARGUMENT, "glu: activation %d", activation);
+    if (rows == 0) return HIPATTN_OK;
+    if (!x || !out) return fail(HIPATTN_INVALID_ARGUMENT, "glu: null pointer");
+    const int esz = dtype == HIPATTN_F32 ? 4 : 2;
+    const char* gate = (const char*)x + (gate_first ? 0 : width * esz);
+    const char* up = (const char*)x + (gate_first ? width * esz : 0);
+    EltwiseParams p{gate, up, out, rows * width, width, 2, activation, 1.0f, dtype};
+    const bool vec = width % 8 == 0 && aligned(x, 16) && aligned(out, 16);
+    const int64_t items = vec ? p.count / 8 : p.count;
+    if (blocks_for(items) > 0x7fffffffLL) return fail(HIPATTN_UNSUPPORTED, "glu: too many elements for one launch");
+    if (vec)
+        hipLaunchKernelGGL(eltwise_vec_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(eltwise_scalar_kernel, dim3((unsigned)blocks_for(items)), dim3(256), 0, stream, p);
+    return launched("glu");
 }
 
 // widest power-of-two piece (<= 16 bytes) that divides every size and address given

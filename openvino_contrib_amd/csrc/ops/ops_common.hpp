@@ -19,6 +19,10 @@ hipattn_status gather(const void* data, const void* indices, void* out, int64_t 
                       int64_t inner_bytes, int64_t num_indices, int index_dtype, hipStream_t stream);
 hipattn_status concat(const void* const* inputs, const int64_t* axis_bytes, int num_inputs, int64_t outer, void* out,
                       hipStream_t stream);
+hipattn_status swish(const void* x, void* out, int64_t count, float beta, int dtype, hipStream_t stream);
+hipattn_status multiply(const void* a, const void* b, void* out, int64_t count, int dtype, hipStream_t stream);
+hipattn_status glu(const void* x, void* out, int64_t rows, int64_t width, int activation, int gate_first, int dtype,
+                   hipStream_t stream);
 hipattn_status matmul_workspace_size(const hipops_matmul_desc* desc, size_t* bytes);
 hipattn_status matmul(const hipops_matmul_desc* desc, const void* a, const void* b, void* c, void* workspace,
                       size_t workspace_bytes, hipStream_t stream);

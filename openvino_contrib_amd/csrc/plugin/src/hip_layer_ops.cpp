@@ -1,12 +1,13 @@
 // Operators either side of attention in a decoder layer: RMS normalisation, rotary position
-// embedding, MatMul, Gather, Concat; each a thin adapter from node + runtime shapes to the C ABI of
-// libhipops (include/hipops.h).
+// embedding, MatMul, Gather, Concat, and the gated MLP's Swish / Multiply / GLU; each a thin adapter
+// from node + runtime shapes to the C ABI of libhipops (include/hipops.h).
 //
 // MatMulOp, GatherOp and ConcatOp follow the reference's operators of the same names
 // (modules/nvidia_plugin/src/ops/matmul.cpp:22-76 and 185-227, src/ops/gather.cpp:27-127,
-// src/ops/concat.cpp:20-102).  RmsOp and RopeOp serve OpenVINO's fused internal operators RMS and
-// RoPE, which the reference would receive unfused (Power / ReduceMean / Sqrt / Multiply, and
-// Slice / Multiply / Concat / Add).  As everywhere in this plugin a constructor that throws is how
+// src/ops/concat.cpp:20-102), SwishOp and MultiplyOp likewise (src/ops/swish.cpp:41-59,
+// src/ops/multiply.cpp:43).  GluOp, RmsOp and RopeOp serve OpenVINO's fused internal operators GLU,
+// RMS and RoPE, which the reference would receive unfused (VariadicSplit / Swish / Multiply,
+// Power / ReduceMean / Sqrt / Multiply, and Slice / Multiply / Concat / Add).  As everywhere in this plugin a constructor that throws is how
 // an unsupported node is reported (src/cuda_plugin.cpp:171-188).
 #include <cstring>
 
@@ -16,6 +17,9 @@
 #include "openvino/op/constant.hpp"
 #include "openvino/op/gather.hpp"
 #include "openvino/op/matmul.hpp"
+#include "openvino/op/multiply.hpp"
+#include "openvino/op/swish.hpp"
+#include "ov_ops/glu.hpp"
 #include "ov_ops/rms.hpp"
 #include "ov_ops/rotary_positional_embeddings.hpp"
 
@@ -375,6 +379,102 @@ private:
     int64_t axis_ = 0;
 };
 
+// ------------------------------------------------------------------------------ Swish, Multiply, GLU
+class SwishOp : public OperationBase {
+public:
+    SwishOp(const CreationContext& ctx, const ov::Node& node, IndexCollection&& in, IndexCollection&& out)
+        : OperationBase(ctx, node, std::move(in), std::move(out)) {
+        const std::string who = "Swish '" + node.get_friendly_name() + "': ";
+        if (node.get_input_size() != 1 && node.get_input_size() != 2) HIP_PLUGIN_THROW(who + "x [, beta] expected");
+        if (!float_dtype(node.get_input_element_type(0), dtype_) || node.get_output_element_type(0) != node.get_input_element_type(0))
+            HIP_PLUGIN_THROW(who + "f32, f16 or bf16 expected, output like input");
+        if (node.get_input_size() == 2) {
+            // beta comes from a Constant, as the reference requires (swish.cpp:19-38)
+            auto c = ov::as_type_ptr<const ov::op::v0::Constant>(node.get_input_node_shared_ptr(1));
+            if (!c || c->get_output_element_type(0) != ov::element::f32 || c->get_byte_size() != 4)
+                HIP_PLUGIN_THROW(who + "beta must be an f32 Constant of one value");
+            std::memcpy(&beta_, c->get_data_ptr(), 4);
+        }
+    }
+    std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
+        return {in.at(0).shape};
+    }
+    void Execute(const InferenceRequestContext& context, Inputs in, Outputs out, const Workbuffers&) const override {
+        HIP_OPS_CHECK(hipops_swish(in[0].device, out[0].device, (int64_t)ov::shape_size(in[0].shape), beta_, dtype_, context.stream.get()));
+    }
+
+private:
+    int dtype_ = 0;
+    float beta_ = 1.0f;
+};
+
+class MultiplyOp : public OperationBase {
+public:
+    MultiplyOp(const CreationContext& ctx, const ov::Node& node, IndexCollection&& in, IndexCollection&& out)
+        : OperationBase(ctx, node, std::move(in), std::move(out)) {
+        const std::string who = "Multiply '" + node.get_friendly_name() + "': ";
+        if (node.get_input_size() != 2) HIP_PLUGIN_THROW(who + "two inputs expected");
+        if (node.get_input_element_type(0) != node.get_input_element_type(1)) HIP_PLUGIN_THROW(who + "mixed input precisions");
+        if (!float_dtype(node.get_input_element_type(0), dtype_)) HIP_PLUGIN_THROW(who + "f32, f16 or bf16 expected");
+        if (!node.get_input_partial_shape(0).compatible(node.get_input_partial_shape(1))) HIP_PLUGIN_THROW(who + "broadcasting is not supported");
+    }
+    std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
+        HIP_PLUGIN_ASSERT(in.at(0).shape == in.at(1).shape,
+                          "Multiply of " + shape_str(in[0].shape) + " and " + shape_str(in[1].shape) + ": broadcasting is not supported");
+        return {in[0].shape};
+    }
+    void Execute(const InferenceRequestContext& context, Inputs in, Outputs out, const Workbuffers&) const override {
+        HIP_OPS_CHECK(hipops_multiply(in[0].device, in[1].device, out[0].device, (int64_t)ov::shape_size(in[0].shape), dtype_,
+                                      context.stream.get()));
+    }
+
+private:
+    int dtype_ = 0;
+};
+
+// act(one half of the last axis) * the other half
+class GluOp : public OperationBase {
+public:
+    GluOp(const CreationContext& ctx, const ov::Node& node, IndexCollection&& in, IndexCollection&& out)
+        : OperationBase(ctx, node, std::move(in), std::move(out)) {
+        const std::string who = "GLU '" + node.get_friendly_name() + "': ";
+        auto glu = ov::as_type<const ov::op::internal::GLU>(&node);
+        HIP_PLUGIN_ASSERT(glu != nullptr, "not a GLU node");
+        if (!float_dtype(node.get_input_element_type(0), dtype_) || node.get_output_element_type(0) != node.get_input_element_type(0))
+            HIP_PLUGIN_THROW(who + "f32, f16 or bf16 expected, output like input");
+        const int64_t rank = (int64_t)node.get_input_partial_shape(0).size();
+        int64_t axis = glu->get_axis();
+        if (axis < 0) axis += rank;
+        if (rank < 1 || axis != rank - 1) HIP_PLUGIN_THROW(who + "the split must be along the last axis");
+        width_ = glu->get_split_lengths();
+        if (width_ <= 0) HIP_PLUGIN_THROW(who + "split_lengths " + std::to_string(width_));
+        switch (glu->get_glu_type()) {
+            case ov::op::internal::GLU::GluType::Swish: activation_ = HIPOPS_GLU_SWISH; break;
+            case ov::op::internal::GLU::GluType::Gelu: activation_ = HIPOPS_GLU_GELU; break;
+            case ov::op::internal::GLU::GluType::Gelu_Tanh: activation_ = HIPOPS_GLU_GELU_TANH; break;
+            default: HIP_PLUGIN_THROW(who + "unknown activation");
+        }
+        if (glu->get_split_to_glu_idx() > 1) HIP_PLUGIN_THROW(who + "split_to_glu_idx must be 0 or 1");
+        gate_first_ = glu->get_split_to_glu_idx() == 0;
+    }
+    std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
+        ov::Shape out = in.at(0).shape;
+        HIP_PLUGIN_ASSERT(!out.empty() && out.back() == (size_t)(2 * width_),
+                          "GLU of " + shape_str(out) + " with halves of " + std::to_string(width_));
+        out.back() = (size_t)width_;
+        return {out};
+    }
+    void Execute(const InferenceRequestContext& context, Inputs in, Outputs out, const Workbuffers&) const override {
+        const int64_t rows = (int64_t)(ov::shape_size(in[0].shape) / (size_t)(2 * width_));
+        HIP_OPS_CHECK(hipops_glu(in[0].device, out[0].device, rows, width_, activation_, gate_first_, dtype_, context.stream.get()));
+    }
+
+private:
+    int dtype_ = 0, activation_ = 0;
+    int64_t width_ = 0;
+    bool gate_first_ = true;
+};
+
 }  // namespace
 
 }  // namespace hip_gpu
@@ -382,6 +482,9 @@ private:
 
 using ov::hip_gpu::ConcatOp;
 using ov::hip_gpu::GatherOp;
+using ov::hip_gpu::GluOp;
+using ov::hip_gpu::MultiplyOp;
+using ov::hip_gpu::SwishOp;
 using ov::hip_gpu::MatMulOp;
 using ov::hip_gpu::RmsOp;
 using ov::hip_gpu::RopeOp;
@@ -390,3 +493,6 @@ HIP_OPERATION_REGISTER(RopeOp, RoPE)
 HIP_OPERATION_REGISTER(MatMulOp, MatMul)
 HIP_OPERATION_REGISTER(GatherOp, Gather)
 HIP_OPERATION_REGISTER(ConcatOp, Concat)
+HIP_OPERATION_REGISTER(SwishOp, Swish)
+HIP_OPERATION_REGISTER(MultiplyOp, Multiply)
+HIP_OPERATION_REGISTER(GluOp, GLU)

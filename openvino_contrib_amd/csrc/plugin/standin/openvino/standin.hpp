@@ -731,7 +731,63 @@ public:
 };
 }  // namespace v8
 
+namespace v4 {
+// x [, beta]: x / (1 + exp(-beta x))
+class Swish : public Node {
+public:
+    OPENVINO_OP("Swish", "opset4")
+    explicit Swish(const OutputVector& args) : Node(args) {
+        OPENVINO_ASSERT(args.size() == 1 || args.size() == 2, "Swish takes x [, beta]");
+        set_output_type(0, args[0].get_element_type(), args[0].get_partial_shape());
+    }
+};
+}  // namespace v4
+
+namespace v1 {
+class Multiply : public Node {
+public:
+    OPENVINO_OP("Multiply", "opset1")
+    Multiply(const Output<Node>& a, const Output<Node>& b) : Node(OutputVector{a, b}) {
+        set_output_type(0, a.get_element_type(), a.get_partial_shape());
+    }
+};
+}  // namespace v1
+
 namespace internal {
+// data split in two along `axis` (split_lengths wide each): act(half split_to_glu_idx) * other half
+class GLU : public Node {
+public:
+    OPENVINO_OP("GLU", "ie_internal_opset")
+    enum GluType { Swish = 0, Gelu, Gelu_Tanh };
+    GLU(const Output<Node>& data, int64_t axis, int64_t split_lengths, const GluType glu_type, const size_t split_to_glu_idx,
+        const element::Type output_type = element::dynamic)
+        : Node(OutputVector{data}), axis_(axis), split_lengths_(split_lengths), glu_type_(glu_type),
+          split_to_glu_idx_(split_to_glu_idx), output_type_(output_type) {
+        const PartialShape& ps = data.get_partial_shape();
+        std::vector<Dimension> dims(ps.begin(), ps.end());
+        const int64_t ax = axis < 0 ? axis + (int64_t)dims.size() : axis;
+        OPENVINO_ASSERT(ax >= 0 && ax < (int64_t)dims.size(), "GLU axis out of range");
+        dims[ax] = Dimension(split_lengths);
+        set_output_type(0, output_type == element::dynamic ? data.get_element_type() : output_type, PartialShape(dims));
+    }
+    int64_t get_axis() const { return axis_; }
+    int64_t get_split_lengths() const { return split_lengths_; }
+    GluType get_glu_type() const { return glu_type_; }
+    size_t get_split_to_glu_idx() const { return split_to_glu_idx_; }
+    const element::Type& get_output_type() const { return output_type_; }
+    std::map<std::string, std::string> standin_attributes() const override {
+        return {{"axis", std::to_string(axis_)}, {"split_lengths", std::to_string(split_lengths_)},
+                {"glu_type", std::to_string((int)glu_type_)}, {"split_to_glu_idx", std::to_string(split_to_glu_idx_)},
+                {"output_type", output_type_.get_type_name()}};
+    }
+
+private:
+    int64_t axis_, split_lengths_;
+    GluType glu_type_;
+    size_t split_to_glu_idx_;
+    element::Type output_type_;
+};
+
 // data, gamma; out = data / sqrt(mean(data^2, last axis) + epsilon) * gamma
 class RMS : public Node {
 public:
@@ -1247,6 +1303,15 @@ public:
                 n = a;
             } else if (type == "Add") {
                 n = std::make_shared<op::v1::Add>(inputs.at(0), inputs.at(1));
+            } else if (type == "Swish") {
+                n = std::make_shared<op::v4::Swish>(inputs);
+            } else if (type == "Multiply") {
+                n = std::make_shared<op::v1::Multiply>(inputs.at(0), inputs.at(1));
+            } else if (type == "GLU") {
+                n = std::make_shared<op::internal::GLU>(
+                    inputs.at(0), std::stoll(attrs.at("axis")), std::stoll(attrs.at("split_lengths")),
+                    (op::internal::GLU::GluType)std::stoi(attrs.at("glu_type")), (size_t)std::stoull(attrs.at("split_to_glu_idx")),
+                    attrs.count("output_type") ? element::type_from_name(attrs["output_type"]) : element::dynamic);
             } else if (type == "MatMul") {
                 n = std::make_shared<op::v0::MatMul>(inputs.at(0), inputs.at(1), attrs["transpose_a"] == "true",
                                                      attrs["transpose_b"] == "true");

@@ -57,6 +57,9 @@ SYMBOLS = {
     "hipops_rope": (_i, [_P(RopeDesc), _vp, _vp, _vp, _vp, _vp, _vp]),
     "hipops_matmul_workspace_size": (_i, [_P(MatmulDesc), _P(_sz)]),
     "hipops_matmul": (_i, [_P(MatmulDesc), _vp, _vp, _vp, _vp, _sz, _vp]),
+    "hipops_swish": (_i, [_vp, _vp, _i64, _f, _i, _vp]),
+    "hipops_multiply": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
+    "hipops_glu": (_i, [_vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "hipops_gather": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _vp]),
     "hipops_concat": (_i, [_P(_vp), _P(_i64), _i, _i64, _vp, _vp]),
 }
@@ -117,6 +120,21 @@ def matmul_workspace_size(desc):
 def matmul(desc, a, b, c, workspace=None, stream=None):
     check(lib().hipops_matmul(ctypes.byref(desc), _ptr(a), _ptr(b), _ptr(c), _ptr(workspace),
                               workspace.nbytes if workspace is not None else 0, _h(stream)))
+
+
+GLU_SWISH, GLU_GELU, GLU_GELU_TANH = 0, 1, 2
+
+
+def swish(x, out, count, dtype, beta=1.0, stream=None):
+    check(lib().hipops_swish(_ptr(x), _ptr(out), count, beta, dtype, _h(stream)))
+
+
+def multiply(a, b, out, count, dtype, stream=None):
+    check(lib().hipops_multiply(_ptr(a), _ptr(b), _ptr(out), count, dtype, _h(stream)))
+
+
+def glu(x, out, rows, width, dtype, activation=GLU_SWISH, gate_first=True, stream=None):
+    check(lib().hipops_glu(_ptr(x), _ptr(out), rows, width, activation, int(gate_first), dtype, _h(stream)))
 
 
 def gather(data, indices, out, batch, outer, axis_dim, inner_bytes, num_indices, index_dtype, stream=None):

@@ -27,6 +27,9 @@
  *                         hand-written cases.
  *   oracle_concat_bytes   Concat along an axis (src/ops/concat.cpp:31-56).  Pinned by
  *                         numpy.concatenate.
+ *   oracle_swish_f32 /    Swish (src/ops/swish.cpp:41-59) and OpenVINO's fused gated linear unit
+ *   oracle_glu_f32        act(gate) * up with Swish, Gelu (erf) or Gelu (tanh).  Pinned by
+ *                         torch.nn.functional.silu / gelu in fp64 (fixtures) and the explicit product.
  */
 #include <math.h>
 #include <stdint.h>
@@ -125,4 +128,28 @@ ORACLE_API void oracle_concat_bytes(const uint8_t* const* inputs, const int64_t*
             offset += axis_bytes[i];
         }
     }
+}
+
+/* Swish x / (1 + exp(-beta x)) (src/ops/swish.cpp:41-59, src/kernels/swish.cu:17-19 of the reference);
+ * activation 1: Gelu with erf, 2: Gelu with the tanh approximation (OpenVINO's Gelu modes ERF and
+ * TANH).  Pinned by torch.nn.functional.silu / gelu fixtures in fp64. */
+static double oracle_activate(double x, int activation, double beta) {
+    switch (activation) {
+        case 1: return 0.5 * x * (1.0 + erf(x * 0.70710678118654752440));
+        case 2: return 0.5 * x * (1.0 + tanh(0.79788456080286535588 * (x + 0.044715 * x * x * x)));
+        default: return x / (1.0 + exp(-beta * x));
+    }
+}
+
+ORACLE_API void oracle_swish_f32(const float* x, float* out, int64_t count, float beta) {
+    for (int64_t i = 0; i < count; i++) out[i] = (float)oracle_activate(x[i], 0, beta);
+}
+
+/* out[r, i] = act(x[r, g + i]) * x[r, u + i], x of 2 * width columns: OpenVINO's fused gated linear
+ * unit.  Pinned by act(gate) * up from the torch fixtures and by the plain product for multiply. */
+ORACLE_API void oracle_glu_f32(const float* x, float* out, int64_t rows, int64_t width, int activation, int gate_first) {
+    const int64_t g = gate_first ? 0 : width, u = width - g;
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t i = 0; i < width; i++)
+            out[r * width + i] = (float)(oracle_activate(x[r * 2 * width + g + i], activation, 1.0) * (double)x[r * 2 * width + u + i]);
 }

@@ -70,6 +70,10 @@ def lib():
         L.oracle_rope_f32.restype = None
         L.oracle_matmul_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i32, i32, i64, i64]
         L.oracle_matmul_f32.restype = None
+        L.oracle_swish_f32.argtypes = [vp, vp, i64, f32]
+        L.oracle_swish_f32.restype = None
+        L.oracle_glu_f32.argtypes = [vp, vp, i64, i64, i32, i32]
+        L.oracle_glu_f32.restype = None
         L.oracle_gather_bytes.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64]
         L.oracle_gather_bytes.restype = None
         L.oracle_concat_bytes.argtypes = [vp, vp, i32, i64, vp]
@@ -318,4 +322,20 @@ def concat(arrays, axis):
     out = np.empty(shape, first.dtype)
     ptrs = (ctypes.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
     lib().oracle_concat_bytes(ptrs, _p(widths), len(arrays), outer, _p(out))
+    return out
+
+
+def swish(x, beta=1.0):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().oracle_swish_f32(_p(x), _p(out), x.size, float(beta))
+    return out
+
+
+def glu(x, activation=0, gate_first=True):
+    """x [..., 2 * width] -> act(gate half) * other half; activation 0 swish, 1 gelu (erf), 2 gelu (tanh)."""
+    x = _c(x, np.float32)
+    width = x.shape[-1] // 2
+    out = np.empty(x.shape[:-1] + (width,), np.float32)
+    lib().oracle_glu_f32(_p(x), _p(out), x.size // (2 * width), width, int(activation), int(bool(gate_first)))
     return out

@@ -1,7 +1,8 @@
 """Writes tests/golden/layer_ops_golden.npz: inputs and outputs of library routines for the
 operators around attention - torch.nn.functional.rms_norm on the CPU in fp64, and the rotary
 position embedding helpers of the transformers library (LLaMA's rotate-half form, GPT-J's
-adjacent-pair form) in fp64, whole-head and partial (the first rotary_ndims elements of a head).
+adjacent-pair form) in fp64, whole-head and partial (the first rotary_ndims elements of a head),
+and torch's silu / gelu (erf and tanh forms) in fp64 for the gated MLP.
 
 Nothing from the reference is imported or run.  Usage: python tests/golden/make_layer_ops_golden.py
 """
@@ -50,6 +51,14 @@ def main():
         o = torch.cat([rotated, xd[:, :, rot:]], dim=-1)
         out[name + "/x"], out[name + "/cos"], out[name + "/sin"] = x.numpy(), cos.float().numpy(), sin.float().numpy()
         out[name + "/out"] = o.float().numpy()
+    # activations of the gated MLP: silu with a beta, gelu in both of OpenVINO's modes
+    g = torch.Generator().manual_seed(5300)
+    x = 4.0 * torch.randn(257, generator=g, dtype=torch.float32)
+    out["act/x"] = x.numpy()
+    out["act/silu"] = F.silu(x.double()).float().numpy()
+    out["act/silu_beta1p7"] = (x.double() * torch.sigmoid(1.7 * x.double())).float().numpy()
+    out["act/gelu_erf"] = F.gelu(x.double()).float().numpy()
+    out["act/gelu_tanh"] = F.gelu(x.double(), approximate="tanh").float().numpy()
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "layer_ops_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")

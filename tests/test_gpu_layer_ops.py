@@ -281,3 +281,51 @@ def test_concat(hip, ops, oracle, shape, axis, widths, itemsize):
     do.fill(0xEE)
     ops.concat(bufs, [w * tail for w in widths], outer, do)
     assert np.array_equal(do.download(dt, ref.shape), ref)
+
+
+# ------------------------------------------------------------------------------ Swish, Multiply, GLU
+@pytest.mark.parametrize("count", [1, 8, 37, 4096, 1_000_003])
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+def test_swish_and_multiply(hip, ops, oracle, count, dtype):
+    rng = np.random.default_rng(count)
+    print("[swish, multiply]", count, dtype, flush=True)
+    da, a = upload(hip, rng.standard_normal(count) * 3, dtype)
+    db, b = upload(hip, rng.standard_normal(count), dtype)
+    do = hip.DeviceBuffer(count * hip.DTYPE_BYTES[dtype])
+    ops.swish(da, do, count, dtype)
+    assert scaled_error(download(hip, do, dtype, (count,)), oracle.swish(a)) <= ROUND[dtype]
+    ops.swish(da, do, count, dtype, beta=1.7)
+    assert scaled_error(download(hip, do, dtype, (count,)), oracle.swish(a, 1.7)) <= ROUND[dtype]
+    ops.multiply(da, db, do, count, dtype)
+    assert scaled_error(download(hip, do, dtype, (count,)), a * b) <= ROUND[dtype]
+    ops.multiply(da, db, da, count, dtype)  # in place
+    assert scaled_error(download(hip, da, dtype, (count,)), a * b) <= ROUND[dtype]
+
+
+@pytest.mark.parametrize("rows,width", [(1, 8), (5, 37), (64, 14336), (3, 11008), (4100, 128)])
+@pytest.mark.parametrize("activation", [0, 1, 2])
+@pytest.mark.parametrize("gate_first", [True, False])
+@pytest.mark.parametrize("dtype", [F32, BF16, F16])
+def test_glu(hip, ops, oracle, rows, width, activation, gate_first, dtype):
+    if rows * width > 500_000 and dtype != BF16:
+        pytest.skip("the large shapes run once, in bf16")
+    rng = np.random.default_rng(rows + width + activation)
+    print("[glu]", rows, width, activation, gate_first, dtype, flush=True)
+    dx, x = upload(hip, rng.standard_normal((rows, 2 * width)) * 2, dtype)
+    do = hip.DeviceBuffer(rows * width * hip.DTYPE_BYTES[dtype])
+    ops.glu(dx, do, rows, width, dtype, activation, gate_first)
+    ref = oracle.glu(x, activation, gate_first)
+    assert scaled_error(download(hip, do, dtype, (rows, width)), ref) <= ROUND[dtype]
+
+
+def test_eltwise_rejects_bad_arguments(hip, ops):
+    buf = hip.DeviceBuffer(256)
+    for call in (lambda: ops.swish(buf, buf, -1, F16), lambda: ops.multiply(buf, None, buf, 8, F16),
+                 lambda: ops.glu(buf, buf, 2, 0, F16), lambda: ops.glu(buf, buf, 2, 8, F16, activation=7)):
+        with pytest.raises(ops.HipOpsError) as e:
+            call()
+        assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.swish(buf, buf, 8, W.U8)
+    assert e.value.status == hip.UNSUPPORTED
+    ops.swish(None, None, 0, F16)

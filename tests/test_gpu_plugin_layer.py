@@ -407,3 +407,136 @@ def test_paged_attention_decode_steps_replay_a_graph(hip, oracle):
         assert np.array_equal(o, outs[0])
     assert int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")) == 1 and int(compiled.get_property("HIP_GRAPH_LAUNCHES")) == 3
     np.testing.assert_array_equal(kc.download(np.uint8, case["key_cache"].shape), okc)
+
+
+# ------------------------------------------------------------------------------ a whole small decoder
+class TinyDecoder:
+    """A LLaMA-shaped decoder of `layers` layers as one model in the text form: token ids -> Gather
+    (embedding) -> per layer [RMS -> q/k/v MatMul -> RoPE -> PagedAttentionExtension -> o MatMul ->
+    Add, RMS -> gate|up MatMul -> GLU -> down MatMul -> Add] -> RMS -> lm_head MatMul.  Weights are
+    Constants (uploaded once per request); every layer has a paged KV cache of its own, bound as
+    device tensors; the index tensors are shared by the layers."""
+
+    def __init__(self, rng, layers=2, hidden=256, Hq=2, Hkv=1, D=128, ffn=512, vocab=300, bs=32):
+        self.layers, self.hidden, self.Hq, self.Hkv, self.D, self.ffn, self.vocab, self.bs = layers, hidden, Hq, Hkv, D, ffn, vocab, bs
+        w = lambda *shape: storage(rng.standard_normal(shape) / np.sqrt(shape[-1]), BF16)
+        self.embed = storage(rng.standard_normal((vocab, hidden)), BF16)
+        self.final_gamma = storage(1.0 + 0.1 * rng.standard_normal(hidden), BF16)
+        self.lm_head = w(vocab, hidden)
+        self.layer_w = [{"g1": storage(1.0 + 0.1 * rng.standard_normal(hidden), BF16), "wq": w(Hq * D, hidden),
+                         "wk": w(Hkv * D, hidden), "wv": w(Hkv * D, hidden), "wo": w(hidden, Hq * D),
+                         "g2": storage(1.0 + 0.1 * rng.standard_normal(hidden), BF16), "wgu": w(2 * ffn, hidden),
+                         "wd": w(hidden, ffn)} for _ in range(layers)]
+
+    def graph(self):
+        g = P.GraphText("tiny_decoder")
+        ids = g.parameter("ids", P.I32, [-1])
+        cos_p = g.parameter("cos", F32, [-1, self.D])
+        sin_p = g.parameter("sin", F32, [-1, self.D])
+        pos_p = g.parameter("positions", P.I32, [-1])
+        idx = [g.parameter(n, P.I32, [-1]) for n in ("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")]
+        scale_p = g.parameter("scale", F32, [-1])
+        win_p = g.parameter("sliding_window", P.I32, [-1])
+        alibi_p = g.parameter("alibi_slopes", F32, [0])
+        mcl_p = g.parameter("max_context_len", P.I32, [-1])
+        caches = [(g.parameter("key_cache.%d" % l, F16, [-1, self.Hkv, self.bs, self.D]),
+                   g.parameter("value_cache.%d" % l, F16, [-1, self.Hkv, self.bs, self.D])) for l in range(self.layers)]
+        c = lambda name, pair: g.constant(name, pair[0], "bf16")
+        axis = g.constant("axis", np.array(0, np.int64), "i64")
+        h = g.add("Gather", "embed", [c("embed_w", self.embed), ids, axis], batch_dims=0)
+        mm = lambda name, x, wt: g.add("MatMul", name, [x, wt], transpose_a=False, transpose_b=True)
+        for l, lw in enumerate(self.layer_w):
+            n1 = g.add("RMS", "norm1.%d" % l, [h, c("g1.%d" % l, lw["g1"])], epsilon=1e-5, output_type="dynamic")
+            q = mm("q.%d" % l, n1, c("wq.%d" % l, lw["wq"]))
+            k = mm("k.%d" % l, n1, c("wk.%d" % l, lw["wk"]))
+            v = mm("v.%d" % l, n1, c("wv.%d" % l, lw["wv"]))
+            rope = dict(head_size=self.D, rotary_ndims=self.D, gather_position_arg_id=3)
+            qr = g.add("RoPE", "q_rope.%d" % l, [q, cos_p, sin_p, pos_p], head_cnt=self.Hq, **rope)
+            kr = g.add("RoPE", "k_rope.%d" % l, [k, cos_p, sin_p, pos_p], head_cnt=self.Hkv, **rope)
+            pa = g.add("PagedAttentionExtension", "attention.%d" % l,
+                       [qr, kr, v, caches[l][0], caches[l][1]] + idx + [scale_p, win_p, alibi_p, mcl_p])
+            h = g.add("Add", "res1.%d" % l, [mm("o.%d" % l, pa, c("wo.%d" % l, lw["wo"])), h])
+            n2 = g.add("RMS", "norm2.%d" % l, [h, c("g2.%d" % l, lw["g2"])], epsilon=1e-5, output_type="dynamic")
+            gu = mm("gate_up.%d" % l, n2, c("wgu.%d" % l, lw["wgu"]))
+            act = g.add("GLU", "glu.%d" % l, [gu], axis=-1, split_lengths=self.ffn, glu_type=0, split_to_glu_idx=0, output_type="dynamic")
+            h = g.add("Add", "res2.%d" % l, [mm("down.%d" % l, act, c("wd.%d" % l, lw["wd"])), h])
+        nf = g.add("RMS", "final_norm", [h, c("final_gamma", self.final_gamma)], epsilon=1e-5, output_type="dynamic")
+        g.result("logits", mm("lm_head", nf, c("lm_head_w", self.lm_head)))
+        return g
+
+    def reference(self, oracle, ids, cos, sin, positions, cases):
+        """The chain of oracle functions with a bf16 rounding behind every operator; cases[l] holds
+        layer l's cache and tables (the caches are updated in place, as the operator does)."""
+        r = lambda a: oracle.round_to(a, BF16)
+        mm = lambda x, wt: r(oracle.matmul(x, wt[1], False, True))
+        T = len(ids)
+        h = self.embed[1][ids]
+        for lw, case in zip(self.layer_w, cases):
+            n1 = r(oracle.rms_norm(h, lw["g1"][1], 1e-5))
+            q, k, v = mm(n1, lw["wq"]), mm(n1, lw["wk"]), mm(n1, lw["wv"])
+            qr = r(oracle.rope(q.reshape(T, self.Hq, self.D), cos, sin, positions)).reshape(T, -1)
+            kr = r(oracle.rope(k.reshape(T, self.Hkv, self.D), cos, sin, positions)).reshape(T, -1)
+            att = r(oracle.paged_attention(qr, kr, v, case["key_cache"], case["value_cache"], F16, case["past_lens"],
+                                           case["subsequence_begins"], case["block_indices"], case["block_indices_begins"],
+                                           self.Hq, self.Hkv, self.D, self.bs))
+            h = r(mm(att, lw["wo"]) + h)
+            n2 = r(oracle.rms_norm(h, lw["g2"][1], 1e-5))
+            h = r(mm(r(oracle.glu(mm(n2, lw["wgu"]), 0, True)), lw["wd"]) + h)
+        return mm(r(oracle.rms_norm(h, self.final_gamma[1], 1e-5)), self.lm_head)
+
+
+def test_a_whole_small_decoder_runs_on_the_device(hip, oracle):
+    """Two decoder layers, embedding to logits, one mixed prefill + decode step on device "HIP": 35
+    operators, one infer, against the oracle chain; then the same step twice more, which records and
+    replays a graph (the caches are rewritten with the same rows, so the logits repeat)."""
+    rng = np.random.default_rng(12)
+    model = TinyDecoder(rng)
+    seqs = [(0, 40), (70, 1), (33, 1), (5, 20)]
+    cases = [W.make_paged_case(120 + l, seqs, model.Hq, model.Hkv, model.D, model.bs, BF16, BF16, F16) for l in range(model.layers)]
+    for c in cases[1:]:  # one set of tables for all layers; every pool is random throughout, so any table fits it
+        assert c["key_cache"].shape == cases[0]["key_cache"].shape
+        for n in ("past_lens", "subsequence_begins", "block_indices", "block_indices_begins"):
+            c[n] = cases[0][n]
+    T = cases[0]["q"].shape[0]
+    ids = rng.integers(0, model.vocab, T).astype(np.int32)
+    positions = np.concatenate([np.arange(p, p + n) for p, n in seqs]).astype(np.int32)
+    cos, sin = rope_tables(int(positions.max()) + 1, model.D)
+    plugin = P.Plugin()
+    g = model.graph()
+    supported = set(plugin.query_model(g.model()))
+    assert {"embed", "glu.0", "glu.1", "attention.1", "lm_head", "res2.1"} <= supported
+    compiled = plugin.compile_model(g.model())
+    req = compiled.create_infer_request()
+    dev_caches = [(hip.DeviceBuffer.from_numpy(c["key_cache"]), hip.DeviceBuffer.from_numpy(c["value_cache"])) for c in cases]
+    case = cases[0]
+    host = {"ids": (ids, P.I32), "cos": (cos, F32), "sin": (sin, F32), "positions": (positions, P.I32),
+            "past_lens": (case["past_lens"], P.I32), "subsequence_begins": (case["subsequence_begins"], P.I32),
+            "block_indices": (case["block_indices"], P.I32), "block_indices_begins": (case["block_indices_begins"], P.I32),
+            "scale": (np.zeros((0,), np.float32), F32), "sliding_window": (np.array([0], np.int32), P.I32),
+            "alibi_slopes": (np.zeros((0,), np.float32), F32),
+            "max_context_len": (np.array([case["max_context_len"]], np.int32), P.I32)}
+    cache_shape = list(case["key_cache"].shape[:3]) + [model.D]
+    for i, n in enumerate(compiled.input_names()):
+        if n in host:
+            req.set_input(i, *host[n])
+        else:
+            kind, l = n.split(".")
+            req.set_device_input(i, dev_caches[int(l)][0 if kind == "key_cache" else 1].ptr, F16, cache_shape)
+    req.infer()
+    logits, _ = req.output(0)
+    got = H.storage_to_f32(logits, BF16)
+    ref = model.reference(oracle, ids, cos, sin, positions, cases)
+    assert got.shape == ref.shape == (T, model.vocab)
+    err = scaled_error(got, ref)
+    print("tiny decoder: scaled max error of the logits %.4g" % err, flush=True)
+    assert err <= 6e-2  # 35 bf16 roundings deep; a wrong operator anywhere is off by order one
+    # the ranking of the logits is what a sampler sees: the top token agrees wherever the reference's
+    # margin over the runner-up is larger than the error
+    top_ref, top_got = ref.argmax(-1), got.argmax(-1)
+    margin = np.sort(ref, -1)[:, -1] - np.sort(ref, -1)[:, -2]
+    assert np.all((top_ref == top_got) | (margin <= 2 * err * np.maximum(1.0, np.abs(ref).max(-1))))
+    for _ in range(2):
+        req.infer()
+        again, _ = req.output(0)
+        assert np.array_equal(again, logits)
+    assert int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")) == 1 and int(compiled.get_property("HIP_GRAPH_LAUNCHES")) == 2

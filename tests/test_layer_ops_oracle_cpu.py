@@ -118,3 +118,16 @@ def test_concat_matches_numpy(oracle):
             shape[axis] = w
             parts.append(rng.standard_normal(shape).astype(np.float32))
         assert np.array_equal(oracle.concat(parts, axis), np.concatenate(parts, axis))
+
+
+def test_swish_and_glu_match_torch_fixtures(oracle, golden):
+    x = golden["act/x"]
+    np.testing.assert_allclose(oracle.swish(x), golden["act/silu"], rtol=2e-6, atol=1e-7)
+    np.testing.assert_allclose(oracle.swish(x, 1.7), golden["act/silu_beta1p7"], rtol=2e-6, atol=1e-7)
+    up = np.linspace(-2, 3, x.size).astype(np.float32)
+    for act, name in ((0, "silu"), (1, "gelu_erf"), (2, "gelu_tanh")):
+        packed = np.stack([np.concatenate([x, up]), np.concatenate([x[::-1], up])])  # [gate | up]
+        want = np.stack([golden["act/" + name].astype(np.float64) * up, golden["act/" + name][::-1].astype(np.float64) * up])
+        np.testing.assert_allclose(oracle.glu(packed, act, True), want, rtol=3e-6, atol=1e-6)
+        swapped = np.stack([np.concatenate([up, x]), np.concatenate([up, x[::-1]])])     # [up | gate]
+        np.testing.assert_allclose(oracle.glu(swapped, act, False), want, rtol=3e-6, atol=1e-6)

@@ -17,7 +17,7 @@ def declared_functions():
 
 def test_header_and_binding_agree():
     names = declared_functions()
-    assert len(names) == 8
+    assert len(names) == 11
     assert sorted(ops_capi.SYMBOLS) == names
 
 
@@ -37,7 +37,7 @@ def test_struct_layout_matches_header():
 
 def test_validation_needs_no_device():
     L = ops_capi.lib()
-    assert L.hipops_version() == 1
+    assert L.hipops_version() == 2
     n = ctypes.c_size_t(0)
     ok = ops_capi.MatmulDesc(capi.BF16, capi.BF16, 64, 6144, 4096, 1, 0, 1, 0, 0)
     assert L.hipops_matmul_workspace_size(ctypes.byref(ok), ctypes.byref(n)) == capi.OK and n.value == 32 << 20
