@@ -191,10 +191,11 @@ hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q,
  * those blocks (probability zero); the MFMA chunked-prefill kernel redirects them to a valid
  * block, so reads stay inside the cache and the affected rows are unspecified.
  * A mixed batch (single-token and multi-token sequences) with decode_waves == 0 runs its two
- * parts side by side: the call forks from `stream` onto a side stream that the library keeps per
- * device (created by the first such call, default priority, never destroyed) and joins before it
- * returns, so `stream` order is all the caller has to know, also under stream capture (make the
- * first such call on a device outside a capture: creating a stream is not a capturable operation).  The
+ * parts side by side: the call forks from `stream` onto a side stream that the library keeps for
+ * that stream (created by the first such call on it, default priority, destroyed by
+ * hipattn_stream_destroy; the library keeps at most 32, further streams share one) and joins before
+ * it returns, so `stream` order is all the caller has to know, also under stream capture (make the
+ * first such call on a stream outside a capture: creating a stream is not a capturable operation).  The
  * option "mixed_overlap" = 0 (hipattn_set_option) switches that off. */
 enum {
     HIPATTN_PA_SKIP_CACHE_WRITE = 1, /* attention only; k_new / v_new may be NULL */

@@ -219,6 +219,7 @@ HIPATTN_EXPORT hipattn_status hipattn_stream_create(hipattn_stream* stream) {
     return HIPATTN_OK;
 }
 HIPATTN_EXPORT hipattn_status hipattn_stream_destroy(hipattn_stream stream) {
+    hipattn::release_side_stream(as_stream(stream));
     HIP_TRY(hipStreamDestroy(as_stream(stream)));
     return HIPATTN_OK;
 }

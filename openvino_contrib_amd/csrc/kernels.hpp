@@ -143,6 +143,7 @@ hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream);
 bool paged_fast_supported(const PagedParams& p);
 size_t paged_fast_workspace_bytes(const PagedParams& p);
 void paged_fast_plan(PagedParams& p, void* workspace);  // fills chunking fields and workspace pointers
+void release_side_stream(hipStream_t owner);  // drops the side stream mixed batches on `owner` used, if any
 // write == nullptr skips the KV-cache write of the new tokens
 hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
                              const KernelProbe& probe);

@@ -1074,31 +1074,82 @@ hipError_t paged_static_scratch(void** ptr, size_t* bytes) {
     return hipSuccess;
 }
 
-// One side stream and a fork/join pair of events per device, made on first use and kept until the
-// process ends.  The mutex keeps the record/wait pairs of concurrent callers apart.
+// A side stream and a fork/join pair of events per (device, caller's stream), made on the first
+// mixed batch that stream carries, so that mixed batches on different streams do not wait for each
+// other's chunk kernels.  An entry lives until its stream is destroyed through the C ABI
+// (release_side_stream) or the process ends; beyond kMaxSideStreams entries further caller streams
+// share the device's first entry.  The entry's mutex keeps the record/wait pairs of concurrent
+// callers apart.
 struct SideStream {
+    int device = 0;
+    hipStream_t owner = nullptr;
     hipStream_t stream = nullptr;
     hipEvent_t fork = nullptr, join = nullptr;
     std::mutex mutex;
 };
 
-static SideStream* side_stream() {
-    static std::mutex table_mutex;
-    static SideStream* table[64] = {};
+constexpr int kMaxSideStreams = 32;
+static std::mutex g_side_mutex;
+static SideStream* g_side[kMaxSideStreams] = {};
+
+static SideStream* side_stream(hipStream_t owner) {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    std::lock_guard<std::mutex> guard(table_mutex);
-    if (!table[dev]) {
-        SideStream* s = new SideStream;
-        if (hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking) != hipSuccess ||
-            hipEventCreateWithFlags(&s->fork, hipEventDisableTiming) != hipSuccess ||
-            hipEventCreateWithFlags(&s->join, hipEventDisableTiming) != hipSuccess) {
-            delete s;
-            return nullptr;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> guard(g_side_mutex);
+    int free_slot = -1;
+    SideStream* shared = nullptr;
+    for (int i = 0; i < kMaxSideStreams; i++) {
+        SideStream* s = g_side[i];
+        if (!s) {
+            if (free_slot < 0) free_slot = i;
+            continue;
         }
-        table[dev] = s;
+        if (s->device != dev) continue;
+        if (s->owner == owner) return s;
+        if (!shared) shared = s;
     }
-    return table[dev];
+    if (free_slot < 0) return shared;  // table full: share (nullptr if this device has none, the caller reports it)
+    SideStream* s = new SideStream;
+    s->device = dev;
+    s->owner = owner;
+    if (hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&s->fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&s->join, hipEventDisableTiming) != hipSuccess) {
+        if (s->stream) (void)hipStreamDestroy(s->stream);
+        if (s->fork) (void)hipEventDestroy(s->fork);
+        if (s->join) (void)hipEventDestroy(s->join);
+        delete s;
+        return nullptr;
+    }
+    g_side[free_slot] = s;
+    return s;
+}
+
+// Called before a stream is destroyed: whatever its side stream still runs is waited for, then the
+// side stream and its events go.  Streams other callers share through a full table are not owned by
+// the stream being destroyed and stay.
+void release_side_stream(hipStream_t owner) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    SideStream* s = nullptr;
+    {
+        std::lock_guard<std::mutex> guard(g_side_mutex);
+        for (int i = 0; i < kMaxSideStreams; i++)
+            if (g_side[i] && g_side[i]->device == dev && g_side[i]->owner == owner) {
+                s = g_side[i];
+                g_side[i] = nullptr;
+                break;
+            }
+    }
+    if (!s) return;
+    {
+        std::lock_guard<std::mutex> guard(s->mutex);
+        (void)hipStreamSynchronize(s->stream);
+        (void)hipStreamDestroy(s->stream);
+        (void)hipEventDestroy(s->fork);
+        (void)hipEventDestroy(s->join);
+    }
+    delete s;
 }
 
 hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
@@ -1139,7 +1190,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         // chunks' flash kernel, on a side stream, has the others; both only need the prologue's
         // results.  The decode kernel stays on the caller's stream, directly behind the prologue,
         // so that it is dispatched first and gets its compute units at once.
-        SideStream* side = side_stream();
+        SideStream* side = side_stream(stream);
         if (!side) return hipErrorOutOfMemory;
         std::lock_guard<std::mutex> guard(side->mutex);
         if ((e = hipEventRecord(side->fork, stream)) != hipSuccess) return e;

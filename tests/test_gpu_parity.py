@@ -652,8 +652,8 @@ def test_paged_generic_skips_blocks_outside_the_cache(hip, oracle):
 
 
 def test_paged_mixed_batches_from_two_host_threads(hip, oracle):
-    """Mixed-batch calls share one side stream per device; two host threads with a stream, a
-    workspace and tensors of their own each must not disturb each other."""
+    """Every caller stream gets a side stream of its own for the chunk kernel of a mixed batch; two
+    host threads with a stream, a workspace and tensors of their own each must not disturb each other."""
     import threading
 
     announce("paged mixed, two host threads")
@@ -685,6 +685,30 @@ def test_paged_mixed_batches_from_two_host_threads(hip, oracle):
         assert H.max_abs(results[i], refs[i]) <= 2e-3
         devs[i].free()
         streams[i].close()
+
+
+def test_paged_mixed_batches_on_many_short_lived_streams(hip, oracle):
+    """A side stream lives as long as the caller's stream: 40 streams in turn (more than the table
+    of side streams holds), each created, used for one mixed batch and destroyed, and then three
+    streams alive at once, all give the first result bit for bit."""
+    announce("paged mixed, short-lived streams")
+    case = W.make_paged_case(131, [(0, 130), (37, 1), (500, 1), (100, 257), (999, 1)], 16, 4, 128, 32, W.F16, W.F16, W.F16)
+    ref = H.oracle_paged(oracle, case)[0]
+    dev = H.PagedDeviceCase(hip, case)
+    first, _ = dev.run()
+    assert H.max_abs(first, ref) <= 2e-3
+    for _ in range(40):
+        s = hip.Stream()
+        out, _ = dev.run(stream=s)
+        s.close()
+        np.testing.assert_array_equal(out, first)
+    streams = [hip.Stream() for _ in range(3)]
+    for _ in range(2):
+        for s in streams:
+            np.testing.assert_array_equal(dev.run(stream=s)[0], first)
+    for s in streams:
+        s.close()
+    dev.free()
 
 
 @pytest.mark.parametrize("shape", [(6, 2, 64, 16, W.F16, W.F16), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
