@@ -369,10 +369,12 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
         return sum(times) / len(times), len(times)
 
     # HBM bytes per launch from rocprofv3 FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB (recorded, not measured in this run)
-    source = "recorded, not measured in this run: profiles/layer_ops_8192x4096_bf16.txt"
-    recorded = {"rms_norm_vec_kernel": (32883.2 * 2 + 65536.0) * 1024, "rope_vec_kernel": (36228.1 * 2 + 65536.0) * 1024,
-                "gather_kernel": (32501.6 * 2 + 65536.0) * 1024, "concat_kernel": (32787.9 * 2 + 65536.0) * 1024,
-                "matmul_prefill": (320729.2 * 2 + 98356.2) * 1024, "matmul_decode": (27236.2 * 2 + 768.0) * 1024}
+    source = "recorded, not measured in this run: profiles/layer_ops_bf16.txt"
+    recorded = {"rms_norm_vec_kernel": (32888.8 * 2 + 65536.0) * 1024, "rope_vec_kernel": (36550.8 * 2 + 65536.0) * 1024,
+                "gather_kernel": (32508.4 * 2 + 65536.0) * 1024, "concat_kernel": (32787.9 * 2 + 65536.0) * 1024,
+                "transpose_rows_kernel": (32783.3 * 2 + 65536.0) * 1024, "transpose_tiles_kernel": (32796.0 * 2 + 65536.0) * 1024,
+                "convert_kernel": (262155.5 * 2 + 262144.0) * 1024,
+                "matmul_prefill": (320733.2 * 2 + 98347.4) * 1024, "matmul_decode": (29104.8 * 2 + 5385.0) * 1024}
 
     def hbm(name, ms, nbytes, kernel):
         a = nbytes / (ms * 1e-3) / 1e9
@@ -451,6 +453,32 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
     out["multiply"] = hbm("Multiply, %d x %d bf16" % (Tm, ffn), ms, 3 * Tm * ffn * 2, "eltwise_vec_kernel(multiply)")
     dgu.free()
     dmo.free()
+
+    # Transpose [tokens, heads, size] -> [heads, tokens, size] (runs of 256 bytes move whole), the K^T form whose
+    # innermost axis changes (tiles through LDS), and Convert f32 -> bf16
+    dqt = hip.DeviceBuffer(T * Hq * D * 2)
+    ms = timed(lambda: ops.transpose(dq, dqt, (T, Hq, D), (1, 0, 2), 2))
+    out["transpose_rows"] = hbm("Transpose [%d, %d, %d] bf16 -> heads first" % (T, Hq, D), ms, 2 * T * Hq * D * 2, "transpose_rows_kernel")
+    ms = timed(lambda: ops.transpose(dq, dqt, (Hq, T, D), (0, 2, 1), 2))
+    out["transpose_tiles"] = hbm("Transpose [%d, %d, %d] bf16 -> [%d, %d, %d]" % (Hq, T, D, Hq, D, T), ms, 2 * T * Hq * D * 2, "transpose_tiles_kernel")
+    if with_cpu:
+        t, n = cpu_time(lambda: O.transpose(q[:sample], (1, 0, 2)))
+        out["transpose_rows"]["cpu_baseline"] = {"value": (2 * sample * Hq * D * 4) / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                                 "sample": "oracle (fp32 elements, one thread) on %d of %d tokens, mean of %d passes" % (sample, T, n)}
+    Tc = 4 * T  # 805 MB in and out: more than the 256 MB last-level cache holds from one launch to the next
+    df32 = hip.DeviceBuffer(Tc * hidden * 4)
+    dbf = hip.DeviceBuffer(Tc * hidden * 2)
+    df32.fill(0)
+    ms = timed(lambda: ops.convert(df32, dbf, Tc * hidden, 0, 2))
+    out["convert"] = hbm("Convert f32 -> bf16, %d x %d" % (Tc, hidden), ms, Tc * hidden * 6, "convert_kernel")
+    if with_cpu:
+        xs = np.ascontiguousarray(x[:sample])
+        t, n = cpu_time(lambda: O.convert(xs, 0, 2))
+        out["convert"]["cpu_baseline"] = {"value": (sample * hidden * 6) / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                          "sample": "oracle (one thread) on %d of %d rows, mean of %d passes" % (sample, Tc, n)}
+    dqt.free()
+    df32.free()
+    dbf.free()
 
     # MatMul: fused q|k|v projection of a prefill batch (MFMA-bound) and of a decode step (HBM-bound)
     N = (Hq + 2 * Hkv) * D

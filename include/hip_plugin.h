@@ -11,7 +11,7 @@
  * All functions return 0 on success and a non-zero code on failure (1 ov::Exception, 2 other
  * exception, 3 ov::NotImplemented, 4 ov::Cancelled, 5 ov::Busy); hip_plugin_last_error() then
  * holds the exception text.  dtype arguments are hipattn_dtype values, HIP_PLUGIN_I32 for index
- * tensors or HIP_PLUGIN_BOOL for boolean masks.
+ * tensors, HIP_PLUGIN_BOOL for boolean masks, HIP_PLUGIN_I64 / HIP_PLUGIN_I8 for what Convert may produce.
  */
 #ifndef HIP_PLUGIN_H_
 #define HIP_PLUGIN_H_
@@ -25,6 +25,8 @@ extern "C" {
 
 #define HIP_PLUGIN_I32 100
 #define HIP_PLUGIN_BOOL 101
+#define HIP_PLUGIN_I64 102
+#define HIP_PLUGIN_I8 103
 
 typedef struct hip_plugin_s hip_plugin_t;
 typedef struct hip_model_s hip_model_t;

@@ -1,7 +1,7 @@
 /*
  * hipops - thin C ABI over the operators that stand either side of attention in a decoder layer
- * on MI355X (gfx950): RMS normalisation, rotary position embedding, MatMul, Gather, Concat and the
- * gated MLP's Swish, Multiply and GLU.
+ * on MI355X (gfx950): RMS normalisation, rotary position embedding, MatMul, Gather, Concat, the gated
+ * MLP's Swish, Multiply and GLU, and Transpose and Convert between them.
  *
  * Same conventions as hipattn.h, whose status codes, dtype codes and stream type it uses: plain C,
  * device pointers of the current HIP device, asynchronous on the given stream, nothing allocated
@@ -21,7 +21,9 @@ extern "C" {
 #endif
 
 #define HIPOPS_VERSION_MAJOR 0
-#define HIPOPS_VERSION_MINOR 2
+#define HIPOPS_VERSION_MINOR 3
+
+#define HIPOPS_I64 101 /* element types beyond hipattn.h's: 64-bit integers (indices, shapes) */
 
 const char* hipops_last_error_string(void);
 int hipops_version(void); /* major * 1000 + minor */
@@ -121,6 +123,35 @@ hipattn_status hipops_multiply(const void* device_a, const void* device_b, void*
 hipattn_status hipops_glu(const void* device_x, void* device_out, int64_t rows, int64_t width, int activation,
                           int gate_first, int dtype, hipattn_stream stream);
 
+/* ---- Transpose -----------------------------------------------------------------------------
+ * out = in with its axes permuted: output axis k is input axis order[k], as TransposeOp
+ * (src/ops/transpose.cpp:54-135; the reference calls cuTENSOR, or its own gather kernel where
+ * cuTENSOR has no code for the GPU, :215-270).  dims: the input's extents, rank <=
+ * HIPOPS_TRANSPOSE_MAX_RANK; both tensors contiguous; the operator moves elements of
+ * element_bytes (1, 2, 4 or 8) whatever their type.  dims and order are host arrays.  Not in place.
+ * A permutation that keeps the innermost axis moves contiguous runs in pieces of up to 16 bytes;
+ * one that changes it goes through 64 x 64 tiles in LDS. */
+#define HIPOPS_TRANSPOSE_MAX_RANK 8
+hipattn_status hipops_transpose(const void* device_in, void* device_out, int rank, const int64_t* dims,
+                                const int32_t* order, int element_bytes, hipattn_stream stream);
+
+/* ---- Convert -------------------------------------------------------------------------------
+ * out[i] = (to_dtype) in[i], ConvertOp (src/ops/convert.cpp:19-58, src/kernels/convert.cuh:24-49:
+ * static_cast, through float where a 16-bit floating type is involved).  Types: HIPATTN_F32 / F16 /
+ * BF16 / I32, HIPOPS_I64 / U8 / I8 / BOOL (one byte, 0 or 1).
+ *   floating -> floating   one rounding to nearest even
+ *   integer  -> floating   through float, to nearest even
+ *   floating -> integer    towards zero; values beyond the target's range saturate and NaN gives 0
+ *                          (C leaves both undefined)
+ *   integer  -> integer    modulo 2^bits, as a C cast
+ *   any      -> boolean    1 where the value is not zero (NaN included)
+ * Equal types copy (nothing at all when in == out). */
+#define HIPOPS_U8 102 /* plain bytes; HIPATTN_U8 names the quantised KV-cache rows */
+#define HIPOPS_I8 103
+#define HIPOPS_BOOL 104
+hipattn_status hipops_convert(const void* device_in, void* device_out, int64_t count, int from_dtype, int to_dtype,
+                              hipattn_stream stream);
+
 /* ---- Gather -----------------------------------------------------------------------------
  * Gather (opset 1/7/8) with batch_dims, as GatherOp sets it up (src/ops/gather.cpp:60-127) and
  * the kernel executes it (src/kernels/gather.cu:19-47): data seen as
@@ -128,7 +159,6 @@ hipattn_status hipops_glu(const void* device_x, void* device_out, int64_t rows, 
  * [batch, outer, num_indices, inner].  A negative index counts from the end; an index outside
  * the axis after that yields zeros.  inner_bytes = elements after the axis x element size: the
  * operator moves bytes, whatever the element type.  index_dtype: HIPATTN_I32 or HIPOPS_I64. */
-#define HIPOPS_I64 101
 hipattn_status hipops_gather(const void* device_data, const void* device_indices, void* device_out, int64_t batch,
                              int64_t outer, int64_t axis_dim, int64_t inner_bytes, int64_t num_indices,
                              int index_dtype, hipattn_stream stream);

@@ -81,6 +81,16 @@ HIPOPS_API hipattn_status hipops_multiply(const void* a, const void* b, void* ou
     return guarded("hipops_multiply", [&] { return multiply(a, b, out, count, dtype, (hipStream_t)stream); });
 }
 
+HIPOPS_API hipattn_status hipops_transpose(const void* in, void* out, int rank, const int64_t* dims, const int32_t* order,
+                                           int element_bytes, hipattn_stream stream) {
+    return guarded("hipops_transpose", [&] { return transpose(in, out, rank, dims, order, element_bytes, (hipStream_t)stream); });
+}
+
+HIPOPS_API hipattn_status hipops_convert(const void* in, void* out, int64_t count, int from_dtype, int to_dtype,
+                                         hipattn_stream stream) {
+    return guarded("hipops_convert", [&] { return convert(in, out, count, from_dtype, to_dtype, (hipStream_t)stream); });
+}
+
 HIPOPS_API hipattn_status hipops_glu(const void* x, void* out, int64_t rows, int64_t width, int activation, int gate_first,
                                      int dtype, hipattn_stream stream) {
     return guarded("hipops_glu", [&] { return glu(x, out, rows, width, activation, gate_first, dtype, (hipStream_t)stream); });

@@ -23,6 +23,9 @@ hipattn_status swish(const void* x, void* out, int64_t count, float beta, int dt
 hipattn_status multiply(const void* a, const void* b, void* out, int64_t count, int dtype, hipStream_t stream);
 hipattn_status glu(const void* x, void* out, int64_t rows, int64_t width, int activation, int gate_first, int dtype,
                    hipStream_t stream);
+hipattn_status transpose(const void* in, void* out, int rank, const int64_t* dims, const int32_t* order, int element_bytes,
+                         hipStream_t stream);
+hipattn_status convert(const void* in, void* out, int64_t count, int from_dtype, int to_dtype, hipStream_t stream);
 hipattn_status matmul_workspace_size(const hipops_matmul_desc* desc, size_t* bytes);
 hipattn_status matmul(const hipops_matmul_desc* desc, const void* a, const void* b, void* c, void* workspace,
                       size_t workspace_bytes, hipStream_t stream);

@@ -724,6 +724,8 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
             if (alias >= 0) {
                 v.device = ps.in.at(alias).device;
                 v.host = ps.in.at(alias).host;
+                if (bound != remote_outputs.end() && bound->second != v.device && v.byte_size())
+                    ps.copies.push_back({bound->second, v.device, v.byte_size()});
             } else if (bound != remote_outputs.end()) {
                 v.device = bound->second;
             } else {
@@ -768,6 +770,7 @@ void InferRequest::execute_steps(const InferenceRequestContext& context, bool pr
             ev_begin_.back()->record(context.stream);
         }
         step.op->Execute(context, prepared_[si].in, prepared_[si].out, prepared_[si].workbuffers);
+        for (const auto& c : prepared_[si].copies) context.stream.transfer(c.to, c.from, c.bytes);
         if (profiling) ev_end_.back()->record(context.stream);
     }
 }
@@ -798,6 +801,7 @@ std::vector<uint64_t> InferRequest::make_signature() const {
             sig.push_back((uint64_t)(uintptr_t)ps.workbuffers.mutable_buffers[i]);
             sig.push_back(ps.workbuffers.mutable_sizes[i]);
         }
+        for (const auto& c : ps.copies) sig.push_back((uint64_t)(uintptr_t)c.to);
     }
     return sig;
 }

@@ -223,6 +223,14 @@ private:
     struct PreparedStep {
         std::vector<TensorView> in, out;
         Workbuffers workbuffers;
+        // an output that is its input's memory (a view, a pass-through) although its port is bound to a
+        // device tensor of the caller's: copied there behind the operator
+        struct CopyOut {
+            void* to;
+            const void* from;
+            size_t bytes;
+        };
+        std::vector<CopyOut> copies;
     };
     std::vector<PreparedStep> prepared_;
     // Graph replay (the reference's CudaGraphTopologyRunner, src/cuda_graph_topology_runner.cpp, for a

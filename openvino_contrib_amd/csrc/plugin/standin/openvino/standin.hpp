@@ -534,6 +534,25 @@ public:
     }
     const void* get_data_ptr() const { return bytes_.data(); }
     size_t get_byte_size() const { return bytes_.size(); }
+    // the values as T, for the integer constants that carry shapes, axes and orders
+    template <typename T>
+    std::vector<T> cast_vector() const {
+        const element::Type& t = get_output_element_type(0);
+        const size_t n = t.size() ? bytes_.size() / t.size() : 0;
+        std::vector<T> out(n);
+        for (size_t i = 0; i < n; i++) {
+            const uint8_t* at = bytes_.data() + i * t.size();
+            if (t == element::i64) { int64_t v; std::memcpy(&v, at, 8); out[i] = (T)v; }
+            else if (t == element::i32) { int32_t v; std::memcpy(&v, at, 4); out[i] = (T)v; }
+            else if (t == element::u64) { uint64_t v; std::memcpy(&v, at, 8); out[i] = (T)v; }
+            else if (t == element::u32) { uint32_t v; std::memcpy(&v, at, 4); out[i] = (T)v; }
+            else if (t == element::i8) { int8_t v; std::memcpy(&v, at, 1); out[i] = (T)v; }
+            else if (t == element::u8 || t == element::boolean) { out[i] = (T)*at; }
+            else if (t == element::f32) { float v; std::memcpy(&v, at, 4); out[i] = (T)v; }
+            else OPENVINO_THROW("Constant::cast_vector: element type ", t.get_type_name());
+        }
+        return out;
+    }
     std::map<std::string, std::string> standin_attributes() const override {
         std::string hex;
         static const char* digits = "0123456789abcdef";
@@ -730,6 +749,147 @@ public:
     }
 };
 }  // namespace v8
+
+namespace util {
+// the integer values of a Constant input, or nothing when the input is computed at run time
+inline bool constant_values(const Output<Node>& input, std::vector<int64_t>& values) {
+    auto c = std::dynamic_pointer_cast<v0::Constant>(input.get_node_shared_ptr());
+    if (!c) return false;
+    values = c->cast_vector<int64_t>();
+    return true;
+}
+}  // namespace util
+
+namespace v1 {
+// data, pattern: the same elements under the extents of `pattern`; -1 takes what is left, 0 copies
+// the input's extent at that position when special_zero is set
+class Reshape : public Node {
+public:
+    OPENVINO_OP("Reshape", "opset1")
+    Reshape(const Output<Node>& data, const Output<Node>& pattern, bool special_zero)
+        : Node(OutputVector{data, pattern}), special_zero_(special_zero) {
+        std::vector<int64_t> want;
+        const PartialShape& in = data.get_partial_shape();
+        if (util::constant_values(pattern, want)) {
+            std::vector<Dimension> dims;
+            for (size_t i = 0; i < want.size(); i++) {
+                if (want[i] == 0 && special_zero && i < in.size())
+                    dims.push_back(in[i]);
+                else if (want[i] < 0)
+                    dims.push_back(Dimension::dynamic());
+                else
+                    dims.push_back(Dimension(want[i]));
+            }
+            if (in.is_static()) {  // the one -1 can be settled now
+                int64_t known = 1, total = (int64_t)shape_size(in.to_shape());
+                int open = -1;
+                for (size_t i = 0; i < dims.size(); i++) {
+                    if (dims[i].is_dynamic())
+                        open = (int)i;
+                    else
+                        known *= dims[i].get_length();
+                }
+                if (open >= 0 && known > 0) dims[open] = Dimension(total / known);
+            }
+            set_output_type(0, data.get_element_type(), PartialShape(dims));
+        } else {
+            const PartialShape& ps = pattern.get_partial_shape();
+            OPENVINO_ASSERT(ps.size() == 1 && ps[0].is_static(), "Reshape pattern must be a vector of known length");
+            set_output_type(0, data.get_element_type(), PartialShape(std::vector<Dimension>((size_t)ps[0].get_length(), Dimension::dynamic())));
+        }
+    }
+    bool get_special_zero() const { return special_zero_; }
+    std::map<std::string, std::string> standin_attributes() const override { return {{"special_zero", special_zero_ ? "true" : "false"}}; }
+
+private:
+    bool special_zero_;
+};
+
+// data, order: output axis k is input axis order[k]; an empty order reverses the axes
+class Transpose : public Node {
+public:
+    OPENVINO_OP("Transpose", "opset1")
+    Transpose(const Output<Node>& data, const Output<Node>& order) : Node(OutputVector{data, order}) {
+        const PartialShape& in = data.get_partial_shape();
+        std::vector<int64_t> perm;
+        std::vector<Dimension> dims(in.size(), Dimension::dynamic());
+        if (util::constant_values(order, perm)) {
+            if (perm.empty())
+                for (size_t k = 0; k < in.size(); k++) perm.push_back((int64_t)(in.size() - 1 - k));
+            OPENVINO_ASSERT(perm.size() == in.size(), "Transpose order must name every axis");
+            for (size_t k = 0; k < perm.size(); k++) {
+                OPENVINO_ASSERT(perm[k] >= 0 && perm[k] < (int64_t)in.size(), "Transpose order out of range");
+                dims[k] = in[(size_t)perm[k]];
+            }
+        }
+        set_output_type(0, data.get_element_type(), PartialShape(dims));
+    }
+};
+}  // namespace v1
+
+namespace v0 {
+// data [, axes]: axes of extent 1 removed (all of them without the second input)
+class Squeeze : public Node {
+public:
+    OPENVINO_OP("Squeeze", "opset1")
+    explicit Squeeze(const OutputVector& args) : Node(args) {
+        OPENVINO_ASSERT(args.size() == 1 || args.size() == 2, "Squeeze takes data [, axes]");
+        const PartialShape& in = args[0].get_partial_shape();
+        std::vector<int64_t> axes;
+        const bool known = args.size() == 1 || util::constant_values(args[1], axes);
+        OPENVINO_ASSERT(known, "Squeeze axes must be a Constant");
+        std::vector<bool> drop(in.size(), false);
+        for (int64_t a : axes) {
+            if (a < 0) a += (int64_t)in.size();
+            OPENVINO_ASSERT(a >= 0 && a < (int64_t)in.size(), "Squeeze axis out of range");
+            drop[(size_t)a] = true;
+        }
+        std::vector<Dimension> dims;
+        for (size_t k = 0; k < in.size(); k++) {
+            const bool one = in[k].is_static() && in[k].get_length() == 1;
+            if (args.size() == 1 ? one : (drop[k] && (one || in[k].is_dynamic()))) continue;
+            dims.push_back(in[k]);
+        }
+        set_output_type(0, args[0].get_element_type(), PartialShape(dims));
+    }
+};
+
+// data, axes: axes of extent 1 inserted at the given positions of the output
+class Unsqueeze : public Node {
+public:
+    OPENVINO_OP("Unsqueeze", "opset1")
+    Unsqueeze(const Output<Node>& data, const Output<Node>& axes_input) : Node(OutputVector{data, axes_input}) {
+        const PartialShape& in = data.get_partial_shape();
+        std::vector<int64_t> axes;
+        OPENVINO_ASSERT(util::constant_values(axes_input, axes), "Unsqueeze axes must be a Constant");
+        const int64_t rank = (int64_t)(in.size() + axes.size());
+        std::vector<bool> fresh((size_t)rank, false);
+        for (int64_t a : axes) {
+            if (a < 0) a += rank;
+            OPENVINO_ASSERT(a >= 0 && a < rank && !fresh[(size_t)a], "Unsqueeze axis out of range or repeated");
+            fresh[(size_t)a] = true;
+        }
+        std::vector<Dimension> dims;
+        for (size_t k = 0, next = 0; k < (size_t)rank; k++) dims.push_back(fresh[k] ? Dimension(1) : in[next++]);
+        set_output_type(0, data.get_element_type(), PartialShape(dims));
+    }
+};
+
+// data: the same values in another element type
+class Convert : public Node {
+public:
+    OPENVINO_OP("Convert", "opset1")
+    Convert(const Output<Node>& data, const element::Type& destination_type) : Node(OutputVector{data}), destination_(destination_type) {
+        set_output_type(0, destination_type, data.get_partial_shape());
+    }
+    const element::Type& get_destination_type() const { return destination_; }
+    const element::Type& get_convert_element_type() const { return destination_; }
+    std::map<std::string, std::string> standin_attributes() const override { return {{"destination_type", destination_.get_type_name()}}; }
+
+private:
+    element::Type destination_;
+};
+}  // namespace v0
 
 namespace v4 {
 // x [, beta]: x / (1 + exp(-beta x))
@@ -1312,6 +1472,16 @@ public:
                     inputs.at(0), std::stoll(attrs.at("axis")), std::stoll(attrs.at("split_lengths")),
                     (op::internal::GLU::GluType)std::stoi(attrs.at("glu_type")), (size_t)std::stoull(attrs.at("split_to_glu_idx")),
                     attrs.count("output_type") ? element::type_from_name(attrs["output_type"]) : element::dynamic);
+            } else if (type == "Reshape") {
+                n = std::make_shared<op::v1::Reshape>(inputs.at(0), inputs.at(1), attrs.count("special_zero") && attrs["special_zero"] == "true");
+            } else if (type == "Transpose") {
+                n = std::make_shared<op::v1::Transpose>(inputs.at(0), inputs.at(1));
+            } else if (type == "Squeeze") {
+                n = std::make_shared<op::v0::Squeeze>(inputs);
+            } else if (type == "Unsqueeze") {
+                n = std::make_shared<op::v0::Unsqueeze>(inputs.at(0), inputs.at(1));
+            } else if (type == "Convert") {
+                n = std::make_shared<op::v0::Convert>(inputs.at(0), element::type_from_name(attrs.at("destination_type")));
             } else if (type == "MatMul") {
                 n = std::make_shared<op::v0::MatMul>(inputs.at(0), inputs.at(1), attrs["transpose_a"] == "true",
                                                      attrs["transpose_b"] == "true");

@@ -96,6 +96,8 @@ ov::element::Type to_element(int dtype) {
         case HIPATTN_U8: return ov::element::u8;
         case HIP_PLUGIN_I32: return ov::element::i32;
         case HIP_PLUGIN_BOOL: return ov::element::boolean;
+        case HIP_PLUGIN_I64: return ov::element::i64;
+        case HIP_PLUGIN_I8: return ov::element::i8;
     }
     OPENVINO_THROW("unknown dtype code ", dtype);
 }
@@ -105,6 +107,8 @@ int from_element(const ov::element::Type& t) {
     if (t == ov::element::bf16) return HIPATTN_BF16;
     if (t == ov::element::u8) return HIPATTN_U8;
     if (t == ov::element::boolean) return HIP_PLUGIN_BOOL;
+    if (t == ov::element::i64) return HIP_PLUGIN_I64;
+    if (t == ov::element::i8) return HIP_PLUGIN_I8;
     return HIP_PLUGIN_I32;
 }
 

@@ -1,4 +1,5 @@
-"""ctypes binding of libhipops.so (include/hipops.h): RMS norm, RoPE, MatMul, Gather, Concat.
+"""ctypes binding of libhipops.so (include/hipops.h): RMS norm, RoPE, MatMul, Gather, Concat, Swish,
+Multiply, GLU, Transpose, Convert.
 
 Device memory, streams and events come from the hipattn binding (capi.DeviceBuffer & co.); this
 module adds the operator calls.  No fallback: a missing library or a failed call raises.
@@ -11,7 +12,8 @@ from . import capi
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libhipops.so")
 
-I32, I64 = 100, 101
+I32, I64, U8, I8, BOOL = 100, 101, 102, 103, 104
+TRANSPOSE_MAX_RANK = 8
 
 _i, _i64, _f, _vp, _sz = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 _P = ctypes.POINTER
@@ -60,6 +62,8 @@ SYMBOLS = {
     "hipops_swish": (_i, [_vp, _vp, _i64, _f, _i, _vp]),
     "hipops_multiply": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
     "hipops_glu": (_i, [_vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
+    "hipops_transpose": (_i, [_vp, _vp, _i, _P(_i64), _P(ctypes.c_int32), _i, _vp]),
+    "hipops_convert": (_i, [_vp, _vp, _i64, _i, _i, _vp]),
     "hipops_gather": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _vp]),
     "hipops_concat": (_i, [_P(_vp), _P(_i64), _i, _i64, _vp, _vp]),
 }
@@ -135,6 +139,16 @@ def multiply(a, b, out, count, dtype, stream=None):
 
 def glu(x, out, rows, width, dtype, activation=GLU_SWISH, gate_first=True, stream=None):
     check(lib().hipops_glu(_ptr(x), _ptr(out), rows, width, activation, int(gate_first), dtype, _h(stream)))
+
+
+def transpose(x, out, dims, order, element_bytes, stream=None):
+    """out = x with output axis k taken from input axis order[k]; dims are x's extents."""
+    n = len(dims)
+    check(lib().hipops_transpose(_ptr(x), _ptr(out), n, (_i64 * n)(*dims), (ctypes.c_int32 * n)(*order), element_bytes, _h(stream)))
+
+
+def convert(x, out, count, from_dtype, to_dtype, stream=None):
+    check(lib().hipops_convert(_ptr(x), _ptr(out), count, from_dtype, to_dtype, _h(stream)))
 
 
 def gather(data, indices, out, batch, outer, axis_dim, inner_bytes, num_indices, index_dtype, stream=None):

@@ -8,8 +8,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libhip_plugin.so")
 
-F32, F16, BF16, U8, I32, BOOL = 0, 1, 2, 3, 100, 101
-_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, U8: np.uint8, I32: np.int32, BOOL: np.bool_}
+F32, F16, BF16, U8, I32, BOOL, I64, I8 = 0, 1, 2, 3, 100, 101, 102, 103
+_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, U8: np.uint8, I32: np.int32, BOOL: np.bool_, I64: np.int64, I8: np.int8}
 OK, ERROR, OTHER_ERROR, NOT_IMPLEMENTED, CANCELLED, BUSY = range(6)
 
 _vp, _i, _sz, _cp = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_char_p
@@ -99,7 +99,7 @@ def registered_operations():
     return _text(lib().hip_plugin_registered_operations).split(",")
 
 
-_TYPE_NAMES = {F32: "f32", F16: "f16", BF16: "bf16", U8: "u8", I32: "i32", BOOL: "boolean"}
+_TYPE_NAMES = {F32: "f32", F16: "f16", BF16: "bf16", U8: "u8", I32: "i32", BOOL: "boolean", I64: "i64", I8: "i8"}
 
 
 class GraphText:

@@ -27,6 +27,14 @@
  *                         hand-written cases.
  *   oracle_concat_bytes   Concat along an axis (src/ops/concat.cpp:31-56).  Pinned by
  *                         numpy.concatenate.
+ *   oracle_transpose_bytes  Transpose, output axis k = input axis order[k] (src/ops/transpose.cpp:54-135), elements
+ *                         of any size moved as bytes.  Pinned by numpy.transpose.
+ *   oracle_convert        Convert as a C cast, through float where a 16-bit floating type is involved
+ *                         (src/kernels/convert.cuh:24-49), with the two cases C leaves undefined fixed:
+ *                         floating values beyond an integer target's range saturate, NaN gives 0.
+ *                         Pinned by numpy.astype for every pair of types on values inside the range,
+ *                         by torch for the roundings to f16 / bf16, and by hand-written cases for the
+ *                         saturation, NaN and boolean rules.
  *   oracle_swish_f32 /    Swish (src/ops/swish.cpp:41-59) and OpenVINO's fused gated linear unit
  *   oracle_glu_f32        act(gate) * up with Swish, Gelu (erf) or Gelu (tanh).  Pinned by
  *                         torch.nn.functional.silu / gelu in fp64 (fixtures) and the explicit product.
@@ -152,4 +160,74 @@ ORACLE_API void oracle_glu_f32(const float* x, float* out, int64_t rows, int64_t
     for (int64_t r = 0; r < rows; r++)
         for (int64_t i = 0; i < width; i++)
             out[r * width + i] = (float)(oracle_activate(x[r * 2 * width + g + i], activation, 1.0) * (double)x[r * 2 * width + u + i]);
+}
+
+/* out = in with output axis k taken from input axis order[k]; dims are the input's extents */
+ORACLE_API int oracle_transpose_bytes(const uint8_t* in, uint8_t* out, int rank, const int64_t* dims, const int32_t* order,
+                                      int64_t element_bytes) {
+    if (rank < 0 || rank > 16) return 1;
+    int64_t in_stride[16], out_dims[16], step[16], coord[16], total = 1;
+    for (int k = rank - 1; k >= 0; k--) in_stride[k] = k == rank - 1 ? 1 : in_stride[k + 1] * dims[k + 1];
+    for (int k = 0; k < rank; k++) {
+        if (order[k] < 0 || order[k] >= rank) return 1;
+        out_dims[k] = dims[order[k]];
+        step[k] = in_stride[order[k]];
+        coord[k] = 0;
+        total *= out_dims[k];
+    }
+    int64_t src = 0;
+    for (int64_t i = 0; i < total; i++) {
+        memcpy(out + i * element_bytes, in + src * element_bytes, (size_t)element_bytes);
+        for (int k = rank - 1; k >= 0; k--) {  /* odometer over the output's coordinates */
+            src += step[k];
+            if (++coord[k] < out_dims[k]) break;
+            src -= step[k] * out_dims[k];
+            coord[k] = 0;
+        }
+    }
+    return 0;
+}
+
+/* element types as in hipops.h: 0 f32, 1 f16, 2 bf16, 100 i32, 101 i64, 102 u8, 103 i8, 104 boolean */
+float oracle_f16_to_f32(uint16_t h);
+uint16_t oracle_f32_to_f16(float f);
+float oracle_bf16_to_f32(uint16_t b);
+uint16_t oracle_f32_to_bf16(float f);
+
+static int64_t oracle_saturate(float f, float lowest, float beyond, int64_t min_value, int64_t max_value) {
+    if (f != f) return 0;
+    if (f <= lowest) return min_value;
+    if (f >= beyond) return max_value;
+    return (int64_t)f;
+}
+
+ORACLE_API int oracle_convert(const void* in, void* out, int64_t count, int from, int to) {
+    for (int64_t i = 0; i < count; i++) {
+        int is_float = 1;
+        float f = 0.f;
+        int64_t v = 0;
+        switch (from) {
+            case 0: f = ((const float*)in)[i]; break;
+            case 1: f = oracle_f16_to_f32(((const uint16_t*)in)[i]); break;
+            case 2: f = oracle_bf16_to_f32(((const uint16_t*)in)[i]); break;
+            case 100: is_float = 0, v = ((const int32_t*)in)[i]; break;
+            case 101: is_float = 0, v = ((const int64_t*)in)[i]; break;
+            case 102: is_float = 0, v = ((const uint8_t*)in)[i]; break;
+            case 103: is_float = 0, v = ((const int8_t*)in)[i]; break;
+            case 104: is_float = 0, v = ((const uint8_t*)in)[i] != 0; break;
+            default: return 1;
+        }
+        switch (to) {
+            case 0: ((float*)out)[i] = is_float ? f : (float)v; break;
+            case 1: ((uint16_t*)out)[i] = oracle_f32_to_f16(is_float ? f : (float)v); break;
+            case 2: ((uint16_t*)out)[i] = oracle_f32_to_bf16(is_float ? f : (float)v); break;
+            case 100: ((int32_t*)out)[i] = is_float ? (int32_t)oracle_saturate(f, -2147483648.f, 2147483648.f, INT32_MIN, INT32_MAX) : (int32_t)(uint32_t)(uint64_t)v; break;
+            case 101: ((int64_t*)out)[i] = is_float ? oracle_saturate(f, -9223372036854775808.f, 9223372036854775808.f, INT64_MIN, INT64_MAX) : v; break;
+            case 102: ((uint8_t*)out)[i] = is_float ? (uint8_t)oracle_saturate(f, 0.f, 255.f, 0, 255) : (uint8_t)(uint64_t)v; break;
+            case 103: ((int8_t*)out)[i] = is_float ? (int8_t)oracle_saturate(f, -128.f, 127.f, -128, 127) : (int8_t)(uint8_t)(uint64_t)v; break;
+            case 104: ((uint8_t*)out)[i] = is_float ? (f != 0.f) : (v != 0); break;
+            default: return 1;
+        }
+    }
+    return 0;
 }

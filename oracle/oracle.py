@@ -74,6 +74,10 @@ def lib():
         L.oracle_swish_f32.restype = None
         L.oracle_glu_f32.argtypes = [vp, vp, i64, i64, i32, i32]
         L.oracle_glu_f32.restype = None
+        L.oracle_transpose_bytes.restype = i32
+        L.oracle_transpose_bytes.argtypes = [vp, vp, i32, vp, vp, i64]
+        L.oracle_convert.restype = i32
+        L.oracle_convert.argtypes = [vp, vp, i64, i32, i32]
         L.oracle_gather_bytes.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64]
         L.oracle_gather_bytes.restype = None
         L.oracle_concat_bytes.argtypes = [vp, vp, i32, i64, vp]
@@ -322,6 +326,30 @@ def concat(arrays, axis):
     out = np.empty(shape, first.dtype)
     ptrs = (ctypes.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
     lib().oracle_concat_bytes(ptrs, _p(widths), len(arrays), outer, _p(out))
+    return out
+
+
+def transpose(x, order):
+    """x with output axis k taken from input axis order[k] (numpy.transpose's rule), any dtype."""
+    x = np.ascontiguousarray(x)
+    order = [int(o) for o in order]
+    out = np.empty([x.shape[o] for o in order], x.dtype)
+    dims, od = np.array(x.shape, np.int64), np.array(order, np.int32)
+    if lib().oracle_transpose_bytes(_p(x), _p(out), x.ndim, _p(dims), _p(od), x.dtype.itemsize):
+        raise ValueError("oracle_transpose_bytes: bad arguments")
+    return out
+
+
+# element types of the Convert operator: code -> numpy storage type (f16 / bf16 travel as their bits)
+CONVERT_STORAGE = {0: np.float32, 1: np.uint16, 2: np.uint16, 100: np.int32, 101: np.int64, 102: np.uint8, 103: np.int8, 104: np.uint8}
+
+
+def convert(x, from_dtype, to_dtype):
+    """Convert on storage arrays (CONVERT_STORAGE); returns the storage array of to_dtype."""
+    x = _c(x, CONVERT_STORAGE[from_dtype])
+    out = np.empty(x.shape, CONVERT_STORAGE[to_dtype])
+    if lib().oracle_convert(_p(x), _p(out), x.size, from_dtype, to_dtype):
+        raise ValueError("oracle_convert: unknown element type")
     return out
 
 

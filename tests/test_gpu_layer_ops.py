@@ -1,4 +1,5 @@
-"""GPU parity of libhipops.so (RMS norm, RoPE, MatMul, Gather, Concat) against the CPU oracle,
+"""GPU parity of libhipops.so (RMS norm, RoPE, MatMul, Gather, Concat, the gated MLP's element-wise
+operators, Transpose, Convert) against the CPU oracle,
 through the C ABI.  Byte movers are compared bit for bit; floating results against the oracle's
 fp64-accumulated value, within one rounding of the output type plus the fp32 accumulation error
 stated at each test.
@@ -329,3 +330,138 @@ def test_eltwise_rejects_bad_arguments(hip, ops):
         ops.swish(buf, buf, 8, W.U8)
     assert e.value.status == hip.UNSUPPORTED
     ops.swish(None, None, 0, F16)
+
+
+# ------------------------------------------------------------------------------ Transpose, Convert
+TRANSPOSE_CASES = [
+    ((5,), (0,)), ((3, 4), (1, 0)), ((2, 3, 4), (0, 2, 1)), ((2, 3, 4), (2, 0, 1)), ((2, 1, 3, 4), (3, 1, 0, 2)),
+    ((2, 3, 2, 3, 2, 3), (5, 3, 1, 4, 2, 0)), ((4, 1, 6), (1, 0, 2)), ((2, 3, 4, 5, 2, 3, 2, 2), (7, 0, 6, 1, 5, 2, 4, 3)),
+    ((3, 77, 5, 64), (0, 2, 1, 3)),       # [b, l, h, d] -> [b, h, l, d]: rows of 64 elements move whole
+    ((2, 300, 8, 128), (0, 2, 1, 3)),
+    ((2, 8, 300, 128), (0, 2, 1, 3)),
+    ((300, 8, 3, 128), (2, 0, 1, 3)),     # a packed q|k|v split into three tensors
+    ((5, 130, 70), (0, 2, 1)),            # the innermost axis changes: tiles, with ragged edges
+    ((1000, 3), (1, 0)), ((3, 1000), (1, 0)), ((65, 2, 67), (2, 1, 0)), ((4, 66, 3, 65), (3, 0, 2, 1)),
+    ((3, 72, 200), (0, 2, 1)),            # tiles with 16-byte accesses on both sides and ragged edges
+    ((2, 10, 3, 24), (0, 3, 2, 1)), ((2, 100, 4, 36), (0, 3, 2, 1)),  # wide reads, narrow writes; a row end inside a wide access
+    ((2, 3, 4), (0, 1, 2)), ((6, 1, 1, 7), (0, 2, 1, 3)),  # nothing moves
+]
+
+
+@pytest.mark.parametrize("shape,order", TRANSPOSE_CASES)
+@pytest.mark.parametrize("itemsize", [1, 2, 4, 8])
+def test_transpose(hip, ops, oracle, shape, order, itemsize):
+    rng = np.random.default_rng(sum(shape) * 7 + itemsize)
+    print("[transpose]", shape, order, itemsize, flush=True)
+    dt = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[itemsize]
+    x = rng.integers(0, 2 ** (8 * min(itemsize, 4)) - 1, shape).astype(dt)
+    ref = oracle.transpose(x, order)
+    dx = hip.DeviceBuffer.from_numpy(x)
+    do = hip.DeviceBuffer(max(ref.nbytes, 16))
+    do.fill(0xEE)
+    ops.transpose(dx, do, shape, order, itemsize)
+    assert np.array_equal(do.download(dt, ref.shape), ref)
+
+
+def test_transpose_odd_addresses_and_errors(hip, ops, oracle):
+    rng = np.random.default_rng(5)
+    x = rng.integers(0, 65535, (1 + 6 * 10 * 24,)).astype(np.uint16)
+    dx = hip.DeviceBuffer.from_numpy(x)
+    do = hip.DeviceBuffer(x.nbytes + 16)
+
+    class In:   # two bytes into the allocation: pieces of 2 bytes only
+        ptr = ctypes.c_void_p(dx.ptr.value + 2)
+
+    class Out:
+        ptr = ctypes.c_void_p(do.ptr.value + 6)
+
+    ops.transpose(In, Out, (6, 10, 24), (1, 0, 2), 2)
+    got = do.download(np.uint16, (3 + 6 * 10 * 24,))[3:].reshape(10, 6, 24)
+    assert np.array_equal(got, oracle.transpose(x[1:].reshape(6, 10, 24), (1, 0, 2)))
+    ops.transpose(dx, do, (0, 4), (1, 0), 2)  # empty: nothing to do
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.transpose(dx, do, (2, 3), (1, 1), 2)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.transpose(dx, dx, (2, 3), (1, 0), 2)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.transpose(dx, do, (2, 3), (1, 0), 3)
+    assert e.value.status == hip.UNSUPPORTED
+
+
+CONVERT_TYPES = [0, 1, 2, 100, 101, 102, 103, 104]
+
+
+def convert_input(rng, src, n):
+    """Storage array of element type `src`: ordinary values, ties, and everything the rules single out
+    (NaN, infinities, values beyond every integer range, negative zero, bytes that are neither 0 nor 1)."""
+    import torch
+    if src in (0, 1, 2):
+        v = np.concatenate([rng.uniform(-300, 300, n - 24), rng.uniform(-1, 1, 8) * 1e-3,
+                            [np.nan, np.inf, -np.inf, 3e9, -3e9, 1e20, -1e20, 65504.0, 70000.0, 255.5, 127.5, -128.5, 0.0, -0.0, 0.5, -0.5]]).astype(np.float32)
+        v[: n // 4] = np.round(v[: n // 4])
+        v[n // 4: n // 2] = np.round(v[n // 4: n // 2]) + 0.5
+        if src == 1:
+            with np.errstate(over="ignore"):
+                return v.astype(np.float16).view(np.uint16)
+        if src == 2:
+            return torch.from_numpy(v).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        return v
+    storage = {100: np.int32, 101: np.int64, 102: np.uint8, 103: np.int8, 104: np.uint8}[src]
+    info = np.iinfo(storage)
+    v = rng.integers(info.min, info.max, n, dtype=np.int64, endpoint=True)
+    v[: n // 2] = rng.integers(max(info.min, -300), min(info.max, 300), n // 2, endpoint=True)
+    v[-4:] = [info.min, info.max, 0, 1]
+    if src in (100, 101):
+        v[-8:-4] = [2 ** 24 + 1, 2 ** 24 + 3, -(2 ** 24) - 1, 65519]  # ties of the roundings to f32 and f16
+    return v.astype(storage)
+
+
+@pytest.mark.parametrize("src", CONVERT_TYPES)
+@pytest.mark.parametrize("dst", CONVERT_TYPES)
+def test_convert(hip, ops, oracle, src, dst):
+    rng = np.random.default_rng(100 * src + dst)
+    print("[convert]", src, dst, flush=True)
+    for n in (24, 4099, 100_000):
+        x = convert_input(rng, src, n)
+        ref = oracle.convert(x, src, dst)
+        dx = hip.DeviceBuffer.from_numpy(x)
+        do = hip.DeviceBuffer(ref.nbytes)
+        do.fill(0xEE)
+        ops.convert(dx, do, n, src, dst)
+        got = do.download(ref.dtype, ref.shape)
+        if dst in (0, 1, 2):  # NaN payloads are not part of the contract; everything else is, -0.0 included
+            floats = lambda a: a if dst == 0 else (oracle.f16_bits_to_f32(a) if dst == 1 else oracle.bf16_bits_to_f32(a))
+            assert np.array_equal(np.isnan(floats(got)), np.isnan(floats(ref)))
+            keep = ~np.isnan(floats(ref))
+            got, ref = got[keep], ref[keep]
+            if dst == 0:
+                got, ref = got.view(np.uint32), ref.view(np.uint32)
+        assert np.array_equal(got, ref), (src, dst, n, np.flatnonzero(got != ref)[:5])
+
+
+def test_convert_odd_addresses_in_place_and_errors(hip, ops, oracle):
+    rng = np.random.default_rng(9)
+    x = rng.uniform(-100, 100, 1001).astype(np.float32)
+    dx = hip.DeviceBuffer.from_numpy(x)
+    do = hip.DeviceBuffer(4096)
+
+    class In:   # four bytes in: no 16-byte loads
+        ptr = ctypes.c_void_p(dx.ptr.value + 4)
+
+    class Out:
+        ptr = ctypes.c_void_p(do.ptr.value + 2)
+
+    ops.convert(In, Out, 1000, 0, 1)
+    got = do.download(np.uint16, (1001,))[1:]
+    assert np.array_equal(got, oracle.convert(x[1:], 0, 1))
+    ops.convert(dx, dx, 1001, 0, 0)  # equal types in place: nothing
+    assert np.array_equal(dx.download(np.float32, (1001,)), x)
+    ops.convert(dx, do, 0, 0, 1)
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.convert(dx, do, 8, 0, 3)  # 3 names the quantised KV-cache rows, not an element type
+    assert e.value.status == hip.UNSUPPORTED
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.convert(dx, do, -1, 0, 1)
+    assert e.value.status == hip.INVALID_ARGUMENT

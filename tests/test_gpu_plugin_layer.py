@@ -540,3 +540,136 @@ def test_a_whole_small_decoder_runs_on_the_device(hip, oracle):
         again, _ = req.output(0)
         assert np.array_equal(again, logits)
     assert int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")) == 1 and int(compiled.get_property("HIP_GRAPH_LAUNCHES")) == 2
+
+
+# ------------------------------------------------------------------------------ views, Transpose, Convert
+def test_reshape_transpose_convert_chain(hip, oracle):
+    """[batch, length, heads * size] f32 -> Reshape (0, 0, heads, size) -> Transpose (0, 2, 1, 3) ->
+    Convert to f16 -> Unsqueeze / Squeeze -> Reshape (-1, size): the views cost nothing, Transpose and
+    Convert are compared with the oracle bit for bit; shapes change from infer to infer."""
+    rng = np.random.default_rng(21)
+    Hh, S = 3, 16
+    g = P.GraphText("formats")
+    x = g.parameter("x", F32, [-1, -1, Hh * S])
+    i64 = lambda name, values: g.constant(name, np.array(values, np.int64), "i64")
+    split = g.add("Reshape", "split_heads", [x, i64("p0", [0, 0, Hh, S])], special_zero=True)
+    moved = g.add("Transpose", "heads_first", [split, i64("order", [0, 2, 1, 3])])
+    half = g.add("Convert", "to_f16", [moved], destination_type="f16")
+    up = g.add("Unsqueeze", "up", [half, i64("ax_up", [0, -1])])
+    down = g.add("Squeeze", "down", [up, i64("ax_down", [0])])
+    g.result("heads", g.add("Squeeze", "down_all", [down]))
+    g.result("rows", g.add("Reshape", "rows", [half, i64("p1", [-1, S])], special_zero=False))
+    plugin = P.Plugin()
+    assert {"split_heads", "heads_first", "to_f16", "up", "down", "down_all", "rows"} <= set(plugin.query_model(g.model()))
+    compiled = plugin.compile_model(g.model())
+    req = compiled.create_infer_request()
+    for B, L in ((2, 5), (1, 1), (3, 70), (2, 0)):
+        xv = (rng.standard_normal((B, L, Hh * S)) * 4).astype(np.float32)
+        req.set_input(0, xv, F32)
+        req.infer()
+        heads, dt = req.output(0)
+        rows, _ = req.output(1)
+        want = oracle.convert(oracle.transpose(xv.reshape(B, L, Hh, S), (0, 2, 1, 3)), 0, 1)
+        assert dt == F16
+        squeezed = tuple(d for d in (B, Hh, L, S) if d != 1)
+        assert heads.shape == squeezed and rows.shape == (B * Hh * L, S)
+        assert np.array_equal(heads.reshape(-1), want.reshape(-1)) and np.array_equal(rows.reshape(-1), want.reshape(-1))
+
+
+def test_transpose_order_from_a_host_tensor_and_reversal(hip, oracle):
+    """The order may arrive as a tensor at run time (the reference reads it from the input then too,
+    src/ops/transpose.cpp:272-300); an empty order reverses the axes."""
+    rng = np.random.default_rng(22)
+    g = P.GraphText("orders")
+    x = g.parameter("x", BF16, [-1, -1, -1])
+    order = g.parameter("order", P.I32, [-1])
+    g.result("out", g.add("Transpose", "t", [x, order]))
+    compiled = P.Plugin().compile_model(g.model())
+    xs = rng.integers(0, 65535, (4, 70, 9)).astype(np.uint16)
+    for perm in ((2, 0, 1), (0, 2, 1), (1, 0, 2), ()):
+        out, _ = run(compiled, [(xs, BF16), (np.array(perm, np.int32), P.I32)]).output(0)
+        want = oracle.transpose(xs, perm if perm else (2, 1, 0))
+        assert out.shape == want.shape and np.array_equal(out, want)
+    req = compiled.create_infer_request()
+    req.set_input(0, xs, BF16)
+    req.set_input(1, np.array([0, 0, 1], np.int32), P.I32)
+    with pytest.raises(P.PluginError):
+        req.infer()
+
+
+@pytest.mark.parametrize("src,dst", [(F32, BF16), (BF16, F32), (F16, P.I32), (P.I32, F16), (F32, P.I64), (P.I64, F32), (F32, P.BOOL),
+                                     (P.BOOL, F16), (F32, P.I8), (P.I8, BF16)])
+def test_convert_through_the_plugin(hip, oracle, src, dst):
+    codes = {F32: 0, F16: 1, BF16: 2, P.I32: 100, P.I64: 101, P.I8: 103, P.BOOL: 104}
+    rng = np.random.default_rng(23 + src + dst)
+    g = P.GraphText("convert")
+    x = g.parameter("x", src, [-1, 33])
+    g.result("out", g.add("Convert", "c", [x], destination_type=P._TYPE_NAMES[dst]))
+    compiled = P.Plugin().compile_model(g.model())
+    v = rng.uniform(-100, 100, (7, 33)).astype(np.float32)
+    v[0, :4] = [0.0, -0.0, 0.5, -0.5]
+    if src in (F16, BF16):
+        xs = W.to_storage(v, src)[0]
+    elif src == P.BOOL:
+        xs = (v > 0)
+    else:
+        xs = v.astype(P._NP[src])
+    out, dt = run(compiled, [(xs, src)]).output(0)
+    want = oracle.convert(xs.view(np.uint8) if src == P.BOOL else xs, codes[src], codes[dst])
+    assert dt == dst and out.shape == (7, 33)
+    assert np.array_equal(np.asarray(out).view(want.dtype) if dst == P.BOOL else out, want)
+
+
+def test_format_operators_the_plugin_refuses(hip):
+    plugin = P.Plugin()
+    g = P.GraphText("bad")
+    x = g.parameter("x", F32, [-1, 8])
+    g.result("out", g.add("Convert", "to_f64", [x], destination_type="f64"))
+    assert "to_f64" not in plugin.query_model(g.model())
+    g = P.GraphText("bad2")
+    x = g.parameter("x", F32, [-1, 8])
+    pattern = g.parameter("pattern", F32, [2])
+    g.result("out", g.add("Reshape", "float_pattern", [x, pattern], special_zero=False))
+    assert "float_pattern" not in plugin.query_model(g.model())
+    # a pattern that does not fit the data is reported at infer time, by name
+    g = P.GraphText("bad3")
+    x = g.parameter("x", F32, [-1, 8])
+    g.result("out", g.add("Reshape", "misfit", [x, g.constant("p", np.array([-1, 3], np.int64), "i64")], special_zero=False))
+    req = plugin.compile_model(g.model()).create_infer_request()
+    req.set_input(0, np.zeros((2, 8), np.float32), F32)
+    with pytest.raises(P.PluginError) as e:
+        req.infer()
+    assert "misfit" in str(e.value)
+
+
+def test_sdpa_attention_block_with_split_heads(hip, oracle):
+    """The prefill form of an attention block as a converted model carries it: q/k/v MatMul ->
+    Reshape to [batch, length, heads, size] -> Transpose to heads first -> causal
+    ScaledDotProductAttention -> Transpose back -> Reshape -> output MatMul -> residual Add."""
+    rng = np.random.default_rng(24)
+    hidden, Hh, S = 256, 2, 128
+    w = lambda *shape: storage(rng.standard_normal(shape) / np.sqrt(shape[-1]), BF16)
+    wq, wk, wv, wo = w(Hh * S, hidden), w(Hh * S, hidden), w(Hh * S, hidden), w(hidden, Hh * S)
+    g = P.GraphText("sdpa_block")
+    x = g.parameter("x", BF16, [-1, -1, hidden])
+    i64 = lambda name, values: g.constant(name, np.array(values, np.int64), "i64")
+    mm = lambda name, a, wt: g.add("MatMul", name, [a, g.constant(name + "_w", wt[0], "bf16")], transpose_a=False, transpose_b=True)
+    heads = lambda name, t: g.add("Transpose", name + "_t", [g.add("Reshape", name + "_r", [t, i64(name + "_p", [0, 0, Hh, S])], special_zero=True),
+                                                             i64(name + "_o", [0, 2, 1, 3])])
+    att = g.add("ScaledDotProductAttention", "sdpa", [heads("q", mm("q", x, wq)), heads("k", mm("k", x, wk)), heads("v", mm("v", x, wv))], causal=True)
+    back = g.add("Reshape", "merge", [g.add("Transpose", "back", [att, i64("back_o", [0, 2, 1, 3])]), i64("merge_p", [0, 0, Hh * S])], special_zero=True)
+    g.result("out", g.add("Add", "residual", [mm("o", back, wo), x]))
+    compiled = P.Plugin().compile_model(g.model())
+    r = lambda a: oracle.round_to(a, BF16)
+    for B, L in ((2, 200), (1, 37)):
+        x_st, xv = storage(rng.standard_normal((B, L, hidden)), BF16)
+        out, _ = run(compiled, [(x_st, BF16)]).output(0)
+        proj = lambda wt: r(oracle.matmul(xv.reshape(B * L, hidden), wt[1], False, True)).reshape(B, L, Hh, S).transpose(0, 2, 1, 3)
+        a = r(oracle.sdpa(np.ascontiguousarray(proj(wq)), np.ascontiguousarray(proj(wk)), np.ascontiguousarray(proj(wv)), causal=True))
+        merged = np.ascontiguousarray(a.transpose(0, 2, 1, 3)).reshape(B * L, Hh * S)
+        ref = r(r(oracle.matmul(merged, wo[1], False, True)) + xv.reshape(B * L, hidden)).reshape(B, L, hidden)
+        got = H.storage_to_f32(out, BF16)
+        assert got.shape == ref.shape
+        err = scaled_error(got, ref)
+        print("sdpa block %dx%d: scaled max error %.4g" % (B, L, err), flush=True)
+        assert err <= 3e-2

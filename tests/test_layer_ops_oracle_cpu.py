@@ -131,3 +131,93 @@ def test_swish_and_glu_match_torch_fixtures(oracle, golden):
         np.testing.assert_allclose(oracle.glu(packed, act, True), want, rtol=3e-6, atol=1e-6)
         swapped = np.stack([np.concatenate([up, x]), np.concatenate([up, x[::-1]])])     # [up | gate]
         np.testing.assert_allclose(oracle.glu(swapped, act, False), want, rtol=3e-6, atol=1e-6)
+
+
+TRANSPOSE_CASES = [((5,), (0,)), ((3, 4), (1, 0)), ((2, 3, 4), (0, 2, 1)), ((2, 3, 4), (2, 0, 1)), ((2, 5, 3, 8), (0, 2, 1, 3)),
+                   ((2, 1, 3, 4), (3, 1, 0, 2)), ((2, 3, 2, 3, 2, 3), (5, 3, 1, 4, 2, 0)), ((4, 1, 6), (1, 0, 2)), ((0, 3), (1, 0))]
+
+
+@pytest.mark.parametrize("shape,order", TRANSPOSE_CASES)
+def test_transpose_matches_numpy(oracle, shape, order):
+    rng = np.random.default_rng(3)
+    for dt in (np.uint8, np.uint16, np.float32, np.int64):
+        x = rng.integers(0, 200, shape).astype(dt)
+        out = oracle.transpose(x, order)
+        assert out.shape == tuple(shape[o] for o in order)
+        np.testing.assert_array_equal(out, np.transpose(x, order))
+
+
+def convert_with_numpy(x_storage, src, dst):
+    """Convert restated with numpy / torch casts; valid for values inside the target's range."""
+    import torch
+    F32, F16, BF16, BOOL = 0, 1, 2, 104
+    if src == F16:
+        v = x_storage.view(np.float16).astype(np.float32)
+    elif src == BF16:
+        v = (x_storage.astype(np.uint32) << 16).view(np.float32)
+    elif src == BOOL:
+        v = (x_storage != 0).astype(np.int64)
+    else:
+        v = x_storage
+    if dst == BOOL:
+        return (v != 0).astype(np.uint8)
+    if dst in (F16, BF16):
+        v32 = v.astype(np.float32)  # the reference casts through float (kernels/convert.cuh:24-33)
+        if dst == F16:
+            with np.errstate(over="ignore"):
+                return v32.astype(np.float16).view(np.uint16)
+        return torch.from_numpy(v32).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    target = {F32: np.float32, 100: np.int32, 101: np.int64, 102: np.uint8, 103: np.int8}[dst]
+    return v.astype(target)
+
+
+CONVERT_TYPES = [0, 1, 2, 100, 101, 102, 103, 104]
+
+
+def convert_samples(rng, src, dst, n=4096):
+    """Storage array of type `src` whose values lie inside the range of `dst` (fractions included)."""
+    limit = {102: (0, 255), 103: (-128, 127), 104: (0, 1)}.get(dst, (-30000, 30000))
+    if src in (0, 1, 2):
+        v = rng.uniform(limit[0], limit[1], n).astype(np.float32)
+        v[: n // 8] = np.round(v[: n // 8])          # exact integers and ties
+        v[n // 8: n // 4] = np.round(v[n // 8: n // 4]) + 0.5 * (limit[1] > 1)
+        v = np.clip(v, limit[0], limit[1])
+        v[-3:] = [0.0, -0.0, limit[1]]
+        if src == 1:
+            return v.astype(np.float16).view(np.uint16)
+        if src == 2:
+            import torch
+            return torch.from_numpy(v).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        return v
+    storage = {100: np.int32, 101: np.int64, 102: np.uint8, 103: np.int8, 104: np.uint8}[src]
+    lo, hi = {100: (-2**31, 2**31 - 1), 101: (-2**62, 2**62), 102: (0, 255), 103: (-128, 127), 104: (0, 2)}[src]
+    v = rng.integers(lo, hi, n, dtype=np.int64, endpoint=True)
+    v[: n // 2] = rng.integers(max(lo, -300), min(hi, 300), n // 2, endpoint=True)  # small values too
+    return v.astype(storage)
+
+
+@pytest.mark.parametrize("src", CONVERT_TYPES)
+@pytest.mark.parametrize("dst", CONVERT_TYPES)
+def test_convert_matches_numpy_casts(oracle, src, dst):
+    rng = np.random.default_rng(100 * src + dst)
+    x = convert_samples(rng, src, dst)
+    got = oracle.convert(x, src, dst)
+    want = convert_with_numpy(x, src, dst)
+    assert got.dtype == want.dtype
+    np.testing.assert_array_equal(got, want)
+
+
+def test_convert_rules_c_leaves_open(oracle):
+    f = np.array([np.nan, np.inf, -np.inf, 3e9, -3e9, 1e20, -1e20, 300.7, -300.7, 255.9, -0.9, 127.5, -128.9], np.float32)
+    np.testing.assert_array_equal(oracle.convert(f, 0, 100), [0, 2**31 - 1, -2**31, 2**31 - 1, -2**31, 2**31 - 1, -2**31, 300, -300, 255, 0, 127, -128])
+    np.testing.assert_array_equal(oracle.convert(f, 0, 101), [0, 2**63 - 1, -2**63, 3000000000, -3000000000, 2**63 - 1, -2**63, 300, -300, 255, 0, 127, -128])
+    np.testing.assert_array_equal(oracle.convert(f, 0, 102), [0, 255, 0, 255, 0, 255, 0, 255, 0, 255, 0, 127, 0])
+    np.testing.assert_array_equal(oracle.convert(f, 0, 103), [0, 127, -128, 127, -128, 127, -128, 127, -128, 127, 0, 127, -128])
+    np.testing.assert_array_equal(oracle.convert(f, 0, 104), [1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1])
+    np.testing.assert_array_equal(oracle.convert(np.array([0.0, -0.0, 1e-30], np.float32), 0, 104), [0, 0, 1])
+    # integers narrow modulo 2^bits, booleans read any non-zero byte as 1
+    np.testing.assert_array_equal(oracle.convert(np.array([2**32 + 5, -1, 2**31], np.int64), 101, 100), [5, -1, -2**31])
+    np.testing.assert_array_equal(oracle.convert(np.array([256 + 7, -1, 128], np.int32), 100, 102), [7, 255, 128])
+    np.testing.assert_array_equal(oracle.convert(np.array([0, 1, 2, 255], np.uint8), 104, 100), [0, 1, 1, 1])
+    # 2^24 + 1 is not a float: to nearest even
+    np.testing.assert_array_equal(oracle.convert(np.array([2**24 + 1, 2**24 + 3], np.int64), 101, 0), np.array([2**24, 2**24 + 4], np.float32))

@@ -17,7 +17,7 @@ def declared_functions():
 
 def test_header_and_binding_agree():
     names = declared_functions()
-    assert len(names) == 11
+    assert len(names) == 13
     assert sorted(ops_capi.SYMBOLS) == names
 
 
@@ -37,7 +37,7 @@ def test_struct_layout_matches_header():
 
 def test_validation_needs_no_device():
     L = ops_capi.lib()
-    assert L.hipops_version() == 2
+    assert L.hipops_version() == 3
     n = ctypes.c_size_t(0)
     ok = ops_capi.MatmulDesc(capi.BF16, capi.BF16, 64, 6144, 4096, 1, 0, 1, 0, 0)
     assert L.hipops_matmul_workspace_size(ctypes.byref(ok), ctypes.byref(n)) == capi.OK and n.value == 32 << 20
@@ -50,3 +50,12 @@ def test_validation_needs_no_device():
     assert b"rotary_ndims" in L.hipops_last_error_string()
     assert L.hipops_gather(None, None, None, 1, 1, 4, 8, 2, 5, None) == capi.UNSUPPORTED
     assert L.hipops_concat(None, None, 0, 1, None, None) == capi.INVALID_ARGUMENT
+    order = (ctypes.c_int32 * 3)(0, 0, 1)
+    dims = (ctypes.c_int64 * 3)(2, 3, 4)
+    assert L.hipops_transpose(None, None, 3, dims, order, 2, None) == capi.INVALID_ARGUMENT
+    assert b"permutation" in L.hipops_last_error_string()
+    order = (ctypes.c_int32 * 3)(0, 2, 1)
+    assert L.hipops_transpose(None, None, 3, dims, order, 3, None) == capi.UNSUPPORTED
+    assert L.hipops_transpose(None, None, 9, dims, order, 2, None) == capi.INVALID_ARGUMENT
+    assert L.hipops_convert(None, None, 8, capi.F32, 7, None) == capi.UNSUPPORTED
+    assert L.hipops_convert(None, None, 0, capi.F32, ops_capi.I64, None) == capi.OK

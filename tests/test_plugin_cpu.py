@@ -26,7 +26,8 @@ def test_header_binding_and_exports_agree():
 def test_registry_holds_the_attention_operators():
     ops = P.registered_operations()
     for name in ("Parameter", "Result", "Constant", "ScaledDotProductAttention", "PagedAttentionExtension", "ReadValue",
-                 "Assign", "Add", "RMS", "RoPE", "MatMul", "Gather", "Concat"):
+                 "Assign", "Add", "RMS", "RoPE", "MatMul", "Gather", "Concat", "Swish", "Multiply", "GLU", "Reshape", "Squeeze",
+                 "Unsqueeze", "Transpose", "Convert"):
         assert name in ops
 
 
@@ -149,3 +150,20 @@ def test_compile_without_a_device_or_with_unknown_operator_fails():
         plugin.compile_model(P.Model.unsupported())
     # either there is no device here, or the unknown operator is rejected: both are errors, never a fallback
     assert "SuperOperation" in str(e.value) or "no HIP device" in str(e.value)
+
+
+def test_query_model_on_views_transpose_and_convert():
+    """Static shapes of the stand-in nodes and the constructors' verdicts, without a device."""
+    import numpy as np
+
+    g = P.GraphText("formats")
+    x = g.parameter("x", P.F32, [2, 5, 48])
+    i64 = lambda name, values: g.constant(name, np.array(values, np.int64), "i64")
+    split = g.add("Reshape", "split", [x, i64("p", [0, -1, 3, 16])], special_zero=True)
+    moved = g.add("Transpose", "moved", [split, i64("o", [0, 2, 1, 3])])
+    wide = g.add("Unsqueeze", "wide", [moved, i64("a", [0])])
+    g.result("out", g.add("Convert", "half", [g.add("Squeeze", "narrow", [wide, i64("b", [0])])], destination_type="f16"))
+    g.result("bad", g.add("Convert", "to_u16", [x], destination_type="u16"))
+    supported = P.Plugin().query_model(g.model())
+    assert {"split", "moved", "wide", "narrow", "half"} <= set(supported)
+    assert "to_u16" not in supported
