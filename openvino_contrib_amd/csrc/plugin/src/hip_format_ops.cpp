@@ -57,6 +57,7 @@ public:
     using OperationBase::OperationBase;
     void Execute(const InferenceRequestContext&, Inputs, Outputs, const Workbuffers&) const override {}
     int InplaceInputOf(size_t) const override { return 0; }
+    bool InputIsHostOnly(size_t input) const override { return input == 1; }  // the pattern or the axes
 };
 
 class ReshapeOp : public ViewOp {
@@ -170,6 +171,7 @@ public:
             HIP_PLUGIN_THROW(who_ + "rank " + std::to_string(node.get_input_partial_shape(0).size()) + " (at most " +
                              std::to_string(HIPOPS_TRANSPOSE_MAX_RANK) + ")");
     }
+    bool InputIsHostOnly(size_t input) const override { return input == 1; }  // the order
     std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
         const ov::Shape& from = in.at(0).shape;
         const std::vector<int32_t> order = order_of(in);

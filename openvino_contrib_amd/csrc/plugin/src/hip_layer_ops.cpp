@@ -307,6 +307,7 @@ public:
         if (axis_ < 0 || axis_ >= data_rank || batch_dims_ < 0 || batch_dims_ > axis_ || batch_dims_ > index_rank)
             HIP_PLUGIN_THROW(who + "axis " + std::to_string(axis_) + " / batch_dims " + std::to_string(batch_dims_));
     }
+    bool InputIsHostOnly(size_t input) const override { return input == 2; }  // the axis was read from its Constant
     std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
         const ov::Shape &d = in.at(0).shape, &i = in.at(1).shape;
         for (int64_t b = 0; b < batch_dims_; b++)
@@ -396,6 +397,7 @@ public:
             std::memcpy(&beta_, c->get_data_ptr(), 4);
         }
     }
+    bool InputIsHostOnly(size_t input) const override { return input == 1; }  // beta was read from its Constant
     std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
         return {in.at(0).shape};
     }

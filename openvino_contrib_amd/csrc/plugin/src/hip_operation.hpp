@@ -121,6 +121,10 @@ public:
     // When such an input was bound as a host tensor the request copies it back after the operator,
     // so the caller's memory holds the update; device-resident tensors need nothing.
     virtual std::vector<size_t> UpdatedInputs() const { return {}; }
+    // True for an input the operator only ever reads through TensorView::host (a scale, a window, a
+    // shape pattern, an order): a tensor all of whose consumers say so is not uploaded, and its
+    // TensorView::device is null.
+    virtual bool InputIsHostOnly(size_t /*input*/) const { return false; }
     // Told once, while the model is compiled, that nothing consumes this output: an operator may then
     // skip producing it (the scores of PagedAttentionExtension).
     virtual void MarkOutputUnused(size_t /*output*/) {}

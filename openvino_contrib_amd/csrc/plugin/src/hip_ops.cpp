@@ -128,6 +128,7 @@ public:
         }
     }
 
+    bool InputIsHostOnly(size_t input) const override { return input == 4; }  // the scale: a launch parameter
     std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
         return {in.at(0).shape};
     }
@@ -299,6 +300,11 @@ public:
     }
 
     std::vector<size_t> UpdatedInputs() const override { return {kKeyCache, kValueCache}; }
+    // launch parameters, and inputs that must be empty: none of them is handed to a kernel
+    bool InputIsHostOnly(size_t input) const override {
+        return input == kScale || input == kSlidingWindow || input == kAlibiSlopes || input == kMaxContextLen ||
+               (input >= kPaRequiredInputs && input != kScoreAggregationWindow);
+    }
 
     WorkbufferRequest GetWorkBufferRequest(const std::vector<TensorView>& inputs) const override {
         const hipattn_pa_desc d = describe(inputs);

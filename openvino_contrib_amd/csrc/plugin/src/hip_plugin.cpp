@@ -483,6 +483,21 @@ CompiledModel::CompiledModel(const std::shared_ptr<const ov::Model>& model, cons
     for (const auto& step : exec_sequence_)
         for (size_t o = 0; o < step.node->get_output_size(); o++)
             if (!consumed.count({step.node.get(), o})) step.op->MarkOutputUnused(o);
+    // tensors every consumer reads on the host only (launch parameters, shape patterns) stay off the device
+    std::map<TensorID, bool> host_only;
+    for (const auto& step : exec_sequence_) {
+        const auto& in_ids = step.op->GetInputIds();
+        for (size_t i = 0; i < in_ids.size(); i++) {
+            const bool here = step.op->InputIsHostOnly(i);
+            auto it = host_only.find(in_ids[i]);
+            if (it == host_only.end())
+                host_only[in_ids[i]] = here;
+            else
+                it->second = it->second && here;
+        }
+    }
+    for (const auto& kv : host_only)
+        if (kv.second) host_only_tensors_.insert(kv.first);
 }
 
 std::shared_ptr<ov::ISyncInferRequest> CompiledModel::create_sync_infer_request() const {
@@ -706,8 +721,10 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
                 v.device = remote->device_ptr();
             } else {
                 v.host = t->data();
-                v.device = tensor_buffers_[out_ids[0]].reserve(std::max<size_t>(v.byte_size(), 16));
-                if (v.byte_size()) stream.upload(v.device, v.host, v.byte_size());
+                if (!compiled_->is_host_only(out_ids[0])) {
+                    v.device = tensor_buffers_[out_ids[0]].reserve(std::max<size_t>(v.byte_size(), 16));
+                    if (v.byte_size()) stream.upload(v.device, v.host, v.byte_size());
+                }
             }
             views_[out_ids[0]] = v;
             ps.out.push_back(v);
@@ -728,6 +745,8 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
                     ps.copies.push_back({bound->second, v.device, v.byte_size()});
             } else if (bound != remote_outputs.end()) {
                 v.device = bound->second;
+            } else if (step.op->HostData(o) && compiled_->is_host_only(out_ids[o])) {
+                v.host = step.op->HostData(o);  // a Constant only ever read on the host
             } else {
                 v.device = tensor_buffers_[out_ids[o]].reserve(std::max<size_t>(v.byte_size(), 16));
                 if (const void* host = step.op->HostData(o)) {  // a Constant: uploaded once per request

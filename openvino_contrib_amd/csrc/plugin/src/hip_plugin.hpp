@@ -169,6 +169,8 @@ public:
     const std::vector<ExecStep>& exec_sequence() const { return exec_sequence_; }
     size_t num_tensors() const { return num_tensors_; }
     const std::vector<TensorID>& output_ids(const ov::Node* node) const { return output_ids_.at(node); }
+    // no consumer of this tensor reads it on the device (OperationBase::InputIsHostOnly)
+    bool is_host_only(TensorID id) const { return host_only_tensors_.count(id) != 0; }
     const Configuration& config() const { return config_; }
     const ov::ParameterVector& parameters() const { return exec_model_->get_parameters(); }
     const ov::ResultVector& results() const { return exec_model_->get_results(); }
@@ -186,6 +188,7 @@ private:
     bool loaded_from_cache_;
     std::vector<ExecStep> exec_sequence_;
     std::map<const ov::Node*, std::vector<TensorID>> output_ids_;  // per node: one TensorID per output port
+    std::set<TensorID> host_only_tensors_;
     size_t num_tensors_ = 0;
     mutable std::atomic<size_t> graphs_captured_{0}, graph_launches_{0};
 };
