@@ -480,6 +480,23 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
     df32.free()
     dbf.free()
 
+    # the decomposed form of attention: mask added to the scores of 32 heads (broadcast over the heads), softmax over the keys
+    Hs, Ls = 32, 2048
+    dsc, _ = dev((Hs, Ls, Ls))
+    dmask, _ = dev((1, Ls, Ls))
+    dso = hip.DeviceBuffer(Hs * Ls * Ls * 2)
+    ms = timed(lambda: ops.binary(ops.ADD, dsc, dmask, dso, (Hs, Ls, Ls), (Hs, Ls, Ls), (1, Ls, Ls), BF16))
+    out["add_broadcast"] = hbm("Add [%d, %d, %d] + [1, %d, %d] bf16" % (Hs, Ls, Ls, Ls, Ls), ms, (2 * Hs + 1) * Ls * Ls * 2, "binary_kernel")
+    ms = timed(lambda: ops.softmax(dsc, dso, Hs * Ls, Ls, 1, BF16))
+    out["softmax"] = hbm("Softmax over the last axis of [%d, %d, %d] bf16" % (Hs, Ls, Ls), ms, 2 * Hs * Ls * Ls * 2, "softmax_rows_kernel")
+    if with_cpu:
+        xs = np.ascontiguousarray(x[:sample, :Ls])
+        t, n = cpu_time(lambda: O.softmax(xs, -1))
+        out["softmax"]["cpu_baseline"] = {"value": (2 * sample * Ls * 4) / t / 1e9, "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+                                          "sample": "oracle (fp32 in, fp64 arithmetic) on %d rows of %d, mean of %d passes" % (sample, Ls, n)}
+    for b in (dsc, dmask, dso):
+        b.free()
+
     # MatMul: fused q|k|v projection of a prefill batch (MFMA-bound) and of a decode step (HBM-bound)
     N = (Hq + 2 * Hkv) * D
     dw, w = dev((N, hidden), 1.0 / 64)

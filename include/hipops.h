@@ -1,7 +1,8 @@
 /*
  * hipops - thin C ABI over the operators that stand either side of attention in a decoder layer
  * on MI355X (gfx950): RMS normalisation, rotary position embedding, MatMul, Gather, Concat, the gated
- * MLP's Swish, Multiply and GLU, and Transpose and Convert between them.
+ * MLP's Swish, Multiply and GLU, Transpose and Convert between them, and the broadcasting
+ * arithmetic and Softmax of attention in its decomposed form.
  *
  * Same conventions as hipattn.h, whose status codes, dtype codes and stream type it uses: plain C,
  * device pointers of the current HIP device, asynchronous on the given stream, nothing allocated
@@ -21,7 +22,7 @@ extern "C" {
 #endif
 
 #define HIPOPS_VERSION_MAJOR 0
-#define HIPOPS_VERSION_MINOR 3
+#define HIPOPS_VERSION_MINOR 4
 
 #define HIPOPS_I64 101 /* element types beyond hipattn.h's: 64-bit integers (indices, shapes) */
 
@@ -122,6 +123,31 @@ hipattn_status hipops_multiply(const void* device_a, const void* device_b, void*
                                hipattn_stream stream);
 hipattn_status hipops_glu(const void* device_x, void* device_out, int64_t rows, int64_t width, int activation,
                           int gate_first, int dtype, hipattn_stream stream);
+
+/* ---- Add / Subtract / Multiply / Divide with broadcasting ---------------------------------------
+ * out = a (op) b under numpy's broadcasting rule, as the reference's ElementwiseBinaryOp
+ * (src/ops/elementwise_binary.hpp:16-76 over src/kernels/details/elementwise_binary.cuh:24-46 and
+ * numpy_broadcast_mapper.cuh; AddOp src/ops/add.cpp:17-43, MultiplyOp src/ops/multiply.cpp:43,
+ * SubtractOp, DivideOp).  The three shapes have one rank (<= HIPOPS_BINARY_MAX_RANK; the caller
+ * pads the shorter ones with leading 1s); an operand's extent is the output's or 1.  fp32
+ * arithmetic, one rounding to `dtype` (HIPATTN_F32 / F16 / BF16); division is correctly rounded.
+ * out may be a or b when that operand has the output's shape. */
+#define HIPOPS_BINARY_MAX_RANK 8
+#define HIPOPS_ADD 0
+#define HIPOPS_SUBTRACT 1
+#define HIPOPS_MULTIPLY 2
+#define HIPOPS_DIVIDE 3
+hipattn_status hipops_binary(int operation, const void* device_a, const void* device_b, void* device_out, int rank,
+                             const int64_t* out_dims, const int64_t* a_dims, const int64_t* b_dims, int dtype,
+                             hipattn_stream stream);
+
+/* ---- Softmax --------------------------------------------------------------------------------
+ * x seen as [outer, length, inner]: out[o, i, n] = exp(x[o, i, n] - max_i) / sum_i exp(x[o, i, n] - max_i),
+ * SoftmaxOp (src/ops/softmax.cpp:73-196: cudnnSoftmaxForward, accurate algorithm, channel mode, after
+ * folding the axes around `axis` the same way).  fp32 arithmetic, one rounding to `dtype`
+ * (HIPATTN_F32 / F16 / BF16).  A slice that is -inf throughout gives NaN.  In place is allowed. */
+hipattn_status hipops_softmax(const void* device_x, void* device_out, int64_t outer, int64_t length, int64_t inner,
+                              int dtype, hipattn_stream stream);
 
 /* ---- Transpose -----------------------------------------------------------------------------
  * out = in with its axes permuted: output axis k is input axis order[k], as TransposeOp

@@ -79,7 +79,7 @@ def build_library(verbose=False, extra_flags=(), jobs=4):
 
 
 OPS_LIB_PATH = os.path.join(CSRC, "libhipops.so")
-OPS_SOURCES = ["ops/hipops_api.hip", "ops/layer_ops.hip", "ops/format_ops.hip", "ops/matmul.hip"]
+OPS_SOURCES = ["ops/hipops_api.hip", "ops/layer_ops.hip", "ops/format_ops.hip", "ops/math_ops.hip", "ops/matmul.hip"]
 
 
 def build_ops_library(verbose=False, extra_flags=(), jobs=4):
@@ -101,7 +101,7 @@ def build_bench_tools():
 
 
 PLUGIN_LIB_PATH = os.path.join(CSRC, "libhip_plugin.so")
-PLUGIN_SOURCES = ["plugin/src/hip_ops.cpp", "plugin/src/hip_layer_ops.cpp", "plugin/src/hip_format_ops.cpp", "plugin/src/hip_plugin.cpp", "plugin/src/hip_create_plugin.cpp",
+PLUGIN_SOURCES = ["plugin/src/hip_ops.cpp", "plugin/src/hip_layer_ops.cpp", "plugin/src/hip_format_ops.cpp", "plugin/src/hip_math_ops.cpp", "plugin/src/hip_plugin.cpp", "plugin/src/hip_create_plugin.cpp",
                   "plugin/test_facade/c_api.cpp"]
 
 

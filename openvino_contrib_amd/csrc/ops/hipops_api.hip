@@ -91,6 +91,16 @@ HIPOPS_API hipattn_status hipops_convert(const void* in, void* out, int64_t coun
     return guarded("hipops_convert", [&] { return convert(in, out, count, from_dtype, to_dtype, (hipStream_t)stream); });
 }
 
+HIPOPS_API hipattn_status hipops_binary(int operation, const void* a, const void* b, void* out, int rank, const int64_t* out_dims,
+                                        const int64_t* a_dims, const int64_t* b_dims, int dtype, hipattn_stream stream) {
+    return guarded("hipops_binary", [&] { return binary(operation, a, b, out, rank, out_dims, a_dims, b_dims, dtype, (hipStream_t)stream); });
+}
+
+HIPOPS_API hipattn_status hipops_softmax(const void* x, void* out, int64_t outer, int64_t length, int64_t inner, int dtype,
+                                         hipattn_stream stream) {
+    return guarded("hipops_softmax", [&] { return softmax(x, out, outer, length, inner, dtype, (hipStream_t)stream); });
+}
+
 HIPOPS_API hipattn_status hipops_glu(const void* x, void* out, int64_t rows, int64_t width, int activation, int gate_first,
                                      int dtype, hipattn_stream stream) {
     return guarded("hipops_glu", [&] { return glu(x, out, rows, width, activation, gate_first, dtype, (hipStream_t)stream); });

@@ -26,6 +26,9 @@ hipattn_status glu(const void* x, void* out, int64_t rows, int64_t width, int ac
 hipattn_status transpose(const void* in, void* out, int rank, const int64_t* dims, const int32_t* order, int element_bytes,
                          hipStream_t stream);
 hipattn_status convert(const void* in, void* out, int64_t count, int from_dtype, int to_dtype, hipStream_t stream);
+hipattn_status binary(int op, const void* a, const void* b, void* out, int rank, const int64_t* out_dims, const int64_t* a_dims,
+                      const int64_t* b_dims, int dtype, hipStream_t stream);
+hipattn_status softmax(const void* x, void* out, int64_t outer, int64_t length, int64_t inner, int dtype, hipStream_t stream);
 hipattn_status matmul_workspace_size(const hipops_matmul_desc* desc, size_t* bytes);
 hipattn_status matmul(const hipops_matmul_desc* desc, const void* a, const void* b, void* c, void* workspace,
                       size_t workspace_bytes, hipStream_t stream);

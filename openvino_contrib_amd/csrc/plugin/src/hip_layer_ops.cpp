@@ -1,11 +1,10 @@
 // Operators either side of attention in a decoder layer: RMS normalisation, rotary position
-// embedding, MatMul, Gather, Concat, and the gated MLP's Swish / Multiply / GLU; each a thin adapter
+// embedding, MatMul, Gather, Concat, and the gated MLP's Swish / GLU; each a thin adapter
 // from node + runtime shapes to the C ABI of libhipops (include/hipops.h).
 //
 // MatMulOp, GatherOp and ConcatOp follow the reference's operators of the same names
 // (modules/nvidia_plugin/src/ops/matmul.cpp:22-76 and 185-227, src/ops/gather.cpp:27-127,
-// src/ops/concat.cpp:20-102), SwishOp and MultiplyOp likewise (src/ops/swish.cpp:41-59,
-// src/ops/multiply.cpp:43).  GluOp, RmsOp and RopeOp serve OpenVINO's fused internal operators GLU,
+// src/ops/concat.cpp:20-102), SwishOp likewise (src/ops/swish.cpp:41-59).  GluOp, RmsOp and RopeOp serve OpenVINO's fused internal operators GLU,
 // RMS and RoPE, which the reference would receive unfused (VariadicSplit / Swish / Multiply,
 // Power / ReduceMean / Sqrt / Multiply, and Slice / Multiply / Concat / Add).  As everywhere in this plugin a constructor that throws is how
 // an unsupported node is reported (src/cuda_plugin.cpp:171-188).
@@ -17,7 +16,6 @@
 #include "openvino/op/constant.hpp"
 #include "openvino/op/gather.hpp"
 #include "openvino/op/matmul.hpp"
-#include "openvino/op/multiply.hpp"
 #include "openvino/op/swish.hpp"
 #include "ov_ops/glu.hpp"
 #include "ov_ops/rms.hpp"
@@ -380,7 +378,7 @@ private:
     int64_t axis_ = 0;
 };
 
-// ------------------------------------------------------------------------------ Swish, Multiply, GLU
+// ------------------------------------------------------------------------------ Swish, GLU
 class SwishOp : public OperationBase {
 public:
     SwishOp(const CreationContext& ctx, const ov::Node& node, IndexCollection&& in, IndexCollection&& out)
@@ -408,30 +406,6 @@ public:
 private:
     int dtype_ = 0;
     float beta_ = 1.0f;
-};
-
-class MultiplyOp : public OperationBase {
-public:
-    MultiplyOp(const CreationContext& ctx, const ov::Node& node, IndexCollection&& in, IndexCollection&& out)
-        : OperationBase(ctx, node, std::move(in), std::move(out)) {
-        const std::string who = "Multiply '" + node.get_friendly_name() + "': ";
-        if (node.get_input_size() != 2) HIP_PLUGIN_THROW(who + "two inputs expected");
-        if (node.get_input_element_type(0) != node.get_input_element_type(1)) HIP_PLUGIN_THROW(who + "mixed input precisions");
-        if (!float_dtype(node.get_input_element_type(0), dtype_)) HIP_PLUGIN_THROW(who + "f32, f16 or bf16 expected");
-        if (!node.get_input_partial_shape(0).compatible(node.get_input_partial_shape(1))) HIP_PLUGIN_THROW(who + "broadcasting is not supported");
-    }
-    std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
-        HIP_PLUGIN_ASSERT(in.at(0).shape == in.at(1).shape,
-                          "Multiply of " + shape_str(in[0].shape) + " and " + shape_str(in[1].shape) + ": broadcasting is not supported");
-        return {in[0].shape};
-    }
-    void Execute(const InferenceRequestContext& context, Inputs in, Outputs out, const Workbuffers&) const override {
-        HIP_OPS_CHECK(hipops_multiply(in[0].device, in[1].device, out[0].device, (int64_t)ov::shape_size(in[0].shape), dtype_,
-                                      context.stream.get()));
-    }
-
-private:
-    int dtype_ = 0;
 };
 
 // act(one half of the last axis) * the other half
@@ -485,7 +459,6 @@ private:
 using ov::hip_gpu::ConcatOp;
 using ov::hip_gpu::GatherOp;
 using ov::hip_gpu::GluOp;
-using ov::hip_gpu::MultiplyOp;
 using ov::hip_gpu::SwishOp;
 using ov::hip_gpu::MatMulOp;
 using ov::hip_gpu::RmsOp;
@@ -496,5 +469,4 @@ HIP_OPERATION_REGISTER(MatMulOp, MatMul)
 HIP_OPERATION_REGISTER(GatherOp, Gather)
 HIP_OPERATION_REGISTER(ConcatOp, Concat)
 HIP_OPERATION_REGISTER(SwishOp, Swish)
-HIP_OPERATION_REGISTER(MultiplyOp, Multiply)
 HIP_OPERATION_REGISTER(GluOp, GLU)

@@ -1,5 +1,5 @@
 // Operators of the "HIP" plugin: Parameter / Result / Constant, the two attention operators, and
-// the stateful pair ReadValue / Assign with the element-wise Add that stateful test models use;
+// the stateful pair ReadValue / Assign;
 // each a thin adapter from node + runtime shapes to calls of the C ABI.
 //
 // SdpaOp stands where the reference lets ScaledDotProductAttentionDecomposition run
@@ -458,41 +458,11 @@ private:
     std::string variable_id_;
 };
 
-// Element-wise sum of two tensors of one shape (src/ops/add.cpp:17-43 without broadcasting).
-class AddOp : public OperationBase {
-public:
-    AddOp(const CreationContext& ctx, const ov::Node& node, IndexCollection&& in, IndexCollection&& out)
-        : OperationBase(ctx, node, std::move(in), std::move(out)) {
-        const std::string who = "Add '" + node.get_friendly_name() + "': ";
-        type_ = node.get_input_element_type(0);
-        if (node.get_input_element_type(1) != type_) HIP_PLUGIN_THROW(who + "mixed input precisions");
-        if (!is_float(type_) && type_ != ov::element::i32)
-            HIP_PLUGIN_THROW(who + "precision " + type_.get_type_name() + " (f32, f16, bf16 or i32 expected)");
-        const auto &a = node.get_input_partial_shape(0), &b = node.get_input_partial_shape(1);
-        if (!a.compatible(b)) HIP_PLUGIN_THROW(who + "broadcasting is not supported");
-    }
-    std::vector<ov::Shape> InferOutputShapes(const std::vector<TensorView>& in, const InferenceRequestContext&) const override {
-        HIP_PLUGIN_ASSERT(in.at(0).shape == in.at(1).shape,
-                          "Add of " + shape_str(in[0].shape) + " and " + shape_str(in[1].shape) + ": broadcasting is not supported");
-        return {in[0].shape};
-    }
-    void Execute(const InferenceRequestContext& context, Inputs in, Outputs out, const Workbuffers&) const override {
-        hipattn_dtype dt;
-        const int dtype = type_ == ov::element::i32 ? HIPATTN_I32 : (to_hipattn_dtype(type_, dt), (int)dt);
-        HIP_PLUGIN_CHECK(hipattn_add_async(out[0].device, in[0].device, in[1].device, (int64_t)ov::shape_size(in[0].shape),
-                                           dtype, context.stream.get()));
-    }
-
-private:
-    ov::element::Type type_;
-};
-
 }  // namespace
 
 }  // namespace hip_gpu
 }  // namespace ov
 
-using ov::hip_gpu::AddOp;
 using ov::hip_gpu::AssignOp;
 using ov::hip_gpu::ConstantOp;
 using ov::hip_gpu::PagedAttentionOp;
@@ -506,4 +476,3 @@ HIP_OPERATION_REGISTER(SdpaOp, ScaledDotProductAttention)
 HIP_OPERATION_REGISTER(PagedAttentionOp, PagedAttentionExtension)
 HIP_OPERATION_REGISTER(ReadValueOp, ReadValue)
 HIP_OPERATION_REGISTER(AssignOp, Assign)
-HIP_OPERATION_REGISTER(AddOp, Add)

@@ -639,16 +639,83 @@ public:
 };
 }  // namespace v6
 
-namespace v1 {
-// element-wise sum, used by the stateful test models
-class Add : public Node {
-public:
-    OPENVINO_OP("Add", "opset1")
-    Add(const Output<Node>& a, const Output<Node>& b) : Node(OutputVector{a, b}) {
-        set_output_type(0, a.get_element_type(), a.get_partial_shape());
+namespace util {
+// numpy's broadcasting rule on shapes that may hold unknown extents
+inline PartialShape broadcast_shapes(const PartialShape& a, const PartialShape& b) {
+    const size_t rank = std::max(a.size(), b.size());
+    std::vector<Dimension> dims(rank);
+    for (size_t k = 0; k < rank; k++) {
+        const Dimension da = k + a.size() >= rank ? a[k + a.size() - rank] : Dimension(1);
+        const Dimension db = k + b.size() >= rank ? b[k + b.size() - rank] : Dimension(1);
+        if (da.is_static() && db.is_static()) {
+            OPENVINO_ASSERT(da.get_length() == db.get_length() || da.get_length() == 1 || db.get_length() == 1,
+                            "shapes ", a.to_string(), " and ", b.to_string(), " do not broadcast");
+            dims[k] = da.get_length() == 1 ? db : da;
+        } else if (da.is_static() && da.get_length() != 1) {
+            dims[k] = da;
+        } else if (db.is_static() && db.get_length() != 1) {
+            dims[k] = db;
+        } else {
+            dims[k] = Dimension::dynamic();
+        }
+    }
+    return PartialShape(dims);
+}
+// element-wise arithmetic of two tensors under numpy broadcasting
+class BinaryElementwiseArithmetic : public Node {
+protected:
+    BinaryElementwiseArithmetic(const Output<Node>& a, const Output<Node>& b) : Node(OutputVector{a, b}) {
+        set_output_type(0, a.get_element_type(), broadcast_shapes(a.get_partial_shape(), b.get_partial_shape()));
     }
 };
+}  // namespace util
+
+namespace v1 {
+class Add : public util::BinaryElementwiseArithmetic {
+public:
+    OPENVINO_OP("Add", "opset1")
+    Add(const Output<Node>& a, const Output<Node>& b) : util::BinaryElementwiseArithmetic(a, b) {}
+};
+class Subtract : public util::BinaryElementwiseArithmetic {
+public:
+    OPENVINO_OP("Subtract", "opset1")
+    Subtract(const Output<Node>& a, const Output<Node>& b) : util::BinaryElementwiseArithmetic(a, b) {}
+};
+class Divide : public util::BinaryElementwiseArithmetic {
+public:
+    OPENVINO_OP("Divide", "opset1")
+    Divide(const Output<Node>& a, const Output<Node>& b) : util::BinaryElementwiseArithmetic(a, b) {}
+};
+// exp(x - max) / sum over one axis
+class Softmax : public Node {
+public:
+    OPENVINO_OP("Softmax", "opset1")
+    Softmax(const Output<Node>& x, size_t axis) : Node(OutputVector{x}), axis_(axis) {
+        set_output_type(0, x.get_element_type(), x.get_partial_shape());
+    }
+    size_t get_axis() const { return axis_; }
+    std::map<std::string, std::string> standin_attributes() const override { return {{"axis", std::to_string(axis_)}, {"opset", "1"}}; }
+
+private:
+    size_t axis_;
+};
 }  // namespace v1
+
+namespace v8 {
+// as v1, the axis may count from the end
+class Softmax : public Node {
+public:
+    OPENVINO_OP("Softmax", "opset8")
+    Softmax(const Output<Node>& x, int64_t axis) : Node(OutputVector{x}), axis_(axis) {
+        set_output_type(0, x.get_element_type(), x.get_partial_shape());
+    }
+    int64_t get_axis() const { return axis_; }
+    std::map<std::string, std::string> standin_attributes() const override { return {{"axis", std::to_string(axis_)}, {"opset", "8"}}; }
+
+private:
+    int64_t axis_;
+};
+}  // namespace v8
 
 namespace v0 {
 // A [.., m, k] x B [.., k, n] with optional transposition of the last two axes of either operand
@@ -904,12 +971,10 @@ public:
 }  // namespace v4
 
 namespace v1 {
-class Multiply : public Node {
+class Multiply : public util::BinaryElementwiseArithmetic {
 public:
     OPENVINO_OP("Multiply", "opset1")
-    Multiply(const Output<Node>& a, const Output<Node>& b) : Node(OutputVector{a, b}) {
-        set_output_type(0, a.get_element_type(), a.get_partial_shape());
-    }
+    Multiply(const Output<Node>& a, const Output<Node>& b) : util::BinaryElementwiseArithmetic(a, b) {}
 };
 }  // namespace v1
 
@@ -1463,6 +1528,15 @@ public:
                 n = a;
             } else if (type == "Add") {
                 n = std::make_shared<op::v1::Add>(inputs.at(0), inputs.at(1));
+            } else if (type == "Subtract") {
+                n = std::make_shared<op::v1::Subtract>(inputs.at(0), inputs.at(1));
+            } else if (type == "Divide") {
+                n = std::make_shared<op::v1::Divide>(inputs.at(0), inputs.at(1));
+            } else if (type == "Softmax") {
+                if (attrs.count("opset") && attrs["opset"] == "1")
+                    n = std::make_shared<op::v1::Softmax>(inputs.at(0), (size_t)std::stoull(attrs.at("axis")));
+                else
+                    n = std::make_shared<op::v8::Softmax>(inputs.at(0), std::stoll(attrs.at("axis")));
             } else if (type == "Swish") {
                 n = std::make_shared<op::v4::Swish>(inputs);
             } else if (type == "Multiply") {

@@ -1,5 +1,5 @@
 """ctypes binding of libhipops.so (include/hipops.h): RMS norm, RoPE, MatMul, Gather, Concat, Swish,
-Multiply, GLU, Transpose, Convert.
+Multiply, GLU, Transpose, Convert, broadcasting arithmetic, Softmax.
 
 Device memory, streams and events come from the hipattn binding (capi.DeviceBuffer & co.); this
 module adds the operator calls.  No fallback: a missing library or a failed call raises.
@@ -64,6 +64,8 @@ SYMBOLS = {
     "hipops_glu": (_i, [_vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "hipops_transpose": (_i, [_vp, _vp, _i, _P(_i64), _P(ctypes.c_int32), _i, _vp]),
     "hipops_convert": (_i, [_vp, _vp, _i64, _i, _i, _vp]),
+    "hipops_binary": (_i, [_i, _vp, _vp, _vp, _i, _P(_i64), _P(_i64), _P(_i64), _i, _vp]),
+    "hipops_softmax": (_i, [_vp, _vp, _i64, _i64, _i64, _i, _vp]),
     "hipops_gather": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _vp]),
     "hipops_concat": (_i, [_P(_vp), _P(_i64), _i, _i64, _vp, _vp]),
 }
@@ -149,6 +151,20 @@ def transpose(x, out, dims, order, element_bytes, stream=None):
 
 def convert(x, out, count, from_dtype, to_dtype, stream=None):
     check(lib().hipops_convert(_ptr(x), _ptr(out), count, from_dtype, to_dtype, _h(stream)))
+
+
+ADD, SUBTRACT, MULTIPLY, DIVIDE = 0, 1, 2, 3
+
+
+def binary(op, a, b, out, out_dims, a_dims, b_dims, dtype, stream=None):
+    """out = a (op) b with numpy broadcasting; the three shapes are given at one rank (leading 1s added here)."""
+    n = max(len(out_dims), len(a_dims), len(b_dims))
+    pad = lambda d: (_i64 * n)(*([1] * (n - len(d)) + [int(x) for x in d]))
+    check(lib().hipops_binary(op, _ptr(a), _ptr(b), _ptr(out), n, pad(out_dims), pad(a_dims), pad(b_dims), dtype, _h(stream)))
+
+
+def softmax(x, out, outer, length, inner, dtype, stream=None):
+    check(lib().hipops_softmax(_ptr(x), _ptr(out), outer, length, inner, dtype, _h(stream)))
 
 
 def gather(data, indices, out, batch, outer, axis_dim, inner_bytes, num_indices, index_dtype, stream=None):

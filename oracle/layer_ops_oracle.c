@@ -35,6 +35,12 @@
  *                         Pinned by numpy.astype for every pair of types on values inside the range,
  *                         by torch for the roundings to f16 / bf16, and by hand-written cases for the
  *                         saturation, NaN and boolean rules.
+ *   oracle_binary_f32     Add / Subtract / Multiply / Divide with numpy broadcasting (src/ops/elementwise_binary.hpp:16-76,
+ *                         src/kernels/details/elementwise_binary.cuh:24-46), one fp32 operation per element.
+ *                         Pinned by numpy's own broadcasting arithmetic in float32, bit for bit.
+ *   oracle_softmax_f32    Softmax over the middle axis of [outer, length, inner] (src/ops/softmax.cpp:73-196)
+ *                         in fp64.  Pinned by scipy.special.softmax and torch.softmax in fp64, rows that sum
+ *                         to 1, shift invariance, and the uniform row.
  *   oracle_swish_f32 /    Swish (src/ops/swish.cpp:41-59) and OpenVINO's fused gated linear unit
  *   oracle_glu_f32        act(gate) * up with Swish, Gelu (erf) or Gelu (tanh).  Pinned by
  *                         torch.nn.functional.silu / gelu in fp64 (fixtures) and the explicit product.
@@ -230,4 +236,48 @@ ORACLE_API int oracle_convert(const void* in, void* out, int64_t count, int from
         }
     }
     return 0;
+}
+
+/* out = a (op) b, the three shapes given at one rank; op: 0 add, 1 subtract, 2 multiply, 3 divide */
+ORACLE_API int oracle_binary_f32(int op, const float* a, const float* b, float* out, int rank, const int64_t* out_dims,
+                                 const int64_t* a_dims, const int64_t* b_dims) {
+    if (rank < 0 || rank > 16) return 1;
+    int64_t sa[16], sb[16], coord[16], total = 1, ra = 1, rb = 1;
+    for (int k = rank - 1; k >= 0; k--) {
+        if ((a_dims[k] != out_dims[k] && a_dims[k] != 1) || (b_dims[k] != out_dims[k] && b_dims[k] != 1)) return 1;
+        sa[k] = a_dims[k] == 1 ? 0 : ra;
+        sb[k] = b_dims[k] == 1 ? 0 : rb;
+        ra *= a_dims[k];
+        rb *= b_dims[k];
+        total *= out_dims[k];
+        coord[k] = 0;
+    }
+    int64_t ia = 0, ib = 0;
+    for (int64_t i = 0; i < total; i++) {
+        const float x = a[ia], y = b[ib];
+        out[i] = op == 1 ? x - y : op == 2 ? x * y : op == 3 ? x / y : x + y;
+        for (int k = rank - 1; k >= 0; k--) {
+            ia += sa[k];
+            ib += sb[k];
+            if (++coord[k] < out_dims[k]) break;
+            ia -= sa[k] * out_dims[k];
+            ib -= sb[k] * out_dims[k];
+            coord[k] = 0;
+        }
+    }
+    return 0;
+}
+
+ORACLE_API void oracle_softmax_f32(const float* x, float* out, int64_t outer, int64_t length, int64_t inner) {
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t o = 0; o < outer; o++)
+        for (int64_t n = 0; n < inner; n++) {
+            const float* xr = x + o * length * inner + n;
+            float* yr = out + o * length * inner + n;
+            double m = -INFINITY, sum = 0.0;
+            for (int64_t i = 0; i < length; i++)
+                if ((double)xr[i * inner] > m) m = xr[i * inner];
+            for (int64_t i = 0; i < length; i++) sum += exp((double)xr[i * inner] - m);
+            for (int64_t i = 0; i < length; i++) yr[i * inner] = (float)(exp((double)xr[i * inner] - m) / sum);
+        }
 }

@@ -78,6 +78,10 @@ def lib():
         L.oracle_transpose_bytes.argtypes = [vp, vp, i32, vp, vp, i64]
         L.oracle_convert.restype = i32
         L.oracle_convert.argtypes = [vp, vp, i64, i32, i32]
+        L.oracle_binary_f32.restype = i32
+        L.oracle_binary_f32.argtypes = [i32, vp, vp, vp, i32, vp, vp, vp]
+        L.oracle_softmax_f32.restype = None
+        L.oracle_softmax_f32.argtypes = [vp, vp, i64, i64, i64]
         L.oracle_gather_bytes.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64]
         L.oracle_gather_bytes.restype = None
         L.oracle_concat_bytes.argtypes = [vp, vp, i32, i64, vp]
@@ -350,6 +354,29 @@ def convert(x, from_dtype, to_dtype):
     out = np.empty(x.shape, CONVERT_STORAGE[to_dtype])
     if lib().oracle_convert(_p(x), _p(out), x.size, from_dtype, to_dtype):
         raise ValueError("oracle_convert: unknown element type")
+    return out
+
+
+def binary(op, a, b):
+    """a (op) b with numpy broadcasting, one fp32 operation per element; op: 0 add, 1 subtract, 2 multiply, 3 divide."""
+    a, b = np.require(np.asarray(a, np.float32), requirements="C"), np.require(np.asarray(b, np.float32), requirements="C")
+    out_shape = np.broadcast_shapes(a.shape, b.shape)
+    n = len(out_shape)
+    pad = lambda s: np.array([1] * (n - len(s)) + list(s), np.int64)
+    out = np.empty(out_shape, np.float32)
+    od, ad, bd = pad(out_shape), pad(a.shape), pad(b.shape)
+    if lib().oracle_binary_f32(op, _p(a), _p(b), _p(out), n, _p(od), _p(ad), _p(bd)):
+        raise ValueError("oracle_binary_f32: shapes do not broadcast")
+    return out
+
+
+def softmax(x, axis=-1):
+    x = _c(x, np.float32)
+    axis = axis % x.ndim
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    out = np.empty_like(x)
+    lib().oracle_softmax_f32(_p(x), _p(out), outer, x.shape[axis], inner)
     return out
 
 

@@ -465,3 +465,95 @@ def test_convert_odd_addresses_in_place_and_errors(hip, ops, oracle):
     with pytest.raises(ops.HipOpsError) as e:
         ops.convert(dx, do, -1, 0, 1)
     assert e.value.status == hip.INVALID_ARGUMENT
+
+
+# ------------------------------------------------------------------------------ broadcasting arithmetic, Softmax
+BINARY_CASES = [((4, 8), (4, 8)), ((2, 3, 40, 64), (1, 1, 40, 64)), ((2, 3, 4, 5), (5,)), ((3, 1, 5), (1, 4, 1)), ((7,), ()), ((), ()),
+                ((2, 1, 16), (2, 3, 1)), ((1, 8), (5, 1)), ((64, 4096), (4096,)), ((64, 4096), (64, 1)), ((3, 5, 24), (3, 1, 24)),
+                ((2, 8, 130, 136), (2, 1, 1, 136)), ((2, 8, 130, 136), (1,)), ((0, 4), (1, 4))]
+
+
+@pytest.mark.parametrize("a_shape,b_shape", BINARY_CASES)
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+def test_binary_broadcasting(hip, ops, oracle, a_shape, b_shape, dtype):
+    rng = np.random.default_rng(len(a_shape) * 7 + len(b_shape))
+    print("[binary]", a_shape, b_shape, dtype, flush=True)
+    da, a = upload(hip, rng.standard_normal(a_shape), dtype)
+    db, b = upload(hip, rng.standard_normal(b_shape) + 3.0, dtype)  # away from zero: the divisor
+    out_shape = np.broadcast_shapes(a_shape, b_shape)
+    n = int(np.prod(out_shape, dtype=np.int64))
+    do = hip.DeviceBuffer(max(n, 1) * hip.DTYPE_BYTES[dtype])
+    for op in (ops.ADD, ops.SUBTRACT, ops.MULTIPLY, ops.DIVIDE):
+        for swap in (False, True):
+            x, y, dx, dy, xs, ys = (b, a, db, da, b_shape, a_shape) if swap else (a, b, da, db, a_shape, b_shape)
+            if swap and op == ops.DIVIDE:
+                continue  # a is not kept away from zero
+            do.fill(0xEE)
+            ops.binary(op, dx, dy, do, out_shape, xs, ys, dtype)
+            if n == 0:
+                continue
+            ref = oracle.round_to(oracle.binary(op, x, y), dtype).reshape(out_shape)
+            got = np.asarray(download(hip, do, dtype, out_shape)).reshape(out_shape)
+            # one fp32 operation, one rounding: the same bits (the oracle rounds its fp32 result the same way)
+            assert np.array_equal(got, ref), (op, swap, np.abs(got - ref).max())
+
+
+def test_binary_in_place_unaligned_and_errors(hip, ops, oracle):
+    rng = np.random.default_rng(4)
+    st, x = W.to_storage(rng.standard_normal((1 + 6 * 24,)).astype(np.float32), F16)
+    dx = hip.DeviceBuffer.from_numpy(st)
+    db, b = upload(hip, rng.standard_normal((24,)), F16)
+
+    class Shifted:  # two bytes in: the scalar path
+        ptr = ctypes.c_void_p(dx.ptr.value + 2)
+
+    ops.binary(ops.ADD, Shifted, db, Shifted, (6, 24), (6, 24), (24,), F16)  # in place on the full-shaped operand
+    got = H.storage_to_f32(dx.download(np.uint16, (1 + 6 * 24,)), F16)[1:].reshape(6, 24)
+    assert np.array_equal(got, oracle.round_to(oracle.binary(0, x[1:].reshape(6, 24), b), F16))
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.binary(ops.ADD, dx, db, dx, (6, 24), (6, 24), (23,), F16)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.binary(7, dx, db, dx, (6, 24), (6, 24), (24,), F16)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.binary(ops.ADD, dx, db, dx, (6, 24), (6, 24), (24,), ops.I64)
+    assert e.value.status == hip.UNSUPPORTED
+
+
+@pytest.mark.parametrize("shape,axis", [((5, 9), 1), ((5, 9), 0), ((2, 3, 4, 5), 2), ((2, 8, 130, 136), 3), ((3, 1000), 1), ((7,), 0),
+                                        ((64, 8192), 1), ((4, 33, 64), 1), ((2, 3, 0), 1), ((1, 1), 1)])
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+def test_softmax(hip, ops, oracle, shape, axis, dtype):
+    rng = np.random.default_rng(sum(shape) + axis)
+    print("[softmax]", shape, axis, dtype, flush=True)
+    dx, x = upload(hip, rng.standard_normal(shape) * 4, dtype)
+    n = int(np.prod(shape, dtype=np.int64))
+    do = hip.DeviceBuffer(max(n, 1) * hip.DTYPE_BYTES[dtype])
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    ops.softmax(dx, do, outer, shape[axis], inner, dtype)
+    if n == 0:
+        return
+    got = download(hip, do, dtype, shape)
+    ref = oracle.softmax(x, axis)
+    # probabilities are at most 1: absolute error of one rounding plus the fast exponential's few ulps
+    assert np.abs(got - ref).max() <= {F32: 2e-6, F16: 6e-4, BF16: 4.5e-3}[dtype]
+    ops.softmax(dx, dx, outer, shape[axis], inner, dtype)  # in place
+    assert np.array_equal(download(hip, dx, dtype, shape), got)
+
+
+def test_softmax_masked_entries_and_errors(hip, ops, oracle):
+    x = np.array([[0.0, -np.inf, 1.0, -np.inf, 0.5, -np.inf, -np.inf, -np.inf], [-np.inf] * 7 + [2.0], [-np.inf] * 8], np.float32)
+    dx = hip.DeviceBuffer.from_numpy(x)
+    do = hip.DeviceBuffer(x.nbytes)
+    ops.softmax(dx, do, 3, 8, 1, F32)
+    got = do.download(np.float32, x.shape)
+    ref = oracle.softmax(x, 1)
+    assert np.abs(got[:2] - ref[:2]).max() <= 2e-6 and np.isnan(got[2]).all() and np.isnan(ref[2]).all()
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.softmax(dx, do, 3, -1, 1, F32)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(ops.HipOpsError) as e:
+        ops.softmax(dx, do, 3, 8, 1, W.U8)
+    assert e.value.status == hip.UNSUPPORTED

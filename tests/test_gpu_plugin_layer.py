@@ -673,3 +673,90 @@ def test_sdpa_attention_block_with_split_heads(hip, oracle):
         err = scaled_error(got, ref)
         print("sdpa block %dx%d: scaled max error %.4g" % (B, L, err), flush=True)
         assert err <= 3e-2
+
+
+# ------------------------------------------------------------------------------ arithmetic, Softmax, decomposed attention
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_broadcasting_arithmetic_through_the_plugin(hip, oracle, dtype):
+    """(x * scale + bias - row) / column with numpy broadcasting, shapes changing from infer to infer."""
+    rng = np.random.default_rng(31)
+    g = P.GraphText("arith")
+    x = g.parameter("x", dtype, [-1, -1, 24])
+    row = g.parameter("row", dtype, [-1, 1, 24])
+    col = g.parameter("col", dtype, [-1, 1])
+    scale_st, scale = storage(np.array([0.25]), dtype)
+    bias_st, bias = storage(rng.standard_normal(24), dtype)
+    t = g.add("Multiply", "scaled", [x, g.constant("scale", scale_st, P._TYPE_NAMES[dtype])])
+    t = g.add("Add", "biased", [t, g.constant("bias", bias_st, P._TYPE_NAMES[dtype])])
+    t = g.add("Subtract", "centred", [t, row])
+    g.result("out", g.add("Divide", "divided", [t, col]))
+    plugin = P.Plugin()
+    assert {"scaled", "biased", "centred", "divided"} <= set(plugin.query_model(g.model()))
+    compiled = plugin.compile_model(g.model())
+    r = lambda a: oracle.round_to(a, dtype)
+    for B, L in ((2, 5), (1, 1), (3, 40)):
+        x_st, xv = storage(rng.standard_normal((B, L, 24)), dtype)
+        row_st, rv = storage(rng.standard_normal((B, 1, 24)), dtype)
+        col_st, cv = storage(rng.standard_normal((L, 1)) + 3.0, dtype)
+        out, _ = run(compiled, [(x_st, dtype), (row_st, dtype), (col_st, dtype)]).output(0)
+        ref = r(oracle.binary(3, r(oracle.binary(1, r(oracle.binary(0, r(oracle.binary(2, xv, scale)), bias)), rv)), cv))
+        assert out.shape == (B, L, 24) and np.array_equal(H.storage_to_f32(out, dtype), ref)
+    req = compiled.create_infer_request()
+    for i, a in enumerate((np.zeros((2, 5, 24)), np.zeros((3, 1, 24)), np.zeros((5, 1)))):
+        req.set_input(i, storage(a, dtype)[0], dtype)
+    with pytest.raises(P.PluginError) as e:  # batch 2 against batch 3
+        req.infer()
+    assert "centred" in str(e.value)
+
+
+@pytest.mark.parametrize("opset,axis,shape", [(8, -1, (2, 3, 40)), (8, 1, (2, 3, 40)), (1, 0, (5, 7)), (8, -2, (4, 9, 16))])
+def test_softmax_through_the_plugin(hip, oracle, opset, axis, shape):
+    rng = np.random.default_rng(32)
+    g = P.GraphText("softmax")
+    x = g.parameter("x", F16, [-1] * len(shape))
+    g.result("out", g.add("Softmax", "sm", [x], axis=axis, opset=opset))
+    compiled = P.Plugin().compile_model(g.model())
+    x_st, xv = storage(rng.standard_normal(shape) * 3, F16)
+    out, _ = run(compiled, [(x_st, F16)]).output(0)
+    assert out.shape == shape and np.abs(H.storage_to_f32(out, F16) - oracle.softmax(xv, axis)).max() <= 6e-4
+
+
+def decomposed_attention_graph(dtype, Hh, D, L, scale):
+    """Attention as the reference executes it once ScaledDotProductAttentionDecomposition has run
+    (transformer/cuda_graph_transformer.cpp:151-156): Multiply by the scale, Transpose of the keys,
+    MatMul, Add of the mask, Softmax, MatMul; beside it the fused operator on the same inputs."""
+    g = P.GraphText("decomposed")
+    q = g.parameter("q", dtype, [-1, Hh, -1, D])
+    k = g.parameter("k", dtype, [-1, Hh, -1, D])
+    v = g.parameter("v", dtype, [-1, Hh, -1, D])
+    mask = g.parameter("mask", dtype, [1, 1, -1, -1])
+    scale_st, _ = storage(np.array([scale]), dtype)
+    qs = g.add("Multiply", "scale_q", [q, g.constant("scale", scale_st, P._TYPE_NAMES[dtype])])
+    kt = g.add("Transpose", "k_t", [k, g.constant("order", np.array([0, 1, 3, 2], np.int64), "i64")])
+    scores = g.add("Add", "masked", [g.add("MatMul", "qk", [qs, kt], transpose_a=False, transpose_b=False), mask])
+    probs = g.add("Softmax", "softmax", [scores], axis=-1, opset=8)
+    g.result("decomposed", g.add("MatMul", "pv", [probs, v], transpose_a=False, transpose_b=False))
+    g.result("fused", g.add("ScaledDotProductAttention", "sdpa", [q, k, v], causal=True))
+    return g
+
+
+@pytest.mark.parametrize("dtype,B,Hh,L,D,tol", [(F32, 1, 8, 128, 64, 2e-5), (BF16, 2, 4, 200, 128, 1.5e-2), (F16, 1, 2, 77, 64, 3e-3)])
+def test_decomposed_attention_matches_the_fused_operator(hip, oracle, dtype, B, Hh, L, D, tol):
+    """The first case is the reference's own CPU-runnable configuration (fp32, 1 x 8 x 128 x 64, causal,
+    scale 1/sqrt(64)); both forms run on device "HIP" in one infer and are held against the oracle."""
+    rng = np.random.default_rng(33)
+    scale = 1.0 / np.sqrt(D)
+    g = decomposed_attention_graph(dtype, Hh, D, L, scale)
+    compiled = P.Plugin().compile_model(g.model())
+    q_st, q = storage(rng.standard_normal((B, Hh, L, D)), dtype)
+    k_st, k = storage(rng.standard_normal((B, Hh, L, D)), dtype)
+    v_st, v = storage(rng.standard_normal((B, Hh, L, D)), dtype)
+    big = -np.inf if dtype == F32 else -60000.0  # f16 has no room for more; exp of it is 0 all the same
+    mask_st, _ = storage(np.triu(np.full((L, L), big, np.float32), 1)[None, None], dtype)
+    req = run(compiled, [(q_st, dtype), (k_st, dtype), (v_st, dtype), (mask_st, dtype)])
+    outs = {name: H.storage_to_f32(req.output(i)[0], dtype) for i, name in enumerate(("decomposed", "fused"))}  # in the order of the results
+    ref = oracle.sdpa(q, k, v, causal=True)
+    for name in ("decomposed", "fused"):
+        err = float(np.abs(outs[name] - ref).max())
+        print("%s attention, dtype %d: max abs error %.3g" % (name, dtype, err), flush=True)
+        assert outs[name].shape == ref.shape and err <= tol, (name, err)

@@ -221,3 +221,48 @@ def test_convert_rules_c_leaves_open(oracle):
     np.testing.assert_array_equal(oracle.convert(np.array([0, 1, 2, 255], np.uint8), 104, 100), [0, 1, 1, 1])
     # 2^24 + 1 is not a float: to nearest even
     np.testing.assert_array_equal(oracle.convert(np.array([2**24 + 1, 2**24 + 3], np.int64), 101, 0), np.array([2**24, 2**24 + 4], np.float32))
+
+
+BROADCAST_CASES = [((4, 8), (4, 8)), ((2, 3, 4, 5), (1, 1, 4, 5)), ((2, 3, 4, 5), (5,)), ((3, 1, 5), (1, 4, 1)), ((7,), ()), ((), ()),
+                   ((2, 1, 6), (2, 3, 1)), ((1, 8), (5, 1)), ((0, 4), (1, 4))]
+
+
+@pytest.mark.parametrize("a_shape,b_shape", BROADCAST_CASES)
+@pytest.mark.parametrize("op", [0, 1, 2, 3])
+def test_binary_matches_numpy_broadcasting(oracle, a_shape, b_shape, op):
+    rng = np.random.default_rng(len(a_shape) * 10 + op)
+    a = rng.standard_normal(a_shape).astype(np.float32)
+    b = (rng.standard_normal(b_shape) + 3.0).astype(np.float32)
+    want = [np.add, np.subtract, np.multiply, np.divide][op](a, b)
+    got = oracle.binary(op, a, b)
+    assert got.shape == want.shape
+    np.testing.assert_array_equal(got, want)
+    got = oracle.binary(op, b, a + 5.0)  # operands the other way round
+    np.testing.assert_array_equal(got, [np.add, np.subtract, np.multiply, np.divide][op](b, a + 5.0))
+
+
+def test_binary_refuses_shapes_that_do_not_broadcast(oracle):
+    with pytest.raises(ValueError):
+        oracle.binary(0, np.zeros((2, 3), np.float32), np.zeros((2, 4), np.float32))
+
+
+@pytest.mark.parametrize("shape,axis", [((5, 9), 1), ((5, 9), 0), ((2, 3, 4, 5), 2), ((2, 3, 4, 5), -1), ((3, 1000), 1), ((7,), 0)])
+def test_softmax_matches_scipy_and_torch(oracle, shape, axis):
+    import scipy.special
+    import torch
+    rng = np.random.default_rng(sum(shape) + axis)
+    x = (rng.standard_normal(shape) * 6).astype(np.float32)
+    got = oracle.softmax(x, axis)
+    np.testing.assert_allclose(got, scipy.special.softmax(x.astype(np.float64), axis=axis), rtol=2e-7, atol=1e-12)
+    np.testing.assert_allclose(got, torch.softmax(torch.from_numpy(x).double(), axis).numpy(), rtol=2e-7, atol=1e-12)
+    np.testing.assert_allclose(got.astype(np.float64).sum(axis), 1.0, rtol=1e-6)
+    np.testing.assert_allclose(oracle.softmax(x + 100.0, axis), got, rtol=2e-5, atol=1e-9)  # shift invariance (x + 100 rounds)
+    np.testing.assert_allclose(oracle.softmax(np.full(shape, -3.5, np.float32), axis), 1.0 / shape[axis], rtol=1e-7)
+
+
+def test_softmax_with_masked_entries(oracle):
+    x = np.array([[0.0, -np.inf, 1.0, -np.inf], [-np.inf, -np.inf, -np.inf, 2.0]], np.float32)
+    got = oracle.softmax(x, 1)
+    e = np.exp(1.0)
+    np.testing.assert_allclose(got, [[1 / (1 + e), 0, e / (1 + e), 0], [0, 0, 0, 1]], rtol=1e-7)
+    assert np.isnan(oracle.softmax(np.full((1, 4), -np.inf, np.float32), 1)).all()

@@ -17,7 +17,7 @@ def declared_functions():
 
 def test_header_and_binding_agree():
     names = declared_functions()
-    assert len(names) == 13
+    assert len(names) == 15
     assert sorted(ops_capi.SYMBOLS) == names
 
 
@@ -37,7 +37,7 @@ def test_struct_layout_matches_header():
 
 def test_validation_needs_no_device():
     L = ops_capi.lib()
-    assert L.hipops_version() == 3
+    assert L.hipops_version() == 4
     n = ctypes.c_size_t(0)
     ok = ops_capi.MatmulDesc(capi.BF16, capi.BF16, 64, 6144, 4096, 1, 0, 1, 0, 0)
     assert L.hipops_matmul_workspace_size(ctypes.byref(ok), ctypes.byref(n)) == capi.OK and n.value == 32 << 20
@@ -59,3 +59,10 @@ def test_validation_needs_no_device():
     assert L.hipops_transpose(None, None, 9, dims, order, 2, None) == capi.INVALID_ARGUMENT
     assert L.hipops_convert(None, None, 8, capi.F32, 7, None) == capi.UNSUPPORTED
     assert L.hipops_convert(None, None, 0, capi.F32, ops_capi.I64, None) == capi.OK
+    d3 = (ctypes.c_int64 * 2)(4, 8)
+    d1 = (ctypes.c_int64 * 2)(4, 3)
+    assert L.hipops_binary(0, None, None, None, 2, d3, d3, d1, capi.F32, None) == capi.INVALID_ARGUMENT
+    assert b"broadcast" in L.hipops_last_error_string()
+    assert L.hipops_binary(9, None, None, None, 2, d3, d3, d3, capi.F32, None) == capi.INVALID_ARGUMENT
+    assert L.hipops_softmax(None, None, 4, 0, 1, capi.F16, None) == capi.OK
+    assert L.hipops_softmax(None, None, 4, 8, 1, ops_capi.I64, None) == capi.UNSUPPORTED

@@ -27,7 +27,7 @@ def test_registry_holds_the_attention_operators():
     ops = P.registered_operations()
     for name in ("Parameter", "Result", "Constant", "ScaledDotProductAttention", "PagedAttentionExtension", "ReadValue",
                  "Assign", "Add", "RMS", "RoPE", "MatMul", "Gather", "Concat", "Swish", "Multiply", "GLU", "Reshape", "Squeeze",
-                 "Unsqueeze", "Transpose", "Convert"):
+                 "Unsqueeze", "Transpose", "Convert", "Subtract", "Divide", "Softmax"):
         assert name in ops
 
 
