@@ -977,9 +977,12 @@ static int resident_decode_waves() {
 // evenly over the compute units 5-10 % slower.
 // Upper bound of the 128-row query tiles of the batch's multi-token sequences (the lengths stay
 // on the device): each such sequence has at least 2 tokens and wastes at most one tile.
+// 0 selects the row-per-token form of the plan, which takes the batch to hold as many rows as
+// sequences: only a batch with exactly that many tokens may get it (a single token spread over two
+// or more sequences, all but one of them empty, has a bound of 0 by the formula and must not).
 static int query_tile_bound(const PagedParams& p) {
     if (p.num_tokens == p.num_seqs && !p.any_lengths) return 0;  // one token per sequence: a pure decode batch
-    return p.num_tokens / 128 + std::min(p.num_seqs, p.num_tokens / 2);
+    return std::max(1, p.num_tokens / 128 + std::min(p.num_seqs, p.num_tokens / 2));
 }
 
 // Mixed batches run the decode kernel beside the chunks' flash kernel unless the caller fixed the

@@ -612,6 +612,27 @@ def test_paged_as_many_tokens_as_sequences_but_not_one_each(hip, oracle, flags):
             dev.free()
 
 
+@pytest.mark.parametrize("seqs", [[(33, 0), (33, 1)], [(0, 0), (5, 1), (7, 0)], [(64, 1), (10, 0)], [(3, 0), (0, 1)]])
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.BF16, W.U8])
+def test_paged_one_token_among_several_sequences(hip, oracle, seqs, cache_dtype):
+    """Fewer tokens than sequences: one sequence brings a token, the others none.  The plan must not
+    take the batch for one row per sequence (a second row would read beyond q and write beyond out and
+    into the cache position behind the token's)."""
+    announce("paged one token, several sequences", seqs, cache_dtype)
+    case = W.make_paged_case(77, seqs, 6, 3, 128, 32, W.BF16, W.BF16, cache_dtype, sliding_window=64)
+    assert case["T"] == 1 and case["S"] == len(seqs)
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    for flags in (0, hip.PA_ANY_LENGTHS):
+        dev = H.PagedDeviceCase(hip, case)
+        out, path = dev.run(flags=flags)
+        assert path == "paged_mfma"
+        kc, vc = dev.caches()
+        np.testing.assert_array_equal(kc, okc)
+        np.testing.assert_array_equal(vc, ovc)
+        assert H.max_abs(out, ref) <= (2e-2 if cache_dtype == W.BF16 else 1e-2)
+        dev.free()
+
+
 def test_paged_decode_row_with_an_empty_block_table_is_zeros(hip, oracle):
     """A single-token sequence whose block table is empty has nothing to attend: zeros on every path."""
     announce("paged decode empty table")
