@@ -88,6 +88,10 @@ __global__ __launch_bounds__(256) void binary_kernel(BinaryParams p) {
 }
 
 // ------------------------------------------------------------------------------ softmax
+// f32 tensors get the accurate exponential (the fast one's error grows with the argument, to a few
+// 1e-6 of the result at |x| = 30, which an f32 result shows and a 16-bit one does not)
+__device__ __forceinline__ float exp_of(int dtype, float x) { return dtype == HIPATTN_F32 ? expf(x) : __expf(x); }
+
 struct SoftmaxParams {
     const void* x;
     void* out;
@@ -121,22 +125,22 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxParams p) {
         if (m_new > -INFINITY) {  // a row of -inf so far keeps l = 0
             float add = 0.f;
 #pragma unroll
-            for (int k = 0; k < kPer; k++) add += __expf(v[k] - m_new);
-            l = l * __expf(m - m_new) + add;
+            for (int k = 0; k < kPer; k++) add += exp_of(p.dtype, v[k] - m_new);
+            l = l * exp_of(p.dtype, m - m_new) + add;
             m = m_new;
         }
     }
     const float row_max = wave_max(m);
-    l = row_max > -INFINITY ? l * __expf(m - row_max) : 0.f;
+    l = row_max > -INFINITY ? l * exp_of(p.dtype, m - row_max) : 0.f;
     const float inv = 1.0f / wave_sum(l);  // a row that is -inf throughout divides 0 by 0: NaN, as exp(-inf + inf) gives
     for (int64_t i = (int64_t)lane * kPer; i < p.length; i += 64 * kPer) {
         if constexpr (kWide) {
             Float8 r = load8(p.x, base + i, p.dtype);
 #pragma unroll
-            for (int k = 0; k < 8; k++) r.v[k] = __expf(r.v[k] - row_max) * inv;
+            for (int k = 0; k < 8; k++) r.v[k] = exp_of(p.dtype, r.v[k] - row_max) * inv;
             store8(p.out, base + i, p.dtype, r);
         } else {
-            store_scalar(p.out, base + i, p.dtype, __expf(load_scalar(p.x, base + i, p.dtype) - row_max) * inv);
+            store_scalar(p.out, base + i, p.dtype, exp_of(p.dtype, load_scalar(p.x, base + i, p.dtype) - row_max) * inv);
         }
     }
 }
@@ -168,7 +172,7 @@ __global__ __launch_bounds__(256) void softmax_kept_rows_kernel(SoftmaxParams p)
         if (i < p.length) {
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                keep[c].v[k] = __expf(keep[c].v[k] - m);  // a row of -inf throughout: exp(nan), as the other kernels give
+                keep[c].v[k] = exp_of(p.dtype, keep[c].v[k] - m);  // a row of -inf throughout: exp(nan), as the other kernels give
                 l += keep[c].v[k];
             }
         }
@@ -196,13 +200,13 @@ __global__ __launch_bounds__(256) void softmax_strided_kernel(SoftmaxParams p) {
         const float v = load_scalar(p.x, base + i * p.inner, p.dtype);
         const float m_new = fmaxf(m, v);
         if (m_new > -INFINITY) {
-            l = l * __expf(m - m_new) + __expf(v - m_new);
+            l = l * exp_of(p.dtype, m - m_new) + exp_of(p.dtype, v - m_new);
             m = m_new;
         }
     }
     const float inv = 1.0f / l;
     for (int64_t i = 0; i < p.length; i++)
-        store_scalar(p.out, base + i * p.inner, p.dtype, __expf(load_scalar(p.x, base + i * p.inner, p.dtype) - m) * inv);
+        store_scalar(p.out, base + i * p.inner, p.dtype, exp_of(p.dtype, load_scalar(p.x, base + i * p.inner, p.dtype) - m) * inv);
 }
 
 }  // namespace
