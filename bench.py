@@ -158,6 +158,41 @@ def bench_paged_scores(hip, case, steps, name):
                                  "the figure prices the two passes over the K rows against HBM"}}
 
 
+def bench_sdpa_masked(hip, steps):
+    """Configuration 2's shape with the causality spelt as an attention mask (an additive bf16 triangle of
+    -inf shared by all heads, causal flag off), as converted models carry it: the flash kernel with the
+    mask tile staged through LDS.  FLOPs are those of the full score matrix, which the kernel works
+    through (it cannot know that half of the mask is -inf)."""
+    from openvino_contrib_amd import workloads as W
+    import numpy as np
+
+    B, Hq, Hkv, L, D = 4, 32, 8, 2048, 128
+    case = W.make_sdpa_case(2, B, Hq, Hkv, L, L, D, W.BF16, std=0.5)
+    bufs = [hip.DeviceBuffer.from_numpy(case[n]) for n in ("q_store", "k_store", "v_store")]
+    out = hip.DeviceBuffer(case["q_store"].nbytes)
+    mask = hip.DeviceBuffer.from_numpy(W.to_storage(np.triu(np.full((L, L), -np.inf, np.float32), 1), W.BF16)[0])
+    desc = hip.SdpaDesc(W.BF16, B, Hq, Hkv, L, L, D, 0, 0.0)
+    call = lambda: hip.sdpa_masked(desc, bufs[0], bufs[1], bufs[2], W.BF16, [0, 0, L, 1], mask, out)
+    e0, e1 = hip.Event(), hip.Event()
+    for _ in range(300):  # clock ramp
+        call()
+    e0.record()
+    for _ in range(steps):
+        call()
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / steps
+    path = hip.last_kernel_path()
+    flops = 4.0 * B * Hq * L * L * D
+    a = flops / (ms * 1e-3) / 1e12
+    for b in bufs + [out, mask]:
+        b.free()
+    return {"workload": "SDPA bf16 B=4 Hq=32 Hkv=8 L=2048 D=128, causal flag off, additive bf16 mask [1,1,L,L]", "kernel_path": path,
+            "ms_per_step": ms, "dominant_kernel_ms": ms, "flops": flops, "tflops": a,
+            "roofline": {"bound": "mfma", "achieved": a, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": a / MFMA_BF16_PEAK_TFLOPS,
+                         "traffic": None, "kernel": "sdpa_flash_masked_kernel"}}
+
+
 def bench_paged_through_plugin(hip, case, steps, warmup):
     """The same step through the plugin layer: Plugin -> CompiledModel -> InferRequest::infer ->
     PagedAttentionOp -> C ABI, every tensor device-resident (remote tensors over the buffers of the raw
@@ -655,6 +690,9 @@ def main():
         del case
 
     if not args.no_extra:
+        results["c2_masked"] = bench_sdpa_masked(hip, args.steps)
+        log("c2's shape with the causality as an attention mask: %.3f ms, %.0f TFLOP/s (%s)"
+            % (results["c2_masked"]["ms_per_step"], results["c2_masked"]["tflops"], results["c2_masked"]["kernel_path"]))
         # the operators around attention, each with a roofline and a CPU figure of its own
         results.update(bench_layer_ops(hip, args.steps, args.warmup, not args.no_cpu))
 

@@ -145,7 +145,10 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * stride of 0 broadcasts that dimension.  dtype F32 / F16 / BF16: the value is added to the
  * scaled score; dtype U8: boolean, nonzero = the key takes part, zero = probability zero.  As the
  * operator specifies, the mask is ignored when desc->causal is set.  A query row whose keys are
- * all masked out yields zeros.  mask_desc and mask are both NULL or both set. */
+ * all masked out yields zeros.  mask_desc and mask are both NULL or both set.
+ * At head_dim 128 a mask of the operands' 16-bit type, or a boolean one, whose keys lie side by
+ * side (stride[3] == 1) stays on the matrix cores when the mask pointer and the other strides are
+ * multiples of 16 bytes (8 elements; 16 for boolean); other masks take the shape-generic kernel. */
 typedef struct hipattn_mask_desc {
     hipattn_dtype dtype;
     int64_t stride[4];

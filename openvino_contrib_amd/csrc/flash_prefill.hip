@@ -128,6 +128,11 @@ struct Tile {
     int64_t block_stride;   // paged: bytes between physical blocks
     int block_size;
     int block_shift;        // log2(block_size)
+    // dense SDPA with an attention mask (kMask variants of the kernel): the mask element of the
+    // tile's query row 0 and key 0 for this batch and head; rows mask_row_bytes apart (0: one row
+    // for every query), keys side by side
+    const uint8_t* mask;
+    int64_t mask_row_bytes;
 };
 
 // u8 caches: rows of 8 bytes (float scale, float zero-point) + 128 payload bytes.  The u8 variant
@@ -271,9 +276,14 @@ struct SoftmaxState {
 // Mask, reference update and probabilities of the tile that starts at key ts (register r of s[mt]
 // is key ts + mt*32 + 8*(r/4) + 4*hi + r%4).  `masked` is false for tiles that every query row of
 // the group sees completely (the common case).
-template <bool kBf16>
+// kMask: 0 no attention mask; 2 a mask of the operands' 16-bit type, added to the scaled scores;
+// 1 a boolean mask of one byte per key (zero: the key takes no part).  mask_lds: this wavefront's
+// 32 rows x 64 keys of the mask in LDS (mask_tile_* below), or nullptr for a tile that reaches past
+// the last key, whose mask values are fetched from global memory one by one.
+template <bool kBf16, int kMask = 0>
 __device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], float16_t (&o)[4], SoftmaxState& st,
-                                             typename Mfma<kBf16>::vec8 (&pf)[4], int ts, int my_pos, int hi, bool masked) {
+                                             typename Mfma<kBf16>::vec8 (&pf)[4], int ts, int my_pos, int hi, bool masked,
+                                             const lds_byte* mask_lds = nullptr, int row = 0) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     if (masked) {
@@ -287,6 +297,50 @@ __device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], f
                 if (t.window > 0) ok = ok && key > my_pos - t.window;
                 s[mt][r] = ok ? s[mt][r] : -INFINITY;
             }
+    }
+    if constexpr (kMask != 0) {
+        const int n32 = row & 31;
+        auto add16 = [&](uint32_t bits, float x) __attribute__((always_inline)) -> float {
+            const float m = kBf16 ? bf16_bits_to_float((uint16_t)bits) : f16_bits_to_float((uint16_t)bits);
+            return fmaf(m, kLog2e, x);  // the scores are exponents to base 2
+        };
+        if (mask_lds != nullptr) {
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    if constexpr (kMask == 2) {
+                        typedef __attribute__((address_space(3))) uint2_t lds_uint2;
+                        const int c = mt * 4 + g;
+                        const uint2_t w = *(const lds_uint2*)(mask_lds + n32 * 128 + ((c ^ (n32 & 7)) << 4) + hi * 8);
+                        s[mt][4 * g] = add16(w[0] & 0xffffu, s[mt][4 * g]);
+                        s[mt][4 * g + 1] = add16(w[0] >> 16, s[mt][4 * g + 1]);
+                        s[mt][4 * g + 2] = add16(w[1] & 0xffffu, s[mt][4 * g + 2]);
+                        s[mt][4 * g + 3] = add16(w[1] >> 16, s[mt][4 * g + 3]);
+                    } else {
+                        typedef __attribute__((address_space(3))) uint32_t lds_uint;
+                        const int c = mt * 2 + (g >> 1);
+                        const uint32_t w = *(const lds_uint*)(mask_lds + n32 * 64 + ((c ^ (n32 & 3)) << 4) + 8 * (g & 1) + 4 * hi);
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (((w >> (8 * e)) & 0xffu) == 0) s[mt][4 * g + e] = -INFINITY;
+                    }
+                }
+        } else if (row < t.rows) {
+            const uint8_t* mrow = t.mask + (int64_t)row * t.mask_row_bytes;
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+                    if (key < t.kv_len) {
+                        if constexpr (kMask == 2)
+                            s[mt][r] = add16(((const uint16_t*)mrow)[key], s[mt][r]);
+                        else if (mrow[key] == 0)
+                            s[mt][r] = -INFINITY;
+                    }
+                }
+        }
     }
     // probabilities of the tile against the current reference, and this lane's share of their sum
     auto probabilities = [&]() __attribute__((always_inline)) -> float {
@@ -532,8 +586,12 @@ __device__ __forceinline__ void wait_keeping_loads(int keep) {
     else
         wait_keeping<0>();
 }
-__device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0, 2 or 4 (wave-uniform)
-    if (keep >= 4)
+__device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is even, at most 8 (wave-uniform)
+    if (keep >= 8)
+        barrier_keeping<8>();
+    else if (keep >= 6)
+        barrier_keeping<6>();
+    else if (keep >= 4)
         barrier_keeping<4>();
     else if (keep >= 2)
         barrier_keeping<2>();
@@ -560,9 +618,10 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is 0,
 // read in phase 2j+1.  Between the barriers each group runs one matrix and one vector phase, in
 // opposite order, so that the matrix core and the vector units are both in use; the odd phase
 // boundaries are not enforced, the two groups only drift by what their phases differ in length.
-template <bool kBf16, bool kU8 = false, bool kPaged = true>
+template <bool kBf16, bool kU8 = false, bool kPaged = true, int kMask = 0>
 __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
     static_assert(kPaged || !kU8, "dense K/V are 16-bit");
+    static_assert(kMask == 0 || !kPaged, "attention masks belong to the dense operator");
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16");
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
@@ -590,6 +649,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         return;
     }
     auto unmasked = [&](int j) {
+        if constexpr (kMask != 0) return false;
         const int ts = kv_lo + j * kTileK;
         return (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
@@ -678,6 +738,28 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     };
     auto k_stage = [&](int j) { return k_ring + (j % kStages) * kKBytes; };
     auto v_stage = [&](int j) { return v_ring + (j % kStages) * kKBytes; };
+    // Attention mask: the wavefront's 32 query rows x the 64 keys of tile j go global -> LDS into one
+    // half of the wavefront's own stage (which holds query rows before the loop and output rows after
+    // it, and nothing in between), tile j into half j % 2, one tile ahead of its use.  16-bit masks:
+    // four loads, row r at r * 128 with its 16-byte chunk c at position c ^ (r % 8); boolean masks:
+    // two loads, row r at r * 64, chunk c at c ^ (r % 4).  A tile that reaches past the last key is
+    // not staged (a 16-byte piece would run past the mask row): tile_softmax reads it element-wise.
+    auto mask_tile_staged = [&](int j) { return kMask != 0 && j < n && kv_lo + (j + 1) * kTileK <= t.kv_len; };
+    auto mask_stage = [&](int j) { return wave_stage + (j & 1) * (kWaveStageBytes / 2); };
+    auto load_mask_tile = [&](int j) -> int {
+        if (!mask_tile_staged(j) || t.rows <= 0) return 0;
+        const int ts = kv_lo + j * kTileK;
+        constexpr int kLoads = kMask == 2 ? 4 : 2, kRowsPerLoad = 32 / kLoads, kChunks = 64 / kRowsPerLoad;
+#pragma unroll
+        for (int k = 0; k < kLoads; k++) {
+            const int r = kRowsPerLoad * k + lane / kChunks, q = lane % kChunks;
+            const int c = q ^ (r & (kChunks - 1));
+            const int qrow = min((wave & 3) * 32 + r, t.rows - 1);
+            const uint8_t* src = t.mask + (int64_t)qrow * t.mask_row_bytes + (int64_t)(ts * (kMask == 2 ? 2 : 1)) + (c << 4);
+            load_to_lds_16(src, mask_stage(j) + k * 1024);
+        }
+        return kLoads;
+    };
     // ---- u8 caches: lane l of wavefront w handles 16 payload bytes (piece l % 8) of row 8w + l / 8
     const int u8_row = 8 * wave + (lane >> 3), u8_piece = lane & 7;
     // address of this lane's row of tile j (entry: the block table entry of the wavefront's rows)
@@ -801,6 +883,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) asm volatile("" : "+v"(qf[i]));  // (converted before the wait below, not after)
+    if constexpr (kMask != 0) recent += load_mask_tile(0);  // the query rows have left the stage
     phase_barrier(recent);
     if (group == 1) phase_barrier(recent);  // group 1 sits out phase 0
 
@@ -844,7 +927,15 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         } else {
             recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
         }
-        tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
+        if constexpr (kMask != 0) {
+            recent += load_mask_tile(j + 1);
+            // tile j's mask was issued a vector phase ago, ahead of everything issued in this one
+            wait_keeping_loads(recent);
+            tile_softmax<kBf16, kMask>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, true,
+                                       mask_tile_staged(j) ? mask_stage(j) : nullptr, row);
+        } else {
+            tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
+        }
         // (the probabilities are complete before the barrier: the compiler may not move their
         // arithmetic into the matrix phase)
 #pragma unroll
@@ -961,10 +1052,18 @@ __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) 
     t.block_stride = 0;
     t.block_size = 1;
     t.block_shift = 0;
+    t.mask = nullptr;
+    t.mask_row_bytes = 0;
+    if (p.mask != nullptr) {
+        const int64_t esz = p.mask_dtype == HIPATTN_U8 ? 1 : 2;
+        t.mask = (const uint8_t*)p.mask +
+                 ((int64_t)b * p.mask_stride[0] + (int64_t)h * p.mask_stride[1] + (int64_t)t.pos0 * p.mask_stride[2]) * esz;
+        t.mask_row_bytes = p.mask_stride[2] * esz;
+    }
     return t;
 }
 
-template <bool kBf16, bool kU8 = false, bool kPaged = true>
+template <bool kBf16, bool kU8 = false, bool kPaged = true, int kMask = 0>
 __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t* lds, float scale) {
     int lo0, hi0, lo1, hi1;
     key_range(t0, lo0, hi0);
@@ -981,7 +1080,7 @@ __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t
         kv_hi = max(hi0, hi1);
     }
     const int group = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
-    run_pair<kBf16, kU8, kPaged>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
+    run_pair<kBf16, kU8, kPaged, kMask>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
 }
 
 template <bool kBf16>
@@ -989,6 +1088,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
     const Tile t0 = sdpa_group_tile(p, 0), t1 = sdpa_group_tile(p, 1);
     run_both<kBf16, false, false>(t0, t1, lds, p.scale);
+}
+
+// The same with an attention mask (kMask 2: of the operands' type, added; 1: boolean bytes).
+template <bool kBf16, int kMask>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_masked_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
+    const Tile t0 = sdpa_group_tile(p, 0), t1 = sdpa_group_tile(p, 1);
+    run_both<kBf16, false, false, kMask>(t0, t1, lds, p.scale);
 }
 
 // One workgroup per (128-row query tile of a multi-token sequence, pair of query heads) or, with an
@@ -1023,6 +1130,8 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
     t.block_stride = (int64_t)p.num_heads_kv * p.block_size * row_bytes;
     t.block_size = p.block_size;
     t.block_shift = __builtin_ctz(p.block_size);
+    t.mask = nullptr;
+    t.mask_row_bytes = 0;
     return t;
 }
 
@@ -1081,6 +1190,20 @@ bool sdpa_flash_supported(const SdpaParams& p) {
     return (int64_t)p.batch * p.num_heads_q * q_tiles < (int64_t(1) << 22);
 }
 
+// An attention mask the flash kernel takes: of the operands' type or boolean, its keys side by
+// side, and every 16-byte piece the kernel loads aligned (the mask itself, and the steps from row
+// to row, head to head and batch to batch; a step of 0 broadcasts).
+bool sdpa_flash_mask_supported(const SdpaParams& p) {
+    if (p.mask == nullptr || p.causal) return false;
+    if (p.mask_dtype != p.dtype && p.mask_dtype != HIPATTN_U8) return false;
+    if (p.mask_stride[3] != 1) return false;
+    const int64_t per16 = p.mask_dtype == HIPATTN_U8 ? 16 : 8;
+    if (((uintptr_t)p.mask & 15) != 0) return false;
+    for (int i = 0; i < 3; i++)
+        if (p.mask_stride[i] % per16 != 0) return false;
+    return true;
+}
+
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe) {
     if (p.batch == 0 || p.len_q == 0) return hipSuccess;
     const int G = p.num_heads_q / p.num_heads_kv;
@@ -1089,10 +1212,22 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
     const int per_kv_head = pair_heads ? (G / 2) * n_qt : G * ((n_qt + 1) / 2);
     dim3 grid(per_kv_head * p.num_heads_kv * p.batch);
     if (probe.before) (void)hipEventRecord(probe.before, stream);
-    if (p.dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
-    else
-        hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
+    const int mask = p.mask == nullptr ? 0 : (p.mask_dtype == HIPATTN_U8 ? 1 : 2);
+    if (p.dtype == HIPATTN_BF16) {
+        if (mask == 0)
+            hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
+        else if (mask == 2)
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 2>), grid, dim3(flash::kThreads), 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 1>), grid, dim3(flash::kThreads), 0, stream, p);
+    } else {
+        if (mask == 0)
+            hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
+        else if (mask == 2)
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<false, 2>), grid, dim3(flash::kThreads), 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<false, 1>), grid, dim3(flash::kThreads), 0, stream, p);
+    }
     hipError_t e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     return e;

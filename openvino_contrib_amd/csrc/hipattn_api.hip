@@ -404,8 +404,8 @@ HIPATTN_EXPORT hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc,
         p.mask_dtype = mask_desc->dtype;
         for (int i = 0; i < 4; i++) p.mask_stride[i] = mask_desc->stride[i];
     }
-    if (!p.mask && hipattn::sdpa_flash_supported(p)) {
-        g_kernel_path = "sdpa_flash_mfma";
+    if (hipattn::sdpa_flash_supported(p) && (!p.mask || hipattn::sdpa_flash_mask_supported(p))) {
+        g_kernel_path = p.mask ? "sdpa_flash_mfma_masked" : "sdpa_flash_mfma";
         HIP_TRY(hipattn::launch_sdpa_flash(p, as_stream(stream), g_probe));
     } else if (hipattn::sdpa_flash_small_supported(p)) {
         g_kernel_path = "sdpa_flash_mfma_d64";

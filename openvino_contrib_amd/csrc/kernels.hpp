@@ -134,6 +134,7 @@ hipError_t launch_paged_generic(const PagedParams& p, hipStream_t stream);
 
 // MFMA flash kernels (head_dim 64 or 128, f16 / bf16)
 bool sdpa_flash_supported(const SdpaParams& p);
+bool sdpa_flash_mask_supported(const SdpaParams& p);  // p.mask can ride along in the flash kernel
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
 // head size 64 on the matrix cores (flash_small.hip)
 bool sdpa_flash_small_supported(const SdpaParams& p);

@@ -32,13 +32,16 @@ def run_sdpa(hip, case, causal, scale=0.0):
     return storage_to_f32(res, case["dtype"]), path
 
 
-def run_sdpa_masked(hip, case, mask, scale=0.0):
-    """mask: numpy array broadcastable to [B,Hq,Lq,Lk]; bool (True = take part) or float32 / float16 (additive)."""
+def run_sdpa_masked(hip, case, mask, scale=0.0, mask_dtype=None):
+    """mask: numpy array broadcastable to [B,Hq,Lq,Lk]; bool (True = take part) or float32 / float16 (additive).
+    mask_dtype W.F16 / W.BF16 stores a float mask in that type (rounded to nearest)."""
     desc = hip.SdpaDesc(case["dtype"], case["B"], case["Hq"], case["Hkv"], case["Lq"], case["Lk"], case["D"], 0, scale)
     m = np.asarray(mask)
     while m.ndim < 4:
         m = m[None]
-    if m.dtype == np.bool_:
+    if m.dtype != np.bool_ and mask_dtype in (W.F16, W.BF16):
+        store, mdtype = np.ascontiguousarray(W.to_storage(np.asarray(m, np.float32), mask_dtype)[0]), mask_dtype
+    elif m.dtype == np.bool_:
         store, mdtype = np.ascontiguousarray(m.astype(np.uint8)), W.U8
     elif m.dtype == np.float16:
         store, mdtype = np.ascontiguousarray(m).view(np.uint16), W.F16

@@ -282,6 +282,47 @@ def test_sdpa_with_attention_mask(hip, oracle, dtype, tol, mask_kind):
         assert H.max_abs(out, oracle.sdpa(case["q"], case["k"], case["v"])) <= tol
 
 
+FLASH_MASKS = ["full", "per_batch", "shared", "key_padding", "causal_inf", "bool_shared", "bool_per_batch", "bool_padding"]
+
+
+@pytest.mark.parametrize("dtype", [W.F16, W.BF16])
+@pytest.mark.parametrize("kind", FLASH_MASKS)
+@pytest.mark.parametrize("B,Hq,Hkv,Lq,Lk", [(2, 4, 2, 300, 512), (1, 3, 1, 130, 208), (2, 2, 2, 64, 1000), (1, 8, 2, 1000, 64),
+                                            (1, 2, 1, 5, 48)])
+def test_sdpa_flash_with_mask(hip, oracle, dtype, kind, B, Hq, Hkv, Lq, Lk):
+    """Head size 128 with an attention mask of the operands' type or a boolean one stays on the matrix
+    cores: full, per-batch and shared masks, a key-padding mask (one row for all queries), an additive
+    triangle of -inf (how converted models spell causality), rows that are masked out altogether, and
+    key counts off the 64-key tile (the last tile's mask values are read one by one)."""
+    announce("sdpa flash mask", dtype, kind, B, Hq, Hkv, Lq, Lk)
+    rng = np.random.default_rng(Lq * 7 + Lk + len(kind))
+    case = W.make_sdpa_case(71, B, Hq, Hkv, Lq, Lk, 128, dtype, std=0.5 if dtype == W.BF16 else 1.0)
+    shape = {"full": (B, Hq, Lq, Lk), "per_batch": (B, 1, Lq, Lk), "shared": (Lq, Lk), "key_padding": (B, 1, 1, Lk),
+             "causal_inf": (1, 1, Lq, Lk), "bool_shared": (Lq, Lk), "bool_per_batch": (B, 1, Lq, Lk), "bool_padding": (B, 1, 1, Lk)}[kind]
+    if kind.startswith("bool"):
+        mask = rng.random(shape) < 0.7
+        mask[..., 0] = True
+        if kind == "bool_shared" and Lq > 3:
+            mask[3] = False  # a row with nothing to attend: zeros
+    elif kind == "causal_inf":
+        mask = np.triu(np.full((Lq, Lk), -np.inf, np.float32), 1 + max(Lk - Lq, 0))[None, None]
+    else:
+        mask = (rng.standard_normal(shape) * 2).astype(np.float32)
+        if kind == "key_padding":
+            mask[..., Lk - Lk // 4:] = -np.inf
+    out, path = H.run_sdpa_masked(hip, case, mask, mask_dtype=dtype)
+    per16 = 16 if kind.startswith("bool") else 8
+    if Lk % per16 == 0:
+        assert path == "sdpa_flash_mfma_masked"
+    else:
+        assert path == "sdpa_generic"
+    ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask if kind.startswith("bool") else oracle.round_to(mask, dtype))
+    assert np.isfinite(out).all()
+    rows = np.isfinite(ref).all(-1)  # a row without a key is zeros here and undefined in the oracle
+    assert not out[~rows].any()
+    assert H.max_abs(out[rows], ref[rows]) <= (1e-2 if dtype == W.BF16 else 2e-3)
+
+
 def test_sdpa_mask_is_ignored_when_causal_and_masked_rows_are_zeros(hip, oracle):
     announce("sdpa mask causal / empty rows")
     case = W.make_sdpa_case(63, 1, 8, 2, 200, 200, 128, W.BF16, std=0.5)
