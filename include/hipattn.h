@@ -148,7 +148,8 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * all masked out yields zeros.  mask_desc and mask are both NULL or both set.
  * At head_dim 128 a mask of the operands' 16-bit type, or a boolean one, whose keys lie side by
  * side (stride[3] == 1) stays on the matrix cores when the mask pointer and the other strides are
- * multiples of 16 bytes (8 elements; 16 for boolean); other masks take the shape-generic kernel. */
+ * multiples of 16 bytes (8 elements; 16 for boolean); at head_dim 64 every mask does; other
+ * combinations take the shape-generic kernel. */
 typedef struct hipattn_mask_desc {
     hipattn_dtype dtype;
     int64_t stride[4];

@@ -4,8 +4,9 @@
 // flash_prefill.hip -- S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16, the accumulator of the
 // first being the B operand of the second -- in a plain structure: four wavefronts per workgroup,
 // 32 query rows each, key tiles of 64 staged through registers into a double-buffered, swizzled LDS
-// tile, one workgroup barrier per tile, a straightforward online softmax.  Not tuned beyond
-// conflict-free LDS access; it replaces the fp32 VALU kernel for these shapes.
+// tile, one workgroup barrier per tile, a straightforward online softmax, an optional attention mask
+// of any type the operator allows.  Not tuned beyond conflict-free LDS access; it replaces the fp32
+// VALU kernel for these shapes.
 //
 // Replaces the same decomposed chain as flash_prefill.hip (src/ops/matmul.cpp:185-227,
 // src/ops/softmax.cpp:178-193, src/ops/select.cpp:50-91 of the reference).
@@ -90,7 +91,48 @@ __device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte
     return __builtin_bit_cast(typename Mfma<kBf16>::vec8, a);
 }
 
-template <bool kBf16>
+// The attention-mask values of one query row for the four consecutive keys key .. key + 3, as
+// additions to scores that are exponents to base 2: a floating mask times log2(e), a boolean one 0
+// or -inf.  One 4-, 8- or 16-byte load where the keys lie side by side, all four exist and the
+// address allows it; element by element otherwise (keys past the end give 0: they are masked anyway).
+__device__ __forceinline__ void mask_values4(const uint8_t* row, int64_t key_stride, int dtype, int key, int len_kv, float (&m)[4]) {
+    const int esz = dtype == HIPATTN_U8 ? 1 : (dtype == HIPATTN_F32 ? 4 : 2);
+    auto value = [&](uint32_t bits) __attribute__((always_inline)) -> float {
+        if (dtype == HIPATTN_U8) return bits ? 0.0f : -INFINITY;
+        const float x = dtype == HIPATTN_F32 ? __uint_as_float(bits)
+                                             : (dtype == HIPATTN_F16 ? f16_bits_to_float((uint16_t)bits) : bf16_bits_to_float((uint16_t)bits));
+        return x * kLog2e;
+    };
+    const uint8_t* at = row + (int64_t)key * key_stride * esz;
+    if (key_stride == 1 && key + 3 < len_kv && ((uintptr_t)at & (4 * esz - 1)) == 0) {
+        if (esz == 1) {
+            const uint32_t w = *(const uint32_t*)at;
+#pragma unroll
+            for (int e = 0; e < 4; e++) m[e] = value((w >> (8 * e)) & 0xffu);
+        } else if (esz == 2) {
+            const uint2_t w = *(const uint2_t*)at;
+#pragma unroll
+            for (int e = 0; e < 4; e++) m[e] = value((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        } else {
+            const uint4_t w = *(const uint4_t*)at;
+#pragma unroll
+            for (int e = 0; e < 4; e++) m[e] = value(w[e]);
+        }
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        m[e] = 0.0f;
+        if (key + e < len_kv) {
+            const uint8_t* one = row + (int64_t)(key + e) * key_stride * esz;
+            m[e] = value(esz == 1 ? (uint32_t)*one : (esz == 2 ? (uint32_t) * (const uint16_t*)one : *(const uint32_t*)one));
+        }
+    }
+}
+
+// kMask: the call carries an attention mask (p.mask, ignored under the causal flag): its values are
+// fetched from global memory ahead of the score product of every tile and added behind it.
+template <bool kBf16, bool kMask = false>
 __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams p) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
@@ -168,6 +210,22 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
         const lds_byte* v_lds = (const lds_byte*)lds[buf][1];
         const int ts = j * kTileK;
 
+        float16_t mask_add[2];
+        if constexpr (kMask) {
+            const int row = min(my_row, p.len_q - 1);
+            const int esz = p.mask_dtype == HIPATTN_U8 ? 1 : (p.mask_dtype == HIPATTN_F32 ? 4 : 2);
+            const uint8_t* mrow = (const uint8_t*)p.mask +
+                                  ((int64_t)b * p.mask_stride[0] + (int64_t)h * p.mask_stride[1] + (int64_t)row * p.mask_stride[2]) * esz;
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    float m4[4];
+                    mask_values4(mrow, p.mask_stride[3], p.mask_dtype, ts + mt * 32 + 8 * g + 4 * hi, p.len_kv, m4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) mask_add[mt][4 * g + e] = m4[e];
+                }
+        }
         // scores, transposed: register r of s[mt] is key ts + 32 mt + 8 (r / 4) + 4 hi + r % 4 of query row n32
         float16_t s[2];
 #pragma unroll
@@ -180,6 +238,10 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
                 const vec8 kf = __builtin_bit_cast(vec8, *(const __attribute__((address_space(3))) uint4_t*)(k_lds + k_chunk_offset(row, 2 * i + hi)));
                 s[mt] = M::mma(kf, qf[i], s[mt]);
             }
+        }
+        if constexpr (kMask) {
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++) s[mt] += mask_add[mt];
         }
         // mask: keys past the end, and keys after the query under the causal flag
         const bool edge = ts + kTileK > p.len_kv || (p.causal && ts + kTileK - 1 > q0 + wave * 32);
@@ -257,7 +319,7 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
 }  // namespace flash_small
 
 bool sdpa_flash_small_supported(const SdpaParams& p) {
-    return p.head_dim == flash_small::kD && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16) && p.mask == nullptr &&
+    return p.head_dim == flash_small::kD && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16) &&
            p.len_kv > 0 && p.len_q > 0 && ((uintptr_t)p.q % 16) == 0 && ((uintptr_t)p.k % 16) == 0 &&
            ((uintptr_t)p.v % 16) == 0 && ((uintptr_t)p.out % 8) == 0;
 }
@@ -267,6 +329,13 @@ hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream) {
     const int64_t groups = q_tiles * p.num_heads_q * p.batch;
     if (groups == 0) return hipSuccess;
     if (groups > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (p.mask != nullptr && !p.causal) {
+        if (p.dtype == HIPATTN_BF16)
+            hipLaunchKernelGGL((flash_small::sdpa_flash_d64_kernel<true, true>), dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::sdpa_flash_d64_kernel<false, true>), dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+        return hipGetLastError();
+    }
     if (p.dtype == HIPATTN_BF16)
         hipLaunchKernelGGL(flash_small::sdpa_flash_d64_kernel<true>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
     else

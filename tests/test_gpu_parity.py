@@ -323,6 +323,41 @@ def test_sdpa_flash_with_mask(hip, oracle, dtype, kind, B, Hq, Hkv, Lq, Lk):
     assert H.max_abs(out[rows], ref[rows]) <= (1e-2 if dtype == W.BF16 else 2e-3)
 
 
+@pytest.mark.parametrize("dtype", [W.F16, W.BF16])
+@pytest.mark.parametrize("kind", ["f32_full", "same_type_shared", "bool_per_batch", "f32_key_padding", "per_head_constant", "causal_inf"])
+@pytest.mark.parametrize("B,Hq,Hkv,Lq,Lk", [(2, 4, 2, 300, 513), (1, 3, 1, 130, 208), (1, 2, 1, 5, 47)])
+def test_sdpa_d64_with_mask(hip, oracle, dtype, kind, B, Hq, Hkv, Lq, Lk):
+    """Head size 64 with an attention mask of any type and layout the operator allows stays on the
+    matrix cores (the mask values are fetched from global memory, four keys at a time where the layout
+    allows): fp32 masks beside 16-bit operands, odd key counts and strides of 0 included."""
+    announce("sdpa d64 mask", dtype, kind, B, Hq, Hkv, Lq, Lk)
+    rng = np.random.default_rng(Lq + 3 * Lk + len(kind))
+    case = W.make_sdpa_case(72, B, Hq, Hkv, Lq, Lk, 64, dtype, std=0.5 if dtype == W.BF16 else 1.0)
+    mask_dtype = None
+    if kind == "f32_full":
+        mask = (rng.standard_normal((B, Hq, Lq, Lk)) * 2).astype(np.float32)
+    elif kind == "same_type_shared":
+        mask, mask_dtype = (rng.standard_normal((Lq, Lk)) * 2).astype(np.float32), dtype
+    elif kind == "bool_per_batch":
+        mask = rng.random((B, 1, Lq, Lk)) < 0.6
+        mask[..., 0] = True
+        mask[:, :, min(3, Lq - 1)] = False  # a row with nothing to attend: zeros
+    elif kind == "f32_key_padding":
+        mask = np.zeros((B, 1, 1, Lk), np.float32)
+        mask[..., Lk - Lk // 3:] = -np.inf
+    elif kind == "per_head_constant":
+        mask = rng.standard_normal((1, Hq, 1, 1)).astype(np.float32)  # key stride 0
+    else:
+        mask, mask_dtype = np.triu(np.full((Lq, Lk), -np.inf, np.float32), 1 + max(Lk - Lq, 0))[None, None], dtype
+    out, path = H.run_sdpa_masked(hip, case, mask, mask_dtype=mask_dtype)
+    assert path == "sdpa_flash_mfma_d64"
+    ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask if (mask.dtype == np.bool_ or mask_dtype is None) else oracle.round_to(mask, mask_dtype))
+    assert np.isfinite(out).all()
+    rows = np.isfinite(ref).all(-1)
+    assert not out[~rows].any()
+    assert H.max_abs(out[rows], ref[rows]) <= (1e-2 if dtype == W.BF16 else 2e-3)
+
+
 def test_sdpa_mask_is_ignored_when_causal_and_masked_rows_are_zeros(hip, oracle):
     announce("sdpa mask causal / empty rows")
     case = W.make_sdpa_case(63, 1, 8, 2, 200, 200, 128, W.BF16, std=0.5)
