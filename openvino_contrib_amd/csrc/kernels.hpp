@@ -107,13 +107,14 @@ struct PagedParams {
     int overlap;          // 0: decode, merge and prefill kernels run one after the other
     float overlap_share;
     int32_t* plan_waves;  // [1]
-    int32_t* blk_prefix;  // [num_seqs + 1] exclusive prefix of work-line units of decode sequences
-    void* seq_info;       // [num_seqs] 32-byte records: what each decode sequence attends (written by the plan)
-    float* part_out;      // [num_waves + dyn_pieces + num_seqs*num_heads_kv, G, head_dim] unnormalised outputs
+    int32_t* blk_prefix;  // [num_rows + 1] exclusive prefix of work-line units of the decode rows
+    void* seq_info;       // [num_rows] 32-byte records: what each decode row attends (written by the plan)
+    float* part_out;      // [num_waves + dyn_pieces + num_rows*num_heads_kv, G, head_dim] unnormalised outputs
     float* part_ml;       // [same, G, 2] running max (log2 domain) and sum
     // chunked prefill: query-tile schedule built on the device
     int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
     int max_q_tiles;      // grid upper bound
+    int num_rows;         // records of the decode plan: the sequences, or (max_q_tiles == 0) the tokens
     int any_lengths;      // a batch with num_tokens == num_seqs sends its multi-token sequences to the
                           // chunked-prefill kernel too (HIPATTN_PA_ANY_LENGTHS); without it such a batch is
                           // planned per token and every token is a decode row

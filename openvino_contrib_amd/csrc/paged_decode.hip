@@ -107,10 +107,12 @@ __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int i)
     bool single = true;
     // everything a row of an ordinary decode batch needs is fetched at once, on the guess that row i is
     // sequence i (one level of memory latency instead of two); a guess that fails is redone below
-    const int b0 = p.subsequence_begins[i], b1 = p.subsequence_begins[i + 1];
-    int tb0 = p.block_indices_begins[i], tb1 = p.block_indices_begins[i + 1], past = p.past_lens[i];
+    // (rows beyond the last sequence exist only when rows are tokens: the guess is then made on the last sequence)
+    const int ig = min(i, p.num_seqs - 1);
+    const int b0 = p.subsequence_begins[ig], b1 = p.subsequence_begins[ig + 1];
+    int tb0 = p.block_indices_begins[ig], tb1 = p.block_indices_begins[ig + 1], past = p.past_lens[ig];
     if (p.max_q_tiles == 0) {
-        if (!(b0 == i && b1 == i + 1)) {
+        if (!(ig == i && b0 == i && b1 == i + 1)) {
             s = sequence_of_token(p, i);
             tb0 = p.block_indices_begins[s];
             tb1 = p.block_indices_begins[s + 1];
@@ -118,6 +120,8 @@ __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int i)
         }
         pos_in_seq = i - p.subsequence_begins[s];
         r.token = i;
+        // a token outside every sequence (padding in front of the first or behind the last): no row at all
+        single = i >= p.subsequence_begins[0] && i < p.subsequence_begins[p.num_seqs];
     } else {
         r.token = b0;
         single = (b1 - b0 == 1);
@@ -437,12 +441,13 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
     __shared__ float wave_keys[4];
     const int tid = threadIdx.x;
     if (tid < 64) p.dyn_counter[tid] = 0;  // tickets for the dynamic pieces of this call, one counter per group
-    const int per = (p.num_seqs + 255) / 256;
-    const int s0 = min(tid * per, p.num_seqs), s1 = min(s0 + per, p.num_seqs);
+    const int per = (p.num_rows + 255) / 256;
+    const int s0 = min(tid * per, p.num_rows), s1 = min(s0 + per, p.num_rows);
     int blk = 0, tile = 0;
     float key_tiles = 0.0f;  // 64-key tiles the flash kernel works through, summed over 128-row query tiles
     for (int s = s0; s < s1; s++) {
-        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
+        // (rows are sequences whenever the lengths matter here: max_q_tiles > 0)
+        const int qlen = p.max_q_tiles > 0 ? p.subsequence_begins[s + 1] - p.subsequence_begins[s] : 1;
         blk += line_units(decode_range(p, s).nb, p.switch_cost);
         tile += (qlen > 1 && p.max_q_tiles > 0) ? (qlen + 127) / 128 : 0;
         if (p.overlap && qlen > 1) {
@@ -502,7 +507,7 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
     blk = ahead_blk + scan_blk - blk;
     tile = ahead_tile + scan_tile - tile;
     for (int s = s0; s < s1; s++) {
-        const int qlen = p.subsequence_begins[s + 1] - p.subsequence_begins[s];
+        const int qlen = p.max_q_tiles > 0 ? p.subsequence_begins[s + 1] - p.subsequence_begins[s] : 1;
         p.blk_prefix[s] = blk;
         p.tile_prefix[s] = tile;
         const DecodeRange rg = decode_range(p, s);
@@ -511,9 +516,9 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
         blk += line_units(rg.nb, p.switch_cost);
         tile += (qlen > 1 && p.max_q_tiles > 0) ? (qlen + 127) / 128 : 0;
     }
-    if (s1 == p.num_seqs && s0 < p.num_seqs) {
-        p.blk_prefix[p.num_seqs] = blk;
-        p.tile_prefix[p.num_seqs] = tile;
+    if (s1 == p.num_rows && s0 < p.num_rows) {
+        p.blk_prefix[p.num_rows] = blk;
+        p.tile_prefix[p.num_rows] = tile;
     }
 }
 
@@ -641,11 +646,11 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     __shared__ int plan_prefix[kSelfPlan ? kSelfPlanMaxRows + 1 : 1];
     if constexpr (kSelfPlan) {
         int carry = 0;
-        for (int base = 0; base < p.num_seqs; base += 64) {
+        for (int base = 0; base < p.num_rows; base += 64) {
             const int i = base + lane;
             DecodeRange rg;
             int units = 0;
-            if (i < p.num_seqs) {
+            if (i < p.num_rows) {
                 rg = decode_range(p, i);
                 units = line_units(rg.nb, p.switch_cost);
                 plan_rec[i] = rg;
@@ -656,7 +661,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                 const int up = __shfl_up(scan, d, 64);
                 if (lane >= d) scan += up;
             }
-            if (i < p.num_seqs) {
+            if (i < p.num_rows) {
                 plan_prefix[i] = carry + scan - units;
                 if (w == 0) {  // for the merge kernel
                     ((DecodeRange*)p.seq_info)[i] = rg;
@@ -667,8 +672,8 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
             carry += __shfl(scan, 63, 64);
         }
         if (lane == 0) {
-            plan_prefix[p.num_seqs] = carry;
-            if (w == 0) p.blk_prefix[p.num_seqs] = carry;
+            plan_prefix[p.num_rows] = carry;
+            if (w == 0) p.blk_prefix[p.num_rows] = carry;
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the records are in LDS (the wavefront is the whole workgroup)
         __builtin_amdgcn_wave_barrier();
@@ -679,7 +684,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         else
             return p.blk_prefix[i];
     };
-    const int64_t total = (int64_t)prefix_at(p.num_seqs) * Hkv;
+    const int64_t total = (int64_t)prefix_at(p.num_rows) * Hkv;
     if (total <= 0) return;
     // eight to a workgroup: the plan has chosen how many of the launched wavefronts work
     const int num_waves = kWaves == 1 ? p.num_waves : p.plan_waves[0];
@@ -706,18 +711,18 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         if constexpr (kSelfPlan) {  // the last row whose prefix is <= L / Hkv (the prefix is monotone)
             const int x = (int)(L / Hkv);
             int cnt = 0;
-            for (int base = 0; base < p.num_seqs; base += 64) {
+            for (int base = 0; base < p.num_rows; base += 64) {
                 const int i = base + lane;
-                cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(i < p.num_seqs && plan_prefix[i] <= x));
+                cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(i < p.num_rows && plan_prefix[i] <= x));
             }
             s = max(cnt - 1, 0);
         } else {
-            s = locate_sequence(p.blk_prefix, p.num_seqs, (int)(L / Hkv), lane);
+            s = locate_sequence(p.blk_prefix, p.num_rows, (int)(L / Hkv), lane);
         }
     }
 
     while (L < L_end) {
-        while (s + 1 < p.num_seqs && (int64_t)prefix_at(s + 1) * Hkv <= L) s++;  // next sequence with blocks
+        while (s + 1 < p.num_rows && (int64_t)prefix_at(s + 1) * Hkv <= L) s++;  // next row with blocks
         DecodeRange rg;
         if constexpr (kSelfPlan)
             rg = plan_rec[s];
@@ -890,7 +895,7 @@ __global__ __launch_bounds__(256) void paged_merge_kernel(PagedParams p) {
     const int s = blockIdx.x / Hkv, h = blockIdx.x % Hkv;  // one workgroup per segment
     const DecodeRange rg = ((const DecodeRange*)p.seq_info)[s];
     if (rg.nb <= 0) return;
-    const int64_t total = (int64_t)p.blk_prefix[p.num_seqs] * Hkv;
+    const int64_t total = (int64_t)p.blk_prefix[p.num_rows] * Hkv;
     if (total <= 0) return;
     const Line line(total, p.overlap ? p.plan_waves[0] : p.num_waves, p.dyn_pieces);
     const int seglen = rg.nb + p.switch_cost;
@@ -987,6 +992,9 @@ static int query_tile_bound(const PagedParams& p) {
 
 // Mixed batches run the decode kernel beside the chunks' flash kernel unless the caller fixed the
 // number of decode wavefronts or the option mixed_overlap = 0 asks for one kernel after the other.
+// Records of the decode plan: one per sequence, or one per token when the batch is planned per token.
+static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p.num_tokens : p.num_seqs; }
+
 static bool overlap_wanted(const PagedParams& p) {
     if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
     return option(kOptMixedOverlap) != 0;
@@ -1014,8 +1022,9 @@ size_t paged_fast_workspace_bytes(const PagedParams& p) {
     const bool overlap = overlap_wanted(p);
     const int W = choose_num_waves(p, overlap);
     const int G = p.num_heads_q / p.num_heads_kv;
-    const size_t slots = (size_t)W + choose_dyn_pieces(W, overlap) + (size_t)p.num_seqs * p.num_heads_kv;
-    return 512 + 2 * align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256) + align_up((size_t)p.num_seqs * 32, 256) +
+    const size_t rows = (size_t)plan_rows(p);
+    const size_t slots = (size_t)W + choose_dyn_pieces(W, overlap) + rows * p.num_heads_kv;
+    return 512 + 2 * align_up((rows + 1) * sizeof(int32_t), 256) + align_up(rows * 32, 256) +
            align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
 }
 
@@ -1029,23 +1038,24 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     p.overlap_share = option(kOptSharePercent) / 100.0f;
     p.dyn_groups = std::min(64, std::max(1, p.num_waves / 32));  // every group has at least one wavefront
     const int G = p.num_heads_q / p.num_heads_kv;
-    const size_t slots = (size_t)p.num_waves + p.dyn_pieces + (size_t)p.num_seqs * p.num_heads_kv;
+    p.max_q_tiles = query_tile_bound(p);
+    p.num_rows = plan_rows(p);
+    const size_t slots = (size_t)p.num_waves + p.dyn_pieces + (size_t)p.num_rows * p.num_heads_kv;
     uint8_t* w = (uint8_t*)workspace;
     p.dyn_counter = (int32_t*)w;
     w += 256;
     p.plan_waves = (int32_t*)w;
     w += 256;
     p.tile_prefix = (int32_t*)w;
-    w += align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
+    w += align_up(((size_t)p.num_rows + 1) * sizeof(int32_t), 256);
     p.blk_prefix = (int32_t*)w;
-    w += align_up(((size_t)p.num_seqs + 1) * sizeof(int32_t), 256);
+    w += align_up(((size_t)p.num_rows + 1) * sizeof(int32_t), 256);
     p.seq_info = w;
-    w += align_up((size_t)p.num_seqs * 32, 256);
+    w += align_up((size_t)p.num_rows * 32, 256);
     p.part_out = (float*)w;
     w += align_up(slots * G * kD * sizeof(float), 256);
     p.part_ml = (float*)w;
     w += align_up(slots * G * 2 * sizeof(float), 256);
-    p.max_q_tiles = query_tile_bound(p);
 }
 
 // ---- scratch of the entry point that allocates nothing (hipattn_paged_attention_noalloc) ------
@@ -1167,7 +1177,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     hipError_t e = hipSuccess;
     // A pure decode batch of few rows is one launch less: the decode wavefronts plan for themselves
     // and write the new rows (see kSelfPlanMaxRows).
-    const bool self_plan = p.max_q_tiles == 0 && p.num_seqs <= kSelfPlanMaxRows && p.dyn_pieces == 0 &&
+    const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 &&
                            (!write || wp.vector_rows);
     if (self_plan) {
         if (probe.before) (void)hipEventRecord(probe.before, stream);
@@ -1181,7 +1191,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_seqs * p.num_heads_kv), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
         return hipGetLastError();
     }
     // prologue: KV-cache write of the new tokens (optional) + plan, one launch
@@ -1210,7 +1220,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         if (probe.after) (void)hipEventRecord(probe.after, stream);
         const hipError_t e_prefill = launch_paged_prefill(p, side->stream);
         if (e == hipSuccess) {
-            hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_seqs * p.num_heads_kv), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
             e = hipGetLastError();
         }
         // always join, also after an error, so the caller's stream never runs ahead of the side stream
@@ -1228,7 +1238,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_seqs * p.num_heads_kv), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.max_q_tiles > 0) {
