@@ -690,6 +690,18 @@ def main():
         del case
 
     if not args.no_extra:
+        # config3's batch at the other cache shapes of the matrix-core decode kernel (not reference
+        # configurations; no byte counters recorded for them)
+        for D, bs in ((64, 32), (64, 16), (128, 16)):
+            key = "c3_d%d_blk%d" % (D, bs)
+            case = W.config3(head_dim=D, block_size=bs)
+            r = bench_paged(hip, case, args.steps, args.warmup,
+                            "config3's batch with head size %d and cache blocks of %d tokens" % (D, bs))
+            r["roofline"] = roofline_hbm(r, key)
+            log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f (%s)"
+                % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))
+            results[key] = r
+            del case
         results["c2_masked"] = bench_sdpa_masked(hip, args.steps)
         log("c2's shape with the causality as an attention mask: %.3f ms, %.0f TFLOP/s (%s)"
             % (results["c2_masked"]["ms_per_step"], results["c2_masked"]["tflops"], results["c2_masked"]["kernel_path"]))

@@ -64,8 +64,9 @@
 
 namespace hipattn {
 
-constexpr int kD = 128;   // head size of the fast path
-constexpr int kBS = 32;   // cache block size of the fast path
+constexpr int kD = 128;   // head size of the tuned configurations (the kernels also take 64: template kHD)
+constexpr int kBS = 32;   // their cache block size (also 16: template kBlk)
+constexpr int kUnit = 32; // tokens a wavefront works through at a time: one block of 32, or two of 16
 
 struct alignas(32) DecodeRange {
     int write_pos;    // cache position of the row's own new token when it has a slot in the table, else -1
@@ -73,7 +74,7 @@ struct alignas(32) DecodeRange {
     int ctx;          // attended positions end (exclusive)
     int j0;           // attended positions begin
     int new_begin;    // cache position of the first token its sequence contributes to this batch (past_lens)
-    int nb;           // number of logical blocks attended (0 when not valid)
+    int nb;           // number of 32-token units attended (0 when not valid)
     int table_begin;  // offset of the sequence's block table in block_indices
     int empty_row;    // a single-token row with nothing to attend: its output row is zeros
 };
@@ -134,7 +135,7 @@ __device__ __forceinline__ DecodeRange decode_range(const PagedParams& p, int i)
     r.write_pos = (single && past + pos_in_seq < table_tokens) ? past + pos_in_seq : -1;
     r.empty_row = single && r.ctx <= 0;
     r.new_begin = past;
-    r.nb = valid ? (r.ctx + p.block_size - 1) / p.block_size - r.j0 / p.block_size : 0;
+    r.nb = valid ? (r.ctx + kUnit - 1) / kUnit - r.j0 / kUnit : 0;  // in units of 32 tokens
     r.table_begin = tb0;
     return r;
 }
@@ -236,21 +237,34 @@ __device__ __forceinline__ float row_broadcast(float x) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x150 + kLane, 0xf, 0xf, false));
 }
 
-template <bool kU8>
-__device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* kbase, const uint8_t* vbase, int n16,
-                                           int kg) {
+// kb[t] / vb[t]: the first row of the unit's 16-token tile t in the key / value cache (one block of
+// 32 tokens: kb[1] is sixteen rows behind kb[0]; blocks of 16: two blocks).  Head size kHD: a K row
+// is read in kHD / 32 pieces per lane, a V row by the kHD / 8 lanes that have a piece of it.
+template <bool kU8, int kHD = kD, int kBlk = kBS>
+__device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* const (&kb)[2], const uint8_t* const (&vb)[2],
+                                           int n16, int kg) {
     if constexpr (!kU8) {
+        constexpr int kRow = 2 * kHD;
+        // (with blocks of 32 both tiles are addressed from the block's first row: one base register)
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                b.k[t][i] = *(const uint4_t*)(kbase + (t * 16 + n16) * 256 + kg * 64 + i * 16);
+            for (int i = 0; i < kHD / 32; i++)
+                b.k[t][i] = kBlk == 32 ? *(const uint4_t*)(kb[0] + (t * 16 + n16) * kRow + kg * (kHD / 2) + i * 16)
+                                       : *(const uint4_t*)(kb[t] + n16 * kRow + kg * (kHD / 2) + i * 16);
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-                b.v[t * 4 + r] = *(const uint4_t*)(vbase + (t * 16 + kg * 4 + r) * 256 + n16 * 16);
+            for (int r = 0; r < 4; r++) {
+                if (kHD == 128 || n16 * 8 < kHD)
+                    b.v[t * 4 + r] = kBlk == 32 ? *(const uint4_t*)(vb[0] + (t * 16 + kg * 4 + r) * kRow + n16 * 16)
+                                                : *(const uint4_t*)(vb[t] + (kg * 4 + r) * kRow + n16 * 16);
+                else
+                    b.v[t * 4 + r] = (uint4_t){0u, 0u, 0u, 0u};
+            }
     } else {
+        const uint8_t* const kbase = kb[0];
+        const uint8_t* const vbase = vb[0];
         constexpr int kRow = kD + 8;
 #pragma unroll
         for (int t = 0; t < 2; t++)
@@ -278,16 +292,19 @@ struct WaveState {
     float4_t acc[8];  // acc[e][r] = O[head][(kg*4 + r)*8 + e]
 };
 
-template <bool kU8, bool kBf16>
+// kTileMask (blocks of 16): `tiles_in` has bit t set when tile t of the unit lies in a block of the
+// cache; with blocks of 32 both tiles always do and the argument is ignored.
+template <bool kU8, bool kBf16, int kHD = kD, bool kTileMask = false>
 __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, const typename Op16<kBf16>::vec8 (&qf)[4], float sumq,
-                                              float c, int tok_base, int j0, int ctx, int kg) {
+                                              float c, int tok_base, int j0, int ctx, int kg, int tiles_in = 3) {
+    const int tiles = kTileMask ? tiles_in : 3;
     // ---- S^T = K Q^T : two tiles of 16 tokens x 16 heads
     float4_t s[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         s[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < kHD / 32; i++) {
             typename Op16<kBf16>::vec8 a;
             if constexpr (!kU8) {
                 a = Op16<kBf16>::from_bits(b.k[t][i]);
@@ -307,7 +324,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
     float mloc = -INFINITY;
     // u8: this lane's token's scale, zero-point plus byte bias, and their product (see BlockRegs)
     float sz_scale = 0.0f, sz_zero = 0.0f, sz_prod = 0.0f;
-    const bool partial = (tok_base < j0) || (tok_base + kBS > ctx);  // wavefront-uniform
+    const bool partial = (tok_base < j0) || (tok_base + kUnit > ctx) || tiles != 3;  // wavefront-uniform
     if constexpr (kU8) {
         sz_scale = b.sz.x;
         sz_zero = b.sz.y + kByteBias;
@@ -343,7 +360,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
                     default: x = dequant_score(std::integral_constant<int, 7>{}, x); break;
                 }
             }
-            x = (tok >= j0 && tok < ctx) ? x * c : -INFINITY;
+            x = (tok >= j0 && tok < ctx && ((tiles >> t) & 1)) ? x * c : -INFINITY;
             sv[j] = x;
             mloc = fmaxf(mloc, x);
         }
@@ -359,7 +376,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const int tok = tok_base + (j >> 2) * 16 + kg * 4 + (j & 3);
-                if (!(tok >= j0 && tok < ctx)) b.v[j] = (uint4_t){0u, 0u, 0u, 0u};
+                if (!(tok >= j0 && tok < ctx && ((tiles >> (j >> 2)) & 1))) b.v[j] = (uint4_t){0u, 0u, 0u, 0u};
             }
         }
     }
@@ -581,7 +598,7 @@ __device__ __forceinline__ void store_out8(void* out, int64_t elem, int dtype, c
 // rows are then accumulated with independent loads (lane l owns head-dim 2l and 2l + 1).
 __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const Line& line, int s, int h, int g,
                                                    int token, int id_first, int id_last, int lane) {
-    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
+    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv, D = p.head_dim;
     float m_run = -INFINITY, l_run = 0.0f, ox = 0.0f, oy = 0.0f;
     for (int id0 = id_first; id0 <= id_last; id0 += 64) {
         const int id = id0 + lane;
@@ -606,13 +623,16 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
             if (!((live >> i) & 1)) continue;
             const float fi = __shfl(f, i, 64);
             const int64_t sl = (int64_t)(id0 + i) + (int64_t)s * Hkv + h;
-            const float2 v = *(const float2*)(p.part_out + (sl * G + g) * kD + 2 * lane);
-            ox = fmaf(fi, v.x, ox);
-            oy = fmaf(fi, v.y, oy);
+            if (2 * lane < D) {
+                const float2 v = *(const float2*)(p.part_out + (sl * G + g) * D + 2 * lane);
+                ox = fmaf(fi, v.x, ox);
+                oy = fmaf(fi, v.y, oy);
+            }
         }
     }
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-    const int64_t o = ((int64_t)token * p.num_heads_q + (int64_t)h * G + g) * kD + 2 * lane;
+    if (2 * lane >= D) return;
+    const int64_t o = ((int64_t)token * p.num_heads_q + (int64_t)h * G + g) * D + 2 * lane;
     if (p.out_dtype == HIPATTN_F32) {
         *(float2*)((float*)p.out + o) = make_float2(ox * inv, oy * inv);
     } else {
@@ -634,9 +654,14 @@ constexpr int kSelfPlanMaxRows = 256;
 // kWaves wavefronts to a workgroup.  1 is the ordinary launch.  With 8 a workgroup owns a compute
 // unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
 // leave the others free for a kernel that runs beside this one.
-template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false>
+// kHD, kBlk: head size (128 or 64) and cache block size (32 or 16); u8 caches, the self-planning form
+// and the eight-wavefront form exist for 128 / 32 only.
+template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
+    static_assert((kHD == 128 && kBlk == 32) || (!kU8 && !kSelfPlan && kWaves == 1), "the variants of the tuned shape only");
+    static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32), "head size 64 or 128, blocks of 16 or 32");
+    constexpr int kEntries = kUnit / kBlk;  // block-table entries per unit
     static_assert(!kSelfPlan || kWaves == 1, "a wavefront that plans for itself is a workgroup of its own");
     const int w = kWaves == 1 ? blockIdx.x : blockIdx.x * kWaves + (threadIdx.x >> 6);
     const int lane = kWaves == 1 ? threadIdx.x : (threadIdx.x & 63), n16 = lane & 15, kg = lane >> 4;
@@ -691,8 +716,8 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     if (w >= num_waves) return;
     const Line line(total, num_waves, p.dyn_pieces);
 
-    constexpr int64_t kRowBytes = kU8 ? (kD + 8) : (2 * kD);
-    const int64_t block_stride = (int64_t)Hkv * kBS * kRowBytes;
+    constexpr int64_t kRowBytes = kU8 ? (kHD + 8) : (2 * kHD);
+    const int64_t block_stride = (int64_t)Hkv * kBlk * kRowBytes;
 
     // The static piece first, then dynamic pieces for as long as there are any.  The ticket for
     // the next dynamic piece is drawn before the current piece is worked on, so its latency is hidden.
@@ -744,9 +769,11 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         const int n = (int)(to - from);  // blocks of this segment in this piece
         const bool whole = (n == nb);
         L = from;
-        const int lb0 = rg.j0 / kBS + b_rel;            // first logical block
-        const int32_t* table = p.block_indices + rg.table_begin + lb0;
-        const int64_t head_off = (int64_t)h * kBS * kRowBytes;
+        const int lb0 = rg.j0 / kUnit + b_rel;          // first unit of 32 tokens
+        const int32_t* table = p.block_indices + rg.table_begin + lb0 * kEntries;
+        // table entries from there on that hold attended tokens (the row's table may end with them)
+        const int entries = (rg.ctx + kBlk - 1) / kBlk - lb0 * kEntries;
+        const int64_t head_off = (int64_t)h * kBlk * kRowBytes;
 
         if constexpr (kSelfPlan) {
             // The new tokens of this call whose cache rows this piece is about to read go into the cache
@@ -755,24 +782,24 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
             // stores and then loads, and the stores are waited for below; a token that several rows
             // attend is written by each of their wavefronts with the same bytes.
             if (do_write && rg.write_pos >= 0) {
-                const int q_lo = max(rg.new_begin, lb0 * kBS), q_hi = min(rg.write_pos, (lb0 + n) * kBS - 1);
+                const int q_lo = max(rg.new_begin, lb0 * kUnit), q_hi = min(rg.write_pos, (lb0 + n) * kUnit - 1);
                 for (int q = q_lo; q <= q_hi; q++) {  // (wave-uniform; one pass for a decode row)
-                    const int pb_new = p.block_indices[rg.table_begin + q / kBS];
+                    const int pb_new = p.block_indices[rg.table_begin + q / kBlk];
                     if (pb_new >= 0 && pb_new < p.num_blocks)
                         kv_cache_write_pair128(wp, rg.token - (rg.write_pos - q), h, pb_new, q, lane);
                 }
                 if (q_lo <= q_hi) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the rows have reached the cache
             }
         }
-        // Q^T operand: lane (head n16, kg) holds Q[head][kg*32 + i*8 .. +8]; padding heads are zero
+        // Q^T operand: lane (head n16, kg) holds Q[head][kg * kHD/4 + i*8 .. +8]; padding heads are zero
         typename Op16<kBf16>::vec8 qf[4];
         float sumq = 0.0f;
         {
-            const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kD;
+            const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kHD;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < kHD / 32; i++) {
                 if (n16 < G) {
-                    qf[i] = load_q8<kBf16>(p.q, qrow + kg * 32 + i * 8, p.q_dtype);
+                    qf[i] = load_q8<kBf16>(p.q, qrow + kg * (kHD / 4) + i * 8, p.q_dtype);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; e++) Op16<kBf16>::set(qf[i], e, 0.0f);
@@ -795,28 +822,46 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
         for (int e = 0; e < 8; e++) st.acc[e] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-        // blocks in groups of 64: one vector load fetches the group's block-table entries
-        for (int g0 = 0; g0 < n; g0 += 64) {
-            const int gn = min(64, n - g0);
-            const int my_pb = lane < gn ? table[g0 + lane] : -1;
-            auto issue = [&](BlockRegs<kU8>& regs, int i) -> bool {
-                const int pb = __builtin_amdgcn_readlane(my_pb, i);
-                if (pb < 0 || pb >= p.num_blocks) return false;  // never read outside the cache
-                const int64_t off = (int64_t)pb * block_stride + head_off;
-                load_block<kU8>(regs, p.key_cache + off, p.value_cache + off, n16, kg);
-                return true;
+        // units in groups of 64 table entries: one vector load fetches the group's block-table entries
+        constexpr int kGroup = 64 / kEntries;
+        for (int g0 = 0; g0 < n; g0 += kGroup) {
+            const int gn = min(kGroup, n - g0);
+            const int my_entry = g0 * kEntries + lane;
+            const int my_pb = (lane < gn * kEntries && my_entry < entries) ? table[my_entry] : -1;
+            // which tiles of unit i were issued (0: none, the unit is skipped); never reads outside the cache
+            auto issue = [&](BlockRegs<kU8>& regs, int i) -> int {
+                if constexpr (kEntries == 1) {
+                    const int pb = __builtin_amdgcn_readlane(my_pb, i);
+                    if (pb < 0 || pb >= p.num_blocks) return 0;
+                    const int64_t off = (int64_t)pb * block_stride + head_off;
+                    const uint8_t* const kb[2] = {p.key_cache + off, p.key_cache + off + 16 * kRowBytes};
+                    const uint8_t* const vb[2] = {p.value_cache + off, p.value_cache + off + 16 * kRowBytes};
+                    load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
+                    return 3;
+                } else {
+                    const int pb0 = __builtin_amdgcn_readlane(my_pb, 2 * i), pb1 = __builtin_amdgcn_readlane(my_pb, 2 * i + 1);
+                    const int ok = (pb0 >= 0 && pb0 < p.num_blocks ? 1 : 0) | (pb1 >= 0 && pb1 < p.num_blocks ? 2 : 0);
+                    if (ok == 0) return 0;
+                    // a tile without a block is read from the other tile's block: valid memory, and masked
+                    const int64_t off0 = (int64_t)((ok & 1) ? pb0 : pb1) * block_stride + head_off;
+                    const int64_t off1 = (int64_t)((ok & 2) ? pb1 : pb0) * block_stride + head_off;
+                    const uint8_t* const kb[2] = {p.key_cache + off0, p.key_cache + off1};
+                    const uint8_t* const vb[2] = {p.value_cache + off0, p.value_cache + off1};
+                    load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
+                    return ok;
+                }
             };
             if constexpr (!kU8) {
                 // two register stages: block i+1 is in flight while block i is consumed
                 BlockRegs<kU8> ra, rb;
-                bool ok_a = issue(ra, 0), ok_b = false;
+                int ok_a = issue(ra, 0), ok_b = 0;
                 int i = 0;
                 while (i < gn) {
-                    ok_b = (i + 1 < gn) ? issue(rb, i + 1) : false;
-                    if (ok_a) process_block<kU8, kBf16>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kBS, rg.j0, rg.ctx, kg);
+                    ok_b = (i + 1 < gn) ? issue(rb, i + 1) : 0;
+                    if (ok_a) process_block<kU8, kBf16, kHD, kEntries != 1>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kUnit, rg.j0, rg.ctx, kg, ok_a);
                     if (i + 1 >= gn) break;
-                    ok_a = (i + 2 < gn) ? issue(ra, i + 2) : false;
-                    if (ok_b) process_block<kU8, kBf16>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kBS, rg.j0, rg.ctx, kg);
+                    ok_a = (i + 2 < gn) ? issue(ra, i + 2) : 0;
+                    if (ok_b) process_block<kU8, kBf16, kHD, kEntries != 1>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kUnit, rg.j0, rg.ctx, kg, ok_b);
                     i += 2;
                 }
             } else {
@@ -825,9 +870,9 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                 // four spill registers and fall to 629 us.)
                 constexpr int kStages = HIPATTN_U8_STAGES;
                 BlockRegs<kU8> regs[kStages];
-                bool ok[kStages];
+                int ok[kStages];
 #pragma unroll
-                for (int u = 0; u < kStages - 1; u++) ok[u] = (u < gn) ? issue(regs[u], u) : false;
+                for (int u = 0; u < kStages - 1; u++) ok[u] = (u < gn) ? issue(regs[u], u) : 0;
                 for (int i = 0; i < gn; i += kStages) {
 #pragma unroll
                     for (int u = 0; u < kStages; u++) {
@@ -835,8 +880,8 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                         if (idx >= gn) break;
                         constexpr int kLast = kStages - 1;
                         ok[(u + kLast) % kStages] =
-                            (idx + kLast < gn) ? issue(regs[(u + kLast) % kStages], idx + kLast) : false;
-                        if (ok[u]) process_block<kU8, kBf16>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kBS, rg.j0, rg.ctx, kg);
+                            (idx + kLast < gn) ? issue(regs[(u + kLast) % kStages], idx + kLast) : 0;
+                        if (ok[u]) process_block<kU8, kBf16>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kUnit, rg.j0, rg.ctx, kg);
                     }
                 }
             }
@@ -864,10 +909,11 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     o[e] = v * inv;
                 }
                 const int d0 = (kg * 4 + r) * 8;
+                if (kHD < 128 && d0 >= kHD) continue;  // (rows of the accumulator beyond the head size hold nothing)
                 if (whole) {
-                    store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * kD + d0, p.out_dtype, o);
+                    store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * kHD + d0, p.out_dtype, o);
                 } else {
-                    float* po = p.part_out + (slot * G + n16) * kD + d0;
+                    float* po = p.part_out + (slot * G + n16) * kHD + d0;
                     *(float4*)(po) = make_float4(o[0], o[1], o[2], o[3]);
                     *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
                 }
@@ -954,11 +1000,16 @@ bool set_option(const char* name, int value) {
 
 // ---- host side of the fast path ---------------------------------------------------------
 
+// The tuned shape -- head size 128, blocks of 32 -- with every cache type; head size 64 and blocks of
+// 16 with 16-bit caches.
+static bool tuned_shape(const PagedParams& p) { return p.head_dim == kD && p.block_size == kBS; }
+
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
-    return p.head_dim == kD && p.block_size == kBS && G <= 16 &&
-           (p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16) &&
-           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
+    if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
+    if (tuned_shape(p)) return p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8;
+    return (p.head_dim == 64 || p.head_dim == 128) && (p.block_size == 16 || p.block_size == 32) &&
+           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16);
 }
 
 // Wavefronts the decode kernel keeps resident: it needs up to 256 registers per lane, i.e. two
@@ -987,6 +1038,7 @@ static int resident_decode_waves() {
 // or more sequences, all but one of them empty, has a bound of 0 by the formula and must not).
 static int query_tile_bound(const PagedParams& p) {
     if (p.num_tokens == p.num_seqs && !p.any_lengths) return 0;  // one token per sequence: a pure decode batch
+    if (p.head_dim != kD) return 0;  // the chunk kernel is head size 128 only: every token a decode row of its own
     return std::max(1, p.num_tokens / 128 + std::min(p.num_seqs, p.num_tokens / 2));
 }
 
@@ -996,7 +1048,7 @@ static int query_tile_bound(const PagedParams& p) {
 static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p.num_tokens : p.num_seqs; }
 
 static bool overlap_wanted(const PagedParams& p) {
-    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
+    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream || !tuned_shape(p)) return false;
     return option(kOptMixedOverlap) != 0;
 }
 
@@ -1025,7 +1077,7 @@ size_t paged_fast_workspace_bytes(const PagedParams& p) {
     const size_t rows = (size_t)plan_rows(p);
     const size_t slots = (size_t)W + choose_dyn_pieces(W, overlap) + rows * p.num_heads_kv;
     return 512 + 2 * align_up((rows + 1) * sizeof(int32_t), 256) + align_up(rows * 32, 256) +
-           align_up(slots * G * kD * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
+           align_up(slots * G * p.head_dim * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
 }
 
 
@@ -1053,7 +1105,7 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     p.seq_info = w;
     w += align_up((size_t)p.num_rows * 32, 256);
     p.part_out = (float*)w;
-    w += align_up(slots * G * kD * sizeof(float), 256);
+    w += align_up(slots * G * p.head_dim * sizeof(float), 256);
     p.part_ml = (float*)w;
     w += align_up(slots * G * 2 * sizeof(float), 256);
 }
@@ -1171,13 +1223,13 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     int write_blocks = 0;
     if (write) {
         wp = *write;
-        if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head_dim 128 only
+        if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head sizes 64 and 128 only
         write_blocks = (int)((kv_write_wavefronts(wp) + 3) / 4);
     }
     hipError_t e = hipSuccess;
     // A pure decode batch of few rows is one launch less: the decode wavefronts plan for themselves
     // and write the new rows (see kSelfPlanMaxRows).
-    const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 &&
+    const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 && tuned_shape(p) &&
                            (!write || wp.vector_rows);
     if (self_plan) {
         if (probe.before) (void)hipEventRecord(probe.before, stream);
@@ -1229,7 +1281,26 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         return e != hipSuccess ? e : (e_prefill != hipSuccess ? e_prefill : e_join);
     }
     if (probe.before) (void)hipEventRecord(probe.before, stream);
-    if (p.cache_dtype == HIPATTN_U8)
+    const dim3 waves(p.num_waves), one(64);
+    const bool bf16 = p.cache_dtype == HIPATTN_BF16;
+    if (!tuned_shape(p)) {  // head size 64 and / or blocks of 16, 16-bit caches
+        if (p.head_dim == 64 && p.block_size == 32) {
+            if (bf16)
+                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 32>), waves, one, 0, stream, p, wp, 0);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 32>), waves, one, 0, stream, p, wp, 0);
+        } else if (p.head_dim == 64) {
+            if (bf16)
+                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 16>), waves, one, 0, stream, p, wp, 0);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 16>), waves, one, 0, stream, p, wp, 0);
+        } else {
+            if (bf16)
+                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 128, 16>), waves, one, 0, stream, p, wp, 0);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 128, 16>), waves, one, 0, stream, p, wp, 0);
+        }
+    } else if (p.cache_dtype == HIPATTN_U8)
         hipLaunchKernelGGL((paged_decode_kernel<true, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);
     else if (p.cache_dtype == HIPATTN_BF16)
         hipLaunchKernelGGL((paged_decode_kernel<false, true, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);

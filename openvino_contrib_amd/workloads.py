@@ -205,12 +205,12 @@ def config2(seed=1002, B=4, Hq=32, Hkv=8, L=2048, D=128):
     return c
 
 
-def config3(seed=1003, S=64, lo=512, hi=8192):
+def config3(seed=1003, S=64, lo=512, hi=8192, head_dim=128, block_size=32):
     """fp16 paged decode: S sequences x 1 new token, contexts uniform in [lo, hi]."""
     rng = np.random.Generator(np.random.PCG64(seed))
     ctx = rng.integers(lo, hi + 1, size=S)
     seqs = [(int(c) - 1, 1) for c in ctx]
-    return make_paged_case(seed + 100000, seqs, 32, 8, 128, 32, F16, F16, F16)
+    return make_paged_case(seed + 100000, seqs, 32, 8, head_dim, block_size, F16, F16, F16)
 
 
 def config4(seed=1004, S=128, lo=1024, hi=16384):

@@ -808,7 +808,62 @@ def test_paged_mixed_batches_on_many_short_lived_streams(hip, oracle):
     dev.free()
 
 
-@pytest.mark.parametrize("shape", [(6, 2, 64, 16, W.F16, W.F16), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
+@pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16)])
+@pytest.mark.parametrize("q_dtype,cache_dtype,Hq,Hkv", [(W.F16, W.F16, 32, 8), (W.BF16, W.BF16, 8, 8), (W.BF16, W.F16, 24, 2),
+                                                        (W.F16, W.BF16, 16, 1)])
+@pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
+def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window):
+    """16-bit caches with head size 64 or blocks of 16 tokens run the matrix-core decode kernel, every
+    token a row of its plan (multi-token sequences included); the shape-generic kernels agree."""
+    announce("paged head/block shapes", D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window)
+    if kind == "decode":
+        seqs = [(c - 1, 1) for c in DECODE_CTX]
+    elif kind == "mixed":
+        seqs = [(0, 9), (37, 1), (31, 2), (5, 40), (64, 1), (200, 1), (15, 1), (16, 1), (17, 33), (0, 1), (1000, 3)]
+    else:
+        seqs = [(0, 70), (0, 16), (3, 17), (0, 1)]
+    case = W.make_paged_case(84, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    tol = 1e-2 if (cache_dtype == W.BF16 or q_dtype == W.BF16) else 2e-3
+    dev = H.PagedDeviceCase(hip, case)
+    for waves in (0, 7, 900):
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if waves else 0)
+        assert path == "paged_mfma"
+        assert np.isfinite(out).all()
+        assert H.max_abs(out, ref) <= tol, waves
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    out_g, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic"
+    assert H.max_abs(out_g, ref) <= tol
+    dev.free()
+
+
+def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle):
+    """A block id outside the pool contributes nothing, whichever half of a 32-token unit it is (checked
+    against the shape-generic kernels, which skip such blocks key by key)."""
+    announce("paged blocks of 16, bad ids")
+    seqs = [(99, 1), (47, 1), (16, 1), (300, 1)]
+    case = W.make_paged_case(85, seqs, 16, 4, 128, 16, W.F16, W.F16, W.F16)
+    ids = case["block_indices"]
+    begins = case["block_indices_begins"]
+    ids[begins[0] + 1] = case["num_blocks"] + 5   # second half of a unit
+    ids[begins[0] + 4] = -3                       # first half of a unit
+    ids[begins[1] + 2] = case["num_blocks"]       # a unit's only block
+    ids[begins[3] + 6] = -1
+    ids[begins[3] + 7] = 1 << 30                  # both halves
+    dev = H.PagedDeviceCase(hip, case)
+    ref, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic" and np.isfinite(ref).all()
+    for waves in (0, 50):
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE)
+        assert path == "paged_mfma"
+        assert H.max_abs(out, ref) <= 2e-3
+    dev.free()
+
+
+@pytest.mark.parametrize("shape", [(6, 2, 96, 16, W.F16, W.F16), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
                                    (4, 1, 128, 16, W.F16, W.U8), (34, 2, 128, 32, W.F16, W.F16)])
 def test_paged_generic_shapes(hip, oracle, shape):
     """Head sizes, block sizes and GQA ratios outside the MFMA fast path."""
