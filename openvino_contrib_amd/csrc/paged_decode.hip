@@ -654,12 +654,13 @@ constexpr int kSelfPlanMaxRows = 256;
 // kWaves wavefronts to a workgroup.  1 is the ordinary launch.  With 8 a workgroup owns a compute
 // unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
 // leave the others free for a kernel that runs beside this one.
-// kHD, kBlk: head size (128 or 64) and cache block size (32 or 16); u8 caches, the self-planning form
-// and the eight-wavefront form exist for 128 / 32 only.
+// kHD, kBlk: head size (128 or 64) and cache block size (32 or 16); u8 caches exist for 128 / 32 only,
+// the self-planning form and the eight-wavefront form for head size 128 only.
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
-    static_assert((kHD == 128 && kBlk == 32) || (!kU8 && !kSelfPlan && kWaves == 1), "the variants of the tuned shape only");
+    static_assert((kHD == 128 && kBlk == 32) || !kU8, "u8 caches: head size 128 and blocks of 32 only");
+    static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
     static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32), "head size 64 or 128, blocks of 16 or 32");
     constexpr int kEntries = kUnit / kBlk;  // block-table entries per unit
     static_assert(!kSelfPlan || kWaves == 1, "a wavefront that plans for itself is a workgroup of its own");
@@ -1048,7 +1049,7 @@ static int query_tile_bound(const PagedParams& p) {
 static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p.num_tokens : p.num_seqs; }
 
 static bool overlap_wanted(const PagedParams& p) {
-    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream || !tuned_shape(p)) return false;
+    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
     return option(kOptMixedOverlap) != 0;
 }
 
@@ -1217,6 +1218,39 @@ void release_side_stream(hipStream_t owner) {
     delete s;
 }
 
+// The decode kernel for p's cache type, head size and block size (a combination paged_fast_supported
+// admits; head size 64 has the ordinary form only).
+template <int kWaves, bool kSelfPlan>
+static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block,
+                          hipStream_t stream) {
+    const bool bf16 = p.cache_dtype == HIPATTN_BF16;
+    if (p.cache_dtype == HIPATTN_U8) {
+        hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan>), grid, block, 0, stream, p, wp, do_write);
+    } else if (p.head_dim == 128 && p.block_size == 32) {
+        if (bf16)
+            hipLaunchKernelGGL((paged_decode_kernel<false, true, kWaves, kSelfPlan>), grid, block, 0, stream, p, wp, do_write);
+        else
+            hipLaunchKernelGGL((paged_decode_kernel<false, false, kWaves, kSelfPlan>), grid, block, 0, stream, p, wp, do_write);
+    } else if (p.head_dim == 128) {
+        if (bf16)
+            hipLaunchKernelGGL((paged_decode_kernel<false, true, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
+        else
+            hipLaunchKernelGGL((paged_decode_kernel<false, false, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
+    } else if constexpr (kWaves == 1 && !kSelfPlan) {
+        if (p.block_size == 32) {
+            if (bf16)
+                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
+        } else {
+            if (bf16)
+                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
+        }
+    }
+}
+
 hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
                              const KernelProbe& probe) {
     KvWriteParams wp{};
@@ -1229,17 +1263,11 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     hipError_t e = hipSuccess;
     // A pure decode batch of few rows is one launch less: the decode wavefronts plan for themselves
     // and write the new rows (see kSelfPlanMaxRows).
-    const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 && tuned_shape(p) &&
+    const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 && p.head_dim == kD &&
                            (!write || wp.vector_rows);
     if (self_plan) {
         if (probe.before) (void)hipEventRecord(probe.before, stream);
-        const int do_write = write ? 1 : 0;
-        if (p.cache_dtype == HIPATTN_U8)
-            hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, true>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, do_write);
-        else if (p.cache_dtype == HIPATTN_BF16)
-            hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, true>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, do_write);
-        else
-            hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, true>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, do_write);
+        launch_decode<1, true>(p, wp, write ? 1 : 0, dim3(p.num_waves), dim3(64), stream);
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
         if (e != hipSuccess) return e;
@@ -1261,13 +1289,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         if ((e = hipEventRecord(side->fork, stream)) != hipSuccess) return e;
         if ((e = hipStreamWaitEvent(side->stream, side->fork, 0)) != hipSuccess) return e;
         if (probe.before) (void)hipEventRecord(probe.before, stream);
-        const dim3 grid(p.num_waves / 8), block(512);
-        if (p.cache_dtype == HIPATTN_U8)
-            hipLaunchKernelGGL((paged_decode_kernel<true, false, 8>), grid, block, 0, stream, p, wp, 0);
-        else if (p.cache_dtype == HIPATTN_BF16)
-            hipLaunchKernelGGL((paged_decode_kernel<false, true, 8>), grid, block, 0, stream, p, wp, 0);
-        else
-            hipLaunchKernelGGL((paged_decode_kernel<false, false, 8>), grid, block, 0, stream, p, wp, 0);
+        launch_decode<8, false>(p, wp, 0, dim3(p.num_waves / 8), dim3(512), stream);
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
         const hipError_t e_prefill = launch_paged_prefill(p, side->stream);
@@ -1281,31 +1303,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         return e != hipSuccess ? e : (e_prefill != hipSuccess ? e_prefill : e_join);
     }
     if (probe.before) (void)hipEventRecord(probe.before, stream);
-    const dim3 waves(p.num_waves), one(64);
-    const bool bf16 = p.cache_dtype == HIPATTN_BF16;
-    if (!tuned_shape(p)) {  // head size 64 and / or blocks of 16, 16-bit caches
-        if (p.head_dim == 64 && p.block_size == 32) {
-            if (bf16)
-                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 32>), waves, one, 0, stream, p, wp, 0);
-            else
-                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 32>), waves, one, 0, stream, p, wp, 0);
-        } else if (p.head_dim == 64) {
-            if (bf16)
-                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 16>), waves, one, 0, stream, p, wp, 0);
-            else
-                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 16>), waves, one, 0, stream, p, wp, 0);
-        } else {
-            if (bf16)
-                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 128, 16>), waves, one, 0, stream, p, wp, 0);
-            else
-                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 128, 16>), waves, one, 0, stream, p, wp, 0);
-        }
-    } else if (p.cache_dtype == HIPATTN_U8)
-        hipLaunchKernelGGL((paged_decode_kernel<true, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);
-    else if (p.cache_dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL((paged_decode_kernel<false, true, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);
-    else
-        hipLaunchKernelGGL((paged_decode_kernel<false, false, 1>), dim3(p.num_waves), dim3(64), 0, stream, p, wp, 0);
+    launch_decode<1, false>(p, wp, 0, dim3(p.num_waves), dim3(64), stream);
     e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     if (e != hipSuccess) return e;

@@ -90,3 +90,16 @@ def test_config5_mixed_batch_u8_cache(hip, oracle):
     """Configuration 5's batch on a u8 cache: the chunks go through the flash kernel's u8 loads."""
     announce("C5 with a u8 cache")
     _run_paged_config(hip, oracle, W.config5(cache_dtype=W.U8), 1e-2, "C5-u8")
+
+
+@pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16)])
+def test_config3_at_head_64_and_blocks_of_16(hip, oracle, D, bs):
+    """Configuration 3's batch on the other cache shapes of the matrix-core decode kernel."""
+    announce("C3's batch, head size", D, "blocks of", bs)
+    _run_paged_config(hip, oracle, W.config3(head_dim=D, block_size=bs), 2e-3, "C3 %d/%d" % (D, bs))
+
+
+def test_config5_mixed_batch_on_blocks_of_16(hip, oracle):
+    """Configuration 5's batch on cache blocks of 16 tokens: the same two kernels side by side."""
+    announce("C5 with blocks of 16")
+    _run_paged_config(hip, oracle, W.config5(block_size=16), 1e-2, "C5 blocks of 16")

@@ -631,13 +631,14 @@ def test_paged_batch_of_thousands_of_sequences(hip, oracle, cache_dtype, mixed):
 
 @pytest.mark.parametrize("env", [{}, {"mixed_decode_share_percent": 10},
                                  {"mixed_decode_share_percent": 1000}, {"mixed_overlap": 0}])
-@pytest.mark.parametrize("q_dtype,cache_dtype,window", [(W.BF16, W.F16, 0), (W.F16, W.U8, 300), (W.BF16, W.BF16, 0)])
-def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, window, schedule_options):
+@pytest.mark.parametrize("q_dtype,cache_dtype,window,bs", [(W.BF16, W.F16, 0, 32), (W.F16, W.U8, 300, 32), (W.BF16, W.BF16, 0, 32),
+                                                           (W.F16, W.F16, 300, 16), (W.BF16, W.BF16, 0, 16)])
+def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, window, bs, schedule_options):
     """With no fixed wavefront count the decode kernel of a mixed batch runs beside the chunks' flash
     kernel on a share of the compute units that the plan picks on the device; whatever the share
     (forced small and large here, and the one-after-the-other order), the results are the same, also
     when calls follow each other without a synchronisation in between."""
-    announce("paged mixed side by side", env, q_dtype, cache_dtype, window)
+    announce("paged mixed side by side", env, q_dtype, cache_dtype, window, bs)
     schedule_options(env)
     batches = [
         [(0, 130), (37, 1), (500, 1), (100, 257), (0, 2), (999, 1), (31, 97), (64, 1), (700, 128), (5, 0)],
@@ -646,7 +647,7 @@ def test_paged_mixed_batch_side_by_side(hip, oracle, env, q_dtype, cache_dtype, 
     ]
     tol = 1e-2
     for i, seqs in enumerate(batches):
-        case = W.make_paged_case(90 + i, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+        case = W.make_paged_case(90 + i, seqs, 16, 4, 128, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
         ref, okc, ovc = H.oracle_paged(oracle, case)
         dev = H.PagedDeviceCase(hip, case)
         out, path = dev.run()
