@@ -702,11 +702,13 @@ def main():
                 % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))
             results[key] = r
             del case
-        case = W.config5(block_size=16)
-        r = bench_paged(hip, case, args.steps, args.warmup, "config5's batch on cache blocks of 16 tokens")
-        log("c5_blk16: %.3f ms/step (%s)" % (r["ms_per_step"], r["kernel_path"]))
-        results["c5_blk16"] = r
-        del case
+        for key, kw, what in (("c5_blk16", {"block_size": 16}, "on cache blocks of 16 tokens"),
+                              ("c5_d64_blk16", {"block_size": 16, "head_dim": 64}, "with head size 64 on cache blocks of 16 tokens")):
+            case = W.config5(**kw)
+            r = bench_paged(hip, case, args.steps, args.warmup, "config5's batch " + what)
+            log("%s: %.3f ms/step (%s)" % (key, r["ms_per_step"], r["kernel_path"]))
+            results[key] = r
+            del case
         results["c2_masked"] = bench_sdpa_masked(hip, args.steps)
         log("c2's shape with the causality as an attention mask: %.3f ms, %.0f TFLOP/s (%s)"
             % (results["c2_masked"]["ms_per_step"], results["c2_masked"]["tflops"], results["c2_masked"]["kernel_path"]))

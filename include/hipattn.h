@@ -190,10 +190,10 @@ hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q,
  * row with its own context length, whichever sequence it belongs to, so the result is right
  * for any split of the tokens over the sequences; HIPATTN_PA_ANY_LENGTHS only changes how fast
  * such a batch runs when it does hold long multi-token sequences.
- * Kernels: 16-bit and u8 caches with head_dim 128 and block_size 32 take the matrix-core decode
- * kernel and, for multi-token sequences, the chunked-prefill kernel; 16-bit caches with head_dim
- * 64 or 128 and block_size 16 or 32 take the decode kernel with every token a row of its own;
- * anything else (fp32, other sizes) takes the shape-generic kernels.
+ * Kernels: 16-bit caches with head_dim 64 or 128 and block_size 16 or 32, and u8 caches with
+ * head_dim 128 and block_size 32, take the matrix-core kernels (stream-K decode for single-token
+ * rows, chunked prefill over the block table for multi-token sequences); anything else (fp32,
+ * other sizes) takes the shape-generic kernels.
  * A single-token row with nothing to attend (an empty block table) gets an output row of zeros.
  * Block ids outside [0, num_blocks) in a table: the decode and the shape-generic kernels skip
  * those blocks (probability zero); the MFMA chunked-prefill kernel redirects them to a valid

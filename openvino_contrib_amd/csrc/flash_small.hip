@@ -6,7 +6,9 @@
 // 32 query rows each, key tiles of 64 staged through registers into a double-buffered, swizzled LDS
 // tile, one workgroup barrier per tile, a straightforward online softmax, an optional attention mask
 // of any type the operator allows.  Not tuned beyond conflict-free LDS access; it replaces the fp32
-// VALU kernel for these shapes.
+// VALU kernel for these shapes.  The same body serves the multi-token sequences of a
+// PagedAttentionExtension batch at head size 64 (16-bit caches): K and V rows are then found
+// through the block table, under the causal order and the sliding window of that operator.
 //
 // Replaces the same decomposed chain as flash_prefill.hip (src/ops/matmul.cpp:185-227,
 // src/ops/softmax.cpp:178-193, src/ops/select.cpp:50-91 of the reference).
@@ -130,43 +132,71 @@ __device__ __forceinline__ void mask_values4(const uint8_t* row, int64_t key_str
     }
 }
 
-// kMask: the call carries an attention mask (p.mask, ignored under the causal flag): its values are
-// fetched from global memory ahead of the score product of every tile and added behind it.
-template <bool kBf16, bool kMask = false>
-__global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams p) {
+// One query tile of one head: what the workgroup reads, where it writes.
+struct Work {
+    const uint16_t* q;      // row 0 of the tile, this head
+    int64_t q_stride;       // elements from one query row to the next
+    int q_dtype;            // HIPATTN_F16 / BF16 (converted to the K/V type on load)
+    void* out;              // as q
+    int64_t out_stride;
+    int out_dtype;          // HIPATTN_F16 / BF16 / F32
+    int rows;               // query rows of the tile that exist (1..128)
+    int pos0;               // position of row 0: under `causal` row r attends keys <= pos0 + r ...
+    int causal;
+    int window;             // ... and, when > 0, keys > pos0 + r - window
+    int kv_len;
+    const uint8_t* k;       // dense: the kv head's rows; paged: the cache at the kv head's offset inside a block
+    const uint8_t* v;
+    const int32_t* table;   // paged: the sequence's block ids
+    int block_shift;        // log2(block size)
+    int num_blocks;
+    int64_t block_stride;   // bytes from one cache block to the next
+    float scale;
+    const uint8_t* mask;    // kMask: the mask row of query row 0 (this batch, this head)
+    int64_t mask_row_stride, mask_key_stride;  // in elements
+    int mask_dtype;
+};
+
+__device__ __forceinline__ uint32_t pack2(int dtype, float lo, float hi) {
+    return dtype == HIPATTN_BF16 ? Mfma<true>::cvt2(lo, hi) : Mfma<false>::cvt2(lo, hi);
+}
+
+// The workgroup's 128 query rows against the keys they attend.
+// kMask: the call carries an attention mask: its values are fetched from global memory ahead of the
+// score product of every tile and added behind it.  kPaged: K and V rows are found through w.table.
+template <bool kBf16, bool kMask, bool kPaged>
+__device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileBytes]) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][kTileBytes];  // [buffer][K, V]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int n32 = lane & 31, hi = lane >> 5;
-    const int q_tiles = (p.len_q + kTileQ - 1) / kTileQ;
-    const int qt = blockIdx.x % q_tiles;
-    const int h = (blockIdx.x / q_tiles) % p.num_heads_q;
-    const int b = blockIdx.x / (q_tiles * p.num_heads_q);
-    const int hkv = h / (p.num_heads_q / p.num_heads_kv);
-    const int q0 = qt * kTileQ;                      // first query row of the workgroup
-    const int my_row = q0 + wave * 32 + n32;         // this lane's query row (may lie beyond len_q)
-    const uint16_t* q = (const uint16_t*)p.q + ((int64_t)(b * p.num_heads_q + h) * p.len_q) * kD;
-    const uint8_t* k = (const uint8_t*)p.k + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
-    const uint8_t* v = (const uint8_t*)p.v + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
+    const int my_row = wave * 32 + n32;          // this lane's query row in the tile (may lie beyond w.rows)
+    const int my_pos = w.pos0 + my_row;
+    const bool windowed = kPaged && w.window > 0;
 
-    // keys this workgroup visits: all, or up to its last query row under the causal mask
-    const int kv_end = p.causal ? min(p.len_kv, min(q0 + kTileQ, p.len_q)) : p.len_kv;
+    // key tiles this workgroup visits: up to its last query row under the causal flag, from the
+    // first row's window start on
+    const int kv_end = w.causal ? min(w.kv_len, w.pos0 + w.rows) : w.kv_len;
     const int tiles = (kv_end + kTileK - 1) / kTileK;
+    const int tile0 = windowed ? max(0, w.pos0 - w.window + 1) / kTileK : 0;
 
     // Q^T fragments (B operand of S^T = K Q^T): lane (n32, hi) holds query row n32, head-dim
     // elements 8 (2i + hi) .. + 7 for k-step i, times scale * log2(e)
     vec8 qf[4];
     {
-        const float c = p.scale * kLog2e;
-        const int row = min(my_row, p.len_q - 1);
+        const float c = w.scale * kLog2e;
+        const int row = min(my_row, w.rows - 1);
+        const bool q_bf16 = w.q_dtype == HIPATTN_BF16;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint4_t raw = *(const uint4_t*)(q + (int64_t)row * kD + 8 * (2 * i + hi));
+            const uint4_t raw = *(const uint4_t*)(w.q + (int64_t)row * w.q_stride + 8 * (2 * i + hi));
             uint4_t cv;
 #pragma unroll
-            for (int w = 0; w < 4; w++)
-                cv[w] = M::cvt2(M::to_float((uint16_t)(raw[w] & 0xffffu)) * c, M::to_float((uint16_t)(raw[w] >> 16)) * c);
+            for (int e = 0; e < 4; e++) {
+                const uint16_t lo = (uint16_t)(raw[e] & 0xffffu), up = (uint16_t)(raw[e] >> 16);
+                cv[e] = q_bf16 ? M::cvt2(bf16_bits_to_float(lo) * c, bf16_bits_to_float(up) * c)
+                               : M::cvt2(f16_bits_to_float(lo) * c, f16_bits_to_float(up) * c);
+            }
             qf[i] = __builtin_bit_cast(vec8, cv);
         }
     }
@@ -177,9 +207,17 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
 #pragma unroll
         for (int s = 0; s < 2; s++) {
             const int piece = tid + 256 * s, r = piece >> 3, c = piece & 7;
-            const int key = min(tile * kTileK + r, p.len_kv - 1);  // rows past the end repeat the last key (masked later)
-            stage[s] = *(const uint4_t*)(k + (int64_t)key * kRowBytes + 16 * c);
-            stage[2 + s] = *(const uint4_t*)(v + (int64_t)key * kRowBytes + 16 * c);
+            const int key = min(tile * kTileK + r, w.kv_len - 1);  // rows past the end repeat the last key (masked later)
+            int64_t at;
+            if constexpr (kPaged) {
+                // a block id outside the cache is redirected into it: the rows that attend it are unspecified
+                const int pb = min(max(w.table[key >> w.block_shift], 0), w.num_blocks - 1);
+                at = (int64_t)pb * w.block_stride + (int64_t)(key & ((1 << w.block_shift) - 1)) * kRowBytes + 16 * c;
+            } else {
+                at = (int64_t)key * kRowBytes + 16 * c;
+            }
+            stage[s] = *(const uint4_t*)(w.k + at);
+            stage[2 + s] = *(const uint4_t*)(w.v + at);
         }
     };
     auto deposit = [&](int buf) {
@@ -198,13 +236,13 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
         for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;  // the row's running maximum (both lanes of a pair agree) and this lane's share of the sum
 
-    if (tiles > 0) {
-        fetch(0);
+    if (tile0 < tiles) {
+        fetch(tile0);
         deposit(0);
     }
     __syncthreads();
-    for (int j = 0; j < tiles; j++) {
-        const int buf = j & 1;
+    for (int j = tile0; j < tiles; j++) {
+        const int buf = (j - tile0) & 1;
         if (j + 1 < tiles) fetch(j + 1);  // in flight while this tile is computed
         const lds_byte* k_lds = (const lds_byte*)lds[buf][0];
         const lds_byte* v_lds = (const lds_byte*)lds[buf][1];
@@ -212,16 +250,15 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
 
         float16_t mask_add[2];
         if constexpr (kMask) {
-            const int row = min(my_row, p.len_q - 1);
-            const int esz = p.mask_dtype == HIPATTN_U8 ? 1 : (p.mask_dtype == HIPATTN_F32 ? 4 : 2);
-            const uint8_t* mrow = (const uint8_t*)p.mask +
-                                  ((int64_t)b * p.mask_stride[0] + (int64_t)h * p.mask_stride[1] + (int64_t)row * p.mask_stride[2]) * esz;
+            const int row = min(my_row, w.rows - 1);
+            const int esz = w.mask_dtype == HIPATTN_U8 ? 1 : (w.mask_dtype == HIPATTN_F32 ? 4 : 2);
+            const uint8_t* mrow = w.mask + (int64_t)row * w.mask_row_stride * esz;
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     float m4[4];
-                    mask_values4(mrow, p.mask_stride[3], p.mask_dtype, ts + mt * 32 + 8 * g + 4 * hi, p.len_kv, m4);
+                    mask_values4(mrow, w.mask_key_stride, w.mask_dtype, ts + mt * 32 + 8 * g + 4 * hi, w.kv_len, m4);
 #pragma unroll
                     for (int e = 0; e < 4; e++) mask_add[mt][4 * g + e] = m4[e];
                 }
@@ -243,15 +280,19 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
 #pragma unroll
             for (int mt = 0; mt < 2; mt++) s[mt] += mask_add[mt];
         }
-        // mask: keys past the end, and keys after the query under the causal flag
-        const bool edge = ts + kTileK > p.len_kv || (p.causal && ts + kTileK - 1 > q0 + wave * 32);
+        // mask: keys past the end, keys after the query under the causal flag, keys that have left
+        // the window (the tile holds one for some row of the wavefront when its first key lies
+        // before the window of the wavefront's last row)
+        const int wave_pos = w.pos0 + wave * 32;
+        const bool edge = ts + kTileK > w.kv_len || (w.causal && ts + kTileK - 1 > wave_pos) ||
+                          (windowed && ts <= wave_pos + 31 - w.window);
         if (edge) {
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
-                    const bool ok = key < p.len_kv && (!p.causal || key <= my_row);
+                    const bool ok = key < w.kv_len && (!w.causal || key <= my_pos) && (!windowed || key > my_pos - w.window);
                     s[mt][r] = ok ? s[mt][r] : -INFINITY;
                 }
         }
@@ -273,10 +314,10 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
         for (int ks = 0; ks < 4; ks++) {
             uint4_t pw;
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w] - m_use);
-                const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * w + 1] - m_use);
-                pw[w] = M::cvt2(p0, p1);
+            for (int e = 0; e < 4; e++) {
+                const float p0 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * e] - m_use);
+                const float p1 = fast_exp2(s[ks >> 1][(ks & 1) * 8 + 2 * e + 1] - m_use);
+                pw[e] = M::cvt2(p0, p1);
                 sum += p0 + p1;
             }
             pf[ks] = __builtin_bit_cast(vec8, pw);
@@ -302,18 +343,120 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
     pair_values(l_run, l_lo, l_hi);
     const float l = l_lo + l_hi;
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    if (my_row < p.len_q) {
-        uint16_t* out = (uint16_t*)p.out + ((int64_t)(b * p.num_heads_q + h) * p.len_q + my_row) * kD;
+    if (my_row < w.rows) {
 #pragma unroll
         for (int dt = 0; dt < 2; dt++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                uint2_t w;
-                w[0] = M::cvt2(o[dt][4 * g] * inv, o[dt][4 * g + 1] * inv);
-                w[1] = M::cvt2(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
-                *(uint2_t*)(out + dt * 32 + 8 * g + 4 * hi) = w;
+                const int d = dt * 32 + 8 * g + 4 * hi;
+                const float x0 = o[dt][4 * g] * inv, x1 = o[dt][4 * g + 1] * inv, x2 = o[dt][4 * g + 2] * inv, x3 = o[dt][4 * g + 3] * inv;
+                if (kPaged && w.out_dtype == HIPATTN_F32) {
+                    *(float4*)((float*)w.out + (int64_t)my_row * w.out_stride + d) = make_float4(x0, x1, x2, x3);
+                } else {
+                    uint2_t pk;
+                    pk[0] = pack2(w.out_dtype, x0, x1);
+                    pk[1] = pack2(w.out_dtype, x2, x3);
+                    *(uint2_t*)((uint16_t*)w.out + (int64_t)my_row * w.out_stride + d) = pk;
+                }
             }
     }
+}
+
+// Dense SDPA: one workgroup per (batch, query head, 128-row query tile).  kMask: p.mask rides along
+// (ignored under the causal flag).
+template <bool kBf16, bool kMask = false>
+__global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][kTileBytes];  // [buffer][K, V]
+    const int q_tiles = (p.len_q + kTileQ - 1) / kTileQ;
+    const int qt = blockIdx.x % q_tiles;
+    const int h = (blockIdx.x / q_tiles) % p.num_heads_q;
+    const int b = blockIdx.x / (q_tiles * p.num_heads_q);
+    const int hkv = h / (p.num_heads_q / p.num_heads_kv);
+    const int q0 = qt * kTileQ;
+    Work w;
+    w.q = (const uint16_t*)p.q + ((int64_t)(b * p.num_heads_q + h) * p.len_q + q0) * kD;
+    w.q_stride = kD;
+    w.q_dtype = p.dtype;
+    w.out = (uint16_t*)p.out + ((int64_t)(b * p.num_heads_q + h) * p.len_q + q0) * kD;
+    w.out_stride = kD;
+    w.out_dtype = p.dtype;
+    w.rows = min(kTileQ, p.len_q - q0);
+    w.pos0 = q0;
+    w.causal = p.causal;
+    w.window = 0;
+    w.kv_len = p.len_kv;
+    w.k = (const uint8_t*)p.k + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
+    w.v = (const uint8_t*)p.v + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
+    w.table = nullptr;
+    w.block_shift = 0;
+    w.num_blocks = 0;
+    w.block_stride = 0;
+    w.scale = p.scale;
+    w.mask = nullptr;
+    w.mask_row_stride = w.mask_key_stride = 0;
+    w.mask_dtype = 0;
+    if constexpr (kMask) {
+        const int esz = p.mask_dtype == HIPATTN_U8 ? 1 : (p.mask_dtype == HIPATTN_F32 ? 4 : 2);
+        w.mask = (const uint8_t*)p.mask +
+                 ((int64_t)b * p.mask_stride[0] + (int64_t)h * p.mask_stride[1] + (int64_t)q0 * p.mask_stride[2]) * esz;
+        w.mask_row_stride = p.mask_stride[2];
+        w.mask_key_stride = p.mask_stride[3];
+        w.mask_dtype = p.mask_dtype;
+    }
+    attend<kBf16, kMask, false>(w, lds);
+}
+
+// Chunked prefill over the block table (PagedAttentionExtension, 16-bit caches, head size 64): one
+// workgroup per (128-row query tile of a multi-token sequence, query head); the tiles of the batch
+// are numbered by p.tile_prefix (written by the plan on the device), the later -- heavier -- tiles
+// of a sequence first, the query heads of a tile side by side.  The grid is an upper bound.
+template <bool kBf16>
+__global__ __launch_bounds__(64 * kWaves) void paged_prefill_d64_kernel(PagedParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][kTileBytes];
+    const int item = blockIdx.x / p.num_heads_q, h = blockIdx.x % p.num_heads_q;
+    if (item >= p.tile_prefix[p.num_seqs]) return;
+    int lo = 0, hi_s = p.num_seqs;  // the sequence owning the tile: largest s with tile_prefix[s] <= item
+    while (hi_s - lo > 1) {
+        const int mid = (lo + hi_s) >> 1;
+        if (p.tile_prefix[mid] <= item)
+            lo = mid;
+        else
+            hi_s = mid;
+    }
+    const int s = lo;
+    const int tiles_s = p.tile_prefix[s + 1] - p.tile_prefix[s];
+    const int qt = tiles_s - 1 - (item - p.tile_prefix[s]);
+    const int t0 = p.subsequence_begins[s];
+    const int qlen = p.subsequence_begins[s + 1] - t0;
+    const int past = p.past_lens[s];
+    const int tb0 = p.block_indices_begins[s];
+    const int table_len = p.block_indices_begins[s + 1] - tb0;
+    const int G = p.num_heads_q / p.num_heads_kv;
+    const int64_t row0 = (int64_t)(t0 + qt * kTileQ) * p.num_heads_q + h;
+    Work w;
+    w.q = (const uint16_t*)p.q + row0 * kD;
+    w.q_stride = (int64_t)p.num_heads_q * kD;
+    w.q_dtype = p.q_dtype;
+    w.out = p.out_dtype == HIPATTN_F32 ? (void*)((float*)p.out + row0 * kD) : (void*)((uint16_t*)p.out + row0 * kD);
+    w.out_stride = (int64_t)p.num_heads_q * kD;
+    w.out_dtype = p.out_dtype;
+    w.rows = min(kTileQ, qlen - qt * kTileQ);
+    w.pos0 = past + qt * kTileQ;
+    w.causal = 1;
+    w.window = p.sliding_window;
+    w.kv_len = min(past + qlen, table_len * p.block_size);
+    const int64_t head_off = (int64_t)(h / G) * p.block_size * kRowBytes;
+    w.k = p.key_cache + head_off;
+    w.v = p.value_cache + head_off;
+    w.table = p.block_indices + tb0;
+    w.block_shift = __builtin_ctz(p.block_size);
+    w.num_blocks = p.num_blocks;
+    w.block_stride = (int64_t)p.num_heads_kv * p.block_size * kRowBytes;
+    w.scale = p.scale;
+    w.mask = nullptr;
+    w.mask_row_stride = w.mask_key_stride = 0;
+    w.mask_dtype = 0;
+    attend<kBf16, false, true>(w, lds);
 }
 
 }  // namespace flash_small
@@ -340,6 +483,18 @@ hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream) {
         hipLaunchKernelGGL(flash_small::sdpa_flash_d64_kernel<true>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
     else
         hipLaunchKernelGGL(flash_small::sdpa_flash_d64_kernel<false>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+    return hipGetLastError();
+}
+
+// The multi-token sequences of a planned batch (p.tile_prefix, p.max_q_tiles), head size 64.
+hipError_t launch_paged_prefill_small(const PagedParams& p, hipStream_t stream) {
+    const int64_t groups = (int64_t)p.max_q_tiles * p.num_heads_q;
+    if (groups == 0) return hipSuccess;
+    if (groups > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (p.cache_dtype == HIPATTN_BF16)
+        hipLaunchKernelGGL(flash_small::paged_prefill_d64_kernel<true>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+    else
+        hipLaunchKernelGGL(flash_small::paged_prefill_d64_kernel<false>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -150,6 +150,7 @@ void release_side_stream(hipStream_t owner);  // drops the side stream mixed bat
 hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, hipStream_t stream,
                              const KernelProbe& probe);
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream);  // flash over the block table (needs the plan)
+hipError_t launch_paged_prefill_small(const PagedParams& p, hipStream_t stream);  // the same at head size 64 (flash_small.hip)
 
 hipError_t launch_fill_bytes(void* dst, int value, size_t bytes, hipStream_t stream);
 // out = a + b over n elements; dtype is a HIPATTN_F32 / F16 / BF16 value, or -1 for int32

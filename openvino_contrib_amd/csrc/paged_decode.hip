@@ -1039,7 +1039,6 @@ static int resident_decode_waves() {
 // or more sequences, all but one of them empty, has a bound of 0 by the formula and must not).
 static int query_tile_bound(const PagedParams& p) {
     if (p.num_tokens == p.num_seqs && !p.any_lengths) return 0;  // one token per sequence: a pure decode batch
-    if (p.head_dim != kD) return 0;  // the chunk kernel is head size 128 only: every token a decode row of its own
     return std::max(1, p.num_tokens / 128 + std::min(p.num_seqs, p.num_tokens / 2));
 }
 
@@ -1050,6 +1049,7 @@ static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p
 
 static bool overlap_wanted(const PagedParams& p) {
     if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
+    if (p.head_dim != kD) return false;  // head size 64 has no eight-wavefront decode kernel
     return option(kOptMixedOverlap) != 0;
 }
 

@@ -222,9 +222,9 @@ def config4(seed=1004, S=128, lo=1024, hi=16384):
 
 
 def config5(seed=1005, n_prefill=8, chunk=512, past_hi=4096, n_decode=120, dec_lo=256, dec_hi=8192, window=4096,
-            cache_dtype=F16, block_size=32):
+            cache_dtype=F16, block_size=32, head_dim=128):
     """Mixed chunked prefill + decode, sliding window, bf16 activations, fp16 cache (or cache_dtype), Hq=64."""
     rng = np.random.Generator(np.random.PCG64(seed))
     seqs = [(int(p), chunk) for p in rng.integers(0, past_hi + 1, size=n_prefill)]
     seqs += [(int(c) - 1, 1) for c in rng.integers(dec_lo, dec_hi + 1, size=n_decode)]
-    return make_paged_case(seed + 100000, seqs, 64, 8, 128, block_size, BF16, BF16, cache_dtype, sliding_window=window)
+    return make_paged_case(seed + 100000, seqs, 64, 8, head_dim, block_size, BF16, BF16, cache_dtype, sliding_window=window)

@@ -103,3 +103,9 @@ def test_config5_mixed_batch_on_blocks_of_16(hip, oracle):
     """Configuration 5's batch on cache blocks of 16 tokens: the same two kernels side by side."""
     announce("C5 with blocks of 16")
     _run_paged_config(hip, oracle, W.config5(block_size=16), 1e-2, "C5 blocks of 16")
+
+
+def test_config5_mixed_batch_at_head_64(hip, oracle):
+    """Configuration 5's batch at head size 64 on blocks of 16: decode rows and the head-64 chunk kernel."""
+    announce("C5 at head size 64, blocks of 16")
+    _run_paged_config(hip, oracle, W.config5(block_size=16, head_dim=64), 1e-2, "C5 64/16")

@@ -814,8 +814,9 @@ def test_paged_mixed_batches_on_many_short_lived_streams(hip, oracle):
                                                         (W.F16, W.BF16, 16, 1)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
 def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window):
-    """16-bit caches with head size 64 or blocks of 16 tokens run the matrix-core decode kernel, every
-    token a row of its plan (multi-token sequences included); the shape-generic kernels agree."""
+    """16-bit caches with head size 64 or blocks of 16 tokens run the matrix-core kernels (decode rows
+    on the stream-K kernel, multi-token sequences on the chunk kernel of their head size); the
+    shape-generic kernels agree."""
     announce("paged head/block shapes", D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window)
     if kind == "decode":
         seqs = [(c - 1, 1) for c in DECODE_CTX]
@@ -838,6 +839,34 @@ def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype
     out_g, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
     assert path_g == "paged_generic"
     assert H.max_abs(out_g, ref) <= tol
+    dev.free()
+
+
+@pytest.mark.parametrize("bs", [16, 32])
+@pytest.mark.parametrize("q_dtype,cache_dtype,out_dtype", [(W.F16, W.F16, None), (W.BF16, W.F16, None), (W.F16, W.BF16, W.F32),
+                                                           (W.BF16, W.BF16, W.F16)])
+@pytest.mark.parametrize("window", [0, 1, 64, 100, 300])
+@pytest.mark.parametrize("heads", [(8, 2), (3, 3)])
+def test_paged_chunks_at_head_64(hip, oracle, bs, q_dtype, cache_dtype, out_dtype, window, heads):
+    """Multi-token sequences at head size 64: the chunk kernel over the block table (query tiles of
+    128 rows that start anywhere in a key tile, windows shorter and longer than a tile, chunks
+    without a past and behind a long one, output types other than the query's)."""
+    announce("paged chunks head 64", bs, q_dtype, cache_dtype, out_dtype, window, heads)
+    seqs = [(0, 130), (37, 1), (500, 1), (100, 257), (0, 2), (999, 1), (31, 97), (64, 1), (700, 128), (5, 0), (1, 127),
+            (63, 129), (0, 64), (2000, 3)]
+    case = W.make_paged_case(86, seqs, heads[0], heads[1], 64, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case, out_dtype=out_dtype)
+    out, path = dev.run()
+    assert path == "paged_mfma"
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    assert np.isfinite(out).all()
+    tol = 1e-2 if (cache_dtype == W.BF16 or q_dtype == W.BF16) else 2e-3
+    assert H.scaled_bound_error(out, ref, "paged chunks head 64") <= tol
+    out2, _ = dev.run(flags=hip.PA_SKIP_CACHE_WRITE, decode_waves=33)
+    assert H.max_abs(out2, out) <= tol
     dev.free()
 
 
