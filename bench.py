@@ -690,14 +690,17 @@ def main():
         del case
 
     if not args.no_extra:
-        # config3's batch at the other cache shapes of the matrix-core decode kernel (not reference
+        # config3's batch at the other cache shapes of the matrix-core decode kernel and, at head size
+        # 96, through the query-tile kernel that takes every other 16-bit shape (not reference
         # configurations; no byte counters recorded for them)
-        for D, bs in ((64, 32), (64, 16), (128, 16)):
+        for D, bs in ((64, 32), (64, 16), (128, 16), (96, 16)):
             key = "c3_d%d_blk%d" % (D, bs)
             case = W.config3(head_dim=D, block_size=bs)
             r = bench_paged(hip, case, args.steps, args.warmup,
                             "config3's batch with head size %d and cache blocks of %d tokens" % (D, bs))
             r["roofline"] = roofline_hbm(r, key)
+            if r["kernel_path"] == "paged_mfma_tiles":
+                r["roofline"]["kernel"] = "paged_tiles_kernel"
             log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f (%s)"
                 % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))
             results[key] = r
@@ -709,6 +712,13 @@ def main():
             log("%s: %.3f ms/step (%s)" % (key, r["ms_per_step"], r["kernel_path"]))
             results[key] = r
             del case
+        case = W.config2(D=96)
+        r = bench_sdpa(hip, case, args.steps, args.warmup, "config2's shape at head size 96 (the plain matrix-core kernel, columns padded to 128)")
+        r["roofline"] = roofline_mfma(r)
+        r["roofline"]["traffic"], r["roofline"]["traffic_source"], r["roofline"]["kernel"] = None, None, "sdpa_flash_small_kernel"
+        log("c2_d96: %.3f ms/step, roofline frac %.3f (%s)" % (r["ms_per_step"], r["roofline"]["frac"], r["kernel_path"]))
+        results["c2_d96"] = r
+        del case
         results["c2_masked"] = bench_sdpa_masked(hip, args.steps)
         log("c2's shape with the causality as an attention mask: %.3f ms, %.0f TFLOP/s (%s)"
             % (results["c2_masked"]["ms_per_step"], results["c2_masked"]["tflops"], results["c2_masked"]["kernel_path"]))

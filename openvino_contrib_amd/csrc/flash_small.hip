@@ -12,6 +12,8 @@
 //
 // Replaces the same decomposed chain as flash_prefill.hip (src/ops/matmul.cpp:185-227,
 // src/ops/softmax.cpp:178-193, src/ops/select.cpp:50-91 of the reference).
+#include <algorithm>
+
 #include "device_common.hpp"
 #include "kernels.hpp"
 
@@ -19,12 +21,13 @@ namespace hipattn {
 
 namespace flash_small {
 
-constexpr int kD = 64;
-constexpr int kRowBytes = kD * 2;           // a K or V row in LDS: 8 chunks of 16 bytes
+// kDP is the head size the kernel is built for, 64 or 128; the call's head size (w.head_dim, a
+// multiple of 8) may be smaller: the missing columns of Q, K and V are zeros in registers and LDS.
 constexpr int kTileK = 64;                  // keys per tile
-constexpr int kTileBytes = kTileK * kRowBytes;
 constexpr int kWaves = 4;
 constexpr int kTileQ = 32 * kWaves;         // query rows per workgroup
+template <int kDP>
+constexpr int tile_bytes() { return kTileK * kDP * 2; }  // a K or V tile in LDS: rows of kDP / 8 chunks of 16 bytes
 
 template <bool kBf16>
 struct Mfma;
@@ -61,12 +64,19 @@ __device__ __forceinline__ void pair_values(float x, float& lo, float& hi) {
     hi = __uint_as_float(r[1]);
 }
 
-// LDS position of the 16-byte chunk c (0..7) of row r of a tile.  K: chunk c ^ ((r >> 1) & 7), so
-// that sixteen lanes reading one chunk index of sixteen consecutive rows (a K fragment) hit sixteen
-// different 16-byte bank groups; V: chunk c ^ (4 * ((r >> 1) & 1)), so that the four rows a
-// transposing read touches at once lie in four different quarters of the banks.
-__device__ __forceinline__ int k_chunk_offset(int r, int c) { return r * kRowBytes + ((c ^ ((r >> 1) & 7)) << 4); }
-__device__ __forceinline__ int v_chunk_offset(int r, int c) { return r * kRowBytes + ((c ^ (((r >> 1) & 1) << 2)) << 4); }
+// LDS position of the 16-byte chunk c of row r of a tile.  K: sixteen lanes reading one chunk index
+// of sixteen consecutive rows (a K fragment) must hit sixteen different 16-byte bank groups: chunk
+// c ^ ((r >> 1) & 7) in 128-byte rows, c ^ (r & 15) in 256-byte rows.  V: the four rows a
+// transposing read touches at once must lie in four different quarters of the banks: chunk
+// c ^ (4 * ((r >> 1) & 1)) in 128-byte rows, c ^ (4 * (r & 3)) in 256-byte rows.
+template <int kDP>
+__device__ __forceinline__ int k_chunk_offset(int r, int c) {
+    return kDP == 64 ? r * 128 + ((c ^ ((r >> 1) & 7)) << 4) : r * 256 + ((c ^ (r & 15)) << 4);
+}
+template <int kDP>
+__device__ __forceinline__ int v_chunk_offset(int r, int c) {
+    return kDP == 64 ? r * 128 + ((c ^ (((r >> 1) & 1) << 2)) << 4) : r * 256 + ((c ^ ((r & 3) << 2)) << 4);
+}
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef short short8_t __attribute__((ext_vector_type(8)));
@@ -79,14 +89,14 @@ typedef __attribute__((address_space(3))) short4_t lds_short4;
 // hands lane i of a 16-lane group element j = what lane 4j + i/4 of the group addressed, at
 // 16-bit index i % 4; so lane i addresses row key0 + i/4, head-dim d0 + 4(i % 4).. and receives
 // V[key0 + j][d0 + i] (d0 = dt*32 + 16(group & 1), key0 = 16ks + 4(group >> 1)).
-template <bool kBf16>
+template <bool kBf16, int kDP>
 __device__ __forceinline__ typename Mfma<kBf16>::vec8 read_v_frag(const lds_byte* v_lds, int lane, int ks, int dt) {
     const int g = lane >> 4, i = lane & 15;
     const int row = 16 * ks + 4 * (g >> 1) + (i >> 2);
     const int d0 = dt * 32 + 16 * (g & 1) + 4 * (i & 3);  // first of this lane's four head-dim elements
     const int c = d0 >> 3, within = (d0 & 7) * 2;
-    const lds_byte* p0 = v_lds + v_chunk_offset(row, c) + within;
-    const lds_byte* p1 = v_lds + v_chunk_offset(row + 8, c) + within;
+    const lds_byte* p0 = v_lds + v_chunk_offset<kDP>(row, c) + within;
+    const lds_byte* p1 = v_lds + v_chunk_offset<kDP>(row + 8, c) + within;
     const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)p0);
     const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)p1);
     const short8_t a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
@@ -140,10 +150,12 @@ struct Work {
     void* out;              // as q
     int64_t out_stride;
     int out_dtype;          // HIPATTN_F16 / BF16 / F32
+    int head_dim;           // <= kDP, a multiple of 8
     int rows;               // query rows of the tile that exist (1..128)
-    int pos0;               // position of row 0: under `causal` row r attends keys <= pos0 + r ...
+    int pos0;               // position of row 0: under `causal` row r attends keys <= pos0 + r * pos_step ...
+    int pos_step;           // 1: rows are consecutive tokens; 0: rows are the query heads of one token
     int causal;
-    int window;             // ... and, when > 0, keys > pos0 + r - window
+    int window;             // ... and, when > 0, keys > that position - window
     int kv_len;
     const uint8_t* k;       // dense: the kv head's rows; paged: the cache at the kv head's offset inside a block
     const uint8_t* v;
@@ -164,32 +176,36 @@ __device__ __forceinline__ uint32_t pack2(int dtype, float lo, float hi) {
 // The workgroup's 128 query rows against the keys they attend.
 // kMask: the call carries an attention mask: its values are fetched from global memory ahead of the
 // score product of every tile and added behind it.  kPaged: K and V rows are found through w.table.
-template <bool kBf16, bool kMask, bool kPaged>
-__device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileBytes]) {
+template <bool kBf16, bool kMask, bool kPaged, int kDP>
+__device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_bytes<kDP>()]) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
+    constexpr int kChunks = kDP / 8;             // 16-byte chunks of a row in LDS
+    const int chunks = w.head_dim >> 3;          // ... of which the call's rows fill this many
+    const int row_bytes = w.head_dim * 2;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int n32 = lane & 31, hi = lane >> 5;
     const int my_row = wave * 32 + n32;          // this lane's query row in the tile (may lie beyond w.rows)
-    const int my_pos = w.pos0 + my_row;
+    const int my_pos = w.pos0 + my_row * w.pos_step;
     const bool windowed = kPaged && w.window > 0;
 
     // key tiles this workgroup visits: up to its last query row under the causal flag, from the
     // first row's window start on
-    const int kv_end = w.causal ? min(w.kv_len, w.pos0 + w.rows) : w.kv_len;
+    const int kv_end = w.causal ? min(w.kv_len, w.pos0 + (w.rows - 1) * w.pos_step + 1) : w.kv_len;
     const int tiles = (kv_end + kTileK - 1) / kTileK;
     const int tile0 = windowed ? max(0, w.pos0 - w.window + 1) / kTileK : 0;
 
     // Q^T fragments (B operand of S^T = K Q^T): lane (n32, hi) holds query row n32, head-dim
     // elements 8 (2i + hi) .. + 7 for k-step i, times scale * log2(e)
-    vec8 qf[4];
+    vec8 qf[kDP / 16];
     {
         const float c = w.scale * kLog2e;
         const int row = min(my_row, w.rows - 1);
         const bool q_bf16 = w.q_dtype == HIPATTN_BF16;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint4_t raw = *(const uint4_t*)(w.q + (int64_t)row * w.q_stride + 8 * (2 * i + hi));
+        for (int i = 0; i < kDP / 16; i++) {
+            uint4_t raw = {0u, 0u, 0u, 0u};
+            if (2 * i + hi < chunks) raw = *(const uint4_t*)(w.q + (int64_t)row * w.q_stride + 8 * (2 * i + hi));
             uint4_t cv;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -201,49 +217,71 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileByt
         }
     }
 
-    // tile staging: 512 16-byte pieces per K tile and per V tile, two of each per thread
-    uint4_t stage[4];
-    auto fetch = [&](int tile) {
+    // tile staging: 64 * kChunks 16-byte pieces per K tile and per V tile, kPieces of each per thread
+    constexpr int kPieces = kTileK * kChunks / (64 * kWaves);
+    uint4_t stage[2 * kPieces];
+    // paged: the block ids of a tile's rows are looked up one tile ahead of its K/V loads, so that
+    // those loads do not wait for the table
+    int block_of[kPieces];
+    auto lookup = [&](int tile) {
+        if constexpr (kPaged) {
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            const int piece = tid + 256 * s, r = piece >> 3, c = piece & 7;
+            for (int s = 0; s < kPieces; s++) {
+                const int piece = tid + 64 * kWaves * s, r = piece / kChunks;
+                const int key = min(tile * kTileK + r, w.kv_len - 1);
+                block_of[s] = w.table[key >> w.block_shift];
+            }
+        }
+    };
+    auto fetch = [&](int tile) {  // (paged: after lookup(tile))
+#pragma unroll
+        for (int s = 0; s < kPieces; s++) {
+            const int piece = tid + 64 * kWaves * s, r = piece / kChunks, c = piece % kChunks;
             const int key = min(tile * kTileK + r, w.kv_len - 1);  // rows past the end repeat the last key (masked later)
             int64_t at;
             if constexpr (kPaged) {
                 // a block id outside the cache is redirected into it: the rows that attend it are unspecified
-                const int pb = min(max(w.table[key >> w.block_shift], 0), w.num_blocks - 1);
-                at = (int64_t)pb * w.block_stride + (int64_t)(key & ((1 << w.block_shift) - 1)) * kRowBytes + 16 * c;
+                const int pb = min(max(block_of[s], 0), w.num_blocks - 1);
+                at = (int64_t)pb * w.block_stride + (int64_t)(key & ((1 << w.block_shift) - 1)) * row_bytes + 16 * c;
             } else {
-                at = (int64_t)key * kRowBytes + 16 * c;
+                at = (int64_t)key * row_bytes + 16 * c;
             }
-            stage[s] = *(const uint4_t*)(w.k + at);
-            stage[2 + s] = *(const uint4_t*)(w.v + at);
+            stage[s] = stage[kPieces + s] = (uint4_t){0u, 0u, 0u, 0u};
+            if (c < chunks) {
+                stage[s] = *(const uint4_t*)(w.k + at);
+                stage[kPieces + s] = *(const uint4_t*)(w.v + at);
+            }
         }
     };
     auto deposit = [&](int buf) {
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            const int piece = tid + 256 * s, r = piece >> 3, c = piece & 7;
-            *(uint4_t*)(lds[buf][0] + k_chunk_offset(r, c)) = stage[s];
-            *(uint4_t*)(lds[buf][1] + v_chunk_offset(r, c)) = stage[2 + s];
+        for (int s = 0; s < kPieces; s++) {
+            const int piece = tid + 64 * kWaves * s, r = piece / kChunks, c = piece % kChunks;
+            *(uint4_t*)(lds[buf][0] + k_chunk_offset<kDP>(r, c)) = stage[s];
+            *(uint4_t*)(lds[buf][1] + v_chunk_offset<kDP>(r, c)) = stage[kPieces + s];
         }
     };
 
-    float16_t o[2];
+    float16_t o[kDP / 32];
 #pragma unroll
-    for (int dt = 0; dt < 2; dt++)
+    for (int dt = 0; dt < kDP / 32; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;  // the row's running maximum (both lanes of a pair agree) and this lane's share of the sum
 
     if (tile0 < tiles) {
+        lookup(tile0);
         fetch(tile0);
+        if (tile0 + 1 < tiles) lookup(tile0 + 1);
         deposit(0);
     }
     __syncthreads();
     for (int j = tile0; j < tiles; j++) {
         const int buf = (j - tile0) & 1;
-        if (j + 1 < tiles) fetch(j + 1);  // in flight while this tile is computed
+        if (j + 1 < tiles) {
+            fetch(j + 1);  // in flight while this tile is computed
+            if (j + 2 < tiles) lookup(j + 2);
+        }
         const lds_byte* k_lds = (const lds_byte*)lds[buf][0];
         const lds_byte* v_lds = (const lds_byte*)lds[buf][1];
         const int ts = j * kTileK;
@@ -270,9 +308,9 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileByt
 #pragma unroll
             for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < kDP / 16; i++) {
                 const int row = mt * 32 + n32;
-                const vec8 kf = __builtin_bit_cast(vec8, *(const __attribute__((address_space(3))) uint4_t*)(k_lds + k_chunk_offset(row, 2 * i + hi)));
+                const vec8 kf = __builtin_bit_cast(vec8, *(const __attribute__((address_space(3))) uint4_t*)(k_lds + k_chunk_offset<kDP>(row, 2 * i + hi)));
                 s[mt] = M::mma(kf, qf[i], s[mt]);
             }
         }
@@ -283,9 +321,9 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileByt
         // mask: keys past the end, keys after the query under the causal flag, keys that have left
         // the window (the tile holds one for some row of the wavefront when its first key lies
         // before the window of the wavefront's last row)
-        const int wave_pos = w.pos0 + wave * 32;
+        const int wave_pos = w.pos0 + wave * 32 * w.pos_step;
         const bool edge = ts + kTileK > w.kv_len || (w.causal && ts + kTileK - 1 > wave_pos) ||
-                          (windowed && ts <= wave_pos + 31 - w.window);
+                          (windowed && ts <= wave_pos + 31 * w.pos_step - w.window);
         if (edge) {
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
@@ -325,14 +363,14 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileByt
         l_run = l_run * alpha + sum;
         m_run = m_new;
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++)
+        for (int dt = 0; dt < kDP / 32; dt++)
 #pragma unroll
             for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
         // O^T += V^T P^T
 #pragma unroll
         for (int ks = 0; ks < 4; ks++)
 #pragma unroll
-            for (int dt = 0; dt < 2; dt++) o[dt] = M::mma(read_v_frag<kBf16>(v_lds, lane, ks, dt), pf[ks], o[dt]);
+            for (int dt = 0; dt < kDP / 32; dt++) o[dt] = M::mma(read_v_frag<kBf16, kDP>(v_lds, lane, ks, dt), pf[ks], o[dt]);
 
         if (j + 1 < tiles) deposit(buf ^ 1);  // the other buffer was last read before the previous barrier
         __syncthreads();
@@ -345,10 +383,11 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileByt
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
     if (my_row < w.rows) {
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++)
+        for (int dt = 0; dt < kDP / 32; dt++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int d = dt * 32 + 8 * g + 4 * hi;
+                if (d >= w.head_dim) continue;
                 const float x0 = o[dt][4 * g] * inv, x1 = o[dt][4 * g + 1] * inv, x2 = o[dt][4 * g + 2] * inv, x3 = o[dt][4 * g + 3] * inv;
                 if (kPaged && w.out_dtype == HIPATTN_F32) {
                     *(float4*)((float*)w.out + (int64_t)my_row * w.out_stride + d) = make_float4(x0, x1, x2, x3);
@@ -364,29 +403,31 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][kTileByt
 
 // Dense SDPA: one workgroup per (batch, query head, 128-row query tile).  kMask: p.mask rides along
 // (ignored under the causal flag).
-template <bool kBf16, bool kMask = false>
-__global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][kTileBytes];  // [buffer][K, V]
+template <bool kBf16, bool kMask, int kDP>
+__device__ __forceinline__ void sdpa_small_tile(const SdpaParams& p, uint8_t (*lds)[2][tile_bytes<kDP>()]) {
     const int q_tiles = (p.len_q + kTileQ - 1) / kTileQ;
     const int qt = blockIdx.x % q_tiles;
     const int h = (blockIdx.x / q_tiles) % p.num_heads_q;
     const int b = blockIdx.x / (q_tiles * p.num_heads_q);
     const int hkv = h / (p.num_heads_q / p.num_heads_kv);
     const int q0 = qt * kTileQ;
+    const int D = p.head_dim;
     Work w;
-    w.q = (const uint16_t*)p.q + ((int64_t)(b * p.num_heads_q + h) * p.len_q + q0) * kD;
-    w.q_stride = kD;
+    w.q = (const uint16_t*)p.q + ((int64_t)(b * p.num_heads_q + h) * p.len_q + q0) * D;
+    w.q_stride = D;
     w.q_dtype = p.dtype;
-    w.out = (uint16_t*)p.out + ((int64_t)(b * p.num_heads_q + h) * p.len_q + q0) * kD;
-    w.out_stride = kD;
+    w.out = (uint16_t*)p.out + ((int64_t)(b * p.num_heads_q + h) * p.len_q + q0) * D;
+    w.out_stride = D;
     w.out_dtype = p.dtype;
+    w.head_dim = D;
     w.rows = min(kTileQ, p.len_q - q0);
     w.pos0 = q0;
+    w.pos_step = 1;
     w.causal = p.causal;
     w.window = 0;
     w.kv_len = p.len_kv;
-    w.k = (const uint8_t*)p.k + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
-    w.v = (const uint8_t*)p.v + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * kRowBytes;
+    w.k = (const uint8_t*)p.k + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * D * 2;
+    w.v = (const uint8_t*)p.v + ((int64_t)(b * p.num_heads_kv + hkv) * p.len_kv) * D * 2;
     w.table = nullptr;
     w.block_shift = 0;
     w.num_blocks = 0;
@@ -403,16 +444,33 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_d64_kernel(SdpaParams 
         w.mask_key_stride = p.mask_stride[3];
         w.mask_dtype = p.mask_dtype;
     }
-    attend<kBf16, kMask, false>(w, lds);
+    attend<kBf16, kMask, false, kDP>(w, lds);
 }
 
-// Chunked prefill over the block table (PagedAttentionExtension, 16-bit caches, head size 64): one
-// workgroup per (128-row query tile of a multi-token sequence, query head); the tiles of the batch
-// are numbered by p.tile_prefix (written by the plan on the device), the later -- heavier -- tiles
-// of a sequence first, the query heads of a tile side by side.  The grid is an upper bound.
-template <bool kBf16>
-__global__ __launch_bounds__(64 * kWaves) void paged_prefill_d64_kernel(PagedParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][kTileBytes];
+// (two workgroups per compute unit also in the head-128 build: at most 256 registers)
+template <bool kBf16, int kDP>
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))) void sdpa_flash_small_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];  // [buffer][K, V]
+    sdpa_small_tile<kBf16, false, kDP>(p, lds);
+}
+
+// (the mask values of a tile take 32 more registers: no bound on them)
+template <bool kBf16, int kDP>
+__global__ __launch_bounds__(64 * kWaves) void sdpa_flash_small_masked_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];
+    sdpa_small_tile<kBf16, true, kDP>(p, lds);
+}
+
+// Query tiles of a PagedAttentionExtension batch over the block table (16-bit caches): a sequence
+// of n > 1 tokens has ceil(n / 128) tiles per query head; with p.tiles_only a single-token sequence
+// has one tile per kv head whose rows are the query heads of the group (without it such sequences
+// belong to the decode kernel and have no tile).  The tiles of the batch are numbered by
+// p.tile_prefix (written on the device by the plan of the decode path or by paged_tiles_plan_kernel),
+// the later -- heavier -- tiles of a sequence first.  One workgroup per (tile, head); the grid is
+// an upper bound.
+template <bool kBf16, int kDP>
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))) void paged_tiles_kernel(PagedParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];
     const int item = blockIdx.x / p.num_heads_q, h = blockIdx.x % p.num_heads_q;
     if (item >= p.tile_prefix[p.num_seqs]) return;
     int lo = 0, hi_s = p.num_seqs;  // the sequence owning the tile: largest s with tile_prefix[s] <= item
@@ -431,71 +489,167 @@ __global__ __launch_bounds__(64 * kWaves) void paged_prefill_d64_kernel(PagedPar
     const int past = p.past_lens[s];
     const int tb0 = p.block_indices_begins[s];
     const int table_len = p.block_indices_begins[s + 1] - tb0;
-    const int G = p.num_heads_q / p.num_heads_kv;
-    const int64_t row0 = (int64_t)(t0 + qt * kTileQ) * p.num_heads_q + h;
+    const int G = p.num_heads_q / p.num_heads_kv, D = p.head_dim;
+    const bool heads_as_rows = qlen == 1;  // (only tiles_only gives such a sequence a tile)
+    if (heads_as_rows && h >= p.num_heads_kv) return;
+    const int hkv = heads_as_rows ? h : h / G;
+    const int64_t row0 = heads_as_rows ? (int64_t)t0 * p.num_heads_q + (int64_t)h * G
+                                       : (int64_t)(t0 + qt * kTileQ) * p.num_heads_q + h;
     Work w;
-    w.q = (const uint16_t*)p.q + row0 * kD;
-    w.q_stride = (int64_t)p.num_heads_q * kD;
+    w.q = (const uint16_t*)p.q + row0 * D;
+    w.q_stride = heads_as_rows ? D : (int64_t)p.num_heads_q * D;
     w.q_dtype = p.q_dtype;
-    w.out = p.out_dtype == HIPATTN_F32 ? (void*)((float*)p.out + row0 * kD) : (void*)((uint16_t*)p.out + row0 * kD);
-    w.out_stride = (int64_t)p.num_heads_q * kD;
+    w.out = p.out_dtype == HIPATTN_F32 ? (void*)((float*)p.out + row0 * D) : (void*)((uint16_t*)p.out + row0 * D);
+    w.out_stride = w.q_stride;
     w.out_dtype = p.out_dtype;
-    w.rows = min(kTileQ, qlen - qt * kTileQ);
+    w.head_dim = D;
+    w.rows = heads_as_rows ? G : min(kTileQ, qlen - qt * kTileQ);
     w.pos0 = past + qt * kTileQ;
+    w.pos_step = heads_as_rows ? 0 : 1;
     w.causal = 1;
     w.window = p.sliding_window;
     w.kv_len = min(past + qlen, table_len * p.block_size);
-    const int64_t head_off = (int64_t)(h / G) * p.block_size * kRowBytes;
+    const int64_t head_off = (int64_t)hkv * p.block_size * D * 2;
     w.k = p.key_cache + head_off;
     w.v = p.value_cache + head_off;
     w.table = p.block_indices + tb0;
     w.block_shift = __builtin_ctz(p.block_size);
     w.num_blocks = p.num_blocks;
-    w.block_stride = (int64_t)p.num_heads_kv * p.block_size * kRowBytes;
+    w.block_stride = (int64_t)p.num_heads_kv * p.block_size * D * 2;
     w.scale = p.scale;
     w.mask = nullptr;
     w.mask_row_stride = w.mask_key_stride = 0;
     w.mask_dtype = 0;
-    attend<kBf16, false, true>(w, lds);
+    attend<kBf16, false, true, kDP>(w, lds);
+}
+
+// tile_prefix for a batch in which every sequence with tokens goes through paged_tiles_kernel
+// (p.tiles_only): exclusive prefix sums of ceil(tokens / 128) over the sequences.  One workgroup.
+__global__ __launch_bounds__(256) void paged_tiles_plan_kernel(PagedParams p) {
+    __shared__ int wave_total[4];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int per = (p.num_seqs + 255) / 256;
+    const int s0 = min(tid * per, p.num_seqs), s1 = min(s0 + per, p.num_seqs);
+    int mine = 0;
+    for (int s = s0; s < s1; s++) mine += (max(p.subsequence_begins[s + 1] - p.subsequence_begins[s], 0) + kTileQ - 1) / kTileQ;
+    int scan = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(scan, d, 64);
+        if (lane >= d) scan += up;
+    }
+    if (lane == 63) wave_total[wv] = scan;
+    __syncthreads();
+    int tile = scan - mine;
+    for (int w = 0; w < wv; w++) tile += wave_total[w];
+    for (int s = s0; s < s1; s++) {
+        p.tile_prefix[s] = tile;
+        tile += (max(p.subsequence_begins[s + 1] - p.subsequence_begins[s], 0) + kTileQ - 1) / kTileQ;
+    }
+    if (s1 == p.num_seqs && s0 < p.num_seqs) p.tile_prefix[p.num_seqs] = tile;
 }
 
 }  // namespace flash_small
 
+static bool aligned16(const void* q) { return ((uintptr_t)q & 15) == 0; }
+
+// 16-bit operands, head sizes that are multiples of 8 up to 128.
 bool sdpa_flash_small_supported(const SdpaParams& p) {
-    return p.head_dim == flash_small::kD && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16) &&
-           p.len_kv > 0 && p.len_q > 0 && ((uintptr_t)p.q % 16) == 0 && ((uintptr_t)p.k % 16) == 0 &&
-           ((uintptr_t)p.v % 16) == 0 && ((uintptr_t)p.out % 8) == 0;
+    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16) &&
+           p.len_kv > 0 && p.len_q > 0 && aligned16(p.q) && aligned16(p.k) && aligned16(p.v) && ((uintptr_t)p.out % 8) == 0;
 }
 
-hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream) {
+template <bool kMask>
+static void launch_sdpa_small(const SdpaParams& p, unsigned groups, hipStream_t stream) {
+    const dim3 grid(groups), block(64 * flash_small::kWaves);
+    const bool bf16 = p.dtype == HIPATTN_BF16, small = p.head_dim <= 64;
+    if constexpr (kMask) {
+        if (small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<true, 64>), grid, block, 0, stream, p);
+        if (small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<false, 64>), grid, block, 0, stream, p);
+        if (!small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<true, 128>), grid, block, 0, stream, p);
+        if (!small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<false, 128>), grid, block, 0, stream, p);
+    } else {
+        if (small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<true, 64>), grid, block, 0, stream, p);
+        if (small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<false, 64>), grid, block, 0, stream, p);
+        if (!small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<true, 128>), grid, block, 0, stream, p);
+        if (!small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<false, 128>), grid, block, 0, stream, p);
+    }
+}
+
+hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe) {
     const int64_t q_tiles = (p.len_q + flash_small::kTileQ - 1) / flash_small::kTileQ;
     const int64_t groups = q_tiles * p.num_heads_q * p.batch;
     if (groups == 0) return hipSuccess;
     if (groups > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (p.mask != nullptr && !p.causal) {
-        if (p.dtype == HIPATTN_BF16)
-            hipLaunchKernelGGL((flash_small::sdpa_flash_d64_kernel<true, true>), dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
-        else
-            hipLaunchKernelGGL((flash_small::sdpa_flash_d64_kernel<false, true>), dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
-        return hipGetLastError();
-    }
-    if (p.dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL(flash_small::sdpa_flash_d64_kernel<true>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+    if (probe.before) (void)hipEventRecord(probe.before, stream);
+    if (p.mask != nullptr && !p.causal)
+        launch_sdpa_small<true>(p, (unsigned)groups, stream);
     else
-        hipLaunchKernelGGL(flash_small::sdpa_flash_d64_kernel<false>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
-    return hipGetLastError();
+        launch_sdpa_small<false>(p, (unsigned)groups, stream);
+    const hipError_t e = hipGetLastError();
+    if (probe.after) (void)hipEventRecord(probe.after, stream);
+    return e;
 }
 
-// The multi-token sequences of a planned batch (p.tile_prefix, p.max_q_tiles), head size 64.
+static void launch_tiles(const PagedParams& p, unsigned groups, hipStream_t stream) {
+    const dim3 grid(groups), block(64 * flash_small::kWaves);
+    const bool bf16 = p.cache_dtype == HIPATTN_BF16;
+    if (p.head_dim <= 64) {
+        if (bf16)
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 64>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 64>), grid, block, 0, stream, p);
+    } else {
+        if (bf16)
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 128>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 128>), grid, block, 0, stream, p);
+    }
+}
+
+// The multi-token sequences of a batch planned by the decode path (p.tile_prefix, p.max_q_tiles), head size 64.
 hipError_t launch_paged_prefill_small(const PagedParams& p, hipStream_t stream) {
     const int64_t groups = (int64_t)p.max_q_tiles * p.num_heads_q;
     if (groups == 0) return hipSuccess;
     if (groups > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (p.cache_dtype == HIPATTN_BF16)
-        hipLaunchKernelGGL(flash_small::paged_prefill_d64_kernel<true>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
-    else
-        hipLaunchKernelGGL(flash_small::paged_prefill_d64_kernel<false>, dim3((unsigned)groups), dim3(64 * flash_small::kWaves), 0, stream, p);
+    launch_tiles(p, (unsigned)groups, stream);
     return hipGetLastError();
+}
+
+// Whole batches through the tile kernel: 16-bit caches and queries whose shape the decode path
+// does not take -- head sizes that are multiples of 8 up to 128, block sizes that are powers of
+// two, up to 128 query heads per kv head.
+bool paged_tiles_supported(const PagedParams& p) {
+    const int G = p.num_heads_q / p.num_heads_kv;
+    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && G <= flash_small::kTileQ &&
+           p.block_size > 0 && (p.block_size & (p.block_size - 1)) == 0 &&
+           (p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16) &&
+           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16) && aligned16(p.q) && aligned16(p.key_cache) &&
+           aligned16(p.value_cache) && ((uintptr_t)p.out % (p.out_dtype == HIPATTN_F32 ? 16 : 8)) == 0;
+}
+
+static int64_t tiles_bound(const PagedParams& p) {  // every sequence with tokens wastes at most one tile
+    return (int64_t)p.num_tokens / flash_small::kTileQ + std::min(p.num_seqs, p.num_tokens);
+}
+
+size_t paged_tiles_workspace_bytes(const PagedParams& p) { return ((size_t)p.num_seqs + 1) * sizeof(int32_t); }
+
+// (the new tokens are in the cache already)
+hipError_t launch_paged_tiles(const PagedParams& p_in, void* workspace, hipStream_t stream, const KernelProbe& probe) {
+    PagedParams p = p_in;
+    p.tile_prefix = (int32_t*)workspace;
+    p.tiles_only = 1;
+    const int64_t groups = tiles_bound(p) * p.num_heads_q;
+    if (groups == 0) return hipSuccess;
+    if (groups > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(flash_small::paged_tiles_plan_kernel, dim3(1), dim3(256), 0, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (probe.before) (void)hipEventRecord(probe.before, stream);
+    launch_tiles(p, (unsigned)groups, stream);
+    e = hipGetLastError();
+    if (probe.after) (void)hipEventRecord(probe.after, stream);
+    return e;
 }
 
 }  // namespace hipattn

@@ -408,8 +408,8 @@ HIPATTN_EXPORT hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc,
         g_kernel_path = p.mask ? "sdpa_flash_mfma_masked" : "sdpa_flash_mfma";
         HIP_TRY(hipattn::launch_sdpa_flash(p, as_stream(stream), g_probe));
     } else if (hipattn::sdpa_flash_small_supported(p)) {
-        g_kernel_path = "sdpa_flash_mfma_d64";
-        HIP_TRY(hipattn::launch_sdpa_flash_small(p, as_stream(stream)));
+        g_kernel_path = p.head_dim == 64 ? "sdpa_flash_mfma_d64" : "sdpa_flash_mfma_small";
+        HIP_TRY(hipattn::launch_sdpa_flash_small(p, as_stream(stream), g_probe));
     } else {
         g_kernel_path = "sdpa_generic";
         HIP_TRY(hipattn::launch_sdpa_generic(p, as_stream(stream)));
@@ -445,8 +445,11 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention_workspace_size(const hipat
     *bytes = 0;
     if (hipattn_status st = validate_pa(desc, true)) return st;
     hipattn::PagedParams p = make_paged_params(desc);
-    if (!(desc->flags & HIPATTN_PA_FORCE_GENERIC) && hipattn::paged_fast_supported(p))
+    if (desc->flags & HIPATTN_PA_FORCE_GENERIC) return HIPATTN_OK;
+    if (hipattn::paged_fast_supported(p))
         *bytes = hipattn::paged_fast_workspace_bytes(p);
+    else if (hipattn::paged_tiles_supported(p))  // (pointers are not known here: a call with unaligned ones needs none)
+        *bytes = hipattn::paged_tiles_workspace_bytes(p);
     return HIPATTN_OK;
 }
 
@@ -477,8 +480,8 @@ hipattn_status paged_attention_impl(const hipattn_pa_desc* desc, const void* q, 
     p.block_indices_begins = block_indices_begins;
     p.out = out;
     p.no_side_stream = static_scratch ? 1 : 0;  // (creating the side stream of a mixed batch allocates)
-    if (!(desc->flags & HIPATTN_PA_FORCE_GENERIC) && hipattn::paged_fast_supported(p)) {
-        const size_t need = hipattn::paged_fast_workspace_bytes(p);
+    // the caller's workspace, or the static scratch, checked against what the chosen path needs
+    const auto take_workspace = [&](size_t need) -> hipattn_status {
         if (static_scratch) {
             if (need > (size_t)HIPATTN_NOALLOC_SCRATCH_BYTES)
                 return fail(HIPATTN_WORKSPACE_TOO_SMALL,
@@ -491,9 +494,19 @@ hipattn_status paged_attention_impl(const hipattn_pa_desc* desc, const void* q, 
                         need);
         if ((uintptr_t)workspace % 16)
             return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention: workspace must be 16-byte aligned");
+        return HIPATTN_OK;
+    };
+    const bool forced_generic = (desc->flags & HIPATTN_PA_FORCE_GENERIC) != 0;
+    if (!forced_generic && hipattn::paged_fast_supported(p)) {
+        if (hipattn_status st = take_workspace(hipattn::paged_fast_workspace_bytes(p))) return st;
         hipattn::paged_fast_plan(p, workspace);
         g_kernel_path = "paged_mfma";
         HIP_TRY(hipattn::launch_paged_fast(p, do_write ? &w : nullptr, as_stream(stream), g_probe));
+    } else if (!forced_generic && hipattn::paged_tiles_supported(p)) {
+        if (hipattn_status st = take_workspace(hipattn::paged_tiles_workspace_bytes(p))) return st;
+        g_kernel_path = "paged_mfma_tiles";
+        if (do_write) HIP_TRY(hipattn::launch_kv_cache_write(w, as_stream(stream)));
+        HIP_TRY(hipattn::launch_paged_tiles(p, workspace, as_stream(stream), g_probe));
     } else {
         g_kernel_path = "paged_generic";
         if (do_write) HIP_TRY(hipattn::launch_kv_cache_write(w, as_stream(stream)));

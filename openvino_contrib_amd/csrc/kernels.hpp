@@ -119,6 +119,7 @@ struct PagedParams {
                           // chunked-prefill kernel too (HIPATTN_PA_ANY_LENGTHS); without it such a batch is
                           // planned per token and every token is a decode row
     int no_side_stream;   // mixed batches run one kernel after the other on the caller's stream
+    int tiles_only;       // (flash_small.hip) tile_prefix counts single-token sequences too: there are no decode rows
 };
 
 // Optional event pair recorded around the dominant kernel of a call (measurement aid).
@@ -137,9 +138,14 @@ hipError_t launch_paged_generic(const PagedParams& p, hipStream_t stream);
 bool sdpa_flash_supported(const SdpaParams& p);
 bool sdpa_flash_mask_supported(const SdpaParams& p);  // p.mask can ride along in the flash kernel
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
-// head size 64 on the matrix cores (flash_small.hip)
+// head sizes up to 128 that are multiples of 8 on the matrix cores (flash_small.hip)
 bool sdpa_flash_small_supported(const SdpaParams& p);
-hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream);
+hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
+// paged attention of such shapes, 16-bit caches: every sequence of the batch as query tiles over the
+// block table (workspace: paged_tiles_workspace_bytes; the new tokens must be in the cache already)
+bool paged_tiles_supported(const PagedParams& p);
+size_t paged_tiles_workspace_bytes(const PagedParams& p);
+hipError_t launch_paged_tiles(const PagedParams& p, void* workspace, hipStream_t stream, const KernelProbe& probe);
 
 // paged attention fast paths: plan + stream-K decode + merge, and chunked prefill
 bool paged_fast_supported(const PagedParams& p);

@@ -111,8 +111,34 @@ def test_sdpa_small_shapes(hip, oracle, shape, causal, dtype):
     case = W.make_sdpa_case(61, B, Hq, Hkv, Lq, Lk, D, dtype)
     out, path = H.run_sdpa(hip, case, causal)
     ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
-    assert path == ("sdpa_flash_mfma_d64" if (D == 64 and dtype == W.F16) else "sdpa_generic")
+    # 16-bit operands with head sizes up to 128 run on the matrix cores (head size 64 in a kernel built
+    # for it, the others zero-padded to 64 or 128); fp32 and larger heads take the fp32 kernel
+    assert path == ("sdpa_generic" if (dtype == W.F32 or D > 128) else ("sdpa_flash_mfma_d64" if D == 64 else "sdpa_flash_mfma_small"))
     assert H.max_abs(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [W.F16, W.BF16])
+@pytest.mark.parametrize("D", [8, 32, 40, 80, 96, 112, 120])
+@pytest.mark.parametrize("B,Hq,Hkv,Lq,Lk,causal,masked", [(1, 4, 2, 130, 130, True, False), (2, 3, 1, 77, 300, False, False),
+                                                          (1, 2, 2, 300, 515, False, True), (1, 6, 2, 1, 1000, False, True),
+                                                          (2, 2, 1, 257, 64, True, False)])
+def test_sdpa_other_head_sizes_on_the_matrix_cores(hip, oracle, dtype, D, B, Hq, Hkv, Lq, Lk, causal, masked):
+    """Head sizes that are multiples of 8, up to 128: the head-64 / head-128 builds of the plain
+    matrix-core kernel with the missing columns as zeros, with and without an fp32 attention mask."""
+    announce("sdpa other head sizes", dtype, D, B, Hq, Hkv, Lq, Lk, causal, masked)
+    case = W.make_sdpa_case(64, B, Hq, Hkv, Lq, Lk, D, dtype, std=0.5 if dtype == W.BF16 else 1.0)
+    if masked:
+        rng = np.random.default_rng(D + Lk)
+        mask = (rng.standard_normal((B, 1, Lq, Lk)) * 2).astype(np.float32)
+        mask[..., Lk - 7:] = -np.inf
+        out, path = H.run_sdpa_masked(hip, case, mask)
+        ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask)
+    else:
+        out, path = H.run_sdpa(hip, case, causal)
+        ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+    assert path == "sdpa_flash_mfma_small"
+    assert np.isfinite(out).all()
+    assert H.scaled_bound_error(out, ref, "sdpa other head sizes") <= TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [W.F16, W.BF16])
@@ -274,7 +300,8 @@ def test_sdpa_with_attention_mask(hip, oracle, dtype, tol, mask_kind):
     else:
         mask = rng.standard_normal((1, Hq, 1, 1)).astype(np.float16)  # a constant per head: no effect on the result
     out, path = H.run_sdpa_masked(hip, case, mask)
-    assert path == "sdpa_generic"
+    # (130 keys and fp32 masks are off the grid of the tuned kernel's mask tiles)
+    assert path == ("sdpa_generic" if dtype == W.F32 else "sdpa_flash_mfma_small")
     ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask.astype(np.float32) if mask.dtype == np.float16 else mask)
     assert np.isfinite(out).all()
     assert H.max_abs(out, ref) <= tol
@@ -315,7 +342,7 @@ def test_sdpa_flash_with_mask(hip, oracle, dtype, kind, B, Hq, Hkv, Lq, Lk):
     if Lk % per16 == 0:
         assert path == "sdpa_flash_mfma_masked"
     else:
-        assert path == "sdpa_generic"
+        assert path == "sdpa_flash_mfma_small"  # the plain matrix-core kernel reads any mask layout
     ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask if kind.startswith("bool") else oracle.round_to(mask, dtype))
     assert np.isfinite(out).all()
     rows = np.isfinite(ref).all(-1)  # a row without a key is zeros here and undefined in the oracle
@@ -893,10 +920,10 @@ def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle):
     dev.free()
 
 
-@pytest.mark.parametrize("shape", [(6, 2, 96, 16, W.F16, W.F16), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
-                                   (4, 1, 128, 16, W.F16, W.U8), (34, 2, 128, 32, W.F16, W.F16)])
+@pytest.mark.parametrize("shape", [(6, 2, 96, 16, W.F32, W.F32), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
+                                   (4, 1, 128, 16, W.F16, W.U8), (4, 2, 64, 64, W.F16, W.U8)])
 def test_paged_generic_shapes(hip, oracle, shape):
-    """Head sizes, block sizes and GQA ratios outside the MFMA fast path."""
+    """fp32, head sizes above 128 and u8 caches off the tuned shape: the fp32 kernel."""
     announce("paged generic", shape)
     Hq, Hkv, D, bs, qd, cd = shape
     seqs = [(0, 9), (37, 1), (31, 2), (5, 40), (64, 1), (200, 1)]
@@ -909,6 +936,50 @@ def test_paged_generic_shapes(hip, oracle, shape):
     np.testing.assert_array_equal(kc, okc)
     tol = 1e-2 if (cd in (W.U8, W.BF16) or qd == W.BF16) else (1e-4 if qd == W.F32 else 2e-3)
     assert H.max_abs(out, ref) <= tol
+    dev.free()
+
+
+@pytest.mark.parametrize("shape", [(6, 2, 96, 16), (34, 2, 128, 32), (8, 8, 80, 8), (4, 1, 32, 64), (12, 4, 128, 8),
+                                   (3, 3, 8, 4), (16, 2, 112, 128), (40, 1, 64, 32), (128, 1, 48, 16)])
+@pytest.mark.parametrize("q_dtype,cache_dtype,out_dtype", [(W.F16, W.F16, None), (W.BF16, W.BF16, None), (W.BF16, W.F16, W.F32),
+                                                           (W.F16, W.BF16, W.BF16)])
+@pytest.mark.parametrize("window", [0, 50])
+def test_paged_other_shapes_on_the_matrix_cores(hip, oracle, shape, q_dtype, cache_dtype, out_dtype, window):
+    """16-bit caches whose shape the tuned kernels do not take (head sizes that are multiples of 8 up
+    to 128, any power-of-two block size, more than 16 query heads per kv head): every sequence goes
+    through the query-tile kernel over the block table, a single-token sequence as one tile per kv
+    head whose rows are the heads of the group."""
+    announce("paged tiles", shape, q_dtype, cache_dtype, out_dtype, window)
+    Hq, Hkv, D, bs = shape
+    seqs = [(0, 9), (37, 1), (31, 2), (5, 140), (64, 1), (200, 1), (0, 1), (127, 129), (3, 0), (600, 1)]
+    case = W.make_paged_case(87, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case, out_dtype=out_dtype)
+    out, path = dev.run()
+    assert path == "paged_mfma_tiles"
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    assert np.isfinite(out).all()
+    tol = 1e-2 if W.BF16 in (q_dtype, cache_dtype, out_dtype) else 2e-3
+    assert H.scaled_bound_error(out, ref, "paged tiles") <= tol
+    out_g, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic"
+    assert H.scaled_bound_error(out_g, ref, "paged tiles, generic") <= tol
+    dev.free()
+
+
+def test_paged_pure_decode_of_another_shape(hip, oracle):
+    """A decode batch at head size 96: one tile per (sequence, kv head)."""
+    announce("paged tiles decode")
+    seqs = [(c - 1, 1) for c in DECODE_CTX]
+    case = W.make_paged_case(88, seqs, 24, 8, 96, 16, W.F16, W.F16, W.F16)
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run()
+    assert path == "paged_mfma_tiles"
+    np.testing.assert_array_equal(dev.caches()[0], okc)
+    assert H.max_abs(out, ref) <= 2e-3
     dev.free()
 
 
