@@ -149,7 +149,7 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * At head_dim 128 a mask of the operands' 16-bit type, or a boolean one, whose keys lie side by
  * side (stride[3] == 1) rides along in the tuned matrix-core kernel when the mask pointer and the
  * other strides are multiples of 16 bytes (8 elements; 16 for boolean); every other mask beside
- * 16-bit operands with a head_dim that is a multiple of 8 up to 128 takes the plain matrix-core
+ * 16-bit operands with a head_dim that is a multiple of 8 up to 256 takes the plain matrix-core
  * kernel; fp32 operands and larger heads take the shape-generic kernel. */
 typedef struct hipattn_mask_desc {
     hipattn_dtype dtype;
@@ -194,7 +194,7 @@ hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q,
  * Kernels: 16-bit caches with head_dim 64 or 128 and block_size 16 or 32, and u8 caches with
  * head_dim 128 and block_size 32, take the tuned matrix-core kernels (stream-K decode for
  * single-token rows, chunked prefill over the block table for multi-token sequences); other
- * 16-bit caches with 16-bit queries, a head_dim that is a multiple of 8 up to 128 and a block_size
+ * 16-bit caches with 16-bit queries, a head_dim that is a multiple of 8 up to 256 and a block_size
  * that is a power of two take a plain matrix-core kernel (query tiles over the block table);
  * anything else (fp32, larger heads, other u8 shapes) takes the shape-generic fp32 kernels.
  * A single-token row with nothing to attend (an empty block table) gets an output row of zeros.

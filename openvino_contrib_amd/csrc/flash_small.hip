@@ -1,14 +1,15 @@
-// Flash attention on the matrix cores for dense v13::ScaledDotProductAttention at head size 64
-// (f16 / bf16, causal or not, GQA): the shape of the reference's own f16 test and of the small
-// model families.  The same products and the same register layout as the head-size-128 kernel of
-// flash_prefill.hip -- S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16, the accumulator of the
-// first being the B operand of the second -- in a plain structure: four wavefronts per workgroup,
-// 32 query rows each, key tiles of 64 staged through registers into a double-buffered, swizzled LDS
-// tile, one workgroup barrier per tile, a straightforward online softmax, an optional attention mask
-// of any type the operator allows.  Not tuned beyond conflict-free LDS access; it replaces the fp32
-// VALU kernel for these shapes.  The same body serves the multi-token sequences of a
-// PagedAttentionExtension batch at head size 64 (16-bit caches): K and V rows are then found
-// through the block table, under the causal order and the sliding window of that operator.
+// Flash attention on the matrix cores for every 16-bit shape the tuned kernels of flash_prefill.hip
+// and paged_decode.hip do not take: head sizes that are multiples of 8 up to 256 (f16 / bf16, causal
+// or not, GQA, any attention mask) -- among them head size 64, the shape of the reference's own f16
+// test and of the small model families -- dense (v13::ScaledDotProductAttention) and over the block
+// table of PagedAttentionExtension (16-bit caches, any power-of-two block size, causal order and
+// sliding window of that operator).  The same products and the same register layout as the
+// head-size-128 kernel of flash_prefill.hip -- S^T = K Q^T and O^T = V^T P^T on
+// v_mfma_f32_32x32x16, the accumulator of the first being the B operand of the second -- in a plain
+// structure: four wavefronts per workgroup, 32 query rows each, key tiles of 64 staged through
+// registers into a double-buffered, swizzled LDS tile, one workgroup barrier per tile, a
+// straightforward online softmax.  Not tuned beyond conflict-free LDS access; it replaces the fp32
+// VALU kernels for these shapes.
 //
 // Replaces the same decomposed chain as flash_prefill.hip (src/ops/matmul.cpp:185-227,
 // src/ops/softmax.cpp:178-193, src/ops/select.cpp:50-91 of the reference).
@@ -21,7 +22,7 @@ namespace hipattn {
 
 namespace flash_small {
 
-// kDP is the head size the kernel is built for, 64 or 128; the call's head size (w.head_dim, a
+// kDP is the head size the kernel is built for, 64, 128 or 256; the call's head size (w.head_dim, a
 // multiple of 8) may be smaller: the missing columns of Q, K and V are zeros in registers and LDS.
 constexpr int kTileK = 64;                  // keys per tile
 constexpr int kWaves = 4;
@@ -66,16 +67,16 @@ __device__ __forceinline__ void pair_values(float x, float& lo, float& hi) {
 
 // LDS position of the 16-byte chunk c of row r of a tile.  K: sixteen lanes reading one chunk index
 // of sixteen consecutive rows (a K fragment) must hit sixteen different 16-byte bank groups: chunk
-// c ^ ((r >> 1) & 7) in 128-byte rows, c ^ (r & 15) in 256-byte rows.  V: the four rows a
+// c ^ ((r >> 1) & 7) in 128-byte rows, c ^ (r & 15) in 256- and 512-byte rows.  V: the four rows a
 // transposing read touches at once must lie in four different quarters of the banks: chunk
-// c ^ (4 * ((r >> 1) & 1)) in 128-byte rows, c ^ (4 * (r & 3)) in 256-byte rows.
+// c ^ (4 * ((r >> 1) & 1)) in 128-byte rows, c ^ (4 * (r & 3)) in 256- and 512-byte rows.
 template <int kDP>
 __device__ __forceinline__ int k_chunk_offset(int r, int c) {
-    return kDP == 64 ? r * 128 + ((c ^ ((r >> 1) & 7)) << 4) : r * 256 + ((c ^ (r & 15)) << 4);
+    return kDP == 64 ? r * 128 + ((c ^ ((r >> 1) & 7)) << 4) : r * (kDP * 2) + ((c ^ (r & 15)) << 4);
 }
 template <int kDP>
 __device__ __forceinline__ int v_chunk_offset(int r, int c) {
-    return kDP == 64 ? r * 128 + ((c ^ (((r >> 1) & 1) << 2)) << 4) : r * 256 + ((c ^ ((r & 3) << 2)) << 4);
+    return kDP == 64 ? r * 128 + ((c ^ (((r >> 1) & 1) << 2)) << 4) : r * (kDP * 2) + ((c ^ ((r & 3) << 2)) << 4);
 }
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
@@ -286,20 +287,27 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
         const lds_byte* v_lds = (const lds_byte*)lds[buf][1];
         const int ts = j * kTileK;
 
-        float16_t mask_add[2];
-        if constexpr (kMask) {
+        // the mask values of the wavefront's rows for the 32 keys of half mt of the tile
+        auto mask_half = [&](int mt) __attribute__((always_inline)) -> float16_t {
+            float16_t add;
             const int row = min(my_row, w.rows - 1);
             const int esz = w.mask_dtype == HIPATTN_U8 ? 1 : (w.mask_dtype == HIPATTN_F32 ? 4 : 2);
             const uint8_t* mrow = w.mask + (int64_t)row * w.mask_row_stride * esz;
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++)
+            for (int g = 0; g < 4; g++) {
+                float m4[4];
+                mask_values4(mrow, w.mask_key_stride, w.mask_dtype, ts + mt * 32 + 8 * g + 4 * hi, w.kv_len, m4);
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    float m4[4];
-                    mask_values4(mrow, w.mask_key_stride, w.mask_dtype, ts + mt * 32 + 8 * g + 4 * hi, w.kv_len, m4);
+                for (int e = 0; e < 4; e++) add[4 * g + e] = m4[e];
+            }
+            return add;
+        };
+        // (the head-256 build has no registers to hold them across the score product: it fetches them behind it)
+        constexpr bool kMaskAhead = kMask && kDP < 256;
+        float16_t mask_add[2];
+        if constexpr (kMaskAhead) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) mask_add[mt][4 * g + e] = m4[e];
-                }
+            for (int mt = 0; mt < 2; mt++) mask_add[mt] = mask_half(mt);
         }
         // scores, transposed: register r of s[mt] is key ts + 32 mt + 8 (r / 4) + 4 hi + r % 4 of query row n32
         float16_t s[2];
@@ -314,9 +322,22 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
                 s[mt] = M::mma(kf, qf[i], s[mt]);
             }
         }
-        if constexpr (kMask) {
+        if constexpr (kMaskAhead) {
 #pragma unroll
             for (int mt = 0; mt < 2; mt++) s[mt] += mask_add[mt];
+        } else if constexpr (kMask) {
+            const int row = min(my_row, w.rows - 1);
+            const int esz = w.mask_dtype == HIPATTN_U8 ? 1 : (w.mask_dtype == HIPATTN_F32 ? 4 : 2);
+            const uint8_t* mrow = w.mask + (int64_t)row * w.mask_row_stride * esz;
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    float m4[4];
+                    mask_values4(mrow, w.mask_key_stride, w.mask_dtype, ts + mt * 32 + 8 * g + 4 * hi, w.kv_len, m4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) s[mt][4 * g + e] += m4[e];
+                }
         }
         // mask: keys past the end, keys after the query under the causal flag, keys that have left
         // the window (the tile holds one for some row of the wavefront when its first key lies
@@ -447,7 +468,8 @@ __device__ __forceinline__ void sdpa_small_tile(const SdpaParams& p, uint8_t (*l
     attend<kBf16, kMask, false, kDP>(w, lds);
 }
 
-// (two workgroups per compute unit also in the head-128 build: at most 256 registers)
+// (two workgroups per compute unit also in the head-128 build: at most 256 registers; the head-256
+// build needs nearly all 512 and runs one)
 template <bool kBf16, int kDP>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))) void sdpa_flash_small_kernel(SdpaParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];  // [buffer][K, V]
@@ -553,27 +575,37 @@ __global__ __launch_bounds__(256) void paged_tiles_plan_kernel(PagedParams p) {
 
 static bool aligned16(const void* q) { return ((uintptr_t)q & 15) == 0; }
 
-// 16-bit operands, head sizes that are multiples of 8 up to 128.
+// 16-bit operands, head sizes that are multiples of 8 up to 256.
 bool sdpa_flash_small_supported(const SdpaParams& p) {
-    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16) &&
+    return p.head_dim >= 8 && p.head_dim <= 256 && p.head_dim % 8 == 0 && (p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16) &&
            p.len_kv > 0 && p.len_q > 0 && aligned16(p.q) && aligned16(p.k) && aligned16(p.v) && ((uintptr_t)p.out % 8) == 0;
+}
+
+template <bool kMask, int kDP>
+static void launch_sdpa_small(const SdpaParams& p, unsigned groups, hipStream_t stream) {
+    const dim3 grid(groups), block(64 * flash_small::kWaves);
+    const bool bf16 = p.dtype == HIPATTN_BF16;
+    if constexpr (kMask) {
+        if (bf16)
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<true, kDP>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<false, kDP>), grid, block, 0, stream, p);
+    } else {
+        if (bf16)
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<true, kDP>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<false, kDP>), grid, block, 0, stream, p);
+    }
 }
 
 template <bool kMask>
 static void launch_sdpa_small(const SdpaParams& p, unsigned groups, hipStream_t stream) {
-    const dim3 grid(groups), block(64 * flash_small::kWaves);
-    const bool bf16 = p.dtype == HIPATTN_BF16, small = p.head_dim <= 64;
-    if constexpr (kMask) {
-        if (small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<true, 64>), grid, block, 0, stream, p);
-        if (small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<false, 64>), grid, block, 0, stream, p);
-        if (!small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<true, 128>), grid, block, 0, stream, p);
-        if (!small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<false, 128>), grid, block, 0, stream, p);
-    } else {
-        if (small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<true, 64>), grid, block, 0, stream, p);
-        if (small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<false, 64>), grid, block, 0, stream, p);
-        if (!small && bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<true, 128>), grid, block, 0, stream, p);
-        if (!small && !bf16) hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<false, 128>), grid, block, 0, stream, p);
-    }
+    if (p.head_dim <= 64)
+        launch_sdpa_small<kMask, 64>(p, groups, stream);
+    else if (p.head_dim <= 128)
+        launch_sdpa_small<kMask, 128>(p, groups, stream);
+    else
+        launch_sdpa_small<kMask, 256>(p, groups, stream);
 }
 
 hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe) {
@@ -599,6 +631,11 @@ static void launch_tiles(const PagedParams& p, unsigned groups, hipStream_t stre
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 64>), grid, block, 0, stream, p);
         else
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 64>), grid, block, 0, stream, p);
+    } else if (p.head_dim > 128) {
+        if (bf16)
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 256>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 256>), grid, block, 0, stream, p);
     } else {
         if (bf16)
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 128>), grid, block, 0, stream, p);
@@ -617,11 +654,11 @@ hipError_t launch_paged_prefill_small(const PagedParams& p, hipStream_t stream) 
 }
 
 // Whole batches through the tile kernel: 16-bit caches and queries whose shape the decode path
-// does not take -- head sizes that are multiples of 8 up to 128, block sizes that are powers of
+// does not take -- head sizes that are multiples of 8 up to 256, block sizes that are powers of
 // two, up to 128 query heads per kv head.
 bool paged_tiles_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
-    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && G <= flash_small::kTileQ &&
+    return p.head_dim >= 8 && p.head_dim <= 256 && p.head_dim % 8 == 0 && G <= flash_small::kTileQ &&
            p.block_size > 0 && (p.block_size & (p.block_size - 1)) == 0 &&
            (p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16) &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16) && aligned16(p.q) && aligned16(p.key_cache) &&

@@ -138,7 +138,7 @@ hipError_t launch_paged_generic(const PagedParams& p, hipStream_t stream);
 bool sdpa_flash_supported(const SdpaParams& p);
 bool sdpa_flash_mask_supported(const SdpaParams& p);  // p.mask can ride along in the flash kernel
 hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
-// head sizes up to 128 that are multiples of 8 on the matrix cores (flash_small.hip)
+// head sizes up to 256 that are multiples of 8 on the matrix cores (flash_small.hip)
 bool sdpa_flash_small_supported(const SdpaParams& p);
 hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream, const KernelProbe& probe);
 // paged attention of such shapes, 16-bit caches: every sequence of the batch as query tiles over the

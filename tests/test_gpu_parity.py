@@ -111,20 +111,20 @@ def test_sdpa_small_shapes(hip, oracle, shape, causal, dtype):
     case = W.make_sdpa_case(61, B, Hq, Hkv, Lq, Lk, D, dtype)
     out, path = H.run_sdpa(hip, case, causal)
     ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
-    # 16-bit operands with head sizes up to 128 run on the matrix cores (head size 64 in a kernel built
-    # for it, the others zero-padded to 64 or 128); fp32 and larger heads take the fp32 kernel
-    assert path == ("sdpa_generic" if (dtype == W.F32 or D > 128) else ("sdpa_flash_mfma_d64" if D == 64 else "sdpa_flash_mfma_small"))
+    # 16-bit operands with head sizes up to 256 run on the matrix cores (zero-padded to the 64, 128 or
+    # 256 the kernel is built for); fp32 takes the fp32 kernel
+    assert path == ("sdpa_generic" if dtype == W.F32 else ("sdpa_flash_mfma_d64" if D == 64 else "sdpa_flash_mfma_small"))
     assert H.max_abs(out, ref) <= TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [W.F16, W.BF16])
-@pytest.mark.parametrize("D", [8, 32, 40, 80, 96, 112, 120])
+@pytest.mark.parametrize("D", [8, 32, 40, 80, 96, 112, 120, 136, 192, 256])
 @pytest.mark.parametrize("B,Hq,Hkv,Lq,Lk,causal,masked", [(1, 4, 2, 130, 130, True, False), (2, 3, 1, 77, 300, False, False),
                                                           (1, 2, 2, 300, 515, False, True), (1, 6, 2, 1, 1000, False, True),
                                                           (2, 2, 1, 257, 64, True, False)])
 def test_sdpa_other_head_sizes_on_the_matrix_cores(hip, oracle, dtype, D, B, Hq, Hkv, Lq, Lk, causal, masked):
-    """Head sizes that are multiples of 8, up to 128: the head-64 / head-128 builds of the plain
-    matrix-core kernel with the missing columns as zeros, with and without an fp32 attention mask."""
+    """Head sizes that are multiples of 8, up to 256: the head-64 / head-128 / head-256 builds of the
+    plain matrix-core kernel with the missing columns as zeros, with and without an fp32 attention mask."""
     announce("sdpa other head sizes", dtype, D, B, Hq, Hkv, Lq, Lk, causal, masked)
     case = W.make_sdpa_case(64, B, Hq, Hkv, Lq, Lk, D, dtype, std=0.5 if dtype == W.BF16 else 1.0)
     if masked:
@@ -920,10 +920,10 @@ def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle):
     dev.free()
 
 
-@pytest.mark.parametrize("shape", [(6, 2, 96, 16, W.F32, W.F32), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 256, 32, W.BF16, W.BF16),
-                                   (4, 1, 128, 16, W.F16, W.U8), (4, 2, 64, 64, W.F16, W.U8)])
+@pytest.mark.parametrize("shape", [(6, 2, 96, 16, W.F32, W.F32), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 320, 32, W.BF16, W.BF16),
+                                   (4, 1, 128, 16, W.F16, W.U8), (4, 2, 64, 64, W.F16, W.U8), (4, 2, 100, 16, W.F16, W.F16)])
 def test_paged_generic_shapes(hip, oracle, shape):
-    """fp32, head sizes above 128 and u8 caches off the tuned shape: the fp32 kernel."""
+    """fp32, head sizes above 256 or not multiples of 8, u8 caches off the tuned shape: the fp32 kernel."""
     announce("paged generic", shape)
     Hq, Hkv, D, bs, qd, cd = shape
     seqs = [(0, 9), (37, 1), (31, 2), (5, 40), (64, 1), (200, 1)]
@@ -940,13 +940,14 @@ def test_paged_generic_shapes(hip, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(6, 2, 96, 16), (34, 2, 128, 32), (8, 8, 80, 8), (4, 1, 32, 64), (12, 4, 128, 8),
-                                   (3, 3, 8, 4), (16, 2, 112, 128), (40, 1, 64, 32), (128, 1, 48, 16)])
+                                   (3, 3, 8, 4), (16, 2, 112, 128), (40, 1, 64, 32), (128, 1, 48, 16), (8, 2, 256, 32),
+                                   (4, 4, 192, 16), (6, 1, 136, 8)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,out_dtype", [(W.F16, W.F16, None), (W.BF16, W.BF16, None), (W.BF16, W.F16, W.F32),
                                                            (W.F16, W.BF16, W.BF16)])
 @pytest.mark.parametrize("window", [0, 50])
 def test_paged_other_shapes_on_the_matrix_cores(hip, oracle, shape, q_dtype, cache_dtype, out_dtype, window):
     """16-bit caches whose shape the tuned kernels do not take (head sizes that are multiples of 8 up
-    to 128, any power-of-two block size, more than 16 query heads per kv head): every sequence goes
+    to 256, any power-of-two block size, more than 16 query heads per kv head): every sequence goes
     through the query-tile kernel over the block table, a single-token sequence as one tile per kv
     head whose rows are the heads of the group."""
     announce("paged tiles", shape, q_dtype, cache_dtype, out_dtype, window)
