@@ -567,13 +567,48 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
     return out
 
 
+def bench_other_shapes(hip, steps, warmup):
+    """config 3's and config 5's batches at the other cache shapes of the matrix-core decode kernel and, at
+    head size 96, through the query-tile kernel that takes every other 16-bit shape; config 2's shape at
+    head size 96.  Not reference configurations; no byte counters recorded for them."""
+    from openvino_contrib_amd import workloads as W
+
+    results = {}
+    for D, bs in ((64, 32), (64, 16), (128, 16), (96, 16)):
+        key = "c3_d%d_blk%d" % (D, bs)
+        case = W.config3(head_dim=D, block_size=bs)
+        r = bench_paged(hip, case, steps, warmup, "config3's batch with head size %d and cache blocks of %d tokens" % (D, bs))
+        r["roofline"] = roofline_hbm(r, key)
+        if r["kernel_path"] == "paged_mfma_tiles":
+            r["roofline"]["kernel"] = "paged_tiles_kernel"
+        log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f (%s)"
+            % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))
+        results[key] = r
+        del case
+    for key, kw, what in (("c5_blk16", {"block_size": 16}, "on cache blocks of 16 tokens"),
+                          ("c5_d64_blk16", {"block_size": 16, "head_dim": 64}, "with head size 64 on cache blocks of 16 tokens"),
+                          ("c5_d96_blk16", {"block_size": 16, "head_dim": 96}, "with head size 96 on cache blocks of 16 tokens")):
+        case = W.config5(**kw)
+        r = bench_paged(hip, case, steps, warmup, "config5's batch " + what)
+        log("%s: %.3f ms/step (%s)" % (key, r["ms_per_step"], r["kernel_path"]))
+        results[key] = r
+        del case
+    case = W.config2(D=96)
+    r = bench_sdpa(hip, case, steps, warmup, "config2's shape at head size 96 (the plain matrix-core kernel, columns padded to 128)")
+    r["roofline"] = roofline_mfma(r)
+    r["roofline"]["traffic"], r["roofline"]["traffic_source"], r["roofline"]["kernel"] = None, None, "sdpa_flash_small_kernel"
+    log("c2_d96: %.3f ms/step, roofline frac %.3f (%s)" % (r["ms_per_step"], r["roofline"]["frac"], r["kernel_path"]))
+    results["c2_d96"] = r
+    return results
+
+
 def main():
     global CLOCK_RAMP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "copy", "mfma"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "copy", "mfma"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
                          "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
@@ -619,6 +654,11 @@ def main():
     if args.workload == "layer":
         print(json.dumps({"workload": "layer", "steps": args.steps, "warmup": args.warmup,
                           "workloads": bench_layer_ops(hip, args.steps, args.warmup, not args.no_cpu)}))
+        return
+
+    if args.workload == "shapes":
+        print(json.dumps({"workload": "shapes", "steps": args.steps, "warmup": args.warmup,
+                          "workloads": bench_other_shapes(hip, args.steps, args.warmup)}))
         return
 
     if args.workload == "copy":
@@ -690,35 +730,7 @@ def main():
         del case
 
     if not args.no_extra:
-        # config3's batch at the other cache shapes of the matrix-core decode kernel and, at head size
-        # 96, through the query-tile kernel that takes every other 16-bit shape (not reference
-        # configurations; no byte counters recorded for them)
-        for D, bs in ((64, 32), (64, 16), (128, 16), (96, 16)):
-            key = "c3_d%d_blk%d" % (D, bs)
-            case = W.config3(head_dim=D, block_size=bs)
-            r = bench_paged(hip, case, args.steps, args.warmup,
-                            "config3's batch with head size %d and cache blocks of %d tokens" % (D, bs))
-            r["roofline"] = roofline_hbm(r, key)
-            if r["kernel_path"] == "paged_mfma_tiles":
-                r["roofline"]["kernel"] = "paged_tiles_kernel"
-            log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f (%s)"
-                % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))
-            results[key] = r
-            del case
-        for key, kw, what in (("c5_blk16", {"block_size": 16}, "on cache blocks of 16 tokens"),
-                              ("c5_d64_blk16", {"block_size": 16, "head_dim": 64}, "with head size 64 on cache blocks of 16 tokens")):
-            case = W.config5(**kw)
-            r = bench_paged(hip, case, args.steps, args.warmup, "config5's batch " + what)
-            log("%s: %.3f ms/step (%s)" % (key, r["ms_per_step"], r["kernel_path"]))
-            results[key] = r
-            del case
-        case = W.config2(D=96)
-        r = bench_sdpa(hip, case, args.steps, args.warmup, "config2's shape at head size 96 (the plain matrix-core kernel, columns padded to 128)")
-        r["roofline"] = roofline_mfma(r)
-        r["roofline"]["traffic"], r["roofline"]["traffic_source"], r["roofline"]["kernel"] = None, None, "sdpa_flash_small_kernel"
-        log("c2_d96: %.3f ms/step, roofline frac %.3f (%s)" % (r["ms_per_step"], r["roofline"]["frac"], r["kernel_path"]))
-        results["c2_d96"] = r
-        del case
+        results.update(bench_other_shapes(hip, args.steps, args.warmup))
         results["c2_masked"] = bench_sdpa_masked(hip, args.steps)
         log("c2's shape with the causality as an attention mask: %.3f ms, %.0f TFLOP/s (%s)"
             % (results["c2_masked"]["ms_per_step"], results["c2_masked"]["tflops"], results["c2_masked"]["kernel_path"]))
