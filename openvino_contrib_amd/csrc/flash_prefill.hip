@@ -1234,7 +1234,7 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
 }
 
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
-    if (p.head_dim == 64) return launch_paged_prefill_small(p, stream);
+    if (p.head_dim != flash::kD) return launch_paged_prefill_small(p, stream);  // the plain kernel, padded columns
     const int G = p.num_heads_q / p.num_heads_kv;
     dim3 grid((unsigned)((int64_t)p.max_q_tiles * ((G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q)));
     if (p.cache_dtype == HIPATTN_BF16)

@@ -285,6 +285,32 @@ __device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* con
     }
 }
 
+// The same for a head size below kHD (16-bit caches): rows are `row` bytes apart; koff[i] is this
+// lane's offset of K piece i inside a tile -- a piece past the end of the row is pointed at piece 0
+// of the row, which is valid memory and meets zeros in the query operand -- and the lanes whose V
+// columns do not exist (v_ok false) get zeros.
+template <int kHD, int kBlk>
+__device__ __forceinline__ void load_block_padded(BlockRegs<false>& b, const uint8_t* const (&kb)[2], const uint8_t* const (&vb)[2],
+                                                  int row, const int (&koff)[kHD / 32], int voff, bool v_ok) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint8_t* const kt = kBlk == 32 ? kb[0] + t * 16 * row : kb[t];
+#pragma unroll
+        for (int i = 0; i < kHD / 32; i++) b.k[t][i] = *(const uint4_t*)(kt + koff[i]);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint8_t* const vt = kBlk == 32 ? vb[0] + t * 16 * row : vb[t];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            if (v_ok)
+                b.v[t * 4 + r] = *(const uint4_t*)(vt + voff + r * row);
+            else
+                b.v[t * 4 + r] = (uint4_t){0u, 0u, 0u, 0u};
+        }
+    }
+}
+
 struct WaveState {
     float m;          // running max of the scaled scores (log2 domain), per head (lane & 15)
     float l;          // this lane's share of the running sum
@@ -656,9 +682,12 @@ constexpr int kSelfPlanMaxRows = 256;
 // leave the others free for a kernel that runs beside this one.
 // kHD, kBlk: head size (128 or 64) and cache block size (32 or 16); u8 caches exist for 128 / 32 only,
 // the self-planning form and the eight-wavefront form for head size 128 only.
-template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS>
+// kPad: the call's head size (p.head_dim, a multiple of 8) may be smaller than kHD: the missing columns of
+// Q are zeros and those of V are not read.
+template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
+    static_assert(!kPad || (!kU8 && !kSelfPlan && kWaves == 1), "padded head sizes: 16-bit caches, the ordinary launch");
     static_assert((kHD == 128 && kBlk == 32) || !kU8, "u8 caches: head size 128 and blocks of 32 only");
     static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
     static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32), "head size 64 or 128, blocks of 16 or 32");
@@ -717,8 +746,23 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     if (w >= num_waves) return;
     const Line line(total, num_waves, p.dyn_pieces);
 
-    constexpr int64_t kRowBytes = kU8 ? (kHD + 8) : (2 * kHD);
+    constexpr int64_t kRowBytesBuilt = kU8 ? (kHD + 8) : (2 * kHD);
+    const int head_dim = kPad ? p.head_dim : kHD;                       // (a constant unless kPad)
+    const int64_t kRowBytes = kPad ? 2 * p.head_dim : kRowBytesBuilt;
     const int64_t block_stride = (int64_t)Hkv * kBlk * kRowBytes;
+    // kPad: this lane's K piece offsets, V offset and whether its V columns exist
+    int koff[kHD / 32];
+    int voff = 0;
+    bool v_ok = true;
+    if constexpr (kPad) {
+#pragma unroll
+        for (int i = 0; i < kHD / 32; i++) {
+            const int first = kg * (kHD / 4) + i * 8;  // first of the piece's eight columns
+            koff[i] = n16 * (int)kRowBytes + (first < head_dim ? first * 2 : 0);
+        }
+        voff = kg * 4 * (int)kRowBytes + n16 * 16;
+        v_ok = n16 * 8 < head_dim;
+    }
 
     // The static piece first, then dynamic pieces for as long as there are any.  The ticket for
     // the next dynamic piece is drawn before the current piece is worked on, so its latency is hidden.
@@ -796,10 +840,10 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         typename Op16<kBf16>::vec8 qf[4];
         float sumq = 0.0f;
         {
-            const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kHD;
+            const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * head_dim;
 #pragma unroll
             for (int i = 0; i < kHD / 32; i++) {
-                if (n16 < G) {
+                if (n16 < G && (!kPad || kg * (kHD / 4) + i * 8 < head_dim)) {
                     qf[i] = load_q8<kBf16>(p.q, qrow + kg * (kHD / 4) + i * 8, p.q_dtype);
                 } else {
 #pragma unroll
@@ -837,7 +881,10 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     const int64_t off = (int64_t)pb * block_stride + head_off;
                     const uint8_t* const kb[2] = {p.key_cache + off, p.key_cache + off + 16 * kRowBytes};
                     const uint8_t* const vb[2] = {p.value_cache + off, p.value_cache + off + 16 * kRowBytes};
-                    load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
+                    if constexpr (kPad)
+                        load_block_padded<kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok);
+                    else
+                        load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
                     return 3;
                 } else {
                     const int pb0 = __builtin_amdgcn_readlane(my_pb, 2 * i), pb1 = __builtin_amdgcn_readlane(my_pb, 2 * i + 1);
@@ -848,7 +895,10 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     const int64_t off1 = (int64_t)((ok & 2) ? pb1 : pb0) * block_stride + head_off;
                     const uint8_t* const kb[2] = {p.key_cache + off0, p.key_cache + off1};
                     const uint8_t* const vb[2] = {p.value_cache + off0, p.value_cache + off1};
-                    load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
+                    if constexpr (kPad)
+                        load_block_padded<kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok);
+                    else
+                        load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
                     return ok;
                 }
             };
@@ -910,11 +960,11 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     o[e] = v * inv;
                 }
                 const int d0 = (kg * 4 + r) * 8;
-                if (kHD < 128 && d0 >= kHD) continue;  // (rows of the accumulator beyond the head size hold nothing)
+                if ((kPad || kHD < 128) && d0 >= head_dim) continue;  // (rows of the accumulator beyond the head size hold nothing)
                 if (whole) {
-                    store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * kHD + d0, p.out_dtype, o);
+                    store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * head_dim + d0, p.out_dtype, o);
                 } else {
-                    float* po = p.part_out + (slot * G + n16) * kHD + d0;
+                    float* po = p.part_out + (slot * G + n16) * head_dim + d0;
                     *(float4*)(po) = make_float4(o[0], o[1], o[2], o[3]);
                     *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
                 }
@@ -1001,15 +1051,16 @@ bool set_option(const char* name, int value) {
 
 // ---- host side of the fast path ---------------------------------------------------------
 
-// The tuned shape -- head size 128, blocks of 32 -- with every cache type; head size 64 and blocks of
-// 16 with 16-bit caches.
+// The tuned shape -- head size 128, blocks of 32 -- with every cache type; with 16-bit caches also
+// blocks of 16 and every head size up to 128 that is a multiple of 8.
 static bool tuned_shape(const PagedParams& p) { return p.head_dim == kD && p.block_size == kBS; }
 
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
     if (tuned_shape(p)) return p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8;
-    return (p.head_dim == 64 || p.head_dim == 128) && (p.block_size == 16 || p.block_size == 32) &&
+    // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
+    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && (p.block_size == 16 || p.block_size == 32) &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16);
 }
 
@@ -1049,7 +1100,7 @@ static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p
 
 static bool overlap_wanted(const PagedParams& p) {
     if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
-    if (p.head_dim != kD) return false;  // head size 64 has no eight-wavefront decode kernel
+    if (p.head_dim != kD) return false;  // other head sizes have no eight-wavefront decode kernel
     return option(kOptMixedOverlap) != 0;
 }
 
@@ -1219,34 +1270,42 @@ void release_side_stream(hipStream_t owner) {
 }
 
 // The decode kernel for p's cache type, head size and block size (a combination paged_fast_supported
-// admits; head size 64 has the ordinary form only).
+// admits; head sizes other than 128 have the ordinary form only).
+template <bool kBf16, int kWaves, bool kSelfPlan, int kHD, bool kPad>
+static void launch_decode_blk(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block, hipStream_t stream) {
+    if (p.block_size == 32)
+        hipLaunchKernelGGL((paged_decode_kernel<false, kBf16, kWaves, kSelfPlan, kHD, 32, kPad>), grid, block, 0, stream, p, wp, do_write);
+    else
+        hipLaunchKernelGGL((paged_decode_kernel<false, kBf16, kWaves, kSelfPlan, kHD, 16, kPad>), grid, block, 0, stream, p, wp, do_write);
+}
+
 template <int kWaves, bool kSelfPlan>
 static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block,
                           hipStream_t stream) {
     const bool bf16 = p.cache_dtype == HIPATTN_BF16;
     if (p.cache_dtype == HIPATTN_U8) {
         hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan>), grid, block, 0, stream, p, wp, do_write);
-    } else if (p.head_dim == 128 && p.block_size == 32) {
-        if (bf16)
-            hipLaunchKernelGGL((paged_decode_kernel<false, true, kWaves, kSelfPlan>), grid, block, 0, stream, p, wp, do_write);
-        else
-            hipLaunchKernelGGL((paged_decode_kernel<false, false, kWaves, kSelfPlan>), grid, block, 0, stream, p, wp, do_write);
     } else if (p.head_dim == 128) {
         if (bf16)
-            hipLaunchKernelGGL((paged_decode_kernel<false, true, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
+            launch_decode_blk<true, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
         else
-            hipLaunchKernelGGL((paged_decode_kernel<false, false, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
+            launch_decode_blk<false, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
     } else if constexpr (kWaves == 1 && !kSelfPlan) {
-        if (p.block_size == 32) {
+        if (p.head_dim == 64) {
             if (bf16)
-                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
+                launch_decode_blk<true, 1, false, 64, false>(p, wp, do_write, grid, block, stream);
             else
-                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
+                launch_decode_blk<false, 1, false, 64, false>(p, wp, do_write, grid, block, stream);
+        } else if (p.head_dim > 64) {
+            if (bf16)
+                launch_decode_blk<true, 1, false, 128, true>(p, wp, do_write, grid, block, stream);
+            else
+                launch_decode_blk<false, 1, false, 128, true>(p, wp, do_write, grid, block, stream);
         } else {
             if (bf16)
-                hipLaunchKernelGGL((paged_decode_kernel<false, true, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
+                launch_decode_blk<true, 1, false, 64, true>(p, wp, do_write, grid, block, stream);
             else
-                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
+                launch_decode_blk<false, 1, false, 64, true>(p, wp, do_write, grid, block, stream);
         }
     }
 }
@@ -1257,7 +1316,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     int write_blocks = 0;
     if (write) {
         wp = *write;
-        if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head sizes 64 and 128 only
+        if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head sizes up to 128 only
         write_blocks = (int)((kv_write_wavefronts(wp) + 3) / 4);
     }
     hipError_t e = hipSuccess;

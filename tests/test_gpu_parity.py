@@ -836,14 +836,15 @@ def test_paged_mixed_batches_on_many_short_lived_streams(hip, oracle):
     dev.free()
 
 
-@pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16)])
+@pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16), (96, 16), (80, 32), (40, 16), (120, 32), (8, 32), (72, 16)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,Hq,Hkv", [(W.F16, W.F16, 32, 8), (W.BF16, W.BF16, 8, 8), (W.BF16, W.F16, 24, 2),
                                                         (W.F16, W.BF16, 16, 1)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
 def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window):
-    """16-bit caches with head size 64 or blocks of 16 tokens run the matrix-core kernels (decode rows
-    on the stream-K kernel, multi-token sequences on the chunk kernel of their head size); the
-    shape-generic kernels agree."""
+    """16-bit caches on blocks of 16 or 32 tokens with any head size up to 128 that is a multiple of 8
+    run the matrix-core kernels (decode rows on the stream-K kernel -- built for head sizes 64 and
+    128, smaller heads with zero columns -- multi-token sequences on the chunk kernel of their head
+    size); the shape-generic kernels agree."""
     announce("paged head/block shapes", D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window)
     if kind == "decode":
         seqs = [(c - 1, 1) for c in DECODE_CTX]
@@ -939,7 +940,7 @@ def test_paged_generic_shapes(hip, oracle, shape):
     dev.free()
 
 
-@pytest.mark.parametrize("shape", [(6, 2, 96, 16), (34, 2, 128, 32), (8, 8, 80, 8), (4, 1, 32, 64), (12, 4, 128, 8),
+@pytest.mark.parametrize("shape", [(6, 2, 96, 64), (34, 2, 128, 32), (8, 8, 80, 8), (4, 1, 32, 64), (12, 4, 128, 8),
                                    (3, 3, 8, 4), (16, 2, 112, 128), (40, 1, 64, 32), (128, 1, 48, 16), (8, 2, 256, 32),
                                    (4, 4, 192, 16), (6, 1, 136, 8)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,out_dtype", [(W.F16, W.F16, None), (W.BF16, W.BF16, None), (W.BF16, W.F16, W.F32),
@@ -971,10 +972,10 @@ def test_paged_other_shapes_on_the_matrix_cores(hip, oracle, shape, q_dtype, cac
 
 
 def test_paged_pure_decode_of_another_shape(hip, oracle):
-    """A decode batch at head size 96: one tile per (sequence, kv head)."""
+    """A decode batch at head size 96 on blocks of 64: one tile per (sequence, kv head)."""
     announce("paged tiles decode")
     seqs = [(c - 1, 1) for c in DECODE_CTX]
-    case = W.make_paged_case(88, seqs, 24, 8, 96, 16, W.F16, W.F16, W.F16)
+    case = W.make_paged_case(88, seqs, 24, 8, 96, 64, W.F16, W.F16, W.F16)
     ref, okc, ovc = H.oracle_paged(oracle, case)
     dev = H.PagedDeviceCase(hip, case)
     out, path = dev.run()
