@@ -602,13 +602,105 @@ def bench_other_shapes(hip, steps, warmup):
     return results
 
 
+def bench_decoder_layer(hip, steps, warmup):
+    """One decoder layer of LLaMA-3-8B's shape (hidden 4096, 32 query / 8 kv heads of 128, MLP 14336) on
+    configuration 3's decode batch, as ONE compiled model through the plugin layer: RMS -> q/k/v MatMul ->
+    RoPE -> PagedAttentionExtension -> o MatMul -> Add -> RMS -> gate|up MatMul -> GLU -> down MatMul ->
+    Add, thirteen operators per infer() with every tensor device-resident (weights are bound as device
+    inputs) and the recorded graph replayed.  The step has to read the layer's weights (bf16) and the batch's
+    KV cache (fp16) once: that is the HBM roofline it is held against."""
+    from openvino_contrib_amd import plugin_capi as P
+    from openvino_contrib_amd import workloads as W
+    import numpy as np
+
+    hidden, Hq, Hkv, D, ffn, bs = 4096, 32, 8, 128, 14336, 32
+    case = W.config3()
+    T, S = case["T"], case["S"]
+    rng = np.random.default_rng(7)
+    g = P.GraphText("decoder_layer")
+    names, arrays = [], {}
+
+    def dev_param(name, dtype, array):
+        arrays[name] = (hip.DeviceBuffer.from_numpy(np.ascontiguousarray(array)), dtype, list(array.shape))
+        return g.parameter(name, dtype, list(array.shape))
+
+    def weight(name, rows, cols):
+        return dev_param(name, W.BF16, W.to_storage((rng.standard_normal((rows, cols), dtype=np.float32) / np.sqrt(cols)), W.BF16)[0])
+
+    h = dev_param("hidden", W.BF16, W.to_storage(rng.standard_normal((T, hidden), dtype=np.float32), W.BF16)[0])
+    positions = np.concatenate([np.arange(p, p + n) for p, n in zip(case["past_lens"], np.diff(case["subsequence_begins"]))]).astype(np.int32)
+    half = np.arange(0, D, 2, dtype=np.float64) / D
+    ang = np.arange(int(positions.max()) + 1, dtype=np.float64)[:, None] * (10000.0 ** -half)[None, :]
+    cos_p = dev_param("cos", W.F32, np.concatenate([np.cos(ang), np.cos(ang)], 1).astype(np.float32))
+    sin_p = dev_param("sin", W.F32, np.concatenate([np.sin(ang), np.sin(ang)], 1).astype(np.float32))
+    pos_p = dev_param("positions", P.I32, positions)
+    idx = [dev_param(n, P.I32, case[n]) for n in ("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")]
+    scale_p = g.parameter("scale", W.F32, [-1])
+    win_p = g.parameter("sliding_window", P.I32, [-1])
+    alibi_p = g.parameter("alibi_slopes", W.F32, [0])
+    mcl_p = g.parameter("max_context_len", P.I32, [-1])
+    kc = dev_param("key_cache", W.F16, case["key_cache"].view(np.uint16))
+    vc = dev_param("value_cache", W.F16, case["value_cache"].view(np.uint16))
+    gamma = lambda name: g.constant(name, W.to_storage(1.0 + 0.1 * rng.standard_normal(hidden).astype(np.float32), W.BF16)[0], "bf16")
+    mm = lambda name, x, wt: g.add("MatMul", name, [x, wt], transpose_a=False, transpose_b=True)
+    n1 = g.add("RMS", "norm1", [h, gamma("g1")], epsilon=1e-5, output_type="dynamic")
+    q = mm("q", n1, weight("wq", Hq * D, hidden))
+    k = mm("k", n1, weight("wk", Hkv * D, hidden))
+    v = mm("v", n1, weight("wv", Hkv * D, hidden))
+    rope = dict(head_size=D, rotary_ndims=D, gather_position_arg_id=3)
+    qr = g.add("RoPE", "q_rope", [q, cos_p, sin_p, pos_p], head_cnt=Hq, **rope)
+    kr = g.add("RoPE", "k_rope", [k, cos_p, sin_p, pos_p], head_cnt=Hkv, **rope)
+    pa = g.add("PagedAttentionExtension", "attention", [qr, kr, v, kc, vc] + idx + [scale_p, win_p, alibi_p, mcl_p])
+    h1 = g.add("Add", "res1", [mm("o", pa, weight("wo", hidden, Hq * D)), h])
+    n2 = g.add("RMS", "norm2", [h1, gamma("g2")], epsilon=1e-5, output_type="dynamic")
+    gu = mm("gate_up", n2, weight("wgu", 2 * ffn, hidden))
+    act = g.add("GLU", "glu", [gu], axis=-1, split_lengths=ffn, glu_type=0, split_to_glu_idx=0, output_type="dynamic")
+    g.result("out", g.add("Add", "res2", [mm("down", act, weight("wd", hidden, ffn)), h1]))
+
+    plugin = P.Plugin()
+    compiled = plugin.compile_model(g.model())
+    req = compiled.create_infer_request()
+    host = {"scale": (np.zeros((0,), np.float32), W.F32), "sliding_window": (np.array([0], np.int32), P.I32),
+            "alibi_slopes": (np.zeros((0,), np.float32), W.F32),
+            "max_context_len": (np.array([case["max_context_len"]], np.int32), P.I32)}
+    for i, n in enumerate(compiled.input_names()):
+        if n in host:
+            req.set_input(i, *host[n])
+        else:
+            buf, dtype, shape = arrays[n]
+            req.set_device_input(i, buf.ptr, dtype, shape)
+    out = hip.DeviceBuffer(T * hidden * 2)
+    req.set_device_output(0, out.ptr, W.BF16, [T, hidden])
+    for _ in range(max(warmup, 30)):
+        req.infer()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        req.infer()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    graphs, launches = int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")), int(compiled.get_property("HIP_GRAPH_LAUNCHES"))
+    weight_bytes = 2 * (hidden * (Hq + 2 * Hkv) * D + hidden * Hq * D + 3 * hidden * ffn)
+    kv_bytes = W.paged_kv_bytes(case)
+    res = {"workload": "decoder layer (hidden 4096, 32/8 heads of 128, MLP 14336, bf16 weights, fp16 cache) on config3's "
+                       "decode batch through InferRequest::infer, graph replayed",
+           "ms_per_step": ms, "weight_bytes": weight_bytes, "kv_bytes": kv_bytes, "operators": 13,
+           "graphs": graphs, "graph_launches": launches,
+           "roofline": {"bound": "hbm", "achieved": (weight_bytes + kv_bytes) / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                        "unit": "GB/s", "frac": (weight_bytes + kv_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                        "note": "host wall time per synchronous infer() over the bytes one step must read (weights + KV)"}}
+    del req, compiled, plugin
+    for buf, _, _ in arrays.values():
+        buf.free()
+    out.free()
+    return res
+
+
 def main():
     global CLOCK_RAMP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "copy", "mfma"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "decoder", "copy", "mfma"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
                          "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
@@ -654,6 +746,11 @@ def main():
     if args.workload == "layer":
         print(json.dumps({"workload": "layer", "steps": args.steps, "warmup": args.warmup,
                           "workloads": bench_layer_ops(hip, args.steps, args.warmup, not args.no_cpu)}))
+        return
+
+    if args.workload == "decoder":
+        print(json.dumps({"workload": "decoder", "steps": args.steps, "warmup": args.warmup,
+                          "workloads": {"decoder_layer": bench_decoder_layer(hip, args.steps, args.warmup)}}))
         return
 
     if args.workload == "shapes":
@@ -731,6 +828,11 @@ def main():
 
     if not args.no_extra:
         results.update(bench_other_shapes(hip, args.steps, args.warmup))
+        if not args.no_plugin:
+            results["decoder_layer"] = bench_decoder_layer(hip, args.steps, args.warmup)
+            log("decoder layer on c3's batch through the plugin: %.3f ms/step, roofline frac %.3f (%d graph, %d launches)"
+                % (results["decoder_layer"]["ms_per_step"], results["decoder_layer"]["roofline"]["frac"],
+                   results["decoder_layer"]["graphs"], results["decoder_layer"]["graph_launches"]))
         results["c2_masked"] = bench_sdpa_masked(hip, args.steps)
         log("c2's shape with the causality as an attention mask: %.3f ms, %.0f TFLOP/s (%s)"
             % (results["c2_masked"]["ms_per_step"], results["c2_masked"]["tflops"], results["c2_masked"]["kernel_path"]))
