@@ -220,11 +220,16 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 
     // tile staging: 64 * kChunks 16-byte pieces per K tile and per V tile, kPieces of each per thread
     constexpr int kPieces = kTileK * kChunks / (64 * kWaves);
-    uint4_t stage[2 * kPieces];
+    // The head-64 build keeps two tiles in flight in registers (kDeep): the loads of tile j + 2 are
+    // issued a whole iteration before they are written to LDS; the larger builds have the registers
+    // for one.
+    constexpr bool kDeep = kDP == 64;
+    typedef uint4_t Stage[2 * kPieces];
+    Stage stage_a, stage_b;
     // paged: the block ids of a tile's rows are looked up one tile ahead of its K/V loads, so that
     // those loads do not wait for the table
     int block_of[kPieces];
-    auto lookup = [&](int tile) {
+    auto lookup = [&](int tile) __attribute__((always_inline)) {
         if constexpr (kPaged) {
 #pragma unroll
             for (int s = 0; s < kPieces; s++) {
@@ -234,7 +239,7 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
             }
         }
     };
-    auto fetch = [&](int tile) {  // (paged: after lookup(tile))
+    auto fetch = [&](Stage& stage, int tile) __attribute__((always_inline)) {  // (paged: after lookup(tile))
 #pragma unroll
         for (int s = 0; s < kPieces; s++) {
             const int piece = tid + 64 * kWaves * s, r = piece / kChunks, c = piece % kChunks;
@@ -254,7 +259,7 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
             }
         }
     };
-    auto deposit = [&](int buf) {
+    auto deposit = [&](const Stage& stage, int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int s = 0; s < kPieces; s++) {
             const int piece = tid + 64 * kWaves * s, r = piece / kChunks, c = piece % kChunks;
@@ -272,16 +277,31 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 
     if (tile0 < tiles) {
         lookup(tile0);
-        fetch(tile0);
+        fetch(stage_a, tile0);
         if (tile0 + 1 < tiles) lookup(tile0 + 1);
-        deposit(0);
+        deposit(stage_a, 0);
+        if constexpr (kDeep) {
+            if (tile0 + 1 < tiles) {
+                fetch(stage_a, tile0 + 1);
+                if (tile0 + 2 < tiles) lookup(tile0 + 2);
+            }
+        }
     }
     __syncthreads();
-    for (int j = tile0; j < tiles; j++) {
+    // One key tile.  kDeep: `next` holds tile j + 1, on its way since the previous iteration, and
+    // `ahead` takes the loads of tile j + 2; otherwise `next` takes the loads of tile j + 1 now.
+    auto iteration = [&](int j, Stage& next, Stage& ahead) __attribute__((always_inline)) {
         const int buf = (j - tile0) & 1;
-        if (j + 1 < tiles) {
-            fetch(j + 1);  // in flight while this tile is computed
-            if (j + 2 < tiles) lookup(j + 2);
+        if constexpr (kDeep) {
+            if (j + 2 < tiles) {
+                fetch(ahead, j + 2);
+                if (j + 3 < tiles) lookup(j + 3);
+            }
+        } else {
+            if (j + 1 < tiles) {
+                fetch(next, j + 1);  // in flight while this tile is computed
+                if (j + 2 < tiles) lookup(j + 2);
+            }
         }
         const lds_byte* k_lds = (const lds_byte*)lds[buf][0];
         const lds_byte* v_lds = (const lds_byte*)lds[buf][1];
@@ -393,8 +413,12 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 #pragma unroll
             for (int dt = 0; dt < kDP / 32; dt++) o[dt] = M::mma(read_v_frag<kBf16, kDP>(v_lds, lane, ks, dt), pf[ks], o[dt]);
 
-        if (j + 1 < tiles) deposit(buf ^ 1);  // the other buffer was last read before the previous barrier
+        if (j + 1 < tiles) deposit(next, buf ^ 1);  // the other buffer was last read before the previous barrier
         __syncthreads();
+    };
+    for (int j = tile0; j < tiles; j += 2) {
+        iteration(j, stage_a, stage_b);
+        if (j + 1 < tiles) iteration(j + 1, kDeep ? stage_b : stage_a, kDeep ? stage_a : stage_b);
     }
 
     // normalise and store: register r of o[dt] is head-dim 32 dt + 8 (r / 4) + 4 hi + r % 4 of query row n32
