@@ -44,14 +44,15 @@ def hip_runtime():
 
 
 @pytest.mark.parametrize("batch", ["decode", "mixed"])
-@pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
-def test_paged_attention_replays_from_a_graph(hip, oracle, batch, cache_dtype):
-    print("[case] graph capture", batch, cache_dtype, flush=True)
+@pytest.mark.parametrize("cache_dtype,D,bs", [(W.F16, 128, 32), (W.U8, 128, 32), (W.F16, 64, 16), (W.F16, 96, 32),   # the stream-K kernels
+                                              (W.F16, 96, 64), (W.F16, 256, 16)])                                    # the query-tile kernel
+def test_paged_attention_replays_from_a_graph(hip, oracle, batch, cache_dtype, D, bs):
+    print("[case] graph capture", batch, cache_dtype, D, bs, flush=True)
     if batch == "decode":
         seqs = [(c - 1, 1) for c in (700, 64, 1500, 33, 2049, 5)]
     else:
         seqs = [(0, 130), (37, 1), (500, 1), (100, 257), (999, 1), (64, 1), (700, 128)]
-    case = W.make_paged_case(95, seqs, 16, 4, 128, 32, W.F16, W.F16, cache_dtype, sliding_window=0)
+    case = W.make_paged_case(95, seqs, 16, 4, D, bs, W.F16, W.F16, cache_dtype, sliding_window=0)
     ref, okc, ovc = H.oracle_paged(oracle, case)
     rt = hip_runtime()
     stream = hip.Stream()
