@@ -68,6 +68,23 @@ def test_noalloc_mixed_batch_runs_without_the_side_stream(hip, oracle):
     assert H.max_abs(out, H.storage_to_f32(o_ws, W.BF16)) <= 1e-2
 
 
+@pytest.mark.parametrize("D,bs,path", [(96, 16, "paged_mfma"), (64, 32, "paged_mfma"), (96, 64, "paged_mfma_tiles"), (256, 16, "paged_mfma_tiles")])
+def test_noalloc_on_the_other_shapes(hip, oracle, D, bs, path):
+    """The other 16-bit shapes keep their scratch (partials of the stream-K kernel, the tile numbering of
+    the query-tile kernel) in the static array as well: two calls in a row, the second smaller."""
+    print("noalloc other shapes", D, bs, flush=True)
+    batches = ([(c - 1, 1) for c in (3001, 1500, 700, 2049, 33, 1, 900, 257)] + [(10, 140), (0, 3)], [(299, 1), (5, 20)])
+    for i, seqs in enumerate(batches):
+        case = W.make_paged_case(125 + i, seqs, 16, 4, D, bs, W.F16, W.F16, W.F16, sliding_window=0)
+        (o_ws, k_ws, _, _), (o_na, k_na, _, p_na) = run_both(hip, case)
+        assert p_na == path
+        ref, okc, _ = H.oracle_paged(oracle, case)
+        np.testing.assert_array_equal(k_na, okc)
+        np.testing.assert_array_equal(k_ws, okc)
+        assert H.scaled_bound_error(H.storage_to_f32(o_na, W.F16), ref, "noalloc other shapes") <= 2e-3
+        assert H.max_abs(H.storage_to_f32(o_na, W.F16), H.storage_to_f32(o_ws, W.F16)) <= 2e-3
+
+
 def test_noalloc_refuses_a_batch_beyond_its_scratch(hip):
     print("noalloc too big", flush=True)
     # 16 query heads per kv head and 4,096 sequences need far more partial-result slots than 16 MiB hold
