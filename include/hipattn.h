@@ -195,9 +195,9 @@ hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q,
  * and at most 16 query heads per kv head, and u8 caches with head_dim 128 and block_size 32, take
  * the tuned matrix-core kernels (stream-K decode for single-token rows, chunked prefill over the
  * block table for multi-token sequences; fastest at head_dim 128 and 64); other
- * 16-bit caches with 16-bit queries, a head_dim that is a multiple of 8 up to 256 and a block_size
- * that is a power of two take a plain matrix-core kernel (query tiles over the block table);
- * anything else (fp32, larger heads, other u8 shapes) takes the shape-generic fp32 kernels.
+ * 16-bit and u8 caches with 16-bit queries, a head_dim that is a multiple of 8 up to 256 and a
+ * block_size that is a power of two take a plain matrix-core kernel (query tiles over the block
+ * table); anything else (fp32, larger heads) takes the shape-generic fp32 kernels.
  * A single-token row with nothing to attend (an empty block table) gets an output row of zeros.
  * Block ids outside [0, num_blocks) in a table: the decode and the shape-generic kernels skip
  * those blocks (probability zero); the MFMA chunked-prefill kernel redirects them to a valid

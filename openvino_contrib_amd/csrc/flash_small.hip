@@ -143,6 +143,18 @@ __device__ __forceinline__ void mask_values4(const uint8_t* row, int64_t key_str
     }
 }
 
+// Eight u8 values (words 0, 1) of a cache row with scale and zero-point (words 2, 3) as eight fp16 values.
+__device__ __forceinline__ uint4_t dequantised8(uint4_t piece) {
+    const float scale = __uint_as_float(piece[2]), bias = -__uint_as_float(piece[3]) * scale;
+    uint4_t out;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const uint32_t word = piece[e >> 1] >> (16 * (e & 1));
+        out[e] = Mfma<false>::cvt2(fmaf((float)(word & 0xffu), scale, bias), fmaf((float)((word >> 8) & 0xffu), scale, bias));
+    }
+    return out;
+}
+
 // One query tile of one head: what the workgroup reads, where it writes.
 struct Work {
     const uint16_t* q;      // row 0 of the tile, this head
@@ -177,13 +189,17 @@ __device__ __forceinline__ uint32_t pack2(int dtype, float lo, float hi) {
 // The workgroup's 128 query rows against the keys they attend.
 // kMask: the call carries an attention mask: its values are fetched from global memory ahead of the
 // score product of every tile and added behind it.  kPaged: K and V rows are found through w.table.
-template <bool kBf16, bool kMask, bool kPaged, int kDP>
+// kU8 (paged, fp16 products): the cache rows are [scale f32][zero-point f32][head_dim bytes]; a piece
+// travels as its eight bytes and the row's scale and zero-point and becomes eight fp16 values
+// (byte - zero-point) * scale on its way into LDS.
+template <bool kBf16, bool kMask, bool kPaged, int kDP, bool kU8 = false>
 __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_bytes<kDP>()]) {
+    static_assert(!kU8 || (kPaged && !kBf16), "u8 rows exist in paged caches and are multiplied as fp16");
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     constexpr int kChunks = kDP / 8;             // 16-byte chunks of a row in LDS
     const int chunks = w.head_dim >> 3;          // ... of which the call's rows fill this many
-    const int row_bytes = w.head_dim * 2;
+    const int row_bytes = kU8 ? w.head_dim + 8 : w.head_dim * 2;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int n32 = lane & 31, hi = lane >> 5;
     const int my_row = wave * 32 + n32;          // this lane's query row in the tile (may lie beyond w.rows)
@@ -248,14 +264,21 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
             if constexpr (kPaged) {
                 // a block id outside the cache is redirected into it: the rows that attend it are unspecified
                 const int pb = min(max(block_of[s], 0), w.num_blocks - 1);
-                at = (int64_t)pb * w.block_stride + (int64_t)(key & ((1 << w.block_shift) - 1)) * row_bytes + 16 * c;
+                at = (int64_t)pb * w.block_stride + (int64_t)(key & ((1 << w.block_shift) - 1)) * row_bytes + (kU8 ? 0 : 16 * c);
             } else {
                 at = (int64_t)key * row_bytes + 16 * c;
             }
             stage[s] = stage[kPieces + s] = (uint4_t){0u, 0u, 0u, 0u};
             if (c < chunks) {
-                stage[s] = *(const uint4_t*)(w.k + at);
-                stage[kPieces + s] = *(const uint4_t*)(w.v + at);
+                if constexpr (kU8) {
+                    const uint2_t kraw = *(const uint2_t*)(w.k + at + 8 + 8 * c), ksz = *(const uint2_t*)(w.k + at);
+                    const uint2_t vraw = *(const uint2_t*)(w.v + at + 8 + 8 * c), vsz = *(const uint2_t*)(w.v + at);
+                    stage[s] = (uint4_t){kraw[0], kraw[1], ksz[0], ksz[1]};
+                    stage[kPieces + s] = (uint4_t){vraw[0], vraw[1], vsz[0], vsz[1]};
+                } else {
+                    stage[s] = *(const uint4_t*)(w.k + at);
+                    stage[kPieces + s] = *(const uint4_t*)(w.v + at);
+                }
             }
         }
     };
@@ -263,8 +286,13 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 #pragma unroll
         for (int s = 0; s < kPieces; s++) {
             const int piece = tid + 64 * kWaves * s, r = piece / kChunks, c = piece % kChunks;
-            *(uint4_t*)(lds[buf][0] + k_chunk_offset<kDP>(r, c)) = stage[s];
-            *(uint4_t*)(lds[buf][1] + v_chunk_offset<kDP>(r, c)) = stage[kPieces + s];
+            if constexpr (kU8) {
+                *(uint4_t*)(lds[buf][0] + k_chunk_offset<kDP>(r, c)) = dequantised8(stage[s]);
+                *(uint4_t*)(lds[buf][1] + v_chunk_offset<kDP>(r, c)) = dequantised8(stage[kPieces + s]);
+            } else {
+                *(uint4_t*)(lds[buf][0] + k_chunk_offset<kDP>(r, c)) = stage[s];
+                *(uint4_t*)(lds[buf][1] + v_chunk_offset<kDP>(r, c)) = stage[kPieces + s];
+            }
         }
     };
 
@@ -514,7 +542,7 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_small_masked_kernel(Sd
 // p.tile_prefix (written on the device by the plan of the decode path or by paged_tiles_plan_kernel),
 // the later -- heavier -- tiles of a sequence first.  One workgroup per (tile, head); the grid is
 // an upper bound.
-template <bool kBf16, int kDP>
+template <bool kBf16, int kDP, bool kU8 = false>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))) void paged_tiles_kernel(PagedParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];
     const int item = blockIdx.x / p.num_heads_q, h = blockIdx.x % p.num_heads_q;
@@ -555,18 +583,19 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))
     w.causal = 1;
     w.window = p.sliding_window;
     w.kv_len = min(past + qlen, table_len * p.block_size);
-    const int64_t head_off = (int64_t)hkv * p.block_size * D * 2;
+    const int row_bytes = kU8 ? D + 8 : D * 2;
+    const int64_t head_off = (int64_t)hkv * p.block_size * row_bytes;
     w.k = p.key_cache + head_off;
     w.v = p.value_cache + head_off;
     w.table = p.block_indices + tb0;
     w.block_shift = __builtin_ctz(p.block_size);
     w.num_blocks = p.num_blocks;
-    w.block_stride = (int64_t)p.num_heads_kv * p.block_size * D * 2;
+    w.block_stride = (int64_t)p.num_heads_kv * p.block_size * row_bytes;
     w.scale = p.scale;
     w.mask = nullptr;
     w.mask_row_stride = w.mask_key_stride = 0;
     w.mask_dtype = 0;
-    attend<kBf16, false, true, kDP>(w, lds);
+    attend<kBf16, false, true, kDP, kU8>(w, lds);
 }
 
 // tile_prefix for a batch in which every sequence with tokens goes through paged_tiles_kernel
@@ -650,7 +679,14 @@ hipError_t launch_sdpa_flash_small(const SdpaParams& p, hipStream_t stream, cons
 static void launch_tiles(const PagedParams& p, unsigned groups, hipStream_t stream) {
     const dim3 grid(groups), block(64 * flash_small::kWaves);
     const bool bf16 = p.cache_dtype == HIPATTN_BF16;
-    if (p.head_dim <= 64) {
+    if (p.cache_dtype == HIPATTN_U8) {
+        if (p.head_dim <= 64)
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 64, true>), grid, block, 0, stream, p);
+        else if (p.head_dim <= 128)
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 128, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 256, true>), grid, block, 0, stream, p);
+    } else if (p.head_dim <= 64) {
         if (bf16)
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 64>), grid, block, 0, stream, p);
         else
@@ -677,7 +713,7 @@ hipError_t launch_paged_prefill_small(const PagedParams& p, hipStream_t stream) 
     return hipGetLastError();
 }
 
-// Whole batches through the tile kernel: 16-bit caches and queries whose shape the decode path
+// Whole batches through the tile kernel: 16-bit queries on 16-bit or u8 caches whose shape the decode path
 // does not take -- head sizes that are multiples of 8 up to 256, block sizes that are powers of
 // two, up to 128 query heads per kv head.
 bool paged_tiles_supported(const PagedParams& p) {
@@ -685,7 +721,7 @@ bool paged_tiles_supported(const PagedParams& p) {
     return p.head_dim >= 8 && p.head_dim <= 256 && p.head_dim % 8 == 0 && G <= flash_small::kTileQ &&
            p.block_size > 0 && (p.block_size & (p.block_size - 1)) == 0 &&
            (p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16) &&
-           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16) && aligned16(p.q) && aligned16(p.key_cache) &&
+           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8) && aligned16(p.q) && aligned16(p.key_cache) &&
            aligned16(p.value_cache) && ((uintptr_t)p.out % (p.out_dtype == HIPATTN_F32 ? 16 : 8)) == 0;
 }
 
