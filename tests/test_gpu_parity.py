@@ -898,12 +898,39 @@ def test_paged_chunks_at_head_64(hip, oracle, bs, q_dtype, cache_dtype, out_dtyp
     dev.free()
 
 
-def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle):
+@pytest.mark.parametrize("q_dtype,Hq,Hkv", [(W.F16, 32, 8), (W.BF16, 16, 1), (W.F16, 5, 5)])
+@pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
+def test_paged_u8_cache_on_blocks_of_16(hip, oracle, q_dtype, Hq, Hkv, kind, window):
+    """u8 caches at head size 128 on blocks of 16 tokens: the stream-K kernel and the chunk kernel as on
+    blocks of 32; cache bytes bit-exact."""
+    announce("paged u8 blocks of 16", q_dtype, Hq, Hkv, kind, window)
+    if kind == "decode":
+        seqs = [(c - 1, 1) for c in DECODE_CTX]
+    elif kind == "mixed":
+        seqs = [(0, 9), (37, 1), (31, 2), (5, 40), (64, 1), (200, 1), (15, 1), (16, 1), (17, 33), (0, 1), (1000, 3)]
+    else:
+        seqs = [(0, 70), (0, 16), (3, 17), (0, 1)]
+    case = W.make_paged_case(89, seqs, Hq, Hkv, 128, 16, q_dtype, q_dtype, W.U8, sliding_window=window)
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case)
+    for waves in (0, 7, 900):
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if waves else 0)
+        assert path == "paged_mfma"
+        assert np.isfinite(out).all()
+        assert H.scaled_bound_error(out, ref, "paged u8 blocks of 16") <= 1e-2, waves
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    dev.free()
+
+
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
+def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle, cache_dtype):
     """A block id outside the pool contributes nothing, whichever half of a 32-token unit it is (checked
     against the shape-generic kernels, which skip such blocks key by key)."""
-    announce("paged blocks of 16, bad ids")
+    announce("paged blocks of 16, bad ids", cache_dtype)
     seqs = [(99, 1), (47, 1), (16, 1), (300, 1)]
-    case = W.make_paged_case(85, seqs, 16, 4, 128, 16, W.F16, W.F16, W.F16)
+    case = W.make_paged_case(85, seqs, 16, 4, 128, 16, W.F16, W.F16, cache_dtype)
     ids = case["block_indices"]
     begins = case["block_indices_begins"]
     ids[begins[0] + 1] = case["num_blocks"] + 5   # second half of a unit
@@ -917,7 +944,7 @@ def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle):
     for waves in (0, 50):
         out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE)
         assert path == "paged_mfma"
-        assert H.max_abs(out, ref) <= 2e-3
+        assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3)
     dev.free()
 
 
