@@ -263,21 +263,27 @@ __device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* con
                     b.v[t * 4 + r] = (uint4_t){0u, 0u, 0u, 0u};
             }
     } else {
-        constexpr int kRow = kD + 8;
+        constexpr int kRow = kHD + 8;
+        // a lane's K bytes are kHD / 4 consecutive ones of a row, in pieces of eight; its V bytes the
+        // eight of its columns, when the head has them
+        const bool v_cols = kHD == 128 || n16 * 8 < kHD;
         if constexpr (kBlk == 32) {  // both tiles from the block's first row
             const uint8_t* const kbase = kb[0];
             const uint8_t* const vbase = vb[0];
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    b.k[t][i] = *(const uint2_t*)(kbase + (t * 16 + n16) * kRow + 8 + kg * 32 + i * 8);
+                for (int i = 0; i < kHD / 32; i++)
+                    b.k[t][i] = *(const uint2_t*)(kbase + (t * 16 + n16) * kRow + 8 + kg * (kHD / 4) + i * 8);
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int tok = t * 16 + kg * 4 + r;
-                    b.v[t * 4 + r] = *(const uint2_t*)(vbase + tok * kRow + 8 + n16 * 8);
+                    if (v_cols)
+                        b.v[t * 4 + r] = *(const uint2_t*)(vbase + tok * kRow + 8 + n16 * 8);
+                    else
+                        b.v[t * 4 + r] = (uint2_t){0u, 0u};
                 }
             {
                 const int j = n16 & 7, tok = (j >> 2) * 16 + kg * 4 + (j & 3);
@@ -287,13 +293,17 @@ __device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* con
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    b.k[t][i] = *(const uint2_t*)(kb[t] + n16 * kRow + 8 + kg * 32 + i * 8);
+                for (int i = 0; i < kHD / 32; i++)
+                    b.k[t][i] = *(const uint2_t*)(kb[t] + n16 * kRow + 8 + kg * (kHD / 4) + i * 8);
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    b.v[t * 4 + r] = *(const uint2_t*)(vb[t] + (kg * 4 + r) * kRow + 8 + n16 * 8);
+                for (int r = 0; r < 4; r++) {
+                    if (v_cols)
+                        b.v[t * 4 + r] = *(const uint2_t*)(vb[t] + (kg * 4 + r) * kRow + 8 + n16 * 8);
+                    else
+                        b.v[t * 4 + r] = (uint2_t){0u, 0u};
+                }
             {
                 const int j = n16 & 7, row = kg * 4 + (j & 3);
                 b.sz = *(const float2*)((n16 < 8 ? kb[j >> 2] : vb[j >> 2]) + row * kRow);
@@ -697,15 +707,14 @@ constexpr int kSelfPlanMaxRows = 256;
 // kWaves wavefronts to a workgroup.  1 is the ordinary launch.  With 8 a workgroup owns a compute
 // unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
 // leave the others free for a kernel that runs beside this one.
-// kHD, kBlk: head size (128 or 64) and cache block size (32 or 16); u8 caches, the self-planning form
-// and the eight-wavefront form exist for head size 128 only.
+// kHD, kBlk: head size (128 or 64) and cache block size (32 or 16); the self-planning form and the
+// eight-wavefront form exist for head size 128 only.
 // kPad: the call's head size (p.head_dim, a multiple of 8) may be smaller than kHD: the missing columns of
 // Q are zeros and those of V are not read.
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
     static_assert(!kPad || (!kU8 && !kSelfPlan && kWaves == 1), "padded head sizes: 16-bit caches, the ordinary launch");
-    static_assert(kHD == 128 || !kU8, "u8 caches: head size 128 only");
     static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
     static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32), "head size 64 or 128, blocks of 16 or 32");
     constexpr int kEntries = kUnit / kBlk;  // block-table entries per unit
@@ -1068,13 +1077,13 @@ bool set_option(const char* name, int value) {
 
 // ---- host side of the fast path ---------------------------------------------------------
 
-// Head size 128 on blocks of 32 or 16 with every cache type; with 16-bit caches every head size up
-// to 128 that is a multiple of 8.
+// Head sizes 128 and 64 on blocks of 32 or 16 with every cache type; with 16-bit caches every head
+// size up to 128 that is a multiple of 8.
 
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
-    if (p.cache_dtype == HIPATTN_U8) return p.head_dim == kD && (p.block_size == 16 || p.block_size == 32);
+    if (p.cache_dtype == HIPATTN_U8) return (p.head_dim == 128 || p.head_dim == 64) && (p.block_size == 16 || p.block_size == 32);
     // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
     return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && (p.block_size == 16 || p.block_size == 32) &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16);
@@ -1300,10 +1309,17 @@ static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_
                           hipStream_t stream) {
     const bool bf16 = p.cache_dtype == HIPATTN_BF16;
     if (p.cache_dtype == HIPATTN_U8) {
-        if (p.block_size == 32)
-            hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 32>), grid, block, 0, stream, p, wp, do_write);
-        else
-            hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
+        if (p.head_dim == 128) {
+            if (p.block_size == 32)
+                hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 32>), grid, block, 0, stream, p, wp, do_write);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
+        } else if constexpr (kWaves == 1 && !kSelfPlan) {
+            if (p.block_size == 32)
+                hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
+        }
     } else if (p.head_dim == 128) {
         if (bf16)
             launch_decode_blk<true, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);

@@ -898,19 +898,20 @@ def test_paged_chunks_at_head_64(hip, oracle, bs, q_dtype, cache_dtype, out_dtyp
     dev.free()
 
 
+@pytest.mark.parametrize("D,bs", [(128, 16), (64, 16), (64, 32)])
 @pytest.mark.parametrize("q_dtype,Hq,Hkv", [(W.F16, 32, 8), (W.BF16, 16, 1), (W.F16, 5, 5)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
-def test_paged_u8_cache_on_blocks_of_16(hip, oracle, q_dtype, Hq, Hkv, kind, window):
-    """u8 caches at head size 128 on blocks of 16 tokens: the stream-K kernel and the chunk kernel as on
-    blocks of 32; cache bytes bit-exact."""
-    announce("paged u8 blocks of 16", q_dtype, Hq, Hkv, kind, window)
+def test_paged_u8_cache_at_head_64_and_on_blocks_of_16(hip, oracle, D, bs, q_dtype, Hq, Hkv, kind, window):
+    """u8 caches at head size 128 on blocks of 16 tokens and at head size 64: the stream-K kernel and the
+    chunk kernel of the head size; cache bytes bit-exact."""
+    announce("paged u8 head 64 / blocks of 16", D, bs, q_dtype, Hq, Hkv, kind, window)
     if kind == "decode":
         seqs = [(c - 1, 1) for c in DECODE_CTX]
     elif kind == "mixed":
         seqs = [(0, 9), (37, 1), (31, 2), (5, 40), (64, 1), (200, 1), (15, 1), (16, 1), (17, 33), (0, 1), (1000, 3)]
     else:
         seqs = [(0, 70), (0, 16), (3, 17), (0, 1)]
-    case = W.make_paged_case(89, seqs, Hq, Hkv, 128, 16, q_dtype, q_dtype, W.U8, sliding_window=window)
+    case = W.make_paged_case(89, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, W.U8, sliding_window=window)
     ref, okc, ovc = H.oracle_paged(oracle, case)
     dev = H.PagedDeviceCase(hip, case)
     for waves in (0, 7, 900):
