@@ -306,7 +306,12 @@ __device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* con
                 }
             {
                 const int j = n16 & 7, row = kg * 4 + (j & 3);
-                b.sz = *(const float2*)((n16 < 8 ? kb[j >> 2] : vb[j >> 2]) + row * kRow);
+                // One of four tile bases per lane, put together arithmetically: a per-lane index into
+                // (or a select among the elements of) the arrays would move them to scratch memory.
+                const uintptr_t k0 = (uintptr_t)kb[0], k1 = (uintptr_t)kb[1], v0 = (uintptr_t)vb[0], v1 = (uintptr_t)vb[1];
+                const uintptr_t second = (uintptr_t)(j >> 2), value = (uintptr_t)(n16 >> 3);
+                const uintptr_t in_k = k0 + second * (k1 - k0), in_v = v0 + second * (v1 - v0);
+                b.sz = *(const float2*)(in_k + value * (in_v - in_k) + (uintptr_t)(row * kRow));
             }
         }
     }
@@ -1133,7 +1138,10 @@ static int choose_num_waves(const PagedParams& p, bool overlap) {
     if (p.num_waves > 0) return p.num_waves;
     const int resident = resident_decode_waves();
     if (overlap) return resident;  // the most the plan may choose
-    return p.cache_dtype == HIPATTN_U8 ? resident / 4 * 3 : resident / 2;
+    // (u8 at head size 64 has the most arithmetic per byte of all: every resident wavefront, 0.59 against
+    // 0.48 of HBM peak with six per compute unit on the 128-sequence u8 batch)
+    if (p.cache_dtype == HIPATTN_U8) return p.head_dim == 64 ? resident : resident / 4 * 3;
+    return resident / 2;
 }
 
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

@@ -213,12 +213,12 @@ def config3(seed=1003, S=64, lo=512, hi=8192, head_dim=128, block_size=32):
     return make_paged_case(seed + 100000, seqs, 32, 8, head_dim, block_size, F16, F16, F16)
 
 
-def config4(seed=1004, S=128, lo=1024, hi=16384):
+def config4(seed=1004, S=128, lo=1024, hi=16384, head_dim=128, block_size=32):
     """u8-KV paged decode, per-token per-head asymmetric scale / zero-point, Hq=64."""
     rng = np.random.Generator(np.random.PCG64(seed))
     ctx = rng.integers(lo, hi + 1, size=S)
     seqs = [(int(c) - 1, 1) for c in ctx]
-    return make_paged_case(seed + 100000, seqs, 64, 8, 128, 32, F16, F16, U8)
+    return make_paged_case(seed + 100000, seqs, 64, 8, head_dim, block_size, F16, F16, U8)
 
 
 def config5(seed=1005, n_prefill=8, chunk=512, past_hi=4096, n_decode=120, dec_lo=256, dec_hi=8192, window=4096,
