@@ -1,10 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer] [--no-cpu] [--no-extra] [--no-plugin]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer|shapes|decoder] [--no-cpu] [--no-extra] [--no-plugin]
 
-Prints ONE JSON line.  The headline is the fp16 paged-attention decode step (configuration 3
-of BASELINE.json): a "step" is one hipattn_paged_attention call on the whole synthetic batch
+Prints ONE JSON line.  The headline is the fp16 paged-attention decode step (configuration 3, the
+one the headline metric is quoted on): a "step" is one hipattn_paged_attention call on the whole synthetic batch
 (KV-cache write of the new tokens + split-context decode + merge), inputs resident in HBM.
 `value` is algorithmic KV bytes / wall time of a step; `roofline` is the same byte count over
 the average duration of the dominant kernel (the split-context decode kernel), measured with
