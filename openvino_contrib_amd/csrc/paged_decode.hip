@@ -317,28 +317,40 @@ __device__ __forceinline__ void load_block(BlockRegs<kU8>& b, const uint8_t* con
     }
 }
 
-// The same for a head size below kHD (16-bit caches): rows are `row` bytes apart; koff[i] is this
-// lane's offset of K piece i inside a tile -- a piece past the end of the row is pointed at piece 0
-// of the row, which is valid memory and meets zeros in the query operand -- and the lanes whose V
-// columns do not exist (v_ok false) get zeros.
-template <int kHD, int kBlk>
-__device__ __forceinline__ void load_block_padded(BlockRegs<false>& b, const uint8_t* const (&kb)[2], const uint8_t* const (&vb)[2],
-                                                  int row, const int (&koff)[kHD / 32], int voff, bool v_ok) {
+// The same for a head size below kHD: rows are `row` bytes apart; koff[i] is this lane's offset of K
+// piece i inside a tile -- a piece past the end of the row is pointed at the row's first piece, which
+// is valid memory and meets zeros in the query operand -- and the lanes whose V columns do not exist
+// (v_ok false) get zeros.  voff: the lane's offset of its first V row's piece.  u8 rows: the payload
+// behind eight bytes of scale and zero-point, pieces of eight bytes.
+template <bool kU8, int kHD, int kBlk>
+__device__ __forceinline__ void load_block_padded(BlockRegs<kU8>& b, const uint8_t* const (&kb)[2], const uint8_t* const (&vb)[2],
+                                                  int row, const int (&koff)[kHD / 32], int voff, bool v_ok, int n16, int kg) {
+    using Piece = typename std::conditional<kU8, uint2_t, uint4_t>::type;
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const uint8_t* const kt = kBlk == 32 ? kb[0] + t * 16 * row : kb[t];
 #pragma unroll
-        for (int i = 0; i < kHD / 32; i++) b.k[t][i] = *(const uint4_t*)(kt + koff[i]);
+        for (int i = 0; i < kHD / 32; i++) b.k[t][i] = *(const Piece*)(kt + koff[i]);
     }
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const uint8_t* const vt = kBlk == 32 ? vb[0] + t * 16 * row : vb[t];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            if (v_ok)
-                b.v[t * 4 + r] = *(const uint4_t*)(vt + voff + r * row);
-            else
-                b.v[t * 4 + r] = (uint4_t){0u, 0u, 0u, 0u};
+            Piece piece = {};
+            if (v_ok) piece = *(const Piece*)(vt + voff + r * row);
+            b.v[t * 4 + r] = piece;
+        }
+    }
+    if constexpr (kU8) {
+        const int j = n16 & 7, at = (kg * 4 + (j & 3)) * row;
+        if constexpr (kBlk == 32) {
+            b.sz = *(const float2*)((n16 < 8 ? kb[0] : vb[0]) + (j >> 2) * 16 * row + at);
+        } else {  // (one of four tile bases per lane, put together arithmetically: see load_block)
+            const uintptr_t k0 = (uintptr_t)kb[0], k1 = (uintptr_t)kb[1], v0 = (uintptr_t)vb[0], v1 = (uintptr_t)vb[1];
+            const uintptr_t second = (uintptr_t)(j >> 2), value = (uintptr_t)(n16 >> 3);
+            const uintptr_t in_k = k0 + second * (k1 - k0), in_v = v0 + second * (v1 - v0);
+            b.sz = *(const float2*)(in_k + value * (in_v - in_k) + (uintptr_t)at);
         }
     }
 }
@@ -719,7 +731,7 @@ constexpr int kSelfPlanMaxRows = 256;
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
-    static_assert(!kPad || (!kU8 && !kSelfPlan && kWaves == 1), "padded head sizes: 16-bit caches, the ordinary launch");
+    static_assert(!kPad || (!kSelfPlan && kWaves == 1), "padded head sizes: the ordinary launch");
     static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
     static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32), "head size 64 or 128, blocks of 16 or 32");
     constexpr int kEntries = kUnit / kBlk;  // block-table entries per unit
@@ -779,7 +791,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
 
     constexpr int64_t kRowBytesBuilt = kU8 ? (kHD + 8) : (2 * kHD);
     const int head_dim = kPad ? p.head_dim : kHD;                       // (a constant unless kPad)
-    const int64_t kRowBytes = kPad ? 2 * p.head_dim : kRowBytesBuilt;
+    const int64_t kRowBytes = kPad ? (kU8 ? p.head_dim + 8 : 2 * p.head_dim) : kRowBytesBuilt;
     const int64_t block_stride = (int64_t)Hkv * kBlk * kRowBytes;
     // kPad: this lane's K piece offsets, V offset and whether its V columns exist
     int koff[kHD / 32];
@@ -789,9 +801,9 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
         for (int i = 0; i < kHD / 32; i++) {
             const int first = kg * (kHD / 4) + i * 8;  // first of the piece's eight columns
-            koff[i] = n16 * (int)kRowBytes + (first < head_dim ? first * 2 : 0);
+            koff[i] = n16 * (int)kRowBytes + (kU8 ? 8 + (first < head_dim ? first : 0) : (first < head_dim ? first * 2 : 0));
         }
-        voff = kg * 4 * (int)kRowBytes + n16 * 16;
+        voff = kg * 4 * (int)kRowBytes + (kU8 ? 8 + n16 * 8 : n16 * 16);
         v_ok = n16 * 8 < head_dim;
     }
 
@@ -913,7 +925,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     const uint8_t* const kb[2] = {p.key_cache + off, p.key_cache + off + 16 * kRowBytes};
                     const uint8_t* const vb[2] = {p.value_cache + off, p.value_cache + off + 16 * kRowBytes};
                     if constexpr (kPad)
-                        load_block_padded<kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok);
+                        load_block_padded<kU8, kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok, n16, kg);
                     else
                         load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
                     return 3;
@@ -927,7 +939,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     const uint8_t* const kb[2] = {p.key_cache + off0, p.key_cache + off1};
                     const uint8_t* const vb[2] = {p.value_cache + off0, p.value_cache + off1};
                     if constexpr (kPad)
-                        load_block_padded<kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok);
+                        load_block_padded<kU8, kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok, n16, kg);
                     else
                         load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
                     return ok;
@@ -1082,16 +1094,14 @@ bool set_option(const char* name, int value) {
 
 // ---- host side of the fast path ---------------------------------------------------------
 
-// Head sizes 128 and 64 on blocks of 32 or 16 with every cache type; with 16-bit caches every head
-// size up to 128 that is a multiple of 8.
+// Every head size up to 128 that is a multiple of 8, on blocks of 32 or 16, with 16-bit and u8 caches.
 
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
-    if (p.cache_dtype == HIPATTN_U8) return (p.head_dim == 128 || p.head_dim == 64) && (p.block_size == 16 || p.block_size == 32);
     // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
     return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && (p.block_size == 16 || p.block_size == 32) &&
-           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16);
+           (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
 }
 
 // Wavefronts the decode kernel keeps resident: it needs up to 256 registers per lane, i.e. two
@@ -1140,7 +1150,7 @@ static int choose_num_waves(const PagedParams& p, bool overlap) {
     if (overlap) return resident;  // the most the plan may choose
     // (u8 at head size 64 has the most arithmetic per byte of all: every resident wavefront, 0.59 against
     // 0.48 of HBM peak with six per compute unit on the 128-sequence u8 batch)
-    if (p.cache_dtype == HIPATTN_U8) return p.head_dim == 64 ? resident : resident / 4 * 3;
+    if (p.cache_dtype == HIPATTN_U8) return p.head_dim <= 64 ? resident : resident / 4 * 3;
     return resident / 2;
 }
 
@@ -1323,10 +1333,17 @@ static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_
             else
                 hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
         } else if constexpr (kWaves == 1 && !kSelfPlan) {
-            if (p.block_size == 32)
-                hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
-            else
-                hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
+            const bool b32 = p.block_size == 32;
+            if (p.head_dim == 64) {
+                if (b32) hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
+                else hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
+            } else if (p.head_dim > 64) {
+                if (b32) hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 128, 32, true>), grid, block, 0, stream, p, wp, do_write);
+                else hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 128, 16, true>), grid, block, 0, stream, p, wp, do_write);
+            } else {
+                if (b32) hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 32, true>), grid, block, 0, stream, p, wp, do_write);
+                else hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 16, true>), grid, block, 0, stream, p, wp, do_write);
+            }
         }
     } else if (p.head_dim == 128) {
         if (bf16)

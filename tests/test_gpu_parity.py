@@ -898,12 +898,12 @@ def test_paged_chunks_at_head_64(hip, oracle, bs, q_dtype, cache_dtype, out_dtyp
     dev.free()
 
 
-@pytest.mark.parametrize("D,bs", [(128, 16), (64, 16), (64, 32)])
+@pytest.mark.parametrize("D,bs", [(128, 16), (64, 16), (64, 32), (96, 16), (80, 32), (40, 16), (8, 32), (120, 32)])
 @pytest.mark.parametrize("q_dtype,Hq,Hkv", [(W.F16, 32, 8), (W.BF16, 16, 1), (W.F16, 5, 5)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
-def test_paged_u8_cache_at_head_64_and_on_blocks_of_16(hip, oracle, D, bs, q_dtype, Hq, Hkv, kind, window):
-    """u8 caches at head size 128 on blocks of 16 tokens and at head size 64: the stream-K kernel and the
-    chunk kernel of the head size; cache bytes bit-exact."""
+def test_paged_u8_cache_at_other_head_sizes_and_on_blocks_of_16(hip, oracle, D, bs, q_dtype, Hq, Hkv, kind, window):
+    """u8 caches at head size 128 on blocks of 16 tokens and at the other head sizes up to 128: the
+    stream-K kernel and the chunk kernel of the head size; cache bytes bit-exact."""
     announce("paged u8 head 64 / blocks of 16", D, bs, q_dtype, Hq, Hkv, kind, window)
     if kind == "decode":
         seqs = [(c - 1, 1) for c in DECODE_CTX]
