@@ -1,8 +1,9 @@
 // Paged-attention decode for gfx950 (sequences with exactly one new token), scheduled
 // stream-K style over the whole batch.
 //
-// Work decomposition.  The unit of work is one 32-token cache block of one kv head of one
-// sequence ("block-head": 8 KiB of K plus 8 KiB of V in fp16, 2 x 4352 B in u8).  All
+// Work decomposition.  The unit of work is 32 tokens of the cache of one kv head of one sequence
+// -- one cache block of 32 tokens or two of 16 ("block-head": at head size 128, 8 KiB of K plus
+// 8 KiB of V in fp16, 2 x 4352 B in u8).  All
 // block-heads of the batch are laid out on one line, ordered (sequence, kv head, block), and
 // the line is cut into `num_waves` equal pieces; wavefront w owns piece w.  The kernel is
 // launched with exactly as many single-wavefront workgroups as fit on the device at once, so
@@ -35,6 +36,12 @@
 // scale is folded into the score / probability and the zero-point into a rank-one
 // correction (q.(k - zp) s = s (q.k) - s zp sum(q)).
 //
+// Shapes.  The kernel is a template over the head size it is built for (128 or 64: a lane's K
+// piece count and the number of MFMAs per tile follow), the cache block size (32 or 16) and whether
+// the call's head size may be smaller than the built one (any multiple of 8: rows are then
+// head_dim elements apart at run time and the query columns that do not exist are zeros).  The
+// figures and layouts above are those of head size 128.
+//
 // Mixed batches (decode sequences and multi-token chunks in one call).  The chunks go to the flash
 // kernel over the block table, which is bound by the matrix cores; the decode sequences are bound
 // by HBM.  Each of the two kernels needs whole compute units (registers, LDS), so they cannot
@@ -64,7 +71,7 @@
 
 namespace hipattn {
 
-constexpr int kD = 128;   // head size of the tuned configurations (the kernels also take 64: template kHD)
+constexpr int kD = 128;   // head size of the benchmark configurations (the kernels also take 64 and, padded, any multiple of 8 below: templates kHD, kPad)
 constexpr int kBS = 32;   // their cache block size (also 16: template kBlk)
 constexpr int kUnit = 32; // tokens a wavefront works through at a time: one block of 32, or two of 16
 
