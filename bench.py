@@ -574,7 +574,7 @@ def bench_other_shapes(hip, steps, warmup):
     from openvino_contrib_amd import workloads as W
 
     results = {}
-    for D, bs in ((64, 32), (64, 16), (128, 16), (96, 16), (96, 64)):
+    for D, bs in ((64, 32), (64, 16), (128, 16), (96, 16), (96, 64), (256, 16)):
         key = "c3_d%d_blk%d" % (D, bs)
         case = W.config3(head_dim=D, block_size=bs)
         r = bench_paged(hip, case, steps, warmup, "config3's batch with head size %d and cache blocks of %d tokens" % (D, bs))

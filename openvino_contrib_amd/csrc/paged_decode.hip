@@ -621,7 +621,11 @@ __device__ __forceinline__ void plan_block(const PagedParams& p) {
 // plans.  The plan reads lengths only, never the cache, so the two parts do not interact.
 __global__ __launch_bounds__(256) void paged_prologue_kernel(KvWriteParams wp, PagedParams p, int write_blocks) {
     if ((int)blockIdx.x < write_blocks) {
-        kv_cache_write_wave<2>(wp, (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), threadIdx.x & 63);
+        const int64_t wv = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+        if (wp.head_dim <= 128)  // (elements of a row per lane: two up to head size 128, four up to 256)
+            kv_cache_write_wave<2>(wp, wv, threadIdx.x & 63);
+        else
+            kv_cache_write_wave<4>(wp, wv, threadIdx.x & 63);
     } else {
         plan_block(p);
     }
@@ -676,7 +680,8 @@ __device__ __forceinline__ void store_out8(void* out, int64_t elem, int dtype, c
 __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const Line& line, int s, int h, int g,
                                                    int token, int id_first, int id_last, int lane) {
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv, D = p.head_dim;
-    float m_run = -INFINITY, l_run = 0.0f, ox = 0.0f, oy = 0.0f;
+    // lane l owns head-dim 2l, 2l + 1 and, at head size 256, 128 + 2l, 129 + 2l
+    float m_run = -INFINITY, l_run = 0.0f, ox[2] = {0.0f, 0.0f}, oy[2] = {0.0f, 0.0f};
     for (int id0 = id_first; id0 <= id_last; id0 += 64) {
         const int id = id0 + lane;
         const bool have = id <= id_last && line.begin(id) < line.begin(id + 1);  // skip empty pieces
@@ -691,8 +696,11 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
         const float rescale = (m_run == -INFINITY) ? 0.0f : fast_exp2(m_run - m_new);
         const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - m_new);
         l_run = l_run * rescale + wave_sum(f * lw);
-        ox *= rescale;
-        oy *= rescale;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            ox[c] *= rescale;
+            oy[c] *= rescale;
+        }
         m_run = m_new;
         const uint64_t live = __builtin_amdgcn_ballot_w64(have);
         const int n = min(64, id_last - id0 + 1);
@@ -700,22 +708,30 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
             if (!((live >> i) & 1)) continue;
             const float fi = __shfl(f, i, 64);
             const int64_t sl = (int64_t)(id0 + i) + (int64_t)s * Hkv + h;
-            if (2 * lane < D) {
-                const float2 v = *(const float2*)(p.part_out + (sl * G + g) * D + 2 * lane);
-                ox = fmaf(fi, v.x, ox);
-                oy = fmaf(fi, v.y, oy);
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int d = 128 * c + 2 * lane;
+                if (d < D) {
+                    const float2 v = *(const float2*)(p.part_out + (sl * G + g) * D + d);
+                    ox[c] = fmaf(fi, v.x, ox[c]);
+                    oy[c] = fmaf(fi, v.y, oy[c]);
+                }
             }
         }
     }
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-    if (2 * lane >= D) return;
-    const int64_t o = ((int64_t)token * p.num_heads_q + (int64_t)h * G + g) * D + 2 * lane;
-    if (p.out_dtype == HIPATTN_F32) {
-        *(float2*)((float*)p.out + o) = make_float2(ox * inv, oy * inv);
-    } else {
-        const uint32_t lo = p.out_dtype == HIPATTN_F16 ? float_to_f16_bits(ox * inv) : float_to_bf16_bits(ox * inv);
-        const uint32_t hi = p.out_dtype == HIPATTN_F16 ? float_to_f16_bits(oy * inv) : float_to_bf16_bits(oy * inv);
-        *(uint32_t*)((uint16_t*)p.out + o) = lo | (hi << 16);
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int d = 128 * c + 2 * lane;
+        if (d >= D) continue;
+        const int64_t o = ((int64_t)token * p.num_heads_q + (int64_t)h * G + g) * D + d;
+        if (p.out_dtype == HIPATTN_F32) {
+            *(float2*)((float*)p.out + o) = make_float2(ox[c] * inv, oy[c] * inv);
+        } else {
+            const uint32_t lo = p.out_dtype == HIPATTN_F16 ? float_to_f16_bits(ox[c] * inv) : float_to_bf16_bits(ox[c] * inv);
+            const uint32_t hi = p.out_dtype == HIPATTN_F16 ? float_to_f16_bits(oy[c] * inv) : float_to_bf16_bits(oy[c] * inv);
+            *(uint32_t*)((uint16_t*)p.out + o) = lo | (hi << 16);
+        }
     }
 }
 
@@ -1033,6 +1049,280 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     }
 }
 
+// ---- head size 256 (16-bit caches) -------------------------------------------------------------
+// The same schedule, products and lane layouts, with the head dimension worked through in two
+// halves of 128 columns so that the registers hold: a unit of 32 tokens arrives as four
+// half-stages of 32 registers -- K columns 0..127, K columns 128..255, V columns 0..127, V columns
+// 128..255 -- the scores are the sum of the two K halves' products, the probabilities go into two
+// sets of output accumulators, and while one half-stage is consumed the next is in flight.  A
+// wavefront therefore has half as many bytes in flight as the head-128 kernel, and twice as many
+// wavefronts are launched (eight per compute unit).
+struct HalfRegs {
+    uint4_t x[8];  // K: [tile * 4 + piece]; V: [tile * 4 + row]
+};
+
+template <int kBlk>
+__device__ __forceinline__ void load_k_half(HalfRegs& b, const uint8_t* const (&kb)[2], int half, int n16, int kg) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint8_t* const kt = kBlk == 32 ? kb[0] + t * 16 * 512 : kb[t];
+#pragma unroll
+        for (int i = 0; i < 4; i++) b.x[t * 4 + i] = *(const uint4_t*)(kt + n16 * 512 + half * 256 + kg * 64 + i * 16);
+    }
+}
+
+template <int kBlk>
+__device__ __forceinline__ void load_v_half(HalfRegs& b, const uint8_t* const (&vb)[2], int half, int n16, int kg) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint8_t* const vt = kBlk == 32 ? vb[0] + t * 16 * 512 : vb[t];
+#pragma unroll
+        for (int r = 0; r < 4; r++) b.x[t * 4 + r] = *(const uint4_t*)(vt + (kg * 4 + r) * 512 + half * 256 + n16 * 16);
+    }
+}
+
+struct WaveState256 {
+    float m, l;
+    float4_t acc[2][8];  // acc[half][e][r] = O[head][128 * half + (kg*4 + r)*8 + e]
+};
+
+template <bool kBf16>
+__device__ __forceinline__ void scores_half(float4_t (&s)[2], const HalfRegs& k, const typename Op16<kBf16>::vec8 (&q)[4]) {
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) s[t] = Op16<kBf16>::mma(Op16<kBf16>::from_bits(k.x[t * 4 + i]), q[i], s[t]);
+}
+
+// Mask, scale and online softmax of a unit's scores (lane: tokens tok_base + t*16 + kg*4 + r); the
+// accumulators are rescaled when a row's maximum moved.  Returns the probabilities as the B operand.
+template <bool kBf16>
+__device__ __forceinline__ typename Op16<kBf16>::vec8 softmax_unit(WaveState256& st, const float4_t (&s)[2], float c, int tok_base,
+                                                                  int j0, int ctx, int kg, int tiles) {
+    float sv[8];
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int tok = tok_base + t * 16 + kg * 4 + r;
+            const float x = (tok >= j0 && tok < ctx && ((tiles >> t) & 1)) ? s[t][r] * c : -INFINITY;
+            sv[t * 4 + r] = x;
+            mloc = fmaxf(mloc, x);
+        }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    const float m_new = fmaxf(st.m, mloc);
+    // (-inf only while nothing has been attended yet and this unit's blocks both lie outside the cache:
+    // everything stays at zero then; exp2(-inf - -inf) would be NaN)
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+    const float alpha = fast_exp2(st.m - m_use);
+    st.m = m_new;
+    typename Op16<kBf16>::vec8 pf;
+    float lsum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float pj = fast_exp2(sv[j] - m_use);
+        lsum += pj;
+        Op16<kBf16>::set(pf, j, pj);
+    }
+    st.l = st.l * alpha + lsum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) st.acc[h][e] *= alpha;
+    }
+    return pf;
+}
+
+// O^T += V^T P^T for one half of the columns.  Rows outside the attended range may hold anything
+// (never-written cache memory): their probability is exactly zero and they are cleared, so that
+// 0 * NaN cannot occur.
+template <bool kBf16>
+__device__ __forceinline__ void pv_half(float4_t (&acc)[8], HalfRegs& v, typename Op16<kBf16>::vec8 pf, bool partial, int tok_base,
+                                        int j0, int ctx, int kg, int tiles) {
+    if (partial) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int tok = tok_base + (j >> 2) * 16 + kg * 4 + (j & 3);
+            if (!(tok >= j0 && tok < ctx && ((tiles >> (j >> 2)) & 1))) v.x[j] = (uint4_t){0u, 0u, 0u, 0u};
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        uint4_t w;
+#pragma unroll
+        for (int jp = 0; jp < 4; jp++) {
+            const uint32_t lo = v.x[2 * jp][e >> 1], hi = v.x[2 * jp + 1][e >> 1];
+            w[jp] = (e & 1) ? pack_hi(lo, hi) : pack_lo(lo, hi);
+        }
+        acc[e] = Op16<kBf16>::mma(Op16<kBf16>::from_bits(w), pf, acc[e]);
+    }
+}
+
+template <bool kBf16, int kBlk>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode256_kernel(PagedParams p) {
+    constexpr int kHD = 256, kRowBytes = 512;
+    constexpr int kEntries = kUnit / kBlk;
+    const int w = blockIdx.x, lane = threadIdx.x, n16 = lane & 15, kg = lane >> 4;
+    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
+    const float c = p.scale * kLog2e;
+    const int64_t total = (int64_t)p.blk_prefix[p.num_rows] * Hkv;
+    if (total <= 0 || w >= p.num_waves) return;
+    const Line line(total, p.num_waves, 0);
+    const int64_t block_stride = (int64_t)Hkv * kBlk * kRowBytes;
+    int64_t L = line.begin(w);
+    const int64_t L_end = line.begin(w + 1);
+    if (L >= L_end) return;
+    int s = locate_sequence(p.blk_prefix, p.num_rows, (int)(L / Hkv), lane);
+    while (L < L_end) {
+        while (s + 1 < p.num_rows && (int64_t)p.blk_prefix[s + 1] * Hkv <= L) s++;  // next row with units
+        const DecodeRange rg = ((const DecodeRange*)p.seq_info)[s];
+        const int nb = rg.nb;
+        if (nb <= 0) break;  // cannot happen for a consistent plan; never loop forever
+        const int seglen = nb + p.switch_cost;
+        const int64_t seq_L0 = (int64_t)p.blk_prefix[s] * Hkv;
+        const int h = (int)((L - seq_L0) / seglen);
+        const int64_t seg_B0 = seq_L0 + (int64_t)h * seglen + p.switch_cost;
+        const int64_t seg_L1 = seg_B0 + nb;
+        const int64_t from = max(L, seg_B0), to = min(L_end, seg_L1);
+        if (from >= to) {
+            L = to;
+            continue;
+        }
+        const int b_rel = (int)(from - seg_B0);
+        const int n = (int)(to - from);
+        const bool whole = (n == nb);
+        L = from;
+        const int lb0 = rg.j0 / kUnit + b_rel;
+        const int32_t* table = p.block_indices + rg.table_begin + lb0 * kEntries;
+        const int entries = (rg.ctx + kBlk - 1) / kBlk - lb0 * kEntries;
+        const int64_t head_off = (int64_t)h * kBlk * kRowBytes;
+
+        // Q^T operand in two halves: lane (head n16, kg) holds Q[head][128*half + kg*32 + i*8 .. +8]
+        typename Op16<kBf16>::vec8 qf[2][4];
+        {
+            const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kHD;
+#pragma unroll
+            for (int half = 0; half < 2; half++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    if (n16 < G) {
+                        qf[half][i] = load_q8<kBf16>(p.q, qrow + half * 128 + kg * 32 + i * 8, p.q_dtype);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) Op16<kBf16>::set(qf[half][i], e, 0.0f);
+                    }
+                }
+        }
+        WaveState256 st;
+        st.m = -INFINITY;
+        st.l = 0.0f;
+#pragma unroll
+        for (int half = 0; half < 2; half++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) st.acc[half][e] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+        constexpr int kGroup = 64 / kEntries;
+        for (int g0 = 0; g0 < n; g0 += kGroup) {
+            const int gn = min(kGroup, n - g0);
+            const int my_entry = g0 * kEntries + lane;
+            const int my_pb = (lane < gn * kEntries && my_entry < entries) ? table[my_entry] : -1;
+            // Bases of the two tiles of unit i, and which of them lie in a block of the cache.  A block id
+            // outside the cache is replaced by one inside it, so that the loads need no branch; the mask
+            // keeps such a tile out of the scores and clears its V rows.
+            auto unit = [&](int i, const uint8_t* (&kb)[2], const uint8_t* (&vb)[2]) -> int {
+                if constexpr (kEntries == 1) {
+                    const int pb = __builtin_amdgcn_readlane(my_pb, i);
+                    const int ok = (pb >= 0 && pb < p.num_blocks) ? 3 : 0;
+                    const int64_t off = (int64_t)min(max(pb, 0), p.num_blocks - 1) * block_stride + head_off;
+                    kb[0] = p.key_cache + off;
+                    kb[1] = kb[0] + 16 * kRowBytes;
+                    vb[0] = p.value_cache + off;
+                    vb[1] = vb[0] + 16 * kRowBytes;
+                    return ok;
+                } else {
+                    const int pb0 = __builtin_amdgcn_readlane(my_pb, 2 * i), pb1 = __builtin_amdgcn_readlane(my_pb, 2 * i + 1);
+                    const int ok = (pb0 >= 0 && pb0 < p.num_blocks ? 1 : 0) | (pb1 >= 0 && pb1 < p.num_blocks ? 2 : 0);
+                    const int64_t off0 = (int64_t)min(max(pb0, 0), p.num_blocks - 1) * block_stride + head_off;
+                    const int64_t off1 = (int64_t)min(max(pb1, 0), p.num_blocks - 1) * block_stride + head_off;
+                    kb[0] = p.key_cache + off0;
+                    kb[1] = p.key_cache + off1;
+                    vb[0] = p.value_cache + off0;
+                    vb[1] = p.value_cache + off1;
+                    return ok;
+                }
+            };
+            // r0 holds the first K half of unit i when iteration i begins (loaded by the iteration before; the
+            // last iteration loads its own unit's again rather than branching).  No branch in the body: a
+            // unit whose blocks are both outside the cache goes through with every score masked.
+            HalfRegs r0, r1;
+            {
+                const uint8_t *kb[2], *vb[2];
+                (void)unit(0, kb, vb);
+                load_k_half<kBlk>(r0, kb, 0, n16, kg);
+            }
+            for (int i = 0; i < gn; i++) {
+                const int tok_base = (lb0 + g0 + i) * kUnit;
+                const uint8_t *kb[2], *vb[2];
+                const int ok = unit(i, kb, vb);  // (scalar work: the bases are not carried from iteration to iteration)
+                const bool partial = (tok_base < rg.j0) || (tok_base + kUnit > rg.ctx) || ok != 3;  // wavefront-uniform
+                float4_t sc[2] = {(float4_t){0.f, 0.f, 0.f, 0.f}, (float4_t){0.f, 0.f, 0.f, 0.f}};
+                // (the scheduling barriers keep each half-stage's loads behind the use of the registers
+                // they overwrite: hoisted to the top of the iteration they would all be live at once)
+                load_k_half<kBlk>(r1, kb, 1, n16, kg);
+                scores_half<kBf16>(sc, r0, qf[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                load_v_half<kBlk>(r0, vb, 0, n16, kg);
+                scores_half<kBf16>(sc, r1, qf[1]);
+                const typename Op16<kBf16>::vec8 pf = softmax_unit<kBf16>(st, sc, c, tok_base, rg.j0, rg.ctx, kg, ok);
+                __builtin_amdgcn_sched_barrier(0);
+                load_v_half<kBlk>(r1, vb, 1, n16, kg);
+                pv_half<kBf16>(st.acc[0], r0, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
+                __builtin_amdgcn_sched_barrier(0);
+                {
+                    const uint8_t *kbn[2], *vbn[2];
+                    (void)unit(min(i + 1, gn - 1), kbn, vbn);
+                    load_k_half<kBlk>(r0, kbn, 0, n16, kg);
+                }
+                pv_half<kBf16>(st.acc[1], r1, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+
+        // ---- this wavefront's result for the segment
+        float l = st.l;
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        const int64_t slot = (int64_t)w + (int64_t)s * Hkv + h;  // unique per (piece, segment)
+        if (n16 < G) {
+            const float inv = whole ? (l > 0.0f ? 1.0f / l : 0.0f) : 1.0f;
+#pragma unroll
+            for (int half = 0; half < 2; half++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float o[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) o[e] = st.acc[half][e][r] * inv;
+                    const int d0 = half * 128 + (kg * 4 + r) * 8;
+                    if (whole) {
+                        store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * kHD + d0, p.out_dtype, o);
+                    } else {
+                        float* po = p.part_out + (slot * G + n16) * kHD + d0;
+                        *(float4*)(po) = make_float4(o[0], o[1], o[2], o[3]);
+                        *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
+                    }
+                }
+            if (!whole && kg == 0) {
+                p.part_ml[(slot * G + n16) * 2] = st.m;
+                p.part_ml[(slot * G + n16) * 2 + 1] = l;
+            }
+        }
+        L += n;
+    }
+}
+
 // Combines the partials of every (sequence, kv head) segment that more than one piece worked
 // on.  A separate launch: the kernel boundary is what makes the partials visible, which is far
 // cheaper here than device-scope fences inside the streaming kernel (those write back and
@@ -1101,13 +1391,16 @@ bool set_option(const char* name, int value) {
 
 // ---- host side of the fast path ---------------------------------------------------------
 
-// Every head size up to 128 that is a multiple of 8, on blocks of 32 or 16, with 16-bit and u8 caches.
+// Every head size up to 128 that is a multiple of 8 with 16-bit and u8 caches, and head size 256 with 16-bit
+// caches, on blocks of 32 or 16.
 
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
     // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
-    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 && (p.block_size == 16 || p.block_size == 32) &&
+    if (p.block_size != 16 && p.block_size != 32) return false;
+    if (p.head_dim == 256) return p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16;  // (paged_decode256_kernel)
+    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
 }
 
@@ -1158,6 +1451,7 @@ static int choose_num_waves(const PagedParams& p, bool overlap) {
     // (u8 at head size 64 has the most arithmetic per byte of all: every resident wavefront, 0.59 against
     // 0.48 of HBM peak with six per compute unit on the 128-sequence u8 batch)
     if (p.cache_dtype == HIPATTN_U8) return p.head_dim <= 64 ? resident : resident / 4 * 3;
+    if (p.head_dim == 256) return resident;  // half as many bytes in flight per wavefront: twice the wavefronts
     return resident / 2;
 }
 
@@ -1167,8 +1461,8 @@ static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // that starts on a new piece pays a chain of dependent loads (ticket, sequence, block table,
 // first block) before it streams again, and on MI355X that costs more than the better balance
 // at the end of the kernel wins back.  The option decode_dyn_pieces_per_wave switches it on.
-static int choose_dyn_pieces(int num_waves, bool overlap) {
-    if (overlap) return 0;
+static int choose_dyn_pieces(const PagedParams& p, int num_waves, bool overlap) {
+    if (overlap || p.head_dim == 256) return 0;  // (the head-256 kernel has static pieces only)
     return num_waves * option(kOptDynPieces);
 }
 
@@ -1177,7 +1471,7 @@ size_t paged_fast_workspace_bytes(const PagedParams& p) {
     const int W = choose_num_waves(p, overlap);
     const int G = p.num_heads_q / p.num_heads_kv;
     const size_t rows = (size_t)plan_rows(p);
-    const size_t slots = (size_t)W + choose_dyn_pieces(W, overlap) + rows * p.num_heads_kv;
+    const size_t slots = (size_t)W + choose_dyn_pieces(p, W, overlap) + rows * p.num_heads_kv;
     return 512 + 2 * align_up((rows + 1) * sizeof(int32_t), 256) + align_up(rows * 32, 256) +
            align_up(slots * G * p.head_dim * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
 }
@@ -1188,7 +1482,7 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     p.overlap = overlap ? 1 : 0;
     p.num_waves = choose_num_waves(p, overlap);
     p.switch_cost = option(kOptSwitchCost);
-    p.dyn_pieces = choose_dyn_pieces(p.num_waves, overlap);
+    p.dyn_pieces = choose_dyn_pieces(p, p.num_waves, overlap);
     p.overlap_share = option(kOptSharePercent) / 100.0f;
     p.dyn_groups = std::min(64, std::max(1, p.num_waves / 32));  // every group has at least one wavefront
     const int G = p.num_heads_q / p.num_heads_kv;
@@ -1333,7 +1627,15 @@ template <int kWaves, bool kSelfPlan>
 static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block,
                           hipStream_t stream) {
     const bool bf16 = p.cache_dtype == HIPATTN_BF16;
-    if (p.cache_dtype == HIPATTN_U8) {
+    if (p.head_dim == 256) {
+        if constexpr (kWaves == 1 && !kSelfPlan) {
+            const bool b32 = p.block_size == 32;
+            if (bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 32>), grid, block, 0, stream, p);
+            if (bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 16>), grid, block, 0, stream, p);
+            if (!bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 32>), grid, block, 0, stream, p);
+            if (!bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 16>), grid, block, 0, stream, p);
+        }
+    } else if (p.cache_dtype == HIPATTN_U8) {
         if (p.head_dim == 128) {
             if (p.block_size == 32)
                 hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 32>), grid, block, 0, stream, p, wp, do_write);
@@ -1383,7 +1685,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     int write_blocks = 0;
     if (write) {
         wp = *write;
-        if (wp.head_dim > 128) return hipErrorInvalidValue;  // the fast path is head sizes up to 128 only
+        if (wp.head_dim > 256) return hipErrorInvalidValue;  // the fast path is head sizes up to 256 only
         write_blocks = (int)((kv_write_wavefronts(wp) + 3) / 4);
     }
     hipError_t e = hipSuccess;

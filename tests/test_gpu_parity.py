@@ -836,15 +836,16 @@ def test_paged_mixed_batches_on_many_short_lived_streams(hip, oracle):
     dev.free()
 
 
-@pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16), (96, 16), (80, 32), (40, 16), (120, 32), (8, 32), (72, 16)])
+@pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16), (96, 16), (80, 32), (40, 16), (120, 32), (8, 32), (72, 16),
+                                  (256, 32), (256, 16)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,Hq,Hkv", [(W.F16, W.F16, 32, 8), (W.BF16, W.BF16, 8, 8), (W.BF16, W.F16, 24, 2),
                                                         (W.F16, W.BF16, 16, 1)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
 def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window):
-    """16-bit caches on blocks of 16 or 32 tokens with any head size up to 128 that is a multiple of 8
-    run the matrix-core kernels (decode rows on the stream-K kernel -- built for head sizes 64 and
-    128, smaller heads with zero columns -- multi-token sequences on the chunk kernel of their head
-    size); the shape-generic kernels agree."""
+    """16-bit caches on blocks of 16 or 32 tokens with any head size up to 128 that is a multiple of 8,
+    or 256, run the matrix-core kernels (decode rows on the stream-K kernel -- built for head sizes
+    64, 128 and 256, smaller heads with zero columns -- multi-token sequences on the chunk kernel of
+    their head size); the shape-generic kernels agree."""
     announce("paged head/block shapes", D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window)
     if kind == "decode":
         seqs = [(c - 1, 1) for c in DECODE_CTX]
@@ -860,13 +861,15 @@ def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype
         out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if waves else 0)
         assert path == "paged_mfma"
         assert np.isfinite(out).all()
-        assert H.max_abs(out, ref) <= tol, waves
+        # N(0, 1) values and short contexts give outputs beyond 2, where the 16-bit output type alone
+        # rounds by up to 0.008: the bound is relative there (the plain figure is printed)
+        assert H.scaled_bound_error(out, ref, "paged head/block shapes") <= tol, waves
     kc, vc = dev.caches()
     np.testing.assert_array_equal(kc, okc)
     np.testing.assert_array_equal(vc, ovc)
     out_g, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
     assert path_g == "paged_generic"
-    assert H.max_abs(out_g, ref) <= tol
+    assert H.scaled_bound_error(out_g, ref, "paged head/block shapes, generic") <= tol
     dev.free()
 
 
@@ -949,6 +952,33 @@ def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle, cache_dty
     dev.free()
 
 
+@pytest.mark.parametrize("bs", [16, 32])
+def test_paged_head_256_skips_blocks_outside_the_cache(hip, oracle, bs):
+    """Head size 256: the decode kernel reads a block inside the cache in place of one whose id lies
+    outside it and masks its tokens (no branch in its loop); a row whose every block is outside comes
+    out as zeros; checked against the shape-generic kernels, which skip such blocks key by key."""
+    announce("paged head 256, bad ids", bs)
+    seqs = [(99, 1), (47, 1), (16, 1), (300, 1), (20, 1)]
+    case = W.make_paged_case(90, seqs, 8, 4, 256, bs, W.F16, W.F16, W.F16)
+    ids, begins = case["block_indices"], case["block_indices_begins"]
+    per = 32 // bs  # table entries per 32 tokens
+    ids[begins[0] + 1 * per] = case["num_blocks"] + 5      # first block of a unit in the middle
+    ids[begins[0] + 3 * per - 1 + per] = -3 if per == 2 else ids[begins[0] + 3 * per - 1 + per]
+    ids[begins[1] + 1 * per: begins[1] + 2 * per] = case["num_blocks"]  # the last unit, whole
+    ids[begins[3] + 4 * per: begins[3] + 6 * per] = 1 << 30              # two units in a row
+    ids[begins[4]: begins[5]] = -1                                       # every block of the row
+    dev = H.PagedDeviceCase(hip, case)
+    ref, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic" and np.isfinite(ref).all()
+    for waves in (0, 50):
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE)
+        assert path == "paged_mfma"
+        assert np.isfinite(out).all()
+        assert H.max_abs(out, ref) <= 2e-3
+    assert not out[4].any()
+    dev.free()
+
+
 @pytest.mark.parametrize("shape", [(6, 2, 96, 16, W.F32, W.F32), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 320, 32, W.BF16, W.BF16),
                                    (4, 1, 264, 16, W.F16, W.U8), (4, 2, 64, 64, W.F32, W.U8), (4, 2, 100, 16, W.F16, W.F16)])
 def test_paged_generic_shapes(hip, oracle, shape):
@@ -969,7 +999,7 @@ def test_paged_generic_shapes(hip, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(6, 2, 96, 64), (34, 2, 128, 32), (8, 8, 80, 8), (4, 1, 32, 64), (12, 4, 128, 8),
-                                   (3, 3, 8, 4), (16, 2, 112, 128), (40, 1, 64, 32), (128, 1, 48, 16), (8, 2, 256, 32),
+                                   (3, 3, 8, 4), (16, 2, 112, 128), (40, 1, 64, 32), (128, 1, 48, 16), (8, 2, 256, 64),
                                    (4, 4, 192, 16), (6, 1, 136, 8)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,out_dtype", [(W.F16, W.F16, None), (W.BF16, W.BF16, None), (W.BF16, W.F16, W.F32),
                                                            (W.F16, W.BF16, W.BF16), (W.F16, W.U8, None), (W.BF16, W.U8, W.F32)])
