@@ -71,17 +71,62 @@ def test_random_paged_batches(hip, oracle, seed):
     print("worst error / bound: %.2f" % worst)
 
 
+@pytest.mark.parametrize("seed", [31, 32, 33])
+def test_random_paged_batches_of_every_shape(hip, oracle, seed):
+    """The same draws over the shapes the matrix-core paths take besides head size 128 / blocks of 32:
+    head sizes that are multiples of 8 up to 256, block sizes that are powers of two, up to 128 query
+    heads per kv head, 16-bit and u8 caches.  Which kernel takes a call follows from the shape
+    (the stream-K kernels for head sizes up to 128, and 256, on blocks of 16 or 32 with at most 16
+    query heads per kv head; the query-tile kernel for the rest)."""
+    rng = np.random.default_rng(seed)
+    worst = 0.0
+    for it in range(40):
+        kind, _, _, cache, q_dtype, window, seqs = draw_batch(rng)
+        seqs = [(min(past, 800), n) for past, n in seqs][:8]
+        D = 8 * int(rng.integers(1, 33))
+        if rng.random() < 0.3:
+            D = int(rng.choice([64, 96, 128, 256]))
+        bs = int(rng.choice([4, 8, 16, 16, 32, 32, 64, 128]))
+        Hkv = int(rng.choice([1, 2, 3]))
+        G = int(rng.choice([1, 2, 4, 7, 8, 16, 17, 40]))
+        if G * Hkv * D > 8192:
+            G = max(1, 8192 // (Hkv * D))
+        if sum(n for _, n in seqs) == 0:
+            continue
+        if sum(n for _, n in seqs) == len(seqs) and any(n != 1 for _, n in seqs):
+            continue
+        print("[case] random paged shapes", seed, it, kind, "D", D, "bs", bs, "G", G, "Hkv", Hkv, "cache", cache, "q", q_dtype,
+              "window", window, "seqs", seqs, flush=True)
+        case = W.make_paged_case(seed * 100 + it, seqs, G * Hkv, Hkv, D, bs, q_dtype, q_dtype, cache, sliding_window=window)
+        ref, okc, ovc = H.oracle_paged(oracle, case)
+        dev = H.PagedDeviceCase(hip, case)
+        out, path = dev.run()
+        kc, vc = dev.caches()
+        dev.free()
+        stream_k = bs in (16, 32) and G <= 16 and (D <= 128 or (D == 256 and cache != W.U8))
+        assert path == ("paged_mfma" if stream_k else "paged_mfma_tiles")
+        np.testing.assert_array_equal(kc, okc)
+        np.testing.assert_array_equal(vc, ovc)
+        assert np.isfinite(out).all()
+        tol = 2e-2 if cache == W.BF16 else (1e-2 if (cache == W.U8 or q_dtype == W.BF16) else 2e-3)
+        err = H.scaled_bound_error(out, ref, "random paged shapes %d/%d q %d cache %d" % (seed, it, q_dtype, cache))
+        worst = max(worst, err / tol)
+        assert err <= tol, (seed, it)
+    print("worst error / bound: %.2f" % worst)
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_random_sdpa_shapes(hip, oracle, seed):
-    """Dense SDPA: batch, GQA ratio, head size (128 takes the MFMA kernel for 16-bit types, the
-    others and fp32 the shape-generic one), square and rectangular score matrices, causal or not."""
+    """Dense SDPA: batch, GQA ratio, head size (16-bit types take the matrix-core kernels at every
+    multiple of 8 up to 256, fp32 the shape-generic one), square and rectangular score matrices,
+    causal or not."""
     rng = np.random.default_rng(seed)
     worst = {}
     for it in range(24):
         G = int(rng.choice([1, 2, 3, 4, 5, 8]))
         Hkv = int(rng.choice([1, 2, 3]))
         B = int(rng.choice([1, 2, 3]))
-        D = int(rng.choice([128, 128, 128, 64, 32]))
+        D = int(rng.choice([128, 128, 128, 64, 32, 96, 256, 8 * int(rng.integers(1, 33))]))
         dtype = int(rng.choice([W.F16, W.BF16, W.F32]))
         Lq = int(rng.choice([1, 2, 31, 64, 127, 128, 129, 255, 256, 257, 300, 511, 700, int(rng.integers(1, 900))]))
         Lk = Lq if rng.random() < 0.5 else int(rng.choice([1, 63, 64, 65, 200, 513, 1000, int(rng.integers(1, 1200))]))
