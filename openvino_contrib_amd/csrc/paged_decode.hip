@@ -1061,23 +1061,31 @@ struct HalfRegs {
     uint4_t x[8];  // K: [tile * 4 + piece]; V: [tile * 4 + row]
 };
 
+// row: bytes from one cache row to the next (512, or 2 * head_dim for a smaller head).  koff[i]: this
+// lane's offset of K piece i of the half inside a tile (a piece past the end of the row is pointed at
+// the row's first piece: valid memory that meets zeros in the query operand).
 template <int kBlk>
-__device__ __forceinline__ void load_k_half(HalfRegs& b, const uint8_t* const (&kb)[2], int half, int n16, int kg) {
+__device__ __forceinline__ void load_k_half(HalfRegs& b, const uint8_t* const (&kb)[2], int row, const int (&koff)[4]) {
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-        const uint8_t* const kt = kBlk == 32 ? kb[0] + t * 16 * 512 : kb[t];
+        const uint8_t* const kt = kBlk == 32 ? kb[0] + t * 16 * row : kb[t];
 #pragma unroll
-        for (int i = 0; i < 4; i++) b.x[t * 4 + i] = *(const uint4_t*)(kt + n16 * 512 + half * 256 + kg * 64 + i * 16);
+        for (int i = 0; i < 4; i++) b.x[t * 4 + i] = *(const uint4_t*)(kt + koff[i]);
     }
 }
 
+// voff: this lane's offset of its first V row's piece of the half; v_ok: its columns exist.
 template <int kBlk>
-__device__ __forceinline__ void load_v_half(HalfRegs& b, const uint8_t* const (&vb)[2], int half, int n16, int kg) {
+__device__ __forceinline__ void load_v_half(HalfRegs& b, const uint8_t* const (&vb)[2], int row, int voff, bool v_ok) {
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-        const uint8_t* const vt = kBlk == 32 ? vb[0] + t * 16 * 512 : vb[t];
+        const uint8_t* const vt = kBlk == 32 ? vb[0] + t * 16 * row : vb[t];
 #pragma unroll
-        for (int r = 0; r < 4; r++) b.x[t * 4 + r] = *(const uint4_t*)(vt + (kg * 4 + r) * 512 + half * 256 + n16 * 16);
+        for (int r = 0; r < 4; r++) {
+            uint4_t piece = {0u, 0u, 0u, 0u};
+            if (v_ok) piece = *(const uint4_t*)(vt + voff + r * row);
+            b.x[t * 4 + r] = piece;
+        }
     }
 }
 
@@ -1161,11 +1169,26 @@ __device__ __forceinline__ void pv_half(float4_t (&acc)[8], HalfRegs& v, typenam
     }
 }
 
-template <bool kBf16, int kBlk>
+// kPad: the call's head size (p.head_dim, a multiple of 8 above 128) may be smaller than 256.
+template <bool kBf16, int kBlk, bool kPad>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode256_kernel(PagedParams p) {
-    constexpr int kHD = 256, kRowBytes = 512;
     constexpr int kEntries = kUnit / kBlk;
     const int w = blockIdx.x, lane = threadIdx.x, n16 = lane & 15, kg = lane >> 4;
+    const int kHD = kPad ? p.head_dim : 256;  // (a constant unless kPad)
+    const int kRowBytes = 2 * kHD;
+    // this lane's piece offsets inside a tile, per half, and whether its V columns exist
+    int koff[2][4], voff[2];
+    bool v_ok[2];
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int first = half * 128 + kg * 32 + i * 8;  // first of the piece's eight columns
+            koff[half][i] = n16 * kRowBytes + (first < kHD ? first * 2 : 0);
+        }
+        voff[half] = kg * 4 * kRowBytes + half * 256 + n16 * 16;
+        v_ok[half] = half * 128 + n16 * 8 < kHD;
+    }
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
     const float c = p.scale * kLog2e;
     const int64_t total = (int64_t)p.blk_prefix[p.num_rows] * Hkv;
@@ -1208,7 +1231,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             for (int half = 0; half < 2; half++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    if (n16 < G) {
+                    if (n16 < G && half * 128 + kg * 32 + i * 8 < kHD) {
                         qf[half][i] = load_q8<kBf16>(p.q, qrow + half * 128 + kg * 32 + i * 8, p.q_dtype);
                     } else {
 #pragma unroll
@@ -1261,7 +1284,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             {
                 const uint8_t *kb[2], *vb[2];
                 (void)unit(0, kb, vb);
-                load_k_half<kBlk>(r0, kb, 0, n16, kg);
+                load_k_half<kBlk>(r0, kb, kRowBytes, koff[0]);
             }
             for (int i = 0; i < gn; i++) {
                 const int tok_base = (lb0 + g0 + i) * kUnit;
@@ -1271,20 +1294,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 float4_t sc[2] = {(float4_t){0.f, 0.f, 0.f, 0.f}, (float4_t){0.f, 0.f, 0.f, 0.f}};
                 // (the scheduling barriers keep each half-stage's loads behind the use of the registers
                 // they overwrite: hoisted to the top of the iteration they would all be live at once)
-                load_k_half<kBlk>(r1, kb, 1, n16, kg);
+                load_k_half<kBlk>(r1, kb, kRowBytes, koff[1]);
                 scores_half<kBf16>(sc, r0, qf[0]);
                 __builtin_amdgcn_sched_barrier(0);
-                load_v_half<kBlk>(r0, vb, 0, n16, kg);
+                load_v_half<kBlk>(r0, vb, kRowBytes, voff[0], v_ok[0]);
                 scores_half<kBf16>(sc, r1, qf[1]);
                 const typename Op16<kBf16>::vec8 pf = softmax_unit<kBf16>(st, sc, c, tok_base, rg.j0, rg.ctx, kg, ok);
                 __builtin_amdgcn_sched_barrier(0);
-                load_v_half<kBlk>(r1, vb, 1, n16, kg);
+                load_v_half<kBlk>(r1, vb, kRowBytes, voff[1], v_ok[1]);
                 pv_half<kBf16>(st.acc[0], r0, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
                 __builtin_amdgcn_sched_barrier(0);
                 {
                     const uint8_t *kbn[2], *vbn[2];
                     (void)unit(min(i + 1, gn - 1), kbn, vbn);
-                    load_k_half<kBlk>(r0, kbn, 0, n16, kg);
+                    load_k_half<kBlk>(r0, kbn, kRowBytes, koff[0]);
                 }
                 pv_half<kBf16>(st.acc[1], r1, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1306,6 +1329,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
                     for (int e = 0; e < 8; e++) o[e] = st.acc[half][e][r] * inv;
                     const int d0 = half * 128 + (kg * 4 + r) * 8;
+                    if (kPad && d0 >= kHD) continue;  // (columns beyond the head size hold nothing)
                     if (whole) {
                         store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * kHD + d0, p.out_dtype, o);
                     } else {
@@ -1399,7 +1423,8 @@ bool paged_fast_supported(const PagedParams& p) {
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
     // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
     if (p.block_size != 16 && p.block_size != 32) return false;
-    if (p.head_dim == 256) return p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16;  // (paged_decode256_kernel)
+    if (p.head_dim > 128)  // (paged_decode256_kernel)
+        return p.head_dim <= 256 && p.head_dim % 8 == 0 && (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16);
     return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
 }
@@ -1451,7 +1476,7 @@ static int choose_num_waves(const PagedParams& p, bool overlap) {
     // (u8 at head size 64 has the most arithmetic per byte of all: every resident wavefront, 0.59 against
     // 0.48 of HBM peak with six per compute unit on the 128-sequence u8 batch)
     if (p.cache_dtype == HIPATTN_U8) return p.head_dim <= 64 ? resident : resident / 4 * 3;
-    if (p.head_dim == 256) return resident;  // half as many bytes in flight per wavefront: twice the wavefronts
+    if (p.head_dim > 128) return resident;  // half as many bytes in flight per wavefront: twice the wavefronts
     return resident / 2;
 }
 
@@ -1462,7 +1487,7 @@ static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // first block) before it streams again, and on MI355X that costs more than the better balance
 // at the end of the kernel wins back.  The option decode_dyn_pieces_per_wave switches it on.
 static int choose_dyn_pieces(const PagedParams& p, int num_waves, bool overlap) {
-    if (overlap || p.head_dim == 256) return 0;  // (the head-256 kernel has static pieces only)
+    if (overlap || p.head_dim > 128) return 0;  // (the head-256 kernel has static pieces only)
     return num_waves * option(kOptDynPieces);
 }
 
@@ -1627,13 +1652,20 @@ template <int kWaves, bool kSelfPlan>
 static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block,
                           hipStream_t stream) {
     const bool bf16 = p.cache_dtype == HIPATTN_BF16;
-    if (p.head_dim == 256) {
+    if (p.head_dim > 128) {
         if constexpr (kWaves == 1 && !kSelfPlan) {
             const bool b32 = p.block_size == 32;
-            if (bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 32>), grid, block, 0, stream, p);
-            if (bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 16>), grid, block, 0, stream, p);
-            if (!bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 32>), grid, block, 0, stream, p);
-            if (!bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 16>), grid, block, 0, stream, p);
+            if (p.head_dim == 256) {
+                if (bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 32, false>), grid, block, 0, stream, p);
+                if (bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 16, false>), grid, block, 0, stream, p);
+                if (!bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 32, false>), grid, block, 0, stream, p);
+                if (!bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 16, false>), grid, block, 0, stream, p);
+            } else {
+                if (bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 32, true>), grid, block, 0, stream, p);
+                if (bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 16, true>), grid, block, 0, stream, p);
+                if (!bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 32, true>), grid, block, 0, stream, p);
+                if (!bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 16, true>), grid, block, 0, stream, p);
+            }
         }
     } else if (p.cache_dtype == HIPATTN_U8) {
         if (p.head_dim == 128) {

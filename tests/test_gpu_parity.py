@@ -837,15 +837,15 @@ def test_paged_mixed_batches_on_many_short_lived_streams(hip, oracle):
 
 
 @pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16), (96, 16), (80, 32), (40, 16), (120, 32), (8, 32), (72, 16),
-                                  (256, 32), (256, 16)])
+                                  (256, 32), (256, 16), (192, 16), (136, 32), (248, 32)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,Hq,Hkv", [(W.F16, W.F16, 32, 8), (W.BF16, W.BF16, 8, 8), (W.BF16, W.F16, 24, 2),
                                                         (W.F16, W.BF16, 16, 1)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
 def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window):
-    """16-bit caches on blocks of 16 or 32 tokens with any head size up to 128 that is a multiple of 8,
-    or 256, run the matrix-core kernels (decode rows on the stream-K kernel -- built for head sizes
-    64, 128 and 256, smaller heads with zero columns -- multi-token sequences on the chunk kernel of
-    their head size); the shape-generic kernels agree."""
+    """16-bit caches on blocks of 16 or 32 tokens with any head size up to 256 that is a multiple of 8
+    run the matrix-core kernels (decode rows on the stream-K kernel -- built for head sizes 64, 128
+    and 256, smaller heads with zero columns -- multi-token sequences on the chunk kernel of their
+    head size); the shape-generic kernels agree."""
     announce("paged head/block shapes", D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window)
     if kind == "decode":
         seqs = [(c - 1, 1) for c in DECODE_CTX]
@@ -1000,7 +1000,7 @@ def test_paged_generic_shapes(hip, oracle, shape):
 
 @pytest.mark.parametrize("shape", [(6, 2, 96, 64), (34, 2, 128, 32), (8, 8, 80, 8), (4, 1, 32, 64), (12, 4, 128, 8),
                                    (3, 3, 8, 4), (16, 2, 112, 128), (40, 1, 64, 32), (128, 1, 48, 16), (8, 2, 256, 64),
-                                   (4, 4, 192, 16), (6, 1, 136, 8)])
+                                   (4, 4, 192, 64), (6, 1, 136, 8)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,out_dtype", [(W.F16, W.F16, None), (W.BF16, W.BF16, None), (W.BF16, W.F16, W.F32),
                                                            (W.F16, W.BF16, W.BF16), (W.F16, W.U8, None), (W.BF16, W.U8, W.F32)])
 @pytest.mark.parametrize("window", [0, 50])
