@@ -569,12 +569,12 @@ def bench_layer_ops(hip, steps, warmup, with_cpu):
 
 def bench_other_shapes(hip, steps, warmup):
     """config 3's and config 5's batches at the other cache shapes of the matrix-core decode kernel and, at
-    head size 96 on blocks of 64, through the query-tile kernel that takes every other 16-bit shape; config 2's
+    head size 96 on blocks of 8, through the query-tile kernel that takes every other 16-bit shape; config 2's
     shape at head size 96.  Not reference configurations; no byte counters recorded for them."""
     from openvino_contrib_amd import workloads as W
 
     results = {}
-    for D, bs in ((64, 32), (64, 16), (128, 16), (96, 16), (96, 64), (256, 16)):
+    for D, bs in ((64, 32), (64, 16), (128, 16), (128, 64), (96, 16), (96, 64), (96, 8), (256, 16), (256, 128)):
         key = "c3_d%d_blk%d" % (D, bs)
         case = W.config3(head_dim=D, block_size=bs)
         r = bench_paged(hip, case, steps, warmup, "config3's batch with head size %d and cache blocks of %d tokens" % (D, bs))

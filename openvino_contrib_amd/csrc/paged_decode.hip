@@ -2,7 +2,7 @@
 // stream-K style over the whole batch.
 //
 // Work decomposition.  The unit of work is 32 tokens of the cache of one kv head of one sequence
-// -- one cache block of 32 tokens or two of 16 ("block-head": at head size 128, 8 KiB of K plus
+// -- one cache block of 32 tokens, two of 16, or a 32-token part of a larger one ("block-head": at head size 128, 8 KiB of K plus
 // 8 KiB of V in fp16, 2 x 4352 B in u8).  All
 // block-heads of the batch are laid out on one line, ordered (sequence, kv head, block), and
 // the line is cut into `num_waves` equal pieces; wavefront w owns piece w.  The kernel is
@@ -37,7 +37,7 @@
 // correction (q.(k - zp) s = s (q.k) - s zp sum(q)).
 //
 // Shapes.  The kernel is a template over the head size it is built for (128 or 64: a lane's K
-// piece count and the number of MFMAs per tile follow), the cache block size (32 or 16) and whether
+// piece count and the number of MFMAs per tile follow), the cache block size (32, 16, or 0: a larger power of two read from the call) and whether
 // the call's head size may be smaller than the built one (any multiple of 8: rows are then
 // head_dim elements apart at run time and the query columns that do not exist are zeros).  The
 // figures and layouts above are those of head size 128.
@@ -747,8 +747,8 @@ constexpr int kSelfPlanMaxRows = 256;
 // kWaves wavefronts to a workgroup.  1 is the ordinary launch.  With 8 a workgroup owns a compute
 // unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
 // leave the others free for a kernel that runs beside this one.
-// kHD, kBlk: head size (128 or 64) and cache block size (32 or 16); the self-planning form and the
-// eight-wavefront form exist for head size 128 only.
+// kHD, kBlk: head size (128 or 64) and cache block size (32, 16, or 0: a larger power of two); the self-planning form and the
+// eight-wavefront form exist for head size 128 on blocks of 32 or 16 only.
 // kPad: the call's head size (p.head_dim, a multiple of 8) may be smaller than kHD: the missing columns of
 // Q are zeros and those of V are not read.
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false>
@@ -756,8 +756,13 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
     static_assert(!kPad || (!kSelfPlan && kWaves == 1), "padded head sizes: the ordinary launch");
     static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
-    static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32), "head size 64 or 128, blocks of 16 or 32");
-    constexpr int kEntries = kUnit / kBlk;  // block-table entries per unit
+    static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32 || kBlk == 0), "head size 64 or 128, blocks of 16, 32 or more");
+    // kBlk == 0: any larger power of two (p.block_size); a block then holds several units, one after the other
+    static_assert(kBlk != 0 || (!kSelfPlan && kWaves == 1), "larger blocks: the ordinary launch");
+    constexpr int kEntries = kBlk == 16 ? 2 : 1;  // block-table entries per unit
+    constexpr int kTileBlk = kBlk == 16 ? 16 : 32;  // how a unit's two tiles lie: a block each, or sixteen rows apart
+    const int blk = kBlk ? kBlk : p.block_size;
+    const int sub_mask = kBlk ? 0 : (p.block_size >> 5) - 1;  // kBlk == 0: unit u is part (u & sub_mask) of its block
     static_assert(!kSelfPlan || kWaves == 1, "a wavefront that plans for itself is a workgroup of its own");
     const int w = kWaves == 1 ? blockIdx.x : blockIdx.x * kWaves + (threadIdx.x >> 6);
     const int lane = kWaves == 1 ? threadIdx.x : (threadIdx.x & 63), n16 = lane & 15, kg = lane >> 4;
@@ -815,7 +820,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     constexpr int64_t kRowBytesBuilt = kU8 ? (kHD + 8) : (2 * kHD);
     const int head_dim = kPad ? p.head_dim : kHD;                       // (a constant unless kPad)
     const int64_t kRowBytes = kPad ? (kU8 ? p.head_dim + 8 : 2 * p.head_dim) : kRowBytesBuilt;
-    const int64_t block_stride = (int64_t)Hkv * kBlk * kRowBytes;
+    const int64_t block_stride = (int64_t)Hkv * blk * kRowBytes;
     // kPad: this lane's K piece offsets, V offset and whether its V columns exist
     int koff[kHD / 32];
     int voff = 0;
@@ -881,10 +886,12 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         const bool whole = (n == nb);
         L = from;
         const int lb0 = rg.j0 / kUnit + b_rel;          // first unit of 32 tokens
-        const int32_t* table = p.block_indices + rg.table_begin + lb0 * kEntries;
+        // (kBlk == 0: the table is indexed by the block of the absolute unit, lb0 + ... >> log2(units per block))
+        const int32_t* table = p.block_indices + rg.table_begin + (kBlk ? lb0 * kEntries : 0);
         // table entries from there on that hold attended tokens (the row's table may end with them)
-        const int entries = (rg.ctx + kBlk - 1) / kBlk - lb0 * kEntries;
-        const int64_t head_off = (int64_t)h * kBlk * kRowBytes;
+        const int entries = (rg.ctx + blk - 1) / blk - (kBlk ? lb0 * kEntries : 0);
+        const int64_t head_off = (int64_t)h * blk * kRowBytes;
+        const int sub_shift = kBlk ? 0 : __builtin_ctz(p.block_size >> 5);
 
         if constexpr (kSelfPlan) {
             // The new tokens of this call whose cache rows this piece is about to read go into the cache
@@ -895,7 +902,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
             if (do_write && rg.write_pos >= 0) {
                 const int q_lo = max(rg.new_begin, lb0 * kUnit), q_hi = min(rg.write_pos, (lb0 + n) * kUnit - 1);
                 for (int q = q_lo; q <= q_hi; q++) {  // (wave-uniform; one pass for a decode row)
-                    const int pb_new = p.block_indices[rg.table_begin + q / kBlk];
+                    const int pb_new = p.block_indices[rg.table_begin + q / blk];
                     if (pb_new >= 0 && pb_new < p.num_blocks)
                         kv_cache_write_pair128(wp, rg.token - (rg.write_pos - q), h, pb_new, q, lane);
                 }
@@ -937,20 +944,21 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         constexpr int kGroup = 64 / kEntries;
         for (int g0 = 0; g0 < n; g0 += kGroup) {
             const int gn = min(kGroup, n - g0);
-            const int my_entry = g0 * kEntries + lane;
+            const int my_entry = kBlk ? g0 * kEntries + lane : (lb0 + g0 + lane) >> sub_shift;
             const int my_pb = (lane < gn * kEntries && my_entry < entries) ? table[my_entry] : -1;
             // which tiles of unit i were issued (0: none, the unit is skipped); never reads outside the cache
             auto issue = [&](BlockRegs<kU8>& regs, int i) -> int {
                 if constexpr (kEntries == 1) {
                     const int pb = __builtin_amdgcn_readlane(my_pb, i);
                     if (pb < 0 || pb >= p.num_blocks) return 0;
-                    const int64_t off = (int64_t)pb * block_stride + head_off;
+                    int64_t off = (int64_t)pb * block_stride + head_off;
+                    if constexpr (kBlk == 0) off += (int64_t)((lb0 + g0 + i) & sub_mask) * (kUnit * kRowBytes);
                     const uint8_t* const kb[2] = {p.key_cache + off, p.key_cache + off + 16 * kRowBytes};
                     const uint8_t* const vb[2] = {p.value_cache + off, p.value_cache + off + 16 * kRowBytes};
                     if constexpr (kPad)
-                        load_block_padded<kU8, kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok, n16, kg);
+                        load_block_padded<kU8, kHD, kTileBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok, n16, kg);
                     else
-                        load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
+                        load_block<kU8, kHD, kTileBlk>(regs, kb, vb, n16, kg);
                     return 3;
                 } else {
                     const int pb0 = __builtin_amdgcn_readlane(my_pb, 2 * i), pb1 = __builtin_amdgcn_readlane(my_pb, 2 * i + 1);
@@ -962,9 +970,9 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     const uint8_t* const kb[2] = {p.key_cache + off0, p.key_cache + off1};
                     const uint8_t* const vb[2] = {p.value_cache + off0, p.value_cache + off1};
                     if constexpr (kPad)
-                        load_block_padded<kU8, kHD, kBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok, n16, kg);
+                        load_block_padded<kU8, kHD, kTileBlk>(regs, kb, vb, (int)kRowBytes, koff, voff, v_ok, n16, kg);
                     else
-                        load_block<kU8, kHD, kBlk>(regs, kb, vb, n16, kg);
+                        load_block<kU8, kHD, kTileBlk>(regs, kb, vb, n16, kg);
                     return ok;
                 }
             };
@@ -1172,7 +1180,12 @@ __device__ __forceinline__ void pv_half(float4_t (&acc)[8], HalfRegs& v, typenam
 // kPad: the call's head size (p.head_dim, a multiple of 8 above 128) may be smaller than 256.
 template <bool kBf16, int kBlk, bool kPad>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode256_kernel(PagedParams p) {
-    constexpr int kEntries = kUnit / kBlk;
+    // kBlk: 16, 32, or 0 for any larger power of two (p.block_size: a block then holds several units)
+    constexpr int kEntries = kBlk == 16 ? 2 : 1;
+    constexpr int kTileBlk = kBlk == 16 ? 16 : 32;
+    const int blk = kBlk ? kBlk : p.block_size;
+    const int sub_mask = kBlk ? 0 : (p.block_size >> 5) - 1;
+    const int sub_shift = kBlk ? 0 : __builtin_ctz(p.block_size >> 5);
     const int w = blockIdx.x, lane = threadIdx.x, n16 = lane & 15, kg = lane >> 4;
     const int kHD = kPad ? p.head_dim : 256;  // (a constant unless kPad)
     const int kRowBytes = 2 * kHD;
@@ -1194,7 +1207,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int64_t total = (int64_t)p.blk_prefix[p.num_rows] * Hkv;
     if (total <= 0 || w >= p.num_waves) return;
     const Line line(total, p.num_waves, 0);
-    const int64_t block_stride = (int64_t)Hkv * kBlk * kRowBytes;
+    const int64_t block_stride = (int64_t)Hkv * blk * kRowBytes;
     int64_t L = line.begin(w);
     const int64_t L_end = line.begin(w + 1);
     if (L >= L_end) return;
@@ -1219,9 +1232,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         const bool whole = (n == nb);
         L = from;
         const int lb0 = rg.j0 / kUnit + b_rel;
-        const int32_t* table = p.block_indices + rg.table_begin + lb0 * kEntries;
-        const int entries = (rg.ctx + kBlk - 1) / kBlk - lb0 * kEntries;
-        const int64_t head_off = (int64_t)h * kBlk * kRowBytes;
+        const int32_t* table = p.block_indices + rg.table_begin + (kBlk ? lb0 * kEntries : 0);
+        const int entries = (rg.ctx + blk - 1) / blk - (kBlk ? lb0 * kEntries : 0);
+        const int64_t head_off = (int64_t)h * blk * kRowBytes;
 
         // Q^T operand in two halves: lane (head n16, kg) holds Q[head][128*half + kg*32 + i*8 .. +8]
         typename Op16<kBf16>::vec8 qf[2][4];
@@ -1250,7 +1263,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         constexpr int kGroup = 64 / kEntries;
         for (int g0 = 0; g0 < n; g0 += kGroup) {
             const int gn = min(kGroup, n - g0);
-            const int my_entry = g0 * kEntries + lane;
+            const int my_entry = kBlk ? g0 * kEntries + lane : (lb0 + g0 + lane) >> sub_shift;
             const int my_pb = (lane < gn * kEntries && my_entry < entries) ? table[my_entry] : -1;
             // Bases of the two tiles of unit i, and which of them lie in a block of the cache.  A block id
             // outside the cache is replaced by one inside it, so that the loads need no branch; the mask
@@ -1259,7 +1272,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 if constexpr (kEntries == 1) {
                     const int pb = __builtin_amdgcn_readlane(my_pb, i);
                     const int ok = (pb >= 0 && pb < p.num_blocks) ? 3 : 0;
-                    const int64_t off = (int64_t)min(max(pb, 0), p.num_blocks - 1) * block_stride + head_off;
+                    int64_t off = (int64_t)min(max(pb, 0), p.num_blocks - 1) * block_stride + head_off;
+                    if constexpr (kBlk == 0) off += (int64_t)((lb0 + g0 + i) & sub_mask) * (kUnit * kRowBytes);
                     kb[0] = p.key_cache + off;
                     kb[1] = kb[0] + 16 * kRowBytes;
                     vb[0] = p.value_cache + off;
@@ -1284,7 +1298,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             {
                 const uint8_t *kb[2], *vb[2];
                 (void)unit(0, kb, vb);
-                load_k_half<kBlk>(r0, kb, kRowBytes, koff[0]);
+                load_k_half<kTileBlk>(r0, kb, kRowBytes, koff[0]);
             }
             for (int i = 0; i < gn; i++) {
                 const int tok_base = (lb0 + g0 + i) * kUnit;
@@ -1294,20 +1308,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 float4_t sc[2] = {(float4_t){0.f, 0.f, 0.f, 0.f}, (float4_t){0.f, 0.f, 0.f, 0.f}};
                 // (the scheduling barriers keep each half-stage's loads behind the use of the registers
                 // they overwrite: hoisted to the top of the iteration they would all be live at once)
-                load_k_half<kBlk>(r1, kb, kRowBytes, koff[1]);
+                load_k_half<kTileBlk>(r1, kb, kRowBytes, koff[1]);
                 scores_half<kBf16>(sc, r0, qf[0]);
                 __builtin_amdgcn_sched_barrier(0);
-                load_v_half<kBlk>(r0, vb, kRowBytes, voff[0], v_ok[0]);
+                load_v_half<kTileBlk>(r0, vb, kRowBytes, voff[0], v_ok[0]);
                 scores_half<kBf16>(sc, r1, qf[1]);
                 const typename Op16<kBf16>::vec8 pf = softmax_unit<kBf16>(st, sc, c, tok_base, rg.j0, rg.ctx, kg, ok);
                 __builtin_amdgcn_sched_barrier(0);
-                load_v_half<kBlk>(r1, vb, kRowBytes, voff[1], v_ok[1]);
+                load_v_half<kTileBlk>(r1, vb, kRowBytes, voff[1], v_ok[1]);
                 pv_half<kBf16>(st.acc[0], r0, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
                 __builtin_amdgcn_sched_barrier(0);
                 {
                     const uint8_t *kbn[2], *vbn[2];
                     (void)unit(min(i + 1, gn - 1), kbn, vbn);
-                    load_k_half<kBlk>(r0, kbn, kRowBytes, koff[0]);
+                    load_k_half<kTileBlk>(r0, kbn, kRowBytes, koff[0]);
                 }
                 pv_half<kBf16>(st.acc[1], r1, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1415,14 +1429,14 @@ bool set_option(const char* name, int value) {
 
 // ---- host side of the fast path ---------------------------------------------------------
 
-// Every head size up to 128 that is a multiple of 8 with 16-bit and u8 caches, and head size 256 with 16-bit
-// caches, on blocks of 32 or 16.
+// Every head size up to 128 that is a multiple of 8 with 16-bit and u8 caches, and head sizes up to 256 with
+// 16-bit caches, on blocks of 16, 32 or a larger power of two.
 
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
     // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
-    if (p.block_size != 16 && p.block_size != 32) return false;
+    if (p.block_size < 16 || (p.block_size & (p.block_size - 1)) != 0) return false;  // 16, 32, or a larger power of two
     if (p.head_dim > 128)  // (paged_decode256_kernel)
         return p.head_dim <= 256 && p.head_dim % 8 == 0 && (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16);
     return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 &&
@@ -1465,7 +1479,7 @@ static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p
 
 static bool overlap_wanted(const PagedParams& p) {
     if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
-    if (p.head_dim != kD) return false;  // other head sizes have no eight-wavefront decode kernel
+    if (p.head_dim != kD || p.block_size > 32) return false;  // other head sizes and larger blocks have no eight-wavefront decode kernel
     return option(kOptMixedOverlap) != 0;
 }
 
@@ -1639,74 +1653,60 @@ void release_side_stream(hipStream_t owner) {
 }
 
 // The decode kernel for p's cache type, head size and block size (a combination paged_fast_supported
-// admits; head sizes other than 128 have the ordinary form only).
-template <bool kBf16, int kWaves, bool kSelfPlan, int kHD, bool kPad>
+// admits; head sizes other than 128 and blocks of more than 32 tokens have the ordinary form only).
+template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan, int kHD, bool kPad>
 static void launch_decode_blk(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block, hipStream_t stream) {
+    if (p.block_size == 32) {
+        hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, kWaves, kSelfPlan, kHD, 32, kPad>), grid, block, 0, stream, p, wp, do_write);
+    } else if (p.block_size == 16) {
+        hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, kWaves, kSelfPlan, kHD, 16, kPad>), grid, block, 0, stream, p, wp, do_write);
+    } else if constexpr (kWaves == 1 && !kSelfPlan) {
+        hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, 1, false, kHD, 0, kPad>), grid, block, 0, stream, p, wp, do_write);
+    }
+}
+
+template <bool kBf16, bool kPad>
+static void launch_decode256_blk(const PagedParams& p, dim3 grid, dim3 block, hipStream_t stream) {
     if (p.block_size == 32)
-        hipLaunchKernelGGL((paged_decode_kernel<false, kBf16, kWaves, kSelfPlan, kHD, 32, kPad>), grid, block, 0, stream, p, wp, do_write);
+        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 32, kPad>), grid, block, 0, stream, p);
+    else if (p.block_size == 16)
+        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 16, kPad>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((paged_decode_kernel<false, kBf16, kWaves, kSelfPlan, kHD, 16, kPad>), grid, block, 0, stream, p, wp, do_write);
+        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 0, kPad>), grid, block, 0, stream, p);
 }
 
 template <int kWaves, bool kSelfPlan>
 static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block,
                           hipStream_t stream) {
-    const bool bf16 = p.cache_dtype == HIPATTN_BF16;
-    if (p.head_dim > 128) {
-        if constexpr (kWaves == 1 && !kSelfPlan) {
-            const bool b32 = p.block_size == 32;
-            if (p.head_dim == 256) {
-                if (bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 32, false>), grid, block, 0, stream, p);
-                if (bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 16, false>), grid, block, 0, stream, p);
-                if (!bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 32, false>), grid, block, 0, stream, p);
-                if (!bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 16, false>), grid, block, 0, stream, p);
-            } else {
-                if (bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 32, true>), grid, block, 0, stream, p);
-                if (bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<true, 16, true>), grid, block, 0, stream, p);
-                if (!bf16 && b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 32, true>), grid, block, 0, stream, p);
-                if (!bf16 && !b32) hipLaunchKernelGGL((paged_decode256_kernel<false, 16, true>), grid, block, 0, stream, p);
-            }
-        }
-    } else if (p.cache_dtype == HIPATTN_U8) {
-        if (p.head_dim == 128) {
-            if (p.block_size == 32)
-                hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 32>), grid, block, 0, stream, p, wp, do_write);
-            else
-                hipLaunchKernelGGL((paged_decode_kernel<true, false, kWaves, kSelfPlan, 128, 16>), grid, block, 0, stream, p, wp, do_write);
-        } else if constexpr (kWaves == 1 && !kSelfPlan) {
-            const bool b32 = p.block_size == 32;
-            if (p.head_dim == 64) {
-                if (b32) hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 32>), grid, block, 0, stream, p, wp, do_write);
-                else hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 16>), grid, block, 0, stream, p, wp, do_write);
-            } else if (p.head_dim > 64) {
-                if (b32) hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 128, 32, true>), grid, block, 0, stream, p, wp, do_write);
-                else hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 128, 16, true>), grid, block, 0, stream, p, wp, do_write);
-            } else {
-                if (b32) hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 32, true>), grid, block, 0, stream, p, wp, do_write);
-                else hipLaunchKernelGGL((paged_decode_kernel<true, false, 1, false, 64, 16, true>), grid, block, 0, stream, p, wp, do_write);
-            }
-        }
-    } else if (p.head_dim == 128) {
-        if (bf16)
-            launch_decode_blk<true, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
+    const bool bf16 = p.cache_dtype == HIPATTN_BF16, u8 = p.cache_dtype == HIPATTN_U8;
+    if (p.head_dim == 128) {
+        if (u8)
+            launch_decode_blk<true, false, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
+        else if (bf16)
+            launch_decode_blk<false, true, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
         else
-            launch_decode_blk<false, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
+            launch_decode_blk<false, false, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
     } else if constexpr (kWaves == 1 && !kSelfPlan) {
-        if (p.head_dim == 64) {
-            if (bf16)
-                launch_decode_blk<true, 1, false, 64, false>(p, wp, do_write, grid, block, stream);
-            else
-                launch_decode_blk<false, 1, false, 64, false>(p, wp, do_write, grid, block, stream);
+        if (p.head_dim > 128) {
+            if (p.head_dim == 256) {
+                if (bf16) launch_decode256_blk<true, false>(p, grid, block, stream);
+                else launch_decode256_blk<false, false>(p, grid, block, stream);
+            } else {
+                if (bf16) launch_decode256_blk<true, true>(p, grid, block, stream);
+                else launch_decode256_blk<false, true>(p, grid, block, stream);
+            }
+        } else if (p.head_dim == 64) {
+            if (u8) launch_decode_blk<true, false, 1, false, 64, false>(p, wp, do_write, grid, block, stream);
+            else if (bf16) launch_decode_blk<false, true, 1, false, 64, false>(p, wp, do_write, grid, block, stream);
+            else launch_decode_blk<false, false, 1, false, 64, false>(p, wp, do_write, grid, block, stream);
         } else if (p.head_dim > 64) {
-            if (bf16)
-                launch_decode_blk<true, 1, false, 128, true>(p, wp, do_write, grid, block, stream);
-            else
-                launch_decode_blk<false, 1, false, 128, true>(p, wp, do_write, grid, block, stream);
+            if (u8) launch_decode_blk<true, false, 1, false, 128, true>(p, wp, do_write, grid, block, stream);
+            else if (bf16) launch_decode_blk<false, true, 1, false, 128, true>(p, wp, do_write, grid, block, stream);
+            else launch_decode_blk<false, false, 1, false, 128, true>(p, wp, do_write, grid, block, stream);
         } else {
-            if (bf16)
-                launch_decode_blk<true, 1, false, 64, true>(p, wp, do_write, grid, block, stream);
-            else
-                launch_decode_blk<false, 1, false, 64, true>(p, wp, do_write, grid, block, stream);
+            if (u8) launch_decode_blk<true, false, 1, false, 64, true>(p, wp, do_write, grid, block, stream);
+            else if (bf16) launch_decode_blk<false, true, 1, false, 64, true>(p, wp, do_write, grid, block, stream);
+            else launch_decode_blk<false, false, 1, false, 64, true>(p, wp, do_write, grid, block, stream);
         }
     }
 }
@@ -1724,7 +1724,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     // A pure decode batch of few rows is one launch less: the decode wavefronts plan for themselves
     // and write the new rows (see kSelfPlanMaxRows).
     const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 && p.head_dim == kD &&
-                           (!write || wp.vector_rows);
+                           p.block_size <= 32 && (!write || wp.vector_rows);
     if (self_plan) {
         if (probe.before) (void)hipEventRecord(probe.before, stream);
         launch_decode<1, true>(p, wp, write ? 1 : 0, dim3(p.num_waves), dim3(64), stream);

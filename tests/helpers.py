@@ -35,3 +35,12 @@ def scaled_bound_error(out, ref, label=""):
     print("[parity] %s max-abs %.3g, scaled by max(1,|ref|) %.3g, max |ref| %.3g" % (label, plain, scaled, float(np.abs(ref[fin]).max())),
           flush=True)
     return scaled
+
+
+def paged_matrix_core_path(Hq, Hkv, D, bs, cache_dtype):
+    """Kernel path of a paged call with 16-bit queries and a 16-bit or u8 cache at a head size that is a
+    multiple of 8 up to 256 and a power-of-two block size: the stream-K kernels take at most 16 query heads
+    per kv head on blocks of 16 tokens or more (u8 caches up to head size 128), the query-tile kernel the rest."""
+    from openvino_contrib_amd import workloads as W
+    stream_k = bs >= 16 and Hq // Hkv <= 16 and (D <= 128 or cache_dtype != W.U8)
+    return "paged_mfma" if stream_k else "paged_mfma_tiles"

@@ -837,13 +837,14 @@ def test_paged_mixed_batches_on_many_short_lived_streams(hip, oracle):
 
 
 @pytest.mark.parametrize("D,bs", [(64, 16), (64, 32), (128, 16), (96, 16), (80, 32), (40, 16), (120, 32), (8, 32), (72, 16),
-                                  (256, 32), (256, 16), (192, 16), (136, 32), (248, 32)])
+                                  (256, 32), (256, 16), (192, 16), (136, 32), (248, 32),
+                                  (128, 64), (64, 128), (96, 64), (256, 64), (200, 256), (128, 512), (48, 64)])
 @pytest.mark.parametrize("q_dtype,cache_dtype,Hq,Hkv", [(W.F16, W.F16, 32, 8), (W.BF16, W.BF16, 8, 8), (W.BF16, W.F16, 24, 2),
                                                         (W.F16, W.BF16, 16, 1)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
 def test_paged_head_64_and_blocks_of_16(hip, oracle, D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window):
-    """16-bit caches on blocks of 16 or 32 tokens with any head size up to 256 that is a multiple of 8
-    run the matrix-core kernels (decode rows on the stream-K kernel -- built for head sizes 64, 128
+    """16-bit caches on blocks of 16, 32 or a larger power of two with any head size up to 256 that is a multiple
+    of 8 run the matrix-core kernels (decode rows on the stream-K kernel -- built for head sizes 64, 128
     and 256, smaller heads with zero columns -- multi-token sequences on the chunk kernel of their
     head size); the shape-generic kernels agree."""
     announce("paged head/block shapes", D, bs, q_dtype, cache_dtype, Hq, Hkv, kind, window)
@@ -901,12 +902,13 @@ def test_paged_chunks_at_head_64(hip, oracle, bs, q_dtype, cache_dtype, out_dtyp
     dev.free()
 
 
-@pytest.mark.parametrize("D,bs", [(128, 16), (64, 16), (64, 32), (96, 16), (80, 32), (40, 16), (8, 32), (120, 32)])
+@pytest.mark.parametrize("D,bs", [(128, 16), (64, 16), (64, 32), (96, 16), (80, 32), (40, 16), (8, 32), (120, 32),
+                                  (128, 64), (64, 128), (96, 64), (56, 256)])
 @pytest.mark.parametrize("q_dtype,Hq,Hkv", [(W.F16, 32, 8), (W.BF16, 16, 1), (W.F16, 5, 5)])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 100), ("mixed", 0), ("mixed", 45), ("prefill", 0)])
 def test_paged_u8_cache_at_other_head_sizes_and_on_blocks_of_16(hip, oracle, D, bs, q_dtype, Hq, Hkv, kind, window):
-    """u8 caches at head size 128 on blocks of 16 tokens and at the other head sizes up to 128: the
-    stream-K kernel and the chunk kernel of the head size; cache bytes bit-exact."""
+    """u8 caches at head size 128 on blocks of 16 tokens or of more than 32, and at the other head sizes up to
+    128: the stream-K kernel and the chunk kernel of the head size; cache bytes bit-exact."""
     announce("paged u8 head 64 / blocks of 16", D, bs, q_dtype, Hq, Hkv, kind, window)
     if kind == "decode":
         seqs = [(c - 1, 1) for c in DECODE_CTX]
@@ -979,6 +981,35 @@ def test_paged_head_256_skips_blocks_outside_the_cache(hip, oracle, bs):
     dev.free()
 
 
+@pytest.mark.parametrize("D,cache_dtype", [(128, W.F16), (128, W.U8), (72, W.BF16), (256, W.F16), (160, W.BF16)])
+@pytest.mark.parametrize("bs", [64, 128])
+def test_paged_large_blocks_skip_blocks_outside_the_cache(hip, oracle, D, cache_dtype, bs):
+    """Blocks of more than 32 tokens hold several of the stream-K kernels' 32-token units: a block id
+    outside the pool takes all of them out, a row whose every block is outside comes out as zeros
+    (checked against the shape-generic kernels, which skip such blocks key by key)."""
+    announce("paged large blocks, bad ids", D, cache_dtype, bs)
+    seqs = [(399, 1), (47, 1), (bs, 1), (700, 1), (200, 1)]
+    qd = W.BF16 if cache_dtype == W.BF16 else W.F16
+    case = W.make_paged_case(91, seqs, 8, 4, D, bs, qd, qd, cache_dtype)
+    ids, begins = case["block_indices"], case["block_indices_begins"]
+    ids[begins[0] + 1] = case["num_blocks"] + 5   # a block in the middle
+    ids[begins[1]] = case["num_blocks"]           # the row's only block
+    ids[begins[2] + 1] = -7                       # the block that holds the new token alone
+    ids[begins[3] + 2: begins[3] + 4] = 1 << 30   # two blocks in a row
+    ids[begins[3] + 700 // bs] = -1               # the last block
+    ids[begins[4]: begins[5]] = -1                # every block of the row
+    dev = H.PagedDeviceCase(hip, case)
+    ref, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic" and np.isfinite(ref).all()
+    for waves in (0, 50, 3):
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE)
+        assert path == "paged_mfma"
+        assert np.isfinite(out).all()
+        assert H.max_abs(out, ref) <= (2e-3 if cache_dtype == W.F16 else 1e-2)
+    assert not out[1].any() and not out[4].any()
+    dev.free()
+
+
 @pytest.mark.parametrize("shape", [(6, 2, 96, 16, W.F32, W.F32), (4, 4, 80, 8, W.F32, W.F32), (8, 2, 320, 32, W.BF16, W.BF16),
                                    (4, 1, 264, 16, W.F16, W.U8), (4, 2, 64, 64, W.F32, W.U8), (4, 2, 100, 16, W.F16, W.F16)])
 def test_paged_generic_shapes(hip, oracle, shape):
@@ -1005,10 +1036,11 @@ def test_paged_generic_shapes(hip, oracle, shape):
                                                            (W.F16, W.BF16, W.BF16), (W.F16, W.U8, None), (W.BF16, W.U8, W.F32)])
 @pytest.mark.parametrize("window", [0, 50])
 def test_paged_other_shapes_on_the_matrix_cores(hip, oracle, shape, q_dtype, cache_dtype, out_dtype, window):
-    """16-bit and u8 caches whose shape the tuned kernels do not take (head sizes that are multiples of 8
-    up to 256, any power-of-two block size, more than 16 query heads per kv head): every sequence goes
-    through the query-tile kernel over the block table, a single-token sequence as one tile per kv
-    head whose rows are the heads of the group."""
+    """16-bit and u8 caches whose shape the stream-K kernels do not take (blocks of fewer than 16 tokens,
+    more than 16 query heads per kv head, u8 at head sizes above 128): every sequence goes through the
+    query-tile kernel over the block table, a single-token sequence as one tile per kv head whose rows
+    are the heads of the group.  (The list also holds shapes on blocks of 64 and 128 tokens that the
+    stream-K kernels do take.)"""
     announce("paged tiles", shape, q_dtype, cache_dtype, out_dtype, window)
     Hq, Hkv, D, bs = shape
     seqs = [(0, 9), (37, 1), (31, 2), (5, 140), (64, 1), (200, 1), (0, 1), (127, 129), (3, 0), (600, 1)]
@@ -1016,7 +1048,7 @@ def test_paged_other_shapes_on_the_matrix_cores(hip, oracle, shape, q_dtype, cac
     ref, okc, ovc = H.oracle_paged(oracle, case)
     dev = H.PagedDeviceCase(hip, case, out_dtype=out_dtype)
     out, path = dev.run()
-    assert path == "paged_mfma_tiles"
+    assert path == H.paged_matrix_core_path(Hq, Hkv, D, bs, cache_dtype)
     kc, vc = dev.caches()
     np.testing.assert_array_equal(kc, okc)
     np.testing.assert_array_equal(vc, ovc)
@@ -1030,10 +1062,10 @@ def test_paged_other_shapes_on_the_matrix_cores(hip, oracle, shape, q_dtype, cac
 
 
 def test_paged_pure_decode_of_another_shape(hip, oracle):
-    """A decode batch at head size 96 on blocks of 64: one tile per (sequence, kv head)."""
+    """A decode batch at head size 96 on blocks of 8: one tile per (sequence, kv head)."""
     announce("paged tiles decode")
     seqs = [(c - 1, 1) for c in DECODE_CTX]
-    case = W.make_paged_case(88, seqs, 24, 8, 96, 64, W.F16, W.F16, W.F16)
+    case = W.make_paged_case(88, seqs, 24, 8, 96, 8, W.F16, W.F16, W.F16)
     ref, okc, ovc = H.oracle_paged(oracle, case)
     dev = H.PagedDeviceCase(hip, case)
     out, path = dev.run()

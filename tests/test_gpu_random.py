@@ -76,7 +76,7 @@ def test_random_paged_batches_of_every_shape(hip, oracle, seed):
     """The same draws over the shapes the matrix-core paths take besides head size 128 / blocks of 32:
     head sizes that are multiples of 8 up to 256, block sizes that are powers of two, up to 128 query
     heads per kv head, 16-bit and u8 caches.  Which kernel takes a call follows from the shape
-    (the stream-K kernels on blocks of 16 or 32 with at most 16 query heads per kv head -- u8 caches up
+    (the stream-K kernels on blocks of 16 tokens or more with at most 16 query heads per kv head -- u8 caches up
     to head size 128 --; the query-tile kernel for the rest)."""
     rng = np.random.default_rng(seed)
     worst = 0.0
@@ -86,7 +86,7 @@ def test_random_paged_batches_of_every_shape(hip, oracle, seed):
         D = 8 * int(rng.integers(1, 33))
         if rng.random() < 0.3:
             D = int(rng.choice([64, 96, 128, 256]))
-        bs = int(rng.choice([4, 8, 16, 16, 32, 32, 64, 128]))
+        bs = int(rng.choice([4, 8, 16, 16, 32, 32, 64, 128, 256]))
         Hkv = int(rng.choice([1, 2, 3]))
         G = int(rng.choice([1, 2, 4, 7, 8, 16, 17, 40]))
         if G * Hkv * D > 8192:
@@ -103,8 +103,7 @@ def test_random_paged_batches_of_every_shape(hip, oracle, seed):
         out, path = dev.run()
         kc, vc = dev.caches()
         dev.free()
-        stream_k = bs in (16, 32) and G <= 16 and (D <= 128 or cache != W.U8)
-        assert path == ("paged_mfma" if stream_k else "paged_mfma_tiles")
+        assert path == H.paged_matrix_core_path(G * Hkv, Hkv, D, bs, cache)
         np.testing.assert_array_equal(kc, okc)
         np.testing.assert_array_equal(vc, ovc)
         assert np.isfinite(out).all()

@@ -68,7 +68,7 @@ def test_noalloc_mixed_batch_runs_without_the_side_stream(hip, oracle):
     assert H.max_abs(out, H.storage_to_f32(o_ws, W.BF16)) <= 1e-2
 
 
-@pytest.mark.parametrize("D,bs,path", [(96, 16, "paged_mfma"), (64, 32, "paged_mfma"), (96, 64, "paged_mfma_tiles"), (256, 16, "paged_mfma"), (192, 16, "paged_mfma"), (192, 8, "paged_mfma_tiles")])
+@pytest.mark.parametrize("D,bs,path", [(96, 16, "paged_mfma"), (64, 32, "paged_mfma"), (96, 64, "paged_mfma"), (256, 16, "paged_mfma"), (192, 16, "paged_mfma"), (192, 8, "paged_mfma_tiles")])
 def test_noalloc_on_the_other_shapes(hip, oracle, D, bs, path):
     """The other 16-bit shapes keep their scratch (partials of the stream-K kernel, the tile numbering of
     the query-tile kernel) in the static array as well: two calls in a row, the second smaller."""
