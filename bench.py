@@ -585,10 +585,11 @@ def bench_other_shapes(hip, steps, warmup):
             % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))
         results[key] = r
         del case
-    for key, kw in (("c4_blk16", {"block_size": 16}), ("c4_d64_blk32", {"head_dim": 64})):
+    for key, kw in (("c4_blk16", {"block_size": 16}), ("c4_d64_blk32", {"head_dim": 64}),
+                    ("c4_d256_blk16_s64", {"head_dim": 256, "block_size": 16, "S": 64})):
         case = W.config4(**kw)
-        r = bench_paged(hip, case, steps, warmup, "config4's batch (u8 cache) with head size %d and cache blocks of %d tokens"
-                        % (case["D"], case["block_size"]))
+        r = bench_paged(hip, case, steps, warmup, "config4's batch (u8 cache%s) with head size %d and cache blocks of %d tokens"
+                        % (", its first 64 sequences' lengths" if "S" in kw else "", case["D"], case["block_size"]))
         r["roofline"] = roofline_hbm(r, key)
         log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f (%s)"
             % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))

@@ -191,7 +191,7 @@ hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q,
  * row with its own context length, whichever sequence it belongs to, so the result is right
  * for any split of the tokens over the sequences; HIPATTN_PA_ANY_LENGTHS only changes how fast
  * such a batch runs when it does hold long multi-token sequences.
- * Kernels: 16-bit caches with a head_dim that is a multiple of 8 up to 256 (u8 caches: up to 128),
+ * Kernels: 16-bit and u8 caches with a head_dim that is a multiple of 8 up to 256,
  * a block_size that is a power of two from 16 up and at most 16 query heads per kv head take the tuned matrix-core kernels (stream-K decode for single-token rows, chunked prefill over the
  * block table for multi-token sequences; fastest at head_dim 256, 128 and 64); other
  * 16-bit and u8 caches with 16-bit queries, a head_dim that is a multiple of 8 up to 256 and a

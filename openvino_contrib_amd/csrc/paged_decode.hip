@@ -1057,7 +1057,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     }
 }
 
-// ---- head size 256 (16-bit caches) -------------------------------------------------------------
+// ---- head size 256 ------------------------------------------------------------------------------
 // The same schedule, products and lane layouts, with the head dimension worked through in two
 // halves of 128 columns so that the registers hold: a unit of 32 tokens arrives as four
 // half-stages of 32 registers -- K columns 0..127, K columns 128..255, V columns 0..127, V columns
@@ -1099,6 +1099,7 @@ __device__ __forceinline__ void load_v_half(HalfRegs& b, const uint8_t* const (&
 
 struct WaveState256 {
     float m, l;
+    float corr;  // u8 only: this lane's share of sum_j p'_j (zp_j + bias)
     float4_t acc[2][8];  // acc[half][e][r] = O[head][128 * half + (kg*4 + r)*8 + e]
 };
 
@@ -1177,9 +1178,140 @@ __device__ __forceinline__ void pv_half(float4_t (&acc)[8], HalfRegs& v, typenam
     }
 }
 
+// ---- the same for u8 caches: a half-stage is 32 tokens x 128 bytes (16 registers), so K (both halves, plus
+// the tokens' scales and zero-points) and V (both halves) are the two stages that alternate, and a
+// wavefront has as many bytes in flight as with a 16-bit cache.
+struct HalfRegs8 {
+    uint2_t x[8];  // K: [tile * 4 + piece]; V: [tile * 4 + row]
+};
+
+template <int kBlk>
+__device__ __forceinline__ void load_k_half8(HalfRegs8& b, const uint8_t* const (&kb)[2], int row, const int (&koff)[4]) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint8_t* const kt = kBlk == 32 ? kb[0] + t * 16 * row : kb[t];
+#pragma unroll
+        for (int i = 0; i < 4; i++) b.x[t * 4 + i] = *(const uint2_t*)(kt + koff[i]);
+    }
+}
+
+template <int kBlk>
+__device__ __forceinline__ void load_v_half8(HalfRegs8& b, const uint8_t* const (&vb)[2], int row, int voff, bool v_ok) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint8_t* const vt = kBlk == 32 ? vb[0] + t * 16 * row : vb[t];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            uint2_t piece = {0u, 0u};
+            if (v_ok) piece = *(const uint2_t*)(vt + voff + r * row);
+            b.x[t * 4 + r] = piece;
+        }
+    }
+}
+
+// (scale, zp) of one token per lane, laid out as in BlockRegs<true>
+template <int kBlk>
+__device__ __forceinline__ float2 load_scale_zp(const uint8_t* const (&kb)[2], const uint8_t* const (&vb)[2], int row, int n16, int kg) {
+    const int j = n16 & 7, at = (kg * 4 + (j & 3)) * row;
+    if constexpr (kBlk == 32) {
+        return *(const float2*)((n16 < 8 ? kb[0] : vb[0]) + (j >> 2) * 16 * row + at);
+    } else {  // (one of four tile bases per lane, put together arithmetically: see load_block)
+        const uintptr_t k0 = (uintptr_t)kb[0], k1 = (uintptr_t)kb[1], v0 = (uintptr_t)vb[0], v1 = (uintptr_t)vb[1];
+        const uintptr_t second = (uintptr_t)(j >> 2), value = (uintptr_t)(n16 >> 3);
+        const uintptr_t in_k = k0 + second * (k1 - k0), in_v = v0 + second * (v1 - v0);
+        return *(const float2*)(in_k + value * (in_v - in_k) + (uintptr_t)at);
+    }
+}
+
+__device__ __forceinline__ void scores_half8(float4_t (&s)[2], const HalfRegs8& k, const Op16<false>::vec8 (&q)[4]) {
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint4_t w;
+            w[0] = bytes_to_biased_half2(k.x[t * 4 + i][0], 0x04010400u);
+            w[1] = bytes_to_biased_half2(k.x[t * 4 + i][0], 0x04030402u);
+            w[2] = bytes_to_biased_half2(k.x[t * 4 + i][1], 0x04010400u);
+            w[3] = bytes_to_biased_half2(k.x[t * 4 + i][1], 0x04030402u);
+            s[t] = Op16<false>::mma(Op16<false>::from_bits(w), q[i], s[t]);
+        }
+}
+
+// softmax_unit for byte scores: the tokens' scales and zero-points turn them into scores, the
+// probabilities leave multiplied by V's scales, and st.corr collects sum_j p'_j (zp_j + bias).
+__device__ __forceinline__ Op16<false>::vec8 softmax_unit8(WaveState256& st, const float4_t (&s)[2], float2 sz, float sumq, float c,
+                                                          int tok_base, int j0, int ctx, int kg, int tiles, bool partial) {
+    float sz_scale = sz.x, sz_zero = sz.y + kByteBias;
+    if (partial) {  // rows outside the attended range may hold anything: their scale and zero-point are cleared
+        const int j = ((int)threadIdx.x & 7), tok = tok_base + (j >> 2) * 16 + kg * 4 + (j & 3);
+        if (!(tok >= j0 && tok < ctx && ((tiles >> (j >> 2)) & 1))) sz_scale = sz_zero = 0.0f;
+    }
+    const float sz_prod = sz_scale * sz_zero;
+    float ks[8], kp[8], vs[8], vz[8];
+    ks[0] = row_broadcast<0>(sz_scale); kp[0] = row_broadcast<0>(sz_prod); vs[0] = row_broadcast<8>(sz_scale); vz[0] = row_broadcast<8>(sz_zero);
+    ks[1] = row_broadcast<1>(sz_scale); kp[1] = row_broadcast<1>(sz_prod); vs[1] = row_broadcast<9>(sz_scale); vz[1] = row_broadcast<9>(sz_zero);
+    ks[2] = row_broadcast<2>(sz_scale); kp[2] = row_broadcast<2>(sz_prod); vs[2] = row_broadcast<10>(sz_scale); vz[2] = row_broadcast<10>(sz_zero);
+    ks[3] = row_broadcast<3>(sz_scale); kp[3] = row_broadcast<3>(sz_prod); vs[3] = row_broadcast<11>(sz_scale); vz[3] = row_broadcast<11>(sz_zero);
+    ks[4] = row_broadcast<4>(sz_scale); kp[4] = row_broadcast<4>(sz_prod); vs[4] = row_broadcast<12>(sz_scale); vz[4] = row_broadcast<12>(sz_zero);
+    ks[5] = row_broadcast<5>(sz_scale); kp[5] = row_broadcast<5>(sz_prod); vs[5] = row_broadcast<13>(sz_scale); vz[5] = row_broadcast<13>(sz_zero);
+    ks[6] = row_broadcast<6>(sz_scale); kp[6] = row_broadcast<6>(sz_prod); vs[6] = row_broadcast<14>(sz_scale); vz[6] = row_broadcast<14>(sz_zero);
+    ks[7] = row_broadcast<7>(sz_scale); kp[7] = row_broadcast<7>(sz_prod); vs[7] = row_broadcast<15>(sz_scale); vz[7] = row_broadcast<15>(sz_zero);
+    float sv[8];
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int j = t * 4 + r, tok = tok_base + t * 16 + kg * 4 + r;
+            const float x = fmaf(ks[j], s[t][r], -(kp[j] * sumq));
+            sv[j] = (tok >= j0 && tok < ctx && ((tiles >> t) & 1)) ? x * c : -INFINITY;
+            mloc = fmaxf(mloc, sv[j]);
+        }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    const float m_new = fmaxf(st.m, mloc);
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;  // (see softmax_unit)
+    const float alpha = fast_exp2(st.m - m_use);
+    st.m = m_new;
+    Op16<false>::vec8 pf;
+    float lsum = 0.0f, csum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        float pj = fast_exp2(sv[j] - m_use);
+        lsum += pj;
+        pj *= vs[j];
+        Op16<false>::set(pf, j, pj);
+        csum = fmaf(Op16<false>::get(pf, j), vz[j], csum);
+    }
+    st.l = st.l * alpha + lsum;
+    st.corr = st.corr * alpha + csum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) st.acc[h][e] *= alpha;
+    }
+    return pf;
+}
+
+// O^T += V^T P^T for one half of the columns, V as biased bytes (every byte is a finite number, and
+// the probabilities of rows outside the attended range are exactly zero)
+__device__ __forceinline__ void pv_half8(float4_t (&acc)[8], const HalfRegs8& v, Op16<false>::vec8 pf) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        uint4_t w;
+        const uint32_t sel = 0x0c000c00u | ((4u + (e & 3)) << 16) | (uint32_t)(e & 3);
+#pragma unroll
+        for (int jp = 0; jp < 4; jp++) w[jp] = bytes_to_biased_half2(v.x[2 * jp][e >> 2], v.x[2 * jp + 1][e >> 2], sel);
+        acc[e] = Op16<false>::mma(Op16<false>::from_bits(w), pf, acc[e]);
+    }
+}
+
 // kPad: the call's head size (p.head_dim, a multiple of 8 above 128) may be smaller than 256.
-template <bool kBf16, int kBlk, bool kPad>
+// kU8: a u8 cache (fp16 operands).
+template <bool kBf16, int kBlk, bool kPad, bool kU8 = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode256_kernel(PagedParams p) {
+    static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
     // kBlk: 16, 32, or 0 for any larger power of two (p.block_size: a block then holds several units)
     constexpr int kEntries = kBlk == 16 ? 2 : 1;
     constexpr int kTileBlk = kBlk == 16 ? 16 : 32;
@@ -1188,7 +1320,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int sub_shift = kBlk ? 0 : __builtin_ctz(p.block_size >> 5);
     const int w = blockIdx.x, lane = threadIdx.x, n16 = lane & 15, kg = lane >> 4;
     const int kHD = kPad ? p.head_dim : 256;  // (a constant unless kPad)
-    const int kRowBytes = 2 * kHD;
+    const int kRowBytes = kU8 ? kHD + 8 : 2 * kHD;
     // this lane's piece offsets inside a tile, per half, and whether its V columns exist
     int koff[2][4], voff[2];
     bool v_ok[2];
@@ -1197,9 +1329,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int first = half * 128 + kg * 32 + i * 8;  // first of the piece's eight columns
-            koff[half][i] = n16 * kRowBytes + (first < kHD ? first * 2 : 0);
+            koff[half][i] = n16 * kRowBytes + (kU8 ? 8 + (first < kHD ? first : 0) : (first < kHD ? first * 2 : 0));
         }
-        voff[half] = kg * 4 * kRowBytes + half * 256 + n16 * 16;
+        voff[half] = kg * 4 * kRowBytes + (kU8 ? 8 + half * 128 + n16 * 8 : half * 256 + n16 * 16);
         v_ok[half] = half * 128 + n16 * 8 < kHD;
     }
     const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
@@ -1238,6 +1370,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 
         // Q^T operand in two halves: lane (head n16, kg) holds Q[head][128*half + kg*32 + i*8 .. +8]
         typename Op16<kBf16>::vec8 qf[2][4];
+        float sumq = 0.0f;  // u8: the sum of the head's query elements (see process_block)
         {
             const int64_t qrow = ((int64_t)rg.token * p.num_heads_q + (int64_t)h * G + n16) * kHD;
 #pragma unroll
@@ -1250,11 +1383,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
                         for (int e = 0; e < 8; e++) Op16<kBf16>::set(qf[half][i], e, 0.0f);
                     }
+                    if constexpr (kU8) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) sumq += Op16<kBf16>::get(qf[half][i], e);
+                    }
                 }
+            if constexpr (kU8) {
+                sumq += __shfl_xor(sumq, 16, 64);
+                sumq += __shfl_xor(sumq, 32, 64);
+            }
         }
         WaveState256 st;
         st.m = -INFINITY;
         st.l = 0.0f;
+        st.corr = 0.0f;
 #pragma unroll
         for (int half = 0; half < 2; half++)
 #pragma unroll
@@ -1291,47 +1433,89 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                     return ok;
                 }
             };
-            // r0 holds the first K half of unit i when iteration i begins (loaded by the iteration before; the
-            // last iteration loads its own unit's again rather than branching).  No branch in the body: a
-            // unit whose blocks are both outside the cache goes through with every score masked.
-            HalfRegs r0, r1;
-            {
-                const uint8_t *kb[2], *vb[2];
-                (void)unit(0, kb, vb);
-                load_k_half<kTileBlk>(r0, kb, kRowBytes, koff[0]);
-            }
-            for (int i = 0; i < gn; i++) {
-                const int tok_base = (lb0 + g0 + i) * kUnit;
-                const uint8_t *kb[2], *vb[2];
-                const int ok = unit(i, kb, vb);  // (scalar work: the bases are not carried from iteration to iteration)
-                const bool partial = (tok_base < rg.j0) || (tok_base + kUnit > rg.ctx) || ok != 3;  // wavefront-uniform
-                float4_t sc[2] = {(float4_t){0.f, 0.f, 0.f, 0.f}, (float4_t){0.f, 0.f, 0.f, 0.f}};
-                // (the scheduling barriers keep each half-stage's loads behind the use of the registers
-                // they overwrite: hoisted to the top of the iteration they would all be live at once)
-                load_k_half<kTileBlk>(r1, kb, kRowBytes, koff[1]);
-                scores_half<kBf16>(sc, r0, qf[0]);
-                __builtin_amdgcn_sched_barrier(0);
-                load_v_half<kTileBlk>(r0, vb, kRowBytes, voff[0], v_ok[0]);
-                scores_half<kBf16>(sc, r1, qf[1]);
-                const typename Op16<kBf16>::vec8 pf = softmax_unit<kBf16>(st, sc, c, tok_base, rg.j0, rg.ctx, kg, ok);
-                __builtin_amdgcn_sched_barrier(0);
-                load_v_half<kTileBlk>(r1, vb, kRowBytes, voff[1], v_ok[1]);
-                pv_half<kBf16>(st.acc[0], r0, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
-                __builtin_amdgcn_sched_barrier(0);
+            if constexpr (kU8) {
+                // Two stages: K of unit i (both halves, with the scales and zero-points) is there when
+                // iteration i begins; V arrives while the scores are worked out, the next unit's K while
+                // the outputs are.  No branch in the body, as below.
+                HalfRegs8 rk[2], rv[2];
+                float2 sz;
                 {
-                    const uint8_t *kbn[2], *vbn[2];
-                    (void)unit(min(i + 1, gn - 1), kbn, vbn);
-                    load_k_half<kTileBlk>(r0, kbn, kRowBytes, koff[0]);
+                    const uint8_t *kb[2], *vb[2];
+                    (void)unit(0, kb, vb);
+                    load_k_half8<kTileBlk>(rk[0], kb, kRowBytes, koff[0]);
+                    load_k_half8<kTileBlk>(rk[1], kb, kRowBytes, koff[1]);
+                    sz = load_scale_zp<kTileBlk>(kb, vb, kRowBytes, n16, kg);
                 }
-                pv_half<kBf16>(st.acc[1], r1, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int i = 0; i < gn; i++) {
+                    const int tok_base = (lb0 + g0 + i) * kUnit;
+                    const uint8_t *kb[2], *vb[2];
+                    const int ok = unit(i, kb, vb);
+                    const bool partial = (tok_base < rg.j0) || (tok_base + kUnit > rg.ctx) || ok != 3;  // wavefront-uniform
+                    float4_t sc[2] = {(float4_t){0.f, 0.f, 0.f, 0.f}, (float4_t){0.f, 0.f, 0.f, 0.f}};
+                    load_v_half8<kTileBlk>(rv[0], vb, kRowBytes, voff[0], v_ok[0]);
+                    load_v_half8<kTileBlk>(rv[1], vb, kRowBytes, voff[1], v_ok[1]);
+                    scores_half8(sc, rk[0], qf[0]);
+                    scores_half8(sc, rk[1], qf[1]);
+                    const Op16<false>::vec8 pf = softmax_unit8(st, sc, sz, sumq, c, tok_base, rg.j0, rg.ctx, kg, ok, partial);
+                    __builtin_amdgcn_sched_barrier(0);
+                    {
+                        const uint8_t *kbn[2], *vbn[2];
+                        (void)unit(min(i + 1, gn - 1), kbn, vbn);
+                        load_k_half8<kTileBlk>(rk[0], kbn, kRowBytes, koff[0]);
+                        load_k_half8<kTileBlk>(rk[1], kbn, kRowBytes, koff[1]);
+                        sz = load_scale_zp<kTileBlk>(kbn, vbn, kRowBytes, n16, kg);
+                    }
+                    pv_half8(st.acc[0], rv[0], pf);
+                    pv_half8(st.acc[1], rv[1], pf);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                // r0 holds the first K half of unit i when iteration i begins (loaded by the iteration before; the
+                // last iteration loads its own unit's again rather than branching).  No branch in the body: a
+                // unit whose blocks are both outside the cache goes through with every score masked.
+                HalfRegs r0, r1;
+                {
+                    const uint8_t *kb[2], *vb[2];
+                    (void)unit(0, kb, vb);
+                    load_k_half<kTileBlk>(r0, kb, kRowBytes, koff[0]);
+                }
+                for (int i = 0; i < gn; i++) {
+                    const int tok_base = (lb0 + g0 + i) * kUnit;
+                    const uint8_t *kb[2], *vb[2];
+                    const int ok = unit(i, kb, vb);  // (scalar work: the bases are not carried from iteration to iteration)
+                    const bool partial = (tok_base < rg.j0) || (tok_base + kUnit > rg.ctx) || ok != 3;  // wavefront-uniform
+                    float4_t sc[2] = {(float4_t){0.f, 0.f, 0.f, 0.f}, (float4_t){0.f, 0.f, 0.f, 0.f}};
+                    // (the scheduling barriers keep each half-stage's loads behind the use of the registers
+                    // they overwrite: hoisted to the top of the iteration they would all be live at once)
+                    load_k_half<kTileBlk>(r1, kb, kRowBytes, koff[1]);
+                    scores_half<kBf16>(sc, r0, qf[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_v_half<kTileBlk>(r0, vb, kRowBytes, voff[0], v_ok[0]);
+                    scores_half<kBf16>(sc, r1, qf[1]);
+                    const typename Op16<kBf16>::vec8 pf = softmax_unit<kBf16>(st, sc, c, tok_base, rg.j0, rg.ctx, kg, ok);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_v_half<kTileBlk>(r1, vb, kRowBytes, voff[1], v_ok[1]);
+                    pv_half<kBf16>(st.acc[0], r0, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
+                    __builtin_amdgcn_sched_barrier(0);
+                    {
+                        const uint8_t *kbn[2], *vbn[2];
+                        (void)unit(min(i + 1, gn - 1), kbn, vbn);
+                        load_k_half<kTileBlk>(r0, kbn, kRowBytes, koff[0]);
+                    }
+                    pv_half<kBf16>(st.acc[1], r1, pf, partial, tok_base, rg.j0, rg.ctx, kg, ok);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
 
         // ---- this wavefront's result for the segment
-        float l = st.l;
+        float l = st.l, corr = st.corr;
         l += __shfl_xor(l, 16, 64);
         l += __shfl_xor(l, 32, 64);
+        if constexpr (kU8) {
+            corr += __shfl_xor(corr, 16, 64);
+            corr += __shfl_xor(corr, 32, 64);
+        }
         const int64_t slot = (int64_t)w + (int64_t)s * Hkv + h;  // unique per (piece, segment)
         if (n16 < G) {
             const float inv = whole ? (l > 0.0f ? 1.0f / l : 0.0f) : 1.0f;
@@ -1341,7 +1525,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 for (int r = 0; r < 4; r++) {
                     float o[8];
 #pragma unroll
-                    for (int e = 0; e < 8; e++) o[e] = st.acc[half][e][r] * inv;
+                    for (int e = 0; e < 8; e++) o[e] = (kU8 ? st.acc[half][e][r] - corr : st.acc[half][e][r]) * inv;
                     const int d0 = half * 128 + (kg * 4 + r) * 8;
                     if (kPad && d0 >= kHD) continue;  // (columns beyond the head size hold nothing)
                     if (whole) {
@@ -1429,17 +1613,16 @@ bool set_option(const char* name, int value) {
 
 // ---- host side of the fast path ---------------------------------------------------------
 
-// Every head size up to 128 that is a multiple of 8 with 16-bit and u8 caches, and head sizes up to 256 with
-// 16-bit caches, on blocks of 16, 32 or a larger power of two.
+// Every head size up to 256 that is a multiple of 8 with 16-bit and u8 caches, on blocks of 16, 32 or a
+// larger power of two.
 
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
     // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
     if (p.block_size < 16 || (p.block_size & (p.block_size - 1)) != 0) return false;  // 16, 32, or a larger power of two
-    if (p.head_dim > 128)  // (paged_decode256_kernel)
-        return p.head_dim <= 256 && p.head_dim % 8 == 0 && (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16);
-    return p.head_dim >= 8 && p.head_dim <= 128 && p.head_dim % 8 == 0 &&
+    // (above 128: paged_decode256_kernel)
+    return p.head_dim >= 8 && p.head_dim <= 256 && p.head_dim % 8 == 0 &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
 }
 
@@ -1489,8 +1672,8 @@ static int choose_num_waves(const PagedParams& p, bool overlap) {
     if (overlap) return resident;  // the most the plan may choose
     // (u8 at head size 64 has the most arithmetic per byte of all: every resident wavefront, 0.59 against
     // 0.48 of HBM peak with six per compute unit on the 128-sequence u8 batch)
-    if (p.cache_dtype == HIPATTN_U8) return p.head_dim <= 64 ? resident : resident / 4 * 3;
     if (p.head_dim > 128) return resident;  // half as many bytes in flight per wavefront: twice the wavefronts
+    if (p.cache_dtype == HIPATTN_U8) return p.head_dim <= 64 ? resident : resident / 4 * 3;
     return resident / 2;
 }
 
@@ -1665,14 +1848,14 @@ static void launch_decode_blk(const PagedParams& p, const KvWriteParams& wp, int
     }
 }
 
-template <bool kBf16, bool kPad>
+template <bool kBf16, bool kPad, bool kU8 = false>
 static void launch_decode256_blk(const PagedParams& p, dim3 grid, dim3 block, hipStream_t stream) {
     if (p.block_size == 32)
-        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 32, kPad>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 32, kPad, kU8>), grid, block, 0, stream, p);
     else if (p.block_size == 16)
-        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 16, kPad>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 16, kPad, kU8>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 0, kPad>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((paged_decode256_kernel<kBf16, 0, kPad, kU8>), grid, block, 0, stream, p);
 }
 
 template <int kWaves, bool kSelfPlan>
@@ -1689,10 +1872,12 @@ static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_
     } else if constexpr (kWaves == 1 && !kSelfPlan) {
         if (p.head_dim > 128) {
             if (p.head_dim == 256) {
-                if (bf16) launch_decode256_blk<true, false>(p, grid, block, stream);
+                if (u8) launch_decode256_blk<false, false, true>(p, grid, block, stream);
+                else if (bf16) launch_decode256_blk<true, false>(p, grid, block, stream);
                 else launch_decode256_blk<false, false>(p, grid, block, stream);
             } else {
-                if (bf16) launch_decode256_blk<true, true>(p, grid, block, stream);
+                if (u8) launch_decode256_blk<false, true, true>(p, grid, block, stream);
+                else if (bf16) launch_decode256_blk<true, true>(p, grid, block, stream);
                 else launch_decode256_blk<false, true>(p, grid, block, stream);
             }
         } else if (p.head_dim == 64) {

@@ -40,7 +40,6 @@ def scaled_bound_error(out, ref, label=""):
 def paged_matrix_core_path(Hq, Hkv, D, bs, cache_dtype):
     """Kernel path of a paged call with 16-bit queries and a 16-bit or u8 cache at a head size that is a
     multiple of 8 up to 256 and a power-of-two block size: the stream-K kernels take at most 16 query heads
-    per kv head on blocks of 16 tokens or more (u8 caches up to head size 128), the query-tile kernel the rest."""
-    from openvino_contrib_amd import workloads as W
-    stream_k = bs >= 16 and Hq // Hkv <= 16 and (D <= 128 or cache_dtype != W.U8)
+    per kv head on blocks of 16 tokens or more, the query-tile kernel the rest."""
+    stream_k = bs >= 16 and Hq // Hkv <= 16
     return "paged_mfma" if stream_k else "paged_mfma_tiles"

@@ -76,8 +76,8 @@ def test_random_paged_batches_of_every_shape(hip, oracle, seed):
     """The same draws over the shapes the matrix-core paths take besides head size 128 / blocks of 32:
     head sizes that are multiples of 8 up to 256, block sizes that are powers of two, up to 128 query
     heads per kv head, 16-bit and u8 caches.  Which kernel takes a call follows from the shape
-    (the stream-K kernels on blocks of 16 tokens or more with at most 16 query heads per kv head -- u8 caches up
-    to head size 128 --; the query-tile kernel for the rest)."""
+    (the stream-K kernels on blocks of 16 tokens or more with at most 16 query heads per kv head; the query-tile
+    kernel for the rest)."""
     rng = np.random.default_rng(seed)
     worst = 0.0
     for it in range(40):
