@@ -748,7 +748,7 @@ constexpr int kSelfPlanMaxRows = 256;
 // unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
 // leave the others free for a kernel that runs beside this one.
 // kHD, kBlk: head size (128 or 64) and cache block size (32, 16, or 0: a larger power of two); the self-planning form and the
-// eight-wavefront form exist for head size 128 on blocks of 32 or 16 only.
+// eight-wavefront form exist for head size 128 only, the self-planning form on blocks of 32 or 16 only.
 // kPad: the call's head size (p.head_dim, a multiple of 8) may be smaller than kHD: the missing columns of
 // Q are zeros and those of V are not read.
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false>
@@ -758,7 +758,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
     static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32 || kBlk == 0), "head size 64 or 128, blocks of 16, 32 or more");
     // kBlk == 0: any larger power of two (p.block_size); a block then holds several units, one after the other
-    static_assert(kBlk != 0 || (!kSelfPlan && kWaves == 1), "larger blocks: the ordinary launch");
+    static_assert(kBlk != 0 || !kSelfPlan, "larger blocks: no self-planning form");
     constexpr int kEntries = kBlk == 16 ? 2 : 1;  // block-table entries per unit
     constexpr int kTileBlk = kBlk == 16 ? 16 : 32;  // how a unit's two tiles lie: a block each, or sixteen rows apart
     const int blk = kBlk ? kBlk : p.block_size;
@@ -1662,7 +1662,7 @@ static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p
 
 static bool overlap_wanted(const PagedParams& p) {
     if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
-    if (p.head_dim != kD || p.block_size > 32) return false;  // other head sizes and larger blocks have no eight-wavefront decode kernel
+    if (p.head_dim != kD) return false;  // other head sizes have no eight-wavefront decode kernel
     return option(kOptMixedOverlap) != 0;
 }
 
@@ -1836,15 +1836,15 @@ void release_side_stream(hipStream_t owner) {
 }
 
 // The decode kernel for p's cache type, head size and block size (a combination paged_fast_supported
-// admits; head sizes other than 128 and blocks of more than 32 tokens have the ordinary form only).
+// admits; head sizes other than 128 have the ordinary form only, blocks of more than 32 tokens no self-planning form).
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan, int kHD, bool kPad>
 static void launch_decode_blk(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block, hipStream_t stream) {
     if (p.block_size == 32) {
         hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, kWaves, kSelfPlan, kHD, 32, kPad>), grid, block, 0, stream, p, wp, do_write);
     } else if (p.block_size == 16) {
         hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, kWaves, kSelfPlan, kHD, 16, kPad>), grid, block, 0, stream, p, wp, do_write);
-    } else if constexpr (kWaves == 1 && !kSelfPlan) {
-        hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, 1, false, kHD, 0, kPad>), grid, block, 0, stream, p, wp, do_write);
+    } else if constexpr (!kSelfPlan) {
+        hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, kWaves, false, kHD, 0, kPad>), grid, block, 0, stream, p, wp, do_write);
     }
 }
 
@@ -1923,7 +1923,12 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     hipLaunchKernelGGL(paged_prologue_kernel, dim3(write_blocks + 1), dim3(256), 0, stream, wp, p, write_blocks);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    if (p.max_q_tiles > 0 && p.overlap) {
+    // Shapes without the eight-wavefront decode kernel run the two parts side by side all the same when
+    // the decode wavefronts take at most half of every compute unit's registers (and no LDS), so that the
+    // chunks' workgroups find room beside them.
+    const bool beside = p.max_q_tiles > 0 && !p.overlap && !p.no_side_stream && option(kOptMixedOverlap) != 0 &&
+                        p.num_waves * 2 <= resident_decode_waves();
+    if (p.max_q_tiles > 0 && (p.overlap || beside)) {
         // Mixed batch: the decode sequences stream from HBM on a few compute units while the
         // chunks' flash kernel, on a side stream, has the others; both only need the prologue's
         // results.  The decode kernel stays on the caller's stream, directly behind the prologue,
@@ -1934,7 +1939,10 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         if ((e = hipEventRecord(side->fork, stream)) != hipSuccess) return e;
         if ((e = hipStreamWaitEvent(side->stream, side->fork, 0)) != hipSuccess) return e;
         if (probe.before) (void)hipEventRecord(probe.before, stream);
-        launch_decode<8, false>(p, wp, 0, dim3(p.num_waves / 8), dim3(512), stream);
+        if (p.overlap)
+            launch_decode<8, false>(p, wp, 0, dim3(p.num_waves / 8), dim3(512), stream);
+        else
+            launch_decode<1, false>(p, wp, 0, dim3(p.num_waves), dim3(64), stream);
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
         const hipError_t e_prefill = launch_paged_prefill(p, side->stream);
