@@ -73,16 +73,18 @@ MIXED_BATCH = [(0, 130), (37, 1), (500, 1), (100, 257), (999, 1), (64, 1)]
 LOOKS_LIKE_DECODE = [(1500, 1), (100, 2), (31, 0)]  # as many tokens as sequences, but not one each
 
 
+@pytest.mark.parametrize("shape", [(16, 4, 128, 32), (8, 2, 256, 64), (12, 4, 96, 16)])
 @pytest.mark.parametrize("cache_dtype,q_dtype,window,seqs", [(W.F16, W.F16, 0, MIXED_BATCH), (W.U8, W.F16, 0, MIXED_BATCH),
                                                               (W.F16, W.BF16, 200, MIXED_BATCH),
                                                               (W.F16, W.F16, 64, LOOKS_LIKE_DECODE)])
-def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_dtype, window, seqs):
-    print("[plugin] paged attention", cache_dtype, q_dtype, window, seqs, flush=True)
-    case = W.make_paged_case(94, seqs, 16, 4, 128, 32, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_dtype, window, seqs, shape):
+    print("[plugin] paged attention", cache_dtype, q_dtype, window, seqs, shape, flush=True)
+    Hq, Hkv, D, bs = shape  # (nothing in the operator is fixed to a head size or a cache block size)
+    case = W.make_paged_case(94, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
     plugin = P.Plugin()
     plugin.set_property("PERF_COUNT", "YES")
     # the operator's full signature: four empty optional inputs behind max_context_len and the scores output
-    compiled = plugin.compile_model(P.Model.paged_attention(q_dtype, q_dtype, cache_dtype, 16, 4, 128, 32,
+    compiled = plugin.compile_model(P.Model.paged_attention(q_dtype, q_dtype, cache_dtype, Hq, Hkv, D, bs,
                                                             extra_inputs=4, extra_len=0, scores_result=True))
     assert compiled.input_names()[3:5] == ["key_cache", "value_cache"]
     assert compiled.get_property("EXECUTION_DEVICES") == "HIP.0"
@@ -117,7 +119,7 @@ def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_
     ref, okc, ovc = H.oracle_paged(oracle, case)
     # the scores Result is connected, so the second output is produced: every new token aggregated
     ref_scores = oracle.paged_attention_scores(case["q"], okc, cache_dtype, case["past_lens"], case["subsequence_begins"],
-                                               case["block_indices"], case["block_indices_begins"], 16, 4, 128, 32,
+                                               case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
                                                sliding_window=window)
     assert scores.dtype == np.float32 and scores.shape == ref_scores.shape
     assert H.max_abs(scores, ref_scores) <= 2e-5 * max(1.0, float(ref_scores.max()))
