@@ -24,6 +24,8 @@ namespace flash_small {
 
 // kDP is the head size the kernel is built for, 64, 128 or 256; the call's head size (w.head_dim, a
 // multiple of 8) may be smaller: the missing columns of Q, K and V are zeros in registers and LDS.
+// kUsed (head sizes 72..96 in the head-128 build: 96) stops the products at that column: the k-steps and
+// output tiles beyond it are not computed.
 constexpr int kTileK = 64;                  // keys per tile
 constexpr int kWaves = 4;
 constexpr int kTileQ = 32 * kWaves;         // query rows per workgroup
@@ -192,9 +194,13 @@ __device__ __forceinline__ uint32_t pack2(int dtype, float lo, float hi) {
 // kU8 (paged, fp16 products): the cache rows are [scale f32][zero-point f32][head_dim bytes]; a piece
 // travels as its eight bytes and the row's scale and zero-point and becomes eight fp16 values
 // (byte - zero-point) * scale on its way into LDS.
-template <bool kBf16, bool kMask, bool kPaged, int kDP, bool kU8 = false>
+template <bool kBf16, bool kMask, bool kPaged, int kDP, bool kU8 = false, int kUsed = kDP>
 __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_bytes<kDP>()]) {
     static_assert(!kU8 || (kPaged && !kBf16), "u8 rows exist in paged caches and are multiplied as fp16");
+    // kUsed: the columns the products run over (w.head_dim <= kUsed <= kDP, a multiple of 16); the rows in LDS
+    // keep the layout of kDP columns
+    static_assert(kUsed % 16 == 0 && kUsed <= kDP, "whole k-steps of the score product");
+    constexpr int kSteps = kUsed / 16, kOutTiles = (kUsed + 31) / 32;
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     constexpr int kChunks = kDP / 8;             // 16-byte chunks of a row in LDS
@@ -214,13 +220,13 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 
     // Q^T fragments (B operand of S^T = K Q^T): lane (n32, hi) holds query row n32, head-dim
     // elements 8 (2i + hi) .. + 7 for k-step i, times scale * log2(e)
-    vec8 qf[kDP / 16];
+    vec8 qf[kSteps];
     {
         const float c = w.scale * kLog2e;
         const int row = min(my_row, w.rows - 1);
         const bool q_bf16 = w.q_dtype == HIPATTN_BF16;
 #pragma unroll
-        for (int i = 0; i < kDP / 16; i++) {
+        for (int i = 0; i < kSteps; i++) {
             uint4_t raw = {0u, 0u, 0u, 0u};
             if (2 * i + hi < chunks) raw = *(const uint4_t*)(w.q + (int64_t)row * w.q_stride + 8 * (2 * i + hi));
             uint4_t cv;
@@ -296,9 +302,9 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
         }
     };
 
-    float16_t o[kDP / 32];
+    float16_t o[kOutTiles];
 #pragma unroll
-    for (int dt = 0; dt < kDP / 32; dt++)
+    for (int dt = 0; dt < kOutTiles; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;  // the row's running maximum (both lanes of a pair agree) and this lane's share of the sum
@@ -364,7 +370,7 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 #pragma unroll
             for (int r = 0; r < 16; r++) s[mt][r] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < kDP / 16; i++) {
+            for (int i = 0; i < kSteps; i++) {
                 const int row = mt * 32 + n32;
                 const vec8 kf = __builtin_bit_cast(vec8, *(const __attribute__((address_space(3))) uint4_t*)(k_lds + k_chunk_offset<kDP>(row, 2 * i + hi)));
                 s[mt] = M::mma(kf, qf[i], s[mt]);
@@ -432,14 +438,14 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
         l_run = l_run * alpha + sum;
         m_run = m_new;
 #pragma unroll
-        for (int dt = 0; dt < kDP / 32; dt++)
+        for (int dt = 0; dt < kOutTiles; dt++)
 #pragma unroll
             for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
         // O^T += V^T P^T
 #pragma unroll
         for (int ks = 0; ks < 4; ks++)
 #pragma unroll
-            for (int dt = 0; dt < kDP / 32; dt++) o[dt] = M::mma(read_v_frag<kBf16, kDP>(v_lds, lane, ks, dt), pf[ks], o[dt]);
+            for (int dt = 0; dt < kOutTiles; dt++) o[dt] = M::mma(read_v_frag<kBf16, kDP>(v_lds, lane, ks, dt), pf[ks], o[dt]);
 
         if (j + 1 < tiles) deposit(next, buf ^ 1);  // the other buffer was last read before the previous barrier
         __syncthreads();
@@ -456,7 +462,7 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
     if (my_row < w.rows) {
 #pragma unroll
-        for (int dt = 0; dt < kDP / 32; dt++)
+        for (int dt = 0; dt < kOutTiles; dt++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int d = dt * 32 + 8 * g + 4 * hi;
@@ -476,7 +482,7 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 
 // Dense SDPA: one workgroup per (batch, query head, 128-row query tile).  kMask: p.mask rides along
 // (ignored under the causal flag).
-template <bool kBf16, bool kMask, int kDP>
+template <bool kBf16, bool kMask, int kDP, int kUsed>
 __device__ __forceinline__ void sdpa_small_tile(const SdpaParams& p, uint8_t (*lds)[2][tile_bytes<kDP>()]) {
     const int q_tiles = (p.len_q + kTileQ - 1) / kTileQ;
     const int qt = blockIdx.x % q_tiles;
@@ -517,22 +523,22 @@ __device__ __forceinline__ void sdpa_small_tile(const SdpaParams& p, uint8_t (*l
         w.mask_key_stride = p.mask_stride[3];
         w.mask_dtype = p.mask_dtype;
     }
-    attend<kBf16, kMask, false, kDP>(w, lds);
+    attend<kBf16, kMask, false, kDP, false, kUsed>(w, lds);
 }
 
 // (two workgroups per compute unit also in the head-128 build: at most 256 registers; the head-256
 // build needs nearly all 512 and runs one)
-template <bool kBf16, int kDP>
+template <bool kBf16, int kDP, int kUsed = kDP>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))) void sdpa_flash_small_kernel(SdpaParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];  // [buffer][K, V]
-    sdpa_small_tile<kBf16, false, kDP>(p, lds);
+    sdpa_small_tile<kBf16, false, kDP, kUsed>(p, lds);
 }
 
 // (the mask values of a tile take 32 more registers: no bound on them)
-template <bool kBf16, int kDP>
+template <bool kBf16, int kDP, int kUsed = kDP>
 __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_small_masked_kernel(SdpaParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];
-    sdpa_small_tile<kBf16, true, kDP>(p, lds);
+    sdpa_small_tile<kBf16, true, kDP, kUsed>(p, lds);
 }
 
 // Query tiles of a PagedAttentionExtension batch over the block table (16-bit caches): a sequence
@@ -542,7 +548,7 @@ __global__ __launch_bounds__(64 * kWaves) void sdpa_flash_small_masked_kernel(Sd
 // p.tile_prefix (written on the device by the plan of the decode path or by paged_tiles_plan_kernel),
 // the later -- heavier -- tiles of a sequence first.  One workgroup per (tile, head); the grid is
 // an upper bound.
-template <bool kBf16, int kDP, bool kU8 = false>
+template <bool kBf16, int kDP, bool kU8 = false, int kUsed = kDP>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))) void paged_tiles_kernel(PagedParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2][2][tile_bytes<kDP>()];
     const int item = blockIdx.x / p.num_heads_q, h = blockIdx.x % p.num_heads_q;
@@ -595,7 +601,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))
     w.mask = nullptr;
     w.mask_row_stride = w.mask_key_stride = 0;
     w.mask_dtype = 0;
-    attend<kBf16, false, true, kDP, kU8>(w, lds);
+    attend<kBf16, false, true, kDP, kU8, kUsed>(w, lds);
 }
 
 // tile_prefix for a batch in which every sequence with tokens goes through paged_tiles_kernel
@@ -634,20 +640,20 @@ bool sdpa_flash_small_supported(const SdpaParams& p) {
            p.len_kv > 0 && p.len_q > 0 && aligned16(p.q) && aligned16(p.k) && aligned16(p.v) && ((uintptr_t)p.out % 8) == 0;
 }
 
-template <bool kMask, int kDP>
+template <bool kMask, int kDP, int kUsed = kDP>
 static void launch_sdpa_small(const SdpaParams& p, unsigned groups, hipStream_t stream) {
     const dim3 grid(groups), block(64 * flash_small::kWaves);
     const bool bf16 = p.dtype == HIPATTN_BF16;
     if constexpr (kMask) {
         if (bf16)
-            hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<true, kDP>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<true, kDP, kUsed>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<false, kDP>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_masked_kernel<false, kDP, kUsed>), grid, block, 0, stream, p);
     } else {
         if (bf16)
-            hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<true, kDP>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<true, kDP, kUsed>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<false, kDP>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((flash_small::sdpa_flash_small_kernel<false, kDP, kUsed>), grid, block, 0, stream, p);
     }
 }
 
@@ -655,6 +661,8 @@ template <bool kMask>
 static void launch_sdpa_small(const SdpaParams& p, unsigned groups, hipStream_t stream) {
     if (p.head_dim <= 64)
         launch_sdpa_small<kMask, 64>(p, groups, stream);
+    else if (p.head_dim <= 96)  // (the head-128 build without its last two k-steps and its last output tile)
+        launch_sdpa_small<kMask, 128, 96>(p, groups, stream);
     else if (p.head_dim <= 128)
         launch_sdpa_small<kMask, 128>(p, groups, stream);
     else
@@ -682,6 +690,8 @@ static void launch_tiles(const PagedParams& p, unsigned groups, hipStream_t stre
     if (p.cache_dtype == HIPATTN_U8) {
         if (p.head_dim <= 64)
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 64, true>), grid, block, 0, stream, p);
+        else if (p.head_dim <= 96)
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 128, true, 96>), grid, block, 0, stream, p);
         else if (p.head_dim <= 128)
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 128, true>), grid, block, 0, stream, p);
         else
@@ -696,6 +706,11 @@ static void launch_tiles(const PagedParams& p, unsigned groups, hipStream_t stre
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 256>), grid, block, 0, stream, p);
         else
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 256>), grid, block, 0, stream, p);
+    } else if (p.head_dim <= 96) {
+        if (bf16)
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 128, false, 96>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash_small::paged_tiles_kernel<false, 128, false, 96>), grid, block, 0, stream, p);
     } else {
         if (bf16)
             hipLaunchKernelGGL((flash_small::paged_tiles_kernel<true, 128>), grid, block, 0, stream, p);
