@@ -604,9 +604,9 @@ def bench_other_shapes(hip, steps, warmup):
         results[key] = r
         del case
     case = W.config2(D=96)
-    r = bench_sdpa(hip, case, steps, warmup, "config2's shape at head size 96 (the plain matrix-core kernel: 96 columns of its head-128 build)")
+    r = bench_sdpa(hip, case, steps, warmup, "config2's shape at head size 96 (the tuned head-128 kernel on rows of 96 columns)")
     r["roofline"] = roofline_mfma(r)
-    r["roofline"]["traffic"], r["roofline"]["traffic_source"], r["roofline"]["kernel"] = None, None, "sdpa_flash_small_kernel"
+    r["roofline"]["traffic"], r["roofline"]["traffic_source"], r["roofline"]["kernel"] = None, None, "sdpa_flash_padded_kernel"
     log("c2_d96: %.3f ms/step, roofline frac %.3f (%s)" % (r["ms_per_step"], r["roofline"]["frac"], r["kernel_path"]))
     results["c2_d96"] = r
     return results

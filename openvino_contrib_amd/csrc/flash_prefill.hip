@@ -119,6 +119,7 @@ struct Tile {
     int window;
     int q_dtype;         // HIPATTN_F16 / HIPATTN_BF16 (converted to the MFMA type when they differ)
     int out_dtype;
+    int head_dim;        // columns of a row in memory: kD, or fewer in the kPad form of the dense kernel
     // keys / values: the same for both groups of a workgroup
     const uint8_t* k;
     const uint8_t* v;
@@ -178,12 +179,12 @@ __device__ __forceinline__ void key_range(const Tile& t, int& lo, int& hi) {
 // Byte offset of a key's row from t.k / t.v.  Keys past the end are redirected to the last valid
 // key and block ids outside the cache are clamped: such rows only ever meet a probability of
 // zero (or are unspecified input), but they must be readable and finite.
-__device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key) {
+__device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key, int row_bytes = kRowBytes) {
     key = min(key, t.kv_len - 1);
-    if (t.table == nullptr) return (int64_t)key * kRowBytes;
+    if (t.table == nullptr) return (int64_t)key * row_bytes;
     const int lb = key >> t.block_shift;  // block_size is a power of two on this path
     const int pb = min(max(t.table[lb], 0), t.num_blocks - 1);
-    return (int64_t)pb * t.block_stride + (int64_t)(key & (t.block_size - 1)) * kRowBytes;
+    return (int64_t)pb * t.block_stride + (int64_t)(key & (t.block_size - 1)) * row_bytes;
 }
 
 // Q fragment, multiplied by c = scale * log2(e) and rounded to the MFMA element type: the first
@@ -502,6 +503,7 @@ __device__ __forceinline__ void store_rows(const Tile& t, const float16_t (&o)[4
 #pragma unroll
         for (int rq = 0; rq < 4; rq++) {
             const int d = dt * 32 + 8 * rq + 4 * hi;
+            if (d >= t.head_dim) continue;  // (columns the rows in memory do not have)
             const float x0 = o[dt][rq * 4] * inv, x1 = o[dt][rq * 4 + 1] * inv, x2 = o[dt][rq * 4 + 2] * inv,
                         x3 = o[dt][rq * 4 + 3] * inv;
             if constexpr (kOutDtype == HIPATTN_F32) {
@@ -542,16 +544,17 @@ __device__ __forceinline__ void store_rows_via_lds(const Tile& t, const float16_
     for (int k = 0; k < 8; k++) {
         const int r = 4 * k + lrow;
         const uint4_t w = *(const lds_uint4*)(stage + r * kRowBytes + ((chunk ^ (r & 15)) << 4));
-        if (row0 + r < t.rows) *(uint4_t*)((uint16_t*)t.out + (int64_t)(row0 + r) * t.out_stride + chunk * 8) = w;
+        if (row0 + r < t.rows && chunk * 8 < t.head_dim) *(uint4_t*)((uint16_t*)t.out + (int64_t)(row0 + r) * t.out_stride + chunk * 8) = w;
     }
 }
 
 // Wave-uniform address of the 8 consecutive rows that start at key0 (a multiple of 8 below
 // kv_len): they lie in one block of a paged cache, whose table entry is `entry`.
-__device__ __forceinline__ const uint8_t* row_group_base(const Tile& t, const uint8_t* base, int key0, int entry) {
-    if (t.table == nullptr) return base + (int64_t)key0 * kRowBytes;
+__device__ __forceinline__ const uint8_t* row_group_base(const Tile& t, const uint8_t* base, int key0, int entry,
+                                                         int row_bytes = kRowBytes) {
+    if (t.table == nullptr) return base + (int64_t)key0 * row_bytes;
     const int pb = min(max(entry, 0), t.num_blocks - 1);
-    return base + (int64_t)pb * t.block_stride + (int64_t)(key0 & (t.block_size - 1)) * kRowBytes;
+    return base + (int64_t)pb * t.block_stride + (int64_t)(key0 & (t.block_size - 1)) * row_bytes;
 }
 
 // Workgroup barrier that lets the `keep` most recent global->LDS loads of this wavefront stay in
@@ -618,9 +621,17 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is ev
 // read in phase 2j+1.  Between the barriers each group runs one matrix and one vector phase, in
 // opposite order, so that the matrix core and the vector units are both in use; the odd phase
 // boundaries are not enforced, the two groups only drift by what their phases differ in length.
-template <bool kBf16, bool kU8 = false, bool kPaged = true, int kMask = 0>
+// kPad (16-bit K/V, no mask): the rows of Q, K, V and the output have t.head_dim < kD columns in memory (a
+// multiple of 8).  Everything in LDS and in registers keeps the layout of kD columns: a lane whose 16-byte
+// chunk of a row does not exist fetches the row's first chunk instead -- valid, finite data that only
+// ever meets the zeros the query fragments hold in those columns, or lands in output columns that
+// are not stored.
+template <bool kBf16, bool kU8 = false, bool kPaged = true, int kMask = 0, bool kPad = false>
 __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
     static_assert(kPaged || !kU8, "dense K/V are 16-bit");
+    static_assert(!kPad || (!kU8 && kMask == 0), "smaller head sizes: 16-bit K/V, no mask");
+    const int grow = kPad ? 2 * t.head_dim : kRowBytes;  // bytes from row to row in memory
+    const int head_chunks = kPad ? t.head_dim >> 3 : kD / 8;
     static_assert(kMask == 0 || !kPaged, "attention masks belong to the dense operator");
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16");
     using M = Mfma<kBf16>;
@@ -667,7 +678,9 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         for (int k = 0; k < 8; k++) {
             const int r = 4 * k + lr;
             const int qrow = min((wave & 3) * 32 + r, t.rows - 1);
-            const uint8_t* src = (const uint8_t*)(t.q + (int64_t)qrow * t.q_stride) + ((lp ^ (r & 15)) << 4);
+            int q_chunk = lp ^ (r & 15);
+            if constexpr (kPad) q_chunk = q_chunk < head_chunks ? q_chunk : 0;
+            const uint8_t* src = (const uint8_t*)(t.q + (int64_t)qrow * t.q_stride) + (q_chunk << 4);
             load_to_lds_16(src, wave_stage + 4 * k * kRowBytes);
         }
     }
@@ -691,8 +704,14 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     // tile.  Lane l fills chunk position l % 16 of row r = 8w + 4k + l / 16, i.e. it fetches chunk
     // (l % 16) ^ swz(r): for K that is ((l%16) ^ (l/16) ^ 8(w%2)) ^ 4k, for V (l%16) ^ 4(l/16).
     const int lrow = lane >> 4, lpos = lane & 15;
-    const uint32_t k_lane = (uint32_t)(((lpos ^ lrow ^ (8 * (wave & 1))) << 4) + lrow * kRowBytes);
-    const uint32_t v_lane = (uint32_t)(((lpos ^ (4 * lrow)) << 4) + lrow * kRowBytes);
+    // (kPad: chunks past the end of a row in memory become chunk 0, rows are grow bytes apart)
+    auto mem_chunk = [&](int chunk) __attribute__((always_inline)) { return kPad ? (chunk < head_chunks ? chunk : 0) : chunk; };
+    const int k_chunk0 = lpos ^ lrow ^ (8 * (wave & 1)), v_chunk0 = lpos ^ (4 * lrow);
+    const uint32_t k_lane = (uint32_t)((mem_chunk(k_chunk0) << 4) + lrow * grow);
+    const uint32_t v_lane = (uint32_t)((mem_chunk(v_chunk0) << 4) + lrow * grow);
+    // the second instruction of a wavefront's eight rows (four rows further on: K's chunk index has bit 2 flipped)
+    const uint32_t k_lane1 = kPad ? (uint32_t)((mem_chunk(k_chunk0 ^ 4) << 4) + (lrow + 4) * grow) : (k_lane ^ 64u) + 4 * kRowBytes;
+    const uint32_t v_lane1 = v_lane + 4 * grow;
     lds_byte* const k_ring = lds;
     lds_byte* const v_ring = lds + kStages * kKBytes;
     // this wavefront's rows of tile j into `stage`; returns the number of instructions issued
@@ -703,18 +722,22 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         lds_byte* const dst = stage + 8 * wave * kRowBytes;
         const int key0 = kv_lo + j * kTileK + 8 * wave;
         if (key0 + 8 <= t.kv_len) {
-            const uint8_t* gb = row_group_base(t, base, key0, entry);
+            const uint8_t* gb = row_group_base(t, base, key0, entry, grow);
 #pragma unroll
             for (int k = 0; k < 2; k++) {
-                const uint32_t off = (is_k ? (k_lane ^ (uint32_t)(k << 6)) : v_lane) + (uint32_t)(4 * k * kRowBytes);
+                uint32_t off;
+                if constexpr (kPad)
+                    off = (is_k ? (k ? k_lane1 : k_lane) : (k ? v_lane1 : v_lane));
+                else
+                    off = (is_k ? (k_lane ^ (uint32_t)(k << 6)) : v_lane) + (uint32_t)(4 * k * kRowBytes);
                 load_to_lds_16(gb, off, dst + 4 * k * kRowBytes);
             }
         } else {  // the rows at the end of the sequence: per-lane clamped
 #pragma unroll
             for (int k = 0; k < 2; k++) {
                 const int r = 8 * (wave & 1) + 4 * k + lrow;
-                const int chunk = is_k ? (lpos ^ r) : (lpos ^ (4 * lrow));
-                const int64_t off = kv_row_offset(t, key0 + 4 * k + lrow) + (chunk << 4);
+                const int chunk = mem_chunk(is_k ? (lpos ^ r) : (lpos ^ (4 * lrow)));
+                const int64_t off = kv_row_offset(t, key0 + 4 * k + lrow, grow) + (chunk << 4);
                 load_to_lds_16(base + off, dst + 4 * k * kRowBytes);
             }
         }
@@ -832,12 +855,11 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     int fast_tiles = 0;
     const uint8_t* fill_k = nullptr;
     const uint8_t* fill_v = nullptr;
-    const uint32_t k_lane1 = (k_lane ^ 64u) + 4 * kRowBytes, v_lane1 = v_lane + 4 * kRowBytes;
     if constexpr (!kPaged) {
         const int room = t.kv_len - kv_lo - 8 * wave - 8;
         fast_tiles = room >= 0 ? min(n, room / kTileK + 1) : 0;
-        fill_k = t.k + (int64_t)(kv_lo + (group + 2) * kTileK + 8 * wave) * kRowBytes;
-        fill_v = t.v + (int64_t)(kv_lo + (group + 1) * kTileK + 8 * wave) * kRowBytes;
+        fill_k = t.k + (int64_t)(kv_lo + (group + 2) * kTileK + 8 * wave) * grow;
+        fill_v = t.v + (int64_t)(kv_lo + (group + 1) * kTileK + 8 * wave) * grow;
     }
 
     // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
@@ -871,7 +893,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             raw[i] = uint4_t{0u, 0u, 0u, 0u};
-            if (t.rows > 0) raw[i] = *(const lds_uint4*)(wave_stage + (f.k ^ (i << 5)));
+            if (t.rows > 0 && (!kPad || 2 * i + hi < head_chunks)) raw[i] = *(const lds_uint4*)(wave_stage + (f.k ^ (i << 5)));
         }
         if (t.q_dtype == HIPATTN_BF16) {  // (one wave-uniform branch, not a choice per element)
 #pragma unroll
@@ -972,8 +994,8 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             entry_k = table_entry(j + group + 3);
         }
         if constexpr (!kPaged) {
-            fill_k += kTileK * kRowBytes;
-            fill_v += kTileK * kRowBytes;
+            fill_k += kTileK * grow;
+            fill_v += kTileK * grow;
             asm volatile("" : "+s"(fill_k), "+s"(fill_v));
         }
         asm volatile("" : "+s"(i_kn), "+s"(i_vc), "+s"(i_kf), "+s"(i_vf));
@@ -1016,7 +1038,9 @@ __device__ __forceinline__ int small_div(int a, int b) {
     q -= (r < 0) ? 1 : 0;
     return q;
 }
+template <bool kPad = false>
 __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) {
+    const int D = kPad ? p.head_dim : kD;
     const int G = small_div(p.num_heads_q, p.num_heads_kv);
     const int n_qt = (p.len_q + kTileQ - 1) / kTileQ;
     const bool pair_heads = (G & 1) == 0;
@@ -1031,11 +1055,12 @@ __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) 
     const int h = hkv * G + (pair_heads ? 2 * li + group : li);
     const int qt = pair_heads ? slot : 2 * slot + group;
     Tile t;
-    const int64_t qoff = (((int64_t)b * p.num_heads_q + h) * p.len_q + (int64_t)min(qt, n_qt - 1) * kTileQ) * kD;
+    const int64_t qoff = (((int64_t)b * p.num_heads_q + h) * p.len_q + (int64_t)min(qt, n_qt - 1) * kTileQ) * D;
     t.q = (const uint16_t*)p.q + qoff;
-    t.q_stride = kD;
+    t.q_stride = D;
     t.out = (uint16_t*)p.out + qoff;
-    t.out_stride = kD;
+    t.out_stride = D;
+    t.head_dim = D;
     t.rows = qt < n_qt ? min(kTileQ, p.len_q - qt * kTileQ) : 0;
     t.pos0 = qt * kTileQ;
     t.kv_len = p.len_kv;
@@ -1043,7 +1068,7 @@ __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) 
     t.window = 0;
     t.q_dtype = p.dtype;
     t.out_dtype = p.dtype;
-    const int64_t kvoff = ((int64_t)b * p.num_heads_kv + hkv) * p.len_kv * (kD * 2);
+    const int64_t kvoff = ((int64_t)b * p.num_heads_kv + hkv) * p.len_kv * (D * 2);
     t.k = (const uint8_t*)p.k + kvoff;
     t.v = (const uint8_t*)p.v + kvoff;
     t.table = nullptr;
@@ -1063,7 +1088,7 @@ __device__ __forceinline__ Tile sdpa_group_tile(const SdpaParams& p, int group) 
     return t;
 }
 
-template <bool kBf16, bool kU8 = false, bool kPaged = true, int kMask = 0>
+template <bool kBf16, bool kU8 = false, bool kPaged = true, int kMask = 0, bool kPad = false>
 __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t* lds, float scale) {
     int lo0, hi0, lo1, hi1;
     key_range(t0, lo0, hi0);
@@ -1080,7 +1105,7 @@ __device__ __forceinline__ void run_both(const Tile& t0, const Tile& t1, uint8_t
         kv_hi = max(hi0, hi1);
     }
     const int group = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
-    run_pair<kBf16, kU8, kPaged, kMask>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
+    run_pair<kBf16, kU8, kPaged, kMask, kPad>(group ? t1 : t0, kv_lo, kv_hi, lds, scale);
 }
 
 template <bool kBf16>
@@ -1088,6 +1113,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
     const Tile t0 = sdpa_group_tile(p, 0), t1 = sdpa_group_tile(p, 1);
     run_both<kBf16, false, false>(t0, t1, lds, p.scale);
+}
+
+// The same for a head size between 64 and 128 (p.head_dim, a multiple of 8): the kPad form of the loop.
+template <bool kBf16>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_padded_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
+    const Tile t0 = sdpa_group_tile<true>(p, 0), t1 = sdpa_group_tile<true>(p, 1);
+    run_both<kBf16, false, false, 0, true>(t0, t1, lds, p.scale);
 }
 
 // The same with an attention mask (kMask 2: of the operands' type, added; 1: boolean bytes).
@@ -1100,7 +1133,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 // One workgroup per (128-row query tile of a multi-token sequence, pair of query heads) or, with an
 // odd number of query heads per kv head, per (pair of query tiles, query head).
+template <bool kPad = false>
 __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, int qt, int h, bool has_work) {
+    const int D = kPad ? p.head_dim : kD;
     const int G = p.num_heads_q / p.num_heads_kv;
     const int t0 = p.subsequence_begins[s];
     const int qlen = p.subsequence_begins[s + 1] - t0;
@@ -1109,10 +1144,10 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
     const int table_len = p.block_indices_begins[s + 1] - tb0;
     Tile t;
     const int64_t row0 = (int64_t)(t0 + qt * kTileQ) * p.num_heads_q + h;
-    t.q = (const uint16_t*)p.q + row0 * kD;
-    t.q_stride = (int64_t)p.num_heads_q * kD;
-    t.out = (p.out_dtype == HIPATTN_F32) ? (void*)((float*)p.out + row0 * kD) : (void*)((uint16_t*)p.out + row0 * kD);
-    t.out_stride = (int64_t)p.num_heads_q * kD;
+    t.q = (const uint16_t*)p.q + row0 * D;
+    t.q_stride = (int64_t)p.num_heads_q * D;
+    t.out = (p.out_dtype == HIPATTN_F32) ? (void*)((float*)p.out + row0 * D) : (void*)((uint16_t*)p.out + row0 * D);
+    t.out_stride = (int64_t)p.num_heads_q * D;
     t.rows = has_work ? min(kTileQ, qlen - qt * kTileQ) : 0;
     t.pos0 = past + qt * kTileQ;
     t.kv_len = min(past + qlen, table_len * p.block_size);
@@ -1120,7 +1155,8 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
     t.window = p.sliding_window;
     t.q_dtype = p.q_dtype;
     t.out_dtype = p.out_dtype;
-    const int row_bytes = p.cache_dtype == HIPATTN_U8 ? kU8RowBytes : kD * 2;
+    t.head_dim = D;
+    const int row_bytes = p.cache_dtype == HIPATTN_U8 ? kU8RowBytes : D * 2;
     const int64_t head_off = (int64_t)(h / G) * p.block_size * row_bytes;
     t.k = p.key_cache + head_off;
     t.v = p.value_cache + head_off;
@@ -1135,7 +1171,8 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
     return t;
 }
 
-template <bool kBf16, bool kU8>
+// kPad: a head size between 64 and 128 (p.head_dim, a multiple of 8; 16-bit caches).
+template <bool kBf16, bool kU8, bool kPad = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
     // Launch index -> work item.  The workgroups that run on one XCD at a time should share K/V in
@@ -1176,15 +1213,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     // of query heads per kv head, two consecutive query tiles of one head: the item of the even
     // tile does both, the item of the odd tile has nothing left to do.
     if (!pair_heads && (qt & 1)) return;
-    const Tile t0 = paged_group_tile(p, s, qt, h0, true);
-    const Tile t1 = pair_heads ? paged_group_tile(p, s, qt, h0 + 1, true) : paged_group_tile(p, s, qt + 1, h0, qt + 1 < tiles_s);
-    run_both<kBf16, kU8>(t0, t1, lds, p.scale);
+    const Tile t0 = paged_group_tile<kPad>(p, s, qt, h0, true);
+    const Tile t1 = pair_heads ? paged_group_tile<kPad>(p, s, qt, h0 + 1, true) : paged_group_tile<kPad>(p, s, qt + 1, h0, qt + 1 < tiles_s);
+    run_both<kBf16, kU8, true, 0, kPad>(t0, t1, lds, p.scale);
 }
 
 }  // namespace flash
 
+// Head size 128, and -- without a mask -- the head sizes between 64 and 128 that are multiples of 8, which run
+// the same kernel with rows of fewer columns in memory (16-byte aligned operands).
 bool sdpa_flash_supported(const SdpaParams& p) {
-    if (p.head_dim != flash::kD || !(p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16)) return false;
+    if (!(p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16)) return false;
+    if (p.head_dim != flash::kD) {
+        const auto aligned16 = [](const void* q) { return ((uintptr_t)q & 15) == 0; };
+        if (p.head_dim <= 64 || p.head_dim > flash::kD || p.head_dim % 8 != 0 || p.mask != nullptr) return false;
+        if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.out)) return false;
+    }
     // the kernel decodes its launch index with small_div: the number of workgroups must stay below 2^22
     const int64_t q_tiles = ((int64_t)p.len_q + flash::kTileQ - 1) / flash::kTileQ;
     return (int64_t)p.batch * p.num_heads_q * q_tiles < (int64_t(1) << 22);
@@ -1214,14 +1258,18 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     const int mask = p.mask == nullptr ? 0 : (p.mask_dtype == HIPATTN_U8 ? 1 : 2);
     if (p.dtype == HIPATTN_BF16) {
-        if (mask == 0)
+        if (p.head_dim != flash::kD)
+            hipLaunchKernelGGL(flash::sdpa_flash_padded_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
+        else if (mask == 0)
             hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
         else if (mask == 2)
             hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 2>), grid, dim3(flash::kThreads), 0, stream, p);
         else
             hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 1>), grid, dim3(flash::kThreads), 0, stream, p);
     } else {
-        if (mask == 0)
+        if (p.head_dim != flash::kD)
+            hipLaunchKernelGGL(flash::sdpa_flash_padded_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
+        else if (mask == 0)
             hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
         else if (mask == 2)
             hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<false, 2>), grid, dim3(flash::kThreads), 0, stream, p);
@@ -1234,10 +1282,18 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
 }
 
 hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
-    if (p.head_dim != flash::kD) return launch_paged_prefill_small(p, stream);  // the plain kernel, padded columns
+    // the head sizes between 64 and 128 of a 16-bit cache: this kernel on rows of fewer columns
+    const bool padded = p.head_dim > 64 && p.head_dim < flash::kD && p.head_dim % 8 == 0 && p.cache_dtype != HIPATTN_U8 &&
+                        (((uintptr_t)p.q | (uintptr_t)p.key_cache | (uintptr_t)p.value_cache | (uintptr_t)p.out) & 15) == 0;
+    if (p.head_dim != flash::kD && !padded) return launch_paged_prefill_small(p, stream);  // the plain kernel, padded columns
     const int G = p.num_heads_q / p.num_heads_kv;
     dim3 grid((unsigned)((int64_t)p.max_q_tiles * ((G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q)));
-    if (p.cache_dtype == HIPATTN_BF16)
+    if (padded) {
+        if (p.cache_dtype == HIPATTN_BF16)
+            hipLaunchKernelGGL((flash::paged_prefill_kernel<true, false, true>), grid, dim3(flash::kThreads), 0, stream, p);
+        else
+            hipLaunchKernelGGL((flash::paged_prefill_kernel<false, false, true>), grid, dim3(flash::kThreads), 0, stream, p);
+    } else if (p.cache_dtype == HIPATTN_BF16)
         hipLaunchKernelGGL((flash::paged_prefill_kernel<true, false>), grid, dim3(flash::kThreads), 0, stream, p);
     else if (p.cache_dtype == HIPATTN_U8)
         hipLaunchKernelGGL((flash::paged_prefill_kernel<false, true>), grid, dim3(flash::kThreads), 0, stream, p);

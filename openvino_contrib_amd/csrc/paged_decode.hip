@@ -748,13 +748,14 @@ constexpr int kSelfPlanMaxRows = 256;
 // unit's whole register file: `gridDim.x` workgroups then keep exactly that many compute units and
 // leave the others free for a kernel that runs beside this one.
 // kHD, kBlk: head size (128 or 64) and cache block size (32, 16, or 0: a larger power of two); the self-planning form and the
-// eight-wavefront form exist for head size 128 only, the self-planning form on blocks of 32 or 16 only.
+// eight-wavefront form exist for head size 128 only (the eight-wavefront form also for 16-bit caches at the
+// head sizes between 64 and 128, kPad), the self-planning form on blocks of 32 or 16 only.
 // kPad: the call's head size (p.head_dim, a multiple of 8) may be smaller than kHD: the missing columns of
 // Q are zeros and those of V are not read.
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
-    static_assert(!kPad || (!kSelfPlan && kWaves == 1), "padded head sizes: the ordinary launch");
+    static_assert(!kPad || (!kSelfPlan && (kWaves == 1 || (kHD == 128 && !kU8))), "padded head sizes: no self-planning form; eight wavefronts for 16-bit caches in the head-128 build");
     static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
     static_assert((kHD == 64 || kHD == 128) && (kBlk == 16 || kBlk == 32 || kBlk == 0), "head size 64 or 128, blocks of 16, 32 or more");
     // kBlk == 0: any larger power of two (p.block_size); a block then holds several units, one after the other
@@ -1662,7 +1663,8 @@ static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p
 
 static bool overlap_wanted(const PagedParams& p) {
     if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
-    if (p.head_dim != kD) return false;  // other head sizes have no eight-wavefront decode kernel
+    // the eight-wavefront decode kernel: head size 128, and 16-bit caches at the head sizes between 64 and 128
+    if (p.head_dim != kD && !(p.head_dim > 64 && p.head_dim < kD && p.cache_dtype != HIPATTN_U8)) return false;
     return option(kOptMixedOverlap) != 0;
 }
 
@@ -1869,6 +1871,11 @@ static void launch_decode(const PagedParams& p, const KvWriteParams& wp, int do_
             launch_decode_blk<false, true, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
         else
             launch_decode_blk<false, false, kWaves, kSelfPlan, 128, false>(p, wp, do_write, grid, block, stream);
+    } else if constexpr (kWaves == 8) {  // (overlap_wanted: 16-bit caches at head sizes between 64 and 128)
+        if (bf16)
+            launch_decode_blk<false, true, 8, false, 128, true>(p, wp, do_write, grid, block, stream);
+        else
+            launch_decode_blk<false, false, 8, false, 128, true>(p, wp, do_write, grid, block, stream);
     } else if constexpr (kWaves == 1 && !kSelfPlan) {
         if (p.head_dim > 128) {
             if (p.head_dim == 256) {

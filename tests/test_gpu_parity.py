@@ -112,19 +112,21 @@ def test_sdpa_small_shapes(hip, oracle, shape, causal, dtype):
     out, path = H.run_sdpa(hip, case, causal)
     ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
     # 16-bit operands with head sizes up to 256 run on the matrix cores (zero-padded to the 64, 128 or
-    # 256 the kernel is built for); fp32 takes the fp32 kernel
-    assert path == ("sdpa_generic" if dtype == W.F32 else ("sdpa_flash_mfma_d64" if D == 64 else "sdpa_flash_mfma_small"))
+    # 256 the kernel is built for; between 64 and 128 the tuned head-128 kernel); fp32 takes the fp32 kernel
+    assert path == ("sdpa_generic" if dtype == W.F32 else H.sdpa_matrix_core_path(D, masked=False))
     assert H.max_abs(out, ref) <= TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [W.F16, W.BF16])
-@pytest.mark.parametrize("D", [8, 32, 40, 80, 96, 112, 120, 136, 192, 256])
+@pytest.mark.parametrize("D", [8, 32, 40, 72, 80, 96, 104, 112, 120, 136, 192, 256])
 @pytest.mark.parametrize("B,Hq,Hkv,Lq,Lk,causal,masked", [(1, 4, 2, 130, 130, True, False), (2, 3, 1, 77, 300, False, False),
                                                           (1, 2, 2, 300, 515, False, True), (1, 6, 2, 1, 1000, False, True),
-                                                          (2, 2, 1, 257, 64, True, False)])
+                                                          (2, 2, 1, 257, 64, True, False), (2, 8, 2, 1024, 1024, True, False),
+                                                          (1, 5, 5, 700, 900, False, False)])
 def test_sdpa_other_head_sizes_on_the_matrix_cores(hip, oracle, dtype, D, B, Hq, Hkv, Lq, Lk, causal, masked):
     """Head sizes that are multiples of 8, up to 256: the head-64 / head-128 / head-256 builds of the
-    plain matrix-core kernel with the missing columns as zeros, with and without an fp32 attention mask."""
+    plain matrix-core kernel with the missing columns as zeros, with and without an fp32 attention mask;
+    without a mask the head sizes between 64 and 128 run the tuned head-128 kernel on rows of fewer columns."""
     announce("sdpa other head sizes", dtype, D, B, Hq, Hkv, Lq, Lk, causal, masked)
     case = W.make_sdpa_case(64, B, Hq, Hkv, Lq, Lk, D, dtype, std=0.5 if dtype == W.BF16 else 1.0)
     if masked:
@@ -136,7 +138,7 @@ def test_sdpa_other_head_sizes_on_the_matrix_cores(hip, oracle, dtype, D, B, Hq,
     else:
         out, path = H.run_sdpa(hip, case, causal)
         ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
-    assert path == "sdpa_flash_mfma_small"
+    assert path == H.sdpa_matrix_core_path(D, masked)
     assert np.isfinite(out).all()
     assert H.scaled_bound_error(out, ref, "sdpa other head sizes") <= TOL[dtype]
 
