@@ -1172,9 +1172,8 @@ __device__ __forceinline__ Tile paged_group_tile(const PagedParams& p, int s, in
 }
 
 // kPad: a head size between 64 and 128 (p.head_dim, a multiple of 8; 16-bit caches).
-template <bool kBf16, bool kU8, bool kPad = false>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
+template <bool kBf16, bool kU8, bool kPad>
+__device__ __forceinline__ void paged_prefill_item(const PagedParams& p, uint8_t* lds) {
     // Launch index -> work item.  The workgroups that run on one XCD at a time should share K/V in
     // its L2, and the XCDs should get equal work although sequences differ in length.  With a
     // multiple of eight kv heads, XCD x (launch index modulo 8) takes kv heads x, x + 8, ... of
@@ -1216,6 +1215,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const Tile t0 = paged_group_tile<kPad>(p, s, qt, h0, true);
     const Tile t1 = pair_heads ? paged_group_tile<kPad>(p, s, qt, h0 + 1, true) : paged_group_tile<kPad>(p, s, qt + 1, h0, qt + 1 < tiles_s);
     run_both<kBf16, kU8, true, 0, kPad>(t0, t1, lds, p.scale);
+}
+
+template <bool kBf16, bool kU8>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_kernel(PagedParams p) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
+    paged_prefill_item<kBf16, kU8, false>(p, lds);
+}
+
+// The same for a head size between 64 and 128 (16-bit caches): the kPad form of the loop.
+template <bool kBf16>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_padded_kernel(PagedParams p) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
+    paged_prefill_item<kBf16, false, true>(p, lds);
 }
 
 }  // namespace flash
@@ -1290,9 +1302,9 @@ hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
     dim3 grid((unsigned)((int64_t)p.max_q_tiles * ((G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q)));
     if (padded) {
         if (p.cache_dtype == HIPATTN_BF16)
-            hipLaunchKernelGGL((flash::paged_prefill_kernel<true, false, true>), grid, dim3(flash::kThreads), 0, stream, p);
+            hipLaunchKernelGGL(flash::paged_prefill_padded_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
         else
-            hipLaunchKernelGGL((flash::paged_prefill_kernel<false, false, true>), grid, dim3(flash::kThreads), 0, stream, p);
+            hipLaunchKernelGGL(flash::paged_prefill_padded_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
     } else if (p.cache_dtype == HIPATTN_BF16)
         hipLaunchKernelGGL((flash::paged_prefill_kernel<true, false>), grid, dim3(flash::kThreads), 0, stream, p);
     else if (p.cache_dtype == HIPATTN_U8)
