@@ -621,7 +621,7 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is ev
 // read in phase 2j+1.  Between the barriers each group runs one matrix and one vector phase, in
 // opposite order, so that the matrix core and the vector units are both in use; the odd phase
 // boundaries are not enforced, the two groups only drift by what their phases differ in length.
-// kPad (16-bit K/V, no mask): the rows of Q, K, V and the output have t.head_dim < kD columns in memory (a
+// kPad (16-bit K/V): the rows of Q, K, V and the output have t.head_dim < kD columns in memory (a
 // multiple of 8).  Everything in LDS and in registers keeps the layout of kD columns: a lane whose 16-byte
 // chunk of a row does not exist fetches the row's first chunk instead -- valid, finite data that only
 // ever meets the zeros the query fragments hold in those columns, or lands in output columns that
@@ -629,7 +629,7 @@ __device__ __forceinline__ void barrier_keeping_loads(int keep) {  // keep is ev
 template <bool kBf16, bool kU8 = false, bool kPaged = true, int kMask = 0, bool kPad = false>
 __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, uint8_t* lds_generic, float scale) {
     static_assert(kPaged || !kU8, "dense K/V are 16-bit");
-    static_assert(!kPad || (!kU8 && kMask == 0), "smaller head sizes: 16-bit K/V, no mask");
+    static_assert(!kPad || !kU8, "smaller head sizes: 16-bit K/V");
     const int grow = kPad ? 2 * t.head_dim : kRowBytes;  // bytes from row to row in memory
     const int head_chunks = kPad ? t.head_dim >> 3 : kD / 8;
     static_assert(kMask == 0 || !kPaged, "attention masks belong to the dense operator");
@@ -1131,6 +1131,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     run_both<kBf16, false, false, kMask>(t0, t1, lds, p.scale);
 }
 
+// ... and for a head size between 64 and 128.
+template <bool kBf16, int kMask>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_flash_masked_padded_kernel(SdpaParams p) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
+    const Tile t0 = sdpa_group_tile<true>(p, 0), t1 = sdpa_group_tile<true>(p, 1);
+    run_both<kBf16, false, false, kMask, true>(t0, t1, lds, p.scale);
+}
+
 // One workgroup per (128-row query tile of a multi-token sequence, pair of query heads) or, with an
 // odd number of query heads per kv head, per (pair of query tiles, query head).
 template <bool kPad = false>
@@ -1232,13 +1240,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 }  // namespace flash
 
-// Head size 128, and -- without a mask -- the head sizes between 64 and 128 that are multiples of 8, which run
-// the same kernel with rows of fewer columns in memory (16-byte aligned operands).
+// Head size 128, and the head sizes between 64 and 128 that are multiples of 8, which run the same kernel with
+// rows of fewer columns in memory (16-byte aligned operands).
 bool sdpa_flash_supported(const SdpaParams& p) {
     if (!(p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16)) return false;
     if (p.head_dim != flash::kD) {
         const auto aligned16 = [](const void* q) { return ((uintptr_t)q & 15) == 0; };
-        if (p.head_dim <= 64 || p.head_dim > flash::kD || p.head_dim % 8 != 0 || p.mask != nullptr) return false;
+        if (p.head_dim <= 64 || p.head_dim > flash::kD || p.head_dim % 8 != 0) return false;
         if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.out)) return false;
     }
     // the kernel decodes its launch index with small_div: the number of workgroups must stay below 2^22
@@ -1269,24 +1277,37 @@ hipError_t launch_sdpa_flash(const SdpaParams& p, hipStream_t stream, const Kern
     dim3 grid(per_kv_head * p.num_heads_kv * p.batch);
     if (probe.before) (void)hipEventRecord(probe.before, stream);
     const int mask = p.mask == nullptr ? 0 : (p.mask_dtype == HIPATTN_U8 ? 1 : 2);
-    if (p.dtype == HIPATTN_BF16) {
-        if (p.head_dim != flash::kD)
-            hipLaunchKernelGGL(flash::sdpa_flash_padded_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
-        else if (mask == 0)
-            hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, dim3(flash::kThreads), 0, stream, p);
+    const dim3 block(flash::kThreads);
+    if (p.head_dim != flash::kD) {  // (the kPad forms)
+        if (p.dtype == HIPATTN_BF16) {
+            if (mask == 0)
+                hipLaunchKernelGGL(flash::sdpa_flash_padded_kernel<true>, grid, block, 0, stream, p);
+            else if (mask == 2)
+                hipLaunchKernelGGL((flash::sdpa_flash_masked_padded_kernel<true, 2>), grid, block, 0, stream, p);
+            else
+                hipLaunchKernelGGL((flash::sdpa_flash_masked_padded_kernel<true, 1>), grid, block, 0, stream, p);
+        } else {
+            if (mask == 0)
+                hipLaunchKernelGGL(flash::sdpa_flash_padded_kernel<false>, grid, block, 0, stream, p);
+            else if (mask == 2)
+                hipLaunchKernelGGL((flash::sdpa_flash_masked_padded_kernel<false, 2>), grid, block, 0, stream, p);
+            else
+                hipLaunchKernelGGL((flash::sdpa_flash_masked_padded_kernel<false, 1>), grid, block, 0, stream, p);
+        }
+    } else if (p.dtype == HIPATTN_BF16) {
+        if (mask == 0)
+            hipLaunchKernelGGL(flash::sdpa_flash_kernel<true>, grid, block, 0, stream, p);
         else if (mask == 2)
-            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 2>), grid, dim3(flash::kThreads), 0, stream, p);
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 2>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 1>), grid, dim3(flash::kThreads), 0, stream, p);
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<true, 1>), grid, block, 0, stream, p);
     } else {
-        if (p.head_dim != flash::kD)
-            hipLaunchKernelGGL(flash::sdpa_flash_padded_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
-        else if (mask == 0)
-            hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, dim3(flash::kThreads), 0, stream, p);
+        if (mask == 0)
+            hipLaunchKernelGGL(flash::sdpa_flash_kernel<false>, grid, block, 0, stream, p);
         else if (mask == 2)
-            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<false, 2>), grid, dim3(flash::kThreads), 0, stream, p);
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<false, 2>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<false, 1>), grid, dim3(flash::kThreads), 0, stream, p);
+            hipLaunchKernelGGL((flash::sdpa_flash_masked_kernel<false, 1>), grid, block, 0, stream, p);
     }
     hipError_t e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);

@@ -314,18 +314,20 @@ def test_sdpa_with_attention_mask(hip, oracle, dtype, tol, mask_kind):
 FLASH_MASKS = ["full", "per_batch", "shared", "key_padding", "causal_inf", "bool_shared", "bool_per_batch", "bool_padding"]
 
 
+@pytest.mark.parametrize("D", [128, 96, 72])
 @pytest.mark.parametrize("dtype", [W.F16, W.BF16])
 @pytest.mark.parametrize("kind", FLASH_MASKS)
 @pytest.mark.parametrize("B,Hq,Hkv,Lq,Lk", [(2, 4, 2, 300, 512), (1, 3, 1, 130, 208), (2, 2, 2, 64, 1000), (1, 8, 2, 1000, 64),
                                             (1, 2, 1, 5, 48)])
-def test_sdpa_flash_with_mask(hip, oracle, dtype, kind, B, Hq, Hkv, Lq, Lk):
-    """Head size 128 with an attention mask of the operands' type or a boolean one stays on the matrix
-    cores: full, per-batch and shared masks, a key-padding mask (one row for all queries), an additive
-    triangle of -inf (how converted models spell causality), rows that are masked out altogether, and
-    key counts off the 64-key tile (the last tile's mask values are read one by one)."""
-    announce("sdpa flash mask", dtype, kind, B, Hq, Hkv, Lq, Lk)
+def test_sdpa_flash_with_mask(hip, oracle, dtype, kind, B, Hq, Hkv, Lq, Lk, D):
+    """Head size 128 -- and the head sizes between 64 and 128, on rows of fewer columns -- with an attention
+    mask of the operands' type or a boolean one stays in the tuned kernel: full, per-batch and shared masks,
+    a key-padding mask (one row for all queries), an additive triangle of -inf (how converted models spell
+    causality), rows that are masked out altogether, and key counts off the 64-key tile (the last tile's
+    mask values are read one by one)."""
+    announce("sdpa flash mask", dtype, kind, B, Hq, Hkv, Lq, Lk, D)
     rng = np.random.default_rng(Lq * 7 + Lk + len(kind))
-    case = W.make_sdpa_case(71, B, Hq, Hkv, Lq, Lk, 128, dtype, std=0.5 if dtype == W.BF16 else 1.0)
+    case = W.make_sdpa_case(71, B, Hq, Hkv, Lq, Lk, D, dtype, std=0.5 if dtype == W.BF16 else 1.0)
     shape = {"full": (B, Hq, Lq, Lk), "per_batch": (B, 1, Lq, Lk), "shared": (Lq, Lk), "key_padding": (B, 1, 1, Lk),
              "causal_inf": (1, 1, Lq, Lk), "bool_shared": (Lq, Lk), "bool_per_batch": (B, 1, Lq, Lk), "bool_padding": (B, 1, 1, Lk)}[kind]
     if kind.startswith("bool"):
