@@ -146,7 +146,7 @@ hipattn_status hipattn_sdpa(const hipattn_sdpa_desc* desc, const void* q, const 
  * scaled score; dtype U8: boolean, nonzero = the key takes part, zero = probability zero.  As the
  * operator specifies, the mask is ignored when desc->causal is set.  A query row whose keys are
  * all masked out yields zeros.  mask_desc and mask are both NULL or both set.
- * At head_dim 128 (and at the multiples of 8 between 64 and 128) a mask of the operands' 16-bit type, or a boolean one, whose keys lie side by
+ * At head_dim 128 (and at the multiples of 8 below it) a mask of the operands' 16-bit type, or a boolean one, whose keys lie side by
  * side (stride[3] == 1) rides along in the tuned matrix-core kernel when the mask pointer and the
  * other strides are multiples of 16 bytes (8 elements; 16 for boolean); every other mask beside
  * 16-bit operands with a head_dim that is a multiple of 8 up to 256 takes the plain matrix-core
@@ -306,6 +306,8 @@ hipattn_status hipattn_profile_dominant_kernel(hipattn_event before, hipattn_eve
  *                                 work is cut into equal pieces (5)
  *   "decode_dyn_pieces_per_wave"  on-demand pieces per wavefront for the last quarter of the
  *                                 decode work (0 = none)
+ *   "sdpa_padded_rows"            1 (default): dense SDPA at head sizes below 128 (multiples of 8) runs the
+ *                                 tuned head-128 kernel on rows of fewer columns; 0: the plain kernels
  * HIPATTN_<NAME IN CAPITALS> in the environment gives an option its initial value; the
  * environment is read once per process. */
 hipattn_status hipattn_set_option(const char* name, int value);

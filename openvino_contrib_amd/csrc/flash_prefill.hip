@@ -1240,13 +1240,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 }  // namespace flash
 
-// Head size 128, and the head sizes between 64 and 128 that are multiples of 8, which run the same kernel with
-// rows of fewer columns in memory (16-byte aligned operands).
+// Head size 128, and the smaller head sizes that are multiples of 8, which run the same kernel with rows of
+// fewer columns in memory (16-byte aligned operands; the option sdpa_padded_rows = 0 leaves them to the
+// plain kernels).  Measured on 4 x 2,048 tokens, 32 / 8 heads, causal: head size 64 0.124 ms against 0.153 ms
+// in the plain head-64 kernel, head size 32 0.120 ms.
 bool sdpa_flash_supported(const SdpaParams& p) {
     if (!(p.dtype == HIPATTN_F16 || p.dtype == HIPATTN_BF16)) return false;
     if (p.head_dim != flash::kD) {
         const auto aligned16 = [](const void* q) { return ((uintptr_t)q & 15) == 0; };
-        if (p.head_dim <= 64 || p.head_dim > flash::kD || p.head_dim % 8 != 0) return false;
+        if (p.head_dim < 8 || p.head_dim > flash::kD || p.head_dim % 8 != 0 || !sdpa_padded_rows_enabled()) return false;
         if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.out)) return false;
     }
     // the kernel decodes its launch index with small_div: the number of workgroups must stay below 2^22

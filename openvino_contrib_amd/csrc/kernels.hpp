@@ -191,6 +191,7 @@ hipError_t launch_paged_scores(const ScoresParams& p, hipStream_t stream);
 
 // Schedule option by name (see paged_decode.hip); value < 0 restores the default.  false: no such option.
 bool set_option(const char* name, int value);
+bool sdpa_padded_rows_enabled();  // the option sdpa_padded_rows
 // Address and size of the current device's copy of the static scratch array (resolved once per device).
 hipError_t paged_static_scratch(void** ptr, size_t* bytes);
 

@@ -1586,8 +1586,10 @@ Option g_options[] = {
     {"decode_dyn_pieces_per_wave", "HIPATTN_DECODE_DYN_PIECES_PER_WAVE", 0, 0, 64, {0}},
     // scales the compute units the plan gives the decode part of a mixed batch (100 = as modelled)
     {"mixed_decode_share_percent", "HIPATTN_MIXED_DECODE_SHARE_PERCENT", 100, 10, 1000, {100}},
+    // 1: dense SDPA at head sizes below 128 runs the tuned head-128 kernel on rows of fewer columns; 0: the plain kernels
+    {"sdpa_padded_rows", "HIPATTN_SDPA_PADDED_ROWS", 1, 0, 1, {1}},
 };
-enum { kOptMixedOverlap = 0, kOptSwitchCost, kOptDynPieces, kOptSharePercent };
+enum { kOptMixedOverlap = 0, kOptSwitchCost, kOptDynPieces, kOptSharePercent, kOptSdpaPadded };
 
 void init_options_from_environment() {
     static std::once_flag once;
@@ -1601,6 +1603,8 @@ int option(int which) {
     return g_options[which].value.load(std::memory_order_relaxed);
 }
 }  // namespace
+
+bool sdpa_padded_rows_enabled() { return option(kOptSdpaPadded) != 0; }
 
 bool set_option(const char* name, int value) {
     init_options_from_environment();

@@ -48,8 +48,6 @@ def paged_matrix_core_path(Hq, Hkv, D, bs, cache_dtype):
 def sdpa_matrix_core_path(D, masked):
     """Kernel path of a dense SDPA call with 16-bit operands and a head size that is a multiple of 8 up to 256
     (masked: with an attention mask the tuned kernel's mask tiles do not take, or at another head size than 128)."""
-    if D == 128 and not masked:
-        return "sdpa_flash_mfma"
-    if 64 < D < 128 and not masked:
-        return "sdpa_flash_mfma"  # the tuned head-128 kernel on rows of fewer columns
+    if D <= 128 and not masked:
+        return "sdpa_flash_mfma"  # (below 128: the tuned head-128 kernel on rows of fewer columns)
     return "sdpa_flash_mfma_d64" if D == 64 else "sdpa_flash_mfma_small"

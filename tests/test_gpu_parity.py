@@ -141,6 +141,15 @@ def test_sdpa_other_head_sizes_on_the_matrix_cores(hip, oracle, dtype, D, B, Hq,
     assert path == H.sdpa_matrix_core_path(D, masked)
     assert np.isfinite(out).all()
     assert H.scaled_bound_error(out, ref, "sdpa other head sizes") <= TOL[dtype]
+    if not masked and D < 128:  # the plain kernels, which take these head sizes when the option says so
+        hip.set_option("sdpa_padded_rows", 0)
+        try:
+            out, path = H.run_sdpa(hip, case, causal)
+        finally:
+            hip.set_option("sdpa_padded_rows", -1)
+        assert path == "sdpa_flash_mfma_small"
+        assert np.isfinite(out).all()
+        assert H.scaled_bound_error(out, ref, "sdpa other head sizes, plain kernel") <= TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [W.F16, W.BF16])
@@ -152,14 +161,23 @@ def test_sdpa_other_head_sizes_on_the_matrix_cores(hip, oracle, dtype, D, B, Hq,
     ((2, 6, 3, 515, 515, 64), True), ((1, 2, 2, 77, 500, 64), True), ((1, 3, 1, 260, 700, 64), False),
     ((1, 2, 1, 1600, 1600, 64), True), ((3, 5, 5, 1, 700, 64), False)])
 def test_sdpa_flash_head_size_64(hip, oracle, dtype, shape, causal):
-    """Head size 64 runs on the matrix cores too (its own kernel): edge lengths either side of the
+    """Head size 64 runs on the matrix cores too -- by default in the tuned head-128 kernel on rows of 64
+    columns, with the option sdpa_padded_rows = 0 in the plain head-64 kernel: edge lengths either side of the
     64-key tile and the 128-row workgroup, GQA, rectangular shapes with the top-left aligned mask."""
     announce("sdpa flash d64", dtype, shape, causal)
     B, Hq, Hkv, Lq, Lk, D = shape
     case = W.make_sdpa_case(63, B, Hq, Hkv, Lq, Lk, D, dtype)
-    out, path = H.run_sdpa(hip, case, causal)
-    assert path == "sdpa_flash_mfma_d64"
     ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
+    out, path = H.run_sdpa(hip, case, causal)
+    assert path == "sdpa_flash_mfma"
+    assert np.isfinite(out).all()
+    assert H.max_abs(out, ref) <= TOL[dtype]
+    hip.set_option("sdpa_padded_rows", 0)
+    try:
+        out, path = H.run_sdpa(hip, case, causal)
+    finally:
+        hip.set_option("sdpa_padded_rows", -1)
+    assert path == "sdpa_flash_mfma_d64"
     assert np.isfinite(out).all()
     assert H.max_abs(out, ref) <= TOL[dtype]
     out2, _ = H.run_sdpa(hip, case, causal, scale=0.05)
@@ -249,7 +267,7 @@ def test_sdpa_head_size_64_scores_that_grow_along_the_keys(hip, oracle, dtype, p
         case[name + "_store"], case[name] = W.to_storage(x, dtype)
     for causal in (False, True):
         out, path = H.run_sdpa(hip, case, causal)
-        assert path == ("sdpa_generic" if dtype == W.F32 else "sdpa_flash_mfma_d64")  # fp16 at head size 64: the matrix-core kernel
+        assert path == ("sdpa_generic" if dtype == W.F32 else "sdpa_flash_mfma")  # 16-bit at head size 64: the tuned kernel on rows of 64 columns
         ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=causal)
         assert np.isfinite(out).all()
         assert H.scaled_bound_error(out, ref, "sdpa d64 %s dtype %d causal %d" % (profile, dtype, causal)) <= TOL[dtype]
@@ -381,7 +399,9 @@ def test_sdpa_d64_with_mask(hip, oracle, dtype, kind, B, Hq, Hkv, Lq, Lk):
     else:
         mask, mask_dtype = np.triu(np.full((Lq, Lk), -np.inf, np.float32), 1 + max(Lk - Lq, 0))[None, None], dtype
     out, path = H.run_sdpa_masked(hip, case, mask, mask_dtype=mask_dtype)
-    assert path == "sdpa_flash_mfma_d64"
+    # (a mask of the operands' type whose rows are whole 16-byte pieces rides along in the tuned kernel)
+    tuned = (mask_dtype == dtype and Lk % 8 == 0) or (mask.dtype == np.bool_ and Lk % 16 == 0)
+    assert path == ("sdpa_flash_mfma_masked" if tuned else "sdpa_flash_mfma_d64")
     ref = oracle.sdpa_masked(case["q"], case["k"], case["v"], mask if (mask.dtype == np.bool_ or mask_dtype is None) else oracle.round_to(mask, mask_dtype))
     assert np.isfinite(out).all()
     rows = np.isfinite(ref).all(-1)
