@@ -1,11 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer|shapes|decoder] [--no-cpu] [--no-extra] [--no-plugin]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer|shapes|decoder|scores|masked] [--no-cpu] [--no-extra] [--no-plugin]
 
-Prints ONE JSON line.  The headline is the fp16 paged-attention decode step (configuration 3, the
-one the headline metric is quoted on): a "step" is one hipattn_paged_attention call on the whole synthetic batch
-(KV-cache write of the new tokens + split-context decode + merge), inputs resident in HBM.
+The LAST stdout line is ONE compact JSON object (under 3 KB); the full per-workload records go to
+gpurun_out/bench_detail.json when that folder exists, to stderr otherwise.  The headline is the fp16
+paged-attention decode step (configuration 3, the one the headline metric is quoted on): a "step" is
+one hipattn_paged_attention call on the whole synthetic batch (KV-cache write of the new tokens +
+split-context decode + merge), inputs resident in HBM.
 `value` is algorithmic KV bytes / wall time of a step; `roofline` is the same byte count over
 the average duration of the dominant kernel (the split-context decode kernel), measured with
 HIP events recorded by the library around that launch.  Unless --no-extra is given, the other
@@ -14,9 +16,10 @@ configurations are measured the same way and reported under "workloads" in the s
 c5: mixed chunked prefill + decode), each with a `cpu_baseline` of its own.  `cpu_baseline` times
 the CPU oracle (a restatement, not OpenVINO's CPU plugin: OpenVINO is not installed) on a bounded
 sample of the same workload.  `plugin_ms_per_step` of the headline workload is the same step through
-the plugin layer's InferRequest::infer with device-resident tensors.  The operators around attention
-(RMS norm, RoPE, MatMul, Gather, Concat of libhipops.so) ride along under "workloads" too, or alone
-with --workload layer.
+the plugin layer's InferRequest::infer with device-resident tensors.  Everything that is not one of
+the four configurations runs only when asked for: --workload layer (the operators of libhipops.so),
+shapes (other cache shapes), decoder (a decoder layer through the plugin), scores (the operator's
+second output), masked (config 2's shape with the causality as an attention mask).
 """
 import argparse
 import json
@@ -81,7 +84,10 @@ def time_steps(hip, fn, steps, warmup):
     kern = [befores[i].elapsed_ms(afters[i]) for i in range(steps)]
     for e in befores + afters + [start, stop]:
         e.close()
-    return ev_ms, wall_ms, sum(kern) / len(kern)
+    # An event pair brackets the kernel plus the two record packets, so on a step that is one launch
+    # the probed figure can read a microsecond or two above the step itself; a kernel cannot take
+    # longer than the step it is part of, so the step time of the timed pass bounds it.
+    return ev_ms, wall_ms, min(sum(kern) / len(kern), ev_ms)
 
 
 def bench_paged(hip, case, steps, warmup, name):
@@ -326,8 +332,7 @@ def cpu_baseline_paged(case, budget_s=12.0):
     mean = sum(times) / len(times)
     return {"value": W.paged_kv_bytes(case) / mean / 1e9, "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
             "oracle": oracle_kind(),
-            "sample": "oracle paged attention (no cache write) on all %d sequences of the workload, mean of %d passes, "
-                      "%.1f s of CPU work" % (case["S"], len(times), sum(times))}
+            "sample": "all %d sequences, attention only, %d passes, %.1f s" % (case["S"], len(times), sum(times))}
 
 
 def cpu_baseline_sdpa(case, budget_s=20.0):
@@ -349,8 +354,7 @@ def cpu_baseline_sdpa(case, budget_s=20.0):
     fl = W.sdpa_flops(1, G, case["Lq"], case["Lk"], case["D"], True) * len(times)
     return {"value": fl / sum(times) / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
             "oracle": oracle_kind(),
-            "sample": "oracle fp32 SDPA on %d of %d (batch, kv head) groups of the workload, %.1f s of CPU work"
-                      % (len(times), case["B"] * case["Hkv"], sum(times))}
+            "sample": "%d of %d (batch, kv head) groups, %.1f s" % (len(times), case["B"] * case["Hkv"], sum(times))}
 
 
 def bench_layer_ops(hip, steps, warmup, with_cpu):
@@ -704,13 +708,40 @@ def bench_decoder_layer(hip, steps, warmup):
     return res
 
 
+def _r(x, digits=5):
+    """Floats to `digits` significant digits: the compact line is for a reader, the detail file keeps everything."""
+    return float("%.*g" % (digits, x)) if isinstance(x, float) else x
+
+
+def compact_roofline(r):
+    return {k: _r(r[k]) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel") if k in r}
+
+
+def compact_cpu(c):
+    return {k: _r(c[k]) for k in ("value", "unit", "cores", "kind", "sample") if k in c}
+
+
+def compact_workload(r):
+    """What the last stdout line carries per configuration (the whole record goes to stderr and the detail file)."""
+    out = {k: _r(r[k]) for k in ("ms_per_step", "dominant_kernel_ms", "kv_gbs", "tflops", "kernel_path", "ideal_ms",
+                                 "frac_of_ideal", "plugin_ms_per_step") if k in r}
+    if r.get("kernel_path", "").startswith("sdpa"):
+        out.pop("kv_gbs", None)
+    else:
+        out.pop("tflops", None)
+    out["roofline"] = compact_roofline(r["roofline"])
+    if "cpu_baseline" in r:
+        out["cpu_baseline"] = compact_cpu(r["cpu_baseline"])
+    return out
+
+
 def main():
     global CLOCK_RAMP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "decoder", "copy", "mfma"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "decoder", "scores", "masked", "copy", "mfma"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
                          "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
@@ -768,6 +799,15 @@ def main():
                           "workloads": bench_other_shapes(hip, args.steps, args.warmup)}))
         return
 
+    if args.workload == "scores":
+        r = bench_paged_scores(hip, W.config3(), args.steps, "config3's batch: the scores output (all heads, the new token of every sequence)")
+        print(json.dumps({"workload": "scores", "steps": args.steps, "workloads": {"c3_scores": r}}))
+        return
+
+    if args.workload == "masked":
+        print(json.dumps({"workload": "masked", "steps": args.steps, "workloads": {"c2_masked": bench_sdpa_masked(hip, args.steps)}}))
+        return
+
     if args.workload == "copy":
         # Known-size traffic for scaling FETCH_SIZE / WRITE_SIZE: a device-to-device copy of 1 GiB
         # (1 GiB read + 1 GiB written per launch) and a 1 GiB fill kernel (1 GiB written).
@@ -822,9 +862,6 @@ def main():
             r["plugin_overhead_ms"] = r["plugin_ms_per_step"] - r["ms_per_step"]
             log("%s through InferRequest::infer: %.3f ms/step (raw C ABI, back to back: %.3f)"
                 % (w, r["plugin_ms_per_step"], r["ms_per_step"]))
-        if w == "c3" and not args.no_extra:
-            results["c3_scores"] = bench_paged_scores(hip, case, args.steps, "config3's batch: the scores output (all heads, the new token of every sequence)")
-            log("c3 scores output: %.3f ms" % results["c3_scores"]["ms_per_step"])
         if not args.no_cpu:
             # the headline gets the larger budget; every other workload a bounded sample beside its figure
             budget = 12.0 if w == args.workload else 6.0
@@ -835,19 +872,6 @@ def main():
             log("%s cpu baseline:" % w, c)
         results[w] = r
         del case
-
-    if not args.no_extra:
-        results.update(bench_other_shapes(hip, args.steps, args.warmup))
-        if not args.no_plugin:
-            results["decoder_layer"] = bench_decoder_layer(hip, args.steps, args.warmup)
-            log("decoder layer on c3's batch through the plugin: %.3f ms/step, roofline frac %.3f (%d graph, %d launches)"
-                % (results["decoder_layer"]["ms_per_step"], results["decoder_layer"]["roofline"]["frac"],
-                   results["decoder_layer"]["graphs"], results["decoder_layer"]["graph_launches"]))
-        results["c2_masked"] = bench_sdpa_masked(hip, args.steps)
-        log("c2's shape with the causality as an attention mask: %.3f ms, %.0f TFLOP/s (%s)"
-            % (results["c2_masked"]["ms_per_step"], results["c2_masked"]["tflops"], results["c2_masked"]["kernel_path"]))
-        # the operators around attention, each with a roofline and a CPU figure of its own
-        results.update(bench_layer_ops(hip, args.steps, args.warmup, not args.no_cpu))
 
     head = results[args.workload]
     is_sdpa = args.workload == "c2"
@@ -862,11 +886,18 @@ def main():
         "config": {"workload": head["workload"], "kernel_path": head["kernel_path"],
                    "device": dev_name, "arch": info.arch.decode(), "compute_units": info.compute_units,
                    "clock_ramp_ms": CLOCK_RAMP_MS},
-        "roofline": head["roofline"],
-        "cpu_baseline": cpu if cpu else None,
-        "workloads": {k: v for k, v in results.items()},
+        "roofline": compact_roofline(head["roofline"]),
+        "cpu_baseline": compact_cpu(cpu) if cpu else None,
+        "workloads": {k: compact_workload(v) for k, v in results.items()},
     }
-    print(json.dumps(line))
+    detail = dict(line, roofline=head["roofline"], cpu_baseline=cpu if cpu else None, workloads=results)
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "bench_detail.json"), "w") as f:
+            json.dump(detail, f)
+    else:
+        log("detail:", json.dumps(detail))
+    print(json.dumps(line), flush=True)
 
 
 if __name__ == "__main__":
