@@ -306,6 +306,9 @@ hipattn_status hipattn_profile_dominant_kernel(hipattn_event before, hipattn_eve
  *                                 work is cut into equal pieces (5)
  *   "decode_dyn_pieces_per_wave"  on-demand pieces per wavefront for the last quarter of the
  *                                 decode work (0 = none)
+ *   "decode_fused_merge"          where pieces of several wavefronts make up one (sequence, kv head): 2: the
+ *                                 decode kernel combines them itself; 0: a merge launch behind it; 1 (default):
+ *                                 the kernel for u8 caches, the launch for 16-bit ones (whichever measured faster)
  *   "sdpa_padded_rows"            1 (default): dense SDPA at head sizes below 128 (multiples of 8) runs the
  *                                 tuned head-128 kernel on rows of fewer columns; 0: the plain kernels
  * HIPATTN_<NAME IN CAPITALS> in the environment gives an option its initial value; the

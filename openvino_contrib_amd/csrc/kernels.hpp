@@ -111,6 +111,11 @@ struct PagedParams {
     void* seq_info;       // [num_rows] 32-byte records: what each decode row attends (written by the plan)
     float* part_out;      // [num_waves + dyn_pieces + num_rows*num_heads_kv, G, head_dim] unnormalised outputs
     float* part_ml;       // [same, G, 2] running max (log2 domain) and sum
+    // fused_merge: the piece that holds the end of a segment combines the segment's partials inside the
+    // decode kernel (no merge launch); part_flag[slot] == merge_tag says that slot's partial is complete
+    int fused_merge;
+    uint64_t* part_flag;  // [same]
+    unsigned long long merge_tag;  // differs from call to call (and from whatever a fresh workspace holds)
     // chunked prefill: query-tile schedule built on the device
     int32_t* tile_prefix; // [num_seqs + 1] exclusive prefix of query tiles per sequence
     int max_q_tiles;      // grid upper bound

@@ -60,6 +60,7 @@
 // src/ops/softmax.cpp:184-192).
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -735,6 +736,128 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
     }
 }
 
+// ---- partial results that another wavefront of the same launch reads ------------------------
+// The compute units of the device sit behind eight L2 caches that are not kept coherent for
+// ordinary accesses.  Partials, and the flags that announce them, therefore go through agent-scope
+// relaxed atomic accesses (write-through stores, loads that do not take a stale line): no fence,
+// which would write back and invalidate whole L2 caches while the kernel streams through them.
+// Order is kept by hand: a producer waits for its stores (s_waitcnt vmcnt(0)) before it raises
+// the flag, a consumer reads the partial only after it has seen the flag.
+//
+// Layout of such a partial (fused_merge; the merge kernel's partials keep theirs): the wavefront that
+// combines has the lane layout of the one that produced, so a lane's 32 accumulator values and its
+// head's (max, sum) travel as seventeen pairs of floats, pair j of active lane a (a = kg * G + head,
+// 4 G of them) at pair index j * 4 G + a of the slot.  One store instruction then writes 4 G x 8
+// contiguous bytes -- whole cache lines from four query heads per kv head on -- which matters because a
+// write-through store of part of a line is a read-modify-write at the memory (4-byte stores, sixteen
+// lines per instruction, cost configuration 3's kernel 20 us).
+constexpr int kPartPairs = 17;  // per active lane: 16 pairs of outputs, then (max, sum)
+__device__ __forceinline__ void agent_store2(float* p, float x, float y) {
+    const unsigned long long v = (unsigned long long)__float_as_uint(x) | ((unsigned long long)__float_as_uint(y) << 32);
+    __hip_atomic_store((unsigned long long*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void agent_load2(const float* p, float& x, float& y) {
+    const unsigned long long v = __hip_atomic_load((const unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    x = __uint_as_float((uint32_t)v);
+    y = __uint_as_float((uint32_t)(v >> 32));
+}
+__device__ __forceinline__ void stores_done() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// The wavefront that holds the LAST units of a segment which other pieces worked on too combines
+// the partials of all of them (its own among them, left in the workspace like the others) when its
+// own piece is done: a piece meets such a segment only as the first of its run, so it has at most
+// one to combine, and the pieces it waits for have lower numbers, i.e. were dispatched before it.
+// Lane (head n16, kg) owns head-dim (kg*4 + r)*8 + e of its head, as in the accumulators.
+// Waiting is bounded (kMergeSpinLimit polls of about a microsecond each): a flag that never comes --
+// which a consistent plan cannot produce -- leaves the rows unwritten instead of a hung wavefront.
+constexpr int kMergeSpinLimit = 1 << 22;
+struct MergeArgs {
+    float* part_out;
+    float* part_ml;
+    uint64_t* part_flag;
+    unsigned long long merge_tag;
+    void* out;
+    int out_dtype, num_heads_q, num_heads_kv, head_dim;
+};
+template <int kHD, bool kPad>
+__device__ __forceinline__ void merge_in_kernel(const MergeArgs& p, const Line& line, int s, int h, int token,
+                                                int id_first, int id_last, int lane) {
+    const int Hkv = p.num_heads_kv, G = p.num_heads_q / p.num_heads_kv;
+    const int head_dim = kPad ? p.head_dim : kHD;
+    const int n16 = lane & 15, kg = lane >> 4;
+    // flags of the other pieces: lane i polls piece id_first + i (64 at a time)
+    for (int id0 = id_first; id0 < id_last; id0 += 64) {
+        const int id = id0 + lane;
+        const bool have = id < id_last && line.begin(id) < line.begin(id + 1);  // (empty pieces leave nothing)
+        unsigned long long* flag = (unsigned long long*)p.part_flag + ((int64_t)id + (int64_t)s * Hkv + h);
+        bool ready = !have;
+        for (int spin = 0; spin < kMergeSpinLimit; spin++) {
+            if (!ready) ready = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.merge_tag;
+            if (__builtin_amdgcn_ballot_w64(!ready) == 0) break;
+            __builtin_amdgcn_s_sleep(2);
+        }
+        if (__builtin_amdgcn_ballot_w64(!ready) != 0) return;
+        // taken: a replay of a captured call comes with the same tag and must not see this flag again
+        if (have) __hip_atomic_store(flag, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    float m_run = -INFINITY, l_run = 0.0f;
+    float4_t acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    const bool mine = n16 < G;
+    // two pieces at a time, every load of the two issued before the first is used: the merge is a chain
+    // of memory round trips at the very end of the kernel, and four at a time make the register allocator spill
+    for (int id0 = id_first; id0 <= id_last; id0 += 2) {
+        float mw[2], lw[2];
+        float4_t part[2][8];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int id = id0 + u;
+            mw[u] = -INFINITY;
+            lw[u] = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) part[u][e] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            if (mine && id <= id_last && line.begin(id) < line.begin(id + 1)) {
+                const int64_t slot = (int64_t)id + (int64_t)s * Hkv + h;
+                const float* rec = p.part_out + (slot * kPartPairs * 4 * G + (kg * G + n16)) * 2;
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int e2 = 0; e2 < 4; e2++) {
+                        float x, y;
+                        agent_load2(rec + (r * 4 + e2) * 8 * G, x, y);
+                        part[u][2 * e2][r] = x;
+                        part[u][2 * e2 + 1][r] = y;
+                    }
+                agent_load2(rec + 16 * 8 * G, mw[u], lw[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const float m_new = fmaxf(m_run, mw[u]);
+            const float rescale = (m_run == -INFINITY) ? 0.0f : fast_exp2(m_run - m_new);
+            const float f = (mw[u] == -INFINITY) ? 0.0f : fast_exp2(mw[u] - m_new);
+            l_run = l_run * rescale + f * lw[u];
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] = acc[e] * rescale + part[u][e] * f;
+            m_run = m_new;
+        }
+    }
+    if (!mine) return;
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int d0 = (kg * 4 + r) * 8;
+        if ((kPad || kHD < 128) && d0 >= head_dim) continue;
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = acc[e][r] * inv;
+        store_out8(p.out, ((int64_t)token * p.num_heads_q + h * G + n16) * head_dim + d0, p.out_dtype, o);
+    }
+}
+
 // Pure decode batches of up to kSelfPlanMaxRows rows need no prologue launch: every wavefront works
 // out the schedule for itself (one record per row into LDS, lane-parallel, and a wavefront scan for
 // the prefix sums), which is shorter than the chain of dependent global loads through a plan another
@@ -843,6 +966,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     // A group mixes wavefronts of every XCD and of both dispatch halves (w / 8 mod groups).
     const int group = (w >> 3) % p.dyn_groups;
     int piece = w;
+    int merge_seg = -1;  // (fused_merge) the segment this piece has to combine, as sequence * kv heads + kv head
     for (;;) {
     int ticket_lane0 = 0;
     if (p.dyn_pieces > 0 && lane == 0) ticket_lane0 = atomicAdd(p.dyn_counter + group, 1);
@@ -886,6 +1010,9 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         const int n = (int)(to - from);  // blocks of this segment in this piece
         const bool whole = (n == nb);
         L = from;
+        // the segment ends here and began in an earlier piece: this piece combines it when it is done
+        // (one scalar carried through the loop; the rest is worked out again then)
+        if (p.fused_merge && !whole && b_rel + n == nb) merge_seg = s * Hkv + h;
         const int lb0 = rg.j0 / kUnit + b_rel;          // first unit of 32 tokens
         // (kBlk == 0: the table is indexed by the block of the absolute unit, lb0 + ... >> log2(units per block))
         const int32_t* table = p.block_indices + rg.table_begin + (kBlk ? lb0 * kEntries : 0);
@@ -1035,21 +1162,48 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     o[e] = v * inv;
                 }
                 const int d0 = (kg * 4 + r) * 8;
-                if ((kPad || kHD < 128) && d0 >= head_dim) continue;  // (rows of the accumulator beyond the head size hold nothing)
+                // (rows of the accumulator beyond the head size hold nothing; a fused partial carries them all the same)
+                if ((kPad || kHD < 128) && d0 >= head_dim && (whole || !p.fused_merge)) continue;
                 if (whole) {
                     store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * head_dim + d0, p.out_dtype, o);
+                } else if (p.fused_merge) {
+                    float* rec = p.part_out + (slot * kPartPairs * 4 * G + (kg * G + n16)) * 2;
+#pragma unroll
+                    for (int e2 = 0; e2 < 4; e2++) agent_store2(rec + (r * 4 + e2) * 8 * G, o[2 * e2], o[2 * e2 + 1]);
                 } else {
                     float* po = p.part_out + (slot * G + n16) * head_dim + d0;
                     *(float4*)(po) = make_float4(o[0], o[1], o[2], o[3]);
                     *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
                 }
             }
-            if (!whole && kg == 0) {
+            if (!whole && p.fused_merge) {
+                agent_store2(p.part_out + (slot * kPartPairs * 4 * G + (kg * G + n16)) * 2 + 16 * 8 * G, st.m, l);
+            } else if (!whole && kg == 0) {
                 p.part_ml[(slot * G + n16) * 2] = st.m;
                 p.part_ml[(slot * G + n16) * 2 + 1] = l;
             }
         }
+        if (p.fused_merge && !whole && b_rel + n < nb) {
+            // a partial another wavefront will combine: announced once the stores above have completed
+            // (no load is in flight at the end of a segment, so the wait is for these stores alone)
+            stores_done();
+            if (lane == 0)
+                __hip_atomic_store((unsigned long long*)p.part_flag + slot, p.merge_tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         L += n;
+    }
+    if (merge_seg >= 0) {
+        stores_done();  // this wavefront's own partial of that segment
+        const int ms = merge_seg / Hkv, mh = merge_seg - ms * Hkv;
+        DecodeRange mr;
+        if constexpr (kSelfPlan)
+            mr = plan_rec[ms];
+        else
+            mr = ((const DecodeRange*)p.seq_info)[ms];
+        const int64_t first_unit = (int64_t)prefix_at(ms) * Hkv + (int64_t)mh * (mr.nb + p.switch_cost) + p.switch_cost;
+        const MergeArgs ma = {p.part_out, p.part_ml, p.part_flag, p.merge_tag, p.out, p.out_dtype, p.num_heads_q, p.num_heads_kv, p.head_dim};
+        merge_in_kernel<kHD, kPad>(ma, line, ms, mh, mr.token, line.piece_at(first_unit), piece, lane);
+        merge_seg = -1;
     }
     if (p.dyn_pieces <= 0) break;
     const int next = group + __shfl(ticket_lane0, 0, 64) * p.dyn_groups;
@@ -1588,8 +1742,11 @@ Option g_options[] = {
     {"mixed_decode_share_percent", "HIPATTN_MIXED_DECODE_SHARE_PERCENT", 100, 10, 1000, {100}},
     // 1: dense SDPA at head sizes below 128 runs the tuned head-128 kernel on rows of fewer columns; 0: the plain kernels
     {"sdpa_padded_rows", "HIPATTN_SDPA_PADDED_ROWS", 1, 0, 1, {1}},
+    // 2: the decode kernel combines the partials of split segments itself; 0: a merge launch behind it;
+    // 1: whichever measured faster (the kernel itself for u8 caches, the launch for 16-bit ones)
+    {"decode_fused_merge", "HIPATTN_DECODE_FUSED_MERGE", 1, 0, 2, {1}},
 };
-enum { kOptMixedOverlap = 0, kOptSwitchCost, kOptDynPieces, kOptSharePercent, kOptSdpaPadded };
+enum { kOptMixedOverlap = 0, kOptSwitchCost, kOptDynPieces, kOptSharePercent, kOptSdpaPadded, kOptFusedMerge };
 
 void init_options_from_environment() {
     static std::once_flag once;
@@ -1694,6 +1851,13 @@ static int choose_dyn_pieces(const PagedParams& p, int num_waves, bool overlap) 
     return num_waves * option(kOptDynPieces);
 }
 
+// Bytes of one slot of unnormalised partial outputs: [G, head_dim] floats for the merge kernel, or the
+// fused merge's lane layout (kPartPairs pairs for each of 4 G lanes), whichever is larger.
+static size_t part_floats_per_slot(const PagedParams& p) {
+    const size_t G = (size_t)(p.num_heads_q / p.num_heads_kv);
+    return std::max(G * p.head_dim, (size_t)kPartPairs * 4 * G * 2) * sizeof(float);
+}
+
 size_t paged_fast_workspace_bytes(const PagedParams& p) {
     const bool overlap = overlap_wanted(p);
     const int W = choose_num_waves(p, overlap);
@@ -1701,7 +1865,19 @@ size_t paged_fast_workspace_bytes(const PagedParams& p) {
     const size_t rows = (size_t)plan_rows(p);
     const size_t slots = (size_t)W + choose_dyn_pieces(p, W, overlap) + rows * p.num_heads_kv;
     return 512 + 2 * align_up((rows + 1) * sizeof(int32_t), 256) + align_up(rows * 32, 256) +
-           align_up(slots * G * p.head_dim * sizeof(float), 256) + align_up(slots * G * 2 * sizeof(float), 256);
+           align_up(slots * part_floats_per_slot(p), 256) + align_up(slots * G * 2 * sizeof(float), 256) +
+           align_up(slots * sizeof(uint64_t), 256);
+}
+
+// A value no earlier call of this process used and that memory which was never written is unlikely to hold.
+static unsigned long long next_merge_tag() {
+    static std::atomic<unsigned long long> counter{0};
+    static const unsigned long long base = [] {
+        unsigned long long x = 0x9e3779b97f4a7c15ull ^ (unsigned long long)(uintptr_t)&counter;
+        x ^= (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0xbf58476d1ce4e5b9ull;
+        return x | (1ull << 63);
+    }();
+    return base + (counter.fetch_add(1, std::memory_order_relaxed) << 1) + 1;  // never zero: zero means "taken"
 }
 
 
@@ -1729,9 +1905,18 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     p.seq_info = w;
     w += align_up((size_t)p.num_rows * 32, 256);
     p.part_out = (float*)w;
-    w += align_up(slots * G * p.head_dim * sizeof(float), 256);
+    w += align_up(slots * part_floats_per_slot(p), 256);
     p.part_ml = (float*)w;
     w += align_up(slots * G * 2 * sizeof(float), 256);
+    p.part_flag = (uint64_t*)w;
+    w += align_up(slots * sizeof(uint64_t), 256);
+    // the head-256 kernel and on-demand pieces (whose order of completion is not that of their numbers) keep the merge launch
+    // Measured (whole steps, same machine): the 128-sequence u8 batch 0.450 ms fused against 0.454 ms with the
+    // launch; the 64-sequence fp16 batch 0.223 against 0.219 ms -- its kernel has no register to spare, and what
+    // the merge code adds is paid at every wavefront's start.
+    const int fused = option(kOptFusedMerge);
+    p.fused_merge = ((fused == 2 || (fused == 1 && p.cache_dtype == HIPATTN_U8)) && p.dyn_pieces == 0 && p.head_dim <= 128) ? 1 : 0;
+    p.merge_tag = next_merge_tag();
 }
 
 // ---- scratch of the entry point that allocates nothing (hipattn_paged_attention_noalloc) ------
@@ -1926,7 +2111,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         launch_decode<1, true>(p, wp, write ? 1 : 0, dim3(p.num_waves), dim3(64), stream);
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
-        if (e != hipSuccess) return e;
+        if (e != hipSuccess || p.fused_merge) return e;
         hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
         return hipGetLastError();
     }
@@ -1957,7 +2142,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
         const hipError_t e_prefill = launch_paged_prefill(p, side->stream);
-        if (e == hipSuccess) {
+        if (e == hipSuccess && !p.fused_merge) {
             hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
             e = hipGetLastError();
         }
@@ -1971,9 +2156,11 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     e = hipGetLastError();
     if (probe.after) (void)hipEventRecord(probe.after, stream);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (!p.fused_merge) {
+        hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     if (p.max_q_tiles > 0) {
         e = launch_paged_prefill(p, stream);
     }

@@ -494,7 +494,9 @@ def test_paged_decode_sliding_window(hip, oracle, cache_dtype, window):
 
 
 @pytest.mark.parametrize("env", [{"decode_dyn_pieces_per_wave": 4}, {"decode_switch_cost": 0},
-                                 {"decode_dyn_pieces_per_wave": 2, "decode_switch_cost": 9}])
+                                 {"decode_dyn_pieces_per_wave": 2, "decode_switch_cost": 9},
+                                 {"decode_fused_merge": 2}, {"decode_fused_merge": 0},
+                                 {"decode_fused_merge": 2, "decode_switch_cost": 0}])
 @pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
 def test_paged_decode_schedule_knobs(hip, oracle, env, cache_dtype, schedule_options):
     """The schedule of the decode kernel (on-demand pieces, segment-start cost) never changes results."""
@@ -507,6 +509,29 @@ def test_paged_decode_schedule_knobs(hip, oracle, env, cache_dtype, schedule_opt
     for waves in (0, 40, 300, 4000):
         out, _ = dev.run(decode_waves=waves)
         assert H.max_abs(out, ref) <= (1e-2 if cache_dtype == W.U8 else 2e-3), waves
+    dev.free()
+
+
+@pytest.mark.parametrize("fused", [0, 2])
+@pytest.mark.parametrize("D,bs,Hq,Hkv,cache_dtype", [(128, 32, 32, 8, W.F16), (128, 16, 16, 8, W.BF16), (128, 32, 128, 8, W.U8),
+                                                     (64, 32, 8, 8, W.F16), (96, 64, 24, 8, W.F16), (40, 16, 16, 4, W.U8),
+                                                     (128, 128, 64, 8, W.U8), (72, 32, 14, 2, W.BF16)])
+def test_paged_decode_merge_inside_the_kernel_and_behind_it(hip, oracle, fused, D, bs, Hq, Hkv, cache_dtype, schedule_options):
+    """Segments that several wavefronts share are combined by the decode kernel itself or by the merge launch:
+    both against the oracle, at wavefront counts from fewer than segments to many per segment, one call after
+    the other (the allocator hands the freed workspace out again, so a call meets the flags of the one before)."""
+    announce("paged decode merge", fused, D, bs, Hq, Hkv, cache_dtype)
+    schedule_options({"decode_fused_merge": fused})
+    seqs = [(c - 1, 1) for c in DECODE_CTX]
+    case = W.make_paged_case(77, seqs, Hq, Hkv, D, bs, W.F16, W.F16, cache_dtype, sliding_window=0)
+    ref, _, _ = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case)
+    tol = 1e-2 if cache_dtype in (W.U8, W.BF16) else 2e-3
+    for waves in (0, 7, 160, 2048, 160):
+        out, path = dev.run(decode_waves=waves)
+        assert path == "paged_mfma"
+        assert np.isfinite(out).all()
+        assert H.scaled_bound_error(out, ref) <= tol, waves
     dev.free()
 
 
