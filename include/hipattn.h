@@ -198,9 +198,9 @@ hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q,
  * block_size that is a power of two take a plain matrix-core kernel (query tiles over the block
  * table); anything else (fp32, larger heads) takes the shape-generic fp32 kernels.
  * A single-token row with nothing to attend (an empty block table) gets an output row of zeros.
- * Block ids outside [0, num_blocks) in a table: the decode and the shape-generic kernels skip
- * those blocks (probability zero); the MFMA chunked-prefill kernel redirects them to a valid
- * block, so reads stay inside the cache and the affected rows are unspecified.
+ * A table entry outside [0, num_blocks) names no block: the positions it stands for take no part
+ * (probability zero in every kernel; a new token that falls there is not stored), and a row left with
+ * nothing to attend is zeros.  No kernel reads outside the cache for such an entry.
  * A mixed batch (single-token and multi-token sequences) with decode_waves == 0 runs its two
  * parts side by side: the call forks from `stream` onto a side stream that the library keeps for
  * that stream (created by the first such call on it, default priority, destroyed by

@@ -177,8 +177,9 @@ __device__ __forceinline__ void key_range(const Tile& t, int& lo, int& hi) {
 }
 
 // Byte offset of a key's row from t.k / t.v.  Keys past the end are redirected to the last valid
-// key and block ids outside the cache are clamped: such rows only ever meet a probability of
-// zero (or are unspecified input), but they must be readable and finite.
+// key and block ids outside the cache are clamped (the loads stay unconditional and inside the
+// cache): such rows only ever meet a probability of zero -- the softmax masks the keys of a block
+// the table does not name -- but they must be readable and finite.
 __device__ __forceinline__ int64_t kv_row_offset(const Tile& t, int key, int row_bytes = kRowBytes) {
     key = min(key, t.kv_len - 1);
     if (t.table == nullptr) return (int64_t)key * row_bytes;
@@ -281,10 +282,12 @@ struct SoftmaxState {
 // 1 a boolean mask of one byte per key (zero: the key takes no part).  mask_lds: this wavefront's
 // 32 rows x 64 keys of the mask in LDS (mask_tile_* below), or nullptr for a tile that reaches past
 // the last key, whose mask values are fetched from global memory one by one.
+// bad16 (paged caches; wave-uniform): bit b set when keys ts + 16 b .. + 15 lie in a block whose table
+// entry names no block of the cache -- they take no part, like keys past the end (`masked` must be set).
 template <bool kBf16, int kMask = 0>
 __device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], float16_t (&o)[4], SoftmaxState& st,
                                              typename Mfma<kBf16>::vec8 (&pf)[4], int ts, int my_pos, int hi, bool masked,
-                                             const lds_byte* mask_lds = nullptr, int row = 0) {
+                                             const lds_byte* mask_lds = nullptr, int row = 0, uint32_t bad16 = 0) {
     using M = Mfma<kBf16>;
     using vec8 = typename M::vec8;
     if (masked) {
@@ -292,8 +295,8 @@ __device__ __forceinline__ void tile_softmax(const Tile& t, float16_t (&s)[2], f
         for (int mt = 0; mt < 2; mt++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
-                bool ok = key < t.kv_len;
+                const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);  // in sixteenth 2 mt + r / 8 of the tile
+                bool ok = key < t.kv_len && ((bad16 >> (2 * mt + (r >> 3))) & 1u) == 0;
                 if (t.causal) ok = ok && key <= my_pos;
                 if (t.window > 0) ok = ok && key > my_pos - t.window;
                 s[mt][r] = ok ? s[mt][r] : -INFINITY;
@@ -665,6 +668,24 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         return (ts + kTileK <= t.kv_len) && (!t.causal || ts + kTileK <= t.pos0 + 1) &&
                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
     };
+    // Paged caches: table entries that name no block of the cache ([0, num_blocks)) stand for keys that
+    // take no part.  Almost no call has one, so every wavefront first looks through the entries of the
+    // workgroup's key range (up to 256 of them, four loads per lane, issued ahead of everything else and
+    // looked at only after the query rows have been converted); the tiles of a range that has one -- or
+    // is longer than that -- get their entries checked one by one (bad_sixteenths).
+    uint32_t scan_ids[4] = {0u, 0u, 0u, 0u};
+    bool scan_covers = true;
+    if constexpr (kPaged) {
+        if (t.table != nullptr && t.kv_len > 0) {
+            const int e_lo = kv_lo >> t.block_shift, e_hi = (min(kv_hi, t.kv_len) - 1) >> t.block_shift;
+            scan_covers = e_hi - e_lo < 256;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int e = e_lo + lane + 64 * u;
+                if (e <= e_hi) scan_ids[u] = (uint32_t)t.table[e];
+            }
+        }
+    }
 
     // The wavefront's 32 query rows go to its own 8 KB of LDS with eight global->LDS loads of four
     // whole rows each, laid out like a K tile (chunk c of row r at position c ^ (r % 16)): the
@@ -905,6 +926,31 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) asm volatile("" : "+v"(qf[i]));  // (converted before the wait below, not after)
+    bool check_blocks = false;  // wave-uniform
+    if constexpr (kPaged) {
+        bool bad_lane = false;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            asm volatile("" : "+v"(scan_ids[u]));  // (looked at here, not where they were loaded)
+            bad_lane = bad_lane || scan_ids[u] >= (uint32_t)t.num_blocks;
+        }
+        check_blocks = !scan_covers || __builtin_amdgcn_ballot_w64(bad_lane) != 0;
+    }
+    // which sixteenths of tile j lie in blocks the table does not name (only ever called when check_blocks)
+    auto bad_sixteenths = [&](int j) -> uint32_t {
+        uint32_t bits = 0;
+        if constexpr (kPaged) {
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int key0 = kv_lo + j * kTileK + 16 * b;
+                if (key0 >= t.kv_len) continue;  // (keys past the end are masked as such)
+                int entry;
+                asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(entry) : "s"(t.table + (key0 >> t.block_shift)));
+                if ((uint32_t)entry >= (uint32_t)t.num_blocks) bits |= 1u << b;
+            }
+        }
+        return bits;
+    };
     if constexpr (kMask != 0) recent += load_mask_tile(0);  // the query rows have left the stage
     phase_barrier(recent);
     if (group == 1) phase_barrier(recent);  // group 1 sits out phase 0
@@ -955,6 +1001,9 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             wait_keeping_loads(recent);
             tile_softmax<kBf16, kMask>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, true,
                                        mask_tile_staged(j) ? mask_stage(j) : nullptr, row);
+        } else if constexpr (kPaged) {
+            const uint32_t bad16 = check_blocks ? bad_sixteenths(j) : 0u;
+            tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j) || bad16 != 0, nullptr, 0, bad16);
         } else {
             tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j));
         }

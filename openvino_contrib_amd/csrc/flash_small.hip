@@ -248,6 +248,12 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
     constexpr bool kDeep = kDP == 64;
     typedef uint4_t Stage[2 * kPieces];
     Stage stage_a, stage_b;
+    // paged: a table entry that names no block of the cache ([0, num_blocks)) stands for keys that take no
+    // part.  Their rows are read from a block inside the cache all the same (the loads stay unconditional);
+    // which rows of a staged tile they are travels beside the tile: a bit per piece with the registers
+    // (bad_a, bad_b), a byte per row with the tile in LDS (row_bad), and the softmax masks those keys.
+    uint32_t bad_a = 0, bad_b = 0;
+    __shared__ uint8_t row_bad[2][kTileK];
     // paged: the block ids of a tile's rows are looked up one tile ahead of its K/V loads, so that
     // those loads do not wait for the table
     int block_of[kPieces];
@@ -261,15 +267,17 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
             }
         }
     };
-    auto fetch = [&](Stage& stage, int tile) __attribute__((always_inline)) {  // (paged: after lookup(tile))
+    auto fetch = [&](Stage& stage, uint32_t& bad, int tile) __attribute__((always_inline)) {  // (paged: after lookup(tile))
+        bad = 0;
 #pragma unroll
         for (int s = 0; s < kPieces; s++) {
             const int piece = tid + 64 * kWaves * s, r = piece / kChunks, c = piece % kChunks;
             const int key = min(tile * kTileK + r, w.kv_len - 1);  // rows past the end repeat the last key (masked later)
             int64_t at;
             if constexpr (kPaged) {
-                // a block id outside the cache is redirected into it: the rows that attend it are unspecified
+                // a block id outside the cache is redirected into it, and its keys are masked
                 const int pb = min(max(block_of[s], 0), w.num_blocks - 1);
+                if (pb != block_of[s]) bad |= 1u << s;
                 at = (int64_t)pb * w.block_stride + (int64_t)(key & ((1 << w.block_shift) - 1)) * row_bytes + (kU8 ? 0 : 16 * c);
             } else {
                 at = (int64_t)key * row_bytes + 16 * c;
@@ -288,10 +296,13 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
             }
         }
     };
-    auto deposit = [&](const Stage& stage, int buf) __attribute__((always_inline)) {
+    auto deposit = [&](const Stage& stage, uint32_t bad, int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int s = 0; s < kPieces; s++) {
             const int piece = tid + 64 * kWaves * s, r = piece / kChunks, c = piece % kChunks;
+            if constexpr (kPaged) {
+                if (c == 0) row_bad[buf][r] = (uint8_t)((bad >> s) & 1u);
+            }
             if constexpr (kU8) {
                 *(uint4_t*)(lds[buf][0] + k_chunk_offset<kDP>(r, c)) = dequantised8(stage[s]);
                 *(uint4_t*)(lds[buf][1] + v_chunk_offset<kDP>(r, c)) = dequantised8(stage[kPieces + s]);
@@ -311,12 +322,12 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 
     if (tile0 < tiles) {
         lookup(tile0);
-        fetch(stage_a, tile0);
+        fetch(stage_a, bad_a, tile0);
         if (tile0 + 1 < tiles) lookup(tile0 + 1);
-        deposit(stage_a, 0);
+        deposit(stage_a, bad_a, 0);
         if constexpr (kDeep) {
             if (tile0 + 1 < tiles) {
-                fetch(stage_a, tile0 + 1);
+                fetch(stage_a, bad_a, tile0 + 1);
                 if (tile0 + 2 < tiles) lookup(tile0 + 2);
             }
         }
@@ -324,19 +335,22 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
     __syncthreads();
     // One key tile.  kDeep: `next` holds tile j + 1, on its way since the previous iteration, and
     // `ahead` takes the loads of tile j + 2; otherwise `next` takes the loads of tile j + 1 now.
-    auto iteration = [&](int j, Stage& next, Stage& ahead) __attribute__((always_inline)) {
+    auto iteration = [&](int j, Stage& next, uint32_t& next_bad, Stage& ahead, uint32_t& ahead_bad) __attribute__((always_inline)) {
         const int buf = (j - tile0) & 1;
         if constexpr (kDeep) {
             if (j + 2 < tiles) {
-                fetch(ahead, j + 2);
+                fetch(ahead, ahead_bad, j + 2);
                 if (j + 3 < tiles) lookup(j + 3);
             }
         } else {
             if (j + 1 < tiles) {
-                fetch(next, j + 1);  // in flight while this tile is computed
+                fetch(next, next_bad, j + 1);  // in flight while this tile is computed
                 if (j + 2 < tiles) lookup(j + 2);
             }
         }
+        // keys of this tile whose block the table does not name, one bit per key (wave-uniform)
+        uint64_t bad_keys = 0;
+        if constexpr (kPaged) bad_keys = __builtin_amdgcn_ballot_w64(row_bad[buf][lane] != 0);
         const lds_byte* k_lds = (const lds_byte*)lds[buf][0];
         const lds_byte* v_lds = (const lds_byte*)lds[buf][1];
         const int ts = j * kTileK;
@@ -398,14 +412,15 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
         // before the window of the wavefront's last row)
         const int wave_pos = w.pos0 + wave * 32 * w.pos_step;
         const bool edge = ts + kTileK > w.kv_len || (w.causal && ts + kTileK - 1 > wave_pos) ||
-                          (windowed && ts <= wave_pos + 31 * w.pos_step - w.window);
+                          (windowed && ts <= wave_pos + 31 * w.pos_step - w.window) || bad_keys != 0;
         if (edge) {
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
-                    const bool ok = key < w.kv_len && (!w.causal || key <= my_pos) && (!windowed || key > my_pos - w.window);
+                    const int in_tile = mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3), key = ts + in_tile;
+                    const bool ok = key < w.kv_len && (!w.causal || key <= my_pos) && (!windowed || key > my_pos - w.window) &&
+                                    ((bad_keys >> in_tile) & 1u) == 0;
                     s[mt][r] = ok ? s[mt][r] : -INFINITY;
                 }
         }
@@ -447,12 +462,12 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
 #pragma unroll
             for (int dt = 0; dt < kOutTiles; dt++) o[dt] = M::mma(read_v_frag<kBf16, kDP>(v_lds, lane, ks, dt), pf[ks], o[dt]);
 
-        if (j + 1 < tiles) deposit(next, buf ^ 1);  // the other buffer was last read before the previous barrier
+        if (j + 1 < tiles) deposit(next, next_bad, buf ^ 1);  // the other buffer was last read before the previous barrier
         __syncthreads();
     };
     for (int j = tile0; j < tiles; j += 2) {
-        iteration(j, stage_a, stage_b);
-        if (j + 1 < tiles) iteration(j + 1, kDeep ? stage_b : stage_a, kDeep ? stage_a : stage_b);
+        iteration(j, stage_a, bad_a, stage_b, bad_b);
+        if (j + 1 < tiles) iteration(j + 1, kDeep ? stage_b : stage_a, kDeep ? bad_b : bad_a, kDeep ? stage_a : stage_b, kDeep ? bad_a : bad_b);
     }
 
     // normalise and store: register r of o[dt] is head-dim 32 dt + 8 (r / 4) + 4 hi + r % 4 of query row n32

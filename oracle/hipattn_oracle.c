@@ -407,16 +407,30 @@ ORACLE_API int64_t oracle_kv_cache_write(const float* k_new, const float* v_new,
 /*
  * Gather one sequence's first n cache rows of kv head h through its block table into a
  * contiguous fp32 [n, D] array (used by the oracle itself and by tests that reduce the
- * paged case to the dense one).
+ * paged case to the dense one).  A table entry outside [0, num_blocks) names no block: its rows
+ * come out as zeros and, when valid is not NULL, valid[p] is 0 for them (1 for every other row).
+ * num_blocks <= 0: every entry is taken as it is.
  */
-ORACLE_API void oracle_gather_cache_rows(const uint8_t* cache, int cache_dtype, const int32_t* seq_blocks, int n,
-                                         int h, int Hkv, int D, int block_size, float* dst) {
+ORACLE_API void oracle_gather_cache_rows_checked(const uint8_t* cache, int cache_dtype, const int32_t* seq_blocks, int n,
+                                                 int h, int Hkv, int D, int block_size, int num_blocks, float* dst,
+                                                 uint8_t* valid) {
     int64_t rb = cache_row_bytes(cache_dtype, D);
     for (int p = 0; p < n; p++) {
         int pb = seq_blocks[p / block_size];
+        int ok = num_blocks <= 0 || (pb >= 0 && pb < num_blocks);
+        if (valid) valid[p] = (uint8_t)ok;
+        if (!ok) {
+            memset(dst + (int64_t)p * D, 0, sizeof(float) * (size_t)D);
+            continue;
+        }
         int64_t off = (((int64_t)pb * Hkv + h) * block_size + p % block_size) * rb;
         cache_row_load(cache_dtype, cache + off, D, dst + (int64_t)p * D);
     }
+}
+
+ORACLE_API void oracle_gather_cache_rows(const uint8_t* cache, int cache_dtype, const int32_t* seq_blocks, int n,
+                                         int h, int Hkv, int D, int block_size, float* dst) {
+    oracle_gather_cache_rows_checked(cache, cache_dtype, seq_blocks, n, h, Hkv, D, block_size, 0, dst, NULL);
 }
 
 /*
@@ -425,6 +439,16 @@ ORACLE_API void oracle_gather_cache_rows(const uint8_t* cache, int cache_dtype, 
  *   do_write != 0: first scatter k_new / v_new (oracle_kv_cache_write).
  * Query token i of sequence s sits at position p = past_lens[s] + i and attends cache
  * positions j with max(0, p - W + 1) <= j <= p when W = sliding_window > 0, else 0..p.
+ * A table entry outside [0, num_blocks) names no block: the positions it stands for take no part
+ * (probability zero, like the new tokens that oracle_kv_cache_write could not store there), and a
+ * row left with nothing to attend is zeros.
+ * alibi_slopes (NULL, or one float per query head): slope[h] * (j - p) is added to the scaled score
+ * of position j, the linear distance bias of ALiBi (0 at the token itself, more negative with
+ * distance for a positive slope).  A constant added to a whole row does not change its softmax,
+ * so a kernel may measure the distance from any fixed position of the row.
+ * PARITY UNPINNED against OpenVINO for this input (sign and origin restated from the operator's
+ * documentation); pinned against an explicit additive mask through torch's fp64
+ * scaled_dot_product_attention (tests/golden/make_alibi_golden.py) and against the fp64 closed form.
  * scale <= 0 selects 1/sqrt(D).
  */
 ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const float* v_new, uint8_t* key_cache,
@@ -432,7 +456,7 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
                                       const int32_t* subsequence_begins, const int32_t* block_indices,
                                       const int32_t* block_indices_begins, int S, int Hq, int Hkv, int D,
                                       int block_size, int num_blocks, float scale, int sliding_window, int do_write,
-                                      float* out) {
+                                      const float* alibi_slopes, float* out) {
     if (S < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || block_size <= 0) return 1;
     if (scale <= 0.0f) scale = 1.0f / sqrtf((float)D);
     if (do_write)
@@ -459,22 +483,44 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
         float* kbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
         float* vbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
         float* scores = (float*)malloc(sizeof(float) * (size_t)ctx);
+        uint8_t* valid = (uint8_t*)malloc((size_t)ctx);
+        float* bias = (float*)malloc(sizeof(float) * (size_t)ctx); /* 0, or -inf where the table names no block */
+        float* rowbias = (float*)malloc(sizeof(float) * (size_t)ctx); /* bias plus a row's distance term */
         const int32_t* blocks = block_indices + block_indices_begins[s];
-        oracle_gather_cache_rows(key_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, kbuf);
-        oracle_gather_cache_rows(value_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, vbuf);
+        oracle_gather_cache_rows_checked(key_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, num_blocks, kbuf, valid);
+        oracle_gather_cache_rows_checked(value_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, num_blocks, vbuf, NULL);
+        int holes = 0;
+        for (int j = 0; j < ctx; j++) {
+            bias[j] = valid[j] ? 0.0f : -INFINITY;
+            holes += !valid[j];
+        }
         for (int i = 0; i < qlen; i++) {
             int p = past_lens[s] + i;
             int j0 = 0;
             if (sliding_window > 0 && p - sliding_window + 1 > 0) j0 = p - sliding_window + 1;
+            int j1 = p + 1 < ctx ? p + 1 : ctx;
+            if (j0 > ctx) j0 = ctx;
+            int any = 0;
+            for (int j = j0; j < j1 && !any; j++) any = valid[j];
             for (int g = 0; g < G; g++) {
                 int64_t row = ((int64_t)(t0 + i) * Hq + (h * G + g)) * D;
-                attend_row(q + row, kbuf, vbuf, D, j0 < ctx ? j0 : ctx, p + 1 < ctx ? p + 1 : ctx, D, scale, scores,
-                           out + row);
+                if (!any) {
+                    memset(out + row, 0, sizeof(float) * (size_t)D);
+                } else if (alibi_slopes) {
+                    float slope = alibi_slopes[h * G + g];
+                    for (int j = j0; j < j1; j++) rowbias[j] = bias[j] + slope * (float)(j - p);
+                    attend_row_biased(q + row, kbuf, vbuf, D, j0, j1, D, scale, rowbias, 1, scores, out + row);
+                } else {
+                    attend_row_biased(q + row, kbuf, vbuf, D, j0, j1, D, scale, holes ? bias : NULL, 1, scores, out + row);
+                }
             }
         }
         free(kbuf);
         free(vbuf);
         free(scores);
+        free(valid);
+        free(bias);
+        free(rowbias);
     }
     return 0;
 }

@@ -13,6 +13,14 @@ def oracle_paged(oracle, case, scale=0.0):
     return out, kc, vc
 
 
+def oracle_paged_no_write(oracle, case, scale=0.0):
+    """The oracle on the cache as the case holds it (no new rows stored): what a call with
+    HIPATTN_PA_SKIP_CACHE_WRITE on the uploaded cache has to give."""
+    return oracle.paged_attention(case["q"], case["k_new"], case["v_new"], case["key_cache"].copy(), case["value_cache"].copy(),
+                                  case["cache_dtype"], case["past_lens"], case["subsequence_begins"], case["block_indices"],
+                                  case["block_indices_begins"], case["Hq"], case["Hkv"], case["D"], case["block_size"],
+                                  scale=scale, sliding_window=case["sliding_window"], do_write=False)
+
 
 
 def scaled_bound_error(out, ref, label=""):

@@ -983,7 +983,7 @@ def test_paged_u8_cache_at_other_head_sizes_and_on_blocks_of_16(hip, oracle, D, 
 @pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
 def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle, cache_dtype):
     """A block id outside the pool contributes nothing, whichever half of a 32-token unit it is (checked
-    against the shape-generic kernels, which skip such blocks key by key)."""
+    against the oracle, which gives the positions of such an entry probability zero)."""
     announce("paged blocks of 16, bad ids", cache_dtype)
     seqs = [(99, 1), (47, 1), (16, 1), (300, 1)]
     case = W.make_paged_case(85, seqs, 16, 4, 128, 16, W.F16, W.F16, cache_dtype)
@@ -995,8 +995,10 @@ def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle, cache_dty
     ids[begins[3] + 6] = -1
     ids[begins[3] + 7] = 1 << 30                  # both halves
     dev = H.PagedDeviceCase(hip, case)
-    ref, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
-    assert path_g == "paged_generic" and np.isfinite(ref).all()
+    ref = H.oracle_paged_no_write(oracle, case)
+    gen, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic" and np.isfinite(gen).all()
+    assert H.max_abs(gen, ref) <= (1e-2 if case["cache_dtype"] in (W.U8, W.BF16) else 2e-3)
     for waves in (0, 50):
         out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE)
         assert path == "paged_mfma"
@@ -1009,7 +1011,7 @@ def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle, cache_dty
 def test_paged_head_256_skips_blocks_outside_the_cache(hip, oracle, bs, cache_dtype):
     """Head size 256: the decode kernel reads a block inside the cache in place of one whose id lies
     outside it and masks its tokens (no branch in its loop); a row whose every block is outside comes
-    out as zeros; checked against the shape-generic kernels, which skip such blocks key by key."""
+    out as zeros; checked against the oracle, which gives the positions of such an entry probability zero."""
     announce("paged head 256, bad ids", bs, cache_dtype)
     seqs = [(99, 1), (47, 1), (16, 1), (300, 1), (20, 1)]
     case = W.make_paged_case(90, seqs, 8, 4, 256, bs, W.F16, W.F16, cache_dtype)
@@ -1021,8 +1023,10 @@ def test_paged_head_256_skips_blocks_outside_the_cache(hip, oracle, bs, cache_dt
     ids[begins[3] + 4 * per: begins[3] + 6 * per] = 1 << 30              # two units in a row
     ids[begins[4]: begins[5]] = -1                                       # every block of the row
     dev = H.PagedDeviceCase(hip, case)
-    ref, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
-    assert path_g == "paged_generic" and np.isfinite(ref).all()
+    ref = H.oracle_paged_no_write(oracle, case)
+    gen, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic" and np.isfinite(gen).all()
+    assert H.max_abs(gen, ref) <= (1e-2 if case["cache_dtype"] in (W.U8, W.BF16) else 2e-3)
     for waves in (0, 50):
         out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE)
         assert path == "paged_mfma"
@@ -1038,7 +1042,7 @@ def test_paged_head_256_skips_blocks_outside_the_cache(hip, oracle, bs, cache_dt
 def test_paged_large_blocks_skip_blocks_outside_the_cache(hip, oracle, D, cache_dtype, bs):
     """Blocks of more than 32 tokens hold several of the stream-K kernels' 32-token units: a block id
     outside the pool takes all of them out, a row whose every block is outside comes out as zeros
-    (checked against the shape-generic kernels, which skip such blocks key by key)."""
+    (checked against the oracle, which gives the positions of such an entry probability zero)."""
     announce("paged large blocks, bad ids", D, cache_dtype, bs)
     seqs = [(399, 1), (47, 1), (bs, 1), (700, 1), (200, 1)]
     qd = W.BF16 if cache_dtype == W.BF16 else W.F16
@@ -1051,14 +1055,55 @@ def test_paged_large_blocks_skip_blocks_outside_the_cache(hip, oracle, D, cache_
     ids[begins[3] + 700 // bs] = -1               # the last block
     ids[begins[4]: begins[5]] = -1                # every block of the row
     dev = H.PagedDeviceCase(hip, case)
-    ref, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
-    assert path_g == "paged_generic" and np.isfinite(ref).all()
+    ref = H.oracle_paged_no_write(oracle, case)
+    gen, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
+    assert path_g == "paged_generic" and np.isfinite(gen).all()
+    assert H.max_abs(gen, ref) <= (1e-2 if case["cache_dtype"] in (W.U8, W.BF16) else 2e-3)
     for waves in (0, 50, 3):
         out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE)
         assert path == "paged_mfma"
         assert np.isfinite(out).all()
         assert H.max_abs(out, ref) <= (2e-3 if cache_dtype == W.F16 else 1e-2)
     assert not out[1].any() and not out[4].any()
+    dev.free()
+
+
+@pytest.mark.parametrize("D,bs,Hq,Hkv,cache_dtype", [(128, 32, 8, 4, W.F16), (128, 16, 8, 4, W.BF16), (128, 32, 16, 2, W.U8), (128, 64, 6, 2, W.F16),
+                                                     (96, 32, 8, 4, W.F16), (64, 32, 8, 4, W.F16), (64, 16, 4, 4, W.U8), (256, 32, 4, 2, W.BF16),
+                                                     (80, 8, 8, 2, W.F16), (128, 8, 40, 2, W.F16), (48, 4, 4, 1, W.U8)])
+@pytest.mark.parametrize("window", [0, 150])
+def test_paged_chunks_take_no_key_from_a_block_outside_the_cache(hip, oracle, D, bs, Hq, Hkv, cache_dtype, window):
+    """Multi-token sequences (the chunk kernels of every head size, and the query-tile kernel that takes whole
+    batches of the other shapes) with table entries that name no block: those positions get probability zero,
+    as the oracle defines it; the new tokens that fall there are not stored (cache bytes bit-exact); a
+    sequence whose every entry is bad comes out as zeros."""
+    announce("paged chunks, bad ids", D, bs, Hq, Hkv, cache_dtype, window)
+    seqs = [(300, 200), (0, 130), (700, 1), (40, 64), (513, 129), (64, 1), (90, 70)]
+    qd = W.BF16 if cache_dtype == W.BF16 else W.F16
+    case = W.make_paged_case(93, seqs, Hq, Hkv, D, bs, qd, qd, cache_dtype, sliding_window=window)
+    ids, begins, nb = case["block_indices"], case["block_indices_begins"], case["num_blocks"]
+    per = max(1, 64 // bs)  # table entries per 64-key tile
+    ids[begins[0] + 2 * per] = nb + 3               # the first sixteenth (or more) of a tile
+    ids[begins[0] + 5 * per + per - 1] = -1         # the end of a tile
+    ids[begins[0] + (499 // bs)] = nb               # the block of the last new tokens: they are not stored either
+    ids[begins[1] + 0] = 1 << 30                    # the first block of a prefill from position 0
+    ids[begins[2] + 3] = -7                         # a decode row beside the chunks
+    ids[begins[4] + (600 // bs)] = nb               # among the new tokens of a chunk
+    ids[begins[6]: begins[7]] = -2                  # every block of a multi-token sequence
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    assert np.isfinite(ref).all()
+    dev = H.PagedDeviceCase(hip, case)
+    tol = 1e-2 if (cache_dtype in (W.U8, W.BF16)) else 2e-3
+    for waves in (0, 24):
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if waves else 0)
+        assert path in ("paged_mfma", "paged_mfma_tiles"), path
+        assert np.isfinite(out).all()
+        assert H.scaled_bound_error(out, ref, "paged chunks, bad ids") <= tol, waves
+    t6 = case["subsequence_begins"][6]
+    assert not out[t6:t6 + 70].any()
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
     dev.free()
 
 

@@ -323,6 +323,63 @@ def test_paged_attention_block_permutation_invariance_and_window(oracle):
     np.testing.assert_array_equal(kcA, kcB)
 
 
+@pytest.mark.parametrize("cache_dtype,window", [(W.F16, 0), (W.U8, 0), (W.F32, 11)])
+def test_paged_attention_takes_no_key_from_a_block_outside_the_pool(oracle, cache_dtype, window):
+    """A table entry outside [0, num_blocks) names no block: its positions get probability zero.  Pinned by an
+    independent reduction: the rows of the valid blocks, gathered densely from a table whose bad entries are
+    pointed at a real block, through the fp64 closed form with the bad positions masked by hand; a row with
+    nothing left to attend is zeros; a table without bad entries gives what it gave before the rule existed."""
+    bs, Hq, Hkv, D = 8, 4, 2, 16
+    seqs = [(20, 12), (50, 1), (0, 3), (9, 1), (16, 2)]
+    case = W.make_paged_case(34, seqs, Hq, Hkv, D, bs, W.F32, W.F32, cache_dtype, sliding_window=window)
+    nb = case["num_blocks"]
+    ids, begins = case["block_indices"].copy(), case["block_indices_begins"]
+    good = ids.copy()
+    bad_at = [begins[0] + 1, begins[0] + 3, begins[1] + 0, begins[1] + 6, begins[2] + 0, begins[4] + 2]
+    for n, at in enumerate(bad_at):
+        ids[at] = [nb, -1, nb + 7, -(1 << 30), 1 << 30, nb][n]
+    for lb in range(begins[3], begins[4]):  # every block of sequence 3
+        ids[lb] = -5
+    # the cache as the step leaves it, from the table without holes (the holes' tokens are simply not stored)
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    oracle.kv_cache_write(case["k_new"], case["v_new"], kc, vc, cache_dtype, case["past_lens"], case["subsequence_begins"],
+                          good, begins, Hkv, D, bs)
+    out = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc.copy(), vc.copy(), cache_dtype, case["past_lens"],
+                                 case["subsequence_begins"], ids, begins, Hq, Hkv, D, bs, sliding_window=window, do_write=False)
+    assert np.isfinite(out).all()
+    scale = 1.0 / np.sqrt(D)
+    for s, (past, n) in enumerate(seqs):
+        t0 = case["subsequence_begins"][s]
+        ctx = past + n
+        table_bad = (ids[begins[s]:begins[s + 1]] < 0) | (ids[begins[s]:begins[s + 1]] >= nb)
+        key_bad = np.repeat(table_bad, bs)[:ctx]
+        k = np.stack([oracle.gather_cache_rows(kc, cache_dtype, good[begins[s]:begins[s + 1]], ctx, h, Hkv, D, bs) for h in range(Hkv)])
+        v = np.stack([oracle.gather_cache_rows(vc, cache_dtype, good[begins[s]:begins[s + 1]], ctx, h, Hkv, D, bs) for h in range(Hkv)])
+        for i in range(n):
+            pos = past + i
+            j = np.arange(ctx)
+            keep = (j <= pos) & ~key_bad
+            if window > 0:
+                keep &= j > pos - window
+            for h in range(Hq):
+                got = out[t0 + i, h * D:(h + 1) * D]
+                if not keep.any():
+                    assert not got.any()
+                    continue
+                sc = scale * (k[h // (Hq // Hkv)][keep].astype(np.float64) @ case["q"][t0 + i, h * D:(h + 1) * D].astype(np.float64))
+                pr = np.exp(sc - sc.max())
+                ref = (pr / pr.sum()) @ v[h // (Hq // Hkv)][keep].astype(np.float64)
+                np.testing.assert_allclose(got, ref, atol=3e-6, rtol=1e-5)
+    assert not out[case["subsequence_begins"][3]].any()  # sequence 3 has no block at all
+    # without holes nothing changed: the same call on the good table equals the dense reduction used above
+    whole = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc.copy(), vc.copy(), cache_dtype, case["past_lens"],
+                                   case["subsequence_begins"], good, begins, Hq, Hkv, D, bs, sliding_window=window, do_write=False)
+    case["kc_after"], case["vc_after"] = kc, vc
+    for s in range(len(seqs)):
+        t0, t1 = case["subsequence_begins"][s], case["subsequence_begins"][s + 1]
+        np.testing.assert_allclose(whole[t0:t1], _dense_reference(oracle, case, s), atol=3e-6, rtol=1e-5)
+
+
 # ---- the operator's second output ("scores") ----------------------------------------------------
 def _dense_keys(oracle, case, s, h):
     pl, bb = case["past_lens"], case["block_indices_begins"]
