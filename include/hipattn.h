@@ -234,6 +234,12 @@ typedef struct hipattn_pa_desc {
     float scale;       /* <= 0 selects 1/sqrt(head_dim) */
     int flags;         /* HIPATTN_PA_* */
     int decode_waves;  /* wavefronts the decode contexts are spread over; 0 = as many as the device keeps resident */
+    /* The operator's alibi_slopes input: NULL, or num_heads_q floats in device memory.  slope[h] * (j - p) is
+     * added to the scaled score of cache position j for a token at position p (ALiBi's linear distance bias;
+     * sign and origin restated from the operator's documentation, not checked against OpenVINO).  The decode
+     * kernels and the shape-generic kernels take it as one multiply-add per score; multi-token sequences then
+     * go to the plain query-tile kernel rather than the tuned chunk kernel, one kernel after the other. */
+    const float* alibi_slopes;
 } hipattn_pa_desc;
 
 hipattn_status hipattn_paged_attention_workspace_size(const hipattn_pa_desc* desc, size_t* bytes);
@@ -306,9 +312,9 @@ hipattn_status hipattn_profile_dominant_kernel(hipattn_event before, hipattn_eve
  *                                 work is cut into equal pieces (5)
  *   "decode_dyn_pieces_per_wave"  on-demand pieces per wavefront for the last quarter of the
  *                                 decode work (0 = none)
- *   "decode_fused_merge"          where pieces of several wavefronts make up one (sequence, kv head): 2: the
- *                                 decode kernel combines them itself; 0: a merge launch behind it; 1 (default):
- *                                 the kernel for u8 caches, the launch for 16-bit ones (whichever measured faster)
+ *   "decode_fused_merge"          where pieces of several wavefronts make up one (sequence, kv head): 1 (default):
+ *                                 the u8 decode kernels combine them themselves (no merge launch); 0: a merge
+ *                                 launch behind every decode kernel (what 16-bit caches always get)
  *   "sdpa_padded_rows"            1 (default): dense SDPA at head sizes below 128 (multiples of 8) runs the
  *                                 tuned head-128 kernel on rows of fewer columns; 0: the plain kernels
  * HIPATTN_<NAME IN CAPITALS> in the environment gives an option its initial value; the

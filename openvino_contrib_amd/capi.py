@@ -78,6 +78,7 @@ class PaDesc(ctypes.Structure):
         ("scale", ctypes.c_float),
         ("flags", ctypes.c_int),
         ("decode_waves", ctypes.c_int),
+        ("alibi_slopes", ctypes.c_void_p),  # device pointer to num_heads_q floats, or None
     ]
 
 

@@ -19,6 +19,13 @@ struct NoBias {
     __device__ __forceinline__ float operator()(int) const { return 0.0f; }
 };
 
+// ALiBi: slope * (key position - query position).
+struct DistanceBias {
+    float slope;
+    int pos;
+    __device__ __forceinline__ float operator()(int j) const { return slope * (float)(j - pos); }
+};
+
 // One row of an attention mask: element j at row + j * stride (stride 0: broadcast over the keys).
 // Boolean masks (u8, nonzero = the key takes part) become 0 / -inf; float masks are added to the
 // scaled scores, as ScaledDotProductAttention specifies.
@@ -189,7 +196,10 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void paged_generic_kernel(Page
     int j0 = 0;
     if (p.sliding_window > 0 && pos - p.sliding_window + 1 > 0) j0 = pos - p.sliding_window + 1;
     float o[kGenericSlots];
-    attend_row_wave(q_lds[wave], kv, NoBias{}, j0, j1, D, p.scale, o);
+    if (p.alibi_slopes)
+        attend_row_wave(q_lds[wave], kv, DistanceBias{p.alibi_slopes[h], pos}, j0, j1, D, p.scale, o);
+    else
+        attend_row_wave(q_lds[wave], kv, NoBias{}, j0, j1, D, p.scale, o);
 #pragma unroll
     for (int sl = 0; sl < kGenericSlots; sl++) {
         const int d = lane + 64 * sl;

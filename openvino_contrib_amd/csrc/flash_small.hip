@@ -179,6 +179,8 @@ struct Work {
     int num_blocks;
     int64_t block_stride;   // bytes from one cache block to the next
     float scale;
+    const float* alibi;     // paged: nullptr, or the ALiBi slope of row 0's query head; row r's is alibi[r * alibi_step]
+    int alibi_step;         // 0: every row belongs to one head; 1: the rows are consecutive query heads
     const uint8_t* mask;    // kMask: the mask row of query row 0 (this batch, this head)
     int64_t mask_row_stride, mask_key_stride;  // in elements
     int mask_dtype;
@@ -407,6 +409,20 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
                     for (int e = 0; e < 4; e++) s[mt][4 * g + e] += m4[e];
                 }
         }
+        // ALiBi: slope * (key - query position) joins the score (an exponent to base 2 here).  The slope is
+        // fetched where it is used: held across the loop it would cost the larger builds a spilled register.
+        if constexpr (kPaged) {
+            if (w.alibi != nullptr) {
+                const float slope = *(const volatile float*)(w.alibi + min(my_row, w.rows - 1) * w.alibi_step) * kLog2e;
+#pragma unroll
+                for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int key = ts + mt * 32 + 8 * (r >> 2) + 4 * hi + (r & 3);
+                        s[mt][r] = fmaf(slope, (float)(key - my_pos), s[mt][r]);
+                    }
+            }
+        }
         // mask: keys past the end, keys after the query under the causal flag, keys that have left
         // the window (the tile holds one for some row of the wavefront when its first key lies
         // before the window of the wavefront's last row)
@@ -527,6 +543,8 @@ __device__ __forceinline__ void sdpa_small_tile(const SdpaParams& p, uint8_t (*l
     w.num_blocks = 0;
     w.block_stride = 0;
     w.scale = p.scale;
+    w.alibi = nullptr;
+    w.alibi_step = 0;
     w.mask = nullptr;
     w.mask_row_stride = w.mask_key_stride = 0;
     w.mask_dtype = 0;
@@ -613,6 +631,8 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))
     w.num_blocks = p.num_blocks;
     w.block_stride = (int64_t)p.num_heads_kv * p.block_size * row_bytes;
     w.scale = p.scale;
+    w.alibi = p.alibi_slopes ? p.alibi_slopes + (heads_as_rows ? h * G : h) : nullptr;
+    w.alibi_step = heads_as_rows ? 1 : 0;
     w.mask = nullptr;
     w.mask_row_stride = w.mask_key_stride = 0;
     w.mask_dtype = 0;

@@ -127,6 +127,7 @@ hipattn::PagedParams make_paged_params(const hipattn_pa_desc* d) {
     p.scale = resolve_scale(d->scale, d->head_dim);
     p.num_waves = d->decode_waves > 0 ? d->decode_waves : 0;
     p.any_lengths = (d->flags & HIPATTN_PA_ANY_LENGTHS) ? 1 : 0;
+    p.alibi_slopes = d->alibi_slopes;
     return p;
 }
 
@@ -558,6 +559,7 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention_scores(const hipattn_pa_de
     if (!q || !key_cache || !past_lens || !subsequence_begins || !block_indices || !block_indices_begins || !scores)
         return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_scores: null pointer");
     if (desc->num_seqs > 65535) return fail(HIPATTN_UNSUPPORTED, "paged_attention_scores: %d sequences (at most 65535)", desc->num_seqs);
+    if (desc->alibi_slopes) return fail(HIPATTN_UNSUPPORTED, "paged_attention_scores: no distance bias (alibi_slopes) in the scores kernels");
     const size_t need = (size_t)desc->num_tokens * desc->num_heads_q * sizeof(float);
     if (!workspace || workspace_bytes < need)
         return fail(HIPATTN_WORKSPACE_TOO_SMALL, "paged_attention_scores: workspace of %zu bytes, %zu needed", workspace_bytes, need);

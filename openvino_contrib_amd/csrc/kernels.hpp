@@ -93,6 +93,7 @@ struct PagedParams {
     int max_context_len;
     int sliding_window;
     float scale;  // already resolved (> 0)
+    const float* alibi_slopes;  // nullptr, or [num_heads_q]: slope * (key position - query position) joins the scaled score
     // decode: the batch's block-heads are cut into num_waves equal pieces (one per wavefront);
     // pieces that do not cover a whole (sequence, kv head) segment leave partials in the workspace
     int num_waves;        // wavefronts (= single-wavefront workgroups) of the decode kernel

@@ -372,9 +372,15 @@ struct WaveState {
 
 // kTileMask (blocks of 16): `tiles_in` has bit t set when tile t of the unit lies in a block of the
 // cache; with blocks of 32 both tiles always do and the argument is ignored.
-template <bool kU8, bool kBf16, int kHD = kD, bool kTileMask = false>
+// kAlibi: slopes holds the ALiBi slopes of the group's query heads (`heads` of them; lane n16 serves head n16),
+// and slope * (token - last attended token) joins the scaled score.  The slope is fetched where it is used:
+// the loop has no register left to hold it (a constant added to a whole row leaves its softmax alone,
+// so the distance may be measured from the row's last attended token instead of its own position).
+// A template argument rather than a test of the pointer: the test alone cost the u8 kernel 1.3 %.
+template <bool kU8, bool kBf16, int kHD = kD, bool kTileMask = false, bool kAlibi = false>
 __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, const typename Op16<kBf16>::vec8 (&qf)[4], float sumq,
-                                              float c, int tok_base, int j0, int ctx, int kg, int tiles_in = 3) {
+                                              float c, int tok_base, int j0, int ctx, int kg, int tiles_in = 3,
+                                              const float* slopes = nullptr, int heads = 0) {
     const int tiles = kTileMask ? tiles_in : 3;
     // ---- S^T = K Q^T : two tiles of 16 tokens x 16 heads
     float4_t s[2];
@@ -440,8 +446,18 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
             }
             x = (tok >= j0 && tok < ctx && ((tiles >> t) & 1)) ? x * c : -INFINITY;
             sv[j] = x;
-            mloc = fmaxf(mloc, x);
+            if constexpr (!kAlibi) mloc = fmaxf(mloc, x);
         }
+    if constexpr (kAlibi) {
+        const int n16 = (int)threadIdx.x & 15;
+        const float slope = *(const volatile float*)(slopes + (n16 < heads ? n16 : 0)) * kLog2e;
+        const float first = (float)(tok_base + kg * 4 - (ctx - 1));
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            sv[j] = fmaf(slope, first + (float)((j >> 2) * 16 + (j & 3)), sv[j]);
+            mloc = fmaxf(mloc, sv[j]);
+        }
+    }
     mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
     const float m_new = fmaxf(st.m, mloc);  // finite: every processed block holds an attended token
@@ -875,8 +891,12 @@ constexpr int kSelfPlanMaxRows = 256;
 // head sizes between 64 and 128, kPad), the self-planning form on blocks of 32 or 16 only.
 // kPad: the call's head size (p.head_dim, a multiple of 8) may be smaller than kHD: the missing columns of
 // Q are zeros and those of V are not read.
-template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false>
+template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false, bool kAlibi = false>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
+    static_assert(!kAlibi || (kWaves == 1 && !kSelfPlan), "the distance bias (p.alibi_slopes) exists in the ordinary launch only");
+    // The merge inside the kernel (p.fused_merge) is built into the u8 instantiations only: the 16-bit ones use
+    // every register in their loop, and with that code behind the loop the allocator spilled 29 of them.
+    constexpr bool kFusedBuilt = kU8;
     static_assert(!(kU8 && kBf16), "u8 caches are dequantised to fp16 operands");
     static_assert(!kPad || (!kSelfPlan && (kWaves == 1 || (kHD == 128 && !kU8))), "padded head sizes: no self-planning form; eight wavefronts for 16-bit caches in the head-128 build");
     static_assert(kHD == 128 || (!kSelfPlan && kWaves == 1), "head size 64 has the ordinary launch only");
@@ -1012,7 +1032,9 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         L = from;
         // the segment ends here and began in an earlier piece: this piece combines it when it is done
         // (one scalar carried through the loop; the rest is worked out again then)
-        if (p.fused_merge && !whole && b_rel + n == nb) merge_seg = s * Hkv + h;
+        if constexpr (kFusedBuilt) {
+            if (p.fused_merge && !whole && b_rel + n == nb) merge_seg = s * Hkv + h;
+        }
         const int lb0 = rg.j0 / kUnit + b_rel;          // first unit of 32 tokens
         // (kBlk == 0: the table is indexed by the block of the absolute unit, lb0 + ... >> log2(units per block))
         const int32_t* table = p.block_indices + rg.table_begin + (kBlk ? lb0 * kEntries : 0);
@@ -1067,6 +1089,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         st.corr = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; e++) st.acc[e] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        const float* const slopes = kAlibi ? p.alibi_slopes + h * G : nullptr;  // ALiBi, this group's heads
 
         // units in groups of 64 table entries: one vector load fetches the group's block-table entries
         constexpr int kGroup = 64 / kEntries;
@@ -1111,10 +1134,10 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                 int i = 0;
                 while (i < gn) {
                     ok_b = (i + 1 < gn) ? issue(rb, i + 1) : 0;
-                    if (ok_a) process_block<kU8, kBf16, kHD, kEntries != 1>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kUnit, rg.j0, rg.ctx, kg, ok_a);
+                    if (ok_a) process_block<kU8, kBf16, kHD, kEntries != 1, kAlibi>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kUnit, rg.j0, rg.ctx, kg, ok_a, slopes, G);
                     if (i + 1 >= gn) break;
                     ok_a = (i + 2 < gn) ? issue(ra, i + 2) : 0;
-                    if (ok_b) process_block<kU8, kBf16, kHD, kEntries != 1>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kUnit, rg.j0, rg.ctx, kg, ok_b);
+                    if (ok_b) process_block<kU8, kBf16, kHD, kEntries != 1, kAlibi>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kUnit, rg.j0, rg.ctx, kg, ok_b, slopes, G);
                     i += 2;
                 }
             } else {
@@ -1134,7 +1157,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                         constexpr int kLast = kStages - 1;
                         ok[(u + kLast) % kStages] =
                             (idx + kLast < gn) ? issue(regs[(u + kLast) % kStages], idx + kLast) : 0;
-                        if (ok[u]) process_block<kU8, kBf16, kHD, kEntries != 1>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kUnit, rg.j0, rg.ctx, kg, ok[u]);
+                        if (ok[u]) process_block<kU8, kBf16, kHD, kEntries != 1, kAlibi>(st, regs[u], qf, sumq, c, (lb0 + g0 + idx) * kUnit, rg.j0, rg.ctx, kg, ok[u], slopes, G);
                     }
                 }
             }
@@ -1163,10 +1186,10 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                 }
                 const int d0 = (kg * 4 + r) * 8;
                 // (rows of the accumulator beyond the head size hold nothing; a fused partial carries them all the same)
-                if ((kPad || kHD < 128) && d0 >= head_dim && (whole || !p.fused_merge)) continue;
+                if ((kPad || kHD < 128) && d0 >= head_dim && (whole || !(kFusedBuilt && p.fused_merge))) continue;
                 if (whole) {
                     store_out8(p.out, ((int64_t)rg.token * p.num_heads_q + h * G + n16) * head_dim + d0, p.out_dtype, o);
-                } else if (p.fused_merge) {
+                } else if (kFusedBuilt && p.fused_merge) {
                     float* rec = p.part_out + (slot * kPartPairs * 4 * G + (kg * G + n16)) * 2;
 #pragma unroll
                     for (int e2 = 0; e2 < 4; e2++) agent_store2(rec + (r * 4 + e2) * 8 * G, o[2 * e2], o[2 * e2 + 1]);
@@ -1176,14 +1199,14 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     *(float4*)(po + 4) = make_float4(o[4], o[5], o[6], o[7]);
                 }
             }
-            if (!whole && p.fused_merge) {
+            if (kFusedBuilt && !whole && p.fused_merge) {
                 agent_store2(p.part_out + (slot * kPartPairs * 4 * G + (kg * G + n16)) * 2 + 16 * 8 * G, st.m, l);
             } else if (!whole && kg == 0) {
                 p.part_ml[(slot * G + n16) * 2] = st.m;
                 p.part_ml[(slot * G + n16) * 2 + 1] = l;
             }
         }
-        if (p.fused_merge && !whole && b_rel + n < nb) {
+        if (kFusedBuilt && p.fused_merge && !whole && b_rel + n < nb) {
             // a partial another wavefront will combine: announced once the stores above have completed
             // (no load is in flight at the end of a segment, so the wait is for these stores alone)
             stores_done();
@@ -1192,7 +1215,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         }
         L += n;
     }
-    if (merge_seg >= 0) {
+    if (kFusedBuilt && merge_seg >= 0) {
         stores_done();  // this wavefront's own partial of that segment
         const int ms = merge_seg / Hkv, mh = merge_seg - ms * Hkv;
         DecodeRange mr;
@@ -1742,9 +1765,9 @@ Option g_options[] = {
     {"mixed_decode_share_percent", "HIPATTN_MIXED_DECODE_SHARE_PERCENT", 100, 10, 1000, {100}},
     // 1: dense SDPA at head sizes below 128 runs the tuned head-128 kernel on rows of fewer columns; 0: the plain kernels
     {"sdpa_padded_rows", "HIPATTN_SDPA_PADDED_ROWS", 1, 0, 1, {1}},
-    // 2: the decode kernel combines the partials of split segments itself; 0: a merge launch behind it;
-    // 1: whichever measured faster (the kernel itself for u8 caches, the launch for 16-bit ones)
-    {"decode_fused_merge", "HIPATTN_DECODE_FUSED_MERGE", 1, 0, 2, {1}},
+    // 1: the decode kernels that have the code for it (u8 caches) combine the partials of split segments
+    // themselves; 0: a merge launch behind every decode kernel
+    {"decode_fused_merge", "HIPATTN_DECODE_FUSED_MERGE", 1, 0, 1, {1}},
 };
 enum { kOptMixedOverlap = 0, kOptSwitchCost, kOptDynPieces, kOptSharePercent, kOptSdpaPadded, kOptFusedMerge };
 
@@ -1783,6 +1806,7 @@ bool paged_fast_supported(const PagedParams& p) {
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
     // (head sizes below 64 / between 64 and 128: the head-64 / head-128 kernel with zero columns)
     if (p.block_size < 16 || (p.block_size & (p.block_size - 1)) != 0) return false;  // 16, 32, or a larger power of two
+    if (p.alibi_slopes && p.head_dim > 128) return false;  // (the head-256 decode kernel has no distance term: the query-tile kernel takes the batch)
     // (above 128: paged_decode256_kernel)
     return p.head_dim >= 8 && p.head_dim <= 256 && p.head_dim % 8 == 0 &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
@@ -1823,7 +1847,7 @@ static int query_tile_bound(const PagedParams& p) {
 static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p.num_tokens : p.num_seqs; }
 
 static bool overlap_wanted(const PagedParams& p) {
-    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream) return false;
+    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream || p.alibi_slopes) return false;
     // the eight-wavefront decode kernel: head size 128, and 16-bit caches at the head sizes between 64 and 128
     if (p.head_dim != kD && !(p.head_dim > 64 && p.head_dim < kD && p.cache_dtype != HIPATTN_U8)) return false;
     return option(kOptMixedOverlap) != 0;
@@ -1911,11 +1935,9 @@ void paged_fast_plan(PagedParams& p, void* workspace) {
     p.part_flag = (uint64_t*)w;
     w += align_up(slots * sizeof(uint64_t), 256);
     // the head-256 kernel and on-demand pieces (whose order of completion is not that of their numbers) keep the merge launch
-    // Measured (whole steps, same machine): the 128-sequence u8 batch 0.450 ms fused against 0.454 ms with the
-    // launch; the 64-sequence fp16 batch 0.223 against 0.219 ms -- its kernel has no register to spare, and what
-    // the merge code adds is paid at every wavefront's start.
-    const int fused = option(kOptFusedMerge);
-    p.fused_merge = ((fused == 2 || (fused == 1 && p.cache_dtype == HIPATTN_U8)) && p.dyn_pieces == 0 && p.head_dim <= 128) ? 1 : 0;
+    // Built into the u8 kernels only (see kFusedBuilt).  Measured, whole steps on one machine: the 128-sequence
+    // u8 batch 0.450 ms fused against 0.454 ms with the merge launch.
+    p.fused_merge = (option(kOptFusedMerge) != 0 && p.cache_dtype == HIPATTN_U8 && p.dyn_pieces == 0 && p.head_dim <= 128) ? 1 : 0;
     p.merge_tag = next_merge_tag();
 }
 
@@ -2030,6 +2052,17 @@ void release_side_stream(hipStream_t owner) {
 // admits; head sizes other than 128 have the ordinary form only, blocks of more than 32 tokens no self-planning form).
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan, int kHD, bool kPad>
 static void launch_decode_blk(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block, hipStream_t stream) {
+    if constexpr (kWaves == 1 && !kSelfPlan) {
+        if (p.alibi_slopes) {  // the instantiations with the distance bias
+            if (p.block_size == 32)
+                hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, 1, false, kHD, 32, kPad, true>), grid, block, 0, stream, p, wp, do_write);
+            else if (p.block_size == 16)
+                hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, 1, false, kHD, 16, kPad, true>), grid, block, 0, stream, p, wp, do_write);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, 1, false, kHD, 0, kPad, true>), grid, block, 0, stream, p, wp, do_write);
+            return;
+        }
+    }
     if (p.block_size == 32) {
         hipLaunchKernelGGL((paged_decode_kernel<kU8, kBf16, kWaves, kSelfPlan, kHD, 32, kPad>), grid, block, 0, stream, p, wp, do_write);
     } else if (p.block_size == 16) {
@@ -2105,7 +2138,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     // A pure decode batch of few rows is one launch less: the decode wavefronts plan for themselves
     // and write the new rows (see kSelfPlanMaxRows).
     const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 && p.head_dim == kD &&
-                           p.block_size <= 32 && (!write || wp.vector_rows);
+                           p.block_size <= 32 && (!write || wp.vector_rows) && !p.alibi_slopes;
     if (self_plan) {
         if (probe.before) (void)hipEventRecord(probe.before, stream);
         launch_decode<1, true>(p, wp, write ? 1 : 0, dim3(p.num_waves), dim3(64), stream);
@@ -2122,7 +2155,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     // Shapes without the eight-wavefront decode kernel run the two parts side by side all the same when
     // the decode wavefronts take at most half of every compute unit's registers (and no LDS), so that the
     // chunks' workgroups find room beside them.
-    const bool beside = p.max_q_tiles > 0 && !p.overlap && !p.no_side_stream && option(kOptMixedOverlap) != 0 &&
+    const bool beside = p.max_q_tiles > 0 && !p.overlap && !p.no_side_stream && !p.alibi_slopes && option(kOptMixedOverlap) != 0 &&
                         p.num_waves * 2 <= resident_decode_waves();
     if (p.max_q_tiles > 0 && (p.overlap || beside)) {
         // Mixed batch: the decode sequences stream from HBM on a few compute units while the

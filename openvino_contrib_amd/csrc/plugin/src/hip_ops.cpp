@@ -271,8 +271,11 @@ public:
             if (node.get_input_element_type(i) != ov::element::i32) HIP_PLUGIN_THROW(who + "index inputs must be i32");
         if (node.get_input_partial_shape(kKeyCache).size() != 4)
             HIP_PLUGIN_THROW(who + "key_cache must be [num_blocks, num_kv_heads, block_size, head_size]");
-        if (!statically_empty(node.get_input_partial_shape(kAlibiSlopes)))
-            HIP_PLUGIN_THROW(who + "alibi_slopes are not supported (expected shape [0])");
+        // alibi_slopes: empty, or one f32 slope per query head (checked against the head count at run time)
+        if (node.get_input_element_type(kAlibiSlopes) != ov::element::f32 && !statically_empty(node.get_input_partial_shape(kAlibiSlopes)))
+            HIP_PLUGIN_THROW(who + "alibi_slopes must be f32");
+        if (node.get_input_partial_shape(kAlibiSlopes).rank().is_static() && node.get_input_partial_shape(kAlibiSlopes).size() != 1)
+            HIP_PLUGIN_THROW(who + "alibi_slopes must be a vector ([0] or [query heads])");
         out1_type_ = num_outputs_ > 1 ? node.get_output_element_type(1) : ov::element::dynamic;
     }
 
@@ -302,7 +305,7 @@ public:
     std::vector<size_t> UpdatedInputs() const override { return {kKeyCache, kValueCache}; }
     // launch parameters, and inputs that must be empty: none of them is handed to a kernel
     bool InputIsHostOnly(size_t input) const override {
-        return input == kScale || input == kSlidingWindow || input == kAlibiSlopes || input == kMaxContextLen ||
+        return input == kScale || input == kSlidingWindow || input == kMaxContextLen ||
                (input >= kPaRequiredInputs && input != kScoreAggregationWindow);
     }
 
@@ -392,6 +395,12 @@ private:
         d.max_context_len = host_scalar<int32_t>(in[kMaxContextLen], "max_context_len", 0, false);
         d.flags = 0;  // any split of the tokens over the sequences comes out right without a hint
         d.decode_waves = 0;
+        if (ov::shape_size(in[kAlibiSlopes].shape) > 0) {
+            HIP_PLUGIN_ASSERT(ov::shape_size(in[kAlibiSlopes].shape) == (size_t)d.num_heads_q,
+                              "alibi_slopes must hold one value per query head (" + std::to_string(d.num_heads_q) + "), got " +
+                                  shape_str(in[kAlibiSlopes].shape));
+            d.alibi_slopes = (const float*)in[kAlibiSlopes].device;
+        }
         return d;
     }
     ov::element::Type q_type_, kv_type_, cache_type_, out1_type_;

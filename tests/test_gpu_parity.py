@@ -495,8 +495,8 @@ def test_paged_decode_sliding_window(hip, oracle, cache_dtype, window):
 
 @pytest.mark.parametrize("env", [{"decode_dyn_pieces_per_wave": 4}, {"decode_switch_cost": 0},
                                  {"decode_dyn_pieces_per_wave": 2, "decode_switch_cost": 9},
-                                 {"decode_fused_merge": 2}, {"decode_fused_merge": 0},
-                                 {"decode_fused_merge": 2, "decode_switch_cost": 0}])
+                                 {"decode_fused_merge": 1}, {"decode_fused_merge": 0},
+                                 {"decode_fused_merge": 1, "decode_switch_cost": 0}])
 @pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
 def test_paged_decode_schedule_knobs(hip, oracle, env, cache_dtype, schedule_options):
     """The schedule of the decode kernel (on-demand pieces, segment-start cost) never changes results."""
@@ -512,12 +512,12 @@ def test_paged_decode_schedule_knobs(hip, oracle, env, cache_dtype, schedule_opt
     dev.free()
 
 
-@pytest.mark.parametrize("fused", [0, 2])
+@pytest.mark.parametrize("fused", [0, 1])
 @pytest.mark.parametrize("D,bs,Hq,Hkv,cache_dtype", [(128, 32, 32, 8, W.F16), (128, 16, 16, 8, W.BF16), (128, 32, 128, 8, W.U8),
                                                      (64, 32, 8, 8, W.F16), (96, 64, 24, 8, W.F16), (40, 16, 16, 4, W.U8),
                                                      (128, 128, 64, 8, W.U8), (72, 32, 14, 2, W.BF16)])
 def test_paged_decode_merge_inside_the_kernel_and_behind_it(hip, oracle, fused, D, bs, Hq, Hkv, cache_dtype, schedule_options):
-    """Segments that several wavefronts share are combined by the decode kernel itself or by the merge launch:
+    """Segments that several wavefronts share are combined by the decode kernel itself (u8 caches) or by the merge launch:
     both against the oracle, at wavefront counts from fewer than segments to many per segment, one call after
     the other (the allocator hands the freed workspace out again, so a call meets the flags of the one before)."""
     announce("paged decode merge", fused, D, bs, Hq, Hkv, cache_dtype)
@@ -1104,6 +1104,62 @@ def test_paged_chunks_take_no_key_from_a_block_outside_the_cache(hip, oracle, D,
     kc, vc = dev.caches()
     np.testing.assert_array_equal(kc, okc)
     np.testing.assert_array_equal(vc, ovc)
+    dev.free()
+
+
+def alibi_slopes(Hq):
+    """ALiBi's geometric slopes, 2^(-8 h / Hq) for h = 1..Hq (any head count: the formula, not the paper's rule for
+    counts that are not powers of two)."""
+    return (2.0 ** (-8.0 * np.arange(1, Hq + 1) / Hq)).astype(np.float32)
+
+
+@pytest.mark.parametrize("D,bs,Hq,Hkv,q_dtype,cache_dtype,path", [
+    (128, 32, 32, 8, W.F16, W.F16, "paged_mfma"), (128, 16, 16, 8, W.BF16, W.BF16, "paged_mfma"), (128, 32, 64, 8, W.F16, W.U8, "paged_mfma"),
+    (128, 64, 8, 2, W.BF16, W.F16, "paged_mfma"), (64, 32, 8, 8, W.F16, W.F16, "paged_mfma"), (96, 16, 12, 4, W.F16, W.U8, "paged_mfma"),
+    (256, 32, 8, 2, W.F16, W.F16, "paged_mfma_tiles"), (80, 8, 8, 2, W.F16, W.F16, "paged_mfma_tiles"), (128, 16, 40, 2, W.BF16, W.U8, "paged_mfma_tiles"),
+    (64, 16, 4, 2, W.F32, W.F32, "paged_generic"), (72, 32, 6, 3, W.F16, W.F32, "paged_generic")])
+@pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 300), ("mixed", 0), ("mixed", 70), ("prefill", 0)])
+def test_paged_attention_with_alibi_slopes(hip, oracle, D, bs, Hq, Hkv, q_dtype, cache_dtype, path, kind, window):
+    """The operator's alibi_slopes input: slope[h] * (j - p) joins the scaled scores in the decode kernels, the
+    query-tile kernel (which takes the multi-token sequences of such a call) and the shape-generic kernels; all
+    against the oracle, whose distance term is pinned by a torch fixture.  Slopes of zero change nothing."""
+    announce("paged alibi", D, bs, Hq, Hkv, q_dtype, cache_dtype, kind, window)
+    if kind == "decode":
+        seqs = [(c - 1, 1) for c in DECODE_CTX]
+    elif kind == "mixed":
+        seqs = [(0, 9), (37, 1), (31, 2), (5, 140), (64, 1), (700, 1), (15, 1), (300, 130), (0, 1), (1000, 3)]
+    else:
+        seqs = [(0, 200), (0, 16), (3, 17), (0, 1)]
+    case = W.make_paged_case(97, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    slopes = alibi_slopes(Hq)
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    ref = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc, vc, cache_dtype, case["past_lens"],
+                                 case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
+                                 sliding_window=window, alibi_slopes=slopes)
+    plain, _, _ = H.oracle_paged(oracle, case)
+    assert np.abs(plain - ref).max() > 1e-2  # the bias matters on these contexts
+    dev = H.PagedDeviceCase(hip, case)
+    dslopes = hip.DeviceBuffer.from_numpy(slopes)
+    tol = 1e-4 if q_dtype == W.F32 else (1e-2 if (cache_dtype in (W.U8, W.BF16) or q_dtype == W.BF16) else 2e-3)
+    for waves in (0, 9):
+        out, got_path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if waves else 0, alibi=dslopes)
+        assert got_path == path
+        assert np.isfinite(out).all()
+        assert H.scaled_bound_error(out, ref, "paged alibi") <= tol, waves
+    kc_dev, vc_dev = dev.caches()
+    np.testing.assert_array_equal(kc_dev, kc)
+    np.testing.assert_array_equal(vc_dev, vc)
+    gen, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC, alibi=dslopes)
+    assert path_g == "paged_generic" and H.scaled_bound_error(gen, ref, "paged alibi, generic") <= tol
+    dzero = hip.DeviceBuffer.from_numpy(np.zeros(Hq, np.float32))
+    out0, _ = dev.run(flags=hip.PA_SKIP_CACHE_WRITE, alibi=dzero)
+    out1, _ = dev.run(flags=hip.PA_SKIP_CACHE_WRITE)
+    if path == "paged_mfma" and kind == "decode":
+        np.testing.assert_array_equal(out0, out1)  # the same kernel, the same arithmetic plus zeros
+    else:
+        assert H.scaled_bound_error(out0, plain, "paged alibi, zero slopes") <= tol
+    for b in (dslopes, dzero):
+        b.free()
     dev.free()
 
 

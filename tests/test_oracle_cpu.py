@@ -380,6 +380,48 @@ def test_paged_attention_takes_no_key_from_a_block_outside_the_pool(oracle, cach
         np.testing.assert_allclose(whole[t0:t1], _dense_reference(oracle, case, s), atol=3e-6, rtol=1e-5)
 
 
+ALIBI_GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "alibi_golden.npz")
+
+
+@pytest.mark.parametrize("name", ["decode", "chunk", "prefill", "window"])
+@pytest.mark.parametrize("block_size", [4, 16])
+def test_paged_attention_alibi_matches_torch_fixture(oracle, name, block_size):
+    """alibi_slopes: slope[h] * (j - p) added to the scaled scores.  The fixture is torch's fp64
+    scaled_dot_product_attention with that bias as an explicit mask on dense K/V; here the same K/V rows sit in
+    a paged f32 cache behind a shuffled block table (the new tokens come in through the operator's own write)."""
+    z = np.load(ALIBI_GOLDEN)
+    Hq, Hkv, D, past, n, window = (int(x) for x in z[name + "/meta"])
+    q, k, v, slopes = z[name + "/q"][0], z[name + "/k"][0], z[name + "/v"][0], z[name + "/slopes"]
+    ctx = past + n
+    nblk = (ctx + block_size - 1) // block_size
+    rng = np.random.default_rng(5)
+    table = rng.permutation(nblk + 3)[:nblk].astype(np.int32)
+    kc = np.zeros((nblk + 3, Hkv, block_size, D), np.float32)
+    vc = np.zeros_like(kc)
+    for j in range(past):  # the cached tokens; the new ones are written by the call
+        kc[table[j // block_size], :, j % block_size] = k[:, j]
+        vc[table[j // block_size], :, j % block_size] = v[:, j]
+    kc8, vc8 = kc.view(np.uint8).reshape(nblk + 3, Hkv, block_size, D * 4), vc.view(np.uint8).reshape(nblk + 3, Hkv, block_size, D * 4)
+    k_new = k[:, past:].transpose(1, 0, 2).reshape(n, Hkv * D)
+    v_new = v[:, past:].transpose(1, 0, 2).reshape(n, Hkv * D)
+    out = oracle.paged_attention(q.transpose(1, 0, 2).reshape(n, Hq * D), k_new, v_new, kc8, vc8, W.F32,
+                                 np.array([past], np.int32), np.array([0, n], np.int32), table, np.array([0, nblk], np.int32),
+                                 Hq, Hkv, D, block_size, sliding_window=window, alibi_slopes=slopes)
+    ref = z[name + "/out"][0].transpose(1, 0, 2).reshape(n, Hq * D)
+    np.testing.assert_allclose(out, ref, atol=3e-6, rtol=1e-5)
+    # the bias matters (the fixture is not met without it), and slopes of zero are no bias
+    kc8b, vc8b = kc8.copy(), vc8.copy()
+    plain = oracle.paged_attention(q.transpose(1, 0, 2).reshape(n, Hq * D), k_new, v_new, kc8b, vc8b, W.F32,
+                                   np.array([past], np.int32), np.array([0, n], np.int32), table, np.array([0, nblk], np.int32),
+                                   Hq, Hkv, D, block_size, sliding_window=window)
+    if ctx > 2:
+        assert np.abs(plain - ref).max() > 1e-3
+    zero = oracle.paged_attention(q.transpose(1, 0, 2).reshape(n, Hq * D), k_new, v_new, kc8b, vc8b, W.F32,
+                                  np.array([past], np.int32), np.array([0, n], np.int32), table, np.array([0, nblk], np.int32),
+                                  Hq, Hkv, D, block_size, sliding_window=window, alibi_slopes=np.zeros(Hq, np.float32), do_write=False)
+    np.testing.assert_array_equal(zero, plain)
+
+
 # ---- the operator's second output ("scores") ----------------------------------------------------
 def _dense_keys(oracle, case, s, h):
     pl, bb = case["past_lens"], case["block_indices_begins"]

@@ -110,7 +110,7 @@ def test_paged_attention_takes_the_operators_full_signature():
     unknown_inputs = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=9, extra_len=0)
     assert "paged_attention" not in plugin.query_model(unknown_inputs)
     alibi = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, alibi_len=32)
-    assert "paged_attention" not in plugin.query_model(alibi)
+    assert "paged_attention" in plugin.query_model(alibi)  # one slope per query head: ALiBi
 
 
 def test_import_model_rejects_a_foreign_stream():
