@@ -100,6 +100,9 @@ int hip_compiled_model_create_infer_request(hip_compiled_model_t* compiled, hip_
 void hip_infer_request_destroy(hip_infer_request_t* request); /* waits for a pending start_async */
 int hip_infer_request_set_input(hip_infer_request_t* request, int index, void* data, int on_device, int dtype,
                                 int rank, const int64_t* shape);
+/* set_tensors: `count` host tensors of `shape` (first extent 1), one batch entry each, for one input */
+int hip_infer_request_set_input_batch(hip_infer_request_t* request, int index, void* const* data, int count, int dtype,
+                                      int rank, const int64_t* shape);
 int hip_infer_request_set_output(hip_infer_request_t* request, int index, void* data, int on_device, int dtype,
                                  int rank, const int64_t* shape);
 int hip_infer_request_infer(hip_infer_request_t* request);
@@ -110,6 +113,9 @@ int hip_infer_request_cancel(hip_infer_request_t* request);
 int hip_infer_request_output_info(hip_infer_request_t* request, int index, int* dtype, int* rank, int64_t* shape,
                                   size_t* bytes);
 int hip_infer_request_copy_output(hip_infer_request_t* request, int index, void* dst, size_t dst_bytes);
+/* get_runtime_model: "node_name|layerType|execOrder|execTimeMcs|runtimePrecision|primitiveType" per line, in
+ * execution order; execTimeMcs is the average over the infers profiled so far, or "not_executed" */
+int hip_compiled_model_runtime_info(hip_compiled_model_t* compiled, char* text, size_t text_size);
 /* "node_name|node_type|microseconds" per line */
 int hip_infer_request_profiling(hip_infer_request_t* request, char* text, size_t text_size);
 /* variable states (query_state; src/cuda_variable_state.hpp:62-105) */

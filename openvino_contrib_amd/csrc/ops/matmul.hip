@@ -2,7 +2,9 @@
 // are row-major; hipBLASLt is column-major, so the product is taken transposed
 // (C^T = op(B)^T * op(A)^T) with the operands swapped and no data movement.  Descriptors and the
 // algorithm are kept per (device, shape), so a repeated shape costs one hipblasLtMatmul call; the
-// algorithm is the fastest of the heuristic's candidates, timed once when the shape is first seen.
+// algorithm is the fastest of the heuristic's candidates, timed once when the shape is first seen
+// outside a stream capture (that call synchronises with its stream; calls on other devices are not
+// held up by it: every device has a lock of its own).
 #include <hipblaslt/hipblaslt.h>
 
 #include <map>
@@ -22,16 +24,34 @@ struct Plan {
     hipblasLtMatrixLayout_t first = nullptr, second = nullptr, result = nullptr;
     hipblasLtMatmulAlgo_t algo{};
     size_t workspace = 0;
+    bool tuned = false;  // false: the heuristic's first candidate (picked under a stream capture); timed by the next call outside one
+    void destroy() {
+        if (desc) hipblasLtMatmulDescDestroy(desc);
+        if (first) hipblasLtMatrixLayoutDestroy(first);
+        if (second) hipblasLtMatrixLayoutDestroy(second);
+        if (result) hipblasLtMatrixLayoutDestroy(result);
+        desc = nullptr;
+        first = second = result = nullptr;
+    }
+};
+// destroys what a plan under construction holds unless it reaches the cache
+struct PlanGuard {
+    Plan& plan;
+    bool keep = false;
+    ~PlanGuard() {
+        if (!keep) plan.destroy();
+    }
 };
 
 using Key = std::tuple<int, int, int, int64_t, int64_t, int64_t, int64_t, int, int, int64_t, int64_t, size_t>;
 
 struct DeviceState {
+    std::mutex mutex;  // the handle and the plans of this device
     hipblasLtHandle_t handle = nullptr;
     std::map<Key, Plan> plans;
 };
 
-std::mutex g_mutex;
+std::mutex g_mutex;  // the map of devices only
 std::map<int, DeviceState> g_devices;  // never destroyed: the library may outlive static teardown order
 
 bool blas_type(int dtype, hipDataType* t) {
@@ -96,14 +116,27 @@ hipattn_status matmul(const hipops_matmul_desc* d, const void* a, const void* b,
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) return fail(HIPATTN_NO_DEVICE, "matmul: no current device");
 
-    std::lock_guard<std::mutex> lock(g_mutex);
-    DeviceState& dev = g_devices[device];
+    DeviceState* dev_ptr = nullptr;
+    {
+        std::lock_guard<std::mutex> devices_lock(g_mutex);
+        dev_ptr = &g_devices[device];  // (map nodes do not move)
+    }
+    DeviceState& dev = *dev_ptr;
+    std::lock_guard<std::mutex> lock(dev.mutex);
     if (!dev.handle) BLAS_CHECK(hipblasLtCreate(&dev.handle));
     const Key key{device, d->ab_dtype, d->c_dtype, d->m, d->n, d->k, d->batch, d->transpose_a != 0, d->transpose_b != 0,
                   d->batch_stride_a, d->batch_stride_b, workspace_bytes};
     auto it = dev.plans.find(key);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    const bool can_time = hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone;
+    if (it != dev.plans.end() && !it->second.tuned && can_time) {  // picked under a capture: time the candidates now
+        it->second.destroy();
+        dev.plans.erase(it);
+        it = dev.plans.end();
+    }
     if (it == dev.plans.end()) {
         Plan plan;
+        PlanGuard guard{plan};
         hipDataType ab, ct;
         blas_type(d->ab_dtype, &ab);
         blas_type(d->c_dtype, &ct);
@@ -146,8 +179,7 @@ hipattn_status matmul(const hipops_matmul_desc* d, const void* a, const void* b,
         // The heuristic's order is a guess: the first time a shape is seen, and unless the stream is
         // being captured, every candidate runs a few times on the caller's own operands (each writes the
         // same C) and the fastest is kept.  A candidate that fails to run is skipped.
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (usable > 1 && hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
+        if (usable > 1 && can_time) {
             hipEvent_t e0 = nullptr, e1 = nullptr;
             if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
                 const float one = 1.0f, zero = 0.0f;
@@ -173,7 +205,9 @@ hipattn_status matmul(const hipops_matmul_desc* d, const void* a, const void* b,
         }
         plan.algo = found[pick].algo;
         plan.workspace = found[pick].workspaceSize;
+        plan.tuned = can_time || usable <= 1;
         it = dev.plans.emplace(key, plan).first;
+        guard.keep = true;
     }
     const Plan& plan = it->second;
     const float alpha = 1.0f, beta = 0.0f;

@@ -125,6 +125,11 @@ public:
     // shape pattern, an order): a tensor all of whose consumers say so is not uploaded, and its
     // TensorView::device is null.
     virtual bool InputIsHostOnly(size_t /*input*/) const { return false; }
+    // False for a host-side input whose VALUE changes nothing the operator launches (a bound that is only
+    // advisory): the request leaves such a value out of the signature by which it recognises a repeat of
+    // the previous infer, so that a value that moves with every step does not keep it from replaying the
+    // recorded graph.
+    virtual bool InputValueShapesLaunch(size_t /*input*/) const { return true; }
     // Told once, while the model is compiled, that nothing consumes this output: an operator may then
     // skip producing it (the scores of PagedAttentionExtension).
     virtual void MarkOutputUnused(size_t /*output*/) {}

@@ -309,6 +309,11 @@ public:
                (input >= kPaRequiredInputs && input != kScoreAggregationWindow);
     }
 
+    // max_context_len is advisory for the attention kernels; only the scores kernels size a grid by it
+    bool InputValueShapesLaunch(size_t input) const override {
+        return input != kMaxContextLen || (scores_wanted_ && num_outputs_ > 1);
+    }
+
     WorkbufferRequest GetWorkBufferRequest(const std::vector<TensorView>& inputs) const override {
         const hipattn_pa_desc d = describe(inputs);
         size_t bytes = 0;

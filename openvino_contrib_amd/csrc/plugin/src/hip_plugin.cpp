@@ -18,6 +18,7 @@
 #include "openvino/op/read_value.hpp"
 #include "openvino/op/result.hpp"
 #include "openvino/pass/serialize.hpp"
+#include "openvino/runtime/exec_model_info.hpp"
 #include "openvino/runtime/icore.hpp"
 #include "openvino/runtime/internal_properties.hpp"
 
@@ -293,7 +294,7 @@ Configuration Plugin::get_full_config(const ov::AnyMap& properties, bool throw_o
 
 std::shared_ptr<ov::threading::ITaskExecutor> Plugin::get_stream_executor(const Configuration& config) const {
     std::lock_guard<std::mutex> lock(mutex_);
-    auto& pool = device_thread_pool_[config.device_id];
+    auto& pool = device_thread_pool_[{config.device_id, config.num_streams}];
     if (!pool) pool = std::make_shared<ThreadPool>(config.device_id, (unsigned)config.num_streams);
     return pool;
 }
@@ -498,6 +499,21 @@ CompiledModel::CompiledModel(const std::shared_ptr<const ov::Model>& model, cons
     }
     for (const auto& kv : host_only)
         if (kv.second) host_only_tensors_.insert(kv.first);
+    // tensors whose host-side value no consumer's launches depend on (OperationBase::InputValueShapesLaunch)
+    std::map<TensorID, bool> advisory;
+    for (const auto& step : exec_sequence_) {
+        const auto& in_ids = step.op->GetInputIds();
+        for (size_t i = 0; i < in_ids.size(); i++) {
+            const bool here = !step.op->InputValueShapesLaunch(i);
+            auto it = advisory.find(in_ids[i]);
+            if (it == advisory.end())
+                advisory[in_ids[i]] = here;
+            else
+                it->second = it->second && here;
+        }
+    }
+    for (const auto& kv : advisory)
+        if (kv.second) advisory_value_tensors_.insert(kv.first);
 }
 
 std::shared_ptr<ov::ISyncInferRequest> CompiledModel::create_sync_infer_request() const {
@@ -531,6 +547,35 @@ ov::Any CompiledModel::get_property(const std::string& name) const {
         return all;
     }
     return config_.get(name);
+}
+
+void CompiledModel::record_execution_time(const std::string& node_name, uint64_t microseconds) const {
+    std::lock_guard<std::mutex> lock(perf_mutex_);
+    auto& entry = perf_[node_name];
+    entry.first += microseconds;
+    entry.second += 1;
+}
+
+std::shared_ptr<const ov::Model> CompiledModel::get_runtime_model() const {
+    auto model = model_->clone();
+    size_t exec_order = 0;
+    std::lock_guard<std::mutex> lock(perf_mutex_);
+    for (const auto& op : model->get_ordered_ops()) {
+        auto& info = op->get_rt_info();
+        info[ov::exec_model_info::LAYER_TYPE] = std::string(op->get_type_info().name);
+        info[ov::exec_model_info::EXECUTION_ORDER] = std::to_string(exec_order++);
+        info[ov::exec_model_info::IMPL_TYPE] = std::string("HIP");
+        const auto it = perf_.find(op->get_friendly_name());
+        const bool timed = config_.enable_profiling && it != perf_.end() && it->second.second > 0 && it->second.first > 0;
+        info[ov::exec_model_info::PERF_COUNTER] = timed ? std::to_string(it->second.first / it->second.second) : std::string("not_executed");
+        info[ov::exec_model_info::ORIGINAL_NAMES] = op->get_friendly_name();
+        std::string precisions;
+        for (size_t i = 0; i < op->get_output_size(); i++) precisions += (i ? "," : "") + op->get_output_element_type(i).get_type_name();
+        info[ov::exec_model_info::OUTPUT_PRECISIONS] = precisions;
+        info[ov::exec_model_info::RUNTIME_PRECISION] =
+            op->get_output_size() ? op->get_output_element_type(0).get_type_name() : std::string("undefined");
+    }
+    return model;
 }
 
 void CompiledModel::export_model(std::ostream& model_stream) const {
@@ -601,7 +646,54 @@ void InferRequest::infer() {
     infer_postprocess();
 }
 
+void InferRequest::set_tensors_impl(const ov::Output<const ov::Node> port, const std::vector<ov::SoPtr<ov::ITensor>>& tensors) {
+    for (const auto& input : get_inputs()) {
+        if (!(input == port)) continue;
+        OPENVINO_ASSERT(!tensors.empty(), "set_tensors: no tensors for input '", port.get_node()->get_friendly_name(), "'");
+        const ov::Shape& first = tensors[0]->get_shape();
+        for (const auto& t : tensors) {
+            OPENVINO_ASSERT(t, "set_tensors: a tensor is not initialized");
+            OPENVINO_ASSERT(std::dynamic_pointer_cast<RemoteTensor>(t._ptr) == nullptr,
+                            "set_tensors: device tensors cannot be put together into a batch; pass one tensor");
+            OPENVINO_ASSERT(port.get_element_type().compatible(t->get_element_type()), "set_tensors: element type ",
+                            t->get_element_type(), " does not match the input's ", port.get_element_type());
+            OPENVINO_ASSERT(!first.empty() && first[0] == 1 && t->get_shape() == first,
+                            "set_tensors: every tensor must hold one batch entry of the same shape, got ", t->get_shape());
+        }
+        ov::Shape whole = first;
+        whole[0] = tensors.size();
+        OPENVINO_ASSERT(port.get_partial_shape().compatible(ov::PartialShape(whole)), "set_tensors: ", tensors.size(),
+                        " tensors of shape ", first, " do not fit the input's ", port.get_partial_shape());
+        batched_tensors_[{port.get_node(), port.get_index()}] = tensors;
+        return;
+    }
+    OPENVINO_THROW("Cannot find input tensors for port ", port.get_node()->get_friendly_name());
+}
+
+// (a single tensor set later replaces a batch set before)
+void InferRequest::set_tensor(const ov::Output<const ov::Node>& port, const ov::SoPtr<ov::ITensor>& tensor) {
+    ov::ISyncInferRequest::set_tensor(port, tensor);
+    batched_tensors_.erase({port.get_node(), port.get_index()});
+}
+
+// The batches set with set_tensors become one host tensor each, entry after entry along the first axis
+// (what ISyncInferRequest::convert_batched_tensors does for the reference, src/cuda_infer_request.cpp:111).
+void InferRequest::bind_batched_tensors() {
+    for (const auto& input : get_inputs()) {
+        const auto it = batched_tensors_.find({input.get_node(), input.get_index()});
+        if (it == batched_tensors_.end()) continue;
+        const auto& parts = it->second;
+        ov::Shape whole = parts[0]->get_shape();
+        whole[0] = parts.size();
+        auto joined = ov::make_tensor(parts[0]->get_element_type(), whole);
+        const size_t bytes = parts[0]->get_byte_size();
+        for (size_t i = 0; i < parts.size(); i++) std::memcpy((uint8_t*)joined->data() + i * bytes, parts[i]->data(), bytes);
+        ov::ISyncInferRequest::set_tensor(input, ov::SoPtr<ov::ITensor>{joined, nullptr});
+    }
+}
+
 void InferRequest::infer_preprocess() {
+    bind_batched_tensors();
     check_tensors();
     cancellation_.reset();
 }
@@ -800,12 +892,12 @@ void InferRequest::execute_steps(const InferenceRequestContext& context, bool pr
 // small; the shapes cover what larger host tensors decide (the extent of the scores output).
 std::vector<uint64_t> InferRequest::make_signature() const {
     std::vector<uint64_t> sig;
-    auto add_view = [&](const TensorView& v) {
+    auto add_view = [&](const TensorView& v, bool value_matters = true) {
         sig.push_back((uint64_t)(uintptr_t)v.device);
         sig.push_back(v.shape.size());
         for (size_t d : v.shape) sig.push_back(d);
         const size_t bytes = v.byte_size();
-        if (v.host != nullptr && bytes > 0 && bytes <= 64) {
+        if (v.host != nullptr && bytes > 0 && bytes <= 64 && value_matters) {
             uint64_t words[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             std::memcpy(words, v.host, bytes);
             sig.insert(sig.end(), words, words + (bytes + 7) / 8);
@@ -813,9 +905,14 @@ std::vector<uint64_t> InferRequest::make_signature() const {
             sig.push_back(v.host != nullptr);
         }
     };
-    for (const auto& ps : prepared_) {
-        for (const auto& v : ps.in) add_view(v);
-        for (const auto& v : ps.out) add_view(v);
+    const auto& sequence = compiled_->exec_sequence();
+    for (size_t si = 0; si < prepared_.size(); si++) {
+        const auto& ps = prepared_[si];
+        // (small host-side values are part of the signature unless every consumer says the value is advisory)
+        const auto& in_ids = sequence[si].op->GetInputIds();
+        const auto& out_ids = compiled_->output_ids(sequence[si].node.get());
+        for (size_t i = 0; i < ps.in.size(); i++) add_view(ps.in[i], i >= in_ids.size() || !compiled_->has_advisory_value(in_ids[i]));
+        for (size_t o = 0; o < ps.out.size(); o++) add_view(ps.out[o], o >= out_ids.size() || !compiled_->has_advisory_value(out_ids[o]));
         for (size_t i = 0; i < ps.workbuffers.mutable_buffers.size(); i++) {
             sig.push_back((uint64_t)(uintptr_t)ps.workbuffers.mutable_buffers[i]);
             sig.push_back(ps.workbuffers.mutable_sizes[i]);
@@ -839,6 +936,7 @@ void InferRequest::infer_postprocess() {
         info.node_type = step.op->GetTypeName();
         info.exec_type = "HIP";
         profiling_.push_back(info);
+        compiled_->record_execution_time(info.node_name, (uint64_t)info.real_time.count());
     }
 }
 

@@ -156,7 +156,10 @@ public:
                   const std::shared_ptr<ov::threading::ITaskExecutor>& wait_executor,
                   const std::shared_ptr<const ov::IPlugin>& plugin, bool loaded_from_cache);
 
-    std::shared_ptr<const ov::Model> get_runtime_model() const override { return model_; }
+    // the model with execution information in every node's rt_info (src/cuda_compiled_model.cpp:336-371)
+    std::shared_ptr<const ov::Model> get_runtime_model() const override;
+    // what an infer request measured for one operator (profiling on): feeds the runtime model's execTimeMcs
+    void record_execution_time(const std::string& node_name, uint64_t microseconds) const;
     void export_model(std::ostream& model) const override;
     std::shared_ptr<ov::IAsyncInferRequest> create_infer_request() const override;
     void set_property(const ov::AnyMap& properties) override;
@@ -171,6 +174,8 @@ public:
     const std::vector<TensorID>& output_ids(const ov::Node* node) const { return output_ids_.at(node); }
     // no consumer of this tensor reads it on the device (OperationBase::InputIsHostOnly)
     bool is_host_only(TensorID id) const { return host_only_tensors_.count(id) != 0; }
+    // every consumer takes this tensor's host-side value as advisory (OperationBase::InputValueShapesLaunch)
+    bool has_advisory_value(TensorID id) const { return advisory_value_tensors_.count(id) != 0; }
     const Configuration& config() const { return config_; }
     const ov::ParameterVector& parameters() const { return exec_model_->get_parameters(); }
     const ov::ResultVector& results() const { return exec_model_->get_results(); }
@@ -189,8 +194,11 @@ private:
     std::vector<ExecStep> exec_sequence_;
     std::map<const ov::Node*, std::vector<TensorID>> output_ids_;  // per node: one TensorID per output port
     std::set<TensorID> host_only_tensors_;
+    std::set<TensorID> advisory_value_tensors_;
     size_t num_tensors_ = 0;
     mutable std::atomic<size_t> graphs_captured_{0}, graph_launches_{0};
+    mutable std::mutex perf_mutex_;
+    mutable std::map<std::string, std::pair<uint64_t, uint64_t>> perf_;  // node name -> (microseconds in all, runs)
 };
 
 class InferRequest : public ov::ISyncInferRequest {
@@ -201,6 +209,10 @@ public:
     void infer() override;
     std::vector<ov::SoPtr<ov::IVariableState>> query_state() const override;
     std::vector<ov::ProfilingInfo> get_profiling_info() const override;
+    // several tensors, one batch entry each, for one input (src/cuda_infer_request.cpp:263-272): kept per
+    // port and put together along the batch axis when the request runs (infer_preprocess)
+    void set_tensors_impl(const ov::Output<const ov::Node> port, const std::vector<ov::SoPtr<ov::ITensor>>& tensors) override;
+    void set_tensor(const ov::Output<const ov::Node>& port, const ov::SoPtr<ov::ITensor>& tensor) override;
 
     // stages of the asynchronous pipeline (src/cuda_infer_request.cpp:107-254)
     void infer_preprocess();
@@ -212,6 +224,8 @@ public:
 private:
     std::shared_ptr<const CompiledModel> compiled_;
     std::shared_ptr<ov::threading::ITaskExecutor> wait_executor_;
+    std::map<std::pair<const ov::Node*, size_t>, std::vector<ov::SoPtr<ov::ITensor>>> batched_tensors_;
+    void bind_batched_tensors();
     std::vector<TensorView> views_;               // per TensorID, rebuilt by every infer
     std::vector<Allocation> tensor_buffers_;      // per TensorID, grow-only
     Allocation workbuffer_;                       // scratch arena shared by the steps of one infer
@@ -303,7 +317,9 @@ private:
     int device_count_ = 0;
     Configuration config_;
     mutable std::mutex mutex_;
-    mutable std::map<int, std::shared_ptr<ThreadPool>> device_thread_pool_;
+    // one pool of stream-owning workers per (device, NUM_STREAMS): compiled models that ask for different
+    // numbers of streams get pools of their own size
+    mutable std::map<std::pair<int, int>, std::shared_ptr<ThreadPool>> device_thread_pool_;
 };
 
 }  // namespace hip_gpu

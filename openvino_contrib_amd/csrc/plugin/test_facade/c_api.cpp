@@ -10,6 +10,7 @@
 
 #include "hip_operation.hpp"
 #include "hip_plugin.hpp"
+#include "openvino/runtime/exec_model_info.hpp"
 #include "openvino/op/add.hpp"
 #include "openvino/op/assign.hpp"
 #include "openvino/op/constant.hpp"
@@ -368,6 +369,16 @@ API int hip_infer_request_set_input(hip_infer_request_t* request, int index, voi
         request->impl->set_tensor(ports[index], wrap(request, data, on_device, dtype, rank, shape));
     });
 }
+API int hip_infer_request_set_input_batch(hip_infer_request_t* request, int index, void* const* data, int count, int dtype,
+                                          int rank, const int64_t* shape) {
+    return guarded([&] {
+        const auto& ports = request->impl->get_inputs();
+        if (index < 0 || (size_t)index >= ports.size()) OPENVINO_THROW("input index ", index, " is out of range");
+        std::vector<ov::SoPtr<ov::ITensor>> tensors;
+        for (int i = 0; i < count; i++) tensors.push_back(wrap(request, data[i], 0, dtype, rank, shape));
+        request->impl->set_tensors(ports[index], tensors);
+    });
+}
 API int hip_infer_request_set_output(hip_infer_request_t* request, int index, void* data, int on_device, int dtype,
                                      int rank, const int64_t* shape) {
     return guarded([&] {
@@ -405,6 +416,20 @@ API int hip_infer_request_copy_output(hip_infer_request_t* request, int index, v
         auto t = request->impl->get_tensor(request->impl->get_outputs().at(index));
         if (dst_bytes < t->get_byte_size()) OPENVINO_THROW("destination too small");
         if (t->get_byte_size()) std::memcpy(dst, t->data(), t->get_byte_size());
+    });
+}
+API int hip_compiled_model_runtime_info(hip_compiled_model_t* compiled, char* text, size_t text_size) {
+    return guarded([&] {
+        std::string all;
+        const auto model = compiled->impl->get_runtime_model();
+        for (const auto& op : model->get_ordered_ops()) {
+            const auto& info = op->get_rt_info();
+            const auto field = [&](const char* key) { return info.count(key) ? info.at(key).as<std::string>() : std::string("?"); };
+            all += op->get_friendly_name() + "|" + field(ov::exec_model_info::LAYER_TYPE) + "|" + field(ov::exec_model_info::EXECUTION_ORDER) +
+                   "|" + field(ov::exec_model_info::PERF_COUNTER) + "|" + field(ov::exec_model_info::RUNTIME_PRECISION) + "|" +
+                   field(ov::exec_model_info::IMPL_TYPE) + "\n";
+        }
+        copy_out(all, text, text_size);
     });
 }
 API int hip_infer_request_profiling(hip_infer_request_t* request, char* text, size_t text_size) {

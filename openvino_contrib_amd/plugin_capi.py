@@ -38,9 +38,11 @@ SYMBOLS = {
     "hip_compiled_model_input_name": (_i, [_vp, _i, ctypes.c_char_p, _sz]),
     "hip_compiled_model_get_property": (_i, [_vp, _cp, ctypes.c_char_p, _sz]),
     "hip_compiled_model_export": (_i, [_vp, _vp, _sz, _P(_sz)]),
+    "hip_compiled_model_runtime_info": (_i, [_vp, ctypes.c_char_p, _sz]),
     "hip_compiled_model_create_infer_request": (_i, [_vp, _P(_vp)]),
     "hip_infer_request_destroy": (None, [_vp]),
     "hip_infer_request_set_input": (_i, [_vp, _i, _vp, _i, _i, _i, _i64p]),
+    "hip_infer_request_set_input_batch": (_i, [_vp, _i, _P(_vp), _i, _i, _i, _i64p]),
     "hip_infer_request_set_output": (_i, [_vp, _i, _vp, _i, _i, _i, _i64p]),
     "hip_infer_request_infer": (_i, [_vp]),
     "hip_infer_request_start_async": (_i, [_vp]),
@@ -199,6 +201,14 @@ class InferRequest:
         _check(lib().hip_infer_request_set_input(self.handle, index, array.ctypes.data_as(_vp), 0, dtype, array.ndim,
                                                  _shape(array.shape)))
 
+    def set_input_batch(self, index, arrays, dtype):
+        """set_tensors: one host tensor per batch entry (each of shape [1, ...]), wrapped, not copied."""
+        arrays = [np.asarray(a, dtype=_NP[dtype], order="C") for a in arrays]
+        self._keep[index] = arrays
+        ptrs = (_vp * len(arrays))(*[a.ctypes.data_as(_vp) for a in arrays])
+        shape = arrays[0].shape if arrays else (1,)
+        _check(lib().hip_infer_request_set_input_batch(self.handle, index, ptrs, len(arrays), dtype, len(shape), _shape(shape)))
+
     def set_device_input(self, index, device_ptr, dtype, shape):
         _check(lib().hip_infer_request_set_input(self.handle, index, device_ptr, 1, dtype, len(shape), _shape(shape)))
 
@@ -274,6 +284,10 @@ class CompiledModel:
 
     def num_outputs(self):
         return lib().hip_compiled_model_num_outputs(self.handle)
+
+    def runtime_info(self):
+        """get_runtime_model: (node name, layerType, execOrder, execTimeMcs, runtimePrecision, primitiveType) per node."""
+        return [tuple(line.split("|")) for line in _text(lib().hip_compiled_model_runtime_info, self.handle, size=65536).splitlines()]
 
     def export_model(self):
         """The bytes CompiledModel::export_model writes."""

@@ -69,6 +69,69 @@ def test_sdpa_dynamic_shapes_one_compiled_model(hip, oracle):
         compiled.create_infer_request().infer()
 
 
+def test_set_tensors_puts_one_tensor_per_batch_entry_together(hip, oracle):
+    """set_tensors on an input (several tensors, one batch entry each, src/cuda_infer_request.cpp:263-272):
+    the request joins them along the batch axis when it runs; a single tensor set later replaces them;
+    tensors that do not fit are refused with an error."""
+    print("[plugin] set_tensors", flush=True)
+    B, Hh, L, D = 3, 4, 40, 64
+    case = W.make_sdpa_case(99, B, Hh, Hh, L, L, D, W.F16)
+    plugin = P.Plugin()
+    compiled = plugin.compile_model(P.Model.sdpa(W.F16, [-1, Hh, -1, D], [-1, Hh, -1, D], True))
+    req = compiled.create_infer_request()
+    req.set_input_batch(0, [case["q_store"][b:b + 1] for b in range(B)], W.F16)
+    req.set_input(1, case["k_store"], W.F16)
+    req.set_input_batch(2, [case["v_store"][b:b + 1] for b in range(B)], W.F16)
+    req.infer()
+    out, _ = req.output(0)
+    ref = oracle.sdpa(case["q"], case["k"], case["v"], causal=True)
+    assert out.shape == (B, Hh, L, D) and H.max_abs(H.storage_to_f32(out, W.F16), ref) <= 2e-3
+    # the tensors are read again by every infer: new values in the same memory, new result
+    case2 = W.make_sdpa_case(100, B, Hh, Hh, L, L, D, W.F16)
+    req.set_input_batch(0, [case2["q_store"][b:b + 1] for b in range(B)], W.F16)
+    req.infer()
+    out2, _ = req.output(0)
+    assert H.max_abs(H.storage_to_f32(out2, W.F16), oracle.sdpa(case2["q"], case["k"], case["v"], causal=True)) <= 2e-3
+    # one tensor for the whole input takes the place of the batch
+    req.set_input(0, case["q_store"], W.F16)
+    req.infer()
+    out3, _ = req.output(0)
+    np.testing.assert_array_equal(out3, out)
+    with pytest.raises(P.PluginError):  # an entry that is more than one batch entry
+        req.set_input_batch(0, [case["q_store"][0:2], case["q_store"][1:3]], W.F16)
+    with pytest.raises(P.PluginError):  # the wrong precision
+        req.set_input_batch(0, [np.zeros((1, Hh, L, D), np.float32)] * 2, W.F32)
+
+
+def test_runtime_model_carries_execution_information(hip, oracle):
+    """get_runtime_model (src/cuda_compiled_model.cpp:336-371): every node with its type, place in the execution
+    order, precision and, with profiling on, the average time of its executions so far."""
+    print("[plugin] runtime model", flush=True)
+    case = W.make_sdpa_case(101, 1, 4, 4, 64, 64, 64, W.F16)
+    plugin = P.Plugin()
+    plugin.set_property("PERF_COUNT", "YES")
+    compiled = plugin.compile_model(P.Model.sdpa(W.F16, [1, 4, 64, 64], [1, 4, 64, 64], True))
+    before = compiled.runtime_info()
+    assert [r[2] for r in before] == [str(i) for i in range(len(before))]
+    assert "ScaledDotProductAttention" in [r[1] for r in before]
+    assert all(r[3] == "not_executed" and r[5] == "HIP" for r in before)
+    req = compiled.create_infer_request()
+    for i, name in enumerate(("q", "k", "v")):
+        req.set_input(i, case[name + "_store"], W.F16)
+    for _ in range(3):
+        req.infer()
+    after = {r[1]: r for r in compiled.runtime_info()}
+    sdpa = after["ScaledDotProductAttention"]
+    assert sdpa[3] != "not_executed" and int(sdpa[3]) > 0 and sdpa[4] == "f16"
+    # without profiling nothing is timed
+    quiet = P.Plugin().compile_model(P.Model.sdpa(W.F16, [1, 4, 64, 64], [1, 4, 64, 64], True))
+    r2 = quiet.create_infer_request()
+    for i, name in enumerate(("q", "k", "v")):
+        r2.set_input(i, case[name + "_store"], W.F16)
+    r2.infer()
+    assert all(r[3] == "not_executed" for r in quiet.runtime_info())
+
+
 MIXED_BATCH = [(0, 130), (37, 1), (500, 1), (100, 257), (999, 1), (64, 1)]
 LOOKS_LIKE_DECODE = [(1500, 1), (100, 2), (31, 0)]  # as many tokens as sequences, but not one each
 
@@ -133,6 +196,97 @@ def test_paged_attention_with_device_resident_cache(hip, oracle, cache_dtype, q_
     assert prof[0][2] > 0
     kc.free()
     vc.free()
+
+
+@pytest.mark.parametrize("cache_dtype,seqs", [(W.F16, MIXED_BATCH), (W.U8, [(700, 1), (31, 1), (1500, 1)])])
+def test_paged_attention_with_alibi_slopes_through_the_plugin(hip, oracle, cache_dtype, seqs):
+    """alibi_slopes with one value per query head: the model is supported, the slopes go to the device with the
+    other inputs and the result is the oracle's with its distance term; an empty input is no bias."""
+    print("[plugin] paged attention with alibi slopes", cache_dtype, flush=True)
+    Hq, Hkv, D, bs = 16, 4, 128, 32
+    case = W.make_paged_case(98, seqs, Hq, Hkv, D, bs, W.F16, W.F16, cache_dtype)
+    slopes = (2.0 ** (-8.0 * np.arange(1, Hq + 1) / Hq)).astype(np.float32)
+    plugin = P.Plugin()
+    model = P.Model.paged_attention(W.F16, W.F16, cache_dtype, Hq, Hkv, D, bs, alibi_len=Hq)
+    assert "paged_attention" in plugin.query_model(model)
+    compiled = plugin.compile_model(model)
+    kc_ref, vc_ref = case["key_cache"].copy(), case["value_cache"].copy()
+    ref = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc_ref, vc_ref, cache_dtype, case["past_lens"],
+                                 case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
+                                 alibi_slopes=slopes)
+    kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
+    vc = hip.DeviceBuffer.from_numpy(case["value_cache"])
+    req = compiled.create_infer_request()
+    elem_shape = list(case["key_cache"].shape[:3]) + [case["key_cache"].shape[3] // hip.DTYPE_BYTES[cache_dtype]]
+    for i, a in enumerate((case["q_store"], case["k_new_store"], case["v_new_store"])):
+        req.set_input(i, a, W.F16)
+    req.set_device_input(3, kc.ptr, cache_dtype, elem_shape)
+    req.set_device_input(4, vc.ptr, cache_dtype, elem_shape)
+    for i, n in enumerate(("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")):
+        req.set_input(5 + i, case[n], P.I32)
+    req.set_input(9, np.zeros((0,), np.float32), W.F32)
+    req.set_input(10, np.array([0], np.int32), P.I32)
+    req.set_input(11, slopes, W.F32)
+    req.set_input(12, np.array([case["max_context_len"]], np.int32), P.I32)
+    req.infer()
+    out, _ = req.output(0)
+    tol = 1e-2 if cache_dtype == W.U8 else 2e-3
+    assert H.scaled_bound_error(H.storage_to_f32(out, W.F16), ref, "plugin alibi") <= tol
+    np.testing.assert_array_equal(kc.download(np.uint8, case["key_cache"].shape), kc_ref)
+    with pytest.raises(P.PluginError):  # one slope per query head, or none
+        req.set_input(11, slopes[:3], W.F32)
+        req.infer()
+    kc.free()
+    vc.free()
+
+
+def test_decode_steps_replay_the_graph_while_the_context_bound_grows(hip, oracle):
+    """A decode loop as a server runs it: every tensor device-resident, past_lens advanced in place, and
+    max_context_len (a host scalar, advisory for the attention kernels) one larger every step.  The steps
+    after the second replay the recorded graph all the same, and the last one still matches the oracle."""
+    print("[plugin] decode loop under graph replay", flush=True)
+    from openvino_contrib_amd import device_case as DC
+    Hq, Hkv, D, bs = 16, 4, 128, 32
+    past0 = [700, 64, 1500, 33]
+    steps = 5
+    # room in the block tables for the tokens of every step
+    case = W.make_paged_case(102, [(p + steps, 1) for p in past0], Hq, Hkv, D, bs, W.F16, W.F16, W.F16)
+    dev = DC.PagedDeviceCase(hip, case)
+    plugin = P.Plugin()
+    compiled = plugin.compile_model(P.Model.paged_attention(W.F16, W.F16, W.F16, Hq, Hkv, D, bs), {"HIP_GRAPH_MIN_OPERATORS": "1"})
+    req = compiled.create_infer_request()
+    T, S = case["T"], case["S"]
+    cache_shape = list(case["key_cache"].shape[:3]) + [D]
+    req.set_device_input(0, dev.q.ptr, W.F16, [T, Hq * D])
+    req.set_device_input(1, dev.k_new.ptr, W.F16, [T, Hkv * D])
+    req.set_device_input(2, dev.v_new.ptr, W.F16, [T, Hkv * D])
+    req.set_device_input(3, dev.key_cache.ptr, W.F16, cache_shape)
+    req.set_device_input(4, dev.value_cache.ptr, W.F16, cache_shape)
+    req.set_device_input(5, dev.past_lens.ptr, P.I32, [S])
+    req.set_device_input(6, dev.subsequence_begins.ptr, P.I32, [S + 1])
+    req.set_device_input(7, dev.block_indices.ptr, P.I32, [len(case["block_indices"])])
+    req.set_device_input(8, dev.block_indices_begins.ptr, P.I32, [S + 1])
+    req.set_input(9, np.zeros((0,), np.float32), W.F32)
+    req.set_input(10, np.array([0], np.int32), P.I32)
+    req.set_input(11, np.zeros((0,), np.float32), W.F32)
+    req.set_device_output(0, dev.out.ptr, W.F16, [T, Hq * D])
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    launches = []
+    for step in range(steps):
+        lens = np.array([p + step for p in past0], np.int32)
+        dev.past_lens.upload(lens)
+        req.set_input(12, np.array([int(lens.max()) + 1], np.int32), P.I32)  # grows with every step
+        req.infer()
+        launches.append(int(compiled.get_property("HIP_GRAPH_LAUNCHES")))
+        ref = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc, vc, W.F16, lens, case["subsequence_begins"],
+                                     case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs)
+        out = H.storage_to_f32(dev.out.download(np.uint16, (T, Hq * D)), W.F16)
+        assert H.max_abs(out, ref) <= 2e-3, step
+    assert launches == [0, 1, 2, 3, 4], launches  # recorded at the second step, replayed from then on
+    got_kc, got_vc = dev.caches()
+    np.testing.assert_array_equal(got_kc, kc)
+    np.testing.assert_array_equal(got_vc, vc)
+    dev.free()
 
 
 def test_paged_attention_scores_over_an_aggregation_window(hip, oracle):
