@@ -3,8 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer|shapes|decoder|scores|masked] [--no-cpu] [--no-extra] [--no-plugin]
 
-The LAST stdout line is ONE compact JSON object (under 3 KB); the full per-workload records go to
-gpurun_out/bench_detail.json when that folder exists, to stderr otherwise.  The headline is the fp16
+The LAST stdout line is ONE compact JSON object (under 3 KB); the full per-workload records go to the
+file --detail names, or to stderr.  The headline is the fp16
 paged-attention decode step (configuration 3, the one the headline metric is quoted on): a "step" is
 one hipattn_paged_attention call on the whole synthetic batch (KV-cache write of the new tokens +
 split-context decode + merge), inputs resident in HBM.
@@ -747,6 +747,7 @@ def main():
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
                     help="untimed GPU time of the step run ahead of the warmup steps (0 for hardware-counter runs, "
                          "which only count bytes)")
+    ap.add_argument("--detail", default="", help="file for the full per-workload records (default: one line on stderr)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="measure the headline workload only")
     ap.add_argument("--no-plugin", action="store_true", help="skip the timing through the plugin layer")
@@ -891,9 +892,8 @@ def main():
         "workloads": {k: compact_workload(v) for k, v in results.items()},
     }
     detail = dict(line, roofline=head["roofline"], cpu_baseline=cpu if cpu else None, workloads=results)
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
-        with open(os.path.join(out_dir, "bench_detail.json"), "w") as f:
+    if args.detail:
+        with open(args.detail, "w") as f:
             json.dump(detail, f)
     else:
         log("detail:", json.dumps(detail))
