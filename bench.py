@@ -695,7 +695,8 @@ def bench_decoder_layer(hip, steps, warmup):
     weight_bytes = 2 * (hidden * (Hq + 2 * Hkv) * D + hidden * Hq * D + 3 * hidden * ffn)
     kv_bytes = W.paged_kv_bytes(case)
     res = {"workload": "decoder layer (hidden 4096, 32/8 heads of 128, MLP 14336, bf16 weights, fp16 cache) on config3's "
-                       "decode batch through InferRequest::infer, graph replayed",
+                       "decode batch through InferRequest::infer; the same inputs every infer, so every infer after the "
+                       "second replays the recorded graph (a serving loop replays as long as shapes and pointers stay)",
            "ms_per_step": ms, "weight_bytes": weight_bytes, "kv_bytes": kv_bytes, "operators": 13,
            "graphs": graphs, "graph_launches": launches,
            "roofline": {"bound": "hbm", "achieved": (weight_bytes + kv_bytes) / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
