@@ -669,21 +669,36 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
                (t.window <= 0 || ts >= t.pos0 + t.rows - t.window);
     };
     // Paged caches: table entries that name no block of the cache ([0, num_blocks)) stand for keys that
-    // take no part.  Almost no call has one, so every wavefront first looks through the entries of the
-    // workgroup's key range (up to 256 of them, four loads per lane, issued ahead of everything else and
-    // looked at only after the query rows have been converted); the tiles of a range that has one -- or
-    // is longer than that -- get their entries checked one by one (bad_sixteenths).
+    // take no part.  Almost no call has one, so every wavefront looks through the table in windows of 256
+    // entries (four loads per lane and a ballot): the first window of the workgroup's key range is loaded
+    // ahead of everything else and looked at only after the query rows have been converted, later windows
+    // when the loop reaches them (one stall in 64 to 256 key tiles).  Only the tiles of a window that has
+    // such an entry get their own entries checked and their keys masked (bad_sixteenths).
+    constexpr int kScanWindow = 256;
     uint32_t scan_ids[4] = {0u, 0u, 0u, 0u};
-    bool scan_covers = true;
+    int scan_end = 0, last_entry = -1;  // entries below scan_end have been looked at; the range's last entry
+    // a window looked at on the spot (the loop's later windows)
+    auto scan_now = [&](int first) __attribute__((always_inline)) -> bool {
+        bool bad_lane = false;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int e = first + lane + 64 * u;
+            const uint32_t id = e <= last_entry ? (uint32_t)t.table[e] : 0u;
+            bad_lane = bad_lane || id >= (uint32_t)t.num_blocks;
+        }
+        scan_end = first + kScanWindow;
+        return __builtin_amdgcn_ballot_w64(bad_lane) != 0;
+    };
     if constexpr (kPaged) {
         if (t.table != nullptr && t.kv_len > 0) {
-            const int e_lo = kv_lo >> t.block_shift, e_hi = (min(kv_hi, t.kv_len) - 1) >> t.block_shift;
-            scan_covers = e_hi - e_lo < 256;
+            last_entry = (min(kv_hi, t.kv_len) - 1) >> t.block_shift;
+            const int first = kv_lo >> t.block_shift;
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                const int e = e_lo + lane + 64 * u;
-                if (e <= e_hi) scan_ids[u] = (uint32_t)t.table[e];
+                const int e = first + lane + 64 * u;
+                if (e <= last_entry) scan_ids[u] = (uint32_t)t.table[e];
             }
+            scan_end = first + kScanWindow;
         }
     }
 
@@ -926,7 +941,7 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) asm volatile("" : "+v"(qf[i]));  // (converted before the wait below, not after)
-    bool check_blocks = false;  // wave-uniform
+    bool check_blocks = false;  // wave-uniform: the window of the table the loop is in has an entry outside the cache
     if constexpr (kPaged) {
         bool bad_lane = false;
 #pragma unroll
@@ -934,19 +949,41 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             asm volatile("" : "+v"(scan_ids[u]));  // (looked at here, not where they were loaded)
             bad_lane = bad_lane || scan_ids[u] >= (uint32_t)t.num_blocks;
         }
-        check_blocks = !scan_covers || __builtin_amdgcn_ballot_w64(bad_lane) != 0;
+        check_blocks = __builtin_amdgcn_ballot_w64(bad_lane) != 0;
     }
     // which sixteenths of tile j lie in blocks the table does not name (only ever called when check_blocks)
     auto bad_sixteenths = [&](int j) -> uint32_t {
         uint32_t bits = 0;
         if constexpr (kPaged) {
+            const int key0 = kv_lo + j * kTileK;
+            const int32_t* const first = t.table + (key0 >> t.block_shift);
+            const auto bad = [&](int entry) { return (uint32_t)entry >= (uint32_t)t.num_blocks; };
+            if (key0 + kTileK <= t.kv_len && t.block_shift >= 4) {
+                // the whole tile exists: its one, two or four entries in one scalar load (waited for inside the
+                // statement: no LDS read is outstanding at the head of a vector phase)
+                if (t.block_shift >= 6) {
+                    int e0;
+                    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e0) : "s"(first));
+                    bits = bad(e0) ? 0xfu : 0u;
+                } else if (t.block_shift == 5) {
+                    uint2_t e;
+                    asm volatile("s_load_dwordx2 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e) : "s"(first));
+                    bits = (bad((int)e[0]) ? 0x3u : 0u) | (bad((int)e[1]) ? 0xcu : 0u);
+                } else {
+                    uint4_t e;
+                    asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e) : "s"(first));
 #pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const int key0 = kv_lo + j * kTileK + 16 * b;
-                if (key0 >= t.kv_len) continue;  // (keys past the end are masked as such)
-                int entry;
-                asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(entry) : "s"(t.table + (key0 >> t.block_shift)));
-                if ((uint32_t)entry >= (uint32_t)t.num_blocks) bits |= 1u << b;
+                    for (int b = 0; b < 4; b++) bits |= bad((int)e[b]) ? 1u << b : 0u;
+                }
+            } else {
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const int k = key0 + 16 * b;
+                    if (k >= t.kv_len) continue;  // (keys past the end are masked as such)
+                    int entry;
+                    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(entry) : "s"(t.table + (k >> t.block_shift)));
+                    if (bad(entry)) bits |= 1u << b;
+                }
             }
         }
         return bits;
@@ -1002,6 +1039,11 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             tile_softmax<kBf16, kMask>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, true,
                                        mask_tile_staged(j) ? mask_stage(j) : nullptr, row);
         } else if constexpr (kPaged) {
+            // the loop has reached entries nobody has looked at: the next window of the table
+            const int tile_entry = (kv_lo + j * kTileK) >> t.block_shift;
+            if (tile_entry + (kTileK >> t.block_shift) >= scan_end && tile_entry <= last_entry) {
+                check_blocks = scan_now(tile_entry);
+            }
             const uint32_t bad16 = check_blocks ? bad_sixteenths(j) : 0u;
             tile_softmax<kBf16>(t, s, o, st, pf, kv_lo + j * kTileK, my_pos, hi, !unmasked(j) || bad16 != 0, nullptr, 0, bad16);
         } else {

@@ -1150,6 +1150,33 @@ def test_paged_chunks_take_no_key_from_a_block_outside_the_cache(hip, oracle, D,
     dev.free()
 
 
+@pytest.mark.parametrize("bs,cache_dtype,entries", [(16, W.F16, 600), (32, W.U8, 530), (8, W.BF16, 600), (64, W.F16, 300)])
+def test_paged_chunks_find_bad_ids_anywhere_in_a_long_table(hip, oracle, bs, cache_dtype, entries):
+    """The chunk kernel looks through a sequence's table 256 entries at a time; bad entries on either side of
+    those borders, in the last entry and nowhere at all (a sequence of the same length beside it) all match
+    the oracle."""
+    announce("paged chunks, bad ids in a long table", bs, cache_dtype)
+    past = entries * bs + 5
+    seqs = [(past, 130), (past, 130), (17, 64)]
+    qd = W.BF16 if cache_dtype == W.BF16 else W.F16
+    case = W.make_paged_case(101, seqs, 8, 2, 128, bs, qd, qd, cache_dtype)
+    ids, begins, nb = case["block_indices"], case["block_indices_begins"], case["num_blocks"]
+    for e, bad in ((3, -1), (255, nb), (256, nb + 9), (257, -4), (entries - 1, 1 << 29), (511, -1), (512, nb), (599, -2)):
+        if e < entries:
+            ids[begins[0] + e] = bad
+    ids[begins[1] - 1] = nb + 1  # the last entry of the first sequence: some of its new tokens
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case)
+    out, path = dev.run()
+    assert path == ("paged_mfma" if bs >= 16 else "paged_mfma_tiles"), path  # blocks under 16 tokens: the query-tile kernel
+    assert np.isfinite(out).all()
+    assert H.scaled_bound_error(out, ref, "paged chunks, long table") <= (1e-2 if cache_dtype in (W.U8, W.BF16) else 2e-3)
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    dev.free()
+
+
 def alibi_slopes(Hq):
     """ALiBi's geometric slopes, 2^(-8 h / Hq) for h = 1..Hq (any head count: the formula, not the paper's rule for
     counts that are not powers of two)."""
