@@ -1113,7 +1113,12 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                     return 3;
                 } else {
                     const int pb0 = __builtin_amdgcn_readlane(my_pb, 2 * i), pb1 = __builtin_amdgcn_readlane(my_pb, 2 * i + 1);
-                    const int ok = (pb0 >= 0 && pb0 < p.num_blocks ? 1 : 0) | (pb1 >= 0 && pb1 < p.num_blocks ? 2 : 0);
+                    // A tile counts only if it holds an attended token: a unit whose one valid block lies wholly
+                    // ahead of the window (or behind the context) is skipped like a unit without blocks, so that
+                    // every processed unit has a finite score.
+                    const int tok0 = (lb0 + g0 + i) * kUnit;
+                    const int ok = (pb0 >= 0 && pb0 < p.num_blocks && tok0 + 16 > rg.j0 && tok0 < rg.ctx ? 1 : 0) |
+                                   (pb1 >= 0 && pb1 < p.num_blocks && tok0 + 32 > rg.j0 && tok0 + 16 < rg.ctx ? 2 : 0);
                     if (ok == 0) return 0;
                     // a tile without a block is read from the other tile's block: valid memory, and masked
                     const int64_t off0 = (int64_t)((ok & 1) ? pb0 : pb1) * block_stride + head_off;

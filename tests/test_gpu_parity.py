@@ -1049,6 +1049,44 @@ def test_paged_blocks_of_16_skip_blocks_outside_the_cache(hip, oracle, cache_dty
     dev.free()
 
 
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.BF16, W.U8])
+@pytest.mark.parametrize("D", [128, 64, 96, 256])
+def test_paged_blocks_of_16_with_a_window_that_starts_in_a_bad_block(hip, oracle, cache_dtype, D):
+    """Blocks of 16 tokens are read two to a unit.  When the sliding window starts in the second block of
+    a unit and that block's entry names no block, the first block (valid, but wholly ahead of the window)
+    holds no attended token: the unit contributes nothing and the row stays finite.  The same at the other
+    end (context ends in the first block, which is bad) and with both ends in one unit."""
+    announce("paged blocks of 16, window starts in a bad block", cache_dtype, D)
+    window = 64
+    seqs = [(1500, 1), (1500, 1), (200, 1), (70, 1), (17, 1)]
+    qd = W.BF16 if cache_dtype == W.BF16 else W.F16
+    case = W.make_paged_case(107, seqs, 8, 2, D, 16, qd, qd, cache_dtype, sliding_window=window)
+    ids, begins, nb = case["block_indices"], case["block_indices_begins"], case["num_blocks"]
+    # context 1501, window 64: keys 1437..1500, i.e. entries 89..93; entry 88 shares a unit with 89
+    ids[begins[0] + 89] = -9
+    ids[begins[1] + 89] = nb + 1
+    ids[begins[1] + 90] = -1          # the whole next unit as well
+    ids[begins[1] + 91] = nb
+    # context 201: keys 137..200, entries 8..12; entry 12 is the first block of its unit and holds the row's own token
+    ids[begins[2] + 12] = -1
+    # context 71: keys 7..70, entries 0..4
+    ids[begins[3] + 0] = nb + 7
+    # context 18: keys 0..17, entries 0..1 of one unit, the second bad
+    ids[begins[4] + 1] = -2
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    assert np.isfinite(ref).all()
+    dev = H.PagedDeviceCase(hip, case)
+    for waves in (0, 7):
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if waves else 0)
+        assert path == "paged_mfma", path
+        assert np.isfinite(out).all(), waves
+        assert H.scaled_bound_error(out, ref, "blocks of 16, window in a bad block") <= (1e-2 if cache_dtype in (W.U8, W.BF16) else 2e-3)
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    dev.free()
+
+
 @pytest.mark.parametrize("cache_dtype", [W.F16, W.U8])
 @pytest.mark.parametrize("bs", [16, 32])
 def test_paged_head_256_skips_blocks_outside_the_cache(hip, oracle, bs, cache_dtype):
