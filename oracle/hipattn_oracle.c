@@ -530,6 +530,9 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
  * score_window[s] query tokens of the sequence (all of them when score_window is NULL).
  * Reads the cache as it stands (call after the write).  scores must hold
  * sum(past_lens[s] + new_tokens(s)) floats; sequence s starts where s-1 ends.  fp64 throughout.
+ * A table entry outside [0, num_blocks) names no block, as in oracle_paged_attention: its positions
+ * get probability zero and take no part in a row's softmax; a row with nothing left adds nothing
+ * (num_blocks <= 0: every entry is taken as it is).
  * PARITY UNPINNED against OpenVINO (which tokens and heads are aggregated is restated from its
  * operator documentation).  Pinned by: a numpy restatement over a dense gather of the keys, the sum
  * of a sequence's scores (= heads x aggregated tokens), and agreement of the probabilities with
@@ -538,7 +541,7 @@ ORACLE_API int oracle_paged_attention_scores(const float* q, const uint8_t* key_
                                              const int32_t* past_lens, const int32_t* subsequence_begins,
                                              const int32_t* block_indices, const int32_t* block_indices_begins,
                                              const int32_t* score_window, int S, int Hq, int Hkv, int D, int block_size,
-                                             float scale, int sliding_window, float* scores) {
+                                             int num_blocks, float scale, int sliding_window, float* scores) {
     if (S < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || block_size <= 0) return 1;
     if (scale <= 0.0f) scale = 1.0f / sqrtf((float)D);
     const int G = Hq / Hkv;
@@ -560,9 +563,10 @@ ORACLE_API int oracle_paged_attention_scores(const float* q, const uint8_t* key_
         double* acc = (double*)calloc((size_t)ctx, sizeof(double));
         double* sc = (double*)malloc(sizeof(double) * (size_t)ctx);
         float* kbuf = (float*)malloc(sizeof(float) * (size_t)ctx * D);
+        uint8_t* valid = (uint8_t*)malloc((size_t)ctx);
         const int32_t* blocks = block_indices + block_indices_begins[s];
         for (int h = 0; h < Hkv; h++) {
-            oracle_gather_cache_rows(key_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, kbuf);
+            oracle_gather_cache_rows_checked(key_cache, cache_dtype, blocks, ctx, h, Hkv, D, block_size, num_blocks, kbuf, valid);
             for (int i = qlen - w; i < qlen; i++) {
                 const int p = past_lens[s] + i;
                 int j0 = 0, j1 = p + 1 < ctx ? p + 1 : ctx;
@@ -572,13 +576,17 @@ ORACLE_API int oracle_paged_attention_scores(const float* q, const uint8_t* key_
                     const float* qr = q + ((int64_t)(t0 + i) * Hq + (h * G + g)) * D;
                     double m = -INFINITY, l = 0.0;
                     for (int j = j0; j < j1; j++) {
+                        if (!valid[j]) continue;
                         double d = 0.0;
                         for (int e = 0; e < D; e++) d += (double)qr[e] * (double)kbuf[(int64_t)j * D + e];
                         sc[j] = d * (double)scale;
                         if (sc[j] > m) m = sc[j];
                     }
-                    for (int j = j0; j < j1; j++) l += exp(sc[j] - m);
-                    for (int j = j0; j < j1; j++) acc[j] += exp(sc[j] - m) / l;
+                    if (m == -INFINITY) continue; /* every attended position lies in a block the table does not name */
+                    for (int j = j0; j < j1; j++)
+                        if (valid[j]) l += exp(sc[j] - m);
+                    for (int j = j0; j < j1; j++)
+                        if (valid[j]) acc[j] += exp(sc[j] - m) / l;
                 }
             }
         }
@@ -586,6 +594,7 @@ ORACLE_API int oracle_paged_attention_scores(const float* q, const uint8_t* key_
         free(acc);
         free(sc);
         free(kbuf);
+        free(valid);
     }
     free(starts);
     return 0;

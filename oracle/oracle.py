@@ -62,7 +62,7 @@ def lib():
         L.oracle_paged_attention.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                              f32, i32, i32, vp, vp]
         L.oracle_paged_attention.restype = i32
-        L.oracle_paged_attention_scores.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp]
+        L.oracle_paged_attention_scores.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp]
         L.oracle_paged_attention_scores.restype = i32
         L.oracle_rms_norm_f32.argtypes = [vp, vp, vp, i64, i64, f32]
         L.oracle_rms_norm_f32.restype = None
@@ -261,7 +261,7 @@ def paged_attention_scores(q, key_cache, cache_dtype, past_lens, subsequence_beg
     out = np.zeros(total, np.float32)
     rc = lib().oracle_paged_attention_scores(_p(q), _p(key_cache), cache_dtype, _p(pl), _p(sb), _p(bi), _p(bb),
                                              _p(sw) if sw is not None else None, len(pl), Hq, Hkv, D, block_size,
-                                             float(scale), int(sliding_window), _p(out))
+                                             key_cache.shape[0], float(scale), int(sliding_window), _p(out))
     if rc:
         raise ValueError("oracle_paged_attention_scores: bad arguments")
     return out

@@ -1396,6 +1396,33 @@ def test_paged_attention_scores(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, b
     dev.free()
 
 
+@pytest.mark.parametrize("cache_dtype,q_dtype,Hq,Hkv,D,bs", [(W.F16, W.F16, 8, 2, 128, 32), (W.U8, W.BF16, 4, 4, 128, 16),
+                                                             (W.F32, W.F32, 4, 2, 64, 16), (W.BF16, W.BF16, 6, 3, 96, 8)])
+@pytest.mark.parametrize("window", [0, 40])
+def test_paged_attention_scores_with_entries_outside_the_cache(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, bs, window):
+    """The scores output where the table names no block: such positions score zero and the rest of a row's
+    probability stays among the others, as the oracle defines it; a sequence with no valid entry scores zeros."""
+    announce("scores, bad ids", cache_dtype, q_dtype, Hq, Hkv, D, bs, window)
+    seqs = [(300, 5), (0, 70), (650, 1), (12, 4), (100, 1)]
+    case = W.make_paged_case(331, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    ids, begins, nb = case["block_indices"], case["block_indices_begins"], case["num_blocks"]
+    ids[begins[0] + 2] = nb + 1
+    ids[begins[0] + 304 // bs] = -1           # the block of the new tokens
+    ids[begins[1] + 1] = 1 << 30
+    ids[begins[2] + 640 // bs] = -3           # inside the window of the decode row
+    ids[begins[4]:begins[5]] = nb             # every entry of a sequence
+    dev = H.PagedDeviceCase(hip, case)
+    dev.run()
+    got = dev.scores(None)
+    kc, _ = dev.caches()
+    ref = oracle.paged_attention_scores(case["q"], kc, cache_dtype, case["past_lens"], case["subsequence_begins"],
+                                        ids, begins, Hq, Hkv, D, bs, sliding_window=window)
+    assert not ref[-101:].any() and ref[:305].any()
+    bound = 2e-5 * max(1.0, float(ref.max()))
+    assert H.max_abs(got[:ref.size], ref) <= bound, (H.max_abs(got[:ref.size], ref), bound)
+    dev.free()
+
+
 def test_paged_attention_scores_arguments(hip):
     case = W.make_paged_case(310, [(10, 2)], 4, 2, 64, 16, W.F16, W.F16, W.F16)
     dev = H.PagedDeviceCase(hip, case)

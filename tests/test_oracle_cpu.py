@@ -461,6 +461,45 @@ def test_paged_scores_match_a_numpy_restatement(oracle, cache_dtype, window, sco
     np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
 
 
+def test_paged_scores_give_nothing_to_positions_without_a_block(oracle):
+    """Table entries outside the pool: their positions get no probability and the others share a row's
+    whole unit of it, as if those positions were not there (numpy over the remaining keys); a sequence with
+    no valid entry scores zeros."""
+    seqs = [(30, 5), (0, 9), (65, 1), (12, 4)]
+    Hq, Hkv, D, bs = 4, 2, 16, 8
+    case = W.make_paged_case(73, seqs, Hq, Hkv, D, bs, W.F32, W.F32, W.F16)
+    ids, bb, nb = case["block_indices"], case["block_indices_begins"], case["num_blocks"]
+    ids[bb[0] + 1] = nb + 2
+    ids[bb[0] + 4] = -1  # the block of the new tokens
+    ids[bb[2] + 3] = 1 << 30
+    ids[bb[3]:bb[4]] = -5
+    oracle.kv_cache_write(case["k_new"], case["v_new"], case["key_cache"], case["value_cache"], W.F16, case["past_lens"],
+                          case["subsequence_begins"], ids, bb, Hkv, D, bs)
+    got = oracle.paged_attention_scores(case["q"], case["key_cache"], W.F16, case["past_lens"], case["subsequence_begins"],
+                                        ids, bb, Hq, Hkv, D, bs)
+    q = case["q"].reshape(-1, Hq, D).astype(np.float64)
+    ref, start = np.zeros_like(got, dtype=np.float64), 0
+    for s, (past, qlen) in enumerate(seqs):
+        ctx, t0 = past + qlen, case["subsequence_begins"][s]
+        table = ids[bb[s]:bb[s + 1]]
+        there = np.array([0 <= table[j // bs] < nb for j in range(ctx)])
+        safe = np.where((table >= 0) & (table < nb), table, 0).astype(np.int32)
+        for h in range(Hq):
+            K = oracle.gather_cache_rows(case["key_cache"], W.F16, safe, ctx, h // (Hq // Hkv), Hkv, D, bs).astype(np.float64)
+            for i in range(qlen):
+                p = past + i
+                keep = np.nonzero(there[:p + 1])[0]
+                if keep.size == 0:
+                    continue
+                sc = (K[keep] @ q[t0 + i, h]) / np.sqrt(D)
+                e = np.exp(sc - sc.max())
+                ref[start + keep] += e / e.sum()
+        assert not got[start:start + ctx][~there].any()
+        start += ctx
+    assert not got[-16:].any() and ref[:35].any()
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+
+
 def test_paged_scores_are_the_probabilities_of_the_attention(oracle):
     """One head, one new token: out = sum_j scores[j] * v[j], with out from the attention oracle."""
     seqs = [(37, 1), (5, 1)]
