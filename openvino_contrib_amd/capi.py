@@ -307,11 +307,12 @@ def paged_attention_noalloc(desc, q, k_new, v_new, key_cache, value_cache, past_
 
 
 def paged_attention_scores(desc, q, key_cache, past_lens, subsequence_begins, block_indices, block_indices_begins,
-                           score_window, scores, capacity, stream=None):
-    """scores: DeviceBuffer of `capacity` floats.  The scratch (one float per token and head) is allocated here."""
+                           score_window, scores, capacity, stream=None, lse_only=False):
+    """scores: DeviceBuffer of `capacity` floats.  The workspace is allocated here: what the size query asks for
+    or, with lse_only, one float per token and head, which leaves the call to the fp32 kernels."""
     n = _sz(0)
     check(lib().hipattn_paged_attention_scores_workspace_size(ctypes.byref(desc), ctypes.byref(n)))
-    ws = DeviceBuffer(n.value)
+    ws = DeviceBuffer(desc.num_tokens * desc.num_heads_q * 4 if lse_only else n.value)
     check(lib().hipattn_paged_attention_scores(ctypes.byref(desc), q.ptr, key_cache.ptr, past_lens.ptr,
                                                subsequence_begins.ptr, block_indices.ptr, block_indices_begins.ptr,
                                                score_window.ptr if score_window is not None else None, scores.ptr,

@@ -542,7 +542,11 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention_scores_workspace_size(cons
     if (!bytes) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_scores_workspace_size: null output");
     *bytes = 0;
     if (hipattn_status st = validate_pa(desc, true)) return st;
-    *bytes = (size_t)desc->num_tokens * desc->num_heads_q * sizeof(float);
+    // (the bound the call itself will use, short of the output's capacity, which can only lower it)
+    int64_t bound = (int64_t)desc->num_blocks * desc->block_size;
+    if (desc->max_context_len > 0) bound = std::min<int64_t>(bound, desc->max_context_len);
+    *bytes = hipattn::paged_scores_workspace(desc->q_dtype, desc->cache_dtype, desc->head_dim, desc->block_size, desc->num_heads_q,
+                                             desc->num_heads_kv, desc->num_tokens, bound, nullptr, nullptr);
     return HIPATTN_OK;
 }
 
@@ -591,6 +595,17 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention_scores(const hipattn_pa_de
     p.max_context_len = (int)std::min<int64_t>(bound, 0x7fffffff);
     p.sliding_window = desc->sliding_window;
     p.scale = desc->scale > 0.f ? desc->scale : 1.0f / sqrtf((float)desc->head_dim);
+    // the matrix-core form when the workspace holds its raw scores (a caller that sized the workspace for the
+    // log-sum-exps alone gets the fp32 kernels)
+    size_t lse_bytes = 0, part_bytes = 0;
+    const size_t full = hipattn::paged_scores_workspace(p.q_dtype, p.cache_dtype, p.head_dim, p.block_size, p.num_heads_q, p.num_heads_kv,
+                                                        p.num_tokens, p.max_context_len, &lse_bytes, &part_bytes);
+    if (part_bytes != 0 && workspace_bytes >= full && (((uintptr_t)workspace | (uintptr_t)key_cache | (uintptr_t)q) & 15) == 0) {
+        p.part = (float2*)((uint8_t*)workspace + lse_bytes);
+        p.raw = (float*)((uint8_t*)workspace + lse_bytes + part_bytes);
+        p.raw_stride = (int)((full - lse_bytes - part_bytes) / sizeof(float) / ((size_t)p.num_tokens * p.num_heads_q));
+    }
+    g_kernel_path = p.raw ? "scores_mfma" : "scores_fp32";
     HIP_TRY(hipattn::launch_paged_scores(p, as_stream(stream)));
     return HIPATTN_OK;
 }

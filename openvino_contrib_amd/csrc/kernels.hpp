@@ -180,6 +180,9 @@ struct ScoresParams {
     float* scores;
     int64_t scores_capacity;      // floats
     float* lse;                   // [num_tokens, num_heads_q] log2-domain log-sum-exp (workspace)
+    float2* part;                 // matrix-core form: [num_tokens, num_heads_q, chunks] (max, sum) per wavefront
+    float* raw;                   // matrix-core form: [num_tokens, num_heads_q, raw_stride] scaled scores; null: fp32 kernels
+    int raw_stride;
     int q_dtype;
     int cache_dtype;
     int num_heads_q;
@@ -194,6 +197,11 @@ struct ScoresParams {
     float scale;                  // already resolved (> 0)
 };
 hipError_t launch_paged_scores(const ScoresParams& p, hipStream_t stream);
+// Workspace of the scores kernels: the log-sum-exps alone (the return value when the shape stays with the fp32
+// kernels or the raw scores would exceed 256 MiB), or those, the wavefronts' partial sums and the raw scores of
+// the matrix-core form, in that order (lse_bytes / part_bytes: the aligned sizes of the first two areas).
+size_t paged_scores_workspace(int q_dtype, int cache_dtype, int head_dim, int block_size, int heads_q, int heads_kv, int num_tokens,
+                              int64_t max_context_len, size_t* lse_bytes, size_t* part_bytes);
 
 // Schedule option by name (see paged_decode.hip); value < 0 restores the default.  false: no such option.
 bool set_option(const char* name, int value);

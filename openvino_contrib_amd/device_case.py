@@ -106,9 +106,9 @@ class PagedDeviceCase:
             ws.free()
         return storage_to_f32(res, self.out_dtype), path
 
-    def scores(self, score_window=None, scale=0.0, max_context_len=None, stream=None):
+    def scores(self, score_window=None, scale=0.0, max_context_len=None, stream=None, lse_only=False):
         """The operator's second output for the cache as it stands (call run() first): f32
-        [sum(past_lens) + tokens]."""
+        [sum(past_lens) + tokens].  lse_only: the smallest workspace the call accepts (the fp32 kernels)."""
         hip, case = self.hip, self.case
         desc = pa_desc(hip, case, self.out_dtype, 0, 0, scale, max_context_len)
         total = int(np.sum(case["past_lens"])) + case["T"]
@@ -116,7 +116,7 @@ class PagedDeviceCase:
         out.fill(0xEE)
         sw = None if score_window is None else hip.DeviceBuffer.from_numpy(np.asarray(score_window, np.int32))
         hip.paged_attention_scores(desc, self.q, self.key_cache, self.past_lens, self.subsequence_begins,
-                                   self.block_indices, self.block_indices_begins, sw, out, total, stream)
+                                   self.block_indices, self.block_indices_begins, sw, out, total, stream, lse_only=lse_only)
         res = out.download(np.float32, (total + 16,), stream)
         out.free()
         if sw is not None:

@@ -1376,7 +1376,10 @@ SCORE_BATCHES = [
 
 @pytest.mark.parametrize("cache_dtype,q_dtype,Hq,Hkv,D,bs", [(W.F16, W.F16, 8, 2, 128, 32), (W.U8, W.BF16, 4, 4, 128, 32),
                                                              (W.F32, W.F32, 4, 2, 64, 16), (W.BF16, W.BF16, 6, 3, 96, 8),
-                                                             (W.F16, W.F16, 16, 1, 64, 32), (W.F16, W.F32, 2, 2, 256, 16)])
+                                                             (W.F16, W.F16, 16, 1, 64, 32), (W.F16, W.F32, 2, 2, 256, 16),
+                                                             (W.BF16, W.BF16, 12, 4, 128, 16), (W.U8, W.F16, 32, 2, 64, 16),
+                                                             (W.F16, W.BF16, 5, 1, 128, 64), (W.BF16, W.F16, 4, 2, 128, 32),
+                                                             (W.U8, W.F16, 14, 2, 128, 128)])
 @pytest.mark.parametrize("batch", range(len(SCORE_BATCHES)))
 @pytest.mark.parametrize("window", [0, 40])
 def test_paged_attention_scores(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, bs, batch, window):
@@ -1385,14 +1388,18 @@ def test_paged_attention_scores(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, b
     case = W.make_paged_case(300 + batch, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
     dev = H.PagedDeviceCase(hip, case)
     dev.run()  # writes the new tokens' keys
-    got = dev.scores(score_window)
     kc, _ = dev.caches()
     ref = oracle.paged_attention_scores(case["q"], kc, cache_dtype, case["past_lens"], case["subsequence_begins"],
                                         case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
                                         score_window=score_window, sliding_window=window)
-    # a sum of up to heads x tokens probabilities, each from an fp32 dot product and exp2
+    # a sum of up to heads x tokens probabilities, each from an fp32 dot product (or an MFMA accumulating in fp32) and exp2
     bound = 2e-5 * max(1.0, float(ref.max()))
-    assert H.max_abs(got, ref) <= bound, (H.max_abs(got, ref), bound)
+    # the workspace the size query asks for (the matrix-core kernels where the shape is theirs), then the smallest one
+    mma = D in (64, 128) and bs >= 16 and q_dtype != W.F32 and cache_dtype != W.F32 and not (cache_dtype == W.BF16 and q_dtype == W.F16)
+    for lse_only in (False, True):
+        got = dev.scores(score_window, lse_only=lse_only)
+        assert hip.last_kernel_path() == ("scores_mfma" if mma and not lse_only else "scores_fp32")
+        assert H.max_abs(got, ref) <= bound, (lse_only, H.max_abs(got, ref), bound)
     dev.free()
 
 
@@ -1413,13 +1420,14 @@ def test_paged_attention_scores_with_entries_outside_the_cache(hip, oracle, cach
     ids[begins[4]:begins[5]] = nb             # every entry of a sequence
     dev = H.PagedDeviceCase(hip, case)
     dev.run()
-    got = dev.scores(None)
     kc, _ = dev.caches()
     ref = oracle.paged_attention_scores(case["q"], kc, cache_dtype, case["past_lens"], case["subsequence_begins"],
                                         ids, begins, Hq, Hkv, D, bs, sliding_window=window)
     assert not ref[-101:].any() and ref[:305].any()
     bound = 2e-5 * max(1.0, float(ref.max()))
-    assert H.max_abs(got[:ref.size], ref) <= bound, (H.max_abs(got[:ref.size], ref), bound)
+    for lse_only in (False, True):  # the matrix-core kernels where the shape is theirs, then the fp32 ones
+        got = dev.scores(None, lse_only=lse_only)
+        assert H.max_abs(got[:ref.size], ref) <= bound, (lse_only, hip.last_kernel_path(), H.max_abs(got[:ref.size], ref), bound)
     dev.free()
 
 
