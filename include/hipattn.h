@@ -192,7 +192,7 @@ hipattn_status hipattn_sdpa_masked(const hipattn_sdpa_desc* desc, const void* q,
  * for any split of the tokens over the sequences; HIPATTN_PA_ANY_LENGTHS only changes how fast
  * such a batch runs when it does hold long multi-token sequences.
  * Kernels: 16-bit and u8 caches with a head_dim that is a multiple of 8 up to 256,
- * a block_size that is a power of two from 16 up and at most 16 query heads per kv head take the tuned matrix-core kernels (stream-K decode for single-token rows, chunked prefill over the
+ * a block_size that is a power of two from 16 up and at most 16 query heads per kv head -- or more that split into equal groups of 8 to 16, each kv head's rows then being read once per group (multi-query models: 32, 48, 64 ... heads on one kv head) -- take the tuned matrix-core kernels (stream-K decode for single-token rows, chunked prefill over the
  * block table for multi-token sequences; fastest at head_dim 256, 128 and 64; head sizes between 64 and 128 run the head-128 kernels on rows of fewer columns); other
  * 16-bit and u8 caches with 16-bit queries, a head_dim that is a multiple of 8 up to 256 and a
  * block_size that is a power of two take a plain matrix-core kernel (query tiles over the block

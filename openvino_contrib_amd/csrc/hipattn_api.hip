@@ -128,6 +128,9 @@ hipattn::PagedParams make_paged_params(const hipattn_pa_desc* d) {
     p.num_waves = d->decode_waves > 0 ? d->decode_waves : 0;
     p.any_lengths = (d->flags & HIPATTN_PA_ANY_LENGTHS) ? 1 : 0;
     p.alibi_slopes = d->alibi_slopes;
+    p.kv_share = 1;
+    // (more than 16 query heads per kv head: see split_kv_heads; the forced shape-generic path keeps the heads as they are)
+    if (!(d->flags & HIPATTN_PA_FORCE_GENERIC)) p = hipattn::split_kv_heads(p);
     return p;
 }
 

@@ -93,6 +93,11 @@ struct PagedParams {
     int max_context_len;
     int sliding_window;
     float scale;  // already resolved (> 0)
+    // More than 16 query heads per kv head (multi-query models): the stream-K kernels serve 16 heads per
+    // (sequence, kv head) segment, so each kv head is entered kv_share times, as num_heads_kv * kv_share heads
+    // of num_heads_q / that many query heads each, consecutive ones sharing the K/V rows of kv head h / kv_share
+    // (split_kv_heads; 1 otherwise).  Only the K/V addresses divide by it; the chunk kernels get the heads undivided.
+    int kv_share;
     const float* alibi_slopes;  // nullptr, or [num_heads_q]: slope * (key position - query position) joins the scaled score
     // decode: the batch's block-heads are cut into num_waves equal pieces (one per wavefront);
     // pieces that do not cover a whole (sequence, kv head) segment leave partials in the workspace
@@ -155,6 +160,9 @@ hipError_t launch_paged_tiles(const PagedParams& p, void* workspace, hipStream_t
 
 // paged attention fast paths: plan + stream-K decode + merge, and chunked prefill
 bool paged_fast_supported(const PagedParams& p);
+// p with its kv heads entered several times when that brings a call with more than 16 query heads per kv head
+// within the stream-K kernels' reach (paged_fast_supported of the result), else p as it is.
+PagedParams split_kv_heads(const PagedParams& p);
 size_t paged_fast_workspace_bytes(const PagedParams& p);
 void paged_fast_plan(PagedParams& p, void* workspace);  // fills chunking fields and workspace pointers
 void release_side_stream(hipStream_t owner);  // drops the side stream mixed batches on `owner` used, if any

@@ -898,7 +898,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
     constexpr int64_t kRowBytesBuilt = kU8 ? (kHD + 8) : (2 * kHD);
     const int head_dim = kPad ? p.head_dim : kHD;                       // (a constant unless kPad)
     const int64_t kRowBytes = kPad ? (kU8 ? p.head_dim + 8 : 2 * p.head_dim) : kRowBytesBuilt;
-    const int64_t block_stride = (int64_t)Hkv * blk * kRowBytes;
+    const int64_t block_stride = (int64_t)(Hkv / p.kv_share) * blk * kRowBytes;  // (kv_share: see PagedParams)
     // kPad: this lane's K piece offsets, V offset and whether its V columns exist
     int koff[kHD / 32];
     int voff = 0;
@@ -974,7 +974,8 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         const int32_t* table = p.block_indices + rg.table_begin + (kBlk ? lb0 * kEntries : 0);
         // table entries from there on that hold attended tokens (the row's table may end with them)
         const int entries = (rg.ctx + blk - 1) / blk - (kBlk ? lb0 * kEntries : 0);
-        const int64_t head_off = (int64_t)h * blk * kRowBytes;
+        const int h_kv = p.kv_share == 1 ? h : h / p.kv_share;  // the kv head whose rows this segment reads
+        const int64_t head_off = (int64_t)h_kv * blk * kRowBytes;
         const int sub_shift = kBlk ? 0 : __builtin_ctz(p.block_size >> 5);
 
         if constexpr (kSelfPlan) {
@@ -988,7 +989,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                 for (int q = q_lo; q <= q_hi; q++) {  // (wave-uniform; one pass for a decode row)
                     const int pb_new = p.block_indices[rg.table_begin + q / blk];
                     if (pb_new >= 0 && pb_new < p.num_blocks)
-                        kv_cache_write_pair128(wp, rg.token - (rg.write_pos - q), h, pb_new, q, lane);
+                        kv_cache_write_pair128(wp, rg.token - (rg.write_pos - q), h_kv, pb_new, q, lane);
                 }
                 if (q_lo <= q_hi) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the rows have reached the cache
             }
@@ -1456,7 +1457,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const int64_t total = (int64_t)p.blk_prefix[p.num_rows] * Hkv;
     if (total <= 0 || w >= p.num_waves) return;
     const Line line(total, p.num_waves, 0);
-    const int64_t block_stride = (int64_t)Hkv * blk * kRowBytes;
+    const int64_t block_stride = (int64_t)(Hkv / p.kv_share) * blk * kRowBytes;
     int64_t L = line.begin(w);
     const int64_t L_end = line.begin(w + 1);
     if (L >= L_end) return;
@@ -1483,7 +1484,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         const int lb0 = rg.j0 / kUnit + b_rel;
         const int32_t* table = p.block_indices + rg.table_begin + (kBlk ? lb0 * kEntries : 0);
         const int entries = (rg.ctx + blk - 1) / blk - (kBlk ? lb0 * kEntries : 0);
-        const int64_t head_off = (int64_t)h * blk * kRowBytes;
+        const int64_t head_off = (int64_t)(p.kv_share == 1 ? h : h / p.kv_share) * blk * kRowBytes;
 
         // Q^T operand in two halves: lane (head n16, kg) holds Q[head][128*half + kg*32 + i*8 .. +8]
         typename Op16<kBf16>::vec8 qf[2][4];
@@ -1749,6 +1750,29 @@ bool paged_fast_supported(const PagedParams& p) {
     // (above 128: paged_decode256_kernel)
     return p.head_dim >= 8 && p.head_dim <= 256 && p.head_dim % 8 == 0 &&
            (p.cache_dtype == HIPATTN_F16 || p.cache_dtype == HIPATTN_BF16 || p.cache_dtype == HIPATTN_U8);
+}
+
+PagedParams split_kv_heads(const PagedParams& p) {
+    const int G = p.num_heads_q / p.num_heads_kv;
+    if (G <= 16 || p.kv_share != 1) return p;
+    for (int share = 2; share <= G; share++) {
+        if (G % share != 0 || G / share > 16) continue;
+        if (G / share < 8) break;  // (groups that fill less than half of a 16-row product: the K/V rows would be read too often)
+        if ((int64_t)p.num_heads_kv * share > 0x7fff) break;
+        PagedParams s = p;
+        s.num_heads_kv = p.num_heads_kv * share;
+        s.kv_share = share;
+        return paged_fast_supported(s) ? s : p;
+    }
+    return p;  // (a prime number of heads, say: the query-tile kernel keeps the call)
+}
+
+// The chunk kernels address K and V by the cache's own kv heads.
+static PagedParams with_cache_heads(const PagedParams& p) {
+    PagedParams r = p;
+    r.num_heads_kv = p.num_heads_kv / p.kv_share;
+    r.kv_share = 1;
+    return r;
 }
 
 // Wavefronts the decode kernel keeps resident: it needs up to 256 registers per lane, i.e. two
@@ -2113,7 +2137,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
             launch_decode<1, false>(p, wp, 0, dim3(p.num_waves), dim3(64), stream);
         e = hipGetLastError();
         if (probe.after) (void)hipEventRecord(probe.after, stream);
-        const hipError_t e_prefill = launch_paged_prefill(p, side->stream);
+        const hipError_t e_prefill = launch_paged_prefill(with_cache_heads(p), side->stream);
         if (e == hipSuccess && !p.fused_merge) {
             hipLaunchKernelGGL(paged_merge_kernel, dim3(p.num_rows * p.num_heads_kv), dim3(256), 0, stream, p);
             e = hipGetLastError();
@@ -2134,7 +2158,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
         if (e != hipSuccess) return e;
     }
     if (p.max_q_tiles > 0) {
-        e = launch_paged_prefill(p, stream);
+        e = launch_paged_prefill(with_cache_heads(p), stream);
     }
     return e;
 }

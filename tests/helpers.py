@@ -47,10 +47,12 @@ def scaled_bound_error(out, ref, label=""):
 
 def paged_matrix_core_path(Hq, Hkv, D, bs, cache_dtype):
     """Kernel path of a paged call with 16-bit queries and a 16-bit or u8 cache at a head size that is a
-    multiple of 8 up to 256 and a power-of-two block size: the stream-K kernels take at most 16 query heads
-    per kv head on blocks of 16 tokens or more, the query-tile kernel the rest."""
-    stream_k = bs >= 16 and Hq // Hkv <= 16
-    return "paged_mfma" if stream_k else "paged_mfma_tiles"
+    multiple of 8 up to 256 and a power-of-two block size: the stream-K kernels on blocks of 16 tokens or more
+    with at most 16 query heads per kv head, or a number of them that splits into equal groups of 8 to 16
+    (each kv head is then entered once per group); the query-tile kernel the rest."""
+    G = Hq // Hkv
+    splits = G <= 16 or any(G % share == 0 and 8 <= G // share <= 16 for share in range(2, G + 1))
+    return "paged_mfma" if bs >= 16 and splits else "paged_mfma_tiles"
 
 
 def sdpa_matrix_core_path(D, masked):

@@ -1224,7 +1224,8 @@ def alibi_slopes(Hq):
 @pytest.mark.parametrize("D,bs,Hq,Hkv,q_dtype,cache_dtype,path", [
     (128, 32, 32, 8, W.F16, W.F16, "paged_mfma"), (128, 16, 16, 8, W.BF16, W.BF16, "paged_mfma"), (128, 32, 64, 8, W.F16, W.U8, "paged_mfma"),
     (128, 64, 8, 2, W.BF16, W.F16, "paged_mfma"), (64, 32, 8, 8, W.F16, W.F16, "paged_mfma"), (96, 16, 12, 4, W.F16, W.U8, "paged_mfma"),
-    (256, 32, 8, 2, W.F16, W.F16, "paged_mfma_tiles"), (80, 8, 8, 2, W.F16, W.F16, "paged_mfma_tiles"), (128, 16, 40, 2, W.BF16, W.U8, "paged_mfma_tiles"),
+    (256, 32, 8, 2, W.F16, W.F16, "paged_mfma_tiles"), (80, 8, 8, 2, W.F16, W.F16, "paged_mfma_tiles"), (128, 16, 34, 2, W.BF16, W.U8, "paged_mfma_tiles"),
+    (128, 16, 40, 2, W.BF16, W.U8, "paged_mfma"), (128, 32, 48, 1, W.F16, W.F16, "paged_mfma"),
     (64, 16, 4, 2, W.F32, W.F32, "paged_generic"), (72, 32, 6, 3, W.F16, W.F32, "paged_generic")])
 @pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 300), ("mixed", 0), ("mixed", 70), ("prefill", 0)])
 def test_paged_attention_with_alibi_slopes(hip, oracle, D, bs, Hq, Hkv, q_dtype, cache_dtype, path, kind, window):
@@ -1319,6 +1320,40 @@ def test_paged_other_shapes_on_the_matrix_cores(hip, oracle, shape, q_dtype, cac
     out_g, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC)
     assert path_g == "paged_generic"
     assert H.scaled_bound_error(out_g, ref, "paged tiles, generic") <= tol
+    dev.free()
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 1), (48, 1), (40, 2), (64, 2), (20, 1), (96, 3)])
+@pytest.mark.parametrize("D,bs,cache_dtype", [(128, 32, W.F16), (128, 16, W.U8), (64, 32, W.BF16), (256, 32, W.F16), (96, 64, W.U8), (128, 128, W.BF16)])
+@pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 300), ("mixed", 0)])
+def test_paged_more_than_16_query_heads_per_kv_head(hip, oracle, Hq, Hkv, D, bs, cache_dtype, kind, window):
+    """Multi-query shapes: the stream-K kernels serve 16 query heads per segment, so a kv head with more of them
+    (in equal groups of at most 16) is entered once per group, every group reading the same K/V rows.  Decode rows at
+    several wavefront counts, with the merge inside the kernel and behind it, a bad table entry, the step's own
+    cache write bit-exact; the chunks of a mixed batch take the heads undivided."""
+    announce("paged, more than 16 heads per kv head", Hq, Hkv, D, bs, cache_dtype, kind, window)
+    if kind == "decode":
+        seqs = [(c - 1, 1) for c in DECODE_CTX]
+    else:
+        seqs = [(0, 9), (37, 1), (31, 2), (5, 140), (64, 1), (700, 1), (15, 1), (300, 130), (0, 1), (1000, 3)]
+    qd = W.BF16 if cache_dtype == W.BF16 else W.F16
+    case = W.make_paged_case(111, seqs, Hq, Hkv, D, bs, qd, qd, cache_dtype, sliding_window=window)
+    ids, begins = case["block_indices"], case["block_indices_begins"]
+    ids[begins[5] + 1] = case["num_blocks"] + 2
+    ref, okc, ovc = H.oracle_paged(oracle, case)
+    dev = H.PagedDeviceCase(hip, case)
+    # (chunk rows on a bf16 cache: probabilities enter the second product with 8 significant bits, held to 2e-2 as elsewhere)
+    tol = 2e-2 if (cache_dtype == W.BF16 and kind == "mixed") else (1e-2 if cache_dtype in (W.U8, W.BF16) else 2e-3)
+    for waves, fused in ((0, 1), (0, 0), (13, 1), (700, 0)):
+        hip.set_option("decode_fused_merge", fused)
+        out, path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if (waves, fused) != (0, 1) else 0)
+        assert path == "paged_mfma", path
+        assert np.isfinite(out).all()
+        assert H.scaled_bound_error(out, ref, "more than 16 heads per kv head") <= tol, (waves, fused)
+    hip.set_option("decode_fused_merge", -1)
+    kc, vc = dev.caches()
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
     dev.free()
 
 
