@@ -260,7 +260,7 @@ hipattn_status hipattn_paged_attention(const hipattn_pa_desc* desc, const void* 
  * new tokens' keys.  Positions outside a query's sliding window and keys in blocks outside the cache
  * count as probability zero, as in the attention itself.  The call needs a workspace of one float
  * per (token, query head).  The size query asks for more where that pays: for head sizes 64 and 128
- * with 16-bit queries (blocks of 16 tokens or more, at most 16 query heads per kv head) it adds room
+ * with 16-bit queries (blocks of 16 tokens or more, query heads per kv head as for the tuned attention kernels) it adds room
  * for the scaled scores themselves, num_tokens x num_heads_q x max_context_len floats as long as that
  * stays below 256 MiB, and the call then reads the key rows once, on the matrix cores, instead of
  * twice (a decode batch of 64 sequences of 512..8,192 keys: 0.17 against 0.82 ms); with the smaller

@@ -13,7 +13,7 @@
 // the plain pair covers every other shape the ABI accepts.
 //
 // Head sizes 64 and 128 with 16-bit queries on fp16 / bf16 / u8 caches (blocks of 16 tokens or more, up to
-// 16 query heads per kv head) take the matrix cores instead, when the caller's workspace has room
+// 16 query heads per kv head, or more in equal groups of 8 to 16) take the matrix cores instead, when the caller's workspace has room
 // for the raw scores: the K rows are read ONCE,
 //
 //   paged_scores_mma_kernel      one wavefront per (aggregated token, kv head, 512 keys): S^T = K Q^T on
@@ -356,6 +356,18 @@ __host__ __device__ inline int mma_units_bound(int max_context_len) { return (ma
 __host__ __device__ inline int mma_chunks(int max_context_len) { return (mma_units_bound(max_context_len) + kMmaChunkUnits - 1) / kMmaChunkUnits; }
 __host__ __device__ inline int mma_stride(int max_context_len) { return mma_units_bound(max_context_len) * kMmaUnit; }
 
+// More than 16 query heads per kv head: in equal groups of 8 to 16, each group an item of its own that reads the
+// kv head's rows again (0: no such split).
+__host__ __device__ inline int mma_kv_share(int heads_q, int heads_kv) {
+    const int G = heads_q / heads_kv;
+    if (G <= 16) return 1;
+    for (int share = 2; share <= G; share++) {
+        if (G % share != 0 || G / share > 16) continue;
+        return G / share >= 8 ? share : 0;
+    }
+    return 0;
+}
+
 // The keys an aggregated token's scores cover, and whether it has any.
 struct MmaRow {
     int s, j0, j1;
@@ -397,17 +409,20 @@ __global__ __launch_bounds__(64 * kMmaWaves) void paged_scores_mma_kernel(Scores
     using O = Op16<kBf16>;
     const int lane = threadIdx.x & 63, n16 = lane & 15, kg = lane >> 4;
     const int chunks = mma_chunks(p.max_context_len);
-    const int G = p.num_heads_q / p.num_heads_kv;
+    const int share = mma_kv_share(p.num_heads_q, p.num_heads_kv);  // (1 unless a kv head has more than 16 query heads)
+    const int heads = p.num_heads_kv * share;                        // items per (token, chunk): head groups
+    const int G = p.num_heads_q / heads;
     const int shift = __builtin_ctz(p.block_size);
     constexpr int kRow = kU8 ? kHD + 8 : 2 * kHD;
     const float c = p.scale * kLog2e;
     // Items are (token, chunk, kv head), kv heads side by side, four to a workgroup; an item beyond its sequence's
     // end leaves at once.  (A workgroup per item, wavefronts walking the item list in steps of the grid, 4, 8 or 16
     // units per item: all within 5 % of each other on 64 decode rows of 512..8,192 keys, 0.17-0.18 ms.)
-    const int64_t items = (int64_t)p.num_heads_kv * p.num_tokens * chunks;
+    const int64_t items = (int64_t)heads * p.num_tokens * chunks;
     const int64_t item = (int64_t)blockIdx.x * kMmaWaves + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     if (item >= items) return;
-    const int kvh = (int)(item % p.num_heads_kv), chunk = (int)((item / p.num_heads_kv) % chunks), t = (int)(item / ((int64_t)p.num_heads_kv * chunks));
+    // kvh: the head group (query heads kvh * G ...), whose K rows are those of kv head kvh / share
+    const int kvh = (int)(item % heads), chunk = (int)((item / heads) % chunks), t = (int)(item / ((int64_t)heads * chunks));
     SeqView v;
     MmaRow row = mma_row(p, t, v);
     if (!row.scored) return;
@@ -459,7 +474,7 @@ __global__ __launch_bounds__(64 * kMmaWaves) void paged_scores_mma_kernel(Scores
             const int pb = __builtin_amdgcn_readlane(my_pb, (u - u_first) * 2 + tl);  // (-1: no attended key in the tile)
             const bool ok = pb >= 0 && pb < p.num_blocks;
             r.ok |= ok ? 1 << tl : 0;
-            const uint8_t* const base = p.key_cache + (((int64_t)(ok ? pb : 0) * p.num_heads_kv + kvh) * p.block_size + (tok & (p.block_size - 1))) * kRow;
+            const uint8_t* const base = p.key_cache + (((int64_t)(ok ? pb : 0) * p.num_heads_kv + kvh / share) * p.block_size + (tok & (p.block_size - 1))) * kRow;
 #pragma unroll
             for (int i = 0; i < kHD / 32; i++) {
                 if constexpr (kU8)
@@ -600,7 +615,7 @@ __global__ __launch_bounds__(256) void paged_scores_sum_kernel(ScoresParams p) {
 static bool mma_shape(int q_dtype, int cache_dtype, int head_dim, int block_size, int heads_q, int heads_kv) {
     if (!(head_dim == 64 || head_dim == 128)) return false;
     if (block_size < 16 || (block_size & (block_size - 1))) return false;
-    if (heads_q / heads_kv > 16) return false;
+    if (mma_kv_share(heads_q, heads_kv) == 0) return false;
     if (!(q_dtype == HIPATTN_F16 || q_dtype == HIPATTN_BF16)) return false;
     // fp16 queries on a bf16 cache would be rounded to eight bits for the product: the fp32 kernels keep them
     if (cache_dtype == HIPATTN_BF16) return q_dtype == HIPATTN_BF16;
@@ -624,7 +639,7 @@ size_t paged_scores_workspace(int q_dtype, int cache_dtype, int head_dim, int bl
 
 template <bool kU8, bool kBf16>
 static hipError_t launch_mma(const ScoresParams& p, hipStream_t stream) {
-    const int64_t items = (int64_t)p.num_tokens * mma_chunks(p.max_context_len) * p.num_heads_kv;
+    const int64_t items = (int64_t)p.num_tokens * mma_chunks(p.max_context_len) * p.num_heads_kv * mma_kv_share(p.num_heads_q, p.num_heads_kv);
     if ((items + kMmaWaves - 1) / kMmaWaves > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((items + kMmaWaves - 1) / kMmaWaves));
     if (p.head_dim == 128)

@@ -1414,7 +1414,8 @@ SCORE_BATCHES = [
                                                              (W.F16, W.F16, 16, 1, 64, 32), (W.F16, W.F32, 2, 2, 256, 16),
                                                              (W.BF16, W.BF16, 12, 4, 128, 16), (W.U8, W.F16, 32, 2, 64, 16),
                                                              (W.F16, W.BF16, 5, 1, 128, 64), (W.BF16, W.F16, 4, 2, 128, 32),
-                                                             (W.U8, W.F16, 14, 2, 128, 128)])
+                                                             (W.U8, W.F16, 14, 2, 128, 128), (W.F16, W.F16, 48, 1, 128, 32),
+                                                             (W.U8, W.F16, 40, 2, 64, 16), (W.BF16, W.BF16, 17, 1, 128, 32)])
 @pytest.mark.parametrize("batch", range(len(SCORE_BATCHES)))
 @pytest.mark.parametrize("window", [0, 40])
 def test_paged_attention_scores(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, bs, batch, window):
@@ -1430,7 +1431,8 @@ def test_paged_attention_scores(hip, oracle, cache_dtype, q_dtype, Hq, Hkv, D, b
     # a sum of up to heads x tokens probabilities, each from an fp32 dot product (or an MFMA accumulating in fp32) and exp2
     bound = 2e-5 * max(1.0, float(ref.max()))
     # the workspace the size query asks for (the matrix-core kernels where the shape is theirs), then the smallest one
-    mma = D in (64, 128) and bs >= 16 and q_dtype != W.F32 and cache_dtype != W.F32 and not (cache_dtype == W.BF16 and q_dtype == W.F16)
+    mma = (D in (64, 128) and bs >= 16 and q_dtype != W.F32 and cache_dtype != W.F32 and not (cache_dtype == W.BF16 and q_dtype == W.F16)
+           and H.paged_matrix_core_path(Hq, Hkv, D, bs, cache_dtype) == "paged_mfma")  # (head groups: as for the attention kernels)
     for lse_only in (False, True):
         got = dev.scores(score_window, lse_only=lse_only)
         assert hip.last_kernel_path() == ("scores_mfma" if mma and not lse_only else "scores_fp32")
