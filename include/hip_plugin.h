@@ -118,6 +118,13 @@ int hip_infer_request_copy_output(hip_infer_request_t* request, int index, void*
 int hip_compiled_model_runtime_info(hip_compiled_model_t* compiled, char* text, size_t text_size);
 /* "node_name|node_type|microseconds" per line */
 int hip_infer_request_profiling(hip_infer_request_t* request, char* text, size_t text_size);
+/* The last infer's intermediate tensors (operator outputs that are neither views, nor constants, nor bound to
+ * the caller's device memory): bytes of the one blob they were packed into by lifetime (the reference's mutable
+ * blob, src/memory_manager/model/cuda_memory_model_builder.cpp:11-25), and what they take one beside the other. */
+int hip_infer_request_intermediate_memory(hip_infer_request_t* request, size_t* blob_bytes, size_t* apart_bytes);
+/* The packing itself, for tests: box i is bytes[i] alive from step start[i] to step end[i]; offsets[i] out,
+ * returns the blob size (offsets and sizes in multiples of 256). */
+size_t hip_memory_solver_pack(int count, const size_t* bytes, const int* start, const int* end, size_t* offsets);
 /* variable states (query_state; src/cuda_variable_state.hpp:62-105) */
 int hip_infer_request_num_states(hip_infer_request_t* request);
 int hip_infer_request_state_name(hip_infer_request_t* request, int index, char* name, size_t name_size);

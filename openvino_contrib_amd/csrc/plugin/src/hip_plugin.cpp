@@ -8,6 +8,7 @@
 // sync) -> infer_postprocess (src/cuda_infer_request.cpp:107-254), the middle two on a worker
 // thread of the device's pool, which owns the stream.
 #include "hip_plugin.hpp"
+#include "hip_memory_solver.hpp"
 
 #include <algorithm>
 #include <sstream>
@@ -794,9 +795,22 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
     }
     const auto& sequence = compiled_->exec_sequence();
     prepared_.assign(sequence.size(), PreparedStep{});
-    // scratch: one arena for all steps (they run one after the other on the request's stream), sized
-    // for the largest request before any pointer into it is handed out
-    std::vector<WorkbufferRequest> requests(sequence.size());
+    // Intermediate tensors -- operator outputs that are neither views of an input, nor bound to a caller's
+    // device tensor, nor constants -- live in one blob, at offsets worked out from their lifetimes once every
+    // shape of this infer is known (hip_memory_solver.hpp; the reference's mutable blob,
+    // src/memory_manager/model/cuda_memory_model_builder.cpp:11-25).  First pass: shapes, and the memory
+    // that is known without the blob; second pass: the blob's addresses, then the scratch requests (an
+    // operator may size its scratch by which of its inputs are there).
+    struct Packed {
+        TensorID id;
+        size_t bytes;
+        int step;
+    };
+    std::vector<Packed> packed;
+    std::vector<TensorID> owner(views_.size());  // the tensor whose memory a tensor is (itself, unless it is a view)
+    for (size_t id = 0; id < owner.size(); id++) owner[id] = (TensorID)id;
+    const int kToTheEnd = (int)sequence.size();
+    std::vector<int> last_use(views_.size(), -1);
     for (size_t si = 0; si < sequence.size(); si++) {
         const auto& step = sequence[si];
         const ov::Node& node = *step.node;
@@ -822,7 +836,10 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
             ps.out.push_back(v);
             continue;
         }
-        for (TensorID id : step.op->GetInputIds()) ps.in.push_back(views_[id]);
+        for (TensorID id : step.op->GetInputIds()) {
+            ps.in.push_back(views_[id]);
+            last_use[owner[id]] = std::max(last_use[owner[id]], (int)si);
+        }
         const std::vector<ov::Shape> out_shapes = step.op->InferOutputShapes(ps.in, context);
         for (size_t o = 0; o < out_ids.size(); o++) {
             TensorView v;
@@ -831,24 +848,64 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
             const int alias = step.op->InplaceInputOf(o);
             auto bound = remote_outputs.find(out_ids[o]);
             if (alias >= 0) {
-                v.device = ps.in.at(alias).device;
+                v.device = ps.in.at(alias).device;  // (of a tensor in the blob: filled in by the second pass)
                 v.host = ps.in.at(alias).host;
-                if (bound != remote_outputs.end() && bound->second != v.device && v.byte_size())
-                    ps.copies.push_back({bound->second, v.device, v.byte_size()});
+                owner[out_ids[o]] = owner[step.op->GetInputIds().at(alias)];
+                if (bound != remote_outputs.end() && v.byte_size()) ps.copies.push_back({bound->second, nullptr, v.byte_size(), o});
             } else if (bound != remote_outputs.end()) {
                 v.device = bound->second;
             } else if (step.op->HostData(o) && compiled_->is_host_only(out_ids[o])) {
                 v.host = step.op->HostData(o);  // a Constant only ever read on the host
-            } else {
+            } else if (const void* host = step.op->HostData(o)) {  // a Constant: uploaded once per request
                 v.device = tensor_buffers_[out_ids[o]].reserve(std::max<size_t>(v.byte_size(), 16));
-                if (const void* host = step.op->HostData(o)) {  // a Constant: uploaded once per request
-                    v.host = host;
-                    if (v.byte_size() && constants_on_device_.insert(out_ids[o]).second) stream.upload(v.device, host, v.byte_size());
-                }
+                v.host = host;
+                if (v.byte_size() && constants_on_device_.insert(out_ids[o]).second) stream.upload(v.device, host, v.byte_size());
+            } else {
+                packed.push_back({out_ids[o], std::max<size_t>(v.byte_size(), 16), (int)si});
             }
             ps.out.push_back(v);
             views_[out_ids[o]] = v;
         }
+    }
+    // what the caller reads after the last step stays to the end
+    for (size_t i = 0; i < results.size(); i++) {
+        const auto src = results[i]->input_value(0);
+        last_use[owner[compiled_->output_ids(src.get_node()).at(src.get_index())]] = kToTheEnd;
+    }
+    std::vector<MemoryBox> boxes;
+    size_t apart = 0;
+    for (const Packed& t : packed) {
+        boxes.push_back({t.bytes, t.step, std::max(last_use[t.id], t.step)});
+        apart += (t.bytes + 255) / 256 * 256;
+    }
+    // (a decode loop asks for the same boxes infer after infer: the solution is kept)
+    const auto same_box = [](const MemoryBox& a, const MemoryBox& b) { return a.bytes == b.bytes && a.start == b.start && a.end == b.end; };
+    if (!(boxes.size() == solved_boxes_.size() && std::equal(boxes.begin(), boxes.end(), solved_boxes_.begin(), same_box))) {
+        packed_bytes_ = solve_memory(boxes, solved_offsets_);
+        solved_boxes_ = boxes;
+    }
+    char* const blob = packed_bytes_ ? (char*)blob_.reserve(packed_bytes_) : nullptr;
+    for (size_t i = 0; i < packed.size(); i++) views_[packed[i].id].device = blob + solved_offsets_[i];
+    unpacked_bytes_ = apart;
+
+    // second pass: every view with its final address; scratch -- one arena for all steps (they run one after
+    // the other on the request's stream), sized for the largest request before any pointer into it is handed out
+    std::vector<WorkbufferRequest> requests(sequence.size());
+    for (size_t si = 0; si < sequence.size(); si++) {
+        const auto& step = sequence[si];
+        if (ov::as_type<const ov::op::v0::Parameter>(step.node.get())) continue;
+        PreparedStep& ps = prepared_[si];
+        const auto& in_ids = step.op->GetInputIds();
+        const auto& out_ids = step.op->GetOutputIds();
+        for (size_t i = 0; i < ps.in.size(); i++) ps.in[i].device = views_[in_ids[i]].device;
+        for (size_t o = 0; o < ps.out.size(); o++) {
+            const int alias = step.op->InplaceInputOf(o);
+            if (alias >= 0) views_[out_ids[o]].device = ps.in.at(alias).device;
+            ps.out[o].device = views_[out_ids[o]].device;
+        }
+        for (auto& c : ps.copies) c.from = ps.out.at(c.output).device;
+        ps.copies.erase(std::remove_if(ps.copies.begin(), ps.copies.end(), [](const PreparedStep::CopyOut& c) { return c.to == c.from; }),
+                        ps.copies.end());
         requests[si] = step.op->GetWorkBufferRequest(ps.in);
     }
     size_t arena = 0;

@@ -24,6 +24,7 @@
 #include <vector>
 
 #include "hip_device.hpp"
+#include "hip_memory_solver.hpp"
 #include "hip_operation.hpp"
 #include "openvino/core/any.hpp"
 #include "openvino/core/model.hpp"
@@ -220,6 +221,8 @@ public:
     void wait_pipeline(const ThreadContext& thread_context);
     void infer_postprocess();
     void cancel();
+    // bytes of the blob that holds the last infer's intermediate tensors, and what they would take one beside the other
+    std::pair<size_t, size_t> intermediate_memory() const { return {packed_bytes_, unpacked_bytes_}; }
 
 private:
     std::shared_ptr<const CompiledModel> compiled_;
@@ -227,7 +230,11 @@ private:
     std::map<std::pair<const ov::Node*, size_t>, std::vector<ov::SoPtr<ov::ITensor>>> batched_tensors_;
     void bind_batched_tensors();
     std::vector<TensorView> views_;               // per TensorID, rebuilt by every infer
-    std::vector<Allocation> tensor_buffers_;      // per TensorID, grow-only
+    std::vector<Allocation> tensor_buffers_;      // per TensorID, grow-only: uploaded inputs and constants
+    Allocation blob_;                             // every other operator output of one infer, packed by lifetime
+    size_t packed_bytes_ = 0, unpacked_bytes_ = 0;  // the blob of the last infer; what its tensors take side by side
+    std::vector<MemoryBox> solved_boxes_;         // the boxes the offsets below were worked out for
+    std::vector<size_t> solved_offsets_;
     Allocation workbuffer_;                       // scratch arena shared by the steps of one infer
     std::set<TensorID> constants_on_device_;      // Constant outputs already uploaded
     std::vector<std::unique_ptr<Event>> ev_begin_, ev_end_;
@@ -246,6 +253,7 @@ private:
             void* to;
             const void* from;
             size_t bytes;
+            size_t output;  // the output it copies
         };
         std::vector<CopyOut> copies;
     };
@@ -277,6 +285,7 @@ public:
     ~AsyncInferRequest() override;
     void cancel() override;
     void infer_thread_unsafe() override;
+    const std::shared_ptr<InferRequest>& sync_request() const { return request_; }
 
 private:
     std::shared_ptr<InferRequest> request_;

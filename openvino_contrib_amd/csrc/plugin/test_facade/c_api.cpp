@@ -8,6 +8,7 @@
 #include <cstring>
 #include <sstream>
 
+#include "hip_memory_solver.hpp"
 #include "hip_operation.hpp"
 #include "hip_plugin.hpp"
 #include "openvino/runtime/exec_model_info.hpp"
@@ -431,6 +432,23 @@ API int hip_compiled_model_runtime_info(hip_compiled_model_t* compiled, char* te
         }
         copy_out(all, text, text_size);
     });
+}
+API int hip_infer_request_intermediate_memory(hip_infer_request_t* request, size_t* blob_bytes, size_t* apart_bytes) {
+    return guarded([&] {
+        auto async = std::dynamic_pointer_cast<ov::hip_gpu::AsyncInferRequest>(request->impl);
+        if (!async) OPENVINO_THROW("not a request of this plugin");
+        const auto m = async->sync_request()->intermediate_memory();
+        *blob_bytes = m.first;
+        *apart_bytes = m.second;
+    });
+}
+API size_t hip_memory_solver_pack(int count, const size_t* bytes, const int* start, const int* end, size_t* offsets) {
+    std::vector<ov::hip_gpu::MemoryBox> boxes;
+    for (int i = 0; i < count; i++) boxes.push_back({bytes[i], start[i], end[i]});
+    std::vector<size_t> at;
+    const size_t total = ov::hip_gpu::solve_memory(boxes, at);
+    for (int i = 0; i < count; i++) offsets[i] = at[i];
+    return total;
 }
 API int hip_infer_request_profiling(hip_infer_request_t* request, char* text, size_t text_size) {
     return guarded([&] {

@@ -51,6 +51,8 @@ SYMBOLS = {
     "hip_infer_request_output_info": (_i, [_vp, _i, _P(_i), _P(_i), _i64p, _P(_sz)]),
     "hip_infer_request_copy_output": (_i, [_vp, _i, _vp, _sz]),
     "hip_infer_request_profiling": (_i, [_vp, ctypes.c_char_p, _sz]),
+    "hip_infer_request_intermediate_memory": (_i, [_vp, _P(_sz), _P(_sz)]),
+    "hip_memory_solver_pack": (_sz, [_i, _P(_sz), _P(_i), _P(_i), _P(_sz)]),
     "hip_infer_request_num_states": (_i, [_vp]),
     "hip_infer_request_state_name": (_i, [_vp, _i, ctypes.c_char_p, _sz]),
     "hip_infer_request_state_reset": (_i, [_vp, _i]),
@@ -201,6 +203,12 @@ class InferRequest:
         _check(lib().hip_infer_request_set_input(self.handle, index, array.ctypes.data_as(_vp), 0, dtype, array.ndim,
                                                  _shape(array.shape)))
 
+    def intermediate_memory(self):
+        """(bytes of the blob the last infer's intermediate tensors were packed into, bytes they take side by side)."""
+        blob, apart = _sz(0), _sz(0)
+        _check(lib().hip_infer_request_intermediate_memory(self.handle, ctypes.byref(blob), ctypes.byref(apart)))
+        return blob.value, apart.value
+
     def set_input_batch(self, index, arrays, dtype):
         """set_tensors: one host tensor per batch entry (each of shape [1, ...]), wrapped, not copied."""
         arrays = [np.asarray(a, dtype=_NP[dtype], order="C") for a in arrays]
@@ -343,3 +351,11 @@ class Plugin:
         if self.handle:
             lib().hip_plugin_destroy(self.handle)
             self.handle = None
+
+
+def memory_solver_pack(bytes_, start, end):
+    """hip_memory_solver_pack: (offsets, blob size) for boxes of bytes_[i] alive from step start[i] to end[i]."""
+    n = len(bytes_)
+    offsets = (_sz * n)()
+    total = lib().hip_memory_solver_pack(n, (_sz * n)(*bytes_), (_i * n)(*start), (_i * n)(*end), offsets)
+    return list(offsets), total

@@ -540,6 +540,10 @@ def test_a_whole_small_decoder_runs_on_the_device(hip, oracle):
         again, _ = req.output(0)
         assert np.array_equal(again, logits)
     assert int(compiled.get_property("HIP_NUMBER_OF_GRAPHS")) == 1 and int(compiled.get_property("HIP_GRAPH_LAUNCHES")) == 2
+    # the intermediate tensors of the 35 operators share one blob by lifetime: a few tensors' worth, not all of them
+    blob, apart = req.intermediate_memory()
+    print("tiny decoder: intermediate tensors %d bytes packed, %d side by side" % (blob, apart), flush=True)
+    assert 0 < blob <= apart // 3
 
 
 # ------------------------------------------------------------------------------ views, Transpose, Convert

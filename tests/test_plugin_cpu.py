@@ -167,3 +167,47 @@ def test_query_model_on_views_transpose_and_convert():
     supported = P.Plugin().query_model(g.model())
     assert {"split", "moved", "wide", "narrow", "half"} <= set(supported)
     assert "to_u16" not in supported
+
+
+def test_memory_solver_packs_boxes_by_lifetime():
+    """The offsets of the request's intermediate tensors (the reference packs its mutable blob with
+    ov::MemorySolver, NP/src/memory_manager/model/cuda_memory_model_builder.cpp:11-25): boxes alive at the
+    same step never share an address, a chain needs two buffers, and no packing beats the peak of live bytes."""
+    import numpy as np
+
+    def check(sizes, start, end):
+        offsets, total = P.memory_solver_pack(sizes, start, end)
+        n = len(sizes)
+        up = [(b + 255) // 256 * 256 for b in sizes]
+        assert all(o % 256 == 0 for o in offsets) and total == max([o + u for o, u in zip(offsets, up)] + [0])
+        for i in range(n):
+            for j in range(i + 1, n):
+                if start[i] <= end[j] and start[j] <= end[i]:
+                    assert offsets[i] + up[i] <= offsets[j] or offsets[j] + up[j] <= offsets[i], (i, j)
+        peak = max([sum(up[i] for i in range(n) if start[i] <= t <= end[i]) for t in range(max(end) + 1)] + [0])
+        assert peak <= total <= sum(up)
+        return total, peak
+
+    # a chain: tensor i is written by step i and read by step i + 1
+    total, peak = check([1000] * 12, list(range(12)), list(range(1, 13)))
+    assert total == peak == 2 * 1024
+    # a residual stream: one tensor lives through, the others are a chain
+    total, peak = check([4096] + [3000] * 8, [0] + list(range(1, 9)), [9] + list(range(2, 10)))
+    assert total == peak
+    # nothing overlaps in time: one buffer of the largest size
+    total, _ = check([300, 70000, 5, 256], [0, 2, 4, 6], [1, 3, 5, 7])
+    assert total == 70144
+    # everything alive at once: the sum
+    total, peak = check([100, 200, 300], [0, 0, 0], [5, 5, 5])
+    assert total == peak == 256 * 4
+    assert P.memory_solver_pack([], [], []) == ([], 0)
+    rng = np.random.default_rng(3)
+    worst = 1.0
+    for _ in range(200):
+        n = int(rng.integers(1, 40))
+        start = [int(x) for x in rng.integers(0, 30, n)]
+        end = [s + int(x) for s, x in zip(start, rng.integers(0, 8, n))]
+        sizes = [int(x) for x in rng.integers(1, 100000, n)]
+        total, peak = check(sizes, start, end)
+        worst = max(worst, total / peak)
+    assert worst <= 1.5, worst  # (greedy, largest first: close to the peak on such mixes)
