@@ -173,6 +173,25 @@ struct BlockRegs<true> {
     float2 sz;
 };
 
+// A bf16 block turned into fp16 operands in its registers (fp16 queries on a bf16 cache: rounding the queries to
+// bf16's eight bits instead costs the decode rows their 2e-3).  bf16 -> fp16 is exact inside fp16's range; beyond it
+// the conversion (towards zero) stops at the largest finite fp16 number.
+__device__ __forceinline__ uint32_t bf16x2_to_f16x2(uint32_t w) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u)));
+}
+__device__ __forceinline__ void bf16_block_to_f16(BlockRegs<false>& b) {
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) b.k[t][i][e] = bf16x2_to_f16x2(b.k[t][i][e]);
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) b.v[j][e] = bf16x2_to_f16x2(b.v[j][e]);
+}
+
 // value of lane kLane of the caller's 16-lane row (v_mov_b32 row_newbcast, folded into the consumer where possible)
 template <int kLane>
 __device__ __forceinline__ float row_broadcast(float x) {
@@ -825,8 +844,10 @@ constexpr int kSelfPlanMaxRows = 256;
 // head sizes between 64 and 128, kPad), the self-planning form on blocks of 32 or 16 only.
 // kPad: the call's head size (p.head_dim, a multiple of 8) may be smaller than kHD: the missing columns of
 // Q are zeros and those of V are not read.
-template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false, bool kAlibi = false>
+template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan = false, int kHD = kD, int kBlk = kBS, bool kPad = false, bool kAlibi = false, bool kHalfFromBf16 = false>
 __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_decode_kernel(PagedParams p, KvWriteParams wp, int do_write) {
+    // kHalfFromBf16: the cache holds bf16, the operands are fp16 (fp16 queries): blocks are converted as they arrive
+    static_assert(!kHalfFromBf16 || (!kU8 && !kBf16 && kWaves == 1 && !kSelfPlan && kHD == 128 && !kPad && !kAlibi), "bf16 blocks as fp16 operands: the ordinary launch at head size 128 only");
     static_assert(!kAlibi || (kWaves == 1 && !kSelfPlan), "the distance bias (p.alibi_slopes) exists in the ordinary launch only");
     // The merge inside the kernel (p.fused_merge) is built into the u8 instantiations only: the 16-bit ones use
     // every register in their loop, and with that code behind the loop the allocator spilled 29 of them.
@@ -1074,9 +1095,11 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
                 int i = 0;
                 while (i < gn) {
                     ok_b = (i + 1 < gn) ? issue(rb, i + 1) : 0;
+                    if constexpr (kHalfFromBf16) bf16_block_to_f16(ra);
                     if (ok_a) process_block<kU8, kBf16, kHD, kEntries != 1, kAlibi>(st, ra, qf, sumq, c, (lb0 + g0 + i) * kUnit, rg.j0, rg.ctx, kg, ok_a, slopes, G);
                     if (i + 1 >= gn) break;
                     ok_a = (i + 2 < gn) ? issue(ra, i + 2) : 0;
+                    if constexpr (kHalfFromBf16) bf16_block_to_f16(rb);
                     if (ok_b) process_block<kU8, kBf16, kHD, kEntries != 1, kAlibi>(st, rb, qf, sumq, c, (lb0 + g0 + i + 1) * kUnit, rg.j0, rg.ctx, kg, ok_b, slopes, G);
                     i += 2;
                 }
@@ -1741,6 +1764,12 @@ bool set_option(const char* name, int value) {
 // Every head size up to 256 that is a multiple of 8 with 16-bit and u8 caches, on blocks of 16, 32 or a
 // larger power of two.
 
+// fp16 queries on a bf16 cache at head size 128: the ordinary launch with the blocks converted to fp16 operands
+// (kHalfFromBf16; no self-planning or eight-wavefront form of it is built, nor one with the distance bias).
+static bool half_operands_from_bf16(const PagedParams& p) {
+    return p.cache_dtype == HIPATTN_BF16 && p.q_dtype == HIPATTN_F16 && p.head_dim == kD && !p.alibi_slopes;
+}
+
 bool paged_fast_supported(const PagedParams& p) {
     const int G = p.num_heads_q / p.num_heads_kv;
     if (G > 16 || !(p.q_dtype == HIPATTN_F16 || p.q_dtype == HIPATTN_BF16)) return false;
@@ -1810,7 +1839,7 @@ static int query_tile_bound(const PagedParams& p) {
 static int plan_rows(const PagedParams& p) { return query_tile_bound(p) == 0 ? p.num_tokens : p.num_seqs; }
 
 static bool overlap_wanted(const PagedParams& p) {
-    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream || p.alibi_slopes) return false;
+    if (query_tile_bound(p) == 0 || p.num_waves > 0 || p.no_side_stream || p.alibi_slopes || half_operands_from_bf16(p)) return false;
     // the eight-wavefront decode kernel: head size 128, and 16-bit caches at the head sizes between 64 and 128
     if (p.head_dim != kD && !(p.head_dim > 64 && p.head_dim < kD && p.cache_dtype != HIPATTN_U8)) return false;
     return option(kOptMixedOverlap) != 0;
@@ -2015,6 +2044,17 @@ void release_side_stream(hipStream_t owner) {
 // admits; head sizes other than 128 have the ordinary form only, blocks of more than 32 tokens no self-planning form).
 template <bool kU8, bool kBf16, int kWaves, bool kSelfPlan, int kHD, bool kPad>
 static void launch_decode_blk(const PagedParams& p, const KvWriteParams& wp, int do_write, dim3 grid, dim3 block, hipStream_t stream) {
+    if constexpr (kWaves == 1 && !kSelfPlan && kBf16 && kHD == 128 && !kPad) {
+        if (half_operands_from_bf16(p)) {
+            if (p.block_size == 32)
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 128, 32, false, false, true>), grid, block, 0, stream, p, wp, do_write);
+            else if (p.block_size == 16)
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 128, 16, false, false, true>), grid, block, 0, stream, p, wp, do_write);
+            else
+                hipLaunchKernelGGL((paged_decode_kernel<false, false, 1, false, 128, 0, false, false, true>), grid, block, 0, stream, p, wp, do_write);
+            return;
+        }
+    }
     if constexpr (kWaves == 1 && !kSelfPlan) {
         if (p.alibi_slopes) {  // the instantiations with the distance bias
             if (p.block_size == 32)
@@ -2101,7 +2141,7 @@ hipError_t launch_paged_fast(const PagedParams& p, const KvWriteParams* write, h
     // A pure decode batch of few rows is one launch less: the decode wavefronts plan for themselves
     // and write the new rows (see kSelfPlanMaxRows).
     const bool self_plan = p.max_q_tiles == 0 && p.num_rows <= kSelfPlanMaxRows && p.dyn_pieces == 0 && p.head_dim == kD &&
-                           p.block_size <= 32 && (!write || wp.vector_rows) && !p.alibi_slopes;
+                           p.block_size <= 32 && (!write || wp.vector_rows) && !p.alibi_slopes && !half_operands_from_bf16(p);
     if (self_plan) {
         if (probe.before) (void)hipEventRecord(probe.before, stream);
         launch_decode<1, true>(p, wp, write ? 1 : 0, dim3(p.num_waves), dim3(64), stream);

@@ -659,15 +659,15 @@ def test_paged_scores_that_grow_along_the_context(hip, oracle, q_dtype, cache_dt
 
 @pytest.mark.parametrize("q_dtype,cache_dtype,bound,wide_bound", [
     (W.F16, W.F16, 2e-3, 2e-3), (W.BF16, W.F16, 1e-2, 1e-2), (W.F16, W.U8, 1e-2, 1e-2), (W.BF16, W.U8, 1e-2, 1e-2),
-    (W.BF16, W.BF16, 1e-2, 1e-2), (W.F16, W.BF16, 1e-2, 2e-2)])
+    (W.BF16, W.BF16, 1e-2, 1e-2), (W.F16, W.BF16, 1e-2, 1e-2)])
 @pytest.mark.parametrize("profile", ["normal", "wide"])
 def test_decode_rows_meet_the_stated_bounds_as_plain_max_abs(hip, oracle, q_dtype, cache_dtype, bound, wide_bound, profile):
     """Single-token rows through the stream-K decode kernel, held to the plain max-abs bounds (2e-3 for fp16
     throughout, 1e-2 where bf16 or u8 is involved) against the fp32 oracle, on N(0,1) data and on scores three
     times as wide (std 3 nats, peaked rows).  The output is taken in fp32 so that the kernel is measured and not
-    the rounding of a 16-bit output type (a bf16 output alone moves a value near 4 by up to 0.0156).  One
-    combination stays above its bound on the wide profile: fp16 queries on a bf16 cache, whose queries are
-    rounded to bf16 for the product (measured 1.7e-2; every other entry is below a third of its bound)."""
+    the rounding of a 16-bit output type (a bf16 output alone moves a value near 4 by up to 0.0156).  fp16
+    queries on a bf16 cache take fp16 operands, the cache blocks converted in registers: rounding the queries
+    to bf16 instead measured 1.7e-2 on the wide profile."""
     announce("decode rows, plain max-abs", q_dtype, cache_dtype, profile)
     ctxs = [5, 17, 33, 64, 200, 900, 1500, 2000, 63, 3000, 4097, 700]
     Hq, Hkv, D, bs = 16, 4, 128, 32
