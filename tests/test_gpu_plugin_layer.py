@@ -546,6 +546,56 @@ def test_a_whole_small_decoder_runs_on_the_device(hip, oracle):
     assert 0 < blob <= apart // 3
 
 
+def test_one_request_through_batches_of_changing_size(hip, oracle):
+    """The request's blob of intermediate tensors is laid out per infer: a decode step, a longer prefill (the blob
+    grows and every offset moves), the decode step's size again (the blob is larger than needed), each against the
+    oracle chain, on one request."""
+    rng = np.random.default_rng(14)
+    model = TinyDecoder(rng)
+    plugin = P.Plugin()
+    compiled = plugin.compile_model(model.graph().model())
+    req = compiled.create_infer_request()
+    blobs = []
+    for step, seqs in enumerate([[(70, 1), (33, 1), (5, 1)], [(0, 150), (64, 1), (10, 70)], [(9, 1), (200, 1), (31, 1)]]):
+        cases = [W.make_paged_case(140 + 10 * step + l, seqs, model.Hq, model.Hkv, model.D, model.bs, BF16, BF16, F16) for l in range(model.layers)]
+        for c in cases[1:]:
+            for n in ("past_lens", "subsequence_begins", "block_indices", "block_indices_begins"):
+                c[n] = cases[0][n]
+        case = cases[0]
+        T = case["q"].shape[0]
+        ids = rng.integers(0, model.vocab, T).astype(np.int32)
+        positions = np.concatenate([np.arange(p, p + n) for p, n in seqs]).astype(np.int32)
+        cos, sin = rope_tables(int(positions.max()) + 1, model.D)
+        dev_caches = [(hip.DeviceBuffer.from_numpy(c["key_cache"]), hip.DeviceBuffer.from_numpy(c["value_cache"])) for c in cases]
+        host = {"ids": (ids, P.I32), "cos": (cos, F32), "sin": (sin, F32), "positions": (positions, P.I32),
+                "past_lens": (case["past_lens"], P.I32), "subsequence_begins": (case["subsequence_begins"], P.I32),
+                "block_indices": (case["block_indices"], P.I32), "block_indices_begins": (case["block_indices_begins"], P.I32),
+                "scale": (np.zeros((0,), np.float32), F32), "sliding_window": (np.array([0], np.int32), P.I32),
+                "alibi_slopes": (np.zeros((0,), np.float32), F32),
+                "max_context_len": (np.array([case["max_context_len"]], np.int32), P.I32)}
+        cache_shape = list(case["key_cache"].shape[:3]) + [model.D]
+        for i, n in enumerate(compiled.input_names()):
+            if n in host:
+                req.set_input(i, *host[n])
+            else:
+                kind, l = n.split(".")
+                req.set_device_input(i, dev_caches[int(l)][0 if kind == "key_cache" else 1].ptr, F16, cache_shape)
+        req.infer()
+        logits, _ = req.output(0)
+        got = H.storage_to_f32(logits, BF16)
+        ref = model.reference(oracle, ids, cos, sin, positions, cases)
+        assert got.shape == ref.shape == (T, model.vocab)
+        err = scaled_error(got, ref)
+        blobs.append(req.intermediate_memory())
+        print("changing sizes, step %d: %d tokens, scaled max error %.4g, blob %d of %d bytes" % ((step, T, err) + blobs[-1]), flush=True)
+        assert err <= 6e-2
+        for kc, vc in dev_caches:
+            kc.free()
+            vc.free()
+    assert blobs[1][0] > blobs[0][0] and blobs[2][0] < blobs[1][0]  # (the figure is what the infer needs, not the allocation)
+    assert all(0 < b <= a // 3 for b, a in blobs)
+
+
 # ------------------------------------------------------------------------------ views, Transpose, Convert
 def test_reshape_transpose_convert_chain(hip, oracle):
     """[batch, length, heads * size] f32 -> Reshape (0, 0, heads, size) -> Transpose (0, 2, 1, 3) ->
