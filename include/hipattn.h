@@ -291,6 +291,24 @@ hipattn_status hipattn_paged_attention_noalloc(const hipattn_pa_desc* desc, cons
                                                const int32_t* block_indices, const int32_t* block_indices_begins,
                                                void* out, hipattn_stream stream);
 
+/* The operator's cache rotation (inputs rotated_block_indices, rotation_deltas, rotation_trig_lut; no
+ * counterpart in the reference): the key rows of the listed cache blocks, all kv heads, are turned by the
+ * rotary-embedding angle of a table row -- x'[i] = x[i] cos[i] - x[i + D/2] sin[i], x'[i + D/2] = x[i] sin[i]
+ * + x[i + D/2] cos[i] for i < D/2 -- which is what moving a token by `delta` positions does to a key stored
+ * with its rotary embedding applied.  rotation_deltas is [num_rotated_blocks, deltas_per_block] with
+ * deltas_per_block 1 (one table row for the whole block) or block_size (one per token); rotation_trig_lut is
+ * [lut_rows, head_dim] of lut_dtype (f32, f16 or bf16), a row holding head_dim / 2 cosines, then as many
+ * sines.  A block id outside [0, num_blocks) and a delta outside [0, lut_rows) leave their rows as they are.
+ * Computed in fp32 and stored in the cache's type (a u8 row is quantised again).  A caller runs it before
+ * hipattn_paged_attention of the step, on the same stream; the value cache is not touched.  Of desc, the
+ * cache type, num_heads_kv, head_dim (even), block_size and num_blocks are used.  Table layout, pairing and
+ * order are restated from the operator's documentation, not checked against OpenVINO. */
+hipattn_status hipattn_rotate_key_cache(const hipattn_pa_desc* desc, void* key_cache,
+                                        const int32_t* rotated_block_indices, int num_rotated_blocks,
+                                        const int32_t* rotation_deltas, int deltas_per_block,
+                                        const void* rotation_trig_lut, int lut_dtype, int lut_rows,
+                                        hipattn_stream stream);
+
 /* Step 1 alone: the device-side KV-cache block writer. */
 hipattn_status hipattn_kv_cache_write(const hipattn_pa_desc* desc, const void* k_new, const void* v_new,
                                       void* key_cache, void* value_cache, const int32_t* past_lens,

@@ -125,6 +125,7 @@ SYMBOLS = {
     "hipattn_paged_attention_scores": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int64, _vp, _sz, _vp]),
     "hipattn_set_option": (_i, [ctypes.c_char_p, _i]),
     "hipattn_kv_cache_write": (_i, [_P(PaDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "hipattn_rotate_key_cache": (_i, [_P(PaDesc), _vp, _vp, _i, _vp, _i, _vp, _i, _i, _vp]),
     "hipattn_cache_row_bytes": (_sz, [_i, _i]),
     "hipattn_last_kernel_path": (ctypes.c_char_p, []),
     "hipattn_profile_dominant_kernel": (_i, [_vp, _vp]),
@@ -327,6 +328,14 @@ def set_option(name, value):
 
 
 NOALLOC_SCRATCH_BYTES = 16 << 20
+
+
+def rotate_key_cache(desc, key_cache, rotated_block_indices, rotation_deltas, deltas_per_block, trig_lut, lut_dtype, lut_rows,
+                     stream=None):
+    """DeviceBuffers: block ids [n] and deltas [n, deltas_per_block] int32, the table [lut_rows, head_dim] of lut_dtype."""
+    n = rotated_block_indices.nbytes // 4
+    check(lib().hipattn_rotate_key_cache(ctypes.byref(desc), key_cache.ptr, rotated_block_indices.ptr, n, rotation_deltas.ptr,
+                                         deltas_per_block, trig_lut.ptr, lut_dtype, lut_rows, _h(stream)))
 
 
 def kv_cache_write(desc, k_new, v_new, key_cache, value_cache, past_lens, subsequence_begins, block_indices,

@@ -444,6 +444,38 @@ HIPATTN_EXPORT hipattn_status hipattn_kv_cache_write(const hipattn_pa_desc* desc
     return HIPATTN_OK;
 }
 
+HIPATTN_EXPORT hipattn_status hipattn_rotate_key_cache(const hipattn_pa_desc* desc, void* key_cache,
+                                                       const int32_t* rotated_block_indices, int num_rotated_blocks,
+                                                       const int32_t* rotation_deltas, int deltas_per_block,
+                                                       const void* rotation_trig_lut, int lut_dtype, int lut_rows,
+                                                       hipattn_stream stream) {
+    if (hipattn_status st = validate_pa(desc, false)) return st;
+    if (num_rotated_blocks < 0 || lut_rows < 0) return fail(HIPATTN_INVALID_ARGUMENT, "rotate_key_cache: negative count");
+    if (num_rotated_blocks == 0) return HIPATTN_OK;
+    if (!key_cache || !rotated_block_indices || !rotation_deltas || !rotation_trig_lut)
+        return fail(HIPATTN_INVALID_ARGUMENT, "rotate_key_cache: null pointer");
+    if (deltas_per_block != 1 && deltas_per_block != desc->block_size)
+        return fail(HIPATTN_INVALID_ARGUMENT, "rotate_key_cache: %d deltas per block (1 or block_size = %d)", deltas_per_block, desc->block_size);
+    if (!is_float_dtype(lut_dtype)) return fail(HIPATTN_INVALID_ARGUMENT, "rotate_key_cache: table dtype %d", lut_dtype);
+    if (desc->head_dim % 2 != 0) return fail(HIPATTN_UNSUPPORTED, "rotate_key_cache: odd head size %d", desc->head_dim);
+    hipattn::KeyRotationParams p{};
+    p.key_cache = (uint8_t*)key_cache;
+    p.rotated_block_indices = rotated_block_indices;
+    p.rotation_deltas = rotation_deltas;
+    p.trig_lut = rotation_trig_lut;
+    p.lut_dtype = lut_dtype;
+    p.lut_rows = lut_rows;
+    p.num_rotated = num_rotated_blocks;
+    p.deltas_per_block = deltas_per_block;
+    p.cache_dtype = desc->cache_dtype;
+    p.num_heads_kv = desc->num_heads_kv;
+    p.head_dim = desc->head_dim;
+    p.block_size = desc->block_size;
+    p.num_blocks = desc->num_blocks;
+    HIP_TRY(hipattn::launch_rotate_key_cache(p, as_stream(stream)));
+    return HIPATTN_OK;
+}
+
 HIPATTN_EXPORT hipattn_status hipattn_paged_attention_workspace_size(const hipattn_pa_desc* desc, size_t* bytes) {
     if (!bytes) return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_workspace_size: null output");
     *bytes = 0;

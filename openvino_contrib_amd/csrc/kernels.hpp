@@ -34,6 +34,24 @@ struct KvWriteParams {
     int vector_rows;
 };
 
+// The operator's cache rotation: the key rows of the listed blocks turned by the angles of their table rows.
+struct KeyRotationParams {
+    uint8_t* key_cache;
+    const int32_t* rotated_block_indices;  // [num_rotated]
+    const int32_t* rotation_deltas;        // [num_rotated, deltas_per_block]
+    const void* trig_lut;                  // [lut_rows, head_dim]: head_dim / 2 cosines, then as many sines
+    int lut_dtype;
+    int lut_rows;
+    int num_rotated;
+    int deltas_per_block;                  // 1 or block_size
+    int cache_dtype;
+    int num_heads_kv;
+    int head_dim;
+    int block_size;
+    int num_blocks;
+};
+hipError_t launch_rotate_key_cache(const KeyRotationParams& p, hipStream_t stream);
+
 // Wavefronts the writer needs for p (and p.heads_per_wave, which it sets).
 inline int64_t kv_write_wavefronts(KvWriteParams& p) {
     const auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };

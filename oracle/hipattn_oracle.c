@@ -525,6 +525,60 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
     return 0;
 }
 
+/*
+ * Cache rotation of PagedAttentionExtension (inputs rotated_block_indices, rotation_deltas,
+ * rotation_trig_lut): the keys of the listed cache blocks are turned by a rotary-embedding angle, which is
+ * what moving a token to another position does to a key that was stored with its rotary embedding applied
+ * (a cache-eviction policy closes the gaps it leaves and re-rotates the blocks behind them).
+ *   rotated_block_indices [n]        blocks of the cache (ids outside [0, num_blocks) are skipped)
+ *   rotation_deltas [n, per_block]   per_block = 1: one row of the table for the whole block;
+ *                                    per_block = block_size: one per token of the block
+ *   rotation_trig_lut [lut_rows, D]  row r: D/2 cosines, then D/2 sines (a delta outside [0, lut_rows)
+ *                                    leaves its token as it is)
+ * Every key row x of a listed block (all kv heads) becomes, for i < D/2,
+ *   x'[i] = x[i] cos[i] - x[i + D/2] sin[i],   x'[i + D/2] = x[i] sin[i] + x[i + D/2] cos[i]
+ * (the "rotate-half" pairing), computed in fp32 and stored in the cache's type (u8 rows are dequantised,
+ * turned and quantised again).  The value cache is not touched.  In the operator this happens before the
+ * step's new keys are stored.
+ * PARITY UNPINNED against OpenVINO (the operator is not in the reference tree, OpenVINO is not installed):
+ * table layout, pairing and order restated from the operator's documentation.  Pinned by: two rotations
+ * compose to the rotation by the summed angle, a rotation and its inverse restore the rows, norms are kept,
+ * and a key stored with the rotary embedding of position p (oracle_rope_f32, itself pinned by transformers'
+ * apply_rotary_pos_emb) and turned by delta equals the key embedded at position p + delta
+ * (tests/test_oracle_cpu.py).
+ */
+ORACLE_API int oracle_rotate_key_cache(uint8_t* key_cache, int cache_dtype, const int32_t* rotated_block_indices, int n,
+                                       const int32_t* rotation_deltas, int per_block, const float* rotation_trig_lut,
+                                       int lut_rows, int Hkv, int D, int block_size, int num_blocks) {
+    if (n < 0 || Hkv <= 0 || D <= 0 || (D & 1) || block_size <= 0 || (per_block != 1 && per_block != block_size)) return 1;
+    const int64_t rb = cache_row_bytes(cache_dtype, D);
+    const int half = D / 2;
+    float* x = (float*)malloc(sizeof(float) * (size_t)D);
+    float* y = (float*)malloc(sizeof(float) * (size_t)D);
+    for (int b = 0; b < n; b++) {
+        const int pb = rotated_block_indices[b];
+        if (pb < 0 || pb >= num_blocks) continue;
+        for (int t = 0; t < block_size; t++) {
+            const int delta = rotation_deltas[(int64_t)b * per_block + (per_block == 1 ? 0 : t)];
+            if (delta < 0 || delta >= lut_rows) continue;
+            const float* cs = rotation_trig_lut + (int64_t)delta * D;
+            for (int h = 0; h < Hkv; h++) {
+                uint8_t* row = key_cache + (((int64_t)pb * Hkv + h) * block_size + t) * rb;
+                cache_row_load(cache_dtype, row, D, x);
+                for (int i = 0; i < half; i++) { /* (one product rounded, the other fused: spelled out so that a kernel can match to the bit) */
+                    const float t0 = x[i + half] * cs[half + i], t1 = x[i + half] * cs[i];
+                    y[i] = fmaf(x[i], cs[i], -t0);
+                    y[i + half] = fmaf(x[i], cs[half + i], t1);
+                }
+                cache_row_store(cache_dtype, y, D, row);
+            }
+        }
+    }
+    free(x);
+    free(y);
+    return 0;
+}
+
 /* Second output of PagedAttentionExtension ("scores"): for every cache position of every
  * sequence, the probability it received, summed over the query heads and over the last
  * score_window[s] query tokens of the sequence (all of them when score_window is NULL).

@@ -64,6 +64,8 @@ def lib():
         L.oracle_paged_attention.restype = i32
         L.oracle_paged_attention_scores.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp]
         L.oracle_paged_attention_scores.restype = i32
+        L.oracle_rotate_key_cache.argtypes = [vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32]
+        L.oracle_rotate_key_cache.restype = i32
         L.oracle_rms_norm_f32.argtypes = [vp, vp, vp, i64, i64, f32]
         L.oracle_rms_norm_f32.restype = None
         L.oracle_rope_f32.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i64]
@@ -265,6 +267,20 @@ def paged_attention_scores(q, key_cache, cache_dtype, past_lens, subsequence_beg
     if rc:
         raise ValueError("oracle_paged_attention_scores: bad arguments")
     return out
+
+
+def rotate_key_cache(key_cache, cache_dtype, rotated_block_indices, rotation_deltas, rotation_trig_lut, Hkv, D, block_size):
+    """The operator's cache rotation, in place on key_cache (a uint8 view).  rotation_deltas: [n, 1] or
+    [n, block_size] int32; rotation_trig_lut: [rows, D] fp32 (D/2 cosines, then D/2 sines per row)."""
+    assert key_cache.dtype == np.uint8 and key_cache.flags.c_contiguous
+    idx = _c(rotated_block_indices, np.int32)
+    deltas = _c(rotation_deltas, np.int32).reshape(len(idx), -1)
+    lut = _c(rotation_trig_lut, np.float32)
+    assert lut.ndim == 2 and lut.shape[1] == D
+    rc = lib().oracle_rotate_key_cache(_p(key_cache), cache_dtype, _p(idx), len(idx), _p(deltas), deltas.shape[1] if len(idx) else 1,
+                                       _p(lut), lut.shape[0], Hkv, D, block_size, key_cache.shape[0])
+    if rc:
+        raise ValueError("oracle_rotate_key_cache: bad arguments")
 
 
 # ---- the operators either side of attention (oracle/layer_ops_oracle.c) ------------------------

@@ -5,6 +5,8 @@ Bars: cache bytes after the writer / the op's step 1 are bit-exact; attention ou
 within max-abs 2e-3 (fp16), 1e-2 (bf16 or u8 cache), 1e-4 for the fp32 kernel, against the
 oracle's fp32 result computed from the same stored (rounded / quantised) inputs.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -1398,6 +1400,64 @@ def test_paged_errors(hip):
         np.testing.assert_array_equal(before, dev.out.download(np.uint16, (case["T"], 32 * 128)))
     dev.free()
 
+
+
+# ---- the operator's cache rotation ---------------------------------------------------------------
+def trig_lut(rows, D, base=10000.0):
+    theta = base ** (-np.arange(D // 2, dtype=np.float64) * 2.0 / D)
+    ang = np.arange(rows, dtype=np.float64)[:, None] * theta[None, :]
+    return np.concatenate([np.cos(ang), np.sin(ang)], axis=1).astype(np.float32)
+
+
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.BF16, W.U8, W.F32])
+@pytest.mark.parametrize("D,bs,Hkv", [(128, 32, 8), (64, 16, 2), (96, 8, 3), (256, 32, 1), (512, 16, 1), (8, 4, 5)])
+@pytest.mark.parametrize("per_token", [False, True])
+@pytest.mark.parametrize("lut_dtype", [W.F32, W.F16])
+def test_rotate_key_cache_matches_the_oracle_to_the_bit(hip, oracle, cache_dtype, D, bs, Hkv, per_token, lut_dtype):
+    """hipattn_rotate_key_cache against the oracle on the same cache bytes: every cache type, per block and per
+    token, block ids outside the pool and deltas outside the table skipped, a block listed twice (turned twice,
+    in list order only when the two deltas are equal -- the test lists it with one delta), the value cache and
+    every other key block untouched; bit-exact, u8 rows included."""
+    announce("rotate key cache", cache_dtype, D, bs, Hkv, per_token, lut_dtype)
+    if cache_dtype == W.F32 and D > 256:
+        pytest.skip("one shape per type is enough at this size")
+    rng = np.random.default_rng(D + bs)
+    seqs = [(5 * bs + 3, 1), (2 * bs, 4)]
+    qd = W.F32 if cache_dtype == W.F32 else W.F16
+    case = W.make_paged_case(150, seqs, Hkv, Hkv, D, bs, qd, qd, cache_dtype)
+    nb = case["num_blocks"]
+    rows = 300
+    lut32 = trig_lut(rows, D)
+    lut_store, lut_used = (lut32, lut32) if lut_dtype == W.F32 else W.to_storage(lut32, W.F16)
+    blocks = np.array([1, nb + 3, 0, -1, nb - 1, 2], np.int32)
+    deltas = rng.integers(0, rows, (len(blocks), bs if per_token else 1)).astype(np.int32)
+    deltas[2, 0] = rows      # outside the table
+    deltas[4, -1] = -1
+    desc = H.pa_desc(hip, case)
+    kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
+    d_blocks, d_deltas, d_lut = (hip.DeviceBuffer.from_numpy(a) for a in (blocks, deltas, np.ascontiguousarray(lut_store)))
+    hip.rotate_key_cache(desc, kc, d_blocks, d_deltas, deltas.shape[1], d_lut, lut_dtype, rows)
+    got = kc.download(np.uint8, case["key_cache"].shape)
+    want = case["key_cache"].copy()
+    oracle.rotate_key_cache(want, cache_dtype, blocks, deltas, lut_used, Hkv, D, bs)
+    assert not np.array_equal(want, case["key_cache"])
+    np.testing.assert_array_equal(got, want)
+    for b in (kc, d_blocks, d_deltas, d_lut):
+        b.free()
+
+
+def test_rotate_key_cache_arguments(hip):
+    announce("rotate key cache arguments")
+    case = W.make_paged_case(151, [(40, 1)], 4, 2, 64, 16, W.F16, W.F16, W.F16)
+    desc = H.pa_desc(hip, case)
+    L = hip.lib()
+    one = ctypes.c_void_p(256)
+    assert L.hipattn_rotate_key_cache(ctypes.byref(desc), one, one, 0, one, 1, one, hip.F32, 10, None) == hip.OK  # nothing listed
+    assert L.hipattn_rotate_key_cache(ctypes.byref(desc), one, one, 2, one, 5, one, hip.F32, 10, None) == hip.INVALID_ARGUMENT
+    assert b"deltas per block" in L.hipattn_last_error_string()
+    assert L.hipattn_rotate_key_cache(ctypes.byref(desc), one, None, 2, one, 1, one, hip.F32, 10, None) == hip.INVALID_ARGUMENT
+    assert L.hipattn_rotate_key_cache(ctypes.byref(desc), one, one, 2, one, 1, one, hip.U8, 10, None) == hip.INVALID_ARGUMENT
+    assert L.hipattn_rotate_key_cache(ctypes.byref(desc), one, one, -1, one, 1, one, hip.F32, 10, None) == hip.INVALID_ARGUMENT
 
 
 # ---- the operator's second output ("scores") ----------------------------------------------------

@@ -515,3 +515,98 @@ def test_paged_scores_are_the_probabilities_of_the_attention(oracle):
         V = oracle.gather_cache_rows(vc, W.F32, case["block_indices"][bb[s]:bb[s + 1]], past + 1, 0, 1, 32, 16)
         np.testing.assert_allclose(sc[start:start + past + 1] @ V, out[s], rtol=1e-5, atol=1e-6)
         start += past + 1
+
+
+# ---- the operator's cache rotation ----------------------------------------------------------------
+def _trig_lut(rows, D, base=10000.0, sign=1.0):
+    """Row r: cos(r theta_i) for i < D/2, then sign * sin(r theta_i), with the rotary embedding's frequencies."""
+    theta = base ** (-np.arange(D // 2, dtype=np.float64) * 2.0 / D)
+    ang = np.arange(rows, dtype=np.float64)[:, None] * theta[None, :]
+    return np.concatenate([np.cos(ang), sign * np.sin(ang)], axis=1).astype(np.float32)
+
+
+def _f32_cache(rng, num_blocks, Hkv, bs, D):
+    rows = rng.standard_normal((num_blocks, Hkv, bs, D)).astype(np.float32)
+    return rows, np.ascontiguousarray(rows).view(np.uint8).reshape(num_blocks, Hkv, bs, D * 4)
+
+
+def test_cache_rotation_composes_inverts_and_keeps_norms(oracle):
+    rng = np.random.default_rng(5)
+    nb, Hkv, bs, D = 9, 3, 8, 32
+    rows, cache = _f32_cache(rng, nb, Hkv, bs, D)
+    lut = _trig_lut(64, D)
+    blocks = [4, 1, 7]
+    one = cache.copy()
+    oracle.rotate_key_cache(one, W.F32, blocks, [[5], [9], [0]], lut, Hkv, D, bs)
+    oracle.rotate_key_cache(one, W.F32, blocks, [[12], [3], [40]], lut, Hkv, D, bs)
+    both = cache.copy()
+    oracle.rotate_key_cache(both, W.F32, blocks, [[17], [12], [40]], lut, Hkv, D, bs)
+    a, b = one.view(np.float32).reshape(rows.shape), both.view(np.float32).reshape(rows.shape)
+    np.testing.assert_allclose(a, b, rtol=0, atol=3e-6)
+    # the blocks that are not listed keep their bytes; the listed ones moved (but for the rotation by row 0) and kept their norms
+    for blk in range(nb):
+        if blk not in blocks:
+            assert np.array_equal(b[blk], rows[blk])
+    assert np.abs(b[4] - rows[4]).max() > 0.1 and np.abs(b[1] - rows[1]).max() > 0.1
+    np.testing.assert_allclose(np.linalg.norm(b, axis=-1), np.linalg.norm(rows, axis=-1), rtol=1e-5)
+    # the table with the sines negated turns back
+    back = both.copy()
+    oracle.rotate_key_cache(back, W.F32, blocks, [[17], [12], [40]], _trig_lut(64, D, sign=-1.0), Hkv, D, bs)
+    np.testing.assert_allclose(back.view(np.float32).reshape(rows.shape), rows, rtol=0, atol=3e-6)
+
+
+def test_cache_rotation_moves_a_rotary_embedded_key_to_another_position(oracle):
+    """Keys stored with the rotary embedding of their positions (rotate-half layout, the embedding oracle that
+    transformers' apply_rotary_pos_emb pins), turned by delta, are the keys embedded at position + delta: per
+    block and per token."""
+    rng = np.random.default_rng(6)
+    Hkv, bs, D, nb = 2, 4, 64, 5
+    plain = rng.standard_normal((nb * bs, Hkv, D)).astype(np.float32)
+    lut = _trig_lut(200, D)
+    cos = np.concatenate([lut[:, :D // 2], lut[:, :D // 2]], axis=1)
+    sin = np.concatenate([lut[:, D // 2:], lut[:, D // 2:]], axis=1)
+    positions = rng.integers(0, 60, nb * bs).astype(np.int32)
+    def cache_of(pos):
+        e = oracle.rope(plain, cos, sin, pos.astype(np.int32))                        # [tokens, Hkv, D]
+        return np.ascontiguousarray(e.reshape(nb, bs, Hkv, D).transpose(0, 2, 1, 3))  # [block, head, token, D]
+    cache = cache_of(positions).view(np.uint8).reshape(nb, Hkv, bs, D * 4).copy()
+    per_block = rng.integers(0, 100, (2, 1)).astype(np.int32)
+    per_token = rng.integers(0, 100, (2, bs)).astype(np.int32)
+    oracle.rotate_key_cache(cache, W.F32, [3, 0], per_block, lut, Hkv, D, bs)
+    oracle.rotate_key_cache(cache, W.F32, [1, 4], per_token, lut, Hkv, D, bs)
+    shift = np.zeros((nb, bs), np.int32)
+    shift[3], shift[0] = per_block[0, 0], per_block[1, 0]
+    shift[1], shift[4] = per_token[0], per_token[1]
+    want = cache_of(positions + shift.reshape(-1))
+    np.testing.assert_allclose(cache.view(np.float32).reshape(want.shape), want, rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("cache_dtype", [W.F16, W.BF16, W.U8])
+def test_cache_rotation_in_the_cache_types_and_what_it_skips(oracle, cache_dtype):
+    """16-bit and u8 caches: the fp32 rotation of the stored values, rounded (u8: quantised again, within half a
+    step of the row's new scale); block ids outside the pool and deltas outside the table leave their rows alone."""
+    rng = np.random.default_rng(7)
+    nb, Hkv, bs, D = 6, 2, 8, 32
+    rows = rng.standard_normal((nb, Hkv, bs, D)).astype(np.float32)
+    rb = {W.F16: 2 * D, W.BF16: 2 * D, W.U8: D + 8}[cache_dtype]
+    cache = np.zeros((nb, Hkv, bs, rb), np.uint8)
+    for blk in range(nb):
+        for h in range(Hkv):
+            cache[blk, h] = W.cache_rows_from_f32(rows[blk, h], cache_dtype)
+    stored = np.stack([[oracle.gather_cache_rows(cache, cache_dtype, [blk], bs, h, Hkv, D, bs) for h in range(Hkv)] for blk in range(nb)])
+    lut = _trig_lut(50, D)
+    before = cache.copy()
+    deltas = np.array([[7] * bs, [3] * bs, [49] + [50] * (bs - 1), [1] * bs], np.int32)  # block 5: only token 0 has a row of the table
+    oracle.rotate_key_cache(cache, cache_dtype, [2, -1, 5, nb], deltas, lut, Hkv, D, bs)
+    f32 = np.ascontiguousarray(stored).view(np.uint8).reshape(nb, Hkv, bs, D * 4).copy()
+    oracle.rotate_key_cache(f32, W.F32, [2, -1, 5, nb], deltas, lut, Hkv, D, bs)
+    want = f32.view(np.float32).reshape(stored.shape)
+    got = np.stack([[oracle.gather_cache_rows(cache, cache_dtype, [blk], bs, h, Hkv, D, bs) for h in range(Hkv)] for blk in range(nb)])
+    for blk in (0, 1, 3, 4):
+        assert np.array_equal(cache[blk], before[blk])
+    assert np.array_equal(cache[5, :, 1:], before[5, :, 1:]) and not np.array_equal(cache[5, :, 0], before[5, :, 0])
+    if cache_dtype == W.U8:
+        scale = cache[2].view(np.float32).reshape(Hkv, bs, -1)[:, :, 0]  # (scale, zero-point) lead a row
+        assert np.all(np.abs(got[2] - want[2]) <= 0.5 * scale[:, :, None] + 1e-6)
+    else:
+        np.testing.assert_allclose(got[2], want[2], rtol=2 ** -8 if cache_dtype == W.BF16 else 2 ** -11, atol=1e-6)
