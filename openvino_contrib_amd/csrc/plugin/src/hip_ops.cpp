@@ -230,9 +230,10 @@ private:
 };
 
 // Input order of the OpenVINO operator.  score_aggregation_window belongs to the scores output
-// (built: the aggregated probabilities a cache-eviction policy reads); everything behind it belongs
-// to features this plugin does not implement (cache rotation, sparse attention, sinks): such inputs
-// are accepted when they are empty, as exported models carry them, and refused when they hold data.
+// (built: the aggregated probabilities a cache-eviction policy reads); the three rotation inputs to the
+// cache rotation (built: hipattn_rotate_key_cache ahead of the attention); everything behind them belongs
+// to features this plugin does not implement (sparse attention, sinks): such inputs are accepted when
+// they are empty, as exported models carry them, and refused when they hold data.
 enum PaInput {
     kQuery = 0, kKey, kValue, kKeyCache, kValueCache, kPastLens, kSubsequenceBegins, kBlockIndices,
     kBlockIndicesBegins, kScale, kSlidingWindow, kAlibiSlopes, kMaxContextLen, kPaRequiredInputs,
@@ -254,9 +255,21 @@ public:
         if (num_inputs_ > kPaRequiredInputs + sizeof(kPaOptionalNames) / sizeof(kPaOptionalNames[0]))
             HIP_PLUGIN_THROW(who + std::to_string(num_inputs_) + " inputs: more than this plugin knows of");
         if (num_outputs_ < 1 || num_outputs_ > 2) HIP_PLUGIN_THROW(who + std::to_string(num_outputs_) + " outputs");
-        for (size_t i = kPaRequiredInputs; i < num_inputs_; i++)
-            if (i != kScoreAggregationWindow && statically_non_empty(node.get_input_partial_shape(i)))
+        for (size_t i = kRotationTrigLut + 1; i < num_inputs_; i++)
+            if (statically_non_empty(node.get_input_partial_shape(i)))
                 HIP_PLUGIN_THROW(who + kPaOptionalNames[i - kPaRequiredInputs] + " holds data: the feature is not supported");
+        if (num_inputs_ > kRotationTrigLut) {
+            for (int i : {kRotatedBlockIndices, kRotationDeltas})
+                if (node.get_input_element_type(i) != ov::element::i32 && !statically_empty(node.get_input_partial_shape(i)))
+                    HIP_PLUGIN_THROW(who + kPaOptionalNames[i - kPaRequiredInputs] + " must be i32");
+            lut_type_ = node.get_input_element_type(kRotationTrigLut);
+            if (!is_float(lut_type_) && !statically_empty(node.get_input_partial_shape(kRotationTrigLut)))
+                HIP_PLUGIN_THROW(who + "rotation_trig_lut must be f32, f16 or bf16");
+        } else if (num_inputs_ > kRotatedBlockIndices) {
+            for (size_t i = kRotatedBlockIndices; i < num_inputs_; i++)
+                if (statically_non_empty(node.get_input_partial_shape(i)))
+                    HIP_PLUGIN_THROW(who + "cache rotation needs rotated_block_indices, rotation_deltas and rotation_trig_lut together");
+        }
         if (num_inputs_ > kScoreAggregationWindow && node.get_input_element_type(kScoreAggregationWindow) != ov::element::i32)
             HIP_PLUGIN_THROW(who + "score_aggregation_window must be i32");
         q_type_ = node.get_input_element_type(kQuery);
@@ -305,8 +318,7 @@ public:
     std::vector<size_t> UpdatedInputs() const override { return {kKeyCache, kValueCache}; }
     // launch parameters, and inputs that must be empty: none of them is handed to a kernel
     bool InputIsHostOnly(size_t input) const override {
-        return input == kScale || input == kSlidingWindow || input == kMaxContextLen ||
-               (input >= kPaRequiredInputs && input != kScoreAggregationWindow);
+        return input == kScale || input == kSlidingWindow || input == kMaxContextLen || input > kRotationTrigLut;
     }
 
     // max_context_len is advisory for the attention kernels; only the scores kernels size a grid by it
@@ -331,6 +343,22 @@ public:
         const hipattn_pa_desc d = describe(in);
         void* ws = wb.mutable_buffers.empty() ? nullptr : wb.mutable_buffers[0];
         const size_t ws_bytes = wb.mutable_sizes.empty() ? 0 : wb.mutable_sizes[0];
+        // cache rotation first: the listed key blocks are turned before this step's keys are stored
+        if (num_inputs_ > kRotationTrigLut && ov::shape_size(in[kRotatedBlockIndices].shape) > 0) {
+            const size_t blocks = ov::shape_size(in[kRotatedBlockIndices].shape);
+            const ov::Shape& deltas = in[kRotationDeltas].shape;
+            const ov::Shape& lut = in[kRotationTrigLut].shape;
+            HIP_PLUGIN_ASSERT(ov::shape_size(deltas) == blocks || ov::shape_size(deltas) == blocks * (size_t)d.block_size,
+                              "rotation_deltas must be [rotated blocks, 1] or [rotated blocks, block_size], got " + shape_str(deltas));
+            HIP_PLUGIN_ASSERT(ov::shape_size(lut) > 0 && ov::shape_size(lut) % (size_t)d.head_dim == 0,
+                              "rotation_trig_lut must be [positions, head_size], got " + shape_str(lut));
+            hipattn_dtype lut_dtype = HIPATTN_F32;
+            to_hipattn_dtype(lut_type_, lut_dtype);
+            HIP_PLUGIN_CHECK(hipattn_rotate_key_cache(&d, in[kKeyCache].device, (const int32_t*)in[kRotatedBlockIndices].device, (int)blocks,
+                                                      (const int32_t*)in[kRotationDeltas].device, (int)(ov::shape_size(deltas) / blocks),
+                                                      in[kRotationTrigLut].device, lut_dtype, (int)(ov::shape_size(lut) / (size_t)d.head_dim),
+                                                      context.stream.get()));
+        }
         HIP_PLUGIN_CHECK(hipattn_paged_attention(
             &d, in[kQuery].device, in[kKey].device, in[kValue].device, in[kKeyCache].device, in[kValueCache].device,
             (const int32_t*)in[kPastLens].device, (const int32_t*)in[kSubsequenceBegins].device,
@@ -370,9 +398,12 @@ private:
         const ov::Shape& kc = in[kKeyCache].shape;
         HIP_PLUGIN_ASSERT(q.size() == 2, "query must be [tokens, heads * head_size], got " + shape_str(q));
         HIP_PLUGIN_ASSERT(kc.size() == 4 && in[kValueCache].shape == kc, "key/value cache shapes " + shape_str(kc));
-        for (size_t i = kPaRequiredInputs; i < num_inputs_; i++)
-            HIP_PLUGIN_ASSERT(i == kScoreAggregationWindow || ov::shape_size(in[i].shape) == 0,
+        for (size_t i = kRotationTrigLut + 1; i < num_inputs_; i++)
+            HIP_PLUGIN_ASSERT(ov::shape_size(in[i].shape) == 0,
                               std::string(kPaOptionalNames[i - kPaRequiredInputs]) + " holds data: the feature is not supported");
+        if (num_inputs_ > kRotatedBlockIndices && num_inputs_ <= kRotationTrigLut)
+            for (size_t i = kRotatedBlockIndices; i < num_inputs_; i++)
+                HIP_PLUGIN_ASSERT(ov::shape_size(in[i].shape) == 0, "cache rotation needs rotated_block_indices, rotation_deltas and rotation_trig_lut together");
         hipattn_pa_desc d{};
         to_hipattn_dtype(q_type_, d.q_dtype);
         to_hipattn_dtype(kv_type_, d.kv_dtype);
@@ -408,7 +439,7 @@ private:
         }
         return d;
     }
-    ov::element::Type q_type_, kv_type_, cache_type_, out1_type_;
+    ov::element::Type q_type_, kv_type_, cache_type_, out1_type_, lut_type_ = ov::element::f32;
     size_t num_inputs_ = 0, num_outputs_ = 1;
     bool scores_wanted_ = true;  // until the compiled model says nothing consumes output 1
 };

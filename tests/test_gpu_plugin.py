@@ -577,3 +577,73 @@ def test_paged_attention_with_host_bound_caches_writes_them_back(hip, oracle):
     assert H.max_abs(H.storage_to_f32(req.output(0)[0], W.F16), ref) <= 2e-3
     np.testing.assert_array_equal(kc, okc)  # the caller's own arrays now hold the new rows
     np.testing.assert_array_equal(vc, ovc)
+
+
+@pytest.mark.parametrize("cache_dtype,per_token", [(W.F16, False), (W.U8, True), (W.BF16, True)])
+def test_paged_attention_with_cache_rotation_through_the_plugin(hip, oracle, cache_dtype, per_token):
+    """rotated_block_indices, rotation_deltas and rotation_trig_lut with data: the listed key blocks are turned
+    before the step's keys are stored and the attention runs on the turned cache; against the oracle's rotation
+    followed by its attention, cache bytes bit-exact.  With the three inputs empty nothing is turned."""
+    print("[plugin] paged attention with cache rotation", cache_dtype, per_token, flush=True)
+    Hq, Hkv, D, bs = 8, 2, 128, 32
+    seqs = [(200, 1), (70, 3), (0, 40), (500, 1)]
+    qd = W.BF16 if cache_dtype == W.BF16 else W.F16
+    case = W.make_paged_case(99, seqs, Hq, Hkv, D, bs, qd, qd, cache_dtype)
+    begins, ids, nb = case["block_indices_begins"], case["block_indices"], case["num_blocks"]
+    theta = 10000.0 ** (-np.arange(D // 2, dtype=np.float64) * 2.0 / D)
+    ang = np.arange(64, dtype=np.float64)[:, None] * theta[None, :]
+    lut = np.concatenate([np.cos(ang), np.sin(ang)], axis=1).astype(np.float32)
+    rng = np.random.default_rng(3)
+    rotated = np.array([ids[begins[0] + 1], ids[begins[0] + 2], ids[begins[3] + 7], nb + 1, ids[begins[1]]], np.int32)
+    deltas = rng.integers(0, 64, (len(rotated), bs if per_token else 1)).astype(np.int32)
+    g = P.GraphText("pa_rotation")
+    el = {W.F16: "f16", W.BF16: "bf16", W.U8: "u8"}
+    qp = g.parameter("q", qd, [-1, Hq * D])
+    kp = g.parameter("k", qd, [-1, Hkv * D])
+    vp = g.parameter("v", qd, [-1, Hkv * D])
+    row = case["key_cache"].shape[3] // hip.DTYPE_BYTES[cache_dtype]
+    kcp = g.parameter("key_cache", cache_dtype, [-1, Hkv, bs, row])
+    vcp = g.parameter("value_cache", cache_dtype, [-1, Hkv, bs, row])
+    idx = [g.parameter(n, P.I32, [-1]) for n in ("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")]
+    rest = [g.parameter("scale", W.F32, [-1]), g.parameter("sliding_window", P.I32, [-1]), g.parameter("alibi_slopes", W.F32, [-1]),
+            g.parameter("max_context_len", P.I32, [-1]), g.parameter("score_aggregation_window", P.I32, [-1]),
+            g.parameter("rotated_block_indices", P.I32, [-1]), g.parameter("rotation_deltas", P.I32, [-1, -1]),
+            g.parameter("rotation_trig_lut", W.F32, [-1, D])]
+    pa = g.add("PagedAttentionExtension", "attention", [qp, kp, vp, kcp, vcp] + idx + rest)
+    g.result("out", pa)
+    plugin = P.Plugin()
+    assert "attention" in plugin.query_model(g.model())
+    compiled = plugin.compile_model(g.model())
+    req = compiled.create_infer_request()
+    cache_shape = list(case["key_cache"].shape[:3]) + [row]
+    for use in (True, False):
+        kc_ref, vc_ref = case["key_cache"].copy(), case["value_cache"].copy()
+        if use:
+            oracle.rotate_key_cache(kc_ref, cache_dtype, rotated, deltas, lut, Hkv, D, bs)
+        ref = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc_ref, vc_ref, cache_dtype, case["past_lens"],
+                                     case["subsequence_begins"], ids, begins, Hq, Hkv, D, bs)
+        kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
+        vc = hip.DeviceBuffer.from_numpy(case["value_cache"])
+        host = {"q": (case["q_store"], qd), "k": (case["k_new_store"], qd), "v": (case["v_new_store"], qd),
+                "past_lens": (case["past_lens"], P.I32), "subsequence_begins": (case["subsequence_begins"], P.I32),
+                "block_indices": (ids, P.I32), "block_indices_begins": (begins, P.I32),
+                "scale": (np.zeros((0,), np.float32), W.F32), "sliding_window": (np.array([0], np.int32), P.I32),
+                "alibi_slopes": (np.zeros((0,), np.float32), W.F32),
+                "max_context_len": (np.array([case["max_context_len"]], np.int32), P.I32),
+                "score_aggregation_window": (np.zeros((0,), np.int32), P.I32),
+                "rotated_block_indices": (rotated if use else np.zeros((0,), np.int32), P.I32),
+                "rotation_deltas": (deltas if use else np.zeros((0, 1), np.int32), P.I32),
+                "rotation_trig_lut": (lut if use else np.zeros((0, D), np.float32), W.F32)}
+        for i, n in enumerate(compiled.input_names()):
+            if n in host:
+                req.set_input(i, *host[n])
+            else:
+                req.set_device_input(i, (kc if n == "key_cache" else vc).ptr, cache_dtype, cache_shape)
+        req.infer()
+        out, _ = req.output(0)
+        np.testing.assert_array_equal(kc.download(np.uint8, case["key_cache"].shape), kc_ref)
+        np.testing.assert_array_equal(vc.download(np.uint8, case["value_cache"].shape), vc_ref)
+        tol = 2e-3 if cache_dtype == W.F16 else 1e-2
+        assert H.scaled_bound_error(H.storage_to_f32(out, qd), ref, "plugin cache rotation %s" % use) <= tol
+        kc.free()
+        vc.free()

@@ -95,7 +95,8 @@ def test_sdpa_takes_the_operators_optional_inputs():
 def test_paged_attention_takes_the_operators_full_signature():
     """Exported models carry the inputs behind max_context_len (score aggregation, cache rotation,
     sparse attention, sinks) and the scores output even when the features are off: such a node is
-    supported as long as those inputs are empty, and refused when they hold data."""
+    supported as long as the inputs of what is not built (sparse attention, sinks) are empty, and refused
+    when they hold data; score aggregation and the three cache-rotation inputs may hold data."""
     plugin = P.Plugin()
     assert "paged_attention" in plugin.query_model(P.Model.paged_attention(P.F16, P.F16, P.U8, 32, 8, 128, 32))
     for extra in (1, 4, 8):
@@ -106,7 +107,11 @@ def test_paged_attention_takes_the_operators_full_signature():
     windowed = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=1, extra_len=16, scores_result=True)
     assert "paged_attention" in plugin.query_model(windowed)  # score_aggregation_window may hold data
     rotated = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=4, extra_len=16)
-    assert "paged_attention" not in plugin.query_model(rotated)
+    assert "paged_attention" in plugin.query_model(rotated)  # cache rotation: indices, deltas and the table together
+    half_rotated = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=3, extra_len=16)
+    assert "paged_attention" not in plugin.query_model(half_rotated)  # ... not two of the three
+    sparse = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=5, extra_len=16)
+    assert "paged_attention" not in plugin.query_model(sparse)  # xattention_threshold holds data
     unknown_inputs = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, extra_inputs=9, extra_len=0)
     assert "paged_attention" not in plugin.query_model(unknown_inputs)
     alibi = P.Model.paged_attention(P.F16, P.F16, P.F16, 32, 8, 128, 32, alibi_len=32)
