@@ -240,6 +240,12 @@ typedef struct hipattn_pa_desc {
      * kernels and the shape-generic kernels take it as one multiply-add per score; multi-token sequences then
      * go to the plain query-tile kernel rather than the tuned chunk kernel, one kernel after the other. */
     const float* alibi_slopes;
+    /* The operator's `sinks` input: NULL, or a device pointer to num_heads_q floats, a logit per query head that
+     * takes part in the softmax of every row of that head without a value row of its own ("attention sink"):
+     * out = sum_j exp(s_j) v_j / (sum_j exp(s_j) + exp(sink)).  A row with nothing to attend stays zeros.  The
+     * decode kernels, the query-tile kernel (which takes the multi-token sequences of such a call) and the
+     * shape-generic kernels add the term where they normalise; the scores entry point refuses the call. */
+    const float* sinks;
 } hipattn_pa_desc;
 
 hipattn_status hipattn_paged_attention_workspace_size(const hipattn_pa_desc* desc, size_t* bytes);

@@ -79,6 +79,7 @@ class PaDesc(ctypes.Structure):
         ("flags", ctypes.c_int),
         ("decode_waves", ctypes.c_int),
         ("alibi_slopes", ctypes.c_void_p),  # device pointer to num_heads_q floats, or None
+        ("sinks", ctypes.c_void_p),         # device pointer to num_heads_q floats, or None
     ]
 
 

@@ -44,9 +44,10 @@ struct MaskRow {
 // bias(j) is added to the scaled score of key j.  Every lane of the wavefront must call this; the
 // result for head-dim slot d = lane + 64 * i is returned in o[i], already normalised.  A row that
 // can attend nothing (empty range, every key masked with -inf) yields zeros.
+// sink: -INFINITY, or a logit that joins the row's softmax without a value row (the denominator grows by exp(sink)).
 template <typename KV, typename Bias>
 __device__ __forceinline__ void attend_row_wave(const float* q_lds, const KV& kv, const Bias& bias, int j0, int j1, int D,
-                                                float scale, float (&o)[kGenericSlots]) {
+                                                float scale, float (&o)[kGenericSlots], float sink = -INFINITY) {
     const int lane = threadIdx.x & 63;
     float m = -INFINITY, l = 0.0f;
 #pragma unroll
@@ -81,6 +82,7 @@ __device__ __forceinline__ void attend_row_wave(const float* q_lds, const KV& kv
             }
         }
     }
+    if (l > 0.0f && sink != -INFINITY) l += fast_exp2(sink * kLog2e - m);
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
 #pragma unroll
     for (int i = 0; i < kGenericSlots; i++) o[i] *= inv;
@@ -196,10 +198,11 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void paged_generic_kernel(Page
     int j0 = 0;
     if (p.sliding_window > 0 && pos - p.sliding_window + 1 > 0) j0 = pos - p.sliding_window + 1;
     float o[kGenericSlots];
+    const float sink = p.sinks ? p.sinks[h] : -INFINITY;
     if (p.alibi_slopes)
-        attend_row_wave(q_lds[wave], kv, DistanceBias{p.alibi_slopes[h], pos}, j0, j1, D, p.scale, o);
+        attend_row_wave(q_lds[wave], kv, DistanceBias{p.alibi_slopes[h], pos}, j0, j1, D, p.scale, o, sink);
     else
-        attend_row_wave(q_lds[wave], kv, NoBias{}, j0, j1, D, p.scale, o);
+        attend_row_wave(q_lds[wave], kv, NoBias{}, j0, j1, D, p.scale, o, sink);
 #pragma unroll
     for (int sl = 0; sl < kGenericSlots; sl++) {
         const int d = lane + 64 * sl;

@@ -1411,8 +1411,9 @@ hipError_t launch_paged_prefill(const PagedParams& p, hipStream_t stream) {
     // the head sizes between 64 and 128 of a 16-bit cache: this kernel on rows of fewer columns
     const bool padded = p.head_dim > 64 && p.head_dim < flash::kD && p.head_dim % 8 == 0 && p.cache_dtype != HIPATTN_U8 &&
                         (((uintptr_t)p.q | (uintptr_t)p.key_cache | (uintptr_t)p.value_cache | (uintptr_t)p.out) & 15) == 0;
-    // (ALiBi: the plain kernel has the distance term, the tuned one has no vector slot to spare for it)
-    if ((p.head_dim != flash::kD && !padded) || p.alibi_slopes) return launch_paged_prefill_small(p, stream);  // the plain kernel, padded columns
+    // (ALiBi, attention sinks: the plain kernel has the distance term and the sink in its denominator; the tuned one
+    // has no vector slot to spare for the one and was not given the other)
+    if ((p.head_dim != flash::kD && !padded) || p.alibi_slopes || p.sinks) return launch_paged_prefill_small(p, stream);  // the plain kernel, padded columns
     const int G = p.num_heads_q / p.num_heads_kv;
     dim3 grid((unsigned)((int64_t)p.max_q_tiles * ((G & 1) == 0 ? p.num_heads_q / 2 : p.num_heads_q)));
     if (padded) {

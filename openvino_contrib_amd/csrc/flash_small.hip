@@ -181,6 +181,7 @@ struct Work {
     float scale;
     const float* alibi;     // paged: nullptr, or the ALiBi slope of row 0's query head; row r's is alibi[r * alibi_step]
     int alibi_step;         // 0: every row belongs to one head; 1: the rows are consecutive query heads
+    const float* sink;      // paged: nullptr, or the attention-sink logit of row 0's query head; row r's is sink[r * alibi_step]
     const uint8_t* mask;    // kMask: the mask row of query row 0 (this batch, this head)
     int64_t mask_row_stride, mask_key_stride;  // in elements
     int mask_dtype;
@@ -489,7 +490,10 @@ __device__ __forceinline__ void attend(const Work& w, uint8_t (*lds)[2][tile_byt
     // normalise and store: register r of o[dt] is head-dim 32 dt + 8 (r / 4) + 4 hi + r % 4 of query row n32
     float l_lo, l_hi;
     pair_values(l_run, l_lo, l_hi);
-    const float l = l_lo + l_hi;
+    float l = l_lo + l_hi;
+    if constexpr (kPaged) {  // the attention sink of the row's head: a logit in the denominator without a value row
+        if (w.sink != nullptr && l > 0.0f) l += fast_exp2(w.sink[min(my_row, w.rows - 1) * w.alibi_step] * kLog2e - m_run);
+    }
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
     if (my_row < w.rows) {
 #pragma unroll
@@ -545,6 +549,7 @@ __device__ __forceinline__ void sdpa_small_tile(const SdpaParams& p, uint8_t (*l
     w.scale = p.scale;
     w.alibi = nullptr;
     w.alibi_step = 0;
+    w.sink = nullptr;
     w.mask = nullptr;
     w.mask_row_stride = w.mask_key_stride = 0;
     w.mask_dtype = 0;
@@ -633,6 +638,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2))
     w.scale = p.scale;
     w.alibi = p.alibi_slopes ? p.alibi_slopes + (heads_as_rows ? h * G : h) : nullptr;
     w.alibi_step = heads_as_rows ? 1 : 0;
+    w.sink = p.sinks ? p.sinks + (heads_as_rows ? h * G : h) : nullptr;
     w.mask = nullptr;
     w.mask_row_stride = w.mask_key_stride = 0;
     w.mask_dtype = 0;

@@ -128,6 +128,7 @@ hipattn::PagedParams make_paged_params(const hipattn_pa_desc* d) {
     p.num_waves = d->decode_waves > 0 ? d->decode_waves : 0;
     p.any_lengths = (d->flags & HIPATTN_PA_ANY_LENGTHS) ? 1 : 0;
     p.alibi_slopes = d->alibi_slopes;
+    p.sinks = d->sinks;
     p.kv_share = 1;
     // (more than 16 query heads per kv head: see split_kv_heads; the forced shape-generic path keeps the heads as they are)
     if (!(d->flags & HIPATTN_PA_FORCE_GENERIC)) p = hipattn::split_kv_heads(p);
@@ -599,6 +600,7 @@ HIPATTN_EXPORT hipattn_status hipattn_paged_attention_scores(const hipattn_pa_de
         return fail(HIPATTN_INVALID_ARGUMENT, "paged_attention_scores: null pointer");
     if (desc->num_seqs > 65535) return fail(HIPATTN_UNSUPPORTED, "paged_attention_scores: %d sequences (at most 65535)", desc->num_seqs);
     if (desc->alibi_slopes) return fail(HIPATTN_UNSUPPORTED, "paged_attention_scores: no distance bias (alibi_slopes) in the scores kernels");
+    if (desc->sinks) return fail(HIPATTN_UNSUPPORTED, "paged_attention_scores: no attention sinks in the scores kernels");
     const size_t need = (size_t)desc->num_tokens * desc->num_heads_q * sizeof(float);
     if (!workspace || workspace_bytes < need)
         return fail(HIPATTN_WORKSPACE_TOO_SMALL, "paged_attention_scores: workspace of %zu bytes, %zu needed", workspace_bytes, need);

@@ -116,6 +116,7 @@ struct PagedParams {
     // of num_heads_q / that many query heads each, consecutive ones sharing the K/V rows of kv head h / kv_share
     // (split_kv_heads; 1 otherwise).  Only the K/V addresses divide by it; the chunk kernels get the heads undivided.
     int kv_share;
+    const float* sinks;         // nullptr, or [num_heads_q]: a logit per query head in the denominator of every row's softmax (no value row)
     const float* alibi_slopes;  // nullptr, or [num_heads_q]: slope * (key position - query position) joins the scaled score
     // decode: the batch's block-heads are cut into num_waves equal pieces (one per wavefront);
     // pieces that do not cover a whole (sequence, kv head) segment leave partials in the workspace

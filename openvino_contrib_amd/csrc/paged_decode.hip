@@ -689,6 +689,8 @@ __device__ __forceinline__ void merge_segment_head(const PagedParams& p, const L
             }
         }
     }
+    // (the attention sink of the head, when there is one: a logit in the denominator without a value row)
+    if (p.sinks != nullptr && l_run > 0.0f) l_run += fast_exp2(p.sinks[h * G + g] * kLog2e - m_run);
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
 #pragma unroll
     for (int c = 0; c < 2; c++) {
@@ -749,6 +751,7 @@ struct MergeArgs {
     unsigned long long merge_tag;
     void* out;
     int out_dtype, num_heads_q, num_heads_kv, head_dim;
+    const float* sinks;
 };
 template <int kHD, bool kPad>
 __device__ __forceinline__ void merge_in_kernel(const MergeArgs& p, const Line& line, int s, int h, int token,
@@ -815,6 +818,7 @@ __device__ __forceinline__ void merge_in_kernel(const MergeArgs& p, const Line& 
         }
     }
     if (!mine) return;
+    if (p.sinks != nullptr && l_run > 0.0f) l_run += fast_exp2(p.sinks[h * G + n16] * kLog2e - m_run);
     const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
@@ -1136,6 +1140,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         }
         const int64_t slot = (int64_t)piece + (int64_t)s * Hkv + h;  // unique per (piece, segment)
         if (n16 < G) {
+            if (whole && p.sinks != nullptr && l > 0.0f) l += fast_exp2(p.sinks[h * G + n16] * kLog2e - st.m);
             const float inv = whole ? (l > 0.0f ? 1.0f / l : 0.0f) : 1.0f;
             // acc[e][r] is head-dim (kg*4 + r)*8 + e: eight consecutive outputs per r
 #pragma unroll
@@ -1187,7 +1192,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 
         else
             mr = ((const DecodeRange*)p.seq_info)[ms];
         const int64_t first_unit = (int64_t)prefix_at(ms) * Hkv + (int64_t)mh * (mr.nb + p.switch_cost) + p.switch_cost;
-        const MergeArgs ma = {p.part_out, p.part_ml, p.part_flag, p.merge_tag, p.out, p.out_dtype, p.num_heads_q, p.num_heads_kv, p.head_dim};
+        const MergeArgs ma = {p.part_out, p.part_ml, p.part_flag, p.merge_tag, p.out, p.out_dtype, p.num_heads_q, p.num_heads_kv, p.head_dim, p.sinks};
         merge_in_kernel<kHD, kPad>(ma, line, ms, mh, mr.token, line.piece_at(first_unit), piece, lane);
         merge_seg = -1;
     }
@@ -1659,6 +1664,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         }
         const int64_t slot = (int64_t)w + (int64_t)s * Hkv + h;  // unique per (piece, segment)
         if (n16 < G) {
+            if (whole && p.sinks != nullptr && l > 0.0f) l += fast_exp2(p.sinks[h * G + n16] * kLog2e - st.m);
             const float inv = whole ? (l > 0.0f ? 1.0f / l : 0.0f) : 1.0f;
 #pragma unroll
             for (int half = 0; half < 2; half++)

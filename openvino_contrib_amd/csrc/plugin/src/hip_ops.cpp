@@ -231,13 +231,15 @@ private:
 
 // Input order of the OpenVINO operator.  score_aggregation_window belongs to the scores output
 // (built: the aggregated probabilities a cache-eviction policy reads); the three rotation inputs to the
-// cache rotation (built: hipattn_rotate_key_cache ahead of the attention); everything behind them belongs
-// to features this plugin does not implement (sparse attention, sinks): such inputs are accepted when
-// they are empty, as exported models carry them, and refused when they hold data.
+// cache rotation (built: hipattn_rotate_key_cache ahead of the attention); sinks, the last one, holds one f32
+// logit per query head or nothing (built: the term joins the denominators); the three inputs of sparse
+// attention are not implemented: they are accepted when they are empty, as exported models carry them,
+// and refused when they hold data.
 enum PaInput {
     kQuery = 0, kKey, kValue, kKeyCache, kValueCache, kPastLens, kSubsequenceBegins, kBlockIndices,
     kBlockIndicesBegins, kScale, kSlidingWindow, kAlibiSlopes, kMaxContextLen, kPaRequiredInputs,
-    kScoreAggregationWindow = kPaRequiredInputs, kRotatedBlockIndices, kRotationDeltas, kRotationTrigLut
+    kScoreAggregationWindow = kPaRequiredInputs, kRotatedBlockIndices, kRotationDeltas, kRotationTrigLut,
+    kXattentionThreshold, kXattentionBlockSize, kXattentionStride, kSinks
 };
 const char* const kPaOptionalNames[] = {"score_aggregation_window", "rotated_block_indices", "rotation_deltas",
                                         "rotation_trig_lut",        "xattention_threshold",  "xattention_block_size",
@@ -256,8 +258,10 @@ public:
             HIP_PLUGIN_THROW(who + std::to_string(num_inputs_) + " inputs: more than this plugin knows of");
         if (num_outputs_ < 1 || num_outputs_ > 2) HIP_PLUGIN_THROW(who + std::to_string(num_outputs_) + " outputs");
         for (size_t i = kRotationTrigLut + 1; i < num_inputs_; i++)
-            if (statically_non_empty(node.get_input_partial_shape(i)))
+            if (i != kSinks && statically_non_empty(node.get_input_partial_shape(i)))
                 HIP_PLUGIN_THROW(who + kPaOptionalNames[i - kPaRequiredInputs] + " holds data: the feature is not supported");
+        if (num_inputs_ > kSinks && node.get_input_element_type(kSinks) != ov::element::f32 && !statically_empty(node.get_input_partial_shape(kSinks)))
+            HIP_PLUGIN_THROW(who + "sinks must be f32");
         if (num_inputs_ > kRotationTrigLut) {
             for (int i : {kRotatedBlockIndices, kRotationDeltas})
                 if (node.get_input_element_type(i) != ov::element::i32 && !statically_empty(node.get_input_partial_shape(i)))
@@ -318,7 +322,7 @@ public:
     std::vector<size_t> UpdatedInputs() const override { return {kKeyCache, kValueCache}; }
     // launch parameters, and inputs that must be empty: none of them is handed to a kernel
     bool InputIsHostOnly(size_t input) const override {
-        return input == kScale || input == kSlidingWindow || input == kMaxContextLen || input > kRotationTrigLut;
+        return input == kScale || input == kSlidingWindow || input == kMaxContextLen || (input > kRotationTrigLut && input != kSinks);
     }
 
     // max_context_len is advisory for the attention kernels; only the scores kernels size a grid by it
@@ -399,7 +403,7 @@ private:
         HIP_PLUGIN_ASSERT(q.size() == 2, "query must be [tokens, heads * head_size], got " + shape_str(q));
         HIP_PLUGIN_ASSERT(kc.size() == 4 && in[kValueCache].shape == kc, "key/value cache shapes " + shape_str(kc));
         for (size_t i = kRotationTrigLut + 1; i < num_inputs_; i++)
-            HIP_PLUGIN_ASSERT(ov::shape_size(in[i].shape) == 0,
+            HIP_PLUGIN_ASSERT(i == kSinks || ov::shape_size(in[i].shape) == 0,
                               std::string(kPaOptionalNames[i - kPaRequiredInputs]) + " holds data: the feature is not supported");
         if (num_inputs_ > kRotatedBlockIndices && num_inputs_ <= kRotationTrigLut)
             for (size_t i = kRotatedBlockIndices; i < num_inputs_; i++)
@@ -436,6 +440,11 @@ private:
                               "alibi_slopes must hold one value per query head (" + std::to_string(d.num_heads_q) + "), got " +
                                   shape_str(in[kAlibiSlopes].shape));
             d.alibi_slopes = (const float*)in[kAlibiSlopes].device;
+        }
+        if (num_inputs_ > kSinks && ov::shape_size(in[kSinks].shape) > 0) {
+            HIP_PLUGIN_ASSERT(ov::shape_size(in[kSinks].shape) == (size_t)d.num_heads_q,
+                              "sinks must hold one value per query head (" + std::to_string(d.num_heads_q) + "), got " + shape_str(in[kSinks].shape));
+            d.sinks = (const float*)in[kSinks].device;
         }
         return d;
     }

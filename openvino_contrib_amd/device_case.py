@@ -62,13 +62,14 @@ def run_sdpa_masked(hip, case, mask, scale=0.0, mask_dtype=None):
     return storage_to_f32(res, case["dtype"]), path
 
 
-def pa_desc(hip, case, out_dtype=None, flags=0, decode_waves=0, scale=0.0, max_context_len=None, alibi=None):
-    """alibi: None or a DeviceBuffer of Hq floats (the operator's alibi_slopes input)."""
+def pa_desc(hip, case, out_dtype=None, flags=0, decode_waves=0, scale=0.0, max_context_len=None, alibi=None, sinks=None):
+    """alibi, sinks: None or a DeviceBuffer of Hq floats (the operator's alibi_slopes / sinks input)."""
     return hip.PaDesc(case["q_dtype"], case["kv_dtype"], case["cache_dtype"],
                       case["q_dtype"] if out_dtype is None else out_dtype, case["Hq"], case["Hkv"], case["D"],
                       case["block_size"], case["num_blocks"], case["T"], case["S"],
                       case["max_context_len"] if max_context_len is None else max_context_len,
-                      case["sliding_window"], scale, flags, decode_waves, alibi.ptr if alibi is not None else None)
+                      case["sliding_window"], scale, flags, decode_waves, alibi.ptr if alibi is not None else None,
+                      sinks.ptr if sinks is not None else None)
 
 
 class PagedDeviceCase:
@@ -90,9 +91,9 @@ class PagedDeviceCase:
         self.out_elems = case["T"] * case["Hq"] * case["D"]
         self.out = hip.DeviceBuffer(self.out_elems * hip.DTYPE_BYTES[self.out_dtype])
 
-    def run(self, flags=0, decode_waves=0, scale=0.0, max_context_len=None, stream=None, alibi=None):
+    def run(self, flags=0, decode_waves=0, scale=0.0, max_context_len=None, stream=None, alibi=None, sinks=None):
         hip = self.hip
-        desc = pa_desc(hip, self.case, self.out_dtype, flags, decode_waves, scale, max_context_len, alibi)
+        desc = pa_desc(hip, self.case, self.out_dtype, flags, decode_waves, scale, max_context_len, alibi, sinks)
         nbytes = hip.paged_attention_workspace_size(desc)
         ws = hip.DeviceBuffer(nbytes) if nbytes else None
         self.out.fill(0xFF)

@@ -258,9 +258,11 @@ static inline float dotf(const float* a, const float* b, int n) {
  * One query row against keys [j0, j1) given as row pointers computed by the caller's
  * stride; scores buffer must hold j1 - j0 floats.
  */
-static void attend_row_biased(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0,
-                              int j1, int D, float scale, const float* bias, int64_t bias_stride, float* scores,
-                              float* out) {
+/* sink: -INFINITY, or a logit that takes part in the row's softmax without a value row of its own (an
+ * "attention sink": the row's probabilities then sum to less than one). */
+static void attend_row_sink(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0,
+                            int j1, int D, float scale, const float* bias, int64_t bias_stride, float sink, float* scores,
+                            float* out) {
     int n = j1 - j0;
     if (n <= 0) {
         for (int d = 0; d < D; d++) out[d] = 0.0f;
@@ -273,7 +275,8 @@ static void attend_row_biased(const float* q, const float* kbase, const float* v
         scores[j] = s;
         m = s > m ? s : m;
     }
-    double l = 0.0;
+    if (sink > m) m = sink;
+    double l = sink > -INFINITY ? exp((double)sink - (double)m) : 0.0;
     for (int j = 0; j < n; j++) {
         float p = expf(scores[j] - m);
         scores[j] = p;
@@ -287,6 +290,12 @@ static void attend_row_biased(const float* q, const float* kbase, const float* v
     }
     float inv = (float)(1.0 / l);
     for (int d = 0; d < D; d++) out[d] *= inv;
+}
+
+static void attend_row_biased(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0,
+                              int j1, int D, float scale, const float* bias, int64_t bias_stride, float* scores,
+                              float* out) {
+    attend_row_sink(q, kbase, vbase, kv_stride, j0, j1, D, scale, bias, bias_stride, -INFINITY, scores, out);
 }
 
 static void attend_row(const float* q, const float* kbase, const float* vbase, int64_t kv_stride, int j0, int j1,
@@ -449,6 +458,11 @@ ORACLE_API void oracle_gather_cache_rows(const uint8_t* cache, int cache_dtype, 
  * PARITY UNPINNED against OpenVINO for this input (sign and origin restated from the operator's
  * documentation); pinned against an explicit additive mask through torch's fp64
  * scaled_dot_product_attention (tests/golden/make_alibi_golden.py) and against the fp64 closed form.
+ * sinks (NULL, or one float per query head): a logit that joins every row's softmax of that head without a
+ * value row ("attention sink"): out = sum_j exp(s_j) v_j / (sum_j exp(s_j) + exp(sink)); a row left with
+ * nothing to attend is zeros all the same.  PARITY UNPINNED against OpenVINO (restated from the operator's
+ * documentation and the models that carry the input); pinned by the fp64 closed form, by "a sink of -inf
+ * changes nothing" and by the equivalent extra key with a value row of zeros (tests/test_oracle_cpu.py).
  * scale <= 0 selects 1/sqrt(D).
  */
 ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const float* v_new, uint8_t* key_cache,
@@ -456,7 +470,7 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
                                       const int32_t* subsequence_begins, const int32_t* block_indices,
                                       const int32_t* block_indices_begins, int S, int Hq, int Hkv, int D,
                                       int block_size, int num_blocks, float scale, int sliding_window, int do_write,
-                                      const float* alibi_slopes, float* out) {
+                                      const float* alibi_slopes, const float* sinks, float* out) {
     if (S < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || block_size <= 0) return 1;
     if (scale <= 0.0f) scale = 1.0f / sqrtf((float)D);
     if (do_write)
@@ -509,9 +523,11 @@ ORACLE_API int oracle_paged_attention(const float* q, const float* k_new, const 
                 } else if (alibi_slopes) {
                     float slope = alibi_slopes[h * G + g];
                     for (int j = j0; j < j1; j++) rowbias[j] = bias[j] + slope * (float)(j - p);
-                    attend_row_biased(q + row, kbuf, vbuf, D, j0, j1, D, scale, rowbias, 1, scores, out + row);
+                    attend_row_sink(q + row, kbuf, vbuf, D, j0, j1, D, scale, rowbias, 1, sinks ? sinks[h * G + g] : -INFINITY, scores,
+                                    out + row);
                 } else {
-                    attend_row_biased(q + row, kbuf, vbuf, D, j0, j1, D, scale, holes ? bias : NULL, 1, scores, out + row);
+                    attend_row_sink(q + row, kbuf, vbuf, D, j0, j1, D, scale, holes ? bias : NULL, 1, sinks ? sinks[h * G + g] : -INFINITY,
+                                    scores, out + row);
                 }
             }
         }

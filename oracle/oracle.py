@@ -60,7 +60,7 @@ def lib():
         L.oracle_gather_cache_rows.argtypes = [vp, i32, vp, i32, i32, i32, i32, i32, vp]
         L.oracle_gather_cache_rows.restype = None
         L.oracle_paged_attention.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
-                                             f32, i32, i32, vp, vp]
+                                             f32, i32, i32, vp, vp, vp]
         L.oracle_paged_attention.restype = i32
         L.oracle_paged_attention_scores.argtypes = [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp]
         L.oracle_paged_attention_scores.restype = i32
@@ -231,8 +231,8 @@ def gather_cache_rows(cache, cache_dtype, seq_blocks, n, h, Hkv, D, block_size):
 
 def paged_attention(q, k_new, v_new, key_cache, value_cache, cache_dtype, past_lens, subsequence_begins,
                     block_indices, block_indices_begins, Hq, Hkv, D, block_size, scale=0.0, sliding_window=0,
-                    do_write=True, alibi_slopes=None):
-    """q [T, Hq*D] fp32; caches are uint8 views, updated in place when do_write; alibi_slopes: None or [Hq] f32.
+                    do_write=True, alibi_slopes=None, sinks=None):
+    """q [T, Hq*D] fp32; caches are uint8 views, updated in place when do_write; alibi_slopes, sinks: None or [Hq] f32.
     Returns out [T, Hq*D]."""
     q = _c(q, np.float32)
     k_new, v_new = _c(k_new, np.float32), _c(v_new, np.float32)
@@ -242,10 +242,12 @@ def paged_attention(q, k_new, v_new, key_cache, value_cache, cache_dtype, past_l
     out = np.zeros_like(q)
     al = None if alibi_slopes is None else _c(alibi_slopes, np.float32)
     assert al is None or al.shape == (Hq,)
+    sk = None if sinks is None else _c(sinks, np.float32)
+    assert sk is None or sk.shape == (Hq,)
     rc = lib().oracle_paged_attention(_p(q), _p(k_new), _p(v_new), _p(key_cache), _p(value_cache), cache_dtype,
                                       _p(pl), _p(sb), _p(bi), _p(bb), len(pl), Hq, Hkv, D, block_size,
                                       key_cache.shape[0], float(scale), int(sliding_window), int(bool(do_write)),
-                                      _p(al) if al is not None else None, _p(out))
+                                      _p(al) if al is not None else None, _p(sk) if sk is not None else None, _p(out))
     if rc:
         raise ValueError("oracle_paged_attention: bad arguments")
     return out

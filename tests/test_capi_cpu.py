@@ -28,9 +28,9 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_layout_matches_header():
-    # 9 four-byte fields; 16 four-byte fields and one pointer, no padding
+    # 9 four-byte fields; 16 four-byte fields and two pointers, no padding
     assert ctypes.sizeof(capi.SdpaDesc) == 36
-    assert ctypes.sizeof(capi.PaDesc) == 72 and capi.PaDesc.alibi_slopes.offset == 64
+    assert ctypes.sizeof(capi.PaDesc) == 80 and capi.PaDesc.alibi_slopes.offset == 64 and capi.PaDesc.sinks.offset == 72
     # int + four int64, the int64s aligned to 8
     assert ctypes.sizeof(capi.MaskDesc) == 40 and capi.MaskDesc.stride.offset == 8
 

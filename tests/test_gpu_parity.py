@@ -1402,6 +1402,60 @@ def test_paged_errors(hip):
 
 
 
+# ---- attention sinks ------------------------------------------------------------------------------
+@pytest.mark.parametrize("D,bs,Hq,Hkv,q_dtype,cache_dtype,path", [
+    (64, 32, 64, 8, W.BF16, W.BF16, "paged_mfma"), (128, 32, 32, 8, W.F16, W.F16, "paged_mfma"), (128, 16, 16, 8, W.BF16, W.U8, "paged_mfma"),
+    (64, 16, 8, 2, W.F16, W.U8, "paged_mfma"), (96, 64, 12, 4, W.F16, W.F16, "paged_mfma"), (256, 32, 8, 2, W.F16, W.F16, "paged_mfma"),
+    (128, 32, 48, 1, W.F16, W.F16, "paged_mfma"), (80, 8, 8, 2, W.F16, W.F16, "paged_mfma_tiles"), (128, 16, 34, 2, W.BF16, W.U8, "paged_mfma_tiles"),
+    (64, 16, 4, 2, W.F32, W.F32, "paged_generic")])
+@pytest.mark.parametrize("kind,window", [("decode", 0), ("decode", 128), ("mixed", 0), ("mixed", 128), ("prefill", 0)])
+def test_paged_attention_with_sinks(hip, oracle, D, bs, Hq, Hkv, q_dtype, cache_dtype, path, kind, window):
+    """The operator's sinks input: a logit per query head in the denominator of every row's softmax, no value row;
+    the decode kernels (rows that one wavefront finishes, rows combined inside the kernel and behind it), the
+    query-tile kernel (which takes the multi-token sequences of such a call) and the shape-generic kernels,
+    against the oracle, whose term the closed form pins.  No sinks and sinks of -1e30 give the same bits."""
+    announce("paged sinks", D, bs, Hq, Hkv, q_dtype, cache_dtype, kind, window)
+    if kind == "decode":
+        seqs = [(c - 1, 1) for c in DECODE_CTX]
+    elif kind == "mixed":
+        seqs = [(0, 9), (37, 1), (31, 2), (5, 140), (64, 1), (700, 1), (15, 1), (300, 130), (0, 1), (1000, 3)]
+    else:
+        seqs = [(0, 200), (0, 16), (3, 17), (0, 1)]
+    case = W.make_paged_case(117, seqs, Hq, Hkv, D, bs, q_dtype, q_dtype, cache_dtype, sliding_window=window)
+    sinks = np.random.default_rng(Hq).uniform(-2.0, 3.0, Hq).astype(np.float32)
+    kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+    ref = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc, vc, cache_dtype, case["past_lens"],
+                                 case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
+                                 sliding_window=window, sinks=sinks)
+    plain, _, _ = H.oracle_paged(oracle, case)
+    assert np.abs(plain - ref).max() > 1e-2
+    dev = H.PagedDeviceCase(hip, case)
+    dsinks = hip.DeviceBuffer.from_numpy(sinks)
+    tol = 1e-4 if q_dtype == W.F32 else (1e-2 if (cache_dtype in (W.U8, W.BF16) or q_dtype == W.BF16) else 2e-3)
+    for waves, fused in ((0, 1), (9, 1), (9, 0), (300, 0)):
+        hip.set_option("decode_fused_merge", fused)
+        out, got_path = dev.run(decode_waves=waves, flags=hip.PA_SKIP_CACHE_WRITE if (waves, fused) != (0, 1) else 0, sinks=dsinks)
+        assert got_path == path
+        assert np.isfinite(out).all()
+        assert H.scaled_bound_error(out, ref, "paged sinks") <= tol, (waves, fused)
+    hip.set_option("decode_fused_merge", -1)
+    kc_dev, vc_dev = dev.caches()
+    np.testing.assert_array_equal(kc_dev, kc)
+    np.testing.assert_array_equal(vc_dev, vc)
+    gen, path_g = dev.run(flags=hip.PA_SKIP_CACHE_WRITE | hip.PA_FORCE_GENERIC, sinks=dsinks)
+    assert path_g == "paged_generic" and H.scaled_bound_error(gen, ref, "paged sinks, generic") <= tol
+    dnone = hip.DeviceBuffer.from_numpy(np.full(Hq, -1e30, np.float32))
+    out0, _ = dev.run(flags=hip.PA_SKIP_CACHE_WRITE, sinks=dnone)
+    if kind == "decode" or path != "paged_mfma":
+        out1, _ = dev.run(flags=hip.PA_SKIP_CACHE_WRITE)
+        np.testing.assert_array_equal(out0, out1)
+    else:  # (the chunks of a call with sinks go to the query-tile kernel: another kernel than without)
+        assert H.scaled_bound_error(out0, plain, "paged sinks of -1e30") <= tol
+    for b in (dsinks, dnone):
+        b.free()
+    dev.free()
+
+
 # ---- the operator's cache rotation ---------------------------------------------------------------
 def trig_lut(rows, D, base=10000.0):
     theta = base ** (-np.arange(D // 2, dtype=np.float64) * 2.0 / D)

@@ -647,3 +647,61 @@ def test_paged_attention_with_cache_rotation_through_the_plugin(hip, oracle, cac
         assert H.scaled_bound_error(H.storage_to_f32(out, qd), ref, "plugin cache rotation %s" % use) <= tol
         kc.free()
         vc.free()
+
+
+@pytest.mark.parametrize("seqs", [[(300, 1), (70, 1), (1000, 1), (5, 1)], [(200, 1), (70, 3), (0, 140), (500, 1)]])
+def test_paged_attention_with_sinks_through_the_plugin(hip, oracle, seqs):
+    """The operator's last input, sinks, with one f32 logit per query head (as [1, heads, 1, 1]), on a shape of the
+    models that carry it: head size 64, 64 query heads on 8 kv heads, a sliding window of 128, bf16.  Against the
+    oracle; the sparse-attention inputs in front of it stay empty."""
+    print("[plugin] paged attention with sinks", len(seqs), flush=True)
+    Hq, Hkv, D, bs, window = 64, 8, 64, 32, 128
+    case = W.make_paged_case(100, seqs, Hq, Hkv, D, bs, W.BF16, W.BF16, W.BF16, sliding_window=window)
+    sinks = np.random.default_rng(8).uniform(-1.0, 3.0, Hq).astype(np.float32)
+    g = P.GraphText("pa_sinks")
+    qp = g.parameter("q", W.BF16, [-1, Hq * D])
+    kp = g.parameter("k", W.BF16, [-1, Hkv * D])
+    vp = g.parameter("v", W.BF16, [-1, Hkv * D])
+    kcp = g.parameter("key_cache", W.BF16, [-1, Hkv, bs, D])
+    vcp = g.parameter("value_cache", W.BF16, [-1, Hkv, bs, D])
+    idx = [g.parameter(n, P.I32, [-1]) for n in ("past_lens", "subsequence_begins", "block_indices", "block_indices_begins")]
+    rest = [g.parameter("scale", W.F32, [-1]), g.parameter("sliding_window", P.I32, [-1]), g.parameter("alibi_slopes", W.F32, [-1]),
+            g.parameter("max_context_len", P.I32, [-1]), g.parameter("score_aggregation_window", P.I32, [-1]),
+            g.parameter("rotated_block_indices", P.I32, [-1]), g.parameter("rotation_deltas", P.I32, [-1, -1]),
+            g.parameter("rotation_trig_lut", W.F32, [-1, D]), g.parameter("xattention_threshold", W.F32, [-1]),
+            g.parameter("xattention_block_size", P.I32, [-1]), g.parameter("xattention_stride", P.I32, [-1]),
+            g.parameter("sinks", W.F32, [1, -1, 1, 1])]
+    g.result("out", g.add("PagedAttentionExtension", "attention", [qp, kp, vp, kcp, vcp] + idx + rest))
+    plugin = P.Plugin()
+    assert "attention" in plugin.query_model(g.model())
+    compiled = plugin.compile_model(g.model())
+    req = compiled.create_infer_request()
+    kc_ref, vc_ref = case["key_cache"].copy(), case["value_cache"].copy()
+    ref = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc_ref, vc_ref, W.BF16, case["past_lens"],
+                                 case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs,
+                                 sliding_window=window, sinks=sinks)
+    kc = hip.DeviceBuffer.from_numpy(case["key_cache"])
+    vc = hip.DeviceBuffer.from_numpy(case["value_cache"])
+    empty_i, empty_f = (np.zeros((0,), np.int32), P.I32), (np.zeros((0,), np.float32), W.F32)
+    host = {"q": (case["q_store"], W.BF16), "k": (case["k_new_store"], W.BF16), "v": (case["v_new_store"], W.BF16),
+            "past_lens": (case["past_lens"], P.I32), "subsequence_begins": (case["subsequence_begins"], P.I32),
+            "block_indices": (case["block_indices"], P.I32), "block_indices_begins": (case["block_indices_begins"], P.I32),
+            "scale": empty_f, "sliding_window": (np.array([window], np.int32), P.I32), "alibi_slopes": empty_f,
+            "max_context_len": (np.array([case["max_context_len"]], np.int32), P.I32), "score_aggregation_window": empty_i,
+            "rotated_block_indices": empty_i, "rotation_deltas": (np.zeros((0, 1), np.int32), P.I32),
+            "rotation_trig_lut": (np.zeros((0, D), np.float32), W.F32), "xattention_threshold": empty_f,
+            "xattention_block_size": empty_i, "xattention_stride": empty_i, "sinks": (sinks.reshape(1, Hq, 1, 1), W.F32)}
+    cache_shape = list(case["key_cache"].shape[:3]) + [D]
+    for i, n in enumerate(compiled.input_names()):
+        if n in host:
+            req.set_input(i, *host[n])
+        else:
+            req.set_device_input(i, (kc if n == "key_cache" else vc).ptr, W.BF16, cache_shape)
+    req.infer()
+    out, _ = req.output(0)
+    np.testing.assert_array_equal(kc.download(np.uint8, case["key_cache"].shape), kc_ref)
+    assert H.scaled_bound_error(H.storage_to_f32(out, W.BF16), ref, "plugin sinks") <= 2e-2
+    plain, _, _ = H.oracle_paged(oracle, case)
+    assert np.abs(plain - ref).max() > 1e-2
+    kc.free()
+    vc.free()

@@ -517,6 +517,49 @@ def test_paged_scores_are_the_probabilities_of_the_attention(oracle):
         start += past + 1
 
 
+# ---- attention sinks --------------------------------------------------------------------------------
+@pytest.mark.parametrize("window,alibi", [(0, False), (9, False), (0, True)])
+def test_paged_attention_sinks_match_the_closed_form(oracle, window, alibi):
+    """sinks: a per-head logit in the denominator of every row's softmax, no value row.  Against numpy in fp64 over
+    the gathered keys and values; sinks of -inf change nothing, to the bit; a large sink takes nearly all of the
+    probability and the output goes to zero."""
+    seqs = [(20, 3), (0, 6), (33, 1)]
+    Hq, Hkv, D, bs = 4, 2, 16, 8
+    case = W.make_paged_case(75, seqs, Hq, Hkv, D, bs, W.F32, W.F32, W.F32, sliding_window=window)
+    sinks = np.array([0.3, -1.5, 2.0, 0.0], np.float32)
+    slopes = np.array([0.5, 0.25, 0.125, 0.0625], np.float32) if alibi else None
+    def run(sk):
+        kc, vc = case["key_cache"].copy(), case["value_cache"].copy()
+        out = oracle.paged_attention(case["q"], case["k_new"], case["v_new"], kc, vc, W.F32, case["past_lens"], case["subsequence_begins"],
+                                     case["block_indices"], case["block_indices_begins"], Hq, Hkv, D, bs, sliding_window=window,
+                                     alibi_slopes=slopes, sinks=sk)
+        return out, kc, vc
+    got, kc, vc = run(sinks)
+    plain, _, _ = run(None)
+    none, _, _ = run(np.full(Hq, -np.inf, np.float32))
+    assert np.array_equal(plain, none)
+    assert np.abs(got - plain).max() > 1e-2
+    q = case["q"].reshape(-1, Hq, D).astype(np.float64)
+    bb = case["block_indices_begins"]
+    for s, (past, qlen) in enumerate(seqs):
+        t0 = case["subsequence_begins"][s]
+        blocks = case["block_indices"][bb[s]:bb[s + 1]]
+        for h in range(Hq):
+            K = oracle.gather_cache_rows(kc, W.F32, blocks, past + qlen, h // (Hq // Hkv), Hkv, D, bs).astype(np.float64)
+            V = oracle.gather_cache_rows(vc, W.F32, blocks, past + qlen, h // (Hq // Hkv), Hkv, D, bs).astype(np.float64)
+            for i in range(qlen):
+                p = past + i
+                j0 = max(0, p - window + 1) if window > 0 else 0
+                sc = (K[j0:p + 1] @ q[t0 + i, h]) / np.sqrt(D)
+                if alibi:
+                    sc = sc + float(slopes[h]) * (np.arange(j0, p + 1) - p)
+                e = np.exp(sc - sc.max())
+                want = (e @ V[j0:p + 1]) / (e.sum() + np.exp(float(sinks[h]) - sc.max()))
+                np.testing.assert_allclose(got[t0 + i].reshape(Hq, D)[h], want, rtol=2e-5, atol=2e-6)
+    big, _, _ = run(np.full(Hq, 60.0, np.float32))
+    assert np.abs(big).max() < 1e-15 * 1e3
+
+
 # ---- the operator's cache rotation ----------------------------------------------------------------
 def _trig_lut(rows, D, base=10000.0, sign=1.0):
     """Row r: cos(r theta_i) for i < D/2, then sign * sin(r theta_i), with the rotary embedding's frequencies."""
