@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer|shapes|decoder|scores|masked] [--no-cpu] [--no-extra] [--no-plugin]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|layer|shapes|mqa|decoder|scores|masked] [--no-cpu] [--no-extra] [--no-plugin]
 
 The LAST stdout line is ONE compact JSON object (under 3 KB); the full per-workload records go to the
 file --detail names, or to stderr.  The headline is the fp16
@@ -623,6 +623,30 @@ def bench_other_shapes(hip, steps, warmup):
     return results
 
 
+def bench_multi_query(hip, steps, warmup):
+    """config 3's sequences (64 decode rows, contexts U[512,8192], head size 128, blocks of 32) with more than 16 query
+    heads per kv head -- the stream-K kernel enters a kv head once per group of 8..16 heads, so its K/V rows are read
+    once per group -- and with fp16 queries on a bf16 cache (fp16 operands, blocks converted in registers).  Bytes
+    counted are the cache rows once, as everywhere."""
+    import numpy as np
+    from openvino_contrib_amd import workloads as W
+
+    rng = np.random.Generator(np.random.PCG64(1003))
+    seqs = [(int(c) - 1, 1) for c in rng.integers(512, 8193, size=64)]
+    results = {}
+    for key, Hq, Hkv, qd, cache in (("mq_48_1_f16", 48, 1, W.F16, W.F16), ("mq_32_1_f16", 32, 1, W.F16, W.F16),
+                                    ("mq_64_2_u8", 64, 2, W.F16, W.U8), ("mq_40_2_f16", 40, 2, W.F16, W.F16),
+                                    ("f16q_bf16cache_32_8", 32, 8, W.F16, W.BF16), ("bf16q_bf16cache_32_8", 32, 8, W.BF16, W.BF16)):
+        case = W.make_paged_case(101003, seqs, Hq, Hkv, 128, 32, qd, qd, cache)
+        r = bench_paged(hip, case, steps, warmup, "config3's sequences with %d query heads on %d kv heads, q dtype %d, cache dtype %d" % (Hq, Hkv, qd, cache))
+        r["roofline"] = roofline_hbm(r, key)
+        log("%s: %.3f ms/step, dominant kernel %.3f ms, roofline frac %.3f (%s)"
+            % (key, r["ms_per_step"], r["dominant_kernel_ms"], r["roofline"]["frac"], r["kernel_path"]))
+        results[key] = r
+        del case
+    return results
+
+
 def bench_decoder_layer(hip, steps, warmup):
     """One decoder layer of LLaMA-3-8B's shape (hidden 4096, 32 query / 8 kv heads of 128, MLP 14336) on
     configuration 3's decode batch, as ONE compiled model through the plugin layer: RMS -> q/k/v MatMul ->
@@ -749,7 +773,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "decoder", "scores", "masked", "copy", "mfma"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "mqa", "decoder", "scores", "masked", "copy", "mfma"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
                          "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
@@ -803,6 +827,9 @@ def main():
                           "workloads": {"decoder_layer": bench_decoder_layer(hip, args.steps, args.warmup)}}))
         return
 
+    if args.workload == "mqa":
+        print(json.dumps({"workload": "mqa", "steps": args.steps, "warmup": args.warmup, "workloads": bench_multi_query(hip, args.steps, args.warmup)}))
+        return
     if args.workload == "shapes":
         print(json.dumps({"workload": "shapes", "steps": args.steps, "warmup": args.warmup,
                           "workloads": bench_other_shapes(hip, args.steps, args.warmup)}))
