@@ -24,7 +24,7 @@ extern "C" {
 #endif
 
 #define HIPATTN_VERSION_MAJOR 0
-#define HIPATTN_VERSION_MINOR 3
+#define HIPATTN_VERSION_MINOR 4
 
 typedef enum hipattn_status {
     HIPATTN_OK = 0,
