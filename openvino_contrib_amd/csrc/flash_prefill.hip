@@ -897,6 +897,11 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
         fill_k = t.k + (int64_t)(kv_lo + (group + 2) * kTileK + 8 * wave) * grow;
         fill_v = t.v + (int64_t)(kv_lo + (group + 1) * kTileK + 8 * wave) * grow;
     }
+    // Paged 16-bit caches: the same two instructions per tile whenever all eight rows exist; their source
+    // addresses (block table entry times block stride plus the rows' place in the block) are worked out one
+    // iteration ahead, at the end of a matrix phase.  fill_whole: both tiles of the coming batch are of that kind.
+    bool fill_whole = false;
+    auto whole_rows = [&](int j) __attribute__((always_inline)) { return j < n && kv_lo + j * kTileK + 8 * wave + 8 <= t.kv_len; };
 
     // ---- prologue: K(0), V(0), K(1); group 1 also issues its rows of B(0)
     const int e0 = table_entry(0), e1 = table_entry(1), e2 = table_entry(2), e3 = table_entry(3);
@@ -915,6 +920,11 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
     }
     // entries of the tiles the first iteration loads: K(group + 2) and V(group + 1)
     int entry_v = group ? e2 : e1, entry_k = group ? e3 : e2;
+    if constexpr (kPaged && !kU8) {
+        fill_whole = whole_rows(group + 2);  // (then the rows of V(group + 1) exist as well)
+        fill_k = row_group_base(t, t.k, kv_lo + (group + 2) * kTileK + 8 * wave, entry_k, grow);
+        fill_v = row_group_base(t, t.v, kv_lo + (group + 1) * kTileK + 8 * wave, entry_v, grow);
+    }
     // The query rows were issued first and nobody else reads them: they are converted while the
     // K and V tiles are still on their way.
     if constexpr (kU8)
@@ -1030,7 +1040,17 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
                 recent = load_rows(true, j + group + 2, k_fill, 0) + load_rows(false, j + group + 1, v_fill, 0);
             }
         } else {
-            recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
+            if (fill_whole) {
+                lds_byte* const kd = k_fill + 8 * wave * kRowBytes;
+                lds_byte* const vd = v_fill + 8 * wave * kRowBytes;
+                load_to_lds_16(fill_k, k_lane, kd);
+                load_to_lds_16(fill_k, k_lane1, kd + 4 * kRowBytes);
+                load_to_lds_16(fill_v, v_lane, vd);
+                load_to_lds_16(fill_v, v_lane1, vd + 4 * kRowBytes);
+                recent = 4;
+            } else {
+                recent = load_rows(true, j + group + 2, k_fill, entry_k) + load_rows(false, j + group + 1, v_fill, entry_v);
+            }
         }
         if constexpr (kMask != 0) {
             recent += load_mask_tile(j + 1);
@@ -1083,6 +1103,12 @@ __device__ __forceinline__ void run_pair(const Tile& t, int kv_lo, int kv_hi, ui
             // load's own wait costs the phase nothing)
             entry_v = entry_k;  // the next iteration loads V of the tile whose K was loaded now
             entry_k = table_entry(j + group + 3);
+            if constexpr (!kU8) {
+                fill_v = t.v + (fill_k - t.k);  // the same rows of the same block
+                fill_whole = whole_rows(j + group + 3);
+                fill_k = row_group_base(t, t.k, kv_lo + (j + group + 3) * kTileK + 8 * wave, entry_k, grow);
+                asm volatile("" : "+s"(fill_k), "+s"(fill_v));
+            }
         }
         if constexpr (!kPaged) {
             fill_k += kTileK * grow;
