@@ -5,8 +5,21 @@
 
 namespace hipattn {
 
-__device__ __forceinline__ uint32_t pack_lo(uint32_t a, uint32_t b) { return (a & 0xffffu) | (b << 16); }
-__device__ __forceinline__ uint32_t pack_hi(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xffff0000u); }
+// the low (high) halves of a and b side by side, a's first: one v_perm_b32 each
+__device__ __forceinline__ uint32_t pack_lo(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
+__device__ __forceinline__ uint32_t pack_hi(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
+
+// The largest of the values that lanes l, l ^ 16, l ^ 32 and l ^ 48 hold, in the vector ALU: v_permlane16_swap
+// (the odd rows of sixteen lanes of the first operand change places with the even rows of the second) and
+// v_permlane32_swap (the same for the two halves of the wavefront) on two copies of the value leave every
+// lane with both partners' values; through LDS (ds_bpermute) each step is a round trip that the softmax of
+// every block would wait for.
+__device__ __forceinline__ float max_over_rows(float x) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(y), __float_as_uint(y), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
 
 __device__ __forceinline__ half8_t as_half8(uint4_t v) { return __builtin_bit_cast(half8_t, v); }
 

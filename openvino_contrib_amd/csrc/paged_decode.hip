@@ -411,8 +411,7 @@ __device__ __forceinline__ void process_block(WaveState& st, BlockRegs<kU8>& b, 
             mloc = fmaxf(mloc, sv[j]);
         }
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    mloc = max_over_rows(mloc);
     const float m_new = fmaxf(st.m, mloc);  // finite: every processed block holds an attended token
     const float alpha = fast_exp2(st.m - m_new);
     st.m = m_new;
@@ -1273,8 +1272,7 @@ __device__ __forceinline__ typename Op16<kBf16>::vec8 softmax_unit(WaveState256&
             sv[t * 4 + r] = x;
             mloc = fmaxf(mloc, x);
         }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    mloc = max_over_rows(mloc);
     const float m_new = fmaxf(st.m, mloc);
     // (-inf only while nothing has been attended yet and this unit's blocks both lie outside the cache:
     // everything stays at zero then; exp2(-inf - -inf) would be NaN)
@@ -1413,8 +1411,7 @@ __device__ __forceinline__ Op16<false>::vec8 softmax_unit8(WaveState256& st, con
             sv[j] = (tok >= j0 && tok < ctx && ((tiles >> t) & 1)) ? x * c : -INFINITY;
             mloc = fmaxf(mloc, sv[j]);
         }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    mloc = max_over_rows(mloc);
     const float m_new = fmaxf(st.m, mloc);
     const float m_use = m_new == -INFINITY ? 0.0f : m_new;  // (see softmax_unit)
     const float alpha = fast_exp2(st.m - m_use);
