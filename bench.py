@@ -275,10 +275,10 @@ def bench_sdpa(hip, case, steps, warmup, name):
 # rocprofv3 --pmc runs of this script on the default seeds (scale factors from a plain 1 GiB copy,
 # profiles/copy_calibration.txt); the file each pair of numbers was read from is named beside it.
 RECORDED_TRAFFIC = {
-    "c3": ((563542.9 * 2.0 + 3258.1) * 1024, "profiles/paged_decode_kernel_config3_fp16.txt"),
-    "c4": ((1225893.3 * 2.0 + 12670.5) * 1024, "profiles/paged_decode_kernel_config4_u8.txt"),
-    "c2": ((49302.8 * 2.0 + 65536.0) * 1024, "profiles/sdpa_flash_kernel_config2_bf16.txt"),
-    "c5": ((786149.2 * 2.0 + 6319.5) * 1024, "profiles/paged_attention_config5_mixed.txt"),  # the decode kernel of the mixed step
+    "c3": ((563582.6 * 2.0 + 3258.4) * 1024, "profiles/paged_decode_kernel_config3_fp16.txt"),
+    "c4": ((1225872.7 * 2.0 + 12671.2) * 1024, "profiles/paged_decode_kernel_config4_u8.txt"),
+    "c2": ((49302.7 * 2.0 + 65536.0) * 1024, "profiles/sdpa_flash_kernel_config2_bf16.txt"),
+    "c5": ((786147.1 * 2.0 + 6318.8) * 1024, "profiles/paged_attention_config5_mixed.txt"),  # the decode kernel of the mixed step
 }
 
 
