@@ -647,6 +647,78 @@ def bench_multi_query(hip, steps, warmup):
     return results
 
 
+def bench_stream_reader(hip):
+    """What N compute units stream when each runs one workgroup that only reads (stream_yardstick.hip): alone, and
+    launched just ahead of config 5's chunk sequences (the flash kernel over the block table, which then has the
+    other compute units), as the decode kernel of a mixed batch is."""
+    import ctypes
+    from openvino_contrib_amd import build as hip_build
+    from openvino_contrib_amd import device_case as H
+    from openvino_contrib_amd import workloads as W
+    if not os.path.exists(hip_build.YARDSTICK_LIB_PATH):
+        sys.exit("bench.py: %s is missing (python -m openvino_contrib_amd.build)" % hip_build.YARDSTICK_LIB_PATH)
+    yard = ctypes.CDLL(hip_build.YARDSTICK_LIB_PATH)
+    yard.stream_yardstick_launch.argtypes = [ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                             ctypes.POINTER(ctypes.c_longlong)]
+    total = 2 << 30
+    buf, sink = hip.DeviceBuffer(total), hip.DeviceBuffer(256)
+    buf.fill(3)
+    side, main = hip.Stream(), hip.Stream()
+    case = W.config5(n_decode=0)
+    dev = H.PagedDeviceCase(hip, case)
+    desc = H.pa_desc(hip, case, flags=hip.PA_SKIP_CACHE_WRITE)
+    ws = hip.DeviceBuffer(hip.paged_attention_workspace_size(desc))
+
+    def chunks():
+        hip.paged_attention(desc, dev.q, dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                            dev.subsequence_begins, dev.block_indices, dev.block_indices_begins, dev.out, ws, stream=main)
+
+    def timed(workgroups, beside):
+        best, chunk_ms = None, None
+        for _ in range(5):
+            r0, r1, c0, c1 = hip.Event(), hip.Event(), hip.Event(), hip.Event()
+            nread = ctypes.c_longlong()
+            r0.record(side)
+            rc = yard.stream_yardstick_launch(buf.ptr, total, workgroups, sink.ptr, side.handle, ctypes.byref(nread))
+            if rc != 0:
+                sys.exit("bench.py: stream_yardstick_launch failed with HIP error %d" % rc)
+            r1.record(side)
+            if beside:
+                c0.record(main)
+                chunks()
+                c1.record(main)
+            r1.synchronize()
+            main.synchronize()
+            ms = r0.elapsed_ms(r1)
+            if best is None or ms < best:
+                best, chunk_ms = ms, (c0.elapsed_ms(c1) if beside else None)
+            for e in (r0, r1, c0, c1):
+                e.close()
+        gbs = nread.value / (best * 1e-3) / 1e9
+        return {"workgroups": workgroups, "reader_gb_per_s": _r(gbs), "per_cu_gb_per_s": _r(gbs / workgroups), "frac_of_hbm_peak": _r(gbs / HBM_PEAK_GBS),
+                "chunks_ms_beside": None if chunk_ms is None else _r(chunk_ms)}
+
+    for _ in range(40):  # clock ramp
+        chunks()
+    main.synchronize()
+    c0, c1 = hip.Event(), hip.Event()
+    c0.record(main)
+    for _ in range(20):
+        chunks()
+    c1.record(main)
+    c1.synchronize()
+    cus = hip.device_info(0).compute_units
+    out = {"workload": "stream", "reader": "512 threads and all LDS of a compute unit per workgroup, 64 KB in flight per workgroup, 2 GiB read once",
+           "chunks_alone_ms": _r(c0.elapsed_ms(c1) / 20),
+           "alone": [timed(n, False) for n in (cus, cus // 2, 90, 64, 32)],
+           "ahead_of_config5_chunks": [timed(n, True) for n in (90, 64)]}
+    for r in out["alone"] + out["ahead_of_config5_chunks"]:
+        log("reader on %3d compute units%s: %.0f GB/s, %.1f per compute unit" %
+            (r["workgroups"], "" if r["chunks_ms_beside"] is None else " ahead of the chunks (%.3f ms)" % r["chunks_ms_beside"],
+             r["reader_gb_per_s"], r["per_cu_gb_per_s"]))
+    return out
+
+
 def bench_decoder_layer(hip, steps, warmup):
     """One decoder layer of LLaMA-3-8B's shape (hidden 4096, 32 query / 8 kv heads of 128, MLP 14336) on
     configuration 3's decode batch, as ONE compiled model through the plugin layer: RMS -> q/k/v MatMul ->
@@ -773,9 +845,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "mqa", "decoder", "scores", "masked", "copy", "mfma"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "mqa", "decoder", "scores", "masked", "copy", "mfma", "stream"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
-                         "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels")
+                         "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels; "
+                         "stream = a plain reader on a share of the compute units, alone and beside config 5's chunks")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
                     help="untimed GPU time of the step run ahead of the warmup steps (0 for hardware-counter runs, "
                          "which only count bytes)")
@@ -815,6 +888,10 @@ def main():
                 sys.exit("bench.py: mfma_yardstick failed with HIP error %d" % rc)
             out[name] = {"tflops": tf.value, "shader_ghz": ghz.value, "frac_of_peak": tf.value / MFMA_BF16_PEAK_TFLOPS}
         print(json.dumps(out))
+        return
+
+    if args.workload == "stream":
+        print(json.dumps(bench_stream_reader(hip)))
         return
 
     if args.workload == "layer":

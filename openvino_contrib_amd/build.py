@@ -92,11 +92,12 @@ YARDSTICK_LIB_PATH = os.path.join(CSRC, "bench", "libmfma_yardstick.so")
 
 
 def build_bench_tools():
-    """The MFMA yardstick of bench.py --workload mfma: a library of its own, not part of libhipattn."""
-    cmd = [hipcc()] + HIPCC_FLAGS + ["-shared", os.path.join(CSRC, "bench", "mfma_yardstick.hip"), "-o", YARDSTICK_LIB_PATH]
+    """The yardsticks of bench.py --workload mfma and --workload stream: a library of its own, not part of libhipattn."""
+    sources = [os.path.join(CSRC, "bench", name) for name in ("mfma_yardstick.hip", "stream_yardstick.hip")]
+    cmd = [hipcc()] + HIPCC_FLAGS + ["-shared"] + sources + ["-o", YARDSTICK_LIB_PATH]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
-        raise RuntimeError("hipcc failed on mfma_yardstick.hip:\n%s" % r.stderr[-4000:])
+        raise RuntimeError("hipcc failed on the yardsticks:\n%s" % r.stderr[-4000:])
     return YARDSTICK_LIB_PATH
 
 
