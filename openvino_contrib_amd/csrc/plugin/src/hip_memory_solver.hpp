@@ -2,8 +2,8 @@
 // not meet share addresses.  The reference packs its "mutable blob" the same way with ov::MemorySolver
 // (src/memory_manager/model/cuda_memory_model_builder.cpp:11-25, one box per tensor with the indices of
 // its producing and its last consuming operation) and hands a blob to each running request from a pool
-// (src/memory_manager/cuda_memory_pool.cpp:34-42); here every request owns its blob, which grows when an
-// infer with larger shapes needs it to.
+// (src/memory_manager/cuda_memory_pool.cpp:34-42); here the blob belongs to the worker thread that runs the
+// request (one per stream) and grows when an infer with larger shapes needs it to.
 #pragma once
 
 #include <algorithm>

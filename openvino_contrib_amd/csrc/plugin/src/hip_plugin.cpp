@@ -599,8 +599,7 @@ InferRequest::InferRequest(const std::shared_ptr<const CompiledModel>& compiled,
       compiled_(compiled),
       wait_executor_(wait_executor),
       views_(compiled->num_tensors()),
-      tensor_buffers_(compiled->num_tensors()),
-      workbuffer_() {
+      tensor_buffers_(compiled->num_tensors()) {
     HIP_PLUGIN_CHECK(hipattn_set_device(compiled_->config().device_id));
     // host tensors for ports of known shape; dynamic outputs are shaped by infer_postprocess
     auto host_tensor = [](const ov::Output<const ov::Node>& port) {
@@ -884,7 +883,7 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
         packed_bytes_ = solve_memory(boxes, solved_offsets_);
         solved_boxes_ = boxes;
     }
-    char* const blob = packed_bytes_ ? (char*)blob_.reserve(packed_bytes_) : nullptr;
+    char* const blob = packed_bytes_ ? (char*)thread_context.blob.reserve(packed_bytes_) : nullptr;
     for (size_t i = 0; i < packed.size(); i++) views_[packed[i].id].device = blob + solved_offsets_[i];
     unpacked_bytes_ = apart;
 
@@ -914,7 +913,7 @@ void InferRequest::prepare_steps(const ThreadContext& thread_context, const Infe
         for (size_t b : req.mutable_sizes) total += (b + 255) / 256 * 256;
         arena = std::max(arena, total);
     }
-    char* const arena_base = arena ? (char*)workbuffer_.reserve(arena) : nullptr;
+    char* const arena_base = arena ? (char*)thread_context.workbuffer.reserve(arena) : nullptr;
     for (size_t si = 0; si < sequence.size(); si++) {
         char* base = arena_base;
         for (size_t b : requests[si].mutable_sizes) {

@@ -128,8 +128,15 @@ private:
 
 // Worker threads of one device; each owns a stream.  Tasks handed to run() execute on one of them
 // (src/cuda_thread_pool.cpp:11-72); the stream of the executing thread is get_thread_context().
+// A worker also owns the memory of whatever request it is running: the blob that holds an infer's intermediate
+// tensors and the scratch arena of its operators.  A compiled model with NUM_STREAMS = n thus holds n blobs however
+// many requests exist, and a request that finds every worker busy waits in the pool's queue -- what the reference
+// gets from a pool of n blobs that a request blocks on (src/memory_manager/cuda_memory_pool.cpp:34-42).  Both only
+// grow; they are touched by the thread that owns the context alone (mutable: handed out as const ThreadContext&).
 struct ThreadContext {
     Stream stream;
+    mutable Allocation blob;        // every operator output of the running infer that nothing else owns, packed by lifetime
+    mutable Allocation workbuffer;  // scratch arena shared by the steps of the running infer
 };
 class ThreadPool : public ov::threading::ITaskExecutor {
 public:
@@ -231,11 +238,10 @@ private:
     void bind_batched_tensors();
     std::vector<TensorView> views_;               // per TensorID, rebuilt by every infer
     std::vector<Allocation> tensor_buffers_;      // per TensorID, grow-only: uploaded inputs and constants
-    Allocation blob_;                             // every other operator output of one infer, packed by lifetime
-    size_t packed_bytes_ = 0, unpacked_bytes_ = 0;  // the blob of the last infer; what its tensors take side by side
+    // every other operator output of one infer lies in the blob of the worker that runs it (ThreadContext), packed by lifetime
+    size_t packed_bytes_ = 0, unpacked_bytes_ = 0;  // what the last infer took of that blob; what its tensors take side by side
     std::vector<MemoryBox> solved_boxes_;         // the boxes the offsets below were worked out for
     std::vector<size_t> solved_offsets_;
-    Allocation workbuffer_;                       // scratch arena shared by the steps of one infer
     std::set<TensorID> constants_on_device_;      // Constant outputs already uploaded
     std::vector<std::unique_ptr<Event>> ev_begin_, ev_end_;
     std::vector<size_t> ev_step_;

@@ -334,6 +334,51 @@ def test_infer_request_replays_a_graph(hip, oracle):
     assert np.array_equal(step(x3_st, positions3), got3) and counts() == (2, 5)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("streams", [1, 2])
+def test_requests_share_the_blobs_of_the_device_workers(hip, oracle, streams):
+    """Intermediate tensors live in the blob of the worker thread that runs a request (one per stream), not in the
+    request: three requests of one compiled model with inputs of three sizes, run in turn and in flight together,
+    each get their own results, also when an infer replays a graph recorded before the other requests used the blob."""
+    rng = np.random.default_rng(21)
+    g, gamma = _small_chain()
+    compiled = P.Plugin().compile_model(g.model(), {"HIP_GRAPH_MIN_OPERATORS": "1", "NUM_STREAMS": str(streams)})
+    w_st, wv = storage(rng.standard_normal((256, 256)) / 16, BF16)
+    dw = hip.DeviceBuffer.from_numpy(w_st)
+    cos, sin = rope_tables(100, 64)
+    requests, inputs, refs = [], [], []
+    for T in (24, 56, 9):
+        req = compiled.create_infer_request()
+        req.set_device_input(1, dw.ptr, BF16, [256, 256])
+        req.set_input(2, cos, F32)
+        req.set_input(3, sin, F32)
+        x_st, xv = storage(rng.standard_normal((T, 256)), BF16)
+        positions = rng.integers(0, 100, T).astype(np.int32)
+        req.set_input(0, x_st, BF16)
+        req.set_input(4, positions, P.I32)
+        requests.append(req)
+        inputs.append((x_st, positions))
+        refs.append(_chain_reference(oracle, xv, wv, gamma, cos, sin, positions))
+    first = []
+    for req, ref in zip(requests, refs):
+        req.infer()
+        first.append(H.storage_to_f32(req.output(0)[0], BF16))
+        assert first[-1].shape == ref.shape and scaled_error(first[-1], ref) <= 3e-2
+    for round_ in range(3):  # in turn: from the second round on every request replays its graph
+        for req, want in zip(requests, first):
+            req.infer()
+            assert np.array_equal(H.storage_to_f32(req.output(0)[0], BF16), want), round_
+    for round_ in range(3):  # in flight together
+        for req in requests:
+            req.start_async()
+        for req, want in zip(requests, first):
+            req.wait()
+            assert np.array_equal(H.storage_to_f32(req.output(0)[0], BF16), want), round_
+    sizes = [req.intermediate_memory()[0] for req in requests]
+    assert sizes[1] > sizes[0] > sizes[2] > 0  # what each request's last infer took of its worker's blob
+    dw.free()
+
+
 def test_graph_replay_can_be_switched_off(hip, oracle):
     rng = np.random.default_rng(9)
     g, gamma = _small_chain()
@@ -547,7 +592,7 @@ def test_a_whole_small_decoder_runs_on_the_device(hip, oracle):
 
 
 def test_one_request_through_batches_of_changing_size(hip, oracle):
-    """The request's blob of intermediate tensors is laid out per infer: a decode step, a longer prefill (the blob
+    """The blob of intermediate tensors (the running worker's) is laid out per infer: a decode step, a longer prefill (the blob
     grows and every offset moves), the decode step's size again (the blob is larger than needed), each against the
     oracle chain, on one request."""
     rng = np.random.default_rng(14)
