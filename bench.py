@@ -647,6 +647,45 @@ def bench_multi_query(hip, steps, warmup):
     return results
 
 
+def bench_kv_cache_writer(hip, steps, warmup):
+    """hipattn_kv_cache_write alone on a prefill-sized batch: 32 sequences x 4,096 new tokens, 8 kv heads x 128, fp16 rows
+    into an fp16, a bf16 and a u8 cache (about 1 GB per call: several times the 256 MB of the last-level cache, so that a
+    call does not find the previous call's lines there).  Bytes per call: the new K and V rows read once, their cache
+    rows written once."""
+    from openvino_contrib_amd import device_case as H
+    from openvino_contrib_amd import workloads as W
+    out = {}
+    for cache_dtype, name in ((W.F16, "writer_f16_cache"), (W.BF16, "writer_bf16_cache"), (W.U8, "writer_u8_cache")):
+        case = W.make_paged_case(77, [(0, 4096)] * 32, 8, 8, 128, 32, W.F16, W.F16, cache_dtype)
+        dev = H.PagedDeviceCase(hip, case)
+        desc = H.pa_desc(hip, case)
+
+        def step(_):
+            hip.kv_cache_write(desc, dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                               dev.subsequence_begins, dev.block_indices, dev.block_indices_begins)
+
+        for i in range(warmup + 100):  # (the clock ramp as well)
+            step(i)
+        e0, e1 = hip.Event(), hip.Event()
+        e0.record()
+        for i in range(steps):
+            step(i)
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_ms(e1) / steps
+        e0.close()
+        e1.close()
+        rows = case["T"] * case["Hkv"] * 2
+        nbytes = rows * (128 * 2 + W.cache_row_bytes(cache_dtype, 128))
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out[name] = {"workload": name, "ms_per_step": ms, "bytes": nbytes, "gb_per_s": gbs,
+                     "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                                  "traffic": None, "kernel": "kv_cache_write_kernel"}}
+        log("%s: %.4f ms per call, %.0f MB, %.0f GB/s (%.2f of the HBM peak)" % (name, ms, nbytes / 1e6, gbs, gbs / HBM_PEAK_GBS))
+        dev.free()
+    return out
+
+
 def bench_stream_reader(hip):
     """What N compute units stream when each runs one workgroup that only reads (stream_yardstick.hip): alone, and
     launched just ahead of config 5's chunk sequences (the flash kernel over the block table, which then has the
@@ -845,10 +884,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "mqa", "decoder", "scores", "masked", "copy", "mfma", "stream"],
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "c5u8", "layer", "shapes", "mqa", "decoder", "scores", "masked", "copy", "mfma", "stream", "writer"],
                     help="copy = plain 1 GiB device copy and fill, the yardstick for hardware byte counters; "
                          "mfma = register-fed bf16 MFMAs only, the yardstick for the MFMA-bound kernels; "
-                         "stream = a plain reader on a share of the compute units, alone and beside config 5's chunks")
+                         "stream = a plain reader on a share of the compute units, alone and beside config 5's chunks; "
+                         "writer = hipattn_kv_cache_write alone on a prefill-sized batch")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
                     help="untimed GPU time of the step run ahead of the warmup steps (0 for hardware-counter runs, "
                          "which only count bytes)")
@@ -892,6 +932,11 @@ def main():
 
     if args.workload == "stream":
         print(json.dumps(bench_stream_reader(hip)))
+        return
+
+    if args.workload == "writer":
+        print(json.dumps({"workload": "writer", "steps": args.steps, "warmup": args.warmup,
+                          "workloads": bench_kv_cache_writer(hip, args.steps, args.warmup)}))
         return
 
     if args.workload == "layer":
