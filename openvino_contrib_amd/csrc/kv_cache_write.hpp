@@ -2,6 +2,8 @@
 // paged-attention prologue kernel (which also plans the decode schedule in the same launch).
 #pragma once
 
+#include <type_traits>
+
 #include "device_common.hpp"
 #include "kernels.hpp"
 
@@ -45,6 +47,20 @@ __device__ __forceinline__ uint32_t float_to_bits16(float x, int dtype) {
     return dtype == HIPATTN_F16 ? float_to_f16_bits(x) : float_to_bf16_bits(x);
 }
 
+// Minimum (maximum) of a value over each group of sixteen consecutive lanes, every lane getting the result.
+template <bool kMax>
+__device__ __forceinline__ float row16_reduce(float x) {
+    const auto pick = [](float a, float b) { return kMax ? fmaxf(a, b) : fminf(a, b); };
+    const auto dpp = [](float v, auto ctrl) {
+        return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), decltype(ctrl)::value, 0xf, 0xf, false));
+    };
+    x = pick(x, dpp(x, std::integral_constant<int, 0xB1>{}));   // quad_perm [1, 0, 3, 2]
+    x = pick(x, dpp(x, std::integral_constant<int, 0x4E>{}));   // quad_perm [2, 3, 0, 1]
+    x = pick(x, dpp(x, std::integral_constant<int, 0x141>{}));  // row_half_mirror
+    x = pick(x, dpp(x, std::integral_constant<int, 0x140>{}));  // row_mirror
+    return x;
+}
+
 // Eight consecutive elements (d0 .. d0 + 7) of a new 128-element row, given as the 16 bytes `raw` of
 // the kv type, go into the cache row at `row`, converted or quantised.  Sixteen consecutive lanes
 // (a 16-lane group) hold one row between them; the u8 quantiser's minimum and maximum are reduced
@@ -67,11 +83,10 @@ __device__ __forceinline__ void kv_store_row8(const KvWriteParams& p, uint4_t ra
             mn = fminf(mn, x[i]);
             mx = fmaxf(mx, x[i]);
         }
-#pragma unroll
-        for (int m = 1; m < 16; m <<= 1) {  // over the 16 lanes of the row
-            mn = fminf(mn, __shfl_xor(mn, m, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, m, 64));
-        }
+        // over the 16 lanes of the row, in the vector ALU (DPP: lane ^ 1, lane ^ 2, then the mirror image inside
+        // eight and inside sixteen lanes, which by then holds the other half's result)
+        mn = row16_reduce<false>(mn);
+        mx = row16_reduce<true>(mx);
         float scale = (mx - mn) / 255.0f;
         if (scale == 0.0f) scale = 0.0001f;
         const float zp = -mn / scale + 0.0f;  // -0 becomes +0

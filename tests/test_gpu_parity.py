@@ -78,6 +78,31 @@ def test_kv_cache_write_head_counts(hip, oracle, Hkv, kv_dtype, cache_dtype):
     dev.free()
 
 
+@pytest.mark.parametrize("kv_dtype,cache_dtype", [(W.F16, W.F16), (W.BF16, W.U8), (W.F16, W.BF16)])
+def test_kv_cache_write_large_batch_bit_exact(hip, oracle, kv_dtype, cache_dtype):
+    """A batch of some twenty thousand tokens (more wavefronts than the device holds at a time): odd sequence lengths,
+    an empty sequence and two table entries outside the pool -- byte for byte against the oracle."""
+    announce("kv_write large", kv_dtype, cache_dtype)
+    seqs = [(0, 4099), (31, 1), (17, 6001), (5, 0), (100, 2), (64, 7003), (3, 1022), (1000, 5), (0, 3)]
+    case = W.make_paged_case(58, seqs, 8, 8, 128, 32, W.F16, kv_dtype, cache_dtype)
+    assert case["T"] * 2 >= 4 * 8192  # (eight kv heads: two wavefronts per token)
+    case["block_indices"][5] = case["num_blocks"] + 3
+    case["block_indices"][int(case["block_indices_begins"][2]) + 40] = -1
+    case["block_indices_begins"] = case["block_indices_begins"].copy()
+    dev = H.PagedDeviceCase(hip, case)
+    desc = H.pa_desc(hip, case)
+    hip.kv_cache_write(desc, dev.k_new, dev.v_new, dev.key_cache, dev.value_cache, dev.past_lens,
+                       dev.subsequence_begins, dev.block_indices, dev.block_indices_begins)
+    kc, vc = dev.caches()
+    okc, ovc = case["key_cache"].copy(), case["value_cache"].copy()
+    oracle.kv_cache_write(case["k_new"], case["v_new"], okc, ovc, cache_dtype, case["past_lens"],
+                          case["subsequence_begins"], case["block_indices"], case["block_indices_begins"], 8, 128, 32)
+    np.testing.assert_array_equal(kc, okc)
+    np.testing.assert_array_equal(vc, ovc)
+    assert (okc != case["key_cache"]).any(axis=-1).sum() > case["T"] * 8 - 2 * 32 * 8 - 8  # (all but the rows of the two bad blocks)
+    dev.free()
+
+
 def test_kv_cache_write_skips_invalid_targets(hip, oracle):
     announce("kv_write invalid targets")
     case = W.make_paged_case(52, [(3, 40), (0, 33)], 4, 2, 64, 16, W.F16, W.F16, W.F16)
